@@ -1,0 +1,207 @@
+/*
+ * kinetics_amd.h -- C ABI of the MI355X (gfx950) block top-k sparse paged
+ * decode-attention path.
+ *
+ * Every entry point is extern "C", takes plain device pointers and sizes,
+ * returns an int status (KIN_OK == 0), never throws, never allocates or frees
+ * device memory and never synchronises the device (kin_check_page_table, a
+ * debugging aid, is the one documented exception).  All work is enqueued on
+ * the HIP stream passed as the last argument (NULL = the default stream).
+ *
+ * Citations "ref:" are file:line in the Infini-AI-Lab/Kinetics tree and name
+ * the reference interface each entry point stands in for.
+ *
+ * Tensor conventions (all device memory, densely packed, row-major):
+ *   bf16 tensors are passed as uint16_t* (raw bfloat16 bit patterns).
+ *   q, out        [batch, num_q_heads, head_dim]                    bf16
+ *   k, v          [batch, num_kv_heads, head_dim]                   bf16
+ *   kv_cache      [num_pages, 2, page_size, num_kv_heads, head_dim] bf16
+ *                 ("NHD" paged layout, K plane then V plane per page;
+ *                  ref: benchmark/blocktopk_decoder.py:161-164)
+ *   kbar          [batch, kbar_pages, num_kv_heads, head_dim]       bf16
+ *                 per-page representative (mean) key, indexed by LOGICAL page
+ *                 (ref: benchmark/blocktopk_decoder.py:166-168)
+ *   page_indices  [nnz] int32, page_indptr [batch+1] int32,
+ *   last_page_len [batch] int32 in [1, page_size]
+ *                 CSR page table: sequence b owns physical pages
+ *                 page_indices[page_indptr[b] : page_indptr[b+1]] in logical
+ *                 order and holds (n_pages-1)*page_size + last_page_len[b]
+ *                 tokens (ref: benchmark/blocktopk_decoder.py:141-149).
+ *   sel_pages     [batch, num_kv_heads, sel_stride] int32 physical page ids,
+ *   sel_count     [batch, num_kv_heads] int32
+ *                 per-(sequence, KV head) list of pages to attend to; the
+ *                 final entry is always the sequence's last page
+ *                 (ref: benchmark/blocktopk_decoder.py:143,217-221).
+ *
+ * Supported shapes: head_dim == 128, page_size == 16,
+ * num_q_heads % num_kv_heads == 0 and group size num_q_heads/num_kv_heads <= 8.
+ */
+#ifndef KINETICS_AMD_H
+#define KINETICS_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t kin_bf16_t;  /* raw bfloat16 bits */
+typedef void* kin_stream_t;   /* a hipStream_t */
+
+enum kin_status {
+  KIN_OK = 0,
+  KIN_ERR_NULL_POINTER = 1,  /* a required pointer argument is NULL */
+  KIN_ERR_BAD_SHAPE = 2,     /* a size argument is out of range / inconsistent */
+  KIN_ERR_UNSUPPORTED = 3,   /* valid request outside the compiled fast paths */
+  KIN_ERR_WORKSPACE = 4,     /* workspace missing or too small */
+  KIN_ERR_LAUNCH = 5,        /* the HIP runtime refused a launch / call */
+  KIN_ERR_PAGE_TABLE = 6,    /* kin_check_page_table found an invalid entry */
+  KIN_ERR_MISALIGNED = 7     /* a tensor pointer is not 16-byte aligned */
+};
+
+/* Library version (major*10000 + minor*100 + patch). */
+int kin_version(void);
+
+/* Human-readable text of the last non-OK status on the calling thread
+ * (thread-local; empty string if none). */
+const char* kin_last_error(void);
+
+/* Static name of a status code ("KIN_OK", "KIN_ERR_BAD_SHAPE", ...). */
+const char* kin_status_string(int status);
+
+/*
+ * (1) Paged KV append -- replaces mylib::update_kv ->
+ * flashinfer.append_paged_kv_cache (ref: benchmark/blocktopk_decoder.py:23-46,
+ * 209-213; semantics of LiteSys copy_to_cache,
+ * ref: LiteSys/litesys/attention/cache_utils.py:5-51).
+ *
+ * The page table describes the cache AFTER the append: the new token of
+ * sequence b is written at slot last_page_len[b]-1 of its last page.  When
+ * that write fills the page (last_page_len[b] == page_size) and kbar != NULL,
+ * kbar[b, n_pages-1, h, :] is set to the mean of the page's page_size keys
+ * (fp32 sum in slot order, times 1/page_size, round-to-nearest-even to bf16).
+ * Sequences with an empty page list are skipped.  kbar may be NULL.
+ */
+int kin_append_paged_kv(const kin_bf16_t* k, const kin_bf16_t* v,
+                        kin_bf16_t* kv_cache, kin_bf16_t* kbar,
+                        const int32_t* page_indices, const int32_t* page_indptr,
+                        const int32_t* last_page_len,
+                        int batch, int num_kv_heads, int head_dim, int page_size,
+                        int64_t num_pages, int kbar_pages, kin_stream_t stream);
+
+/*
+ * Representative keys for every FULL page of every sequence (what a prefill
+ * has to leave behind for the scorer).  The reference fills
+ * compressed_key_cache with random numbers and never maintains it
+ * (ref: benchmark/blocktopk_decoder.py:166-168); this is the missing producer.
+ * Same arithmetic as the append-time update.
+ */
+int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar,
+                   const int32_t* page_indices, const int32_t* page_indptr,
+                   const int32_t* last_page_len,
+                   int batch, int num_kv_heads, int head_dim, int page_size,
+                   int64_t num_pages, int kbar_pages, kin_stream_t stream);
+
+/*
+ * (2)+(3) Page scoring and top-k page selection, fused -- replaces
+ *   csim = einsum("b g d, b n d -> b g n", q, kbar).mean(1); topk(csim, k);
+ *   logical->physical translation; cat(last page)
+ * (ref: benchmark/blocktopk_decoder.py:216-221) and, per KV head, LiteSys
+ * blockwise_topk_sparsity (ref: LiteSys/litesys/attention/sparsity_utils.py:24-47).
+ *
+ * For sequence b and KV head h the candidates are the n_cand = n_pages-1 pages
+ * before the last one.  score[n] = dot(mean_g q[b, h*G+g, :], kbar[b, n, h, :])
+ * in fp32.  k_eff = min(topk, n_cand) pages are selected: descending score,
+ * equal scores by ascending logical index (deterministic).  Outputs:
+ *   sel_pages[b,h,0:k_eff]   physical ids of the selected pages, in that order
+ *   sel_pages[b,h,k_eff]     the sequence's last page (always attended)
+ *   sel_pages[b,h,k_eff+1:]  -1
+ *   sel_count[b,h]           k_eff + 1   (0 for an empty page list)
+ *   sel_logical[b,h,0:k_eff] logical page indices (== torch.topk(...).indices),
+ *                            stride topk; may be NULL
+ *   scores_out[b,h,0:n_cand] fp32 scores, stride kbar_pages; may be NULL
+ *                            (debug/parity only: costs an HBM write)
+ * Requires 1 <= topk < sel_stride, topk <= 2048, n_cand <= kbar_pages <= 16384.
+ */
+int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
+                         const int32_t* page_indices, const int32_t* page_indptr,
+                         int topk,
+                         int32_t* sel_pages, int32_t* sel_count,
+                         int32_t* sel_logical, float* scores_out,
+                         int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                         int kbar_pages, int sel_stride, kin_stream_t stream);
+
+/*
+ * Bytes of workspace kin_sparse_paged_decode / kin_dense_paged_decode need for
+ * the given problem when num_splits is chosen automatically (0) or forced.
+ * max_pages_per_list is an upper bound on any list length (sel_stride, or the
+ * longest sequence's page count).  Returns 0 when no workspace is needed.
+ */
+size_t kin_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads,
+                                  int head_dim, int max_pages_per_list,
+                                  int num_splits);
+
+/* The split count the decode entry points use for num_splits == 0. */
+int kin_decode_auto_splits(int batch, int num_kv_heads, int max_pages_per_list);
+
+/*
+ * (4) Sparse paged gather-attention -- replaces mylib::decode ->
+ * flashinfer BatchDecodeWithPagedKVCacheWrapper.run over the k+1 listed pages
+ * (ref: benchmark/blocktopk_decoder.py:171-184,223-225,255-265: NHD layout,
+ * no positional encoding, sm_scale = 1/sqrt(head_dim) by default).
+ *
+ * out[b, hq, :] = softmax(sm_scale * q[b,hq,:] . K[tokens]) V[tokens] over the
+ * tokens of the pages sel_pages[b,h,0:sel_count[b,h]], h = hq / G; every listed
+ * page is full except the final one, which holds last_page_len[b] tokens.
+ * Accumulation in fp32, output bf16.  lse (may be NULL) receives the natural-log
+ * sum-exp of the scaled logits, [batch, num_q_heads] fp32.  sm_scale <= 0 means
+ * 1/sqrt(head_dim).  num_splits: 0 = automatic, else the number of split-K
+ * partitions per list (>1 needs workspace, see kin_decode_workspace_bytes).
+ * An empty list yields out = 0, lse = -inf.
+ */
+int kin_sparse_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
+                            const int32_t* sel_pages, const int32_t* sel_count,
+                            const int32_t* last_page_len,
+                            kin_bf16_t* out, float* lse,
+                            void* workspace, size_t workspace_bytes,
+                            int batch, int num_q_heads, int num_kv_heads,
+                            int head_dim, int page_size, int64_t num_pages,
+                            int sel_stride, float sm_scale, int num_splits,
+                            kin_stream_t stream);
+
+/*
+ * Dense paged decode attention over every page of each sequence -- replaces
+ * the dense layer's mylib::decode (ref: benchmark/dense_decoder.py:149-170,
+ * 211-219).  Same arithmetic and kernel as kin_sparse_paged_decode; the page
+ * list of sequence b is page_indices[page_indptr[b]:page_indptr[b+1]], shared
+ * by all KV heads.  max_pages_per_seq bounds the longest list (used only to
+ * choose the split count).
+ */
+int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
+                           const int32_t* page_indices, const int32_t* page_indptr,
+                           const int32_t* last_page_len,
+                           kin_bf16_t* out, float* lse,
+                           void* workspace, size_t workspace_bytes,
+                           int batch, int num_q_heads, int num_kv_heads,
+                           int head_dim, int page_size, int64_t num_pages,
+                           int max_pages_per_seq, float sm_scale, int num_splits,
+                           kin_stream_t stream);
+
+/*
+ * Debugging aid, SYNCHRONOUS (waits for the stream): verifies on the device
+ * that page_indptr is non-decreasing from 0 and never exceeds nnz (the length
+ * of page_indices), every page id lies in [0, num_pages), and every
+ * last_page_len lies in [1, page_size] for non-empty sequences.  Returns KIN_ERR_PAGE_TABLE if not.  scratch must
+ * point to at least 4 bytes of device memory (the caller's, not allocated
+ * here).  The reference has no counterpart: flashinfer trusts its metadata.
+ */
+int kin_check_page_table(const int32_t* page_indices, const int32_t* page_indptr,
+                         const int32_t* last_page_len, int batch, int page_size,
+                         int64_t num_pages, int64_t nnz, int32_t* scratch,
+                         kin_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KINETICS_AMD_H */

@@ -1,0 +1,75 @@
+// Shared host/device helpers for the gfx950 block top-k decode kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kinetics_amd.h"
+
+namespace kin {
+
+constexpr int kHeadDim = 128;    // elements per head row (256 B in bf16)
+constexpr int kPageSize = 16;    // tokens per page
+constexpr int kRowBytes = kHeadDim * 2;
+constexpr int kMaxGroup = 8;     // largest supported num_q_heads / num_kv_heads
+constexpr int kMaxTopk = 2048;
+constexpr int kMaxCandidates = 16384;
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+// ---- host side: status + thread-local message -----------------------------
+int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int check_hip(hipError_t e, const char* what);
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Shape rules every entry point shares.  Returns KIN_OK or records an error.
+int check_common_dims(const char* fn, int batch, int num_q_heads, int num_kv_heads,
+                      int head_dim, int page_size);
+
+// ---- device side -----------------------------------------------------------
+#if defined(__HIPCC__)
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// fp32 -> bf16 bits, round-to-nearest-even, NaN kept quiet.
+__device__ __forceinline__ uint32_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+// DPP lane permutes inside a row of 16 lanes (no LDS traffic).
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+constexpr int kDppQuadXor1 = 0xB1;     // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;     // quad_perm:[2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // row_half_mirror: lane i <- 7-i (per 8)
+constexpr int kDppMirror = 0x140;      // row_mirror:      lane i <- 15-i (per 16)
+
+// Sum over each aligned group of 16 lanes; every lane of the group gets it.
+__device__ __forceinline__ float row16_sum(float x) {
+  x += dpp_f<kDppQuadXor1>(x);
+  x += dpp_f<kDppQuadXor2>(x);
+  x += dpp_f<kDppHalfMirror>(x);
+  x += dpp_f<kDppMirror>(x);
+  return x;
+}
+
+// Value of lane (quad base + I) broadcast to the 4 lanes of each quad.
+template <int I>
+__device__ __forceinline__ float quad_bcast(float x) {
+  return dpp_f<(I) | (I << 2) | (I << 4) | (I << 6)>(x);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+#endif  // __HIPCC__
+
+}  // namespace kin

@@ -1,0 +1,287 @@
+// Fused page scoring + top-k page selection.
+//
+// One 256-thread workgroup per (sequence, KV head):
+//   phase 1  stream the sequence's representative keys (256 B each) once,
+//            16 lanes per key with 16-byte loads, fp32 dot with the group-mean
+//            query, DPP reduction inside each 16-lane row; scores stay in LDS
+//            as order-preserving 32-bit keys (never written to HBM);
+//   phase 2  4-pass 8-bit radix select in LDS for the k-th largest key;
+//   phase 3  gather the winners (ties at the threshold by lowest index),
+//            bitonic sort them (score descending, index ascending) in LDS,
+//            translate logical -> physical page ids and append the last page.
+// The kernel is HBM-bound on phase 1: n_cand * 256 B per workgroup.
+#include "kin_common.h"
+
+namespace kin {
+
+struct ScoreTopkParams {
+  const uint16_t* q;
+  const uint16_t* kbar;
+  const int32_t* page_indices;
+  const int32_t* page_indptr;
+  int32_t* sel_pages;
+  int32_t* sel_count;
+  int32_t* sel_logical;  // may be null
+  float* scores_out;     // may be null
+  int num_q_heads, num_kv_heads, group;
+  int kbar_pages, sel_stride, topk;
+  int sort_cap;  // power of two >= topk: slots of the bitonic sort
+};
+
+// Monotone map float -> uint32: a < b  <=>  key(a) < key(b)  (-0 < +0).
+__device__ __forceinline__ uint32_t order_key(float f) {
+  const uint32_t u = __float_as_uint(f);
+  return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
+}
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 8;  // independent 16-byte loads in flight per lane
+
+// Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap]
+__global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t wave_tot[4];
+  __shared__ uint32_t sh_bin, sh_remaining, sh_count;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int item = blockIdx.x;
+  const int b = item / p.num_kv_heads, h = item - b * p.num_kv_heads;
+
+  const int ps = p.page_indptr[b], pe = p.page_indptr[b + 1];
+  const int n_pages = pe - ps;
+  int32_t* sel = p.sel_pages + (int64_t)item * p.sel_stride;
+  if (n_pages <= 0) {
+    for (int i = tid; i < p.sel_stride; i += kThreads) sel[i] = -1;
+    if (tid == 0) p.sel_count[item] = 0;
+    return;
+  }
+  const int n_cand = min(n_pages - 1, p.kbar_pages);
+  const int k_eff = min(p.topk, n_cand);
+
+  const int keys_cap = (p.kbar_pages + 3) & ~3;
+  uint32_t* keys = reinterpret_cast<uint32_t*>(smem);
+  unsigned long long* sortbuf = reinterpret_cast<unsigned long long*>(smem + (size_t)keys_cap * 4);
+
+  // ---- phase 1: scores --------------------------------------------------
+  // Lane owns columns d = 8*(lane%16) .. +7 of the mean query.
+  const int c16 = lane & 15;
+  float qm[8];
+  {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) qm[u] = 0.f;
+    const uint16_t* qp = p.q + ((int64_t)b * p.num_q_heads + (int64_t)h * p.group) * kHeadDim + 8 * c16;
+    for (int g = 0; g < p.group; ++g) {
+      const uint4 w = *reinterpret_cast<const uint4*>(qp + (int64_t)g * kHeadDim);
+      qm[0] += bf16_lo(w.x); qm[1] += bf16_hi(w.x);
+      qm[2] += bf16_lo(w.y); qm[3] += bf16_hi(w.y);
+      qm[4] += bf16_lo(w.z); qm[5] += bf16_hi(w.z);
+      qm[6] += bf16_lo(w.w); qm[7] += bf16_hi(w.w);
+    }
+    const float inv = 1.0f / (float)p.group;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) qm[u] *= inv;
+  }
+  const int64_t row_stride = (int64_t)p.num_kv_heads * kHeadDim;  // elements between logical pages
+  const uint16_t* kb = p.kbar + ((int64_t)b * p.kbar_pages * p.num_kv_heads + h) * kHeadDim + 8 * c16;
+  float* sc_out = p.scores_out ? p.scores_out + (int64_t)item * p.kbar_pages : nullptr;
+  const int sub = tid >> 4;  // 0..15: which of the 16 rows of a pass this lane helps with
+  for (int base = 0; base < n_cand; base += 16 * kUnroll) {
+    uint4 w[kUnroll];
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      const int row = base + j * 16 + sub;
+      w[j] = (row < n_cand) ? *reinterpret_cast<const uint4*>(kb + (int64_t)row * row_stride)
+                            : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      float acc = 0.f;
+      acc = fmaf(qm[0], bf16_lo(w[j].x), acc); acc = fmaf(qm[1], bf16_hi(w[j].x), acc);
+      acc = fmaf(qm[2], bf16_lo(w[j].y), acc); acc = fmaf(qm[3], bf16_hi(w[j].y), acc);
+      acc = fmaf(qm[4], bf16_lo(w[j].z), acc); acc = fmaf(qm[5], bf16_hi(w[j].z), acc);
+      acc = fmaf(qm[6], bf16_lo(w[j].w), acc); acc = fmaf(qm[7], bf16_hi(w[j].w), acc);
+      acc = row16_sum(acc);
+      const int row = base + j * 16 + sub;
+      if (c16 == 0 && row < n_cand) {
+        keys[row] = order_key(acc);
+        if (sc_out) sc_out[row] = acc;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 2: radix select of the k_eff-th largest key -------------------
+  uint32_t prefix = 0, mask = 0;
+  uint32_t remaining = (uint32_t)k_eff;  // how many keys equal to the threshold are taken
+  if (k_eff > 0 && k_eff < n_cand) {
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      hist[tid] = 0;
+      __syncthreads();
+      for (int i = tid; i < n_cand; i += kThreads) {
+        const uint32_t key = keys[i];
+        if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+      }
+      __syncthreads();
+      // Thread t owns bin 255-t, so an inclusive scan over t counts keys in
+      // bins >= 255-t.  The bin where the scan first reaches `remaining` holds
+      // the threshold digit.
+      const uint32_t mine = hist[255 - tid];
+      uint32_t incl = mine;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t up = __shfl_up(incl, off);
+        if (lane >= off) incl += up;
+      }
+      if (lane == 63) wave_tot[wave] = incl;
+      __syncthreads();
+      uint32_t before = 0;
+      for (int wv = 0; wv < wave; ++wv) before += wave_tot[wv];
+      incl += before;
+      const uint32_t excl = incl - mine;
+      if (excl < remaining && remaining <= incl) {
+        sh_bin = 255u - (uint32_t)tid;
+        sh_remaining = remaining - excl;
+      }
+      __syncthreads();
+      prefix |= sh_bin << shift;
+      mask |= 255u << shift;
+      remaining = sh_remaining;
+      __syncthreads();
+    }
+  }
+  const bool take_all = (k_eff >= n_cand);
+  const uint32_t thr = prefix;
+
+  // ---- phase 3: gather, sort, translate --------------------------------------
+  for (int i = tid; i < p.sort_cap; i += kThreads) sortbuf[i] = 0ull;
+  if (tid == 0) sh_count = 0;
+  __syncthreads();
+  if (k_eff > 0) {
+    // Keys above the threshold: any order (the sort fixes it).
+    // Keys equal to it: the `remaining` lowest indices, found by an ordered count.
+    const int per = (n_cand + kThreads - 1) / kThreads;
+    const int lo = min(tid * per, n_cand), hi = min(lo + per, n_cand);
+    uint32_t eq_cnt = 0;
+    for (int i = lo; i < hi; ++i) {
+      const uint32_t key = keys[i];
+      if (take_all || key > thr) {
+        const uint32_t slot = atomicAdd(&sh_count, 1u);
+        sortbuf[slot] = ((unsigned long long)key << 32) | (uint32_t)(0xffffffffu - (uint32_t)i);
+      } else if (key == thr) {
+        eq_cnt++;
+      }
+    }
+    if (!take_all) {
+      // exclusive block scan of eq_cnt in thread order (== index order)
+      uint32_t incl = eq_cnt;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t up = __shfl_up(incl, off);
+        if (lane >= off) incl += up;
+      }
+      if (lane == 63) wave_tot[wave] = incl;
+      __syncthreads();
+      uint32_t before = 0;
+      for (int wv = 0; wv < wave; ++wv) before += wave_tot[wv];
+      uint32_t rank = incl - eq_cnt + before;
+      for (int i = lo; i < hi && rank < remaining; ++i) {
+        const uint32_t key = keys[i];
+        if (key == thr) {
+          const uint32_t slot = atomicAdd(&sh_count, 1u);
+          sortbuf[slot] = ((unsigned long long)key << 32) | (uint32_t)(0xffffffffu - (uint32_t)i);
+          rank++;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // Bitonic sort, descending, over sort_cap (power of two) 64-bit entries; the
+  // zero padding sinks to the end.
+  for (int size = 2; size <= p.sort_cap; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      for (int i = tid; i < (p.sort_cap >> 1); i += kThreads) {
+        const int lo_i = 2 * i - (i & (stride - 1));
+        const int hi_i = lo_i + stride;
+        const bool desc = ((lo_i & size) == 0);
+        const unsigned long long a = sortbuf[lo_i], c = sortbuf[hi_i];
+        if ((a < c) == desc) {
+          sortbuf[lo_i] = c;
+          sortbuf[hi_i] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  const int32_t* table = p.page_indices + ps;
+  for (int i = tid; i < p.sel_stride; i += kThreads) {
+    int32_t out = -1;
+    if (i < k_eff) {
+      const uint32_t logical = 0xffffffffu - (uint32_t)(sortbuf[i] & 0xffffffffull);
+      out = table[logical];
+      if (p.sel_logical) p.sel_logical[(int64_t)item * p.topk + i] = (int32_t)logical;
+    } else if (i == k_eff) {
+      out = table[n_pages - 1];
+    }
+    sel[i] = out;
+  }
+  if (tid == 0) p.sel_count[item] = k_eff + 1;
+}
+
+}  // namespace kin
+
+extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar, const int32_t* page_indices,
+                                    const int32_t* page_indptr, int topk, int32_t* sel_pages, int32_t* sel_count,
+                                    int32_t* sel_logical, float* scores_out, int batch, int num_q_heads,
+                                    int num_kv_heads, int head_dim, int kbar_pages, int sel_stride,
+                                    kin_stream_t stream) {
+  using namespace kin;
+  const char* fn = "kin_block_score_topk";
+  if (!q || !kbar || !page_indices || !page_indptr || !sel_pages || !sel_count)
+    return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
+  int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, kPageSize);
+  if (st) return st;
+  if (topk < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: topk=%d must be >= 1", fn, topk);
+  if (sel_stride <= topk)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must exceed topk=%d (room for the last page)", fn, sel_stride,
+                topk);
+  if (kbar_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: kbar_pages=%d must be >= 1", fn, kbar_pages);
+  if (topk > kMaxTopk) return fail(KIN_ERR_UNSUPPORTED, "%s: topk=%d exceeds the limit %d", fn, topk, kMaxTopk);
+  if (kbar_pages > kMaxCandidates)
+    return fail(KIN_ERR_UNSUPPORTED, "%s: kbar_pages=%d exceeds the limit %d", fn, kbar_pages, kMaxCandidates);
+  if (!aligned16(q) || !aligned16(kbar)) return fail(KIN_ERR_MISALIGNED, "%s: q and kbar must be 16-byte aligned", fn);
+  if (batch == 0) return KIN_OK;
+
+  ScoreTopkParams p;
+  p.q = q;
+  p.kbar = kbar;
+  p.page_indices = page_indices;
+  p.page_indptr = page_indptr;
+  p.sel_pages = sel_pages;
+  p.sel_count = sel_count;
+  p.sel_logical = sel_logical;
+  p.scores_out = scores_out;
+  p.num_q_heads = num_q_heads;
+  p.num_kv_heads = num_kv_heads;
+  p.group = num_q_heads / num_kv_heads;
+  p.kbar_pages = kbar_pages;
+  p.sel_stride = sel_stride;
+  p.topk = topk;
+  const int need = topk < kbar_pages ? topk : kbar_pages;  // k_eff never exceeds either
+  int cap = 2;
+  while (cap < need) cap <<= 1;
+  p.sort_cap = cap;
+  const size_t lds = (size_t)((kbar_pages + 3) & ~3) * 4 + (size_t)cap * 8;
+  const int64_t items = (int64_t)batch * num_kv_heads;
+  if (items > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
+  if (lds > 48 * 1024) {
+    // Above the default dynamic-LDS allowance the runtime wants an explicit opt-in.
+    st = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&score_topk_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                   "hipFuncSetAttribute(score_topk_kernel)");
+    if (st) return st;
+  }
+  score_topk_kernel<<<(unsigned)items, kThreads, lds, static_cast<hipStream_t>(stream)>>>(p);
+  return check_hip(hipGetLastError(), "score_topk_kernel launch");
+}

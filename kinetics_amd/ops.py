@@ -1,0 +1,340 @@
+"""Tensor-level entry points of the block top-k decode path.
+
+Each function checks its tensors (dtype, device, contiguity, shape), then hands
+raw device pointers and the current HIP stream to the C ABI
+(include/kinetics_amd.h).  Nothing here computes: without the HIP library the
+import of ``_lib`` fails.  The same functions are registered as
+``torch.ops.kinetics.*`` custom ops with fake (meta) implementations, the way
+the reference wraps its kernels as ``mylib::update_kv`` / ``mylib::decode``
+(benchmark/blocktopk_decoder.py:23-58,171-184), so a layer built on them stays
+traceable by ``torch.compile(fullgraph=True)``.
+"""
+from __future__ import annotations
+
+from ctypes import c_void_p
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+HEAD_DIM = 128
+PAGE_SIZE = 16
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else c_void_p(t.data_ptr())
+
+
+def _stream(device) -> c_void_p:
+    return c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _require(t: torch.Tensor, name: str, dtype: torch.dtype, ndim=None, device=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
+    if t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if t.device.type != "cuda":
+        raise ValueError(f"{name} must live on the GPU (device 'cuda'), got {t.device}")
+    if device is not None and t.device != device:
+        raise ValueError(f"{name} is on {t.device}, expected {device}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if ndim is not None and t.dim() not in (ndim if isinstance(ndim, tuple) else (ndim,)):
+        raise ValueError(f"{name} must have {ndim} dimensions, got shape {tuple(t.shape)}")
+
+
+def _cache_dims(kv_cache: torch.Tensor):
+    _require(kv_cache, "kv_cache", torch.bfloat16, 5)
+    num_pages, two, page_size, num_kv_heads, head_dim = kv_cache.shape
+    if two != 2:
+        raise ValueError(f"kv_cache must be [num_pages, 2, page_size, num_kv_heads, head_dim], got {tuple(kv_cache.shape)}")
+    return num_pages, page_size, num_kv_heads, head_dim
+
+
+def _kbar_pages(kbar: torch.Tensor, batch: int, num_kv_heads: int, head_dim: int) -> int:
+    """kbar is [B, pages, Hkv, D], or the reference's [B, pages, D] when Hkv == 1."""
+    _require(kbar, "kbar", torch.bfloat16, (3, 4))
+    if kbar.dim() == 3:
+        ok = num_kv_heads == 1 and kbar.shape[0] == batch and kbar.shape[2] == head_dim
+    else:
+        ok = kbar.shape[0] == batch and kbar.shape[2] == num_kv_heads and kbar.shape[3] == head_dim
+    if not ok:
+        raise ValueError(
+            f"kbar shape {tuple(kbar.shape)} does not match batch={batch}, num_kv_heads={num_kv_heads}, head_dim={head_dim}"
+        )
+    return kbar.shape[1]
+
+
+def _table(page_indices, page_indptr, last_page_len, batch, device):
+    _require(page_indices, "page_indices", torch.int32, 1, device)
+    _require(page_indptr, "page_indptr", torch.int32, 1, device)
+    if page_indptr.numel() != batch + 1:
+        raise ValueError(f"page_indptr must have batch+1={batch + 1} entries, got {page_indptr.numel()}")
+    if last_page_len is not None:
+        _require(last_page_len, "last_page_len", torch.int32, 1, device)
+        if last_page_len.numel() != batch:
+            raise ValueError(f"last_page_len must have batch={batch} entries, got {last_page_len.numel()}")
+
+
+# ---------------------------------------------------------------------------
+# (1) append
+# ---------------------------------------------------------------------------
+
+
+def append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len) -> None:
+    """Write one new token per sequence into the paged cache (and refresh the
+    mean key of a page that becomes full).  Stands in for ``mylib::update_kv``
+    (benchmark/blocktopk_decoder.py:23-46,209-213).  The page table describes
+    the cache after the append.  ``kbar`` may be None."""
+    num_pages, page_size, num_kv_heads, head_dim = _cache_dims(kv_cache)
+    dev = kv_cache.device
+    _require(k, "k", torch.bfloat16, 3, dev)
+    _require(v, "v", torch.bfloat16, 3, dev)
+    batch = k.shape[0]
+    if tuple(k.shape) != (batch, num_kv_heads, head_dim) or k.shape != v.shape:
+        raise ValueError(f"k and v must be [batch, {num_kv_heads}, {head_dim}], got {tuple(k.shape)} and {tuple(v.shape)}")
+    _table(page_indices, page_indptr, last_page_len, batch, dev)
+    kbar_pages = 0
+    if kbar is not None:
+        kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim)
+        if kbar.device != dev:
+            raise ValueError("kbar must be on the same device as kv_cache")
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(
+            lib.kin_append_paged_kv(
+                _ptr(k), _ptr(v), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
+                _ptr(last_page_len), batch, num_kv_heads, head_dim, page_size, num_pages, kbar_pages, _stream(dev),
+            )
+        )
+
+
+def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len) -> None:
+    """Fill ``kbar`` with the mean key of every full page (prefill-side producer
+    of what the reference calls compressed_key_cache,
+    benchmark/blocktopk_decoder.py:166-168)."""
+    num_pages, page_size, num_kv_heads, head_dim = _cache_dims(kv_cache)
+    dev = kv_cache.device
+    batch = page_indptr.numel() - 1
+    _table(page_indices, page_indptr, last_page_len, batch, dev)
+    kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(
+            lib.kin_build_kbar(
+                _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len),
+                batch, num_kv_heads, head_dim, page_size, num_pages, kbar_pages, _stream(dev),
+            )
+        )
+
+
+# ---------------------------------------------------------------------------
+# (2)+(3) score + select
+# ---------------------------------------------------------------------------
+
+
+def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count, sel_logical=None, scores_out=None) -> None:
+    """Score every candidate page with the group-mean query and write the
+    top-``topk`` pages plus the last page into ``sel_pages`` / ``sel_count``
+    (in place: fixed buffers, as the reference registers with its decode
+    wrapper, benchmark/blocktopk_decoder.py:143,156-159).  Stands in for
+    lines 216-221 of that file."""
+    _require(q, "q", torch.bfloat16, 3)
+    dev = q.device
+    batch, num_q_heads, head_dim = q.shape
+    _require(sel_pages, "sel_pages", torch.int32, 3, dev)
+    num_kv_heads, sel_stride = sel_pages.shape[1], sel_pages.shape[2]
+    if sel_pages.shape[0] != batch:
+        raise ValueError(f"sel_pages must be [batch, num_kv_heads, stride], got {tuple(sel_pages.shape)}")
+    _require(sel_count, "sel_count", torch.int32, 2, dev)
+    if tuple(sel_count.shape) != (batch, num_kv_heads):
+        raise ValueError(f"sel_count must be [{batch}, {num_kv_heads}], got {tuple(sel_count.shape)}")
+    kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim)
+    _table(page_indices, page_indptr, None, batch, dev)
+    if sel_logical is not None:
+        _require(sel_logical, "sel_logical", torch.int32, 3, dev)
+        if tuple(sel_logical.shape) != (batch, num_kv_heads, topk):
+            raise ValueError(f"sel_logical must be [{batch}, {num_kv_heads}, {topk}], got {tuple(sel_logical.shape)}")
+    if scores_out is not None:
+        _require(scores_out, "scores_out", torch.float32, 3, dev)
+        if tuple(scores_out.shape) != (batch, num_kv_heads, kbar_pages):
+            raise ValueError(f"scores_out must be [{batch}, {num_kv_heads}, {kbar_pages}], got {tuple(scores_out.shape)}")
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(
+            lib.kin_block_score_topk(
+                _ptr(q), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), int(topk), _ptr(sel_pages),
+                _ptr(sel_count), _ptr(sel_logical), _ptr(scores_out), batch, num_q_heads, num_kv_heads, head_dim,
+                kbar_pages, sel_stride, _stream(dev),
+            )
+        )
+
+
+# ---------------------------------------------------------------------------
+# (4) attention
+# ---------------------------------------------------------------------------
+
+
+def decode_workspace_bytes(batch, num_q_heads, num_kv_heads, max_pages_per_list, num_splits=0, head_dim=HEAD_DIM) -> int:
+    return int(_lib.load().kin_decode_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, max_pages_per_list, num_splits))
+
+
+def decode_auto_splits(batch, num_kv_heads, max_pages_per_list) -> int:
+    return int(_lib.load().kin_decode_auto_splits(batch, num_kv_heads, max_pages_per_list))
+
+
+def _decode_common(q, kv_cache, last_page_len, out, lse, workspace):
+    num_pages, page_size, num_kv_heads, head_dim = _cache_dims(kv_cache)
+    dev = kv_cache.device
+    _require(q, "q", torch.bfloat16, 3, dev)
+    batch, num_q_heads, qd = q.shape
+    if qd != head_dim:
+        raise ValueError(f"q head_dim {qd} != kv_cache head_dim {head_dim}")
+    _require(last_page_len, "last_page_len", torch.int32, 1, dev)
+    if last_page_len.numel() != batch:
+        raise ValueError(f"last_page_len must have batch={batch} entries, got {last_page_len.numel()}")
+    if out is None:
+        out = torch.empty_like(q)
+    else:
+        _require(out, "out", torch.bfloat16, 3, dev)
+        if out.shape != q.shape:
+            raise ValueError(f"out shape {tuple(out.shape)} != q shape {tuple(q.shape)}")
+    if lse is not None:
+        _require(lse, "lse", torch.float32, 2, dev)
+        if tuple(lse.shape) != (batch, num_q_heads):
+            raise ValueError(f"lse must be [{batch}, {num_q_heads}], got {tuple(lse.shape)}")
+    ws_bytes = 0
+    if workspace is not None:
+        _require(workspace, "workspace", torch.uint8, 1, dev)
+        ws_bytes = workspace.numel()
+    return dev, batch, num_q_heads, num_kv_heads, head_dim, page_size, num_pages, out, ws_bytes
+
+
+def sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, out=None, lse=None, workspace=None,
+                        sm_scale: float = 0.0, num_splits: int = 0):
+    """Attention of one query token per sequence over the listed pages; stands
+    in for ``mylib::decode`` (benchmark/blocktopk_decoder.py:171-184,223-225).
+    Returns ``out`` [batch, num_q_heads, head_dim] bf16."""
+    dev, batch, hq, hkv, d, ps, num_pages, out, ws_bytes = _decode_common(q, kv_cache, last_page_len, out, lse, workspace)
+    _require(sel_pages, "sel_pages", torch.int32, 3, dev)
+    _require(sel_count, "sel_count", torch.int32, 2, dev)
+    if sel_pages.shape[:2] != (batch, hkv) or tuple(sel_count.shape) != (batch, hkv):
+        raise ValueError(
+            f"sel_pages/sel_count must be [{batch}, {hkv}, stride] / [{batch}, {hkv}], got {tuple(sel_pages.shape)} / {tuple(sel_count.shape)}"
+        )
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(
+            lib.kin_sparse_paged_decode(
+                _ptr(q), _ptr(kv_cache), _ptr(sel_pages), _ptr(sel_count), _ptr(last_page_len), _ptr(out), _ptr(lse),
+                _ptr(workspace), ws_bytes, batch, hq, hkv, d, ps, num_pages, sel_pages.shape[2], float(sm_scale),
+                int(num_splits), _stream(dev),
+            )
+        )
+    return out
+
+
+def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, max_pages_per_seq, out=None, lse=None,
+                       workspace=None, sm_scale: float = 0.0, num_splits: int = 0):
+    """Attention over every page of each sequence; the dense baseline
+    (benchmark/dense_decoder.py:149-170,211-219)."""
+    dev, batch, hq, hkv, d, ps, num_pages, out, ws_bytes = _decode_common(q, kv_cache, last_page_len, out, lse, workspace)
+    _table(page_indices, page_indptr, None, batch, dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(
+            lib.kin_dense_paged_decode(
+                _ptr(q), _ptr(kv_cache), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), _ptr(out),
+                _ptr(lse), _ptr(workspace), ws_bytes, batch, hq, hkv, d, ps, num_pages, int(max_pages_per_seq),
+                float(sm_scale), int(num_splits), _stream(dev),
+            )
+        )
+    return out
+
+
+def check_page_table(page_indices, page_indptr, last_page_len, page_size, num_pages) -> None:
+    """Synchronous device-side validation of a page table (debugging aid);
+    raises KineticsError on an invalid entry."""
+    _require(page_indices, "page_indices", torch.int32, 1)
+    dev = page_indices.device
+    batch = page_indptr.numel() - 1
+    _table(page_indices, page_indptr, last_page_len, batch, dev)
+    scratch = torch.zeros(1, dtype=torch.int32, device=dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(
+            lib.kin_check_page_table(
+                _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), batch, int(page_size), int(num_pages),
+                page_indices.numel(), _ptr(scratch), _stream(dev),
+            )
+        )
+
+
+# ---------------------------------------------------------------------------
+# torch.library registration (namespace "kinetics", defined once at import)
+# ---------------------------------------------------------------------------
+
+torch.library.define(
+    "kinetics::append_paged_kv",
+    "(Tensor k, Tensor v, Tensor(a!) kv_cache, Tensor(b!)? kbar, Tensor page_indices, Tensor page_indptr, "
+    "Tensor last_page_len) -> ()",
+)
+torch.library.define(
+    "kinetics::block_score_topk",
+    "(Tensor q, Tensor kbar, Tensor page_indices, Tensor page_indptr, int topk, Tensor(a!) sel_pages, "
+    "Tensor(b!) sel_count) -> ()",
+)
+torch.library.define(
+    "kinetics::sparse_paged_decode",
+    "(Tensor q, Tensor kv_cache, Tensor sel_pages, Tensor sel_count, Tensor last_page_len, Tensor? workspace, "
+    "float sm_scale, int num_splits) -> Tensor",
+)
+torch.library.define(
+    "kinetics::dense_paged_decode",
+    "(Tensor q, Tensor kv_cache, Tensor page_indices, Tensor page_indptr, Tensor last_page_len, "
+    "int max_pages_per_seq, Tensor? workspace, float sm_scale, int num_splits) -> Tensor",
+)
+
+
+@torch.library.impl("kinetics::append_paged_kv", "cuda")
+def _append_impl(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len):
+    append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len)
+
+
+@torch.library.register_fake("kinetics::append_paged_kv")
+def _append_fake(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len):
+    return None
+
+
+@torch.library.impl("kinetics::block_score_topk", "cuda")
+def _select_impl(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count):
+    block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count)
+
+
+@torch.library.register_fake("kinetics::block_score_topk")
+def _select_fake(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count):
+    return None
+
+
+@torch.library.impl("kinetics::sparse_paged_decode", "cuda")
+def _sparse_impl(q, kv_cache, sel_pages, sel_count, last_page_len, workspace, sm_scale, num_splits):
+    return sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, workspace=workspace,
+                               sm_scale=sm_scale, num_splits=num_splits)
+
+
+@torch.library.register_fake("kinetics::sparse_paged_decode")
+def _sparse_fake(q, kv_cache, sel_pages, sel_count, last_page_len, workspace, sm_scale, num_splits):
+    return torch.empty_like(q)
+
+
+@torch.library.impl("kinetics::dense_paged_decode", "cuda")
+def _dense_impl(q, kv_cache, page_indices, page_indptr, last_page_len, max_pages_per_seq, workspace, sm_scale, num_splits):
+    return dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, max_pages_per_seq,
+                              workspace=workspace, sm_scale=sm_scale, num_splits=num_splits)
+
+
+@torch.library.register_fake("kinetics::dense_paged_decode")
+def _dense_fake(q, kv_cache, page_indices, page_indptr, last_page_len, max_pages_per_seq, workspace, sm_scale, num_splits):
+    return torch.empty_like(q)

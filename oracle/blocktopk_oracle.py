@@ -1,0 +1,320 @@
+"""CPU oracle for block top-k sparse paged decode attention.  TEST INFRASTRUCTURE.
+
+This file is the checker, not the product: only ``tests/``,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may
+import it.  The shipped path (``kinetics_amd``) never does and fails loudly
+when its HIP library is missing.
+
+It restates, in numpy with float64 arithmetic on bfloat16-rounded inputs, the
+algorithm of the reference's block top-k decoder path:
+
+* append            benchmark/blocktopk_decoder.py:209-213 (flashinfer
+                    append_paged_kv_cache; same effect as LiteSys
+                    copy_to_cache, LiteSys/litesys/attention/cache_utils.py:40-51)
+* page scores       benchmark/blocktopk_decoder.py:216
+* top-k pages       benchmark/blocktopk_decoder.py:217; per KV head as in
+                    LiteSys/litesys/attention/sparsity_utils.py:36-38
+* page list         benchmark/blocktopk_decoder.py:218-221 (logical->physical,
+                    last page always appended) -- applied ONCE; the reference
+                    file applies the translation twice and never hands the
+                    result to the decode kernel, which is a defect of that
+                    timing harness, not behaviour to reproduce
+* attention         benchmark/blocktopk_decoder.py:223-225,255-265 (NHD pages,
+                    no positional encoding, scale 1/sqrt(D)); the arithmetic is
+                    LiteSys/litesys/attention/cache_utils.py:54-169
+                    (logits*scale, -inf mask past the length, fp32 softmax,
+                    P.V) with the new token attended
+                    (LiteSys/litesys/attention/batch_cache.py:154-168)
+* dense baseline    benchmark/dense_decoder.py:211-219
+
+flashinfer 0.1.6 (the wheel the reference calls, README.md:81) is not in the
+reference tree; its page-table convention is restated here: sequence b owns
+``page_indices[page_indptr[b]:page_indptr[b+1]]`` and holds
+``(n_pages-1)*page_size + last_page_len[b]`` tokens, the metadata describing
+the cache AFTER the append.
+
+Pinning (tests/test_oracle.py): the reference ships no tests or golden
+vectors for this path, so each function is pinned by what the mathematics
+fixes -- append: clone-and-compare of every byte; mean key: float64 mean
+within one bf16 ulp; scores: mean_g(q_g.k) == (mean_g q_g).k and LiteSys'
+group-mean/block-mean order up to the constant 1/sqrt(D); selection:
+numpy/torch library top-k on the same scores plus hand-built tie cases;
+attention: torch scaled_dot_product_attention on the de-paged K/V when every
+page is selected, out == v for one token, out == V for constant V, q == 0 gives
+the mean of V, permutation invariance of the page list, split-K merge
+invariance, lse == logsumexp.
+
+bfloat16 tensors are numpy uint16 arrays of raw bit patterns throughout.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+# ---------------------------------------------------------------------------
+# bfloat16 <-> float32
+# ---------------------------------------------------------------------------
+
+
+def bf16_to_f32(bits: np.ndarray) -> np.ndarray:
+    """Exact widening of bfloat16 bit patterns (uint16) to float32."""
+    bits = np.ascontiguousarray(bits, dtype=np.uint16)
+    return (bits.astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def f32_to_bf16(x: np.ndarray) -> np.ndarray:
+    """float32 -> bfloat16 bits, round-to-nearest-even (NaN stays NaN)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32)
+    rounded = (u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)
+    nan = (u & np.uint32(0x7FFFFFFF)) > np.uint32(0x7F800000)
+    out = np.where(nan, (u >> np.uint32(16)) | np.uint32(0x40), rounded)
+    return out.astype(np.uint16)
+
+
+# ---------------------------------------------------------------------------
+# page-table helpers
+# ---------------------------------------------------------------------------
+
+
+def seq_pages(page_indices, page_indptr, b):
+    """Physical page ids of sequence ``b`` in logical order."""
+    return np.asarray(page_indices[int(page_indptr[b]) : int(page_indptr[b + 1])], dtype=np.int64)
+
+
+def seq_len(page_indptr, last_page_len, b, page_size):
+    n_pages = int(page_indptr[b + 1]) - int(page_indptr[b])
+    return 0 if n_pages <= 0 else (n_pages - 1) * page_size + int(last_page_len[b])
+
+
+# ---------------------------------------------------------------------------
+# (1) append  -- benchmark/blocktopk_decoder.py:209-213
+# ---------------------------------------------------------------------------
+
+
+def page_mean_key(page_k_bits: np.ndarray) -> np.ndarray:
+    """Representative key of full pages: ``page_k_bits`` is [..., page_size, D]
+    bf16 bits; float32 sum in slot order, times 1/page_size, RNE to bf16."""
+    rows = bf16_to_f32(page_k_bits)
+    ps = rows.shape[-2]
+    acc = np.zeros(rows.shape[:-2] + rows.shape[-1:], dtype=np.float32)
+    for t in range(ps):
+        acc = (acc + rows[..., t, :]).astype(np.float32)
+    return f32_to_bf16(acc * np.float32(1.0 / ps))
+
+
+def append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len):
+    """In place.  k, v: [B, Hkv, D] bits; kv_cache: [P, 2, ps, Hkv, D] bits;
+    kbar: [B, kbar_pages, Hkv, D] bits or None.  Writes the new token at slot
+    ``last_page_len[b]-1`` of the last page; a page that becomes full gets its
+    mean key stored at its logical index."""
+    B, Hkv, _ = k.shape
+    ps = kv_cache.shape[2]
+    for b in range(B):
+        pages = seq_pages(page_indices, page_indptr, b)
+        if len(pages) == 0:
+            continue
+        pid, pos = int(pages[-1]), int(last_page_len[b]) - 1
+        kv_cache[pid, 0, pos] = k[b]
+        kv_cache[pid, 1, pos] = v[b]
+        if kbar is not None and pos == ps - 1 and len(pages) - 1 < kbar.shape[1]:
+            for h in range(Hkv):
+                kbar[b, len(pages) - 1, h] = page_mean_key(kv_cache[pid, 0, :, h, :])
+
+
+def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len):
+    """Mean key of every FULL page of every sequence (in place on ``kbar``)."""
+    B = len(page_indptr) - 1
+    ps = kv_cache.shape[2]
+    for b in range(B):
+        pages = seq_pages(page_indices, page_indptr, b)
+        if len(pages) == 0:
+            continue
+        n_full = len(pages) if int(last_page_len[b]) >= ps else len(pages) - 1
+        n_full = min(n_full, kbar.shape[1])
+        if n_full > 0:
+            # [n_full, ps, Hkv, D] -> [n_full, Hkv, ps, D]
+            kbar[b, :n_full] = page_mean_key(kv_cache[pages[:n_full], 0].transpose(0, 2, 1, 3))
+
+
+# ---------------------------------------------------------------------------
+# (2) scores  -- benchmark/blocktopk_decoder.py:216
+# ---------------------------------------------------------------------------
+
+
+def block_scores(q, kbar, page_indptr):
+    """score[b][h][n] = mean_g q[b, h*G+g, :] . kbar[b, n, h, :] in float64, over
+    the n_cand = n_pages-1 candidate pages.  Returns a list (b) of lists (h) of
+    float64 arrays."""
+    B, Hq, D = q.shape
+    Hkv = kbar.shape[2]
+    G = Hq // Hkv
+    qf = bf16_to_f32(q).astype(np.float64)
+    out = []
+    for b in range(B):
+        n_pages = int(page_indptr[b + 1]) - int(page_indptr[b])
+        n_cand = max(0, min(n_pages - 1, kbar.shape[1]))
+        kb = bf16_to_f32(kbar[b, :n_cand]).astype(np.float64)  # [n, Hkv, D]
+        per_head = []
+        for h in range(Hkv):
+            per_q = np.einsum("gd,nd->gn", qf[b, h * G : (h + 1) * G], kb[:, h, :])  # [G, n]
+            per_head.append(per_q.mean(axis=0))
+        out.append(per_head)
+    return out
+
+
+# ---------------------------------------------------------------------------
+# (3) selection  -- benchmark/blocktopk_decoder.py:217-221
+# ---------------------------------------------------------------------------
+
+
+def select_topk(scores: np.ndarray, k: int) -> np.ndarray:
+    """Indices of the min(k, n) largest scores: descending score, equal scores
+    by ascending index."""
+    n = len(scores)
+    order = np.lexsort((np.arange(n), -np.asarray(scores, dtype=np.float64)))
+    return order[: min(k, n)].astype(np.int64)
+
+
+def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_stride=None):
+    """Returns (sel_pages [B,Hkv,stride] int32 padded with -1, sel_count [B,Hkv],
+    sel_logical list[b][h] of index arrays, scores list[b][h])."""
+    B = q.shape[0]
+    Hkv = kbar.shape[2]
+    stride = topk + 1 if sel_stride is None else sel_stride
+    scores = block_scores(q, kbar, page_indptr)
+    sel_pages = np.full((B, Hkv, stride), -1, dtype=np.int32)
+    sel_count = np.zeros((B, Hkv), dtype=np.int32)
+    sel_logical = []
+    for b in range(B):
+        pages = seq_pages(page_indices, page_indptr, b)
+        row = []
+        for h in range(Hkv):
+            if len(pages) == 0:
+                row.append(np.zeros(0, dtype=np.int64))
+                continue
+            idx = select_topk(scores[b][h], topk)
+            sel_pages[b, h, : len(idx)] = pages[idx]
+            sel_pages[b, h, len(idx)] = pages[-1]
+            sel_count[b, h] = len(idx) + 1
+            row.append(idx)
+        sel_logical.append(row)
+    return sel_pages, sel_count, sel_logical, scores
+
+
+# ---------------------------------------------------------------------------
+# (4) attention  -- benchmark/blocktopk_decoder.py:223-225
+# ---------------------------------------------------------------------------
+
+
+def attend_pages(q_bh, kv_cache, pages, h, last_len, sm_scale):
+    """Softmax attention of the G query rows ``q_bh`` ([G, D] float64) over the
+    tokens of ``pages`` for KV head ``h``; every page full except the final one
+    (``last_len`` tokens).  Returns (out [G, D] float64, lse [G] float64,
+    natural log)."""
+    G, D = q_bh.shape
+    if len(pages) == 0:
+        return np.zeros((G, D)), np.full(G, -np.inf)
+    ps = kv_cache.shape[2]
+    K = bf16_to_f32(kv_cache[np.asarray(pages), 0, :, h, :]).astype(np.float64).reshape(-1, D)
+    V = bf16_to_f32(kv_cache[np.asarray(pages), 1, :, h, :]).astype(np.float64).reshape(-1, D)
+    n_tok = (len(pages) - 1) * ps + int(last_len)
+    K, V = K[:n_tok], V[:n_tok]
+    logits = (q_bh @ K.T) * sm_scale  # [G, n_tok]
+    m = logits.max(axis=1, keepdims=True)
+    p = np.exp(logits - m)
+    s = p.sum(axis=1, keepdims=True)
+    return (p / s) @ V, (m + np.log(s))[:, 0]
+
+
+def sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, sm_scale=None):
+    """out [B, Hq, D] float64 and lse [B, Hq] float64 over the listed pages."""
+    B, Hq, D = q.shape
+    Hkv = kv_cache.shape[3]
+    G = Hq // Hkv
+    scale = 1.0 / np.sqrt(D) if sm_scale is None else sm_scale
+    qf = bf16_to_f32(q).astype(np.float64)
+    out = np.zeros((B, Hq, D))
+    lse = np.full((B, Hq), -np.inf)
+    for b in range(B):
+        for h in range(Hkv):
+            pages = sel_pages[b, h, : int(sel_count[b, h])]
+            o, l = attend_pages(qf[b, h * G : (h + 1) * G], kv_cache, pages, h, last_page_len[b], scale)
+            out[b, h * G : (h + 1) * G] = o
+            lse[b, h * G : (h + 1) * G] = l
+    return out, lse
+
+
+def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, sm_scale=None):
+    """Attention over every page of each sequence -- benchmark/dense_decoder.py:211-219."""
+    B, Hq, D = q.shape
+    Hkv = kv_cache.shape[3]
+    G = Hq // Hkv
+    scale = 1.0 / np.sqrt(D) if sm_scale is None else sm_scale
+    qf = bf16_to_f32(q).astype(np.float64)
+    out = np.zeros((B, Hq, D))
+    lse = np.full((B, Hq), -np.inf)
+    for b in range(B):
+        pages = seq_pages(page_indices, page_indptr, b)
+        for h in range(Hkv):
+            o, l = attend_pages(qf[b, h * G : (h + 1) * G], kv_cache, pages, h, last_page_len[b], scale)
+            out[b, h * G : (h + 1) * G] = o
+            lse[b, h * G : (h + 1) * G] = l
+    return out, lse
+
+
+def merge_partials(outs, lses):
+    """Online-softmax merge of partial attention results over disjoint token
+    sets: outs [S, ..., D], lses [S, ...] (natural log)."""
+    lses = np.asarray(lses, dtype=np.float64)
+    m = lses.max(axis=0)
+    m_safe = np.where(np.isfinite(m), m, 0.0)
+    w = np.exp(lses - m_safe)
+    den = w.sum(axis=0)
+    num = (np.asarray(outs) * w[..., None]).sum(axis=0)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        out = np.where(den[..., None] > 0, num / den[..., None], 0.0)
+        lse = np.where(den > 0, m_safe + np.log(den), -np.inf)
+    return out, lse
+
+
+# ---------------------------------------------------------------------------
+# one decode step  -- benchmark/blocktopk_decoder.py:209-225
+# ---------------------------------------------------------------------------
+
+
+def decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sm_scale=None):
+    """append -> score -> select -> attend.  Mutates kv_cache / kbar.  Returns
+    dict(out, lse, sel_pages, sel_count, sel_logical, scores)."""
+    append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len)
+    sel_pages, sel_count, sel_logical, scores = block_score_topk(q, kbar, page_indices, page_indptr, topk)
+    out, lse = sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, sm_scale)
+    return dict(out=out, lse=lse, sel_pages=sel_pages, sel_count=sel_count, sel_logical=sel_logical, scores=scores)
+
+
+# ---------------------------------------------------------------------------
+# The tie rule of the parity contract
+# ---------------------------------------------------------------------------
+
+
+def selection_matches(got_idx, scores, k, rel_tol=1e-3):
+    """True iff ``got_idx`` is an acceptable top-k of ``scores``: the same set
+    as the oracle's, except that indices may differ where their scores tie
+    with the k-th score within ``rel_tol`` relative.  Returns (ok, message)."""
+    scores = np.asarray(scores, dtype=np.float64)
+    want = select_topk(scores, k)
+    got = np.asarray(got_idx, dtype=np.int64)
+    if len(got) != len(want):
+        return False, f"length {len(got)} != {len(want)}"
+    if len(set(got.tolist())) != len(got):
+        return False, "duplicate indices"
+    if len(got) and (got.min() < 0 or got.max() >= len(scores)):
+        return False, "index out of range"
+    if len(want) == 0:
+        return True, ""
+    kth = scores[want[-1]]
+    tol = rel_tol * max(abs(kth), np.finfo(np.float32).tiny)
+    diff = set(got.tolist()) ^ set(want.tolist())
+    for i in diff:
+        if abs(scores[i] - kth) > tol:
+            return False, f"index {i} score {scores[i]!r} is not within {rel_tol} rel of k-th score {kth!r}"
+    return True, ""

@@ -1,0 +1,146 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol the header
+declares, and rejects bad arguments with the documented status codes before
+touching the device."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from kinetics_amd import _lib
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = ROOT / "include" / "kinetics_amd.h"
+
+A = 0x1000  # a non-null, 16-byte aligned dummy address; never dereferenced on these paths
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+def declared_symbols():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(kin_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree(lib):
+    syms = declared_symbols()
+    assert len(syms) >= 11
+    assert sorted(_lib.SIGNATURES) == syms
+    for s in syms:
+        assert hasattr(lib, s), f"{s} is declared in the header but not exported"
+
+
+def test_version_and_status_strings(lib):
+    assert lib.kin_version() >= 100
+    assert lib.kin_status_string(0) == b"KIN_OK"
+    assert lib.kin_status_string(_lib.KIN_ERR_BAD_SHAPE) == b"KIN_ERR_BAD_SHAPE"
+    assert lib.kin_status_string(99) == b"KIN_ERR_UNKNOWN"
+
+
+def append(lib, k=A, v=A, kv=A, kbar=A, idx=A, ptr=A, last=A, B=2, Hkv=1, D=128, ps=16, P=8, kp=4):
+    return lib.kin_append_paged_kv(k, v, kv, kbar, idx, ptr, last, B, Hkv, D, ps, P, kp, None)
+
+
+def test_append_argument_errors(lib):
+    assert append(lib, k=None) == _lib.KIN_ERR_NULL_POINTER
+    assert append(lib, ptr=None) == _lib.KIN_ERR_NULL_POINTER
+    assert append(lib, B=-1) == _lib.KIN_ERR_BAD_SHAPE
+    assert append(lib, Hkv=0) == _lib.KIN_ERR_BAD_SHAPE
+    assert append(lib, P=0) == _lib.KIN_ERR_BAD_SHAPE
+    assert append(lib, kp=0) == _lib.KIN_ERR_BAD_SHAPE
+    assert append(lib, D=64) == _lib.KIN_ERR_UNSUPPORTED
+    assert append(lib, ps=32) == _lib.KIN_ERR_UNSUPPORTED
+    assert append(lib, kv=A + 2) == _lib.KIN_ERR_MISALIGNED
+    assert b"kv_cache" in lib.kin_last_error()
+    assert append(lib, B=0) == _lib.KIN_OK  # nothing to do, nothing launched
+
+
+def select(lib, q=A, kbar=A, idx=A, ptr=A, topk=4, sel=A, cnt=A, B=2, Hq=4, Hkv=1, D=128, kp=64, stride=5):
+    return lib.kin_block_score_topk(q, kbar, idx, ptr, topk, sel, cnt, None, None, B, Hq, Hkv, D, kp, stride, None)
+
+
+def test_select_argument_errors(lib):
+    assert select(lib, q=None) == _lib.KIN_ERR_NULL_POINTER
+    assert select(lib, cnt=None) == _lib.KIN_ERR_NULL_POINTER
+    assert select(lib, topk=0) == _lib.KIN_ERR_BAD_SHAPE
+    assert select(lib, stride=4) == _lib.KIN_ERR_BAD_SHAPE          # no room for the last page
+    assert select(lib, Hq=5, Hkv=2) == _lib.KIN_ERR_BAD_SHAPE
+    assert select(lib, Hq=16, Hkv=1) == _lib.KIN_ERR_UNSUPPORTED    # group 16 > 8
+    assert select(lib, topk=4096, stride=4097) == _lib.KIN_ERR_UNSUPPORTED
+    assert select(lib, kp=20000) == _lib.KIN_ERR_UNSUPPORTED
+    assert select(lib, kbar=A + 8) == _lib.KIN_ERR_MISALIGNED
+    assert select(lib, B=0) == _lib.KIN_OK
+
+
+def sparse(lib, q=A, kv=A, sel=A, cnt=A, last=A, out=A, ws=None, wsb=0, B=2, Hq=4, Hkv=1, D=128, ps=16, P=8,
+           stride=5, splits=1):
+    return lib.kin_sparse_paged_decode(q, kv, sel, cnt, last, out, None, ws, wsb, B, Hq, Hkv, D, ps, P, stride, 0.0,
+                                       splits, None)
+
+
+def test_decode_argument_errors(lib):
+    assert sparse(lib, out=None) == _lib.KIN_ERR_NULL_POINTER
+    assert sparse(lib, sel=None) == _lib.KIN_ERR_NULL_POINTER
+    assert sparse(lib, stride=0) == _lib.KIN_ERR_BAD_SHAPE
+    assert sparse(lib, splits=-1) == _lib.KIN_ERR_BAD_SHAPE
+    assert sparse(lib, D=256) == _lib.KIN_ERR_UNSUPPORTED
+    assert sparse(lib, q=A + 4) == _lib.KIN_ERR_MISALIGNED
+    # split-K without (enough) workspace
+    assert sparse(lib, splits=3) == _lib.KIN_ERR_WORKSPACE
+    need = lib.kin_decode_workspace_bytes(2, 4, 1, 128, 5, 3)
+    assert need == 2 * 4 * 3 * 129 * 4
+    assert sparse(lib, splits=3, ws=A, wsb=need - 1) == _lib.KIN_ERR_WORKSPACE
+    assert b"workspace" in lib.kin_last_error()
+    assert sparse(lib, B=0) == _lib.KIN_OK
+    dense = lib.kin_dense_paged_decode(A, A, None, A, A, A, None, None, 0, 2, 4, 1, 128, 16, 8, 9, 0.0, 1, None)
+    assert dense == _lib.KIN_ERR_NULL_POINTER
+    dense = lib.kin_dense_paged_decode(A, A, A, A, A, A, None, None, 0, 2, 4, 1, 128, 16, 8, 0, 0.0, 1, None)
+    assert dense == _lib.KIN_ERR_BAD_SHAPE
+
+
+def test_auto_splits_policy(lib):
+    assert lib.kin_decode_auto_splits(4096, 1, 129) == 1      # enough lists to fill the chip
+    assert lib.kin_decode_auto_splits(8, 1, 65) > 1           # few lists: split along pages
+    assert lib.kin_decode_auto_splits(8, 1, 3) == 1           # nothing to split
+    assert lib.kin_decode_workspace_bytes(4096, 4, 1, 128, 129, 0) == 0
+
+
+def test_python_wrapper_maps_status_to_exceptions():
+    with pytest.raises(ValueError, match="KIN_ERR_BAD_SHAPE"):
+        _lib.check(_lib.load().kin_block_score_topk(A, A, A, A, 0, A, A, None, None, 2, 4, 1, 128, 64, 5, None))
+    with pytest.raises(_lib.KineticsError, match="KIN_ERR_WORKSPACE"):
+        _lib.check(sparse(_lib.load(), splits=3))
+
+
+def test_ops_reject_cpu_tensors_loudly():
+    import torch
+
+    from kinetics_amd import ops
+
+    q = torch.zeros(2, 4, 128, dtype=torch.bfloat16)
+    kv = torch.zeros(8, 2, 16, 1, 128, dtype=torch.bfloat16)
+    i32 = torch.zeros(2, dtype=torch.int32)
+    with pytest.raises(ValueError, match="GPU"):
+        ops.sparse_paged_decode(q, kv, torch.zeros(2, 1, 5, dtype=torch.int32), torch.zeros(2, 1, dtype=torch.int32), i32)
+    with pytest.raises(TypeError):
+        ops.sparse_paged_decode(q, kv.float(), None, None, i32)
+
+
+def test_custom_ops_are_registered_with_fake_kernels():
+    import torch
+
+    import kinetics_amd  # noqa: F401
+
+    for name in ("append_paged_kv", "block_score_topk", "sparse_paged_decode", "dense_paged_decode"):
+        assert hasattr(torch.ops.kinetics, name)
+    # the fake kernel gives shape/dtype without running anything (what torch.compile needs)
+    q = torch.empty(3, 4, 128, dtype=torch.bfloat16, device="meta")
+    kv = torch.empty(8, 2, 16, 1, 128, dtype=torch.bfloat16, device="meta")
+    i = torch.empty(3, 1, 5, dtype=torch.int32, device="meta")
+    c = torch.empty(3, 1, dtype=torch.int32, device="meta")
+    l = torch.empty(3, dtype=torch.int32, device="meta")
+    out = torch.ops.kinetics.sparse_paged_decode(q, kv, i, c, l, None, 0.0, 0)
+    assert out.shape == q.shape and out.dtype == torch.bfloat16

@@ -1,0 +1,441 @@
+"""Parity of the HIP path (through the C ABI) against the CPU oracle on the
+same seeded inputs.  Bars: byte moves bit-exact; selected page indices equal
+to the oracle's except where scores tie within 1e-3 relative; bf16 attention
+output within 2e-2 abs/rel of the oracle (float64 on bf16-rounded inputs).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import blocktopk_oracle as O
+from tests import problems as P
+
+pytestmark = pytest.mark.gpu
+
+D, PS = P.HEAD_DIM, P.PAGE_SIZE
+DEV = "cuda"
+OUT_ATOL, OUT_RTOL = 2e-2, 2e-2     # the contract
+TIGHT_ATOL, TIGHT_RTOL = 4e-3, 8e-3  # what fp32 accumulation + one bf16 rounding should give
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from kinetics_amd import ops as _ops
+
+    return _ops
+
+
+class Gpu:
+    """A Problem uploaded to the GPU."""
+
+    def __init__(self, pb: P.Problem):
+        self.pb = pb
+        self.q, self.k, self.v = (P.to_torch(x, DEV) for x in (pb.q, pb.k, pb.v))
+        self.kv = P.to_torch(pb.kv_cache, DEV)
+        self.kbar = P.to_torch(pb.kbar, DEV)
+        self.indices = P.int_tensor(pb.page_indices, DEV)
+        self.indptr = P.int_tensor(pb.page_indptr, DEV)
+        self.last = P.int_tensor(pb.last_page_len, DEV)
+        self.sel = torch.full((pb.B, pb.Hkv, pb.topk + 1), -7, dtype=torch.int32, device=DEV)
+        self.cnt = torch.full((pb.B, pb.Hkv), -7, dtype=torch.int32, device=DEV)
+        self.logical = torch.full((pb.B, pb.Hkv, pb.topk), -7, dtype=torch.int32, device=DEV)
+        self.scores = torch.full((pb.B, pb.Hkv, pb.kbar.shape[1]), float("nan"), dtype=torch.float32, device=DEV)
+
+
+def check_table(ops, g: Gpu):
+    ops.check_page_table(g.indices, g.indptr, g.last, PS, g.pb.num_pages)
+
+
+def assert_out_close(got_bf16: torch.Tensor, want: np.ndarray, what=""):
+    got = got_bf16.float().cpu().numpy().astype(np.float64)
+    err = np.abs(got - want)
+    assert np.all(err <= OUT_ATOL + OUT_RTOL * np.abs(want)), f"{what}: max err {err.max()} (contract)"
+    assert np.all(err <= TIGHT_ATOL + TIGHT_RTOL * np.abs(want)), f"{what}: max err {err.max()} (tight)"
+
+
+def workspace(ops, pb, max_pages, splits):
+    n = ops.decode_workspace_bytes(pb.B, pb.Hq, pb.Hkv, max_pages, splits)
+    return torch.empty(max(n, 16), dtype=torch.uint8, device=DEV)
+
+
+# --------------------------------------------------------------------------- append / kbar
+
+
+@pytest.mark.parametrize("hkv,group", [(1, 4), (2, 2), (8, 2)])
+def test_append_bit_exact(ops, hkv, group):
+    lengths = [3 * PS + r + 1 for r in range(PS)] + [1, PS, 0, 5 * PS]
+    pb = P.make_problem(200 + hkv, lengths, num_kv_heads=hkv, group=group)
+    g = Gpu(pb)
+    check_table(ops, g)
+    ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
+    torch.cuda.synchronize()
+    want_kv, want_kbar = pb.kv_cache.copy(), pb.kbar.copy()
+    O.append_paged_kv(pb.k, pb.v, want_kv, want_kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    assert np.array_equal(P.from_torch(g.kv), want_kv)        # every byte, touched or not
+    assert np.array_equal(P.from_torch(g.kbar), want_kbar)
+    assert not np.array_equal(want_kbar, pb.kbar)             # some page did fill up
+    # without kbar
+    g2 = Gpu(pb)
+    ops.append_paged_kv(g2.k, g2.v, g2.kv, None, g2.indices, g2.indptr, g2.last)
+    assert np.array_equal(P.from_torch(g2.kv), want_kv)
+
+
+def test_build_kbar_bit_exact(ops):
+    lengths = [PS * 37, PS * 5 + 3, 1, 0, PS, PS * 64 + 16]
+    pb = P.make_problem(210, lengths, num_kv_heads=2, group=2, build_kbar=False)
+    g = Gpu(pb)
+    g.kbar.fill_(float("nan"))
+    ops.build_kbar(g.kv, g.kbar, g.indices, g.indptr, g.last)
+    want = P.from_torch(torch.full_like(g.kbar, float("nan")))
+    O.build_kbar(pb.kv_cache, want, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    assert np.array_equal(P.from_torch(g.kbar), want)
+
+
+# --------------------------------------------------------------------------- score + select
+
+
+def run_select(ops, g: Gpu):
+    pb = g.pb
+    ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, pb.topk, g.sel, g.cnt, g.logical, g.scores)
+    torch.cuda.synchronize()
+    return g.sel.cpu().numpy(), g.cnt.cpu().numpy(), g.logical.cpu().numpy(), g.scores.cpu().numpy()
+
+
+def check_selection(pb, sel, cnt, logical, scores, exact=False):
+    want_sel, want_cnt, want_logical, want_scores = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    assert np.array_equal(cnt, want_cnt)
+    for b in range(pb.B):
+        pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+        for h in range(pb.Hkv):
+            c = int(cnt[b, h])
+            if c == 0:
+                assert np.all(sel[b, h] == -1)
+                continue
+            ws = want_scores[b][h]
+            got_idx = logical[b, h, : c - 1]
+            # scores: fp32 on the GPU vs float64
+            gs = scores[b, h, : len(ws)].astype(np.float64)
+            assert np.allclose(gs, ws, rtol=1e-5, atol=1e-5), f"scores b={b} h={h}"
+            ok, msg = O.selection_matches(got_idx, ws, pb.topk)
+            assert ok, f"b={b} h={h}: {msg}"
+            if exact:
+                assert np.array_equal(got_idx, want_logical[b][h])
+            # order: descending GPU score, ties ascending index
+            s_sel = scores[b, h][got_idx]
+            assert np.all(s_sel[:-1] >= s_sel[1:])
+            same = s_sel[:-1] == s_sel[1:]
+            assert np.all(got_idx[:-1][same] < got_idx[1:][same])
+            # translation applied once, last page appended, tail padded
+            assert np.array_equal(sel[b, h, : c - 1], pages[got_idx])
+            assert sel[b, h, c - 1] == pages[-1]
+            assert np.all(sel[b, h, c:] == -1)
+
+
+@pytest.mark.parametrize("hkv,group,topk", [(1, 4, 8), (2, 2, 5), (8, 2, 16), (1, 8, 64), (1, 1, 3)])
+def test_score_topk_small(ops, hkv, group, topk):
+    lengths = [PS * 40 + 3, PS * 9, 1, 0, PS * 3 + 1, PS * 130 + 16, PS * topk + 1, PS * (topk + 1) + 1]
+    pb = P.make_problem(300 + hkv + topk, lengths, num_kv_heads=hkv, group=group, topk=topk)
+    g = Gpu(pb)
+    check_selection(pb, *run_select(ops, g))
+
+
+def test_score_topk_ties_take_lowest_index(ops):
+    # every candidate page has the same mean key -> all scores equal, bit for bit
+    pb = P.make_problem(320, [PS * 50 + 2, PS * 20 + 2], topk=7)
+    pb.kbar[:] = pb.kbar[0, 0, 0]
+    g = Gpu(pb)
+    sel, cnt, logical, scores = run_select(ops, g)
+    for b in range(2):
+        assert logical[b, 0].tolist() == list(range(7))
+    # two-level ties: a few pages much larger, the rest tied
+    pb2 = P.make_problem(321, [PS * 300 + 2], topk=12)
+    base = pb2.kbar[0, 0, 0].copy()
+    pb2.kbar[:] = base
+    qm = O.bf16_to_f32(pb2.q[0]).astype(np.float64).mean(axis=0)
+    big = O.f32_to_bf16((qm * 4).astype(np.float32))  # aligned with the mean query: clearly the largest score
+    for p in (17, 200, 5):
+        pb2.kbar[0, p, 0] = big
+    g2 = Gpu(pb2)
+    sel, cnt, logical, scores = run_select(ops, g2)
+    assert sorted(logical[0, 0, :3].tolist()) == [5, 17, 200]
+    assert logical[0, 0, :3].tolist() == [5, 17, 200]       # equal big scores: ascending index
+    assert logical[0, 0, 3:].tolist() == [0, 1, 2, 3, 4, 6, 7, 8, 9]
+    check_selection(pb2, sel, cnt, logical, scores, exact=True)
+
+
+def test_score_topk_many_candidates(ops):
+    # 12000 candidate pages (192k tokens): dynamic LDS above the default allowance
+    pb = P.make_problem(330, [PS * 12000 + 5, PS * 700 + 1], topk=512, kbar_slack=3)
+    g = Gpu(pb)
+    check_selection(pb, *run_select(ops, g))
+
+
+# --------------------------------------------------------------------------- attention
+
+
+def oracle_sparse(pb, kv=None):
+    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    out, lse = O.sparse_paged_decode(pb.q, pb.kv_cache if kv is None else kv, sel, cnt, pb.last_page_len)
+    return sel, cnt, out, lse
+
+
+@pytest.mark.parametrize("hkv,group", [(1, 4), (1, 8), (8, 2), (2, 1), (1, 3), (2, 6)])
+@pytest.mark.parametrize("splits", [1, 3, 0])
+def test_sparse_decode_matches_oracle(ops, hkv, group, splits):
+    lengths = [PS * 30 + r for r in (1, 2, 7, 15, 16)] + [1, 0, PS, PS * 3 + 4, PS * 100 + 9]
+    pb = P.make_problem(400 + 10 * hkv + group, lengths, num_kv_heads=hkv, group=group, topk=12)
+    sel, cnt, want, want_lse = oracle_sparse(pb)
+    g = Gpu(pb)
+    check_table(ops, g)
+    lse = torch.empty(pb.B, pb.Hq, dtype=torch.float32, device=DEV)
+    out = ops.sparse_paged_decode(g.q, g.kv, P.int_tensor(sel, DEV), P.int_tensor(cnt, DEV), g.last, lse=lse,
+                                  workspace=workspace(ops, pb, pb.topk + 1, splits), num_splits=splits)
+    torch.cuda.synchronize()
+    assert_out_close(out, want, f"hkv={hkv} G={group} splits={splits}")
+    got_lse = lse.cpu().numpy().astype(np.float64)
+    fin = np.isfinite(want_lse)
+    assert np.array_equal(np.isneginf(got_lse), ~fin)
+    assert np.allclose(got_lse[fin], want_lse[fin], rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("hkv,group", [(1, 4), (8, 2), (1, 8)])
+@pytest.mark.parametrize("splits", [1, 4, 0])
+def test_dense_decode_matches_oracle(ops, hkv, group, splits):
+    lengths = [PS * 70 + 5, PS * 33, 1, 0, 17, PS * 257 + 16]
+    pb = P.make_problem(500 + hkv + group, lengths, num_kv_heads=hkv, group=group, table="fragmented")
+    want, want_lse = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    g = Gpu(pb)
+    check_table(ops, g)
+    lse = torch.empty(pb.B, pb.Hq, dtype=torch.float32, device=DEV)
+    out = ops.dense_paged_decode(g.q, g.kv, g.indices, g.indptr, g.last, pb.max_pages, lse=lse,
+                                 workspace=workspace(ops, pb, pb.max_pages, splits), num_splits=splits)
+    torch.cuda.synchronize()
+    assert_out_close(out, want, f"dense hkv={hkv} G={group} splits={splits}")
+    fin = np.isfinite(want_lse)
+    assert np.allclose(lse.cpu().numpy()[fin], want_lse[fin], rtol=1e-4, atol=1e-4)
+
+
+def test_attention_closed_forms_on_gpu(ops):
+    pb = P.make_problem(47, [1, PS * 4 + 3, PS * 9 + 16], num_kv_heads=1, group=4, topk=2)
+    O.append_paged_kv(pb.k, pb.v, pb.kv_cache, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    sel_t, cnt_t = P.int_tensor(sel, DEV), P.int_tensor(cnt, DEV)
+    g = Gpu(pb)
+    out = ops.sparse_paged_decode(g.q, g.kv, sel_t, cnt_t, g.last).float().cpu().numpy()
+    # single token: out == v exactly (weight 1, value already bf16)
+    assert np.array_equal(out[0], np.broadcast_to(O.bf16_to_f32(pb.v[0, 0]), (4, D)))
+    # constant V: out == that constant up to one output rounding
+    cv = pb.v[1, 0]
+    kv2 = pb.kv_cache.copy()
+    kv2[:, 1] = cv
+    out2 = ops.sparse_paged_decode(g.q, P.to_torch(kv2, DEV), sel_t, cnt_t, g.last).float().cpu().numpy()
+    c = O.bf16_to_f32(cv)
+    assert np.all(np.abs(out2 - c) <= np.abs(c) * 2.0 ** -7 + 1e-30)
+    # q = 0: mean of the attended values, lse = log(#tokens)
+    lse = torch.empty(pb.B, pb.Hq, dtype=torch.float32, device=DEV)
+    out3 = ops.sparse_paged_decode(torch.zeros_like(g.q), g.kv, sel_t, cnt_t, g.last, lse=lse).float().cpu().numpy()
+    for b, ntok in [(1, 2 * PS + 3), (2, 2 * PS + 16)]:
+        pages = sel[b, 0, : cnt[b, 0]]
+        V = O.bf16_to_f32(pb.kv_cache[pages, 1, :, 0]).reshape(-1, D)[:ntok].astype(np.float64)
+        assert np.allclose(out3[b], V.mean(axis=0), rtol=8e-3, atol=2e-3)
+        assert np.allclose(lse[b].cpu().numpy(), math.log(ntok), rtol=1e-5)
+
+
+def test_page_list_order_does_not_matter(ops):
+    pb = P.make_problem(610, [PS * 90 + 5] * 3, num_kv_heads=2, group=4, topk=33)
+    sel, cnt, want, _ = oracle_sparse(pb)
+    g = Gpu(pb)
+    a = ops.sparse_paged_decode(g.q, g.kv, P.int_tensor(sel, DEV), P.int_tensor(cnt, DEV), g.last)
+    sel2 = sel.copy()
+    sel2[:, :, :33] = sel[:, :, :33][:, :, ::-1]
+    b = ops.sparse_paged_decode(g.q, g.kv, P.int_tensor(sel2, DEV), P.int_tensor(cnt, DEV), g.last)
+    assert_out_close(a, want)
+    assert_out_close(b, want)
+    assert (a.float() - b.float()).abs().max().item() <= 2e-2
+
+
+def test_out_of_range_page_ids_are_skipped_not_followed(ops):
+    # a corrupt list entry must not be dereferenced: the kernel leaves that page out
+    pb = P.make_problem(620, [PS * 20 + 5], topk=6)
+    sel, cnt, _, _ = oracle_sparse(pb)
+    bad = sel.copy()
+    bad[0, 0, 2] = pb.num_pages + 12345
+    bad[0, 0, 4] = -3
+    keep = np.array([0, 1, 3, 5, 6])
+    want_sel = np.full_like(sel, -1)
+    want_sel[0, 0, :5] = sel[0, 0, keep]
+    want, _ = O.sparse_paged_decode(pb.q, pb.kv_cache, want_sel, np.array([[5]], dtype=np.int32), pb.last_page_len)
+    g = Gpu(pb)
+    out = ops.sparse_paged_decode(g.q, g.kv, P.int_tensor(bad, DEV), P.int_tensor(cnt, DEV), g.last)
+    assert_out_close(out, want)
+
+
+# --------------------------------------------------------------------------- whole step
+
+
+def run_step(ops, g: Gpu, splits=0):
+    pb = g.pb
+    ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
+    ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, pb.topk, g.sel, g.cnt, g.logical, g.scores)
+    out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, workspace=workspace(ops, pb, pb.topk + 1, splits),
+                                  num_splits=splits)
+    torch.cuda.synchronize()
+    return out
+
+
+def check_step(ops, pb, splits=0):
+    g = Gpu(pb)
+    check_table(ops, g)
+    out = run_step(ops, g, splits)
+    kv, kbar = pb.kv_cache.copy(), pb.kbar.copy()
+    res = O.decode_step(pb.q, pb.k, pb.v, kv, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
+    assert np.array_equal(P.from_torch(g.kv), kv)
+    assert np.array_equal(P.from_torch(g.kbar), kbar)
+    pb_after = P.Problem(**{**pb.__dict__, "kv_cache": kv, "kbar": kbar})
+    sel, cnt, logical, scores = (x.cpu().numpy() for x in (g.sel, g.cnt, g.logical, g.scores))
+    check_selection(pb_after, sel, cnt, logical, scores)
+    # Attention is judged on the pages the GPU selected (they may differ from the
+    # oracle's only inside the tie tolerance checked above).
+    want, _ = O.sparse_paged_decode(pb.q, kv, sel, cnt, pb.last_page_len)
+    assert_out_close(out, want, "decode step")
+    same = all(set(logical[b, h, : cnt[b, h] - 1].tolist()) == set(res["sel_logical"][b][h].tolist())
+               for b in range(pb.B) for h in range(pb.Hkv))
+    if same:
+        assert_out_close(out, res["out"], "decode step vs oracle end to end")
+    return same
+
+
+def test_decode_step_tiny_config(ops):
+    """Batch 8, context 4096 (+1 appended), 1 KV head, 4 Q heads, budget 64 pages,
+    random page table."""
+    pb = P.make_problem(0, [4096 + 1] * 8, num_kv_heads=1, group=4, topk=64, table="random")
+    assert check_step(ops, pb)
+
+
+def test_decode_step_qwen3_32b_share_small(ops):
+    """8 Q heads per KV head, budget 256 pages, reference page layout p*B+b."""
+    pb = P.make_problem(3, [8192 + 1] * 6, num_kv_heads=1, group=8, topk=256, table="strided")
+    check_step(ops, pb)
+
+
+def test_decode_step_continuous_batching_mix(ops):
+    """8 KV heads x 2, ragged lengths, per-KV-head selection, fragmented table,
+    budget min(64, pages)."""
+    rng = np.random.default_rng(4)
+    lengths = rng.integers(1024, 8192, size=12).tolist() + [1, 17, PS * 64 + 1, PS * 65 + 1]
+    pb = P.make_problem(4, lengths, num_kv_heads=8, group=2, topk=64, table="fragmented")
+    check_step(ops, pb)
+
+
+def test_decode_step_fills_a_page(ops):
+    # the appended token completes a page: its mean key must appear, and the page
+    # (being the last one) is attended but is not a candidate
+    pb = P.make_problem(5, [PS * 21, PS * 2, PS], num_kv_heads=2, group=4, topk=4)
+    check_step(ops, pb)
+
+
+# --------------------------------------------------------------------------- larger, property-based
+
+
+def test_properties_at_scale(ops):
+    """Sizes the oracle cannot finish quickly: B=256, context 16K, budget 128
+    pages.  Checked through size-independent properties: split-K invariance,
+    dense == sparse when every page is listed, and a spot check of 3 sequences
+    against the oracle."""
+    B, n_pages, topk = 256, 1025, 128
+    torch.manual_seed(1)
+    num_pages = B * n_pages
+    kv = torch.randn(num_pages, 2, PS, 1, D, device=DEV, dtype=torch.float32).to(torch.bfloat16)
+    q = torch.randn(B, 4, D, device=DEV, dtype=torch.float32).to(torch.bfloat16)
+    table = (torch.arange(n_pages, device=DEV, dtype=torch.int32) * B + torch.arange(B, device=DEV, dtype=torch.int32)[:, None])
+    indices = table.reshape(-1).contiguous()
+    indptr = (torch.arange(B + 1, device=DEV, dtype=torch.int32) * n_pages).contiguous()
+    last = torch.full((B,), 1, dtype=torch.int32, device=DEV)
+    kbar = torch.zeros(B, n_pages, 1, D, dtype=torch.bfloat16, device=DEV)
+    ops.build_kbar(kv, kbar, indices, indptr, last)
+    sel = torch.empty(B, 1, topk + 1, dtype=torch.int32, device=DEV)
+    cnt = torch.empty(B, 1, dtype=torch.int32, device=DEV)
+    logical = torch.empty(B, 1, topk, dtype=torch.int32, device=DEV)
+    ops.block_score_topk(q, kbar, indices, indptr, topk, sel, cnt, logical)
+    assert bool((cnt == topk + 1).all())
+    # selected ids: unique, candidates only, last entry the last page
+    lg = logical[:, 0].sort(dim=1).values
+    assert bool((lg[:, 1:] > lg[:, :-1]).all()) and int(lg.min()) >= 0 and int(lg.max()) < n_pages - 1
+    assert torch.equal(sel[:, 0, topk], table[:, -1])
+    assert torch.equal(sel[:, 0, :topk].long(), torch.gather(table.long(), 1, logical[:, 0].long()))
+    # split-K invariance
+    ws = torch.empty(ops.decode_workspace_bytes(B, 4, 1, topk + 1, 4), dtype=torch.uint8, device=DEV)
+    o1 = ops.sparse_paged_decode(q, kv, sel, cnt, last, num_splits=1)
+    o4 = ops.sparse_paged_decode(q, kv, sel, cnt, last, workspace=ws, num_splits=4)
+    assert (o1.float() - o4.float()).abs().max().item() <= 1e-2
+    # dense == sparse over the full table
+    full_cnt = torch.full((B, 1), n_pages, dtype=torch.int32, device=DEV)
+    od = ops.dense_paged_decode(q, kv, indices, indptr, last, n_pages, num_splits=1)
+    os_ = ops.sparse_paged_decode(q, kv, table.reshape(B, 1, n_pages).contiguous(), full_cnt, last, num_splits=1)
+    assert torch.equal(od, os_)
+    # spot check against the oracle
+    rows = [0, 101, 255]
+    kv_np = P.from_torch(kv.reshape(n_pages, B, 2, PS, 1, D)[:, rows].reshape(-1, 2, PS, 1, D))  # pages p*3+j
+    sub_idx = (np.arange(n_pages)[None, :] * 3 + np.arange(3)[:, None]).reshape(-1).astype(np.int32)
+    sub_ptr = (np.arange(4) * n_pages).astype(np.int32)
+    q_np = P.from_torch(q[rows])
+    kbar_np = P.from_torch(kbar[rows])
+    want_sel, want_cnt, want_logical, want_scores = O.block_score_topk(q_np, kbar_np, sub_idx, sub_ptr, topk)
+    for j, b in enumerate(rows):
+        ok, msg = O.selection_matches(logical[b, 0].cpu().numpy(), want_scores[j][0], topk)
+        assert ok, msg
+    want, _ = O.sparse_paged_decode(q_np, kv_np, want_sel, want_cnt, np.ones(3, dtype=np.int32))
+    assert_out_close(o1[rows], want, "scale spot check")
+
+
+# --------------------------------------------------------------------------- layer objects + custom ops
+
+
+def test_layer_objects_follow_the_reference_call_order(ops):
+    from kinetics_amd import BlockTopkPagedAttention, DensePagedAttention
+
+    B, prefix, topk = 5, PS * 48, 8
+    layer = BlockTopkPagedAttention(4, 1, D, B, prefix, prefix + 512, PS, topk, device=DEV, seed=3)
+    torch.manual_seed(7)
+    q = torch.randn(B, 4, D, device=DEV).to(torch.bfloat16)
+    k = torch.randn(B, 1, D, device=DEV).to(torch.bfloat16)
+    v = torch.randn(B, 1, D, device=DEV).to(torch.bfloat16)
+    kv_before = P.from_torch(layer.kv_cache)
+    kbar_before = P.from_torch(layer.compressed_key_cache)
+    out = layer(q, k, v)
+    torch.cuda.synchronize()
+    idx = layer.paged_kv_indices.cpu().numpy()
+    ptr = layer.paged_kv_indptr.cpu().numpy()
+    last = layer.last_kv_lens.cpu().numpy()
+    assert idx.reshape(B, -1)[2, 3] == 3 * B + 2  # reference layout p*B + b
+    res = O.decode_step(P.from_torch(q), P.from_torch(k), P.from_torch(v), kv_before, kbar_before, idx, ptr, last, topk)
+    assert np.array_equal(P.from_torch(layer.kv_cache), kv_before)
+    assert np.array_equal(layer.topk_page_count.cpu().numpy(), res["sel_count"])
+    assert np.array_equal(layer.topk_page_indices.cpu().numpy(), res["sel_pages"])
+    assert_out_close(out, res["out"], "layer")
+    dense = DensePagedAttention(4, 1, D, B, prefix, prefix + 512, PS, share_cache_with=layer)
+    od = dense.decode(q)
+    want, _ = O.dense_paged_decode(P.from_torch(q), kv_before, idx, ptr, last)
+    assert_out_close(od, want, "dense layer")
+
+
+def test_check_page_table_flags_bad_metadata(ops):
+    from kinetics_amd._lib import KineticsError
+
+    pb = P.make_problem(700, [PS * 3 + 1, PS + 5])
+    g = Gpu(pb)
+    check_table(ops, g)
+    bad = g.indices.clone()
+    bad[2] = pb.num_pages
+    with pytest.raises(KineticsError, match="KIN_ERR_PAGE_TABLE"):
+        ops.check_page_table(bad, g.indptr, g.last, PS, pb.num_pages)
+    bad_last = g.last.clone()
+    bad_last[1] = PS + 1
+    with pytest.raises(KineticsError):
+        ops.check_page_table(g.indices, g.indptr, bad_last, PS, pb.num_pages)
+    bad_ptr = g.indptr.clone()
+    bad_ptr[1] = 100
+    with pytest.raises(KineticsError):
+        ops.check_page_table(g.indices, bad_ptr, g.last, PS, pb.num_pages)

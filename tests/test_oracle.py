@@ -1,0 +1,346 @@
+"""Pins the CPU oracle (oracle/blocktopk_oracle.py, oracle/torch_path.py).
+
+The reference ships no tests, golden vectors or fixtures for this path, so the
+oracle is pinned by library routines (torch bf16 casts, torch.topk, torch SDPA,
+scipy logsumexp) and by what the mathematics fixes (closed forms, invariants,
+brute force on small inputs).  Every check is chosen so that a plausible slip
+-- wrong slot, transposed operand, dropped scale, off-by-one page, wrong mask --
+breaks it.  No GPU needed.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+from scipy.special import logsumexp
+
+from oracle import blocktopk_oracle as O
+from oracle import torch_path
+from tests import problems as P
+
+D, PS = P.HEAD_DIM, P.PAGE_SIZE
+
+
+# --------------------------------------------------------------------------- bf16
+
+
+def test_bf16_roundtrip_matches_torch():
+    rng = np.random.default_rng(0)
+    x = np.concatenate([
+        rng.standard_normal(4096).astype(np.float32) * 10,
+        np.array([0.0, -0.0, 1.0, -1.0, 65504.0, 1e-40, 3.3895314e38, np.inf, -np.inf], dtype=np.float32),
+        # exact ties between two bf16 values: must round to even
+        np.array([1.00390625, 1.01171875, -1.00390625], dtype=np.float32),
+    ])
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = O.f32_to_bf16(x)
+    assert np.array_equal(got, want)
+    back = torch.from_numpy(got.view(np.int16)).view(torch.bfloat16).float().numpy()
+    assert np.array_equal(O.bf16_to_f32(got), back)
+    nan = O.f32_to_bf16(np.array([np.nan], dtype=np.float32))
+    assert np.isnan(O.bf16_to_f32(nan))[0]
+
+
+# --------------------------------------------------------------------------- append
+
+
+@pytest.mark.parametrize("residue", list(range(PS)))
+def test_append_writes_exactly_one_slot(residue):
+    # one length per residue class of L mod page_size, random page table
+    lengths = [3 * PS + residue + 1, residue + 1, 7 * PS + residue + 1]
+    pb = P.make_problem(100 + residue, lengths, num_kv_heads=2, group=2)
+    before = pb.kv_cache.copy()
+    kbar = pb.kbar.copy()
+    O.append_paged_kv(pb.k, pb.v, pb.kv_cache, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    changed = np.zeros(pb.kv_cache.shape[:3], dtype=bool)
+    for b, L in enumerate(lengths):
+        pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+        pid, pos = pages[(L - 1) // PS], (L - 1) % PS  # closed form of "last token's slot"
+        assert np.array_equal(pb.kv_cache[pid, 0, pos], pb.k[b])
+        assert np.array_equal(pb.kv_cache[pid, 1, pos], pb.v[b])
+        changed[pid, :, pos] = True
+    # every other byte is untouched
+    assert np.array_equal(pb.kv_cache[~changed], before[~changed])
+    # kbar changes only where a page became full
+    for b, L in enumerate(lengths):
+        n_pages = (L + PS - 1) // PS
+        if L % PS == 0:
+            pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+            want = O.page_mean_key(pb.kv_cache[pages[-1], 0].transpose(1, 0, 2))
+            assert np.array_equal(kbar[b, n_pages - 1], want)
+            mask = np.ones(kbar.shape[1], dtype=bool)
+            mask[n_pages - 1] = False
+            assert np.array_equal(kbar[b, mask], pb.kbar[b, mask])
+        else:
+            assert np.array_equal(kbar[b], pb.kbar[b])
+
+
+def test_append_skips_empty_sequences():
+    pb = P.make_problem(7, [0, 5, 0, 33])
+    before = pb.kv_cache.copy()
+    O.append_paged_kv(pb.k, pb.v, pb.kv_cache, None, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    assert (pb.kv_cache != before).any(axis=(1, 2, 3, 4)).sum() == 2  # exactly two pages touched
+
+
+def test_page_mean_key_against_float64_and_closed_forms():
+    rng = np.random.default_rng(3)
+    pages = P.randn_bf16(rng, (64, PS, D), scale=3.0)
+    got = O.bf16_to_f32(O.page_mean_key(pages)).astype(np.float64)
+    exact = O.bf16_to_f32(pages).astype(np.float64).mean(axis=1)
+    ulp = np.maximum(np.abs(exact), 2.0 ** -126) * 2.0 ** -7  # one bf16 ulp is <= 2^-7 relative
+    assert np.all(np.abs(got - exact) <= ulp)
+    # constant rows: the mean is that row, exactly
+    row = P.randn_bf16(rng, (1, D))
+    assert np.array_equal(O.page_mean_key(np.repeat(row, PS, axis=0)), row[0])
+    # a single non-zero row of value 16*x gives x
+    z = np.zeros((PS, D), dtype=np.uint16)
+    z[5] = O.f32_to_bf16(np.full(D, 48.0, dtype=np.float32))
+    assert np.array_equal(O.bf16_to_f32(O.page_mean_key(z)), np.full(D, 3.0, dtype=np.float32))
+
+
+def test_build_kbar_covers_full_pages_only():
+    pb = P.make_problem(11, [PS * 4, PS * 2 + 3, 1, 0], num_kv_heads=2, group=1, build_kbar=False)
+    sentinel = np.uint16(0x7FC0)
+    kbar = np.full_like(pb.kbar, sentinel)
+    O.build_kbar(pb.kv_cache, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    full = [4, 2, 0, 0]
+    for b in range(4):
+        pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+        for p in range(kbar.shape[1]):
+            if p < full[b]:
+                for h in range(2):
+                    want = O.page_mean_key(pb.kv_cache[pages[p], 0, :, h, :])
+                    assert np.array_equal(kbar[b, p, h], want)
+            else:
+                assert np.all(kbar[b, p] == sentinel)
+
+
+# --------------------------------------------------------------------------- scores
+
+
+def test_scores_identities():
+    pb = P.make_problem(21, [PS * 9 + 4, PS * 5 + 1], num_kv_heads=2, group=4)
+    sc = O.block_scores(pb.q, pb.kbar, pb.page_indptr)
+    qf = O.bf16_to_f32(pb.q).astype(np.float64)
+    for b in range(pb.B):
+        n_cand = (pb.lengths[b] + PS - 1) // PS - 1
+        for h in range(2):
+            assert sc[b][h].shape == (n_cand,)
+            # mean_g (q_g . k) == (mean_g q_g) . k
+            qbar = qf[b, 4 * h : 4 * h + 4].mean(axis=0)
+            kb = O.bf16_to_f32(pb.kbar[b, :n_cand, h]).astype(np.float64)
+            assert np.allclose(sc[b][h], kb @ qbar, rtol=1e-12, atol=1e-12)
+            # not the other head's keys, not the other head's queries
+            other = O.bf16_to_f32(pb.kbar[b, :n_cand, 1 - h]).astype(np.float64) @ qbar
+            assert not np.allclose(sc[b][h], other)
+
+
+def test_scores_equal_litesys_group_mean_then_block_mean():
+    """LiteSys ranks blocks by mean over the query group, then mean over the
+    block's tokens, of q.k/sqrt(D) (sparsity_utils.py:36-37).  With keys whose
+    page mean is exactly representable this equals score/sqrt(D)."""
+    rng = np.random.default_rng(5)
+    n_pages, G = 6, 4
+    # small integers: sums and the /16 mean are exact in bf16
+    K = (rng.integers(-8, 9, size=(n_pages, PS, D)) * 16).astype(np.float32)
+    kv = np.zeros((n_pages + 1, 2, PS, 1, D), dtype=np.uint16)
+    kv[:n_pages, 0, :, 0] = O.f32_to_bf16(K)
+    indices = np.arange(n_pages + 1, dtype=np.int32)
+    indptr = np.array([0, n_pages + 1], dtype=np.int32)
+    kbar = np.zeros((1, n_pages + 1, 1, D), dtype=np.uint16)
+    O.build_kbar(kv, kbar, indices, indptr, np.array([1], dtype=np.int32))
+    q = P.randn_bf16(rng, (1, G, D))
+    sc = O.block_scores(q, kbar, indptr)[0][0]
+    logits = np.einsum("gd,ptd->gpt", O.bf16_to_f32(q[0]).astype(np.float64), K.astype(np.float64)) / math.sqrt(D)
+    litesys = logits.mean(axis=0).mean(axis=-1)
+    assert np.allclose(sc / math.sqrt(D), litesys, rtol=1e-12, atol=1e-12)
+
+
+# --------------------------------------------------------------------------- selection
+
+
+def test_select_topk_against_library_routines():
+    rng = np.random.default_rng(9)
+    for n, k in [(1, 1), (5, 3), (257, 64), (2048, 128), (100, 100), (100, 250)]:
+        s = rng.standard_normal(n)
+        got = O.select_topk(s, k)
+        kk = min(k, n)
+        want_t = torch.topk(torch.from_numpy(s), kk).indices.numpy()
+        assert np.array_equal(got, want_t)  # distinct values: order is fixed too
+        part = np.argpartition(-s, kk - 1)[:kk]
+        assert set(got.tolist()) == set(part.tolist())
+
+
+def test_select_topk_tie_break_is_lowest_index():
+    assert O.select_topk(np.zeros(10), 4).tolist() == [0, 1, 2, 3]
+    s = np.array([1.0, 5.0, 5.0, 2.0, 5.0, 0.0])
+    assert O.select_topk(s, 2).tolist() == [1, 2]
+    assert O.select_topk(s, 4).tolist() == [1, 2, 4, 3]
+    assert O.select_topk(np.array([]), 3).tolist() == []
+
+
+def test_block_score_topk_page_list_layout():
+    pb = P.make_problem(31, [PS * 20 + 7, PS * 3, 1, 0, PS * 2 + 1], topk=4)
+    sel, cnt, logical, scores = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    assert sel.shape == (5, 1, 5)
+    assert cnt[:, 0].tolist() == [5, 3, 1, 0, 3]  # min(k, n_cand) + 1, 0 for the empty sequence
+    for b in range(5):
+        pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+        c = cnt[b, 0]
+        if c == 0:
+            assert np.all(sel[b] == -1)
+            continue
+        assert sel[b, 0, c - 1] == pages[-1]                # last page always attended, applied once
+        assert np.array_equal(sel[b, 0, : c - 1], pages[logical[b][0]])  # logical -> physical, once
+        assert np.all(sel[b, 0, c:] == -1)
+        assert pages[-1] not in sel[b, 0, : c - 1]          # the last page is not a candidate
+        s = scores[b][0]
+        if len(s) > c - 1:
+            assert s[logical[b][0]].min() >= np.delete(s, logical[b][0]).max()
+
+
+def test_selection_matches_rule():
+    s = np.array([10.0, 9.0, 5.0, 5.0 + 1e-6, 1.0])
+    assert O.selection_matches([0, 1, 3], s, 3)[0]
+    assert O.selection_matches([0, 1, 2], s, 3)[0]        # tie within 1e-3 relative
+    assert not O.selection_matches([0, 1, 4], s, 3)[0]    # 1.0 is no tie of 5.0
+    assert not O.selection_matches([0, 1], s, 3)[0]
+    assert not O.selection_matches([0, 0, 1], s, 3)[0]
+    assert not O.selection_matches([0, 1, 7], s, 3)[0]
+
+
+# --------------------------------------------------------------------------- attention
+
+
+def _depaged(pb, b, h):
+    pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+    L = int(pb.lengths[b])
+    K = O.bf16_to_f32(pb.kv_cache[pages, 0, :, h]).reshape(-1, D)[:L]
+    V = O.bf16_to_f32(pb.kv_cache[pages, 1, :, h]).reshape(-1, D)[:L]
+    return K.astype(np.float64), V.astype(np.float64)
+
+
+def test_dense_attention_equals_torch_sdpa():
+    pb = P.make_problem(41, [PS * 6 + 5, PS * 2, 9], num_kv_heads=2, group=4)
+    out, lse = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    qf = O.bf16_to_f32(pb.q).astype(np.float64)
+    for b in range(pb.B):
+        for h in range(2):
+            K, V = _depaged(pb, b, h)
+            qt = torch.from_numpy(qf[b, 4 * h : 4 * h + 4])[None, :, None, :]       # [1, G, 1, D]
+            Kt = torch.from_numpy(K)[None, None].expand(1, 4, -1, -1)
+            Vt = torch.from_numpy(V)[None, None].expand(1, 4, -1, -1)
+            want = torch.nn.functional.scaled_dot_product_attention(qt, Kt, Vt)[0, :, 0].numpy()
+            assert np.allclose(out[b, 4 * h : 4 * h + 4], want, rtol=1e-9, atol=1e-9)
+            logits = qf[b, 4 * h : 4 * h + 4] @ K.T / math.sqrt(D)
+            assert np.allclose(lse[b, 4 * h : 4 * h + 4], logsumexp(logits, axis=1), rtol=1e-12)
+
+
+def test_sparse_with_every_page_selected_equals_dense():
+    pb = P.make_problem(43, [PS * 5 + 2, PS * 3 + 16], num_kv_heads=1, group=4, topk=64)
+    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    a, la = O.sparse_paged_decode(pb.q, pb.kv_cache, sel, cnt, pb.last_page_len)
+    d, ld = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    assert np.allclose(a, d, rtol=1e-10, atol=1e-12) and np.allclose(la, ld, rtol=1e-12)
+
+
+def test_attention_closed_forms():
+    rng = np.random.default_rng(47)
+    pb = P.make_problem(47, [1, PS * 4 + 3], num_kv_heads=1, group=4, topk=2)
+    O.append_paged_kv(pb.k, pb.v, pb.kv_cache, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    out, lse = O.sparse_paged_decode(pb.q, pb.kv_cache, sel, cnt, pb.last_page_len)
+    # one token: softmax over one logit is 1 -> out is that token's value, lse its logit
+    v0 = O.bf16_to_f32(pb.v[0, 0]).astype(np.float64)
+    assert np.allclose(out[0], np.broadcast_to(v0, (4, D)), rtol=0, atol=1e-12)
+    logit = O.bf16_to_f32(pb.q[0]).astype(np.float64) @ O.bf16_to_f32(pb.k[0, 0]).astype(np.float64) / math.sqrt(D)
+    assert np.allclose(lse[0], logit, rtol=1e-12)
+    # constant V: out is that constant whatever the weights
+    cv = P.randn_bf16(rng, (D,))
+    kv2 = pb.kv_cache.copy()
+    kv2[:, 1] = cv
+    out2, _ = O.sparse_paged_decode(pb.q, kv2, sel, cnt, pb.last_page_len)
+    assert np.allclose(out2, O.bf16_to_f32(cv).astype(np.float64), rtol=0, atol=1e-12)
+    # q = 0: uniform weights -> mean of the attended values (2 full pages + 3 tokens of the last)
+    q0 = np.zeros_like(pb.q)
+    out3, lse3 = O.sparse_paged_decode(q0, pb.kv_cache, sel, cnt, pb.last_page_len)
+    pages = sel[1, 0, : cnt[1, 0]]
+    V = O.bf16_to_f32(pb.kv_cache[pages, 1, :, 0]).reshape(-1, D)[: 2 * PS + 3].astype(np.float64)
+    assert np.allclose(out3[1], V.mean(axis=0), rtol=1e-12, atol=1e-12)
+    assert np.allclose(lse3[1], math.log(2 * PS + 3), rtol=1e-12)
+
+
+def test_attention_permutation_and_split_invariance():
+    pb = P.make_problem(53, [PS * 12 + 9], num_kv_heads=1, group=4, topk=7)
+    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    out, lse = O.sparse_paged_decode(pb.q, pb.kv_cache, sel, cnt, pb.last_page_len)
+    # shuffle the full pages (the final, partial page keeps its place)
+    c = cnt[0, 0]
+    sel2 = sel.copy()
+    sel2[0, 0, : c - 1] = sel[0, 0, : c - 1][::-1]
+    out2, lse2 = O.sparse_paged_decode(pb.q, pb.kv_cache, sel2, cnt, pb.last_page_len)
+    assert np.allclose(out, out2, rtol=1e-12, atol=1e-13) and np.allclose(lse, lse2, rtol=1e-13)
+    # any partition of the page list merged by (out, lse) gives the same answer
+    qf = O.bf16_to_f32(pb.q[0]).astype(np.float64)
+    pages = sel[0, 0, :c]
+    for cuts in ([3], [1, 2, 5], [c - 1]):
+        outs, lses = [], []
+        bounds = [0, *cuts, c]
+        for lo, hi in zip(bounds[:-1], bounds[1:]):
+            ll = pb.last_page_len[0] if hi == c else PS
+            o, l = O.attend_pages(qf, pb.kv_cache, pages[lo:hi], 0, ll, 1 / math.sqrt(D))
+            outs.append(o)
+            lses.append(l)
+        # an empty part must be neutral
+        outs.append(np.zeros_like(outs[0]))
+        lses.append(np.full_like(lses[0], -np.inf))
+        mo, ml = O.merge_partials(outs, lses)
+        assert np.allclose(mo, out[0], rtol=1e-12, atol=1e-13) and np.allclose(ml, lse[0], rtol=1e-13)
+
+
+def test_decode_step_equals_masked_dense_formulation():
+    """LiteSys expresses block sparsity as a -inf mask on full-context logits
+    (sparsity_utils.py:39-45) followed by softmax and P.V; the gather form must
+    give the same numbers."""
+    pb = P.make_problem(59, [PS * 10 + 5, PS * 7 + 16], num_kv_heads=2, group=2, topk=3)
+    res = O.decode_step(pb.q, pb.k, pb.v, pb.kv_cache, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
+    qf = O.bf16_to_f32(pb.q).astype(np.float64)
+    for b in range(pb.B):
+        L = int(pb.lengths[b])
+        n_pages = (L + PS - 1) // PS
+        for h in range(2):
+            K, V = _depaged(pb, b, h)
+            keep = np.zeros(n_pages * PS, dtype=bool)
+            for p in res["sel_logical"][b][h]:
+                keep[p * PS : (p + 1) * PS] = True
+            keep[(n_pages - 1) * PS :] = True
+            keep = keep[:L]
+            logits = qf[b, 2 * h : 2 * h + 2] @ K.T / math.sqrt(D)
+            logits[:, ~keep] = -np.inf
+            w = np.exp(logits - logits.max(axis=1, keepdims=True))
+            w /= w.sum(axis=1, keepdims=True)
+            assert np.allclose(res["out"][b, 2 * h : 2 * h + 2], w @ V, rtol=1e-10, atol=1e-12)
+
+
+# --------------------------------------------------------------------------- torch path
+
+
+def test_torch_path_agrees_with_oracle():
+    B, n_pages, topk = 4, 40, 8
+    pb = P.make_problem(61, [PS * (n_pages - 1) + 6] * B, num_kv_heads=1, group=4, topk=topk)
+    kv_t = P.to_torch(pb.kv_cache.copy())
+    table = torch.from_numpy(pb.page_indices.astype(np.int64)).reshape(B, n_pages)
+    out_t, idx_t = torch_path.blocktopk_decode_step(
+        P.to_torch(pb.q), P.to_torch(pb.k), P.to_torch(pb.v), kv_t, P.to_torch(pb.kbar[:, : n_pages - 1, 0]),
+        table, torch.from_numpy(pb.last_page_len.astype(np.int64)), topk)
+    res = O.decode_step(pb.q, pb.k, pb.v, pb.kv_cache, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, topk)
+    assert np.array_equal(P.from_torch(kv_t), pb.kv_cache)  # same append
+    for b in range(B):
+        ok, msg = O.selection_matches(idx_t[b].numpy(), res["scores"][b][0], topk)
+        assert ok, msg
+    got = out_t.float().numpy().astype(np.float64)
+    assert np.allclose(got, res["out"], rtol=2e-2, atol=2e-2)
+    dense_t = torch_path.dense_decode_step(P.to_torch(pb.q), P.to_torch(pb.k), P.to_torch(pb.v), kv_t, table,
+                                           torch.from_numpy(pb.last_page_len.astype(np.int64)))
+    dense_o, _ = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    assert np.allclose(dense_t.float().numpy(), dense_o, rtol=2e-2, atol=2e-2)
