@@ -205,11 +205,20 @@ def _decode_common(q, kv_cache, last_page_len, out, lse, workspace):
         _require(lse, "lse", torch.float32, 2, dev)
         if tuple(lse.shape) != (batch, num_q_heads):
             raise ValueError(f"lse must be [{batch}, {num_q_heads}], got {tuple(lse.shape)}")
-    ws_bytes = 0
     if workspace is not None:
         _require(workspace, "workspace", torch.uint8, 1, dev)
-        ws_bytes = workspace.numel()
-    return dev, batch, num_q_heads, num_kv_heads, head_dim, page_size, num_pages, out, ws_bytes
+    return dev, batch, num_q_heads, num_kv_heads, head_dim, page_size, num_pages, out
+
+
+def _workspace(workspace, dev, batch, hq, hkv, max_pages, num_splits):
+    """The caller's workspace, or a fresh one when none was given and the split
+    count needs it (like ``out``: allocated here only as a convenience; loops
+    that must not allocate pass both)."""
+    if workspace is None:
+        need = decode_workspace_bytes(batch, hq, hkv, max_pages, num_splits)
+        if need:
+            workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    return workspace, (0 if workspace is None else workspace.numel())
 
 
 def sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, out=None, lse=None, workspace=None,
@@ -217,13 +226,14 @@ def sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, out=No
     """Attention of one query token per sequence over the listed pages; stands
     in for ``mylib::decode`` (benchmark/blocktopk_decoder.py:171-184,223-225).
     Returns ``out`` [batch, num_q_heads, head_dim] bf16."""
-    dev, batch, hq, hkv, d, ps, num_pages, out, ws_bytes = _decode_common(q, kv_cache, last_page_len, out, lse, workspace)
+    dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, workspace)
     _require(sel_pages, "sel_pages", torch.int32, 3, dev)
     _require(sel_count, "sel_count", torch.int32, 2, dev)
     if sel_pages.shape[:2] != (batch, hkv) or tuple(sel_count.shape) != (batch, hkv):
         raise ValueError(
             f"sel_pages/sel_count must be [{batch}, {hkv}, stride] / [{batch}, {hkv}], got {tuple(sel_pages.shape)} / {tuple(sel_count.shape)}"
         )
+    workspace, ws_bytes = _workspace(workspace, dev, batch, hq, hkv, sel_pages.shape[2], int(num_splits))
     lib = _lib.load()
     with torch.cuda.device(dev):
         _lib.check(
@@ -240,8 +250,9 @@ def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, ma
                        workspace=None, sm_scale: float = 0.0, num_splits: int = 0):
     """Attention over every page of each sequence; the dense baseline
     (benchmark/dense_decoder.py:149-170,211-219)."""
-    dev, batch, hq, hkv, d, ps, num_pages, out, ws_bytes = _decode_common(q, kv_cache, last_page_len, out, lse, workspace)
+    dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, workspace)
     _table(page_indices, page_indptr, None, batch, dev)
+    workspace, ws_bytes = _workspace(workspace, dev, batch, hq, hkv, int(max_pages_per_seq), int(num_splits))
     lib = _lib.load()
     with torch.cuda.device(dev):
         _lib.check(
