@@ -1,0 +1,255 @@
+#!/usr/bin/env python3
+"""Throughput of one block top-k sparse decode step on one MI355X.
+
+A "step" is what benchmark/blocktopk_decoder.py:209-225 does for one batch:
+append the new token's K/V, score every page against the group-mean query,
+take the top-k pages plus the last page, attend over them.  The harness mirrors
+benchmark/blocktopk.py:47-61: W untimed warm-up steps, then K timed steps
+between device synchronisations, throughput = K * batch / elapsed (tokens/s for
+one layer on one GPU's share of the heads).  Sequence lengths stay fixed across
+steps, as in the reference harness whose metadata never changes.
+
+Prints ONE JSON line.  ``value`` is decode tokens/s per layer with every input
+already resident in HBM.  ``roofline`` describes the dominant kernel (the sparse
+paged attention), ``step_hbm`` the whole step against the algorithmic-bytes
+model, ``cpu_baseline`` the torch-CPU restatement of the reference path timed on
+this machine's host cores, ``dense_baseline`` the dense paged decode on the same
+tensors.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+PS, D = 16, 128
+
+WORKLOADS = {
+    # name: (batch, ctx, H_kv, group, topk, description)
+    "qwen3-8b-share": (4096, 32768, 1, 4, 128, "Qwen3-8B one-GPU share (TP=8): 1 KV head, 4 Q heads"),
+    "qwen3-32b-share": (1024, 32768, 1, 8, 256, "Qwen3-32B one-GPU share: 1 KV head, 8 Q heads"),
+    "tiny": (8, 4096, 1, 4, 64, "CPU-runnable tiny case"),
+}
+
+
+def algorithmic_bytes(B, Hkv, G, n_cand, k_eff, last_len):
+    """Bytes per step that the algorithm has to move (bf16 K/V, int32 indices)."""
+    Hq = Hkv * G
+    kbar = Hkv * n_cand * D * 2
+    kv_sel = Hkv * (k_eff * PS + last_len) * 2 * D * 2
+    append = Hkv * 2 * D * 2
+    qo = 2 * Hq * D * 2
+    idx = 2 * Hkv * k_eff * 4
+    per_seq = kbar + kv_sel + append + qo + idx
+    attn_per_seq = kv_sel + qo + Hkv * (k_eff + 1) * 4
+    score_per_seq = kbar + Hq * D * 2 + Hkv * (k_eff + 1) * 4
+    return dict(step=B * per_seq, attention=B * attn_per_seq, score_select=B * score_per_seq,
+                append=B * (append + Hkv * 2 * D * 2), per_seq=per_seq)
+
+
+def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2):
+    """Paged cache in the reference layout (page id = p*B + b, max_len = ctx+512),
+    K ~ N(0,1) + per-page mean offset N(0,0.5), V ~ N(0,1); kbar = true page means."""
+    n_full = ctx // PS
+    max_pages = (ctx + 512) // PS
+    num_pages = max_pages * B
+    gen = torch.Generator(device=device).manual_seed(seed)
+    kv = torch.empty(num_pages, 2, PS, Hkv, D, dtype=torch.bfloat16, device=device)
+    chunk = max(1, (1 << 28) // (2 * PS * Hkv * D))
+    for s in range(0, num_pages, chunk):
+        e = min(num_pages, s + chunk)
+        x = torch.randn(e - s, 2, PS, Hkv, D, generator=gen, device=device, dtype=torch.float32)
+        mu = torch.randn(e - s, 1, 1, Hkv, 1, generator=gen, device=device, dtype=torch.float32) * 0.5
+        x[:, 0:1] += mu
+        kv[s:e] = x.to(torch.bfloat16)
+        del x, mu
+    table = torch.arange(n_full + 1, dtype=torch.int32, device=device) * B + torch.arange(B, dtype=torch.int32, device=device)[:, None]
+    st = dict(
+        kv=kv,
+        indices=table.reshape(-1).contiguous(),
+        indptr=(torch.arange(B + 1, dtype=torch.int32, device=device) * (n_full + 1)).contiguous(),
+        last=torch.ones(B, dtype=torch.int32, device=device),
+        kbar=torch.zeros(B, max_pages, Hkv, D, dtype=torch.bfloat16, device=device),
+        sel=torch.full((B, Hkv, topk + 1), -1, dtype=torch.int32, device=device),
+        cnt=torch.zeros(B, Hkv, dtype=torch.int32, device=device),
+        q=torch.randn(B, Hkv * G, D, generator=gen, device=device, dtype=torch.float32).to(torch.bfloat16),
+        k=torch.randn(B, Hkv, D, generator=gen, device=device, dtype=torch.float32).to(torch.bfloat16),
+        v=torch.randn(B, Hkv, D, generator=gen, device=device, dtype=torch.float32).to(torch.bfloat16),
+        out=torch.empty(B, Hkv * G, D, dtype=torch.bfloat16, device=device),
+        n_full=n_full, max_pages=max_pages, num_pages=num_pages,
+    )
+    ops.build_kbar(st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
+    ws = ops.decode_workspace_bytes(B, Hkv * G, Hkv, topk + 1)
+    st["ws"] = torch.empty(max(ws, 16), dtype=torch.uint8, device=device)
+    wsd = ops.decode_workspace_bytes(B, Hkv * G, Hkv, n_full + 1)
+    st["ws_dense"] = torch.empty(max(wsd, 16), dtype=torch.uint8, device=device)
+    return st
+
+
+def cpu_baseline(torch, B_cpu, ctx, G, topk, budget_s=20.0):
+    """The reference's torch path (oracle/torch_path.py) on the host cores, on a
+    slice of the workload: B_cpu sequences of the same context length."""
+    from oracle import torch_path
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    n_full = ctx // PS
+    n_pages = n_full + 1
+    g = torch.Generator().manual_seed(5)
+    kv = torch.empty(B_cpu * n_pages, 2, PS, 1, D, dtype=torch.bfloat16)
+    chunk = 1 << 13
+    for s in range(0, kv.shape[0], chunk):
+        e = min(kv.shape[0], s + chunk)
+        kv[s:e] = torch.randn(e - s, 2, PS, 1, D, generator=g).to(torch.bfloat16)
+    table = (torch.arange(n_pages)[None, :] * B_cpu + torch.arange(B_cpu)[:, None]).contiguous()
+    kbar = kv[table[:, :-1], 0, :, 0].float().mean(dim=2).to(torch.bfloat16)  # [B, n_full, D]
+    q = torch.randn(B_cpu, G, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(B_cpu, 1, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(B_cpu, 1, D, generator=g).to(torch.bfloat16)
+    last = torch.ones(B_cpu, dtype=torch.int64)
+    times = []
+    for _ in range(3):
+        torch_path.blocktopk_decode_step(q, k, v, kv, kbar, table, last, topk)
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 10 or (time.perf_counter() < t_end and len(times) < 200):
+        t0 = time.perf_counter()
+        torch_path.blocktopk_decode_step(q, k, v, kv, kbar, table, last, topk)
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
+    return dict(value=B_cpu / med, unit="tokens/s", cores=cores, kind="port",
+                sample=f"torch-CPU restatement of the reference path (oracle/torch_path.py), {B_cpu} of the batch's "
+                       f"sequences at ctx={ctx}, k={topk}, median of {len(times)} steps after 3 warm-ups, "
+                       f"{med * 1e3:.2f} ms/step; tokens/s is linear in batch")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="qwen3-8b-share", choices=sorted(WORKLOADS))
+    ap.add_argument("--batch", type=int, default=0, help="override the workload's batch size")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-dense", action="store_true")
+    ap.add_argument("--cpu-batch", type=int, default=128)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: the path is independent per (sequence, KV head) and is run on "
+              "one GPU's share of the heads; --gpus above 1 is not supported.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from kinetics_amd import _lib, ops
+
+    _lib.load()  # fail loudly if the HIP library is missing
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    device = torch.device("cuda:0")
+    B, ctx, Hkv, G, topk, desc = WORKLOADS[args.workload]
+    if args.batch:
+        B = args.batch
+    t_setup = time.perf_counter()
+    st = build_state(torch, ops, B, ctx, Hkv, G, topk, device)
+    torch.cuda.synchronize()
+    print(f"[bench] {args.workload}: B={B} ctx={ctx} H_kv={Hkv} G={G} topk={topk}, "
+          f"KV {st['kv'].numel() * 2 / 1e9:.1f} GB resident, setup {time.perf_counter() - t_setup:.1f}s", file=sys.stderr)
+
+    def step():
+        ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
+        ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], topk, st["sel"], st["cnt"])
+        ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"], out=st["out"], workspace=st["ws"])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    # -- the timed region: K steps; HIP events on the launch stream bracket each kernel
+    K = args.steps
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(K)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        ev[i][0].record()
+        ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
+        ev[i][1].record()
+        ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], topk, st["sel"], st["cnt"])
+        ev[i][2].record()
+        ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"], out=st["out"], workspace=st["ws"])
+        ev[i][3].record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_step = elapsed / K * 1e3
+    t_append = statistics.fmean(e[0].elapsed_time(e[1]) for e in ev)
+    t_select = statistics.fmean(e[1].elapsed_time(e[2]) for e in ev)
+    t_attn = statistics.fmean(e[2].elapsed_time(e[3]) for e in ev)
+
+    k_eff = min(topk, st["n_full"])
+    ab = algorithmic_bytes(B, Hkv, G, st["n_full"], k_eff, 1)
+    attn_gbs = ab["attention"] / (t_attn * 1e-3) / 1e9
+    step_gbs = ab["step"] / (ms_step * 1e-3) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get(f"{args.workload}:B={B}", {}).get("paged_decode_kernel")
+
+    result = {
+        "metric": "decode tok/s per layer, Qwen3-8B 1-GPU share B=4096 ctx=32K; HBM GB/s % peak",
+        "value": B * K / elapsed,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "description": desc, "batch": B, "ctx": ctx, "num_kv_heads": Hkv,
+                   "num_q_heads": Hkv * G, "head_dim": D, "page_size": PS, "topk_pages": topk,
+                   "page_table": "reference layout p*B+b", "kv_resident_gb": round(st["kv"].numel() * 2 / 1e9, 2)},
+        "roofline": {"bound": "hbm", "kernel": "paged_decode_kernel (sparse gather-attention)",
+                     "achieved": attn_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": attn_gbs / HBM_PEAK_GBS,
+                     "traffic": traffic, "algorithmic_bytes_per_launch": ab["attention"],
+                     "avg_launch_ms": t_attn},
+        "step_hbm": {"algorithmic_bytes_per_step": ab["step"], "bytes_per_seq": ab["per_seq"], "achieved": step_gbs,
+                     "unit": "GB/s", "frac": step_gbs / HBM_PEAK_GBS},
+        "kernels_ms": {"append": t_append, "score_topk": t_select, "sparse_attention": t_attn,
+                       "score_topk_gbs": ab["score_select"] / (t_select * 1e-3) / 1e9},
+    }
+
+    if not args.no_dense:
+        nd = max(3, min(10, K // 10))
+        for _ in range(2):
+            ops.dense_paged_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], st["n_full"] + 1,
+                                   out=st["out"], workspace=st["ws_dense"])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(nd):
+            ops.append_paged_kv(st["k"], st["v"], st["kv"], None, st["indices"], st["indptr"], st["last"])
+            ops.dense_paged_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], st["n_full"] + 1,
+                                   out=st["out"], workspace=st["ws_dense"])
+        torch.cuda.synchronize()
+        td = (time.perf_counter() - t0) / nd
+        dense_bytes = B * (Hkv * ((st["n_full"] * PS + 1) * 2 * D * 2 + 2 * D * 2) + 2 * Hkv * G * D * 2)
+        result["dense_baseline"] = {"value": B / td, "unit": "tokens/s", "ms_per_step": td * 1e3, "steps": nd,
+                                    "achieved_gbs": dense_bytes / td / 1e9, "frac": dense_bytes / td / 1e9 / HBM_PEAK_GBS,
+                                    "sparse_over_dense": (B * K / elapsed) / (B / td)}
+    del st
+    torch.cuda.empty_cache()
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(torch, min(args.cpu_batch, B), ctx, G, topk)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -48,8 +48,73 @@ struct DecodeParams {
 constexpr float kNegInf = -INFINITY;
 constexpr float kLn2 = 0.6931471805599453f;
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Buffer descriptor covering `bytes` bytes from `base` (0 bytes: every load
+// through it returns zeros without touching memory).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+
+// One page for one wave: scores, online softmax update, O += P V.
+// kq: this lane's 4 K chunks in MFMA A layout; vr: its 4 V rows (row 4*kg + r).
 template <int NG>
-__global__ __launch_bounds__(256) void paged_decode_kernel(DecodeParams p) {
+__device__ __forceinline__ void process_page(const uint4 (&ka)[4], const u32x4 (&vr)[4], const bf16x8 (&qB)[NG][4],
+                                             float (&m_run)[NG], float (&l_run)[NG], floatx4 (&O)[NG][8],
+                                             float scale_log2, int valid_tokens, int kg) {
+  floatx4 S[NG];
+#pragma unroll
+  for (int half = 0; half < NG; ++half) S[half] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const bf16x8 a = __builtin_bit_cast(bf16x8, ka[c]);
+#pragma unroll
+    for (int half = 0; half < NG; ++half)
+      S[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qB[half][c], S[half], 0, 0, 0);
+  }
+  float pr[NG][4];
+#pragma unroll
+  for (int half = 0; half < NG; ++half) {
+    float s[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) s[r] = (4 * kg + r < valid_tokens) ? S[half][r] * scale_log2 : kNegInf;
+    const float m_new = fmaxf(m_run[half], fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
+    if (__any(m_new > m_run[half])) {
+      const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
+      const float alpha = fast_exp2(m_run[half] - m_safe);
+      l_run[half] *= alpha;
+      const float a0 = quad_bcast<0>(alpha), a1 = quad_bcast<1>(alpha);
+      const float a2 = quad_bcast<2>(alpha), a3 = quad_bcast<3>(alpha);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        O[half][u][0] *= a0;
+        O[half][u][1] *= a1;
+        O[half][u][2] *= a2;
+        O[half][u][3] *= a3;
+      }
+      m_run[half] = m_new;
+    }
+    const float m_use = (m_run[half] == kNegInf) ? 0.f : m_run[half];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) pr[half][r] = fast_exp2(s[r] - m_use);
+    l_run[half] += (pr[half][0] + pr[half][1]) + (pr[half][2] + pr[half][3]);
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const u32x4 vv = vr[r];
+    const float vf[8] = {bf16_lo(vv.x), bf16_hi(vv.x), bf16_lo(vv.y), bf16_hi(vv.y),
+                         bf16_lo(vv.z), bf16_hi(vv.z), bf16_lo(vv.w), bf16_hi(vv.w)};
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+#pragma unroll
+      for (int half = 0; half < NG; ++half)
+        O[half][u] = __builtin_amdgcn_mfma_f32_4x4x1f32(pr[half][r], vf[u], O[half][u], 0, 0, 0);
+    }
+  }
+}
+
+template <int NG>
+__global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
   // 4 KiB of K staging per wave; reused as the [wave][head][128] merge buffer.
   __shared__ __attribute__((aligned(16))) unsigned char lds[16384];
   __shared__ float sm_m[4][4 * NG];
@@ -62,7 +127,7 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(DecodeParams p) {
   const int b = list / p.num_kv_heads, h = list - b * p.num_kv_heads;
   const int G = p.group;
 
-  const int32_t* pl;
+  const int32_t* __restrict__ pl;
   int n;
   if (p.list_indptr) {
     const int s = p.list_indptr[b];
@@ -88,14 +153,15 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(DecodeParams p) {
       qB[half][c] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(qp + 32 * c));
   }
 
-  const int64_t row_bytes = (int64_t)p.num_kv_heads * kRowBytes;
-  const int64_t page_bytes = 2 * kPageSize * row_bytes;
+  const int row_bytes = p.num_kv_heads * kRowBytes;
+  const int page_bytes = 2 * kPageSize * row_bytes;
+  const int span = page_bytes - h * kRowBytes;  // bytes addressable from this head's first row
   const char* kvb = reinterpret_cast<const char*>(p.kv) + (int64_t)h * kRowBytes;
   int koff[4], voff[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
-    koff[c] = (int)((4 * c + kg) * row_bytes) + c16 * 16;
-    voff[c] = (int)((kPageSize + 4 * kg + c) * row_bytes) + c16 * 16;
+    koff[c] = (4 * c + kg) * row_bytes + c16 * 16;
+    voff[c] = (kPageSize + 4 * kg + c) * row_bytes + c16 * 16;
   }
   unsigned char* kl = lds + w * 4096;
   int lds_w[4], lds_r[4];
@@ -117,110 +183,47 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(DecodeParams p) {
     for (int u = 0; u < 8; ++u) O[half][u] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // Page ids for this wave's next 64 iterations live one per lane.
+  // This wave takes list entries my_first, my_first+4, ...  The loop below is
+  // branch-free: a page past the end (or with an id outside the cache) is read
+  // through an empty buffer descriptor -- zeros, no memory traffic -- and all
+  // of its tokens are masked.
   const int my_first = p0 + w;
   const int iters = (p1 > my_first) ? (p1 - my_first + 3) / 4 : 0;
-  int ids = -1;
-  auto fetch_ids = [&](int it0) {
-    const int idx = my_first + 4 * (it0 + l);
-    ids = (idx < p1) ? pl[idx] : -1;
+  const int n_last = n - 1;
+  auto page_rsrc = [&](int it, int& valid_tokens) {
+    const int idx = my_first + 4 * it;
+    const bool in_list = idx < p1;
+    const int id = pl[in_list ? idx : 0];  // uniform address: a scalar load
+    const bool ok = in_list && id >= 0 && (int64_t)id < p.num_pages;
+    valid_tokens = ok ? (idx == n_last ? last_len : kPageSize) : 0;
+    return make_rsrc(kvb + (int64_t)(ok ? id : 0) * page_bytes, ok ? span : 0);
   };
-  auto page_base = [&](int it) -> const char* {
-    const int id = __builtin_amdgcn_readlane(ids, it & 63);
-    const bool ok = (id >= 0) && ((int64_t)id < p.num_pages);
-    return ok ? kvb + (int64_t)id * page_bytes : nullptr;
+  auto load_page = [&](__amdgpu_buffer_rsrc_t r, u32x4 (&kk)[4], u32x4 (&vv)[4]) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) kk[c] = __builtin_amdgcn_raw_buffer_load_b128(r, koff[c], 0, 0);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) vv[c] = __builtin_amdgcn_raw_buffer_load_b128(r, voff[c], 0, 0);
+  };
+  auto stage_k = [&](const u32x4 (&kk)[4], uint4 (&ka)[4]) {
+    // K: registers -> wave-private LDS (row-major, swizzled) -> MFMA A layout.
+#pragma unroll
+    for (int c = 0; c < 4; ++c) *reinterpret_cast<u32x4*>(kl + lds_w[c]) = kk[c];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) ka[c] = *reinterpret_cast<const uint4*>(kl + lds_r[c]);
   };
 
-  uint4 kr[4], vr[4];
-  const char* cur = nullptr;
-  if (iters > 0) {
-    fetch_ids(0);
-    cur = page_base(0);
-    if (cur) {
-#pragma unroll
-      for (int c = 0; c < 4; ++c) kr[c] = *reinterpret_cast<const uint4*>(cur + koff[c]);
-#pragma unroll
-      for (int c = 0; c < 4; ++c) vr[c] = *reinterpret_cast<const uint4*>(cur + voff[c]);
-    }
-  }
-  for (int it = 0; it < iters; ++it) {
-    // Prefetch the next page while this one is processed.
-    uint4 kn[4], vn[4];
-    const char* nxt = nullptr;
-    if (it + 1 < iters) {
-      if (((it + 1) & 63) == 0) fetch_ids(it + 1);
-      nxt = page_base(it + 1);
-      if (nxt) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) kn[c] = *reinterpret_cast<const uint4*>(nxt + koff[c]);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) vn[c] = *reinterpret_cast<const uint4*>(nxt + voff[c]);
-      }
-    }
-    if (cur) {
-      const bool is_last = (my_first + 4 * it == n - 1);
-      // K: registers -> LDS (row-major, swizzled) -> MFMA A layout.
-#pragma unroll
-      for (int c = 0; c < 4; ++c) *reinterpret_cast<uint4*>(kl + lds_w[c]) = kr[c];
-      floatx4 S[NG];
-#pragma unroll
-      for (int half = 0; half < NG; ++half) S[half] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(kl + lds_r[c]));
-#pragma unroll
-        for (int half = 0; half < NG; ++half)
-          S[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qB[half][c], S[half], 0, 0, 0);
-      }
-      float pr[NG][4];
-#pragma unroll
-      for (int half = 0; half < NG; ++half) {
-        float s[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          s[r] = S[half][r] * p.scale_log2;
-          if (is_last && (4 * kg + r >= last_len)) s[r] = kNegInf;
-        }
-        const float m_new = fmaxf(m_run[half], fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
-        if (__any(m_new > m_run[half])) {
-          const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
-          const float alpha = fast_exp2(m_run[half] - m_safe);
-          l_run[half] *= alpha;
-          const float a0 = quad_bcast<0>(alpha), a1 = quad_bcast<1>(alpha);
-          const float a2 = quad_bcast<2>(alpha), a3 = quad_bcast<3>(alpha);
-#pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            O[half][u][0] *= a0;
-            O[half][u][1] *= a1;
-            O[half][u][2] *= a2;
-            O[half][u][3] *= a3;
-          }
-          m_run[half] = m_new;
-        }
-        const float m_use = (m_run[half] == kNegInf) ? 0.f : m_run[half];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) pr[half][r] = fast_exp2(s[r] - m_use);
-        l_run[half] += (pr[half][0] + pr[half][1]) + (pr[half][2] + pr[half][3]);
-      }
-      // O += P V.
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const uint4 vv = vr[r];
-        const float vf[8] = {bf16_lo(vv.x), bf16_hi(vv.x), bf16_lo(vv.y), bf16_hi(vv.y),
-                             bf16_lo(vv.z), bf16_hi(vv.z), bf16_lo(vv.w), bf16_hi(vv.w)};
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-#pragma unroll
-          for (int half = 0; half < NG; ++half)
-            O[half][u] = __builtin_amdgcn_mfma_f32_4x4x1f32(pr[half][r], vf[u], O[half][u], 0, 0, 0);
-        }
-      }
-    }
-    cur = nxt;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      kr[c] = kn[c];
-      vr[c] = vn[c];
+  if (iters > 0 && n > 0) {
+    u32x4 kA[4], vA[4], kB[4], vB[4];
+    uint4 ka[4];
+    int validA, validB;
+    load_page(page_rsrc(0, validA), kA, vA);
+    for (int it = 0; it < iters; it += 2) {
+      load_page(page_rsrc(it + 1, validB), kB, vB);
+      stage_k(kA, ka);
+      process_page<NG>(ka, vA, qB, m_run, l_run, O, p.scale_log2, validA, kg);
+      load_page(page_rsrc(it + 2, validA), kA, vA);
+      stage_k(kB, ka);
+      process_page<NG>(ka, vB, qB, m_run, l_run, O, p.scale_log2, validB, kg);
     }
   }
 
