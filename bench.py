@@ -141,6 +141,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--cpu-batch", type=int, default=128)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (known bytes) to scale profiler byte counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the path is independent per (sequence, KV head) and is run on "
@@ -226,6 +228,14 @@ def main():
         "kernels_ms": {"append": t_append, "score_topk": t_select, "sparse_attention": t_attn,
                        "score_topk_gbs": ab["score_select"] / (t_select * 1e-3) / 1e9},
     }
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 29, dtype=torch.bfloat16, device=device).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     if not args.no_dense:
         nd = max(3, min(10, K // 10))
