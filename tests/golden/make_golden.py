@@ -1,0 +1,55 @@
+#!/usr/bin/env python3
+"""Writes the golden fixtures in this directory: small seeded decode problems
+(inputs) and the results the oracle gives for them (expected outputs).
+
+The reference repository holds no tests, golden vectors or fixtures for this
+path, and its implementation cannot run here (it imports flashinfer), so these
+vectors come from ``oracle/blocktopk_oracle.py``, which tests/test_oracle.py
+pins against library routines and closed forms.  They freeze the oracle's
+behaviour (a later change to it shows up as a diff) and give the HIP path a
+fixed target that does not depend on numpy's random streams.
+
+Run from the repository root:  python tests/golden/make_golden.py
+"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+
+from oracle import blocktopk_oracle as O  # noqa: E402
+from tests import problems as P  # noqa: E402
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+PS = P.PAGE_SIZE
+
+CASES = {
+    # name: (seed, lengths, num_kv_heads, group, topk, table, all_equal_kbar)
+    "basic": (1001, [PS * 5 + 3, PS * 2, 7], 1, 4, 2, "random", False),
+    "hkv2_fills_page": (1002, [PS * 4 + 16, PS * 3 + 1], 2, 2, 2, "random", False),
+    "ties": (1003, [PS * 8 + 2], 1, 4, 3, "random", True),
+}
+
+
+def make(name):
+    seed, lengths, hkv, group, topk, table, equal = CASES[name]
+    pb = P.make_problem(seed, lengths, num_kv_heads=hkv, group=group, topk=topk, table=table, extra_pages=1, kbar_slack=1)
+    if equal:
+        pb.kbar[:] = pb.kbar[0, 0, 0]
+    inputs = dict(q=pb.q, k=pb.k, v=pb.v, kv_cache=pb.kv_cache.copy(), kbar=pb.kbar.copy(),
+                  page_indices=pb.page_indices, page_indptr=pb.page_indptr, last_page_len=pb.last_page_len,
+                  topk=np.int32(topk))
+    res = O.decode_step(pb.q, pb.k, pb.v, pb.kv_cache, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, topk)
+    dense, dense_lse = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    expected = dict(exp_kv_cache=pb.kv_cache, exp_kbar=pb.kbar, exp_sel_pages=res["sel_pages"],
+                    exp_sel_count=res["sel_count"], exp_out=res["out"], exp_lse=res["lse"], exp_dense_out=dense,
+                    exp_dense_lse=dense_lse)
+    np.savez_compressed(os.path.join(HERE, f"{name}.npz"), **inputs, **expected)
+
+
+if __name__ == "__main__":
+    for n in CASES:
+        make(n)
+        print("wrote", n, os.path.getsize(os.path.join(HERE, f"{n}.npz")), "bytes")
