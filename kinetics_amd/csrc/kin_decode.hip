@@ -200,9 +200,9 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
   };
   auto load_page = [&](__amdgpu_buffer_rsrc_t r, u32x4 (&kk)[4], u32x4 (&vv)[4]) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) kk[c] = __builtin_amdgcn_raw_buffer_load_b128(r, koff[c], 0, 0);
+    for (int c = 0; c < 4; ++c) kk[c] = __builtin_amdgcn_raw_buffer_load_b128(r, koff[c], 0, kStreamLoad);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) vv[c] = __builtin_amdgcn_raw_buffer_load_b128(r, voff[c], 0, 0);
+    for (int c = 0; c < 4; ++c) vv[c] = __builtin_amdgcn_raw_buffer_load_b128(r, voff[c], 0, kStreamLoad);
   };
   auto stage_k = [&](const u32x4 (&kk)[4], uint4 (&ka)[4]) {
     // K: registers -> wave-private LDS (row-major, swizzled) -> MFMA A layout.

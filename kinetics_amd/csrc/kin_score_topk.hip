@@ -6,9 +6,10 @@
 //            query, DPP reduction inside each 16-lane row; scores stay in LDS
 //            as order-preserving 32-bit keys (never written to HBM);
 //   phase 2  4-pass 8-bit radix select in LDS for the k-th largest key;
-//   phase 3  gather the winners (ties at the threshold by lowest index),
-//            bitonic sort them (score descending, index ascending) in LDS,
-//            translate logical -> physical page ids and append the last page.
+//   phase 3  gather the winners (ties at the threshold by lowest index), order
+//            them (score descending, index ascending) in LDS -- by counting for
+//            k <= 512, by bitonic sort above -- translate logical -> physical
+//            page ids and append the last page.
 // The kernel is HBM-bound on phase 1: n_cand * 256 B per workgroup.
 #include "kin_common.h"
 
@@ -34,8 +35,11 @@ __device__ __forceinline__ uint32_t order_key(float f) {
   return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
 }
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
 constexpr int kThreads = 256;
-constexpr int kUnroll = 8;  // independent 16-byte loads in flight per lane
+constexpr int kUnroll = 4;  // independent 16-byte loads in flight per lane
+constexpr int kRankSortMax = 512;  // up to here winners are ordered by counting, above by bitonic sort
 
 // Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap]
 __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p) {
@@ -83,25 +87,34 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
 #pragma unroll
     for (int u = 0; u < 8; ++u) qm[u] *= inv;
   }
-  const int64_t row_stride = (int64_t)p.num_kv_heads * kHeadDim;  // elements between logical pages
-  const uint16_t* kb = p.kbar + ((int64_t)b * p.kbar_pages * p.num_kv_heads + h) * kHeadDim + 8 * c16;
+  // The candidates of (b, h) are rows of 256 B at a fixed stride.  They are read
+  // through a buffer descriptor that ends after the last candidate, so loads past
+  // the end return zeros without touching memory and the loop needs no branches:
+  // each lane keeps kUnroll 16-byte loads in flight, re-issuing slot j for the
+  // next pass as soon as it has consumed it.
+  const int row_stride_b = p.num_kv_heads * kRowBytes;  // bytes between logical pages
+  const char* kb = reinterpret_cast<const char*>(p.kbar) +
+                   ((int64_t)b * p.kbar_pages * p.num_kv_heads + h) * kRowBytes;
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(kb), 0, n_cand > 0 ? (n_cand - 1) * row_stride_b + kRowBytes : 0, 0x00020000);
   float* sc_out = p.scores_out ? p.scores_out + (int64_t)item * p.kbar_pages : nullptr;
-  const int sub = tid >> 4;  // 0..15: which of the 16 rows of a pass this lane helps with
+  const int sub = tid >> 4;  // 0..15: which of the 16 rows of a slot this lane helps with
+  const int lane_off = sub * row_stride_b + c16 * 16;
+  u32x4 w[kUnroll];
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j)
+    w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + j * 16 * row_stride_b, 0, kStreamLoad);
   for (int base = 0; base < n_cand; base += 16 * kUnroll) {
-    uint4 w[kUnroll];
+    const int next_off = (base + 16 * kUnroll) * row_stride_b;
 #pragma unroll
     for (int j = 0; j < kUnroll; ++j) {
-      const int row = base + j * 16 + sub;
-      w[j] = (row < n_cand) ? *reinterpret_cast<const uint4*>(kb + (int64_t)row * row_stride)
-                            : make_uint4(0, 0, 0, 0);
-    }
-#pragma unroll
-    for (int j = 0; j < kUnroll; ++j) {
+      const u32x4 x = w[j];
+      w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + j * 16 * row_stride_b, next_off, kStreamLoad);
       float acc = 0.f;
-      acc = fmaf(qm[0], bf16_lo(w[j].x), acc); acc = fmaf(qm[1], bf16_hi(w[j].x), acc);
-      acc = fmaf(qm[2], bf16_lo(w[j].y), acc); acc = fmaf(qm[3], bf16_hi(w[j].y), acc);
-      acc = fmaf(qm[4], bf16_lo(w[j].z), acc); acc = fmaf(qm[5], bf16_hi(w[j].z), acc);
-      acc = fmaf(qm[6], bf16_lo(w[j].w), acc); acc = fmaf(qm[7], bf16_hi(w[j].w), acc);
+      acc = fmaf(qm[0], bf16_lo(x.x), acc); acc = fmaf(qm[1], bf16_hi(x.x), acc);
+      acc = fmaf(qm[2], bf16_lo(x.y), acc); acc = fmaf(qm[3], bf16_hi(x.y), acc);
+      acc = fmaf(qm[4], bf16_lo(x.z), acc); acc = fmaf(qm[5], bf16_hi(x.z), acc);
+      acc = fmaf(qm[6], bf16_lo(x.w), acc); acc = fmaf(qm[7], bf16_hi(x.w), acc);
       acc = row16_sum(acc);
       const int row = base + j * 16 + sub;
       if (c16 == 0 && row < n_cand) {
@@ -124,38 +137,46 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
         if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
       }
       __syncthreads();
-      // Thread t owns bin 255-t, so an inclusive scan over t counts keys in
-      // bins >= 255-t.  The bin where the scan first reaches `remaining` holds
-      // the threshold digit.
-      const uint32_t mine = hist[255 - tid];
-      uint32_t incl = mine;
+      if (wave == 0) {
+        // Lane j owns bins 255-4j .. 252-4j (highest first); an inclusive scan
+        // over lanes counts the keys in all bins at or above the lane's lowest.
+        // The bin where the running count first reaches `remaining` holds the
+        // threshold digit.
+        const int top = 255 - 4 * lane;
+        const uint32_t c0 = hist[top], c1 = hist[top - 1], c2 = hist[top - 2], c3 = hist[top - 3];
+        const uint32_t mine = c0 + c1 + c2 + c3;
+        uint32_t incl = mine;
 #pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const uint32_t up = __shfl_up(incl, off);
-        if (lane >= off) incl += up;
-      }
-      if (lane == 63) wave_tot[wave] = incl;
-      __syncthreads();
-      uint32_t before = 0;
-      for (int wv = 0; wv < wave; ++wv) before += wave_tot[wv];
-      incl += before;
-      const uint32_t excl = incl - mine;
-      if (excl < remaining && remaining <= incl) {
-        sh_bin = 255u - (uint32_t)tid;
-        sh_remaining = remaining - excl;
+        for (int off = 1; off < 64; off <<= 1) {
+          const uint32_t up = __shfl_up(incl, off);
+          if (lane >= off) incl += up;
+        }
+        uint32_t run = incl - mine;  // keys in bins above this lane's
+        if (run < remaining && remaining <= incl) {
+          int bin = top;
+          uint32_t c = c0;
+          if (run + c < remaining) { run += c; bin = top - 1; c = c1; }
+          if (run + c < remaining) { run += c; bin = top - 2; c = c2; }
+          if (run + c < remaining) { run += c; bin = top - 3; }
+          sh_bin = (uint32_t)bin;
+          sh_remaining = remaining - run;
+        }
       }
       __syncthreads();
       prefix |= sh_bin << shift;
       mask |= 255u << shift;
       remaining = sh_remaining;
-      __syncthreads();
+      // The two barriers at the top of the next pass order these reads before
+      // the next write of sh_bin / sh_remaining.
     }
   }
   const bool take_all = (k_eff >= n_cand);
   const uint32_t thr = prefix;
 
   // ---- phase 3: gather, sort, translate --------------------------------------
-  for (int i = tid; i < p.sort_cap; i += kThreads) sortbuf[i] = 0ull;
+  const bool rank_sort = (k_eff <= kRankSortMax);
+  if (!rank_sort)
+    for (int i = tid; i < p.sort_cap; i += kThreads) sortbuf[i] = 0ull;
   if (tid == 0) sh_count = 0;
   __syncthreads();
   if (k_eff > 0) {
@@ -197,8 +218,26 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
     }
   }
   __syncthreads();
-  // Bitonic sort, descending, over sort_cap (power of two) 64-bit entries; the
-  // zero padding sinks to the end.
+  const int32_t* table = p.page_indices + ps;
+  if (rank_sort) {
+    // Small k: every winner counts the winners that beat it (entries are
+    // distinct, so the counts are a permutation) and writes itself to that slot.
+    // All lanes read the same LDS word per step: a broadcast, no conflicts.
+    for (int i = tid; i < k_eff; i += kThreads) {
+      const unsigned long long mine = sortbuf[i];
+      int rank = 0;
+#pragma unroll 8
+      for (int j = 0; j < k_eff; ++j) rank += (sortbuf[j] > mine) ? 1 : 0;
+      const uint32_t logical = 0xffffffffu - (uint32_t)(mine & 0xffffffffull);
+      sel[rank] = table[logical];
+      if (p.sel_logical) p.sel_logical[(int64_t)item * p.topk + rank] = (int32_t)logical;
+    }
+    for (int i = k_eff + tid; i < p.sel_stride; i += kThreads) sel[i] = (i == k_eff) ? table[n_pages - 1] : -1;
+    if (tid == 0) p.sel_count[item] = k_eff + 1;
+    return;
+  }
+  // Large k: bitonic sort, descending, over sort_cap (power of two) 64-bit
+  // entries; the zero padding sinks to the end.
   for (int size = 2; size <= p.sort_cap; size <<= 1) {
     for (int stride = size >> 1; stride > 0; stride >>= 1) {
       for (int i = tid; i < (p.sort_cap >> 1); i += kThreads) {
@@ -214,7 +253,6 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
       __syncthreads();
     }
   }
-  const int32_t* table = p.page_indices + ps;
   for (int i = tid; i < p.sel_stride; i += kThreads) {
     int32_t out = -1;
     if (i < k_eff) {

@@ -167,7 +167,7 @@ def test_score_topk_ties_take_lowest_index(ops):
 
 def test_score_topk_many_candidates(ops):
     # 12000 candidate pages (192k tokens): dynamic LDS above the default allowance
-    pb = P.make_problem(330, [PS * 12000 + 5, PS * 700 + 1], topk=512, kbar_slack=3)
+    pb = P.make_problem(330, [PS * 12000 + 5, PS * 700 + 1, PS * 650 + 1], topk=700, kbar_slack=3)  # k > 512: bitonic path
     g = Gpu(pb)
     check_selection(pb, *run_select(ops, g))
 
