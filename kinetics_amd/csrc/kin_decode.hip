@@ -45,6 +45,10 @@ struct DecodeParams {
   float scale_log2;  // sm_scale * log2(e)
 };
 
+// s_waitcnt immediate for "vmcnt <= 4, no wait on expcnt / lgkmcnt" (gfx9 encoding:
+// vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]).
+constexpr int kWaitVm4 = 4 | (7 << 4) | (15 << 8);
+
 constexpr float kNegInf = -INFINITY;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -56,12 +60,13 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, in
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
 
-// One page for one wave: scores, online softmax update, O += P V.
-// kq: this lane's 4 K chunks in MFMA A layout; vr: its 4 V rows (row 4*kg + r).
+// One page for one wave, first half: scores and the online softmax update.
+// ka: this lane's 4 K chunks in MFMA A layout.  Leaves the probabilities of
+// this lane's 4 tokens in pr.
 template <int NG>
-__device__ __forceinline__ void process_page(const uint4 (&ka)[4], const u32x4 (&vr)[4], const bf16x8 (&qB)[NG][4],
-                                             float (&m_run)[NG], float (&l_run)[NG], floatx4 (&O)[NG][8],
-                                             float scale_log2, int valid_tokens, int kg) {
+__device__ __forceinline__ void page_scores(const uint4 (&ka)[4], const bf16x8 (&qB)[NG][4], float (&m_run)[NG],
+                                            float (&l_run)[NG], floatx4 (&O)[NG][8], float (&pr)[NG][4],
+                                            float scale_log2, int valid_tokens, int kg) {
   floatx4 S[NG];
 #pragma unroll
   for (int half = 0; half < NG; ++half) S[half] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -72,7 +77,6 @@ __device__ __forceinline__ void process_page(const uint4 (&ka)[4], const u32x4 (
     for (int half = 0; half < NG; ++half)
       S[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qB[half][c], S[half], 0, 0, 0);
   }
-  float pr[NG][4];
 #pragma unroll
   for (int half = 0; half < NG; ++half) {
     float s[4];
@@ -99,6 +103,11 @@ __device__ __forceinline__ void process_page(const uint4 (&ka)[4], const u32x4 (
     for (int r = 0; r < 4; ++r) pr[half][r] = fast_exp2(s[r] - m_use);
     l_run[half] += (pr[half][0] + pr[half][1]) + (pr[half][2] + pr[half][3]);
   }
+}
+
+// Second half: O += P V.  vr: this lane's 4 V rows (row 4*kg + r).
+template <int NG>
+__device__ __forceinline__ void page_pv(const u32x4 (&vr)[4], const float (&pr)[NG][4], floatx4 (&O)[NG][8]) {
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const u32x4 vv = vr[r];
@@ -115,8 +124,8 @@ __device__ __forceinline__ void process_page(const uint4 (&ka)[4], const u32x4 (
 
 template <int NG>
 __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
-  // 4 KiB of K staging per wave; reused as the [wave][head][128] merge buffer.
-  __shared__ __attribute__((aligned(16))) unsigned char lds[16384];
+  // 2 x 4 KiB of K staging per wave; reused as the [wave][head][128] merge buffer.
+  __shared__ __attribute__((aligned(16))) unsigned char lds[32768];
   __shared__ float sm_m[4][4 * NG];
   __shared__ float sm_l[4][4 * NG];
 
@@ -157,18 +166,19 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
   const int page_bytes = 2 * kPageSize * row_bytes;
   const int span = page_bytes - h * kRowBytes;  // bytes addressable from this head's first row
   const char* kvb = reinterpret_cast<const char*>(p.kv) + (int64_t)h * kRowBytes;
-  int koff[4], voff[4];
+  int voff[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) voff[c] = (kPageSize + 4 * kg + c) * row_bytes + c16 * 16;
+  // K staging: two 4 KiB stages per wave, filled by LDS-direct buffer loads
+  // (no VGPRs while in flight).  Load c brings rows 4c..4c+3: lane (kg, c16)
+  // lands at LDS row 4c+kg, position c16, and fetches the chunk that belongs
+  // there under the XOR swizzle (position p of row R holds chunk p ^ R).
+  unsigned char* kl = lds + w * (2 * 4096);
+  int kdma_off[4], lds_r[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
-    koff[c] = (4 * c + kg) * row_bytes + c16 * 16;
-    voff[c] = (kPageSize + 4 * kg + c) * row_bytes + c16 * 16;
-  }
-  unsigned char* kl = lds + w * 4096;
-  int lds_w[4], lds_r[4];
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    const int row_w = 4 * c + kg;  // row this lane's load c brought
-    lds_w[c] = row_w * 256 + ((c16 ^ row_w) & 15) * 16;
+    const int row = 4 * c + kg;
+    kdma_off[c] = row * row_bytes + ((c16 ^ row) & 15) * 16;
     const int chunk_r = 4 * c + kg;  // chunk of row c16 that MFMA c wants from this lane
     lds_r[c] = c16 * 256 + ((chunk_r ^ c16) & 15) * 16;
   }
@@ -190,42 +200,92 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
   const int my_first = p0 + w;
   const int iters = (p1 > my_first) ? (p1 - my_first + 3) / 4 : 0;
   const int n_last = n - 1;
-  auto page_rsrc = [&](int it, int& valid_tokens) {
+  // Page ids come through scalar loads issued one half-step before they are
+  // needed.  The list is read-only for the whole kernel; the constant address
+  // space makes the uniform load a scalar one (off the vector-memory counter
+  // that the page prefetch relies on).
+  const __attribute__((address_space(4))) int32_t* pl_c =
+      reinterpret_cast<const __attribute__((address_space(4))) int32_t*>(reinterpret_cast<uintptr_t>(pl));
+  auto load_id = [&](int it) -> int {
     const int idx = my_first + 4 * it;
-    const bool in_list = idx < p1;
-    const int id = pl[in_list ? idx : 0];  // uniform address: a scalar load
-    const bool ok = in_list && id >= 0 && (int64_t)id < p.num_pages;
+    return pl_c[idx < p1 ? idx : 0];
+  };
+  auto page_rsrc = [&](int it, int id, int& valid_tokens) {
+    const int idx = my_first + 4 * it;
+    const bool ok = idx < p1 && id >= 0 && (int64_t)id < p.num_pages;
     valid_tokens = ok ? (idx == n_last ? last_len : kPageSize) : 0;
     return make_rsrc(kvb + (int64_t)(ok ? id : 0) * page_bytes, ok ? span : 0);
   };
-  auto load_page = [&](__amdgpu_buffer_rsrc_t r, u32x4 (&kk)[4], u32x4 (&vv)[4]) {
-#pragma unroll
-    for (int c = 0; c < 4; ++c) kk[c] = __builtin_amdgcn_raw_buffer_load_b128(r, koff[c], 0, kStreamLoad);
+  auto issue_v = [&](__amdgpu_buffer_rsrc_t r, u32x4 (&vv)[4]) {
 #pragma unroll
     for (int c = 0; c < 4; ++c) vv[c] = __builtin_amdgcn_raw_buffer_load_b128(r, voff[c], 0, kStreamLoad);
   };
-  auto stage_k = [&](const u32x4 (&kk)[4], uint4 (&ka)[4]) {
-    // K: registers -> wave-private LDS (row-major, swizzled) -> MFMA A layout.
+  auto issue_k = [&](__amdgpu_buffer_rsrc_t r, int stage) {
+    __attribute__((address_space(3))) unsigned char* dst =
+        (__attribute__((address_space(3))) unsigned char*)(kl + stage * 4096);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) *reinterpret_cast<u32x4*>(kl + lds_w[c]) = kk[c];
+    for (int c = 0; c < 4; ++c)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, dst + c * 1024, 16, kdma_off[c], 0, 0, kStreamLoad);
+  };
+  auto read_k = [&](int stage, uint4 (&ka)[4]) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) ka[c] = *reinterpret_cast<const uint4*>(kl + lds_r[c]);
+    for (int c = 0; c < 4; ++c) ka[c] = *reinterpret_cast<const uint4*>(kl + stage * 4096 + lds_r[c]);
   };
 
+  // The compiler does not order LDS reads after LDS-direct loads by itself, so
+  // the wait is explicit: when it executes, exactly the 4 V loads issued just
+  // before it are allowed to be outstanding, which means the K stage about to
+  // be read (and the V registers about to be used) have landed.  The scheduling
+  // fences keep the instruction order this count relies on.
   if (iters > 0 && n > 0) {
-    u32x4 kA[4], vA[4], kB[4], vB[4];
+    u32x4 vA[4], vB[4];
     uint4 ka[4];
+    float pr[NG][4];
     int validA, validB;
-    load_page(page_rsrc(0, validA), kA, vA);
+    {
+      const __amdgpu_buffer_rsrc_t r0 = page_rsrc(0, load_id(0), validA);
+      issue_k(r0, 0);
+      issue_v(r0, vA);
+    }
+    int id_next = load_id(1);
     for (int it = 0; it < iters; it += 2) {
-      load_page(page_rsrc(it + 1, validB), kB, vB);
-      stage_k(kA, ka);
-      process_page<NG>(ka, vA, qB, m_run, l_run, O, p.scale_log2, validA, kg);
-      load_page(page_rsrc(it + 2, validA), kA, vA);
-      stage_k(kB, ka);
-      process_page<NG>(ka, vB, qB, m_run, l_run, O, p.scale_log2, validB, kg);
+      {
+        const __amdgpu_buffer_rsrc_t r1 = page_rsrc(it + 1, id_next, validB);
+        __builtin_amdgcn_sched_barrier(0);
+        issue_v(r1, vB);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(kWaitVm4);
+        __builtin_amdgcn_sched_barrier(0);
+        read_k(0, ka);
+        __builtin_amdgcn_sched_barrier(0);
+        issue_k(r1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        page_scores<NG>(ka, qB, m_run, l_run, O, pr, p.scale_log2, validA, kg);
+        __builtin_amdgcn_sched_barrier(0);
+        id_next = load_id(it + 2);  // lands while the P V products run
+        page_pv<NG>(vA, pr, O);
+      }
+      {
+        const __amdgpu_buffer_rsrc_t r2 = page_rsrc(it + 2, id_next, validA);
+        __builtin_amdgcn_sched_barrier(0);
+        issue_v(r2, vA);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(kWaitVm4);
+        __builtin_amdgcn_sched_barrier(0);
+        read_k(1, ka);
+        __builtin_amdgcn_sched_barrier(0);
+        issue_k(r2, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        page_scores<NG>(ka, qB, m_run, l_run, O, pr, p.scale_log2, validB, kg);
+        __builtin_amdgcn_sched_barrier(0);
+        id_next = load_id(it + 3);
+        page_pv<NG>(vB, pr, O);
+      }
     }
   }
+  // LDS-direct loads that are still in flight (masked tail pages) must land
+  // before the staging area is reused below.
+  __builtin_amdgcn_s_waitcnt(0);
 
   // ---- merge the 4 row groups of the wave (lanes l, l^16, l^32, l^48) --------
   float m_w[NG], l_w[NG];
