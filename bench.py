@@ -187,6 +187,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--cpu-batch", type=int, default=128)
+    ap.add_argument("--three-kernels", action="store_true",
+                    help="time the append / score+select / attention launches separately instead of the fused step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) to scale profiler byte counters")
     args = ap.parse_args()
@@ -211,42 +213,58 @@ def main():
     print(f"[bench] {args.workload}: B={B} ctx={ctx} H_kv={Hkv} G={G} topk={topk}, "
           f"KV {st['kv'].numel() * 2 / 1e9:.1f} GB resident, setup {time.perf_counter() - t_setup:.1f}s", file=sys.stderr)
 
-    def step():
-        ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
-        ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], topk, st["sel"], st["cnt"])
-        ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"], out=st["out"], workspace=st["ws"])
+    fused = not args.three_kernels
 
+    def launches():
+        """The step's kernel launches, in order, as (name, callable)."""
+        if fused:
+            return [("fused_step", lambda: ops.blocktopk_decode_step(
+                st["q"], st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"], topk,
+                out=st["out"]))]
+        return [
+            ("append", lambda: ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"],
+                                                   st["last"])),
+            ("score_topk", lambda: ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], topk,
+                                                        st["sel"], st["cnt"])),
+            ("sparse_attention", lambda: ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"],
+                                                                 out=st["out"], workspace=st["ws"])),
+        ]
+
+    kernels = launches()
     for _ in range(args.warmup):
-        step()
+        for _, fn in kernels:
+            fn()
     torch.cuda.synchronize()
     # -- the timed region: K steps; HIP events on the launch stream bracket each kernel
     K = args.steps
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(K)]
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(kernels) + 1)] for _ in range(K)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(K):
         ev[i][0].record()
-        ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
-        ev[i][1].record()
-        ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], topk, st["sel"], st["cnt"])
-        ev[i][2].record()
-        ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"], out=st["out"], workspace=st["ws"])
-        ev[i][3].record()
+        for j, (_, fn) in enumerate(kernels):
+            fn()
+            ev[i][j + 1].record()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_step = elapsed / K * 1e3
-    t_append = statistics.fmean(e[0].elapsed_time(e[1]) for e in ev)
-    t_select = statistics.fmean(e[1].elapsed_time(e[2]) for e in ev)
-    t_attn = statistics.fmean(e[2].elapsed_time(e[3]) for e in ev)
+    kernel_ms = {name: statistics.fmean(e[j].elapsed_time(e[j + 1]) for e in ev) for j, (name, _) in enumerate(kernels)}
 
     ab = algorithmic_bytes(st["lengths"], Hkv, G, topk)
-    attn_gbs = ab["attention"] / (t_attn * 1e-3) / 1e9
     step_gbs = ab["step"] / (ms_step * 1e-3) / 1e9
+    if fused:
+        dom_name, dom_kernel, dom_bytes, dom_ms = ("blocktopk_step_kernel (append + score + select + attention, fused)",
+                                                   "blocktopk_step_kernel", ab["step"], kernel_ms["fused_step"])
+    else:
+        dom_name, dom_kernel, dom_bytes, dom_ms = ("paged_decode_kernel (sparse gather-attention)",
+                                                   "paged_decode_kernel", ab["attention"], kernel_ms["sparse_attention"])
+        kernel_ms["score_topk_gbs"] = ab["score_select"] / (kernel_ms["score_topk"] * 1e-3) / 1e9
+    dom_gbs = dom_bytes / (dom_ms * 1e-3) / 1e9
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get(f"{args.workload}:B={B}", {}).get("paged_decode_kernel")
+            traffic = json.load(f).get(f"{args.workload}:B={B}", {}).get(dom_kernel)
 
     result = {
         "metric": "decode tok/s per layer, Qwen3-8B 1-GPU share B=4096 ctx=32K; HBM GB/s % peak",
@@ -264,15 +282,15 @@ def main():
         "config": {"workload": args.workload, "description": desc, "batch": B, "ctx": ctx, "num_kv_heads": Hkv,
                    "num_q_heads": Hkv * G, "head_dim": D, "page_size": PS, "topk_pages": topk,
                    "page_table": "ragged, half fragmented" if args.workload in RAGGED else "reference layout p*B+b",
-                   "kv_resident_gb": round(st["kv"].numel() * 2 / 1e9, 2)},
-        "roofline": {"bound": "hbm", "kernel": "paged_decode_kernel (sparse gather-attention)",
-                     "achieved": attn_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": attn_gbs / HBM_PEAK_GBS,
-                     "traffic": traffic, "algorithmic_bytes_per_launch": ab["attention"],
-                     "avg_launch_ms": t_attn},
+                   "kv_resident_gb": round(st["kv"].numel() * 2 / 1e9, 2),
+                   "launches_per_step": len(kernels)},
+        "roofline": {"bound": "hbm", "kernel": dom_name,
+                     "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom_gbs / HBM_PEAK_GBS,
+                     "traffic": traffic, "algorithmic_bytes_per_launch": dom_bytes,
+                     "avg_launch_ms": dom_ms},
         "step_hbm": {"algorithmic_bytes_per_step": ab["step"], "bytes_per_seq": ab["per_seq"], "achieved": step_gbs,
                      "unit": "GB/s", "frac": step_gbs / HBM_PEAK_GBS},
-        "kernels_ms": {"append": t_append, "score_topk": t_select, "sparse_attention": t_attn,
-                       "score_topk_gbs": ab["score_select"] / (t_select * 1e-3) / 1e9},
+        "kernels_ms": kernel_ms,
     }
 
     if args.calibrate_copy:

@@ -189,6 +189,32 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
                            kin_stream_t stream);
 
 /*
+ * The whole decode step in ONE launch -- replaces lines 209-225 of the
+ * reference layer's forward (ref: benchmark/blocktopk_decoder.py:209-225):
+ * append (kin_append_paged_kv), scoring + selection (kin_block_score_topk) and
+ * attention over the selected pages (kin_sparse_paged_decode), with the same
+ * arithmetic, results and argument meaning as those three calls in sequence.
+ * One workgroup per (sequence, KV head) runs all phases, so the page list never
+ * leaves the chip and phases of different sequences overlap.
+ *
+ * k and v may both be NULL (no append).  sel_pages / sel_count are optional
+ * outputs (both NULL, or both given with 1 <= topk < sel_stride); lse is
+ * optional.  Needs no workspace.  Intended for batch * num_kv_heads large
+ * enough to fill the GPU (>= ~1000 lists); for small batches the three-call
+ * path with split-K is faster.
+ */
+int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
+                              kin_bf16_t* kv_cache, kin_bf16_t* kbar,
+                              const int32_t* page_indices, const int32_t* page_indptr,
+                              const int32_t* last_page_len, int topk,
+                              int32_t* sel_pages, int32_t* sel_count,
+                              kin_bf16_t* out, float* lse,
+                              int batch, int num_q_heads, int num_kv_heads,
+                              int head_dim, int page_size, int64_t num_pages,
+                              int kbar_pages, int sel_stride, float sm_scale,
+                              kin_stream_t stream);
+
+/*
  * Debugging aid, SYNCHRONOUS (waits for the stream): verifies on the device
  * that page_indptr is non-decreasing from 0 and never exceeds nnz (the length
  * of page_indices), every page id lies in [0, num_pages), and every

@@ -47,6 +47,11 @@ SIGNATURES = {
         c_int,
         [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int64, c_int, c_float, c_int, _P],
     ),
+    "kin_blocktopk_decode_step": (
+        c_int,
+        [_P, _P, _P, _P, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int64, c_int, c_int,
+         c_float, _P],
+    ),
     "kin_check_page_table": (c_int, [_P, _P, _P, c_int, c_int, c_int64, c_int64, _P, _P]),
 }
 

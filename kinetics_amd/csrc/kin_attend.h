@@ -1,0 +1,336 @@
+// Device-side building block: attention of one decode token over a list of
+// KV pages, for one (sequence, KV head, split) handled by one 256-thread
+// workgroup.  Shared by the stand-alone paged decode kernel and the fused
+// decode-step kernel.
+//
+// Work decomposition: the workgroup's 4 waves take the list's pages round-robin,
+// one 8 KiB page (16 keys + 16 values of 128 bf16) per wave per iteration, and
+// keep private online-softmax state that is merged once at the end.
+//
+// Per page and wave (lane l, row group kg = l/16, 16-byte column chunk c = l%16):
+//   K  4 x 16-byte LDS-direct buffer loads, each instruction covering 4 whole
+//      256-byte rows, into a wave-private, XOR-swizzled staging area (two
+//      stages); read back in the MFMA operand layout "row = l%16".
+//   S  = K q^T with 4 x v_mfma_f32_16x16x32_bf16; the 16 output columns hold
+//      the (<=4) query heads of the group replicated 4x, so lane l ends up with
+//      S[g = l%4][t = 4*kg + r] (r = 0..3) and no cross-lane traffic is needed.
+//   softmax state (m, l) is kept per (row group, head): 4 independent partial
+//      softmaxes per wave, so the running max needs no cross-lane reduction.
+//   V  4 x 16-byte buffer loads straight into registers: load r fetches row 4*kg + r.
+//   O += P V with v_mfma_f32_4x4x1_16B_f32 (16 independent 4x4 outer products):
+//      block = 4 lanes = one token row, A = p[g][t] (lane%4 = g), B = V[t][d]
+//      (d = 8*c + u), so values feed the matrix unit in the layout they were
+//      loaded in; P and V stay fp32.
+// Query groups larger than 4 run NG = 2 passes of the S / PV tiles per page.
+#pragma once
+
+#include <cmath>
+
+#include "kin_common.h"
+
+namespace kin {
+
+// s_waitcnt immediate for "vmcnt <= 4, no wait on expcnt / lgkmcnt" (gfx9 encoding:
+// vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]).
+constexpr int kWaitVm4 = 4 | (7 << 4) | (15 << 8);
+
+constexpr float kNegInf = -INFINITY;
+constexpr float kLn2 = 0.6931471805599453f;
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Buffer descriptor covering `bytes` bytes from `base` (0 bytes: every load
+// through it returns zeros without touching memory).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+
+// One page for one wave, first half: scores and the online softmax update.
+// ka: this lane's 4 K chunks in MFMA A layout.  Leaves the probabilities of
+// this lane's 4 tokens in pr.
+template <int NG>
+__device__ __forceinline__ void page_scores(const uint4 (&ka)[4], const bf16x8 (&qB)[NG][4], float (&m_run)[NG],
+                                            float (&l_run)[NG], floatx4 (&O)[NG][8], float (&pr)[NG][4],
+                                            float scale_log2, int valid_tokens, int kg) {
+  floatx4 S[NG];
+#pragma unroll
+  for (int half = 0; half < NG; ++half) S[half] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const bf16x8 a = __builtin_bit_cast(bf16x8, ka[c]);
+#pragma unroll
+    for (int half = 0; half < NG; ++half)
+      S[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qB[half][c], S[half], 0, 0, 0);
+  }
+#pragma unroll
+  for (int half = 0; half < NG; ++half) {
+    float s[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) s[r] = (4 * kg + r < valid_tokens) ? S[half][r] * scale_log2 : kNegInf;
+    const float m_new = fmaxf(m_run[half], fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
+    if (__any(m_new > m_run[half])) {
+      const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
+      const float alpha = fast_exp2(m_run[half] - m_safe);
+      l_run[half] *= alpha;
+      const float a0 = quad_bcast<0>(alpha), a1 = quad_bcast<1>(alpha);
+      const float a2 = quad_bcast<2>(alpha), a3 = quad_bcast<3>(alpha);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        O[half][u][0] *= a0;
+        O[half][u][1] *= a1;
+        O[half][u][2] *= a2;
+        O[half][u][3] *= a3;
+      }
+      m_run[half] = m_new;
+    }
+    const float m_use = (m_run[half] == kNegInf) ? 0.f : m_run[half];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) pr[half][r] = fast_exp2(s[r] - m_use);
+    l_run[half] += (pr[half][0] + pr[half][1]) + (pr[half][2] + pr[half][3]);
+  }
+}
+
+// Second half: O += P V.  vr: this lane's 4 V rows (row 4*kg + r).
+template <int NG>
+__device__ __forceinline__ void page_pv(const u32x4 (&vr)[4], const float (&pr)[NG][4], floatx4 (&O)[NG][8]) {
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const u32x4 vv = vr[r];
+    const float vf[8] = {bf16_lo(vv.x), bf16_hi(vv.x), bf16_lo(vv.y), bf16_hi(vv.y),
+                         bf16_lo(vv.z), bf16_hi(vv.z), bf16_lo(vv.w), bf16_hi(vv.w)};
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+#pragma unroll
+      for (int half = 0; half < NG; ++half)
+        O[half][u] = __builtin_amdgcn_mfma_f32_4x4x1f32(pr[half][r], vf[u], O[half][u], 0, 0, 0);
+    }
+  }
+}
+
+
+// Wave-uniform description of one list for attend_list().
+struct AttendArgs {
+  const uint16_t* q_bh;  // the group's G query rows (contiguous, 128 bf16 each)
+  const char* kvb;       // kv_cache base + h * 256 bytes
+  int row_bytes;         // bytes between token rows of a page (H_kv * 256)
+  int page_bytes;        // 2 * 16 * row_bytes
+  int span;              // bytes addressable from kvb within one page
+  int64_t num_pages;
+  int G;
+  float scale_log2;      // sm_scale * log2(e)
+  int n;                 // list length
+  int p0, p1;            // this workgroup's part of the list [p0, p1)
+  int last_len;          // tokens in the list's final page
+};
+
+constexpr int kAttendLdsBytes = 32768;  // 4 waves x 2 stages x 4 KiB; reused for the merge
+
+// id_at(i) returns the (wave-uniform) physical page id of list entry i, 0 <= i < n.
+// emit(g, d, o, lse2) receives, once per (head g < G, column d), the normalised
+// output and the base-2 log-sum-exp (-inf and o = 0 for an empty part).
+// lds: kAttendLdsBytes, 16-byte aligned; sm_m / sm_l: 4 x (4*NG) floats each.
+template <int NG, typename IdAt, typename Emit>
+__device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, unsigned char* lds,
+                                            float (*sm_m)[4 * NG], float (*sm_l)[4 * NG], Emit emit) {
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l = tid & 63, kg = l >> 4, c16 = l & 15, gq = l & 3;
+  const int G = a.G;
+  const int n = a.n, p0 = a.p0, p1 = a.p1, last_len = a.last_len;
+
+  // Query operands: B[k][j], j = l%16 -> head 4*half + l%4, k-chunk = l/16.
+  bf16x8 qB[NG][4];
+#pragma unroll
+  for (int half = 0; half < NG; ++half) {
+    const int g = min(4 * half + gq, G - 1);
+    const uint16_t* qp = a.q_bh + (int64_t)g * kHeadDim + 8 * kg;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      qB[half][c] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(qp + 32 * c));
+  }
+
+  const int row_bytes = a.row_bytes;
+  const int page_bytes = a.page_bytes;
+  const int span = a.span;
+  const char* kvb = a.kvb;
+  int voff[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) voff[c] = (kPageSize + 4 * kg + c) * row_bytes + c16 * 16;
+  // K staging: two 4 KiB stages per wave, filled by LDS-direct buffer loads
+  // (no VGPRs while in flight).  Load c brings rows 4c..4c+3: lane (kg, c16)
+  // lands at LDS row 4c+kg, position c16, and fetches the chunk that belongs
+  // there under the XOR swizzle (position p of row R holds chunk p ^ R).
+  unsigned char* kl = lds + w * (2 * 4096);
+  int kdma_off[4], lds_r[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int row = 4 * c + kg;
+    kdma_off[c] = row * row_bytes + ((c16 ^ row) & 15) * 16;
+    const int chunk_r = 4 * c + kg;  // chunk of row c16 that MFMA c wants from this lane
+    lds_r[c] = c16 * 256 + ((chunk_r ^ c16) & 15) * 16;
+  }
+
+  float m_run[NG], l_run[NG];
+  floatx4 O[NG][8];
+#pragma unroll
+  for (int half = 0; half < NG; ++half) {
+    m_run[half] = kNegInf;
+    l_run[half] = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) O[half][u] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // This wave takes list entries my_first, my_first+4, ...  The loop below is
+  // branch-free: a page past the end (or with an id outside the cache) is read
+  // through an empty buffer descriptor -- zeros, no memory traffic -- and all
+  // of its tokens are masked.
+  const int my_first = p0 + w;
+  const int iters = (p1 > my_first) ? (p1 - my_first + 3) / 4 : 0;
+  const int n_last = n - 1;
+  // Page ids are fetched one half-step before they are needed.
+  auto load_id = [&](int it) -> int {
+    const int idx = my_first + 4 * it;
+    return id_at(idx < p1 ? idx : p0);
+  };
+  auto page_rsrc = [&](int it, int id, int& valid_tokens) {
+    const int idx = my_first + 4 * it;
+    const bool ok = idx < p1 && id >= 0 && (int64_t)id < a.num_pages;
+    valid_tokens = ok ? (idx == n_last ? last_len : kPageSize) : 0;
+    return make_rsrc(kvb + (int64_t)(ok ? id : 0) * page_bytes, ok ? span : 0);
+  };
+  auto issue_v = [&](__amdgpu_buffer_rsrc_t r, u32x4 (&vv)[4]) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) vv[c] = __builtin_amdgcn_raw_buffer_load_b128(r, voff[c], 0, kStreamLoad);
+  };
+  auto issue_k = [&](__amdgpu_buffer_rsrc_t r, int stage) {
+    __attribute__((address_space(3))) unsigned char* dst =
+        (__attribute__((address_space(3))) unsigned char*)(kl + stage * 4096);
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, dst + c * 1024, 16, kdma_off[c], 0, 0, kStreamLoad);
+  };
+  auto read_k = [&](int stage, uint4 (&ka)[4]) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) ka[c] = *reinterpret_cast<const uint4*>(kl + stage * 4096 + lds_r[c]);
+  };
+
+  // The compiler does not order LDS reads after LDS-direct loads by itself, so
+  // the wait is explicit: when it executes, exactly the 4 V loads issued just
+  // before it are allowed to be outstanding, which means the K stage about to
+  // be read (and the V registers about to be used) have landed.  The scheduling
+  // fences keep the instruction order this count relies on.
+  if (iters > 0 && n > 0) {
+    u32x4 vA[4], vB[4];
+    uint4 ka[4];
+    float pr[NG][4];
+    int validA, validB;
+    {
+      const __amdgpu_buffer_rsrc_t r0 = page_rsrc(0, load_id(0), validA);
+      issue_k(r0, 0);
+      issue_v(r0, vA);
+    }
+    int id_next = load_id(1);
+    for (int it = 0; it < iters; it += 2) {
+      {
+        const __amdgpu_buffer_rsrc_t r1 = page_rsrc(it + 1, id_next, validB);
+        __builtin_amdgcn_sched_barrier(0);
+        issue_v(r1, vB);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(kWaitVm4);
+        __builtin_amdgcn_sched_barrier(0);
+        read_k(0, ka);
+        __builtin_amdgcn_sched_barrier(0);
+        issue_k(r1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validA, kg);
+        __builtin_amdgcn_sched_barrier(0);
+        id_next = load_id(it + 2);  // lands while the P V products run
+        page_pv<NG>(vA, pr, O);
+      }
+      {
+        const __amdgpu_buffer_rsrc_t r2 = page_rsrc(it + 2, id_next, validA);
+        __builtin_amdgcn_sched_barrier(0);
+        issue_v(r2, vA);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(kWaitVm4);
+        __builtin_amdgcn_sched_barrier(0);
+        read_k(1, ka);
+        __builtin_amdgcn_sched_barrier(0);
+        issue_k(r2, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validB, kg);
+        __builtin_amdgcn_sched_barrier(0);
+        id_next = load_id(it + 3);
+        page_pv<NG>(vB, pr, O);
+      }
+    }
+  }
+  // LDS-direct loads that are still in flight (masked tail pages) must land
+  // before the staging area is reused below.
+  __builtin_amdgcn_s_waitcnt(0);
+
+  // ---- merge the 4 row groups of the wave (lanes l, l^16, l^32, l^48) --------
+  float m_w[NG], l_w[NG];
+#pragma unroll
+  for (int half = 0; half < NG; ++half) {
+    float mm = m_run[half];
+    mm = fmaxf(mm, __shfl_xor(mm, 16));
+    mm = fmaxf(mm, __shfl_xor(mm, 32));
+    const float m_safe = (mm == kNegInf) ? 0.f : mm;
+    const float sc = fast_exp2(m_run[half] - m_safe);
+    float ll = l_run[half] * sc;
+    ll += __shfl_xor(ll, 16);
+    ll += __shfl_xor(ll, 32);
+    m_w[half] = mm;
+    l_w[half] = ll;
+    const float s0 = quad_bcast<0>(sc), s1 = quad_bcast<1>(sc), s2 = quad_bcast<2>(sc), s3 = quad_bcast<3>(sc);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      float x0 = O[half][u][0] * s0, x1 = O[half][u][1] * s1, x2 = O[half][u][2] * s2, x3 = O[half][u][3] * s3;
+      x0 += __shfl_xor(x0, 16); x1 += __shfl_xor(x1, 16); x2 += __shfl_xor(x2, 16); x3 += __shfl_xor(x3, 16);
+      x0 += __shfl_xor(x0, 32); x1 += __shfl_xor(x1, 32); x2 += __shfl_xor(x2, 32); x3 += __shfl_xor(x3, 32);
+      O[half][u] = floatx4{x0, x1, x2, x3};
+    }
+  }
+  __syncthreads();  // every wave is done with its K staging area
+  float* ow = reinterpret_cast<float*>(lds);  // [4 waves][4*NG heads][128]
+  if (kg == 0) {
+#pragma unroll
+    for (int half = 0; half < NG; ++half) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float* dst = ow + ((w * 4 * NG + 4 * half + i) * kHeadDim + 8 * c16);
+        *reinterpret_cast<float4*>(dst) = make_float4(O[half][0][i], O[half][1][i], O[half][2][i], O[half][3][i]);
+        *reinterpret_cast<float4*>(dst + 4) = make_float4(O[half][4][i], O[half][5][i], O[half][6][i], O[half][7][i]);
+      }
+      if (l < 4) {
+        sm_m[w][4 * half + l] = m_w[half];
+        sm_l[w][4 * half + l] = l_w[half];
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- merge the 4 waves and hand the results out -------------------------------
+#pragma unroll
+  for (int j = 0; j < 2 * NG; ++j) {
+    const int idx = tid + 256 * j;
+    const int g = idx >> 7, d = idx & 127;
+    if (g < G) {
+      float mm = fmaxf(fmaxf(sm_m[0][g], sm_m[1][g]), fmaxf(sm_m[2][g], sm_m[3][g]));
+      const float m_safe = (mm == kNegInf) ? 0.f : mm;
+      float num = 0.f, den = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < 4; ++wv) {
+        const float sc = fast_exp2(sm_m[wv][g] - m_safe);
+        num += ow[(wv * 4 * NG + g) * kHeadDim + d] * sc;
+        den += sm_l[wv][g] * sc;
+      }
+      const float o = (den > 0.f) ? num / den : 0.f;
+      const float lse2 = (den > 0.f) ? mm + fast_log2(den) : kNegInf;
+      emit(g, d, o, lse2);
+    }
+  }
+}
+
+}  // namespace kin

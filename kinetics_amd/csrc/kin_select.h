@@ -1,0 +1,269 @@
+// Device-side building block: page scoring + top-k page selection for one
+// (sequence, KV head), run by one 256-thread workgroup.  Shared by the
+// stand-alone selector kernel and the fused decode-step kernel.
+//
+//   phase 1  stream the sequence's representative keys (256 B each) once,
+//            16 lanes per key with 16-byte loads, fp32 dot with the group-mean
+//            query, DPP reduction inside each 16-lane row; scores stay in LDS
+//            as order-preserving 32-bit keys (never written to HBM);
+//   phase 2  4-pass 8-bit radix select in LDS for the k-th largest key;
+//   phase 3  gather the winners (ties at the threshold by lowest index), order
+//            them (score descending, index ascending) in LDS -- by counting for
+//            k <= 512, by bitonic sort above -- translate logical -> physical
+//            page ids and append the last page.
+// HBM-bound on phase 1: n_cand * 256 B per workgroup.
+#pragma once
+
+#include "kin_common.h"
+
+namespace kin {
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Monotone map float -> uint32: a < b  <=>  key(a) < key(b)  (-0 < +0).
+__device__ __forceinline__ uint32_t order_key(float f) {
+  const uint32_t u = __float_as_uint(f);
+  return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
+}
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;          // independent 16-byte loads in flight per lane
+constexpr int kRankSortMax = 512;   // up to here winners are ordered by counting, above by bitonic sort
+
+// Wave-uniform description of one selection problem.
+struct SelectArgs {
+  const uint16_t* q_bh;       // the group's G query rows
+  int G;
+  const char* kb;             // first representative key of (b, h)
+  int row_stride_b;           // bytes between consecutive logical pages
+  int n_pages;                // pages of the sequence (>= 1)
+  int n_cand;                 // candidates: min(n_pages - 1, capacity)
+  int topk;
+  const int32_t* table;       // the sequence's page table (logical -> physical)
+  int32_t* sel_logical;       // HBM, topk entries, or null
+  float* scores_out;          // HBM, n_cand entries, or null
+  uint32_t* keys;             // LDS, >= n_cand entries
+  unsigned long long* sortbuf;  // LDS, sort_cap entries
+  int sort_cap;               // power of two >= min(topk, capacity)
+};
+
+__host__ __device__ inline size_t select_lds_bytes(int kbar_pages, int sort_cap) {
+  return (size_t)((kbar_pages + 3) & ~3) * 4 + (size_t)sort_cap * 8;
+}
+
+__host__ __device__ inline int select_sort_cap(int topk, int kbar_pages) {
+  const int need = topk < kbar_pages ? topk : kbar_pages;  // k_eff never exceeds either
+  int cap = 2;
+  while (cap < need) cap <<= 1;
+  return cap;
+}
+
+// Writes the ordered physical ids of the k_eff winners to sel_lds[0 .. k_eff)
+// and the sequence's last page to sel_lds[k_eff] (LDS, >= topk + 1 entries);
+// returns k_eff.  Ends with a workgroup barrier: sel_lds is visible to every
+// thread and keys / sortbuf are free for reuse.
+__device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_lds) {
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t wave_tot[4];
+  __shared__ uint32_t sh_bin, sh_remaining, sh_count;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n_cand = a.n_cand, n_pages = a.n_pages;
+  const int k_eff = min(a.topk, n_cand);
+  uint32_t* keys = a.keys;
+  unsigned long long* sortbuf = a.sortbuf;
+
+  // ---- phase 1: scores --------------------------------------------------
+  // Lane owns columns d = 8*(lane%16) .. +7 of the mean query.
+  const int c16 = lane & 15;
+  float qm[8];
+  {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) qm[u] = 0.f;
+    const uint16_t* qp = a.q_bh + 8 * c16;
+    for (int g = 0; g < a.G; ++g) {
+      const uint4 w = *reinterpret_cast<const uint4*>(qp + (int64_t)g * kHeadDim);
+      qm[0] += bf16_lo(w.x); qm[1] += bf16_hi(w.x);
+      qm[2] += bf16_lo(w.y); qm[3] += bf16_hi(w.y);
+      qm[4] += bf16_lo(w.z); qm[5] += bf16_hi(w.z);
+      qm[6] += bf16_lo(w.w); qm[7] += bf16_hi(w.w);
+    }
+    const float inv = 1.0f / (float)a.G;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) qm[u] *= inv;
+  }
+  // The candidates of (b, h) are rows of 256 B at a fixed stride.  They are read
+  // through a buffer descriptor that ends after the last candidate, so loads past
+  // the end return zeros without touching memory and the loop needs no branches:
+  // each lane keeps kUnroll 16-byte loads in flight, re-issuing slot j for the
+  // next pass as soon as it has consumed it.
+  const int row_stride_b = a.row_stride_b;  // bytes between logical pages
+  const char* kb = a.kb;
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(kb), 0, n_cand > 0 ? (n_cand - 1) * row_stride_b + kRowBytes : 0, 0x00020000);
+  float* sc_out = a.scores_out;
+  const int sub = tid >> 4;  // 0..15: which of the 16 rows of a slot this lane helps with
+  const int lane_off = sub * row_stride_b + c16 * 16;
+  u32x4 w[kUnroll];
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j)
+    w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + j * 16 * row_stride_b, 0, kStreamLoad);
+  for (int base = 0; base < n_cand; base += 16 * kUnroll) {
+    const int next_off = (base + 16 * kUnroll) * row_stride_b;
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      const u32x4 x = w[j];
+      w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + j * 16 * row_stride_b, next_off, kStreamLoad);
+      float acc = 0.f;
+      acc = fmaf(qm[0], bf16_lo(x.x), acc); acc = fmaf(qm[1], bf16_hi(x.x), acc);
+      acc = fmaf(qm[2], bf16_lo(x.y), acc); acc = fmaf(qm[3], bf16_hi(x.y), acc);
+      acc = fmaf(qm[4], bf16_lo(x.z), acc); acc = fmaf(qm[5], bf16_hi(x.z), acc);
+      acc = fmaf(qm[6], bf16_lo(x.w), acc); acc = fmaf(qm[7], bf16_hi(x.w), acc);
+      acc = row16_sum(acc);
+      const int row = base + j * 16 + sub;
+      if (c16 == 0 && row < n_cand) {
+        keys[row] = order_key(acc);
+        if (sc_out) sc_out[row] = acc;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 2: radix select of the k_eff-th largest key -------------------
+  uint32_t prefix = 0, mask = 0;
+  uint32_t remaining = (uint32_t)k_eff;  // how many keys equal to the threshold are taken
+  if (k_eff > 0 && k_eff < n_cand) {
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      hist[tid] = 0;
+      __syncthreads();
+      for (int i = tid; i < n_cand; i += kThreads) {
+        const uint32_t key = keys[i];
+        if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+      }
+      __syncthreads();
+      if (wave == 0) {
+        // Lane j owns bins 255-4j .. 252-4j (highest first); an inclusive scan
+        // over lanes counts the keys in all bins at or above the lane's lowest.
+        // The bin where the running count first reaches `remaining` holds the
+        // threshold digit.
+        const int top = 255 - 4 * lane;
+        const uint32_t c0 = hist[top], c1 = hist[top - 1], c2 = hist[top - 2], c3 = hist[top - 3];
+        const uint32_t mine = c0 + c1 + c2 + c3;
+        uint32_t incl = mine;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+          const uint32_t up = __shfl_up(incl, off);
+          if (lane >= off) incl += up;
+        }
+        uint32_t run = incl - mine;  // keys in bins above this lane's
+        if (run < remaining && remaining <= incl) {
+          int bin = top;
+          uint32_t c = c0;
+          if (run + c < remaining) { run += c; bin = top - 1; c = c1; }
+          if (run + c < remaining) { run += c; bin = top - 2; c = c2; }
+          if (run + c < remaining) { run += c; bin = top - 3; }
+          sh_bin = (uint32_t)bin;
+          sh_remaining = remaining - run;
+        }
+      }
+      __syncthreads();
+      prefix |= sh_bin << shift;
+      mask |= 255u << shift;
+      remaining = sh_remaining;
+      // The two barriers at the top of the next pass order these reads before
+      // the next write of sh_bin / sh_remaining.
+    }
+  }
+  const bool take_all = (k_eff >= n_cand);
+  const uint32_t thr = prefix;
+
+  // ---- phase 3: gather, sort, translate --------------------------------------
+  const bool rank_sort = (k_eff <= kRankSortMax);
+  if (!rank_sort)
+    for (int i = tid; i < a.sort_cap; i += kThreads) sortbuf[i] = 0ull;
+  if (tid == 0) sh_count = 0;
+  __syncthreads();
+  if (k_eff > 0) {
+    // Keys above the threshold: any order (the sort fixes it).
+    // Keys equal to it: the `remaining` lowest indices, found by an ordered count.
+    const int per = (n_cand + kThreads - 1) / kThreads;
+    const int lo = min(tid * per, n_cand), hi = min(lo + per, n_cand);
+    uint32_t eq_cnt = 0;
+    for (int i = lo; i < hi; ++i) {
+      const uint32_t key = keys[i];
+      if (take_all || key > thr) {
+        const uint32_t slot = atomicAdd(&sh_count, 1u);
+        sortbuf[slot] = ((unsigned long long)key << 32) | (uint32_t)(0xffffffffu - (uint32_t)i);
+      } else if (key == thr) {
+        eq_cnt++;
+      }
+    }
+    if (!take_all) {
+      // exclusive block scan of eq_cnt in thread order (== index order)
+      uint32_t incl = eq_cnt;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t up = __shfl_up(incl, off);
+        if (lane >= off) incl += up;
+      }
+      if (lane == 63) wave_tot[wave] = incl;
+      __syncthreads();
+      uint32_t before = 0;
+      for (int wv = 0; wv < wave; ++wv) before += wave_tot[wv];
+      uint32_t rank = incl - eq_cnt + before;
+      for (int i = lo; i < hi && rank < remaining; ++i) {
+        const uint32_t key = keys[i];
+        if (key == thr) {
+          const uint32_t slot = atomicAdd(&sh_count, 1u);
+          sortbuf[slot] = ((unsigned long long)key << 32) | (uint32_t)(0xffffffffu - (uint32_t)i);
+          rank++;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  const int32_t* table = a.table;
+  if (rank_sort) {
+    // Small k: every winner counts the winners that beat it (entries are
+    // distinct, so the counts are a permutation) and writes itself to that slot.
+    // All lanes read the same LDS word per step: a broadcast, no conflicts.
+    for (int i = tid; i < k_eff; i += kThreads) {
+      const unsigned long long mine = sortbuf[i];
+      int rank = 0;
+#pragma unroll 8
+      for (int j = 0; j < k_eff; ++j) rank += (sortbuf[j] > mine) ? 1 : 0;
+      const uint32_t logical = 0xffffffffu - (uint32_t)(mine & 0xffffffffull);
+      sel_lds[rank] = table[logical];
+      if (a.sel_logical) a.sel_logical[rank] = (int32_t)logical;
+    }
+  } else {
+    // Large k: bitonic sort, descending, over sort_cap (power of two) 64-bit
+    // entries; the zero padding sinks to the end.
+    for (int size = 2; size <= a.sort_cap; size <<= 1) {
+      for (int stride = size >> 1; stride > 0; stride >>= 1) {
+        for (int i = tid; i < (a.sort_cap >> 1); i += kThreads) {
+          const int lo_i = 2 * i - (i & (stride - 1));
+          const int hi_i = lo_i + stride;
+          const bool desc = ((lo_i & size) == 0);
+          const unsigned long long x = sortbuf[lo_i], y = sortbuf[hi_i];
+          if ((x < y) == desc) {
+            sortbuf[lo_i] = y;
+            sortbuf[hi_i] = x;
+          }
+        }
+        __syncthreads();
+      }
+    }
+    for (int i = tid; i < k_eff; i += kThreads) {
+      const uint32_t logical = 0xffffffffu - (uint32_t)(sortbuf[i] & 0xffffffffull);
+      sel_lds[i] = table[logical];
+      if (a.sel_logical) a.sel_logical[i] = (int32_t)logical;
+    }
+  }
+  if (tid == 0) sel_lds[k_eff] = table[n_pages - 1];
+  __syncthreads();
+  return k_eff;
+}
+
+}  // namespace kin

@@ -1,0 +1,221 @@
+// Fused decode step: append -> score -> select -> attend in ONE launch, one
+// 256-thread workgroup per (sequence, KV head).
+//
+// Compared with the three stand-alone kernels this removes two dependent
+// dispatches, the selector's drain (its last workgroups finish their LDS-only
+// select phase with the memory system idle) and the attention kernel's ramp-up;
+// workgroups drift out of phase, so one workgroup's select overlaps its
+// neighbours' streaming.  The selected page ids stay in LDS (HBM copies are
+// optional outputs).  Same building blocks and arithmetic as the stand-alone
+// kernels: score_select() (kin_select.h) and attend_list() (kin_attend.h).
+#include "kin_attend.h"
+#include "kin_select.h"
+
+namespace kin {
+
+struct StepParams {
+  const uint16_t* q;
+  const uint32_t* k;  // new token's K/V rows as dwords; null = no append
+  const uint32_t* v;
+  uint16_t* kv;
+  uint16_t* kbar;
+  const int32_t* page_indices;
+  const int32_t* page_indptr;
+  const int32_t* last_page_len;
+  int32_t* sel_pages;  // optional HBM copy of the page lists
+  int32_t* sel_count;  // optional
+  uint16_t* out;
+  float* lse;  // optional
+  int num_q_heads, num_kv_heads, group;
+  int kbar_pages, sel_stride, topk, sort_cap;
+  int region0_bytes;  // LDS: max(attend staging, select scratch); the page list follows it
+  int64_t num_pages;
+  float scale_log2;
+};
+
+template <int NG>
+__global__ __launch_bounds__(256, 2) void blocktopk_step_kernel(StepParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  __shared__ float sm_m[4][4 * NG];
+  __shared__ float sm_l[4][4 * NG];
+
+  const int tid = threadIdx.x;
+  const int item = blockIdx.x;
+  const int b = item / p.num_kv_heads, h = item - b * p.num_kv_heads;
+  const int G = p.group;
+  const int64_t hq0 = (int64_t)b * p.num_q_heads + (int64_t)h * G;
+
+  const int ps = p.page_indptr[b], pe = p.page_indptr[b + 1];
+  const int n_pages = pe - ps;
+  if (n_pages <= 0) {  // empty sequence: nothing to append, select or attend
+    if (p.sel_pages)
+      for (int i = tid; i < p.sel_stride; i += 256) p.sel_pages[(int64_t)item * p.sel_stride + i] = -1;
+    if (p.sel_count && tid == 0) p.sel_count[item] = 0;
+    for (int i = tid; i < G * kHeadDim; i += 256) p.out[hq0 * kHeadDim + i] = 0;
+    if (p.lse && tid < G) p.lse[hq0 + tid] = kNegInf;
+    return;
+  }
+  const int last_len = p.last_page_len[b];
+  const int row_dw = p.num_kv_heads * (kHeadDim / 2);  // dwords per token row
+
+  // ---- append (wave 0): same byte moves and mean-key update as append_kernel ----
+  if (p.k != nullptr && tid < 64) {
+    const int lane = tid;
+    const int pos = last_len - 1;
+    const int64_t pid = p.page_indices[pe - 1];
+    if (pos >= 0 && pos < kPageSize && pid >= 0 && pid < p.num_pages) {
+      uint32_t* kplane = reinterpret_cast<uint32_t*>(p.kv) + pid * (2LL * kPageSize * row_dw) + h * (kHeadDim / 2);
+      uint32_t* vplane = kplane + (int64_t)kPageSize * row_dw;
+      const int64_t src = (int64_t)item * (kHeadDim / 2) + lane;
+      const uint32_t kw = p.k[src], vw = p.v[src];
+      kplane[(int64_t)pos * row_dw + lane] = kw;
+      vplane[(int64_t)pos * row_dw + lane] = vw;
+      if (p.kbar != nullptr && pos == kPageSize - 1 && n_pages - 1 < p.kbar_pages) {
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int t = 0; t < kPageSize - 1; ++t) {
+          const uint32_t w = kplane[(int64_t)t * row_dw + lane];
+          s0 += bf16_lo(w);
+          s1 += bf16_hi(w);
+        }
+        s0 += bf16_lo(kw);
+        s1 += bf16_hi(kw);
+        const float inv = 1.0f / kPageSize;
+        reinterpret_cast<uint32_t*>(p.kbar)[(((int64_t)b * p.kbar_pages + (n_pages - 1)) * p.num_kv_heads + h) *
+                                                (kHeadDim / 2) +
+                                            lane] = f32_to_bf16(s0 * inv) | (f32_to_bf16(s1 * inv) << 16);
+      }
+    }
+    // The attention phase of this workgroup reads the row back: make the stores
+    // visible before the barriers that separate the phases.
+    __threadfence_block();
+  }
+
+  // ---- score + select: page list into LDS -------------------------------------
+  int32_t* sel_lds = reinterpret_cast<int32_t*>(smem + p.region0_bytes);
+  SelectArgs s;
+  s.q_bh = p.q + hq0 * kHeadDim;
+  s.G = G;
+  s.row_stride_b = p.num_kv_heads * kRowBytes;
+  s.kb = reinterpret_cast<const char*>(p.kbar) + ((int64_t)b * p.kbar_pages * p.num_kv_heads + h) * kRowBytes;
+  s.n_pages = n_pages;
+  s.n_cand = min(n_pages - 1, p.kbar_pages);
+  s.topk = p.topk;
+  s.table = p.page_indices + ps;
+  s.sel_logical = nullptr;
+  s.scores_out = nullptr;
+  s.keys = reinterpret_cast<uint32_t*>(smem);
+  s.sortbuf = reinterpret_cast<unsigned long long*>(smem + (size_t)((p.kbar_pages + 3) & ~3) * 4);
+  s.sort_cap = p.sort_cap;
+  const int k_eff = score_select(s, sel_lds);
+  const int n = k_eff + 1;
+  if (p.sel_pages) {
+    int32_t* sel = p.sel_pages + (int64_t)item * p.sel_stride;
+    for (int i = tid; i < p.sel_stride; i += 256) sel[i] = (i < n) ? sel_lds[i] : -1;
+  }
+  if (p.sel_count && tid == 0) p.sel_count[item] = n;
+
+  // ---- attend over the listed pages (select scratch is dead: reuse as staging) ---
+  AttendArgs a;
+  a.q_bh = s.q_bh;
+  a.kvb = reinterpret_cast<const char*>(p.kv) + (int64_t)h * kRowBytes;
+  a.row_bytes = p.num_kv_heads * kRowBytes;
+  a.page_bytes = 2 * kPageSize * a.row_bytes;
+  a.span = a.page_bytes - h * kRowBytes;
+  a.num_pages = p.num_pages;
+  a.G = G;
+  a.scale_log2 = p.scale_log2;
+  a.n = n;
+  a.p0 = 0;
+  a.p1 = n;
+  a.last_len = last_len;
+  attend_list<NG>(
+      a, [&](int i) -> int { return __builtin_amdgcn_readfirstlane(sel_lds[i]); }, smem, sm_m, sm_l,
+      [&](int g, int d, float o, float lse2) {
+        p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_bf16(o);
+        if (p.lse && d == 0) p.lse[hq0 + g] = lse2 * kLn2;
+      });
+}
+
+}  // namespace kin
+
+extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
+                                         kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
+                                         const int32_t* page_indptr, const int32_t* last_page_len, int topk,
+                                         int32_t* sel_pages, int32_t* sel_count, kin_bf16_t* out, float* lse,
+                                         int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
+                                         int64_t num_pages, int kbar_pages, int sel_stride, float sm_scale,
+                                         kin_stream_t stream) {
+  using namespace kin;
+  const char* fn = "kin_blocktopk_decode_step";
+  if (!q || !kv_cache || !kbar || !page_indices || !page_indptr || !last_page_len || !out)
+    return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
+  if ((k == nullptr) != (v == nullptr))
+    return fail(KIN_ERR_NULL_POINTER, "%s: k and v must both be given or both be null", fn);
+  int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size);
+  if (st) return st;
+  if (num_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_pages=%lld must be >= 1", fn, (long long)num_pages);
+  if (topk < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: topk=%d must be >= 1", fn, topk);
+  if (kbar_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: kbar_pages=%d must be >= 1", fn, kbar_pages);
+  if (sel_pages && sel_stride <= topk)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must exceed topk=%d (room for the last page)", fn, sel_stride,
+                topk);
+  if (sel_pages && !sel_count) return fail(KIN_ERR_NULL_POINTER, "%s: sel_pages given without sel_count", fn);
+  if (topk > kMaxTopk) return fail(KIN_ERR_UNSUPPORTED, "%s: topk=%d exceeds the limit %d", fn, topk, kMaxTopk);
+  if (kbar_pages > kMaxCandidates)
+    return fail(KIN_ERR_UNSUPPORTED, "%s: kbar_pages=%d exceeds the limit %d", fn, kbar_pages, kMaxCandidates);
+  if (!aligned16(q) || !aligned16(kv_cache) || !aligned16(kbar) || !aligned16(out) || (k && !aligned16(k)) ||
+      (v && !aligned16(v)))
+    return fail(KIN_ERR_MISALIGNED, "%s: q, k, v, kv_cache, kbar and out must be 16-byte aligned", fn);
+  if (batch == 0) return KIN_OK;
+
+  StepParams p;
+  p.q = q;
+  p.k = reinterpret_cast<const uint32_t*>(k);
+  p.v = reinterpret_cast<const uint32_t*>(v);
+  p.kv = kv_cache;
+  p.kbar = kbar;
+  p.page_indices = page_indices;
+  p.page_indptr = page_indptr;
+  p.last_page_len = last_page_len;
+  p.sel_pages = sel_pages;
+  p.sel_count = sel_count;
+  p.out = out;
+  p.lse = lse;
+  p.num_q_heads = num_q_heads;
+  p.num_kv_heads = num_kv_heads;
+  p.group = num_q_heads / num_kv_heads;
+  p.kbar_pages = kbar_pages;
+  p.sel_stride = sel_stride;
+  p.topk = topk;
+  p.sort_cap = select_sort_cap(topk, kbar_pages);
+  const size_t sel_scratch = select_lds_bytes(kbar_pages, p.sort_cap);
+  size_t region0 = sel_scratch > (size_t)kAttendLdsBytes ? sel_scratch : (size_t)kAttendLdsBytes;
+  region0 = (region0 + 15) & ~(size_t)15;
+  p.region0_bytes = (int)region0;
+  p.num_pages = num_pages;
+  const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
+  p.scale_log2 = scale * 1.4426950408889634f;
+  const size_t lds = region0 + (size_t)(topk + 1) * 4;
+  const int64_t items = (int64_t)batch * num_kv_heads;
+  if (items > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (p.group <= 4) {
+    if (lds > 48 * 1024) {
+      st = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&blocktopk_step_kernel<1>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                     "hipFuncSetAttribute(blocktopk_step_kernel)");
+      if (st) return st;
+    }
+    blocktopk_step_kernel<1><<<(unsigned)items, 256, lds, s>>>(p);
+  } else {
+    if (lds > 48 * 1024) {
+      st = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&blocktopk_step_kernel<2>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                     "hipFuncSetAttribute(blocktopk_step_kernel)");
+      if (st) return st;
+    }
+    blocktopk_step_kernel<2><<<(unsigned)items, 256, lds, s>>>(p);
+  }
+  return check_hip(hipGetLastError(), "blocktopk_step_kernel launch");
+}

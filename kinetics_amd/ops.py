@@ -265,6 +265,43 @@ def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, ma
     return out
 
 
+def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, out=None, lse=None,
+                          sel_pages=None, sel_count=None, sm_scale: float = 0.0):
+    """append -> score -> select -> attend in one launch: lines 209-225 of the
+    reference layer's forward (benchmark/blocktopk_decoder.py) as a single
+    kernel.  ``k``/``v`` may be None (no append); ``sel_pages``/``sel_count`` are
+    optional outputs.  Returns ``out`` [batch, num_q_heads, head_dim] bf16."""
+    dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, None)
+    _table(page_indices, page_indptr, last_page_len, batch, dev)
+    kbar_pages = _kbar_pages(kbar, batch, hkv, d)
+    if (k is None) != (v is None):
+        raise ValueError("k and v must both be given or both be None")
+    if k is not None:
+        _require(k, "k", torch.bfloat16, 3, dev)
+        _require(v, "v", torch.bfloat16, 3, dev)
+        if tuple(k.shape) != (batch, hkv, d) or k.shape != v.shape:
+            raise ValueError(f"k and v must be [{batch}, {hkv}, {d}], got {tuple(k.shape)} and {tuple(v.shape)}")
+    sel_stride = 0
+    if (sel_pages is None) != (sel_count is None):
+        raise ValueError("sel_pages and sel_count must both be given or both be None")
+    if sel_pages is not None:
+        _require(sel_pages, "sel_pages", torch.int32, 3, dev)
+        _require(sel_count, "sel_count", torch.int32, 2, dev)
+        if sel_pages.shape[:2] != (batch, hkv) or tuple(sel_count.shape) != (batch, hkv):
+            raise ValueError(f"sel_pages/sel_count must be [{batch}, {hkv}, stride] / [{batch}, {hkv}]")
+        sel_stride = sel_pages.shape[2]
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(
+            lib.kin_blocktopk_decode_step(
+                _ptr(q), _ptr(k), _ptr(v), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
+                _ptr(last_page_len), int(topk), _ptr(sel_pages), _ptr(sel_count), _ptr(out), _ptr(lse), batch, hq, hkv,
+                d, ps, num_pages, kbar_pages, sel_stride, float(sm_scale), _stream(dev),
+            )
+        )
+    return out
+
+
 def check_page_table(page_indices, page_indptr, last_page_len, page_size, num_pages) -> None:
     """Synchronous device-side validation of a page table (debugging aid);
     raises KineticsError on an invalid entry."""
@@ -307,6 +344,24 @@ torch.library.define(
     "(Tensor q, Tensor kv_cache, Tensor page_indices, Tensor page_indptr, Tensor last_page_len, "
     "int max_pages_per_seq, Tensor? workspace, float sm_scale, int num_splits) -> Tensor",
 )
+
+
+torch.library.define(
+    "kinetics::blocktopk_decode_step",
+    "(Tensor q, Tensor k, Tensor v, Tensor(a!) kv_cache, Tensor(b!) kbar, Tensor page_indices, Tensor page_indptr, "
+    "Tensor last_page_len, int topk, Tensor(c!)? sel_pages, Tensor(d!)? sel_count, float sm_scale) -> Tensor",
+)
+
+
+@torch.library.impl("kinetics::blocktopk_decode_step", "cuda")
+def _step_impl(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sm_scale):
+    return blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk,
+                                 sel_pages=sel_pages, sel_count=sel_count, sm_scale=sm_scale)
+
+
+@torch.library.register_fake("kinetics::blocktopk_decode_step")
+def _step_fake(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sm_scale):
+    return torch.empty_like(q)
 
 
 @torch.library.impl("kinetics::append_paged_kv", "cuda")
