@@ -187,8 +187,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--cpu-batch", type=int, default=128)
-    ap.add_argument("--three-kernels", action="store_true",
-                    help="time the append / score+select / attention launches separately instead of the fused step")
+    ap.add_argument("--mode", default="auto", choices=["auto", "fused", "three"],
+                    help="decode-step path: one fused launch, three launches (append / score+select / attention), "
+                         "or what kinetics_amd.ops.prefer_fused_step picks for the shape")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) to scale profiler byte counters")
     args = ap.parse_args()
@@ -213,7 +214,7 @@ def main():
     print(f"[bench] {args.workload}: B={B} ctx={ctx} H_kv={Hkv} G={G} topk={topk}, "
           f"KV {st['kv'].numel() * 2 / 1e9:.1f} GB resident, setup {time.perf_counter() - t_setup:.1f}s", file=sys.stderr)
 
-    fused = not args.three_kernels
+    fused = args.mode == "fused" or (args.mode == "auto" and ops.prefer_fused_step(B, Hkv, st["max_pages_used"], topk))
 
     def launches():
         """The step's kernel launches, in order, as (name, callable)."""

@@ -29,7 +29,7 @@ from . import ops
 class BlockTopkPagedAttention:
     def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, batch_size: int, prefix_len: int,
                  max_len: int, page_size: int, topk_page: int, device="cuda", dtype=torch.bfloat16,
-                 init_cache: str = "randn", seed: int = 0):
+                 init_cache: str = "randn", seed: int = 0, fused: Optional[bool] = None):
         if dtype != torch.bfloat16:
             raise ValueError("the HIP kernels are built for bfloat16")
         if prefix_len % page_size != 0:
@@ -72,6 +72,8 @@ class BlockTopkPagedAttention:
         self.refresh_compressed_keys()
 
         self.sm_scale = 1.0 / math.sqrt(head_dim)
+        # one launch or three: same results, the faster one for this shape unless told otherwise
+        self.fused = ops.prefer_fused_step(B, num_kv_heads, n + 1, topk_page) if fused is None else bool(fused)
         ws = ops.decode_workspace_bytes(B, num_heads, num_kv_heads, topk_page + 1)
         self.workspace: Optional[torch.Tensor] = torch.empty(ws, dtype=torch.uint8, device=dev) if ws else None
 
@@ -98,6 +100,11 @@ class BlockTopkPagedAttention:
 
     def forward(self, query_states, key_states, value_states) -> torch.Tensor:
         """q [B, H_q, D], k/v [B, H_kv, D] -> [B, H_q, D]."""
+        if self.fused:
+            return torch.ops.kinetics.blocktopk_decode_step(
+                query_states, key_states, value_states, self.kv_cache, self.compressed_key_cache,
+                self.paged_kv_indices, self.paged_kv_indptr, self.last_kv_lens, self.topk_page,
+                self.topk_page_indices, self.topk_page_count, self.sm_scale)
         self.update_kv(key_states, value_states)
         self.select_pages(query_states)
         return self.decode(query_states)

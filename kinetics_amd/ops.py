@@ -265,6 +265,20 @@ def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, ma
     return out
 
 
+def prefer_fused_step(batch: int, num_kv_heads: int, max_pages_per_seq: int, topk: int) -> bool:
+    """Which of the two equivalent decode-step paths is faster (measured on
+    MI355X).  The single-launch kernel saves two dependent dispatches and the
+    selector's drain, which wins while a step moves less than about 4 GB; its
+    workgroups live longer, so on bigger steps the end-of-kernel imbalance costs
+    more than the dispatches saved and three launches are (slightly) faster.
+    Needs enough lists to fill the GPU without split-K either way."""
+    lists = batch * num_kv_heads
+    if decode_auto_splits(batch, num_kv_heads, topk + 1) > 1:
+        return False
+    step_bytes = lists * (max_pages_per_seq * 256 + (min(topk, max_pages_per_seq) + 1) * 8192)
+    return step_bytes < 4e9
+
+
 def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, out=None, lse=None,
                           sel_pages=None, sel_count=None, sm_scale: float = 0.0):
     """append -> score -> select -> attend in one launch: lines 209-225 of the

@@ -393,11 +393,12 @@ def test_properties_at_scale(ops):
 # --------------------------------------------------------------------------- layer objects + custom ops
 
 
-def test_layer_objects_follow_the_reference_call_order(ops):
+@pytest.mark.parametrize("fused", [False, True])
+def test_layer_objects_follow_the_reference_call_order(ops, fused):
     from kinetics_amd import BlockTopkPagedAttention, DensePagedAttention
 
     B, prefix, topk = 5, PS * 48, 8
-    layer = BlockTopkPagedAttention(4, 1, D, B, prefix, prefix + 512, PS, topk, device=DEV, seed=3)
+    layer = BlockTopkPagedAttention(4, 1, D, B, prefix, prefix + 512, PS, topk, device=DEV, seed=3, fused=fused)
     torch.manual_seed(7)
     q = torch.randn(B, 4, D, device=DEV).to(torch.bfloat16)
     k = torch.randn(B, 1, D, device=DEV).to(torch.bfloat16)
