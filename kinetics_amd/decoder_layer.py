@@ -1,0 +1,148 @@
+"""Whole decoder layers with the constructor and ``forward`` of the reference's
+benchmark layers, for like-for-like whole-layer throughput runs.
+
+``BlockTopkDecoderLayer`` mirrors benchmark/blocktopk_decoder.py:96-240 and
+``DenseDecoderLayer`` mirrors benchmark/dense_decoder.py: RMSNorm -> fused
+``wqkv`` -> q/k RMSNorm -> [append, page scoring, top-k, attention] -> ``wo`` ->
+residual -> RMSNorm -> SwiGLU MLP -> residual, for one tensor-parallel shard
+(head counts and MLP width divided by ``world_size``, as the reference does at
+:101-106).  Everything between the q/k norms and ``wo`` runs on the HIP kernels
+of this package; the norms and GEMMs are plain PyTorch (rocBLAS/hipBLASLt), which
+is what the reference does too apart from using flashinfer's RMSNorm
+(benchmark/model_utils.py:4-25).
+
+The reference reads the model shape from the Hugging Face hub
+(benchmark/blocktopk.py:65); ``qwen3_config`` provides the same fields offline.
+"""
+from __future__ import annotations
+
+import math
+from types import SimpleNamespace
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .blocktopk_decoder import BlockTopkPagedAttention, DensePagedAttention
+
+# Published Qwen3 shapes (general knowledge; the reference fetches them from the hub).
+_QWEN3 = {
+    "Qwen3-0.6B": dict(hidden_size=1024, intermediate_size=3072, num_attention_heads=16, num_key_value_heads=8, num_hidden_layers=28),
+    "Qwen3-1.7B": dict(hidden_size=2048, intermediate_size=6144, num_attention_heads=16, num_key_value_heads=8, num_hidden_layers=28),
+    "Qwen3-4B": dict(hidden_size=2560, intermediate_size=9728, num_attention_heads=32, num_key_value_heads=8, num_hidden_layers=36),
+    "Qwen3-8B": dict(hidden_size=4096, intermediate_size=12288, num_attention_heads=32, num_key_value_heads=8, num_hidden_layers=36),
+    "Qwen3-14B": dict(hidden_size=5120, intermediate_size=17408, num_attention_heads=40, num_key_value_heads=8, num_hidden_layers=40),
+    "Qwen3-32B": dict(hidden_size=5120, intermediate_size=25600, num_attention_heads=64, num_key_value_heads=8, num_hidden_layers=64),
+}
+
+_ACT = {"silu": F.silu, "gelu": F.gelu, "relu": F.relu}
+
+
+def qwen3_config(name: str) -> SimpleNamespace:
+    """The config fields the layers read (benchmark/blocktopk_decoder.py:101-121)."""
+    key = name.split("/")[-1]
+    if key not in _QWEN3:
+        raise KeyError(f"unknown model {name!r}; known: {sorted(_QWEN3)}")
+    return SimpleNamespace(head_dim=128, rms_norm_eps=1e-6, hidden_act="silu", max_position_embeddings=40960,
+                           rope_theta=1000000.0, eos_token_id=151645, **_QWEN3[key])
+
+
+def rms_norm(x: torch.Tensor, eps: float, weight: torch.Tensor) -> torch.Tensor:
+    """RMSNorm over the last dimension, computed in fp32 (benchmark/model_utils.py:4-25)."""
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps) * weight.float()).to(x.dtype)
+
+
+def init_weights(m):
+    """benchmark/blocktopk_decoder.py:88-94."""
+    if isinstance(m, nn.Linear):
+        nn.init.kaiming_uniform_(m.weight, a=math.sqrt(5))
+        if m.bias is not None:
+            fan_in, _ = nn.init._calculate_fan_in_and_fan_out(m.weight)
+            bound = 1 / math.sqrt(fan_in)
+            nn.init.uniform_(m.bias, -bound, bound)
+
+
+class _LayerBase(nn.Module):
+    def __init__(self, config, world_size, batch_size, device, dtype):
+        super().__init__()
+        self.num_heads = config.num_attention_heads // world_size
+        self.num_kv_heads = config.num_key_value_heads // world_size
+        if self.num_heads < 1 or self.num_kv_heads < 1:
+            raise ValueError("world_size exceeds the number of heads")
+        self.num_key_value_groups = self.num_heads // self.num_kv_heads
+        self.head_dim = config.head_dim
+        self.dim = config.hidden_size
+        self.intermediate_size = config.intermediate_size // world_size
+        self.eps = config.rms_norm_eps
+        self.activation = _ACT[config.hidden_act]
+        self.batch_size = batch_size
+
+        self.qnorm_weight = nn.Parameter(torch.ones(self.head_dim))
+        self.knorm_weight = nn.Parameter(torch.ones(self.head_dim))
+        self.input_layernorm_weight = nn.Parameter(torch.ones(self.dim))
+        self.post_attention_layernorm_weight = nn.Parameter(torch.ones(self.dim))
+        total_head_dim = (self.num_heads + 2 * self.num_kv_heads) * self.head_dim
+        self.wqkv = nn.Linear(self.dim, total_head_dim, bias=True)
+        self.wo = nn.Linear(self.head_dim * self.num_heads, self.dim, bias=False)
+        self.up_proj = nn.Linear(self.dim, self.intermediate_size, bias=False)
+        self.gate_proj = nn.Linear(self.dim, self.intermediate_size, bias=False)
+        self.down_proj = nn.Linear(self.intermediate_size, self.dim, bias=False)
+
+    def _qkv(self, hidden_states):
+        """benchmark/blocktopk_decoder.py:192-207: norm, fused projection, split, q/k norm."""
+        bsz, q_len, _ = hidden_states.size()
+        if q_len != 1:
+            raise ValueError("decode layers take one token per sequence")
+        x = rms_norm(hidden_states, self.eps, self.input_layernorm_weight)
+        q_dim, kv_dim = self.head_dim * self.num_heads, self.head_dim * self.num_kv_heads
+        q, k, v = self.wqkv(x).split((q_dim, kv_dim, kv_dim), dim=-1)
+        q = rms_norm(q.reshape(bsz, self.num_heads, self.head_dim), self.eps, self.qnorm_weight).contiguous()
+        k = rms_norm(k.reshape(bsz, self.num_kv_heads, self.head_dim), self.eps, self.knorm_weight).contiguous()
+        v = v.reshape(bsz, self.num_kv_heads, self.head_dim).contiguous()
+        return q, k, v
+
+    def _finish(self, residual, o):
+        """benchmark/blocktopk_decoder.py:226-240: wo, residual, norm, SwiGLU MLP, residual."""
+        bsz = o.shape[0]
+        h = residual + self.wo(o.reshape(bsz, 1, self.head_dim * self.num_heads))
+        x = rms_norm(h, self.eps, self.post_attention_layernorm_weight)
+        return h + self.down_proj(self.activation(self.gate_proj(x)) * self.up_proj(x))
+
+
+class BlockTopkDecoderLayer(_LayerBase):
+    """Constructor arguments as benchmark/blocktopk_decoder.py:97-99."""
+
+    def __init__(self, config, world_size, batch_size, prefix_len, max_len, page_size, topk_page, device, dtype, seed: int = 0):
+        super().__init__(config, world_size, batch_size, device, dtype)
+        self.attn = BlockTopkPagedAttention(self.num_heads, self.num_kv_heads, self.head_dim, batch_size, prefix_len, max_len,
+                                            page_size, topk_page, device=device, dtype=dtype, seed=seed)
+
+    def prepare_wrapper(self, prefix_len=None, topk_page_indices=None):
+        """Present for call compatibility (benchmark/blocktopk_decoder.py:243-265): the
+        HIP kernels need no planning step."""
+        return None
+
+    @torch.inference_mode()
+    def forward(self, hidden_states):
+        q, k, v = self._qkv(hidden_states)
+        o = self.attn(q, k, v)
+        return self._finish(hidden_states, o)
+
+
+class DenseDecoderLayer(_LayerBase):
+    """The dense baseline layer (benchmark/dense_decoder.py)."""
+
+    def __init__(self, config, world_size, batch_size, prefix_len, max_len, page_size, device, dtype, seed: int = 0):
+        super().__init__(config, world_size, batch_size, device, dtype)
+        self.attn = DensePagedAttention(self.num_heads, self.num_kv_heads, self.head_dim, batch_size, prefix_len, max_len,
+                                        page_size, device=device, dtype=dtype, seed=seed)
+
+    def prepare_wrapper(self):
+        return None
+
+    @torch.inference_mode()
+    def forward(self, hidden_states):
+        q, k, v = self._qkv(hidden_states)
+        o = self.attn(q, k, v)
+        return self._finish(hidden_states, o)

@@ -770,3 +770,72 @@ def test_fused_step_full_size(ops):
     assert torch.equal(st["sel"], sel_b) and torch.equal(st["cnt"], cnt_b) and torch.equal(out_a, out_b)
     del st
     torch.cuda.empty_cache()
+
+
+# --------------------------------------------------------------------------- whole decoder layer
+
+
+@pytest.mark.parametrize("dense", [False, True])
+def test_decoder_layer_matches_fp32_reference(ops, dense):
+    """The drop-in layers: norms/GEMMs in PyTorch around the HIP attention.  The
+    attention inside is checked against the oracle on the layer's own q, k, v;
+    the rest against an fp32 restatement of the same layer."""
+    from types import SimpleNamespace
+
+    from kinetics_amd.decoder_layer import BlockTopkDecoderLayer, DenseDecoderLayer, init_weights, qwen3_config, rms_norm
+
+    assert qwen3_config("Qwen/Qwen3-8B").num_key_value_heads == 8
+    cfg = SimpleNamespace(num_attention_heads=8, num_key_value_heads=2, head_dim=D, hidden_size=512, intermediate_size=1024,
+                          rms_norm_eps=1e-6, hidden_act="silu")
+    B, prefix, topk = 6, PS * 40, 8
+    torch.manual_seed(11)
+    if dense:
+        layer = DenseDecoderLayer(cfg, 2, B, prefix, prefix + 512, PS, DEV, torch.bfloat16, seed=5)
+    else:
+        layer = BlockTopkDecoderLayer(cfg, 2, B, prefix, prefix + 512, PS, topk, DEV, torch.bfloat16, seed=5)
+    layer.apply(init_weights)
+    layer.eval().to(DEV, dtype=torch.bfloat16)
+    assert (layer.num_heads, layer.num_kv_heads) == (4, 1)  # world_size 2 shard
+    layer.prepare_wrapper() if dense else layer.prepare_wrapper(prefix)
+    hidden = torch.randn(B, 1, 512, device=DEV).to(torch.bfloat16)
+    st = layer.attn.state if dense else layer.attn
+    kv_before = P.from_torch(st.kv_cache)
+    kbar_before = P.from_torch(st.compressed_key_cache)
+    with torch.inference_mode():
+        q, k, v = layer._qkv(hidden)
+    out = layer(hidden.clone())
+    torch.cuda.synchronize()
+    assert out.shape == hidden.shape and out.dtype == torch.bfloat16
+    # q, k, v against fp32
+    W = {n: p.detach().float().cpu() for n, p in layer.named_parameters()}
+    h32 = hidden.float().cpu()
+
+    def rn(x, w):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * w
+
+    x = rn(h32, W["input_layernorm_weight"]).to(torch.bfloat16).float()
+    qkv = x @ W["wqkv.weight"].T + W["wqkv.bias"]
+    q32, k32, v32 = qkv.split((512, 128, 128), dim=-1)
+    q32 = rn(q32.reshape(B, 4, D), W["qnorm_weight"])
+    k32 = rn(k32.reshape(B, 1, D), W["knorm_weight"])
+    assert torch.allclose(q.float().cpu(), q32, rtol=3e-2, atol=3e-2)
+    assert torch.allclose(k.float().cpu(), k32, rtol=3e-2, atol=3e-2)
+    assert torch.allclose(v.float().cpu(), v32.reshape(B, 1, D), rtol=3e-2, atol=3e-2)
+    # attention on the layer's own q, k, v
+    idx, ptr, last = (t.cpu().numpy() for t in (st.paged_kv_indices, st.paged_kv_indptr, st.last_kv_lens))
+    if dense:
+        O.append_paged_kv(P.from_torch(k), P.from_torch(v), kv_before, None, idx, ptr, last)
+        attn, _ = O.dense_paged_decode(P.from_torch(q), kv_before, idx, ptr, last)
+    else:
+        res = O.decode_step(P.from_torch(q), P.from_torch(k), P.from_torch(v), kv_before, kbar_before, idx, ptr, last, topk)
+        attn = res["out"]
+        assert np.array_equal(layer.attn.topk_page_indices.cpu().numpy(), res["sel_pages"])
+    assert np.array_equal(P.from_torch(st.kv_cache), kv_before)
+    # the rest of the layer in fp32
+    o32 = torch.from_numpy(attn).float().to(torch.bfloat16).float().reshape(B, 1, 512)
+    h1 = h32 + o32 @ W["wo.weight"].T
+    y = rn(h1, W["post_attention_layernorm_weight"])
+    want = h1 + (torch.nn.functional.silu(y @ W["gate_proj.weight"].T) * (y @ W["up_proj.weight"].T)) @ W["down_proj.weight"].T
+    got = out.float().cpu()
+    assert torch.allclose(got, want, rtol=5e-2, atol=5e-2), (got - want).abs().max()
+    assert rms_norm(hidden, 1e-6, layer.input_layernorm_weight).dtype == torch.bfloat16
