@@ -215,6 +215,25 @@ int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const ki
                               kin_stream_t stream);
 
 /*
+ * Page-table metadata for a slot-based cache -- the paged replacement of
+ * LiteSys' contiguous per-slot caches and kv_offset counters
+ * (ref: LiteSys/litesys/attention/batch_cache.py:40-62,76-84).  Slot s owns the
+ * physical pages s*pages_per_slot .. (s+1)*pages_per_slot-1.  For sequence b
+ * living in slot slot_ids[b] (NULL = identity) with seq_lens[b] tokens, writes
+ *   page_indptr[0..batch]   CSR offsets (n_pages = ceil(len / page_size),
+ *                           clamped to pages_per_slot; 0 pages for len <= 0)
+ *   page_indices[...]       slot*pages_per_slot + p, packed per sequence
+ *                           (capacity batch*pages_per_slot entries)
+ *   last_page_len[b]        tokens in the final page (1 for empty sequences)
+ * No host synchronisation.  batch <= 65535.  (The batch == 0 case records a
+ * memset; do not capture that case in a HIP graph.)
+ */
+int kin_build_slot_page_table(const int32_t* slot_ids, const int32_t* seq_lens, int batch,
+                              int pages_per_slot, int page_size,
+                              int32_t* page_indices, int32_t* page_indptr,
+                              int32_t* last_page_len, kin_stream_t stream);
+
+/*
  * Debugging aid, SYNCHRONOUS (waits for the stream): verifies on the device
  * that page_indptr is non-decreasing from 0 and never exceeds nnz (the length
  * of page_indices), every page id lies in [0, num_pages), and every

@@ -1,0 +1,168 @@
+"""A KV manager with the interface of LiteSys' ``BatchKVManager``
+(LiteSys/litesys/attention/batch_cache.py) on top of the paged HIP kernels.
+
+LiteSys keeps contiguous per-slot caches ``[max_batch, H_kv, max_len, D]`` and,
+for block-sparse decoding, computes full-context logits, masks all but the
+top-k blocks and runs softmax and P.V over the whole context
+(batch_cache.py:154-168, sparsity_utils.py:24-47).  Here every slot owns a fixed
+run of 16-token pages of one paged cache per layer; decode appends the token,
+scores the per-page mean keys, selects the top-k pages per KV head and attends
+only to those pages plus the open page -- the same result as the mask
+formulation with page-aligned blocks, without touching the rest of the context.
+
+Supported configurations (anything else raises at construction):
+  * no sparsity arguments                      -> dense paged decode
+  * ``attn_block_topk=k`` (+ ``attn_local``)    -> block top-k with block size 16
+Differences from LiteSys, by design of the paged layout: blocks are page
+aligned (LiteSys starts them after 4 hard-wired "sink" tokens,
+sparsity_utils.py:24,240), and the always-attended local window is the open page
+(1..16 newest tokens) rather than ``attn_local`` tokens.  ``attn_layer_skip``
+(default ``[0]``: layer 0 stays dense, sparsity_utils.py:211) is honoured.
+Prefill is not the accelerated path: it writes pages with PyTorch indexing and
+runs PyTorch's scaled_dot_product_attention (LiteSys calls flashinfer there,
+batch_cache.py:112-145).
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+from . import ops
+
+PAGE = 16
+
+_UNSUPPORTED = ("attn_topk", "attn_random_select", "attn_random_nsample", "attn_stride")
+
+
+class PagedBatchKVManager:
+    def __init__(self, config, max_batch_size: int, max_seq_len: int, device, dtype, **kwargs):
+        if dtype != torch.bfloat16:
+            raise ValueError("the HIP kernels are built for bfloat16")
+        self.config = config
+        self.max_length = max_seq_len
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self.max_batch_size = max_batch_size
+        self.head_dim = getattr(config, "head_dim", config.hidden_size // config.num_attention_heads)
+        import torch.distributed as dist
+
+        self.world_size = dist.get_world_size() if dist.is_available() and dist.is_initialized() else 1
+        self.num_layers = config.num_hidden_layers
+        self.hidden_size = self.head_dim * config.num_attention_heads // self.world_size
+        self.num_key_value_heads = config.num_key_value_heads // self.world_size
+        self.num_attention_heads = config.num_attention_heads // self.world_size
+        self.num_key_value_groups = config.num_attention_heads // config.num_key_value_heads
+
+        for name in _UNSUPPORTED:
+            if kwargs.get(name) is not None:
+                raise NotImplementedError(f"{name} is a LiteSys research ablation that the paged kernels do not implement")
+        self.block_topk = kwargs.get("attn_block_topk")
+        if self.block_topk is not None:
+            if kwargs.get("attn_local") is None:
+                # same rule as LiteSys (sparsity_utils.py:207-208)
+                raise AssertionError("attn_local must be provided if use_nonlocal_sparsity is True")
+            if kwargs.get("attn_block_size", PAGE) != PAGE:
+                raise NotImplementedError("block size must equal the page size (16)")
+        elif kwargs.get("attn_local") is not None:
+            raise NotImplementedError("local-window-only sparsity is not implemented")
+        self.layer_skip = list(kwargs.get("attn_layer_skip", [0]))
+
+        B, Hq, Hkv, D = max_batch_size, self.num_attention_heads, self.num_key_value_heads, self.head_dim
+        self.pages_per_slot = P = (max_seq_len + PAGE - 1) // PAGE
+        dev = self.device
+        self.kv_cache = [torch.zeros(B * P, 2, PAGE, Hkv, D, dtype=dtype, device=dev) for _ in range(self.num_layers)]
+        self.kbar = [torch.zeros(B, P, Hkv, D, dtype=dtype, device=dev) for _ in range(self.num_layers)]
+        self.kv_offset = [torch.zeros(B, dtype=torch.int32, device=dev) for _ in range(self.num_layers)]
+        # page-table metadata (rebuilt on the device each decode call) and full-batch staging buffers
+        self.page_indices = torch.zeros(B * P, dtype=torch.int32, device=dev)
+        self.page_indptr = torch.zeros(B + 1, dtype=torch.int32, device=dev)
+        self.last_page_len = torch.ones(B, dtype=torch.int32, device=dev)
+        self._lens = torch.zeros(B, dtype=torch.int32, device=dev)
+        self._q = torch.zeros(B, Hq, D, dtype=dtype, device=dev)
+        self._k = torch.zeros(B, Hkv, D, dtype=dtype, device=dev)
+        self._v = torch.zeros(B, Hkv, D, dtype=dtype, device=dev)
+        self._out = torch.zeros(B, Hq, D, dtype=dtype, device=dev)
+        k = self.block_topk or 1
+        self._sel = torch.full((B, Hkv, k + 1), -1, dtype=torch.int32, device=dev)
+        self._cnt = torch.zeros(B, Hkv, dtype=torch.int32, device=dev)
+        self._fused = ops.prefer_fused_step(B, Hkv, P, k)
+        ws = max(ops.decode_workspace_bytes(B, Hq, Hkv, P), ops.decode_workspace_bytes(B, Hq, Hkv, k + 1), 16)
+        self._ws = torch.empty(ws, dtype=torch.uint8, device=dev)
+
+    # ------------------------------------------------------------------ LiteSys interface
+    def compute_attention(self, query_states, key_states, value_states, layer_idx, batch_idx):
+        """query [B, H_q, s, D], key/value [B, H_kv, s, D] -> [B, s, H_q*D]
+        (batch_cache.py:86-110).  s > 1 is a prefill of one request."""
+        bsz, seq_len = query_states.shape[0], query_states.shape[2]
+        if seq_len > 1:
+            return self.prefill_or_append(query_states, key_states, value_states, layer_idx, batch_idx)
+        out = self.decode(query_states, key_states, value_states, batch_idx, layer_idx)
+        return out.reshape(bsz, seq_len, self.hidden_size)
+
+    def clear_cache(self, batch_idx: int):
+        """batch_cache.py:147-152.  Pages need no zeroing: an empty page list hides them."""
+        for i in range(self.num_layers):
+            self.kv_offset[i][batch_idx] = 0
+
+    # ------------------------------------------------------------------ decode
+    def decode(self, query, key, value, batch_idx, layer_idx):
+        """append -> (select ->) attend for the active slots (batch_cache.py:154-168)."""
+        slots = batch_idx.to(self.device, torch.long)
+        off = self.kv_offset[layer_idx]
+        off[slots] += 1
+        # Sequence b of the kernels == slot b; inactive slots get an empty page list.
+        self._lens.zero_()
+        self._lens[slots] = off[slots]
+        ops.build_slot_page_table(self._lens, self.pages_per_slot, PAGE, self.page_indices, self.page_indptr, self.last_page_len)
+        self._q[slots] = query[:, :, 0, :]
+        self._k[slots] = key[:, :, 0, :]
+        self._v[slots] = value[:, :, 0, :]
+        kv, kbar = self.kv_cache[layer_idx], self.kbar[layer_idx]
+        sparse = self.block_topk is not None and layer_idx not in self.layer_skip
+        if sparse and self._fused:
+            ops.blocktopk_decode_step(self._q, self._k, self._v, kv, kbar, self.page_indices, self.page_indptr,
+                                      self.last_page_len, self.block_topk, out=self._out)
+        else:
+            ops.append_paged_kv(self._k, self._v, kv, kbar, self.page_indices, self.page_indptr, self.last_page_len)
+            if sparse:
+                ops.block_score_topk(self._q, kbar, self.page_indices, self.page_indptr, self.block_topk, self._sel, self._cnt)
+                ops.sparse_paged_decode(self._q, kv, self._sel, self._cnt, self.last_page_len, out=self._out, workspace=self._ws)
+            else:
+                ops.dense_paged_decode(self._q, kv, self.page_indices, self.page_indptr, self.last_page_len,
+                                       self.pages_per_slot, out=self._out, workspace=self._ws)
+        return self._out[slots]
+
+    # ------------------------------------------------------------------ prefill (not the accelerated path)
+    def prefill_or_append(self, query_states, key_states, value_states, layer_idx, batch_idx):
+        """One request: write its K/V rows into the slot's pages, refresh the
+        mean keys of the pages that are now full, causal attention over the
+        slot's whole context (batch_cache.py:112-145)."""
+        bsz, seq_len = query_states.shape[0], query_states.shape[2]
+        slot = int(batch_idx.item())
+        offset = int(self.kv_offset[layer_idx][slot].item())
+        total = offset + seq_len
+        if total > self.pages_per_slot * PAGE:
+            raise ValueError(f"sequence of {total} tokens exceeds max_seq_len")
+        P, Hkv, D = self.pages_per_slot, self.num_key_value_heads, self.head_dim
+        view = self.kv_cache[layer_idx].view(self.max_batch_size, P, 2, PAGE, Hkv, D)
+        tok = torch.arange(offset, total, device=self.device)
+        view[slot, tok // PAGE, 0, tok % PAGE] = key_states[0].transpose(0, 1)
+        view[slot, tok // PAGE, 1, tok % PAGE] = value_states[0].transpose(0, 1)
+        self.kv_offset[layer_idx][slot] += seq_len
+        n_pages = (total + PAGE - 1) // PAGE
+        idx = (slot * P + torch.arange(n_pages, device=self.device, dtype=torch.int32)).contiguous()
+        ptr = torch.tensor([0, n_pages], dtype=torch.int32, device=self.device)
+        last = torch.tensor([total - (n_pages - 1) * PAGE], dtype=torch.int32, device=self.device)
+        ops.build_kbar(self.kv_cache[layer_idx], self.kbar[layer_idx][slot:slot + 1], idx, ptr, last)
+        k_all = view[slot, :n_pages, 0].reshape(n_pages * PAGE, Hkv, D)[:total].transpose(0, 1)  # [Hkv, total, D]
+        v_all = view[slot, :n_pages, 1].reshape(n_pages * PAGE, Hkv, D)[:total].transpose(0, 1)
+        G = self.num_attention_heads // Hkv
+        q = query_states[0]                                                                    # [Hq, s, D]
+        pos_q = torch.arange(offset, total, device=self.device)[:, None]
+        mask = torch.arange(total, device=self.device)[None, :] <= pos_q                       # causal with history
+        o = F.scaled_dot_product_attention(q[None], k_all.repeat_interleave(G, dim=0)[None],
+                                           v_all.repeat_interleave(G, dim=0)[None], attn_mask=mask[None, None],
+                                           scale=1.0 / math.sqrt(D))[0]                       # [Hq, s, D]
+        return o.transpose(0, 1).reshape(bsz, seq_len, self.hidden_size)

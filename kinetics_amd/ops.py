@@ -316,6 +316,33 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
     return out
 
 
+def build_slot_page_table(seq_lens, pages_per_slot, page_size, page_indices, page_indptr, last_page_len, slot_ids=None) -> None:
+    """CSR page table for a cache where slot ``s`` owns pages
+    ``s*pages_per_slot ...`` (the paged stand-in for LiteSys' contiguous
+    per-slot caches, LiteSys/litesys/attention/batch_cache.py:40-62).  Fills the
+    three output tensors in place from the token counts ``seq_lens``."""
+    _require(seq_lens, "seq_lens", torch.int32, 1)
+    dev = seq_lens.device
+    batch = seq_lens.numel()
+    _require(page_indices, "page_indices", torch.int32, 1, dev)
+    _require(page_indptr, "page_indptr", torch.int32, 1, dev)
+    _require(last_page_len, "last_page_len", torch.int32, 1, dev)
+    if page_indptr.numel() != batch + 1 or last_page_len.numel() != batch:
+        raise ValueError("page_indptr needs batch+1 entries and last_page_len batch entries")
+    if page_indices.numel() < batch * pages_per_slot:
+        raise ValueError(f"page_indices needs room for batch*pages_per_slot = {batch * pages_per_slot} entries")
+    if slot_ids is not None:
+        _require(slot_ids, "slot_ids", torch.int32, 1, dev)
+        if slot_ids.numel() != batch:
+            raise ValueError("slot_ids must have one entry per sequence")
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(
+            lib.kin_build_slot_page_table(_ptr(slot_ids), _ptr(seq_lens), batch, int(pages_per_slot), int(page_size),
+                                          _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), _stream(dev))
+        )
+
+
 def check_page_table(page_indices, page_indptr, last_page_len, page_size, num_pages) -> None:
     """Synchronous device-side validation of a page table (debugging aid);
     raises KineticsError on an invalid entry."""

@@ -1,0 +1,140 @@
+"""The LiteSys-style KV manager (kinetics_amd/batch_cache.py) against the
+oracle and against a contiguous-cache restatement of LiteSys' flow
+(LiteSys/litesys/attention/batch_cache.py:86-168)."""
+import math
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import blocktopk_oracle as O
+from tests import problems as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+D, PS = P.HEAD_DIM, P.PAGE_SIZE
+
+
+def bf(x):
+    return x.to(torch.bfloat16)
+
+
+def make_manager(**sparse):
+    from kinetics_amd.batch_cache import PagedBatchKVManager
+
+    cfg = SimpleNamespace(num_attention_heads=4, num_key_value_heads=2, head_dim=D, hidden_size=512, num_hidden_layers=2)
+    return PagedBatchKVManager(cfg, max_batch_size=6, max_seq_len=PS * 24, device=DEV, dtype=torch.bfloat16, **sparse)
+
+
+def test_rejects_what_it_does_not_implement():
+    from kinetics_amd.batch_cache import PagedBatchKVManager
+
+    cfg = SimpleNamespace(num_attention_heads=4, num_key_value_heads=2, head_dim=D, hidden_size=512, num_hidden_layers=1)
+    with pytest.raises(NotImplementedError):
+        PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_topk=8, attn_local=4)
+    with pytest.raises(AssertionError):
+        PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_block_topk=2)          # LiteSys: local required
+    with pytest.raises(NotImplementedError):
+        PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_block_topk=2, attn_local=4, attn_block_size=32)
+
+
+@pytest.mark.parametrize("sparse", [dict(), dict(attn_block_topk=3, attn_local=16)])
+def test_prefill_then_decode_like_litesys(sparse):
+    torch.manual_seed(5)
+    m = make_manager(**sparse)
+    L, Hq, Hkv = 2, 4, 2
+    hist = {}  # (layer, slot) -> (K [t, Hkv, D], V) float32 of the bf16 values fed so far
+
+    def feed(layer, slot, k, v):  # k, v: [Hkv, s, D] bf16
+        K, V = hist.get((layer, slot), (torch.zeros(0, Hkv, D), torch.zeros(0, Hkv, D)))
+        hist[(layer, slot)] = (torch.cat([K, k.float().cpu().transpose(0, 1)]), torch.cat([V, v.float().cpu().transpose(0, 1)]))
+
+    def dense_ref(layer, slot, q):  # q [Hq, s, D]; causal over history
+        K, V = hist[(layer, slot)]
+        s, total = q.shape[1], K.shape[0]
+        out = torch.zeros(Hq, s, D)
+        for hq in range(Hq):
+            h = hq // 2
+            logits = q[hq].float().cpu() @ K[:, h].T / math.sqrt(D)
+            pos = torch.arange(total - s, total)[:, None]
+            logits = logits.masked_fill(torch.arange(total)[None, :] > pos, float("-inf"))
+            out[hq] = torch.softmax(logits, -1) @ V[:, h]
+        return out
+
+    # ---- prefill three requests, one at a time, in two chunks for slot 5 (append to history)
+    for slot, lens in ((0, [PS * 7 + 5]), (2, [PS * 3]), (5, [PS * 2 + 1, PS * 6 + 9])):
+        for s in lens:
+            for layer in range(L):
+                q, k, v = bf(torch.randn(1, Hq, s, D, device=DEV)), bf(torch.randn(1, Hkv, s, D, device=DEV)), bf(torch.randn(1, Hkv, s, D, device=DEV))
+                feed(layer, slot, k[0], v[0])
+                out = m.compute_attention(q, k, v, layer, torch.tensor([slot]))
+                assert out.shape == (1, s, Hq * D)
+                want = dense_ref(layer, slot, q[0]).transpose(0, 1).reshape(1, s, Hq * D)
+                assert torch.allclose(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
+    assert m.kv_offset[0].cpu().tolist() == [PS * 7 + 5, 0, PS * 3, 0, 0, PS * 8 + 10]
+
+    def decode_round(batch_slots):
+        for layer in range(L):
+            bsz = len(batch_slots)
+            q, k, v = bf(torch.randn(bsz, Hq, 1, D, device=DEV)), bf(torch.randn(bsz, Hkv, 1, D, device=DEV)), bf(torch.randn(bsz, Hkv, 1, D, device=DEV))
+            kv_before, kbar_before = P.from_torch(m.kv_cache[layer]), P.from_torch(m.kbar[layer])
+            off_before = m.kv_offset[layer].cpu().numpy().copy()
+            out = m.compute_attention(q, k, v, layer, torch.tensor(batch_slots))
+            torch.cuda.synchronize()
+            assert out.shape == (bsz, 1, Hq * D)
+            for i, slot in enumerate(batch_slots):
+                feed(layer, slot, k[i], v[i])
+            # the paged cache holds exactly the history that was fed
+            view = m.kv_cache[layer].view(6, m.pages_per_slot, 2, PS, Hkv, D)
+            for slot in batch_slots:
+                K, V = hist[(layer, slot)]
+                t = K.shape[0]
+                assert m.kv_offset[layer][slot].item() == t == off_before[slot] + 1
+                got_k = view[slot, :, 0].reshape(-1, Hkv, D)[:t].float().cpu()
+                assert torch.equal(got_k, K)
+            # oracle on the manager's own state before the call
+            lens = np.zeros(6, dtype=np.int64)
+            lens[batch_slots] = off_before[batch_slots] + 1
+            n_pages = (lens + PS - 1) // PS
+            indptr = np.zeros(7, dtype=np.int32)
+            indptr[1:] = np.cumsum(n_pages)
+            idx = np.concatenate([s * m.pages_per_slot + np.arange(n_pages[s]) for s in range(6)]).astype(np.int32)
+            last = np.where(lens > 0, lens - (n_pages - 1) * PS, 1).astype(np.int32)
+            assert np.array_equal(m.page_indptr.cpu().numpy(), indptr)
+            assert np.array_equal(m.page_indices.cpu().numpy()[: len(idx)], idx)
+            assert np.array_equal(m.last_page_len.cpu().numpy(), last)
+            qf = np.zeros((6, Hq, D), dtype=np.uint16)
+            kf = np.zeros((6, Hkv, D), dtype=np.uint16)
+            vf = np.zeros((6, Hkv, D), dtype=np.uint16)
+            qf[batch_slots], kf[batch_slots], vf[batch_slots] = P.from_torch(q[:, :, 0]), P.from_torch(k[:, :, 0]), P.from_torch(v[:, :, 0])
+            is_sparse = bool(sparse) and layer not in (0,)   # layer 0 stays dense (attn_layer_skip default)
+            if is_sparse:
+                res = O.decode_step(qf, kf, vf, kv_before, kbar_before, idx, indptr, last, sparse["attn_block_topk"])
+                want = res["out"]
+                # really sparse for the long sequences: fewer pages than the context has
+                assert res["sel_count"][batch_slots].max() == sparse["attn_block_topk"] + 1
+            else:
+                O.append_paged_kv(kf, vf, kv_before, kbar_before, idx, indptr, last)
+                want, _ = O.dense_paged_decode(qf, kv_before, idx, indptr, last)
+            assert np.array_equal(P.from_torch(m.kv_cache[layer]), kv_before)
+            assert np.array_equal(P.from_torch(m.kbar[layer]), kbar_before)
+            got = out.float().cpu().numpy().reshape(bsz, Hq, D)
+            err = np.abs(got - want[batch_slots])
+            assert np.all(err <= 2e-2 + 2e-2 * np.abs(want[batch_slots]))
+            if not is_sparse:  # dense layers also equal the contiguous-cache restatement
+                for i, slot in enumerate(batch_slots):
+                    ref = dense_ref(layer, slot, q[i])[:, 0]
+                    assert torch.allclose(torch.from_numpy(got[i]).float(), ref, rtol=2e-2, atol=2e-2)
+
+    for _ in range(12):           # crosses page boundaries (mean keys refreshed) for every slot
+        decode_round([0, 2, 5])
+    decode_round([5, 0])          # a subset, in another order
+    m.clear_cache(2)              # recycle slot 2
+    assert m.kv_offset[1][2].item() == 0
+    for layer in range(L):
+        hist.pop((layer, 2))
+        q, k, v = bf(torch.randn(1, Hq, 20, D, device=DEV)), bf(torch.randn(1, Hkv, 20, D, device=DEV)), bf(torch.randn(1, Hkv, 20, D, device=DEV))
+        feed(layer, 2, k[0], v[0])
+        m.compute_attention(q, k, v, layer, torch.tensor([2]))
+    decode_round([2, 5])
