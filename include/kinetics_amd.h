@@ -110,23 +110,33 @@ int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar,
  * (ref: benchmark/blocktopk_decoder.py:216-221) and, per KV head, LiteSys
  * blockwise_topk_sparsity (ref: LiteSys/litesys/attention/sparsity_utils.py:24-47).
  *
- * For sequence b and KV head h the candidates are the n_cand = n_pages-1 pages
- * before the last one.  score[n] = dot(mean_g q[b, h*G+g, :], kbar[b, n, h, :])
- * in fp32.  k_eff = min(topk, n_cand) pages are selected: descending score,
- * equal scores by ascending logical index (deterministic).  Outputs:
+ * The pages of sequence b split into n_local = min(local_pages, n_pages)
+ * trailing pages and n_sink = min(sink_pages, rest) leading pages, which are
+ * always attended, and the candidates in between (logical pages n_sink ..
+ * n_pages-n_local-1).  sink_pages = 0, local_pages = 1 is the reference's rule
+ * ("top-k plus the last page", blocktopk_decoder.py:220); larger values give the
+ * page-aligned form of LiteSys' sink tokens and local window
+ * (sparsity_utils.py:24-35).  score[p] = dot(mean_g q[b, h*G+g, :],
+ * kbar[b, p, h, :]) in fp32.  k_eff = min(topk, n_cand) candidates are selected:
+ * descending score, equal scores by ascending logical index (deterministic).
+ * Outputs, with n = k_eff + n_sink + n_local:
  *   sel_pages[b,h,0:k_eff]   physical ids of the selected pages, in that order
- *   sel_pages[b,h,k_eff]     the sequence's last page (always attended)
- *   sel_pages[b,h,k_eff+1:]  -1
- *   sel_count[b,h]           k_eff + 1   (0 for an empty page list)
- *   sel_logical[b,h,0:k_eff] logical page indices (== torch.topk(...).indices),
- *                            stride topk; may be NULL
- *   scores_out[b,h,0:n_cand] fp32 scores, stride kbar_pages; may be NULL
- *                            (debug/parity only: costs an HBM write)
- * Requires 1 <= topk < sel_stride, topk <= 2048, n_cand <= kbar_pages <= 16384.
+ *   sel_pages[b,h,k_eff:n]   the sink pages, then the local pages (the open
+ *                            page last)
+ *   sel_pages[b,h,n:]        -1
+ *   sel_count[b,h]           n   (0 for an empty page list)
+ *   sel_logical[b,h,0:k_eff] logical page indices (== n_sink +
+ *                            torch.topk(...).indices), stride topk; may be NULL
+ *   scores_out[b,h,p]        fp32 score of candidate page p (logical index),
+ *                            stride kbar_pages; may be NULL (debug/parity only:
+ *                            costs an HBM write)
+ * Requires topk >= 1, 0 <= sink_pages <= 64, 1 <= local_pages <= 64,
+ * sel_stride >= topk + sink_pages + local_pages, topk <= 2048,
+ * kbar_pages <= 16384.
  */
 int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
                          const int32_t* page_indices, const int32_t* page_indptr,
-                         int topk,
+                         int topk, int sink_pages, int local_pages,
                          int32_t* sel_pages, int32_t* sel_count,
                          int32_t* sel_logical, float* scores_out,
                          int batch, int num_q_heads, int num_kv_heads, int head_dim,
@@ -198,7 +208,8 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  * leaves the chip and phases of different sequences overlap.
  *
  * k and v may both be NULL (no append).  sel_pages / sel_count are optional
- * outputs (both NULL, or both given with 1 <= topk < sel_stride); lse is
+ * outputs (both NULL, or both given with sel_stride >= topk + sink_pages +
+ * local_pages); sink_pages / local_pages as in kin_block_score_topk; lse is
  * optional.  Needs no workspace.  Intended for batch * num_kv_heads large
  * enough to fill the GPU (>= ~1000 lists); for small batches the three-call
  * path with split-K is faster.
@@ -207,6 +218,7 @@ int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const ki
                               kin_bf16_t* kv_cache, kin_bf16_t* kbar,
                               const int32_t* page_indices, const int32_t* page_indptr,
                               const int32_t* last_page_len, int topk,
+                              int sink_pages, int local_pages,
                               int32_t* sel_pages, int32_t* sel_count,
                               kin_bf16_t* out, float* lse,
                               int batch, int num_q_heads, int num_kv_heads,

@@ -13,11 +13,14 @@ formulation with page-aligned blocks, without touching the rest of the context.
 Supported configurations (anything else raises at construction):
   * no sparsity arguments                      -> dense paged decode
   * ``attn_block_topk=k`` (+ ``attn_local``)    -> block top-k with block size 16
-Differences from LiteSys, by design of the paged layout: blocks are page
-aligned (LiteSys starts them after 4 hard-wired "sink" tokens,
-sparsity_utils.py:24,240), and the always-attended local window is the open page
-(1..16 newest tokens) rather than ``attn_local`` tokens.  ``attn_layer_skip``
-(default ``[0]``: layer 0 stays dense, sparsity_utils.py:211) is honoured.
+Differences from LiteSys, by design of the paged layout: everything is page
+aligned.  LiteSys always attends 4 hard-wired "sink" tokens and the newest
+``attn_local`` tokens and starts its blocks after the sink
+(sparsity_utils.py:24-35,240); here the first page (16 tokens, a superset of the
+sink) and the last ``ceil(attn_local/16) + 1`` pages (a superset of the local
+window) are pinned into every list and the blocks are the pages in between.
+``attn_layer_skip`` (default ``[0]``: layer 0 stays dense, sparsity_utils.py:211)
+is honoured.
 Prefill is not the accelerated path: it writes pages with PyTorch indexing and
 runs PyTorch's scaled_dot_product_attention (LiteSys calls flashinfer there,
 batch_cache.py:112-145).
@@ -68,6 +71,8 @@ class PagedBatchKVManager:
         elif kwargs.get("attn_local") is not None:
             raise NotImplementedError("local-window-only sparsity is not implemented")
         self.layer_skip = list(kwargs.get("attn_layer_skip", [0]))
+        self.sink_pages = 1
+        self.local_pages = (int(kwargs["attn_local"]) + PAGE - 1) // PAGE + 1 if self.block_topk is not None else 1
 
         B, Hq, Hkv, D = max_batch_size, self.num_attention_heads, self.num_key_value_heads, self.head_dim
         self.pages_per_slot = P = (max_seq_len + PAGE - 1) // PAGE
@@ -85,10 +90,10 @@ class PagedBatchKVManager:
         self._v = torch.zeros(B, Hkv, D, dtype=dtype, device=dev)
         self._out = torch.zeros(B, Hq, D, dtype=dtype, device=dev)
         k = self.block_topk or 1
-        self._sel = torch.full((B, Hkv, k + 1), -1, dtype=torch.int32, device=dev)
+        self._sel = torch.full((B, Hkv, k + self.sink_pages + self.local_pages), -1, dtype=torch.int32, device=dev)
         self._cnt = torch.zeros(B, Hkv, dtype=torch.int32, device=dev)
         self._fused = ops.prefer_fused_step(B, Hkv, P, k)
-        ws = max(ops.decode_workspace_bytes(B, Hq, Hkv, P), ops.decode_workspace_bytes(B, Hq, Hkv, k + 1), 16)
+        ws = max(ops.decode_workspace_bytes(B, Hq, Hkv, P), ops.decode_workspace_bytes(B, Hq, Hkv, self._sel.shape[2]), 16)
         self._ws = torch.empty(ws, dtype=torch.uint8, device=dev)
 
     # ------------------------------------------------------------------ LiteSys interface
@@ -123,11 +128,13 @@ class PagedBatchKVManager:
         sparse = self.block_topk is not None and layer_idx not in self.layer_skip
         if sparse and self._fused:
             ops.blocktopk_decode_step(self._q, self._k, self._v, kv, kbar, self.page_indices, self.page_indptr,
-                                      self.last_page_len, self.block_topk, out=self._out)
+                                      self.last_page_len, self.block_topk, out=self._out, sink_pages=self.sink_pages,
+                                      local_pages=self.local_pages)
         else:
             ops.append_paged_kv(self._k, self._v, kv, kbar, self.page_indices, self.page_indptr, self.last_page_len)
             if sparse:
-                ops.block_score_topk(self._q, kbar, self.page_indices, self.page_indptr, self.block_topk, self._sel, self._cnt)
+                ops.block_score_topk(self._q, kbar, self.page_indices, self.page_indptr, self.block_topk, self._sel, self._cnt,
+                                     sink_pages=self.sink_pages, local_pages=self.local_pages)
                 ops.sparse_paged_decode(self._q, kv, self._sel, self._cnt, self.last_page_len, out=self._out, workspace=self._ws)
             else:
                 ops.dense_paged_decode(self._q, kv, self.page_indices, self.page_indptr, self.last_page_len,

@@ -14,6 +14,7 @@ constexpr int kRowBytes = kHeadDim * 2;
 constexpr int kMaxGroup = 8;     // largest supported num_q_heads / num_kv_heads
 constexpr int kMaxTopk = 2048;
 constexpr int kMaxCandidates = 16384;
+constexpr int kMaxFixedPages = 64;  // most sink / local pages that can be pinned into every list
 
 // Cache-policy bits for buffer loads of read-once data (K/V pages, mean keys):
 // the non-temporal hint keeps streams from displacing each other in L2/MALL and

@@ -15,11 +15,11 @@ struct ScoreTopkParams {
   int32_t* sel_logical;  // may be null
   float* scores_out;     // may be null
   int num_q_heads, num_kv_heads, group;
-  int kbar_pages, sel_stride, topk;
+  int kbar_pages, sel_stride, topk, sink_pages, local_pages;
   int sort_cap;
 };
 
-// Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap] | int32 sel[topk + 1]
+// Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap] | int32 sel[topk + sink + local]
 __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x;
@@ -41,26 +41,28 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
   a.q_bh = p.q + ((int64_t)b * p.num_q_heads + (int64_t)h * p.group) * kHeadDim;
   a.G = p.group;
   a.row_stride_b = p.num_kv_heads * kRowBytes;
-  a.kb = reinterpret_cast<const char*>(p.kbar) + ((int64_t)b * p.kbar_pages * p.num_kv_heads + h) * kRowBytes;
   a.n_pages = n_pages;
-  a.n_cand = min(n_pages - 1, p.kbar_pages);
+  split_pages(n_pages, p.sink_pages, p.local_pages, p.kbar_pages, a.n_sink, a.n_cand, a.n_local);
+  a.kb = reinterpret_cast<const char*>(p.kbar) +
+         (((int64_t)b * p.kbar_pages + a.n_sink) * p.num_kv_heads + h) * kRowBytes;
   a.topk = p.topk;
   a.table = p.page_indices + ps;
   a.sel_logical = p.sel_logical ? p.sel_logical + (int64_t)item * p.topk : nullptr;
-  a.scores_out = p.scores_out ? p.scores_out + (int64_t)item * p.kbar_pages : nullptr;
+  a.scores_out = p.scores_out ? p.scores_out + (int64_t)item * p.kbar_pages + a.n_sink : nullptr;
   a.keys = reinterpret_cast<uint32_t*>(smem);
   a.sortbuf = reinterpret_cast<unsigned long long*>(smem + (size_t)((p.kbar_pages + 3) & ~3) * 4);
   a.sort_cap = p.sort_cap;
-  const int k_eff = score_select(a, sel_lds);
+  const int n_list = score_select(a, sel_lds);
 
-  for (int i = tid; i < p.sel_stride; i += kThreads) sel[i] = (i <= k_eff) ? sel_lds[i] : -1;
-  if (tid == 0) p.sel_count[item] = k_eff + 1;
+  for (int i = tid; i < p.sel_stride; i += kThreads) sel[i] = (i < n_list) ? sel_lds[i] : -1;
+  if (tid == 0) p.sel_count[item] = n_list;
 }
 
 }  // namespace kin
 
 extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar, const int32_t* page_indices,
-                                    const int32_t* page_indptr, int topk, int32_t* sel_pages, int32_t* sel_count,
+                                    const int32_t* page_indptr, int topk, int sink_pages, int local_pages,
+                                    int32_t* sel_pages, int32_t* sel_count,
                                     int32_t* sel_logical, float* scores_out, int batch, int num_q_heads,
                                     int num_kv_heads, int head_dim, int kbar_pages, int sel_stride,
                                     kin_stream_t stream) {
@@ -71,9 +73,12 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
   int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, kPageSize);
   if (st) return st;
   if (topk < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: topk=%d must be >= 1", fn, topk);
-  if (sel_stride <= topk)
-    return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must exceed topk=%d (room for the last page)", fn, sel_stride,
-                topk);
+  if (sink_pages < 0 || sink_pages > kMaxFixedPages || local_pages < 1 || local_pages > kMaxFixedPages)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: sink_pages=%d must be in [0, %d] and local_pages=%d in [1, %d]", fn, sink_pages,
+                kMaxFixedPages, local_pages, kMaxFixedPages);
+  if (sel_stride < topk + sink_pages + local_pages)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must be at least topk + sink_pages + local_pages = %d", fn,
+                sel_stride, topk + sink_pages + local_pages);
   if (kbar_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: kbar_pages=%d must be >= 1", fn, kbar_pages);
   if (topk > kMaxTopk) return fail(KIN_ERR_UNSUPPORTED, "%s: topk=%d exceeds the limit %d", fn, topk, kMaxTopk);
   if (kbar_pages > kMaxCandidates)
@@ -96,8 +101,10 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
   p.kbar_pages = kbar_pages;
   p.sel_stride = sel_stride;
   p.topk = topk;
+  p.sink_pages = sink_pages;
+  p.local_pages = local_pages;
   p.sort_cap = select_sort_cap(topk, kbar_pages);
-  const size_t lds = select_lds_bytes(kbar_pages, p.sort_cap) + (size_t)(topk + 1) * 4;
+  const size_t lds = select_lds_bytes(kbar_pages, p.sort_cap) + (size_t)(topk + sink_pages + local_pages) * 4;
   const int64_t items = (int64_t)batch * num_kv_heads;
   if (items > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   if (lds > 48 * 1024) {

@@ -34,14 +34,16 @@ constexpr int kRankSortMax = 512;   // up to here winners are ordered by countin
 struct SelectArgs {
   const uint16_t* q_bh;       // the group's G query rows
   int G;
-  const char* kb;             // first representative key of (b, h)
+  const char* kb;             // representative key of the first candidate of (b, h)
   int row_stride_b;           // bytes between consecutive logical pages
   int n_pages;                // pages of the sequence (>= 1)
-  int n_cand;                 // candidates: min(n_pages - 1, capacity)
+  int n_sink;                 // leading pages that are always attended (not candidates)
+  int n_cand;                 // candidates: logical pages n_sink .. n_sink + n_cand - 1
+  int n_local;                // trailing pages that are always attended (>= 1: the open page)
   int topk;
   const int32_t* table;       // the sequence's page table (logical -> physical)
   int32_t* sel_logical;       // HBM, topk entries, or null
-  float* scores_out;          // HBM, n_cand entries, or null
+  float* scores_out;          // HBM, entry n = score of candidate n, or null
   uint32_t* keys;             // LDS, >= n_cand entries
   unsigned long long* sortbuf;  // LDS, sort_cap entries
   int sort_cap;               // power of two >= min(topk, capacity)
@@ -58,10 +60,25 @@ __host__ __device__ inline int select_sort_cap(int topk, int kbar_pages) {
   return cap;
 }
 
-// Writes the ordered physical ids of the k_eff winners to sel_lds[0 .. k_eff)
-// and the sequence's last page to sel_lds[k_eff] (LDS, >= topk + 1 entries);
-// returns k_eff.  Ends with a workgroup barrier: sel_lds is visible to every
-// thread and keys / sortbuf are free for reuse.
+// Splits a sequence's pages into always-attended leading ("sink") pages,
+// candidates and always-attended trailing ("local") pages; the final local page
+// is the open one.  kbar_pages bounds the logical pages that have a mean key.
+__host__ __device__ inline void split_pages(int n_pages, int sink_pages, int local_pages, int kbar_pages, int& n_sink,
+                                            int& n_cand, int& n_local) {
+  n_local = local_pages < n_pages ? local_pages : n_pages;
+  const int rest = n_pages - n_local;
+  n_sink = sink_pages < rest ? sink_pages : rest;
+  const int cap = kbar_pages - n_sink;
+  n_cand = rest - n_sink;
+  if (n_cand > cap) n_cand = cap;
+  if (n_cand < 0) n_cand = 0;
+}
+
+// Writes the page list to sel_lds (LDS, >= topk + n_sink + n_local entries):
+// the ordered physical ids of the k_eff winners, then the sink pages, then the
+// local pages (the open page last).  Returns the list length.  Ends with a
+// workgroup barrier: sel_lds is visible to every thread and keys / sortbuf are
+// free for reuse.
 __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_lds) {
   __shared__ uint32_t hist[256];
   __shared__ uint32_t wave_tot[4];
@@ -234,8 +251,8 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
 #pragma unroll 8
       for (int j = 0; j < k_eff; ++j) rank += (sortbuf[j] > mine) ? 1 : 0;
       const uint32_t logical = 0xffffffffu - (uint32_t)(mine & 0xffffffffull);
-      sel_lds[rank] = table[logical];
-      if (a.sel_logical) a.sel_logical[rank] = (int32_t)logical;
+      sel_lds[rank] = table[a.n_sink + logical];
+      if (a.sel_logical) a.sel_logical[rank] = (int32_t)(a.n_sink + logical);
     }
   } else {
     // Large k: bitonic sort, descending, over sort_cap (power of two) 64-bit
@@ -257,13 +274,14 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
     }
     for (int i = tid; i < k_eff; i += kThreads) {
       const uint32_t logical = 0xffffffffu - (uint32_t)(sortbuf[i] & 0xffffffffull);
-      sel_lds[i] = table[logical];
-      if (a.sel_logical) a.sel_logical[i] = (int32_t)logical;
+      sel_lds[i] = table[a.n_sink + logical];
+      if (a.sel_logical) a.sel_logical[i] = (int32_t)(a.n_sink + logical);
     }
   }
-  if (tid == 0) sel_lds[k_eff] = table[n_pages - 1];
+  for (int i = tid; i < a.n_sink + a.n_local; i += kThreads)
+    sel_lds[k_eff + i] = (i < a.n_sink) ? table[i] : table[n_pages - a.n_local + (i - a.n_sink)];
   __syncthreads();
-  return k_eff;
+  return k_eff + a.n_sink + a.n_local;
 }
 
 }  // namespace kin

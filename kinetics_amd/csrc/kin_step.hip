@@ -27,7 +27,7 @@ struct StepParams {
   uint16_t* out;
   float* lse;  // optional
   int num_q_heads, num_kv_heads, group;
-  int kbar_pages, sel_stride, topk, sort_cap;
+  int kbar_pages, sel_stride, topk, sink_pages, local_pages, sort_cap;
   int region0_bytes;  // LDS: max(attend staging, select scratch); the page list follows it
   int64_t num_pages;
   float scale_log2;
@@ -97,9 +97,10 @@ __global__ __launch_bounds__(256, 2) void blocktopk_step_kernel(StepParams p) {
   s.q_bh = p.q + hq0 * kHeadDim;
   s.G = G;
   s.row_stride_b = p.num_kv_heads * kRowBytes;
-  s.kb = reinterpret_cast<const char*>(p.kbar) + ((int64_t)b * p.kbar_pages * p.num_kv_heads + h) * kRowBytes;
   s.n_pages = n_pages;
-  s.n_cand = min(n_pages - 1, p.kbar_pages);
+  split_pages(n_pages, p.sink_pages, p.local_pages, p.kbar_pages, s.n_sink, s.n_cand, s.n_local);
+  s.kb = reinterpret_cast<const char*>(p.kbar) +
+         (((int64_t)b * p.kbar_pages + s.n_sink) * p.num_kv_heads + h) * kRowBytes;
   s.topk = p.topk;
   s.table = p.page_indices + ps;
   s.sel_logical = nullptr;
@@ -107,8 +108,7 @@ __global__ __launch_bounds__(256, 2) void blocktopk_step_kernel(StepParams p) {
   s.keys = reinterpret_cast<uint32_t*>(smem);
   s.sortbuf = reinterpret_cast<unsigned long long*>(smem + (size_t)((p.kbar_pages + 3) & ~3) * 4);
   s.sort_cap = p.sort_cap;
-  const int k_eff = score_select(s, sel_lds);
-  const int n = k_eff + 1;
+  const int n = score_select(s, sel_lds);
   if (p.sel_pages) {
     int32_t* sel = p.sel_pages + (int64_t)item * p.sel_stride;
     for (int i = tid; i < p.sel_stride; i += 256) sel[i] = (i < n) ? sel_lds[i] : -1;
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256, 2) void blocktopk_step_kernel(StepParams p) {
 extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
                                          kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
                                          const int32_t* page_indptr, const int32_t* last_page_len, int topk,
-                                         int32_t* sel_pages, int32_t* sel_count, kin_bf16_t* out, float* lse,
+                                         int sink_pages, int local_pages, int32_t* sel_pages, int32_t* sel_count, kin_bf16_t* out, float* lse,
                                          int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
                                          int64_t num_pages, int kbar_pages, int sel_stride, float sm_scale,
                                          kin_stream_t stream) {
@@ -157,9 +157,12 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
   if (num_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_pages=%lld must be >= 1", fn, (long long)num_pages);
   if (topk < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: topk=%d must be >= 1", fn, topk);
   if (kbar_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: kbar_pages=%d must be >= 1", fn, kbar_pages);
-  if (sel_pages && sel_stride <= topk)
-    return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must exceed topk=%d (room for the last page)", fn, sel_stride,
-                topk);
+  if (sink_pages < 0 || sink_pages > kMaxFixedPages || local_pages < 1 || local_pages > kMaxFixedPages)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: sink_pages=%d must be in [0, %d] and local_pages=%d in [1, %d]", fn, sink_pages,
+                kMaxFixedPages, local_pages, kMaxFixedPages);
+  if (sel_pages && sel_stride < topk + sink_pages + local_pages)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must be at least topk + sink_pages + local_pages = %d", fn,
+                sel_stride, topk + sink_pages + local_pages);
   if (sel_pages && !sel_count) return fail(KIN_ERR_NULL_POINTER, "%s: sel_pages given without sel_count", fn);
   if (topk > kMaxTopk) return fail(KIN_ERR_UNSUPPORTED, "%s: topk=%d exceeds the limit %d", fn, topk, kMaxTopk);
   if (kbar_pages > kMaxCandidates)
@@ -188,6 +191,8 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
   p.kbar_pages = kbar_pages;
   p.sel_stride = sel_stride;
   p.topk = topk;
+  p.sink_pages = sink_pages;
+  p.local_pages = local_pages;
   p.sort_cap = select_sort_cap(topk, kbar_pages);
   const size_t sel_scratch = select_lds_bytes(kbar_pages, p.sort_cap);
   size_t region0 = sel_scratch > (size_t)kAttendLdsBytes ? sel_scratch : (size_t)kAttendLdsBytes;
@@ -196,7 +201,7 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
   p.num_pages = num_pages;
   const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
   p.scale_log2 = scale * 1.4426950408889634f;
-  const size_t lds = region0 + (size_t)(topk + 1) * 4;
+  const size_t lds = region0 + (size_t)(topk + sink_pages + local_pages) * 4;
   const int64_t items = (int64_t)batch * num_kv_heads;
   if (items > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   hipStream_t s = static_cast<hipStream_t>(stream);

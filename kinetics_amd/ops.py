@@ -135,12 +135,15 @@ def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len) -> None
 # ---------------------------------------------------------------------------
 
 
-def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count, sel_logical=None, scores_out=None) -> None:
+def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count, sel_logical=None, scores_out=None,
+                     sink_pages: int = 0, local_pages: int = 1) -> None:
     """Score every candidate page with the group-mean query and write the
     top-``topk`` pages plus the last page into ``sel_pages`` / ``sel_count``
     (in place: fixed buffers, as the reference registers with its decode
     wrapper, benchmark/blocktopk_decoder.py:143,156-159).  Stands in for
-    lines 216-221 of that file."""
+    lines 216-221 of that file.  ``sink_pages`` leading and ``local_pages``
+    trailing pages are always attended and never candidates (0 and 1 give the
+    reference's "top-k plus the last page")."""
     _require(q, "q", torch.bfloat16, 3)
     dev = q.device
     batch, num_q_heads, head_dim = q.shape
@@ -165,8 +168,8 @@ def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_co
     with torch.cuda.device(dev):
         _lib.check(
             lib.kin_block_score_topk(
-                _ptr(q), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), int(topk), _ptr(sel_pages),
-                _ptr(sel_count), _ptr(sel_logical), _ptr(scores_out), batch, num_q_heads, num_kv_heads, head_dim,
+                _ptr(q), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), int(topk), int(sink_pages), int(local_pages),
+                _ptr(sel_pages), _ptr(sel_count), _ptr(sel_logical), _ptr(scores_out), batch, num_q_heads, num_kv_heads, head_dim,
                 kbar_pages, sel_stride, _stream(dev),
             )
         )
@@ -280,7 +283,8 @@ def prefer_fused_step(batch: int, num_kv_heads: int, max_pages_per_seq: int, top
 
 
 def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, out=None, lse=None,
-                          sel_pages=None, sel_count=None, sm_scale: float = 0.0):
+                          sel_pages=None, sel_count=None, sm_scale: float = 0.0, sink_pages: int = 0,
+                          local_pages: int = 1):
     """append -> score -> select -> attend in one launch: lines 209-225 of the
     reference layer's forward (benchmark/blocktopk_decoder.py) as a single
     kernel.  ``k``/``v`` may be None (no append); ``sel_pages``/``sel_count`` are
@@ -309,7 +313,8 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
         _lib.check(
             lib.kin_blocktopk_decode_step(
                 _ptr(q), _ptr(k), _ptr(v), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
-                _ptr(last_page_len), int(topk), _ptr(sel_pages), _ptr(sel_count), _ptr(out), _ptr(lse), batch, hq, hkv,
+                _ptr(last_page_len), int(topk), int(sink_pages), int(local_pages), _ptr(sel_pages), _ptr(sel_count), _ptr(out),
+                _ptr(lse), batch, hq, hkv,
                 d, ps, num_pages, kbar_pages, sel_stride, float(sm_scale), _stream(dev),
             )
         )
@@ -373,7 +378,7 @@ torch.library.define(
 torch.library.define(
     "kinetics::block_score_topk",
     "(Tensor q, Tensor kbar, Tensor page_indices, Tensor page_indptr, int topk, Tensor(a!) sel_pages, "
-    "Tensor(b!) sel_count) -> ()",
+    "Tensor(b!) sel_count, int sink_pages=0, int local_pages=1) -> ()",
 )
 torch.library.define(
     "kinetics::sparse_paged_decode",
@@ -390,18 +395,22 @@ torch.library.define(
 torch.library.define(
     "kinetics::blocktopk_decode_step",
     "(Tensor q, Tensor k, Tensor v, Tensor(a!) kv_cache, Tensor(b!) kbar, Tensor page_indices, Tensor page_indptr, "
-    "Tensor last_page_len, int topk, Tensor(c!)? sel_pages, Tensor(d!)? sel_count, float sm_scale) -> Tensor",
+    "Tensor last_page_len, int topk, Tensor(c!)? sel_pages, Tensor(d!)? sel_count, float sm_scale, "
+    "int sink_pages=0, int local_pages=1) -> Tensor",
 )
 
 
 @torch.library.impl("kinetics::blocktopk_decode_step", "cuda")
-def _step_impl(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sm_scale):
+def _step_impl(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sm_scale,
+               sink_pages=0, local_pages=1):
     return blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk,
-                                 sel_pages=sel_pages, sel_count=sel_count, sm_scale=sm_scale)
+                                 sel_pages=sel_pages, sel_count=sel_count, sm_scale=sm_scale, sink_pages=sink_pages,
+                                 local_pages=local_pages)
 
 
 @torch.library.register_fake("kinetics::blocktopk_decode_step")
-def _step_fake(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sm_scale):
+def _step_fake(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sm_scale,
+               sink_pages=0, local_pages=1):
     return torch.empty_like(q)
 
 
@@ -416,12 +425,13 @@ def _append_fake(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len)
 
 
 @torch.library.impl("kinetics::block_score_topk", "cuda")
-def _select_impl(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count):
-    block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count)
+def _select_impl(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count, sink_pages=0, local_pages=1):
+    block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count, sink_pages=sink_pages,
+                     local_pages=local_pages)
 
 
 @torch.library.register_fake("kinetics::block_score_topk")
-def _select_fake(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count):
+def _select_fake(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count, sink_pages=0, local_pages=1):
     return None
 
 

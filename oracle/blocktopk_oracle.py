@@ -141,9 +141,22 @@ def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len):
 # ---------------------------------------------------------------------------
 
 
-def block_scores(q, kbar, page_indptr):
-    """score[b][h][n] = mean_g q[b, h*G+g, :] . kbar[b, n, h, :] in float64, over
-    the n_cand = n_pages-1 candidate pages.  Returns a list (b) of lists (h) of
+def split_pages(n_pages, sink_pages, local_pages, kbar_pages):
+    """(n_sink, n_cand, n_local): trailing ``local_pages`` pages (at least the
+    open page) and leading ``sink_pages`` pages are always attended; the pages in
+    between are the candidates.  sink 0 / local 1 is the reference's rule
+    (benchmark/blocktopk_decoder.py:220); larger values are the page-aligned form
+    of LiteSys' sink tokens and local window (sparsity_utils.py:24-35)."""
+    n_local = min(local_pages, n_pages)
+    rest = n_pages - n_local
+    n_sink = min(sink_pages, rest)
+    n_cand = max(0, min(rest - n_sink, kbar_pages - n_sink))
+    return n_sink, n_cand, n_local
+
+
+def block_scores(q, kbar, page_indptr, sink_pages=0, local_pages=1):
+    """score[b][h][n] = mean_g q[b, h*G+g, :] . kbar[b, n_sink + n, h, :] in
+    float64 over the candidate pages.  Returns a list (b) of lists (h) of
     float64 arrays."""
     B, Hq, D = q.shape
     Hkv = kbar.shape[2]
@@ -152,8 +165,8 @@ def block_scores(q, kbar, page_indptr):
     out = []
     for b in range(B):
         n_pages = int(page_indptr[b + 1]) - int(page_indptr[b])
-        n_cand = max(0, min(n_pages - 1, kbar.shape[1]))
-        kb = bf16_to_f32(kbar[b, :n_cand]).astype(np.float64)  # [n, Hkv, D]
+        n_sink, n_cand, _ = split_pages(max(n_pages, 0), sink_pages, local_pages, kbar.shape[1])
+        kb = bf16_to_f32(kbar[b, n_sink : n_sink + n_cand]).astype(np.float64)  # [n, Hkv, D]
         per_head = []
         for h in range(Hkv):
             per_q = np.einsum("gd,nd->gn", qf[b, h * G : (h + 1) * G], kb[:, h, :])  # [G, n]
@@ -175,13 +188,15 @@ def select_topk(scores: np.ndarray, k: int) -> np.ndarray:
     return order[: min(k, n)].astype(np.int64)
 
 
-def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_stride=None):
+def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_stride=None, sink_pages=0, local_pages=1):
     """Returns (sel_pages [B,Hkv,stride] int32 padded with -1, sel_count [B,Hkv],
-    sel_logical list[b][h] of index arrays, scores list[b][h])."""
+    sel_logical list[b][h] of logical page index arrays, scores list[b][h] over
+    the candidates).  List order: winners (descending score), sink pages, local
+    pages with the open page last."""
     B = q.shape[0]
     Hkv = kbar.shape[2]
-    stride = topk + 1 if sel_stride is None else sel_stride
-    scores = block_scores(q, kbar, page_indptr)
+    stride = topk + sink_pages + local_pages if sel_stride is None else sel_stride
+    scores = block_scores(q, kbar, page_indptr, sink_pages, local_pages)
     sel_pages = np.full((B, Hkv, stride), -1, dtype=np.int32)
     sel_count = np.zeros((B, Hkv), dtype=np.int32)
     sel_logical = []
@@ -192,10 +207,12 @@ def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_stride=None):
             if len(pages) == 0:
                 row.append(np.zeros(0, dtype=np.int64))
                 continue
-            idx = select_topk(scores[b][h], topk)
+            n_sink, _, n_local = split_pages(len(pages), sink_pages, local_pages, kbar.shape[1])
+            idx = n_sink + select_topk(scores[b][h], topk)
+            fixed = np.concatenate([pages[:n_sink], pages[len(pages) - n_local :]])
             sel_pages[b, h, : len(idx)] = pages[idx]
-            sel_pages[b, h, len(idx)] = pages[-1]
-            sel_count[b, h] = len(idx) + 1
+            sel_pages[b, h, len(idx) : len(idx) + len(fixed)] = fixed
+            sel_count[b, h] = len(idx) + len(fixed)
             row.append(idx)
         sel_logical.append(row)
     return sel_pages, sel_count, sel_logical, scores
@@ -282,11 +299,13 @@ def merge_partials(outs, lses):
 # ---------------------------------------------------------------------------
 
 
-def decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sm_scale=None):
+def decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sm_scale=None, sink_pages=0,
+                local_pages=1):
     """append -> score -> select -> attend.  Mutates kv_cache / kbar.  Returns
     dict(out, lse, sel_pages, sel_count, sel_logical, scores)."""
     append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len)
-    sel_pages, sel_count, sel_logical, scores = block_score_topk(q, kbar, page_indices, page_indptr, topk)
+    sel_pages, sel_count, sel_logical, scores = block_score_topk(q, kbar, page_indices, page_indptr, topk,
+                                                                 sink_pages=sink_pages, local_pages=local_pages)
     out, lse = sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, sm_scale)
     return dict(out=out, lse=lse, sel_pages=sel_pages, sel_count=sel_count, sel_logical=sel_logical, scores=scores)
 

@@ -58,8 +58,8 @@ def test_append_argument_errors(lib):
     assert append(lib, B=0) == _lib.KIN_OK  # nothing to do, nothing launched
 
 
-def select(lib, q=A, kbar=A, idx=A, ptr=A, topk=4, sel=A, cnt=A, B=2, Hq=4, Hkv=1, D=128, kp=64, stride=5):
-    return lib.kin_block_score_topk(q, kbar, idx, ptr, topk, sel, cnt, None, None, B, Hq, Hkv, D, kp, stride, None)
+def select(lib, q=A, kbar=A, idx=A, ptr=A, topk=4, sel=A, cnt=A, B=2, Hq=4, Hkv=1, D=128, kp=64, stride=5, sink=0, local=1):
+    return lib.kin_block_score_topk(q, kbar, idx, ptr, topk, sink, local, sel, cnt, None, None, B, Hq, Hkv, D, kp, stride, None)
 
 
 def test_select_argument_errors(lib):
@@ -67,6 +67,10 @@ def test_select_argument_errors(lib):
     assert select(lib, cnt=None) == _lib.KIN_ERR_NULL_POINTER
     assert select(lib, topk=0) == _lib.KIN_ERR_BAD_SHAPE
     assert select(lib, stride=4) == _lib.KIN_ERR_BAD_SHAPE          # no room for the last page
+    assert select(lib, stride=5, sink=1) == _lib.KIN_ERR_BAD_SHAPE  # nor for a sink page on top
+    assert select(lib, local=0) == _lib.KIN_ERR_BAD_SHAPE           # the open page is always attended
+    assert select(lib, sink=-1) == _lib.KIN_ERR_BAD_SHAPE
+    assert select(lib, stride=200, local=65) == _lib.KIN_ERR_BAD_SHAPE
     assert select(lib, Hq=5, Hkv=2) == _lib.KIN_ERR_BAD_SHAPE
     assert select(lib, Hq=16, Hkv=1) == _lib.KIN_ERR_UNSUPPORTED    # group 16 > 8
     assert select(lib, topk=4096, stride=4097) == _lib.KIN_ERR_UNSUPPORTED
@@ -110,7 +114,7 @@ def test_auto_splits_policy(lib):
 
 def test_python_wrapper_maps_status_to_exceptions():
     with pytest.raises(ValueError, match="KIN_ERR_BAD_SHAPE"):
-        _lib.check(_lib.load().kin_block_score_topk(A, A, A, A, 0, A, A, None, None, 2, 4, 1, 128, 64, 5, None))
+        _lib.check(_lib.load().kin_block_score_topk(A, A, A, A, 0, 0, 1, A, A, None, None, 2, 4, 1, 128, 64, 5, None))
     with pytest.raises(_lib.KineticsError, match="KIN_ERR_WORKSPACE"):
         _lib.check(sparse(_lib.load(), splits=3))
 

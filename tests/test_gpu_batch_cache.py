@@ -110,10 +110,13 @@ def test_prefill_then_decode_like_litesys(sparse):
             qf[batch_slots], kf[batch_slots], vf[batch_slots] = P.from_torch(q[:, :, 0]), P.from_torch(k[:, :, 0]), P.from_torch(v[:, :, 0])
             is_sparse = bool(sparse) and layer not in (0,)   # layer 0 stays dense (attn_layer_skip default)
             if is_sparse:
-                res = O.decode_step(qf, kf, vf, kv_before, kbar_before, idx, indptr, last, sparse["attn_block_topk"])
+                # first page (sink) and the last ceil(local/16)+1 pages are pinned, 3 blocks chosen in between
+                res = O.decode_step(qf, kf, vf, kv_before, kbar_before, idx, indptr, last, sparse["attn_block_topk"],
+                                    sink_pages=1, local_pages=2)
                 want = res["out"]
                 # really sparse for the long sequences: fewer pages than the context has
-                assert res["sel_count"][batch_slots].max() == sparse["attn_block_topk"] + 1
+                assert res["sel_count"][batch_slots].max() == sparse["attn_block_topk"] + 3
+                assert res["sel_count"][batch_slots].max() < n_pages[batch_slots].max()
             else:
                 O.append_paged_kv(kf, vf, kv_before, kbar_before, idx, indptr, last)
                 want, _ = O.dense_paged_decode(qf, kv_before, idx, indptr, last)

@@ -839,3 +839,41 @@ def test_decoder_layer_matches_fp32_reference(ops, dense):
     got = out.float().cpu()
     assert torch.allclose(got, want, rtol=5e-2, atol=5e-2), (got - want).abs().max()
     assert rms_norm(hidden, 1e-6, layer.input_layernorm_weight).dtype == torch.bfloat16
+
+
+@pytest.mark.parametrize("sink,local", [(1, 2), (2, 3), (0, 4), (3, 1)])
+@pytest.mark.parametrize("fused", [False, True])
+def test_sink_and_local_pages(ops, sink, local, fused):
+    """Pinned leading / trailing pages (LiteSys' sink and local window, page aligned)."""
+    topk = 6
+    lengths = [PS * 40 + 3, PS * 9, 1, 0, PS * 3 + 1, PS * 130 + 16, PS * (topk + sink + local) + 1, PS * 2 + 5]
+    pb = P.make_problem(950 + sink * 10 + local, lengths, num_kv_heads=2, group=4, topk=topk)
+    g = Gpu(pb)
+    stride = topk + sink + local
+    g.sel = torch.full((pb.B, pb.Hkv, stride), -7, dtype=torch.int32, device=DEV)
+    check_table(ops, g)
+    if fused:
+        out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, topk, sel_pages=g.sel,
+                                        sel_count=g.cnt, sink_pages=sink, local_pages=local)
+    else:
+        ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
+        ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, topk, g.sel, g.cnt, g.logical, g.scores, sink_pages=sink,
+                             local_pages=local)
+        out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last)
+    torch.cuda.synchronize()
+    kv, kbar = pb.kv_cache.copy(), pb.kbar.copy()
+    res = O.decode_step(pb.q, pb.k, pb.v, kv, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, topk,
+                        sink_pages=sink, local_pages=local)
+    assert np.array_equal(g.cnt.cpu().numpy(), res["sel_count"])
+    assert np.array_equal(g.sel.cpu().numpy(), res["sel_pages"])
+    assert_out_close(out, res["out"], f"sink={sink} local={local} fused={fused}")
+    if not fused:
+        logical, scores = g.logical.cpu().numpy(), g.scores.cpu().numpy()
+        for b in range(pb.B):
+            for h in range(pb.Hkv):
+                want = res["sel_logical"][b][h]
+                assert np.array_equal(logical[b, h, : len(want)], want)
+                ws = res["scores"][b][h]
+                n_pages = (lengths[b] + PS - 1) // PS
+                n_sink = O.split_pages(n_pages, sink, local, pb.kbar.shape[1])[0]
+                assert np.allclose(scores[b, h, n_sink : n_sink + len(ws)], ws, rtol=1e-5, atol=1e-5)

@@ -344,3 +344,39 @@ def test_torch_path_agrees_with_oracle():
                                            torch.from_numpy(pb.last_page_len.astype(np.int64)))
     dense_o, _ = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len)
     assert np.allclose(dense_t.float().numpy(), dense_o, rtol=2e-2, atol=2e-2)
+
+
+def test_sink_and_local_pages_are_pinned_not_candidates():
+    """Page-aligned form of LiteSys' sink tokens and local window
+    (sparsity_utils.py:24-35): pinned pages are always in the list, never scored."""
+    pb = P.make_problem(71, [PS * 20 + 7, PS * 4 + 2, PS * 2, 5, 0], topk=3)
+    sel, cnt, logical, scores = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, 3, sink_pages=2, local_pages=3)
+    assert sel.shape[2] == 3 + 2 + 3
+    # n_pages = 21, 5, 2, 1, 0 -> (sink, cand, local) = (2,16,3), (2,0,3), (0,0,2), (0,0,1), -
+    assert cnt[:, 0].tolist() == [3 + 5, 5, 2, 1, 0]
+    pages = O.seq_pages(pb.page_indices, pb.page_indptr, 0)
+    assert len(scores[0][0]) == 16
+    assert sel[0, 0, 3:8].tolist() == [pages[0], pages[1], pages[18], pages[19], pages[20]]
+    assert all(2 <= i < 18 for i in logical[0][0])
+    # scores are those of logical pages 2..17
+    full = O.block_scores(pb.q, pb.kbar, pb.page_indptr)[0][0]  # default split: candidates 0..19
+    assert np.allclose(scores[0][0], full[2:18])
+    # short sequences: everything pinned, in logical order, open page last
+    p1 = O.seq_pages(pb.page_indices, pb.page_indptr, 1)
+    assert sel[1, 0, :5].tolist() == p1.tolist()
+    # attending to the pinned list equals the masked-dense formulation
+    out, _ = O.sparse_paged_decode(pb.q, pb.kv_cache, sel, cnt, pb.last_page_len)
+    K, V = _depaged(pb, 0, 0)
+    keep = np.zeros(21 * PS, dtype=bool)
+    for p_ in list(logical[0][0]) + [0, 1, 18, 19, 20]:
+        keep[p_ * PS : (p_ + 1) * PS] = True
+    keep = keep[: PS * 20 + 7]
+    logits = O.bf16_to_f32(pb.q[0]).astype(np.float64) @ K.T / math.sqrt(D)
+    logits[:, ~keep] = -np.inf
+    w = np.exp(logits - logits.max(axis=1, keepdims=True))
+    w /= w.sum(axis=1, keepdims=True)
+    assert np.allclose(out[0], w @ V, rtol=1e-10, atol=1e-12)
+    # defaults reproduce the reference rule
+    a = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, 3)
+    b = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, 3, sink_pages=0, local_pages=1)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
