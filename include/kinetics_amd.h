@@ -211,8 +211,8 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  * outputs (both NULL, or both given with sel_stride >= topk + sink_pages +
  * local_pages); sink_pages / local_pages as in kin_block_score_topk; lse is
  * optional.  Needs no workspace.  Intended for batch * num_kv_heads large
- * enough to fill the GPU (>= ~1000 lists); for small batches the three-call
- * path with split-K is faster.
+ * enough to fill the GPU (kin_decode_auto_splits(...) == 1, i.e. >= 1024
+ * lists); for small batches the three-call path with split-K is faster.
  */
 int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
                               kin_bf16_t* kv_cache, kin_bf16_t* kbar,

@@ -269,17 +269,13 @@ def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, ma
 
 
 def prefer_fused_step(batch: int, num_kv_heads: int, max_pages_per_seq: int, topk: int) -> bool:
-    """Which of the two equivalent decode-step paths is faster (measured on
-    MI355X).  The single-launch kernel saves two dependent dispatches and the
-    selector's drain, which wins while a step moves less than about 4 GB; its
-    workgroups live longer, so on bigger steps the end-of-kernel imbalance costs
-    more than the dispatches saved and three launches are (slightly) faster.
-    Needs enough lists to fill the GPU without split-K either way."""
-    lists = batch * num_kv_heads
-    if decode_auto_splits(batch, num_kv_heads, topk + 1) > 1:
-        return False
-    step_bytes = lists * (max_pages_per_seq * 256 + (min(topk, max_pages_per_seq) + 1) * 8192)
-    return step_bytes < 4e9
+    """Which of the two equivalent decode-step paths to use.  The single-launch
+    kernel saves two dependent dispatches, the selector's drain and the attention
+    ramp-up (3-5 % per step on MI355X at every benchmark shape), but it has no
+    split-K: with too few (sequence, KV head) lists to fill the GPU the
+    three-launch path, which splits lists across workgroups, is the faster one."""
+    del max_pages_per_seq
+    return decode_auto_splits(batch, num_kv_heads, topk + 1) == 1
 
 
 def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, out=None, lse=None,
