@@ -130,6 +130,8 @@ int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar,
  *   scores_out[b,h,p]        fp32 score of candidate page p (logical index),
  *                            stride kbar_pages; may be NULL (debug/parity only:
  *                            costs an HBM write)
+ * Only logical pages below kbar_pages have a mean key: candidates at or beyond
+ * kbar_pages are never selected (size kbar for the longest sequence).
  * Requires topk >= 1, 0 <= sink_pages <= 64, 1 <= local_pages <= 64,
  * sel_stride >= topk + sink_pages + local_pages, topk <= 2048,
  * kbar_pages <= 16384.

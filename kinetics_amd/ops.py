@@ -22,8 +22,21 @@ HEAD_DIM = 128
 PAGE_SIZE = 16
 
 
+_EMPTY_STANDIN = {}
+
+
 def _ptr(t: Optional[torch.Tensor]):
-    return None if t is None else c_void_p(t.data_ptr())
+    """Device pointer of a tensor (None -> NULL).  An empty tensor has no storage
+    and would read as NULL ("argument missing" to the C ABI); it is passed as a
+    pointer to a small per-device buffer that nothing dereferences."""
+    if t is None:
+        return None
+    if t.numel() == 0:
+        buf = _EMPTY_STANDIN.get(t.device)
+        if buf is None:
+            buf = _EMPTY_STANDIN[t.device] = torch.zeros(64, dtype=torch.uint8, device=t.device)
+        return c_void_p(buf.data_ptr())
+    return c_void_p(t.data_ptr())
 
 
 def _stream(device) -> c_void_p:

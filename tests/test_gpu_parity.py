@@ -877,3 +877,77 @@ def test_sink_and_local_pages(ops, sink, local, fused):
                 n_pages = (lengths[b] + PS - 1) // PS
                 n_sink = O.split_pages(n_pages, sink, local, pb.kbar.shape[1])[0]
                 assert np.allclose(scores[b, h, n_sink : n_sink + len(ws)], ws, rtol=1e-5, atol=1e-5)
+
+
+# --------------------------------------------------------------------------- seeded sweep over odd shapes
+
+
+def test_seeded_sweep_of_shapes(ops):
+    """40 seeded random configurations -- head counts, group sizes 1..8, ragged
+    lengths with empty and one-token sequences, budgets above and below the
+    candidate count, pinned pages, table layouts, split counts, both step
+    paths -- each checked end to end against the oracle."""
+    rng = np.random.default_rng(2024)
+    for trial in range(40):
+        hkv = int(rng.choice([1, 1, 2, 3, 4, 8]))
+        group = int(rng.integers(1, 9))
+        B = int(rng.integers(1, 7))
+        lengths = []
+        for _ in range(B):
+            kind = rng.integers(0, 6)
+            if kind == 0:
+                lengths.append(0)
+            elif kind == 1:
+                lengths.append(int(rng.integers(1, PS + 1)))
+            elif kind == 2:
+                lengths.append(PS * int(rng.integers(1, 40)))           # ends exactly on a page boundary
+            else:
+                lengths.append(int(rng.integers(PS, PS * 90)))
+        topk = int(rng.choice([1, 2, 5, 17, 64, 100]))
+        sink, local = int(rng.integers(0, 3)), int(rng.integers(1, 4))
+        table = str(rng.choice(["random", "fragmented"]))
+        fused = bool(rng.integers(0, 2))
+        splits = int(rng.choice([0, 1, 2, 5]))
+        what = f"trial {trial}: hkv={hkv} G={group} lengths={lengths} topk={topk} sink={sink} local={local} {table} fused={fused} splits={splits}"
+        pb = P.make_problem(3000 + trial, lengths, num_kv_heads=hkv, group=group, topk=topk, table=table)
+        g = Gpu(pb)
+        g.sel = torch.full((pb.B, hkv, topk + sink + local), -7, dtype=torch.int32, device=DEV)
+        check_table(ops, g)
+        lse = torch.full((pb.B, pb.Hq), float("nan"), dtype=torch.float32, device=DEV)
+        if fused:
+            out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, topk, lse=lse,
+                                            sel_pages=g.sel, sel_count=g.cnt, sink_pages=sink, local_pages=local)
+        else:
+            ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
+            ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, topk, g.sel, g.cnt, sink_pages=sink, local_pages=local)
+            out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, lse=lse, num_splits=splits)
+        torch.cuda.synchronize()
+        kv, kbar = pb.kv_cache.copy(), pb.kbar.copy()
+        res = O.decode_step(pb.q, pb.k, pb.v, kv, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, topk,
+                            sink_pages=sink, local_pages=local)
+        assert np.array_equal(P.from_torch(g.kv), kv), what
+        assert np.array_equal(P.from_torch(g.kbar), kbar), what
+        sel, cnt = g.sel.cpu().numpy(), g.cnt.cpu().numpy()
+        assert np.array_equal(cnt, res["sel_count"]), what
+        # selection: exact, or within the tie rule
+        if not np.array_equal(sel, res["sel_pages"]):
+            for b in range(pb.B):
+                pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+                n_sink = O.split_pages(len(pages), sink, local, pb.kbar.shape[1])[0]
+                lookup = {int(p): i for i, p in enumerate(pages)}
+                for h in range(hkv):
+                    k_eff = len(res["sel_logical"][b][h])
+                    got = np.array([lookup[int(p)] for p in sel[b, h, :k_eff]]) - n_sink
+                    ok, msg = O.selection_matches(got, res["scores"][b][h], topk)
+                    assert ok, f"{what}: {msg}"
+                    assert np.array_equal(sel[b, h, k_eff:], res["sel_pages"][b, h, k_eff:]), what
+        want, want_lse = O.sparse_paged_decode(pb.q, kv, sel, cnt, pb.last_page_len)
+        assert_out_close(out, want, what)
+        got_lse = lse.cpu().numpy().astype(np.float64)
+        fin = np.isfinite(want_lse)
+        assert np.array_equal(np.isneginf(got_lse), ~fin), what
+        assert np.allclose(got_lse[fin], want_lse[fin], rtol=1e-4, atol=1e-4), what
+        # dense on the same cache
+        od = ops.dense_paged_decode(g.q, g.kv, g.indices, g.indptr, g.last, max(pb.max_pages, 1), num_splits=splits)
+        wd, _ = O.dense_paged_decode(pb.q, kv, pb.page_indices, pb.page_indptr, pb.last_page_len)
+        assert_out_close(od, wd, what + " (dense)")
