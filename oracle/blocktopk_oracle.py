@@ -77,7 +77,8 @@ def f32_to_bf16(x: np.ndarray) -> np.ndarray:
 
 
 def seq_pages(page_indices, page_indptr, b):
-    """Physical page ids of sequence ``b`` in logical order."""
+    """Physical page ids of sequence ``b`` in logical order (CSR convention of
+    benchmark/blocktopk_decoder.py:141-147)."""
     return np.asarray(page_indices[int(page_indptr[b]) : int(page_indptr[b + 1])], dtype=np.int64)
 
 
@@ -93,7 +94,10 @@ def seq_len(page_indptr, last_page_len, b, page_size):
 
 def page_mean_key(page_k_bits: np.ndarray) -> np.ndarray:
     """Representative key of full pages: ``page_k_bits`` is [..., page_size, D]
-    bf16 bits; float32 sum in slot order, times 1/page_size, RNE to bf16."""
+    bf16 bits; float32 sum in slot order, times 1/page_size, RNE to bf16.  The
+    reference leaves compressed_key_cache random
+    (benchmark/blocktopk_decoder.py:166-168); the block mean is what LiteSys ranks
+    blocks by (sparsity_utils.py:37) up to the query projection."""
     rows = bf16_to_f32(page_k_bits)
     ps = rows.shape[-2]
     acc = np.zeros(rows.shape[:-2] + rows.shape[-1:], dtype=np.float32)
@@ -103,7 +107,8 @@ def page_mean_key(page_k_bits: np.ndarray) -> np.ndarray:
 
 
 def append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len):
-    """In place.  k, v: [B, Hkv, D] bits; kv_cache: [P, 2, ps, Hkv, D] bits;
+    """benchmark/blocktopk_decoder.py:209-213 (LiteSys copy_to_cache,
+    cache_utils.py:5-51).  In place.  k, v: [B, Hkv, D] bits; kv_cache: [P, 2, ps, Hkv, D] bits;
     kbar: [B, kbar_pages, Hkv, D] bits or None.  Writes the new token at slot
     ``last_page_len[b]-1`` of the last page; a page that becomes full gets its
     mean key stored at its logical index."""
@@ -181,8 +186,9 @@ def block_scores(q, kbar, page_indptr, sink_pages=0, local_pages=1):
 
 
 def select_topk(scores: np.ndarray, k: int) -> np.ndarray:
-    """Indices of the min(k, n) largest scores: descending score, equal scores
-    by ascending index."""
+    """benchmark/blocktopk_decoder.py:217 / sparsity_utils.py:38 (torch.topk).
+    Indices of the min(k, n) largest scores: descending score, equal scores by
+    ascending index."""
     n = len(scores)
     order = np.lexsort((np.arange(n), -np.asarray(scores, dtype=np.float64)))
     return order[: min(k, n)].astype(np.int64)
@@ -224,7 +230,9 @@ def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_stride=None, 
 
 
 def attend_pages(q_bh, kv_cache, pages, h, last_len, sm_scale):
-    """Softmax attention of the G query rows ``q_bh`` ([G, D] float64) over the
+    """LiteSys cache_utils.py:54-169 restated for pages: logits * scale, softmax in
+    one pass over the valid tokens, P.V.
+    Softmax attention of the G query rows ``q_bh`` ([G, D] float64) over the
     tokens of ``pages`` for KV head ``h``; every page full except the final one
     (``last_len`` tokens).  Returns (out [G, D] float64, lse [G] float64,
     natural log)."""
@@ -244,7 +252,8 @@ def attend_pages(q_bh, kv_cache, pages, h, last_len, sm_scale):
 
 
 def sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, sm_scale=None):
-    """out [B, Hq, D] float64 and lse [B, Hq] float64 over the listed pages."""
+    """benchmark/blocktopk_decoder.py:223-225.  out [B, Hq, D] float64 and lse
+    [B, Hq] float64 over the listed pages."""
     B, Hq, D = q.shape
     Hkv = kv_cache.shape[3]
     G = Hq // Hkv
@@ -281,7 +290,8 @@ def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, sm
 
 def merge_partials(outs, lses):
     """Online-softmax merge of partial attention results over disjoint token
-    sets: outs [S, ..., D], lses [S, ...] (natural log)."""
+    sets (what LiteSys' split-K partial sums amount to, cache_utils.py:193-212):
+    outs [S, ..., D], lses [S, ...] (natural log)."""
     lses = np.asarray(lses, dtype=np.float64)
     m = lses.max(axis=0)
     m_safe = np.where(np.isfinite(m), m, 0.0)

@@ -148,3 +148,18 @@ def test_custom_ops_are_registered_with_fake_kernels():
     l = torch.empty(3, dtype=torch.int32, device="meta")
     out = torch.ops.kinetics.sparse_paged_decode(q, kv, i, c, l, None, 0.0, 0)
     assert out.shape == q.shape and out.dtype == torch.bfloat16
+
+
+def test_bench_byte_model_matches_the_documented_figures():
+    """The algorithmic-bytes model behind the roofline figures: 1 576 960 B per
+    sequence at the headline shape (k-bar stream + selected K/V + append + q/out +
+    index write/read), 16 780 288 B for the dense baseline."""
+    import bench
+
+    ab = bench.algorithmic_bytes([32768 + 1] * 4096, 1, 4, 128)
+    assert ab["step"] == 4096 * 1576960 == 6459228160
+    assert ab["step"] // 4096 == 524288 + 1049088 + 512 + 2048 + 1024
+    assert ab["dense"] == 4096 * 16780288
+    assert ab["attention"] == 4096 * (1049088 + 2048 + 129 * 4)
+    small = bench.algorithmic_bytes([17], 2, 2, 8)       # 2 pages: 1 candidate, budget clamps to 1
+    assert small["step"] == 2 * (1 * 256 + (16 + 1) * 512 + 512) + 2 * 4 * 256 + 2 * 2 * 1 * 4
