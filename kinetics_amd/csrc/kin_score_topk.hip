@@ -20,6 +20,7 @@ struct ScoreTopkParams {
 };
 
 // Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap] | int32 sel[topk + sink + local]
+template <int UNROLL>
 __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x;
@@ -52,7 +53,7 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
   a.keys = reinterpret_cast<uint32_t*>(smem);
   a.sortbuf = reinterpret_cast<unsigned long long*>(smem + (size_t)((p.kbar_pages + 3) & ~3) * 4);
   a.sort_cap = p.sort_cap;
-  const int n_list = score_select(a, sel_lds);
+  const int n_list = score_select<UNROLL>(a, sel_lds);
 
   for (int i = tid; i < p.sel_stride; i += kThreads) sel[i] = (i < n_list) ? sel_lds[i] : -1;
   if (tid == 0) p.sel_count[item] = n_list;
@@ -107,13 +108,20 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
   const size_t lds = select_lds_bytes(kbar_pages, p.sort_cap) + (size_t)(topk + sink_pages + local_pages) * 4;
   const int64_t items = (int64_t)batch * num_kv_heads;
   if (items > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
+  // Few workgroups cannot saturate HBM with 4 loads per lane in flight: give a
+  // small grid 16 (more registers, which it can afford).
+  const bool small_grid = items < 512;
+  const void* fn_ptr = small_grid ? reinterpret_cast<const void*>(&score_topk_kernel<16>)
+                                  : reinterpret_cast<const void*>(&score_topk_kernel<4>);
   if (lds > 48 * 1024) {
     // Above the default dynamic-LDS allowance the runtime wants an explicit opt-in.
-    st = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&score_topk_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+    st = check_hip(hipFuncSetAttribute(fn_ptr, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
                    "hipFuncSetAttribute(score_topk_kernel)");
     if (st) return st;
   }
-  score_topk_kernel<<<(unsigned)items, kThreads, lds, static_cast<hipStream_t>(stream)>>>(p);
+  if (small_grid)
+    score_topk_kernel<16><<<(unsigned)items, kThreads, lds, static_cast<hipStream_t>(stream)>>>(p);
+  else
+    score_topk_kernel<4><<<(unsigned)items, kThreads, lds, static_cast<hipStream_t>(stream)>>>(p);
   return check_hip(hipGetLastError(), "score_topk_kernel launch");
 }

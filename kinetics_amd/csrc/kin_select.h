@@ -27,7 +27,6 @@ __device__ __forceinline__ uint32_t order_key(float f) {
 }
 
 constexpr int kThreads = 256;
-constexpr int kUnroll = 4;          // independent 16-byte loads in flight per lane
 constexpr int kRankSortMax = 512;   // up to here winners are ordered by counting, above by bitonic sort
 
 // Wave-uniform description of one selection problem.
@@ -79,7 +78,12 @@ __host__ __device__ inline void split_pages(int n_pages, int sink_pages, int loc
 // local pages (the open page last).  Returns the list length.  Ends with a
 // workgroup barrier: sel_lds is visible to every thread and keys / sortbuf are
 // free for reuse.
+// UNROLL: independent 16-byte loads each lane keeps in flight while streaming the
+// mean keys (4 saturates HBM when thousands of workgroups run; a small grid
+// needs more per workgroup).
+template <int UNROLL = 4>
 __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_lds) {
+  constexpr int kUnroll = UNROLL;
   __shared__ uint32_t hist[256];
   __shared__ uint32_t wave_tot[4];
   __shared__ uint32_t sh_bin, sh_remaining, sh_count;
