@@ -177,6 +177,37 @@ def cpu_baseline(torch, B_cpu, ctx, G, topk, budget_s=20.0):
                        f"{med * 1e3:.2f} ms/step; tokens/s is linear in batch")
 
 
+WHOLE_LAYER_MODEL = {"qwen3-8b-share": ("Qwen3-8B", 8), "qwen3-32b-share": ("Qwen3-32B", 8)}
+
+
+def whole_layer(torch, args, B, ctx, topk, device):
+    """One whole decoder layer of the TP shard, timed like benchmark/blocktopk.py:47-61
+    (hidden_states.clone() -> forward, warm-up then K timed calls).  The printed figure
+    of the reference additionally divides by world_size * num_hidden_layers (:82)."""
+    from kinetics_amd.decoder_layer import BlockTopkDecoderLayer, init_weights, qwen3_config
+
+    name, world = WHOLE_LAYER_MODEL[args.workload]
+    cfg = qwen3_config(name)
+    layer = BlockTopkDecoderLayer(cfg, world, B, ctx, ctx + 512, PS, topk, device, torch.bfloat16)
+    layer.apply(init_weights)
+    layer.eval().to(device, dtype=torch.bfloat16)
+    hidden = torch.randn(B, 1, cfg.hidden_size, device=device, dtype=torch.bfloat16)
+    for _ in range(args.warmup):
+        layer(hidden.clone())
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        layer(hidden.clone())
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    out = {"model": name, "world_size": world, "ms_per_layer_step": dt * 1e3, "tokens_per_s_per_layer": B / dt,
+           "normalised_like_reference_print": B / dt / (world * cfg.num_hidden_layers),
+           "note": "norms and GEMMs are plain PyTorch (rocBLAS/hipBLASLt); only the attention path is this repository's kernels"}
+    del layer
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -190,6 +221,9 @@ def main():
     ap.add_argument("--mode", default="auto", choices=["auto", "fused", "three"],
                     help="decode-step path: one fused launch, three launches (append / score+select / attention), "
                          "or what kinetics_amd.ops.prefer_fused_step picks for the shape")
+    ap.add_argument("--whole-layer", action="store_true",
+                    help="also time the whole decoder layer (norms, GEMMs, MLP around the attention path), "
+                         "the quantity benchmark/blocktopk.py prints")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) to scale profiler byte counters")
     args = ap.parse_args()
@@ -321,6 +355,8 @@ def main():
                                     "sparse_over_dense": (B * K / elapsed) / (B / td)}
     del st
     torch.cuda.empty_cache()
+    if args.whole_layer and args.workload in WHOLE_LAYER_MODEL:
+        result["whole_layer"] = whole_layer(torch, args, B, ctx, topk, device)
     if not args.no_cpu_baseline and Hkv == 1 and args.workload not in RAGGED:
         result["cpu_baseline"] = cpu_baseline(torch, min(args.cpu_batch, B), ctx, G, topk)
     print(json.dumps(result))
