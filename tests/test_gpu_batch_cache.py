@@ -39,10 +39,13 @@ def test_rejects_what_it_does_not_implement():
         PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_block_topk=2, attn_local=4, attn_block_size=32)
 
 
-@pytest.mark.parametrize("sparse", [dict(), dict(attn_block_topk=3, attn_local=16)])
-def test_prefill_then_decode_like_litesys(sparse):
+@pytest.mark.parametrize("sparse,fused", [(dict(), None), (dict(attn_block_topk=3, attn_local=16), True),
+                                          (dict(attn_block_topk=3, attn_local=16), False)])
+def test_prefill_then_decode_like_litesys(sparse, fused):
     torch.manual_seed(5)
     m = make_manager(**sparse)
+    if fused is not None:
+        m._fused = fused          # both routes of decode(): one launch, or append + select + attend
     L, Hq, Hkv = 2, 4, 2
     hist = {}  # (layer, slot) -> (K [t, Hkv, D], V) float32 of the bf16 values fed so far
 
