@@ -259,7 +259,7 @@ def main():
         return [
             ("append", lambda: ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"],
                                                    st["last"])),
-            ("score_topk", lambda: ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], topk,
+            ("score_topk", lambda: ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], st["last"], topk,
                                                         st["sel"], st["cnt"])),
             ("sparse_attention", lambda: ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"],
                                                                  out=st["out"], workspace=st["ws"])),

@@ -110,19 +110,27 @@ int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar,
  * (ref: benchmark/blocktopk_decoder.py:216-221) and, per KV head, LiteSys
  * blockwise_topk_sparsity (ref: LiteSys/litesys/attention/sparsity_utils.py:24-47).
  *
- * The pages of sequence b split into n_local = min(local_pages, n_pages)
- * trailing pages and n_sink = min(sink_pages, rest) leading pages, which are
- * always attended, and the candidates in between (logical pages n_sink ..
- * n_pages-n_local-1).  sink_pages = 0, local_pages = 1 is the reference's rule
- * ("top-k plus the last page", blocktopk_decoder.py:220); larger values give the
- * page-aligned form of LiteSys' sink tokens and local window
- * (sparsity_utils.py:24-35).  score[p] = dot(mean_g q[b, h*G+g, :],
- * kbar[b, p, h, :]) in fp32.  k_eff = min(topk, n_cand) candidates are selected:
- * descending score, equal scores by ascending logical index (deterministic).
- * Outputs, with n = k_eff + n_sink + n_local:
- *   sel_pages[b,h,0:k_eff]   physical ids of the selected pages, in that order
- *   sel_pages[b,h,k_eff:n]   the sink pages, then the local pages (the open
- *                            page last)
+ * With kv_len = 16*(n_pages-1) + last_page_len[b], the pages of sequence b
+ * split into
+ *   n_sink  = min(sink_pages, n_pages-1) leading pages, always attended,
+ *   n_cand  = max(0, floor((kv_len - 16*n_sink - local_tokens) / 16)) candidate
+ *             pages after them (the whole pages that lie before the newest
+ *             local_tokens tokens), and
+ *   n_local = n_pages - n_sink - n_cand trailing pages, always attended; the
+ *             open page is one of them (local_tokens >= 1), even when full.
+ * sink_pages = 0, local_tokens = 1 is the reference's rule ("top-k plus the
+ * last page", blocktopk_decoder.py:220); local_tokens = 16*(L-1)+1 pins exactly
+ * the last L pages.  sink_pages = 1 with the sequences stored 12 slots into
+ * their first page (see first_page_offset below) and local_tokens = LiteSys'
+ * `local` reproduces blockwise_topk_sparsity with its hard-wired 4 sink tokens
+ * and 16-token blocks that start at token 4 (sparsity_utils.py:24-35).
+ * score[p] = dot(mean_g q[b, h*G+g, :], kbar[b, p, h, :]) in fp32.
+ * k_eff = min(topk, n_cand) candidates are selected: descending score, equal
+ * scores by ascending logical index (deterministic).
+ * Outputs, with n = n_sink + k_eff + n_local:
+ *   sel_pages[b,h,0:n_sink]          physical ids of the sink pages
+ *   sel_pages[b,h,n_sink:n_sink+k_eff]  the selected pages, in that order
+ *   sel_pages[b,h,n_sink+k_eff:n]    the local pages (the open page last)
  *   sel_pages[b,h,n:]        -1
  *   sel_count[b,h]           n   (0 for an empty page list)
  *   sel_logical[b,h,0:k_eff] logical page indices (== n_sink +
@@ -132,17 +140,26 @@ int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar,
  *                            costs an HBM write)
  * Only logical pages below kbar_pages have a mean key: candidates at or beyond
  * kbar_pages are never selected (size kbar for the longest sequence).
- * Requires topk >= 1, 0 <= sink_pages <= 64, 1 <= local_pages <= 64,
- * sel_stride >= topk + sink_pages + local_pages, topk <= 2048,
- * kbar_pages <= 16384.
+ * Requires topk >= 0 (0: sink and local pages only, no key is read),
+ * 0 <= sink_pages <= 64, 1 <= local_tokens <= 1009,
+ * sel_stride >= kin_sel_list_capacity(topk, sink_pages, local_tokens),
+ * topk <= 2048, kbar_pages <= 16384.
  */
 int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
                          const int32_t* page_indices, const int32_t* page_indptr,
-                         int topk, int sink_pages, int local_pages,
+                         const int32_t* last_page_len,
+                         int topk, int sink_pages, int local_tokens,
                          int32_t* sel_pages, int32_t* sel_count,
                          int32_t* sel_logical, float* scores_out,
                          int batch, int num_q_heads, int num_kv_heads, int head_dim,
                          int kbar_pages, int sel_stride, kin_stream_t stream);
+
+/*
+ * Longest page list the selector can write for these settings:
+ * topk + sink_pages + 1 + ceil((local_tokens - 1) / 16).  0 for arguments out
+ * of range.
+ */
+int kin_sel_list_capacity(int topk, int sink_pages, int local_tokens);
 
 /*
  * Bytes of workspace kin_sparse_paged_decode / kin_dense_paged_decode need for
@@ -171,6 +188,12 @@ int kin_decode_auto_splits(int batch, int num_kv_heads, int max_pages_per_list);
  * 1/sqrt(head_dim).  num_splits: 0 = automatic, else the number of split-K
  * partitions per list (>1 needs workspace, see kin_decode_workspace_bytes).
  * An empty list yields out = 0, lse = -inf.
+ * first_page_offset (0..15): the first that many token slots of the FIRST listed
+ * page of every list hold no token and are skipped -- for caches that store
+ * each sequence shifted into its first page so that pages line up with blocks
+ * that do not start at token 0 (LiteSys' blocks start after 4 sink tokens,
+ * sparsity_utils.py:24-35: offset 12).  The selector lists the sequence's first
+ * page first whenever sink_pages >= 1.
  */
 int kin_sparse_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
                             const int32_t* sel_pages, const int32_t* sel_count,
@@ -179,8 +202,8 @@ int kin_sparse_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
                             void* workspace, size_t workspace_bytes,
                             int batch, int num_q_heads, int num_kv_heads,
                             int head_dim, int page_size, int64_t num_pages,
-                            int sel_stride, float sm_scale, int num_splits,
-                            kin_stream_t stream);
+                            int sel_stride, int first_page_offset,
+                            float sm_scale, int num_splits, kin_stream_t stream);
 
 /*
  * Dense paged decode attention over every page of each sequence -- replaces
@@ -188,7 +211,7 @@ int kin_sparse_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  * 211-219).  Same arithmetic and kernel as kin_sparse_paged_decode; the page
  * list of sequence b is page_indices[page_indptr[b]:page_indptr[b+1]], shared
  * by all KV heads.  max_pages_per_seq bounds the longest list (used only to
- * choose the split count).
+ * choose the split count).  first_page_offset as above.
  */
 int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
                            const int32_t* page_indices, const int32_t* page_indptr,
@@ -197,8 +220,8 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
                            void* workspace, size_t workspace_bytes,
                            int batch, int num_q_heads, int num_kv_heads,
                            int head_dim, int page_size, int64_t num_pages,
-                           int max_pages_per_seq, float sm_scale, int num_splits,
-                           kin_stream_t stream);
+                           int max_pages_per_seq, int first_page_offset,
+                           float sm_scale, int num_splits, kin_stream_t stream);
 
 /*
  * The whole decode step in ONE launch -- replaces lines 209-225 of the
@@ -210,23 +233,26 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  * leaves the chip and phases of different sequences overlap.
  *
  * k and v may both be NULL (no append).  sel_pages / sel_count are optional
- * outputs (both NULL, or both given with sel_stride >= topk + sink_pages +
- * local_pages); sink_pages / local_pages as in kin_block_score_topk; lse is
- * optional.  Needs no workspace.  Intended for batch * num_kv_heads large
- * enough to fill the GPU (kin_decode_auto_splits(...) == 1, i.e. >= 1024
- * lists); for small batches the three-call path with split-K is faster.
+ * outputs (both NULL, or both given with sel_stride >=
+ * kin_sel_list_capacity(...)); topk / sink_pages / local_tokens as in
+ * kin_block_score_topk, first_page_offset as in kin_sparse_paged_decode (a
+ * non-zero offset requires sink_pages >= 1: a padded page has no valid mean
+ * key); lse is optional.  Needs no workspace.  One workgroup walks a whole
+ * list (no split-K): faster than the three calls from about 256 lists
+ * (batch * num_kv_heads) up, and for lists of up to ~129 pages at any batch
+ * size; few long lists are better served by the three-call path.
  */
 int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
                               kin_bf16_t* kv_cache, kin_bf16_t* kbar,
                               const int32_t* page_indices, const int32_t* page_indptr,
                               const int32_t* last_page_len, int topk,
-                              int sink_pages, int local_pages,
+                              int sink_pages, int local_tokens,
                               int32_t* sel_pages, int32_t* sel_count,
                               kin_bf16_t* out, float* lse,
                               int batch, int num_q_heads, int num_kv_heads,
                               int head_dim, int page_size, int64_t num_pages,
-                              int kbar_pages, int sel_stride, float sm_scale,
-                              kin_stream_t stream);
+                              int kbar_pages, int sel_stride, int first_page_offset,
+                              float sm_scale, kin_stream_t stream);
 
 /*
  * Page-table metadata for a slot-based cache -- the paged replacement of

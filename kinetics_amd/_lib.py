@@ -35,22 +35,25 @@ SIGNATURES = {
     "kin_build_kbar": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int64, c_int, _P]),
     "kin_block_score_topk": (
         c_int,
-        [_P, _P, _P, _P, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+        [_P, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P],
     ),
+    "kin_sel_list_capacity": (c_int, [c_int, c_int, c_int]),
     "kin_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "kin_decode_auto_splits": (c_int, [c_int, c_int, c_int]),
     "kin_sparse_paged_decode": (
         c_int,
-        [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int64, c_int, c_float, c_int, _P],
+        [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int64, c_int, c_int, c_float,
+         c_int, _P],
     ),
     "kin_dense_paged_decode": (
         c_int,
-        [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int64, c_int, c_float, c_int, _P],
+        [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int64, c_int, c_int, c_float,
+         c_int, _P],
     ),
     "kin_blocktopk_decode_step": (
         c_int,
         [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int64,
-         c_int, c_int, c_float, _P],
+         c_int, c_int, c_int, c_float, _P],
     ),
     "kin_build_slot_page_table": (c_int, [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P]),
     "kin_check_page_table": (c_int, [_P, _P, _P, c_int, c_int, c_int64, c_int64, _P, _P]),

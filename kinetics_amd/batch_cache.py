@@ -7,18 +7,26 @@ top-k blocks and runs softmax and P.V over the whole context
 (batch_cache.py:154-168, sparsity_utils.py:24-47).  Here every slot owns a fixed
 run of 16-token pages of one paged cache per layer; decode appends the token,
 scores the per-page mean keys, selects the top-k pages per KV head and attends
-only to those pages plus the open page -- the same result as the mask
-formulation with page-aligned blocks, without touching the rest of the context.
+only to those pages plus the pinned ones -- the same result as the mask
+formulation, without touching the rest of the context.
 
 Supported configurations (anything else raises at construction):
   * no sparsity arguments                      -> dense paged decode
   * ``attn_block_topk=k`` (+ ``attn_local``)    -> block top-k with block size 16
-Differences from LiteSys, by design of the paged layout: everything is page
-aligned.  LiteSys always attends 4 hard-wired "sink" tokens and the newest
-``attn_local`` tokens and starts its blocks after the sink
-(sparsity_utils.py:24-35,240); here the first page (16 tokens, a superset of the
-sink) and the last ``ceil(attn_local/16) + 1`` pages (a superset of the local
-window) are pinned into every list and the blocks are the pages in between.
+  * ``attn_local`` alone                        -> sink + local window only: block top-k with
+                                                  k = 0, whose window is LiteSys' ``local``
+                                                  rounded up to the block grid (a superset, by
+                                                  at most 15 tokens, of local_sparsity,
+                                                  sparsity_utils.py:107-114)
+LiteSys always attends 4 hard-wired "sink" tokens, starts its 16-token blocks
+right after them and always attends the ``_local`` newest tokens that remain
+after the last whole block (sparsity_utils.py:24-35,240).  To keep that exact
+geometry on 16-token pages, a sparse manager stores every sequence 12 slots
+into its first page: the sink tokens are slots 12..15 of page 0, block j is
+page j+1, and the kernels are told to skip the 12 padding slots
+(``first_page_offset``), to pin one sink page and to keep the newest
+``attn_local`` tokens out of the candidates (``local_tokens``).  The attended
+token set is then LiteSys' own, token for token.
 ``attn_layer_skip`` (default ``[0]``: layer 0 stays dense, sparsity_utils.py:211)
 is honoured.
 Prefill is not the accelerated path: it writes pages with PyTorch indexing and
@@ -68,14 +76,19 @@ class PagedBatchKVManager:
                 raise AssertionError("attn_local must be provided if use_nonlocal_sparsity is True")
             if kwargs.get("attn_block_size", PAGE) != PAGE:
                 raise NotImplementedError("block size must equal the page size (16)")
-        elif kwargs.get("attn_local") is not None:
-            raise NotImplementedError("local-window-only sparsity is not implemented")
+        self.sparse = kwargs.get("attn_local") is not None
+        if self.sparse and self.block_topk is None:
+            self.block_topk = 0                      # sink + local window only
         self.layer_skip = list(kwargs.get("attn_layer_skip", [0]))
-        self.sink_pages = 1
-        self.local_pages = (int(kwargs["attn_local"]) + PAGE - 1) // PAGE + 1 if self.block_topk is not None else 1
+        self.sink_pages = 1 if self.sparse else 0
+        self.local_tokens = int(kwargs["attn_local"]) if self.sparse else 1
+        if self.sparse and not 1 <= self.local_tokens <= 1009:
+            raise NotImplementedError("attn_local must be in [1, 1009]")
+        # padding slots in front of every sequence: LiteSys' 4 sink tokens end page 0, its blocks are pages 1, 2, ...
+        self.pad = PAGE - 4 if self.sparse else 0
 
         B, Hq, Hkv, D = max_batch_size, self.num_attention_heads, self.num_key_value_heads, self.head_dim
-        self.pages_per_slot = P = (max_seq_len + PAGE - 1) // PAGE
+        self.pages_per_slot = P = (max_seq_len + self.pad + PAGE - 1) // PAGE
         dev = self.device
         self.kv_cache = [torch.zeros(B * P, 2, PAGE, Hkv, D, dtype=dtype, device=dev) for _ in range(self.num_layers)]
         self.kbar = [torch.zeros(B, P, Hkv, D, dtype=dtype, device=dev) for _ in range(self.num_layers)]
@@ -89,8 +102,9 @@ class PagedBatchKVManager:
         self._k = torch.zeros(B, Hkv, D, dtype=dtype, device=dev)
         self._v = torch.zeros(B, Hkv, D, dtype=dtype, device=dev)
         self._out = torch.zeros(B, Hq, D, dtype=dtype, device=dev)
-        k = self.block_topk or 1
-        self._sel = torch.full((B, Hkv, k + self.sink_pages + self.local_pages), -1, dtype=torch.int32, device=dev)
+        k = self.block_topk or 0
+        self._sel = torch.full((B, Hkv, ops.sel_list_capacity(k, self.sink_pages, self.local_tokens)), -1,
+                               dtype=torch.int32, device=dev)
         self._cnt = torch.zeros(B, Hkv, dtype=torch.int32, device=dev)
         self._fused = ops.prefer_fused_step(B, Hkv, P, k)
         ws = max(ops.decode_workspace_bytes(B, Hq, Hkv, P), ops.decode_workspace_bytes(B, Hq, Hkv, self._sel.shape[2]), 16)
@@ -119,26 +133,29 @@ class PagedBatchKVManager:
         off[slots] += 1
         # Sequence b of the kernels == slot b; inactive slots get an empty page list.
         self._lens.zero_()
-        self._lens[slots] = off[slots]
+        self._lens[slots] = off[slots] + self.pad
         ops.build_slot_page_table(self._lens, self.pages_per_slot, PAGE, self.page_indices, self.page_indptr, self.last_page_len)
         self._q[slots] = query[:, :, 0, :]
         self._k[slots] = key[:, :, 0, :]
         self._v[slots] = value[:, :, 0, :]
         kv, kbar = self.kv_cache[layer_idx], self.kbar[layer_idx]
-        sparse = self.block_topk is not None and layer_idx not in self.layer_skip
+        sparse = self.sparse and layer_idx not in self.layer_skip
         if sparse and self._fused:
             ops.blocktopk_decode_step(self._q, self._k, self._v, kv, kbar, self.page_indices, self.page_indptr,
                                       self.last_page_len, self.block_topk, out=self._out, sink_pages=self.sink_pages,
-                                      local_pages=self.local_pages)
+                                      local_tokens=self.local_tokens, first_page_offset=self.pad)
         else:
             ops.append_paged_kv(self._k, self._v, kv, kbar, self.page_indices, self.page_indptr, self.last_page_len)
             if sparse:
-                ops.block_score_topk(self._q, kbar, self.page_indices, self.page_indptr, self.block_topk, self._sel, self._cnt,
-                                     sink_pages=self.sink_pages, local_pages=self.local_pages)
-                ops.sparse_paged_decode(self._q, kv, self._sel, self._cnt, self.last_page_len, out=self._out, workspace=self._ws)
+                ops.block_score_topk(self._q, kbar, self.page_indices, self.page_indptr, self.last_page_len,
+                                     self.block_topk, self._sel, self._cnt, sink_pages=self.sink_pages,
+                                     local_tokens=self.local_tokens)
+                ops.sparse_paged_decode(self._q, kv, self._sel, self._cnt, self.last_page_len, out=self._out,
+                                        workspace=self._ws, first_page_offset=self.pad)
             else:
                 ops.dense_paged_decode(self._q, kv, self.page_indices, self.page_indptr, self.last_page_len,
-                                       self.pages_per_slot, out=self._out, workspace=self._ws)
+                                       self.pages_per_slot, out=self._out, workspace=self._ws,
+                                       first_page_offset=self.pad)
         return self._out[slots]
 
     # ------------------------------------------------------------------ prefill (not the accelerated path)
@@ -150,21 +167,22 @@ class PagedBatchKVManager:
         slot = int(batch_idx.item())
         offset = int(self.kv_offset[layer_idx][slot].item())
         total = offset + seq_len
-        if total > self.pages_per_slot * PAGE:
+        pad = self.pad                                   # token t lives in cache slot t + pad
+        if total + pad > self.pages_per_slot * PAGE:
             raise ValueError(f"sequence of {total} tokens exceeds max_seq_len")
         P, Hkv, D = self.pages_per_slot, self.num_key_value_heads, self.head_dim
         view = self.kv_cache[layer_idx].view(self.max_batch_size, P, 2, PAGE, Hkv, D)
-        tok = torch.arange(offset, total, device=self.device)
-        view[slot, tok // PAGE, 0, tok % PAGE] = key_states[0].transpose(0, 1)
-        view[slot, tok // PAGE, 1, tok % PAGE] = value_states[0].transpose(0, 1)
+        pos = torch.arange(offset, total, device=self.device) + pad
+        view[slot, pos // PAGE, 0, pos % PAGE] = key_states[0].transpose(0, 1)
+        view[slot, pos // PAGE, 1, pos % PAGE] = value_states[0].transpose(0, 1)
         self.kv_offset[layer_idx][slot] += seq_len
-        n_pages = (total + PAGE - 1) // PAGE
+        n_pages = (total + pad + PAGE - 1) // PAGE
         idx = (slot * P + torch.arange(n_pages, device=self.device, dtype=torch.int32)).contiguous()
         ptr = torch.tensor([0, n_pages], dtype=torch.int32, device=self.device)
-        last = torch.tensor([total - (n_pages - 1) * PAGE], dtype=torch.int32, device=self.device)
+        last = torch.tensor([total + pad - (n_pages - 1) * PAGE], dtype=torch.int32, device=self.device)
         ops.build_kbar(self.kv_cache[layer_idx], self.kbar[layer_idx][slot:slot + 1], idx, ptr, last)
-        k_all = view[slot, :n_pages, 0].reshape(n_pages * PAGE, Hkv, D)[:total].transpose(0, 1)  # [Hkv, total, D]
-        v_all = view[slot, :n_pages, 1].reshape(n_pages * PAGE, Hkv, D)[:total].transpose(0, 1)
+        k_all = view[slot, :n_pages, 0].reshape(n_pages * PAGE, Hkv, D)[pad:total + pad].transpose(0, 1)  # [Hkv, total, D]
+        v_all = view[slot, :n_pages, 1].reshape(n_pages * PAGE, Hkv, D)[pad:total + pad].transpose(0, 1)
         G = self.num_attention_heads // Hkv
         q = query_states[0]                                                                    # [Hq, s, D]
         pos_q = torch.arange(offset, total, device=self.device)[:, None]

@@ -30,7 +30,7 @@ class BlockTopkPagedAttention:
     def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, batch_size: int, prefix_len: int,
                  max_len: int, page_size: int, topk_page: int, device="cuda", dtype=torch.bfloat16,
                  init_cache: str = "randn", seed: int = 0, fused: Optional[bool] = None, sink_pages: int = 0,
-                 local_pages: int = 1):
+                 local_tokens: int = 1):
         if dtype != torch.bfloat16:
             raise ValueError("the HIP kernels are built for bfloat16")
         if prefix_len % page_size != 0:
@@ -53,10 +53,11 @@ class BlockTopkPagedAttention:
         self.paged_kv_indptr = (torch.arange(B + 1, dtype=torch.int32, device=dev) * (n + 1)).contiguous()
         # The open page holds exactly the token being decoded after the append.
         self.last_kv_lens = torch.ones(B, dtype=torch.int32, device=dev)
-        # sink_pages leading and local_pages trailing pages are always attended (0 / 1: the reference's rule)
-        self.sink_pages, self.local_pages = sink_pages, local_pages
-        self.topk_page_indices = torch.full((B, num_kv_heads, topk_page + sink_pages + local_pages), -1, dtype=torch.int32,
-                                            device=dev)
+        # the first sink_pages pages and the pages of the newest local_tokens tokens are always attended
+        # (0 / 1: the reference's rule, top-k plus the last page)
+        self.sink_pages, self.local_tokens = sink_pages, local_tokens
+        self.list_capacity = ops.sel_list_capacity(topk_page, sink_pages, local_tokens)
+        self.topk_page_indices = torch.full((B, num_kv_heads, self.list_capacity), -1, dtype=torch.int32, device=dev)
         self.topk_page_count = torch.zeros(B, num_kv_heads, dtype=torch.int32, device=dev)
 
         shape = (max_num_pages * B, 2, page_size, num_kv_heads, head_dim)
@@ -78,7 +79,7 @@ class BlockTopkPagedAttention:
         self.sm_scale = 1.0 / math.sqrt(head_dim)
         # one launch or three: same results, the faster one for this shape unless told otherwise
         self.fused = ops.prefer_fused_step(B, num_kv_heads, n + 1, topk_page) if fused is None else bool(fused)
-        ws = ops.decode_workspace_bytes(B, num_heads, num_kv_heads, topk_page + sink_pages + local_pages)
+        ws = ops.decode_workspace_bytes(B, num_heads, num_kv_heads, self.list_capacity)
         self.workspace: Optional[torch.Tensor] = torch.empty(ws, dtype=torch.uint8, device=dev) if ws else None
 
     # -- the three stages, each a custom op --------------------------------
@@ -93,8 +94,9 @@ class BlockTopkPagedAttention:
     def select_pages(self, query_states: torch.Tensor) -> None:
         """benchmark/blocktopk_decoder.py:216-221; result lands in ``topk_page_indices``."""
         torch.ops.kinetics.block_score_topk(query_states, self.compressed_key_cache, self.paged_kv_indices,
-                                            self.paged_kv_indptr, self.topk_page, self.topk_page_indices,
-                                            self.topk_page_count, self.sink_pages, self.local_pages)
+                                            self.paged_kv_indptr, self.last_kv_lens, self.topk_page,
+                                            self.topk_page_indices, self.topk_page_count, self.sink_pages,
+                                            self.local_tokens)
 
     def decode(self, query_states: torch.Tensor) -> torch.Tensor:
         """benchmark/blocktopk_decoder.py:223-225."""
@@ -108,7 +110,7 @@ class BlockTopkPagedAttention:
             return torch.ops.kinetics.blocktopk_decode_step(
                 query_states, key_states, value_states, self.kv_cache, self.compressed_key_cache,
                 self.paged_kv_indices, self.paged_kv_indptr, self.last_kv_lens, self.topk_page,
-                self.topk_page_indices, self.topk_page_count, self.sm_scale, self.sink_pages, self.local_pages)
+                self.topk_page_indices, self.topk_page_count, self.sm_scale, self.sink_pages, self.local_tokens)
         self.update_kv(key_states, value_states)
         self.select_pages(query_states)
         return self.decode(query_states)

@@ -41,6 +41,19 @@ int check_common_dims(const char* fn, int batch, int num_q_heads, int num_kv_hea
   return KIN_OK;
 }
 
+int check_fixed_pages(const char* fn, int sink_pages, int local_tokens) {
+  if (sink_pages < 0 || sink_pages > kMaxFixedPages || local_tokens < 1 || local_tokens > kMaxLocalTokens)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: sink_pages=%d must be in [0, %d] and local_tokens=%d in [1, %d]", fn, sink_pages,
+                kMaxFixedPages, local_tokens, kMaxLocalTokens);
+  return KIN_OK;
+}
+
+int check_first_page_offset(const char* fn, int first_page_offset) {
+  if (first_page_offset < 0 || first_page_offset >= kPageSize)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: first_page_offset=%d must be in [0, %d)", fn, first_page_offset, kPageSize);
+  return KIN_OK;
+}
+
 // One thread per sequence checks its indptr step, last_page_len and page ids.
 __global__ void check_page_table_kernel(const int32_t* __restrict__ page_indices,
                                         const int32_t* __restrict__ page_indptr,
@@ -70,7 +83,12 @@ __global__ void check_page_table_kernel(const int32_t* __restrict__ page_indices
 
 extern "C" {
 
-int kin_version(void) { return 100; }
+int kin_version(void) { return 110; }
+
+int kin_sel_list_capacity(int topk, int sink_pages, int local_tokens) {
+  if (topk < 0 || sink_pages < 0 || local_tokens < 1) return 0;
+  return topk + sink_pages + kin::max_local_pages(local_tokens);
+}
 
 const char* kin_last_error(void) { return kin::g_last_error; }
 

@@ -47,11 +47,12 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, in
 
 // One page for one wave, first half: scores and the online softmax update.
 // ka: this lane's 4 K chunks in MFMA A layout.  Leaves the probabilities of
-// this lane's 4 tokens in pr.
+// this lane's 4 tokens in pr.  Requires 0 <= first_token <= 16 and
+// 0 <= valid_tokens <= 16 (an empty range masks the whole page).
 template <int NG>
 __device__ __forceinline__ void page_scores(const uint4 (&ka)[4], const bf16x8 (&qB)[NG][4], float (&m_run)[NG],
                                             float (&l_run)[NG], floatx4 (&O)[NG][8], float (&pr)[NG][4],
-                                            float scale_log2, int valid_tokens, int kg) {
+                                            float scale_log2, int first_token, int valid_tokens, int kg) {
   floatx4 S[NG];
 #pragma unroll
   for (int half = 0; half < NG; ++half) S[half] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -66,7 +67,9 @@ __device__ __forceinline__ void page_scores(const uint4 (&ka)[4], const bf16x8 (
   for (int half = 0; half < NG; ++half) {
     float s[4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) s[r] = (4 * kg + r < valid_tokens) ? S[half][r] * scale_log2 : kNegInf;
+    for (int r = 0; r < 4; ++r)  // token slots [first_token, valid_tokens) of the page count
+      s[r] = ((unsigned)(4 * kg + r - first_token) < (unsigned)(valid_tokens - first_token)) ? S[half][r] * scale_log2
+                                                                                             : kNegInf;
     const float m_new = fmaxf(m_run[half], fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
     if (__any(m_new > m_run[half])) {
       const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
@@ -121,6 +124,7 @@ struct AttendArgs {
   int n;                 // list length
   int p0, p1;            // this workgroup's part of the list [p0, p1)
   int last_len;          // tokens in the list's final page
+  int first_skip;        // leading token slots of list entry 0 that hold no token (0..15)
 };
 
 constexpr int kAttendLdsBytes = 32768;  // 4 waves x 2 stages x 4 KiB; reused for the merge
@@ -192,10 +196,15 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
     const int idx = my_first + 4 * it;
     return id_at(idx < p1 ? idx : p0);
   };
+  const int first_skip = a.first_skip;
   auto page_rsrc = [&](int it, int id, int& valid_tokens) {
     const int idx = my_first + 4 * it;
     const bool ok = idx < p1 && id >= 0 && (int64_t)id < a.num_pages;
-    valid_tokens = ok ? (idx == n_last ? last_len : kPageSize) : 0;
+    // The skipped slots of entry 0 are folded into one number: bits 8.. hold
+    // the first counted slot, bits 0..7 one past the last.
+    const int hi = idx == n_last ? last_len : kPageSize;
+    const int lo = idx == 0 ? min(first_skip, hi) : 0;
+    valid_tokens = ok ? (hi | (lo << 8)) : 0;
     return make_rsrc(kvb + (int64_t)(ok ? id : 0) * page_bytes, ok ? span : 0);
   };
   auto issue_v = [&](__amdgpu_buffer_rsrc_t r, u32x4 (&vv)[4]) {
@@ -242,7 +251,7 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
         __builtin_amdgcn_sched_barrier(0);
         issue_k(r1, 1);
         __builtin_amdgcn_sched_barrier(0);
-        page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validA, kg);
+        page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validA >> 8, validA & 255, kg);
         __builtin_amdgcn_sched_barrier(0);
         id_next = load_id(it + 2);  // lands while the P V products run
         page_pv<NG>(vA, pr, O);
@@ -258,7 +267,7 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
         __builtin_amdgcn_sched_barrier(0);
         issue_k(r2, 0);
         __builtin_amdgcn_sched_barrier(0);
-        page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validB, kg);
+        page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validB >> 8, validB & 255, kg);
         __builtin_amdgcn_sched_barrier(0);
         id_next = load_id(it + 3);
         page_pv<NG>(vB, pr, O);

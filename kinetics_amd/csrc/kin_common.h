@@ -15,6 +15,10 @@ constexpr int kMaxGroup = 8;     // largest supported num_q_heads / num_kv_heads
 constexpr int kMaxTopk = 2048;
 constexpr int kMaxCandidates = 16384;
 constexpr int kMaxFixedPages = 64;  // most sink / local pages that can be pinned into every list
+constexpr int kMaxLocalTokens = (kMaxFixedPages - 1) * kPageSize + 1;
+
+// Most trailing pages that local_tokens always-attended trailing tokens can span.
+__host__ __device__ inline int max_local_pages(int local_tokens) { return 1 + (local_tokens + kPageSize - 2) / kPageSize; }
 
 // Cache-policy bits for buffer loads of read-once data (K/V pages, mean keys):
 // the non-temporal hint keeps streams from displacing each other in L2/MALL and
@@ -34,6 +38,10 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // Shape rules every entry point shares.  Returns KIN_OK or records an error.
 int check_common_dims(const char* fn, int batch, int num_q_heads, int num_kv_heads,
                       int head_dim, int page_size);
+// Range rules for the always-attended parts of a page list.
+int check_fixed_pages(const char* fn, int sink_pages, int local_tokens);
+// first_page_offset: padding slots at the start of every sequence's first page.
+int check_first_page_offset(const char* fn, int first_page_offset);
 
 // ---- device side -----------------------------------------------------------
 #if defined(__HIPCC__)

@@ -20,6 +20,7 @@ struct DecodeParams {
   float* ws_lse;  // [batch*Hq, splits]      fp32 (log2 domain)
   int num_q_heads, num_kv_heads, group;
   int list_stride, num_splits;
+  int first_page_offset;  // padding slots at the start of list entry 0
   int64_t num_pages;
   float scale_log2;  // sm_scale * log2(e)
 };
@@ -60,6 +61,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
   a.p0 = min(split * per_split, n);
   a.p1 = min(n, a.p0 + per_split);
   a.last_len = p.last_page_len[b];
+  a.first_skip = p.first_page_offset;
 
   // The list is read-only for the whole kernel; the constant address space
   // makes the uniform id load a scalar one (off the vector-memory counter that
@@ -158,9 +160,11 @@ static int launch_decode(const char* fn, DecodeParams& p, int batch, void* works
 
 static int check_decode_args(const char* fn, const void* q, const void* kv_cache, const void* last_page_len,
                              const void* out, int batch, int num_q_heads, int num_kv_heads, int head_dim,
-                             int page_size, int64_t num_pages, int num_splits) {
+                             int page_size, int64_t num_pages, int first_page_offset, int num_splits) {
   if (!q || !kv_cache || !last_page_len || !out) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size);
+  if (st) return st;
+  st = check_first_page_offset(fn, first_page_offset);
   if (st) return st;
   if (num_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_pages=%lld must be >= 1", fn, (long long)num_pages);
   if (num_splits < 0) return fail(KIN_ERR_BAD_SHAPE, "%s: num_splits=%d is negative", fn, num_splits);
@@ -188,13 +192,13 @@ size_t kin_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads, 
 int kin_sparse_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const int32_t* sel_pages,
                             const int32_t* sel_count, const int32_t* last_page_len, kin_bf16_t* out, float* lse,
                             void* workspace, size_t workspace_bytes, int batch, int num_q_heads, int num_kv_heads,
-                            int head_dim, int page_size, int64_t num_pages, int sel_stride, float sm_scale,
-                            int num_splits, kin_stream_t stream) {
+                            int head_dim, int page_size, int64_t num_pages, int sel_stride, int first_page_offset,
+                            float sm_scale, int num_splits, kin_stream_t stream) {
   using namespace kin;
   const char* fn = "kin_sparse_paged_decode";
   if (!sel_pages || !sel_count) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_decode_args(fn, q, kv_cache, last_page_len, out, batch, num_q_heads, num_kv_heads, head_dim,
-                             page_size, num_pages, num_splits);
+                             page_size, num_pages, first_page_offset, num_splits);
   if (st) return st;
   if (sel_stride < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must be >= 1", fn, sel_stride);
   if (batch == 0) return KIN_OK;
@@ -212,6 +216,7 @@ int kin_sparse_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, con
   p.group = num_q_heads / num_kv_heads;
   p.list_stride = sel_stride;
   p.num_pages = num_pages;
+  p.first_page_offset = first_page_offset;
   const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
   p.scale_log2 = scale * 1.4426950408889634f;
   return launch_decode(fn, p, batch, workspace, workspace_bytes, sel_stride, num_splits,
@@ -221,13 +226,13 @@ int kin_sparse_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, con
 int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const int32_t* page_indices,
                            const int32_t* page_indptr, const int32_t* last_page_len, kin_bf16_t* out, float* lse,
                            void* workspace, size_t workspace_bytes, int batch, int num_q_heads, int num_kv_heads,
-                           int head_dim, int page_size, int64_t num_pages, int max_pages_per_seq, float sm_scale,
-                           int num_splits, kin_stream_t stream) {
+                           int head_dim, int page_size, int64_t num_pages, int max_pages_per_seq,
+                           int first_page_offset, float sm_scale, int num_splits, kin_stream_t stream) {
   using namespace kin;
   const char* fn = "kin_dense_paged_decode";
   if (!page_indices || !page_indptr) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_decode_args(fn, q, kv_cache, last_page_len, out, batch, num_q_heads, num_kv_heads, head_dim,
-                             page_size, num_pages, num_splits);
+                             page_size, num_pages, first_page_offset, num_splits);
   if (st) return st;
   if (max_pages_per_seq < 1)
     return fail(KIN_ERR_BAD_SHAPE, "%s: max_pages_per_seq=%d must be >= 1", fn, max_pages_per_seq);
@@ -246,6 +251,7 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, cons
   p.group = num_q_heads / num_kv_heads;
   p.list_stride = 0;
   p.num_pages = num_pages;
+  p.first_page_offset = first_page_offset;
   const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
   p.scale_log2 = scale * 1.4426950408889634f;
   return launch_decode(fn, p, batch, workspace, workspace_bytes, max_pages_per_seq, num_splits,

@@ -10,16 +10,17 @@ struct ScoreTopkParams {
   const uint16_t* kbar;
   const int32_t* page_indices;
   const int32_t* page_indptr;
+  const int32_t* last_page_len;
   int32_t* sel_pages;
   int32_t* sel_count;
   int32_t* sel_logical;  // may be null
   float* scores_out;     // may be null
   int num_q_heads, num_kv_heads, group;
-  int kbar_pages, sel_stride, topk, sink_pages, local_pages;
+  int kbar_pages, sel_stride, topk, sink_pages, local_tokens;
   int sort_cap;
 };
 
-// Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap] | int32 sel[topk + sink + local]
+// Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap] | int32 sel[sink + topk + local]
 template <int UNROLL>
 __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -43,7 +44,7 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
   a.G = p.group;
   a.row_stride_b = p.num_kv_heads * kRowBytes;
   a.n_pages = n_pages;
-  split_pages(n_pages, p.sink_pages, p.local_pages, p.kbar_pages, a.n_sink, a.n_cand, a.n_local);
+  split_pages(n_pages, p.last_page_len[b], p.sink_pages, p.local_tokens, p.kbar_pages, a.n_sink, a.n_cand, a.n_local);
   a.kb = reinterpret_cast<const char*>(p.kbar) +
          (((int64_t)b * p.kbar_pages + a.n_sink) * p.num_kv_heads + h) * kRowBytes;
   a.topk = p.topk;
@@ -62,24 +63,25 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
 }  // namespace kin
 
 extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar, const int32_t* page_indices,
-                                    const int32_t* page_indptr, int topk, int sink_pages, int local_pages,
+                                    const int32_t* page_indptr, const int32_t* last_page_len, int topk,
+                                    int sink_pages, int local_tokens,
                                     int32_t* sel_pages, int32_t* sel_count,
                                     int32_t* sel_logical, float* scores_out, int batch, int num_q_heads,
                                     int num_kv_heads, int head_dim, int kbar_pages, int sel_stride,
                                     kin_stream_t stream) {
   using namespace kin;
   const char* fn = "kin_block_score_topk";
-  if (!q || !kbar || !page_indices || !page_indptr || !sel_pages || !sel_count)
+  if (!q || !kbar || !page_indices || !page_indptr || !last_page_len || !sel_pages || !sel_count)
     return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, kPageSize);
   if (st) return st;
-  if (topk < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: topk=%d must be >= 1", fn, topk);
-  if (sink_pages < 0 || sink_pages > kMaxFixedPages || local_pages < 1 || local_pages > kMaxFixedPages)
-    return fail(KIN_ERR_BAD_SHAPE, "%s: sink_pages=%d must be in [0, %d] and local_pages=%d in [1, %d]", fn, sink_pages,
-                kMaxFixedPages, local_pages, kMaxFixedPages);
-  if (sel_stride < topk + sink_pages + local_pages)
-    return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must be at least topk + sink_pages + local_pages = %d", fn,
-                sel_stride, topk + sink_pages + local_pages);
+  if (topk < 0) return fail(KIN_ERR_BAD_SHAPE, "%s: topk=%d is negative", fn, topk);
+  st = check_fixed_pages(fn, sink_pages, local_tokens);
+  if (st) return st;
+  const int list_cap = topk + sink_pages + max_local_pages(local_tokens);
+  if (sel_stride < list_cap)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must be at least kin_sel_list_capacity(topk, sink_pages, local_tokens) = %d",
+                fn, sel_stride, list_cap);
   if (kbar_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: kbar_pages=%d must be >= 1", fn, kbar_pages);
   if (topk > kMaxTopk) return fail(KIN_ERR_UNSUPPORTED, "%s: topk=%d exceeds the limit %d", fn, topk, kMaxTopk);
   if (kbar_pages > kMaxCandidates)
@@ -92,6 +94,7 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
   p.kbar = kbar;
   p.page_indices = page_indices;
   p.page_indptr = page_indptr;
+  p.last_page_len = last_page_len;
   p.sel_pages = sel_pages;
   p.sel_count = sel_count;
   p.sel_logical = sel_logical;
@@ -103,9 +106,9 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
   p.sel_stride = sel_stride;
   p.topk = topk;
   p.sink_pages = sink_pages;
-  p.local_pages = local_pages;
+  p.local_tokens = local_tokens;
   p.sort_cap = select_sort_cap(topk, kbar_pages);
-  const size_t lds = select_lds_bytes(kbar_pages, p.sort_cap) + (size_t)(topk + sink_pages + local_pages) * 4;
+  const size_t lds = select_lds_bytes(kbar_pages, p.sort_cap) + (size_t)list_cap * 4;
   const int64_t items = (int64_t)batch * num_kv_heads;
   if (items > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   // Few workgroups cannot saturate HBM with 4 loads per lane in flight: give a

@@ -38,7 +38,7 @@ struct SelectArgs {
   int n_pages;                // pages of the sequence (>= 1)
   int n_sink;                 // leading pages that are always attended (not candidates)
   int n_cand;                 // candidates: logical pages n_sink .. n_sink + n_cand - 1
-  int n_local;                // trailing pages that are always attended (>= 1: the open page)
+  int n_local;                // trailing pages that are always attended (>= 1: the open page last)
   int topk;
   const int32_t* table;       // the sequence's page table (logical -> physical)
   int32_t* sel_logical;       // HBM, topk entries, or null
@@ -59,22 +59,24 @@ __host__ __device__ inline int select_sort_cap(int topk, int kbar_pages) {
   return cap;
 }
 
-// Splits a sequence's pages into always-attended leading ("sink") pages,
-// candidates and always-attended trailing ("local") pages; the final local page
-// is the open one.  kbar_pages bounds the logical pages that have a mean key.
-__host__ __device__ inline void split_pages(int n_pages, int sink_pages, int local_pages, int kbar_pages, int& n_sink,
-                                            int& n_cand, int& n_local) {
-  n_local = local_pages < n_pages ? local_pages : n_pages;
-  const int rest = n_pages - n_local;
-  n_sink = sink_pages < rest ? sink_pages : rest;
+// Splits a sequence of n_pages pages (the last one holding last_len tokens)
+// into always-attended leading ("sink") pages, candidates and always-attended
+// trailing ("local") pages.  The candidates are the whole pages between the sink
+// pages and the newest local_tokens tokens, so the open page (local_tokens >= 1)
+// is always local.  kbar_pages bounds the logical pages that have a mean key.
+__host__ __device__ inline void split_pages(int n_pages, int last_len, int sink_pages, int local_tokens,
+                                            int kbar_pages, int& n_sink, int& n_cand, int& n_local) {
+  last_len = last_len < 1 ? 1 : (last_len > kPageSize ? kPageSize : last_len);
+  n_sink = sink_pages < n_pages - 1 ? sink_pages : n_pages - 1;
+  const int between = (n_pages - 1 - n_sink) * kPageSize + last_len - local_tokens;  // tokens after the sink, before the local part
+  n_cand = between > 0 ? between / kPageSize : 0;
+  n_local = n_pages - n_sink - n_cand;
   const int cap = kbar_pages - n_sink;
-  n_cand = rest - n_sink;
-  if (n_cand > cap) n_cand = cap;
-  if (n_cand < 0) n_cand = 0;
+  if (n_cand > cap) n_cand = cap > 0 ? cap : 0;
 }
 
-// Writes the page list to sel_lds (LDS, >= topk + n_sink + n_local entries):
-// the ordered physical ids of the k_eff winners, then the sink pages, then the
+// Writes the page list to sel_lds (LDS, >= n_sink + topk + n_local entries):
+// the sink pages, then the ordered physical ids of the k_eff winners, then the
 // local pages (the open page last).  Returns the list length.  Ends with a
 // workgroup barrier: sel_lds is visible to every thread and keys / sortbuf are
 // free for reuse.
@@ -121,16 +123,18 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
   // next pass as soon as it has consumed it.
   const int row_stride_b = a.row_stride_b;  // bytes between logical pages
   const char* kb = a.kb;
-  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<char*>(kb), 0, n_cand > 0 ? (n_cand - 1) * row_stride_b + kRowBytes : 0, 0x00020000);
   float* sc_out = a.scores_out;
+  // Nothing to choose (topk == 0) and nobody asked for the scores: stream nothing.
+  const int n_score = (k_eff > 0 || sc_out) ? n_cand : 0;
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(kb), 0, n_score > 0 ? (n_score - 1) * row_stride_b + kRowBytes : 0, 0x00020000);
   const int sub = tid >> 4;  // 0..15: which of the 16 rows of a slot this lane helps with
   const int lane_off = sub * row_stride_b + c16 * 16;
   u32x4 w[kUnroll];
 #pragma unroll
   for (int j = 0; j < kUnroll; ++j)
     w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + j * 16 * row_stride_b, 0, kStreamLoad);
-  for (int base = 0; base < n_cand; base += 16 * kUnroll) {
+  for (int base = 0; base < n_score; base += 16 * kUnroll) {
     const int next_off = (base + 16 * kUnroll) * row_stride_b;
 #pragma unroll
     for (int j = 0; j < kUnroll; ++j) {
@@ -143,7 +147,7 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
       acc = fmaf(qm[6], bf16_lo(x.w), acc); acc = fmaf(qm[7], bf16_hi(x.w), acc);
       acc = row16_sum(acc);
       const int row = base + j * 16 + sub;
-      if (c16 == 0 && row < n_cand) {
+      if (c16 == 0 && row < n_score) {
         keys[row] = order_key(acc);
         if (sc_out) sc_out[row] = acc;
       }
@@ -255,7 +259,7 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
 #pragma unroll 8
       for (int j = 0; j < k_eff; ++j) rank += (sortbuf[j] > mine) ? 1 : 0;
       const uint32_t logical = 0xffffffffu - (uint32_t)(mine & 0xffffffffull);
-      sel_lds[rank] = table[a.n_sink + logical];
+      sel_lds[a.n_sink + rank] = table[a.n_sink + logical];
       if (a.sel_logical) a.sel_logical[rank] = (int32_t)(a.n_sink + logical);
     }
   } else {
@@ -278,12 +282,16 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
     }
     for (int i = tid; i < k_eff; i += kThreads) {
       const uint32_t logical = 0xffffffffu - (uint32_t)(sortbuf[i] & 0xffffffffull);
-      sel_lds[i] = table[a.n_sink + logical];
+      sel_lds[a.n_sink + i] = table[a.n_sink + logical];
       if (a.sel_logical) a.sel_logical[i] = (int32_t)(a.n_sink + logical);
     }
   }
-  for (int i = tid; i < a.n_sink + a.n_local; i += kThreads)
-    sel_lds[k_eff + i] = (i < a.n_sink) ? table[i] : table[n_pages - a.n_local + (i - a.n_sink)];
+  for (int i = tid; i < a.n_sink + a.n_local; i += kThreads) {
+    if (i < a.n_sink)
+      sel_lds[i] = table[i];
+    else
+      sel_lds[k_eff + i] = table[n_pages - a.n_local + (i - a.n_sink)];
+  }
   __syncthreads();
   return k_eff + a.n_sink + a.n_local;
 }

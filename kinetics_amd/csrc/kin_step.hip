@@ -27,7 +27,7 @@ struct StepParams {
   uint16_t* out;
   float* lse;  // optional
   int num_q_heads, num_kv_heads, group;
-  int kbar_pages, sel_stride, topk, sink_pages, local_pages, sort_cap;
+  int kbar_pages, sel_stride, topk, sink_pages, local_tokens, first_page_offset, sort_cap;
   int region0_bytes;  // LDS: max(attend staging, select scratch); the page list follows it
   int64_t num_pages;
   float scale_log2;
@@ -98,7 +98,7 @@ __global__ __launch_bounds__(256, 2) void blocktopk_step_kernel(StepParams p) {
   s.G = G;
   s.row_stride_b = p.num_kv_heads * kRowBytes;
   s.n_pages = n_pages;
-  split_pages(n_pages, p.sink_pages, p.local_pages, p.kbar_pages, s.n_sink, s.n_cand, s.n_local);
+  split_pages(n_pages, last_len, p.sink_pages, p.local_tokens, p.kbar_pages, s.n_sink, s.n_cand, s.n_local);
   s.kb = reinterpret_cast<const char*>(p.kbar) +
          (((int64_t)b * p.kbar_pages + s.n_sink) * p.num_kv_heads + h) * kRowBytes;
   s.topk = p.topk;
@@ -129,6 +129,7 @@ __global__ __launch_bounds__(256, 2) void blocktopk_step_kernel(StepParams p) {
   a.p0 = 0;
   a.p1 = n;
   a.last_len = last_len;
+  a.first_skip = p.first_page_offset;
   attend_list<NG>(
       a, [&](int i) -> int { return __builtin_amdgcn_readfirstlane(sel_lds[i]); }, smem, sm_m, sm_l,
       [&](int g, int d, float o, float lse2) {
@@ -142,10 +143,10 @@ __global__ __launch_bounds__(256, 2) void blocktopk_step_kernel(StepParams p) {
 extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
                                          kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
                                          const int32_t* page_indptr, const int32_t* last_page_len, int topk,
-                                         int sink_pages, int local_pages, int32_t* sel_pages, int32_t* sel_count, kin_bf16_t* out, float* lse,
-                                         int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
-                                         int64_t num_pages, int kbar_pages, int sel_stride, float sm_scale,
-                                         kin_stream_t stream) {
+                                         int sink_pages, int local_tokens, int32_t* sel_pages, int32_t* sel_count,
+                                         kin_bf16_t* out, float* lse, int batch, int num_q_heads, int num_kv_heads,
+                                         int head_dim, int page_size, int64_t num_pages, int kbar_pages,
+                                         int sel_stride, int first_page_offset, float sm_scale, kin_stream_t stream) {
   using namespace kin;
   const char* fn = "kin_blocktopk_decode_step";
   if (!q || !kv_cache || !kbar || !page_indices || !page_indptr || !last_page_len || !out)
@@ -155,14 +156,19 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
   int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size);
   if (st) return st;
   if (num_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_pages=%lld must be >= 1", fn, (long long)num_pages);
-  if (topk < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: topk=%d must be >= 1", fn, topk);
+  if (topk < 0) return fail(KIN_ERR_BAD_SHAPE, "%s: topk=%d is negative", fn, topk);
   if (kbar_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: kbar_pages=%d must be >= 1", fn, kbar_pages);
-  if (sink_pages < 0 || sink_pages > kMaxFixedPages || local_pages < 1 || local_pages > kMaxFixedPages)
-    return fail(KIN_ERR_BAD_SHAPE, "%s: sink_pages=%d must be in [0, %d] and local_pages=%d in [1, %d]", fn, sink_pages,
-                kMaxFixedPages, local_pages, kMaxFixedPages);
-  if (sel_pages && sel_stride < topk + sink_pages + local_pages)
-    return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must be at least topk + sink_pages + local_pages = %d", fn,
-                sel_stride, topk + sink_pages + local_pages);
+  st = check_fixed_pages(fn, sink_pages, local_tokens);
+  if (st) return st;
+  st = check_first_page_offset(fn, first_page_offset);
+  if (st) return st;
+  if (first_page_offset > 0 && sink_pages < 1)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: first_page_offset=%d needs sink_pages >= 1 (a padded page has no mean key)", fn,
+                first_page_offset);
+  const int list_cap = topk + sink_pages + max_local_pages(local_tokens);
+  if (sel_pages && sel_stride < list_cap)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must be at least kin_sel_list_capacity(topk, sink_pages, local_tokens) = %d",
+                fn, sel_stride, list_cap);
   if (sel_pages && !sel_count) return fail(KIN_ERR_NULL_POINTER, "%s: sel_pages given without sel_count", fn);
   if (topk > kMaxTopk) return fail(KIN_ERR_UNSUPPORTED, "%s: topk=%d exceeds the limit %d", fn, topk, kMaxTopk);
   if (kbar_pages > kMaxCandidates)
@@ -192,7 +198,8 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
   p.sel_stride = sel_stride;
   p.topk = topk;
   p.sink_pages = sink_pages;
-  p.local_pages = local_pages;
+  p.local_tokens = local_tokens;
+  p.first_page_offset = first_page_offset;
   p.sort_cap = select_sort_cap(topk, kbar_pages);
   const size_t sel_scratch = select_lds_bytes(kbar_pages, p.sort_cap);
   size_t region0 = sel_scratch > (size_t)kAttendLdsBytes ? sel_scratch : (size_t)kAttendLdsBytes;
@@ -201,7 +208,7 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
   p.num_pages = num_pages;
   const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
   p.scale_log2 = scale * 1.4426950408889634f;
-  const size_t lds = region0 + (size_t)(topk + sink_pages + local_pages) * 4;
+  const size_t lds = region0 + (size_t)list_cap * 4;
   const int64_t items = (int64_t)batch * num_kv_heads;
   if (items > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   hipStream_t s = static_cast<hipStream_t>(stream);

@@ -148,15 +148,23 @@ def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len) -> None
 # ---------------------------------------------------------------------------
 
 
-def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count, sel_logical=None, scores_out=None,
-                     sink_pages: int = 0, local_pages: int = 1) -> None:
+def sel_list_capacity(topk: int, sink_pages: int = 0, local_tokens: int = 1) -> int:
+    """Longest page list the selector writes: the stride ``sel_pages`` needs."""
+    return int(_lib.load().kin_sel_list_capacity(int(topk), int(sink_pages), int(local_tokens)))
+
+
+def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sel_logical=None,
+                     scores_out=None, sink_pages: int = 0, local_tokens: int = 1) -> None:
     """Score every candidate page with the group-mean query and write the
     top-``topk`` pages plus the last page into ``sel_pages`` / ``sel_count``
     (in place: fixed buffers, as the reference registers with its decode
     wrapper, benchmark/blocktopk_decoder.py:143,156-159).  Stands in for
-    lines 216-221 of that file.  ``sink_pages`` leading and ``local_pages``
-    trailing pages are always attended and never candidates (0 and 1 give the
-    reference's "top-k plus the last page")."""
+    lines 216-221 of that file.  The first ``sink_pages`` pages and the pages
+    that hold the newest ``local_tokens`` tokens are always attended and never
+    candidates (0 and 1 give the reference's "top-k plus the last page"; 1 and
+    LiteSys' ``local`` on a cache stored 12 slots into its first page give
+    LiteSys/litesys/attention/sparsity_utils.py:24-47).  List order: sink pages,
+    selected pages by descending score, local pages."""
     _require(q, "q", torch.bfloat16, 3)
     dev = q.device
     batch, num_q_heads, head_dim = q.shape
@@ -168,7 +176,9 @@ def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_co
     if tuple(sel_count.shape) != (batch, num_kv_heads):
         raise ValueError(f"sel_count must be [{batch}, {num_kv_heads}], got {tuple(sel_count.shape)}")
     kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim)
-    _table(page_indices, page_indptr, None, batch, dev)
+    _table(page_indices, page_indptr, last_page_len, batch, dev)
+    if last_page_len is None:
+        raise TypeError("last_page_len is required")
     if sel_logical is not None:
         _require(sel_logical, "sel_logical", torch.int32, 3, dev)
         if tuple(sel_logical.shape) != (batch, num_kv_heads, topk):
@@ -181,8 +191,8 @@ def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_co
     with torch.cuda.device(dev):
         _lib.check(
             lib.kin_block_score_topk(
-                _ptr(q), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), int(topk), int(sink_pages), int(local_pages),
-                _ptr(sel_pages), _ptr(sel_count), _ptr(sel_logical), _ptr(scores_out), batch, num_q_heads, num_kv_heads, head_dim,
+                _ptr(q), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), int(topk), int(sink_pages),
+                int(local_tokens), _ptr(sel_pages), _ptr(sel_count), _ptr(sel_logical), _ptr(scores_out), batch, num_q_heads, num_kv_heads, head_dim,
                 kbar_pages, sel_stride, _stream(dev),
             )
         )
@@ -238,10 +248,11 @@ def _workspace(workspace, dev, batch, hq, hkv, max_pages, num_splits):
 
 
 def sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, out=None, lse=None, workspace=None,
-                        sm_scale: float = 0.0, num_splits: int = 0):
+                        sm_scale: float = 0.0, num_splits: int = 0, first_page_offset: int = 0):
     """Attention of one query token per sequence over the listed pages; stands
     in for ``mylib::decode`` (benchmark/blocktopk_decoder.py:171-184,223-225).
-    Returns ``out`` [batch, num_q_heads, head_dim] bf16."""
+    ``first_page_offset`` leading token slots of each list's first page are
+    padding.  Returns ``out`` [batch, num_q_heads, head_dim] bf16."""
     dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, workspace)
     _require(sel_pages, "sel_pages", torch.int32, 3, dev)
     _require(sel_count, "sel_count", torch.int32, 2, dev)
@@ -255,15 +266,15 @@ def sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, out=No
         _lib.check(
             lib.kin_sparse_paged_decode(
                 _ptr(q), _ptr(kv_cache), _ptr(sel_pages), _ptr(sel_count), _ptr(last_page_len), _ptr(out), _ptr(lse),
-                _ptr(workspace), ws_bytes, batch, hq, hkv, d, ps, num_pages, sel_pages.shape[2], float(sm_scale),
-                int(num_splits), _stream(dev),
+                _ptr(workspace), ws_bytes, batch, hq, hkv, d, ps, num_pages, sel_pages.shape[2], int(first_page_offset),
+                float(sm_scale), int(num_splits), _stream(dev),
             )
         )
     return out
 
 
 def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, max_pages_per_seq, out=None, lse=None,
-                       workspace=None, sm_scale: float = 0.0, num_splits: int = 0):
+                       workspace=None, sm_scale: float = 0.0, num_splits: int = 0, first_page_offset: int = 0):
     """Attention over every page of each sequence; the dense baseline
     (benchmark/dense_decoder.py:149-170,211-219)."""
     dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, workspace)
@@ -275,7 +286,7 @@ def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, ma
             lib.kin_dense_paged_decode(
                 _ptr(q), _ptr(kv_cache), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), _ptr(out),
                 _ptr(lse), _ptr(workspace), ws_bytes, batch, hq, hkv, d, ps, num_pages, int(max_pages_per_seq),
-                float(sm_scale), int(num_splits), _stream(dev),
+                int(first_page_offset), float(sm_scale), int(num_splits), _stream(dev),
             )
         )
     return out
@@ -296,7 +307,7 @@ def prefer_fused_step(batch: int, num_kv_heads: int, max_pages_per_seq: int, top
 
 def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, out=None, lse=None,
                           sel_pages=None, sel_count=None, sm_scale: float = 0.0, sink_pages: int = 0,
-                          local_pages: int = 1):
+                          local_tokens: int = 1, first_page_offset: int = 0):
     """append -> score -> select -> attend in one launch: lines 209-225 of the
     reference layer's forward (benchmark/blocktopk_decoder.py) as a single
     kernel.  ``k``/``v`` may be None (no append); ``sel_pages``/``sel_count`` are
@@ -325,9 +336,9 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
         _lib.check(
             lib.kin_blocktopk_decode_step(
                 _ptr(q), _ptr(k), _ptr(v), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
-                _ptr(last_page_len), int(topk), int(sink_pages), int(local_pages), _ptr(sel_pages), _ptr(sel_count), _ptr(out),
-                _ptr(lse), batch, hq, hkv,
-                d, ps, num_pages, kbar_pages, sel_stride, float(sm_scale), _stream(dev),
+                _ptr(last_page_len), int(topk), int(sink_pages), int(local_tokens), _ptr(sel_pages), _ptr(sel_count),
+                _ptr(out), _ptr(lse), batch, hq, hkv, d, ps, num_pages, kbar_pages, sel_stride, int(first_page_offset),
+                float(sm_scale), _stream(dev),
             )
         )
     return out
@@ -389,18 +400,18 @@ torch.library.define(
 )
 torch.library.define(
     "kinetics::block_score_topk",
-    "(Tensor q, Tensor kbar, Tensor page_indices, Tensor page_indptr, int topk, Tensor(a!) sel_pages, "
-    "Tensor(b!) sel_count, int sink_pages=0, int local_pages=1) -> ()",
+    "(Tensor q, Tensor kbar, Tensor page_indices, Tensor page_indptr, Tensor last_page_len, int topk, "
+    "Tensor(a!) sel_pages, Tensor(b!) sel_count, int sink_pages=0, int local_tokens=1) -> ()",
 )
 torch.library.define(
     "kinetics::sparse_paged_decode",
     "(Tensor q, Tensor kv_cache, Tensor sel_pages, Tensor sel_count, Tensor last_page_len, Tensor? workspace, "
-    "float sm_scale, int num_splits) -> Tensor",
+    "float sm_scale, int num_splits, int first_page_offset=0) -> Tensor",
 )
 torch.library.define(
     "kinetics::dense_paged_decode",
     "(Tensor q, Tensor kv_cache, Tensor page_indices, Tensor page_indptr, Tensor last_page_len, "
-    "int max_pages_per_seq, Tensor? workspace, float sm_scale, int num_splits) -> Tensor",
+    "int max_pages_per_seq, Tensor? workspace, float sm_scale, int num_splits, int first_page_offset=0) -> Tensor",
 )
 
 
@@ -408,21 +419,21 @@ torch.library.define(
     "kinetics::blocktopk_decode_step",
     "(Tensor q, Tensor k, Tensor v, Tensor(a!) kv_cache, Tensor(b!) kbar, Tensor page_indices, Tensor page_indptr, "
     "Tensor last_page_len, int topk, Tensor(c!)? sel_pages, Tensor(d!)? sel_count, float sm_scale, "
-    "int sink_pages=0, int local_pages=1) -> Tensor",
+    "int sink_pages=0, int local_tokens=1, int first_page_offset=0) -> Tensor",
 )
 
 
 @torch.library.impl("kinetics::blocktopk_decode_step", "cuda")
 def _step_impl(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sm_scale,
-               sink_pages=0, local_pages=1):
+               sink_pages=0, local_tokens=1, first_page_offset=0):
     return blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk,
                                  sel_pages=sel_pages, sel_count=sel_count, sm_scale=sm_scale, sink_pages=sink_pages,
-                                 local_pages=local_pages)
+                                 local_tokens=local_tokens, first_page_offset=first_page_offset)
 
 
 @torch.library.register_fake("kinetics::blocktopk_decode_step")
 def _step_fake(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sm_scale,
-               sink_pages=0, local_pages=1):
+               sink_pages=0, local_tokens=1, first_page_offset=0):
     return torch.empty_like(q)
 
 
@@ -437,33 +448,38 @@ def _append_fake(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len)
 
 
 @torch.library.impl("kinetics::block_score_topk", "cuda")
-def _select_impl(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count, sink_pages=0, local_pages=1):
-    block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count, sink_pages=sink_pages,
-                     local_pages=local_pages)
+def _select_impl(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sink_pages=0,
+                 local_tokens=1):
+    block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count,
+                     sink_pages=sink_pages, local_tokens=local_tokens)
 
 
 @torch.library.register_fake("kinetics::block_score_topk")
-def _select_fake(q, kbar, page_indices, page_indptr, topk, sel_pages, sel_count, sink_pages=0, local_pages=1):
+def _select_fake(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sink_pages=0,
+                 local_tokens=1):
     return None
 
 
 @torch.library.impl("kinetics::sparse_paged_decode", "cuda")
-def _sparse_impl(q, kv_cache, sel_pages, sel_count, last_page_len, workspace, sm_scale, num_splits):
+def _sparse_impl(q, kv_cache, sel_pages, sel_count, last_page_len, workspace, sm_scale, num_splits, first_page_offset=0):
     return sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, workspace=workspace,
-                               sm_scale=sm_scale, num_splits=num_splits)
+                               sm_scale=sm_scale, num_splits=num_splits, first_page_offset=first_page_offset)
 
 
 @torch.library.register_fake("kinetics::sparse_paged_decode")
-def _sparse_fake(q, kv_cache, sel_pages, sel_count, last_page_len, workspace, sm_scale, num_splits):
+def _sparse_fake(q, kv_cache, sel_pages, sel_count, last_page_len, workspace, sm_scale, num_splits, first_page_offset=0):
     return torch.empty_like(q)
 
 
 @torch.library.impl("kinetics::dense_paged_decode", "cuda")
-def _dense_impl(q, kv_cache, page_indices, page_indptr, last_page_len, max_pages_per_seq, workspace, sm_scale, num_splits):
+def _dense_impl(q, kv_cache, page_indices, page_indptr, last_page_len, max_pages_per_seq, workspace, sm_scale, num_splits,
+                first_page_offset=0):
     return dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, max_pages_per_seq,
-                              workspace=workspace, sm_scale=sm_scale, num_splits=num_splits)
+                              workspace=workspace, sm_scale=sm_scale, num_splits=num_splits,
+                              first_page_offset=first_page_offset)
 
 
 @torch.library.register_fake("kinetics::dense_paged_decode")
-def _dense_fake(q, kv_cache, page_indices, page_indptr, last_page_len, max_pages_per_seq, workspace, sm_scale, num_splits):
+def _dense_fake(q, kv_cache, page_indices, page_indptr, last_page_len, max_pages_per_seq, workspace, sm_scale, num_splits,
+                first_page_offset=0):
     return torch.empty_like(q)

@@ -26,6 +26,10 @@ algorithm of the reference's block top-k decoder path:
                     P.V) with the new token attended
                     (LiteSys/litesys/attention/batch_cache.py:154-168)
 * dense baseline    benchmark/dense_decoder.py:211-219
+* LiteSys' mask form LiteSys/litesys/attention/sparsity_utils.py:24-47 on a
+                    contiguous cache (litesys_decode), the cross-check that the
+                    page lists with sink_pages=1, local_tokens=local and a
+                    12-slot first-page offset are the same function
 
 flashinfer 0.1.6 (the wheel the reference calls, README.md:81) is not in the
 reference tree; its page-table convention is restated here: sequence b owns
@@ -146,20 +150,25 @@ def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len):
 # ---------------------------------------------------------------------------
 
 
-def split_pages(n_pages, sink_pages, local_pages, kbar_pages):
-    """(n_sink, n_cand, n_local): trailing ``local_pages`` pages (at least the
-    open page) and leading ``sink_pages`` pages are always attended; the pages in
-    between are the candidates.  sink 0 / local 1 is the reference's rule
-    (benchmark/blocktopk_decoder.py:220); larger values are the page-aligned form
-    of LiteSys' sink tokens and local window (sparsity_utils.py:24-35)."""
-    n_local = min(local_pages, n_pages)
-    rest = n_pages - n_local
-    n_sink = min(sink_pages, rest)
-    n_cand = max(0, min(rest - n_sink, kbar_pages - n_sink))
+def split_pages(n_pages, last_len, sink_pages, local_tokens, kbar_pages):
+    """(n_sink, n_cand, n_local).  The first ``sink_pages`` pages (never the
+    open page) and the pages that hold the newest ``local_tokens`` tokens are
+    always attended; the candidates are the whole pages in between.  sink 0 /
+    local 1 is the reference's rule (benchmark/blocktopk_decoder.py:220).  With
+    the sequence stored 12 slots into its first page, sink 1 / local = LiteSys'
+    ``local`` is LiteSys/litesys/attention/sparsity_utils.py:31-33:
+    ``_n_dynamic = (seq_len - local - sink) // block_size * block_size`` with
+    sink = 4, the rest of the tokens being the local part.  Candidates beyond
+    ``kbar_pages`` have no mean key and are dropped."""
+    n_sink = min(sink_pages, n_pages - 1)
+    kv_len = (n_pages - 1) * 16 + min(max(int(last_len), 1), 16)
+    n_cand = max(0, (kv_len - 16 * n_sink - local_tokens) // 16)
+    n_local = n_pages - n_sink - n_cand
+    n_cand = max(0, min(n_cand, kbar_pages - n_sink))
     return n_sink, n_cand, n_local
 
 
-def block_scores(q, kbar, page_indptr, sink_pages=0, local_pages=1):
+def block_scores(q, kbar, page_indptr, last_page_len, sink_pages=0, local_tokens=1):
     """score[b][h][n] = mean_g q[b, h*G+g, :] . kbar[b, n_sink + n, h, :] in
     float64 over the candidate pages.  Returns a list (b) of lists (h) of
     float64 arrays."""
@@ -170,7 +179,10 @@ def block_scores(q, kbar, page_indptr, sink_pages=0, local_pages=1):
     out = []
     for b in range(B):
         n_pages = int(page_indptr[b + 1]) - int(page_indptr[b])
-        n_sink, n_cand, _ = split_pages(max(n_pages, 0), sink_pages, local_pages, kbar.shape[1])
+        if n_pages <= 0:
+            out.append([np.zeros(0) for _ in range(Hkv)])
+            continue
+        n_sink, n_cand, _ = split_pages(n_pages, last_page_len[b], sink_pages, local_tokens, kbar.shape[1])
         kb = bf16_to_f32(kbar[b, n_sink : n_sink + n_cand]).astype(np.float64)  # [n, Hkv, D]
         per_head = []
         for h in range(Hkv):
@@ -194,15 +206,21 @@ def select_topk(scores: np.ndarray, k: int) -> np.ndarray:
     return order[: min(k, n)].astype(np.int64)
 
 
-def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_stride=None, sink_pages=0, local_pages=1):
+def sel_list_capacity(topk, sink_pages=0, local_tokens=1):
+    """Longest list block_score_topk can produce."""
+    return topk + sink_pages + 1 + (local_tokens + 14) // 16
+
+
+def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_stride=None, sink_pages=0,
+                     local_tokens=1):
     """Returns (sel_pages [B,Hkv,stride] int32 padded with -1, sel_count [B,Hkv],
     sel_logical list[b][h] of logical page index arrays, scores list[b][h] over
-    the candidates).  List order: winners (descending score), sink pages, local
+    the candidates).  List order: sink pages, winners (descending score), local
     pages with the open page last."""
     B = q.shape[0]
     Hkv = kbar.shape[2]
-    stride = topk + sink_pages + local_pages if sel_stride is None else sel_stride
-    scores = block_scores(q, kbar, page_indptr, sink_pages, local_pages)
+    stride = sel_list_capacity(topk, sink_pages, local_tokens) if sel_stride is None else sel_stride
+    scores = block_scores(q, kbar, page_indptr, last_page_len, sink_pages, local_tokens)
     sel_pages = np.full((B, Hkv, stride), -1, dtype=np.int32)
     sel_count = np.zeros((B, Hkv), dtype=np.int32)
     sel_logical = []
@@ -213,12 +231,11 @@ def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_stride=None, 
             if len(pages) == 0:
                 row.append(np.zeros(0, dtype=np.int64))
                 continue
-            n_sink, _, n_local = split_pages(len(pages), sink_pages, local_pages, kbar.shape[1])
+            n_sink, _, n_local = split_pages(len(pages), last_page_len[b], sink_pages, local_tokens, kbar.shape[1])
             idx = n_sink + select_topk(scores[b][h], topk)
-            fixed = np.concatenate([pages[:n_sink], pages[len(pages) - n_local :]])
-            sel_pages[b, h, : len(idx)] = pages[idx]
-            sel_pages[b, h, len(idx) : len(idx) + len(fixed)] = fixed
-            sel_count[b, h] = len(idx) + len(fixed)
+            full = np.concatenate([pages[:n_sink], pages[idx], pages[len(pages) - n_local :]])
+            sel_pages[b, h, : len(full)] = full
+            sel_count[b, h] = len(full)
             row.append(idx)
         sel_logical.append(row)
     return sel_pages, sel_count, sel_logical, scores
@@ -229,12 +246,13 @@ def block_score_topk(q, kbar, page_indices, page_indptr, topk, sel_stride=None, 
 # ---------------------------------------------------------------------------
 
 
-def attend_pages(q_bh, kv_cache, pages, h, last_len, sm_scale):
+def attend_pages(q_bh, kv_cache, pages, h, last_len, sm_scale, first_skip=0):
     """LiteSys cache_utils.py:54-169 restated for pages: logits * scale, softmax in
     one pass over the valid tokens, P.V.
     Softmax attention of the G query rows ``q_bh`` ([G, D] float64) over the
     tokens of ``pages`` for KV head ``h``; every page full except the final one
-    (``last_len`` tokens).  Returns (out [G, D] float64, lse [G] float64,
+    (``last_len`` tokens); the first ``first_skip`` token slots of the first
+    listed page are padding.  Returns (out [G, D] float64, lse [G] float64,
     natural log)."""
     G, D = q_bh.shape
     if len(pages) == 0:
@@ -243,7 +261,9 @@ def attend_pages(q_bh, kv_cache, pages, h, last_len, sm_scale):
     K = bf16_to_f32(kv_cache[np.asarray(pages), 0, :, h, :]).astype(np.float64).reshape(-1, D)
     V = bf16_to_f32(kv_cache[np.asarray(pages), 1, :, h, :]).astype(np.float64).reshape(-1, D)
     n_tok = (len(pages) - 1) * ps + int(last_len)
-    K, V = K[:n_tok], V[:n_tok]
+    K, V = K[first_skip:n_tok], V[first_skip:n_tok]
+    if len(K) == 0:
+        return np.zeros((G, D)), np.full(G, -np.inf)
     logits = (q_bh @ K.T) * sm_scale  # [G, n_tok]
     m = logits.max(axis=1, keepdims=True)
     p = np.exp(logits - m)
@@ -251,7 +271,7 @@ def attend_pages(q_bh, kv_cache, pages, h, last_len, sm_scale):
     return (p / s) @ V, (m + np.log(s))[:, 0]
 
 
-def sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, sm_scale=None):
+def sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, sm_scale=None, first_page_offset=0):
     """benchmark/blocktopk_decoder.py:223-225.  out [B, Hq, D] float64 and lse
     [B, Hq] float64 over the listed pages."""
     B, Hq, D = q.shape
@@ -264,13 +284,13 @@ def sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, sm_sca
     for b in range(B):
         for h in range(Hkv):
             pages = sel_pages[b, h, : int(sel_count[b, h])]
-            o, l = attend_pages(qf[b, h * G : (h + 1) * G], kv_cache, pages, h, last_page_len[b], scale)
+            o, l = attend_pages(qf[b, h * G : (h + 1) * G], kv_cache, pages, h, last_page_len[b], scale, first_page_offset)
             out[b, h * G : (h + 1) * G] = o
             lse[b, h * G : (h + 1) * G] = l
     return out, lse
 
 
-def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, sm_scale=None):
+def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, sm_scale=None, first_page_offset=0):
     """Attention over every page of each sequence -- benchmark/dense_decoder.py:211-219."""
     B, Hq, D = q.shape
     Hkv = kv_cache.shape[3]
@@ -282,7 +302,7 @@ def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, sm
     for b in range(B):
         pages = seq_pages(page_indices, page_indptr, b)
         for h in range(Hkv):
-            o, l = attend_pages(qf[b, h * G : (h + 1) * G], kv_cache, pages, h, last_page_len[b], scale)
+            o, l = attend_pages(qf[b, h * G : (h + 1) * G], kv_cache, pages, h, last_page_len[b], scale, first_page_offset)
             out[b, h * G : (h + 1) * G] = o
             lse[b, h * G : (h + 1) * G] = l
     return out, lse
@@ -310,14 +330,69 @@ def merge_partials(outs, lses):
 
 
 def decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sm_scale=None, sink_pages=0,
-                local_pages=1):
+                local_tokens=1, first_page_offset=0):
     """append -> score -> select -> attend.  Mutates kv_cache / kbar.  Returns
     dict(out, lse, sel_pages, sel_count, sel_logical, scores)."""
     append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len)
-    sel_pages, sel_count, sel_logical, scores = block_score_topk(q, kbar, page_indices, page_indptr, topk,
-                                                                 sink_pages=sink_pages, local_pages=local_pages)
-    out, lse = sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, sm_scale)
+    sel_pages, sel_count, sel_logical, scores = block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk,
+                                                                 sink_pages=sink_pages, local_tokens=local_tokens)
+    out, lse = sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, sm_scale, first_page_offset)
     return dict(out=out, lse=lse, sel_pages=sel_pages, sel_count=sel_count, sel_logical=sel_logical, scores=scores)
+
+
+# ---------------------------------------------------------------------------
+# LiteSys' own formulation on a contiguous cache (mask on full logits)
+# ---------------------------------------------------------------------------
+
+
+def litesys_blockwise_topk_mask(mean_logits, seq_len, topk_block, local, sink=4, block_size=16):
+    """LiteSys/litesys/attention/sparsity_utils.py:24-47 for one sequence and one
+    KV head.  ``mean_logits`` [seq_len]: the logits averaged over the query group
+    (:36).  Returns a bool array [seq_len], True where a token stays attended:
+    everything when ``seq_len <= n_full`` (:27-32), otherwise the ``sink`` first
+    tokens, the top ``topk_block`` blocks of the dynamic part by block-mean logit
+    (:37-45) and the ``_local`` newest tokens (:33-35)."""
+    n_full = sink + local + topk_block * block_size
+    n_full = (n_full + block_size - 1) // block_size * block_size
+    keep = np.ones(seq_len, dtype=bool)
+    if seq_len <= n_full:
+        return keep
+    n_dynamic = (seq_len - local - sink) // block_size * block_size
+    n_local = seq_len - n_dynamic - sink
+    dyn = np.asarray(mean_logits[sink : seq_len - n_local], dtype=np.float64)
+    block_means = dyn.reshape(-1, block_size).mean(axis=1)
+    top = select_topk(block_means, topk_block)
+    block_keep = np.zeros(len(block_means), dtype=bool)
+    block_keep[top] = True
+    keep[sink : seq_len - n_local] = np.repeat(block_keep, block_size)
+    return keep
+
+
+def litesys_decode(q, K, V, topk_block, local, sink=4, block_size=16, sm_scale=None):
+    """One sequence of LiteSys' sparse decode on its contiguous cache
+    (LiteSys/litesys/attention/batch_cache.py:154-168): logits of every token
+    (cache_utils.py:54-93, scale 1/sqrt(D)), blockwise_topk_sparsity per KV head
+    on the group-mean logits (sparsity_utils.py:24-47), softmax over what stays
+    (cache_utils.py:216-226), P.V (cache_utils.py:97-169).  q [Hq, D], K / V
+    [seq_len, Hkv, D] float (the new token included).  ``topk_block=None`` is the
+    dense layer.  Returns (out [Hq, D] float64, keep [Hkv, seq_len] bool)."""
+    q = np.asarray(q, dtype=np.float64)
+    K = np.asarray(K, dtype=np.float64)
+    V = np.asarray(V, dtype=np.float64)
+    Hq, D = q.shape
+    seq_len, Hkv, _ = K.shape
+    G = Hq // Hkv
+    scale = 1.0 / np.sqrt(D) if sm_scale is None else sm_scale
+    out = np.zeros((Hq, D))
+    keep_all = np.ones((Hkv, seq_len), dtype=bool)
+    for h in range(Hkv):
+        logits = (q[h * G : (h + 1) * G] @ K[:, h, :].T) * scale  # [G, seq_len]
+        if topk_block is not None:
+            keep_all[h] = litesys_blockwise_topk_mask(logits.mean(axis=0), seq_len, topk_block, local, sink, block_size)
+        masked = np.where(keep_all[h][None, :], logits, -np.inf)
+        p = np.exp(masked - masked.max(axis=1, keepdims=True))
+        out[h * G : (h + 1) * G] = (p / p.sum(axis=1, keepdims=True)) @ V[:, h, :]
+    return out, keep_all
 
 
 # ---------------------------------------------------------------------------

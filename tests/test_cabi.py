@@ -58,19 +58,24 @@ def test_append_argument_errors(lib):
     assert append(lib, B=0) == _lib.KIN_OK  # nothing to do, nothing launched
 
 
-def select(lib, q=A, kbar=A, idx=A, ptr=A, topk=4, sel=A, cnt=A, B=2, Hq=4, Hkv=1, D=128, kp=64, stride=5, sink=0, local=1):
-    return lib.kin_block_score_topk(q, kbar, idx, ptr, topk, sink, local, sel, cnt, None, None, B, Hq, Hkv, D, kp, stride, None)
+def select(lib, q=A, kbar=A, idx=A, ptr=A, last=A, topk=4, sel=A, cnt=A, B=2, Hq=4, Hkv=1, D=128, kp=64, stride=5, sink=0,
+           local=1):
+    return lib.kin_block_score_topk(q, kbar, idx, ptr, last, topk, sink, local, sel, cnt, None, None, B, Hq, Hkv, D, kp,
+                                    stride, None)
 
 
 def test_select_argument_errors(lib):
     assert select(lib, q=None) == _lib.KIN_ERR_NULL_POINTER
     assert select(lib, cnt=None) == _lib.KIN_ERR_NULL_POINTER
-    assert select(lib, topk=0) == _lib.KIN_ERR_BAD_SHAPE
+    assert select(lib, last=None) == _lib.KIN_ERR_NULL_POINTER
+    assert select(lib, topk=-1) == _lib.KIN_ERR_BAD_SHAPE
     assert select(lib, stride=4) == _lib.KIN_ERR_BAD_SHAPE          # no room for the last page
     assert select(lib, stride=5, sink=1) == _lib.KIN_ERR_BAD_SHAPE  # nor for a sink page on top
+    assert select(lib, stride=5, local=2) == _lib.KIN_ERR_BAD_SHAPE  # 2 local tokens can span 2 pages
+    assert b"kin_sel_list_capacity" in lib.kin_last_error()
     assert select(lib, local=0) == _lib.KIN_ERR_BAD_SHAPE           # the open page is always attended
     assert select(lib, sink=-1) == _lib.KIN_ERR_BAD_SHAPE
-    assert select(lib, stride=200, local=65) == _lib.KIN_ERR_BAD_SHAPE
+    assert select(lib, stride=200, local=1010) == _lib.KIN_ERR_BAD_SHAPE
     assert select(lib, Hq=5, Hkv=2) == _lib.KIN_ERR_BAD_SHAPE
     assert select(lib, Hq=16, Hkv=1) == _lib.KIN_ERR_UNSUPPORTED    # group 16 > 8
     assert select(lib, topk=4096, stride=4097) == _lib.KIN_ERR_UNSUPPORTED
@@ -80,8 +85,8 @@ def test_select_argument_errors(lib):
 
 
 def sparse(lib, q=A, kv=A, sel=A, cnt=A, last=A, out=A, ws=None, wsb=0, B=2, Hq=4, Hkv=1, D=128, ps=16, P=8,
-           stride=5, splits=1):
-    return lib.kin_sparse_paged_decode(q, kv, sel, cnt, last, out, None, ws, wsb, B, Hq, Hkv, D, ps, P, stride, 0.0,
+           stride=5, splits=1, offset=0):
+    return lib.kin_sparse_paged_decode(q, kv, sel, cnt, last, out, None, ws, wsb, B, Hq, Hkv, D, ps, P, stride, offset, 0.0,
                                        splits, None)
 
 
@@ -90,6 +95,8 @@ def test_decode_argument_errors(lib):
     assert sparse(lib, sel=None) == _lib.KIN_ERR_NULL_POINTER
     assert sparse(lib, stride=0) == _lib.KIN_ERR_BAD_SHAPE
     assert sparse(lib, splits=-1) == _lib.KIN_ERR_BAD_SHAPE
+    assert sparse(lib, offset=16) == _lib.KIN_ERR_BAD_SHAPE
+    assert sparse(lib, offset=-1) == _lib.KIN_ERR_BAD_SHAPE
     assert sparse(lib, D=256) == _lib.KIN_ERR_UNSUPPORTED
     assert sparse(lib, q=A + 4) == _lib.KIN_ERR_MISALIGNED
     # split-K without (enough) workspace
@@ -99,10 +106,42 @@ def test_decode_argument_errors(lib):
     assert sparse(lib, splits=3, ws=A, wsb=need - 1) == _lib.KIN_ERR_WORKSPACE
     assert b"workspace" in lib.kin_last_error()
     assert sparse(lib, B=0) == _lib.KIN_OK
-    dense = lib.kin_dense_paged_decode(A, A, None, A, A, A, None, None, 0, 2, 4, 1, 128, 16, 8, 9, 0.0, 1, None)
+    dense = lib.kin_dense_paged_decode(A, A, None, A, A, A, None, None, 0, 2, 4, 1, 128, 16, 8, 9, 0, 0.0, 1, None)
     assert dense == _lib.KIN_ERR_NULL_POINTER
-    dense = lib.kin_dense_paged_decode(A, A, A, A, A, A, None, None, 0, 2, 4, 1, 128, 16, 8, 0, 0.0, 1, None)
+    dense = lib.kin_dense_paged_decode(A, A, A, A, A, A, None, None, 0, 2, 4, 1, 128, 16, 8, 0, 0, 0.0, 1, None)
     assert dense == _lib.KIN_ERR_BAD_SHAPE
+    dense = lib.kin_dense_paged_decode(A, A, A, A, A, A, None, None, 0, 2, 4, 1, 128, 16, 8, 9, 16, 0.0, 1, None)
+    assert dense == _lib.KIN_ERR_BAD_SHAPE
+
+
+def step(lib, q=A, k=A, v=A, kv=A, kbar=A, idx=A, ptr=A, last=A, topk=4, sink=0, local=1, sel=None, cnt=None, out=A, B=2,
+         Hq=4, Hkv=1, D=128, ps=16, P=8, kp=64, stride=0, offset=0):
+    return lib.kin_blocktopk_decode_step(q, k, v, kv, kbar, idx, ptr, last, topk, sink, local, sel, cnt, out, None, B, Hq, Hkv,
+                                         D, ps, P, kp, stride, offset, 0.0, None)
+
+
+def test_step_argument_errors(lib):
+    assert step(lib, kbar=None) == _lib.KIN_ERR_NULL_POINTER
+    assert step(lib, v=None) == _lib.KIN_ERR_NULL_POINTER            # k without v
+    assert step(lib, topk=-1) == _lib.KIN_ERR_BAD_SHAPE
+    assert step(lib, local=0) == _lib.KIN_ERR_BAD_SHAPE
+    assert step(lib, offset=16) == _lib.KIN_ERR_BAD_SHAPE
+    assert step(lib, offset=12) == _lib.KIN_ERR_BAD_SHAPE            # a padded first page must be a sink page
+    assert b"sink_pages" in lib.kin_last_error()
+    assert step(lib, sel=A, cnt=A, stride=4) == _lib.KIN_ERR_BAD_SHAPE
+    assert step(lib, sel=A, stride=5) == _lib.KIN_ERR_NULL_POINTER   # list without its count
+    assert step(lib, topk=4096) == _lib.KIN_ERR_UNSUPPORTED
+    assert step(lib, out=A + 2) == _lib.KIN_ERR_MISALIGNED
+    assert step(lib, B=0, sink=1, offset=12) == _lib.KIN_OK
+
+
+def test_sel_list_capacity(lib):
+    assert lib.kin_sel_list_capacity(128, 0, 1) == 129               # the reference's k + 1
+    assert lib.kin_sel_list_capacity(64, 1, 16) == 64 + 1 + 2
+    assert lib.kin_sel_list_capacity(64, 1, 17) == 64 + 1 + 2
+    assert lib.kin_sel_list_capacity(64, 1, 18) == 64 + 1 + 3
+    assert lib.kin_sel_list_capacity(0, 0, 1) == 1
+    assert lib.kin_sel_list_capacity(4, 0, 0) == 0
 
 
 def test_auto_splits_policy(lib):
@@ -114,7 +153,7 @@ def test_auto_splits_policy(lib):
 
 def test_python_wrapper_maps_status_to_exceptions():
     with pytest.raises(ValueError, match="KIN_ERR_BAD_SHAPE"):
-        _lib.check(_lib.load().kin_block_score_topk(A, A, A, A, 0, 0, 1, A, A, None, None, 2, 4, 1, 128, 64, 5, None))
+        _lib.check(_lib.load().kin_block_score_topk(A, A, A, A, A, -1, 0, 1, A, A, None, None, 2, 4, 1, 128, 64, 5, None))
     with pytest.raises(_lib.KineticsError, match="KIN_ERR_WORKSPACE"):
         _lib.check(sparse(_lib.load(), splits=3))
 

@@ -40,7 +40,9 @@ def test_rejects_what_it_does_not_implement():
 
 
 @pytest.mark.parametrize("sparse,fused", [(dict(), None), (dict(attn_block_topk=3, attn_local=16), True),
-                                          (dict(attn_block_topk=3, attn_local=16), False)])
+                                          (dict(attn_block_topk=3, attn_local=16), False),
+                                          (dict(attn_block_topk=2, attn_local=21), True),
+                                          (dict(attn_local=24), False)])
 def test_prefill_then_decode_like_litesys(sparse, fused):
     torch.manual_seed(5)
     m = make_manager(**sparse)
@@ -48,6 +50,18 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
         m._fused = fused          # both routes of decode(): one launch, or append + select + attend
     L, Hq, Hkv = 2, 4, 2
     hist = {}  # (layer, slot) -> (K [t, Hkv, D], V) float32 of the bf16 values fed so far
+
+    pad = 12 if sparse else 0
+    topk_block, local = sparse.get("attn_block_topk", 0), sparse.get("attn_local")
+    gen = torch.Generator().manual_seed(11)
+    block_bias = torch.randn(64, Hkv, 1, generator=gen) * 0.5   # separates the block scores well beyond bf16 rounding
+
+    def keys(slot_len, n, bsz=1):
+        """n new key rows per sequence that start at token slot_len: N(0,1) plus
+        a per-(LiteSys block, head) shift."""
+        t = torch.arange(slot_len, slot_len + n)
+        blk = torch.clamp((t - 4) // PS + 1, min=0)
+        return bf(torch.randn(bsz, Hkv, n, D) + block_bias[blk].permute(1, 0, 2)[None]).to(DEV)
 
     def feed(layer, slot, k, v):  # k, v: [Hkv, s, D] bf16
         K, V = hist.get((layer, slot), (torch.zeros(0, Hkv, D), torch.zeros(0, Hkv, D)))
@@ -69,7 +83,8 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
     for slot, lens in ((0, [PS * 7 + 5]), (2, [PS * 3]), (5, [PS * 2 + 1, PS * 6 + 9])):
         for s in lens:
             for layer in range(L):
-                q, k, v = bf(torch.randn(1, Hq, s, D, device=DEV)), bf(torch.randn(1, Hkv, s, D, device=DEV)), bf(torch.randn(1, Hkv, s, D, device=DEV))
+                q, v = bf(torch.randn(1, Hq, s, D, device=DEV)), bf(torch.randn(1, Hkv, s, D, device=DEV))
+                k = keys(int(m.kv_offset[layer][slot].item()), s)
                 feed(layer, slot, k[0], v[0])
                 out = m.compute_attention(q, k, v, layer, torch.tensor([slot]))
                 assert out.shape == (1, s, Hq * D)
@@ -80,7 +95,8 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
     def decode_round(batch_slots):
         for layer in range(L):
             bsz = len(batch_slots)
-            q, k, v = bf(torch.randn(bsz, Hq, 1, D, device=DEV)), bf(torch.randn(bsz, Hkv, 1, D, device=DEV)), bf(torch.randn(bsz, Hkv, 1, D, device=DEV))
+            q, v = bf(torch.randn(bsz, Hq, 1, D, device=DEV)), bf(torch.randn(bsz, Hkv, 1, D, device=DEV))
+            k = torch.cat([keys(int(m.kv_offset[layer][slot].item()), 1) for slot in batch_slots])
             kv_before, kbar_before = P.from_torch(m.kv_cache[layer]), P.from_torch(m.kbar[layer])
             off_before = m.kv_offset[layer].cpu().numpy().copy()
             out = m.compute_attention(q, k, v, layer, torch.tensor(batch_slots))
@@ -94,11 +110,11 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
                 K, V = hist[(layer, slot)]
                 t = K.shape[0]
                 assert m.kv_offset[layer][slot].item() == t == off_before[slot] + 1
-                got_k = view[slot, :, 0].reshape(-1, Hkv, D)[:t].float().cpu()
+                got_k = view[slot, :, 0].reshape(-1, Hkv, D)[pad:pad + t].float().cpu()
                 assert torch.equal(got_k, K)
             # oracle on the manager's own state before the call
             lens = np.zeros(6, dtype=np.int64)
-            lens[batch_slots] = off_before[batch_slots] + 1
+            lens[batch_slots] = off_before[batch_slots] + 1 + pad
             n_pages = (lens + PS - 1) // PS
             indptr = np.zeros(7, dtype=np.int32)
             indptr[1:] = np.cumsum(n_pages)
@@ -113,25 +129,29 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
             qf[batch_slots], kf[batch_slots], vf[batch_slots] = P.from_torch(q[:, :, 0]), P.from_torch(k[:, :, 0]), P.from_torch(v[:, :, 0])
             is_sparse = bool(sparse) and layer not in (0,)   # layer 0 stays dense (attn_layer_skip default)
             if is_sparse:
-                # first page (sink) and the last ceil(local/16)+1 pages are pinned, 3 blocks chosen in between
-                res = O.decode_step(qf, kf, vf, kv_before, kbar_before, idx, indptr, last, sparse["attn_block_topk"],
-                                    sink_pages=1, local_pages=2)
+                # the paged oracle on the manager's own state: one sink page, `local` newest tokens, 12 padding slots
+                res = O.decode_step(qf, kf, vf, kv_before, kbar_before, idx, indptr, last, topk_block,
+                                    sink_pages=1, local_tokens=local, first_page_offset=pad)
                 want = res["out"]
                 # really sparse for the long sequences: fewer pages than the context has
-                assert res["sel_count"][batch_slots].max() == sparse["attn_block_topk"] + 3
                 assert res["sel_count"][batch_slots].max() < n_pages[batch_slots].max()
             else:
                 O.append_paged_kv(kf, vf, kv_before, kbar_before, idx, indptr, last)
-                want, _ = O.dense_paged_decode(qf, kv_before, idx, indptr, last)
+                want, _ = O.dense_paged_decode(qf, kv_before, idx, indptr, last, first_page_offset=pad)
             assert np.array_equal(P.from_torch(m.kv_cache[layer]), kv_before)
             assert np.array_equal(P.from_torch(m.kbar[layer]), kbar_before)
             got = out.float().cpu().numpy().reshape(bsz, Hq, D)
             err = np.abs(got - want[batch_slots])
             assert np.all(err <= 2e-2 + 2e-2 * np.abs(want[batch_slots]))
-            if not is_sparse:  # dense layers also equal the contiguous-cache restatement
-                for i, slot in enumerate(batch_slots):
-                    ref = dense_ref(layer, slot, q[i])[:, 0]
-                    assert torch.allclose(torch.from_numpy(got[i]).float(), ref, rtol=2e-2, atol=2e-2)
+            # and LiteSys' own formulation on the contiguous history that was fed: full logits, its mask
+            # (4 sink tokens, blocks from token 4, `local` newest tokens), softmax, P.V
+            for i, slot in enumerate(batch_slots):
+                K, V = hist[(layer, slot)]
+                ref, keep = O.litesys_decode(q[i, :, 0].float().cpu().numpy(), K.numpy(), V.numpy(),
+                                             topk_block if is_sparse else None, local)
+                if is_sparse and K.shape[0] > 100:
+                    assert not keep.all()
+                assert np.all(np.abs(got[i] - ref) <= 2e-2 + 2e-2 * np.abs(ref)), (layer, slot)
 
     for _ in range(12):           # crosses page boundaries (mean keys refreshed) for every slot
         decode_round([0, 2, 5])

@@ -98,13 +98,13 @@ def test_build_kbar_bit_exact(ops):
 
 def run_select(ops, g: Gpu):
     pb = g.pb
-    ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, pb.topk, g.sel, g.cnt, g.logical, g.scores)
+    ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, pb.topk, g.sel, g.cnt, g.logical, g.scores)
     torch.cuda.synchronize()
     return g.sel.cpu().numpy(), g.cnt.cpu().numpy(), g.logical.cpu().numpy(), g.scores.cpu().numpy()
 
 
 def check_selection(pb, sel, cnt, logical, scores, exact=False):
-    want_sel, want_cnt, want_logical, want_scores = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    want_sel, want_cnt, want_logical, want_scores = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
     assert np.array_equal(cnt, want_cnt)
     for b in range(pb.B):
         pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
@@ -176,7 +176,7 @@ def test_score_topk_many_candidates(ops):
 
 
 def oracle_sparse(pb, kv=None):
-    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
     out, lse = O.sparse_paged_decode(pb.q, pb.kv_cache if kv is None else kv, sel, cnt, pb.last_page_len)
     return sel, cnt, out, lse
 
@@ -220,7 +220,7 @@ def test_dense_decode_matches_oracle(ops, hkv, group, splits):
 def test_attention_closed_forms_on_gpu(ops):
     pb = P.make_problem(47, [1, PS * 4 + 3, PS * 9 + 16], num_kv_heads=1, group=4, topk=2)
     O.append_paged_kv(pb.k, pb.v, pb.kv_cache, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
-    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
     sel_t, cnt_t = P.int_tensor(sel, DEV), P.int_tensor(cnt, DEV)
     g = Gpu(pb)
     out = ops.sparse_paged_decode(g.q, g.kv, sel_t, cnt_t, g.last).float().cpu().numpy()
@@ -278,7 +278,7 @@ def test_out_of_range_page_ids_are_skipped_not_followed(ops):
 def run_step(ops, g: Gpu, splits=0):
     pb = g.pb
     ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
-    ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, pb.topk, g.sel, g.cnt, g.logical, g.scores)
+    ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, pb.topk, g.sel, g.cnt, g.logical, g.scores)
     out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, workspace=workspace(ops, pb, pb.topk + 1, splits),
                                   num_splits=splits)
     torch.cuda.synchronize()
@@ -358,7 +358,7 @@ def test_properties_at_scale(ops):
     sel = torch.empty(B, 1, topk + 1, dtype=torch.int32, device=DEV)
     cnt = torch.empty(B, 1, dtype=torch.int32, device=DEV)
     logical = torch.empty(B, 1, topk, dtype=torch.int32, device=DEV)
-    ops.block_score_topk(q, kbar, indices, indptr, topk, sel, cnt, logical)
+    ops.block_score_topk(q, kbar, indices, indptr, last, topk, sel, cnt, logical)
     assert bool((cnt == topk + 1).all())
     # selected ids: unique, candidates only, last entry the last page
     lg = logical[:, 0].sort(dim=1).values
@@ -382,7 +382,7 @@ def test_properties_at_scale(ops):
     sub_ptr = (np.arange(4) * n_pages).astype(np.int32)
     q_np = P.from_torch(q[rows])
     kbar_np = P.from_torch(kbar[rows])
-    want_sel, want_cnt, want_logical, want_scores = O.block_score_topk(q_np, kbar_np, sub_idx, sub_ptr, topk)
+    want_sel, want_cnt, want_logical, want_scores = O.block_score_topk(q_np, kbar_np, sub_idx, sub_ptr, np.ones(len(sub_ptr) - 1, dtype=np.int32), topk)
     for j, b in enumerate(rows):
         ok, msg = O.selection_matches(logical[b, 0].cpu().numpy(), want_scores[j][0], topk)
         assert ok, msg
@@ -478,7 +478,7 @@ def _check_full_size(ops, st, spot_rows):
     B, hkv, group, topk, n_pages = st["B"], st["hkv"], st["group"], st["topk"], st["n_pages"]
     ops.build_kbar(st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
     ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
-    ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], topk, st["sel"], st["cnt"], st["logical"])
+    ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], st["last"], topk, st["sel"], st["cnt"], st["logical"])
     out = ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"], num_splits=1)
     torch.cuda.synchronize()
     # append landed in slot 0 of every sequence's last page, bit for bit
@@ -494,7 +494,7 @@ def _check_full_size(ops, st, spot_rows):
     # idempotence: lengths are static, so a second step reproduces the first exactly
     sel1, out1 = st["sel"].clone(), out.clone()
     ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
-    ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], topk, st["sel"], st["cnt"], st["logical"])
+    ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], st["last"], topk, st["sel"], st["cnt"], st["logical"])
     out2 = ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"], num_splits=1)
     assert torch.equal(sel1, st["sel"]) and torch.equal(out1, out2)
     # split-K invariance (fp32 merge vs in-kernel merge; one bf16 rounding each)
@@ -507,7 +507,7 @@ def _check_full_size(ops, st, spot_rows):
     sub_idx = np.arange(len(spot_rows) * n_pages, dtype=np.int32)
     sub_ptr = (np.arange(len(spot_rows) + 1) * n_pages).astype(np.int32)
     q_np, kbar_np = P.from_torch(st["q"][rows]), P.from_torch(st["kbar"][rows])
-    want_sel, want_cnt, want_logical, want_scores = O.block_score_topk(q_np, kbar_np, sub_idx, sub_ptr, topk)
+    want_sel, want_cnt, want_logical, want_scores = O.block_score_topk(q_np, kbar_np, sub_idx, sub_ptr, np.ones(len(sub_ptr) - 1, dtype=np.int32), topk)
     got_logical = st["logical"][rows].cpu().numpy()
     for j in range(len(spot_rows)):
         for h in range(hkv):
@@ -603,7 +603,7 @@ def test_full_size_continuous_batching_mix(ops):
     pre_last = torch.clamp(last_t - 1, min=0)  # the cache before this step's append
     ops.build_kbar(kv, kbar, indices, ptr, pre_last)
     ops.append_paged_kv(k, v, kv, kbar, indices, ptr, last_t)
-    ops.block_score_topk(q, kbar, indices, ptr, topk, sel, cnt, logical)
+    ops.block_score_topk(q, kbar, indices, ptr, last_t, topk, sel, cnt, logical)
     out = ops.sparse_paged_decode(q, kv, sel, cnt, last_t)
     torch.cuda.synchronize()
     want_cnt = np.minimum(topk, n_pages - 1) + 1
@@ -617,7 +617,7 @@ def test_full_size_continuous_batching_mix(ops):
     sub_idx = np.arange(sub_ptr[-1], dtype=np.int32)
     sub_kbar = P.from_torch(kbar[rows])
     q_np = P.from_torch(q[rows])
-    want_sel, want_cnt2, want_logical, want_scores = O.block_score_topk(q_np, sub_kbar, sub_idx, sub_ptr, topk)
+    want_sel, want_cnt2, want_logical, want_scores = O.block_score_topk(q_np, sub_kbar, sub_idx, sub_ptr, last[rows], topk)
     got_logical = logical[rows].cpu().numpy()
     got_cnt = cnt[rows].cpu().numpy()
     sel_sub = np.full((len(rows), hkv, topk + 1), -1, dtype=np.int32)
@@ -651,7 +651,7 @@ def test_step_replays_under_hip_graph(ops):
 
     def step():
         ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
-        ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, pb.topk, g.sel, g.cnt)
+        ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, pb.topk, g.sel, g.cnt)
         ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, out=out, workspace=ws)
 
     step()
@@ -689,7 +689,7 @@ def test_custom_ops_trace_with_fullgraph(ops):
 
     def fn(q, k, v):
         torch.ops.kinetics.append_paged_kv(k, v, g.kv, g.kbar, g.indices, g.indptr, g.last)
-        torch.ops.kinetics.block_score_topk(q, g.kbar, g.indices, g.indptr, pb.topk, g.sel, g.cnt)
+        torch.ops.kinetics.block_score_topk(q, g.kbar, g.indices, g.indptr, g.last, pb.topk, g.sel, g.cnt)
         o = torch.ops.kinetics.sparse_paged_decode(q, g.kv, g.sel, g.cnt, g.last, None, 0.0, 1)
         return o * 1.0
 
@@ -725,7 +725,7 @@ def test_fused_step_equals_three_calls(ops, case):
     lse_a = torch.empty(pb.B, pb.Hq, dtype=torch.float32, device=DEV)
     lse_b = torch.empty_like(lse_a)
     ops.append_paged_kv(a.k, a.v, a.kv, a.kbar, a.indices, a.indptr, a.last)
-    ops.block_score_topk(a.q, a.kbar, a.indices, a.indptr, pb.topk, a.sel, a.cnt)
+    ops.block_score_topk(a.q, a.kbar, a.indices, a.indptr, a.last, pb.topk, a.sel, a.cnt)
     out_a = ops.sparse_paged_decode(a.q, a.kv, a.sel, a.cnt, a.last, lse=lse_a, num_splits=1)
     out_b = ops.blocktopk_decode_step(b.q, b.k, b.v, b.kv, b.kbar, b.indices, b.indptr, b.last, pb.topk, lse=lse_b,
                                       sel_pages=b.sel, sel_count=b.cnt)
@@ -761,7 +761,7 @@ def test_fused_step_full_size(ops):
     st = _uniform_state(4096, 32768, 1, 4, 128, seed=2)
     ops.build_kbar(st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
     ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
-    ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], 128, st["sel"], st["cnt"])
+    ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], st["last"], 128, st["sel"], st["cnt"])
     out_a = ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"], num_splits=1)
     sel_b, cnt_b = torch.empty_like(st["sel"]), torch.empty_like(st["cnt"])
     out_b = ops.blocktopk_decode_step(st["q"], st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"],
@@ -841,32 +841,42 @@ def test_decoder_layer_matches_fp32_reference(ops, dense):
     assert rms_norm(hidden, 1e-6, layer.input_layernorm_weight).dtype == torch.bfloat16
 
 
-@pytest.mark.parametrize("sink,local", [(1, 2), (2, 3), (0, 4), (3, 1)])
+@pytest.mark.parametrize("sink,local,offset", [(1, 17, 0), (2, 33, 0), (0, 49, 0), (3, 1, 0), (1, 16, 12), (1, 5, 12),
+                                               (2, 40, 7), (1, 1, 15)])
 @pytest.mark.parametrize("fused", [False, True])
-def test_sink_and_local_pages(ops, sink, local, fused):
-    """Pinned leading / trailing pages (LiteSys' sink and local window, page aligned)."""
+def test_sink_and_local_pages(ops, sink, local, offset, fused):
+    """Pinned leading pages and trailing tokens (LiteSys' sink and local window),
+    with and without padding slots at the start of the first page."""
     topk = 6
-    lengths = [PS * 40 + 3, PS * 9, 1, 0, PS * 3 + 1, PS * 130 + 16, PS * (topk + sink + local) + 1, PS * 2 + 5]
+    lengths = [PS * 40 + 3, PS * 9, 1, 0, PS * 3 + 1, PS * 130 + 16, PS * (topk + sink) + local + 1, PS * 2 + 5,
+               PS * (topk + sink) + local + 16, 16, 13]
     pb = P.make_problem(950 + sink * 10 + local, lengths, num_kv_heads=2, group=4, topk=topk)
     g = Gpu(pb)
-    stride = topk + sink + local
+    stride = ops.sel_list_capacity(topk, sink, local)
+    assert stride == O.sel_list_capacity(topk, sink, local)
     g.sel = torch.full((pb.B, pb.Hkv, stride), -7, dtype=torch.int32, device=DEV)
     check_table(ops, g)
     if fused:
         out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, topk, sel_pages=g.sel,
-                                        sel_count=g.cnt, sink_pages=sink, local_pages=local)
+                                        sel_count=g.cnt, sink_pages=sink, local_tokens=local, first_page_offset=offset)
     else:
         ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
-        ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, topk, g.sel, g.cnt, g.logical, g.scores, sink_pages=sink,
-                             local_pages=local)
-        out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last)
+        ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, topk, g.sel, g.cnt, g.logical, g.scores, sink_pages=sink,
+                             local_tokens=local)
+        out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, first_page_offset=offset)
     torch.cuda.synchronize()
     kv, kbar = pb.kv_cache.copy(), pb.kbar.copy()
     res = O.decode_step(pb.q, pb.k, pb.v, kv, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, topk,
-                        sink_pages=sink, local_pages=local)
+                        sink_pages=sink, local_tokens=local, first_page_offset=offset)
     assert np.array_equal(g.cnt.cpu().numpy(), res["sel_count"])
     assert np.array_equal(g.sel.cpu().numpy(), res["sel_pages"])
-    assert_out_close(out, res["out"], f"sink={sink} local={local} fused={fused}")
+    assert_out_close(out, res["out"], f"sink={sink} local={local} offset={offset} fused={fused}")
+    if offset:  # the padding slots really are left out: the result differs from the unpadded one on the long rows
+        plain, _ = O.sparse_paged_decode(pb.q, kv, res["sel_pages"], res["sel_count"], pb.last_page_len)
+        assert np.abs(plain[0] - res["out"][0]).max() > 1e-3
+        od = ops.dense_paged_decode(g.q, g.kv, g.indices, g.indptr, g.last, pb.max_pages, first_page_offset=offset)
+        wd, _ = O.dense_paged_decode(pb.q, kv, pb.page_indices, pb.page_indptr, pb.last_page_len, first_page_offset=offset)
+        assert_out_close(od, wd, f"dense offset={offset}")
     if not fused:
         logical, scores = g.logical.cpu().numpy(), g.scores.cpu().numpy()
         for b in range(pb.B):
@@ -875,8 +885,37 @@ def test_sink_and_local_pages(ops, sink, local, fused):
                 assert np.array_equal(logical[b, h, : len(want)], want)
                 ws = res["scores"][b][h]
                 n_pages = (lengths[b] + PS - 1) // PS
-                n_sink = O.split_pages(n_pages, sink, local, pb.kbar.shape[1])[0]
-                assert np.allclose(scores[b, h, n_sink : n_sink + len(ws)], ws, rtol=1e-5, atol=1e-5)
+                if n_pages:
+                    n_sink = O.split_pages(n_pages, pb.last_page_len[b], sink, local, pb.kbar.shape[1])[0]
+                    assert np.allclose(scores[b, h, n_sink : n_sink + len(ws)], ws, rtol=1e-5, atol=1e-5)
+
+
+def test_topk_zero_is_sink_plus_local_window(ops):
+    """topk = 0: only the pinned pages are attended (LiteSys' local_sparsity,
+    sparsity_utils.py:107-114) and no mean key is read."""
+    lengths = [PS * 40 + 3, PS * 2, 5, 0, PS * 12 + 16]
+    pb = P.make_problem(77, lengths, num_kv_heads=2, group=2, topk=1)
+    for fused in (False, True):
+        g = Gpu(pb)
+        g.kbar.fill_(float("nan"))   # must not matter
+        stride = ops.sel_list_capacity(0, 1, 40)
+        g.sel = torch.full((pb.B, pb.Hkv, stride), -7, dtype=torch.int32, device=DEV)
+        if fused:
+            out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, 0, sel_pages=g.sel,
+                                            sel_count=g.cnt, sink_pages=1, local_tokens=40)
+        else:
+            ops.append_paged_kv(g.k, g.v, g.kv, None, g.indices, g.indptr, g.last)
+            ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, 0, g.sel, g.cnt, sink_pages=1, local_tokens=40)
+            out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last)
+        torch.cuda.synchronize()
+        kv = pb.kv_cache.copy()
+        O.append_paged_kv(pb.k, pb.v, kv, None, pb.page_indices, pb.page_indptr, pb.last_page_len)
+        sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, 0,
+                                            sink_pages=1, local_tokens=40)
+        assert np.array_equal(g.cnt.cpu().numpy(), cnt) and np.array_equal(g.sel.cpu().numpy(), sel)
+        assert cnt[0, 0] == 1 + 4 and cnt[1, 0] == 2 and cnt[3, 0] == 0
+        want, _ = O.sparse_paged_decode(pb.q, kv, sel, cnt, pb.last_page_len)
+        assert_out_close(out, want, f"topk=0 fused={fused}")
 
 
 # --------------------------------------------------------------------------- seeded sweep over odd shapes
@@ -904,27 +943,31 @@ def test_seeded_sweep_of_shapes(ops):
             else:
                 lengths.append(int(rng.integers(PS, PS * 90)))
         topk = int(rng.choice([1, 2, 5, 17, 64, 100]))
-        sink, local = int(rng.integers(0, 3)), int(rng.integers(1, 4))
+        sink, local = int(rng.integers(0, 3)), int(rng.choice([1, 1, 17, 33, int(rng.integers(1, 60))]))
+        offset = int(rng.integers(0, PS)) if sink and rng.integers(0, 2) else 0
         table = str(rng.choice(["random", "fragmented"]))
         fused = bool(rng.integers(0, 2))
         splits = int(rng.choice([0, 1, 2, 5]))
-        what = f"trial {trial}: hkv={hkv} G={group} lengths={lengths} topk={topk} sink={sink} local={local} {table} fused={fused} splits={splits}"
+        what = f"trial {trial}: hkv={hkv} G={group} lengths={lengths} topk={topk} sink={sink} local={local} offset={offset} {table} fused={fused} splits={splits}"
         pb = P.make_problem(3000 + trial, lengths, num_kv_heads=hkv, group=group, topk=topk, table=table)
         g = Gpu(pb)
-        g.sel = torch.full((pb.B, hkv, topk + sink + local), -7, dtype=torch.int32, device=DEV)
+        g.sel = torch.full((pb.B, hkv, ops.sel_list_capacity(topk, sink, local)), -7, dtype=torch.int32, device=DEV)
         check_table(ops, g)
         lse = torch.full((pb.B, pb.Hq), float("nan"), dtype=torch.float32, device=DEV)
         if fused:
             out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, topk, lse=lse,
-                                            sel_pages=g.sel, sel_count=g.cnt, sink_pages=sink, local_pages=local)
+                                            sel_pages=g.sel, sel_count=g.cnt, sink_pages=sink, local_tokens=local,
+                                            first_page_offset=offset)
         else:
             ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
-            ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, topk, g.sel, g.cnt, sink_pages=sink, local_pages=local)
-            out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, lse=lse, num_splits=splits)
+            ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, topk, g.sel, g.cnt, sink_pages=sink,
+                                 local_tokens=local)
+            out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, lse=lse, num_splits=splits,
+                                          first_page_offset=offset)
         torch.cuda.synchronize()
         kv, kbar = pb.kv_cache.copy(), pb.kbar.copy()
         res = O.decode_step(pb.q, pb.k, pb.v, kv, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, topk,
-                            sink_pages=sink, local_pages=local)
+                            sink_pages=sink, local_tokens=local, first_page_offset=offset)
         assert np.array_equal(P.from_torch(g.kv), kv), what
         assert np.array_equal(P.from_torch(g.kbar), kbar), what
         sel, cnt = g.sel.cpu().numpy(), g.cnt.cpu().numpy()
@@ -933,21 +976,25 @@ def test_seeded_sweep_of_shapes(ops):
         if not np.array_equal(sel, res["sel_pages"]):
             for b in range(pb.B):
                 pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
-                n_sink = O.split_pages(len(pages), sink, local, pb.kbar.shape[1])[0]
+                if len(pages) == 0:
+                    continue
+                n_sink = O.split_pages(len(pages), pb.last_page_len[b], sink, local, pb.kbar.shape[1])[0]
                 lookup = {int(p): i for i, p in enumerate(pages)}
                 for h in range(hkv):
                     k_eff = len(res["sel_logical"][b][h])
-                    got = np.array([lookup[int(p)] for p in sel[b, h, :k_eff]]) - n_sink
+                    got = np.array([lookup[int(p)] for p in sel[b, h, n_sink : n_sink + k_eff]]) - n_sink
                     ok, msg = O.selection_matches(got, res["scores"][b][h], topk)
                     assert ok, f"{what}: {msg}"
-                    assert np.array_equal(sel[b, h, k_eff:], res["sel_pages"][b, h, k_eff:]), what
-        want, want_lse = O.sparse_paged_decode(pb.q, kv, sel, cnt, pb.last_page_len)
+                    assert np.array_equal(sel[b, h, :n_sink], res["sel_pages"][b, h, :n_sink]), what
+                    assert np.array_equal(sel[b, h, n_sink + k_eff :], res["sel_pages"][b, h, n_sink + k_eff :]), what
+        want, want_lse = O.sparse_paged_decode(pb.q, kv, sel, cnt, pb.last_page_len, first_page_offset=offset)
         assert_out_close(out, want, what)
         got_lse = lse.cpu().numpy().astype(np.float64)
         fin = np.isfinite(want_lse)
         assert np.array_equal(np.isneginf(got_lse), ~fin), what
         assert np.allclose(got_lse[fin], want_lse[fin], rtol=1e-4, atol=1e-4), what
         # dense on the same cache
-        od = ops.dense_paged_decode(g.q, g.kv, g.indices, g.indptr, g.last, max(pb.max_pages, 1), num_splits=splits)
-        wd, _ = O.dense_paged_decode(pb.q, kv, pb.page_indices, pb.page_indptr, pb.last_page_len)
+        od = ops.dense_paged_decode(g.q, g.kv, g.indices, g.indptr, g.last, max(pb.max_pages, 1), num_splits=splits,
+                                    first_page_offset=offset)
+        wd, _ = O.dense_paged_decode(pb.q, kv, pb.page_indices, pb.page_indptr, pb.last_page_len, first_page_offset=offset)
         assert_out_close(od, wd, what + " (dense)")

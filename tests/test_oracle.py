@@ -120,7 +120,7 @@ def test_build_kbar_covers_full_pages_only():
 
 def test_scores_identities():
     pb = P.make_problem(21, [PS * 9 + 4, PS * 5 + 1], num_kv_heads=2, group=4)
-    sc = O.block_scores(pb.q, pb.kbar, pb.page_indptr)
+    sc = O.block_scores(pb.q, pb.kbar, pb.page_indptr, pb.last_page_len)
     qf = O.bf16_to_f32(pb.q).astype(np.float64)
     for b in range(pb.B):
         n_cand = (pb.lengths[b] + PS - 1) // PS - 1
@@ -150,7 +150,7 @@ def test_scores_equal_litesys_group_mean_then_block_mean():
     kbar = np.zeros((1, n_pages + 1, 1, D), dtype=np.uint16)
     O.build_kbar(kv, kbar, indices, indptr, np.array([1], dtype=np.int32))
     q = P.randn_bf16(rng, (1, G, D))
-    sc = O.block_scores(q, kbar, indptr)[0][0]
+    sc = O.block_scores(q, kbar, indptr, np.array([1], dtype=np.int32))[0][0]
     logits = np.einsum("gd,ptd->gpt", O.bf16_to_f32(q[0]).astype(np.float64), K.astype(np.float64)) / math.sqrt(D)
     litesys = logits.mean(axis=0).mean(axis=-1)
     assert np.allclose(sc / math.sqrt(D), litesys, rtol=1e-12, atol=1e-12)
@@ -181,7 +181,7 @@ def test_select_topk_tie_break_is_lowest_index():
 
 def test_block_score_topk_page_list_layout():
     pb = P.make_problem(31, [PS * 20 + 7, PS * 3, 1, 0, PS * 2 + 1], topk=4)
-    sel, cnt, logical, scores = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    sel, cnt, logical, scores = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
     assert sel.shape == (5, 1, 5)
     assert cnt[:, 0].tolist() == [5, 3, 1, 0, 3]  # min(k, n_cand) + 1, 0 for the empty sequence
     for b in range(5):
@@ -238,7 +238,7 @@ def test_dense_attention_equals_torch_sdpa():
 
 def test_sparse_with_every_page_selected_equals_dense():
     pb = P.make_problem(43, [PS * 5 + 2, PS * 3 + 16], num_kv_heads=1, group=4, topk=64)
-    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
     a, la = O.sparse_paged_decode(pb.q, pb.kv_cache, sel, cnt, pb.last_page_len)
     d, ld = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len)
     assert np.allclose(a, d, rtol=1e-10, atol=1e-12) and np.allclose(la, ld, rtol=1e-12)
@@ -248,7 +248,7 @@ def test_attention_closed_forms():
     rng = np.random.default_rng(47)
     pb = P.make_problem(47, [1, PS * 4 + 3], num_kv_heads=1, group=4, topk=2)
     O.append_paged_kv(pb.k, pb.v, pb.kv_cache, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
-    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
     out, lse = O.sparse_paged_decode(pb.q, pb.kv_cache, sel, cnt, pb.last_page_len)
     # one token: softmax over one logit is 1 -> out is that token's value, lse its logit
     v0 = O.bf16_to_f32(pb.v[0, 0]).astype(np.float64)
@@ -272,7 +272,7 @@ def test_attention_closed_forms():
 
 def test_attention_permutation_and_split_invariance():
     pb = P.make_problem(53, [PS * 12 + 9], num_kv_heads=1, group=4, topk=7)
-    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.topk)
+    sel, cnt, _, _ = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
     out, lse = O.sparse_paged_decode(pb.q, pb.kv_cache, sel, cnt, pb.last_page_len)
     # shuffle the full pages (the final, partial page keeps its place)
     c = cnt[0, 0]
@@ -347,19 +347,22 @@ def test_torch_path_agrees_with_oracle():
 
 
 def test_sink_and_local_pages_are_pinned_not_candidates():
-    """Page-aligned form of LiteSys' sink tokens and local window
-    (sparsity_utils.py:24-35): pinned pages are always in the list, never scored."""
+    """Sink pages and the pages of the newest local tokens (LiteSys' sink and
+    local window, sparsity_utils.py:24-35) are always in the list, never scored."""
     pb = P.make_problem(71, [PS * 20 + 7, PS * 4 + 2, PS * 2, 5, 0], topk=3)
-    sel, cnt, logical, scores = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, 3, sink_pages=2, local_pages=3)
-    assert sel.shape[2] == 3 + 2 + 3
-    # n_pages = 21, 5, 2, 1, 0 -> (sink, cand, local) = (2,16,3), (2,0,3), (0,0,2), (0,0,1), -
+    sel, cnt, logical, scores = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, 3,
+                                                   sink_pages=2, local_tokens=2 * PS + 1)
+    assert sel.shape[2] == 3 + 2 + 3 == O.sel_list_capacity(3, 2, 2 * PS + 1)
+    # n_pages = 21, 5, 2, 1, 0 -> (sink, cand, local) = (2,16,3), (2,0,3), (1,0,1), (0,0,1), -
     assert cnt[:, 0].tolist() == [3 + 5, 5, 2, 1, 0]
     pages = O.seq_pages(pb.page_indices, pb.page_indptr, 0)
     assert len(scores[0][0]) == 16
-    assert sel[0, 0, 3:8].tolist() == [pages[0], pages[1], pages[18], pages[19], pages[20]]
+    assert sel[0, 0, :2].tolist() == [pages[0], pages[1]]                    # sink pages first
+    assert sel[0, 0, 2:5].tolist() == pages[logical[0][0]].tolist()          # then the winners, best first
+    assert sel[0, 0, 5:8].tolist() == [pages[18], pages[19], pages[20]]      # then the local pages, open page last
     assert all(2 <= i < 18 for i in logical[0][0])
     # scores are those of logical pages 2..17
-    full = O.block_scores(pb.q, pb.kbar, pb.page_indptr)[0][0]  # default split: candidates 0..19
+    full = O.block_scores(pb.q, pb.kbar, pb.page_indptr, pb.last_page_len)[0][0]  # default split: candidates 0..19
     assert np.allclose(scores[0][0], full[2:18])
     # short sequences: everything pinned, in logical order, open page last
     p1 = O.seq_pages(pb.page_indices, pb.page_indptr, 1)
@@ -377,6 +380,95 @@ def test_sink_and_local_pages_are_pinned_not_candidates():
     w /= w.sum(axis=1, keepdims=True)
     assert np.allclose(out[0], w @ V, rtol=1e-10, atol=1e-12)
     # defaults reproduce the reference rule
-    a = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, 3)
-    b = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, 3, sink_pages=0, local_pages=1)
+    a = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, 3)
+    b = O.block_score_topk(pb.q, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, 3, sink_pages=0, local_tokens=1)
     assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+
+
+def test_split_pages_against_token_level_definition():
+    """Brute force: a page is a candidate iff it comes after the sink pages and
+    ends at or before the first of the newest ``local_tokens`` tokens."""
+    for kv_len in list(range(1, 200)) + [1000, 1009, 4096]:
+        n_pages = (kv_len + PS - 1) // PS
+        last = kv_len - (n_pages - 1) * PS
+        for sink in (0, 1, 2, 5):
+            for local in (1, 2, 15, 16, 17, 18, 33, 100):
+                n_sink, n_cand, n_local = O.split_pages(n_pages, last, sink, local, 10 ** 6)
+                want_sink = min(sink, n_pages - 1)
+                cand = [p for p in range(want_sink, n_pages) if (p + 1) * PS <= kv_len - local]
+                assert (n_sink, n_cand) == (want_sink, len(cand)), (kv_len, sink, local)
+                assert cand == list(range(want_sink, want_sink + len(cand)))
+                assert n_sink + n_cand + n_local == n_pages and n_local >= 1
+                assert n_local <= 1 + (local + 14) // PS
+    # local_tokens = 16 (L - 1) + 1 pins exactly the last L pages whatever the open page holds
+    for n_pages in range(1, 12):
+        for last in range(1, PS + 1):
+            for L in (1, 2, 3):
+                n_sink, n_cand, n_local = O.split_pages(n_pages, last, 0, PS * (L - 1) + 1, 10 ** 6)
+                assert n_local == min(L, n_pages) and n_cand == n_pages - n_local
+    # mean keys exist for the first kbar_pages pages only
+    assert O.split_pages(100, 3, 2, 1, 50) == (2, 48, 1)
+
+
+def test_litesys_mask_hand_case():
+    """sparsity_utils.py:24-47 on a case small enough to do by hand: 57 tokens,
+    sink 4, local 5, one block of 16 kept out of three."""
+    seq_len, local = 4 + 3 * 16 + 5, 5
+    mean_logits = np.zeros(seq_len)
+    mean_logits[4 + 16 : 4 + 32] = 1.0      # block 1 has the largest mean
+    mean_logits[4] = 10.0                    # one large token does not make block 0 win: mean 10/16 < 1
+    keep = O.litesys_blockwise_topk_mask(mean_logits, seq_len, 1, local)
+    want = np.zeros(seq_len, dtype=bool)
+    want[:4] = True
+    want[20:36] = True
+    want[52:] = True
+    assert np.array_equal(keep, want)
+    # a non-aligned tail: the local part absorbs the remainder (58 tokens -> 6 local tokens)
+    keep = O.litesys_blockwise_topk_mask(np.append(mean_logits, 0.0), seq_len + 1, 1, local)
+    assert keep[52:].all() and keep[20:36].all() and keep.sum() == 4 + 16 + 6
+    # at or below n_full = roundup16(4 + 5 + 16) = 32 tokens everything stays
+    assert O.litesys_blockwise_topk_mask(np.zeros(32), 32, 1, local).all()
+    assert O.litesys_blockwise_topk_mask(np.arange(33.0), 33, 1, local).sum() == 4 + 16 + 13
+
+
+def test_page_lists_with_offset_12_equal_litesys_mask_formulation():
+    """The paged formulation (sink_pages=1, local_tokens=local, sequences stored
+    12 slots into their first page) and LiteSys' mask on full logits
+    (sparsity_utils.py:24-47, batch_cache.py:154-168) are the same function:
+    same kept tokens, same output.  Keys are multiples of 16 so that page means
+    are exact in bfloat16 and no score is perturbed by rounding."""
+    rng = np.random.default_rng(123)
+    Hkv, G, pad = 2, 2, 12
+    for seq_len, topk, local in [(300, 3, 20), (301, 3, 16), (52, 2, 5), (53, 2, 5), (40, 4, 7), (5, 2, 3), (4, 1, 1),
+                                 (1, 1, 1), (1000, 10, 64), (999, 10, 1), (131, 1, 100), (307, 5, 33)]:
+        K = (rng.integers(-8, 9, size=(seq_len, Hkv, D)) * 16).astype(np.float32)
+        V = O.bf16_to_f32(P.randn_bf16(rng, (seq_len, Hkv, D)))
+        q = P.randn_bf16(rng, (1, Hkv * G, D))
+        cache_len = seq_len + pad
+        n_pages = (cache_len + PS - 1) // PS
+        perm = rng.permutation(n_pages + 3).astype(np.int32)[:n_pages]
+        kv = P.randn_bf16(rng, (n_pages + 3, 2, PS, Hkv, D))            # padding slots hold garbage
+        flat_k = np.zeros((n_pages * PS, Hkv, D), dtype=np.uint16)
+        flat_v = np.zeros_like(flat_k)
+        flat_k[:pad], flat_v[:pad] = P.randn_bf16(rng, (pad, Hkv, D)), P.randn_bf16(rng, (pad, Hkv, D))
+        flat_k[pad:cache_len], flat_v[pad:cache_len] = O.f32_to_bf16(K), O.f32_to_bf16(V)
+        kv[perm, 0] = flat_k.reshape(n_pages, PS, Hkv, D)
+        kv[perm, 1] = flat_v.reshape(n_pages, PS, Hkv, D)
+        indptr = np.array([0, n_pages], dtype=np.int32)
+        last = np.array([cache_len - (n_pages - 1) * PS], dtype=np.int32)
+        kbar = np.zeros((1, n_pages, Hkv, D), dtype=np.uint16)
+        O.build_kbar(kv, kbar, perm, indptr, last)
+        sel, cnt, logical, _ = O.block_score_topk(q, kbar, perm, indptr, last, topk, sink_pages=1, local_tokens=local)
+        out, _ = O.sparse_paged_decode(q, kv, sel, cnt, last, first_page_offset=pad)
+        want, keep = O.litesys_decode(O.bf16_to_f32(q[0]), K, V, topk, local)
+        lookup = {int(p): i for i, p in enumerate(perm)}
+        for h in range(Hkv):
+            got_keep = np.zeros(n_pages * PS, dtype=bool)
+            for pid in sel[0, h, : cnt[0, h]]:
+                got_keep[lookup[int(pid)] * PS : (lookup[int(pid)] + 1) * PS] = True
+            assert np.array_equal(got_keep[pad:cache_len], keep[h]), (seq_len, topk, local, h)
+        assert np.allclose(out[0], want, rtol=1e-9, atol=1e-11), (seq_len, topk, local)
+        # the dense layer (attn_layer_skip) on the same cache
+        dense, _ = O.dense_paged_decode(q, kv, perm, indptr, last, first_page_offset=pad)
+        want_dense, _ = O.litesys_decode(O.bf16_to_f32(q[0]), K, V, None, local)
+        assert np.allclose(dense[0], want_dense, rtol=1e-9, atol=1e-11)
