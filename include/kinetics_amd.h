@@ -104,6 +104,31 @@ int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar,
                    int64_t num_pages, int kbar_pages, kin_stream_t stream);
 
 /*
+ * Ragged multi-token append -- the general form of
+ * flashinfer.append_paged_kv_cache behind mylib::update_kv, whose signature
+ * carries kv_append_indptr (ref: benchmark/blocktopk_decoder.py:23-46), and the
+ * paged counterpart of LiteSys' prefill write
+ * (ref: LiteSys/litesys/attention/batch_cache.py:112-131).
+ *
+ * k, v: [nnz, num_kv_heads, head_dim]; sequence b appends the rows
+ * append_indptr[b] .. append_indptr[b+1]-1 (n_b of them).  The page table
+ * describes the cache AFTER the append: row i of sequence b lands at token
+ * position kv_len_b - n_b + i, kv_len_b = 16*(n_pages_b-1) + last_page_len[b].
+ * When kbar is given, the mean key of every page the append completed is
+ * (re)computed, with the arithmetic of kin_append_paged_kv.  max_append_len is
+ * an upper bound on n_b (nnz always works; a tighter bound launches fewer idle
+ * workgroups).  Sequences whose metadata is out of contract are skipped.
+ */
+int kin_append_paged_kv_ragged(const kin_bf16_t* k, const kin_bf16_t* v,
+                               const int32_t* append_indptr,
+                               kin_bf16_t* kv_cache, kin_bf16_t* kbar,
+                               const int32_t* page_indices, const int32_t* page_indptr,
+                               const int32_t* last_page_len,
+                               int batch, int64_t nnz, int max_append_len,
+                               int num_kv_heads, int head_dim, int page_size,
+                               int64_t num_pages, int kbar_pages, kin_stream_t stream);
+
+/*
  * (2)+(3) Page scoring and top-k page selection, fused -- replaces
  *   csim = einsum("b g d, b n d -> b g n", q, kbar).mean(1); topk(csim, k);
  *   logical->physical translation; cat(last page)

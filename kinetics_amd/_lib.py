@@ -32,6 +32,10 @@ SIGNATURES = {
     "kin_last_error": (c_char_p, []),
     "kin_status_string": (c_char_p, [c_int]),
     "kin_append_paged_kv": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int64, c_int, _P]),
+    "kin_append_paged_kv_ragged": (
+        c_int,
+        [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int64, c_int, c_int, c_int, c_int, c_int64, c_int, _P],
+    ),
     "kin_build_kbar": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int64, c_int, _P]),
     "kin_block_score_topk": (
         c_int,

@@ -29,8 +29,9 @@ page j+1, and the kernels are told to skip the 12 padding slots
 token set is then LiteSys' own, token for token.
 ``attn_layer_skip`` (default ``[0]``: layer 0 stays dense, sparsity_utils.py:211)
 is honoured.
-Prefill is not the accelerated path: it writes pages with PyTorch indexing and
-runs PyTorch's scaled_dot_product_attention (LiteSys calls flashinfer there,
+Prefill writes its rows and the mean keys of the pages it completes with the
+ragged append kernel; its attention is not the accelerated path and runs on
+PyTorch's scaled_dot_product_attention (LiteSys calls flashinfer there,
 batch_cache.py:112-145).
 """
 from __future__ import annotations
@@ -160,9 +161,9 @@ class PagedBatchKVManager:
 
     # ------------------------------------------------------------------ prefill (not the accelerated path)
     def prefill_or_append(self, query_states, key_states, value_states, layer_idx, batch_idx):
-        """One request: write its K/V rows into the slot's pages, refresh the
-        mean keys of the pages that are now full, causal attention over the
-        slot's whole context (batch_cache.py:112-145)."""
+        """One request: write its K/V rows into the slot's pages and refresh the
+        mean keys of the pages that are now full (one ragged append), then causal
+        attention over the slot's whole context (batch_cache.py:112-145)."""
         bsz, seq_len = query_states.shape[0], query_states.shape[2]
         slot = int(batch_idx.item())
         offset = int(self.kv_offset[layer_idx][slot].item())
@@ -172,15 +173,15 @@ class PagedBatchKVManager:
             raise ValueError(f"sequence of {total} tokens exceeds max_seq_len")
         P, Hkv, D = self.pages_per_slot, self.num_key_value_heads, self.head_dim
         view = self.kv_cache[layer_idx].view(self.max_batch_size, P, 2, PAGE, Hkv, D)
-        pos = torch.arange(offset, total, device=self.device) + pad
-        view[slot, pos // PAGE, 0, pos % PAGE] = key_states[0].transpose(0, 1)
-        view[slot, pos // PAGE, 1, pos % PAGE] = value_states[0].transpose(0, 1)
         self.kv_offset[layer_idx][slot] += seq_len
         n_pages = (total + pad + PAGE - 1) // PAGE
         idx = (slot * P + torch.arange(n_pages, device=self.device, dtype=torch.int32)).contiguous()
         ptr = torch.tensor([0, n_pages], dtype=torch.int32, device=self.device)
         last = torch.tensor([total + pad - (n_pages - 1) * PAGE], dtype=torch.int32, device=self.device)
-        ops.build_kbar(self.kv_cache[layer_idx], self.kbar[layer_idx][slot:slot + 1], idx, ptr, last)
+        # rows to their page slots, mean keys of the pages that are now full
+        ops.append_paged_kv_ragged(key_states[0].transpose(0, 1).contiguous(), value_states[0].transpose(0, 1).contiguous(),
+                                   torch.tensor([0, seq_len], dtype=torch.int32, device=self.device),
+                                   self.kv_cache[layer_idx], self.kbar[layer_idx][slot:slot + 1], idx, ptr, last)
         k_all = view[slot, :n_pages, 0].reshape(n_pages * PAGE, Hkv, D)[pad:total + pad].transpose(0, 1)  # [Hkv, total, D]
         v_all = view[slot, :n_pages, 1].reshape(n_pages * PAGE, Hkv, D)[pad:total + pad].transpose(0, 1)
         G = self.num_attention_heads // Hkv

@@ -124,6 +124,43 @@ def append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_l
         )
 
 
+def append_paged_kv_ragged(k, v, append_indptr, kv_cache, kbar, page_indices, page_indptr, last_page_len,
+                           max_append_len: Optional[int] = None) -> None:
+    """Write ``append_indptr[b+1] - append_indptr[b]`` new tokens per sequence
+    (rows of ``k`` / ``v`` [nnz, num_kv_heads, head_dim]) into the paged cache and
+    refresh the mean key of every page that becomes full: the general form of
+    ``mylib::update_kv`` (benchmark/blocktopk_decoder.py:23-46) and the paged
+    counterpart of LiteSys' prefill write (batch_cache.py:112-131).  The page
+    table describes the cache after the append.  ``max_append_len`` bounds the
+    longest append (default: nnz)."""
+    num_pages, page_size, num_kv_heads, head_dim = _cache_dims(kv_cache)
+    dev = kv_cache.device
+    _require(k, "k", torch.bfloat16, 3, dev)
+    _require(v, "v", torch.bfloat16, 3, dev)
+    nnz = k.shape[0]
+    if tuple(k.shape) != (nnz, num_kv_heads, head_dim) or k.shape != v.shape:
+        raise ValueError(f"k and v must be [nnz, {num_kv_heads}, {head_dim}], got {tuple(k.shape)} and {tuple(v.shape)}")
+    _require(append_indptr, "append_indptr", torch.int32, 1, dev)
+    batch = append_indptr.numel() - 1
+    if batch < 0:
+        raise ValueError("append_indptr must have batch+1 entries")
+    _table(page_indices, page_indptr, last_page_len, batch, dev)
+    kbar_pages = 0
+    if kbar is not None:
+        kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim)
+        if kbar.device != dev:
+            raise ValueError("kbar must be on the same device as kv_cache")
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(
+            lib.kin_append_paged_kv_ragged(
+                _ptr(k), _ptr(v), _ptr(append_indptr), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
+                _ptr(last_page_len), batch, nnz, nnz if max_append_len is None else int(max_append_len), num_kv_heads,
+                head_dim, page_size, num_pages, kbar_pages, _stream(dev),
+            )
+        )
+
+
 def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len) -> None:
     """Fill ``kbar`` with the mean key of every full page (prefill-side producer
     of what the reference calls compressed_key_cache,
@@ -398,6 +435,13 @@ torch.library.define(
     "(Tensor k, Tensor v, Tensor(a!) kv_cache, Tensor(b!)? kbar, Tensor page_indices, Tensor page_indptr, "
     "Tensor last_page_len) -> ()",
 )
+# Same argument order as the reference's mylib::update_kv
+# (benchmark/blocktopk_decoder.py:23-26), plus the mean-key cache it has to keep current.
+torch.library.define(
+    "kinetics::update_kv",
+    "(Tensor k, Tensor v, Tensor kv_append_indptr, Tensor(a!) kv_cache, Tensor kv_page_indices, Tensor kv_page_indptr, "
+    "Tensor cachelen, Tensor(b!)? kbar=None) -> ()",
+)
 torch.library.define(
     "kinetics::block_score_topk",
     "(Tensor q, Tensor kbar, Tensor page_indices, Tensor page_indptr, Tensor last_page_len, int topk, "
@@ -444,6 +488,16 @@ def _append_impl(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len)
 
 @torch.library.register_fake("kinetics::append_paged_kv")
 def _append_fake(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len):
+    return None
+
+
+@torch.library.impl("kinetics::update_kv", "cuda")
+def _update_kv_impl(k, v, kv_append_indptr, kv_cache, kv_page_indices, kv_page_indptr, cachelen, kbar=None):
+    append_paged_kv_ragged(k, v, kv_append_indptr, kv_cache, kbar, kv_page_indices, kv_page_indptr, cachelen)
+
+
+@torch.library.register_fake("kinetics::update_kv")
+def _update_kv_fake(k, v, kv_append_indptr, kv_cache, kv_page_indices, kv_page_indptr, cachelen, kbar=None):
     return None
 
 

@@ -130,6 +130,33 @@ def append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_l
                 kbar[b, len(pages) - 1, h] = page_mean_key(kv_cache[pid, 0, :, h, :])
 
 
+def append_paged_kv_ragged(k, v, append_indptr, kv_cache, kbar, page_indices, page_indptr, last_page_len):
+    """flashinfer.append_paged_kv_cache in its general form (the call behind
+    mylib::update_kv, benchmark/blocktopk_decoder.py:38-46, which carries
+    kv_append_indptr): sequence b appends rows append_indptr[b]:append_indptr[b+1]
+    of k / v [nnz, Hkv, D]; the page table describes the cache after the append,
+    so row i lands at token position kv_len_b - n_b + i.  Same effect as LiteSys'
+    prefill write into its contiguous cache (batch_cache.py:112-131).  The mean
+    key of every page the append completed is recomputed.  In place."""
+    ps = kv_cache.shape[2]
+    B = len(page_indptr) - 1
+    for b in range(B):
+        a0, a1 = int(append_indptr[b]), int(append_indptr[b + 1])
+        pages = seq_pages(page_indices, page_indptr, b)
+        if a1 <= a0 or len(pages) == 0:
+            continue
+        kv_len = (len(pages) - 1) * ps + int(last_page_len[b])
+        first = kv_len - (a1 - a0)
+        for i in range(a1 - a0):
+            pos = first + i
+            kv_cache[pages[pos // ps], 0, pos % ps] = k[a0 + i]
+            kv_cache[pages[pos // ps], 1, pos % ps] = v[a0 + i]
+        if kbar is not None:
+            for p in range(first // ps, kv_len // ps):
+                if p < kbar.shape[1]:
+                    kbar[b, p] = page_mean_key(kv_cache[pages[p], 0].transpose(1, 0, 2))
+
+
 def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len):
     """Mean key of every FULL page of every sequence (in place on ``kbar``)."""
     B = len(page_indptr) - 1

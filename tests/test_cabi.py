@@ -58,6 +58,19 @@ def test_append_argument_errors(lib):
     assert append(lib, B=0) == _lib.KIN_OK  # nothing to do, nothing launched
 
 
+def test_ragged_append_argument_errors(lib):
+    def ragged(k=A, ind=A, B=2, nnz=10, mx=10, kv=A):
+        return lib.kin_append_paged_kv_ragged(k, A, ind, kv, A, A, A, A, B, nnz, mx, 1, 128, 16, 8, 4, None)
+
+    assert ragged(k=None) == _lib.KIN_ERR_NULL_POINTER
+    assert ragged(ind=None) == _lib.KIN_ERR_NULL_POINTER
+    assert ragged(nnz=-1) == _lib.KIN_ERR_BAD_SHAPE
+    assert ragged(nnz=4, mx=5) == _lib.KIN_ERR_BAD_SHAPE
+    assert ragged(kv=A + 4) == _lib.KIN_ERR_MISALIGNED
+    assert ragged(nnz=0, mx=0) == _lib.KIN_OK
+    assert ragged(B=0) == _lib.KIN_OK
+
+
 def select(lib, q=A, kbar=A, idx=A, ptr=A, last=A, topk=4, sel=A, cnt=A, B=2, Hq=4, Hkv=1, D=128, kp=64, stride=5, sink=0,
            local=1):
     return lib.kin_block_score_topk(q, kbar, idx, ptr, last, topk, sink, local, sel, cnt, None, None, B, Hq, Hkv, D, kp,
@@ -177,7 +190,7 @@ def test_custom_ops_are_registered_with_fake_kernels():
 
     import kinetics_amd  # noqa: F401
 
-    for name in ("append_paged_kv", "block_score_topk", "sparse_paged_decode", "dense_paged_decode"):
+    for name in ("append_paged_kv", "update_kv", "block_score_topk", "sparse_paged_decode", "dense_paged_decode"):
         assert hasattr(torch.ops.kinetics, name)
     # the fake kernel gives shape/dtype without running anything (what torch.compile needs)
     q = torch.empty(3, 4, 128, dtype=torch.bfloat16, device="meta")

@@ -637,6 +637,50 @@ def test_full_size_continuous_batching_mix(ops):
     torch.cuda.empty_cache()
 
 
+# --------------------------------------------------------------------------- ragged multi-token append
+
+
+@pytest.mark.parametrize("hkv", [1, 2, 8])
+def test_ragged_append_bit_exact(ops, hkv):
+    """Multi-token appends of mixed lengths (none, one, page-crossing, page-filling,
+    a long prefill) land bit for bit where the oracle puts them, and the mean keys
+    of the completed pages are refreshed; also through the update_kv custom op."""
+    rng = np.random.default_rng(500 + hkv)
+    before = [0, 5, PS * 2, PS * 3 + 15, 40, 7, PS, 0, 3]
+    new = [PS * 2 + 3, 1, 0, 18, PS * 40 + 5, 9, PS, 0, 13]
+    after = [a + n for a, n in zip(before, new)]
+    pb = P.make_problem(600 + hkv, after, num_kv_heads=hkv, group=1, table="fragmented")
+    nnz = sum(new)
+    k, v = P.randn_bf16(rng, (nnz, hkv, D)), P.randn_bf16(rng, (nnz, hkv, D))
+    append_indptr = np.concatenate([[0], np.cumsum(new)]).astype(np.int32)
+    for use_op in (False, True):
+        g = Gpu(pb)
+        g.kbar.zero_()
+        kt, vt, at = P.to_torch(k, DEV), P.to_torch(v, DEV), P.int_tensor(append_indptr, DEV)
+        if use_op:
+            torch.ops.kinetics.update_kv(kt, vt, at, g.kv, g.indices, g.indptr, g.last, g.kbar)
+        else:
+            ops.append_paged_kv_ragged(kt, vt, at, g.kv, g.kbar, g.indices, g.indptr, g.last, max_append_len=max(new))
+        torch.cuda.synchronize()
+        want_kv, want_kbar = pb.kv_cache.copy(), np.zeros_like(pb.kbar)
+        O.append_paged_kv_ragged(k, v, append_indptr, want_kv, want_kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
+        assert np.array_equal(P.from_torch(g.kv), want_kv)
+        assert np.array_equal(P.from_torch(g.kbar), want_kbar)
+        assert want_kbar.any()
+    # without a mean-key cache only the rows move
+    g = Gpu(pb)
+    ops.append_paged_kv_ragged(P.to_torch(k, DEV), P.to_torch(v, DEV), P.int_tensor(append_indptr, DEV), g.kv, None,
+                               g.indices, g.indptr, g.last)
+    assert np.array_equal(P.from_torch(g.kv), want_kv)
+    # one token per sequence is the decode append
+    pb1 = P.make_problem(700 + hkv, [PS * 3 + 16, 1, PS * 2 + 4], num_kv_heads=hkv, group=1)
+    g1, g2 = Gpu(pb1), Gpu(pb1)
+    ops.append_paged_kv(g1.k, g1.v, g1.kv, g1.kbar, g1.indices, g1.indptr, g1.last)
+    ops.append_paged_kv_ragged(g2.k, g2.v, P.int_tensor(np.arange(4, dtype=np.int32), DEV), g2.kv, g2.kbar, g2.indices,
+                               g2.indptr, g2.last)
+    assert torch.equal(g1.kv, g2.kv) and torch.equal(g1.kbar, g2.kbar)
+
+
 # --------------------------------------------------------------------------- graph capture / tracing
 
 

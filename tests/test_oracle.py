@@ -115,6 +115,57 @@ def test_build_kbar_covers_full_pages_only():
                 assert np.all(kbar[b, p] == sentinel)
 
 
+def _ragged_case(seed, before, new, hkv=2, slack=2):
+    """A cache holding ``before[b]`` tokens per sequence, the table after
+    appending ``new[b]`` more, and the rows to append."""
+    rng = np.random.default_rng(seed)
+    after = [a + n for a, n in zip(before, new)]
+    pb = P.make_problem(seed, after, num_kv_heads=hkv, group=1, kbar_slack=slack)
+    nnz = sum(new)
+    k, v = P.randn_bf16(rng, (nnz, hkv, D)), P.randn_bf16(rng, (nnz, hkv, D))
+    append_indptr = np.concatenate([[0], np.cumsum(new)]).astype(np.int32)
+    return pb, k, v, append_indptr, after
+
+
+def test_ragged_append_equals_token_by_token_append():
+    """The multi-token append is the single-token append (pinned above) applied
+    once per new token with the table of that moment; nothing else changes."""
+    before = [0, 5, PS * 2, PS * 3 + 15, 40, 7, PS]
+    new = [PS * 2 + 3, 1, 0, 18, PS * 4, 9, PS]
+    pb, k, v, append_indptr, after = _ragged_case(77, before, new)
+    kv_a, kbar_a = pb.kv_cache.copy(), pb.kbar.copy()
+    O.append_paged_kv_ragged(k, v, append_indptr, kv_a, kbar_a, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    kv_b, kbar_b = pb.kv_cache.copy(), pb.kbar.copy()
+    for b in range(pb.B):
+        pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+        for i in range(new[b]):
+            length = before[b] + i + 1
+            n_pages = (length + PS - 1) // PS
+            one_k = np.zeros((1, pb.Hkv, D), dtype=np.uint16)
+            one_v = np.zeros_like(one_k)
+            one_k[0], one_v[0] = k[append_indptr[b] + i], v[append_indptr[b] + i]
+            sub_kbar = kbar_b[b : b + 1]
+            O.append_paged_kv(one_k, one_v, kv_b, sub_kbar, pages[:n_pages].astype(np.int32),
+                              np.array([0, n_pages], dtype=np.int32), np.array([length - (n_pages - 1) * PS], dtype=np.int32))
+    assert np.array_equal(kv_a, kv_b)
+    assert np.array_equal(kbar_a, kbar_b)
+    # rows land where the closed form says, bit for bit
+    for b in range(pb.B):
+        pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+        for i in range(new[b]):
+            pos = before[b] + i
+            assert np.array_equal(kv_a[pages[pos // PS], 0, pos % PS], k[append_indptr[b] + i])
+            assert np.array_equal(kv_a[pages[pos // PS], 1, pos % PS], v[append_indptr[b] + i])
+    # bytes outside the appended rows are untouched
+    touched = np.zeros(kv_a.shape[:3], dtype=bool)
+    for b in range(pb.B):
+        pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+        for i in range(new[b]):
+            pos = before[b] + i
+            touched[pages[pos // PS], :, pos % PS] = True
+    assert np.array_equal(kv_a[~touched], pb.kv_cache[~touched])
+
+
 # --------------------------------------------------------------------------- scores
 
 
