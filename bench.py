@@ -38,6 +38,8 @@ WORKLOADS = {
     "qwen3-8b-share": (4096, 32768, 1, 4, 128, "Qwen3-8B one-GPU share (TP=8): 1 KV head, 4 Q heads"),
     "qwen3-32b-share": (1024, 32768, 1, 8, 256, "Qwen3-32B one-GPU share: 1 KV head, 8 Q heads"),
     "tiny": (8, 4096, 1, 4, 64, "CPU-runnable tiny case"),
+    # the command in the reference's benchmark/README.md: --batch_size 256 --gen_len 32768 (ctx 16384) --topk_page 64
+    "qwen3-8b-readme": (256, 16384, 1, 4, 64, "reference README example: Qwen3-8B share, B=256, ctx 16K, 64 pages"),
     # ragged: contexts uniform in [1024, ctx], budget min(topk, pages), half the tables fragmented
     "qwen3-0.6b-mix": (512, 32768, 8, 2, 64, "continuous-batching mix, Qwen3-0.6B attention: 8 KV heads, 16 Q heads"),
 }

@@ -263,9 +263,10 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  * kin_block_score_topk, first_page_offset as in kin_sparse_paged_decode (a
  * non-zero offset requires sink_pages >= 1: a padded page has no valid mean
  * key); lse is optional.  Needs no workspace.  One workgroup walks a whole
- * list (no split-K): faster than the three calls from about 256 lists
- * (batch * num_kv_heads) up, and for lists of up to ~129 pages at any batch
- * size; few long lists are better served by the three-call path.
+ * list (no split-K); with few lists it runs 8 or 16 waves instead of 4, which
+ * changes the fp32 summation order of the output (not the page lists or cache
+ * bytes).  Faster than the three calls except for few (< 256) and very long
+ * (topk > 512) lists.
  */
 int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
                               kin_bf16_t* kv_cache, kin_bf16_t* kbar,

@@ -1,9 +1,10 @@
 // Device-side building block: attention of one decode token over a list of
-// KV pages, for one (sequence, KV head, split) handled by one 256-thread
-// workgroup.  Shared by the stand-alone paged decode kernel and the fused
+// KV pages, for one (sequence, KV head, split) handled by one workgroup of NW
+// waves (4 in the stand-alone kernel; the fused step uses up to 16 when few
+// lists have to fill the GPU).  Shared by the stand-alone paged decode kernel and the fused
 // decode-step kernel.
 //
-// Work decomposition: the workgroup's 4 waves take the list's pages round-robin,
+// Work decomposition: the workgroup's NW waves take the list's pages round-robin,
 // one 8 KiB page (16 keys + 16 values of 128 bf16) per wave per iteration, and
 // keep private online-softmax state that is merged once at the end.
 //
@@ -128,12 +129,15 @@ struct AttendArgs {
 };
 
 constexpr int kAttendLdsBytes = 32768;  // 4 waves x 2 stages x 4 KiB; reused for the merge
+// K staging for NW waves, also large enough for the merge buffer [NW][4*NG][128] fp32 (NG <= 2).
+constexpr int attend_lds_bytes(int nw) { return nw * 8192; }
 
 // id_at(i) returns the (wave-uniform) physical page id of list entry i, 0 <= i < n.
 // emit(g, d, o, lse2) receives, once per (head g < G, column d), the normalised
 // output and the base-2 log-sum-exp (-inf and o = 0 for an empty part).
-// lds: kAttendLdsBytes, 16-byte aligned; sm_m / sm_l: 4 x (4*NG) floats each.
-template <int NG, typename IdAt, typename Emit>
+// lds: attend_lds_bytes(NW), 16-byte aligned; sm_m / sm_l: NW x (4*NG) floats each.
+// Every one of the workgroup's NW*64 threads calls this.
+template <int NG, int NW, typename IdAt, typename Emit>
 __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, unsigned char* lds,
                                             float (*sm_m)[4 * NG], float (*sm_l)[4 * NG], Emit emit) {
   const int tid = threadIdx.x;
@@ -184,21 +188,21 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
     for (int u = 0; u < 8; ++u) O[half][u] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // This wave takes list entries my_first, my_first+4, ...  The loop below is
+  // This wave takes list entries my_first, my_first+NW, ...  The loop below is
   // branch-free: a page past the end (or with an id outside the cache) is read
   // through an empty buffer descriptor -- zeros, no memory traffic -- and all
   // of its tokens are masked.
   const int my_first = p0 + w;
-  const int iters = (p1 > my_first) ? (p1 - my_first + 3) / 4 : 0;
+  const int iters = (p1 > my_first) ? (p1 - my_first + NW - 1) / NW : 0;
   const int n_last = n - 1;
   // Page ids are fetched one half-step before they are needed.
   auto load_id = [&](int it) -> int {
-    const int idx = my_first + 4 * it;
+    const int idx = my_first + NW * it;
     return id_at(idx < p1 ? idx : p0);
   };
   const int first_skip = a.first_skip;
   auto page_rsrc = [&](int it, int id, int& valid_tokens) {
-    const int idx = my_first + 4 * it;
+    const int idx = my_first + NW * it;
     const bool ok = idx < p1 && id >= 0 && (int64_t)id < a.num_pages;
     // The skipped slots of entry 0 are folded into one number: bits 8.. hold
     // the first counted slot, bits 0..7 one past the last.
@@ -302,7 +306,7 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
     }
   }
   __syncthreads();  // every wave is done with its K staging area
-  float* ow = reinterpret_cast<float*>(lds);  // [4 waves][4*NG heads][128]
+  float* ow = reinterpret_cast<float*>(lds);  // [NW waves][4*NG heads][128]
   if (kg == 0) {
 #pragma unroll
     for (int half = 0; half < NG; ++half) {
@@ -320,17 +324,17 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
   }
   __syncthreads();
 
-  // ---- merge the 4 waves and hand the results out -------------------------------
-#pragma unroll
-  for (int j = 0; j < 2 * NG; ++j) {
-    const int idx = tid + 256 * j;
+  // ---- merge the NW waves and hand the results out ------------------------------
+  for (int idx = tid; idx < 4 * NG * kHeadDim; idx += NW * 64) {
     const int g = idx >> 7, d = idx & 127;
     if (g < G) {
-      float mm = fmaxf(fmaxf(sm_m[0][g], sm_m[1][g]), fmaxf(sm_m[2][g], sm_m[3][g]));
+      float mm = kNegInf;
+#pragma unroll
+      for (int wv = 0; wv < NW; ++wv) mm = fmaxf(mm, sm_m[wv][g]);
       const float m_safe = (mm == kNegInf) ? 0.f : mm;
       float num = 0.f, den = 0.f;
 #pragma unroll
-      for (int wv = 0; wv < 4; ++wv) {
+      for (int wv = 0; wv < NW; ++wv) {
         const float sc = fast_exp2(sm_m[wv][g] - m_safe);
         num += ow[(wv * 4 * NG + g) * kHeadDim + d] * sc;
         den += sm_l[wv][g] * sc;

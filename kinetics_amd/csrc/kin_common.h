@@ -14,6 +14,7 @@ constexpr int kRowBytes = kHeadDim * 2;
 constexpr int kMaxGroup = 8;     // largest supported num_q_heads / num_kv_heads
 constexpr int kMaxTopk = 2048;
 constexpr int kMaxCandidates = 16384;
+constexpr int kNumCus = 256;     // compute units of the target GPU (MI355X)
 constexpr int kMaxFixedPages = 64;  // most sink / local pages that can be pinned into every list
 constexpr int kMaxLocalTokens = (kMaxFixedPages - 1) * kPageSize + 1;
 

@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
   const __attribute__((address_space(4))) int32_t* pl_c =
       reinterpret_cast<const __attribute__((address_space(4))) int32_t*>(reinterpret_cast<uintptr_t>(pl));
   const int64_t hq0 = (int64_t)b * p.num_q_heads + (int64_t)h * G;
-  attend_list<NG>(
+  attend_list<NG, 4>(
       a, [&](int i) -> int { return pl_c[i]; }, lds, sm_m, sm_l,
       [&](int g, int d, float o, float lse2) {
         const int64_t hq = hq0 + g;

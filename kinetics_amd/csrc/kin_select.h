@@ -1,5 +1,5 @@
 // Device-side building block: page scoring + top-k page selection for one
-// (sequence, KV head), run by one 256-thread workgroup.  Shared by the
+// (sequence, KV head), run by one workgroup of NT = 256 .. 1024 threads.  Shared by the
 // stand-alone selector kernel and the fused decode-step kernel.
 //
 //   phase 1  stream the sequence's representative keys (256 B each) once,
@@ -26,7 +26,7 @@ __device__ __forceinline__ uint32_t order_key(float f) {
   return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
 }
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 256;  // workgroup size of the stand-alone selector
 constexpr int kRankSortMax = 512;   // up to here winners are ordered by counting, above by bitonic sort
 
 // Wave-uniform description of one selection problem.
@@ -80,14 +80,16 @@ __host__ __device__ inline void split_pages(int n_pages, int last_len, int sink_
 // local pages (the open page last).  Returns the list length.  Ends with a
 // workgroup barrier: sel_lds is visible to every thread and keys / sortbuf are
 // free for reuse.
+// NT: threads of the workgroup (a multiple of 256, all of them call this).
 // UNROLL: independent 16-byte loads each lane keeps in flight while streaming the
 // mean keys (4 saturates HBM when thousands of workgroups run; a small grid
 // needs more per workgroup).
-template <int UNROLL = 4>
+template <int UNROLL = 4, int NT = kThreads>
 __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_lds) {
   constexpr int kUnroll = UNROLL;
+  constexpr int kRows = NT / 16;  // mean keys one pass of the workgroup covers
   __shared__ uint32_t hist[256];
-  __shared__ uint32_t wave_tot[4];
+  __shared__ uint32_t wave_tot[NT / 64];
   __shared__ uint32_t sh_bin, sh_remaining, sh_count;
 
   const int tid = threadIdx.x;
@@ -128,25 +130,25 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
   const int n_score = (k_eff > 0 || sc_out) ? n_cand : 0;
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(kb), 0, n_score > 0 ? (n_score - 1) * row_stride_b + kRowBytes : 0, 0x00020000);
-  const int sub = tid >> 4;  // 0..15: which of the 16 rows of a slot this lane helps with
+  const int sub = tid >> 4;  // which of the kRows rows of a slot this lane helps with
   const int lane_off = sub * row_stride_b + c16 * 16;
   u32x4 w[kUnroll];
 #pragma unroll
   for (int j = 0; j < kUnroll; ++j)
-    w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + j * 16 * row_stride_b, 0, kStreamLoad);
-  for (int base = 0; base < n_score; base += 16 * kUnroll) {
-    const int next_off = (base + 16 * kUnroll) * row_stride_b;
+    w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + j * kRows * row_stride_b, 0, kStreamLoad);
+  for (int base = 0; base < n_score; base += kRows * kUnroll) {
+    const int next_off = (base + kRows * kUnroll) * row_stride_b;
 #pragma unroll
     for (int j = 0; j < kUnroll; ++j) {
       const u32x4 x = w[j];
-      w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + j * 16 * row_stride_b, next_off, kStreamLoad);
+      w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + j * kRows * row_stride_b, next_off, kStreamLoad);
       float acc = 0.f;
       acc = fmaf(qm[0], bf16_lo(x.x), acc); acc = fmaf(qm[1], bf16_hi(x.x), acc);
       acc = fmaf(qm[2], bf16_lo(x.y), acc); acc = fmaf(qm[3], bf16_hi(x.y), acc);
       acc = fmaf(qm[4], bf16_lo(x.z), acc); acc = fmaf(qm[5], bf16_hi(x.z), acc);
       acc = fmaf(qm[6], bf16_lo(x.w), acc); acc = fmaf(qm[7], bf16_hi(x.w), acc);
       acc = row16_sum(acc);
-      const int row = base + j * 16 + sub;
+      const int row = base + j * kRows + sub;
       if (c16 == 0 && row < n_score) {
         keys[row] = order_key(acc);
         if (sc_out) sc_out[row] = acc;
@@ -160,9 +162,9 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
   uint32_t remaining = (uint32_t)k_eff;  // how many keys equal to the threshold are taken
   if (k_eff > 0 && k_eff < n_cand) {
     for (int shift = 24; shift >= 0; shift -= 8) {
-      hist[tid] = 0;
+      if (tid < 256) hist[tid] = 0;
       __syncthreads();
-      for (int i = tid; i < n_cand; i += kThreads) {
+      for (int i = tid; i < n_cand; i += NT) {
         const uint32_t key = keys[i];
         if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
       }
@@ -206,13 +208,13 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
   // ---- phase 3: gather, sort, translate --------------------------------------
   const bool rank_sort = (k_eff <= kRankSortMax);
   if (!rank_sort)
-    for (int i = tid; i < a.sort_cap; i += kThreads) sortbuf[i] = 0ull;
+    for (int i = tid; i < a.sort_cap; i += NT) sortbuf[i] = 0ull;
   if (tid == 0) sh_count = 0;
   __syncthreads();
   if (k_eff > 0) {
     // Keys above the threshold: any order (the sort fixes it).
     // Keys equal to it: the `remaining` lowest indices, found by an ordered count.
-    const int per = (n_cand + kThreads - 1) / kThreads;
+    const int per = (n_cand + NT - 1) / NT;
     const int lo = min(tid * per, n_cand), hi = min(lo + per, n_cand);
     uint32_t eq_cnt = 0;
     for (int i = lo; i < hi; ++i) {
@@ -253,7 +255,7 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
     // Small k: every winner counts the winners that beat it (entries are
     // distinct, so the counts are a permutation) and writes itself to that slot.
     // All lanes read the same LDS word per step: a broadcast, no conflicts.
-    for (int i = tid; i < k_eff; i += kThreads) {
+    for (int i = tid; i < k_eff; i += NT) {
       const unsigned long long mine = sortbuf[i];
       int rank = 0;
 #pragma unroll 8
@@ -267,7 +269,7 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
     // entries; the zero padding sinks to the end.
     for (int size = 2; size <= a.sort_cap; size <<= 1) {
       for (int stride = size >> 1; stride > 0; stride >>= 1) {
-        for (int i = tid; i < (a.sort_cap >> 1); i += kThreads) {
+        for (int i = tid; i < (a.sort_cap >> 1); i += NT) {
           const int lo_i = 2 * i - (i & (stride - 1));
           const int hi_i = lo_i + stride;
           const bool desc = ((lo_i & size) == 0);
@@ -280,13 +282,13 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
         __syncthreads();
       }
     }
-    for (int i = tid; i < k_eff; i += kThreads) {
+    for (int i = tid; i < k_eff; i += NT) {
       const uint32_t logical = 0xffffffffu - (uint32_t)(sortbuf[i] & 0xffffffffull);
       sel_lds[a.n_sink + i] = table[a.n_sink + logical];
       if (a.sel_logical) a.sel_logical[i] = (int32_t)(a.n_sink + logical);
     }
   }
-  for (int i = tid; i < a.n_sink + a.n_local; i += kThreads) {
+  for (int i = tid; i < a.n_sink + a.n_local; i += NT) {
     if (i < a.n_sink)
       sel_lds[i] = table[i];
     else

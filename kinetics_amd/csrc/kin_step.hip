@@ -1,5 +1,7 @@
 // Fused decode step: append -> score -> select -> attend in ONE launch, one
-// 256-thread workgroup per (sequence, KV head).
+// workgroup of NW waves per (sequence, KV head): 4 waves when there are enough
+// lists to fill the GPU, 8 or 16 when there are few (one wide workgroup per CU
+// then keeps as many loads in flight as four narrow ones would).
 //
 // Compared with the three stand-alone kernels this removes two dependent
 // dispatches, the selector's drain (its last workgroups finish their LDS-only
@@ -33,11 +35,12 @@ struct StepParams {
   float scale_log2;
 };
 
-template <int NG>
-__global__ __launch_bounds__(256, 2) void blocktopk_step_kernel(StepParams p) {
+template <int NG, int NW>
+__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kernel(StepParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  __shared__ float sm_m[4][4 * NG];
-  __shared__ float sm_l[4][4 * NG];
+  __shared__ float sm_m[NW][4 * NG];
+  __shared__ float sm_l[NW][4 * NG];
+  constexpr int NT = NW * 64;
 
   const int tid = threadIdx.x;
   const int item = blockIdx.x;
@@ -49,9 +52,9 @@ __global__ __launch_bounds__(256, 2) void blocktopk_step_kernel(StepParams p) {
   const int n_pages = pe - ps;
   if (n_pages <= 0) {  // empty sequence: nothing to append, select or attend
     if (p.sel_pages)
-      for (int i = tid; i < p.sel_stride; i += 256) p.sel_pages[(int64_t)item * p.sel_stride + i] = -1;
+      for (int i = tid; i < p.sel_stride; i += NT) p.sel_pages[(int64_t)item * p.sel_stride + i] = -1;
     if (p.sel_count && tid == 0) p.sel_count[item] = 0;
-    for (int i = tid; i < G * kHeadDim; i += 256) p.out[hq0 * kHeadDim + i] = 0;
+    for (int i = tid; i < G * kHeadDim; i += NT) p.out[hq0 * kHeadDim + i] = 0;
     if (p.lse && tid < G) p.lse[hq0 + tid] = kNegInf;
     return;
   }
@@ -108,10 +111,10 @@ __global__ __launch_bounds__(256, 2) void blocktopk_step_kernel(StepParams p) {
   s.keys = reinterpret_cast<uint32_t*>(smem);
   s.sortbuf = reinterpret_cast<unsigned long long*>(smem + (size_t)((p.kbar_pages + 3) & ~3) * 4);
   s.sort_cap = p.sort_cap;
-  const int n = score_select(s, sel_lds);
+  const int n = score_select<4, NT>(s, sel_lds);
   if (p.sel_pages) {
     int32_t* sel = p.sel_pages + (int64_t)item * p.sel_stride;
-    for (int i = tid; i < p.sel_stride; i += 256) sel[i] = (i < n) ? sel_lds[i] : -1;
+    for (int i = tid; i < p.sel_stride; i += NT) sel[i] = (i < n) ? sel_lds[i] : -1;
   }
   if (p.sel_count && tid == 0) p.sel_count[item] = n;
 
@@ -130,7 +133,7 @@ __global__ __launch_bounds__(256, 2) void blocktopk_step_kernel(StepParams p) {
   a.p1 = n;
   a.last_len = last_len;
   a.first_skip = p.first_page_offset;
-  attend_list<NG>(
+  attend_list<NG, NW>(
       a, [&](int i) -> int { return __builtin_amdgcn_readfirstlane(sel_lds[i]); }, smem, sm_m, sm_l,
       [&](int g, int d, float o, float lse2) {
         p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_bf16(o);
@@ -201,33 +204,40 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
   p.local_tokens = local_tokens;
   p.first_page_offset = first_page_offset;
   p.sort_cap = select_sort_cap(topk, kbar_pages);
+  // Waves per workgroup: aim for 16 waves per CU (8 with the two-pass kernel for
+  // groups above 4, whose registers allow no more) when the lists are few.
+  const int64_t items = (int64_t)batch * num_kv_heads;
+  if (items > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
+  int nw = 4;
+  if (p.group <= 4)
+    nw = items <= kNumCus ? 16 : (items <= 2 * kNumCus ? 8 : 4);
+  else
+    nw = items <= kNumCus ? 8 : 4;
   const size_t sel_scratch = select_lds_bytes(kbar_pages, p.sort_cap);
-  size_t region0 = sel_scratch > (size_t)kAttendLdsBytes ? sel_scratch : (size_t)kAttendLdsBytes;
+  size_t region0 = sel_scratch > (size_t)attend_lds_bytes(nw) ? sel_scratch : (size_t)attend_lds_bytes(nw);
   region0 = (region0 + 15) & ~(size_t)15;
   p.region0_bytes = (int)region0;
   p.num_pages = num_pages;
   const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
   p.scale_log2 = scale * 1.4426950408889634f;
   const size_t lds = region0 + (size_t)list_cap * 4;
-  const int64_t items = (int64_t)batch * num_kv_heads;
-  if (items > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (p.group <= 4) {
-    if (lds > 48 * 1024) {
-      st = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&blocktopk_step_kernel<1>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
-                     "hipFuncSetAttribute(blocktopk_step_kernel)");
-      if (st) return st;
-    }
-    blocktopk_step_kernel<1><<<(unsigned)items, 256, lds, s>>>(p);
-  } else {
-    if (lds > 48 * 1024) {
-      st = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&blocktopk_step_kernel<2>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
-                     "hipFuncSetAttribute(blocktopk_step_kernel)");
-      if (st) return st;
-    }
-    blocktopk_step_kernel<2><<<(unsigned)items, 256, lds, s>>>(p);
+  const void* kernel;
+  if (p.group <= 4)
+    kernel = nw == 16  ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 16>)
+             : nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 8>)
+                       : reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 4>);
+  else
+    kernel = nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<2, 8>)
+                     : reinterpret_cast<const void*>(&blocktopk_step_kernel<2, 4>);
+  if (lds > 48 * 1024) {
+    // Above the default dynamic-LDS allowance the runtime wants an explicit opt-in.
+    st = check_hip(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                   "hipFuncSetAttribute(blocktopk_step_kernel)");
+    if (st) return st;
   }
-  return check_hip(hipGetLastError(), "blocktopk_step_kernel launch");
+  void* args[] = {&p};
+  st = check_hip(hipLaunchKernel(kernel, dim3((unsigned)items), dim3(nw * 64), args, lds, s),
+                 "blocktopk_step_kernel launch");
+  return st;
 }

@@ -332,14 +332,15 @@ def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, ma
 def prefer_fused_step(batch: int, num_kv_heads: int, max_pages_per_seq: int, topk: int) -> bool:
     """Which of the two equivalent decode-step paths to use.  The single-launch
     kernel saves two dependent dispatches, the selector's drain and the attention
-    ramp-up (3-12 % per step on MI355X, the more the smaller the step), but one
+    ramp-up (3-30 % per step on MI355X, the more the smaller the step), and
+    widens its workgroups to 8 or 16 waves when there are few lists; but one
     workgroup walks a whole list: it has no split-K.  Measured on MI355X it wins
-    from 256 (sequence, KV head) lists up at every top-k, and for lists of up to
-    129 pages at every batch size; with fewer and longer lists the three-launch
-    path, which splits each list across workgroups, is faster (up to 2.8x at one
-    sequence with top-k 2048)."""
+    from 256 (sequence, KV head) lists up at every top-k, and for top-k up to 512
+    at every batch size; only few lists that are also very long (64 sequences
+    with top-k 2048: 377 vs 268 us) are served better by the three-launch path,
+    which splits each list across workgroups."""
     del max_pages_per_seq
-    return batch * num_kv_heads >= 256 or topk <= 128
+    return batch * num_kv_heads >= 256 or topk <= 512
 
 
 def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, out=None, lse=None,

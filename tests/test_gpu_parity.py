@@ -747,10 +747,13 @@ def test_custom_ops_trace_with_fullgraph(ops):
 # --------------------------------------------------------------------------- fused step
 
 
-@pytest.mark.parametrize("case", ["mixed", "hkv8", "g8", "fills", "ties", "long"])
+@pytest.mark.parametrize("case", ["mixed", "hkv8", "g8", "fills", "ties", "long", "many", "many_g8", "mid"])
 def test_fused_step_equals_three_calls(ops, case):
-    """kin_blocktopk_decode_step must give exactly what append + score/select +
-    attend give (same code, same order of operations), and match the oracle."""
+    """kin_blocktopk_decode_step must give what append + score/select + attend
+    give and match the oracle: cache bytes, mean keys and page lists bit for bit;
+    the output bit for bit when the fused kernel runs 4 waves per list like the
+    stand-alone one (more than 512 lists), else to fp32 summation order (wider
+    workgroups deal the pages to more waves)."""
     if case == "mixed":
         pb = P.make_problem(900, [PS * 40 + 3, PS * 9, 1, 0, PS * 3 + 1, PS * 130 + 16, 17], num_kv_heads=1, group=4, topk=8)
     elif case == "hkv8":
@@ -762,8 +765,17 @@ def test_fused_step_equals_three_calls(ops, case):
     elif case == "ties":
         pb = P.make_problem(904, [PS * 50 + 2, PS * 20 + 2], topk=7)
         pb.kbar[:] = pb.kbar[0, 0, 0]
-    else:
+    elif case == "long":
         pb = P.make_problem(905, [PS * 5000 + 5, PS * 900 + 1], topk=600, kbar_slack=3)  # bitonic path, big LDS
+    elif case == "many":       # > 512 lists: 4 waves per list
+        rng = np.random.default_rng(906)
+        pb = P.make_problem(906, [int(x) for x in rng.integers(1, PS * 30, size=600)], num_kv_heads=1, group=4, topk=6)
+    elif case == "many_g8":    # > 256 lists with a group above 4: 4 waves per list
+        rng = np.random.default_rng(907)
+        pb = P.make_problem(907, [int(x) for x in rng.integers(1, PS * 30, size=300)], num_kv_heads=1, group=8, topk=6)
+    else:                      # 257..512 lists: 8 waves per list
+        rng = np.random.default_rng(908)
+        pb = P.make_problem(908, [int(x) for x in rng.integers(1, PS * 40, size=150)], num_kv_heads=2, group=3, topk=9)
     a, b = Gpu(pb), Gpu(pb)
     check_table(ops, a)
     lse_a = torch.empty(pb.B, pb.Hq, dtype=torch.float32, device=DEV)
@@ -776,8 +788,12 @@ def test_fused_step_equals_three_calls(ops, case):
     torch.cuda.synchronize()
     assert torch.equal(a.kv, b.kv) and torch.equal(a.kbar, b.kbar)
     assert torch.equal(a.cnt, b.cnt) and torch.equal(a.sel, b.sel)
-    assert torch.equal(out_a, out_b)
-    assert torch.equal(lse_a, lse_b)
+    if case in ("many", "many_g8"):
+        assert torch.equal(out_a, out_b)
+        assert torch.equal(lse_a, lse_b)
+    else:
+        assert torch.allclose(out_a.float(), out_b.float(), rtol=1e-2, atol=1e-2)
+        assert torch.allclose(lse_a, lse_b, rtol=1e-5, atol=1e-5)
     # and against the oracle, end to end
     kv, kbar = pb.kv_cache.copy(), pb.kbar.copy()
     res = O.decode_step(pb.q, pb.k, pb.v, kv, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
@@ -788,7 +804,7 @@ def test_fused_step_equals_three_calls(ops, case):
     if np.array_equal(sel, res["sel_pages"]):
         assert_out_close(out_b, res["out"], f"fused {case} vs oracle end to end")
     else:
-        assert case in ("long",)  # only near-ties may reorder; checked by selection_matches elsewhere
+        assert case in ("long", "many", "many_g8", "mid")  # only near-ties may reorder; checked by selection_matches elsewhere
     # optional outputs may be omitted; no append when k, v are None
     c = Gpu(pb)
     ops.append_paged_kv(c.k, c.v, c.kv, c.kbar, c.indices, c.indptr, c.last)
