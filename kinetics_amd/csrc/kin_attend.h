@@ -112,6 +112,15 @@ __device__ __forceinline__ void page_pv(const u32x4 (&vr)[4], const float (&pr)[
 }
 
 
+// Zeroes the V rows of token slots outside [first_token, valid_tokens): their
+// probabilities are 0, but 0 * NaN would still poison the accumulator when an
+// unused cache slot happens to hold a NaN or Inf bit pattern.
+__device__ __forceinline__ void clear_unused_v_rows(u32x4 (&vr)[4], int first_token, int valid_tokens, int kg) {
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    if (!((unsigned)(4 * kg + r - first_token) < (unsigned)(valid_tokens - first_token))) vr[r] = u32x4{0u, 0u, 0u, 0u};
+}
+
 // Wave-uniform description of one list for attend_list().
 struct AttendArgs {
   const uint16_t* q_bh;  // the group's G query rows (contiguous, 128 bf16 each)
@@ -258,6 +267,7 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
         page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validA >> 8, validA & 255, kg);
         __builtin_amdgcn_sched_barrier(0);
         id_next = load_id(it + 2);  // lands while the P V products run
+        if (validA != kPageSize) clear_unused_v_rows(vA, validA >> 8, validA & 255, kg);  // partial page: rare
         page_pv<NG>(vA, pr, O);
       }
       {
@@ -274,6 +284,7 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
         page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validB >> 8, validB & 255, kg);
         __builtin_amdgcn_sched_barrier(0);
         id_next = load_id(it + 3);
+        if (validB != kPageSize) clear_unused_v_rows(vB, validB >> 8, validB & 255, kg);
         page_pv<NG>(vB, pr, O);
       }
     }

@@ -637,6 +637,49 @@ def test_full_size_continuous_batching_mix(ops):
     torch.cuda.empty_cache()
 
 
+def test_unused_cache_slots_may_hold_nan(ops):
+    """Slots past a sequence's last token, padding slots in front of it and pages
+    nobody owns are never initialised by a real cache: NaN and Inf bit patterns
+    there must not reach the output (0 * NaN) on any path."""
+    lengths = [PS * 30 + 3, PS * 4 + 13, 14, PS * 2, PS * 9 + 1, 0]
+    pb = P.make_problem(1234, lengths, num_kv_heads=2, group=3, topk=4)
+    kv = pb.kv_cache.copy()
+    offset = 12
+    used = np.zeros(kv.shape[0] * PS, dtype=bool)
+    for b, n in enumerate(lengths):
+        pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+        for t in range(offset if pages.size else 0, n):
+            used[pages[t // PS] * PS + t % PS] = True
+    poison = np.where(np.arange(used.size) % 2 == 0, 0x7FC0, 0xFF80).astype(np.uint16)   # NaN / -Inf
+    flat = kv.reshape(kv.shape[0], 2, PS, -1)            # a view: kv is contiguous
+    unused = (~used).reshape(kv.shape[0], PS)
+    for plane in range(2):
+        flat[:, plane][unused] = poison[~used, None]
+    assert np.shares_memory(flat, kv) and (kv == 0x7FC0).any()
+    pb.kv_cache = kv
+    for fused in (False, True):
+        g = Gpu(pb)
+        g.sel = torch.full((pb.B, pb.Hkv, ops.sel_list_capacity(pb.topk, 1, 20)), -7, dtype=torch.int32, device=DEV)
+        if fused:
+            out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, pb.topk, sel_pages=g.sel,
+                                            sel_count=g.cnt, sink_pages=1, local_tokens=20, first_page_offset=offset)
+        else:
+            ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
+            ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, pb.topk, g.sel, g.cnt, sink_pages=1, local_tokens=20)
+            out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, first_page_offset=offset, num_splits=2)
+        dense = ops.dense_paged_decode(g.q, g.kv, g.indices, g.indptr, g.last, pb.max_pages, first_page_offset=offset)
+        torch.cuda.synchronize()
+        assert torch.isfinite(out.float()).all() and torch.isfinite(dense.float()).all()
+        kv_o, kbar_o = pb.kv_cache.copy(), pb.kbar.copy()
+        res = O.decode_step(pb.q, pb.k, pb.v, kv_o, kbar_o, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk,
+                            sink_pages=1, local_tokens=20, first_page_offset=offset)
+        want, _ = O.sparse_paged_decode(pb.q, kv_o, g.sel.cpu().numpy(), g.cnt.cpu().numpy(), pb.last_page_len,
+                                        first_page_offset=offset)
+        assert_out_close(out, want, f"poisoned cache, fused={fused}")
+        wd, _ = O.dense_paged_decode(pb.q, kv_o, pb.page_indices, pb.page_indptr, pb.last_page_len, first_page_offset=offset)
+        assert_out_close(dense, wd, "poisoned cache, dense")
+
+
 # --------------------------------------------------------------------------- ragged multi-token append
 
 
