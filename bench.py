@@ -226,6 +226,9 @@ def main():
     ap.add_argument("--whole-layer", action="store_true",
                     help="also time the whole decoder layer (norms, GEMMs, MLP around the attention path), "
                          "the quantity benchmark/blocktopk.py prints")
+    ap.add_argument("--token-topk", action="store_true",
+                    help="also time token-level top-k decode (LiteSys' attn_topk policy) with the same token budget "
+                         "(topk_pages * 16 tokens, 4 sink tokens, a 16-token window)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) to scale profiler byte counters")
     args = ap.parse_args()
@@ -355,6 +358,31 @@ def main():
         result["dense_baseline"] = {"value": B / td, "unit": "tokens/s", "ms_per_step": td * 1e3, "steps": nd,
                                     "achieved_gbs": dense_bytes / td / 1e9, "frac": dense_bytes / td / 1e9 / HBM_PEAK_GBS,
                                     "sparse_over_dense": (B * K / elapsed) / (B / td)}
+    if args.token_topk:
+        # every key of the context is streamed once (256 B per token), then the listed tokens' K and V rows
+        ntok, sink, window = topk * PS, 4, 16
+        ws_tok = torch.empty(max(16, ops.token_topk_workspace_bytes(B, Hkv, st["max_pages_used"])), dtype=torch.uint8,
+                             device=device)
+        nt = max(3, min(20, K // 5))
+
+        def token_step():
+            ops.append_paged_kv(st["k"], st["v"], st["kv"], None, st["indices"], st["indptr"], st["last"])
+            ops.token_topk_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], ntok, st["max_pages_used"],
+                                  sink_tokens=sink, local_tokens=window, out=st["out"], workspace=ws_tok)
+
+        for _ in range(2):
+            token_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(nt):
+            token_step()
+        torch.cuda.synchronize()
+        tt = (time.perf_counter() - t0) / nt
+        tok_bytes = sum(Hkv * (L * 256 + min(L, ntok + sink + window) * 512 + 512) + 2 * Hkv * G * 256 for L in st["lengths"])
+        result["token_topk"] = {"topk_tokens": ntok, "sink_tokens": sink, "local_tokens": window, "ms_per_step": tt * 1e3,
+                                "value": B / tt, "unit": "tokens/s", "steps": nt, "algorithmic_bytes_per_step": tok_bytes,
+                                "achieved_gbs": tok_bytes / tt / 1e9, "frac": tok_bytes / tt / 1e9 / HBM_PEAK_GBS}
+        del ws_tok
     del st
     torch.cuda.empty_cache()
     if args.whole_layer and args.workload in WHOLE_LAYER_MODEL:

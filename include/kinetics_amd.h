@@ -281,6 +281,44 @@ int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const ki
                               float sm_scale, kin_stream_t stream);
 
 /*
+ * Token-level top-k sparse decode attention in one launch -- LiteSys'
+ * topk_sparsity policy (ref: LiteSys/litesys/attention/sparsity_utils.py:6-21)
+ * inside BatchKVManager.decode (ref: LiteSys/litesys/attention/batch_cache.py:154-168),
+ * on the paged cache.  Per (sequence, KV head): the logits of every token are
+ * averaged over the query group; the first sink_tokens tokens and the newest
+ * local_tokens tokens are always attended; of the tokens in between, the
+ * topk_tokens with the largest mean logit (ties: lowest position) are attended
+ * too; everything when the sequence has no more than sink + topk + local tokens.
+ * Attention itself is that of kin_sparse_paged_decode.  The token just appended
+ * must already be in the cache (kin_append_paged_kv first).
+ *
+ * A sequence of n_pages pages holds 16*(n_pages-1) + last_page_len[b] -
+ * first_page_offset tokens; token t sits in cache slot t + first_page_offset.
+ * Optional outputs: sel_tokens[b,h,0:n] (stride sel_stride >= topk + sink +
+ * local) the attended token positions -- sink tokens, selected tokens in
+ * ascending order, local tokens -- padded with -1, and sel_count[b,h] = n
+ * (-1 for a sequence with more than max_pages_per_seq pages, which is skipped:
+ * out = 0).  workspace: kin_token_topk_workspace_bytes(...) bytes of scratch
+ * (4 bytes per cache slot and KV head).  Reads every key of the context once:
+ * HBM traffic is about half of dense decode's.
+ * Limits: topk_tokens <= 4096, sink_tokens <= 64, local_tokens <= 1024.
+ */
+size_t kin_token_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq);
+
+int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
+                          const int32_t* page_indices, const int32_t* page_indptr,
+                          const int32_t* last_page_len,
+                          int topk_tokens, int sink_tokens, int local_tokens,
+                          int first_page_offset,
+                          int32_t* sel_tokens, int32_t* sel_count,
+                          kin_bf16_t* out, float* lse,
+                          void* workspace, size_t workspace_bytes,
+                          int batch, int num_q_heads, int num_kv_heads,
+                          int head_dim, int page_size, int64_t num_pages,
+                          int max_pages_per_seq, int sel_stride, float sm_scale,
+                          kin_stream_t stream);
+
+/*
  * Page-table metadata for a slot-based cache -- the paged replacement of
  * LiteSys' contiguous per-slot caches and kv_offset counters
  * (ref: LiteSys/litesys/attention/batch_cache.py:40-62,76-84).  Slot s owns the

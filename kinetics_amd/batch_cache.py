@@ -13,6 +13,9 @@ formulation, without touching the rest of the context.
 Supported configurations (anything else raises at construction):
   * no sparsity arguments                      -> dense paged decode
   * ``attn_block_topk=k`` (+ ``attn_local``)    -> block top-k with block size 16
+  * ``attn_topk=k`` (+ ``attn_local``)          -> token-level top-k (topk_sparsity,
+                                                  sparsity_utils.py:6-21), one launch that
+                                                  reads every key of the context once
   * ``attn_local`` alone                        -> sink + local window only: block top-k with
                                                   k = 0, whose window is LiteSys' ``local``
                                                   rounded up to the block grid (a superset, by
@@ -45,7 +48,7 @@ from . import ops
 
 PAGE = 16
 
-_UNSUPPORTED = ("attn_topk", "attn_random_select", "attn_random_nsample", "attn_stride")
+_UNSUPPORTED = ("attn_random_select", "attn_random_nsample", "attn_stride")
 
 
 class PagedBatchKVManager:
@@ -71,13 +74,22 @@ class PagedBatchKVManager:
             if kwargs.get(name) is not None:
                 raise NotImplementedError(f"{name} is a LiteSys research ablation that the paged kernels do not implement")
         self.block_topk = kwargs.get("attn_block_topk")
+        self.token_topk = kwargs.get("attn_topk")
+        if self.token_topk is not None:
+            # same rules as LiteSys (sparsity_utils.py:203-208)
+            assert self.block_topk is None, "Only one of the sparsity parameters can be provided"
+            if kwargs.get("attn_local") is None:
+                raise AssertionError("attn_local must be provided if use_nonlocal_sparsity is True")
+            if not 0 <= int(self.token_topk) <= 4096 or not 0 <= int(kwargs["attn_local"]) <= 1024:
+                raise NotImplementedError("attn_topk must be in [0, 4096] and attn_local in [0, 1024]")
         if self.block_topk is not None:
             if kwargs.get("attn_local") is None:
                 # same rule as LiteSys (sparsity_utils.py:207-208)
                 raise AssertionError("attn_local must be provided if use_nonlocal_sparsity is True")
             if kwargs.get("attn_block_size", PAGE) != PAGE:
                 raise NotImplementedError("block size must equal the page size (16)")
-        self.sparse = kwargs.get("attn_local") is not None
+        self.sparse = kwargs.get("attn_local") is not None and self.token_topk is None
+        self.token_local = int(kwargs["attn_local"]) if self.token_topk is not None else 0
         if self.sparse and self.block_topk is None:
             self.block_topk = 0                      # sink + local window only
         self.layer_skip = list(kwargs.get("attn_layer_skip", [0]))
@@ -109,6 +121,8 @@ class PagedBatchKVManager:
         self._cnt = torch.zeros(B, Hkv, dtype=torch.int32, device=dev)
         self._fused = ops.prefer_fused_step(B, Hkv, P, k)
         ws = max(ops.decode_workspace_bytes(B, Hq, Hkv, P), ops.decode_workspace_bytes(B, Hq, Hkv, self._sel.shape[2]), 16)
+        if self.token_topk is not None:
+            ws = max(ws, ops.token_topk_workspace_bytes(B, Hkv, P))
         self._ws = torch.empty(ws, dtype=torch.uint8, device=dev)
 
     # ------------------------------------------------------------------ LiteSys interface
@@ -141,7 +155,13 @@ class PagedBatchKVManager:
         self._v[slots] = value[:, :, 0, :]
         kv, kbar = self.kv_cache[layer_idx], self.kbar[layer_idx]
         sparse = self.sparse and layer_idx not in self.layer_skip
-        if sparse and self._fused:
+        if self.token_topk is not None and layer_idx not in self.layer_skip:
+            # token-level top-k: LiteSys' 4 sink tokens, the top tokens of the middle, the newest attn_local tokens
+            ops.append_paged_kv(self._k, self._v, kv, None, self.page_indices, self.page_indptr, self.last_page_len)
+            ops.token_topk_decode(self._q, kv, self.page_indices, self.page_indptr, self.last_page_len, self.token_topk,
+                                  self.pages_per_slot, sink_tokens=4, local_tokens=self.token_local, out=self._out,
+                                  workspace=self._ws)
+        elif sparse and self._fused:
             ops.blocktopk_decode_step(self._q, self._k, self._v, kv, kbar, self.page_indices, self.page_indptr,
                                       self.last_page_len, self.block_topk, out=self._out, sink_pages=self.sink_pages,
                                       local_tokens=self.local_tokens, first_page_offset=self.pad)

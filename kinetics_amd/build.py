@@ -17,7 +17,8 @@ INCLUDE = REPO_ROOT / "include"
 LIB_PATH = PKG_DIR / "libkinetics_amd.so"
 OBJ_DIR = PKG_DIR / "build"
 
-SOURCES = ["kin_api.hip", "kin_append.hip", "kin_score_topk.hip", "kin_decode.hip", "kin_step.hip", "kin_table.hip"]
+SOURCES = ["kin_api.hip", "kin_append.hip", "kin_score_topk.hip", "kin_decode.hip", "kin_step.hip", "kin_token_topk.hip",
+           "kin_table.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -141,6 +141,84 @@ constexpr int kAttendLdsBytes = 32768;  // 4 waves x 2 stages x 4 KiB; reused fo
 // K staging for NW waves, also large enough for the merge buffer [NW][4*NG][128] fp32 (NG <= 2).
 constexpr int attend_lds_bytes(int nw) { return nw * 8192; }
 
+// Common tail of the attention loops: merges the wave's 4 row groups, then the
+// workgroup's NW waves through LDS, and hands out the normalised results.
+// m_run / l_run / O: this lane's online-softmax state (see page_scores).
+template <int NG, int NW, typename Emit>
+__device__ __forceinline__ void attend_finish(float (&m_run)[NG], float (&l_run)[NG], floatx4 (&O)[NG][8], int G,
+                                              unsigned char* lds, float (*sm_m)[4 * NG], float (*sm_l)[4 * NG],
+                                              Emit emit) {
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l = tid & 63, kg = l >> 4, c16 = l & 15;
+  // LDS-direct loads that are still in flight (masked tail pages) must land
+  // before the staging area is reused below.
+  __builtin_amdgcn_s_waitcnt(0);
+
+  // ---- merge the 4 row groups of the wave (lanes l, l^16, l^32, l^48) --------
+  float m_w[NG], l_w[NG];
+#pragma unroll
+  for (int half = 0; half < NG; ++half) {
+    float mm = m_run[half];
+    mm = fmaxf(mm, __shfl_xor(mm, 16));
+    mm = fmaxf(mm, __shfl_xor(mm, 32));
+    const float m_safe = (mm == kNegInf) ? 0.f : mm;
+    const float sc = fast_exp2(m_run[half] - m_safe);
+    float ll = l_run[half] * sc;
+    ll += __shfl_xor(ll, 16);
+    ll += __shfl_xor(ll, 32);
+    m_w[half] = mm;
+    l_w[half] = ll;
+    const float s0 = quad_bcast<0>(sc), s1 = quad_bcast<1>(sc), s2 = quad_bcast<2>(sc), s3 = quad_bcast<3>(sc);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      float x0 = O[half][u][0] * s0, x1 = O[half][u][1] * s1, x2 = O[half][u][2] * s2, x3 = O[half][u][3] * s3;
+      x0 += __shfl_xor(x0, 16); x1 += __shfl_xor(x1, 16); x2 += __shfl_xor(x2, 16); x3 += __shfl_xor(x3, 16);
+      x0 += __shfl_xor(x0, 32); x1 += __shfl_xor(x1, 32); x2 += __shfl_xor(x2, 32); x3 += __shfl_xor(x3, 32);
+      O[half][u] = floatx4{x0, x1, x2, x3};
+    }
+  }
+  __syncthreads();  // every wave is done with its K staging area
+  float* ow = reinterpret_cast<float*>(lds);  // [NW waves][4*NG heads][128]
+  if (kg == 0) {
+#pragma unroll
+    for (int half = 0; half < NG; ++half) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float* dst = ow + ((w * 4 * NG + 4 * half + i) * kHeadDim + 8 * c16);
+        *reinterpret_cast<float4*>(dst) = make_float4(O[half][0][i], O[half][1][i], O[half][2][i], O[half][3][i]);
+        *reinterpret_cast<float4*>(dst + 4) = make_float4(O[half][4][i], O[half][5][i], O[half][6][i], O[half][7][i]);
+      }
+      if (l < 4) {
+        sm_m[w][4 * half + l] = m_w[half];
+        sm_l[w][4 * half + l] = l_w[half];
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- merge the NW waves and hand the results out ------------------------------
+  for (int idx = tid; idx < 4 * NG * kHeadDim; idx += NW * 64) {
+    const int g = idx >> 7, d = idx & 127;
+    if (g < G) {
+      float mm = kNegInf;
+#pragma unroll
+      for (int wv = 0; wv < NW; ++wv) mm = fmaxf(mm, sm_m[wv][g]);
+      const float m_safe = (mm == kNegInf) ? 0.f : mm;
+      float num = 0.f, den = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < NW; ++wv) {
+        const float sc = fast_exp2(sm_m[wv][g] - m_safe);
+        num += ow[(wv * 4 * NG + g) * kHeadDim + d] * sc;
+        den += sm_l[wv][g] * sc;
+      }
+      const float o = (den > 0.f) ? num / den : 0.f;
+      const float lse2 = (den > 0.f) ? mm + fast_log2(den) : kNegInf;
+      emit(g, d, o, lse2);
+    }
+  }
+}
+
 // id_at(i) returns the (wave-uniform) physical page id of list entry i, 0 <= i < n.
 // emit(g, d, o, lse2) receives, once per (head g < G, column d), the normalised
 // output and the base-2 log-sum-exp (-inf and o = 0 for an empty part).
@@ -289,72 +367,7 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
       }
     }
   }
-  // LDS-direct loads that are still in flight (masked tail pages) must land
-  // before the staging area is reused below.
-  __builtin_amdgcn_s_waitcnt(0);
-
-  // ---- merge the 4 row groups of the wave (lanes l, l^16, l^32, l^48) --------
-  float m_w[NG], l_w[NG];
-#pragma unroll
-  for (int half = 0; half < NG; ++half) {
-    float mm = m_run[half];
-    mm = fmaxf(mm, __shfl_xor(mm, 16));
-    mm = fmaxf(mm, __shfl_xor(mm, 32));
-    const float m_safe = (mm == kNegInf) ? 0.f : mm;
-    const float sc = fast_exp2(m_run[half] - m_safe);
-    float ll = l_run[half] * sc;
-    ll += __shfl_xor(ll, 16);
-    ll += __shfl_xor(ll, 32);
-    m_w[half] = mm;
-    l_w[half] = ll;
-    const float s0 = quad_bcast<0>(sc), s1 = quad_bcast<1>(sc), s2 = quad_bcast<2>(sc), s3 = quad_bcast<3>(sc);
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      float x0 = O[half][u][0] * s0, x1 = O[half][u][1] * s1, x2 = O[half][u][2] * s2, x3 = O[half][u][3] * s3;
-      x0 += __shfl_xor(x0, 16); x1 += __shfl_xor(x1, 16); x2 += __shfl_xor(x2, 16); x3 += __shfl_xor(x3, 16);
-      x0 += __shfl_xor(x0, 32); x1 += __shfl_xor(x1, 32); x2 += __shfl_xor(x2, 32); x3 += __shfl_xor(x3, 32);
-      O[half][u] = floatx4{x0, x1, x2, x3};
-    }
-  }
-  __syncthreads();  // every wave is done with its K staging area
-  float* ow = reinterpret_cast<float*>(lds);  // [NW waves][4*NG heads][128]
-  if (kg == 0) {
-#pragma unroll
-    for (int half = 0; half < NG; ++half) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float* dst = ow + ((w * 4 * NG + 4 * half + i) * kHeadDim + 8 * c16);
-        *reinterpret_cast<float4*>(dst) = make_float4(O[half][0][i], O[half][1][i], O[half][2][i], O[half][3][i]);
-        *reinterpret_cast<float4*>(dst + 4) = make_float4(O[half][4][i], O[half][5][i], O[half][6][i], O[half][7][i]);
-      }
-      if (l < 4) {
-        sm_m[w][4 * half + l] = m_w[half];
-        sm_l[w][4 * half + l] = l_w[half];
-      }
-    }
-  }
-  __syncthreads();
-
-  // ---- merge the NW waves and hand the results out ------------------------------
-  for (int idx = tid; idx < 4 * NG * kHeadDim; idx += NW * 64) {
-    const int g = idx >> 7, d = idx & 127;
-    if (g < G) {
-      float mm = kNegInf;
-#pragma unroll
-      for (int wv = 0; wv < NW; ++wv) mm = fmaxf(mm, sm_m[wv][g]);
-      const float m_safe = (mm == kNegInf) ? 0.f : mm;
-      float num = 0.f, den = 0.f;
-#pragma unroll
-      for (int wv = 0; wv < NW; ++wv) {
-        const float sc = fast_exp2(sm_m[wv][g] - m_safe);
-        num += ow[(wv * 4 * NG + g) * kHeadDim + d] * sc;
-        den += sm_l[wv][g] * sc;
-      }
-      const float o = (den > 0.f) ? num / den : 0.f;
-      const float lse2 = (den > 0.f) ? mm + fast_log2(den) : kNegInf;
-      emit(g, d, o, lse2);
-    }
-  }
+  attend_finish<NG, NW>(m_run, l_run, O, G, lds, sm_m, sm_l, emit);
 }
 
 }  // namespace kin

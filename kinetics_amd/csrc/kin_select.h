@@ -75,6 +75,36 @@ __host__ __device__ inline void split_pages(int n_pages, int last_len, int sink_
   if (n_cand > cap) n_cand = cap > 0 ? cap : 0;
 }
 
+// One digit of a most-significant-digit-first radix select, run by ONE wave:
+// hist[256] counts the keys that match the digits fixed so far, by their next
+// digit; `remaining` of them are wanted, largest first.  Writes the digit that
+// holds the threshold and how many keys of that digit are still wanted.
+__device__ __forceinline__ void radix_pick_bin(const uint32_t* hist, uint32_t remaining, int lane, uint32_t* out_bin,
+                                               uint32_t* out_remaining) {
+  // Lane j owns bins 255-4j .. 252-4j (highest first); an inclusive scan over
+  // lanes counts the keys in all bins at or above the lane's lowest.  The bin
+  // where the running count first reaches `remaining` holds the threshold digit.
+  const int top = 255 - 4 * lane;
+  const uint32_t c0 = hist[top], c1 = hist[top - 1], c2 = hist[top - 2], c3 = hist[top - 3];
+  const uint32_t mine = c0 + c1 + c2 + c3;
+  uint32_t incl = mine;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t up = __shfl_up(incl, off);
+    if (lane >= off) incl += up;
+  }
+  uint32_t run = incl - mine;  // keys in bins above this lane's
+  if (run < remaining && remaining <= incl) {
+    int bin = top;
+    uint32_t c = c0;
+    if (run + c < remaining) { run += c; bin = top - 1; c = c1; }
+    if (run + c < remaining) { run += c; bin = top - 2; c = c2; }
+    if (run + c < remaining) { run += c; bin = top - 3; }
+    *out_bin = (uint32_t)bin;
+    *out_remaining = remaining - run;
+  }
+}
+
 // Writes the page list to sel_lds (LDS, >= n_sink + topk + n_local entries):
 // the sink pages, then the ordered physical ids of the k_eff winners, then the
 // local pages (the open page last).  Returns the list length.  Ends with a
@@ -169,31 +199,7 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
         if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
       }
       __syncthreads();
-      if (wave == 0) {
-        // Lane j owns bins 255-4j .. 252-4j (highest first); an inclusive scan
-        // over lanes counts the keys in all bins at or above the lane's lowest.
-        // The bin where the running count first reaches `remaining` holds the
-        // threshold digit.
-        const int top = 255 - 4 * lane;
-        const uint32_t c0 = hist[top], c1 = hist[top - 1], c2 = hist[top - 2], c3 = hist[top - 3];
-        const uint32_t mine = c0 + c1 + c2 + c3;
-        uint32_t incl = mine;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-          const uint32_t up = __shfl_up(incl, off);
-          if (lane >= off) incl += up;
-        }
-        uint32_t run = incl - mine;  // keys in bins above this lane's
-        if (run < remaining && remaining <= incl) {
-          int bin = top;
-          uint32_t c = c0;
-          if (run + c < remaining) { run += c; bin = top - 1; c = c1; }
-          if (run + c < remaining) { run += c; bin = top - 2; c = c2; }
-          if (run + c < remaining) { run += c; bin = top - 3; }
-          sh_bin = (uint32_t)bin;
-          sh_remaining = remaining - run;
-        }
-      }
+      if (wave == 0) radix_pick_bin(hist, remaining, lane, &sh_bin, &sh_remaining);
       __syncthreads();
       prefix |= sh_bin << shift;
       mask |= 255u << shift;

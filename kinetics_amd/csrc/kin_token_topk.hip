@@ -1,0 +1,199 @@
+// Token-level top-k sparse decode attention in one launch: one workgroup per
+// (sequence, KV head) scores every token of the context, keeps the sink tokens,
+// the local window and the top-k tokens in between, and attends to them
+// (token_score_select() + attend_tokens(), kin_token.h).
+#include "kin_token.h"
+
+namespace kin {
+
+struct TokenTopkParams {
+  const uint16_t* q;
+  const uint16_t* kv;
+  const int32_t* page_indices;
+  const int32_t* page_indptr;
+  const int32_t* last_page_len;
+  int32_t* sel_tokens;  // optional [lists, sel_stride]
+  int32_t* sel_count;   // optional [lists]
+  uint16_t* out;
+  float* lse;           // optional
+  uint32_t* keys;       // workspace: [lists, max_pages_per_seq * 16]
+  int num_q_heads, num_kv_heads, group;
+  int topk, sink_tokens, local_tokens, first_page_offset;
+  int max_pages_per_seq, sel_stride;
+  int64_t num_pages;
+  float scale_log2;
+};
+
+// Dynamic LDS: K staging attend_lds_bytes(NW) | int32 list[sink + topk + local]
+template <int NG, int NW>
+__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(TokenTopkParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  __shared__ float sm_m[NW][4 * NG];
+  __shared__ float sm_l[NW][4 * NG];
+  constexpr int NT = NW * 64;
+
+  const int tid = threadIdx.x;
+  const int item = blockIdx.x;
+  const int b = item / p.num_kv_heads, h = item - b * p.num_kv_heads;
+  const int G = p.group;
+  const int64_t hq0 = (int64_t)b * p.num_q_heads + (int64_t)h * G;
+
+  const int ps = p.page_indptr[b], pe = p.page_indptr[b + 1];
+  const int n_pages = pe - ps;
+  const int last_len = p.last_page_len[b];
+  const int kv_len = (n_pages - 1) * kPageSize + min(max(last_len, 1), kPageSize);
+  const int seq_len = kv_len - p.first_page_offset;  // tokens of the sequence
+  int32_t* sel_out = p.sel_tokens ? p.sel_tokens + (int64_t)item * p.sel_stride : nullptr;
+  if (n_pages <= 0 || seq_len <= 0 || n_pages > p.max_pages_per_seq) {
+    // Nothing to attend (or a sequence longer than the scratch array was sized for:
+    // reported as count -1 rather than written past its end).
+    if (sel_out)
+      for (int i = tid; i < p.sel_stride; i += NT) sel_out[i] = -1;
+    if (p.sel_count && tid == 0) p.sel_count[item] = (n_pages > p.max_pages_per_seq) ? -1 : 0;
+    for (int i = tid; i < G * kHeadDim; i += NT) p.out[hq0 * kHeadDim + i] = 0;
+    if (p.lse && tid < G) p.lse[hq0 + tid] = kNegInf;
+    return;
+  }
+
+  int32_t* list = reinterpret_cast<int32_t*>(smem + attend_lds_bytes(NW));
+  TokenArgs t;
+  t.q_bh = p.q + hq0 * kHeadDim;
+  t.kvb = reinterpret_cast<const char*>(p.kv) + (int64_t)h * kRowBytes;
+  t.row_bytes = p.num_kv_heads * kRowBytes;
+  t.page_bytes = 2 * kPageSize * t.row_bytes;
+  t.span = t.page_bytes - h * kRowBytes;
+  t.num_pages = p.num_pages;
+  t.G = G;
+  t.table = p.page_indices + ps;
+  t.n_pages = n_pages;
+  t.pad = p.first_page_offset;
+  t.n_sink = min(p.sink_tokens, seq_len);
+  t.n_local = min(p.local_tokens, seq_len - t.n_sink);
+  t.n_dyn = seq_len - t.n_sink - t.n_local;
+  t.topk = p.topk;
+  t.keys = p.keys + (int64_t)item * p.max_pages_per_seq * kPageSize;
+  t.list = list;
+  t.sel_tokens = sel_out;
+  const int n = token_score_select<NG, NW>(t, smem);
+  if (sel_out)
+    for (int i = n + tid; i < p.sel_stride; i += NT) sel_out[i] = -1;
+  if (p.sel_count && tid == 0) p.sel_count[item] = n;
+
+  AttendArgs a;
+  a.q_bh = t.q_bh;
+  a.kvb = t.kvb;
+  a.row_bytes = t.row_bytes;
+  a.page_bytes = t.page_bytes;
+  a.span = t.span;
+  a.num_pages = p.num_pages;
+  a.G = G;
+  a.scale_log2 = p.scale_log2;
+  a.n = n;
+  a.p0 = 0;
+  a.p1 = n;
+  a.last_len = kPageSize;
+  a.first_skip = 0;
+  attend_tokens<NG, NW>(a, list, smem, sm_m, sm_l, [&](int g, int d, float o, float lse2) {
+    p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_bf16(o);
+    if (p.lse && d == 0) p.lse[hq0 + g] = lse2 * kLn2;
+  });
+}
+
+}  // namespace kin
+
+extern "C" {
+
+size_t kin_token_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq) {
+  if (batch <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0) return 0;
+  return (size_t)batch * num_kv_heads * max_pages_per_seq * kin::kPageSize * sizeof(uint32_t);
+}
+
+int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const int32_t* page_indices,
+                          const int32_t* page_indptr, const int32_t* last_page_len, int topk_tokens,
+                          int sink_tokens, int local_tokens, int first_page_offset, int32_t* sel_tokens,
+                          int32_t* sel_count, kin_bf16_t* out, float* lse, void* workspace, size_t workspace_bytes,
+                          int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
+                          int64_t num_pages, int max_pages_per_seq, int sel_stride, float sm_scale,
+                          kin_stream_t stream) {
+  using namespace kin;
+  const char* fn = "kin_token_topk_decode";
+  if (!q || !kv_cache || !page_indices || !page_indptr || !last_page_len || !out)
+    return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
+  int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size);
+  if (st) return st;
+  st = check_first_page_offset(fn, first_page_offset);
+  if (st) return st;
+  if (num_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_pages=%lld must be >= 1", fn, (long long)num_pages);
+  if (num_pages > 0x7fffffffLL / kPageSize)
+    return fail(KIN_ERR_UNSUPPORTED, "%s: num_pages=%lld: token ids do not fit 31 bits", fn, (long long)num_pages);
+  if (topk_tokens < 0 || sink_tokens < 0 || local_tokens < 0)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: topk_tokens=%d, sink_tokens=%d and local_tokens=%d must not be negative", fn,
+                topk_tokens, sink_tokens, local_tokens);
+  if (topk_tokens > kMaxTopkTokens || sink_tokens > kMaxSinkTokens || local_tokens > kMaxWindowTokens)
+    return fail(KIN_ERR_UNSUPPORTED, "%s: limits are topk_tokens <= %d, sink_tokens <= %d, local_tokens <= %d", fn,
+                kMaxTopkTokens, kMaxSinkTokens, kMaxWindowTokens);
+  if (max_pages_per_seq < 1)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: max_pages_per_seq=%d must be >= 1", fn, max_pages_per_seq);
+  const int list_cap = topk_tokens + sink_tokens + local_tokens;
+  if (sel_tokens && sel_stride < list_cap)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must be at least topk + sink + local tokens = %d", fn, sel_stride,
+                list_cap);
+  if (sel_tokens && !sel_count) return fail(KIN_ERR_NULL_POINTER, "%s: sel_tokens given without sel_count", fn);
+  if (!aligned16(q) || !aligned16(kv_cache) || !aligned16(out))
+    return fail(KIN_ERR_MISALIGNED, "%s: q, kv_cache and out must be 16-byte aligned", fn);
+  const size_t need = kin_token_topk_workspace_bytes(batch, num_kv_heads, max_pages_per_seq);
+  if (batch == 0) return KIN_OK;
+  if (!workspace || workspace_bytes < need)
+    return fail(KIN_ERR_WORKSPACE, "%s: needs %zu workspace bytes, got %zu", fn, need,
+                workspace ? workspace_bytes : (size_t)0);
+  if (!aligned16(workspace)) return fail(KIN_ERR_MISALIGNED, "%s: workspace must be 16-byte aligned", fn);
+
+  TokenTopkParams p;
+  p.q = q;
+  p.kv = kv_cache;
+  p.page_indices = page_indices;
+  p.page_indptr = page_indptr;
+  p.last_page_len = last_page_len;
+  p.sel_tokens = sel_tokens;
+  p.sel_count = sel_count;
+  p.out = out;
+  p.lse = lse;
+  p.keys = static_cast<uint32_t*>(workspace);
+  p.num_q_heads = num_q_heads;
+  p.num_kv_heads = num_kv_heads;
+  p.group = num_q_heads / num_kv_heads;
+  p.topk = topk_tokens;
+  p.sink_tokens = sink_tokens;
+  p.local_tokens = local_tokens;
+  p.first_page_offset = first_page_offset;
+  p.max_pages_per_seq = max_pages_per_seq;
+  p.sel_stride = sel_stride;
+  p.num_pages = num_pages;
+  const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
+  p.scale_log2 = scale * 1.4426950408889634f;
+
+  const int64_t items = (int64_t)batch * num_kv_heads;
+  if (items > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
+  // Waves per workgroup: 8 when the lists are too few to fill the GPU with 4-wave
+  // workgroups (the per-token addressing needs ~140 registers, so 16 do not fit).
+  const int nw = items <= 2 * kNumCus ? 8 : 4;
+  const size_t lds = (size_t)attend_lds_bytes(nw) + (size_t)(list_cap > 0 ? list_cap : 1) * 4;
+  const void* kernel;
+  if (p.group <= 4)
+    kernel = nw == 8 ? reinterpret_cast<const void*>(&token_topk_kernel<1, 8>)
+                     : reinterpret_cast<const void*>(&token_topk_kernel<1, 4>);
+  else
+    kernel = nw == 8 ? reinterpret_cast<const void*>(&token_topk_kernel<2, 8>)
+                     : reinterpret_cast<const void*>(&token_topk_kernel<2, 4>);
+  if (lds > 48 * 1024) {
+    st = check_hip(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                   "hipFuncSetAttribute(token_topk_kernel)");
+    if (st) return st;
+  }
+  void* args[] = {&p};
+  return check_hip(hipLaunchKernel(kernel, dim3((unsigned)items), dim3(nw * 64), args, lds,
+                                   static_cast<hipStream_t>(stream)),
+                   "token_topk_kernel launch");
+}
+
+}  // extern "C"

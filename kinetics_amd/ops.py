@@ -382,6 +382,48 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
     return out
 
 
+def token_topk_workspace_bytes(batch: int, num_kv_heads: int, max_pages_per_seq: int) -> int:
+    return int(_lib.load().kin_token_topk_workspace_bytes(int(batch), int(num_kv_heads), int(max_pages_per_seq)))
+
+
+def token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, topk_tokens: int, max_pages_per_seq: int,
+                      sink_tokens: int = 4, local_tokens: int = 1, first_page_offset: int = 0, out=None, lse=None,
+                      sel_tokens=None, sel_count=None, workspace=None, sm_scale: float = 0.0):
+    """Token-level top-k sparse decode attention: LiteSys' ``topk_sparsity``
+    (LiteSys/litesys/attention/sparsity_utils.py:6-21) inside its decode
+    (batch_cache.py:154-168) in one launch on the paged cache.  The first
+    ``sink_tokens`` and newest ``local_tokens`` tokens are always attended; of
+    the rest, the ``topk_tokens`` with the largest group-mean logit per KV
+    head.  The new token must already be appended.  Returns ``out``."""
+    dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, None)
+    _table(page_indices, page_indptr, last_page_len, batch, dev)
+    sel_stride = 0
+    if (sel_tokens is None) != (sel_count is None):
+        raise ValueError("sel_tokens and sel_count must both be given or both be None")
+    if sel_tokens is not None:
+        _require(sel_tokens, "sel_tokens", torch.int32, 3, dev)
+        _require(sel_count, "sel_count", torch.int32, 2, dev)
+        if sel_tokens.shape[:2] != (batch, hkv) or tuple(sel_count.shape) != (batch, hkv):
+            raise ValueError(f"sel_tokens/sel_count must be [{batch}, {hkv}, stride] / [{batch}, {hkv}]")
+        sel_stride = sel_tokens.shape[2]
+    need = token_topk_workspace_bytes(batch, hkv, max_pages_per_seq)
+    if workspace is None:
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+    else:
+        _require(workspace, "workspace", torch.uint8, 1, dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(
+            lib.kin_token_topk_decode(
+                _ptr(q), _ptr(kv_cache), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), int(topk_tokens),
+                int(sink_tokens), int(local_tokens), int(first_page_offset), _ptr(sel_tokens), _ptr(sel_count), _ptr(out),
+                _ptr(lse), _ptr(workspace), workspace.numel(), batch, hq, hkv, d, ps, num_pages, int(max_pages_per_seq),
+                sel_stride, float(sm_scale), _stream(dev),
+            )
+        )
+    return out
+
+
 def build_slot_page_table(seq_lens, pages_per_slot, page_size, page_indices, page_indptr, last_page_len, slot_ids=None) -> None:
     """CSR page table for a cache where slot ``s`` owns pages
     ``s*pages_per_slot ...`` (the paged stand-in for LiteSys' contiguous
@@ -458,6 +500,28 @@ torch.library.define(
     "(Tensor q, Tensor kv_cache, Tensor page_indices, Tensor page_indptr, Tensor last_page_len, "
     "int max_pages_per_seq, Tensor? workspace, float sm_scale, int num_splits, int first_page_offset=0) -> Tensor",
 )
+
+
+torch.library.define(
+    "kinetics::token_topk_decode",
+    "(Tensor q, Tensor kv_cache, Tensor page_indices, Tensor page_indptr, Tensor last_page_len, int topk_tokens, "
+    "int max_pages_per_seq, int sink_tokens, int local_tokens, int first_page_offset, Tensor(a!) workspace, "
+    "float sm_scale) -> Tensor",
+)
+
+
+@torch.library.impl("kinetics::token_topk_decode", "cuda")
+def _token_impl(q, kv_cache, page_indices, page_indptr, last_page_len, topk_tokens, max_pages_per_seq, sink_tokens,
+                local_tokens, first_page_offset, workspace, sm_scale):
+    return token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, topk_tokens, max_pages_per_seq,
+                             sink_tokens=sink_tokens, local_tokens=local_tokens, first_page_offset=first_page_offset,
+                             workspace=workspace, sm_scale=sm_scale)
+
+
+@torch.library.register_fake("kinetics::token_topk_decode")
+def _token_fake(q, kv_cache, page_indices, page_indptr, last_page_len, topk_tokens, max_pages_per_seq, sink_tokens,
+                local_tokens, first_page_offset, workspace, sm_scale):
+    return torch.empty_like(q)
 
 
 torch.library.define(

@@ -395,14 +395,63 @@ def litesys_blockwise_topk_mask(mean_logits, seq_len, topk_block, local, sink=4,
     return keep
 
 
-def litesys_decode(q, K, V, topk_block, local, sink=4, block_size=16, sm_scale=None):
+def litesys_topk_mask(mean_logits, seq_len, topk, local, sink=4):
+    """LiteSys/litesys/attention/sparsity_utils.py:6-21 for one sequence and one
+    KV head: everything when ``seq_len <= sink + topk + local`` (:9-12);
+    otherwise the ``sink`` first tokens, the ``local`` newest and, of the tokens
+    in between, the ``topk`` with the largest group-mean logit (:13-19)."""
+    keep = np.ones(seq_len, dtype=bool)
+    if seq_len <= sink + topk + local:
+        return keep
+    dyn = np.asarray(mean_logits[sink : seq_len - local], dtype=np.float64)
+    dyn_keep = np.zeros(len(dyn), dtype=bool)
+    dyn_keep[select_topk(dyn, topk)] = True
+    keep[sink : seq_len - local] = dyn_keep
+    return keep
+
+
+def token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, topk, sink=4, local=1, first_page_offset=0,
+                      sm_scale=None):
+    """Token-level top-k decode on the paged cache: per sequence the cache is
+    read back into LiteSys' contiguous form (token t = cache slot t +
+    first_page_offset) and litesys_decode(policy "topk") does the rest.
+    Returns (out [B, Hq, D] float64, keep list[b] of bool [Hkv, seq_len],
+    mean_logits list[b] of float64 [Hkv, seq_len])."""
+    B, Hq, D = q.shape
+    ps = kv_cache.shape[2]
+    out = np.zeros((B, Hq, D))
+    keeps, means = [], []
+    qf = bf16_to_f32(q).astype(np.float64)
+    for b in range(B):
+        pages = seq_pages(page_indices, page_indptr, b)
+        kv_len = (len(pages) - 1) * ps + int(last_page_len[b]) if len(pages) else 0
+        if kv_len - first_page_offset <= 0:
+            keeps.append(None)
+            means.append(None)
+            continue
+        K = bf16_to_f32(kv_cache[pages, 0]).reshape(len(pages) * ps, -1, D)[first_page_offset:kv_len]
+        V = bf16_to_f32(kv_cache[pages, 1]).reshape(len(pages) * ps, -1, D)[first_page_offset:kv_len]
+        o, keep, mean = litesys_decode(qf[b], K, V, topk, local, sink=sink, sm_scale=sm_scale, policy="topk",
+                                       return_mean_logits=True)
+        out[b] = o
+        keeps.append(keep)
+        means.append(mean)
+    return out, keeps, means
+
+
+def litesys_decode(q, K, V, topk_block, local, sink=4, block_size=16, sm_scale=None, policy="block",
+                   return_mean_logits=False, keep=None):
     """One sequence of LiteSys' sparse decode on its contiguous cache
     (LiteSys/litesys/attention/batch_cache.py:154-168): logits of every token
-    (cache_utils.py:54-93, scale 1/sqrt(D)), blockwise_topk_sparsity per KV head
-    on the group-mean logits (sparsity_utils.py:24-47), softmax over what stays
+    (cache_utils.py:54-93, scale 1/sqrt(D)), the sparsity policy per KV head on
+    the group-mean logits -- blockwise_topk_sparsity (sparsity_utils.py:24-47,
+    ``policy="block"``) or topk_sparsity (:6-21, ``policy="topk"``, where
+    ``topk_block`` counts tokens) --, softmax over what stays
     (cache_utils.py:216-226), P.V (cache_utils.py:97-169).  q [Hq, D], K / V
     [seq_len, Hkv, D] float (the new token included).  ``topk_block=None`` is the
-    dense layer.  Returns (out [Hq, D] float64, keep [Hkv, seq_len] bool)."""
+    dense layer.  ``keep`` [Hkv, seq_len] overrides the policy's choice (to
+    price a selection that differs from it only by ties).  Returns (out [Hq, D]
+    float64, keep [Hkv, seq_len] bool)."""
     q = np.asarray(q, dtype=np.float64)
     K = np.asarray(K, dtype=np.float64)
     V = np.asarray(V, dtype=np.float64)
@@ -412,13 +461,21 @@ def litesys_decode(q, K, V, topk_block, local, sink=4, block_size=16, sm_scale=N
     scale = 1.0 / np.sqrt(D) if sm_scale is None else sm_scale
     out = np.zeros((Hq, D))
     keep_all = np.ones((Hkv, seq_len), dtype=bool)
+    mean_all = np.zeros((Hkv, seq_len))
     for h in range(Hkv):
         logits = (q[h * G : (h + 1) * G] @ K[:, h, :].T) * scale  # [G, seq_len]
-        if topk_block is not None:
-            keep_all[h] = litesys_blockwise_topk_mask(logits.mean(axis=0), seq_len, topk_block, local, sink, block_size)
+        mean_all[h] = logits.mean(axis=0)
+        if keep is not None:
+            keep_all[h] = keep[h]
+        elif topk_block is not None and policy == "block":
+            keep_all[h] = litesys_blockwise_topk_mask(mean_all[h], seq_len, topk_block, local, sink, block_size)
+        elif topk_block is not None:
+            keep_all[h] = litesys_topk_mask(mean_all[h], seq_len, topk_block, local, sink)
         masked = np.where(keep_all[h][None, :], logits, -np.inf)
         p = np.exp(masked - masked.max(axis=1, keepdims=True))
         out[h * G : (h + 1) * G] = (p / p.sum(axis=1, keepdims=True)) @ V[:, h, :]
+    if return_mean_logits:
+        return out, keep_all, mean_all
     return out, keep_all
 
 

@@ -148,6 +148,27 @@ def test_step_argument_errors(lib):
     assert step(lib, B=0, sink=1, offset=12) == _lib.KIN_OK
 
 
+def test_token_topk_argument_errors(lib):
+    def tok(q=A, topk=8, sink=4, local=1, offset=0, sel=None, cnt=None, ws=A, wsb=1 << 20, B=2, Hq=4, Hkv=1, P=8, mp=4,
+            stride=0):
+        return lib.kin_token_topk_decode(q, A, A, A, A, topk, sink, local, offset, sel, cnt, A, None, ws, wsb, B, Hq, Hkv,
+                                         128, 16, P, mp, stride, 0.0, None)
+
+    assert tok(q=None) == _lib.KIN_ERR_NULL_POINTER
+    assert tok(topk=-1) == _lib.KIN_ERR_BAD_SHAPE
+    assert tok(offset=16) == _lib.KIN_ERR_BAD_SHAPE
+    assert tok(mp=0) == _lib.KIN_ERR_BAD_SHAPE
+    assert tok(topk=5000) == _lib.KIN_ERR_UNSUPPORTED
+    assert tok(local=2000) == _lib.KIN_ERR_UNSUPPORTED
+    assert tok(sel=A, cnt=A, stride=12) == _lib.KIN_ERR_BAD_SHAPE      # 8 + 4 + 1 entries needed
+    assert tok(sel=A, stride=13) == _lib.KIN_ERR_NULL_POINTER
+    assert lib.kin_token_topk_workspace_bytes(2, 1, 4) == 2 * 4 * 16 * 4
+    assert tok(wsb=2 * 4 * 16 * 4 - 1) == _lib.KIN_ERR_WORKSPACE
+    assert tok(ws=None) == _lib.KIN_ERR_WORKSPACE
+    assert tok(P=1 << 28) == _lib.KIN_ERR_UNSUPPORTED                  # token ids would not fit 31 bits
+    assert tok(B=0) == _lib.KIN_OK
+
+
 def test_sel_list_capacity(lib):
     assert lib.kin_sel_list_capacity(128, 0, 1) == 129               # the reference's k + 1
     assert lib.kin_sel_list_capacity(64, 1, 16) == 64 + 1 + 2

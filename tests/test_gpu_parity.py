@@ -724,6 +724,111 @@ def test_ragged_append_bit_exact(ops, hkv):
     assert torch.equal(g1.kv, g2.kv) and torch.equal(g1.kbar, g2.kbar)
 
 
+# --------------------------------------------------------------------------- token-level top-k
+
+
+def _check_token_topk(ops, pb, topk, sink, local, offset, what):
+    g = Gpu(pb)
+    ops.append_paged_kv(g.k, g.v, g.kv, None, g.indices, g.indptr, g.last)
+    stride = topk + sink + local
+    sel = torch.full((pb.B, pb.Hkv, stride), -7, dtype=torch.int32, device=DEV)
+    cnt = torch.full((pb.B, pb.Hkv), -7, dtype=torch.int32, device=DEV)
+    lse = torch.full((pb.B, pb.Hq), float("nan"), dtype=torch.float32, device=DEV)
+    out = ops.token_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, topk, max(pb.max_pages, 1), sink_tokens=sink,
+                                local_tokens=local, first_page_offset=offset, lse=lse, sel_tokens=sel, sel_count=cnt)
+    torch.cuda.synchronize()
+    kv = pb.kv_cache.copy()
+    O.append_paged_kv(pb.k, pb.v, kv, None, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    want, keeps, means = O.token_topk_decode(pb.q, kv, pb.page_indices, pb.page_indptr, pb.last_page_len, topk, sink=sink,
+                                             local=local, first_page_offset=offset)
+    sel, cnt, got = sel.cpu().numpy(), cnt.cpu().numpy(), out.float().cpu().numpy()
+    G = pb.Hq // pb.Hkv
+    qf = O.bf16_to_f32(pb.q).astype(np.float64)
+    for b in range(pb.B):
+        if keeps[b] is None:
+            assert (cnt[b] == 0).all() and (sel[b] == -1).all() and (got[b] == 0).all(), what
+            continue
+        S = keeps[b].shape[1]
+        n_sink = min(sink, S)
+        n_local = min(local, S - n_sink)
+        n_dyn = S - n_sink - n_local
+        k_eff = min(topk, n_dyn)
+        pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+        K = O.bf16_to_f32(kv[pages, 0]).reshape(-1, pb.Hkv, D)[offset : offset + S]
+        V = O.bf16_to_f32(kv[pages, 1]).reshape(-1, pb.Hkv, D)[offset : offset + S]
+        got_keep = np.zeros((pb.Hkv, S), dtype=bool)
+        for h in range(pb.Hkv):
+            n = cnt[b, h]
+            assert n == n_sink + k_eff + n_local, f"{what}: b={b} h={h} count {n}"
+            row = sel[b, h]
+            assert (row[n:] == -1).all(), what
+            assert row[:n_sink].tolist() == list(range(n_sink)), what
+            assert row[n - n_local : n].tolist() == list(range(S - n_local, S)), what
+            mid = row[n_sink : n - n_local]
+            assert np.all(np.diff(mid) > 0), f"{what}: selected tokens are not in ascending order"
+            ok, msg = O.selection_matches(mid - n_sink, means[b][h][n_sink : n_sink + n_dyn], topk)
+            assert ok, f"{what}: b={b} h={h}: {msg}"
+            got_keep[h, row[:n]] = True
+        # the output for the selection the kernel made (identical to the oracle's except for ties)
+        ref, _ = O.litesys_decode(qf[b], K, V, topk, local, sink=sink, policy="topk", keep=got_keep)
+        err = np.abs(got[b] - ref)
+        assert np.all(err <= 2e-2 + 2e-2 * np.abs(ref)), f"{what}: b={b} max err {err.max()}"
+        if np.array_equal(got_keep, keeps[b]):
+            assert np.all(np.abs(got[b] - want[b]) <= 2e-2 + 2e-2 * np.abs(want[b])), what
+    return lse.cpu().numpy()
+
+
+@pytest.mark.parametrize("case", ["mixed", "hkv8", "g8", "many", "offset", "all", "window_only"])
+def test_token_topk_decode(ops, case):
+    """LiteSys' token-level top-k (sparsity_utils.py:6-21): sink tokens, the
+    top-k tokens of the middle by group-mean logit, the local window."""
+    if case == "mixed":
+        pb = P.make_problem(1300, [PS * 40 + 3, PS * 9, 1, 0, PS * 3 + 1, PS * 130 + 16, 17, 5], num_kv_heads=1, group=4)
+        args = (64, 4, 16, 0)
+    elif case == "hkv8":
+        pb = P.make_problem(1301, [PS * 70 + 5, PS * 20 + 16, 0, 5], num_kv_heads=8, group=2, table="fragmented")
+        args = (100, 4, 7, 0)
+    elif case == "g8":
+        pb = P.make_problem(1302, [PS * 300 + 9] * 3, num_kv_heads=1, group=8, table="strided")
+        args = (1024, 4, 64, 0)
+    elif case == "many":     # > 512 lists: 4 waves per list
+        rng = np.random.default_rng(1303)
+        pb = P.make_problem(1303, [int(x) for x in rng.integers(1, PS * 30, size=600)], num_kv_heads=1, group=3)
+        args = (48, 4, 8, 0)
+    elif case == "offset":   # sequences stored 12 slots into their first page
+        pb = P.make_problem(1304, [PS * 25 + 2, PS * 2, 13, 12, 30], num_kv_heads=2, group=4)
+        args = (32, 4, 10, 12)
+    elif case == "all":      # budget covers everything: dense
+        pb = P.make_problem(1305, [PS * 5 + 2, 7], num_kv_heads=1, group=4)
+        args = (4096, 4, 1, 0)
+    else:                    # topk = 0: sink + local window
+        pb = P.make_problem(1306, [PS * 20 + 2, 40], num_kv_heads=2, group=1)
+        args = (0, 4, 33, 0)
+    topk, sink, local, offset = args
+    lse = _check_token_topk(ops, pb, topk, sink, local, offset, f"token top-k {case}")
+    assert not np.isnan(lse).any()
+    if case == "all":
+        kv = pb.kv_cache.copy()
+        O.append_paged_kv(pb.k, pb.v, kv, None, pb.page_indices, pb.page_indptr, pb.last_page_len)
+        _, want_lse = O.dense_paged_decode(pb.q, kv, pb.page_indices, pb.page_indptr, pb.last_page_len)
+        assert np.allclose(lse, want_lse, rtol=1e-4, atol=1e-4)
+
+
+def test_token_topk_rejects_short_workspace_and_long_sequences(ops):
+    pb = P.make_problem(1310, [PS * 6 + 2, PS * 2], num_kv_heads=1, group=4)
+    g = Gpu(pb)
+    with pytest.raises(Exception, match="KIN_ERR_WORKSPACE"):
+        ops.token_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, 8, pb.max_pages,
+                              workspace=torch.empty(64, dtype=torch.uint8, device=DEV))
+    # a sequence with more pages than the scratch array was sized for is skipped and flagged
+    sel = torch.zeros(pb.B, 1, 8 + 4 + 1, dtype=torch.int32, device=DEV)
+    cnt = torch.zeros(pb.B, 1, dtype=torch.int32, device=DEV)
+    out = ops.token_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, 8, 3, sel_tokens=sel, sel_count=cnt)
+    torch.cuda.synchronize()
+    assert cnt.cpu().numpy().reshape(-1).tolist() == [-1, 4 + 8 + 1]
+    assert (out[0] == 0).all()
+
+
 # --------------------------------------------------------------------------- graph capture / tracing
 
 

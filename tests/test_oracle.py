@@ -523,3 +523,54 @@ def test_page_lists_with_offset_12_equal_litesys_mask_formulation():
         dense, _ = O.dense_paged_decode(q, kv, perm, indptr, last, first_page_offset=pad)
         want_dense, _ = O.litesys_decode(O.bf16_to_f32(q[0]), K, V, None, local)
         assert np.allclose(dense[0], want_dense, rtol=1e-9, atol=1e-11)
+
+
+def test_litesys_token_topk_mask():
+    """sparsity_utils.py:6-21 by hand and against torch.topk."""
+    seq_len, local, sink, topk = 30, 3, 4, 5
+    ml = np.zeros(seq_len)
+    ml[[6, 9, 10, 20, 26]] = [5.0, 4.0, 3.0, 2.0, 1.0]
+    ml[[1, 28]] = 100.0                      # sink / local tokens are not candidates
+    keep = O.litesys_topk_mask(ml, seq_len, topk, local, sink)
+    want = np.zeros(seq_len, dtype=bool)
+    want[:4] = True
+    want[27:] = True
+    want[[6, 9, 10, 20, 26]] = True
+    assert np.array_equal(keep, want)
+    assert O.litesys_topk_mask(ml, 12, topk, local, sink).all()        # seq_len <= sink + topk + local: dense
+    assert O.litesys_topk_mask(ml[:13], 13, topk, local, sink).sum() == 12
+    rng = np.random.default_rng(3)
+    for seq_len, topk, local in [(500, 64, 16), (77, 10, 1), (4096, 1024, 64)]:
+        ml = rng.standard_normal(seq_len)
+        keep = O.litesys_topk_mask(ml, seq_len, topk, local)
+        idx = torch.topk(torch.from_numpy(ml[4 : seq_len - local]), topk).indices.numpy() + 4
+        want = np.zeros(seq_len, dtype=bool)
+        want[:4] = True
+        want[seq_len - local :] = True
+        want[idx] = True
+        assert np.array_equal(keep, want)
+
+
+def test_token_topk_decode_on_pages_is_litesys_on_the_contiguous_cache():
+    """The paged wrapper only de-pages; with a budget that covers everything the
+    result is dense attention; with first_page_offset the padding slots vanish."""
+    pb = P.make_problem(88, [PS * 12 + 5, 9, PS * 3], num_kv_heads=2, group=2)
+    O.append_paged_kv(pb.k, pb.v, pb.kv_cache, None, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    out, keeps, means = O.token_topk_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len, 10 ** 6)
+    dense, _ = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    assert np.allclose(out, dense, rtol=1e-10, atol=1e-12) and all(k.all() for k in keeps)
+    out, keeps, means = O.token_topk_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len, 20,
+                                            sink=4, local=8)
+    assert keeps[0].sum(axis=1).tolist() == [32, 32] and keeps[1].all()
+    K, V = _depaged(pb, 0, 1)
+    q = O.bf16_to_f32(pb.q[0, 2:4]).astype(np.float64)
+    logits = q @ K.T / math.sqrt(D)
+    assert np.allclose(means[0][1], logits.mean(axis=0), rtol=1e-12)
+    logits[:, ~keeps[0][1]] = -np.inf
+    w = np.exp(logits - logits.max(axis=1, keepdims=True))
+    assert np.allclose(out[0, 2:4], (w / w.sum(axis=1, keepdims=True)) @ V, rtol=1e-10, atol=1e-12)
+    off, _, _ = O.token_topk_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len, 10 ** 6,
+                                    first_page_offset=7)
+    dense_off, _ = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len,
+                                        first_page_offset=7)
+    assert np.allclose(off, dense_off, rtol=1e-10, atol=1e-12)
