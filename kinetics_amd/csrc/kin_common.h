@@ -15,6 +15,13 @@ constexpr int kMaxGroup = 8;     // largest supported num_q_heads / num_kv_heads
 constexpr int kMaxTopk = 2048;
 constexpr int kMaxCandidates = 16384;
 constexpr int kNumCus = 256;     // compute units of the target GPU (MI355X)
+constexpr int kNumXcds = 8;      // accelerator dies, each with its own L2
+
+// Workgroups to launch for one list per (sequence, KV head) under xcd_list_of().
+inline int64_t xcd_grid_size(int batch, int num_kv_heads) {
+  if (num_kv_heads == 1) return batch;
+  return ((int64_t)batch + kNumXcds - 1) / kNumXcds * kNumXcds * num_kv_heads;
+}
 constexpr int kMaxFixedPages = 64;  // most sink / local pages that can be pinned into every list
 constexpr int kMaxLocalTokens = (kMaxFixedPages - 1) * kPageSize + 1;
 
@@ -46,6 +53,25 @@ int check_first_page_offset(const char* fn, int first_page_offset);
 
 // ---- device side -----------------------------------------------------------
 #if defined(__HIPCC__)
+
+// Workgroups are handed to the GPU's 8 XCDs round-robin by index; every XCD has
+// its own L2 and address-translation caches.  The lists of one sequence's KV
+// heads read different parts of the same KV pages and the same page-table
+// entries, so they go to workgroups of ONE XCD: with t = bid / 8 and x = bid % 8,
+// workgroup bid handles head t % hkv of sequence (t / hkv) * 8 + x.  The grid
+// is xcd_grid_size(batch, hkv) workgroups; false marks a padding workgroup.
+__device__ __forceinline__ bool xcd_list_of(int bid, int batch, int hkv, int& b, int& h) {
+  if (hkv == 1) {
+    b = bid;
+    h = 0;
+    return true;
+  }
+  const int t = bid / kNumXcds, x = bid - t * kNumXcds;
+  const int tb = t / hkv;
+  h = t - tb * hkv;
+  b = tb * kNumXcds + x;
+  return b < batch;
+}
 
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }

@@ -18,7 +18,7 @@ struct DecodeParams {
   float* lse;     // may be null
   float* ws_o;    // [batch*Hq, splits, 128] fp32, splits > 1 only
   float* ws_lse;  // [batch*Hq, splits]      fp32 (log2 domain)
-  int num_q_heads, num_kv_heads, group;
+  int batch, num_q_heads, num_kv_heads, group;
   int list_stride, num_splits;
   int first_page_offset;  // padding slots at the start of list entry 0
   int64_t num_pages;
@@ -31,8 +31,10 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
   __shared__ float sm_m[4][4 * NG];
   __shared__ float sm_l[4][4 * NG];
 
-  const int list = blockIdx.x, split = blockIdx.y;
-  const int b = list / p.num_kv_heads, h = list - b * p.num_kv_heads;
+  const int split = blockIdx.y;
+  int b, h;
+  if (!xcd_list_of(blockIdx.x, p.batch, p.num_kv_heads, b, h)) return;
+  const int list = b * p.num_kv_heads + h;
   const int G = p.group;
 
   const int32_t* __restrict__ pl;
@@ -141,8 +143,9 @@ static int launch_decode(const char* fn, DecodeParams& p, int batch, void* works
     p.ws_o = nullptr;
     p.ws_lse = nullptr;
   }
-  const int64_t lists = (int64_t)batch * p.num_kv_heads;
+  const int64_t lists = xcd_grid_size(batch, p.num_kv_heads);
   if (lists > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
+  p.batch = batch;
   dim3 grid((unsigned)lists, (unsigned)splits);
   if (p.group <= 4)
     paged_decode_kernel<1><<<grid, 256, 0, stream>>>(p);

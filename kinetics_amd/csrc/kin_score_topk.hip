@@ -15,7 +15,7 @@ struct ScoreTopkParams {
   int32_t* sel_count;
   int32_t* sel_logical;  // may be null
   float* scores_out;     // may be null
-  int num_q_heads, num_kv_heads, group;
+  int batch, num_q_heads, num_kv_heads, group;
   int kbar_pages, sel_stride, topk, sink_pages, local_tokens;
   int sort_cap;
 };
@@ -25,8 +25,9 @@ template <int UNROLL>
 __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x;
-  const int item = blockIdx.x;
-  const int b = item / p.num_kv_heads, h = item - b * p.num_kv_heads;
+  int b, h;
+  if (!xcd_list_of(blockIdx.x, p.batch, p.num_kv_heads, b, h)) return;
+  const int item = b * p.num_kv_heads + h;
 
   const int ps = p.page_indptr[b], pe = p.page_indptr[b + 1];
   const int n_pages = pe - ps;
@@ -99,6 +100,7 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
   p.sel_count = sel_count;
   p.sel_logical = sel_logical;
   p.scores_out = scores_out;
+  p.batch = batch;
   p.num_q_heads = num_q_heads;
   p.num_kv_heads = num_kv_heads;
   p.group = num_q_heads / num_kv_heads;
@@ -110,7 +112,8 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
   p.sort_cap = select_sort_cap(topk, kbar_pages);
   const size_t lds = select_lds_bytes(kbar_pages, p.sort_cap) + (size_t)list_cap * 4;
   const int64_t items = (int64_t)batch * num_kv_heads;
-  if (items > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
+  if (xcd_grid_size(batch, num_kv_heads) > 0x7fffffffLL)
+    return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   // Few workgroups cannot saturate HBM with 4 loads per lane in flight: give a
   // small grid 16 (more registers, which it can afford).
   const bool small_grid = items < 512;
@@ -123,8 +126,8 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
     if (st) return st;
   }
   if (small_grid)
-    score_topk_kernel<16><<<(unsigned)items, kThreads, lds, static_cast<hipStream_t>(stream)>>>(p);
+    score_topk_kernel<16><<<(unsigned)xcd_grid_size(batch, num_kv_heads), kThreads, lds, static_cast<hipStream_t>(stream)>>>(p);
   else
-    score_topk_kernel<4><<<(unsigned)items, kThreads, lds, static_cast<hipStream_t>(stream)>>>(p);
+    score_topk_kernel<4><<<(unsigned)xcd_grid_size(batch, num_kv_heads), kThreads, lds, static_cast<hipStream_t>(stream)>>>(p);
   return check_hip(hipGetLastError(), "score_topk_kernel launch");
 }

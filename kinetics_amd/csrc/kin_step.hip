@@ -28,7 +28,7 @@ struct StepParams {
   int32_t* sel_count;  // optional
   uint16_t* out;
   float* lse;  // optional
-  int num_q_heads, num_kv_heads, group;
+  int batch, num_q_heads, num_kv_heads, group;
   int kbar_pages, sel_stride, topk, sink_pages, local_tokens, first_page_offset, sort_cap;
   int region0_bytes;  // LDS: max(attend staging, select scratch); the page list follows it
   int64_t num_pages;
@@ -43,8 +43,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   constexpr int NT = NW * 64;
 
   const int tid = threadIdx.x;
-  const int item = blockIdx.x;
-  const int b = item / p.num_kv_heads, h = item - b * p.num_kv_heads;
+  int b, h;
+  if (!xcd_list_of(blockIdx.x, p.batch, p.num_kv_heads, b, h)) return;
+  const int item = b * p.num_kv_heads + h;
   const int G = p.group;
   const int64_t hq0 = (int64_t)b * p.num_q_heads + (int64_t)h * G;
 
@@ -194,6 +195,7 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
   p.sel_count = sel_count;
   p.out = out;
   p.lse = lse;
+  p.batch = batch;
   p.num_q_heads = num_q_heads;
   p.num_kv_heads = num_kv_heads;
   p.group = num_q_heads / num_kv_heads;
@@ -207,7 +209,8 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
   // Waves per workgroup: aim for 16 waves per CU (8 with the two-pass kernel for
   // groups above 4, whose registers allow no more) when the lists are few.
   const int64_t items = (int64_t)batch * num_kv_heads;
-  if (items > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
+  if (xcd_grid_size(batch, num_kv_heads) > 0x7fffffffLL)
+    return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   int nw = 4;
   if (p.group <= 4)
     nw = items <= kNumCus ? 16 : (items <= 2 * kNumCus ? 8 : 4);
@@ -237,7 +240,7 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
     if (st) return st;
   }
   void* args[] = {&p};
-  st = check_hip(hipLaunchKernel(kernel, dim3((unsigned)items), dim3(nw * 64), args, lds, s),
+  st = check_hip(hipLaunchKernel(kernel, dim3((unsigned)xcd_grid_size(batch, num_kv_heads)), dim3(nw * 64), args, lds, s),
                  "blocktopk_step_kernel launch");
   return st;
 }

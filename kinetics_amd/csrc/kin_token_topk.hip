@@ -17,7 +17,7 @@ struct TokenTopkParams {
   uint16_t* out;
   float* lse;           // optional
   uint32_t* keys;       // workspace: [lists, max_pages_per_seq * 16]
-  int num_q_heads, num_kv_heads, group;
+  int batch, num_q_heads, num_kv_heads, group;
   int topk, sink_tokens, local_tokens, first_page_offset;
   int max_pages_per_seq, sel_stride;
   int64_t num_pages;
@@ -33,8 +33,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
   constexpr int NT = NW * 64;
 
   const int tid = threadIdx.x;
-  const int item = blockIdx.x;
-  const int b = item / p.num_kv_heads, h = item - b * p.num_kv_heads;
+  int b, h;
+  if (!xcd_list_of(blockIdx.x, p.batch, p.num_kv_heads, b, h)) return;
+  const int item = b * p.num_kv_heads + h;
   const int G = p.group;
   const int64_t hq0 = (int64_t)b * p.num_q_heads + (int64_t)h * G;
 
@@ -159,6 +160,7 @@ int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const
   p.out = out;
   p.lse = lse;
   p.keys = static_cast<uint32_t*>(workspace);
+  p.batch = batch;
   p.num_q_heads = num_q_heads;
   p.num_kv_heads = num_kv_heads;
   p.group = num_q_heads / num_kv_heads;
@@ -173,7 +175,8 @@ int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const
   p.scale_log2 = scale * 1.4426950408889634f;
 
   const int64_t items = (int64_t)batch * num_kv_heads;
-  if (items > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
+  if (xcd_grid_size(batch, num_kv_heads) > 0x7fffffffLL)
+    return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   // Waves per workgroup: 8 when the lists are too few to fill the GPU with 4-wave
   // workgroups (the per-token addressing needs ~140 registers, so 16 do not fit).
   const int nw = items <= 2 * kNumCus ? 8 : 4;
@@ -191,7 +194,7 @@ int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const
     if (st) return st;
   }
   void* args[] = {&p};
-  return check_hip(hipLaunchKernel(kernel, dim3((unsigned)items), dim3(nw * 64), args, lds,
+  return check_hip(hipLaunchKernel(kernel, dim3((unsigned)xcd_grid_size(batch, num_kv_heads)), dim3(nw * 64), args, lds,
                                    static_cast<hipStream_t>(stream)),
                    "token_topk_kernel launch");
 }
