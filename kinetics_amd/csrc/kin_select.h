@@ -105,31 +105,20 @@ __device__ __forceinline__ void radix_pick_bin(const uint32_t* hist, uint32_t re
   }
 }
 
-// Writes the page list to sel_lds (LDS, >= n_sink + topk + n_local entries):
-// the sink pages, then the ordered physical ids of the k_eff winners, then the
-// local pages (the open page last).  Returns the list length.  Ends with a
-// workgroup barrier: sel_lds is visible to every thread and keys / sortbuf are
-// free for reuse.
+// Scores the candidates r0 <= r < r1 of one (sequence, KV head) with the
+// group-mean query and stores them as order-preserving keys in keys_out[r] (LDS
+// or global memory) and, if a.scores_out is set, as fp32 in scores_out[r].
+// Streams (r1 - r0) * 256 B; no barrier inside.
 // NT: threads of the workgroup (a multiple of 256, all of them call this).
 // UNROLL: independent 16-byte loads each lane keeps in flight while streaming the
 // mean keys (4 saturates HBM when thousands of workgroups run; a small grid
 // needs more per workgroup).
-template <int UNROLL = 4, int NT = kThreads>
-__device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_lds) {
+template <int UNROLL, int NT>
+__device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, uint32_t* keys_out) {
   constexpr int kUnroll = UNROLL;
   constexpr int kRows = NT / 16;  // mean keys one pass of the workgroup covers
-  __shared__ uint32_t hist[256];
-  __shared__ uint32_t wave_tot[NT / 64];
-  __shared__ uint32_t sh_bin, sh_remaining, sh_count;
-
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int n_cand = a.n_cand, n_pages = a.n_pages;
-  const int k_eff = min(a.topk, n_cand);
-  uint32_t* keys = a.keys;
-  unsigned long long* sortbuf = a.sortbuf;
-
-  // ---- phase 1: scores --------------------------------------------------
+  const int lane = tid & 63;
   // Lane owns columns d = 8*(lane%16) .. +7 of the mean query.
   const int c16 = lane & 15;
   float qm[8];
@@ -149,24 +138,23 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
     for (int u = 0; u < 8; ++u) qm[u] *= inv;
   }
   // The candidates of (b, h) are rows of 256 B at a fixed stride.  They are read
-  // through a buffer descriptor that ends after the last candidate, so loads past
+  // through a buffer descriptor that ends after the last wanted row, so loads past
   // the end return zeros without touching memory and the loop needs no branches:
   // each lane keeps kUnroll 16-byte loads in flight, re-issuing slot j for the
   // next pass as soon as it has consumed it.
   const int row_stride_b = a.row_stride_b;  // bytes between logical pages
-  const char* kb = a.kb;
+  const int n = r1 > r0 ? r1 - r0 : 0;
+  const char* kb = a.kb + (int64_t)r0 * row_stride_b;
   float* sc_out = a.scores_out;
-  // Nothing to choose (topk == 0) and nobody asked for the scores: stream nothing.
-  const int n_score = (k_eff > 0 || sc_out) ? n_cand : 0;
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<char*>(kb), 0, n_score > 0 ? (n_score - 1) * row_stride_b + kRowBytes : 0, 0x00020000);
+      const_cast<char*>(kb), 0, n > 0 ? (n - 1) * row_stride_b + kRowBytes : 0, 0x00020000);
   const int sub = tid >> 4;  // which of the kRows rows of a slot this lane helps with
   const int lane_off = sub * row_stride_b + c16 * 16;
   u32x4 w[kUnroll];
 #pragma unroll
   for (int j = 0; j < kUnroll; ++j)
     w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + j * kRows * row_stride_b, 0, kStreamLoad);
-  for (int base = 0; base < n_score; base += kRows * kUnroll) {
+  for (int base = 0; base < n; base += kRows * kUnroll) {
     const int next_off = (base + kRows * kUnroll) * row_stride_b;
 #pragma unroll
     for (int j = 0; j < kUnroll; ++j) {
@@ -179,13 +167,32 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
       acc = fmaf(qm[6], bf16_lo(x.w), acc); acc = fmaf(qm[7], bf16_hi(x.w), acc);
       acc = row16_sum(acc);
       const int row = base + j * kRows + sub;
-      if (c16 == 0 && row < n_score) {
-        keys[row] = order_key(acc);
-        if (sc_out) sc_out[row] = acc;
+      if (c16 == 0 && row < n) {
+        keys_out[r0 + row] = order_key(acc);
+        if (sc_out) sc_out[r0 + row] = acc;
       }
     }
   }
-  __syncthreads();
+}
+
+// Selects from the keys of the n_cand candidates in a.keys (LDS) and writes the
+// page list to sel_lds (LDS, >= n_sink + topk + n_local entries): the sink
+// pages, then the ordered physical ids of the k_eff winners, then the local
+// pages (the open page last).  Returns the list length.  The caller has put a
+// workgroup barrier between the last key write and this call; it ends with one:
+// sel_lds is visible to every thread and keys / sortbuf are free for reuse.
+template <int NT>
+__device__ __forceinline__ int select_from_keys(const SelectArgs& a, int32_t* sel_lds) {
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t wave_tot[NT / 64];
+  __shared__ uint32_t sh_bin, sh_remaining, sh_count;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n_cand = a.n_cand, n_pages = a.n_pages;
+  const int k_eff = min(a.topk, n_cand);
+  uint32_t* keys = a.keys;
+  unsigned long long* sortbuf = a.sortbuf;
 
   // ---- phase 2: radix select of the k_eff-th largest key -------------------
   uint32_t prefix = 0, mask = 0;
@@ -302,6 +309,16 @@ __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_ld
   }
   __syncthreads();
   return k_eff + a.n_sink + a.n_local;
+}
+
+// score_rows() over every candidate into a.keys, then select_from_keys().
+template <int UNROLL = 4, int NT = kThreads>
+__device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_lds) {
+  // Nothing to choose (topk == 0) and nobody asked for the scores: stream nothing.
+  const int n_score = (min(a.topk, a.n_cand) > 0 || a.scores_out) ? a.n_cand : 0;
+  score_rows<UNROLL, NT>(a, 0, n_score, a.keys);
+  __syncthreads();
+  return select_from_keys<NT>(a, sel_lds);
 }
 
 }  // namespace kin
