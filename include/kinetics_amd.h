@@ -266,7 +266,7 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  * list (no split-K); with few lists it runs 8 or 16 waves instead of 4, which
  * changes the fp32 summation order of the output (not the page lists or cache
  * bytes).  Faster than the three calls except for few (< 256) and very long
- * (topk > 512) lists.
+ * (topk > 512) lists.  workspace: optional, see kin_step_workspace_bytes.
  */
 int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
                               kin_bf16_t* kv_cache, kin_bf16_t* kbar,
@@ -278,7 +278,19 @@ int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const ki
                               int batch, int num_q_heads, int num_kv_heads,
                               int head_dim, int page_size, int64_t num_pages,
                               int kbar_pages, int sel_stride, int first_page_offset,
-                              float sm_scale, kin_stream_t stream);
+                              float sm_scale, void* workspace, size_t workspace_bytes,
+                              kin_stream_t stream);
+
+/*
+ * Workspace kin_blocktopk_decode_step can use for the given problem: 0 unless
+ * the lists are few (batch * num_kv_heads <= 64) and long (kbar_pages >= 2048),
+ * where the step spreads the scoring of each list over several workgroups that
+ * meet through this memory (4 bytes per candidate page and an arrival counter
+ * per list; contents need no initialisation and are of no use afterwards).
+ * Passing NULL or too little is allowed: the step then scores each list with a
+ * single workgroup, as it does for every other shape.
+ */
+size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages);
 
 /*
  * Token-level top-k sparse decode attention in one launch -- LiteSys'

@@ -123,6 +123,7 @@ class PagedBatchKVManager:
         ws = max(ops.decode_workspace_bytes(B, Hq, Hkv, P), ops.decode_workspace_bytes(B, Hq, Hkv, self._sel.shape[2]), 16)
         if self.token_topk is not None:
             ws = max(ws, ops.token_topk_workspace_bytes(B, Hkv, P))
+        ws = max(ws, ops.step_workspace_bytes(B, Hkv, P))
         self._ws = torch.empty(ws, dtype=torch.uint8, device=dev)
 
     # ------------------------------------------------------------------ LiteSys interface
@@ -164,7 +165,7 @@ class PagedBatchKVManager:
         elif sparse and self._fused:
             ops.blocktopk_decode_step(self._q, self._k, self._v, kv, kbar, self.page_indices, self.page_indptr,
                                       self.last_page_len, self.block_topk, out=self._out, sink_pages=self.sink_pages,
-                                      local_tokens=self.local_tokens, first_page_offset=self.pad)
+                                      local_tokens=self.local_tokens, first_page_offset=self.pad, workspace=self._ws)
         else:
             ops.append_paged_kv(self._k, self._v, kv, kbar, self.page_indices, self.page_indptr, self.last_page_len)
             if sparse:

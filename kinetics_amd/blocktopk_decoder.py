@@ -81,6 +81,9 @@ class BlockTopkPagedAttention:
         self.fused = ops.prefer_fused_step(B, num_kv_heads, n + 1, topk_page) if fused is None else bool(fused)
         ws = ops.decode_workspace_bytes(B, num_heads, num_kv_heads, self.list_capacity)
         self.workspace: Optional[torch.Tensor] = torch.empty(ws, dtype=torch.uint8, device=dev) if ws else None
+        # few, long sequences: the fused step spreads each list's scoring over several workgroups through this
+        sws = ops.step_workspace_bytes(B, num_kv_heads, max_num_pages)
+        self.step_workspace: Optional[torch.Tensor] = torch.empty(sws, dtype=torch.uint8, device=dev) if sws else None
 
     # -- the three stages, each a custom op --------------------------------
     def refresh_compressed_keys(self) -> None:
@@ -110,7 +113,8 @@ class BlockTopkPagedAttention:
             return torch.ops.kinetics.blocktopk_decode_step(
                 query_states, key_states, value_states, self.kv_cache, self.compressed_key_cache,
                 self.paged_kv_indices, self.paged_kv_indptr, self.last_kv_lens, self.topk_page,
-                self.topk_page_indices, self.topk_page_count, self.sm_scale, self.sink_pages, self.local_tokens)
+                self.topk_page_indices, self.topk_page_count, self.sm_scale, self.sink_pages, self.local_tokens, 0,
+                self.step_workspace)
         self.update_kv(key_states, value_states)
         self.select_pages(query_states)
         return self.decode(query_states)

@@ -108,12 +108,14 @@ __device__ __forceinline__ void radix_pick_bin(const uint32_t* hist, uint32_t re
 // Scores the candidates r0 <= r < r1 of one (sequence, KV head) with the
 // group-mean query and stores them as order-preserving keys in keys_out[r] (LDS
 // or global memory) and, if a.scores_out is set, as fp32 in scores_out[r].
-// Streams (r1 - r0) * 256 B; no barrier inside.
+// Streams (r1 - r0) * 256 B; no barrier inside.  DEVICE_VISIBLE: keys_out is global
+// memory that a workgroup on another XCD will read in this launch: the stores
+// are made at device scope (past this XCD's L2).
 // NT: threads of the workgroup (a multiple of 256, all of them call this).
 // UNROLL: independent 16-byte loads each lane keeps in flight while streaming the
 // mean keys (4 saturates HBM when thousands of workgroups run; a small grid
 // needs more per workgroup).
-template <int UNROLL, int NT>
+template <int UNROLL, int NT, bool DEVICE_VISIBLE = false>
 __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, uint32_t* keys_out) {
   constexpr int kUnroll = UNROLL;
   constexpr int kRows = NT / 16;  // mean keys one pass of the workgroup covers
@@ -168,7 +170,10 @@ __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, 
       acc = row16_sum(acc);
       const int row = base + j * kRows + sub;
       if (c16 == 0 && row < n) {
-        keys_out[r0 + row] = order_key(acc);
+        if (DEVICE_VISIBLE)
+          __hip_atomic_store(keys_out + r0 + row, order_key(acc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else
+          keys_out[r0 + row] = order_key(acc);
         if (sc_out) sc_out[r0 + row] = acc;
       }
     }

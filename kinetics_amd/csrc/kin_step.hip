@@ -31,6 +31,11 @@ struct StepParams {
   int batch, num_q_heads, num_kv_heads, group;
   int kbar_pages, sel_stride, topk, sink_pages, local_tokens, first_page_offset, sort_cap;
   int region0_bytes;  // LDS: max(attend staging, select scratch); the page list follows it
+  // Split scoring (few, long sequences): `chunks` workgroups per list score a slice of the
+  // candidates each into ws_keys; the last one to finish selects and attends.
+  int chunks;
+  int32_t* ws_count;   // [lists], zero at launch and left zero
+  uint32_t* ws_keys;   // [lists, kbar_pages]
   int64_t num_pages;
   float scale_log2;
 };
@@ -42,9 +47,17 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   __shared__ float sm_l[NW][4 * NG];
   constexpr int NT = NW * 64;
 
+  __shared__ int sh_last;
   const int tid = threadIdx.x;
-  int b, h;
-  if (!xcd_list_of(blockIdx.x, p.batch, p.num_kv_heads, b, h)) return;
+  int b, h, chunk = 0;
+  if (p.chunks > 1) {
+    const int list = blockIdx.x / p.chunks;
+    chunk = blockIdx.x - list * p.chunks;
+    b = list / p.num_kv_heads;
+    h = list - b * p.num_kv_heads;
+  } else if (!xcd_list_of(blockIdx.x, p.batch, p.num_kv_heads, b, h)) {
+    return;
+  }
   const int item = b * p.num_kv_heads + h;
   const int G = p.group;
   const int64_t hq0 = (int64_t)b * p.num_q_heads + (int64_t)h * G;
@@ -52,6 +65,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   const int ps = p.page_indptr[b], pe = p.page_indptr[b + 1];
   const int n_pages = pe - ps;
   if (n_pages <= 0) {  // empty sequence: nothing to append, select or attend
+    if (chunk != 0) return;
     if (p.sel_pages)
       for (int i = tid; i < p.sel_stride; i += NT) p.sel_pages[(int64_t)item * p.sel_stride + i] = -1;
     if (p.sel_count && tid == 0) p.sel_count[item] = 0;
@@ -63,37 +77,42 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   const int row_dw = p.num_kv_heads * (kHeadDim / 2);  // dwords per token row
 
   // ---- append (wave 0): same byte moves and mean-key update as append_kernel ----
-  if (p.k != nullptr && tid < 64) {
-    const int lane = tid;
-    const int pos = last_len - 1;
-    const int64_t pid = p.page_indices[pe - 1];
-    if (pos >= 0 && pos < kPageSize && pid >= 0 && pid < p.num_pages) {
-      uint32_t* kplane = reinterpret_cast<uint32_t*>(p.kv) + pid * (2LL * kPageSize * row_dw) + h * (kHeadDim / 2);
-      uint32_t* vplane = kplane + (int64_t)kPageSize * row_dw;
-      const int64_t src = (int64_t)item * (kHeadDim / 2) + lane;
-      const uint32_t kw = p.k[src], vw = p.v[src];
-      kplane[(int64_t)pos * row_dw + lane] = kw;
-      vplane[(int64_t)pos * row_dw + lane] = vw;
-      if (p.kbar != nullptr && pos == kPageSize - 1 && n_pages - 1 < p.kbar_pages) {
-        float s0 = 0.f, s1 = 0.f;
+  // With split scoring the workgroup that ends up attending does it (see below).
+  auto append_token = [&]() {
+    if (p.k != nullptr && tid < 64) {
+      const int lane = tid;
+      const int pos = last_len - 1;
+      const int64_t pid = p.page_indices[pe - 1];
+      if (pos >= 0 && pos < kPageSize && pid >= 0 && pid < p.num_pages) {
+        uint32_t* kplane = reinterpret_cast<uint32_t*>(p.kv) + pid * (2LL * kPageSize * row_dw) + h * (kHeadDim / 2);
+        uint32_t* vplane = kplane + (int64_t)kPageSize * row_dw;
+        const int64_t src = (int64_t)item * (kHeadDim / 2) + lane;
+        const uint32_t kw = p.k[src], vw = p.v[src];
+        kplane[(int64_t)pos * row_dw + lane] = kw;
+        vplane[(int64_t)pos * row_dw + lane] = vw;
+        if (p.kbar != nullptr && pos == kPageSize - 1 && n_pages - 1 < p.kbar_pages) {
+          float s0 = 0.f, s1 = 0.f;
 #pragma unroll
-        for (int t = 0; t < kPageSize - 1; ++t) {
-          const uint32_t w = kplane[(int64_t)t * row_dw + lane];
-          s0 += bf16_lo(w);
-          s1 += bf16_hi(w);
+          for (int t = 0; t < kPageSize - 1; ++t) {
+            const uint32_t w = kplane[(int64_t)t * row_dw + lane];
+            s0 += bf16_lo(w);
+            s1 += bf16_hi(w);
+          }
+          s0 += bf16_lo(kw);
+          s1 += bf16_hi(kw);
+          const float inv = 1.0f / kPageSize;
+          reinterpret_cast<uint32_t*>(p.kbar)[(((int64_t)b * p.kbar_pages + (n_pages - 1)) * p.num_kv_heads + h) *
+                                                  (kHeadDim / 2) +
+                                              lane] = f32_to_bf16(s0 * inv) | (f32_to_bf16(s1 * inv) << 16);
         }
-        s0 += bf16_lo(kw);
-        s1 += bf16_hi(kw);
-        const float inv = 1.0f / kPageSize;
-        reinterpret_cast<uint32_t*>(p.kbar)[(((int64_t)b * p.kbar_pages + (n_pages - 1)) * p.num_kv_heads + h) *
-                                                (kHeadDim / 2) +
-                                            lane] = f32_to_bf16(s0 * inv) | (f32_to_bf16(s1 * inv) << 16);
       }
+      // The attention phase of this workgroup reads the row back: make the stores
+      // visible before the barriers that separate the phases.
+      __threadfence_block();
     }
-    // The attention phase of this workgroup reads the row back: make the stores
-    // visible before the barriers that separate the phases.
-    __threadfence_block();
-  }
+
+  };
+  if (p.chunks <= 1) append_token();
 
   // ---- score + select: page list into LDS -------------------------------------
   int32_t* sel_lds = reinterpret_cast<int32_t*>(smem + p.region0_bytes);
@@ -112,7 +131,35 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   s.keys = reinterpret_cast<uint32_t*>(smem);
   s.sortbuf = reinterpret_cast<unsigned long long*>(smem + (size_t)((p.kbar_pages + 3) & ~3) * 4);
   s.sort_cap = p.sort_cap;
-  const int n = score_select<4, NT>(s, sel_lds);
+  int n;
+  if (p.chunks > 1) {
+    // This workgroup's slice of the candidates -> keys in HBM.
+    uint32_t* gkeys = p.ws_keys + (int64_t)item * p.kbar_pages;
+    const int n_score = min(s.topk, s.n_cand) > 0 ? s.n_cand : 0;
+    const int per = ((n_score + p.chunks - 1) / p.chunks + 63) & ~63;
+    const int r0 = min(chunk * per, n_score), r1 = min(r0 + per, n_score);
+    score_rows<4, NT, true>(s, r0, r1, gkeys);
+    // The slices meet through memory without cache maintenance: keys and the
+    // arrival counter are written and read at device scope (they bypass the
+    // XCD-private L2), and every wave waits for its own stores to be acknowledged
+    // before the workgroup counts in.  Whoever counts in last sees everybody's
+    // keys and carries on alone; the others are done.
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0)
+      sh_last = (__hip_atomic_fetch_add(&p.ws_count[item], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.chunks - 1)
+                    ? 1 : 0;
+    __syncthreads();
+    if (!sh_last) return;
+    if (tid == 0) __hip_atomic_store(&p.ws_count[item], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+    append_token();
+    for (int i = tid; i < n_score; i += NT)
+      s.keys[i] = __hip_atomic_load(gkeys + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    n = select_from_keys<NT>(s, sel_lds);
+  } else {
+    n = score_select<4, NT>(s, sel_lds);
+  }
   if (p.sel_pages) {
     int32_t* sel = p.sel_pages + (int64_t)item * p.sel_stride;
     for (int i = tid; i < p.sel_stride; i += NT) sel[i] = (i < n) ? sel_lds[i] : -1;
@@ -142,7 +189,32 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
       });
 }
 
+__global__ void fill_zero_kernel(int32_t* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// Workgroups per list for the scoring phase: 1 unless the lists are few (at most a
+// quarter of the CUs) and long, then enough to put a workgroup on every CU, each
+// with at least 256 candidates.
+static int step_score_chunks(int batch, int num_kv_heads, int kbar_pages) {
+  const int64_t items = (int64_t)batch * num_kv_heads;
+  if (items <= 0 || items * 4 > kNumCus || kbar_pages < 2048) return 1;
+  int64_t c = kNumCus / items;
+  const int64_t by_rows = kbar_pages / 256;
+  if (c > by_rows) c = by_rows;
+  return c < 2 ? 1 : (int)c;
+}
+
+static size_t step_count_bytes(int64_t items) { return ((size_t)items * sizeof(int32_t) + 255) & ~(size_t)255; }
+
 }  // namespace kin
+
+extern "C" size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages) {
+  if (kin::step_score_chunks(batch, num_kv_heads, kbar_pages) <= 1) return 0;
+  const int64_t items = (int64_t)batch * num_kv_heads;
+  return kin::step_count_bytes(items) + (size_t)items * kbar_pages * sizeof(uint32_t);
+}
 
 extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
                                          kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
@@ -150,7 +222,8 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
                                          int sink_pages, int local_tokens, int32_t* sel_pages, int32_t* sel_count,
                                          kin_bf16_t* out, float* lse, int batch, int num_q_heads, int num_kv_heads,
                                          int head_dim, int page_size, int64_t num_pages, int kbar_pages,
-                                         int sel_stride, int first_page_offset, float sm_scale, kin_stream_t stream) {
+                                         int sel_stride, int first_page_offset, float sm_scale, void* workspace,
+                                         size_t workspace_bytes, kin_stream_t stream) {
   using namespace kin;
   const char* fn = "kin_blocktopk_decode_step";
   if (!q || !kv_cache || !kbar || !page_indices || !page_indptr || !last_page_len || !out)
@@ -216,6 +289,17 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
     nw = items <= kNumCus ? 16 : (items <= 2 * kNumCus ? 8 : 4);
   else
     nw = items <= kNumCus ? 8 : 4;
+  // Few long sequences: spread the scoring of each list over several workgroups.
+  p.chunks = step_score_chunks(batch, num_kv_heads, kbar_pages);
+  if (p.chunks > 1 && workspace && aligned16(workspace) &&
+      workspace_bytes >= kin_step_workspace_bytes(batch, num_kv_heads, kbar_pages)) {
+    p.ws_count = static_cast<int32_t*>(workspace);
+    p.ws_keys = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + step_count_bytes(items));
+  } else {
+    p.chunks = 1;
+    p.ws_count = nullptr;
+    p.ws_keys = nullptr;
+  }
   const size_t sel_scratch = select_lds_bytes(kbar_pages, p.sort_cap);
   size_t region0 = sel_scratch > (size_t)attend_lds_bytes(nw) ? sel_scratch : (size_t)attend_lds_bytes(nw);
   region0 = (region0 + 15) & ~(size_t)15;
@@ -239,8 +323,15 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
                    "hipFuncSetAttribute(blocktopk_step_kernel)");
     if (st) return st;
   }
+  unsigned grid = (unsigned)xcd_grid_size(batch, num_kv_heads);
+  if (p.chunks > 1) {
+    // the arrival counters start at zero (a fill kernel, so that the launch pair can be captured in a graph)
+    fill_zero_kernel<<<(unsigned)((items + 255) / 256), 256, 0, s>>>(p.ws_count, (int)items);
+    st = check_hip(hipGetLastError(), "fill_zero_kernel launch");
+    if (st) return st;
+    grid = (unsigned)(items * p.chunks);
+  }
   void* args[] = {&p};
-  st = check_hip(hipLaunchKernel(kernel, dim3((unsigned)xcd_grid_size(batch, num_kv_heads)), dim3(nw * 64), args, lds, s),
-                 "blocktopk_step_kernel launch");
+  st = check_hip(hipLaunchKernel(kernel, dim3(grid), dim3(nw * 64), args, lds, s), "blocktopk_step_kernel launch");
   return st;
 }

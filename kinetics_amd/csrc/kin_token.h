@@ -2,9 +2,10 @@
 // one (sequence, KV head), run by one workgroup of NW waves:
 //
 //   token_score_select()  streams every key of the sequence once (the K half of
-//       each page, through the same LDS-direct staging and MFMA tile as the
-//       page attention), turns the group-mean logit of every token of the
-//       "dynamic" part (after the sink tokens, before the local window) into an
+//       each page, 16-byte loads straight to registers; the mean over the
+//       group's heads of q_g . k_t is (mean_g q_g) . k_t, one fp32 dot product
+//       per token), turns the score of every token of the "dynamic" part
+//       (after the sink tokens, before the local window) into an
 //       order-preserving 32-bit key in an HBM scratch array, radix-selects the
 //       k-th largest key and compacts the winners, in ascending token order,
 //       into a token list in LDS: sink tokens, winners, local-window tokens;

@@ -244,6 +244,11 @@ def decode_workspace_bytes(batch, num_q_heads, num_kv_heads, max_pages_per_list,
     return int(_lib.load().kin_decode_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, max_pages_per_list, num_splits))
 
 
+def step_workspace_bytes(batch: int, num_kv_heads: int, kbar_pages: int) -> int:
+    """Bytes of workspace the fused step can use for this shape (0: none)."""
+    return int(_lib.load().kin_step_workspace_bytes(int(batch), int(num_kv_heads), int(kbar_pages)))
+
+
 def decode_auto_splits(batch, num_kv_heads, max_pages_per_list) -> int:
     return int(_lib.load().kin_decode_auto_splits(batch, num_kv_heads, max_pages_per_list))
 
@@ -345,12 +350,14 @@ def prefer_fused_step(batch: int, num_kv_heads: int, max_pages_per_seq: int, top
 
 def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, out=None, lse=None,
                           sel_pages=None, sel_count=None, sm_scale: float = 0.0, sink_pages: int = 0,
-                          local_tokens: int = 1, first_page_offset: int = 0):
+                          local_tokens: int = 1, first_page_offset: int = 0, workspace=None):
     """append -> score -> select -> attend in one launch: lines 209-225 of the
     reference layer's forward (benchmark/blocktopk_decoder.py) as a single
     kernel.  ``k``/``v`` may be None (no append); ``sel_pages``/``sel_count`` are
-    optional outputs.  Returns ``out`` [batch, num_q_heads, head_dim] bf16."""
-    dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, None)
+    optional outputs.  ``workspace`` (``step_workspace_bytes``; allocated here when
+    None and the shape profits) lets few, long sequences spread their scoring over
+    the GPU.  Returns ``out`` [batch, num_q_heads, head_dim] bf16."""
+    dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, workspace)
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     kbar_pages = _kbar_pages(kbar, batch, hkv, d)
     if (k is None) != (v is None):
@@ -369,6 +376,10 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
         if sel_pages.shape[:2] != (batch, hkv) or tuple(sel_count.shape) != (batch, hkv):
             raise ValueError(f"sel_pages/sel_count must be [{batch}, {hkv}, stride] / [{batch}, {hkv}]")
         sel_stride = sel_pages.shape[2]
+    if workspace is None:
+        need = step_workspace_bytes(batch, hkv, kbar_pages)
+        if need:
+            workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
         _lib.check(
@@ -376,7 +387,7 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
                 _ptr(q), _ptr(k), _ptr(v), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
                 _ptr(last_page_len), int(topk), int(sink_pages), int(local_tokens), _ptr(sel_pages), _ptr(sel_count),
                 _ptr(out), _ptr(lse), batch, hq, hkv, d, ps, num_pages, kbar_pages, sel_stride, int(first_page_offset),
-                float(sm_scale), _stream(dev),
+                float(sm_scale), _ptr(workspace), 0 if workspace is None else workspace.numel(), _stream(dev),
             )
         )
     return out
@@ -528,21 +539,21 @@ torch.library.define(
     "kinetics::blocktopk_decode_step",
     "(Tensor q, Tensor k, Tensor v, Tensor(a!) kv_cache, Tensor(b!) kbar, Tensor page_indices, Tensor page_indptr, "
     "Tensor last_page_len, int topk, Tensor(c!)? sel_pages, Tensor(d!)? sel_count, float sm_scale, "
-    "int sink_pages=0, int local_tokens=1, int first_page_offset=0) -> Tensor",
+    "int sink_pages=0, int local_tokens=1, int first_page_offset=0, Tensor(e!)? workspace=None) -> Tensor",
 )
 
 
 @torch.library.impl("kinetics::blocktopk_decode_step", "cuda")
 def _step_impl(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sm_scale,
-               sink_pages=0, local_tokens=1, first_page_offset=0):
+               sink_pages=0, local_tokens=1, first_page_offset=0, workspace=None):
     return blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk,
                                  sel_pages=sel_pages, sel_count=sel_count, sm_scale=sm_scale, sink_pages=sink_pages,
-                                 local_tokens=local_tokens, first_page_offset=first_page_offset)
+                                 local_tokens=local_tokens, first_page_offset=first_page_offset, workspace=workspace)
 
 
 @torch.library.register_fake("kinetics::blocktopk_decode_step")
 def _step_fake(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sm_scale,
-               sink_pages=0, local_tokens=1, first_page_offset=0):
+               sink_pages=0, local_tokens=1, first_page_offset=0, workspace=None):
     return torch.empty_like(q)
 
 

@@ -130,7 +130,7 @@ def test_decode_argument_errors(lib):
 def step(lib, q=A, k=A, v=A, kv=A, kbar=A, idx=A, ptr=A, last=A, topk=4, sink=0, local=1, sel=None, cnt=None, out=A, B=2,
          Hq=4, Hkv=1, D=128, ps=16, P=8, kp=64, stride=0, offset=0):
     return lib.kin_blocktopk_decode_step(q, k, v, kv, kbar, idx, ptr, last, topk, sink, local, sel, cnt, out, None, B, Hq, Hkv,
-                                         D, ps, P, kp, stride, offset, 0.0, None)
+                                         D, ps, P, kp, stride, offset, 0.0, None, 0, None)
 
 
 def test_step_argument_errors(lib):

@@ -680,6 +680,44 @@ def test_unused_cache_slots_may_hold_nan(ops):
         assert_out_close(dense, wd, "poisoned cache, dense")
 
 
+@pytest.mark.parametrize("hkv,group", [(1, 4), (2, 8), (8, 1)])
+def test_fused_step_split_scoring_for_few_long_sequences(ops, hkv, group):
+    """Few lists with thousands of candidate pages: the step spreads the scoring
+    of each list over several workgroups that meet through the workspace; same
+    cache bytes, page lists and output as without it, call after call."""
+    lengths = [PS * 2500 + 3, PS * 2100 + 16, 5, 0, PS * 300 + 1][: max(2, 10 // hkv)]
+    pb = P.make_problem(1400 + hkv, lengths, num_kv_heads=hkv, group=group, topk=40)
+    kbar_pages = pb.kbar.shape[1]
+    need = ops.step_workspace_bytes(pb.B, hkv, kbar_pages)
+    assert need > 0 and ops.step_workspace_bytes(4096, 1, kbar_pages) == 0 and ops.step_workspace_bytes(2, 1, 512) == 0
+    ws = torch.full((need,), 0xAB, dtype=torch.uint8, device=DEV)       # contents need no initialisation
+    a, b = Gpu(pb), Gpu(pb)
+    out_a = ops.blocktopk_decode_step(a.q, a.k, a.v, a.kv, a.kbar, a.indices, a.indptr, a.last, pb.topk, sel_pages=a.sel,
+                                      sel_count=a.cnt, workspace=torch.empty(0, dtype=torch.uint8, device=DEV))
+    outs = []
+    for _ in range(3):   # the arrival counters are reusable
+        b2 = Gpu(pb)
+        outs.append(ops.blocktopk_decode_step(b2.q, b2.k, b2.v, b2.kv, b2.kbar, b2.indices, b2.indptr, b2.last, pb.topk,
+                                              sel_pages=b2.sel, sel_count=b2.cnt, workspace=ws, sink_pages=0))
+        torch.cuda.synchronize()
+        assert torch.equal(a.kv, b2.kv) and torch.equal(a.kbar, b2.kbar)
+        assert torch.equal(a.cnt, b2.cnt) and torch.equal(a.sel, b2.sel)
+        assert torch.equal(out_a, outs[-1])
+    kv, kbar = pb.kv_cache.copy(), pb.kbar.copy()
+    res = O.decode_step(pb.q, pb.k, pb.v, kv, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
+    assert np.array_equal(P.from_torch(a.kv), kv) and np.array_equal(P.from_torch(a.kbar), kbar)
+    assert np.array_equal(a.cnt.cpu().numpy(), res["sel_count"])
+    sel = a.sel.cpu().numpy()
+    want, _ = O.sparse_paged_decode(pb.q, kv, sel, res["sel_count"], pb.last_page_len)
+    assert_out_close(out_a, want, "split scoring")
+    if np.array_equal(sel, res["sel_pages"]):
+        assert_out_close(out_a, res["out"], "split scoring vs oracle end to end")
+    # the wrapper allocates the workspace itself when none is given
+    c = Gpu(pb)
+    out_c = ops.blocktopk_decode_step(c.q, c.k, c.v, c.kv, c.kbar, c.indices, c.indptr, c.last, pb.topk)
+    assert torch.equal(out_c, out_a)
+
+
 # --------------------------------------------------------------------------- ragged multi-token append
 
 
