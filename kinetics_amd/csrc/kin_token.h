@@ -45,13 +45,160 @@ struct TokenArgs {
   int32_t* sel_tokens;   // HBM, the listed tokens' positions in the sequence, or null
 };
 
-__device__ __forceinline__ float quad_sum(float x) {
-  return (quad_bcast<0>(x) + quad_bcast<1>(x)) + (quad_bcast<2>(x) + quad_bcast<3>(x));
-}
-
 // Physical token id (page * 16 + slot) of cache slot c of the sequence.
 __device__ __forceinline__ int phys_token(const int32_t* table, int c) {
   return table[c >> 4] * kPageSize + (c & (kPageSize - 1));
+}
+
+// LDS scratch of the two functions below.
+struct KeySelectShared {
+  uint32_t hist[256];
+  uint32_t wave_gt[16], wave_eq[16];
+  uint32_t bin, remaining;
+};
+
+// Most-significant-digit-first radix select over n_keys (a multiple of 16) 32-bit
+// keys in global memory, run by a workgroup of NW waves: finds the k-th largest
+// non-zero key (zero keys are "not a candidate"; at least k keys are non-zero).
+// thr receives it, remaining how many keys equal to thr belong to the k largest.
+// first_digit_counted: sh->hist already holds the histogram of the top byte of
+// the non-zero keys (counted while they were produced).  The keys are written by
+// this workgroup; a barrier separates their last write from this call.
+template <int NW>
+__device__ __forceinline__ void radix_threshold(const uint32_t* keys, int n_keys, uint32_t k, bool first_digit_counted,
+                                                KeySelectShared* sh, uint32_t& thr, uint32_t& remaining) {
+  constexpr int NT = NW * 64;
+  const int tid = threadIdx.x;
+  const int w = tid >> 6, l = tid & 63;
+  uint32_t prefix = 0, mask = 0;
+  remaining = k;
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    if (shift != 24 || !first_digit_counted) {
+      if (tid < 256) sh->hist[tid] = 0;
+      __syncthreads();
+      // 4 independent 16-byte loads per thread in flight: the keys come from L2 / HBM
+      for (int base = tid * 4; base < n_keys; base += NT * 16) {
+        uint4 kk[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = base + u * NT * 4;
+          kk[u] = (i < n_keys) ? *reinterpret_cast<const uint4*>(keys + i) : make_uint4(0u, 0u, 0u, 0u);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (k4[j] && (k4[j] & mask) == prefix) atomicAdd(&sh->hist[(k4[j] >> shift) & 255u], 1u);
+        }
+      }
+      __syncthreads();
+    }
+    if (w == 0) radix_pick_bin(sh->hist, remaining, l, &sh->bin, &sh->remaining);
+    __syncthreads();
+    prefix |= sh->bin << shift;
+    mask |= 255u << shift;
+    remaining = sh->remaining;
+  }
+  thr = prefix;  // >= 1
+}
+
+// Calls emit(pos, index) for every key above thr and for the `remaining` lowest-
+// indexed keys equal to it, pos = 0, 1, ... in ascending index order.  Each wave
+// owns a contiguous run of indices and walks it 256 at a time (4 consecutive keys
+// per lane, two such loads in flight).  n_keys is a multiple of 16.
+template <int NW, typename Emit>
+__device__ __forceinline__ void compact_winners(const uint32_t* keys, int n_keys, uint32_t thr, uint32_t remaining,
+                                                KeySelectShared* sh, Emit emit) {
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63;
+  const int seg = ((n_keys + NW - 1) / NW + 255) & ~255;
+  const int seg_lo = min(w * seg, n_keys), seg_hi = min(seg_lo + seg, n_keys);  // multiples of 16
+  auto load4 = [&](int c) { return (c < seg_hi) ? *reinterpret_cast<const uint4*>(keys + c) : make_uint4(0u, 0u, 0u, 0u); };
+  uint32_t gt = 0, eq = 0;
+  for (int i = seg_lo; i < seg_hi; i += 1024) {
+    uint4 kk[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) kk[u] = load4(i + u * 256 + 4 * l);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        gt += (k4[j] > thr) ? 1u : 0u;
+        eq += (k4[j] == thr) ? 1u : 0u;
+      }
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    gt += __shfl_xor(gt, off);
+    eq += __shfl_xor(eq, off);
+  }
+  if (l == 0) {
+    sh->wave_gt[w] = gt;
+    sh->wave_eq[w] = eq;
+  }
+  __syncthreads();
+  uint32_t run = 0, eq_run = 0;  // winners / threshold-equal keys in the runs before this wave's
+  for (int wv = 0; wv < w; ++wv) {
+    const uint32_t e = sh->wave_eq[wv];
+    const uint32_t left = remaining > eq_run ? remaining - eq_run : 0u;
+    run += sh->wave_gt[wv] + min(e, left);
+    eq_run += e;
+  }
+  const unsigned long long below = (1ull << l) - 1ull;
+  for (int i = seg_lo; i < seg_hi; i += 512) {
+    uint4 kk[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) kk[u] = load4(i + u * 256 + 4 * l);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c0 = i + u * 256 + 4 * l;  // this lane's 4 consecutive indices
+      const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
+      // Keys equal to the threshold are rare: rank them (lane-major, then j) only when there are any.
+      bool is_eq[4];
+      uint32_t eq_mine = 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        is_eq[j] = k4[j] == thr;
+        eq_mine += is_eq[j] ? 1u : 0u;
+      }
+      uint32_t eq_before = eq_run;  // equal keys at lower indices
+      uint32_t eq_total = 0;
+      if (__ballot(eq_mine != 0) != 0ull) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const unsigned long long be = __ballot(is_eq[j]);
+          eq_before += __popcll(be & below);
+          eq_total += __popcll(be);
+        }
+      }
+      bool take[4];
+      uint32_t mine_eq_seen = 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        take[j] = k4[j] > thr || (is_eq[j] && eq_before + mine_eq_seen < remaining);
+        mine_eq_seen += is_eq[j] ? 1u : 0u;
+      }
+      uint32_t pos = run, total = 0;  // winners at lower indices
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const unsigned long long bt = __ballot(take[j]);
+        pos += __popcll(bt & below);
+        total += __popcll(bt);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (take[j]) {
+          emit((int)pos, c0 + j);
+          ++pos;
+        }
+      }
+      run += total;
+      eq_run += eq_total;
+    }
+  }
 }
 
 // Writes the token list (physical token ids) to a.list and returns its length.
@@ -60,13 +207,13 @@ __device__ __forceinline__ int phys_token(const int32_t* table, int c) {
 template <int NG, int NW>
 __device__ __forceinline__ int token_score_select(const TokenArgs& a, unsigned char* lds) {
   constexpr int NT = NW * 64;
-  __shared__ uint32_t hist[256];
-  __shared__ uint32_t wave_gt[NW], wave_eq[NW];
-  __shared__ uint32_t sh_bin, sh_remaining;
+  __shared__ KeySelectShared sh_store;
+  KeySelectShared* sh = &sh_store;
+  uint32_t* hist = sh->hist;
 
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int l = tid & 63, kg = l >> 4, c16 = l & 15, gq = l & 3;
+  const int l = tid & 63, kg = l >> 4, c16 = l & 15;
   const int G = a.G;
   const int n_pages = a.n_pages;
   const int k_eff = min(a.topk, a.n_dyn);
@@ -142,130 +289,13 @@ __device__ __forceinline__ int token_score_select(const TokenArgs& a, unsigned c
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();  // keys[] and hist[] complete and visible to the whole workgroup
 
-    // ---- phase 2: 4-digit radix select of the k_eff-th largest key -------------
-    uint32_t prefix = 0, mask = 0;
-    uint32_t remaining = (uint32_t)k_eff;
-    for (int shift = 24; shift >= 0; shift -= 8) {
-      if (shift != 24) {
-        if (tid < 256) hist[tid] = 0;
-        __syncthreads();
-        // 4 independent 16-byte loads per thread in flight: the keys come from L2 / HBM
-        for (int base = tid * 4; base < n_keys; base += NT * 16) {
-          uint4 kk[4];
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const int i = base + u * NT * 4;
-            kk[u] = (i < n_keys) ? *reinterpret_cast<const uint4*>(a.keys + i) : make_uint4(0u, 0u, 0u, 0u);
-          }
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-              if (k4[j] && (k4[j] & mask) == prefix) atomicAdd(&hist[(k4[j] >> shift) & 255u], 1u);
-          }
-        }
-        __syncthreads();
-      }
-      if (w == 0) radix_pick_bin(hist, remaining, l, &sh_bin, &sh_remaining);
-      __syncthreads();
-      prefix |= sh_bin << shift;
-      mask |= 255u << shift;
-      remaining = sh_remaining;
-    }
-    const uint32_t thr = prefix;  // >= 1; `remaining` keys equal to it are taken, lowest tokens first
-
-    // ---- phase 3: ordered compaction of the winners (ascending token order) ------
-    // Each wave owns a contiguous run of cache slots and walks it 256 at a time
-    // (4 consecutive keys per lane, two such loads in flight).
-    const int seg = ((n_keys + NW - 1) / NW + 255) & ~255;
-    const int seg_lo = min(w * seg, n_keys), seg_hi = min(seg_lo + seg, n_keys);  // multiples of 16
-    auto load4 = [&](int c) { return (c < seg_hi) ? *reinterpret_cast<const uint4*>(a.keys + c) : make_uint4(0u, 0u, 0u, 0u); };
-    uint32_t gt = 0, eq = 0;
-    for (int i = seg_lo; i < seg_hi; i += 1024) {
-      uint4 kk[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) kk[u] = load4(i + u * 256 + 4 * l);
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          gt += (k4[j] > thr) ? 1u : 0u;
-          eq += (k4[j] == thr) ? 1u : 0u;
-        }
-      }
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      gt += __shfl_xor(gt, off);
-      eq += __shfl_xor(eq, off);
-    }
-    if (l == 0) {
-      wave_gt[w] = gt;
-      wave_eq[w] = eq;
-    }
-    __syncthreads();
-    uint32_t run = 0, eq_run = 0;  // winners / threshold-equal keys in the runs before this wave's
-    for (int wv = 0; wv < w; ++wv) {
-      const uint32_t e = wave_eq[wv];
-      const uint32_t left = remaining > eq_run ? remaining - eq_run : 0u;
-      run += wave_gt[wv] + min(e, left);
-      eq_run += e;
-    }
-    const unsigned long long below = (1ull << l) - 1ull;
-    for (int i = seg_lo; i < seg_hi; i += 512) {
-      uint4 kk[2];
-#pragma unroll
-      for (int u = 0; u < 2; ++u) kk[u] = load4(i + u * 256 + 4 * l);
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int c0 = i + u * 256 + 4 * l;  // this lane's 4 consecutive cache slots
-        const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
-        // Keys equal to the threshold are rare: rank them (lane-major, then j) only when there are any.
-        bool is_eq[4];
-        uint32_t eq_mine = 0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          is_eq[j] = k4[j] == thr;
-          eq_mine += is_eq[j] ? 1u : 0u;
-        }
-        uint32_t eq_before = eq_run;   // equal keys in lower slots
-        uint32_t eq_total = 0;
-        if (__ballot(eq_mine != 0) != 0ull) {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const unsigned long long be = __ballot(is_eq[j]);
-            eq_before += __popcll(be & below);
-            eq_total += __popcll(be);
-          }
-        }
-        bool take[4];
-        uint32_t mine_eq_seen = 0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          take[j] = k4[j] > thr || (is_eq[j] && eq_before + mine_eq_seen < remaining);
-          mine_eq_seen += is_eq[j] ? 1u : 0u;
-        }
-        uint32_t pos = run, total = 0;  // winners in lower slots
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const unsigned long long bt = __ballot(take[j]);
-          pos += __popcll(bt & below);
-          total += __popcll(bt);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (take[j]) {
-            list[a.n_sink + pos] = phys_token(table, c0 + j);
-            if (a.sel_tokens) a.sel_tokens[a.n_sink + pos] = c0 + j - a.pad;
-            ++pos;
-          }
-        }
-        run += total;
-        eq_run += eq_total;
-      }
-    }
+    // ---- phases 2 and 3: threshold, then the winners in ascending token order ----
+    uint32_t thr, remaining;
+    radix_threshold<NW>(a.keys, n_keys, (uint32_t)k_eff, true, sh, thr, remaining);
+    compact_winners<NW>(a.keys, n_keys, thr, remaining, sh, [&](int pos, int c) {
+      list[a.n_sink + pos] = phys_token(table, c);
+      if (a.sel_tokens) a.sel_tokens[a.n_sink + pos] = c - a.pad;
+    });
   } else if (k_eff > 0) {
     // Budget covers every candidate: all of them, no key needed.
     for (int i = tid; i < k_eff; i += NT) {
