@@ -331,6 +331,38 @@ int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
                           kin_stream_t stream);
 
 /*
+ * Strided overlapping-block top-k decode attention in one launch -- LiteSys'
+ * strided_blockwise_topk_sparsity policy
+ * (ref: LiteSys/litesys/attention/sparsity_utils.py:49-105) inside
+ * BatchKVManager.decode (ref: LiteSys/litesys/attention/batch_cache.py:154-168).
+ * Per (sequence, KV head), with L candidate tokens between the sink tokens and
+ * the local window: block i covers candidates [i*stride, i*stride + block_size),
+ * i < (L - block_size) / stride + 1; the min(2*topk_blocks, num_blocks) blocks
+ * with the largest mean group-mean logit are chosen, their tokens united, and
+ * the topk_blocks * block_size lowest-positioned of those attended together with
+ * the sink and local tokens.  Candidates no chosen block covers are dropped,
+ * also when the budget would have room for them; with L < block_size every token
+ * is attended.  Arguments, outputs and token layout as in kin_token_topk_decode
+ * (sel_stride >= max(topk_blocks, 1) * block_size + sink + local).  workspace:
+ * kin_strided_topk_workspace_bytes(...).  Limits: block_size <= 64,
+ * topk_blocks * block_size <= 4096, sink_tokens <= 64, local_tokens <= 1024.
+ */
+size_t kin_strided_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq);
+
+int kin_strided_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
+                            const int32_t* page_indices, const int32_t* page_indptr,
+                            const int32_t* last_page_len,
+                            int topk_blocks, int block_size, int stride,
+                            int sink_tokens, int local_tokens, int first_page_offset,
+                            int32_t* sel_tokens, int32_t* sel_count,
+                            kin_bf16_t* out, float* lse,
+                            void* workspace, size_t workspace_bytes,
+                            int batch, int num_q_heads, int num_kv_heads,
+                            int head_dim, int page_size, int64_t num_pages,
+                            int max_pages_per_seq, int sel_stride, float sm_scale,
+                            kin_stream_t stream);
+
+/*
  * Page-table metadata for a slot-based cache -- the paged replacement of
  * LiteSys' contiguous per-slot caches and kv_offset counters
  * (ref: LiteSys/litesys/attention/batch_cache.py:40-62,76-84).  Slot s owns the

@@ -66,6 +66,12 @@ SIGNATURES = {
         [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int, c_int,
          c_int64, c_int, c_int, c_float, _P],
     ),
+    "kin_strided_topk_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "kin_strided_topk_decode": (
+        c_int,
+        [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int,
+         c_int, c_int, c_int64, c_int, c_int, c_float, _P],
+    ),
     "kin_build_slot_page_table": (c_int, [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P]),
     "kin_check_page_table": (c_int, [_P, _P, _P, c_int, c_int, c_int64, c_int64, _P, _P]),
 }

@@ -16,6 +16,9 @@ Supported configurations (anything else raises at construction):
   * ``attn_topk=k`` (+ ``attn_local``)          -> token-level top-k (topk_sparsity,
                                                   sparsity_utils.py:6-21), one launch that
                                                   reads every key of the context once
+  * ``attn_block_topk=k, attn_stride=s``        -> overlapping blocks every s tokens
+                                                  (strided_blockwise_topk_sparsity,
+                                                  sparsity_utils.py:49-105), also one launch
   * ``attn_local`` alone                        -> sink + local window only: block top-k with
                                                   k = 0, whose window is LiteSys' ``local``
                                                   rounded up to the block grid (a superset, by
@@ -48,7 +51,7 @@ from . import ops
 
 PAGE = 16
 
-_UNSUPPORTED = ("attn_random_select", "attn_random_nsample", "attn_stride")
+_UNSUPPORTED = ("attn_random_select", "attn_random_nsample")
 
 
 class PagedBatchKVManager:
@@ -82,14 +85,26 @@ class PagedBatchKVManager:
                 raise AssertionError("attn_local must be provided if use_nonlocal_sparsity is True")
             if not 0 <= int(self.token_topk) <= 4096 or not 0 <= int(kwargs["attn_local"]) <= 1024:
                 raise NotImplementedError("attn_topk must be in [0, 4096] and attn_local in [0, 1024]")
+        self.strided = None
         if self.block_topk is not None:
             if kwargs.get("attn_local") is None:
                 # same rule as LiteSys (sparsity_utils.py:207-208)
                 raise AssertionError("attn_local must be provided if use_nonlocal_sparsity is True")
-            if kwargs.get("attn_block_size", PAGE) != PAGE:
+            if kwargs.get("attn_stride") is not None:
+                # overlapping blocks (sparsity_utils.py:245-246): a token-granular policy, any block size up to 64
+                self.strided = (int(self.block_topk), int(kwargs.get("attn_block_size", PAGE)), int(kwargs["attn_stride"]))
+                self.token_local = int(kwargs["attn_local"])
+                if not (1 <= self.strided[1] <= 64 and self.strided[2] >= 1 and self.strided[0] * self.strided[1] <= 4096
+                        and 0 <= self.token_local <= 1024):
+                    raise NotImplementedError("strided blocks: block size <= 64, budget <= 4096 tokens, attn_local <= 1024")
+                self.block_topk = None
+            elif kwargs.get("attn_block_size", PAGE) != PAGE:
                 raise NotImplementedError("block size must equal the page size (16)")
-        self.sparse = kwargs.get("attn_local") is not None and self.token_topk is None
-        self.token_local = int(kwargs["attn_local"]) if self.token_topk is not None else 0
+        elif kwargs.get("attn_stride") is not None:
+            raise NotImplementedError("attn_stride needs attn_block_topk")
+        self.sparse = kwargs.get("attn_local") is not None and self.token_topk is None and self.strided is None
+        if self.token_topk is not None:
+            self.token_local = int(kwargs["attn_local"])
         if self.sparse and self.block_topk is None:
             self.block_topk = 0                      # sink + local window only
         self.layer_skip = list(kwargs.get("attn_layer_skip", [0]))
@@ -123,6 +138,8 @@ class PagedBatchKVManager:
         ws = max(ops.decode_workspace_bytes(B, Hq, Hkv, P), ops.decode_workspace_bytes(B, Hq, Hkv, self._sel.shape[2]), 16)
         if self.token_topk is not None:
             ws = max(ws, ops.token_topk_workspace_bytes(B, Hkv, P))
+        if self.strided is not None:
+            ws = max(ws, ops.strided_topk_workspace_bytes(B, Hkv, P))
         ws = max(ws, ops.step_workspace_bytes(B, Hkv, P))
         self._ws = torch.empty(ws, dtype=torch.uint8, device=dev)
 
@@ -162,6 +179,11 @@ class PagedBatchKVManager:
             ops.token_topk_decode(self._q, kv, self.page_indices, self.page_indptr, self.last_page_len, self.token_topk,
                                   self.pages_per_slot, sink_tokens=4, local_tokens=self.token_local, out=self._out,
                                   workspace=self._ws)
+        elif self.strided is not None and layer_idx not in self.layer_skip:
+            ops.append_paged_kv(self._k, self._v, kv, None, self.page_indices, self.page_indptr, self.last_page_len)
+            ops.strided_topk_decode(self._q, kv, self.page_indices, self.page_indptr, self.last_page_len, self.strided[0],
+                                    self.pages_per_slot, block_size=self.strided[1], stride=self.strided[2], sink_tokens=4,
+                                    local_tokens=self.token_local, out=self._out, workspace=self._ws)
         elif sparse and self._fused:
             ops.blocktopk_decode_step(self._q, self._k, self._v, kv, kbar, self.page_indices, self.page_indptr,
                                       self.last_page_len, self.block_topk, out=self._out, sink_pages=self.sink_pages,

@@ -201,20 +201,87 @@ __device__ __forceinline__ void compact_winners(const uint32_t* keys, int n_keys
   }
 }
 
-// Writes the token list (physical token ids) to a.list and returns its length.
-// lds: attend_lds_bytes(NW) of staging, 16-byte aligned.  Every thread of the
-// workgroup calls this; it ends with a workgroup barrier.
+// Streams the K plane of every page of the sequence once and calls
+// emit(c, score) -- from one lane per key row -- with score = (mean_g q_g) . k_c
+// in fp32 for every cache slot c of those pages (slots past the last token
+// included).  16-byte loads straight to registers, kU of them in flight per
+// lane; no LDS, no barrier.
+template <int NW, typename Emit>
+__device__ __forceinline__ void stream_token_scores(const TokenArgs& a, Emit emit) {
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l = tid & 63, kg = l >> 4, c16 = l & 15;
+  const int G = a.G;
+  const int n_pages = a.n_pages;
+  const int32_t* table = a.table;
+  // The mean over the group's heads of q_g . k_t is (mean_g q_g) . k_t: one dot
+  // product per token.  Lane owns columns d = 8*(lane%16) .. +7 of the mean query;
+  // 16 lanes share a key row, a wave covers 4 rows, 4 waves one page.
+  float qm[8];
+  {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) qm[u] = 0.f;
+    const uint16_t* qp = a.q_bh + 8 * c16;
+    for (int g = 0; g < G; ++g) {
+      const uint4 x = *reinterpret_cast<const uint4*>(qp + (int64_t)g * kHeadDim);
+      qm[0] += bf16_lo(x.x); qm[1] += bf16_hi(x.x);
+      qm[2] += bf16_lo(x.y); qm[3] += bf16_hi(x.y);
+      qm[4] += bf16_lo(x.z); qm[5] += bf16_hi(x.z);
+      qm[6] += bf16_lo(x.w); qm[7] += bf16_hi(x.w);
+    }
+    const float inv = 1.0f / (float)G;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) qm[u] *= inv;
+  }
+  constexpr int kPP = NW / 4;   // pages one pass of the workgroup covers
+  constexpr int kU = 16;        // passes (16-byte loads per lane) kept in flight
+  const __attribute__((address_space(4))) int32_t* tab_c =
+      reinterpret_cast<const __attribute__((address_space(4))) int32_t*>(reinterpret_cast<uintptr_t>(table));
+  const int row = 4 * (w & 3) + kg;                 // key row of the page this lane helps with
+  const int voff = row * a.row_bytes + c16 * 16;
+  const int k_span = kPageSize * a.row_bytes - (a.span < a.page_bytes ? a.page_bytes - a.span : 0);  // K plane only
+  auto load_page = [&](int p) -> u32x4 {
+    // Pages past the end (or with an id outside the cache) are read through an
+    // empty descriptor: zeros, no memory traffic.
+    const bool in = p < n_pages;
+    const int id = tab_c[in ? p : 0];
+    const bool ok = in && id >= 0 && (int64_t)id < a.num_pages;
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(a.kvb + (int64_t)(ok ? id : 0) * a.page_bytes, ok ? k_span : 0);
+    return __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, kStreamLoad);
+  };
+  const int p_first = w >> 2;  // this wave's page within a pass
+  u32x4 x[kU];
+#pragma unroll
+  for (int u = 0; u < kU; ++u) x[u] = load_page(p_first + u * kPP);
+  for (int base = 0; base < n_pages; base += kU * kPP) {
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      const u32x4 kx = x[u];
+      const int p = base + u * kPP + p_first;
+      x[u] = load_page(p + kU * kPP);
+      float acc = 0.f;
+      acc = fmaf(qm[0], bf16_lo(kx.x), acc); acc = fmaf(qm[1], bf16_hi(kx.x), acc);
+      acc = fmaf(qm[2], bf16_lo(kx.y), acc); acc = fmaf(qm[3], bf16_hi(kx.y), acc);
+      acc = fmaf(qm[4], bf16_lo(kx.z), acc); acc = fmaf(qm[5], bf16_hi(kx.z), acc);
+      acc = fmaf(qm[6], bf16_lo(kx.w), acc); acc = fmaf(qm[7], bf16_hi(kx.w), acc);
+      acc = row16_sum(acc);
+      const int c = p * kPageSize + row;
+      if (c16 == 0 && p < n_pages) emit(c, acc);
+    }
+  }
+}
+
+// Token-level top-k: writes the token list (physical token ids) to a.list and
+// returns its length.  Every thread of the workgroup calls this; it ends with a
+// workgroup barrier.
 template <int NG, int NW>
-__device__ __forceinline__ int token_score_select(const TokenArgs& a, unsigned char* lds) {
+__device__ __forceinline__ int token_score_select(const TokenArgs& a) {
   constexpr int NT = NW * 64;
   __shared__ KeySelectShared sh_store;
   KeySelectShared* sh = &sh_store;
   uint32_t* hist = sh->hist;
 
   const int tid = threadIdx.x;
-  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int l = tid & 63, kg = l >> 4, c16 = l & 15;
-  const int G = a.G;
   const int n_pages = a.n_pages;
   const int k_eff = min(a.topk, a.n_dyn);
   const int dyn_lo = a.pad + a.n_sink, dyn_hi = dyn_lo + a.n_dyn;  // cache slots of the candidates
@@ -226,66 +293,12 @@ __device__ __forceinline__ int token_score_select(const TokenArgs& a, unsigned c
     // ---- phase 1: group-mean logit of every token -> keys[], first radix digit counted on the fly
     if (tid < 256) hist[tid] = 0;
     __syncthreads();
-    // The mean over the group's heads of q_g . k_t is (mean_g q_g) . k_t: one dot
-    // product per token.  Lane owns columns d = 8*(lane%16) .. +7 of the mean query;
-    // 16 lanes share a key row, a wave covers 4 rows, 4 waves one page.
-    float qm[8];
-    {
-#pragma unroll
-      for (int u = 0; u < 8; ++u) qm[u] = 0.f;
-      const uint16_t* qp = a.q_bh + 8 * c16;
-      for (int g = 0; g < G; ++g) {
-        const uint4 x = *reinterpret_cast<const uint4*>(qp + (int64_t)g * kHeadDim);
-        qm[0] += bf16_lo(x.x); qm[1] += bf16_hi(x.x);
-        qm[2] += bf16_lo(x.y); qm[3] += bf16_hi(x.y);
-        qm[4] += bf16_lo(x.z); qm[5] += bf16_hi(x.z);
-        qm[6] += bf16_lo(x.w); qm[7] += bf16_hi(x.w);
-      }
-      const float inv = 1.0f / (float)G;
-#pragma unroll
-      for (int u = 0; u < 8; ++u) qm[u] *= inv;
-    }
-    constexpr int kPP = NW / 4;   // pages one pass of the workgroup covers
-    constexpr int kU = 16;        // passes (16-byte loads per lane) kept in flight
-    const __attribute__((address_space(4))) int32_t* tab_c =
-        reinterpret_cast<const __attribute__((address_space(4))) int32_t*>(reinterpret_cast<uintptr_t>(table));
-    const int row = 4 * (w & 3) + kg;                 // key row of the page this lane helps with
-    const int voff = row * a.row_bytes + c16 * 16;
-    const int k_span = kPageSize * a.row_bytes - (a.span < a.page_bytes ? a.page_bytes - a.span : 0);  // K plane only
-    auto load_page = [&](int p) -> u32x4 {
-      // Pages past the end (or with an id outside the cache) are read through an
-      // empty descriptor: zeros, no memory traffic.
-      const bool in = p < n_pages;
-      const int id = tab_c[in ? p : 0];
-      const bool ok = in && id >= 0 && (int64_t)id < a.num_pages;
-      const __amdgpu_buffer_rsrc_t r = make_rsrc(a.kvb + (int64_t)(ok ? id : 0) * a.page_bytes, ok ? k_span : 0);
-      return __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, kStreamLoad);
-    };
-    const int p_first = w >> 2;  // this wave's page within a pass
-    u32x4 x[kU];
-#pragma unroll
-    for (int u = 0; u < kU; ++u) x[u] = load_page(p_first + u * kPP);
-    for (int base = 0; base < n_pages; base += kU * kPP) {
-#pragma unroll
-      for (int u = 0; u < kU; ++u) {
-        const u32x4 kx = x[u];
-        const int p = base + u * kPP + p_first;
-        x[u] = load_page(p + kU * kPP);
-        float acc = 0.f;
-        acc = fmaf(qm[0], bf16_lo(kx.x), acc); acc = fmaf(qm[1], bf16_hi(kx.x), acc);
-        acc = fmaf(qm[2], bf16_lo(kx.y), acc); acc = fmaf(qm[3], bf16_hi(kx.y), acc);
-        acc = fmaf(qm[4], bf16_lo(kx.z), acc); acc = fmaf(qm[5], bf16_hi(kx.z), acc);
-        acc = fmaf(qm[6], bf16_lo(kx.w), acc); acc = fmaf(qm[7], bf16_hi(kx.w), acc);
-        acc = row16_sum(acc);
-        const int c = p * kPageSize + row;
-        if (c16 == 0 && p < n_pages) {
-          // 0 marks "not a candidate" (order_key is never 0 for a finite score)
-          const uint32_t key = (c >= dyn_lo && c < dyn_hi) ? order_key(acc) : 0u;
-          a.keys[c] = key;
-          if (key) atomicAdd(&hist[key >> 24], 1u);
-        }
-      }
-    }
+    stream_token_scores<NW>(a, [&](int c, float score) {
+      // 0 marks "not a candidate" (order_key is never 0 for a finite score)
+      const uint32_t key = (c >= dyn_lo && c < dyn_hi) ? order_key(score) : 0u;
+      a.keys[c] = key;
+      if (key) atomicAdd(&hist[key >> 24], 1u);
+    });
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();  // keys[] and hist[] complete and visible to the whole workgroup
 
@@ -312,6 +325,133 @@ __device__ __forceinline__ int token_score_select(const TokenArgs& a, unsigned c
   }
   __syncthreads();
   return a.n_sink + k_eff + a.n_local;
+}
+
+// What the strided overlapping-block policy needs on top of TokenArgs
+// (a.topk and a.keys are not used by it).
+struct StridedArgs {
+  int block;             // tokens per block
+  int stride;            // tokens between block starts
+  int topk_blocks;       // budget: 2 * topk_blocks blocks are chosen, at most topk_blocks * block tokens kept
+  float* scores;         // HBM scratch, n_pages * 16 entries
+  uint32_t* block_keys;  // HBM scratch, >= n_pages * 16 entries, 16-byte aligned
+  uint32_t* bitmap;      // LDS, one bit per candidate token: (n_dyn + 31) / 32 words
+};
+
+// Strided overlapping-block top-k: block i covers the candidate tokens
+// [i*stride, i*stride + block); the min(2*topk_blocks, num_blocks) blocks with the
+// largest mean score are chosen, their tokens united, and the topk_blocks*block
+// lowest-positioned of those kept.  With fewer candidates than one block every
+// token is listed.  Writes the token list to a.list (sink tokens, kept tokens in
+// ascending order, local tokens) and returns its length; ends with a barrier.
+template <int NG, int NW>
+__device__ __forceinline__ int strided_score_select(const TokenArgs& a, const StridedArgs& sa) {
+  constexpr int NT = NW * 64;
+  __shared__ KeySelectShared sh_store;
+  __shared__ uint32_t wave_cnt[NW];
+  KeySelectShared* sh = &sh_store;
+  uint32_t* hist = sh->hist;
+
+  const int tid = threadIdx.x;
+  const int w = tid >> 6, l = tid & 63;
+  const int dyn_lo = a.pad + a.n_sink;
+  const int L = a.n_dyn;
+  int32_t* list = a.list;
+  const int32_t* table = a.table;
+  int kept = 0;  // candidate tokens listed
+
+  if (L < sa.block) {
+    // Too short for block sparsity: everything is attended.
+    for (int i = tid; i < L; i += NT) {
+      list[a.n_sink + i] = phys_token(table, dyn_lo + i);
+      if (a.sel_tokens) a.sel_tokens[a.n_sink + i] = a.n_sink + i;
+    }
+    kept = L;
+  } else {
+    const int num_blocks = (L - sa.block) / sa.stride + 1;
+    const int k_blocks = min(2 * sa.topk_blocks, num_blocks);
+    const int budget = sa.topk_blocks * sa.block;
+    const int n_words = (L + 31) >> 5;
+    for (int i = tid; i < n_words; i += NT) sa.bitmap[i] = 0u;
+    if (tid < 256) hist[tid] = 0;
+    // ---- token scores -> HBM ------------------------------------------------
+    stream_token_scores<NW>(a, [&](int c, float score) { sa.scores[c] = score; });
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    // ---- block means -> keys (padded with "no candidate" to a multiple of 16) --
+    const int nb_pad = (num_blocks + 15) & ~15;
+    const float inv = 1.0f / (float)sa.block;
+    for (int i = tid; i < nb_pad; i += NT) {
+      uint32_t key = 0u;
+      if (i < num_blocks) {
+        const float* sp = sa.scores + dyn_lo + i * sa.stride;
+        float sum = 0.f;
+        for (int t = 0; t < sa.block; ++t) sum += sp[t];
+        key = order_key(sum * inv);
+        atomicAdd(&hist[key >> 24], 1u);
+      }
+      sa.block_keys[i] = key;
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    // ---- chosen blocks -> token bitmap ---------------------------------------
+    auto mark_block = [&](int i) {
+      const int t0 = i * sa.stride, t1 = t0 + sa.block;  // candidate-relative token range
+      for (int wd = t0 >> 5; wd <= (t1 - 1) >> 5; ++wd) {
+        const int lo = max(t0, wd << 5) & 31, hi = min(t1, (wd + 1) << 5) - (wd << 5);  // bits [lo, hi) of the word
+        const uint32_t m = (hi >= 32 ? 0xffffffffu : ((1u << hi) - 1u)) & ~((1u << lo) - 1u);
+        atomicOr(&sa.bitmap[wd], m);
+      }
+    };
+    if (k_blocks == 0) {
+      // no budget: nothing of the dynamic part is attended
+    } else if (k_blocks < num_blocks) {
+      uint32_t thr, remaining;
+      radix_threshold<NW>(sa.block_keys, nb_pad, (uint32_t)k_blocks, true, sh, thr, remaining);
+      compact_winners<NW>(sa.block_keys, nb_pad, thr, remaining, sh, [&](int, int i) { mark_block(i); });
+    } else {
+      for (int i = tid; i < num_blocks; i += NT) mark_block(i);
+    }
+    __syncthreads();
+    // ---- bitmap -> token list, ascending, the first `budget` tokens ----------------
+    const int per = (n_words + NT - 1) / NT;  // consecutive words per thread
+    const int w_lo = min(tid * per, n_words), w_hi = min(w_lo + per, n_words);
+    uint32_t cnt = 0;
+    for (int i = w_lo; i < w_hi; ++i) cnt += __popc(sa.bitmap[i]);
+    uint32_t incl = cnt;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const uint32_t up = __shfl_up(incl, off);
+      if (l >= off) incl += up;
+    }
+    if (l == 63) wave_cnt[w] = incl;
+    __syncthreads();
+    uint32_t pos = incl - cnt, total = 0;
+    for (int wv = 0; wv < NW; ++wv) {
+      if (wv < w) pos += wave_cnt[wv];
+      total += wave_cnt[wv];
+    }
+    for (int i = w_lo; i < w_hi && pos < (uint32_t)budget; ++i) {
+      uint32_t bits = sa.bitmap[i];
+      while (bits && pos < (uint32_t)budget) {
+        const int t = (i << 5) + __builtin_ctz(bits);
+        bits &= bits - 1u;
+        list[a.n_sink + pos] = phys_token(table, dyn_lo + t);
+        if (a.sel_tokens) a.sel_tokens[a.n_sink + pos] = a.n_sink + t;
+        ++pos;
+      }
+    }
+    kept = (int)min(total, (uint32_t)budget);
+  }
+  for (int i = tid; i < a.n_sink + a.n_local; i += NT) {
+    const bool sink = i < a.n_sink;
+    const int t = sink ? i : a.n_sink + a.n_dyn + (i - a.n_sink);  // position in the sequence
+    const int pos = sink ? i : kept + i;
+    list[pos] = phys_token(table, a.pad + t);
+    if (a.sel_tokens) a.sel_tokens[pos] = t;
+  }
+  __syncthreads();
+  return a.n_sink + kept + a.n_local;
 }
 
 // Attention over a list of n = a.n physical token ids in LDS (a.p0 / a.p1 /

@@ -16,7 +16,10 @@ struct TokenTopkParams {
   int32_t* sel_count;   // optional [lists]
   uint16_t* out;
   float* lse;           // optional
-  uint32_t* keys;       // workspace: [lists, max_pages_per_seq * 16]
+  uint32_t* keys;       // workspace: [lists, max_pages_per_seq * 16] (token keys, or block keys)
+  float* scores;        // workspace, strided blocks only: [lists, max_pages_per_seq * 16]
+  int block, stride;    // strided blocks only
+  int list_cap;         // entries of the LDS token list
   int batch, num_q_heads, num_kv_heads, group;
   int topk, sink_tokens, local_tokens, first_page_offset;
   int max_pages_per_seq, sel_stride;
@@ -24,8 +27,10 @@ struct TokenTopkParams {
   float scale_log2;
 };
 
-// Dynamic LDS: K staging attend_lds_bytes(NW) | int32 list[sink + topk + local]
-template <int NG, int NW>
+// STRIDED = false: token-level top-k (p.topk tokens); true: strided overlapping
+// blocks (p.topk blocks).
+// Dynamic LDS: K staging attend_lds_bytes(NW) | int32 list[list_cap] | uint32 bitmap[] (strided only)
+template <int NG, int NW, bool STRIDED>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(TokenTopkParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ float sm_m[NW][4 * NG];
@@ -75,7 +80,19 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
   t.keys = p.keys + (int64_t)item * p.max_pages_per_seq * kPageSize;
   t.list = list;
   t.sel_tokens = sel_out;
-  const int n = token_score_select<NG, NW>(t, smem);
+  int n;
+  if (STRIDED) {
+    StridedArgs sa;
+    sa.block = p.block;
+    sa.stride = p.stride;
+    sa.topk_blocks = p.topk;
+    sa.scores = p.scores + (int64_t)item * p.max_pages_per_seq * kPageSize;
+    sa.block_keys = t.keys;
+    sa.bitmap = reinterpret_cast<uint32_t*>(list + p.list_cap);
+    n = strided_score_select<NG, NW>(t, sa);
+  } else {
+    n = token_score_select<NG, NW>(t);
+  }
   if (sel_out)
     for (int i = n + tid; i < p.sel_stride; i += NT) sel_out[i] = -1;
   if (p.sel_count && tid == 0) p.sel_count[item] = n;
@@ -102,22 +119,17 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
 
 }  // namespace kin
 
-extern "C" {
+namespace kin {
 
-size_t kin_token_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq) {
-  if (batch <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0) return 0;
-  return (size_t)batch * num_kv_heads * max_pages_per_seq * kin::kPageSize * sizeof(uint32_t);
-}
-
-int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const int32_t* page_indices,
-                          const int32_t* page_indptr, const int32_t* last_page_len, int topk_tokens,
-                          int sink_tokens, int local_tokens, int first_page_offset, int32_t* sel_tokens,
-                          int32_t* sel_count, kin_bf16_t* out, float* lse, void* workspace, size_t workspace_bytes,
-                          int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
-                          int64_t num_pages, int max_pages_per_seq, int sel_stride, float sm_scale,
-                          kin_stream_t stream) {
-  using namespace kin;
-  const char* fn = "kin_token_topk_decode";
+// Shared by the two entry points.  topk counts tokens (block == 0) or blocks.
+static int launch_token_policy(const char* fn, const kin_bf16_t* q, const kin_bf16_t* kv_cache,
+                               const int32_t* page_indices, const int32_t* page_indptr, const int32_t* last_page_len,
+                               int topk, int block, int stride, int sink_tokens, int local_tokens,
+                               int first_page_offset, int32_t* sel_tokens, int32_t* sel_count, kin_bf16_t* out,
+                               float* lse, void* workspace, size_t workspace_bytes, int batch, int num_q_heads,
+                               int num_kv_heads, int head_dim, int page_size, int64_t num_pages,
+                               int max_pages_per_seq, int sel_stride, float sm_scale, kin_stream_t stream) {
+  const bool strided = block > 0;
   if (!q || !kv_cache || !page_indices || !page_indptr || !last_page_len || !out)
     return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size);
@@ -127,22 +139,33 @@ int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const
   if (num_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_pages=%lld must be >= 1", fn, (long long)num_pages);
   if (num_pages > 0x7fffffffLL / kPageSize)
     return fail(KIN_ERR_UNSUPPORTED, "%s: num_pages=%lld: token ids do not fit 31 bits", fn, (long long)num_pages);
-  if (topk_tokens < 0 || sink_tokens < 0 || local_tokens < 0)
-    return fail(KIN_ERR_BAD_SHAPE, "%s: topk_tokens=%d, sink_tokens=%d and local_tokens=%d must not be negative", fn,
-                topk_tokens, sink_tokens, local_tokens);
-  if (topk_tokens > kMaxTopkTokens || sink_tokens > kMaxSinkTokens || local_tokens > kMaxWindowTokens)
-    return fail(KIN_ERR_UNSUPPORTED, "%s: limits are topk_tokens <= %d, sink_tokens <= %d, local_tokens <= %d", fn,
-                kMaxTopkTokens, kMaxSinkTokens, kMaxWindowTokens);
+  if (topk < 0 || sink_tokens < 0 || local_tokens < 0)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: the budget (%d), sink_tokens=%d and local_tokens=%d must not be negative", fn,
+                topk, sink_tokens, local_tokens);
   if (max_pages_per_seq < 1)
     return fail(KIN_ERR_BAD_SHAPE, "%s: max_pages_per_seq=%d must be >= 1", fn, max_pages_per_seq);
-  const int list_cap = topk_tokens + sink_tokens + local_tokens;
+  int budget_tokens = topk;
+  if (strided) {
+    if (block > 64 || stride < 1)
+      return fail(KIN_ERR_BAD_SHAPE, "%s: block_size=%d must be in [1, 64] and stride=%d at least 1", fn, block, stride);
+    if ((int64_t)topk * block > kMaxTopkTokens)
+      return fail(KIN_ERR_UNSUPPORTED, "%s: topk_blocks * block_size = %lld exceeds the limit %d", fn,
+                  (long long)topk * block, kMaxTopkTokens);
+    budget_tokens = topk * block;
+    if (budget_tokens < block) budget_tokens = block;  // sequences shorter than a block are listed whole
+  }
+  if (budget_tokens > kMaxTopkTokens || sink_tokens > kMaxSinkTokens || local_tokens > kMaxWindowTokens)
+    return fail(KIN_ERR_UNSUPPORTED, "%s: limits are %d selected tokens, sink_tokens <= %d, local_tokens <= %d", fn,
+                kMaxTopkTokens, kMaxSinkTokens, kMaxWindowTokens);
+  const int list_cap = budget_tokens + sink_tokens + local_tokens;
   if (sel_tokens && sel_stride < list_cap)
-    return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must be at least topk + sink + local tokens = %d", fn, sel_stride,
-                list_cap);
+    return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must be at least %d (selected + sink + local tokens)", fn,
+                sel_stride, list_cap);
   if (sel_tokens && !sel_count) return fail(KIN_ERR_NULL_POINTER, "%s: sel_tokens given without sel_count", fn);
   if (!aligned16(q) || !aligned16(kv_cache) || !aligned16(out))
     return fail(KIN_ERR_MISALIGNED, "%s: q, kv_cache and out must be 16-byte aligned", fn);
-  const size_t need = kin_token_topk_workspace_bytes(batch, num_kv_heads, max_pages_per_seq);
+  const size_t key_bytes = kin_token_topk_workspace_bytes(batch, num_kv_heads, max_pages_per_seq);
+  const size_t need = strided ? 2 * key_bytes : key_bytes;
   if (batch == 0) return KIN_OK;
   if (!workspace || workspace_bytes < need)
     return fail(KIN_ERR_WORKSPACE, "%s: needs %zu workspace bytes, got %zu", fn, need,
@@ -160,11 +183,15 @@ int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const
   p.out = out;
   p.lse = lse;
   p.keys = static_cast<uint32_t*>(workspace);
+  p.scores = strided ? reinterpret_cast<float*>(static_cast<char*>(workspace) + key_bytes) : nullptr;
+  p.block = block;
+  p.stride = stride;
+  p.list_cap = list_cap > 0 ? list_cap : 1;
   p.batch = batch;
   p.num_q_heads = num_q_heads;
   p.num_kv_heads = num_kv_heads;
   p.group = num_q_heads / num_kv_heads;
-  p.topk = topk_tokens;
+  p.topk = topk;
   p.sink_tokens = sink_tokens;
   p.local_tokens = local_tokens;
   p.first_page_offset = first_page_offset;
@@ -180,14 +207,27 @@ int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const
   // Waves per workgroup: 8 when the lists are too few to fill the GPU with 4-wave
   // workgroups (the per-token addressing needs ~140 registers, so 16 do not fit).
   const int nw = items <= 2 * kNumCus ? 8 : 4;
-  const size_t lds = (size_t)attend_lds_bytes(nw) + (size_t)(list_cap > 0 ? list_cap : 1) * 4;
+  const size_t bitmap_bytes = strided ? ((size_t)max_pages_per_seq * kPageSize / 32 + 1) * 4 : 0;
+  const size_t lds = (size_t)attend_lds_bytes(nw) + (size_t)p.list_cap * 4 + bitmap_bytes;
+  if (lds > 150 * 1024)
+    return fail(KIN_ERR_UNSUPPORTED, "%s: max_pages_per_seq=%d is too long for the strided policy's token bitmap", fn,
+                max_pages_per_seq);
   const void* kernel;
-  if (p.group <= 4)
-    kernel = nw == 8 ? reinterpret_cast<const void*>(&token_topk_kernel<1, 8>)
-                     : reinterpret_cast<const void*>(&token_topk_kernel<1, 4>);
-  else
-    kernel = nw == 8 ? reinterpret_cast<const void*>(&token_topk_kernel<2, 8>)
-                     : reinterpret_cast<const void*>(&token_topk_kernel<2, 4>);
+  if (strided) {
+    if (p.group <= 4)
+      kernel = nw == 8 ? reinterpret_cast<const void*>(&token_topk_kernel<1, 8, true>)
+                       : reinterpret_cast<const void*>(&token_topk_kernel<1, 4, true>);
+    else
+      kernel = nw == 8 ? reinterpret_cast<const void*>(&token_topk_kernel<2, 8, true>)
+                       : reinterpret_cast<const void*>(&token_topk_kernel<2, 4, true>);
+  } else {
+    if (p.group <= 4)
+      kernel = nw == 8 ? reinterpret_cast<const void*>(&token_topk_kernel<1, 8, false>)
+                       : reinterpret_cast<const void*>(&token_topk_kernel<1, 4, false>);
+    else
+      kernel = nw == 8 ? reinterpret_cast<const void*>(&token_topk_kernel<2, 8, false>)
+                       : reinterpret_cast<const void*>(&token_topk_kernel<2, 4, false>);
+  }
   if (lds > 48 * 1024) {
     st = check_hip(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
                    "hipFuncSetAttribute(token_topk_kernel)");
@@ -197,6 +237,48 @@ int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const
   return check_hip(hipLaunchKernel(kernel, dim3((unsigned)xcd_grid_size(batch, num_kv_heads)), dim3(nw * 64), args, lds,
                                    static_cast<hipStream_t>(stream)),
                    "token_topk_kernel launch");
+}
+
+}  // namespace kin
+
+extern "C" {
+
+size_t kin_token_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq) {
+  if (batch <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0) return 0;
+  return (size_t)batch * num_kv_heads * max_pages_per_seq * kin::kPageSize * sizeof(uint32_t);
+}
+
+size_t kin_strided_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq) {
+  return 2 * kin_token_topk_workspace_bytes(batch, num_kv_heads, max_pages_per_seq);
+}
+
+int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const int32_t* page_indices,
+                          const int32_t* page_indptr, const int32_t* last_page_len, int topk_tokens,
+                          int sink_tokens, int local_tokens, int first_page_offset, int32_t* sel_tokens,
+                          int32_t* sel_count, kin_bf16_t* out, float* lse, void* workspace, size_t workspace_bytes,
+                          int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
+                          int64_t num_pages, int max_pages_per_seq, int sel_stride, float sm_scale,
+                          kin_stream_t stream) {
+  return kin::launch_token_policy("kin_token_topk_decode", q, kv_cache, page_indices, page_indptr, last_page_len,
+                                  topk_tokens, 0, 0, sink_tokens, local_tokens, first_page_offset, sel_tokens,
+                                  sel_count, out, lse, workspace, workspace_bytes, batch, num_q_heads, num_kv_heads,
+                                  head_dim, page_size, num_pages, max_pages_per_seq, sel_stride, sm_scale, stream);
+}
+
+int kin_strided_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const int32_t* page_indices,
+                            const int32_t* page_indptr, const int32_t* last_page_len, int topk_blocks,
+                            int block_size, int stride, int sink_tokens, int local_tokens, int first_page_offset,
+                            int32_t* sel_tokens, int32_t* sel_count, kin_bf16_t* out, float* lse, void* workspace,
+                            size_t workspace_bytes, int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                            int page_size, int64_t num_pages, int max_pages_per_seq, int sel_stride, float sm_scale,
+                            kin_stream_t stream) {
+  if (block_size < 1)
+    return kin::fail(KIN_ERR_BAD_SHAPE, "kin_strided_topk_decode: block_size=%d must be in [1, 64]", block_size);
+  return kin::launch_token_policy("kin_strided_topk_decode", q, kv_cache, page_indices, page_indptr, last_page_len,
+                                  topk_blocks, block_size, stride, sink_tokens, local_tokens, first_page_offset,
+                                  sel_tokens, sel_count, out, lse, workspace, workspace_bytes, batch, num_q_heads,
+                                  num_kv_heads, head_dim, page_size, num_pages, max_pages_per_seq, sel_stride,
+                                  sm_scale, stream);
 }
 
 }  // extern "C"

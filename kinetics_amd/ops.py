@@ -397,15 +397,8 @@ def token_topk_workspace_bytes(batch: int, num_kv_heads: int, max_pages_per_seq:
     return int(_lib.load().kin_token_topk_workspace_bytes(int(batch), int(num_kv_heads), int(max_pages_per_seq)))
 
 
-def token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, topk_tokens: int, max_pages_per_seq: int,
-                      sink_tokens: int = 4, local_tokens: int = 1, first_page_offset: int = 0, out=None, lse=None,
-                      sel_tokens=None, sel_count=None, workspace=None, sm_scale: float = 0.0):
-    """Token-level top-k sparse decode attention: LiteSys' ``topk_sparsity``
-    (LiteSys/litesys/attention/sparsity_utils.py:6-21) inside its decode
-    (batch_cache.py:154-168) in one launch on the paged cache.  The first
-    ``sink_tokens`` and newest ``local_tokens`` tokens are always attended; of
-    the rest, the ``topk_tokens`` with the largest group-mean logit per KV
-    head.  The new token must already be appended.  Returns ``out``."""
+def _token_policy(q, kv_cache, page_indices, page_indptr, last_page_len, out, lse, sel_tokens, sel_count, workspace,
+                  need_bytes):
     dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, None)
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     sel_stride = 0
@@ -417,11 +410,25 @@ def token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, top
         if sel_tokens.shape[:2] != (batch, hkv) or tuple(sel_count.shape) != (batch, hkv):
             raise ValueError(f"sel_tokens/sel_count must be [{batch}, {hkv}, stride] / [{batch}, {hkv}]")
         sel_stride = sel_tokens.shape[2]
-    need = token_topk_workspace_bytes(batch, hkv, max_pages_per_seq)
     if workspace is None:
-        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+        workspace = torch.empty(max(need_bytes(batch, hkv), 16), dtype=torch.uint8, device=dev)
     else:
         _require(workspace, "workspace", torch.uint8, 1, dev)
+    return dev, batch, hq, hkv, d, ps, num_pages, out, sel_stride, workspace
+
+
+def token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, topk_tokens: int, max_pages_per_seq: int,
+                      sink_tokens: int = 4, local_tokens: int = 1, first_page_offset: int = 0, out=None, lse=None,
+                      sel_tokens=None, sel_count=None, workspace=None, sm_scale: float = 0.0):
+    """Token-level top-k sparse decode attention: LiteSys' ``topk_sparsity``
+    (LiteSys/litesys/attention/sparsity_utils.py:6-21) inside its decode
+    (batch_cache.py:154-168) in one launch on the paged cache.  The first
+    ``sink_tokens`` and newest ``local_tokens`` tokens are always attended; of
+    the rest, the ``topk_tokens`` with the largest group-mean logit per KV
+    head.  The new token must already be appended.  Returns ``out``."""
+    dev, batch, hq, hkv, d, ps, num_pages, out, sel_stride, workspace = _token_policy(
+        q, kv_cache, page_indices, page_indptr, last_page_len, out, lse, sel_tokens, sel_count, workspace,
+        lambda b, h: token_topk_workspace_bytes(b, h, max_pages_per_seq))
     lib = _lib.load()
     with torch.cuda.device(dev):
         _lib.check(
@@ -430,6 +437,36 @@ def token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, top
                 int(sink_tokens), int(local_tokens), int(first_page_offset), _ptr(sel_tokens), _ptr(sel_count), _ptr(out),
                 _ptr(lse), _ptr(workspace), workspace.numel(), batch, hq, hkv, d, ps, num_pages, int(max_pages_per_seq),
                 sel_stride, float(sm_scale), _stream(dev),
+            )
+        )
+    return out
+
+
+def strided_topk_workspace_bytes(batch: int, num_kv_heads: int, max_pages_per_seq: int) -> int:
+    return int(_lib.load().kin_strided_topk_workspace_bytes(int(batch), int(num_kv_heads), int(max_pages_per_seq)))
+
+
+def strided_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, topk_blocks: int, max_pages_per_seq: int,
+                        block_size: int = 16, stride: int = 8, sink_tokens: int = 4, local_tokens: int = 1,
+                        first_page_offset: int = 0, out=None, lse=None, sel_tokens=None, sel_count=None, workspace=None,
+                        sm_scale: float = 0.0):
+    """Strided overlapping-block top-k sparse decode attention: LiteSys'
+    ``strided_blockwise_topk_sparsity`` (sparsity_utils.py:49-105) inside its
+    decode, in one launch on the paged cache.  Blocks of ``block_size`` candidate
+    tokens start every ``stride`` tokens; the ``2 * topk_blocks`` best by mean
+    logit are united and the ``topk_blocks * block_size`` lowest-positioned of
+    their tokens attended, with the sink and local tokens.  Returns ``out``."""
+    dev, batch, hq, hkv, d, ps, num_pages, out, sel_stride, workspace = _token_policy(
+        q, kv_cache, page_indices, page_indptr, last_page_len, out, lse, sel_tokens, sel_count, workspace,
+        lambda b, h: strided_topk_workspace_bytes(b, h, max_pages_per_seq))
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(
+            lib.kin_strided_topk_decode(
+                _ptr(q), _ptr(kv_cache), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), int(topk_blocks),
+                int(block_size), int(stride), int(sink_tokens), int(local_tokens), int(first_page_offset),
+                _ptr(sel_tokens), _ptr(sel_count), _ptr(out), _ptr(lse), _ptr(workspace), workspace.numel(), batch, hq,
+                hkv, d, ps, num_pages, int(max_pages_per_seq), sel_stride, float(sm_scale), _stream(dev),
             )
         )
     return out

@@ -410,11 +410,49 @@ def litesys_topk_mask(mean_logits, seq_len, topk, local, sink=4):
     return keep
 
 
+def litesys_strided_mask(mean_logits, seq_len, topk_block, local, sink=4, block_size=16, stride=8):
+    """LiteSys/litesys/attention/sparsity_utils.py:49-105 for one sequence and one
+    KV head.  Nothing is masked when ``seq_len <= sink + local`` (:56-57) or the
+    dynamic part is shorter than a block (:63-64).  Otherwise overlapping blocks
+    start every ``stride`` dynamic tokens (:74-77), their mean logit ranks them
+    (:80-81), ``min(2 * topk_block, num_blocks)`` are taken (:84-85), their tokens
+    united in position order and cut to ``topk_block * block_size`` (:88-95); the
+    rest of the dynamic part is masked (:101-103)."""
+    keep = np.ones(seq_len, dtype=bool)
+    if seq_len <= sink + local:
+        return keep
+    dyn = np.asarray(mean_logits[sink : seq_len - local], dtype=np.float64)
+    L = len(dyn)
+    if L < block_size:
+        return keep
+    num_blocks = (L - block_size) // stride + 1
+    starts = np.arange(num_blocks) * stride
+    block_means = np.array([dyn[s0 : s0 + block_size].mean() for s0 in starts])
+    top = select_topk(block_means, min(2 * topk_block, num_blocks))
+    tokens = np.unique(np.concatenate([np.arange(starts[i], starts[i] + block_size) for i in top])) if len(top) else \
+        np.zeros(0, dtype=np.int64)
+    tokens = tokens[: topk_block * block_size]
+    dyn_keep = np.zeros(L, dtype=bool)
+    dyn_keep[tokens] = True
+    keep[sink : seq_len - local] = dyn_keep
+    return keep
+
+
+def strided_block_means(mean_logits, seq_len, local, sink=4, block_size=16, stride=8):
+    """The block means litesys_strided_mask ranks (empty when nothing is masked)."""
+    if seq_len <= sink + local or seq_len - sink - local < block_size:
+        return np.zeros(0)
+    dyn = np.asarray(mean_logits[sink : seq_len - local], dtype=np.float64)
+    num_blocks = (len(dyn) - block_size) // stride + 1
+    return np.array([dyn[i * stride : i * stride + block_size].mean() for i in range(num_blocks)])
+
+
 def token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, topk, sink=4, local=1, first_page_offset=0,
-                      sm_scale=None):
+                      sm_scale=None, policy="topk", block_size=16, stride=8):
     """Token-level top-k decode on the paged cache: per sequence the cache is
     read back into LiteSys' contiguous form (token t = cache slot t +
-    first_page_offset) and litesys_decode(policy "topk") does the rest.
+    first_page_offset) and litesys_decode (``policy`` "topk" or "strided") does
+    the rest.
     Returns (out [B, Hq, D] float64, keep list[b] of bool [Hkv, seq_len],
     mean_logits list[b] of float64 [Hkv, seq_len])."""
     B, Hq, D = q.shape
@@ -431,8 +469,8 @@ def token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, top
             continue
         K = bf16_to_f32(kv_cache[pages, 0]).reshape(len(pages) * ps, -1, D)[first_page_offset:kv_len]
         V = bf16_to_f32(kv_cache[pages, 1]).reshape(len(pages) * ps, -1, D)[first_page_offset:kv_len]
-        o, keep, mean = litesys_decode(qf[b], K, V, topk, local, sink=sink, sm_scale=sm_scale, policy="topk",
-                                       return_mean_logits=True)
+        o, keep, mean = litesys_decode(qf[b], K, V, topk, local, sink=sink, sm_scale=sm_scale, policy=policy,
+                                       block_size=block_size, stride=stride, return_mean_logits=True)
         out[b] = o
         keeps.append(keep)
         means.append(mean)
@@ -440,13 +478,14 @@ def token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, top
 
 
 def litesys_decode(q, K, V, topk_block, local, sink=4, block_size=16, sm_scale=None, policy="block",
-                   return_mean_logits=False, keep=None):
+                   return_mean_logits=False, keep=None, stride=8):
     """One sequence of LiteSys' sparse decode on its contiguous cache
     (LiteSys/litesys/attention/batch_cache.py:154-168): logits of every token
     (cache_utils.py:54-93, scale 1/sqrt(D)), the sparsity policy per KV head on
     the group-mean logits -- blockwise_topk_sparsity (sparsity_utils.py:24-47,
-    ``policy="block"``) or topk_sparsity (:6-21, ``policy="topk"``, where
-    ``topk_block`` counts tokens) --, softmax over what stays
+    ``policy="block"``), topk_sparsity (:6-21, ``policy="topk"``, where
+    ``topk_block`` counts tokens) or strided_blockwise_topk_sparsity (:49-105,
+    ``policy="strided"``) --, softmax over what stays
     (cache_utils.py:216-226), P.V (cache_utils.py:97-169).  q [Hq, D], K / V
     [seq_len, Hkv, D] float (the new token included).  ``topk_block=None`` is the
     dense layer.  ``keep`` [Hkv, seq_len] overrides the policy's choice (to
@@ -469,6 +508,8 @@ def litesys_decode(q, K, V, topk_block, local, sink=4, block_size=16, sm_scale=N
             keep_all[h] = keep[h]
         elif topk_block is not None and policy == "block":
             keep_all[h] = litesys_blockwise_topk_mask(mean_all[h], seq_len, topk_block, local, sink, block_size)
+        elif topk_block is not None and policy == "strided":
+            keep_all[h] = litesys_strided_mask(mean_all[h], seq_len, topk_block, local, sink, block_size, stride)
         elif topk_block is not None:
             keep_all[h] = litesys_topk_mask(mean_all[h], seq_len, topk_block, local, sink)
         masked = np.where(keep_all[h][None, :], logits, -np.inf)

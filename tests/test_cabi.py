@@ -169,6 +169,21 @@ def test_token_topk_argument_errors(lib):
     assert tok(B=0) == _lib.KIN_OK
 
 
+def test_strided_topk_argument_errors(lib):
+    def strided(topk=2, block=16, stride=8, sel=None, cnt=None, wsb=1 << 20, B=2, mp=4, sel_stride=0):
+        return lib.kin_strided_topk_decode(A, A, A, A, A, topk, block, stride, 4, 1, 0, sel, cnt, A, None, A, wsb, B, 4, 1,
+                                           128, 16, 8, mp, sel_stride, 0.0, None)
+
+    assert strided(block=0) == _lib.KIN_ERR_BAD_SHAPE
+    assert strided(block=65) == _lib.KIN_ERR_BAD_SHAPE
+    assert strided(stride=0) == _lib.KIN_ERR_BAD_SHAPE
+    assert strided(topk=300) == _lib.KIN_ERR_UNSUPPORTED              # 300 * 16 tokens > 4096
+    assert strided(sel=A, cnt=A, sel_stride=36) == _lib.KIN_ERR_BAD_SHAPE   # 2 * 16 + 4 + 1 entries needed
+    assert lib.kin_strided_topk_workspace_bytes(2, 1, 4) == 2 * 2 * 4 * 16 * 4
+    assert strided(wsb=2 * 2 * 4 * 16 * 4 - 1) == _lib.KIN_ERR_WORKSPACE
+    assert strided(B=0) == _lib.KIN_OK
+
+
 def test_sel_list_capacity(lib):
     assert lib.kin_sel_list_capacity(128, 0, 1) == 129               # the reference's k + 1
     assert lib.kin_sel_list_capacity(64, 1, 16) == 64 + 1 + 2

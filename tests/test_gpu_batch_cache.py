@@ -32,7 +32,9 @@ def test_rejects_what_it_does_not_implement():
 
     cfg = SimpleNamespace(num_attention_heads=4, num_key_value_heads=2, head_dim=D, hidden_size=512, num_hidden_layers=1)
     with pytest.raises(NotImplementedError):
-        PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_stride=8, attn_block_topk=2, attn_local=4)
+        PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_random_select=8, attn_local=4)
+    with pytest.raises(NotImplementedError):
+        PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_stride=8, attn_local=4)
     with pytest.raises(AssertionError):
         PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_topk=8, attn_block_topk=2, attn_local=4)
     with pytest.raises(AssertionError):
@@ -45,7 +47,9 @@ def test_rejects_what_it_does_not_implement():
                                           (dict(attn_block_topk=3, attn_local=16), False),
                                           (dict(attn_block_topk=2, attn_local=21), True),
                                           (dict(attn_local=24), False),
-                                          (dict(attn_topk=40, attn_local=10), None)])
+                                          (dict(attn_topk=40, attn_local=10), None),
+                                          (dict(attn_block_topk=2, attn_local=9, attn_stride=8), None),
+                                          (dict(attn_block_topk=3, attn_local=5, attn_stride=4, attn_block_size=8), None)])
 def test_prefill_then_decode_like_litesys(sparse, fused):
     torch.manual_seed(5)
     m = make_manager(**sparse)
@@ -54,7 +58,10 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
     L, Hq, Hkv = 2, 4, 2
     hist = {}  # (layer, slot) -> (K [t, Hkv, D], V) float32 of the bf16 values fed so far
 
-    token_policy = "attn_topk" in sparse
+    strided = "attn_stride" in sparse
+    token_policy = "attn_topk" in sparse or strided
+    policy = "strided" if strided else ("topk" if token_policy else "block")
+    block_size, stride = sparse.get("attn_block_size", 16), sparse.get("attn_stride", 8)
     pad = 12 if sparse and not token_policy else 0
     topk_block, local = sparse.get("attn_block_topk", sparse.get("attn_topk", 0)), sparse.get("attn_local")
     gen = torch.Generator().manual_seed(11)
@@ -134,8 +141,9 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
             is_sparse = bool(sparse) and layer not in (0,)   # layer 0 stays dense (attn_layer_skip default)
             if is_sparse and token_policy:
                 O.append_paged_kv(kf, vf, kv_before, None, idx, indptr, last)
-                want, keeps, _ = O.token_topk_decode(qf, kv_before, idx, indptr, last, topk_block, sink=4, local=local)
-                assert not keeps[batch_slots[0]].all() or lens[batch_slots[0]] <= 4 + topk_block + local
+                want, keeps, _ = O.token_topk_decode(qf, kv_before, idx, indptr, last, topk_block, sink=4, local=local,
+                                                     policy=policy, block_size=block_size, stride=stride)
+                assert strided or not keeps[batch_slots[0]].all() or lens[batch_slots[0]] <= 4 + topk_block + local
             elif is_sparse:
                 # the paged oracle on the manager's own state: one sink page, `local` newest tokens, 12 padding slots
                 res = O.decode_step(qf, kf, vf, kv_before, kbar_before, idx, indptr, last, topk_block,
@@ -157,8 +165,8 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
             for i, slot in enumerate(batch_slots):
                 K, V = hist[(layer, slot)]
                 ref, keep = O.litesys_decode(q[i, :, 0].float().cpu().numpy(), K.numpy(), V.numpy(),
-                                             topk_block if is_sparse else None, local,
-                                             policy="topk" if token_policy else "block")
+                                             topk_block if is_sparse else None, local, policy=policy,
+                                             block_size=block_size, stride=stride)
                 if is_sparse and K.shape[0] > 100:
                     assert not keep.all()
                 assert np.all(np.abs(got[i] - ref) <= 2e-2 + 2e-2 * np.abs(ref)), (layer, slot)

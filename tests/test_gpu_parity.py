@@ -852,6 +852,78 @@ def test_token_topk_decode(ops, case):
         assert np.allclose(lse, want_lse, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("case", ["mixed", "hkv8_stride4", "g8", "many", "offset", "stride16", "block8_stride3"])
+def test_strided_topk_decode(ops, case):
+    """LiteSys' strided overlapping-block policy (sparsity_utils.py:49-105)."""
+    block, stride, offset = 16, 8, 0
+    if case == "mixed":
+        pb = P.make_problem(1500, [PS * 40 + 3, PS * 9, 1, 0, PS * 3 + 1, PS * 130 + 16, 17, 5, 23, 24], num_kv_heads=1, group=4)
+        topk, sink, local = 4, 4, 16
+    elif case == "hkv8_stride4":
+        pb = P.make_problem(1501, [PS * 70 + 5, PS * 20 + 16, 0, 5], num_kv_heads=8, group=2, table="fragmented")
+        topk, sink, local, stride = 6, 4, 7, 4
+    elif case == "g8":
+        pb = P.make_problem(1502, [PS * 300 + 9] * 3, num_kv_heads=1, group=8, table="strided")
+        topk, sink, local = 64, 4, 64
+    elif case == "many":     # > 512 lists: 4 waves per list
+        rng = np.random.default_rng(1503)
+        pb = P.make_problem(1503, [int(x) for x in rng.integers(1, PS * 30, size=600)], num_kv_heads=1, group=3)
+        topk, sink, local = 3, 4, 8
+    elif case == "offset":
+        pb = P.make_problem(1504, [PS * 25 + 2, PS * 2, 13, 12, 30], num_kv_heads=2, group=4)
+        topk, sink, local, offset = 2, 4, 10, 12
+    elif case == "stride16":  # disjoint blocks
+        pb = P.make_problem(1505, [PS * 50 + 7, PS * 4], num_kv_heads=1, group=4)
+        topk, sink, local, stride = 5, 4, 3, 16
+    else:
+        pb = P.make_problem(1506, [PS * 33 + 1, 40, 19], num_kv_heads=2, group=1)
+        topk, sink, local, block, stride = 9, 2, 5, 8, 3
+    what = f"strided {case}"
+    g = Gpu(pb)
+    ops.append_paged_kv(g.k, g.v, g.kv, None, g.indices, g.indptr, g.last)
+    cap = max(topk, 1) * block + sink + local
+    sel = torch.full((pb.B, pb.Hkv, cap), -7, dtype=torch.int32, device=DEV)
+    cnt = torch.full((pb.B, pb.Hkv), -7, dtype=torch.int32, device=DEV)
+    lse = torch.full((pb.B, pb.Hq), float("nan"), dtype=torch.float32, device=DEV)
+    out = ops.strided_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, topk, max(pb.max_pages, 1), block_size=block,
+                                  stride=stride, sink_tokens=sink, local_tokens=local, first_page_offset=offset, lse=lse,
+                                  sel_tokens=sel, sel_count=cnt)
+    torch.cuda.synchronize()
+    kv = pb.kv_cache.copy()
+    O.append_paged_kv(pb.k, pb.v, kv, None, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    want, keeps, means = O.token_topk_decode(pb.q, kv, pb.page_indices, pb.page_indptr, pb.last_page_len, topk, sink=sink,
+                                             local=local, first_page_offset=offset, policy="strided", block_size=block,
+                                             stride=stride)
+    sel, cnt, got = sel.cpu().numpy(), cnt.cpu().numpy(), out.float().cpu().numpy()
+    qf = O.bf16_to_f32(pb.q).astype(np.float64)
+    sparse_rows = 0
+    for b in range(pb.B):
+        if keeps[b] is None:
+            assert (cnt[b] == 0).all() and (sel[b] == -1).all() and (got[b] == 0).all(), what
+            continue
+        S = keeps[b].shape[1]
+        pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+        K = O.bf16_to_f32(kv[pages, 0]).reshape(-1, pb.Hkv, D)[offset : offset + S]
+        V = O.bf16_to_f32(kv[pages, 1]).reshape(-1, pb.Hkv, D)[offset : offset + S]
+        got_keep = np.zeros((pb.Hkv, S), dtype=bool)
+        for h in range(pb.Hkv):
+            n = cnt[b, h]
+            row = sel[b, h]
+            assert n >= 0 and (row[n:] == -1).all() and np.all(np.diff(row[:n]) > 0), f"{what}: b={b} h={h}"
+            got_keep[h, row[:n]] = True
+            if not np.array_equal(got_keep[h], keeps[b][h]):
+                # only a near-tie between block means at the cut may change the choice
+                bm = np.sort(O.strided_block_means(means[b][h], S, local, sink, block, stride))[::-1]
+                kb = min(2 * topk, len(bm))
+                assert 0 < kb < len(bm) and abs(bm[kb - 1] - bm[kb]) <= 1e-3 * abs(bm[kb - 1]), f"{what}: b={b} h={h}"
+            sparse_rows += int(not keeps[b][h].all())
+        ref, _ = O.litesys_decode(qf[b], K, V, topk, local, sink=sink, keep=got_keep)
+        err = np.abs(got[b] - ref)
+        assert np.all(err <= 2e-2 + 2e-2 * np.abs(ref)), f"{what}: b={b} max err {err.max()}"
+    assert sparse_rows > 0
+    assert not np.isnan(lse.cpu().numpy()).any()
+
+
 def test_token_topk_rejects_short_workspace_and_long_sequences(ops):
     pb = P.make_problem(1310, [PS * 6 + 2, PS * 2], num_kv_heads=1, group=4)
     g = Gpu(pb)

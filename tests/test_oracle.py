@@ -574,3 +574,44 @@ def test_token_topk_decode_on_pages_is_litesys_on_the_contiguous_cache():
     dense_off, _ = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len,
                                         first_page_offset=7)
     assert np.allclose(off, dense_off, rtol=1e-10, atol=1e-12)
+
+
+def test_litesys_strided_mask():
+    """sparsity_utils.py:49-105 by hand, including its quirks: twice the budget in
+    blocks is chosen, the union is cut in POSITION order, and what no chosen block
+    covers is dropped."""
+    ml = np.zeros(17)
+    ml[4:14] = [0, 0, 5, 5, 5, 5, 0, 0, 9, 9]          # the dynamic part (sink 4, local 3)
+    ml[[0, 15]] = 50.0                                  # sink / local tokens are not candidates
+    keep = O.litesys_strided_mask(ml, 17, 1, 3, sink=4, block_size=4, stride=2)
+    # blocks [0,4) [2,6) [4,8) [6,10): means 2.5, 5, 2.5, 4.5 -> blocks 1 and 3 -> tokens 2..9 -> first 4: 2..5
+    want = np.zeros(17, dtype=bool)
+    want[:4] = True
+    want[14:] = True
+    want[4 + 2 : 4 + 6] = True
+    assert np.array_equal(keep, want)
+    assert np.allclose(O.strided_block_means(ml, 17, 3, sink=4, block_size=4, stride=2), [2.5, 5, 2.5, 4.5])
+    # budget of two blocks: all four blocks are chosen, the first 8 united tokens stay, 8 and 9 are cut
+    keep = O.litesys_strided_mask(ml, 17, 2, 3, sink=4, block_size=4, stride=2)
+    assert keep[4:12].all() and not keep[12:14].any()
+    # a tail no block reaches is dropped even with a huge budget: L = 11 -> still 4 blocks, token 10 uncovered
+    keep = O.litesys_strided_mask(np.append(ml, 0.0), 18, 100, 3, sink=4, block_size=4, stride=2)
+    assert keep[4:14].all() and not keep[14] and keep[15:].all()
+    # too short for a block, or nothing dynamic: nothing masked
+    assert O.litesys_strided_mask(ml, 10, 1, 3, sink=4, block_size=4, stride=2).all()
+    assert O.litesys_strided_mask(ml, 7, 1, 3, sink=4, block_size=4, stride=2).all()
+    # against a direct restatement with torch.topk on random data
+    rng = np.random.default_rng(5)
+    for seq_len, k, local, bs, st in [(500, 8, 16, 16, 8), (333, 5, 7, 16, 4), (2000, 30, 64, 16, 16), (90, 2, 1, 8, 3)]:
+        ml = rng.standard_normal(seq_len)
+        dyn = torch.from_numpy(ml[4 : seq_len - local])
+        nb = (len(dyn) - bs) // st + 1
+        means = dyn.unfold(0, bs, st).mean(dim=-1)
+        assert means.shape[0] == nb
+        top = torch.topk(means, min(2 * k, nb)).indices
+        toks = torch.unique(torch.cat([torch.arange(i * st, i * st + bs) for i in top.tolist()]))[: k * bs]
+        want = np.zeros(seq_len, dtype=bool)
+        want[:4] = True
+        want[seq_len - local :] = True
+        want[4 + toks.numpy()] = True
+        assert np.array_equal(O.litesys_strided_mask(ml, seq_len, k, local, 4, bs, st), want)
