@@ -19,11 +19,11 @@ Supported configurations (anything else raises at construction):
   * ``attn_block_topk=k, attn_stride=s``        -> overlapping blocks every s tokens
                                                   (strided_blockwise_topk_sparsity,
                                                   sparsity_utils.py:49-105), also one launch
-  * ``attn_local`` alone                        -> sink + local window only: block top-k with
-                                                  k = 0, whose window is LiteSys' ``local``
-                                                  rounded up to the block grid (a superset, by
-                                                  at most 15 tokens, of local_sparsity,
-                                                  sparsity_utils.py:107-114)
+  * ``attn_local`` alone                        -> the 4 sink tokens and the newest attn_local
+                                                  tokens only (local_sparsity,
+                                                  sparsity_utils.py:107-114): the token-level
+                                                  kernel with a budget of 0, which reads no key
+                                                  outside that window
 LiteSys always attends 4 hard-wired "sink" tokens, starts its 16-token blocks
 right after them and always attends the ``_local`` newest tokens that remain
 after the last whole block (sparsity_utils.py:24-35,240).  To keep that exact
@@ -102,11 +102,13 @@ class PagedBatchKVManager:
                 raise NotImplementedError("block size must equal the page size (16)")
         elif kwargs.get("attn_stride") is not None:
             raise NotImplementedError("attn_stride needs attn_block_topk")
-        self.sparse = kwargs.get("attn_local") is not None and self.token_topk is None and self.strided is None
+        if kwargs.get("attn_local") is not None and self.block_topk is None and self.strided is None and self.token_topk is None:
+            self.token_topk = 0      # window only (local_sparsity, sparsity_utils.py:107-114): 4 sink + attn_local tokens
+            if not 0 <= int(kwargs["attn_local"]) <= 1024:
+                raise NotImplementedError("attn_local must be in [0, 1024]")
+        self.sparse = self.block_topk is not None
         if self.token_topk is not None:
             self.token_local = int(kwargs["attn_local"])
-        if self.sparse and self.block_topk is None:
-            self.block_topk = 0                      # sink + local window only
         self.layer_skip = list(kwargs.get("attn_layer_skip", [0]))
         self.sink_pages = 1 if self.sparse else 0
         self.local_tokens = int(kwargs["attn_local"]) if self.sparse else 1

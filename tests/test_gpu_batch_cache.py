@@ -59,7 +59,8 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
     hist = {}  # (layer, slot) -> (K [t, Hkv, D], V) float32 of the bf16 values fed so far
 
     strided = "attn_stride" in sparse
-    token_policy = "attn_topk" in sparse or strided
+    window_only = bool(sparse) and "attn_block_topk" not in sparse and "attn_topk" not in sparse
+    token_policy = "attn_topk" in sparse or strided or window_only
     policy = "strided" if strided else ("topk" if token_policy else "block")
     block_size, stride = sparse.get("attn_block_size", 16), sparse.get("attn_stride", 8)
     pad = 12 if sparse and not token_policy else 0
