@@ -942,19 +942,40 @@ def test_token_topk_rejects_short_workspace_and_long_sequences(ops):
 # --------------------------------------------------------------------------- graph capture / tracing
 
 
-def test_step_replays_under_hip_graph(ops):
-    """No allocation, no host sync, fixed buffers: the three launches can be
+@pytest.mark.parametrize("path", ["three", "fused", "fused_split", "token", "strided"])
+def test_step_replays_under_hip_graph(ops, path):
+    """No allocation, no host sync, fixed buffers: every launch sequence can be
     captured once and replayed.  Every replay (with eager work and syncs in
     between) must equal the eager result for the inputs current at replay time."""
-    pb = P.make_problem(800, [PS * 200 + 3] * 64, num_kv_heads=2, group=4, topk=32)
+    if path == "fused_split":   # few long sequences: fill kernel + several workgroups per list
+        pb = P.make_problem(801, [PS * 2300 + 3, PS * 2100 + 9], num_kv_heads=1, group=4, topk=32)
+    else:
+        pb = P.make_problem(800, [PS * 200 + 3] * 64, num_kv_heads=2, group=4, topk=32)
     g = Gpu(pb)
     out = torch.empty_like(g.q)
     ws = workspace(ops, pb, pb.topk + 1, 0)
+    step_ws = torch.empty(max(16, ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[1])), dtype=torch.uint8, device=DEV)
+    tok_ws = torch.empty(max(16, ops.strided_topk_workspace_bytes(pb.B, pb.Hkv, pb.max_pages)), dtype=torch.uint8, device=DEV)
+    tok_sel = torch.full((pb.B, pb.Hkv, 64 * 16 + 4 + 16), -1, dtype=torch.int32, device=DEV)
+    assert (path == "fused_split") == (ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[1]) > 0)
 
     def step():
-        ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
-        ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, pb.topk, g.sel, g.cnt)
-        ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, out=out, workspace=ws)
+        if path == "three":
+            ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
+            ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, pb.topk, g.sel, g.cnt)
+            ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, out=out, workspace=ws)
+        elif path in ("fused", "fused_split"):
+            ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, pb.topk, out=out,
+                                      sel_pages=g.sel, sel_count=g.cnt, workspace=step_ws)
+        else:
+            ops.append_paged_kv(g.k, g.v, g.kv, None, g.indices, g.indptr, g.last)
+            if path == "token":
+                ops.token_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, 300, pb.max_pages, local_tokens=16, out=out,
+                                      sel_tokens=tok_sel, sel_count=g.cnt, workspace=tok_ws)
+            else:
+                ops.strided_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, 20, pb.max_pages, local_tokens=16, out=out,
+                                        sel_tokens=tok_sel, sel_count=g.cnt, workspace=tok_ws)
+            g.sel.copy_(tok_sel[:, :, : g.sel.shape[2]])
 
     step()
     torch.cuda.synchronize()
