@@ -1,0 +1,62 @@
+// Device-side building block: one wave appends one token's K and V rows for one
+// (sequence, KV head) and refreshes the mean key of the page when the row fills
+// it.  Shared by the stand-alone append kernel and the fused decode step.
+#pragma once
+
+#include "kin_common.h"
+
+namespace kin {
+
+// Mean of the kPageSize key rows of one page for one head, for this lane's
+// two columns.  `krow` points at slot 0 of the page's K plane for that head
+// (in dwords); `row_stride` is in dwords.  Sum order is slot 0,1,...,15.
+__device__ __forceinline__ uint32_t page_mean_dword(const uint32_t* krow, int row_stride, int lane) {
+  float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+  for (int t = 0; t < kPageSize; ++t) {
+    const uint32_t w = krow[(int64_t)t * row_stride + lane];
+    s0 += bf16_lo(w);
+    s1 += bf16_hi(w);
+  }
+  const float inv = 1.0f / kPageSize;
+  return f32_to_bf16(s0 * inv) | (f32_to_bf16(s1 * inv) << 16);
+}
+
+// Run by the 64 lanes of one wave (lane = 0..63, 4 bytes each = one 256-byte row).
+// k_row / v_row: the new token's rows for this (sequence, head), in dwords.
+// The row lands in slot last_len-1 of the sequence's last page (physical id
+// last_pid).  If that fills the page and the page has a slot in kbar
+// (n_pages-1 < kbar_pages, kbar may be null), its mean key goes to
+// kbar_page_row, the dword address of kbar[b, n_pages-1, h, 0]: rows 0..14 are
+// read from the cache, row 15 is taken from the register, so the result does not
+// depend on store visibility.  Metadata outside its contract would write
+// outside the cache: the row is skipped.
+__device__ __forceinline__ void append_token_row(const uint32_t* k_row, const uint32_t* v_row, uint32_t* kv_cache,
+                                                 uint32_t* kbar_page_row, int64_t last_pid, int last_len, int n_pages,
+                                                 int kbar_pages, int h, int num_kv_heads, int64_t num_pages, int lane) {
+  const int pos = last_len - 1;
+  if (pos < 0 || pos >= kPageSize || last_pid < 0 || last_pid >= num_pages) return;
+  const int row_stride = num_kv_heads * (kHeadDim / 2);      // dwords per token row
+  const int64_t page_dwords = 2LL * kPageSize * row_stride;  // K plane + V plane
+  uint32_t* kplane = kv_cache + last_pid * page_dwords + h * (kHeadDim / 2);
+  uint32_t* vplane = kplane + (int64_t)kPageSize * row_stride;
+  const uint32_t kw = k_row[lane];
+  const uint32_t vw = v_row[lane];
+  kplane[(int64_t)pos * row_stride + lane] = kw;
+  vplane[(int64_t)pos * row_stride + lane] = vw;
+  if (kbar_page_row != nullptr && pos == kPageSize - 1 && n_pages - 1 < kbar_pages) {
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int t = 0; t < kPageSize - 1; ++t) {
+      const uint32_t w = kplane[(int64_t)t * row_stride + lane];
+      s0 += bf16_lo(w);
+      s1 += bf16_hi(w);
+    }
+    s0 += bf16_lo(kw);
+    s1 += bf16_hi(kw);
+    const float inv = 1.0f / kPageSize;
+    kbar_page_row[lane] = f32_to_bf16(s0 * inv) | (f32_to_bf16(s1 * inv) << 16);
+  }
+}
+
+}  // namespace kin

@@ -1,7 +1,7 @@
 // Paged KV append with per-page mean-key maintenance, and the bulk mean-key
 // builder.  Both are byte movers: one 64-lane wave moves one 256-byte head row
 // per instruction (4 bytes per lane), so every access is a full-row burst.
-#include "kin_common.h"
+#include "kin_append.h"
 
 namespace kin {
 
@@ -17,21 +17,6 @@ struct AppendParams {
   int64_t num_pages;
 };
 
-// Mean of the kPageSize key rows of one page for one head, for this lane's
-// two columns.  `krow` points at slot 0 of the page's K plane for that head
-// (in dwords); `row_stride` is in dwords.  Sum order is slot 0,1,...,15.
-__device__ __forceinline__ uint32_t page_mean_dword(const uint32_t* krow, int row_stride, int lane) {
-  float s0 = 0.f, s1 = 0.f;
-#pragma unroll
-  for (int t = 0; t < kPageSize; ++t) {
-    const uint32_t w = krow[(int64_t)t * row_stride + lane];
-    s0 += bf16_lo(w);
-    s1 += bf16_hi(w);
-  }
-  const float inv = 1.0f / kPageSize;
-  return f32_to_bf16(s0 * inv) | (f32_to_bf16(s1 * inv) << 16);
-}
-
 // grid = ceil(batch*Hkv / 4) blocks of 256 threads; one wave per (sequence, head).
 __global__ __launch_bounds__(256) void append_kernel(AppendParams p) {
   const int lane = threadIdx.x & 63;
@@ -41,38 +26,10 @@ __global__ __launch_bounds__(256) void append_kernel(AppendParams p) {
   const int s = p.page_indptr[b], e = p.page_indptr[b + 1];
   const int n_pages = e - s;
   if (n_pages <= 0) return;
-  const int pos = p.last_page_len[b] - 1;
-  const int64_t pid = p.page_indices[e - 1];
-  // Metadata outside its contract would write outside the cache: skip the row.
-  if (pos < 0 || pos >= kPageSize || pid < 0 || pid >= p.num_pages) return;
-
-  const int row_stride = p.num_kv_heads * (kHeadDim / 2);           // dwords per token row
-  const int64_t page_dwords = 2LL * kPageSize * row_stride;          // K plane + V plane
-  uint32_t* kplane = p.kv_cache + pid * page_dwords + h * (kHeadDim / 2);
-  uint32_t* vplane = kplane + (int64_t)kPageSize * row_stride;
-  const int64_t src = (int64_t)item * (kHeadDim / 2) + lane;
-  const uint32_t kw = p.k[src];
-  const uint32_t vw = p.v[src];
-  kplane[(int64_t)pos * row_stride + lane] = kw;
-  vplane[(int64_t)pos * row_stride + lane] = vw;
-
-  if (p.kbar != nullptr && pos == kPageSize - 1 && n_pages - 1 < p.kbar_pages) {
-    // The page is now full.  Rows 0..14 come from the cache, row 15 is the one
-    // just written (taken from the register so the result does not depend on
-    // store visibility).
-    float s0 = 0.f, s1 = 0.f;
-#pragma unroll
-    for (int t = 0; t < kPageSize - 1; ++t) {
-      const uint32_t w = kplane[(int64_t)t * row_stride + lane];
-      s0 += bf16_lo(w);
-      s1 += bf16_hi(w);
-    }
-    s0 += bf16_lo(kw);
-    s1 += bf16_hi(kw);
-    const float inv = 1.0f / kPageSize;
-    const uint32_t m = f32_to_bf16(s0 * inv) | (f32_to_bf16(s1 * inv) << 16);
-    p.kbar[(((int64_t)b * p.kbar_pages + (n_pages - 1)) * p.num_kv_heads + h) * (kHeadDim / 2) + lane] = m;
-  }
+  uint32_t* kbar_row = p.kbar ? p.kbar + (((int64_t)b * p.kbar_pages + (n_pages - 1)) * p.num_kv_heads + h) * (kHeadDim / 2)
+                              : nullptr;
+  append_token_row(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2), p.kv_cache, kbar_row,
+                   p.page_indices[e - 1], p.last_page_len[b], n_pages, p.kbar_pages, h, p.num_kv_heads, p.num_pages, lane);
 }
 
 // grid = batch * Hkv * ceil(kbar_pages / 4) blocks (flat, so it is not bound by

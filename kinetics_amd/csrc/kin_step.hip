@@ -10,6 +10,7 @@
 // neighbours' streaming.  The selected page ids stay in LDS (HBM copies are
 // optional outputs).  Same building blocks and arithmetic as the stand-alone
 // kernels: score_select() (kin_select.h) and attend_list() (kin_attend.h).
+#include "kin_append.h"
 #include "kin_attend.h"
 #include "kin_select.h"
 
@@ -74,43 +75,20 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     return;
   }
   const int last_len = p.last_page_len[b];
-  const int row_dw = p.num_kv_heads * (kHeadDim / 2);  // dwords per token row
 
   // ---- append (wave 0): same byte moves and mean-key update as append_kernel ----
   // With split scoring the workgroup that ends up attending does it (see below).
   auto append_token = [&]() {
     if (p.k != nullptr && tid < 64) {
-      const int lane = tid;
-      const int pos = last_len - 1;
-      const int64_t pid = p.page_indices[pe - 1];
-      if (pos >= 0 && pos < kPageSize && pid >= 0 && pid < p.num_pages) {
-        uint32_t* kplane = reinterpret_cast<uint32_t*>(p.kv) + pid * (2LL * kPageSize * row_dw) + h * (kHeadDim / 2);
-        uint32_t* vplane = kplane + (int64_t)kPageSize * row_dw;
-        const int64_t src = (int64_t)item * (kHeadDim / 2) + lane;
-        const uint32_t kw = p.k[src], vw = p.v[src];
-        kplane[(int64_t)pos * row_dw + lane] = kw;
-        vplane[(int64_t)pos * row_dw + lane] = vw;
-        if (p.kbar != nullptr && pos == kPageSize - 1 && n_pages - 1 < p.kbar_pages) {
-          float s0 = 0.f, s1 = 0.f;
-#pragma unroll
-          for (int t = 0; t < kPageSize - 1; ++t) {
-            const uint32_t w = kplane[(int64_t)t * row_dw + lane];
-            s0 += bf16_lo(w);
-            s1 += bf16_hi(w);
-          }
-          s0 += bf16_lo(kw);
-          s1 += bf16_hi(kw);
-          const float inv = 1.0f / kPageSize;
-          reinterpret_cast<uint32_t*>(p.kbar)[(((int64_t)b * p.kbar_pages + (n_pages - 1)) * p.num_kv_heads + h) *
-                                                  (kHeadDim / 2) +
-                                              lane] = f32_to_bf16(s0 * inv) | (f32_to_bf16(s1 * inv) << 16);
-        }
-      }
+      uint32_t* kbar_row =
+          reinterpret_cast<uint32_t*>(p.kbar) + (((int64_t)b * p.kbar_pages + (n_pages - 1)) * p.num_kv_heads + h) * (kHeadDim / 2);
+      append_token_row(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2),
+                       reinterpret_cast<uint32_t*>(p.kv), kbar_row, p.page_indices[pe - 1], last_len, n_pages, p.kbar_pages, h,
+                       p.num_kv_heads, p.num_pages, tid);
       // The attention phase of this workgroup reads the row back: make the stores
       // visible before the barriers that separate the phases.
       __threadfence_block();
     }
-
   };
   if (p.chunks <= 1) append_token();
 
