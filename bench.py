@@ -392,6 +392,25 @@ def main():
         if os.path.exists(tpath):
             with open(tpath) as f:
                 result["token_topk"]["traffic"] = json.load(f).get(f"{args.workload}:B={B}", {}).get("token_topk_kernel")
+        # strided overlapping blocks with the same budget: topk blocks of 16 tokens, a block every 8 tokens
+        ws_str = torch.empty(max(16, ops.strided_topk_workspace_bytes(B, Hkv, st["max_pages_used"])), dtype=torch.uint8,
+                             device=device)
+        for _ in range(2):
+            ops.strided_topk_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], topk, st["max_pages_used"],
+                                    sink_tokens=sink, local_tokens=window, out=st["out"], workspace=ws_str)
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nt)]
+        for e0, e1 in evs:
+            e0.record()
+            ops.strided_topk_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], topk, st["max_pages_used"],
+                                    sink_tokens=sink, local_tokens=window, out=st["out"], workspace=ws_str)
+            e1.record()
+        torch.cuda.synchronize()
+        ts = statistics.fmean(e0.elapsed_time(e1) for e0, e1 in evs) * 1e-3
+        result["strided_topk"] = {"topk_blocks": topk, "block_size": PS, "stride": 8, "sink_tokens": sink,
+                                  "local_tokens": window, "kernel_ms": ts * 1e3, "algorithmic_bytes_per_step": tok_bytes,
+                                  "achieved_gbs": tok_bytes / ts / 1e9, "frac": tok_bytes / ts / 1e9 / HBM_PEAK_GBS}
+        del ws_str
         del ws_tok
     del st
     torch.cuda.empty_cache()
