@@ -137,9 +137,16 @@ struct AttendArgs {
   int first_skip;        // leading token slots of list entry 0 that hold no token (0..15)
 };
 
-constexpr int kAttendLdsBytes = 32768;  // 4 waves x 2 stages x 4 KiB; reused for the merge
-// K staging for NW waves, also large enough for the merge buffer [NW][4*NG][128] fp32 (NG <= 2).
-constexpr int attend_lds_bytes(int nw) { return nw * 8192; }
+// K pages a wave keeps staged in LDS in attend_list(): the one being read and 1 or
+// 2 in flight.  The two-pass kernel for groups above 4 runs only 2 waves per SIMD
+// (200 registers), so it keeps one more page (and one more V register set) in
+// flight per wave to cover the memory latency.
+constexpr int attend_k_stages(int ng) { return ng == 1 ? 2 : 3; }
+// K staging for NW waves of `stages` 4 KiB stages each; also large enough for the
+// merge buffer [NW][4*NG][128] fp32 (NG <= 2).
+constexpr int attend_lds_bytes(int nw, int stages = 2) { return nw * stages * 4096; }
+// s_waitcnt immediate for "vmcnt <= 16" (vmcnt[3:0] = 0, vmcnt_hi[15:14] = 1).
+constexpr int kWaitVm16 = 0 | (7 << 4) | (15 << 8) | (1 << 14);
 
 // Common tail of the attention loops: merges the wave's 4 row groups, then the
 // workgroup's NW waves through LDS, and hands out the normalised results.
@@ -222,7 +229,8 @@ __device__ __forceinline__ void attend_finish(float (&m_run)[NG], float (&l_run)
 // id_at(i) returns the (wave-uniform) physical page id of list entry i, 0 <= i < n.
 // emit(g, d, o, lse2) receives, once per (head g < G, column d), the normalised
 // output and the base-2 log-sum-exp (-inf and o = 0 for an empty part).
-// lds: attend_lds_bytes(NW), 16-byte aligned; sm_m / sm_l: NW x (4*NG) floats each.
+// lds: attend_lds_bytes(NW, attend_k_stages(NG)), 16-byte aligned; sm_m / sm_l: NW x
+// (4*NG) floats each.
 // Every one of the workgroup's NW*64 threads calls this.
 template <int NG, int NW, typename IdAt, typename Emit>
 __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, unsigned char* lds,
@@ -251,11 +259,12 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
   int voff[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c) voff[c] = (kPageSize + 4 * kg + c) * row_bytes + c16 * 16;
-  // K staging: two 4 KiB stages per wave, filled by LDS-direct buffer loads
+  // K staging: KS 4 KiB stages per wave, filled by LDS-direct buffer loads
   // (no VGPRs while in flight).  Load c brings rows 4c..4c+3: lane (kg, c16)
   // lands at LDS row 4c+kg, position c16, and fetches the chunk that belongs
   // there under the XOR swizzle (position p of row R holds chunk p ^ R).
-  unsigned char* kl = lds + w * (2 * 4096);
+  constexpr int KS = attend_k_stages(NG);
+  unsigned char* kl = lds + w * (KS * 4096);
   int kdma_off[4], lds_r[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
@@ -319,6 +328,57 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
   // before it are allowed to be outstanding, which means the K stage about to
   // be read (and the V registers about to be used) have landed.  The scheduling
   // fences keep the instruction order this count relies on.
+  if constexpr (KS == 3) {
+    // Three stages: K runs three pages ahead of the one being read, V two.  Issue
+    // order in steady state is ... V(p+1), K(p+2), V(p+2) | wait | read K(p), scores,
+    // K(p+3) ..., so at the wait the loads allowed to be outstanding are K and V of
+    // pages p+1 and p+2: 16 of them; everything older (page p) has landed.  (The
+    // compiler, which sees the LDS reads, tightens this wait to "every LDS-direct
+    // load issued so far", i.e. vmcnt(4); hiding the reads from it in inline
+    // assembly restores vmcnt(16) but was not measurably faster.)
+    if (iters > 0 && n > 0) {
+      u32x4 v[3][4];
+      uint4 ka[4];
+      float pr[NG][4];
+      int valid[3];
+      __amdgpu_buffer_rsrc_t r_v;  // descriptor of the page whose V is issued next
+      {
+        const __amdgpu_buffer_rsrc_t r0 = page_rsrc(0, load_id(0), valid[0]);
+        issue_k(r0, 0);
+        issue_v(r0, v[0]);
+        const __amdgpu_buffer_rsrc_t r1 = page_rsrc(1, load_id(1), valid[1]);
+        issue_k(r1, 1);
+        issue_v(r1, v[1]);
+        r_v = page_rsrc(2, load_id(2), valid[2]);
+        issue_k(r_v, 2);
+      }
+      int id_next = load_id(3);
+      for (int it = 0; it < iters; it += 3) {
+#pragma unroll
+        for (int s3 = 0; s3 < 3; ++s3) {
+          const int cur_valid = valid[s3];
+          __builtin_amdgcn_sched_barrier(0);
+          issue_v(r_v, v[(s3 + 2) % 3]);
+          __builtin_amdgcn_sched_barrier(0);
+          __builtin_amdgcn_s_waitcnt(kWaitVm16);
+          __builtin_amdgcn_sched_barrier(0);
+          read_k(s3, ka);
+          __builtin_amdgcn_sched_barrier(0);
+          page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, cur_valid >> 8, cur_valid & 255, kg);
+          __builtin_amdgcn_sched_barrier(0);
+          // The stage just read is refilled only now that the matrix unit has consumed
+          // it: a load through an empty descriptor (a masked page) returns at once
+          // and would otherwise overtake LDS reads that are still queued.
+          r_v = page_rsrc(it + s3 + 3, id_next, valid[s3]);
+          issue_k(r_v, s3);
+          __builtin_amdgcn_sched_barrier(0);
+          id_next = load_id(it + s3 + 4);  // lands while the P V products run
+          if (cur_valid != kPageSize) clear_unused_v_rows(v[s3], cur_valid >> 8, cur_valid & 255, kg);
+          page_pv<NG>(v[s3], pr, O);
+        }
+      }
+    }
+  } else
   if (iters > 0 && n > 0) {
     u32x4 vA[4], vB[4];
     uint4 ka[4];

@@ -27,7 +27,7 @@ struct DecodeParams {
 
 template <int NG>
 __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
-  __shared__ __attribute__((aligned(16))) unsigned char lds[kAttendLdsBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char lds[attend_lds_bytes(4, attend_k_stages(NG))];
   __shared__ float sm_m[4][4 * NG];
   __shared__ float sm_l[4][4 * NG];
 

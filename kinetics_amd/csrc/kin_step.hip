@@ -279,7 +279,8 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
     p.ws_keys = nullptr;
   }
   const size_t sel_scratch = select_lds_bytes(kbar_pages, p.sort_cap);
-  size_t region0 = sel_scratch > (size_t)attend_lds_bytes(nw) ? sel_scratch : (size_t)attend_lds_bytes(nw);
+  const size_t attend_bytes = (size_t)attend_lds_bytes(nw, attend_k_stages(p.group <= 4 ? 1 : 2));
+  size_t region0 = sel_scratch > attend_bytes ? sel_scratch : attend_bytes;
   region0 = (region0 + 15) & ~(size_t)15;
   p.region0_bytes = (int)region0;
   p.num_pages = num_pages;
