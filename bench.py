@@ -203,7 +203,7 @@ def whole_layer(torch, args, B, ctx, topk, device):
     dt = (time.perf_counter() - t0) / args.steps
     out = {"model": name, "world_size": world, "ms_per_layer_step": dt * 1e3, "tokens_per_s_per_layer": B / dt,
            "normalised_like_reference_print": B / dt / (world * cfg.num_hidden_layers),
-           "note": "norms and GEMMs are plain PyTorch (rocBLAS/hipBLASLt); only the attention path is this repository's kernels"}
+           "note": "GEMMs are hipBLASLt through PyTorch; norms, q/k/v split, attention and the gated activation are this repository's kernels"}
     del layer
     torch.cuda.empty_cache()
     return out

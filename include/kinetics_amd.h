@@ -394,6 +394,60 @@ int kin_check_page_table(const int32_t* page_indices, const int32_t* page_indptr
                          int64_t num_pages, int64_t nnz, int32_t* scratch,
                          kin_stream_t stream);
 
+/* ---- row-wise layer kernels around the attention path ---------------------
+ * The reference's decoder layer (benchmark/blocktopk_decoder.py:187-240) calls
+ * flashinfer's RMSNorm through its custom ops layer_norm and qk_norm
+ * (benchmark/model_utils.py:4-25) and leaves the residual adds, the q/k/v split
+ * and act(gate)*up to PyTorch.  These three entry points cover the same steps
+ * with one pass over the data each.  All tensors are bf16; statistics are fp32.
+ */
+
+/*
+ * RMSNorm over rows of `hidden` elements:
+ *   out[r, :] = bf16( x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight[:] )
+ * which is flashinfer.rmsnorm(x, weight, eps) as layer_norm and qk_norm call it
+ * (benchmark/model_utils.py:8,19).  With residual != NULL ([rows, hidden],
+ * contiguous) the add that precedes the norm in the layer
+ * (benchmark/blocktopk_decoder.py:229-232) is folded in, as
+ * flashinfer.fused_add_rmsnorm does it (benchmark/model_utils.py:27-41):
+ *   residual[r, :] = bf16(x[r, :] + residual[r, :]);  out = RMSNorm(residual)
+ * Row strides are in elements (multiples of 8, >= hidden); out may alias x.
+ * hidden: a multiple of 512 up to 8192, or a multiple of 128 up to 2048
+ * (head_dim 128 rows for qk_norm).
+ */
+int kin_rms_norm(const void* x, void* residual, const void* weight, void* out,
+                 int64_t rows, int hidden, int64_t x_row_stride, int64_t out_row_stride,
+                 float eps, kin_stream_t stream);
+
+/*
+ * The steps between the fused QKV projection and the attention path
+ * (benchmark/blocktopk_decoder.py:196-207): split qkv[b, :] =
+ * [num_q_heads*D | num_kv_heads*D | num_kv_heads*D] into heads, RMSNorm every q
+ * head with q_weight[D] and every k head with k_weight[D] (qk_norm,
+ * benchmark/model_utils.py:15-25), copy the v heads, and write contiguous
+ * q[batch, num_q_heads, D], k[batch, num_kv_heads, D], v[batch, num_kv_heads, D].
+ * qkv_row_stride in elements (multiple of 8).  head_dim must be 128.
+ */
+int kin_qkv_norm_split(const void* qkv, int64_t qkv_row_stride, const void* q_weight,
+                       const void* k_weight, float eps, void* q, void* k, void* v,
+                       int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                       kin_stream_t stream);
+
+#define KIN_ACT_SILU 0
+#define KIN_ACT_GELU 1 /* erf form */
+#define KIN_ACT_RELU 2
+
+/*
+ * out[r, :] = bf16( bf16(act(gate[r, :])) * up[r, :] ), the gated MLP product
+ * (benchmark/blocktopk_decoder.py:234-237) with the rounding of the two bf16
+ * tensor operations it replaces.  gate and up may be the two halves of one
+ * fused projection: row strides in elements (multiples of 8, >= inter); out is
+ * contiguous [rows, inter]; inter a multiple of 8.
+ */
+int kin_gated_act(const void* gate, const void* up, void* out, int64_t rows, int inter,
+                  int64_t gate_row_stride, int64_t up_row_stride, int act,
+                  kin_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -18,7 +18,7 @@ LIB_PATH = PKG_DIR / "libkinetics_amd.so"
 OBJ_DIR = PKG_DIR / "build"
 
 SOURCES = ["kin_api.hip", "kin_append.hip", "kin_score_topk.hip", "kin_decode.hip", "kin_step.hip", "kin_token_topk.hip",
-           "kin_table.hip"]
+           "kin_table.hip", "kin_layer.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -1,0 +1,311 @@
+// Row-wise kernels of a decoder layer on either side of the attention path:
+// RMSNorm with the residual add folded in, the q/k norm + split of the fused QKV
+// projection, and the gated activation of the MLP.  All are HBM-bound: every
+// element is read once and written once with 16-byte accesses, statistics are
+// taken in fp32 inside lane groups (no LDS), and each replaces a chain of
+// elementwise launches that would move the same rows through HBM several times.
+#include "kin_common.h"
+
+namespace kin {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte access: 8 bf16
+
+// 16-byte chunks one lane keeps in registers: a row of up to LPR * 8 * 16 elements.
+constexpr int kNormMaxChunks = 16;
+
+struct NormParams {
+  const u32x4* x;
+  u32x4* residual;      // [rows, hidden] contiguous, updated in place (RES only)
+  const u32x4* weight;  // [hidden]
+  u32x4* out;
+  int64_t rows;
+  int64_t x_stride, out_stride;  // row strides in 16-byte units
+  int chunks;                    // hidden / (LPR * 8)
+  float eps, inv_hidden;
+};
+
+__device__ __forceinline__ float sum_sq8(const u32x4& v) {
+  float s = 0.f;
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float a = bf16_lo(w[i]), b = bf16_hi(w[i]);
+    s = fmaf(a, a, s);
+    s = fmaf(b, b, s);
+  }
+  return s;
+}
+
+// bf16(a + b) per element, as a bf16 tensor add computes it.
+__device__ __forceinline__ uint32_t add_bf16x2(uint32_t a, uint32_t b) {
+  return f32_to_bf16(bf16_lo(a) + bf16_lo(b)) | (f32_to_bf16(bf16_hi(a) + bf16_hi(b)) << 16);
+}
+
+// bf16((x * r) * w) per element.
+__device__ __forceinline__ uint32_t scale_bf16x2(uint32_t x, float r, uint32_t w) {
+  return f32_to_bf16(bf16_lo(x) * r * bf16_lo(w)) | (f32_to_bf16(bf16_hi(x) * r * bf16_hi(w)) << 16);
+}
+
+template <int LPR>
+__device__ __forceinline__ float group_sum(float x) {
+  x = row16_sum(x);
+  if (LPR == 64) {
+    x += __shfl_xor(x, 16);
+    x += __shfl_xor(x, 32);
+  }
+  return x;
+}
+
+// LPR lanes (16 or 64) own one row; a 256-thread workgroup covers 256 / LPR rows.
+// Lane l holds the 16-byte chunks c * LPR + l, so every load instruction of a
+// lane group covers LPR * 16 contiguous bytes.  MAXC bounds the chunks per lane
+// (the row stays in registers between the two passes): the smaller
+// instantiations need fewer registers, so that a grid of a few thousand rows is
+// resident at once instead of running a nearly empty second round.
+template <int LPR, int MAXC, bool RES>
+__global__ __launch_bounds__(256) void rms_norm_kernel(NormParams p) {
+  const int sub = threadIdx.x / LPR, l = threadIdx.x % LPR;
+  const int64_t row = (int64_t)blockIdx.x * (256 / LPR) + sub;
+  if (row >= p.rows) return;  // whole lane groups leave together
+  const u32x4* xr = p.x + row * p.x_stride;
+  u32x4* rr = RES ? p.residual + row * ((int64_t)p.chunks * LPR) : nullptr;
+  u32x4 v[MAXC], r[RES ? MAXC : 1];
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    if (c < p.chunks) {
+      v[c] = __builtin_nontemporal_load(xr + c * LPR + l);
+      if (RES) r[c] = rr[c * LPR + l];
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    if (c < p.chunks) {
+      if (RES) {
+        v[c].x = add_bf16x2(v[c].x, r[c].x);
+        v[c].y = add_bf16x2(v[c].y, r[c].y);
+        v[c].z = add_bf16x2(v[c].z, r[c].z);
+        v[c].w = add_bf16x2(v[c].w, r[c].w);
+        rr[c * LPR + l] = v[c];
+      }
+      ss += sum_sq8(v[c]);
+    }
+  }
+  ss = group_sum<LPR>(ss);
+  const float rinv = rsqrtf(ss * p.inv_hidden + p.eps);
+  u32x4* orow = p.out + row * p.out_stride;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    if (c < p.chunks) {
+      const u32x4 w = p.weight[c * LPR + l];
+      u32x4 o;
+      o.x = scale_bf16x2(v[c].x, rinv, w.x);
+      o.y = scale_bf16x2(v[c].y, rinv, w.y);
+      o.z = scale_bf16x2(v[c].z, rinv, w.z);
+      o.w = scale_bf16x2(v[c].w, rinv, w.w);
+      orow[c * LPR + l] = o;
+    }
+  }
+}
+
+struct QkvParams {
+  const u32x4* qkv;
+  int64_t row_stride;  // 16-byte units
+  const u32x4 *q_weight, *k_weight;
+  u32x4 *q, *k, *v;
+  int batch, hq, hkv;
+  float eps;
+};
+
+// 16 lanes per head row of 128 elements: q and k heads are normalised, v heads
+// copied, each to its own contiguous [batch, heads, 128] tensor.
+__global__ __launch_bounds__(256) void qkv_norm_split_kernel(QkvParams p) {
+  const int heads = p.hq + 2 * p.hkv;
+  const int64_t g = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const int l = threadIdx.x & 15;
+  if (g >= (int64_t)p.batch * heads) return;
+  const int64_t b = g / heads;
+  const int j = (int)(g - b * heads);
+  u32x4 x = __builtin_nontemporal_load(p.qkv + b * p.row_stride + j * 16 + l);
+  u32x4* dst;
+  if (j < p.hq + p.hkv) {
+    const bool is_q = j < p.hq;
+    const float ss = row16_sum(sum_sq8(x));
+    const float rinv = rsqrtf(ss * (1.0f / kHeadDim) + p.eps);
+    const u32x4 w = (is_q ? p.q_weight : p.k_weight)[l];
+    x.x = scale_bf16x2(x.x, rinv, w.x);
+    x.y = scale_bf16x2(x.y, rinv, w.y);
+    x.z = scale_bf16x2(x.z, rinv, w.z);
+    x.w = scale_bf16x2(x.w, rinv, w.w);
+    dst = is_q ? p.q + (b * p.hq + j) * 16 : p.k + (b * p.hkv + (j - p.hq)) * 16;
+  } else {
+    dst = p.v + (b * p.hkv + (j - p.hq - p.hkv)) * 16;
+  }
+  dst[l] = x;
+}
+
+struct GateParams {
+  const u32x4 *gate, *up;
+  u32x4* out;
+  int64_t rows;
+  int64_t gate_stride, up_stride;  // 16-byte units
+  int row_chunks;                  // inter / 8
+};
+
+// Each activation is rounded to bf16 before the product, as the chain
+// act(gate) * up over bf16 tensors rounds it.
+template <int ACT>
+__device__ __forceinline__ float act_bf16(float x) {
+  float y;
+  if (ACT == KIN_ACT_SILU) y = x / (1.0f + expf(-x));
+  else if (ACT == KIN_ACT_GELU) y = 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+  else y = fmaxf(x, 0.f);
+  return __uint_as_float(f32_to_bf16(y) << 16);
+}
+
+template <int ACT>
+__device__ __forceinline__ uint32_t gate_bf16x2(uint32_t g, uint32_t u) {
+  return f32_to_bf16(act_bf16<ACT>(bf16_lo(g)) * bf16_lo(u)) | (f32_to_bf16(act_bf16<ACT>(bf16_hi(g)) * bf16_hi(u)) << 16);
+}
+
+template <int ACT>
+__global__ __launch_bounds__(256) void gated_act_kernel(GateParams p) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= p.rows * p.row_chunks) return;
+  const int64_t row = idx / p.row_chunks;
+  const int c = (int)(idx - row * p.row_chunks);
+  const u32x4 g = __builtin_nontemporal_load(p.gate + row * p.gate_stride + c);
+  const u32x4 u = __builtin_nontemporal_load(p.up + row * p.up_stride + c);
+  u32x4 o;
+  o.x = gate_bf16x2<ACT>(g.x, u.x);
+  o.y = gate_bf16x2<ACT>(g.y, u.y);
+  o.z = gate_bf16x2<ACT>(g.z, u.z);
+  o.w = gate_bf16x2<ACT>(g.w, u.w);
+  p.out[idx] = o;
+}
+
+static int check_row_stride(const char* fn, const char* name, int64_t stride, int width) {
+  if (stride < width || stride % 8 != 0)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: %s=%lld must be a multiple of 8 and at least the row width %d", fn, name,
+                (long long)stride, width);
+  return KIN_OK;
+}
+
+}  // namespace kin
+
+extern "C" int kin_rms_norm(const void* x, void* residual, const void* weight, void* out, int64_t rows, int hidden,
+                            int64_t x_row_stride, int64_t out_row_stride, float eps, kin_stream_t stream) {
+  using namespace kin;
+  const char* fn = "kin_rms_norm";
+  if (!x || !weight || !out) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
+  if (rows < 0 || hidden < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: rows=%lld hidden=%d", fn, (long long)rows, hidden);
+  int lpr;
+  if (hidden % 512 == 0 && hidden <= 512 * kNormMaxChunks) lpr = 64;
+  else if (hidden % 128 == 0 && hidden <= 128 * kNormMaxChunks) lpr = 16;
+  else
+    return fail(KIN_ERR_UNSUPPORTED, "%s: hidden=%d must be a multiple of 128 up to %d or of 512 up to %d", fn, hidden,
+                128 * kNormMaxChunks, 512 * kNormMaxChunks);
+  if (int st = check_row_stride(fn, "x_row_stride", x_row_stride, hidden)) return st;
+  if (int st = check_row_stride(fn, "out_row_stride", out_row_stride, hidden)) return st;
+  if (!aligned16(x) || !aligned16(weight) || !aligned16(out) || !aligned16(residual))
+    return fail(KIN_ERR_MISALIGNED, "%s: pointers must be 16-byte aligned", fn);
+  if (!(eps >= 0.f)) return fail(KIN_ERR_BAD_SHAPE, "%s: eps must be non-negative", fn);
+  const int rows_per_wg = 256 / lpr;
+  const int64_t grid = (rows + rows_per_wg - 1) / rows_per_wg;
+  if (grid > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: rows=%lld is too many", fn, (long long)rows);
+  if (rows == 0) return KIN_OK;
+  NormParams p;
+  p.x = static_cast<const u32x4*>(x);
+  p.residual = static_cast<u32x4*>(residual);
+  p.weight = static_cast<const u32x4*>(weight);
+  p.out = static_cast<u32x4*>(out);
+  p.rows = rows;
+  p.x_stride = x_row_stride / 8;
+  p.out_stride = out_row_stride / 8;
+  p.chunks = hidden / (lpr * 8);
+  p.eps = eps;
+  p.inv_hidden = 1.0f / (float)hidden;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const unsigned g = (unsigned)grid;
+#define KIN_NORM_LAUNCH(LPR, MAXC)                                            \
+  do {                                                                        \
+    if (residual) rms_norm_kernel<LPR, MAXC, true><<<g, 256, 0, s>>>(p);      \
+    else rms_norm_kernel<LPR, MAXC, false><<<g, 256, 0, s>>>(p);              \
+  } while (0)
+  if (lpr == 64) {
+    if (p.chunks <= 4) KIN_NORM_LAUNCH(64, 4);
+    else if (p.chunks <= 8) KIN_NORM_LAUNCH(64, 8);
+    else KIN_NORM_LAUNCH(64, 16);
+  } else {
+    if (p.chunks <= 1) KIN_NORM_LAUNCH(16, 1);
+    else if (p.chunks <= 4) KIN_NORM_LAUNCH(16, 4);
+    else KIN_NORM_LAUNCH(16, 16);
+  }
+#undef KIN_NORM_LAUNCH
+  return check_hip(hipGetLastError(), "rms_norm_kernel launch");
+}
+
+extern "C" int kin_qkv_norm_split(const void* qkv, int64_t qkv_row_stride, const void* q_weight, const void* k_weight,
+                                  float eps, void* q, void* k, void* v, int batch, int num_q_heads, int num_kv_heads,
+                                  int head_dim, kin_stream_t stream) {
+  using namespace kin;
+  const char* fn = "kin_qkv_norm_split";
+  if (!qkv || !q_weight || !k_weight || !q || !k || !v) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
+  if (batch < 0 || num_q_heads < 1 || num_kv_heads < 1)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: batch=%d num_q_heads=%d num_kv_heads=%d", fn, batch, num_q_heads, num_kv_heads);
+  if (head_dim != kHeadDim) return fail(KIN_ERR_UNSUPPORTED, "%s: head_dim=%d, only %d is built", fn, head_dim, kHeadDim);
+  const int64_t heads = (int64_t)num_q_heads + 2 * (int64_t)num_kv_heads;
+  if (heads * kHeadDim > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: too many heads", fn);
+  if (int st = check_row_stride(fn, "qkv_row_stride", qkv_row_stride, (int)(heads * kHeadDim))) return st;
+  if (!aligned16(qkv) || !aligned16(q_weight) || !aligned16(k_weight) || !aligned16(q) || !aligned16(k) || !aligned16(v))
+    return fail(KIN_ERR_MISALIGNED, "%s: pointers must be 16-byte aligned", fn);
+  if (!(eps >= 0.f)) return fail(KIN_ERR_BAD_SHAPE, "%s: eps must be non-negative", fn);
+  const int64_t grid = ((int64_t)batch * heads + 15) / 16;
+  if (grid > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*heads is too large", fn);
+  if (batch == 0) return KIN_OK;
+  QkvParams p;
+  p.qkv = static_cast<const u32x4*>(qkv);
+  p.row_stride = qkv_row_stride / 8;
+  p.q_weight = static_cast<const u32x4*>(q_weight);
+  p.k_weight = static_cast<const u32x4*>(k_weight);
+  p.q = static_cast<u32x4*>(q);
+  p.k = static_cast<u32x4*>(k);
+  p.v = static_cast<u32x4*>(v);
+  p.batch = batch;
+  p.hq = num_q_heads;
+  p.hkv = num_kv_heads;
+  p.eps = eps;
+  qkv_norm_split_kernel<<<(unsigned)grid, 256, 0, static_cast<hipStream_t>(stream)>>>(p);
+  return check_hip(hipGetLastError(), "qkv_norm_split_kernel launch");
+}
+
+extern "C" int kin_gated_act(const void* gate, const void* up, void* out, int64_t rows, int inter,
+                             int64_t gate_row_stride, int64_t up_row_stride, int act, kin_stream_t stream) {
+  using namespace kin;
+  const char* fn = "kin_gated_act";
+  if (!gate || !up || !out) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
+  if (rows < 0 || inter < 1 || inter % 8 != 0)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: rows=%lld inter=%d (inter must be a positive multiple of 8)", fn, (long long)rows, inter);
+  if (int st = check_row_stride(fn, "gate_row_stride", gate_row_stride, inter)) return st;
+  if (int st = check_row_stride(fn, "up_row_stride", up_row_stride, inter)) return st;
+  if (!aligned16(gate) || !aligned16(up) || !aligned16(out))
+    return fail(KIN_ERR_MISALIGNED, "%s: pointers must be 16-byte aligned", fn);
+  if (act != KIN_ACT_SILU && act != KIN_ACT_GELU && act != KIN_ACT_RELU)
+    return fail(KIN_ERR_UNSUPPORTED, "%s: act=%d is not one of KIN_ACT_SILU/GELU/RELU", fn, act);
+  GateParams p;
+  p.gate = static_cast<const u32x4*>(gate);
+  p.up = static_cast<const u32x4*>(up);
+  p.out = static_cast<u32x4*>(out);
+  p.rows = rows;
+  p.gate_stride = gate_row_stride / 8;
+  p.up_stride = up_row_stride / 8;
+  p.row_chunks = inter / 8;
+  const int64_t grid = (rows * p.row_chunks + 255) / 256;
+  if (grid > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: rows*inter is too large", fn);
+  if (rows == 0) return KIN_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (act == KIN_ACT_SILU) gated_act_kernel<KIN_ACT_SILU><<<(unsigned)grid, 256, 0, s>>>(p);
+  else if (act == KIN_ACT_GELU) gated_act_kernel<KIN_ACT_GELU><<<(unsigned)grid, 256, 0, s>>>(p);
+  else gated_act_kernel<KIN_ACT_RELU><<<(unsigned)grid, 256, 0, s>>>(p);
+  return check_hip(hipGetLastError(), "gated_act_kernel launch");
+}

@@ -6,10 +6,13 @@ benchmark layers, for like-for-like whole-layer throughput runs.
 ``wqkv`` -> q/k RMSNorm -> [append, page scoring, top-k, attention] -> ``wo`` ->
 residual -> RMSNorm -> SwiGLU MLP -> residual, for one tensor-parallel shard
 (head counts and MLP width divided by ``world_size``, as the reference does at
-:101-106).  Everything between the q/k norms and ``wo`` runs on the HIP kernels
-of this package; the norms and GEMMs are plain PyTorch (rocBLAS/hipBLASLt), which
-is what the reference does too apart from using flashinfer's RMSNorm
-(benchmark/model_utils.py:4-25).
+:101-106).  Everything except the GEMMs runs on the HIP kernels of this
+package: the RMSNorms (the reference calls flashinfer's through its layer_norm
+and qk_norm ops, benchmark/model_utils.py:4-25) with the first residual add
+folded in, the q/k norm + split of the fused projection, the attention path,
+and the gated activation.  The GEMMs are hipBLASLt through PyTorch; the gate and
+up projections run as one GEMM over their stacked weights, and the last
+residual add rides on the down projection (``addmm``).
 
 The reference reads the model shape from the Hugging Face hub
 (benchmark/blocktopk.py:65); ``qwen3_config`` provides the same fields offline.
@@ -23,6 +26,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import ops
 from .blocktopk_decoder import BlockTopkPagedAttention, DensePagedAttention
 
 # Published Qwen3 shapes (general knowledge; the reference fetches them from the hub).
@@ -35,7 +39,7 @@ _QWEN3 = {
     "Qwen3-32B": dict(hidden_size=5120, intermediate_size=25600, num_attention_heads=64, num_key_value_heads=8, num_hidden_layers=64),
 }
 
-_ACT = {"silu": F.silu, "gelu": F.gelu, "relu": F.relu}
+_ACT = ("silu", "gelu", "relu")
 
 
 def qwen3_config(name: str) -> SimpleNamespace:
@@ -48,9 +52,9 @@ def qwen3_config(name: str) -> SimpleNamespace:
 
 
 def rms_norm(x: torch.Tensor, eps: float, weight: torch.Tensor) -> torch.Tensor:
-    """RMSNorm over the last dimension, computed in fp32 (benchmark/model_utils.py:4-25)."""
-    xf = x.float()
-    return (xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps) * weight.float()).to(x.dtype)
+    """RMSNorm over the last dimension with fp32 statistics, argument order of the
+    reference's layer_norm / qk_norm (benchmark/model_utils.py:4-25)."""
+    return ops.rms_norm(x, weight, eps)
 
 
 def init_weights(m):
@@ -75,7 +79,9 @@ class _LayerBase(nn.Module):
         self.dim = config.hidden_size
         self.intermediate_size = config.intermediate_size // world_size
         self.eps = config.rms_norm_eps
-        self.activation = _ACT[config.hidden_act]
+        if config.hidden_act not in _ACT:
+            raise ValueError(f"hidden_act {config.hidden_act!r} is not one of {_ACT}")
+        self.activation = config.hidden_act
         self.batch_size = batch_size
 
         self.qnorm_weight = nn.Parameter(torch.ones(self.head_dim))
@@ -88,26 +94,42 @@ class _LayerBase(nn.Module):
         self.up_proj = nn.Linear(self.dim, self.intermediate_size, bias=False)
         self.gate_proj = nn.Linear(self.dim, self.intermediate_size, bias=False)
         self.down_proj = nn.Linear(self.intermediate_size, self.dim, bias=False)
+        self._gate_up = None
+
+    def _gate_up_weight(self) -> torch.Tensor:
+        """[2 * intermediate, hidden]: gate_proj over up_proj.  Built on first use
+        (and again after the module moved or changed dtype); the two parameters
+        then become views of it, so no weight is held twice and loading a state
+        dict into them keeps filling the stacked tensor."""
+        g, u = self.gate_proj.weight, self.up_proj.weight
+        w = self._gate_up
+        n = self.intermediate_size
+        if w is None or g.data_ptr() != w.data_ptr() or u.data_ptr() != w[n:].data_ptr() or g.dtype != w.dtype:
+            w = torch.cat([g.data, u.data], dim=0)
+            g.data, u.data = w[:n], w[n:]
+            self._gate_up = w
+        return w
 
     def _qkv(self, hidden_states):
         """benchmark/blocktopk_decoder.py:192-207: norm, fused projection, split, q/k norm."""
         bsz, q_len, _ = hidden_states.size()
         if q_len != 1:
             raise ValueError("decode layers take one token per sequence")
-        x = rms_norm(hidden_states, self.eps, self.input_layernorm_weight)
-        q_dim, kv_dim = self.head_dim * self.num_heads, self.head_dim * self.num_kv_heads
-        q, k, v = self.wqkv(x).split((q_dim, kv_dim, kv_dim), dim=-1)
-        q = rms_norm(q.reshape(bsz, self.num_heads, self.head_dim), self.eps, self.qnorm_weight).contiguous()
-        k = rms_norm(k.reshape(bsz, self.num_kv_heads, self.head_dim), self.eps, self.knorm_weight).contiguous()
-        v = v.reshape(bsz, self.num_kv_heads, self.head_dim).contiguous()
-        return q, k, v
+        x = ops.rms_norm(hidden_states, self.input_layernorm_weight, self.eps)
+        qkv = self.wqkv(x).view(bsz, -1)
+        return ops.qkv_norm_split(qkv, self.qnorm_weight, self.knorm_weight, self.eps, self.num_heads, self.num_kv_heads)
 
     def _finish(self, residual, o):
         """benchmark/blocktopk_decoder.py:226-240: wo, residual, norm, SwiGLU MLP, residual."""
         bsz = o.shape[0]
-        h = residual + self.wo(o.reshape(bsz, 1, self.head_dim * self.num_heads))
-        x = rms_norm(h, self.eps, self.post_attention_layernorm_weight)
-        return h + self.down_proj(self.activation(self.gate_proj(x)) * self.up_proj(x))
+        # h = residual + wo(o), written over the projection's own output (the layer
+        # input stays untouched), and x = norm(h) in the same pass
+        h = self.wo(o.reshape(bsz, self.head_dim * self.num_heads))
+        x = ops.rms_norm(residual.reshape(bsz, self.dim), self.post_attention_layernorm_weight, self.eps, residual=h)
+        n = self.intermediate_size
+        gate_up = F.linear(x, self._gate_up_weight())
+        y = ops.gated_act(gate_up[:, :n], gate_up[:, n:], self.activation)
+        return torch.addmm(h, y, self.down_proj.weight.t()).view(bsz, 1, self.dim)
 
 
 class BlockTopkDecoderLayer(_LayerBase):

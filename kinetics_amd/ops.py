@@ -518,6 +518,111 @@ def check_page_table(page_indices, page_indptr, last_page_len, page_size, num_pa
 
 
 # ---------------------------------------------------------------------------
+# Row-wise layer kernels around the attention path
+# ---------------------------------------------------------------------------
+
+ACTIVATIONS = {"silu": 0, "gelu": 1, "relu": 2}
+
+
+def _row_view(t: torch.Tensor, name: str, device=None):
+    """(rows, width, row stride in elements) of a bf16 tensor whose rows are its
+    last dimension: any contiguous shape, or a 2-D view with a row stride (a
+    slice of a wider projection)."""
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
+    if t.dtype != torch.bfloat16:
+        raise TypeError(f"{name} must be torch.bfloat16, got {t.dtype}")
+    if t.device.type != "cuda":
+        raise ValueError(f"{name} must live on the GPU (device 'cuda'), got {t.device}")
+    if device is not None and t.device != device:
+        raise ValueError(f"{name} is on {t.device}, expected {device}")
+    if t.dim() < 1:
+        raise ValueError(f"{name} must have at least one dimension")
+    width = t.shape[-1]
+    if t.is_contiguous():
+        return t.numel() // max(width, 1), width, width
+    if t.dim() == 2 and t.stride(1) == 1:
+        return t.shape[0], width, t.stride(0)
+    raise ValueError(f"{name} must be contiguous, or 2-D with unit stride along its rows")
+
+
+def rms_norm(x, weight, eps: float, residual=None, out=None) -> torch.Tensor:
+    """RMSNorm over the last dimension with fp32 statistics: what the reference's
+    ``layer_norm`` and ``qk_norm`` ops compute through flashinfer.rmsnorm
+    (benchmark/model_utils.py:4-25).  With ``residual`` (contiguous, same shape)
+    the add in front of the norm is folded in as in ``fused_layer_norm``
+    (benchmark/model_utils.py:27-41): ``residual`` becomes ``x + residual`` and
+    the norm of that sum is returned."""
+    rows, hidden, x_stride = _row_view(x, "x")
+    dev = x.device
+    _require(weight, "weight", torch.bfloat16, 1, dev)
+    if weight.numel() != hidden:
+        raise ValueError(f"weight has {weight.numel()} entries for rows of {hidden}")
+    if out is None:
+        out = torch.empty(x.shape, dtype=x.dtype, device=dev)
+    orows, owidth, out_stride = _row_view(out, "out", dev)
+    if (orows, owidth) != (rows, hidden):
+        raise ValueError(f"out shape {tuple(out.shape)} does not match x {tuple(x.shape)}")
+    if residual is not None:
+        _require(residual, "residual", torch.bfloat16, None, dev)
+        if residual.numel() != rows * hidden or residual.shape[-1] != hidden:
+            raise ValueError(f"residual shape {tuple(residual.shape)} does not match x {tuple(x.shape)}")
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(lib.kin_rms_norm(_ptr(x), _ptr(residual), _ptr(weight), _ptr(out), rows, hidden, x_stride, out_stride,
+                                    float(eps), _stream(dev)))
+    return out
+
+
+def qkv_norm_split(qkv, q_weight, k_weight, eps: float, num_q_heads: int, num_kv_heads: int):
+    """From the fused projection ``qkv[batch, (Hq + 2*Hkv) * 128]`` to contiguous
+    ``q[batch, Hq, 128]``, ``k[batch, Hkv, 128]``, ``v[batch, Hkv, 128]`` with the
+    q and k heads RMS-normalised: the split, qk_norm calls and reshapes of
+    benchmark/blocktopk_decoder.py:196-207 in one pass."""
+    batch, width, stride = _row_view(qkv, "qkv")
+    dev = qkv.device
+    if width != (num_q_heads + 2 * num_kv_heads) * HEAD_DIM:
+        raise ValueError(f"qkv rows have {width} elements, expected (Hq + 2*Hkv) * {HEAD_DIM} = "
+                         f"{(num_q_heads + 2 * num_kv_heads) * HEAD_DIM}")
+    _require(q_weight, "q_weight", torch.bfloat16, 1, dev)
+    _require(k_weight, "k_weight", torch.bfloat16, 1, dev)
+    if q_weight.numel() != HEAD_DIM or k_weight.numel() != HEAD_DIM:
+        raise ValueError(f"q_weight and k_weight must have {HEAD_DIM} entries")
+    q = torch.empty(batch, num_q_heads, HEAD_DIM, dtype=torch.bfloat16, device=dev)
+    k = torch.empty(batch, num_kv_heads, HEAD_DIM, dtype=torch.bfloat16, device=dev)
+    v = torch.empty(batch, num_kv_heads, HEAD_DIM, dtype=torch.bfloat16, device=dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(lib.kin_qkv_norm_split(_ptr(qkv), stride, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(q), _ptr(k),
+                                          _ptr(v), batch, int(num_q_heads), int(num_kv_heads), HEAD_DIM, _stream(dev)))
+    return q, k, v
+
+
+def gated_act(gate, up, act: str = "silu", out=None) -> torch.Tensor:
+    """``act(gate) * up`` of the gated MLP (benchmark/blocktopk_decoder.py:234-237),
+    rounded to bf16 after the activation and after the product as the two tensor
+    operations round.  ``gate`` and ``up`` may be column slices of one fused
+    projection (2-D views with a row stride)."""
+    if act not in ACTIVATIONS:
+        raise ValueError(f"act must be one of {sorted(ACTIVATIONS)}, got {act!r}")
+    rows, inter, g_stride = _row_view(gate, "gate")
+    dev = gate.device
+    urows, uwidth, u_stride = _row_view(up, "up", dev)
+    if (urows, uwidth) != (rows, inter):
+        raise ValueError(f"up shape {tuple(up.shape)} does not match gate {tuple(gate.shape)}")
+    if out is None:
+        out = torch.empty(gate.shape, dtype=torch.bfloat16, device=dev)
+    _require(out, "out", torch.bfloat16, None, dev)
+    if out.numel() != rows * inter or out.shape[-1] != inter:
+        raise ValueError(f"out shape {tuple(out.shape)} does not match gate {tuple(gate.shape)}")
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(lib.kin_gated_act(_ptr(gate), _ptr(up), _ptr(out), rows, inter, g_stride, u_stride, ACTIVATIONS[act],
+                                     _stream(dev)))
+    return out
+
+
+# ---------------------------------------------------------------------------
 # torch.library registration (namespace "kinetics", defined once at import)
 # ---------------------------------------------------------------------------
 
@@ -650,3 +755,68 @@ def _dense_impl(q, kv_cache, page_indices, page_indptr, last_page_len, max_pages
 def _dense_fake(q, kv_cache, page_indices, page_indptr, last_page_len, max_pages_per_seq, workspace, sm_scale, num_splits,
                 first_page_offset=0):
     return torch.empty_like(q)
+
+
+# The reference's norm ops with their names and argument order
+# (mylib::layer_norm, mylib::qk_norm, mylib::fused_layer_norm;
+# benchmark/model_utils.py:4-41), plus the two fused row-wise steps.
+torch.library.define("kinetics::layer_norm", "(Tensor hidden_states, float eps, Tensor weight) -> Tensor")
+torch.library.define("kinetics::qk_norm", "(Tensor hidden_states, float eps, Tensor weight) -> Tensor")
+torch.library.define("kinetics::fused_layer_norm",
+                     "(Tensor hidden_states, Tensor(a!) residual, float eps, Tensor weight) -> Tensor")
+torch.library.define("kinetics::qkv_norm_split",
+                     "(Tensor qkv, Tensor q_weight, Tensor k_weight, float eps, int num_q_heads, int num_kv_heads) "
+                     "-> (Tensor, Tensor, Tensor)")
+torch.library.define("kinetics::gated_act", "(Tensor gate, Tensor up, str act) -> Tensor")
+
+
+@torch.library.impl("kinetics::layer_norm", "cuda")
+def _layer_norm_impl(hidden_states, eps, weight):
+    return rms_norm(hidden_states, weight, eps)
+
+
+@torch.library.register_fake("kinetics::layer_norm")
+def _layer_norm_fake(hidden_states, eps, weight):
+    return torch.empty_like(hidden_states)
+
+
+@torch.library.impl("kinetics::qk_norm", "cuda")
+def _qk_norm_impl(hidden_states, eps, weight):
+    return rms_norm(hidden_states, weight, eps)
+
+
+@torch.library.register_fake("kinetics::qk_norm")
+def _qk_norm_fake(hidden_states, eps, weight):
+    return torch.empty_like(hidden_states)
+
+
+@torch.library.impl("kinetics::fused_layer_norm", "cuda")
+def _fused_layer_norm_impl(hidden_states, residual, eps, weight):
+    return rms_norm(hidden_states, weight, eps, residual=residual)
+
+
+@torch.library.register_fake("kinetics::fused_layer_norm")
+def _fused_layer_norm_fake(hidden_states, residual, eps, weight):
+    return torch.empty_like(hidden_states)
+
+
+@torch.library.impl("kinetics::qkv_norm_split", "cuda")
+def _qkv_norm_split_impl(qkv, q_weight, k_weight, eps, num_q_heads, num_kv_heads):
+    return qkv_norm_split(qkv, q_weight, k_weight, eps, num_q_heads, num_kv_heads)
+
+
+@torch.library.register_fake("kinetics::qkv_norm_split")
+def _qkv_norm_split_fake(qkv, q_weight, k_weight, eps, num_q_heads, num_kv_heads):
+    batch = qkv.numel() // qkv.shape[-1]
+    return (qkv.new_empty(batch, num_q_heads, HEAD_DIM), qkv.new_empty(batch, num_kv_heads, HEAD_DIM),
+            qkv.new_empty(batch, num_kv_heads, HEAD_DIM))
+
+
+@torch.library.impl("kinetics::gated_act", "cuda")
+def _gated_act_impl(gate, up, act):
+    return gated_act(gate, up, act)
+
+
+@torch.library.register_fake("kinetics::gated_act")
+def _gated_act_fake(gate, up, act):
+    return torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)

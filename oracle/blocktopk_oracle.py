@@ -31,6 +31,9 @@ algorithm of the reference's block top-k decoder path:
                     page lists with sink_pages=1, local_tokens=local and a
                     12-slot first-page offset are the same function
 
+* layer row steps   RMSNorm (benchmark/model_utils.py:4-41), q/k norm + split and
+                    act(gate)*up (benchmark/blocktopk_decoder.py:196-207,229-237)
+
 flashinfer 0.1.6 (the wheel the reference calls, README.md:81) is not in the
 reference tree; its page-table convention is restated here: sequence b owns
 ``page_indices[page_indptr[b]:page_indptr[b+1]]`` and holds
@@ -46,7 +49,8 @@ numpy/torch library top-k on the same scores plus hand-built tie cases;
 attention: torch scaled_dot_product_attention on the de-paged K/V when every
 page is selected, out == v for one token, out == V for constant V, q == 0 gives
 the mean of V, permutation invariance of the page list, split-K merge
-invariance, lse == logsumexp.
+invariance, lse == logsumexp; layer row steps: torch's own rms_norm, silu, gelu,
+relu and bf16 tensor add/mul on the CPU, constant rows, scale invariance.
 
 bfloat16 tensors are numpy uint16 arrays of raw bit patterns throughout.
 """
@@ -518,6 +522,60 @@ def litesys_decode(q, K, V, topk_block, local, sink=4, block_size=16, sm_scale=N
     if return_mean_logits:
         return out, keep_all, mean_all
     return out, keep_all
+
+
+# ---------------------------------------------------------------------------
+# Row-wise steps of the decoder layer around the attention path
+# ---------------------------------------------------------------------------
+
+
+def rms_norm(x, weight, eps, residual=None):
+    """RMSNorm over the last axis, bf16 bits in and out: x * rsqrt(mean(x^2) + eps)
+    * weight, which is flashinfer.rmsnorm as the reference's layer_norm and
+    qk_norm call it (benchmark/model_utils.py:4-25).  With ``residual`` the sum
+    x + residual, rounded to bf16 as a bf16 tensor add rounds it
+    (benchmark/blocktopk_decoder.py:229-232; fused_layer_norm,
+    benchmark/model_utils.py:27-41), is normalised instead.  Returns
+    (out_bits, new_residual_bits or None)."""
+    xf = bf16_to_f32(x).astype(np.float64)
+    new_res = None
+    if residual is not None:
+        new_res = f32_to_bf16((xf + bf16_to_f32(residual).astype(np.float64)).astype(np.float32))
+        xf = bf16_to_f32(new_res).astype(np.float64)
+    w = bf16_to_f32(weight).astype(np.float64)
+    r = 1.0 / np.sqrt(np.mean(xf * xf, axis=-1, keepdims=True) + float(eps))
+    return f32_to_bf16((xf * r * w).astype(np.float32)), new_res
+
+
+def qkv_norm_split(qkv, q_weight, k_weight, eps, num_q_heads, num_kv_heads, head_dim=128):
+    """Fused projection rows [Hq*D | Hkv*D | Hkv*D] -> q[B,Hq,D], k[B,Hkv,D] (each
+    head RMS-normalised) and v[B,Hkv,D] (benchmark/blocktopk_decoder.py:196-207)."""
+    qkv = np.asarray(qkv, dtype=np.uint16)
+    B = qkv.shape[0]
+    nq, nk = num_q_heads * head_dim, num_kv_heads * head_dim
+    q = qkv[:, :nq].reshape(B, num_q_heads, head_dim)
+    k = qkv[:, nq:nq + nk].reshape(B, num_kv_heads, head_dim)
+    v = qkv[:, nq + nk:nq + 2 * nk].reshape(B, num_kv_heads, head_dim)
+    return rms_norm(q, q_weight, eps)[0], rms_norm(k, k_weight, eps)[0], np.ascontiguousarray(v)
+
+
+def gated_act(gate, up, act="silu"):
+    """bf16(bf16(act(gate)) * up): the gated MLP product of
+    benchmark/blocktopk_decoder.py:234-237 with the rounding of its two bf16
+    tensor operations.  gelu is the erf form."""
+    from math import erf
+
+    g = bf16_to_f32(gate).astype(np.float64)
+    if act == "silu":
+        a = g / (1.0 + np.exp(-g))
+    elif act == "gelu":
+        a = 0.5 * g * (1.0 + np.vectorize(erf)(g / np.sqrt(2.0)))
+    elif act == "relu":
+        a = np.maximum(g, 0.0)
+    else:
+        raise ValueError(f"unknown activation {act!r}")
+    a = bf16_to_f32(f32_to_bf16(a.astype(np.float32))).astype(np.float64)
+    return f32_to_bf16((a * bf16_to_f32(up).astype(np.float64)).astype(np.float32))
 
 
 # ---------------------------------------------------------------------------

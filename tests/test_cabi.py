@@ -184,6 +184,45 @@ def test_strided_topk_argument_errors(lib):
     assert strided(B=0) == _lib.KIN_OK
 
 
+def test_layer_row_kernel_argument_errors(lib):
+    def norm(x=A, res=None, w=A, out=A, rows=4, hidden=4096, xs=4096, os_=4096, eps=1e-6):
+        return lib.kin_rms_norm(x, res, w, out, rows, hidden, xs, os_, eps, None)
+
+    assert norm(x=None) == _lib.KIN_ERR_NULL_POINTER
+    assert norm(w=None) == _lib.KIN_ERR_NULL_POINTER
+    assert norm(rows=-1) == _lib.KIN_ERR_BAD_SHAPE
+    assert norm(hidden=4100) == _lib.KIN_ERR_UNSUPPORTED   # not a multiple of 128
+    assert norm(hidden=8704, xs=8704, os_=8704) == _lib.KIN_ERR_UNSUPPORTED  # above 8192
+    assert norm(hidden=2176, xs=2176, os_=2176) == _lib.KIN_ERR_UNSUPPORTED  # multiple of 128 only, above 2048
+    assert norm(xs=4000) == _lib.KIN_ERR_BAD_SHAPE         # stride below the row width
+    assert norm(os_=4100) == _lib.KIN_ERR_BAD_SHAPE        # stride not a multiple of 8
+    assert norm(eps=-1.0) == _lib.KIN_ERR_BAD_SHAPE
+    assert norm(out=A + 4) == _lib.KIN_ERR_MISALIGNED
+    assert norm(res=A + 8) == _lib.KIN_ERR_MISALIGNED
+    assert norm(rows=0) == _lib.KIN_OK and norm(rows=0, hidden=128, xs=128, os_=128) == _lib.KIN_OK
+
+    def split(qkv=A, stride=768, qw=A, kw=A, q=A, k=A, v=A, B=2, Hq=4, Hkv=1, D=128):
+        return lib.kin_qkv_norm_split(qkv, stride, qw, kw, 1e-6, q, k, v, B, Hq, Hkv, D, None)
+
+    assert split(kw=None) == _lib.KIN_ERR_NULL_POINTER
+    assert split(v=None) == _lib.KIN_ERR_NULL_POINTER
+    assert split(Hq=0) == _lib.KIN_ERR_BAD_SHAPE
+    assert split(D=64) == _lib.KIN_ERR_UNSUPPORTED
+    assert split(stride=760) == _lib.KIN_ERR_BAD_SHAPE     # narrower than (Hq + 2*Hkv) * 128
+    assert split(q=A + 2) == _lib.KIN_ERR_MISALIGNED
+    assert split(B=0) == _lib.KIN_OK
+
+    def gate(g=A, u=A, out=A, rows=2, inter=1536, gs=3072, us=3072, act=0):
+        return lib.kin_gated_act(g, u, out, rows, inter, gs, us, act, None)
+
+    assert gate(u=None) == _lib.KIN_ERR_NULL_POINTER
+    assert gate(inter=1530) == _lib.KIN_ERR_BAD_SHAPE
+    assert gate(gs=1000) == _lib.KIN_ERR_BAD_SHAPE
+    assert gate(act=3) == _lib.KIN_ERR_UNSUPPORTED
+    assert gate(g=A + 1) == _lib.KIN_ERR_MISALIGNED
+    assert gate(rows=0) == _lib.KIN_OK
+
+
 def test_sel_list_capacity(lib):
     assert lib.kin_sel_list_capacity(128, 0, 1) == 129               # the reference's k + 1
     assert lib.kin_sel_list_capacity(64, 1, 16) == 64 + 1 + 2
@@ -226,7 +265,8 @@ def test_custom_ops_are_registered_with_fake_kernels():
 
     import kinetics_amd  # noqa: F401
 
-    for name in ("append_paged_kv", "update_kv", "block_score_topk", "sparse_paged_decode", "dense_paged_decode"):
+    for name in ("append_paged_kv", "update_kv", "block_score_topk", "sparse_paged_decode", "dense_paged_decode",
+                 "layer_norm", "qk_norm", "fused_layer_norm", "qkv_norm_split", "gated_act"):
         assert hasattr(torch.ops.kinetics, name)
     # the fake kernel gives shape/dtype without running anything (what torch.compile needs)
     q = torch.empty(3, 4, 128, dtype=torch.bfloat16, device="meta")
@@ -236,6 +276,11 @@ def test_custom_ops_are_registered_with_fake_kernels():
     l = torch.empty(3, dtype=torch.int32, device="meta")
     out = torch.ops.kinetics.sparse_paged_decode(q, kv, i, c, l, None, 0.0, 0)
     assert out.shape == q.shape and out.dtype == torch.bfloat16
+    qkv = torch.empty(3, 6 * 128, dtype=torch.bfloat16, device="meta")
+    w = torch.empty(128, dtype=torch.bfloat16, device="meta")
+    fq, fk, fv = torch.ops.kinetics.qkv_norm_split(qkv, w, w, 1e-6, 4, 1)
+    assert fq.shape == (3, 4, 128) and fk.shape == (3, 1, 128) and fv.shape == (3, 1, 128)
+    assert torch.ops.kinetics.gated_act(qkv[:, :256], qkv[:, 256:512], "silu").shape == (3, 256)
 
 
 def test_bench_byte_model_matches_the_documented_figures():

@@ -615,3 +615,88 @@ def test_litesys_strided_mask():
         want[seq_len - local :] = True
         want[4 + toks.numpy()] = True
         assert np.array_equal(O.litesys_strided_mask(ml, seq_len, k, local, 4, bs, st), want)
+
+
+# --------------------------------------------------------------------------- layer row steps
+
+
+def _ulps(a_bits, b_bits):
+    """Largest distance between two bf16 arrays in units of the last place."""
+    def key(b):
+        b = b.astype(np.int32)
+        return np.where(b & 0x8000, 0x8000 - b, b)
+
+    # values that differ by less than 1e-6 count as equal (fp32 against fp64 tails near zero)
+    near = np.abs(O.bf16_to_f32(a_bits).astype(np.float64) - O.bf16_to_f32(b_bits)) <= 1e-6
+    return int(np.where(near, 0, np.abs(key(a_bits) - key(b_bits))).max())
+
+
+def test_rms_norm_against_torch_and_closed_forms():
+    rng = np.random.default_rng(21)
+    x = O.f32_to_bf16(rng.standard_normal((7, 512)).astype(np.float32) * 3)
+    w = O.f32_to_bf16(1 + 0.2 * rng.standard_normal(512).astype(np.float32))
+    got, none = O.rms_norm(x, w, 1e-6)
+    assert none is None
+    xt, wt = P.to_torch(x).double(), P.to_torch(w).double()
+    want = torch.nn.functional.rms_norm(xt, (512,), wt, 1e-6)
+    assert _ulps(got, P.from_torch(want.float().to(torch.bfloat16))) <= 1
+    # a wrong eps placement or a sum instead of a mean shows on small rows
+    tiny = O.f32_to_bf16(np.full((1, 128), 1e-3, dtype=np.float32))
+    got_t, _ = O.rms_norm(tiny, O.f32_to_bf16(np.ones(128, dtype=np.float32)), 1e-6)
+    t = float(O.bf16_to_f32(tiny)[0, 0])
+    assert np.allclose(O.bf16_to_f32(got_t), t / np.sqrt(t * t + 1e-6), rtol=1e-2)
+    # constant row: out == sign(c) * weight; scale invariance
+    c = O.f32_to_bf16(np.full((1, 512), -4.0, dtype=np.float32))
+    got_c, _ = O.rms_norm(c, w, 0.0)
+    assert np.array_equal(got_c[0], O.f32_to_bf16(-O.bf16_to_f32(w)))
+    x4 = O.f32_to_bf16(O.bf16_to_f32(x) * 4.0)
+    assert np.array_equal(O.rms_norm(x4, w, 0.0)[0], O.rms_norm(x, w, 0.0)[0])
+
+
+def test_rms_norm_with_residual_is_norm_of_the_bf16_sum():
+    rng = np.random.default_rng(22)
+    x = O.f32_to_bf16(rng.standard_normal((5, 256)).astype(np.float32))
+    r = O.f32_to_bf16(rng.standard_normal((5, 256)).astype(np.float32) * 2)
+    w = O.f32_to_bf16(1 + 0.1 * rng.standard_normal(256).astype(np.float32))
+    got, new_r = O.rms_norm(x, w, 1e-6, residual=r)
+    want_r = P.from_torch(P.to_torch(x) + P.to_torch(r))  # torch's own bf16 tensor add
+    assert np.array_equal(new_r, want_r)
+    assert np.array_equal(got, O.rms_norm(want_r, w, 1e-6)[0])
+    assert np.array_equal(O.rms_norm(r, w, 1e-6, residual=x)[0], got)  # the add commutes
+
+
+def test_qkv_norm_split_against_torch():
+    rng = np.random.default_rng(23)
+    B, Hq, Hkv = 3, 4, 2
+    qkv = O.f32_to_bf16(rng.standard_normal((B, (Hq + 2 * Hkv) * D)).astype(np.float32) * 2)
+    qw = O.f32_to_bf16(1 + 0.3 * rng.standard_normal(D).astype(np.float32))
+    kw = O.f32_to_bf16(1 + 0.3 * rng.standard_normal(D).astype(np.float32))
+    q, k, v = O.qkv_norm_split(qkv, qw, kw, 1e-6, Hq, Hkv)
+    t = P.to_torch(qkv).double()
+    tq, tk, tv = t.split((Hq * D, Hkv * D, Hkv * D), dim=-1)
+    wq = torch.nn.functional.rms_norm(tq.reshape(B, Hq, D), (D,), P.to_torch(qw).double(), 1e-6)
+    wk = torch.nn.functional.rms_norm(tk.reshape(B, Hkv, D), (D,), P.to_torch(kw).double(), 1e-6)
+    assert q.shape == (B, Hq, D) and k.shape == (B, Hkv, D) and v.shape == (B, Hkv, D)
+    assert _ulps(q, P.from_torch(wq.float().to(torch.bfloat16))) <= 1
+    assert _ulps(k, P.from_torch(wk.float().to(torch.bfloat16))) <= 1
+    assert np.array_equal(v, P.from_torch(tv.reshape(B, Hkv, D).float().to(torch.bfloat16)))
+    # q and k use their own weights
+    assert not np.array_equal(O.qkv_norm_split(qkv, kw, qw, 1e-6, Hq, Hkv)[0], q)
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu", "relu"])
+def test_gated_act_against_torch_bf16_ops(act):
+    rng = np.random.default_rng(24)
+    g = O.f32_to_bf16(rng.standard_normal((4, 64)).astype(np.float32) * 3)
+    u = O.f32_to_bf16(rng.standard_normal((4, 64)).astype(np.float32) * 2)
+    fn = {"silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu, "relu": torch.relu}[act]
+    want = fn(P.to_torch(g)) * P.to_torch(u)  # two bf16 tensor operations
+    got = O.gated_act(g, u, act)
+    assert _ulps(got, P.from_torch(want)) <= 1
+    # closed forms: act(0) = 0; large positive gates pass up through
+    z = O.gated_act(O.f32_to_bf16(np.zeros((1, 8), dtype=np.float32)), u[:1, :8], act)
+    assert np.all(O.bf16_to_f32(z) == 0)
+    big = O.f32_to_bf16(np.full((1, 8), 32.0, dtype=np.float32))
+    assert np.array_equal(O.gated_act(big, u[:1, :8], act), O.f32_to_bf16(32.0 * O.bf16_to_f32(u[:1, :8])))
+    with pytest.raises(ValueError):
+        O.gated_act(g, u, "tanh")
