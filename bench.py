@@ -201,7 +201,20 @@ def whole_layer(torch, args, B, ctx, topk, device):
         layer(hidden.clone())
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
+    # the same forward replayed as one HIP graph (the reference compiles its layer
+    # with mode="max-autotune", benchmark/blocktopk.py:41-43)
+    graphed = layer.graphed(hidden)
+    for _ in range(args.warmup):
+        graphed(hidden)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        graphed(hidden)
+    torch.cuda.synchronize()
+    dt_graph = (time.perf_counter() - t0) / args.steps
+    del graphed
     out = {"model": name, "world_size": world, "ms_per_layer_step": dt * 1e3, "tokens_per_s_per_layer": B / dt,
+           "ms_per_layer_step_hip_graph": dt_graph * 1e3, "tokens_per_s_per_layer_hip_graph": B / dt_graph,
            "normalised_like_reference_print": B / dt / (world * cfg.num_hidden_layers),
            "note": "GEMMs are hipBLASLt through PyTorch; norms, q/k/v split, attention and the gated activation are this repository's kernels"}
     del layer

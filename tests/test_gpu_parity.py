@@ -1178,6 +1178,16 @@ def test_decoder_layer_matches_fp32_reference(ops, dense):
     got = out.float().cpu()
     assert torch.allclose(got, want, rtol=5e-2, atol=5e-2), (got - want).abs().max()
     assert rms_norm(hidden, 1e-6, layer.input_layernorm_weight).dtype == torch.bfloat16
+    # the forward as one HIP graph: every replay equals the eager call on the same input,
+    # with eager work and synchronisations between the replays
+    graphed = layer.graphed(hidden)
+    for i in range(4):
+        h_i = torch.randn(B, 1, 512, device=DEV).to(torch.bfloat16)
+        eager = layer(h_i.clone()).clone()
+        torch.cuda.synchronize()
+        replay = graphed(h_i)
+        torch.cuda.synchronize()
+        assert torch.equal(replay, eager), f"replay {i}: {(replay.float() - eager.float()).abs().max().item()}"
 
 
 @pytest.mark.parametrize("sink,local,offset", [(1, 17, 0), (2, 33, 0), (0, 49, 0), (3, 1, 0), (1, 16, 12), (1, 5, 12),
