@@ -33,6 +33,11 @@ __host__ __device__ inline int max_local_pages(int local_tokens) { return 1 + (l
 // measurably raises achieved HBM read bandwidth (about 6.3 -> 7.0 TB/s on a
 // plain streaming read).
 constexpr int kStreamLoad = 2;  // "nt"
+// Cache-policy bit for buffer loads and stores at device scope ("sc1", what a
+// relaxed agent-scope atomic access uses): the access bypasses the XCD-private
+// L2, so workgroups on different XCDs can hand data to each other through
+// memory inside one launch without cache maintenance.
+constexpr int kDeviceScope = 16;
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;

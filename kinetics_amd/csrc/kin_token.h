@@ -50,6 +50,21 @@ __device__ __forceinline__ int phys_token(const int32_t* table, int c) {
   return table[c >> 4] * kPageSize + (c & (kPageSize - 1));
 }
 
+// list[first .. first + count) holds cache slots (LDS); replaces each by its
+// physical token id and reports the tokens' positions.  One independent table
+// lookup per thread and entry, all in flight together -- inside the ordered
+// compaction the same lookups would be a chain of dependent memory round trips.
+// Barriers before and after are the caller's.
+template <int NT>
+__device__ __forceinline__ void translate_slots(int32_t* list, int first, int count, const int32_t* table, int pad,
+                                                int32_t* sel_tokens) {
+  for (int i = threadIdx.x; i < count; i += NT) {
+    const int c = list[first + i];
+    list[first + i] = phys_token(table, c);
+    if (sel_tokens) sel_tokens[first + i] = c - pad;
+  }
+}
+
 // LDS scratch of the two functions below.
 struct KeySelectShared {
   uint32_t hist[256];
@@ -57,39 +72,60 @@ struct KeySelectShared {
   uint32_t bin, remaining;
 };
 
-// Most-significant-digit-first radix select over n_keys (a multiple of 16) 32-bit
-// keys in global memory, run by a workgroup of NW waves: finds the k-th largest
-// non-zero key (zero keys are "not a candidate"; at least k keys are non-zero).
-// thr receives it, remaining how many keys equal to thr belong to the k largest.
-// first_digit_counted: sh->hist already holds the histogram of the top byte of
-// the non-zero keys (counted while they were produced).  The keys are written by
-// this workgroup; a barrier separates their last write from this call.
+// Keys one trip to memory brings into registers: kSelLoads 16-byte loads per lane.
+// Under a saturated key stream every dependent round trip costs microseconds, so
+// the select passes below make few, wide trips instead of many narrow ones.
+constexpr int kSelLoads = 16;
+
+// Chunk c0 of the key array -> registers: wave w holds the 1024 * kSelLoads / 4
+// consecutive keys from c0 + w * 256 * kSelLoads, load u the keys 256 * u + 4 * lane
+// + 0..3 of them (so wave, u, lane, j ascending is index ascending).  keys covers
+// exactly the n_keys (a multiple of 4) keys: entries past them read as 0, "not a
+// candidate".  Device-scope loads: the keys may come from workgroups on other XCDs.
 template <int NW>
-__device__ __forceinline__ void radix_threshold(const uint32_t* keys, int n_keys, uint32_t k, bool first_digit_counted,
-                                                KeySelectShared* sh, uint32_t& thr, uint32_t& remaining) {
-  constexpr int NT = NW * 64;
+__device__ __forceinline__ void load_key_chunk(__amdgpu_buffer_rsrc_t keys, int c0, u32x4 (&kk)[kSelLoads]) {
+  const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), l = threadIdx.x & 63;
+  const int base = c0 + w * (256 * kSelLoads) + 4 * l;
+#pragma unroll
+  for (int u = 0; u < kSelLoads; ++u) kk[u] = __builtin_amdgcn_raw_buffer_load_b128(keys, (base + u * 256) * 4, 0, kDeviceScope);
+}
+
+// Most-significant-digit-first radix select over n_keys (a multiple of 16) 32-bit
+// keys in global memory (a descriptor over exactly those keys, written at device
+// scope), run by a workgroup of NW waves, followed by the ordered
+// compaction of the winners: finds the k-th largest non-zero key (zero keys are
+// "not a candidate"; at least k >= 1 keys are non-zero), then calls emit(pos, index)
+// for every key above it and for the lowest-indexed keys equal to it that complete
+// the k, pos = 0, 1, ... in ascending index order.
+// first_digit_counted: sh->hist already holds the histogram of the top byte of
+// the non-zero keys (counted while they were produced).  The writes of the keys
+// have completed (s_waitcnt + barrier, or the arrival counter of split scoring).
+// Up to NW * 4096 keys are loaded once and stay in registers through all passes;
+// longer arrays are walked in chunks of that size, one trip per chunk and pass.
+template <int NW, typename Emit>
+__device__ __forceinline__ void radix_select_emit(__amdgpu_buffer_rsrc_t keys, int n_keys, uint32_t k,
+                                                  bool first_digit_counted, KeySelectShared* sh, Emit emit) {
+  constexpr int kChunk = NW * 256 * kSelLoads;
   const int tid = threadIdx.x;
-  const int w = tid >> 6, l = tid & 63;
-  uint32_t prefix = 0, mask = 0;
-  remaining = k;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63;
+  const bool single = n_keys <= kChunk;
+  u32x4 kk[kSelLoads];
+  if (single) load_key_chunk<NW>(keys, 0, kk);
+
+  uint32_t prefix = 0, mask = 0, remaining = k;
   for (int shift = 24; shift >= 0; shift -= 8) {
     if (shift != 24 || !first_digit_counted) {
       if (tid < 256) sh->hist[tid] = 0;
       __syncthreads();
-      // 4 independent 16-byte loads per thread in flight: the keys come from L2 / HBM
-      for (int base = tid * 4; base < n_keys; base += NT * 16) {
-        uint4 kk[4];
+      for (int c0 = 0; c0 < n_keys; c0 += kChunk) {
+        if (!single) load_key_chunk<NW>(keys, c0, kk);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int i = base + u * NT * 4;
-          kk[u] = (i < n_keys) ? *reinterpret_cast<const uint4*>(keys + i) : make_uint4(0u, 0u, 0u, 0u);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < kSelLoads; ++u) {
           const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
 #pragma unroll
           for (int j = 0; j < 4; ++j)
             if (k4[j] && (k4[j] & mask) == prefix) atomicAdd(&sh->hist[(k4[j] >> shift) & 255u], 1u);
+          __builtin_amdgcn_sched_barrier(0);  // keeps the lane masks of one load at a time in scalar registers
         }
       }
       __syncthreads();
@@ -100,28 +136,16 @@ __device__ __forceinline__ void radix_threshold(const uint32_t* keys, int n_keys
     mask |= 255u << shift;
     remaining = sh->remaining;
   }
-  thr = prefix;  // >= 1
-}
+  const uint32_t thr = prefix;  // >= 1
 
-// Calls emit(pos, index) for every key above thr and for the `remaining` lowest-
-// indexed keys equal to it, pos = 0, 1, ... in ascending index order.  Each wave
-// owns a contiguous run of indices and walks it 256 at a time (4 consecutive keys
-// per lane, two such loads in flight).  n_keys is a multiple of 16.
-template <int NW, typename Emit>
-__device__ __forceinline__ void compact_winners(const uint32_t* keys, int n_keys, uint32_t thr, uint32_t remaining,
-                                                KeySelectShared* sh, Emit emit) {
-  const int tid = threadIdx.x;
-  const int w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63;
-  const int seg = ((n_keys + NW - 1) / NW + 255) & ~255;
-  const int seg_lo = min(w * seg, n_keys), seg_hi = min(seg_lo + seg, n_keys);  // multiples of 16
-  auto load4 = [&](int c) { return (c < seg_hi) ? *reinterpret_cast<const uint4*>(keys + c) : make_uint4(0u, 0u, 0u, 0u); };
-  uint32_t gt = 0, eq = 0;
-  for (int i = seg_lo; i < seg_hi; i += 1024) {
-    uint4 kk[4];
+  // Ordered compaction, chunk by chunk: count per wave, prefix over the waves, emit.
+  const unsigned long long below = (1ull << l) - 1ull;
+  uint32_t run_all = 0, eq_all = 0;  // winners / threshold-equal keys in the chunks before this one
+  for (int c0 = 0; c0 < n_keys; c0 += kChunk) {
+    if (!single) load_key_chunk<NW>(keys, c0, kk);
+    uint32_t gt = 0, eq = 0;
 #pragma unroll
-    for (int u = 0; u < 4; ++u) kk[u] = load4(i + u * 256 + 4 * l);
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < kSelLoads; ++u) {
       const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -129,39 +153,47 @@ __device__ __forceinline__ void compact_winners(const uint32_t* keys, int n_keys
         eq += (k4[j] == thr) ? 1u : 0u;
       }
     }
-  }
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    gt += __shfl_xor(gt, off);
-    eq += __shfl_xor(eq, off);
-  }
-  if (l == 0) {
-    sh->wave_gt[w] = gt;
-    sh->wave_eq[w] = eq;
-  }
-  __syncthreads();
-  uint32_t run = 0, eq_run = 0;  // winners / threshold-equal keys in the runs before this wave's
-  for (int wv = 0; wv < w; ++wv) {
-    const uint32_t e = sh->wave_eq[wv];
-    const uint32_t left = remaining > eq_run ? remaining - eq_run : 0u;
-    run += sh->wave_gt[wv] + min(e, left);
-    eq_run += e;
-  }
-  const unsigned long long below = (1ull << l) - 1ull;
-  for (int i = seg_lo; i < seg_hi; i += 512) {
-    uint4 kk[2];
+    for (int off = 32; off > 0; off >>= 1) {
+      gt += __shfl_xor(gt, off);
+      eq += __shfl_xor(eq, off);
+    }
+    if (l == 0) {
+      sh->wave_gt[w] = gt;
+      sh->wave_eq[w] = eq;
+    }
+    __syncthreads();
+    uint32_t run = run_all, eq_run = eq_all;  // ... at lower indices than this wave's keys
+    {
+      uint32_t r = run_all, e_acc = eq_all;
+      for (int wv = 0; wv < NW; ++wv) {
+        if (wv == w) {
+          run = r;
+          eq_run = e_acc;
+        }
+        const uint32_t e = sh->wave_eq[wv];
+        const uint32_t left = remaining > e_acc ? remaining - e_acc : 0u;
+        r += sh->wave_gt[wv] + min(e, left);
+        e_acc += e;
+      }
+      run_all = r;
+      eq_all = e_acc;
+    }
+    const int wave_base = c0 + w * (256 * kSelLoads) + 4 * l;
+    // The comparisons below repeat the counting pass's; an opaque copy of the threshold keeps
+    // the compiler from carrying 128 lane masks from there to here in scalar registers.
+    uint32_t thr_e = thr;
+    asm volatile("" : "+v"(thr_e));
 #pragma unroll
-    for (int u = 0; u < 2; ++u) kk[u] = load4(i + u * 256 + 4 * l);
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int c0 = i + u * 256 + 4 * l;  // this lane's 4 consecutive indices
+    for (int u = 0; u < kSelLoads; ++u) {
+      const int i0 = wave_base + u * 256;  // this lane's 4 consecutive indices
       const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
       // Keys equal to the threshold are rare: rank them (lane-major, then j) only when there are any.
       bool is_eq[4];
       uint32_t eq_mine = 0;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        is_eq[j] = k4[j] == thr;
+        is_eq[j] = k4[j] == thr_e;
         eq_mine += is_eq[j] ? 1u : 0u;
       }
       uint32_t eq_before = eq_run;  // equal keys at lower indices
@@ -178,10 +210,10 @@ __device__ __forceinline__ void compact_winners(const uint32_t* keys, int n_keys
       uint32_t mine_eq_seen = 0;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        take[j] = k4[j] > thr || (is_eq[j] && eq_before + mine_eq_seen < remaining);
+        take[j] = k4[j] > thr_e || (is_eq[j] && eq_before + mine_eq_seen < remaining);
         mine_eq_seen += is_eq[j] ? 1u : 0u;
       }
-      uint32_t pos = run, total = 0;  // winners at lower indices
+      uint32_t pos = run, total = 0;  // winners at lower indices (lower lanes hold lower indices)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const unsigned long long bt = __ballot(take[j]);
@@ -191,32 +223,34 @@ __device__ __forceinline__ void compact_winners(const uint32_t* keys, int n_keys
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if (take[j]) {
-          emit((int)pos, c0 + j);
+          emit((int)pos, i0 + j);
           ++pos;
         }
       }
       run += total;
       eq_run += eq_total;
+      __builtin_amdgcn_sched_barrier(0);  // one load's ballots at a time: they live in scalar registers
     }
+    __syncthreads();  // wave_gt / wave_eq are rewritten by the next chunk
   }
 }
 
-// Streams the K plane of every page of the sequence once and calls
-// emit(c, score) -- from one lane per key row -- with score = (mean_g q_g) . k_c
-// in fp32 for every cache slot c of those pages (slots past the last token
-// included).  16-byte loads straight to registers, kU of them in flight per
+// Streams the K plane of the pages pg0 <= p < pg1 (pg0 a multiple of 4) of the
+// sequence once and calls emit(c, score, valid) from every lane; the calls with
+// valid == true, one per key row, carry score = (mean_g q_g) . k_c in fp32 for every cache slot c of
+// those pages (slots past the last token included).  emit must not branch around
+// vector memory operations (store through a descriptor, out of range when !valid).  16-byte loads straight to registers, 16 of them in flight per
 // lane; no LDS, no barrier.
 template <int NW, typename Emit>
-__device__ __forceinline__ void stream_token_scores(const TokenArgs& a, Emit emit) {
+__device__ __forceinline__ void stream_token_scores(const TokenArgs& a, int pg0, int pg1, Emit emit) {
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l = tid & 63, kg = l >> 4, c16 = l & 15;
   const int G = a.G;
-  const int n_pages = a.n_pages;
   const int32_t* table = a.table;
   // The mean over the group's heads of q_g . k_t is (mean_g q_g) . k_t: one dot
   // product per token.  Lane owns columns d = 8*(lane%16) .. +7 of the mean query;
-  // 16 lanes share a key row, a wave covers 4 rows, 4 waves one page.
+  // 16 lanes share a key row, one load instruction of a wave covers 4 rows.
   float qm[8];
   {
 #pragma unroll
@@ -233,82 +267,113 @@ __device__ __forceinline__ void stream_token_scores(const TokenArgs& a, Emit emi
 #pragma unroll
     for (int u = 0; u < 8; ++u) qm[u] *= inv;
   }
-  constexpr int kPP = NW / 4;   // pages one pass of the workgroup covers
-  constexpr int kU = 16;        // passes (16-byte loads per lane) kept in flight
+  // A wave streams whole K planes (4 KiB contiguous, four 16-byte loads per lane:
+  // load i covers key rows 4*i .. 4*i+3), four consecutive pages at a time: the
+  // quads pg0/4 + w, + NW, ... of the page range, the next quad in flight.  After
+  // a quad every lane holds one score -- lane (kg, c16) that of row 4*(c16%4) + kg
+  // of the quad's page c16/4 -- so one emit per quad covers 64 consecutive cache
+  // slots (256 B of keys: full lines, a quarter of the stores).
+  constexpr int kPF = 4;
   const __attribute__((address_space(4))) int32_t* tab_c =
       reinterpret_cast<const __attribute__((address_space(4))) int32_t*>(reinterpret_cast<uintptr_t>(table));
-  const int row = 4 * (w & 3) + kg;                 // key row of the page this lane helps with
-  const int voff = row * a.row_bytes + c16 * 16;
+  const int voff = kg * a.row_bytes + c16 * 16;
+  const int row_step = 4 * a.row_bytes;
   const int k_span = kPageSize * a.row_bytes - (a.span < a.page_bytes ? a.page_bytes - a.span : 0);  // K plane only
-  auto load_page = [&](int p) -> u32x4 {
+  auto load_page = [&](int p, u32x4 (&dst)[4]) {
     // Pages past the end (or with an id outside the cache) are read through an
     // empty descriptor: zeros, no memory traffic.
-    const bool in = p < n_pages;
+    const bool in = p < pg1;
     const int id = tab_c[in ? p : 0];
     const bool ok = in && id >= 0 && (int64_t)id < a.num_pages;
     const __amdgpu_buffer_rsrc_t r = make_rsrc(a.kvb + (int64_t)(ok ? id : 0) * a.page_bytes, ok ? k_span : 0);
-    return __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, kStreamLoad);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[i] = __builtin_amdgcn_raw_buffer_load_b128(r, voff + i * row_step, 0, kStreamLoad);
   };
-  const int p_first = w >> 2;  // this wave's page within a pass
-  u32x4 x[kU];
+  const int my_page = c16 >> 2, my_row = 4 * (c16 & 3) + kg;
+  const int first = pg0 + kPF * w;  // pg0 is a multiple of 4
+  u32x4 x[kPF][4];
 #pragma unroll
-  for (int u = 0; u < kU; ++u) x[u] = load_page(p_first + u * kPP);
-  for (int base = 0; base < n_pages; base += kU * kPP) {
+  for (int u = 0; u < kPF; ++u) {
+    load_page(first + u, x[u]);
+    // Issue order = consumption order: the wait at the top of the loop is sized for the worse
+    // of the two ways into it, and a reordered prologue would leave only a few loads in flight.
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  for (int base = first; base < pg1; base += kPF * NW) {
+    float mine = 0.f;
 #pragma unroll
-    for (int u = 0; u < kU; ++u) {
-      const u32x4 kx = x[u];
-      const int p = base + u * kPP + p_first;
-      x[u] = load_page(p + kU * kPP);
-      float acc = 0.f;
-      acc = fmaf(qm[0], bf16_lo(kx.x), acc); acc = fmaf(qm[1], bf16_hi(kx.x), acc);
-      acc = fmaf(qm[2], bf16_lo(kx.y), acc); acc = fmaf(qm[3], bf16_hi(kx.y), acc);
-      acc = fmaf(qm[4], bf16_lo(kx.z), acc); acc = fmaf(qm[5], bf16_hi(kx.z), acc);
-      acc = fmaf(qm[6], bf16_lo(kx.w), acc); acc = fmaf(qm[7], bf16_hi(kx.w), acc);
-      acc = row16_sum(acc);
-      const int c = p * kPageSize + row;
-      if (c16 == 0 && p < n_pages) emit(c, acc);
+    for (int u = 0; u < kPF; ++u) {
+      u32x4 kx[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) kx[i] = x[u][i];
+      load_page(base + kPF * NW + u, x[u]);
+      float acc[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float s = 0.f;
+        s = fmaf(qm[0], bf16_lo(kx[i].x), s); s = fmaf(qm[1], bf16_hi(kx[i].x), s);
+        s = fmaf(qm[2], bf16_lo(kx[i].y), s); s = fmaf(qm[3], bf16_hi(kx[i].y), s);
+        s = fmaf(qm[4], bf16_lo(kx[i].z), s); s = fmaf(qm[5], bf16_hi(kx[i].z), s);
+        s = fmaf(qm[6], bf16_lo(kx[i].w), s); s = fmaf(qm[7], bf16_hi(kx[i].w), s);
+        acc[i] = row16_sum(s);
+      }
+      const int i_mine = c16 & 3;
+      const float pick = i_mine == 0 ? acc[0] : i_mine == 1 ? acc[1] : i_mine == 2 ? acc[2] : acc[3];
+      if (my_page == u) mine = pick;
     }
+    // Called by every lane, without a branch: conditionally executed memory operations in
+    // this loop would keep the compiler from counting how many loads may stay in flight.
+    const int p = base + my_page;
+    emit(p * kPageSize + my_row, mine, p < pg1);
   }
 }
 
-// Token-level top-k: writes the token list (physical token ids) to a.list and
-// returns its length.  Every thread of the workgroup calls this; it ends with a
-// workgroup barrier.
-template <int NG, int NW>
-__device__ __forceinline__ int token_score_select(const TokenArgs& a) {
-  constexpr int NT = NW * 64;
-  __shared__ KeySelectShared sh_store;
-  KeySelectShared* sh = &sh_store;
-  uint32_t* hist = sh->hist;
+// Token-level top-k in three steps, so that the scoring of one sequence can be
+// shared by several workgroups: token_needs_scores() (false: the budget covers
+// every candidate, or is zero), token_score_keys() over a page range, and
+// token_select_list().
 
-  const int tid = threadIdx.x;
-  const int n_pages = a.n_pages;
+__device__ __forceinline__ bool token_needs_scores(const TokenArgs& a) {
   const int k_eff = min(a.topk, a.n_dyn);
+  return k_eff > 0 && k_eff < a.n_dyn;
+}
+
+// Scores the tokens of the pages pg0 <= p < pg1 into a.keys (device-scope stores;
+// 0 marks "not a candidate", order_key is never 0 for a finite score).  hist:
+// 256 zeroed LDS counters that receive the histogram of the keys' top byte, or
+// null.  No barrier inside; the stores are complete after s_waitcnt(0).
+template <int NW>
+__device__ __forceinline__ void token_score_keys(const TokenArgs& a, int pg0, int pg1, uint32_t* hist) {
   const int dyn_lo = a.pad + a.n_sink, dyn_hi = dyn_lo + a.n_dyn;  // cache slots of the candidates
-  const int n_keys = n_pages * kPageSize;
+  const __amdgpu_buffer_rsrc_t keys_rsrc = make_rsrc(a.keys, a.n_pages * kPageSize * 4);
+  stream_token_scores<NW>(a, pg0, pg1, [&](int c, float score, bool valid) {
+    const uint32_t key = (c >= dyn_lo && c < dyn_hi) ? order_key(score) : 0u;
+    // lanes without a row store at an offset outside the descriptor: dropped by the hardware
+    __builtin_amdgcn_raw_buffer_store_b32(key, keys_rsrc, valid ? c * 4 : -1, 0, kDeviceScope);
+    if (hist && valid && key) atomicAdd(&hist[key >> 24], 1u);
+  });
+}
+
+// Writes the token list (physical token ids) to a.list: sink tokens, the k
+// candidates with the largest keys in ascending position, local tokens; returns
+// its length.  When token_needs_scores(), a.keys is complete and, if
+// first_digit_counted, sh->hist holds the histogram of the keys' top byte.  Every
+// thread of the workgroup calls this; it ends with a workgroup barrier.
+template <int NG, int NW>
+__device__ __forceinline__ int token_select_list(const TokenArgs& a, KeySelectShared* sh, bool first_digit_counted) {
+  constexpr int NT = NW * 64;
+  const int tid = threadIdx.x;
+  const int k_eff = min(a.topk, a.n_dyn);
+  const int dyn_lo = a.pad + a.n_sink;
+  const int n_keys = a.n_pages * kPageSize;
   int32_t* list = a.list;
   const int32_t* table = a.table;
 
-  if (k_eff > 0 && k_eff < a.n_dyn) {
-    // ---- phase 1: group-mean logit of every token -> keys[], first radix digit counted on the fly
-    if (tid < 256) hist[tid] = 0;
+  if (token_needs_scores(a)) {
+    radix_select_emit<NW>(make_rsrc(a.keys, n_keys * 4), n_keys, (uint32_t)k_eff, first_digit_counted, sh,
+                          [&](int pos, int c) { list[a.n_sink + pos] = c; });
     __syncthreads();
-    stream_token_scores<NW>(a, [&](int c, float score) {
-      // 0 marks "not a candidate" (order_key is never 0 for a finite score)
-      const uint32_t key = (c >= dyn_lo && c < dyn_hi) ? order_key(score) : 0u;
-      a.keys[c] = key;
-      if (key) atomicAdd(&hist[key >> 24], 1u);
-    });
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();  // keys[] and hist[] complete and visible to the whole workgroup
-
-    // ---- phases 2 and 3: threshold, then the winners in ascending token order ----
-    uint32_t thr, remaining;
-    radix_threshold<NW>(a.keys, n_keys, (uint32_t)k_eff, true, sh, thr, remaining);
-    compact_winners<NW>(a.keys, n_keys, thr, remaining, sh, [&](int pos, int c) {
-      list[a.n_sink + pos] = phys_token(table, c);
-      if (a.sel_tokens) a.sel_tokens[a.n_sink + pos] = c - a.pad;
-    });
+    translate_slots<NT>(list, a.n_sink, k_eff, table, a.pad, a.sel_tokens);
   } else if (k_eff > 0) {
     // Budget covers every candidate: all of them, no key needed.
     for (int i = tid; i < k_eff; i += NT) {
@@ -336,20 +401,38 @@ struct StridedArgs {
   float* scores;         // HBM scratch, n_pages * 16 entries
   uint32_t* block_keys;  // HBM scratch, >= n_pages * 16 entries, 16-byte aligned
   uint32_t* bitmap;      // LDS, one bit per candidate token: (n_dyn + 31) / 32 words
+  int32_t* winners;      // LDS, room for 2 * topk_blocks block numbers
 };
 
 // Strided overlapping-block top-k: block i covers the candidate tokens
 // [i*stride, i*stride + block); the min(2*topk_blocks, num_blocks) blocks with the
 // largest mean score are chosen, their tokens united, and the topk_blocks*block
 // lowest-positioned of those kept.  With fewer candidates than one block every
-// token is listed.  Writes the token list to a.list (sink tokens, kept tokens in
-// ascending order, local tokens) and returns its length; ends with a barrier.
+// token is listed.  strided_needs_scores() / strided_score_tokens() over a page
+// range / strided_select_list(), as for the token policy.
+
+__device__ __forceinline__ bool strided_needs_scores(const TokenArgs& a, const StridedArgs& sa) {
+  if (a.n_dyn < sa.block || sa.topk_blocks <= 0) return false;
+  const int num_blocks = (a.n_dyn - sa.block) / sa.stride + 1;
+  return 2 * sa.topk_blocks < num_blocks;  // otherwise every block is chosen
+}
+
+// fp32 scores of the tokens of the pages pg0 <= p < pg1 -> sa.scores (device-scope stores).
+template <int NW>
+__device__ __forceinline__ void strided_score_tokens(const TokenArgs& a, const StridedArgs& sa, int pg0, int pg1) {
+  const __amdgpu_buffer_rsrc_t scores_rsrc = make_rsrc(sa.scores, a.n_pages * kPageSize * 4);
+  stream_token_scores<NW>(a, pg0, pg1, [&](int c, float score, bool valid) {
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(score), scores_rsrc, valid ? c * 4 : -1, 0, kDeviceScope);
+  });
+}
+
+// Writes the token list to a.list (sink tokens, kept tokens in ascending order,
+// local tokens) and returns its length; sa.scores is complete when
+// strided_needs_scores().  Ends with a barrier.
 template <int NG, int NW>
-__device__ __forceinline__ int strided_score_select(const TokenArgs& a, const StridedArgs& sa) {
+__device__ __forceinline__ int strided_select_list(const TokenArgs& a, const StridedArgs& sa, KeySelectShared* sh) {
   constexpr int NT = NW * 64;
-  __shared__ KeySelectShared sh_store;
   __shared__ uint32_t wave_cnt[NW];
-  KeySelectShared* sh = &sh_store;
   uint32_t* hist = sh->hist;
 
   const int tid = threadIdx.x;
@@ -374,25 +457,6 @@ __device__ __forceinline__ int strided_score_select(const TokenArgs& a, const St
     const int n_words = (L + 31) >> 5;
     for (int i = tid; i < n_words; i += NT) sa.bitmap[i] = 0u;
     if (tid < 256) hist[tid] = 0;
-    // ---- token scores -> HBM ------------------------------------------------
-    stream_token_scores<NW>(a, [&](int c, float score) { sa.scores[c] = score; });
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    // ---- block means -> keys (padded with "no candidate" to a multiple of 16) --
-    const int nb_pad = (num_blocks + 15) & ~15;
-    const float inv = 1.0f / (float)sa.block;
-    for (int i = tid; i < nb_pad; i += NT) {
-      uint32_t key = 0u;
-      if (i < num_blocks) {
-        const float* sp = sa.scores + dyn_lo + i * sa.stride;
-        float sum = 0.f;
-        for (int t = 0; t < sa.block; ++t) sum += sp[t];
-        key = order_key(sum * inv);
-        atomicAdd(&hist[key >> 24], 1u);
-      }
-      sa.block_keys[i] = key;
-    }
-    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     // ---- chosen blocks -> token bitmap ---------------------------------------
     auto mark_block = [&](int i) {
@@ -406,9 +470,28 @@ __device__ __forceinline__ int strided_score_select(const TokenArgs& a, const St
     if (k_blocks == 0) {
       // no budget: nothing of the dynamic part is attended
     } else if (k_blocks < num_blocks) {
-      uint32_t thr, remaining;
-      radix_threshold<NW>(sa.block_keys, nb_pad, (uint32_t)k_blocks, true, sh, thr, remaining);
-      compact_winners<NW>(sa.block_keys, nb_pad, thr, remaining, sh, [&](int, int i) { mark_block(i); });
+      // block means -> keys (padded with "no candidate" to a multiple of 16)
+      const int nb_pad = (num_blocks + 15) & ~15;
+      const float inv = 1.0f / (float)sa.block;
+      const __amdgpu_buffer_rsrc_t scores_rsrc = make_rsrc(sa.scores, a.n_pages * kPageSize * 4);
+      const __amdgpu_buffer_rsrc_t bkeys_rsrc = make_rsrc(sa.block_keys, nb_pad * 4);
+      for (int i = tid; i < nb_pad; i += NT) {
+        uint32_t key = 0u;
+        if (i < num_blocks) {
+          const int off = (dyn_lo + i * sa.stride) * 4;
+          float sum = 0.f;
+          for (int t = 0; t < sa.block; ++t)
+            sum += __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(scores_rsrc, off + t * 4, 0, kDeviceScope));
+          key = order_key(sum * inv);
+          atomicAdd(&hist[key >> 24], 1u);
+        }
+        __builtin_amdgcn_raw_buffer_store_b32(key, bkeys_rsrc, i * 4, 0, kDeviceScope);
+      }
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      radix_select_emit<NW>(bkeys_rsrc, nb_pad, (uint32_t)k_blocks, true, sh, [&](int pos, int i) { sa.winners[pos] = i; });
+      __syncthreads();
+      for (int i = tid; i < k_blocks; i += NT) mark_block(sa.winners[i]);
     } else {
       for (int i = tid; i < num_blocks; i += NT) mark_block(i);
     }
@@ -436,12 +519,13 @@ __device__ __forceinline__ int strided_score_select(const TokenArgs& a, const St
       while (bits && pos < (uint32_t)budget) {
         const int t = (i << 5) + __builtin_ctz(bits);
         bits &= bits - 1u;
-        list[a.n_sink + pos] = phys_token(table, dyn_lo + t);
-        if (a.sel_tokens) a.sel_tokens[a.n_sink + pos] = a.n_sink + t;
+        list[a.n_sink + pos] = dyn_lo + t;  // cache slot; translated below
         ++pos;
       }
     }
     kept = (int)min(total, (uint32_t)budget);
+    __syncthreads();
+    translate_slots<NT>(list, a.n_sink, kept, table, a.pad, a.sel_tokens);
   }
   for (int i = tid; i < a.n_sink + a.n_local; i += NT) {
     const bool sink = i < a.n_sink;

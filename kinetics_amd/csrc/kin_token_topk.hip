@@ -1,7 +1,10 @@
-// Token-level top-k sparse decode attention in one launch: one workgroup per
-// (sequence, KV head) scores every token of the context, keeps the sink tokens,
-// the local window and the top-k tokens in between, and attends to them
-// (token_score_select() + attend_tokens(), kin_token.h).
+// Token-level top-k sparse decode attention in one launch: for every (sequence,
+// KV head) every token of the context is scored, the sink tokens, the local
+// window and the top-k tokens in between are listed, and attended to
+// (token_score_keys() / token_select_list() / attend_tokens(), kin_token.h).
+// `chunks` workgroups share the scoring of one list, each a run of pages; the
+// last one to finish selects and attends.  Splitting keeps a few long lists from
+// leaving most of the GPU idle.
 #include "kin_token.h"
 
 namespace kin {
@@ -16,6 +19,8 @@ struct TokenTopkParams {
   int32_t* sel_count;   // optional [lists]
   uint16_t* out;
   float* lse;           // optional
+  int chunks;           // workgroups per list
+  int32_t* count;       // workspace: [lists] arrival counters, zero at launch and left zero
   uint32_t* keys;       // workspace: [lists, max_pages_per_seq * 16] (token keys, or block keys)
   float* scores;        // workspace, strided blocks only: [lists, max_pages_per_seq * 16]
   int block, stride;    // strided blocks only
@@ -35,11 +40,14 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ float sm_m[NW][4 * NG];
   __shared__ float sm_l[NW][4 * NG];
+  __shared__ KeySelectShared sh;
+  __shared__ int sh_last;
   constexpr int NT = NW * 64;
 
   const int tid = threadIdx.x;
+  const int list_id = blockIdx.x / p.chunks, chunk = blockIdx.x - list_id * p.chunks;
   int b, h;
-  if (!xcd_list_of(blockIdx.x, p.batch, p.num_kv_heads, b, h)) return;
+  if (!xcd_list_of(list_id, p.batch, p.num_kv_heads, b, h)) return;
   const int item = b * p.num_kv_heads + h;
   const int G = p.group;
   const int64_t hq0 = (int64_t)b * p.num_q_heads + (int64_t)h * G;
@@ -53,6 +61,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
   if (n_pages <= 0 || seq_len <= 0 || n_pages > p.max_pages_per_seq) {
     // Nothing to attend (or a sequence longer than the scratch array was sized for:
     // reported as count -1 rather than written past its end).
+    if (chunk) return;
     if (sel_out)
       for (int i = tid; i < p.sel_stride; i += NT) sel_out[i] = -1;
     if (p.sel_count && tid == 0) p.sel_count[item] = (n_pages > p.max_pages_per_seq) ? -1 : 0;
@@ -80,19 +89,47 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
   t.keys = p.keys + (int64_t)item * p.max_pages_per_seq * kPageSize;
   t.list = list;
   t.sel_tokens = sel_out;
-  int n;
+  StridedArgs sa;
   if (STRIDED) {
-    StridedArgs sa;
     sa.block = p.block;
     sa.stride = p.stride;
     sa.topk_blocks = p.topk;
     sa.scores = p.scores + (int64_t)item * p.max_pages_per_seq * kPageSize;
     sa.block_keys = t.keys;
     sa.bitmap = reinterpret_cast<uint32_t*>(list + p.list_cap);
-    n = strided_score_select<NG, NW>(t, sa);
-  } else {
-    n = token_score_select<NG, NW>(t);
+    // the K staging area is idle until the attention starts: 2 * topk_blocks <= 2 * kMaxTopkTokens
+    // block numbers fit its attend_lds_bytes(4) = 32 KiB
+    sa.winners = reinterpret_cast<int32_t*>(smem);
   }
+  const bool scored = STRIDED ? strided_needs_scores(t, sa) : token_needs_scores(t);
+  if (!scored && chunk) return;  // nothing to share: chunk 0 does the list alone
+  const bool hist_on_the_fly = !STRIDED && p.chunks == 1;
+  if (scored) {
+    const int per = ((n_pages + p.chunks - 1) / p.chunks + 3) & ~3;  // whole quads of pages
+    const int pg0 = min(chunk * per, n_pages), pg1 = min(pg0 + per, n_pages);
+    if (hist_on_the_fly) {
+      if (tid < 256) sh.hist[tid] = 0;
+      __syncthreads();
+    }
+    if (STRIDED) strided_score_tokens<NW>(t, sa, pg0, pg1);
+    else token_score_keys<NW>(t, pg0, pg1, hist_on_the_fly ? sh.hist : nullptr);
+    // Every wave waits for its own stores to be acknowledged; after the barrier the
+    // workgroup's scores are in memory.
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (p.chunks > 1) {
+      // The slices meet through memory without cache maintenance: scores and the
+      // arrival counter are written and read at device scope.  Whoever counts in
+      // last sees everybody's scores and carries on alone; the others are done.
+      if (tid == 0)
+        sh_last = (__hip_atomic_fetch_add(&p.count[item], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.chunks - 1)
+                      ? 1 : 0;
+      __syncthreads();
+      if (!sh_last) return;
+      if (tid == 0) __hip_atomic_store(&p.count[item], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+    }
+  }
+  const int n = STRIDED ? strided_select_list<NG, NW>(t, sa, &sh) : token_select_list<NG, NW>(t, &sh, hist_on_the_fly);
   if (sel_out)
     for (int i = n + tid; i < p.sel_stride; i += NT) sel_out[i] = -1;
   if (p.sel_count && tid == 0) p.sel_count[item] = n;
@@ -120,6 +157,26 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
 }  // namespace kin
 
 namespace kin {
+
+__global__ void token_fill_zero_kernel(int32_t* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// Bytes of the arrival counters in front of the score arrays.
+static size_t token_count_bytes(int64_t lists) { return ((size_t)lists * sizeof(int32_t) + 255) & ~(size_t)255; }
+
+// Workgroups that share the scoring of one list (each at least 256 pages = 1 MiB
+// of keys): as many as it takes to give every CU one when the lists are fewer than
+// the CUs, otherwise one -- with the GPU already full, splitting only adds
+// workgroups, the extra pass that recounts the first radix digit and a second
+// round of launches (measured: 6.35 -> 7.1 ms at 4096 lists of 32 K tokens).
+static int token_score_chunks(int64_t lists, int max_pages_per_seq) {
+  const int by_len = max_pages_per_seq / 256;
+  const int64_t want = kNumCus / lists;
+  if (by_len < 2 || want < 2) return 1;
+  return (int)(want < by_len ? want : by_len);
+}
 
 // Shared by the two entry points.  topk counts tokens (block == 0) or blocks.
 static int launch_token_policy(const char* fn, const kin_bf16_t* q, const kin_bf16_t* kv_cache,
@@ -164,8 +221,10 @@ static int launch_token_policy(const char* fn, const kin_bf16_t* q, const kin_bf
   if (sel_tokens && !sel_count) return fail(KIN_ERR_NULL_POINTER, "%s: sel_tokens given without sel_count", fn);
   if (!aligned16(q) || !aligned16(kv_cache) || !aligned16(out))
     return fail(KIN_ERR_MISALIGNED, "%s: q, kv_cache and out must be 16-byte aligned", fn);
-  const size_t key_bytes = kin_token_topk_workspace_bytes(batch, num_kv_heads, max_pages_per_seq);
-  const size_t need = strided ? 2 * key_bytes : key_bytes;
+  const int64_t items = (int64_t)batch * num_kv_heads;
+  const size_t count_bytes = token_count_bytes(items);
+  const size_t key_bytes = (size_t)items * max_pages_per_seq * kPageSize * sizeof(uint32_t);
+  const size_t need = count_bytes + (strided ? 2 * key_bytes : key_bytes);
   if (batch == 0) return KIN_OK;
   if (!workspace || workspace_bytes < need)
     return fail(KIN_ERR_WORKSPACE, "%s: needs %zu workspace bytes, got %zu", fn, need,
@@ -182,8 +241,10 @@ static int launch_token_policy(const char* fn, const kin_bf16_t* q, const kin_bf
   p.sel_count = sel_count;
   p.out = out;
   p.lse = lse;
-  p.keys = static_cast<uint32_t*>(workspace);
-  p.scores = strided ? reinterpret_cast<float*>(static_cast<char*>(workspace) + key_bytes) : nullptr;
+  p.count = static_cast<int32_t*>(workspace);
+  p.keys = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + count_bytes);
+  p.scores = strided ? reinterpret_cast<float*>(static_cast<char*>(workspace) + count_bytes + key_bytes) : nullptr;
+  p.chunks = token_score_chunks(items, max_pages_per_seq);
   p.block = block;
   p.stride = stride;
   p.list_cap = list_cap > 0 ? list_cap : 1;
@@ -201,11 +262,12 @@ static int launch_token_policy(const char* fn, const kin_bf16_t* q, const kin_bf
   const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
   p.scale_log2 = scale * 1.4426950408889634f;
 
-  const int64_t items = (int64_t)batch * num_kv_heads;
-  if (xcd_grid_size(batch, num_kv_heads) > 0x7fffffffLL)
-    return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
+  const int64_t grid = xcd_grid_size(batch, num_kv_heads) * p.chunks;
+  if (grid > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   // Waves per workgroup: 8 when the lists are too few to fill the GPU with 4-wave
-  // workgroups (the per-token addressing needs ~140 registers, so 16 do not fit).
+  // workgroups -- whatever the number of chunks: selection and attention are done by
+  // one workgroup per list (the per-token addressing needs ~140 registers, so 16 waves
+  // do not fit).
   const int nw = items <= 2 * kNumCus ? 8 : 4;
   const size_t bitmap_bytes = strided ? ((size_t)max_pages_per_seq * kPageSize / 32 + 1) * 4 : 0;
   const size_t lds = (size_t)attend_lds_bytes(nw) + (size_t)p.list_cap * 4 + bitmap_bytes;
@@ -233,10 +295,15 @@ static int launch_token_policy(const char* fn, const kin_bf16_t* q, const kin_bf
                    "hipFuncSetAttribute(token_topk_kernel)");
     if (st) return st;
   }
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  if (p.chunks > 1) {
+    // a kernel, not a memset node: this launch sequence may be captured into a HIP graph
+    token_fill_zero_kernel<<<(unsigned)((items + 255) / 256), 256, 0, hs>>>(p.count, (int)items);
+    st = check_hip(hipGetLastError(), "token_fill_zero_kernel launch");
+    if (st) return st;
+  }
   void* args[] = {&p};
-  return check_hip(hipLaunchKernel(kernel, dim3((unsigned)xcd_grid_size(batch, num_kv_heads)), dim3(nw * 64), args, lds,
-                                   static_cast<hipStream_t>(stream)),
-                   "token_topk_kernel launch");
+  return check_hip(hipLaunchKernel(kernel, dim3((unsigned)grid), dim3(nw * 64), args, lds, hs), "token_topk_kernel launch");
 }
 
 }  // namespace kin
@@ -245,11 +312,14 @@ extern "C" {
 
 size_t kin_token_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq) {
   if (batch <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0) return 0;
-  return (size_t)batch * num_kv_heads * max_pages_per_seq * kin::kPageSize * sizeof(uint32_t);
+  const int64_t lists = (int64_t)batch * num_kv_heads;
+  return kin::token_count_bytes(lists) + (size_t)lists * max_pages_per_seq * kin::kPageSize * sizeof(uint32_t);
 }
 
 size_t kin_strided_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq) {
-  return 2 * kin_token_topk_workspace_bytes(batch, num_kv_heads, max_pages_per_seq);
+  if (batch <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0) return 0;
+  const int64_t lists = (int64_t)batch * num_kv_heads;
+  return kin::token_count_bytes(lists) + 2 * (size_t)lists * max_pages_per_seq * kin::kPageSize * sizeof(uint32_t);
 }
 
 int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const int32_t* page_indices,

@@ -162,7 +162,7 @@ def test_token_topk_argument_errors(lib):
     assert tok(local=2000) == _lib.KIN_ERR_UNSUPPORTED
     assert tok(sel=A, cnt=A, stride=12) == _lib.KIN_ERR_BAD_SHAPE      # 8 + 4 + 1 entries needed
     assert tok(sel=A, stride=13) == _lib.KIN_ERR_NULL_POINTER
-    assert lib.kin_token_topk_workspace_bytes(2, 1, 4) == 2 * 4 * 16 * 4
+    assert lib.kin_token_topk_workspace_bytes(2, 1, 4) == 256 + 2 * 4 * 16 * 4  # arrival counters + keys
     assert tok(wsb=2 * 4 * 16 * 4 - 1) == _lib.KIN_ERR_WORKSPACE
     assert tok(ws=None) == _lib.KIN_ERR_WORKSPACE
     assert tok(P=1 << 28) == _lib.KIN_ERR_UNSUPPORTED                  # token ids would not fit 31 bits
@@ -179,7 +179,7 @@ def test_strided_topk_argument_errors(lib):
     assert strided(stride=0) == _lib.KIN_ERR_BAD_SHAPE
     assert strided(topk=300) == _lib.KIN_ERR_UNSUPPORTED              # 300 * 16 tokens > 4096
     assert strided(sel=A, cnt=A, sel_stride=36) == _lib.KIN_ERR_BAD_SHAPE   # 2 * 16 + 4 + 1 entries needed
-    assert lib.kin_strided_topk_workspace_bytes(2, 1, 4) == 2 * 2 * 4 * 16 * 4
+    assert lib.kin_strided_topk_workspace_bytes(2, 1, 4) == 256 + 2 * 2 * 4 * 16 * 4
     assert strided(wsb=2 * 2 * 4 * 16 * 4 - 1) == _lib.KIN_ERR_WORKSPACE
     assert strided(B=0) == _lib.KIN_OK
 

@@ -816,7 +816,7 @@ def _check_token_topk(ops, pb, topk, sink, local, offset, what):
     return lse.cpu().numpy()
 
 
-@pytest.mark.parametrize("case", ["mixed", "hkv8", "g8", "many", "offset", "all", "window_only"])
+@pytest.mark.parametrize("case", ["mixed", "hkv8", "g8", "many", "offset", "all", "window_only", "split", "split_many"])
 def test_token_topk_decode(ops, case):
     """LiteSys' token-level top-k (sparsity_utils.py:6-21): sink tokens, the
     top-k tokens of the middle by group-mean logit, the local window."""
@@ -839,6 +839,16 @@ def test_token_topk_decode(ops, case):
     elif case == "all":      # budget covers everything: dense
         pb = P.make_problem(1305, [PS * 5 + 2, 7], num_kv_heads=1, group=4)
         args = (4096, 4, 1, 0)
+    elif case == "split":    # few long lists: several workgroups score each (most of them idle for the short
+        # ones), 8 waves; the longest has more keys than the selecting workgroup holds in registers at once
+        pb = P.make_problem(1307, [PS * 2100 + 7, PS * 1030 + 16, PS * 300 + 1, 17], num_kv_heads=1, group=4)
+        args = (700, 4, 16, 0)
+    elif case == "split_many":  # > 512 lists (4 waves, no splitting), one of them with more keys than the
+        # selecting workgroup holds in registers at once
+        rng = np.random.default_rng(1308)
+        pb = P.make_problem(1308, [PS * 1100 + 3] + [int(x) for x in rng.integers(1, PS * 20, size=519)], num_kv_heads=1,
+                            group=4)
+        args = (40, 4, 8, 0)
     else:                    # topk = 0: sink + local window
         pb = P.make_problem(1306, [PS * 20 + 2, 40], num_kv_heads=2, group=1)
         args = (0, 4, 33, 0)
@@ -852,7 +862,7 @@ def test_token_topk_decode(ops, case):
         assert np.allclose(lse, want_lse, rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("case", ["mixed", "hkv8_stride4", "g8", "many", "offset", "stride16", "block8_stride3"])
+@pytest.mark.parametrize("case", ["mixed", "hkv8_stride4", "g8", "many", "offset", "stride16", "split", "block8_stride3"])
 def test_strided_topk_decode(ops, case):
     """LiteSys' strided overlapping-block policy (sparsity_utils.py:49-105)."""
     block, stride, offset = 16, 8, 0
@@ -875,6 +885,9 @@ def test_strided_topk_decode(ops, case):
     elif case == "stride16":  # disjoint blocks
         pb = P.make_problem(1505, [PS * 50 + 7, PS * 4], num_kv_heads=1, group=4)
         topk, sink, local, stride = 5, 4, 3, 16
+    elif case == "split":     # few long lists: several workgroups score each
+        pb = P.make_problem(1507, [PS * 1290 + 7, PS * 600 + 16, PS * 30 + 1], num_kv_heads=2, group=2)
+        topk, sink, local = 40, 4, 16
     else:
         pb = P.make_problem(1506, [PS * 33 + 1, 40, 19], num_kv_heads=2, group=1)
         topk, sink, local, block, stride = 9, 2, 5, 8, 3
@@ -942,12 +955,12 @@ def test_token_topk_rejects_short_workspace_and_long_sequences(ops):
 # --------------------------------------------------------------------------- graph capture / tracing
 
 
-@pytest.mark.parametrize("path", ["three", "fused", "fused_split", "token", "strided"])
+@pytest.mark.parametrize("path", ["three", "fused", "fused_split", "token", "strided", "token_split", "strided_split"])
 def test_step_replays_under_hip_graph(ops, path):
     """No allocation, no host sync, fixed buffers: every launch sequence can be
     captured once and replayed.  Every replay (with eager work and syncs in
     between) must equal the eager result for the inputs current at replay time."""
-    if path == "fused_split":   # few long sequences: fill kernel + several workgroups per list
+    if path.endswith("_split"):   # few long sequences: fill kernel + several workgroups per list
         pb = P.make_problem(801, [PS * 2300 + 3, PS * 2100 + 9], num_kv_heads=1, group=4, topk=32)
     else:
         pb = P.make_problem(800, [PS * 200 + 3] * 64, num_kv_heads=2, group=4, topk=32)
@@ -957,7 +970,7 @@ def test_step_replays_under_hip_graph(ops, path):
     step_ws = torch.empty(max(16, ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[1])), dtype=torch.uint8, device=DEV)
     tok_ws = torch.empty(max(16, ops.strided_topk_workspace_bytes(pb.B, pb.Hkv, pb.max_pages)), dtype=torch.uint8, device=DEV)
     tok_sel = torch.full((pb.B, pb.Hkv, 64 * 16 + 4 + 16), -1, dtype=torch.int32, device=DEV)
-    assert (path == "fused_split") == (ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[1]) > 0)
+    assert path.endswith("_split") == (ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[1]) > 0)
 
     def step():
         if path == "three":
@@ -969,7 +982,7 @@ def test_step_replays_under_hip_graph(ops, path):
                                       sel_pages=g.sel, sel_count=g.cnt, workspace=step_ws)
         else:
             ops.append_paged_kv(g.k, g.v, g.kv, None, g.indices, g.indptr, g.last)
-            if path == "token":
+            if path.startswith("token"):
                 ops.token_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, 300, pb.max_pages, local_tokens=16, out=out,
                                       sel_tokens=tok_sel, sel_count=g.cnt, workspace=tok_ws)
             else:
