@@ -423,6 +423,9 @@ def main():
         result["strided_topk"] = {"topk_blocks": topk, "block_size": PS, "stride": 8, "sink_tokens": sink,
                                   "local_tokens": window, "kernel_ms": ts * 1e3, "algorithmic_bytes_per_step": tok_bytes,
                                   "achieved_gbs": tok_bytes / ts / 1e9, "frac": tok_bytes / ts / 1e9 / HBM_PEAK_GBS}
+        if os.path.exists(tpath):
+            with open(tpath) as f:
+                result["strided_topk"]["traffic"] = json.load(f).get(f"{args.workload}:B={B}", {}).get("strided_topk_kernel")
         del ws_str
         del ws_tok
     del st

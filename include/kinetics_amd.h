@@ -311,8 +311,12 @@ size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages);
  * ascending order, local tokens -- padded with -1, and sel_count[b,h] = n
  * (-1 for a sequence with more than max_pages_per_seq pages, which is skipped:
  * out = 0).  workspace: kin_token_topk_workspace_bytes(...) bytes of scratch
- * (4 bytes per cache slot and KV head).  Reads every key of the context once:
- * HBM traffic is about half of dense decode's.
+ * (4 bytes per cache slot and KV head, plus an arrival counter per list; any
+ * contents, 16-byte aligned).  Reads every key of the context once: HBM
+ * traffic is about half of dense decode's.  When the lists are fewer than
+ * the GPU's compute units, several workgroups share the scoring of a list;
+ * a small kernel that zeroes the counters is then launched first on the
+ * same stream (no memset, so the call can be captured in a HIP graph).
  * Limits: topk_tokens <= 4096, sink_tokens <= 64, local_tokens <= 1024.
  */
 size_t kin_token_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq);
