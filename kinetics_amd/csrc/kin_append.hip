@@ -32,12 +32,15 @@ __global__ __launch_bounds__(256) void append_kernel(AppendParams p) {
                    p.page_indices[e - 1], p.last_page_len[b], n_pages, p.kbar_pages, h, p.num_kv_heads, p.num_pages, lane);
 }
 
-// grid = batch * Hkv * ceil(kbar_pages / 4) blocks (flat, so it is not bound by
-// the 65535 limit of grid.y); one wave per (sequence, head, logical page).
+// grid = batch * Hkv * ceil(kbar_pages / 16) blocks (flat, so it is not bound by
+// the 65535 limit of grid.y); 16 lanes per (sequence, head, logical page), a lane
+// owns 8 columns of all 16 key rows: 16 loads of 16 B in flight per lane, and the
+// same fp32 sum in slot order that page_mean_dword() makes, so a page's mean key
+// is bit-identical whether it is built here or by the append that fills the page.
 __global__ __launch_bounds__(256) void build_kbar_kernel(AppendParams p, int page_blocks) {
-  const int lane = threadIdx.x & 63;
+  const int sub = threadIdx.x >> 4, c16 = threadIdx.x & 15;
   const int item = blockIdx.x / page_blocks;
-  const int page = (blockIdx.x - item * page_blocks) * 4 + (threadIdx.x >> 6);
+  const int page = (blockIdx.x - item * page_blocks) * 16 + sub;
   const int b = item / p.num_kv_heads, h = item - b * p.num_kv_heads;
   const int s = p.page_indptr[b], e = p.page_indptr[b + 1];
   const int n_pages = e - s;
@@ -46,11 +49,29 @@ __global__ __launch_bounds__(256) void build_kbar_kernel(AppendParams p, int pag
   if (page >= n_full || page >= p.kbar_pages) return;
   const int64_t pid = p.page_indices[s + page];
   if (pid < 0 || pid >= p.num_pages) return;
-  const int row_stride = p.num_kv_heads * (kHeadDim / 2);
+  const int row_stride = p.num_kv_heads * (kHeadDim / 2);  // dwords per token row
   const int64_t page_dwords = 2LL * kPageSize * row_stride;
-  const uint32_t* kplane = p.kv_cache + pid * page_dwords + h * (kHeadDim / 2);
-  const uint32_t m = page_mean_dword(kplane, row_stride, lane);
-  p.kbar[(((int64_t)b * p.kbar_pages + page) * p.num_kv_heads + h) * (kHeadDim / 2) + lane] = m;
+  const u32x4* kplane = reinterpret_cast<const u32x4*>(p.kv_cache + pid * page_dwords + h * (kHeadDim / 2)) + c16;
+  u32x4 x[kPageSize];
+#pragma unroll
+  for (int t = 0; t < kPageSize; ++t) x[t] = __builtin_nontemporal_load(kplane + (int64_t)t * (row_stride / 4));
+  float acc[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) acc[u] = 0.f;
+#pragma unroll
+  for (int t = 0; t < kPageSize; ++t) {
+    acc[0] += bf16_lo(x[t].x); acc[1] += bf16_hi(x[t].x);
+    acc[2] += bf16_lo(x[t].y); acc[3] += bf16_hi(x[t].y);
+    acc[4] += bf16_lo(x[t].z); acc[5] += bf16_hi(x[t].z);
+    acc[6] += bf16_lo(x[t].w); acc[7] += bf16_hi(x[t].w);
+  }
+  const float inv = 1.0f / kPageSize;
+  u32x4 m;
+  m.x = f32_to_bf16(acc[0] * inv) | (f32_to_bf16(acc[1] * inv) << 16);
+  m.y = f32_to_bf16(acc[2] * inv) | (f32_to_bf16(acc[3] * inv) << 16);
+  m.z = f32_to_bf16(acc[4] * inv) | (f32_to_bf16(acc[5] * inv) << 16);
+  m.w = f32_to_bf16(acc[6] * inv) | (f32_to_bf16(acc[7] * inv) << 16);
+  reinterpret_cast<u32x4*>(p.kbar + (((int64_t)b * p.kbar_pages + page) * p.num_kv_heads + h) * (kHeadDim / 2))[c16] = m;
 }
 
 // ---- ragged multi-token append ------------------------------------------------
@@ -197,7 +218,7 @@ int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* 
   if (!aligned16(kbar)) return fail(KIN_ERR_MISALIGNED, "%s: kbar must be 16-byte aligned", fn);
   if (batch == 0) return KIN_OK;
   const int64_t items = (int64_t)batch * num_kv_heads;
-  const int page_blocks = (kbar_pages + 3) / 4;
+  const int page_blocks = (kbar_pages + 15) / 16;
   if (items * page_blocks > 0x7fffffffLL)
     return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads*kbar_pages too large for one launch", fn);
   AppendParams p;

@@ -38,8 +38,6 @@ constexpr int kWaitVm4 = 4 | (7 << 4) | (15 << 8);
 constexpr float kNegInf = -INFINITY;
 constexpr float kLn2 = 0.6931471805599453f;
 
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
 // Buffer descriptor covering `bytes` bytes from `base` (0 bytes: every load
 // through it returns zeros without touching memory).
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int bytes) {

@@ -41,6 +41,7 @@ constexpr int kDeviceScope = 16;
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte access: 8 bf16
 
 // ---- host side: status + thread-local message -----------------------------
 int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));

@@ -8,8 +8,6 @@
 
 namespace kin {
 
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte access: 8 bf16
-
 // 16-byte chunks one lane keeps in registers: a row of up to LPR * 8 * 16 elements.
 constexpr int kNormMaxChunks = 16;
 
