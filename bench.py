@@ -267,17 +267,21 @@ def main():
 
     fused = args.mode == "fused" or (args.mode == "auto" and ops.prefer_fused_step(B, Hkv, st["max_pages_used"], topk))
 
+    # few long lists: the scoring of a list is shared by several workgroups that meet through this
+    sws = ops.step_workspace_bytes(B, Hkv, st["kbar"].shape[1])
+    step_ws = torch.empty(sws, dtype=torch.uint8, device=device) if sws else None
+
     def launches():
         """The step's kernel launches, in order, as (name, callable)."""
         if fused:
             return [("fused_step", lambda: ops.blocktopk_decode_step(
                 st["q"], st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"], topk,
-                out=st["out"]))]
+                out=st["out"], workspace=step_ws))]
         return [
             ("append", lambda: ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"],
                                                    st["last"])),
             ("score_topk", lambda: ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], st["last"], topk,
-                                                        st["sel"], st["cnt"])),
+                                                        st["sel"], st["cnt"], workspace=step_ws)),
             ("sparse_attention", lambda: ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"],
                                                                  out=st["out"], workspace=st["ws"])),
         ]

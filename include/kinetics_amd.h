@@ -169,6 +169,12 @@ int kin_append_paged_kv_ragged(const kin_bf16_t* k, const kin_bf16_t* v,
  * 0 <= sink_pages <= 64, 1 <= local_tokens <= 1009,
  * sel_stride >= kin_sel_list_capacity(topk, sink_pages, local_tokens),
  * topk <= 2048, kbar_pages <= 16384.
+ * workspace: optional (NULL / 0 allowed), kin_step_workspace_bytes(batch,
+ * num_kv_heads, kbar_pages) bytes, 16-byte aligned, any contents.  With it, few
+ * long lists (that function returns non-zero for them) are scored by several
+ * workgroups per list, which meet through this memory; a small kernel that zeroes
+ * its counters is then launched first on the same stream.  Results do not depend
+ * on it.
  */
 int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
                          const int32_t* page_indices, const int32_t* page_indptr,
@@ -177,7 +183,8 @@ int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
                          int32_t* sel_pages, int32_t* sel_count,
                          int32_t* sel_logical, float* scores_out,
                          int batch, int num_q_heads, int num_kv_heads, int head_dim,
-                         int kbar_pages, int sel_stride, kin_stream_t stream);
+                         int kbar_pages, int sel_stride,
+                         void* workspace, size_t workspace_bytes, kin_stream_t stream);
 
 /*
  * Longest page list the selector can write for these settings:
@@ -282,7 +289,8 @@ int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const ki
                               kin_stream_t stream);
 
 /*
- * Workspace kin_blocktopk_decode_step can use for the given problem: 0 unless
+ * Workspace kin_blocktopk_decode_step and kin_block_score_topk can use for the
+ * given problem: 0 unless
  * the lists are few (batch * num_kv_heads <= 64) and long (kbar_pages >= 2048),
  * where the step spreads the scoring of each list over several workgroups that
  * meet through this memory (4 bytes per candidate page and an arrival counter

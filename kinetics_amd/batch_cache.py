@@ -195,7 +195,7 @@ class PagedBatchKVManager:
             if sparse:
                 ops.block_score_topk(self._q, kbar, self.page_indices, self.page_indptr, self.last_page_len,
                                      self.block_topk, self._sel, self._cnt, sink_pages=self.sink_pages,
-                                     local_tokens=self.local_tokens)
+                                     local_tokens=self.local_tokens, workspace=self._ws)
                 ops.sparse_paged_decode(self._q, kv, self._sel, self._cnt, self.last_page_len, out=self._out,
                                         workspace=self._ws, first_page_offset=self.pad)
             else:

@@ -57,6 +57,20 @@ int check_fixed_pages(const char* fn, int sink_pages, int local_tokens);
 // first_page_offset: padding slots at the start of every sequence's first page.
 int check_first_page_offset(const char* fn, int first_page_offset);
 
+// Split scoring of the page selector (few, long lists): workgroups per list.  1
+// unless the lists are at most a quarter of the CUs and long, then enough to put
+// a workgroup on every CU, each with at least 256 candidates.
+inline int score_chunks(int batch, int num_kv_heads, int kbar_pages) {
+  const int64_t items = (int64_t)batch * num_kv_heads;
+  if (items <= 0 || items * 4 > kNumCus || kbar_pages < 2048) return 1;
+  int64_t c = kNumCus / items;
+  const int64_t by_rows = kbar_pages / 256;
+  if (c > by_rows) c = by_rows;
+  return c < 2 ? 1 : (int)c;
+}
+// Bytes of the per-list arrival counters in front of the shared key array.
+inline size_t score_count_bytes(int64_t items) { return ((size_t)items * sizeof(int32_t) + 255) & ~(size_t)255; }
+
 // ---- device side -----------------------------------------------------------
 #if defined(__HIPCC__)
 
@@ -113,6 +127,14 @@ __device__ __forceinline__ float row16_sum(float x) {
 template <int I>
 __device__ __forceinline__ float quad_bcast(float x) {
   return dpp_f<(I) | (I << 2) | (I << 4) | (I << 6)>(x);
+}
+
+// Zeroes n int32 counters.  A kernel rather than a memset so that the launch
+// sequences that use it can be captured into a HIP graph.  (static: every
+// translation unit that launches it gets its own copy.)
+static __global__ __attribute__((unused)) void fill_zero_i32_kernel(int32_t* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

@@ -1,6 +1,8 @@
 // Stand-alone page scoring + top-k page selection kernel: one 256-thread
 // workgroup per (sequence, KV head) runs score_select() (kin_select.h) and
-// copies the page list to HBM.
+// copies the page list to HBM.  With few, long lists and a workspace, `chunks`
+// workgroups score a slice of one list's candidates each into global memory and
+// the last one to finish selects.
 #include "kin_select.h"
 
 namespace kin {
@@ -18,21 +20,27 @@ struct ScoreTopkParams {
   int batch, num_q_heads, num_kv_heads, group;
   int kbar_pages, sel_stride, topk, sink_pages, local_tokens;
   int sort_cap;
+  int chunks;          // workgroups per list
+  int32_t* ws_count;   // [lists] arrival counters, zero at launch and left zero
+  uint32_t* ws_keys;   // [lists, kbar_pages]
 };
 
 // Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap] | int32 sel[sink + topk + local]
 template <int UNROLL>
 __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  __shared__ int sh_last;
   const int tid = threadIdx.x;
+  const int list_id = blockIdx.x / p.chunks, chunk = blockIdx.x - list_id * p.chunks;
   int b, h;
-  if (!xcd_list_of(blockIdx.x, p.batch, p.num_kv_heads, b, h)) return;
+  if (!xcd_list_of(list_id, p.batch, p.num_kv_heads, b, h)) return;
   const int item = b * p.num_kv_heads + h;
 
   const int ps = p.page_indptr[b], pe = p.page_indptr[b + 1];
   const int n_pages = pe - ps;
   int32_t* sel = p.sel_pages + (int64_t)item * p.sel_stride;
   if (n_pages <= 0) {
+    if (chunk) return;
     for (int i = tid; i < p.sel_stride; i += kThreads) sel[i] = -1;
     if (tid == 0) p.sel_count[item] = 0;
     return;
@@ -55,7 +63,31 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
   a.keys = reinterpret_cast<uint32_t*>(smem);
   a.sortbuf = reinterpret_cast<unsigned long long*>(smem + (size_t)((p.kbar_pages + 3) & ~3) * 4);
   a.sort_cap = p.sort_cap;
-  const int n_list = score_select<UNROLL>(a, sel_lds);
+  int n_list;
+  if (p.chunks > 1) {
+    // This workgroup's slice of the candidates -> keys in global memory, written and
+    // (by the workgroup that counts in last) read at device scope: no cache
+    // maintenance, every wave waits for its own stores before the workgroup counts in.
+    uint32_t* gkeys = p.ws_keys + (int64_t)item * p.kbar_pages;
+    const int n_score = (min(a.topk, a.n_cand) > 0 || a.scores_out) ? a.n_cand : 0;
+    const int per = ((n_score + p.chunks - 1) / p.chunks + 63) & ~63;
+    const int r0 = min(chunk * per, n_score), r1 = min(r0 + per, n_score);
+    score_rows<UNROLL, kThreads, true>(a, r0, r1, gkeys);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0)
+      sh_last = (__hip_atomic_fetch_add(&p.ws_count[item], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.chunks - 1)
+                    ? 1 : 0;
+    __syncthreads();
+    if (!sh_last) return;
+    if (tid == 0) __hip_atomic_store(&p.ws_count[item], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+    for (int i = tid; i < n_score; i += kThreads)
+      a.keys[i] = __hip_atomic_load(gkeys + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    n_list = select_from_keys<kThreads>(a, sel_lds);
+  } else {
+    n_list = score_select<UNROLL>(a, sel_lds);
+  }
 
   for (int i = tid; i < p.sel_stride; i += kThreads) sel[i] = (i < n_list) ? sel_lds[i] : -1;
   if (tid == 0) p.sel_count[item] = n_list;
@@ -69,7 +101,7 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
                                     int32_t* sel_pages, int32_t* sel_count,
                                     int32_t* sel_logical, float* scores_out, int batch, int num_q_heads,
                                     int num_kv_heads, int head_dim, int kbar_pages, int sel_stride,
-                                    kin_stream_t stream) {
+                                    void* workspace, size_t workspace_bytes, kin_stream_t stream) {
   using namespace kin;
   const char* fn = "kin_block_score_topk";
   if (!q || !kbar || !page_indices || !page_indptr || !last_page_len || !sel_pages || !sel_count)
@@ -114,6 +146,24 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
   const int64_t items = (int64_t)batch * num_kv_heads;
   if (xcd_grid_size(batch, num_kv_heads) > 0x7fffffffLL)
     return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
+  // Few long lists: spread the scoring of each over several workgroups, given a workspace.
+  p.chunks = score_chunks(batch, num_kv_heads, kbar_pages);
+  const size_t ws_need = score_count_bytes(items) + (size_t)items * kbar_pages * sizeof(uint32_t);
+  if (p.chunks > 1 && workspace && aligned16(workspace) && workspace_bytes >= ws_need) {
+    p.ws_count = static_cast<int32_t*>(workspace);
+    p.ws_keys = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + score_count_bytes(items));
+  } else {
+    p.chunks = 1;
+    p.ws_count = nullptr;
+    p.ws_keys = nullptr;
+  }
+  const int64_t grid = xcd_grid_size(batch, num_kv_heads) * p.chunks;
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  if (p.chunks > 1) {
+    fill_zero_i32_kernel<<<(unsigned)((items + 255) / 256), 256, 0, hs>>>(p.ws_count, (int)items);
+    st = check_hip(hipGetLastError(), "fill_zero_i32_kernel launch");
+    if (st) return st;
+  }
   // Few workgroups cannot saturate HBM with 4 loads per lane in flight: give a
   // small grid 16 (more registers, which it can afford).
   const bool small_grid = items < 512;
@@ -126,8 +176,8 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
     if (st) return st;
   }
   if (small_grid)
-    score_topk_kernel<16><<<(unsigned)xcd_grid_size(batch, num_kv_heads), kThreads, lds, static_cast<hipStream_t>(stream)>>>(p);
+    score_topk_kernel<16><<<(unsigned)grid, kThreads, lds, hs>>>(p);
   else
-    score_topk_kernel<4><<<(unsigned)xcd_grid_size(batch, num_kv_heads), kThreads, lds, static_cast<hipStream_t>(stream)>>>(p);
+    score_topk_kernel<4><<<(unsigned)grid, kThreads, lds, hs>>>(p);
   return check_hip(hipGetLastError(), "score_topk_kernel launch");
 }

@@ -167,31 +167,12 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
       });
 }
 
-__global__ void fill_zero_kernel(int32_t* p, int n) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) p[i] = 0;
-}
-
-// Workgroups per list for the scoring phase: 1 unless the lists are few (at most a
-// quarter of the CUs) and long, then enough to put a workgroup on every CU, each
-// with at least 256 candidates.
-static int step_score_chunks(int batch, int num_kv_heads, int kbar_pages) {
-  const int64_t items = (int64_t)batch * num_kv_heads;
-  if (items <= 0 || items * 4 > kNumCus || kbar_pages < 2048) return 1;
-  int64_t c = kNumCus / items;
-  const int64_t by_rows = kbar_pages / 256;
-  if (c > by_rows) c = by_rows;
-  return c < 2 ? 1 : (int)c;
-}
-
-static size_t step_count_bytes(int64_t items) { return ((size_t)items * sizeof(int32_t) + 255) & ~(size_t)255; }
-
 }  // namespace kin
 
 extern "C" size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages) {
-  if (kin::step_score_chunks(batch, num_kv_heads, kbar_pages) <= 1) return 0;
+  if (kin::score_chunks(batch, num_kv_heads, kbar_pages) <= 1) return 0;
   const int64_t items = (int64_t)batch * num_kv_heads;
-  return kin::step_count_bytes(items) + (size_t)items * kbar_pages * sizeof(uint32_t);
+  return kin::score_count_bytes(items) + (size_t)items * kbar_pages * sizeof(uint32_t);
 }
 
 extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
@@ -268,11 +249,11 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
   else
     nw = items <= kNumCus ? 8 : 4;
   // Few long sequences: spread the scoring of each list over several workgroups.
-  p.chunks = step_score_chunks(batch, num_kv_heads, kbar_pages);
+  p.chunks = score_chunks(batch, num_kv_heads, kbar_pages);
   if (p.chunks > 1 && workspace && aligned16(workspace) &&
       workspace_bytes >= kin_step_workspace_bytes(batch, num_kv_heads, kbar_pages)) {
     p.ws_count = static_cast<int32_t*>(workspace);
-    p.ws_keys = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + step_count_bytes(items));
+    p.ws_keys = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + score_count_bytes(items));
   } else {
     p.chunks = 1;
     p.ws_count = nullptr;
@@ -305,8 +286,8 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
   unsigned grid = (unsigned)xcd_grid_size(batch, num_kv_heads);
   if (p.chunks > 1) {
     // the arrival counters start at zero (a fill kernel, so that the launch pair can be captured in a graph)
-    fill_zero_kernel<<<(unsigned)((items + 255) / 256), 256, 0, s>>>(p.ws_count, (int)items);
-    st = check_hip(hipGetLastError(), "fill_zero_kernel launch");
+    fill_zero_i32_kernel<<<(unsigned)((items + 255) / 256), 256, 0, s>>>(p.ws_count, (int)items);
+    st = check_hip(hipGetLastError(), "fill_zero_i32_kernel launch");
     if (st) return st;
     grid = (unsigned)(items * p.chunks);
   }

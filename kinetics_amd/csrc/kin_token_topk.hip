@@ -158,11 +158,6 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
 
 namespace kin {
 
-__global__ void token_fill_zero_kernel(int32_t* p, int n) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) p[i] = 0;
-}
-
 // Bytes of the arrival counters in front of the score arrays.
 static size_t token_count_bytes(int64_t lists) { return ((size_t)lists * sizeof(int32_t) + 255) & ~(size_t)255; }
 
@@ -298,8 +293,8 @@ static int launch_token_policy(const char* fn, const kin_bf16_t* q, const kin_bf
   hipStream_t hs = static_cast<hipStream_t>(stream);
   if (p.chunks > 1) {
     // a kernel, not a memset node: this launch sequence may be captured into a HIP graph
-    token_fill_zero_kernel<<<(unsigned)((items + 255) / 256), 256, 0, hs>>>(p.count, (int)items);
-    st = check_hip(hipGetLastError(), "token_fill_zero_kernel launch");
+    fill_zero_i32_kernel<<<(unsigned)((items + 255) / 256), 256, 0, hs>>>(p.count, (int)items);
+    st = check_hip(hipGetLastError(), "fill_zero_i32_kernel launch");
     if (st) return st;
   }
   void* args[] = {&p};

@@ -191,7 +191,7 @@ def sel_list_capacity(topk: int, sink_pages: int = 0, local_tokens: int = 1) -> 
 
 
 def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sel_logical=None,
-                     scores_out=None, sink_pages: int = 0, local_tokens: int = 1) -> None:
+                     scores_out=None, sink_pages: int = 0, local_tokens: int = 1, workspace=None) -> None:
     """Score every candidate page with the group-mean query and write the
     top-``topk`` pages plus the last page into ``sel_pages`` / ``sel_count``
     (in place: fixed buffers, as the reference registers with its decode
@@ -201,7 +201,9 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
     candidates (0 and 1 give the reference's "top-k plus the last page"; 1 and
     LiteSys' ``local`` on a cache stored 12 slots into its first page give
     LiteSys/litesys/attention/sparsity_utils.py:24-47).  List order: sink pages,
-    selected pages by descending score, local pages."""
+    selected pages by descending score, local pages.  ``workspace`` (uint8,
+    ``step_workspace_bytes``; optional) lets few, long sequences spread their
+    scoring over the GPU."""
     _require(q, "q", torch.bfloat16, 3)
     dev = q.device
     batch, num_q_heads, head_dim = q.shape
@@ -224,13 +226,15 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
         _require(scores_out, "scores_out", torch.float32, 3, dev)
         if tuple(scores_out.shape) != (batch, num_kv_heads, kbar_pages):
             raise ValueError(f"scores_out must be [{batch}, {num_kv_heads}, {kbar_pages}], got {tuple(scores_out.shape)}")
+    if workspace is not None:
+        _require(workspace, "workspace", torch.uint8, 1, dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
         _lib.check(
             lib.kin_block_score_topk(
                 _ptr(q), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), int(topk), int(sink_pages),
                 int(local_tokens), _ptr(sel_pages), _ptr(sel_count), _ptr(sel_logical), _ptr(scores_out), batch, num_q_heads, num_kv_heads, head_dim,
-                kbar_pages, sel_stride, _stream(dev),
+                kbar_pages, sel_stride, _ptr(workspace), workspace.numel() if workspace is not None else 0, _stream(dev),
             )
         )
 
@@ -641,7 +645,7 @@ torch.library.define(
 torch.library.define(
     "kinetics::block_score_topk",
     "(Tensor q, Tensor kbar, Tensor page_indices, Tensor page_indptr, Tensor last_page_len, int topk, "
-    "Tensor(a!) sel_pages, Tensor(b!) sel_count, int sink_pages=0, int local_tokens=1) -> ()",
+    "Tensor(a!) sel_pages, Tensor(b!) sel_count, int sink_pages=0, int local_tokens=1, Tensor(c!)? workspace=None) -> ()",
 )
 torch.library.define(
     "kinetics::sparse_paged_decode",
@@ -721,14 +725,14 @@ def _update_kv_fake(k, v, kv_append_indptr, kv_cache, kv_page_indices, kv_page_i
 
 @torch.library.impl("kinetics::block_score_topk", "cuda")
 def _select_impl(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sink_pages=0,
-                 local_tokens=1):
+                 local_tokens=1, workspace=None):
     block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count,
-                     sink_pages=sink_pages, local_tokens=local_tokens)
+                     sink_pages=sink_pages, local_tokens=local_tokens, workspace=workspace)
 
 
 @torch.library.register_fake("kinetics::block_score_topk")
 def _select_fake(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sink_pages=0,
-                 local_tokens=1):
+                 local_tokens=1, workspace=None):
     return None
 
 

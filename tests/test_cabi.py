@@ -74,7 +74,7 @@ def test_ragged_append_argument_errors(lib):
 def select(lib, q=A, kbar=A, idx=A, ptr=A, last=A, topk=4, sel=A, cnt=A, B=2, Hq=4, Hkv=1, D=128, kp=64, stride=5, sink=0,
            local=1):
     return lib.kin_block_score_topk(q, kbar, idx, ptr, last, topk, sink, local, sel, cnt, None, None, B, Hq, Hkv, D, kp,
-                                    stride, None)
+                                    stride, None, 0, None)
 
 
 def test_select_argument_errors(lib):
@@ -241,7 +241,7 @@ def test_auto_splits_policy(lib):
 
 def test_python_wrapper_maps_status_to_exceptions():
     with pytest.raises(ValueError, match="KIN_ERR_BAD_SHAPE"):
-        _lib.check(_lib.load().kin_block_score_topk(A, A, A, A, A, -1, 0, 1, A, A, None, None, 2, 4, 1, 128, 64, 5, None))
+        _lib.check(_lib.load().kin_block_score_topk(A, A, A, A, A, -1, 0, 1, A, A, None, None, 2, 4, 1, 128, 64, 5, None, 0, None))
     with pytest.raises(_lib.KineticsError, match="KIN_ERR_WORKSPACE"):
         _lib.check(sparse(_lib.load(), splits=3))
 

@@ -716,6 +716,22 @@ def test_fused_step_split_scoring_for_few_long_sequences(ops, hkv, group):
     c = Gpu(pb)
     out_c = ops.blocktopk_decode_step(c.q, c.k, c.v, c.kv, c.kbar, c.indices, c.indptr, c.last, pb.topk)
     assert torch.equal(out_c, out_a)
+    # the stand-alone selector splits the same way when it is given the workspace: same lists,
+    # same logical indices and scores as alone, call after call
+    one, two = Gpu(pb), Gpu(pb)
+    for g in (one, two):
+        g.kv.copy_(a.kv)
+        g.kbar.copy_(a.kbar)
+    ops.block_score_topk(one.q, one.kbar, one.indices, one.indptr, one.last, pb.topk, one.sel, one.cnt, one.logical, one.scores)
+    for _ in range(3):
+        two.sel.fill_(-9)
+        two.scores.fill_(float("nan"))
+        ops.block_score_topk(two.q, two.kbar, two.indices, two.indptr, two.last, pb.topk, two.sel, two.cnt, two.logical,
+                             two.scores, workspace=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(one.sel, two.sel) and torch.equal(one.cnt, two.cnt) and torch.equal(one.logical, two.logical)
+        assert torch.equal(one.scores.nan_to_num(7.0), two.scores.nan_to_num(7.0))
+    assert torch.equal(one.sel, a.sel)
 
 
 # --------------------------------------------------------------------------- ragged multi-token append
