@@ -1,20 +1,23 @@
 // Device-side building blocks of token-level top-k sparse decode attention for
-// one (sequence, KV head), run by one workgroup of NW waves:
+// one (sequence, KV head), run by workgroups of NW waves:
 //
-//   token_score_select()  streams every key of the sequence once (the K half of
-//       each page, 16-byte loads straight to registers; the mean over the
-//       group's heads of q_g . k_t is (mean_g q_g) . k_t, one fp32 dot product
-//       per token), turns the score of every token of the "dynamic" part
-//       (after the sink tokens, before the local window) into an
-//       order-preserving 32-bit key in an HBM scratch array, radix-selects the
-//       k-th largest key and compacts the winners, in ascending token order,
-//       into a token list in LDS: sink tokens, winners, local-window tokens;
+//   token_score_keys()    streams the K half of a run of the sequence's pages once
+//       (16-byte loads straight to registers; the mean over the group's heads of
+//       q_g . k_t is (mean_g q_g) . k_t, one fp32 dot product per token) and
+//       turns the score of every token of the "dynamic" part (after the sink
+//       tokens, before the local window) into an order-preserving 32-bit key in
+//       an HBM scratch array;
+//   token_select_list()   radix-selects the k-th largest key and compacts the
+//       winners, in ascending token order, into a token list in LDS: sink
+//       tokens, winners, local-window tokens;
+//   strided_score_tokens() / strided_select_list()   the same two steps for the
+//       strided overlapping-block policy (fp32 scores, block means, a bitmap);
 //   attend_tokens()       attention over such a list: the page loop of
 //       attend_list() with one address per token row instead of one per page.
 //
 // HBM-bound on the key stream: 256 B per context token, plus 512 B per listed
-// token; the scratch keys (4 B per token, re-read by the select passes) stay in
-// the cache hierarchy for the most part.
+// token; the scratch keys (4 B per token, written and read back at device scope
+// so that several workgroups can share the scoring of one sequence) add about 5 %.
 #pragma once
 
 #include "kin_attend.h"
