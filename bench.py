@@ -178,7 +178,8 @@ def cpu_baseline(torch, B_cpu, ctx, G, topk, budget_s=20.0):
                        f"{med * 1e3:.2f} ms/step; tokens/s is linear in batch")
 
 
-WHOLE_LAYER_MODEL = {"qwen3-8b-share": ("Qwen3-8B", 8), "qwen3-32b-share": ("Qwen3-32B", 8)}
+WHOLE_LAYER_MODEL = {"qwen3-8b-share": ("Qwen3-8B", 8), "qwen3-32b-share": ("Qwen3-32B", 8),
+                     "qwen3-8b-readme": ("Qwen3-8B", 8)}
 
 
 def whole_layer(torch, args, B, ctx, topk, device):
