@@ -36,6 +36,7 @@ WORKLOADS = {
     # name: (batch, ctx, H_kv, group, topk, description)
     "qwen3-8b-share": (4096, 32768, 1, 4, 128, "Qwen3-8B one-GPU share (TP=8): 1 KV head, 4 Q heads"),
     "qwen3-32b-share": (1024, 32768, 1, 8, 256, "Qwen3-32B one-GPU share: 1 KV head, 8 Q heads"),
+    "qwen3-8b-tp1": (512, 32768, 8, 4, 128, "Qwen3-8B unsharded attention: 8 KV heads, 32 Q heads"),
     "tiny": (8, 4096, 1, 4, 64, "CPU-runnable tiny case"),
     # the command in the reference's benchmark/README.md: --batch_size 256 --gen_len 32768 (ctx 16384) --topk_page 64
     "qwen3-8b-readme": (256, 16384, 1, 4, 64, "reference README example: Qwen3-8B share, B=256, ctx 16K, 64 pages"),
