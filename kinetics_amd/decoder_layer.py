@@ -98,17 +98,23 @@ class _LayerBase(nn.Module):
 
     def _gate_up_weight(self) -> torch.Tensor:
         """[2 * intermediate, hidden]: gate_proj over up_proj.  Built on first use
-        (and again after the module moved or changed dtype); the two parameters
-        then become views of it, so no weight is held twice and loading a state
-        dict into them keeps filling the stacked tensor."""
-        g, u = self.gate_proj.weight, self.up_proj.weight
+        (``prepare_wrapper`` or the first forward; again after the module moved or
+        changed dtype); the two parameters then become views of it, so no weight
+        is held twice and loading a state dict into them keeps filling the stacked
+        tensor."""
         w = self._gate_up
-        n = self.intermediate_size
-        if w is None or g.data_ptr() != w.data_ptr() or u.data_ptr() != w[n:].data_ptr() or g.dtype != w.dtype:
+        if w is None:
+            g, u = self.gate_proj.weight, self.up_proj.weight
+            n = self.intermediate_size
             w = torch.cat([g.data, u.data], dim=0)
             g.data, u.data = w[:n], w[n:]
             self._gate_up = w
         return w
+
+    def _apply(self, fn, recurse=True):
+        # .to() / .cuda() / .half() replace the parameters: the stacked weight is rebuilt on next use
+        self._gate_up = None
+        return super()._apply(fn, recurse)
 
     def graphed(self, example_hidden_states: torch.Tensor) -> GraphedLayer:
         """This layer's forward as one replayable HIP graph (see GraphedLayer)."""
@@ -119,9 +125,10 @@ class _LayerBase(nn.Module):
         bsz, q_len, _ = hidden_states.size()
         if q_len != 1:
             raise ValueError("decode layers take one token per sequence")
-        x = ops.rms_norm(hidden_states, self.input_layernorm_weight, self.eps)
+        x = torch.ops.kinetics.layer_norm(hidden_states, self.eps, self.input_layernorm_weight)
         qkv = self.wqkv(x).view(bsz, -1)
-        return ops.qkv_norm_split(qkv, self.qnorm_weight, self.knorm_weight, self.eps, self.num_heads, self.num_kv_heads)
+        return torch.ops.kinetics.qkv_norm_split(qkv, self.qnorm_weight, self.knorm_weight, self.eps, self.num_heads,
+                                                 self.num_kv_heads)
 
     def _finish(self, residual, o):
         """benchmark/blocktopk_decoder.py:226-240: wo, residual, norm, SwiGLU MLP, residual."""
@@ -129,10 +136,11 @@ class _LayerBase(nn.Module):
         # h = residual + wo(o), written over the projection's own output (the layer
         # input stays untouched), and x = norm(h) in the same pass
         h = self.wo(o.reshape(bsz, self.head_dim * self.num_heads))
-        x = ops.rms_norm(residual.reshape(bsz, self.dim), self.post_attention_layernorm_weight, self.eps, residual=h)
+        x = torch.ops.kinetics.fused_layer_norm(residual.reshape(bsz, self.dim), h, self.eps,
+                                                self.post_attention_layernorm_weight)
         n = self.intermediate_size
         gate_up = F.linear(x, self._gate_up_weight())
-        y = ops.gated_act(gate_up[:, :n], gate_up[:, n:], self.activation)
+        y = torch.ops.kinetics.gated_act(gate_up[:, :n], gate_up[:, n:], self.activation)
         return torch.addmm(h, y, self.down_proj.weight.t()).view(bsz, 1, self.dim)
 
 
@@ -174,7 +182,9 @@ class BlockTopkDecoderLayer(_LayerBase):
 
     def prepare_wrapper(self, prefix_len=None, topk_page_indices=None):
         """Present for call compatibility (benchmark/blocktopk_decoder.py:243-265): the
-        HIP kernels need no planning step."""
+        HIP kernels need no planning step.  Stacks the gate/up weights, so that a
+        compiled forward finds them in place."""
+        self._gate_up_weight()
         return None
 
     @torch.inference_mode()
@@ -193,6 +203,7 @@ class DenseDecoderLayer(_LayerBase):
                                         page_size, device=device, dtype=dtype, seed=seed)
 
     def prepare_wrapper(self):
+        self._gate_up_weight()
         return None
 
     @torch.inference_mode()

@@ -1207,6 +1207,14 @@ def test_decoder_layer_matches_fp32_reference(ops, dense):
     got = out.float().cpu()
     assert torch.allclose(got, want, rtol=5e-2, atol=5e-2), (got - want).abs().max()
     assert rms_norm(hidden, 1e-6, layer.input_layernorm_weight).dtype == torch.bfloat16
+    # the whole forward traces without a graph break (the reference compiles it with fullgraph=True,
+    # benchmark/blocktopk.py:41-43); backend "eager": no code generation, the same kernels run
+    compiled = torch.compile(layer.forward, backend="eager", fullgraph=True)
+    h_c = torch.randn(B, 1, 512, device=DEV).to(torch.bfloat16)
+    want_c = layer(h_c.clone()).clone()
+    got_c = compiled(h_c.clone())
+    torch.cuda.synchronize()
+    assert torch.equal(got_c, want_c)
     # the forward as one HIP graph: every replay equals the eager call on the same input,
     # with eager work and synchronisations between the replays
     graphed = layer.graphed(hidden)
