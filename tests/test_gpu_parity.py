@@ -953,6 +953,48 @@ def test_strided_topk_decode(ops, case):
     assert not np.isnan(lse.cpu().numpy()).any()
 
 
+@pytest.mark.parametrize("lists", [1, 2])
+def test_token_topk_ties_pick_the_lowest_positions(ops, lists):
+    """Equal scores are taken in ascending token position, also across the
+    register-sized chunks the selecting workgroup walks the keys in (more than
+    32768 keys at 8 waves) and across the workgroups that share the scoring."""
+    S = PS * 2100 + 7
+    pb = P.make_problem(1320 + lists, [S] * lists, num_kv_heads=1, group=4)
+    g = Gpu(pb)
+    ops.append_paged_kv(g.k, g.v, g.kv, None, g.indices, g.indptr, g.last)
+    # list 0: every key identical -> every candidate ties; list 1 (if any): two score levels, the
+    # higher one on every ninth token, fewer of them than the budget -> the rest by position
+    row = torch.randn(D, device=DEV).to(torch.bfloat16)
+    for b in range(lists):
+        pages = g.indices[int(pb.page_indptr[b]): int(pb.page_indptr[b + 1])].long()
+        g.kv[pages, 0] = row
+        if b == 1:
+            K = g.kv[pages, 0].reshape(-1, D)        # [slots, D] copy
+            K[::9] = row * 2
+            g.kv[pages, 0] = K.reshape(-1, PS, 1, D)
+    g.q[:] = row.float().sign().to(torch.bfloat16)   # q . row > 0: doubled rows score higher
+    topk, sink, local = 4000, 4, 16
+    sel = torch.full((lists, 1, topk + sink + local), -7, dtype=torch.int32, device=DEV)
+    cnt = torch.zeros(lists, 1, dtype=torch.int32, device=DEV)
+    ops.token_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, topk, pb.max_pages, sink_tokens=sink, local_tokens=local,
+                          sel_tokens=sel, sel_count=cnt)
+    torch.cuda.synchronize()
+    sel, cnt = sel.cpu().numpy(), cnt.cpu().numpy()
+    n_dyn = S - sink - local
+    for b in range(lists):
+        assert cnt[b, 0] == sink + topk + local
+        mid = sel[b, 0, sink: sink + topk]
+        if b == 0:
+            want = np.arange(sink, sink + topk)
+        else:
+            hi = np.arange(0, S, 9)
+            hi = hi[(hi >= sink) & (hi < sink + n_dyn)]
+            assert len(hi) < topk
+            lo = np.setdiff1d(np.arange(sink, sink + n_dyn), hi)[: topk - len(hi)]
+            want = np.sort(np.concatenate([hi, lo]))
+        assert np.array_equal(mid, want), f"list {b}: first difference at {np.flatnonzero(mid != want)[:5]}"
+
+
 def test_token_topk_rejects_short_workspace_and_long_sequences(ops):
     pb = P.make_problem(1310, [PS * 6 + 2, PS * 2], num_kv_heads=1, group=4)
     g = Gpu(pb)
