@@ -1013,7 +1013,8 @@ def test_token_topk_rejects_short_workspace_and_long_sequences(ops):
 # --------------------------------------------------------------------------- graph capture / tracing
 
 
-@pytest.mark.parametrize("path", ["three", "fused", "fused_split", "token", "strided", "token_split", "strided_split"])
+@pytest.mark.parametrize("path", ["three", "three_split", "fused", "fused_split", "token", "strided", "token_split",
+                                  "strided_split"])
 def test_step_replays_under_hip_graph(ops, path):
     """No allocation, no host sync, fixed buffers: every launch sequence can be
     captured once and replayed.  Every replay (with eager work and syncs in
@@ -1031,9 +1032,9 @@ def test_step_replays_under_hip_graph(ops, path):
     assert path.endswith("_split") == (ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[1]) > 0)
 
     def step():
-        if path == "three":
+        if path in ("three", "three_split"):
             ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
-            ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, pb.topk, g.sel, g.cnt)
+            ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, pb.topk, g.sel, g.cnt, workspace=step_ws)
             ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, out=out, workspace=ws)
         elif path in ("fused", "fused_split"):
             ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, pb.topk, out=out,
