@@ -116,8 +116,9 @@ int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar,
  * position kv_len_b - n_b + i, kv_len_b = 16*(n_pages_b-1) + last_page_len[b].
  * When kbar is given, the mean key of every page the append completed is
  * (re)computed, with the arithmetic of kin_append_paged_kv.  max_append_len is
- * an upper bound on n_b (nnz always works; a tighter bound launches fewer idle
- * workgroups).  Sequences whose metadata is out of contract are skipped.
+ * an upper bound on n_b, 0 <= max_append_len <= nnz (checked; the launches are
+ * sized by nnz alone, so nnz is as good a value as any).  Sequences whose
+ * metadata is out of contract are skipped.
  */
 int kin_append_paged_kv_ragged(const kin_bf16_t* k, const kin_bf16_t* v,
                                const int32_t* append_indptr,

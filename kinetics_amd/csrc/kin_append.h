@@ -22,6 +22,34 @@ __device__ __forceinline__ uint32_t page_mean_dword(const uint32_t* krow, int ro
   return f32_to_bf16(s0 * inv) | (f32_to_bf16(s1 * inv) << 16);
 }
 
+// The same mean for 8 columns at once: `kplane16` points at this lane's 16 bytes of
+// slot 0 (lane c16 of 16 owns columns 8*c16 .. 8*c16+7), `row_stride16` is the
+// distance between token rows in 16-byte units.  All 16 loads are in flight
+// together; the sums run in slot order 0,1,...,15 like page_mean_dword(), so both
+// give the same bits.
+__device__ __forceinline__ u32x4 page_mean_16B(const u32x4* kplane16, int row_stride16) {
+  u32x4 x[kPageSize];
+#pragma unroll
+  for (int t = 0; t < kPageSize; ++t) x[t] = __builtin_nontemporal_load(kplane16 + (int64_t)t * row_stride16);
+  float acc[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) acc[u] = 0.f;
+#pragma unroll
+  for (int t = 0; t < kPageSize; ++t) {
+    acc[0] += bf16_lo(x[t].x); acc[1] += bf16_hi(x[t].x);
+    acc[2] += bf16_lo(x[t].y); acc[3] += bf16_hi(x[t].y);
+    acc[4] += bf16_lo(x[t].z); acc[5] += bf16_hi(x[t].z);
+    acc[6] += bf16_lo(x[t].w); acc[7] += bf16_hi(x[t].w);
+  }
+  const float inv = 1.0f / kPageSize;
+  u32x4 m;
+  m.x = f32_to_bf16(acc[0] * inv) | (f32_to_bf16(acc[1] * inv) << 16);
+  m.y = f32_to_bf16(acc[2] * inv) | (f32_to_bf16(acc[3] * inv) << 16);
+  m.z = f32_to_bf16(acc[4] * inv) | (f32_to_bf16(acc[5] * inv) << 16);
+  m.w = f32_to_bf16(acc[6] * inv) | (f32_to_bf16(acc[7] * inv) << 16);
+  return m;
+}
+
 // Run by the 64 lanes of one wave (lane = 0..63, 4 bytes each = one 256-byte row).
 // k_row / v_row: the new token's rows for this (sequence, head), in dwords.
 // The row lands in slot last_len-1 of the sequence's last page (physical id

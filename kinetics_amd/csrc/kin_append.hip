@@ -1,6 +1,6 @@
-// Paged KV append with per-page mean-key maintenance, and the bulk mean-key
-// builder.  Both are byte movers: one 64-lane wave moves one 256-byte head row
-// per instruction (4 bytes per lane), so every access is a full-row burst.
+// Paged KV append with per-page mean-key maintenance (one token per sequence, or
+// a ragged run of tokens per sequence), and the bulk mean-key builder.  All are
+// byte movers.
 #include "kin_append.h"
 
 namespace kin {
@@ -52,25 +52,7 @@ __global__ __launch_bounds__(256) void build_kbar_kernel(AppendParams p, int pag
   const int row_stride = p.num_kv_heads * (kHeadDim / 2);  // dwords per token row
   const int64_t page_dwords = 2LL * kPageSize * row_stride;
   const u32x4* kplane = reinterpret_cast<const u32x4*>(p.kv_cache + pid * page_dwords + h * (kHeadDim / 2)) + c16;
-  u32x4 x[kPageSize];
-#pragma unroll
-  for (int t = 0; t < kPageSize; ++t) x[t] = __builtin_nontemporal_load(kplane + (int64_t)t * (row_stride / 4));
-  float acc[8];
-#pragma unroll
-  for (int u = 0; u < 8; ++u) acc[u] = 0.f;
-#pragma unroll
-  for (int t = 0; t < kPageSize; ++t) {
-    acc[0] += bf16_lo(x[t].x); acc[1] += bf16_hi(x[t].x);
-    acc[2] += bf16_lo(x[t].y); acc[3] += bf16_hi(x[t].y);
-    acc[4] += bf16_lo(x[t].z); acc[5] += bf16_hi(x[t].z);
-    acc[6] += bf16_lo(x[t].w); acc[7] += bf16_hi(x[t].w);
-  }
-  const float inv = 1.0f / kPageSize;
-  u32x4 m;
-  m.x = f32_to_bf16(acc[0] * inv) | (f32_to_bf16(acc[1] * inv) << 16);
-  m.y = f32_to_bf16(acc[2] * inv) | (f32_to_bf16(acc[3] * inv) << 16);
-  m.z = f32_to_bf16(acc[4] * inv) | (f32_to_bf16(acc[5] * inv) << 16);
-  m.w = f32_to_bf16(acc[6] * inv) | (f32_to_bf16(acc[7] * inv) << 16);
+  const u32x4 m = page_mean_16B(kplane, row_stride / 4);
   reinterpret_cast<u32x4*>(p.kbar + (((int64_t)b * p.kbar_pages + page) * p.num_kv_heads + h) * (kHeadDim / 2))[c16] = m;
 }
 
@@ -99,62 +81,122 @@ __device__ __forceinline__ int owner_of_row(const int32_t* indptr, int batch, in
   return lo;
 }
 
-// grid = ceil(nnz*Hkv / 4) blocks of 256 threads; one wave per (appended row, head).
-// The page table describes the cache after the append: row i of sequence b's n_b
-// new rows lands at token position kv_len_b - n_b + i.
+constexpr int kRaggedRows = 32;  // appended token rows one workgroup moves
+
+// grid = ceil(nnz / kRaggedRows) blocks of 256 threads.  A token's K row over all
+// heads is one contiguous run of Hkv*256 bytes in k[] and in its page slot (and
+// likewise V), so the workgroup's rows are moved as 16-byte chunks, several in
+// flight per thread; where each row goes is worked out once per row (threads
+// 0..31) and handed over in LDS.  The page table describes the cache after the
+// append: row i of sequence b's n_b new rows lands at token position
+// kv_len_b - n_b + i.
 __global__ __launch_bounds__(256) void append_ragged_kernel(RaggedAppendParams p) {
-  const int lane = threadIdx.x & 63;
-  const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (item >= p.nnz * p.num_kv_heads) return;
-  const int64_t row = item / p.num_kv_heads;
-  const int h = (int)(item - row * p.num_kv_heads);
-  const int b = owner_of_row(p.append_indptr, p.batch, row);
-  const int a0 = p.append_indptr[b], a1 = p.append_indptr[b + 1];
-  if (row < a0 || row >= a1) return;  // malformed indptr
-  const int s = p.page_indptr[b], e = p.page_indptr[b + 1];
-  const int n_pages = e - s;
-  const int last = p.last_page_len[b];
-  if (n_pages <= 0 || last < 1 || last > kPageSize) return;
-  const int64_t kv_len = (int64_t)(n_pages - 1) * kPageSize + last;
-  const int64_t pos = kv_len - (a1 - a0) + (row - a0);
-  if (pos < 0) return;  // more rows than the sequence holds: out of contract
-  const int64_t pid = p.page_indices[s + (int)(pos / kPageSize)];
-  if (pid < 0 || pid >= p.num_pages) return;
-  const int slot = (int)(pos % kPageSize);
-  const int row_stride = p.num_kv_heads * (kHeadDim / 2);
-  const int64_t page_dwords = 2LL * kPageSize * row_stride;
-  uint32_t* kplane = p.kv_cache + pid * page_dwords + h * (kHeadDim / 2);
-  uint32_t* vplane = kplane + (int64_t)kPageSize * row_stride;
-  const int64_t src = item * (kHeadDim / 2) + lane;
-  kplane[(int64_t)slot * row_stride + lane] = p.k[src];
-  vplane[(int64_t)slot * row_stride + lane] = p.v[src];
+  __shared__ int64_t dst16[kRaggedRows];  // K destination of the row in 16-byte units, -1: skip
+  const int tid = threadIdx.x;
+  const int64_t row0 = (int64_t)blockIdx.x * kRaggedRows;
+  const int rows_here = (int)min((int64_t)kRaggedRows, p.nnz - row0);
+  const int cpr = p.num_kv_heads * (kHeadDim / 8);  // 16-byte chunks per token row (all heads)
+  if (tid < kRaggedRows) {
+    int64_t dst = -1;
+    const int64_t row = row0 + tid;
+    if (tid < rows_here) {
+      const int b = owner_of_row(p.append_indptr, p.batch, row);
+      const int a0 = p.append_indptr[b], a1 = p.append_indptr[b + 1];
+      const int s = p.page_indptr[b], e = p.page_indptr[b + 1];
+      const int n_pages = e - s;
+      const int last = p.last_page_len[b];
+      // rows outside their sequence's range (malformed indptr) or contract are skipped
+      if (row >= a0 && row < a1 && n_pages > 0 && last >= 1 && last <= kPageSize) {
+        const int64_t kv_len = (int64_t)(n_pages - 1) * kPageSize + last;
+        const int64_t pos = kv_len - (a1 - a0) + (row - a0);
+        if (pos >= 0) {
+          const int64_t pid = p.page_indices[s + (int)(pos / kPageSize)];
+          if (pid >= 0 && pid < p.num_pages) dst = (pid * 2 * kPageSize + (pos % kPageSize)) * cpr;
+        }
+      }
+    }
+    dst16[tid] = dst;
+  }
+  __syncthreads();
+  const u32x4* ksrc = reinterpret_cast<const u32x4*>(p.k) + row0 * cpr;
+  const u32x4* vsrc = reinterpret_cast<const u32x4*>(p.v) + row0 * cpr;
+  u32x4* cache = reinterpret_cast<u32x4*>(p.kv_cache);
+  const int64_t v_plane = (int64_t)kPageSize * cpr;  // V plane of a page follows its K plane
+  const int total = rows_here * cpr;
+  constexpr int kU = 4;
+  for (int base = tid; base < total; base += 256 * kU) {
+    u32x4 kk[kU], vv[kU];
+    int64_t d[kU];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      const int c = base + u * 256;
+      d[u] = -1;
+      if (c < total) {
+        const int r = c / cpr;
+        const int64_t dr = dst16[r];
+        if (dr >= 0) d[u] = dr + (c - r * cpr);
+        kk[u] = __builtin_nontemporal_load(ksrc + c);
+        vv[u] = __builtin_nontemporal_load(vsrc + c);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      if (d[u] >= 0) {
+        cache[d[u]] = kk[u];
+        cache[d[u] + v_plane] = vv[u];
+      }
+    }
+  }
 }
 
-// Mean keys of the pages an append completed.  grid = batch*Hkv*page_blocks blocks;
-// one wave per (sequence, head, j-th page touched by the append).  Runs after
+// Mean keys of the pages an append completed: the pages that received an appended
+// row in their last slot.  Same grid and row bookkeeping as append_ragged_kernel
+// (so its cost follows the number of appended rows, whatever their split over the
+// sequences); 16 lanes per (completed page, head).  Runs after
 // append_ragged_kernel on the same stream.
-__global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p, int page_blocks) {
-  const int lane = threadIdx.x & 63;
-  const int item = blockIdx.x / page_blocks;
-  const int j = (blockIdx.x - item * page_blocks) * 4 + (threadIdx.x >> 6);
-  const int b = item / p.num_kv_heads, h = item - b * p.num_kv_heads;
-  const int n_new = p.append_indptr[b + 1] - p.append_indptr[b];
-  const int s = p.page_indptr[b], e = p.page_indptr[b + 1];
-  const int n_pages = e - s;
-  const int last = p.last_page_len[b];
-  if (n_new <= 0 || n_pages <= 0 || last < 1 || last > kPageSize) return;
-  const int64_t kv_len = (int64_t)(n_pages - 1) * kPageSize + last;
-  const int64_t first_pos = kv_len - n_new;
-  if (first_pos < 0) return;
-  const int64_t page = first_pos / kPageSize + j;         // j-th page the append wrote into
-  if (page >= kv_len / kPageSize || page >= p.kbar_pages) return;  // not full (or no slot for its mean key)
-  const int64_t pid = p.page_indices[s + (int)page];
-  if (pid < 0 || pid >= p.num_pages) return;
-  const int row_stride = p.num_kv_heads * (kHeadDim / 2);
-  const int64_t page_dwords = 2LL * kPageSize * row_stride;
-  const uint32_t* kplane = p.kv_cache + pid * page_dwords + h * (kHeadDim / 2);
-  const uint32_t m = page_mean_dword(kplane, row_stride, lane);
-  p.kbar[(((int64_t)b * p.kbar_pages + page) * p.num_kv_heads + h) * (kHeadDim / 2) + lane] = m;
+__global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p) {
+  __shared__ int64_t src16[kRaggedRows];  // K plane of the page a row completed, in 16-byte units; -1: none
+  __shared__ int64_t dst16[kRaggedRows];  // its mean-key row for head 0, in 16-byte units
+  const int tid = threadIdx.x;
+  const int64_t row0 = (int64_t)blockIdx.x * kRaggedRows;
+  const int rows_here = (int)min((int64_t)kRaggedRows, p.nnz - row0);
+  const int cpr = p.num_kv_heads * (kHeadDim / 8);
+  if (tid < kRaggedRows) {
+    int64_t src = -1, dst = 0;
+    const int64_t row = row0 + tid;
+    if (tid < rows_here) {
+      const int b = owner_of_row(p.append_indptr, p.batch, row);
+      const int a0 = p.append_indptr[b], a1 = p.append_indptr[b + 1];
+      const int s = p.page_indptr[b], e = p.page_indptr[b + 1];
+      const int n_pages = e - s;
+      const int last = p.last_page_len[b];
+      if (row >= a0 && row < a1 && n_pages > 0 && last >= 1 && last <= kPageSize) {
+        const int64_t kv_len = (int64_t)(n_pages - 1) * kPageSize + last;
+        const int64_t pos = kv_len - (a1 - a0) + (row - a0);
+        const int64_t page = pos / kPageSize;
+        if (pos >= 0 && pos % kPageSize == kPageSize - 1 && page < p.kbar_pages) {
+          const int64_t pid = p.page_indices[s + (int)page];
+          if (pid >= 0 && pid < p.num_pages) {
+            src = pid * 2 * kPageSize * cpr;
+            dst = (((int64_t)b * p.kbar_pages + page) * p.num_kv_heads) * (kHeadDim / 8);
+          }
+        }
+      }
+    }
+    src16[tid] = src;
+    dst16[tid] = dst;
+  }
+  __syncthreads();
+  const int sub = tid >> 4, c16 = tid & 15;
+  const u32x4* cache = reinterpret_cast<const u32x4*>(p.kv_cache);
+  u32x4* kbar = reinterpret_cast<u32x4*>(p.kbar);
+  for (int pair = sub; pair < rows_here * p.num_kv_heads; pair += 16) {
+    const int r = pair / p.num_kv_heads, h = pair - r * p.num_kv_heads;
+    const int64_t src = src16[r];
+    if (src < 0) continue;
+    const u32x4 m = page_mean_16B(cache + src + h * (kHeadDim / 8) + c16, cpr);
+    kbar[dst16[r] + h * (kHeadDim / 8) + c16] = m;
+  }
 }
 
 static int check_append_args(const char* fn, const void* kv_cache, const void* page_indices,
@@ -254,13 +296,8 @@ int kin_append_paged_kv_ragged(const kin_bf16_t* k, const kin_bf16_t* v, const i
   if (!aligned16(k) || !aligned16(v) || (kbar && !aligned16(kbar)))
     return fail(KIN_ERR_MISALIGNED, "%s: k, v and kbar must be 16-byte aligned", fn);
   if (batch == 0 || nnz == 0) return KIN_OK;
-  const int64_t items = nnz * num_kv_heads;
-  const int64_t blocks = (items + 3) / 4;
-  // pages one sequence's append can touch: a partial page in front plus the pages its rows fill
-  const int page_blocks = ((max_append_len + kPageSize - 1) / kPageSize + 1 + 3) / 4;
-  const int64_t lists = (int64_t)batch * num_kv_heads;
-  if (blocks > 0x7fffffffLL || lists * page_blocks > 0x7fffffffLL)
-    return fail(KIN_ERR_UNSUPPORTED, "%s: problem too large for one launch", fn);
+  const int64_t blocks = (nnz + kRaggedRows - 1) / kRaggedRows;
+  if (blocks > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: problem too large for one launch", fn);
   RaggedAppendParams p;
   p.k = reinterpret_cast<const uint32_t*>(k);
   p.v = reinterpret_cast<const uint32_t*>(v);
@@ -279,7 +316,7 @@ int kin_append_paged_kv_ragged(const kin_bf16_t* k, const kin_bf16_t* v, const i
   append_ragged_kernel<<<(unsigned)blocks, 256, 0, s>>>(p);
   st = check_hip(hipGetLastError(), "append_ragged_kernel launch");
   if (st || !kbar) return st;
-  refresh_kbar_kernel<<<(unsigned)(lists * page_blocks), 256, 0, s>>>(p, page_blocks);
+  refresh_kbar_kernel<<<(unsigned)blocks, 256, 0, s>>>(p);
   return check_hip(hipGetLastError(), "refresh_kbar_kernel launch");
 }
 

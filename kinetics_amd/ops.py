@@ -132,7 +132,7 @@ def append_paged_kv_ragged(k, v, append_indptr, kv_cache, kbar, page_indices, pa
     ``mylib::update_kv`` (benchmark/blocktopk_decoder.py:23-46) and the paged
     counterpart of LiteSys' prefill write (batch_cache.py:112-131).  The page
     table describes the cache after the append.  ``max_append_len`` bounds the
-    longest append (default: nnz)."""
+    longest append (default: nnz; it is checked, the cost does not depend on it)."""
     num_pages, page_size, num_kv_heads, head_dim = _cache_dims(kv_cache)
     dev = kv_cache.device
     _require(k, "k", torch.bfloat16, 3, dev)
