@@ -832,7 +832,7 @@ def _check_token_topk(ops, pb, topk, sink, local, offset, what):
     return lse.cpu().numpy()
 
 
-@pytest.mark.parametrize("case", ["mixed", "hkv8", "g8", "many", "offset", "all", "window_only", "split", "split_many"])
+@pytest.mark.parametrize("case", ["mixed", "hkv8", "g8", "g7", "many", "offset", "all", "window_only", "split", "split_many"])
 def test_token_topk_decode(ops, case):
     """LiteSys' token-level top-k (sparsity_utils.py:6-21): sink tokens, the
     top-k tokens of the middle by group-mean logit, the local window."""
@@ -845,6 +845,9 @@ def test_token_topk_decode(ops, case):
     elif case == "g8":
         pb = P.make_problem(1302, [PS * 300 + 9] * 3, num_kv_heads=1, group=8, table="strided")
         args = (1024, 4, 64, 0)
+    elif case == "g7":       # a group that fills the second head tile only partly
+        pb = P.make_problem(1309, [PS * 50 + 9, PS * 3, 40], num_kv_heads=2, group=7)
+        args = (200, 4, 12, 0)
     elif case == "many":     # > 512 lists: 4 waves per list
         rng = np.random.default_rng(1303)
         pb = P.make_problem(1303, [int(x) for x in rng.integers(1, PS * 30, size=600)], num_kv_heads=1, group=3)
@@ -878,7 +881,7 @@ def test_token_topk_decode(ops, case):
         assert np.allclose(lse, want_lse, rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("case", ["mixed", "hkv8_stride4", "g8", "many", "offset", "stride16", "split", "block8_stride3"])
+@pytest.mark.parametrize("case", ["mixed", "hkv8_stride4", "g8", "g5", "many", "offset", "stride16", "split", "block8_stride3"])
 def test_strided_topk_decode(ops, case):
     """LiteSys' strided overlapping-block policy (sparsity_utils.py:49-105)."""
     block, stride, offset = 16, 8, 0
@@ -891,6 +894,9 @@ def test_strided_topk_decode(ops, case):
     elif case == "g8":
         pb = P.make_problem(1502, [PS * 300 + 9] * 3, num_kv_heads=1, group=8, table="strided")
         topk, sink, local = 64, 4, 64
+    elif case == "g5":
+        pb = P.make_problem(1508, [PS * 50 + 9, PS * 3, 40], num_kv_heads=2, group=5)
+        topk, sink, local = 6, 4, 12
     elif case == "many":     # > 512 lists: 4 waves per list
         rng = np.random.default_rng(1503)
         pb = P.make_problem(1503, [int(x) for x in rng.integers(1, PS * 30, size=600)], num_kv_heads=1, group=3)
