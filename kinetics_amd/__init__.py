@@ -7,7 +7,7 @@ ops, and attention-layer objects shaped like the reference's benchmark layer
 """
 from . import ops  # noqa: F401  (registers torch.ops.kinetics.*)
 from .blocktopk_decoder import BlockTopkPagedAttention, DensePagedAttention  # noqa: F401
-from .decoder_layer import BlockTopkDecoderLayer, DenseDecoderLayer, qwen3_config  # noqa: F401
+from .decoder_layer import BlockTopkDecoderLayer, DenseDecoderLayer, GraphedLayer, qwen3_config  # noqa: F401
 
 __all__ = ["ops", "BlockTopkPagedAttention", "DensePagedAttention", "BlockTopkDecoderLayer", "DenseDecoderLayer",
-           "qwen3_config"]
+           "GraphedLayer", "qwen3_config"]
