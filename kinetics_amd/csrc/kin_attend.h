@@ -38,12 +38,6 @@ constexpr int kWaitVm4 = 4 | (7 << 4) | (15 << 8);
 constexpr float kNegInf = -INFINITY;
 constexpr float kLn2 = 0.6931471805599453f;
 
-// Buffer descriptor covering `bytes` bytes from `base` (0 bytes: every load
-// through it returns zeros without touching memory).
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
-}
-
 // One page for one wave, first half: scores and the online softmax update.
 // ka: this lane's 4 K chunks in MFMA A layout.  Leaves the probabilities of
 // this lane's 4 tokens in pr.  Requires 0 <= first_token <= 16 and

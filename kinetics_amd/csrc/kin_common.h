@@ -70,6 +70,12 @@ inline int score_chunks(int batch, int num_kv_heads, int kbar_pages) {
 }
 // Bytes of the per-list arrival counters in front of the shared key array.
 inline size_t score_count_bytes(int64_t items) { return ((size_t)items * sizeof(int32_t) + 255) & ~(size_t)255; }
+// Keys per list in the shared key array: a multiple of 4, so that every list starts 16-byte aligned.
+__host__ __device__ inline int score_key_stride(int kbar_pages) { return (kbar_pages + 3) & ~3; }
+// Workspace of split scoring: counters, then score_key_stride() keys per list.
+inline size_t score_workspace_bytes(int64_t items, int kbar_pages) {
+  return score_count_bytes(items) + (size_t)items * score_key_stride(kbar_pages) * sizeof(uint32_t);
+}
 
 // ---- device side -----------------------------------------------------------
 #if defined(__HIPCC__)
@@ -127,6 +133,12 @@ __device__ __forceinline__ float row16_sum(float x) {
 template <int I>
 __device__ __forceinline__ float quad_bcast(float x) {
   return dpp_f<(I) | (I << 2) | (I << 4) | (I << 6)>(x);
+}
+
+// Buffer descriptor covering `bytes` bytes from `base` (0 bytes: every load
+// through it returns zeros without touching memory).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
 
 // Zeroes n int32 counters.  A kernel rather than a memset so that the launch

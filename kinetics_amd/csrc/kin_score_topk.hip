@@ -22,7 +22,7 @@ struct ScoreTopkParams {
   int sort_cap;
   int chunks;          // workgroups per list
   int32_t* ws_count;   // [lists] arrival counters, zero at launch and left zero
-  uint32_t* ws_keys;   // [lists, kbar_pages]
+  uint32_t* ws_keys;   // [lists, score_key_stride(kbar_pages)]
 };
 
 // Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap] | int32 sel[sink + topk + local]
@@ -68,7 +68,7 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
     // This workgroup's slice of the candidates -> keys in global memory, written and
     // (by the workgroup that counts in last) read at device scope: no cache
     // maintenance, every wave waits for its own stores before the workgroup counts in.
-    uint32_t* gkeys = p.ws_keys + (int64_t)item * p.kbar_pages;
+    uint32_t* gkeys = p.ws_keys + (int64_t)item * score_key_stride(p.kbar_pages);
     const int n_score = (min(a.topk, a.n_cand) > 0 || a.scores_out) ? a.n_cand : 0;
     const int per = ((n_score + p.chunks - 1) / p.chunks + 63) & ~63;
     const int r0 = min(chunk * per, n_score), r1 = min(r0 + per, n_score);
@@ -81,8 +81,7 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
     __syncthreads();
     if (!sh_last) return;
     if (tid == 0) __hip_atomic_store(&p.ws_count[item], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
-    for (int i = tid; i < n_score; i += kThreads)
-      a.keys[i] = __hip_atomic_load(gkeys + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    load_shared_keys<kThreads>(gkeys, n_score, a.keys);
     __syncthreads();
     n_list = select_from_keys<kThreads>(a, sel_lds);
   } else {
@@ -148,7 +147,7 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
     return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   // Few long lists: spread the scoring of each over several workgroups, given a workspace.
   p.chunks = score_chunks(batch, num_kv_heads, kbar_pages);
-  const size_t ws_need = score_count_bytes(items) + (size_t)items * kbar_pages * sizeof(uint32_t);
+  const size_t ws_need = score_workspace_bytes(items, kbar_pages);
   if (p.chunks > 1 && workspace && aligned16(workspace) && workspace_bytes >= ws_need) {
     p.ws_count = static_cast<int32_t*>(workspace);
     p.ws_keys = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + score_count_bytes(items));

@@ -180,6 +180,26 @@ __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, 
   }
 }
 
+// Copies the n keys that the workgroups sharing one list's scoring wrote to global
+// memory (at device scope, 16-byte aligned) into LDS (16-byte aligned, room for n
+// rounded up to 4): 16-byte device-scope loads, four per thread in flight -- one
+// round trip for up to 16 * NT keys instead of one per key and thread.  The caller
+// puts a barrier after it.
+template <int NT>
+__device__ __forceinline__ void load_shared_keys(const uint32_t* gkeys, int n, uint32_t* keys_lds) {
+  const __amdgpu_buffer_rsrc_t r = make_rsrc(gkeys, n * 4);  // past n: zeros
+  u32x4* dst = reinterpret_cast<u32x4*>(keys_lds);
+  const int n4 = (n + 3) >> 2;
+  for (int base = threadIdx.x; base < n4; base += 4 * NT) {
+    u32x4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = __builtin_amdgcn_raw_buffer_load_b128(r, (base + u * NT) * 16, 0, kDeviceScope);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (base + u * NT < n4) dst[base + u * NT] = v[u];
+  }
+}
+
 // Selects from the keys of the n_cand candidates in a.keys (LDS) and writes the
 // page list to sel_lds (LDS, >= n_sink + topk + n_local entries): the sink
 // pages, then the ordered physical ids of the k_eff winners, then the local

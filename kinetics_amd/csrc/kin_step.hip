@@ -36,7 +36,7 @@ struct StepParams {
   // candidates each into ws_keys; the last one to finish selects and attends.
   int chunks;
   int32_t* ws_count;   // [lists], zero at launch and left zero
-  uint32_t* ws_keys;   // [lists, kbar_pages]
+  uint32_t* ws_keys;   // [lists, score_key_stride(kbar_pages)]
   int64_t num_pages;
   float scale_log2;
 };
@@ -112,7 +112,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   int n;
   if (p.chunks > 1) {
     // This workgroup's slice of the candidates -> keys in HBM.
-    uint32_t* gkeys = p.ws_keys + (int64_t)item * p.kbar_pages;
+    uint32_t* gkeys = p.ws_keys + (int64_t)item * score_key_stride(p.kbar_pages);
     const int n_score = min(s.topk, s.n_cand) > 0 ? s.n_cand : 0;
     const int per = ((n_score + p.chunks - 1) / p.chunks + 63) & ~63;
     const int r0 = min(chunk * per, n_score), r1 = min(r0 + per, n_score);
@@ -131,8 +131,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     if (!sh_last) return;
     if (tid == 0) __hip_atomic_store(&p.ws_count[item], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
     append_token();
-    for (int i = tid; i < n_score; i += NT)
-      s.keys[i] = __hip_atomic_load(gkeys + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    load_shared_keys<NT>(gkeys, n_score, s.keys);
     __syncthreads();
     n = select_from_keys<NT>(s, sel_lds);
   } else {
@@ -172,7 +171,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
 extern "C" size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages) {
   if (kin::score_chunks(batch, num_kv_heads, kbar_pages) <= 1) return 0;
   const int64_t items = (int64_t)batch * num_kv_heads;
-  return kin::score_count_bytes(items) + (size_t)items * kbar_pages * sizeof(uint32_t);
+  return kin::score_workspace_bytes(items, kbar_pages);
 }
 
 extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
