@@ -11,6 +11,7 @@ traceable by ``torch.compile(fullgraph=True)``.
 """
 from __future__ import annotations
 
+import contextlib
 from ctypes import c_void_p
 from typing import Optional
 
@@ -39,23 +40,37 @@ def _ptr(t: Optional[torch.Tensor]):
     return c_void_p(t.data_ptr())
 
 
+_NO_GUARD = contextlib.nullcontext()
+
+
+def _on(device):
+    """Context that makes ``device`` current for a launch; free when it already is."""
+    idx = device.index
+    if idx is None or idx == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(device)
+
+
 def _stream(device) -> c_void_p:
     return c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
 def _require(t: torch.Tensor, name: str, dtype: torch.dtype, ndim=None, device=None):
+    # On the launch path of every call: the cheap tests first, messages built only on failure.
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
-    if t.dtype != dtype:
+    if t.dtype is not dtype:
         raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
-    if t.device.type != "cuda":
+    if not t.is_cuda:
         raise ValueError(f"{name} must live on the GPU (device 'cuda'), got {t.device}")
     if device is not None and t.device != device:
         raise ValueError(f"{name} is on {t.device}, expected {device}")
     if not t.is_contiguous():
         raise ValueError(f"{name} must be contiguous")
-    if ndim is not None and t.dim() not in (ndim if isinstance(ndim, tuple) else (ndim,)):
-        raise ValueError(f"{name} must have {ndim} dimensions, got shape {tuple(t.shape)}")
+    if ndim is not None:
+        d = t.dim()
+        if d != ndim and (not isinstance(ndim, tuple) or d not in ndim):
+            raise ValueError(f"{name} must have {ndim} dimensions, got shape {tuple(t.shape)}")
 
 
 def _cache_dims(kv_cache: torch.Tensor):
@@ -115,7 +130,7 @@ def append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_l
         if kbar.device != dev:
             raise ValueError("kbar must be on the same device as kv_cache")
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(
             lib.kin_append_paged_kv(
                 _ptr(k), _ptr(v), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
@@ -151,7 +166,7 @@ def append_paged_kv_ragged(k, v, append_indptr, kv_cache, kbar, page_indices, pa
         if kbar.device != dev:
             raise ValueError("kbar must be on the same device as kv_cache")
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(
             lib.kin_append_paged_kv_ragged(
                 _ptr(k), _ptr(v), _ptr(append_indptr), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
@@ -171,7 +186,7 @@ def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len) -> None
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(
             lib.kin_build_kbar(
                 _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len),
@@ -229,7 +244,7 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
     if workspace is not None:
         _require(workspace, "workspace", torch.uint8, 1, dev)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(
             lib.kin_block_score_topk(
                 _ptr(q), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), int(topk), int(sink_pages),
@@ -308,7 +323,7 @@ def sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, out=No
         )
     workspace, ws_bytes = _workspace(workspace, dev, batch, hq, hkv, sel_pages.shape[2], int(num_splits))
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(
             lib.kin_sparse_paged_decode(
                 _ptr(q), _ptr(kv_cache), _ptr(sel_pages), _ptr(sel_count), _ptr(last_page_len), _ptr(out), _ptr(lse),
@@ -327,7 +342,7 @@ def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, ma
     _table(page_indices, page_indptr, None, batch, dev)
     workspace, ws_bytes = _workspace(workspace, dev, batch, hq, hkv, int(max_pages_per_seq), int(num_splits))
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(
             lib.kin_dense_paged_decode(
                 _ptr(q), _ptr(kv_cache), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), _ptr(out),
@@ -385,7 +400,7 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
         if need:
             workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(
             lib.kin_blocktopk_decode_step(
                 _ptr(q), _ptr(k), _ptr(v), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
@@ -434,7 +449,7 @@ def token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, top
         q, kv_cache, page_indices, page_indptr, last_page_len, out, lse, sel_tokens, sel_count, workspace,
         lambda b, h: token_topk_workspace_bytes(b, h, max_pages_per_seq))
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(
             lib.kin_token_topk_decode(
                 _ptr(q), _ptr(kv_cache), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), int(topk_tokens),
@@ -464,7 +479,7 @@ def strided_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, t
         q, kv_cache, page_indices, page_indptr, last_page_len, out, lse, sel_tokens, sel_count, workspace,
         lambda b, h: strided_topk_workspace_bytes(b, h, max_pages_per_seq))
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(
             lib.kin_strided_topk_decode(
                 _ptr(q), _ptr(kv_cache), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), int(topk_blocks),
@@ -496,7 +511,7 @@ def build_slot_page_table(seq_lens, pages_per_slot, page_size, page_indices, pag
         if slot_ids.numel() != batch:
             raise ValueError("slot_ids must have one entry per sequence")
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(
             lib.kin_build_slot_page_table(_ptr(slot_ids), _ptr(seq_lens), batch, int(pages_per_slot), int(page_size),
                                           _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), _stream(dev))
@@ -512,7 +527,7 @@ def check_page_table(page_indices, page_indptr, last_page_len, page_size, num_pa
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     scratch = torch.zeros(1, dtype=torch.int32, device=dev)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(
             lib.kin_check_page_table(
                 _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), batch, int(page_size), int(num_pages),
@@ -572,7 +587,7 @@ def rms_norm(x, weight, eps: float, residual=None, out=None) -> torch.Tensor:
         if residual.numel() != rows * hidden or residual.shape[-1] != hidden:
             raise ValueError(f"residual shape {tuple(residual.shape)} does not match x {tuple(x.shape)}")
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(lib.kin_rms_norm(_ptr(x), _ptr(residual), _ptr(weight), _ptr(out), rows, hidden, x_stride, out_stride,
                                     float(eps), _stream(dev)))
     return out
@@ -596,7 +611,7 @@ def qkv_norm_split(qkv, q_weight, k_weight, eps: float, num_q_heads: int, num_kv
     k = torch.empty(batch, num_kv_heads, HEAD_DIM, dtype=torch.bfloat16, device=dev)
     v = torch.empty(batch, num_kv_heads, HEAD_DIM, dtype=torch.bfloat16, device=dev)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(lib.kin_qkv_norm_split(_ptr(qkv), stride, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(q), _ptr(k),
                                           _ptr(v), batch, int(num_q_heads), int(num_kv_heads), HEAD_DIM, _stream(dev)))
     return q, k, v
@@ -620,7 +635,7 @@ def gated_act(gate, up, act: str = "silu", out=None) -> torch.Tensor:
     if out.numel() != rows * inter or out.shape[-1] != inter:
         raise ValueError(f"out shape {tuple(out.shape)} does not match gate {tuple(gate.shape)}")
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.check(lib.kin_gated_act(_ptr(gate), _ptr(up), _ptr(out), rows, inter, g_stride, u_stride, ACTIVATIONS[act],
                                      _stream(dev)))
     return out
