@@ -221,6 +221,28 @@ def whole_layer(torch, args, B, ctx, topk, device):
            "note": "GEMMs are hipBLASLt through PyTorch; norms, q/k/v split, attention and the gated activation are this repository's kernels"}
     del layer
     torch.cuda.empty_cache()
+    if not args.no_dense:
+        # the reference's dense layer (benchmark/dense.py, dense_decoder.py) on the same shape
+        from kinetics_amd.decoder_layer import DenseDecoderLayer
+
+        dense = DenseDecoderLayer(cfg, world, B, ctx, ctx + 512, PS, device, torch.bfloat16)
+        dense.apply(init_weights)
+        dense.eval().to(device, dtype=torch.bfloat16)
+        dense.prepare_wrapper()
+        nd = max(3, min(args.steps, 20))
+        for _ in range(2):
+            dense(hidden.clone())
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(nd):
+            dense(hidden.clone())
+        torch.cuda.synchronize()
+        dd = (time.perf_counter() - t0) / nd
+        out["dense_layer"] = {"ms_per_layer_step": dd * 1e3, "tokens_per_s_per_layer": B / dd, "steps": nd,
+                              "normalised_like_reference_print": B / dd / (world * cfg.num_hidden_layers)}
+        out["sparse_over_dense_layer"] = dd / dt
+        del dense
+        torch.cuda.empty_cache()
     return out
 
 
@@ -229,7 +251,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="qwen3-8b-share", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="qwen3-8b-share", choices=sorted(WORKLOADS) + ["custom"])
     ap.add_argument("--batch", type=int, default=0, help="override the workload's batch size")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
@@ -243,6 +265,14 @@ def main():
     ap.add_argument("--token-topk", action="store_true",
                     help="also time token-level top-k decode (LiteSys' attn_topk policy) with the same token budget "
                          "(topk_pages * 16 tokens, 4 sink tokens, a 16-token window)")
+    # the reference's own command line (benchmark/blocktopk.py:6-19, benchmark/README.md): a context of
+    # gen_len / 2 tokens, the model's heads divided by world_size
+    ap.add_argument("--model", default=None, help="e.g. Qwen/Qwen3-8B: build the workload from the reference's arguments")
+    ap.add_argument("--gen_len", type=int, default=32768)
+    ap.add_argument("--batch_size", type=int, default=256)
+    ap.add_argument("--topk_page", type=int, default=64)
+    ap.add_argument("--page_size", type=int, default=16)
+    ap.add_argument("--world_size", type=int, default=8)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) to scale profiler byte counters")
     args = ap.parse_args()
@@ -250,6 +280,22 @@ def main():
         print("bench.py measures one GPU: the path is independent per (sequence, KV head) and is run on "
               "one GPU's share of the heads; --gpus above 1 is not supported.", file=sys.stderr)
         sys.exit(2)
+
+    if args.model:
+        from kinetics_amd.decoder_layer import qwen3_config
+
+        if args.page_size != PS:
+            print(f"bench.py: the kernels are built for page_size {PS}", file=sys.stderr)
+            sys.exit(2)
+        mcfg = qwen3_config(args.model)
+        hq, hkv = mcfg.num_attention_heads // args.world_size, mcfg.num_key_value_heads // args.world_size
+        if hq < 1 or hkv < 1:
+            print("bench.py: world_size exceeds the number of heads", file=sys.stderr)
+            sys.exit(2)
+        args.workload = "custom"
+        WORKLOADS["custom"] = (args.batch_size, args.gen_len // 2, hkv, hq // hkv, args.topk_page,
+                               f"{args.model} at world_size {args.world_size}: {hkv} KV heads, {hq} Q heads")
+        WHOLE_LAYER_MODEL["custom"] = (args.model, args.world_size)
 
     import torch
 
