@@ -734,6 +734,58 @@ def test_fused_step_split_scoring_for_few_long_sequences(ops, hkv, group):
     assert torch.equal(one.sel, a.sel)
 
 
+def test_seeded_sweep_of_split_scoring(ops):
+    """Six seeded shapes with few, long sequences: the fused step and the three
+    launches, each with and without the workspace that spreads the scoring of a
+    list over several workgroups, must agree on every cache byte and page list
+    (outputs bit-equal within a path), and with the oracle."""
+    rng = np.random.default_rng(61)
+    for trial in range(6):
+        hkv = int(rng.choice([1, 1, 2, 4]))
+        group = int(rng.integers(1, 9))
+        B = int(rng.integers(1, 5))
+        lengths = [int(rng.choice([0, 5, PS * 7, int(rng.integers(PS * 2048, PS * 6000)), int(rng.integers(PS * 100, PS * 3000))]))
+                   for _ in range(B)]
+        if max(lengths) < PS * 2049:
+            lengths[0] = int(rng.integers(PS * 2100, PS * 5000))
+        topk = int(rng.choice([1, 17, 128, 600, 2048]))
+        sink, local = int(rng.integers(0, 3)), int(rng.choice([1, 17, 40]))
+        what = f"trial {trial}: hkv={hkv} G={group} lengths={lengths} topk={topk} sink={sink} local={local}"
+        pb = P.make_problem(6100 + trial, lengths, num_kv_heads=hkv, group=group, topk=topk)
+        need = ops.step_workspace_bytes(pb.B, hkv, pb.kbar.shape[1])
+        assert need > 0, what
+        ws = torch.full((need,), 0xCD, dtype=torch.uint8, device=DEV)
+        cap = ops.sel_list_capacity(topk, sink, local)
+        res = []
+        for mode in ("fused_plain", "fused_split", "three_plain", "three_split"):
+            g = Gpu(pb)
+            g.sel = torch.full((pb.B, hkv, cap), -7, dtype=torch.int32, device=DEV)
+            w = ws if mode.endswith("split") else None
+            if mode.startswith("fused"):
+                out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, topk, sel_pages=g.sel,
+                                                sel_count=g.cnt, sink_pages=sink, local_tokens=local,
+                                                workspace=w if w is not None else torch.empty(0, dtype=torch.uint8, device=DEV))
+            else:
+                ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
+                ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, topk, g.sel, g.cnt, sink_pages=sink,
+                                     local_tokens=local, workspace=w)
+                out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last)
+            torch.cuda.synchronize()
+            res.append((g.sel.clone(), g.cnt.clone(), out.clone(), g.kv, g.kbar))
+        for i in range(1, 4):
+            assert torch.equal(res[0][0], res[i][0]) and torch.equal(res[0][1], res[i][1]), f"{what}: lists differ ({i})"
+            assert torch.equal(res[0][3], res[i][3]) and torch.equal(res[0][4], res[i][4]), f"{what}: cache differs ({i})"
+        assert torch.equal(res[0][2], res[1][2]) and torch.equal(res[2][2], res[3][2]), what
+        kv, kbar = pb.kv_cache.copy(), pb.kbar.copy()
+        r = O.decode_step(pb.q, pb.k, pb.v, kv, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, topk,
+                          sink_pages=sink, local_tokens=local)
+        assert np.array_equal(P.from_torch(res[0][3]), kv) and np.array_equal(P.from_torch(res[0][4]), kbar), what
+        assert np.array_equal(res[0][1].cpu().numpy(), r["sel_count"]), what
+        want, _ = O.sparse_paged_decode(pb.q, kv, res[0][0].cpu().numpy(), r["sel_count"], pb.last_page_len)
+        assert_out_close(res[0][2], want, what)
+        assert_out_close(res[2][2], want, what)
+
+
 # --------------------------------------------------------------------------- ragged multi-token append
 
 
