@@ -386,8 +386,8 @@ int kin_strided_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  *   page_indices[...]       slot*pages_per_slot + p, packed per sequence
  *                           (capacity batch*pages_per_slot entries)
  *   last_page_len[b]        tokens in the final page (1 for empty sequences)
- * No host synchronisation.  batch <= 65535.  (The batch == 0 case records a
- * memset; do not capture that case in a HIP graph.)
+ * No host synchronisation, kernels only (capturable in a HIP graph).
+ * batch <= 65535.
  */
 int kin_build_slot_page_table(const int32_t* slot_ids, const int32_t* seq_lens, int batch,
                               int pages_per_slot, int page_size,

@@ -74,7 +74,8 @@ extern "C" int kin_build_slot_page_table(const int32_t* slot_ids, const int32_t*
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (batch == 0) {
     // nothing to fill, but indptr[0] must still be valid
-    return check_hip(hipMemsetAsync(page_indptr, 0, sizeof(int32_t), s), "clear page_indptr[0]");
+    fill_zero_i32_kernel<<<1, 64, 0, s>>>(page_indptr, 1);
+    return check_hip(hipGetLastError(), "fill_zero_i32_kernel launch");
   }
   slot_table_scan_kernel<<<1, 1024, 0, s>>>(seq_lens, batch, pages_per_slot, page_size, page_indptr, last_page_len);
   int st = check_hip(hipGetLastError(), "slot_table_scan_kernel launch");
