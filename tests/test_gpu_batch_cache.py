@@ -183,3 +183,34 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
         feed(layer, 2, k[0], v[0])
         m.compute_attention(q, k, v, layer, torch.tensor([2]))
     decode_round([2, 5])
+
+
+@pytest.mark.parametrize("batch,with_slots", [(0, False), (1, False), (7, True), (1500, True), (3000, False)])
+def test_slot_page_table_against_numpy(batch, with_slots):
+    """CSR page table of a slot-based cache (kin_build_slot_page_table): page
+    counts clamped to the slot's run, empty and over-long sequences, more
+    sequences than one scan pass, an empty batch."""
+    from kinetics_amd import ops
+
+    rng = np.random.default_rng(batch + 1)
+    pps = 24
+    lens = rng.integers(-3, PS * pps + 40, size=batch).astype(np.int32)
+    if batch >= 7:
+        lens[:4] = [0, 1, PS * pps, PS * pps + 17]
+    slots = rng.permutation(batch + 5)[:batch].astype(np.int32) if with_slots else None
+    idx = torch.full((max(batch * pps, 1),), -1, dtype=torch.int32, device=DEV)
+    ptr = torch.full((batch + 1,), -1, dtype=torch.int32, device=DEV)
+    last = torch.full((batch,), -1, dtype=torch.int32, device=DEV)
+    ops.build_slot_page_table(torch.from_numpy(lens).to(DEV), pps, PS, idx, ptr, last,
+                              slot_ids=None if slots is None else torch.from_numpy(slots).to(DEV))
+    torch.cuda.synchronize()
+    n = np.minimum((np.maximum(lens, 0) + PS - 1) // PS, pps)
+    want_ptr = np.concatenate([[0], np.cumsum(n)]).astype(np.int32)
+    assert np.array_equal(ptr.cpu().numpy(), want_ptr)
+    tokens = np.minimum(np.maximum(lens, 0), n * PS)
+    want_last = np.where(n > 0, tokens - (n - 1) * PS, 1).astype(np.int32)
+    assert np.array_equal(last.cpu().numpy(), want_last)
+    got = idx.cpu().numpy()
+    for b in range(batch):
+        s = b if slots is None else int(slots[b])
+        assert np.array_equal(got[want_ptr[b]: want_ptr[b + 1]], s * pps + np.arange(n[b]))
