@@ -296,3 +296,22 @@ def test_bench_byte_model_matches_the_documented_figures():
     assert ab["attention"] == 4096 * (1049088 + 2048 + 129 * 4)
     small = bench.algorithmic_bytes([17], 2, 2, 8)       # 2 pages: 1 candidate, budget clamps to 1
     assert small["step"] == 2 * (1 * 256 + (16 + 1) * 512 + 512) + 2 * 4 * 256 + 2 * 2 * 1 * 4
+
+
+def test_header_is_plain_c_and_links_from_c(tmp_path):
+    """include/kinetics_amd.h compiles as strict C99 and a C program linked against
+    the library gets versions, sizes and argument errors without a GPU."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    exe = tmp_path / "use_from_c"
+    libdir = _lib.LIB_PATH.parent
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", f"-I{HEADER.parent}",
+                    str(ROOT / "tests" / "cabi" / "use_from_c.c"), "-o", str(exe), f"-L{libdir}", "-lkinetics_amd",
+                    f"-Wl,-rpath,{libdir}"], check=True, capture_output=True, text=True)
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert "ok" in run.stdout.splitlines()[-1]
