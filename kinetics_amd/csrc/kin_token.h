@@ -46,6 +46,7 @@ struct TokenArgs {
   uint32_t* keys;        // HBM scratch, n_pages * 16 entries, 16-byte aligned
   int32_t* list;         // LDS, >= n_sink + min(topk, n_dyn) + n_local entries
   int32_t* sel_tokens;   // HBM, the listed tokens' positions in the sequence, or null
+  unsigned rotate;       // where in its page range this list starts streaming (any value)
 };
 
 // Physical token id (page * 16 + slot) of cache slot c of the sequence.
@@ -293,23 +294,38 @@ __device__ __forceinline__ void stream_token_scores(const TokenArgs& a, int pg0,
     for (int i = 0; i < 4; ++i) dst[i] = __builtin_amdgcn_raw_buffer_load_b128(r, voff + i * row_step, 0, kStreamLoad);
   };
   const int my_page = c16 >> 2, my_row = 4 * (c16 & 3) + kg;
-  const int first = pg0 + kPF * w;  // pg0 is a multiple of 4
+  // The wave's quads are qi = w, w + NW, ... of the range's nq quads, visited from a
+  // list-specific starting quad (a.rotate) and wrapping around: scores are stored by
+  // position, so the order is free, and equal lists that run in step then read from
+  // all over the cache instead of from one narrow window of it (reading only the K
+  // half of consecutive pages loads the memory channels unevenly).
+  const int nq = (pg1 - pg0 + kPF - 1) / kPF;  // pg0 is a multiple of 4
+  const int rot = nq > 0 ? (int)(a.rotate % (unsigned)nq) : 0;
+  auto quad_page = [&](int qi) -> int {  // first page of quad qi, or pg1 (nothing to read) past the end
+    if (qi >= nq) return pg1;
+    const int qq = qi + rot;
+    return pg0 + kPF * (qq >= nq ? qq - nq : qq);
+  };
   u32x4 x[kPF][4];
+  {
+    const int p0 = quad_page(w);
 #pragma unroll
-  for (int u = 0; u < kPF; ++u) {
-    load_page(first + u, x[u]);
-    // Issue order = consumption order: the wait at the top of the loop is sized for the worse
-    // of the two ways into it, and a reordered prologue would leave only a few loads in flight.
-    __builtin_amdgcn_sched_barrier(0);
+    for (int u = 0; u < kPF; ++u) {
+      load_page(p0 + u, x[u]);
+      // Issue order = consumption order: the wait at the top of the loop is sized for the worse
+      // of the two ways into it, and a reordered prologue would leave only a few loads in flight.
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
-  for (int base = first; base < pg1; base += kPF * NW) {
+  for (int qi = w; qi < nq; qi += NW) {
+    const int base = quad_page(qi), next = quad_page(qi + NW);
     float mine = 0.f;
 #pragma unroll
     for (int u = 0; u < kPF; ++u) {
       u32x4 kx[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) kx[i] = x[u][i];
-      load_page(base + kPF * NW + u, x[u]);
+      load_page(next + u, x[u]);
       float acc[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {

@@ -89,6 +89,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
   t.keys = p.keys + (int64_t)item * p.max_pages_per_seq * kPageSize;
   t.list = list;
   t.sel_tokens = sel_out;
+  t.rotate = (unsigned)item * 2654435761u >> 12;  // a different starting point for every list
   StridedArgs sa;
   if (STRIDED) {
     sa.block = p.block;
