@@ -302,6 +302,45 @@ int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const ki
 size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages);
 
 /*
+ * kin_blocktopk_decode_step for callers that cannot allocate -- code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
+ * no counterpart in the reference (which sizes a 128 MiB workspace up front,
+ * benchmark/blocktopk_decoder.py:152).  Same arguments, arithmetic and results as
+ * kin_blocktopk_decode_step given a full workspace, but the split-scoring
+ * workspace is an array of KIN_STATIC_SCRATCH_BYTES bytes inside the library's
+ * device code: each GPU the library runs on holds its own copy until the
+ * process ends.  The call allocates and frees nothing (no hipMalloc, no
+ * hipFree, no allocating library routine); the arrival counters are zeroed by a
+ * small kernel on `stream`, never by a memset.  The first call on a device looks
+ * the array's address up (hipGetSymbolAddress, with that device current; make
+ * that call outside graph capture); the stream must belong to the current
+ * device.
+ * Limit: shapes whose kin_step_workspace_bytes() exceeds
+ * KIN_STATIC_SCRATCH_BYTES are rejected with KIN_ERR_WORKSPACE -- the array
+ * covers up to 524288 candidate pages in total over all lists that split, e.g.
+ * 64 lists of 8192 pages or 32 of 16384; shapes that do not split (that function
+ * returns 0) never touch the array and are always accepted.
+ * All calls on one GPU share the array: calls that overlap in time on the same
+ * GPU (different streams, or different threads) race and must be serialised by
+ * the caller; calls in one stream are ordered by the stream.
+ */
+#define KIN_STATIC_SCRATCH_BYTES (2u * 1024u * 1024u + 256u)
+
+size_t kin_static_scratch_bytes(void);
+
+int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
+                                     kin_bf16_t* kv_cache, kin_bf16_t* kbar,
+                                     const int32_t* page_indices, const int32_t* page_indptr,
+                                     const int32_t* last_page_len, int topk,
+                                     int sink_pages, int local_tokens,
+                                     int32_t* sel_pages, int32_t* sel_count,
+                                     kin_bf16_t* out, float* lse,
+                                     int batch, int num_q_heads, int num_kv_heads,
+                                     int head_dim, int page_size, int64_t num_pages,
+                                     int kbar_pages, int sel_stride, int first_page_offset,
+                                     float sm_scale, kin_stream_t stream);
+
+/*
  * Token-level top-k sparse decode attention in one launch -- LiteSys'
  * topk_sparsity policy (ref: LiteSys/litesys/attention/sparsity_utils.py:6-21)
  * inside BatchKVManager.decode (ref: LiteSys/litesys/attention/batch_cache.py:154-168),

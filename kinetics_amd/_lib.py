@@ -61,6 +61,12 @@ SIGNATURES = {
          c_int, c_int, c_int, c_float, _P, c_size_t, _P],
     ),
     "kin_step_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "kin_static_scratch_bytes": (c_size_t, []),
+    "kin_blocktopk_decode_step_static": (
+        c_int,
+        [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int64,
+         c_int, c_int, c_int, c_float, _P],
+    ),
     "kin_token_topk_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "kin_token_topk_decode": (
         c_int,

@@ -10,6 +10,8 @@
 // neighbours' streaming.  The selected page ids stay in LDS (HBM copies are
 // optional outputs).  Same building blocks and arithmetic as the stand-alone
 // kernels: score_select() (kin_select.h) and attend_list() (kin_attend.h).
+#include <atomic>
+
 #include "kin_append.h"
 #include "kin_attend.h"
 #include "kin_select.h"
@@ -174,16 +176,18 @@ extern "C" size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar
   return kin::score_workspace_bytes(items, kbar_pages);
 }
 
-extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
-                                         kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
-                                         const int32_t* page_indptr, const int32_t* last_page_len, int topk,
-                                         int sink_pages, int local_tokens, int32_t* sel_pages, int32_t* sel_count,
-                                         kin_bf16_t* out, float* lse, int batch, int num_q_heads, int num_kv_heads,
-                                         int head_dim, int page_size, int64_t num_pages, int kbar_pages,
-                                         int sel_stride, int first_page_offset, float sm_scale, void* workspace,
-                                         size_t workspace_bytes, kin_stream_t stream) {
-  using namespace kin;
-  const char* fn = "kin_blocktopk_decode_step";
+namespace kin {
+
+// Validation and launch shared by kin_blocktopk_decode_step (workspace from the
+// caller) and kin_blocktopk_decode_step_static (workspace = this library's own
+// device array).  fn: the entry point's name, for error messages.
+static int launch_step(const char* fn, const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
+                       kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
+                       const int32_t* page_indptr, const int32_t* last_page_len, int topk, int sink_pages,
+                       int local_tokens, int32_t* sel_pages, int32_t* sel_count, kin_bf16_t* out, float* lse,
+                       int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
+                       int64_t num_pages, int kbar_pages, int sel_stride, int first_page_offset, float sm_scale,
+                       void* workspace, size_t workspace_bytes, kin_stream_t stream) {
   if (!q || !kv_cache || !kbar || !page_indices || !page_indptr || !last_page_len || !out)
     return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   if ((k == nullptr) != (v == nullptr))
@@ -293,4 +297,79 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
   void* args[] = {&p};
   st = check_hip(hipLaunchKernel(kernel, dim3(grid), dim3(nw * 64), args, lds, s), "blocktopk_step_kernel launch");
   return st;
+}
+
+// ---- device memory of the entry point that allocates nothing -------------------
+// Split-scoring workspace (arrival counters, then keys) for callers that cannot
+// bring one.  Every GPU the library's code object is loaded on holds its own copy
+// until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; kernels get the address that call returns.
+constexpr size_t kStaticScratchBytes = KIN_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device (looked up once per device).
+static int static_scratch_address(const char* fn, void** ptr) {
+  int dev = -1;
+  int st = check_hip(hipGetDevice(&dev), "hipGetDevice");
+  if (st) return st;
+  if (dev < 0 || dev >= kMaxDevices) return fail(KIN_ERR_UNSUPPORTED, "%s: device ordinal %d is beyond %d", fn, dev, kMaxDevices);
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    st = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+    if (st) return st;
+    if (!p) return fail(KIN_ERR_LAUNCH, "%s: hipGetSymbolAddress returned a null address", fn);
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing threads store the same value
+  }
+  *ptr = p;
+  return KIN_OK;
+}
+
+}  // namespace kin
+
+extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
+                                         kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
+                                         const int32_t* page_indptr, const int32_t* last_page_len, int topk,
+                                         int sink_pages, int local_tokens, int32_t* sel_pages, int32_t* sel_count,
+                                         kin_bf16_t* out, float* lse, int batch, int num_q_heads, int num_kv_heads,
+                                         int head_dim, int page_size, int64_t num_pages, int kbar_pages,
+                                         int sel_stride, int first_page_offset, float sm_scale, void* workspace,
+                                         size_t workspace_bytes, kin_stream_t stream) {
+  return kin::launch_step("kin_blocktopk_decode_step", q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len,
+                          topk, sink_pages, local_tokens, sel_pages, sel_count, out, lse, batch, num_q_heads, num_kv_heads,
+                          head_dim, page_size, num_pages, kbar_pages, sel_stride, first_page_offset, sm_scale, workspace,
+                          workspace_bytes, stream);
+}
+
+extern "C" size_t kin_static_scratch_bytes(void) { return kin::kStaticScratchBytes; }
+
+extern "C" int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
+                                                kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
+                                                const int32_t* page_indptr, const int32_t* last_page_len, int topk,
+                                                int sink_pages, int local_tokens, int32_t* sel_pages,
+                                                int32_t* sel_count, kin_bf16_t* out, float* lse, int batch,
+                                                int num_q_heads, int num_kv_heads, int head_dim, int page_size,
+                                                int64_t num_pages, int kbar_pages, int sel_stride,
+                                                int first_page_offset, float sm_scale, kin_stream_t stream) {
+  using namespace kin;
+  const char* fn = "kin_blocktopk_decode_step_static";
+  // What the split scoring of this shape needs (0: the shape does not split and
+  // no scratch is touched).  Sizes beyond the array are an error, not a silent
+  // fall-back to the slower single-workgroup scoring.
+  const size_t need = kin_step_workspace_bytes(batch, num_kv_heads, kbar_pages);
+  if (need > kStaticScratchBytes)
+    return fail(KIN_ERR_WORKSPACE,
+                "%s: batch=%d x num_kv_heads=%d lists of kbar_pages=%d need %zu bytes of scratch, the built-in array has %zu "
+                "(use kin_blocktopk_decode_step with a workspace of kin_step_workspace_bytes() bytes)",
+                fn, batch, num_kv_heads, kbar_pages, need, kStaticScratchBytes);
+  void* ws = nullptr;
+  if (need > 0) {
+    const int st = static_scratch_address(fn, &ws);
+    if (st) return st;
+  }
+  return launch_step(fn, q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sink_pages, local_tokens,
+                     sel_pages, sel_count, out, lse, batch, num_q_heads, num_kv_heads, head_dim, page_size, num_pages,
+                     kbar_pages, sel_stride, first_page_offset, sm_scale, ws, need > 0 ? kStaticScratchBytes : 0, stream);
 }

@@ -369,13 +369,18 @@ def prefer_fused_step(batch: int, num_kv_heads: int, max_pages_per_seq: int, top
 
 def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, out=None, lse=None,
                           sel_pages=None, sel_count=None, sm_scale: float = 0.0, sink_pages: int = 0,
-                          local_tokens: int = 1, first_page_offset: int = 0, workspace=None):
+                          local_tokens: int = 1, first_page_offset: int = 0, workspace=None, static_scratch: bool = False):
     """append -> score -> select -> attend in one launch: lines 209-225 of the
     reference layer's forward (benchmark/blocktopk_decoder.py) as a single
     kernel.  ``k``/``v`` may be None (no append); ``sel_pages``/``sel_count`` are
     optional outputs.  ``workspace`` (``step_workspace_bytes``; allocated here when
     None and the shape profits) lets few, long sequences spread their scoring over
-    the GPU.  Returns ``out`` [batch, num_q_heads, head_dim] bf16."""
+    the GPU.  ``static_scratch=True`` calls ``kin_blocktopk_decode_step_static``
+    instead: the library's built-in device array is the workspace and nothing is
+    allocated (``out`` must then be given; ``workspace`` must be None).
+    Returns ``out`` [batch, num_q_heads, head_dim] bf16."""
+    if static_scratch and (out is None or workspace is not None):
+        raise ValueError("static_scratch=True needs a caller-provided out and takes no workspace")
     dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, workspace)
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     kbar_pages = _kbar_pages(kbar, batch, hkv, d)
@@ -395,11 +400,22 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
         if sel_pages.shape[:2] != (batch, hkv) or tuple(sel_count.shape) != (batch, hkv):
             raise ValueError(f"sel_pages/sel_count must be [{batch}, {hkv}, stride] / [{batch}, {hkv}]")
         sel_stride = sel_pages.shape[2]
+    lib = _lib.load()
+    if static_scratch:
+        with _on(dev):
+            _lib.check(
+                lib.kin_blocktopk_decode_step_static(
+                    _ptr(q), _ptr(k), _ptr(v), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
+                    _ptr(last_page_len), int(topk), int(sink_pages), int(local_tokens), _ptr(sel_pages), _ptr(sel_count),
+                    _ptr(out), _ptr(lse), batch, hq, hkv, d, ps, num_pages, kbar_pages, sel_stride, int(first_page_offset),
+                    float(sm_scale), _stream(dev),
+                )
+            )
+        return out
     if workspace is None:
         need = step_workspace_bytes(batch, hkv, kbar_pages)
         if need:
             workspace = torch.empty(need, dtype=torch.uint8, device=dev)
-    lib = _lib.load()
     with _on(dev):
         _lib.check(
             lib.kin_blocktopk_decode_step(

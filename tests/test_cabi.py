@@ -315,3 +315,19 @@ def test_header_is_plain_c_and_links_from_c(tmp_path):
     run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
     assert run.returncode == 0, run.stdout + run.stderr
     assert "ok" in run.stdout.splitlines()[-1]
+
+
+def test_static_scratch_step_size_limit_is_checked_before_anything_else(lib):
+    """The entry point that allocates nothing rejects shapes whose split-scoring
+    scratch exceeds its built-in array, from the dimensions alone."""
+    assert lib.kin_static_scratch_bytes() == 2 * 1024 * 1024 + 256
+    assert 0 < lib.kin_step_workspace_bytes(64, 1, 8192) <= lib.kin_static_scratch_bytes()
+    assert lib.kin_step_workspace_bytes(64, 1, 16384) > lib.kin_static_scratch_bytes()
+    st = lib.kin_blocktopk_decode_step_static(None, None, None, None, None, None, None, None, 128, 0, 1, None, None, None,
+                                              None, 64, 4, 1, 128, 16, 1 << 20, 16384, 0, 0, 0.0, None)
+    assert st == _lib.KIN_ERR_WORKSPACE
+    assert b"kin_blocktopk_decode_step_static" in lib.kin_last_error()
+    # a shape that does not split needs no scratch: ordinary argument checking applies
+    st = lib.kin_blocktopk_decode_step_static(None, None, None, None, None, None, None, None, 128, 0, 1, None, None, None,
+                                              None, 4096, 4, 1, 128, 16, 1 << 20, 2048, 0, 0, 0.0, None)
+    assert st == _lib.KIN_ERR_NULL_POINTER
