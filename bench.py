@@ -67,7 +67,7 @@ def algorithmic_bytes(lengths, Hkv, G, topk):
     return dict(step=step, attention=attn, score_select=score, dense=dense, per_seq=step / max(1, len(lengths)))
 
 
-def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2, ragged=False):
+def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2, ragged=False, kv_alloc=None):
     """Paged cache, K ~ N(0,1) + per-page mean offset N(0,0.5), V ~ N(0,1); kbar =
     true page means.  Uniform workloads use the reference layout (page id =
     p*B + b, max_len = ctx+512, every context ``ctx`` tokens + the appended one).
@@ -101,7 +101,8 @@ def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2, ragged=False):
     else:
         num_pages = max_pages * B
         lengths = [ctx + 1] * B
-    kv = torch.empty(num_pages, 2, PS, Hkv, D, dtype=torch.bfloat16, device=device)
+    kv_shape = (num_pages, 2, PS, Hkv, D)
+    kv = kv_alloc(kv_shape) if kv_alloc else torch.empty(kv_shape, dtype=torch.bfloat16, device=device)
     chunk = max(1, (1 << 28) // (2 * PS * Hkv * D))
     for s in range(0, num_pages, chunk):
         e = min(num_pages, s + chunk)
@@ -125,7 +126,7 @@ def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2, ragged=False):
         indptr=indptr,
         last=last,
         lengths=[int(x) for x in lengths],
-        kbar=torch.zeros(B, max_pages, Hkv, D, dtype=torch.bfloat16, device=device),
+        kbar=torch.zeros(B, Hkv, max_pages, D, dtype=torch.bfloat16, device=device),
         sel=torch.full((B, Hkv, topk + 1), -1, dtype=torch.int32, device=device),
         cnt=torch.zeros(B, Hkv, dtype=torch.int32, device=device),
         q=torch.randn(B, Hkv * G, D, generator=gen, device=device, dtype=torch.float32).to(torch.bfloat16),

@@ -18,9 +18,13 @@
  *   kv_cache      [num_pages, 2, page_size, num_kv_heads, head_dim] bf16
  *                 ("NHD" paged layout, K plane then V plane per page;
  *                  ref: benchmark/blocktopk_decoder.py:161-164)
- *   kbar          [batch, kbar_pages, num_kv_heads, head_dim]       bf16
- *                 per-page representative (mean) key, indexed by LOGICAL page
- *                 (ref: benchmark/blocktopk_decoder.py:166-168)
+ *   kbar          [batch, num_kv_heads, kbar_pages, head_dim]       bf16
+ *                 per-page representative (mean) key, indexed by LOGICAL page,
+ *                 head-major: the candidates of one (sequence, KV head) are one
+ *                 contiguous run of rows.  With one KV head this is the
+ *                 reference's compressed_key_cache [batch, pages, head_dim]
+ *                 (ref: benchmark/blocktopk_decoder.py:165-168, which asserts
+ *                 one KV head).
  *   page_indices  [nnz] int32, page_indptr [batch+1] int32,
  *   last_page_len [batch] int32 in [1, page_size]
  *                 CSR page table: sequence b owns physical pages
@@ -79,7 +83,7 @@ const char* kin_status_string(int status);
  * The page table describes the cache AFTER the append: the new token of
  * sequence b is written at slot last_page_len[b]-1 of its last page.  When
  * that write fills the page (last_page_len[b] == page_size) and kbar != NULL,
- * kbar[b, n_pages-1, h, :] is set to the mean of the page's page_size keys
+ * kbar[b, h, n_pages-1, :] is set to the mean of the page's page_size keys
  * (fp32 sum in slot order, times 1/page_size, round-to-nearest-even to bf16).
  * Sequences with an empty page list are skipped.  kbar may be NULL.
  */
@@ -150,7 +154,7 @@ int kin_append_paged_kv_ragged(const kin_bf16_t* k, const kin_bf16_t* v,
  * their first page (see first_page_offset below) and local_tokens = LiteSys'
  * `local` reproduces blockwise_topk_sparsity with its hard-wired 4 sink tokens
  * and 16-token blocks that start at token 4 (sparsity_utils.py:24-35).
- * score[p] = dot(mean_g q[b, h*G+g, :], kbar[b, p, h, :]) in fp32.
+ * score[p] = dot(mean_g q[b, h*G+g, :], kbar[b, h, p, :]) in fp32.
  * k_eff = min(topk, n_cand) candidates are selected: descending score, equal
  * scores by ascending logical index (deterministic).
  * Outputs, with n = n_sink + k_eff + n_local:
@@ -225,8 +229,12 @@ int kin_decode_auto_splits(int batch, int num_kv_heads, int max_pages_per_list);
  * page of every list hold no token and are skipped -- for caches that store
  * each sequence shifted into its first page so that pages line up with blocks
  * that do not start at token 0 (LiteSys' blocks start after 4 sink tokens,
- * sparsity_utils.py:24-35: offset 12).  The selector lists the sequence's first
- * page first whenever sink_pages >= 1.
+ * sparsity_utils.py:24-35: offset 12).  The offset is applied to list entry 0,
+ * which is the sequence's first page only if the list was made with
+ * sink_pages >= 1 (kin_block_score_topk then lists the first page first) or
+ * the sequence has a single page: a caller that passes first_page_offset > 0
+ * must have selected with sink_pages >= 1 (kin_blocktopk_decode_step checks
+ * this pairing; here the list's origin is unknown and nothing can be checked).
  */
 int kin_sparse_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
                             const int32_t* sel_pages, const int32_t* sel_count,
@@ -460,9 +468,13 @@ int kin_check_page_table(const int32_t* page_indices, const int32_t* page_indptr
  * which is flashinfer.rmsnorm(x, weight, eps) as layer_norm and qk_norm call it
  * (benchmark/model_utils.py:8,19).  With residual != NULL ([rows, hidden],
  * contiguous) the add that precedes the norm in the layer
- * (benchmark/blocktopk_decoder.py:229-232) is folded in, as
- * flashinfer.fused_add_rmsnorm does it (benchmark/model_utils.py:27-41):
+ * (benchmark/blocktopk_decoder.py:229-232: a bf16 tensor add, then layer_norm)
+ * is folded in with exactly that arithmetic -- the sum is rounded to bf16
+ * first and the ROUNDED value is normalised:
  *   residual[r, :] = bf16(x[r, :] + residual[r, :]);  out = RMSNorm(residual)
+ * This is the layer's unfused add-then-norm, not flashinfer.fused_add_rmsnorm
+ * (benchmark/model_utils.py:27-41), which is understood to keep the fp32 sum
+ * for the statistics: the two can differ in the last bf16 place.
  * Row strides are in elements (multiples of 8, >= hidden); out may alias x.
  * hidden: a multiple of 512 up to 8192, or a multiple of 128 up to 2048
  * (head_dim 128 rows for qk_norm).

@@ -121,7 +121,7 @@ class PagedBatchKVManager:
         self.pages_per_slot = P = (max_seq_len + self.pad + PAGE - 1) // PAGE
         dev = self.device
         self.kv_cache = [torch.zeros(B * P, 2, PAGE, Hkv, D, dtype=dtype, device=dev) for _ in range(self.num_layers)]
-        self.kbar = [torch.zeros(B, P, Hkv, D, dtype=dtype, device=dev) for _ in range(self.num_layers)]
+        self.kbar = [torch.zeros(B, Hkv, P, D, dtype=dtype, device=dev) for _ in range(self.num_layers)]
         self.kv_offset = [torch.zeros(B, dtype=torch.int32, device=dev) for _ in range(self.num_layers)]
         # page-table metadata (rebuilt on the device each decode call) and full-batch staging buffers
         self.page_indices = torch.zeros(B * P, dtype=torch.int32, device=dev)

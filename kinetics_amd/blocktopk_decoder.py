@@ -73,7 +73,7 @@ class BlockTopkPagedAttention:
             self.kv_cache = torch.empty(shape, dtype=dtype, device=dev)
         else:
             raise ValueError("init_cache must be 'randn' or 'empty'")
-        self.compressed_key_cache = torch.zeros(B, max_num_pages, num_kv_heads, head_dim, dtype=dtype, device=dev)
+        self.compressed_key_cache = torch.zeros(B, num_kv_heads, max_num_pages, head_dim, dtype=dtype, device=dev)
         self.refresh_compressed_keys()
 
         self.sm_scale = 1.0 / math.sqrt(head_dim)

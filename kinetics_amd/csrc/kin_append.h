@@ -55,7 +55,7 @@ __device__ __forceinline__ u32x4 page_mean_16B(const u32x4* kplane16, int row_st
 // The row lands in slot last_len-1 of the sequence's last page (physical id
 // last_pid).  If that fills the page and the page has a slot in kbar
 // (n_pages-1 < kbar_pages, kbar may be null), its mean key goes to
-// kbar_page_row, the dword address of kbar[b, n_pages-1, h, 0]: rows 0..14 are
+// kbar_page_row, the dword address of kbar[b, h, n_pages-1, 0]: rows 0..14 are
 // read from the cache, row 15 is taken from the register, so the result does not
 // depend on store visibility.  Metadata outside its contract would write
 // outside the cache: the row is skipped.

@@ -26,7 +26,7 @@ __global__ __launch_bounds__(256) void append_kernel(AppendParams p) {
   const int s = p.page_indptr[b], e = p.page_indptr[b + 1];
   const int n_pages = e - s;
   if (n_pages <= 0) return;
-  uint32_t* kbar_row = p.kbar ? p.kbar + (((int64_t)b * p.kbar_pages + (n_pages - 1)) * p.num_kv_heads + h) * (kHeadDim / 2)
+  uint32_t* kbar_row = p.kbar ? p.kbar + kbar_row_index(b, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2)
                               : nullptr;
   append_token_row(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2), p.kv_cache, kbar_row,
                    p.page_indices[e - 1], p.last_page_len[b], n_pages, p.kbar_pages, h, p.num_kv_heads, p.num_pages, lane);
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(256) void build_kbar_kernel(AppendParams p, int pag
   const int64_t page_dwords = 2LL * kPageSize * row_stride;
   const u32x4* kplane = reinterpret_cast<const u32x4*>(p.kv_cache + pid * page_dwords + h * (kHeadDim / 2)) + c16;
   const u32x4 m = page_mean_16B(kplane, row_stride / 4);
-  reinterpret_cast<u32x4*>(p.kbar + (((int64_t)b * p.kbar_pages + page) * p.num_kv_heads + h) * (kHeadDim / 2))[c16] = m;
+  reinterpret_cast<u32x4*>(p.kbar + kbar_row_index(b, h, page, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2))[c16] = m;
 }
 
 // ---- ragged multi-token append ------------------------------------------------
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(256) void append_ragged_kernel(RaggedAppendParams p
 // append_ragged_kernel on the same stream.
 __global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p) {
   __shared__ int64_t src16[kRaggedRows];  // K plane of the page a row completed, in 16-byte units; -1: none
-  __shared__ int64_t dst16[kRaggedRows];  // its mean-key row for head 0, in 16-byte units
+  __shared__ int64_t dst16[kRaggedRows];  // its mean-key row for head 0, in 16-byte units (head h: + h * kbar_pages rows)
   const int tid = threadIdx.x;
   const int64_t row0 = (int64_t)blockIdx.x * kRaggedRows;
   const int rows_here = (int)min((int64_t)kRaggedRows, p.nnz - row0);
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p)
           const int64_t pid = p.page_indices[s + (int)page];
           if (pid >= 0 && pid < p.num_pages) {
             src = pid * 2 * kPageSize * cpr;
-            dst = (((int64_t)b * p.kbar_pages + page) * p.num_kv_heads) * (kHeadDim / 8);
+            dst = kbar_row_index(b, 0, (int)page, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 8);
           }
         }
       }
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p)
     const int64_t src = src16[r];
     if (src < 0) continue;
     const u32x4 m = page_mean_16B(cache + src + h * (kHeadDim / 8) + c16, cpr);
-    kbar[dst16[r] + h * (kHeadDim / 8) + c16] = m;
+    kbar[dst16[r] + (int64_t)h * p.kbar_pages * (kHeadDim / 8) + c16] = m;
   }
 }
 

@@ -77,6 +77,13 @@ inline size_t score_workspace_bytes(int64_t items, int kbar_pages) {
   return score_count_bytes(items) + (size_t)items * score_key_stride(kbar_pages) * sizeof(uint32_t);
 }
 
+// Row of kbar[batch, num_kv_heads, kbar_pages, head_dim] that holds the mean key
+// of logical page `page` of (sequence b, KV head h): head-major, so the
+// candidates of one list are one contiguous run of 256-byte rows.
+__host__ __device__ inline int64_t kbar_row_index(int b, int h, int page, int num_kv_heads, int kbar_pages) {
+  return ((int64_t)b * num_kv_heads + h) * kbar_pages + page;
+}
+
 // ---- device side -----------------------------------------------------------
 #if defined(__HIPCC__)
 

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
     n = p.list_indptr[b + 1] - s;
   } else {
     pl = p.page_ids + (int64_t)list * p.list_stride;
-    n = p.list_count[list];
+    n = min(p.list_count[list], p.list_stride);  // a count beyond the row would run into the next list
   }
   n = max(n, 0);
   const int per_split = (n + p.num_splits - 1) / p.num_splits;

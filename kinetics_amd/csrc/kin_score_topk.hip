@@ -51,11 +51,9 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
   SelectArgs a;
   a.q_bh = p.q + ((int64_t)b * p.num_q_heads + (int64_t)h * p.group) * kHeadDim;
   a.G = p.group;
-  a.row_stride_b = p.num_kv_heads * kRowBytes;
   a.n_pages = n_pages;
   split_pages(n_pages, p.last_page_len[b], p.sink_pages, p.local_tokens, p.kbar_pages, a.n_sink, a.n_cand, a.n_local);
-  a.kb = reinterpret_cast<const char*>(p.kbar) +
-         (((int64_t)b * p.kbar_pages + a.n_sink) * p.num_kv_heads + h) * kRowBytes;
+  a.kb = reinterpret_cast<const char*>(p.kbar) + kbar_row_index(b, h, a.n_sink, p.num_kv_heads, p.kbar_pages) * kRowBytes;
   a.topk = p.topk;
   a.table = p.page_indices + ps;
   a.sel_logical = p.sel_logical ? p.sel_logical + (int64_t)item * p.topk : nullptr;

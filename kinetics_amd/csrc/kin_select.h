@@ -33,8 +33,7 @@ constexpr int kRankSortMax = 512;   // up to here winners are ordered by countin
 struct SelectArgs {
   const uint16_t* q_bh;       // the group's G query rows
   int G;
-  const char* kb;             // representative key of the first candidate of (b, h)
-  int row_stride_b;           // bytes between consecutive logical pages
+  const char* kb;             // representative key of the first candidate of (b, h); the others follow, 256 B each
   int n_pages;                // pages of the sequence (>= 1)
   int n_sink;                 // leading pages that are always attended (not candidates)
   int n_cand;                 // candidates: logical pages n_sink .. n_sink + n_cand - 1
@@ -139,12 +138,15 @@ __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, 
 #pragma unroll
     for (int u = 0; u < 8; ++u) qm[u] *= inv;
   }
-  // The candidates of (b, h) are rows of 256 B at a fixed stride.  They are read
+  // The candidates of (b, h) are contiguous rows of 256 B.  They are read
   // through a buffer descriptor that ends after the last wanted row, so loads past
   // the end return zeros without touching memory and the loop needs no branches:
   // each lane keeps kUnroll 16-byte loads in flight, re-issuing slot j for the
-  // next pass as soon as it has consumed it.
-  const int row_stride_b = a.row_stride_b;  // bytes between logical pages
+  // next pass as soon as it has consumed it.  The hardware compares only the
+  // per-lane (VGPR) offset with the descriptor's size -- the scalar offset operand
+  // is added after the range check -- so the whole offset travels in the VGPR and
+  // the scalar operand stays 0.
+  constexpr int row_stride_b = kRowBytes;  // the list's mean keys are contiguous rows (head-major kbar)
   const int n = r1 > r0 ? r1 - r0 : 0;
   const char* kb = a.kb + (int64_t)r0 * row_stride_b;
   float* sc_out = a.scores_out;
@@ -157,11 +159,11 @@ __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, 
   for (int j = 0; j < kUnroll; ++j)
     w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + j * kRows * row_stride_b, 0, kStreamLoad);
   for (int base = 0; base < n; base += kRows * kUnroll) {
-    const int next_off = (base + kRows * kUnroll) * row_stride_b;
+    const int next_off = lane_off + (base + kRows * kUnroll) * row_stride_b;
 #pragma unroll
     for (int j = 0; j < kUnroll; ++j) {
       const u32x4 x = w[j];
-      w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + j * kRows * row_stride_b, next_off, kStreamLoad);
+      w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, next_off + j * kRows * row_stride_b, 0, kStreamLoad);
       float acc = 0.f;
       acc = fmaf(qm[0], bf16_lo(x.x), acc); acc = fmaf(qm[1], bf16_hi(x.x), acc);
       acc = fmaf(qm[2], bf16_lo(x.y), acc); acc = fmaf(qm[3], bf16_hi(x.y), acc);

@@ -83,7 +83,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   auto append_token = [&]() {
     if (p.k != nullptr && tid < 64) {
       uint32_t* kbar_row =
-          reinterpret_cast<uint32_t*>(p.kbar) + (((int64_t)b * p.kbar_pages + (n_pages - 1)) * p.num_kv_heads + h) * (kHeadDim / 2);
+          reinterpret_cast<uint32_t*>(p.kbar) + kbar_row_index(b, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2);
       append_token_row(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2),
                        reinterpret_cast<uint32_t*>(p.kv), kbar_row, p.page_indices[pe - 1], last_len, n_pages, p.kbar_pages, h,
                        p.num_kv_heads, p.num_pages, tid);
@@ -99,11 +99,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   SelectArgs s;
   s.q_bh = p.q + hq0 * kHeadDim;
   s.G = G;
-  s.row_stride_b = p.num_kv_heads * kRowBytes;
   s.n_pages = n_pages;
   split_pages(n_pages, last_len, p.sink_pages, p.local_tokens, p.kbar_pages, s.n_sink, s.n_cand, s.n_local);
-  s.kb = reinterpret_cast<const char*>(p.kbar) +
-         (((int64_t)b * p.kbar_pages + s.n_sink) * p.num_kv_heads + h) * kRowBytes;
+  s.kb = reinterpret_cast<const char*>(p.kbar) + kbar_row_index(b, h, s.n_sink, p.num_kv_heads, p.kbar_pages) * kRowBytes;
   s.topk = p.topk;
   s.table = p.page_indices + ps;
   s.sel_logical = nullptr;

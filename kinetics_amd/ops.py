@@ -82,17 +82,21 @@ def _cache_dims(kv_cache: torch.Tensor):
 
 
 def _kbar_pages(kbar: torch.Tensor, batch: int, num_kv_heads: int, head_dim: int) -> int:
-    """kbar is [B, pages, Hkv, D], or the reference's [B, pages, D] when Hkv == 1."""
+    """kbar is [B, Hkv, pages, D] (head-major), or the reference's [B, pages, D]
+    when Hkv == 1 (the same bytes)."""
     _require(kbar, "kbar", torch.bfloat16, (3, 4))
     if kbar.dim() == 3:
         ok = num_kv_heads == 1 and kbar.shape[0] == batch and kbar.shape[2] == head_dim
+        pages = kbar.shape[1]
     else:
-        ok = kbar.shape[0] == batch and kbar.shape[2] == num_kv_heads and kbar.shape[3] == head_dim
+        ok = kbar.shape[0] == batch and kbar.shape[1] == num_kv_heads and kbar.shape[3] == head_dim
+        pages = kbar.shape[2]
     if not ok:
         raise ValueError(
-            f"kbar shape {tuple(kbar.shape)} does not match batch={batch}, num_kv_heads={num_kv_heads}, head_dim={head_dim}"
+            f"kbar shape {tuple(kbar.shape)} does not match batch={batch}, num_kv_heads={num_kv_heads}, head_dim={head_dim} "
+            "(expected [batch, num_kv_heads, pages, head_dim])"
         )
-    return kbar.shape[1]
+    return pages
 
 
 def _table(page_indices, page_indptr, last_page_len, batch, device):

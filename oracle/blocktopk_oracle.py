@@ -117,7 +117,8 @@ def page_mean_key(page_k_bits: np.ndarray) -> np.ndarray:
 def append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len):
     """benchmark/blocktopk_decoder.py:209-213 (LiteSys copy_to_cache,
     cache_utils.py:5-51).  In place.  k, v: [B, Hkv, D] bits; kv_cache: [P, 2, ps, Hkv, D] bits;
-    kbar: [B, kbar_pages, Hkv, D] bits or None.  Writes the new token at slot
+    kbar: [B, Hkv, kbar_pages, D] bits or None (head-major; [B, pages, D] of
+    the reference, blocktopk_decoder.py:165-168, when Hkv == 1).  Writes the new token at slot
     ``last_page_len[b]-1`` of the last page; a page that becomes full gets its
     mean key stored at its logical index."""
     B, Hkv, _ = k.shape
@@ -129,9 +130,9 @@ def append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_l
         pid, pos = int(pages[-1]), int(last_page_len[b]) - 1
         kv_cache[pid, 0, pos] = k[b]
         kv_cache[pid, 1, pos] = v[b]
-        if kbar is not None and pos == ps - 1 and len(pages) - 1 < kbar.shape[1]:
+        if kbar is not None and pos == ps - 1 and len(pages) - 1 < kbar.shape[2]:
             for h in range(Hkv):
-                kbar[b, len(pages) - 1, h] = page_mean_key(kv_cache[pid, 0, :, h, :])
+                kbar[b, h, len(pages) - 1] = page_mean_key(kv_cache[pid, 0, :, h, :])
 
 
 def append_paged_kv_ragged(k, v, append_indptr, kv_cache, kbar, page_indices, page_indptr, last_page_len):
@@ -157,8 +158,8 @@ def append_paged_kv_ragged(k, v, append_indptr, kv_cache, kbar, page_indices, pa
             kv_cache[pages[pos // ps], 1, pos % ps] = v[a0 + i]
         if kbar is not None:
             for p in range(first // ps, kv_len // ps):
-                if p < kbar.shape[1]:
-                    kbar[b, p] = page_mean_key(kv_cache[pages[p], 0].transpose(1, 0, 2))
+                if p < kbar.shape[2]:
+                    kbar[b, :, p] = page_mean_key(kv_cache[pages[p], 0].transpose(1, 0, 2))
 
 
 def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len):
@@ -170,10 +171,10 @@ def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len):
         if len(pages) == 0:
             continue
         n_full = len(pages) if int(last_page_len[b]) >= ps else len(pages) - 1
-        n_full = min(n_full, kbar.shape[1])
+        n_full = min(n_full, kbar.shape[2])
         if n_full > 0:
-            # [n_full, ps, Hkv, D] -> [n_full, Hkv, ps, D]
-            kbar[b, :n_full] = page_mean_key(kv_cache[pages[:n_full], 0].transpose(0, 2, 1, 3))
+            # [n_full, ps, Hkv, D] -> [Hkv, n_full, ps, D]
+            kbar[b, :, :n_full] = page_mean_key(kv_cache[pages[:n_full], 0].transpose(2, 0, 1, 3))
 
 
 # ---------------------------------------------------------------------------
@@ -200,11 +201,11 @@ def split_pages(n_pages, last_len, sink_pages, local_tokens, kbar_pages):
 
 
 def block_scores(q, kbar, page_indptr, last_page_len, sink_pages=0, local_tokens=1):
-    """score[b][h][n] = mean_g q[b, h*G+g, :] . kbar[b, n_sink + n, h, :] in
+    """score[b][h][n] = mean_g q[b, h*G+g, :] . kbar[b, h, n_sink + n, :] in
     float64 over the candidate pages.  Returns a list (b) of lists (h) of
     float64 arrays."""
     B, Hq, D = q.shape
-    Hkv = kbar.shape[2]
+    Hkv = kbar.shape[1]
     G = Hq // Hkv
     qf = bf16_to_f32(q).astype(np.float64)
     out = []
@@ -213,11 +214,11 @@ def block_scores(q, kbar, page_indptr, last_page_len, sink_pages=0, local_tokens
         if n_pages <= 0:
             out.append([np.zeros(0) for _ in range(Hkv)])
             continue
-        n_sink, n_cand, _ = split_pages(n_pages, last_page_len[b], sink_pages, local_tokens, kbar.shape[1])
-        kb = bf16_to_f32(kbar[b, n_sink : n_sink + n_cand]).astype(np.float64)  # [n, Hkv, D]
+        n_sink, n_cand, _ = split_pages(n_pages, last_page_len[b], sink_pages, local_tokens, kbar.shape[2])
+        kb = bf16_to_f32(kbar[b, :, n_sink : n_sink + n_cand]).astype(np.float64)  # [Hkv, n, D]
         per_head = []
         for h in range(Hkv):
-            per_q = np.einsum("gd,nd->gn", qf[b, h * G : (h + 1) * G], kb[:, h, :])  # [G, n]
+            per_q = np.einsum("gd,nd->gn", qf[b, h * G : (h + 1) * G], kb[h])  # [G, n]
             per_head.append(per_q.mean(axis=0))
         out.append(per_head)
     return out
@@ -249,7 +250,7 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
     the candidates).  List order: sink pages, winners (descending score), local
     pages with the open page last."""
     B = q.shape[0]
-    Hkv = kbar.shape[2]
+    Hkv = kbar.shape[1]
     stride = sel_list_capacity(topk, sink_pages, local_tokens) if sel_stride is None else sel_stride
     scores = block_scores(q, kbar, page_indptr, last_page_len, sink_pages, local_tokens)
     sel_pages = np.full((B, Hkv, stride), -1, dtype=np.int32)
@@ -262,7 +263,7 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
             if len(pages) == 0:
                 row.append(np.zeros(0, dtype=np.int64))
                 continue
-            n_sink, _, n_local = split_pages(len(pages), last_page_len[b], sink_pages, local_tokens, kbar.shape[1])
+            n_sink, _, n_local = split_pages(len(pages), last_page_len[b], sink_pages, local_tokens, kbar.shape[2])
             idx = n_sink + select_topk(scores[b][h], topk)
             full = np.concatenate([pages[:n_sink], pages[idx], pages[len(pages) - n_local :]])
             sel_pages[b, h, : len(full)] = full

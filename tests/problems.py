@@ -22,7 +22,7 @@ class Problem:
     k: np.ndarray               # [B, Hkv, D]
     v: np.ndarray               # [B, Hkv, D]
     kv_cache: np.ndarray        # [P, 2, ps, Hkv, D]
-    kbar: np.ndarray            # [B, kbar_pages, Hkv, D]  (state BEFORE the append)
+    kbar: np.ndarray            # [B, Hkv, kbar_pages, D]  (state BEFORE the append)
     page_indices: np.ndarray    # int32 [nnz]
     page_indptr: np.ndarray     # int32 [B+1]
     last_page_len: np.ndarray   # int32 [B]   (state AFTER the append)
@@ -117,7 +117,7 @@ def make_problem(seed: int, lengths, num_kv_heads: int = 1, group: int = 4, topk
     k = randn_bf16(rng, (B, num_kv_heads, D))
     v = randn_bf16(rng, (B, num_kv_heads, D))
     kbar_pages = int(n_pages.max()) + kbar_slack if B else 1
-    kbar = np.zeros((B, kbar_pages, num_kv_heads, D), dtype=np.uint16)
+    kbar = np.zeros((B, num_kv_heads, kbar_pages, D), dtype=np.uint16)
     if build_kbar:
         # state before the append: the last page is not full yet (its final slot is still unwritten)
         pre_last = np.maximum(last_len - 1, 0).astype(np.int32)

@@ -41,7 +41,7 @@ class Gpu:
         self.sel = torch.full((pb.B, pb.Hkv, pb.topk + 1), -7, dtype=torch.int32, device=DEV)
         self.cnt = torch.full((pb.B, pb.Hkv), -7, dtype=torch.int32, device=DEV)
         self.logical = torch.full((pb.B, pb.Hkv, pb.topk), -7, dtype=torch.int32, device=DEV)
-        self.scores = torch.full((pb.B, pb.Hkv, pb.kbar.shape[1]), float("nan"), dtype=torch.float32, device=DEV)
+        self.scores = torch.full((pb.B, pb.Hkv, pb.kbar.shape[2]), float("nan"), dtype=torch.float32, device=DEV)
 
 
 def check_table(ops, g: Gpu):
@@ -156,7 +156,7 @@ def test_score_topk_ties_take_lowest_index(ops):
     qm = O.bf16_to_f32(pb2.q[0]).astype(np.float64).mean(axis=0)
     big = O.f32_to_bf16((qm * 4).astype(np.float32))  # aligned with the mean query: clearly the largest score
     for p in (17, 200, 5):
-        pb2.kbar[0, p, 0] = big
+        pb2.kbar[0, 0, p] = big
     g2 = Gpu(pb2)
     sel, cnt, logical, scores = run_select(ops, g2)
     assert sorted(logical[0, 0, :3].tolist()) == [5, 17, 200]
@@ -353,7 +353,7 @@ def test_properties_at_scale(ops):
     indices = table.reshape(-1).contiguous()
     indptr = (torch.arange(B + 1, device=DEV, dtype=torch.int32) * n_pages).contiguous()
     last = torch.full((B,), 1, dtype=torch.int32, device=DEV)
-    kbar = torch.zeros(B, n_pages, 1, D, dtype=torch.bfloat16, device=DEV)
+    kbar = torch.zeros(B, 1, n_pages, D, dtype=torch.bfloat16, device=DEV)
     ops.build_kbar(kv, kbar, indices, indptr, last)
     sel = torch.empty(B, 1, topk + 1, dtype=torch.int32, device=DEV)
     cnt = torch.empty(B, 1, dtype=torch.int32, device=DEV)
@@ -463,7 +463,7 @@ def _uniform_state(B, ctx, hkv, group, topk, seed):
     st = dict(kv=kv, table=table, indices=table.reshape(-1).contiguous(),
               indptr=(torch.arange(B + 1, dtype=torch.int32, device=DEV) * n_pages).contiguous(),
               last=torch.ones(B, dtype=torch.int32, device=DEV),
-              kbar=torch.zeros(B, n_pages, hkv, D, dtype=torch.bfloat16, device=DEV),
+              kbar=torch.zeros(B, hkv, n_pages, D, dtype=torch.bfloat16, device=DEV),
               q=torch.randn(B, hkv * group, D, generator=gen, device=DEV).to(torch.bfloat16),
               k=torch.randn(B, hkv, D, generator=gen, device=DEV).to(torch.bfloat16),
               v=torch.randn(B, hkv, D, generator=gen, device=DEV).to(torch.bfloat16),
@@ -593,7 +593,7 @@ def test_full_size_continuous_batching_mix(ops):
     indices, ptr, last_t = P.int_tensor(ids, DEV), P.int_tensor(indptr, DEV), P.int_tensor(last, DEV)
     ops.check_page_table(indices, ptr, last_t, PS, total)
     max_pages = int(n_pages.max())
-    kbar = torch.zeros(B, max_pages, hkv, D, dtype=torch.bfloat16, device=DEV)
+    kbar = torch.zeros(B, hkv, max_pages, D, dtype=torch.bfloat16, device=DEV)
     q = torch.randn(B, hkv * group, D, generator=gen, device=DEV).to(torch.bfloat16)
     k = torch.randn(B, hkv, D, generator=gen, device=DEV).to(torch.bfloat16)
     v = torch.randn(B, hkv, D, generator=gen, device=DEV).to(torch.bfloat16)
@@ -687,7 +687,7 @@ def test_fused_step_split_scoring_for_few_long_sequences(ops, hkv, group):
     cache bytes, page lists and output as without it, call after call."""
     lengths = [PS * 2500 + 3, PS * 2100 + 16, 5, 0, PS * 300 + 1][: max(2, 10 // hkv)]
     pb = P.make_problem(1400 + hkv, lengths, num_kv_heads=hkv, group=group, topk=40)
-    kbar_pages = pb.kbar.shape[1]
+    kbar_pages = pb.kbar.shape[2]
     need = ops.step_workspace_bytes(pb.B, hkv, kbar_pages)
     assert need > 0 and ops.step_workspace_bytes(4096, 1, kbar_pages) == 0 and ops.step_workspace_bytes(2, 1, 512) == 0
     ws = torch.full((need,), 0xAB, dtype=torch.uint8, device=DEV)       # contents need no initialisation
@@ -752,7 +752,7 @@ def test_seeded_sweep_of_split_scoring(ops):
         sink, local = int(rng.integers(0, 3)), int(rng.choice([1, 17, 40]))
         what = f"trial {trial}: hkv={hkv} G={group} lengths={lengths} topk={topk} sink={sink} local={local}"
         pb = P.make_problem(6100 + trial, lengths, num_kv_heads=hkv, group=group, topk=topk)
-        need = ops.step_workspace_bytes(pb.B, hkv, pb.kbar.shape[1])
+        need = ops.step_workspace_bytes(pb.B, hkv, pb.kbar.shape[2])
         assert need > 0, what
         ws = torch.full((need,), 0xCD, dtype=torch.uint8, device=DEV)
         cap = ops.sel_list_capacity(topk, sink, local)
@@ -1127,10 +1127,10 @@ def test_step_replays_under_hip_graph(ops, path):
     g = Gpu(pb)
     out = torch.empty_like(g.q)
     ws = workspace(ops, pb, pb.topk + 1, 0)
-    step_ws = torch.empty(max(16, ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[1])), dtype=torch.uint8, device=DEV)
+    step_ws = torch.empty(max(16, ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[2])), dtype=torch.uint8, device=DEV)
     tok_ws = torch.empty(max(16, ops.strided_topk_workspace_bytes(pb.B, pb.Hkv, pb.max_pages)), dtype=torch.uint8, device=DEV)
     tok_sel = torch.full((pb.B, pb.Hkv, 64 * 16 + 4 + 16), -1, dtype=torch.int32, device=DEV)
-    assert path.endswith("_split") == (ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[1]) > 0)
+    assert path.endswith("_split") == (ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[2]) > 0)
 
     def step():
         if path in ("three", "three_split"):
@@ -1416,7 +1416,7 @@ def test_sink_and_local_pages(ops, sink, local, offset, fused):
                 ws = res["scores"][b][h]
                 n_pages = (lengths[b] + PS - 1) // PS
                 if n_pages:
-                    n_sink = O.split_pages(n_pages, pb.last_page_len[b], sink, local, pb.kbar.shape[1])[0]
+                    n_sink = O.split_pages(n_pages, pb.last_page_len[b], sink, local, pb.kbar.shape[2])[0]
                     assert np.allclose(scores[b, h, n_sink : n_sink + len(ws)], ws, rtol=1e-5, atol=1e-5)
 
 
@@ -1508,7 +1508,7 @@ def test_seeded_sweep_of_shapes(ops):
                 pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
                 if len(pages) == 0:
                     continue
-                n_sink = O.split_pages(len(pages), pb.last_page_len[b], sink, local, pb.kbar.shape[1])[0]
+                n_sink = O.split_pages(len(pages), pb.last_page_len[b], sink, local, pb.kbar.shape[2])[0]
                 lookup = {int(p): i for i, p in enumerate(pages)}
                 for h in range(hkv):
                     k_eff = len(res["sel_logical"][b][h])

@@ -67,10 +67,10 @@ def test_append_writes_exactly_one_slot(residue):
         if L % PS == 0:
             pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
             want = O.page_mean_key(pb.kv_cache[pages[-1], 0].transpose(1, 0, 2))
-            assert np.array_equal(kbar[b, n_pages - 1], want)
-            mask = np.ones(kbar.shape[1], dtype=bool)
+            assert np.array_equal(kbar[b, :, n_pages - 1], want)
+            mask = np.ones(kbar.shape[2], dtype=bool)
             mask[n_pages - 1] = False
-            assert np.array_equal(kbar[b, mask], pb.kbar[b, mask])
+            assert np.array_equal(kbar[b][:, mask], pb.kbar[b][:, mask])
         else:
             assert np.array_equal(kbar[b], pb.kbar[b])
 
@@ -106,13 +106,13 @@ def test_build_kbar_covers_full_pages_only():
     full = [4, 2, 0, 0]
     for b in range(4):
         pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
-        for p in range(kbar.shape[1]):
+        for p in range(kbar.shape[2]):
             if p < full[b]:
                 for h in range(2):
                     want = O.page_mean_key(pb.kv_cache[pages[p], 0, :, h, :])
-                    assert np.array_equal(kbar[b, p, h], want)
+                    assert np.array_equal(kbar[b, h, p], want)
             else:
-                assert np.all(kbar[b, p] == sentinel)
+                assert np.all(kbar[b, :, p] == sentinel)
 
 
 def _ragged_case(seed, before, new, hkv=2, slack=2):
@@ -179,10 +179,10 @@ def test_scores_identities():
             assert sc[b][h].shape == (n_cand,)
             # mean_g (q_g . k) == (mean_g q_g) . k
             qbar = qf[b, 4 * h : 4 * h + 4].mean(axis=0)
-            kb = O.bf16_to_f32(pb.kbar[b, :n_cand, h]).astype(np.float64)
+            kb = O.bf16_to_f32(pb.kbar[b, h, :n_cand]).astype(np.float64)
             assert np.allclose(sc[b][h], kb @ qbar, rtol=1e-12, atol=1e-12)
             # not the other head's keys, not the other head's queries
-            other = O.bf16_to_f32(pb.kbar[b, :n_cand, 1 - h]).astype(np.float64) @ qbar
+            other = O.bf16_to_f32(pb.kbar[b, 1 - h, :n_cand]).astype(np.float64) @ qbar
             assert not np.allclose(sc[b][h], other)
 
 
@@ -198,7 +198,7 @@ def test_scores_equal_litesys_group_mean_then_block_mean():
     kv[:n_pages, 0, :, 0] = O.f32_to_bf16(K)
     indices = np.arange(n_pages + 1, dtype=np.int32)
     indptr = np.array([0, n_pages + 1], dtype=np.int32)
-    kbar = np.zeros((1, n_pages + 1, 1, D), dtype=np.uint16)
+    kbar = np.zeros((1, 1, n_pages + 1, D), dtype=np.uint16)
     O.build_kbar(kv, kbar, indices, indptr, np.array([1], dtype=np.int32))
     q = P.randn_bf16(rng, (1, G, D))
     sc = O.block_scores(q, kbar, indptr, np.array([1], dtype=np.int32))[0][0]
@@ -382,7 +382,7 @@ def test_torch_path_agrees_with_oracle():
     kv_t = P.to_torch(pb.kv_cache.copy())
     table = torch.from_numpy(pb.page_indices.astype(np.int64)).reshape(B, n_pages)
     out_t, idx_t = torch_path.blocktopk_decode_step(
-        P.to_torch(pb.q), P.to_torch(pb.k), P.to_torch(pb.v), kv_t, P.to_torch(pb.kbar[:, : n_pages - 1, 0]),
+        P.to_torch(pb.q), P.to_torch(pb.k), P.to_torch(pb.v), kv_t, P.to_torch(pb.kbar[:, 0, : n_pages - 1]),
         table, torch.from_numpy(pb.last_page_len.astype(np.int64)), topk)
     res = O.decode_step(pb.q, pb.k, pb.v, pb.kv_cache, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, topk)
     assert np.array_equal(P.from_torch(kv_t), pb.kv_cache)  # same append
@@ -507,7 +507,7 @@ def test_page_lists_with_offset_12_equal_litesys_mask_formulation():
         kv[perm, 1] = flat_v.reshape(n_pages, PS, Hkv, D)
         indptr = np.array([0, n_pages], dtype=np.int32)
         last = np.array([cache_len - (n_pages - 1) * PS], dtype=np.int32)
-        kbar = np.zeros((1, n_pages, Hkv, D), dtype=np.uint16)
+        kbar = np.zeros((1, Hkv, n_pages, D), dtype=np.uint16)
         O.build_kbar(kv, kbar, perm, indptr, last)
         sel, cnt, logical, _ = O.block_score_topk(q, kbar, perm, indptr, last, topk, sink_pages=1, local_tokens=local)
         out, _ = O.sparse_paged_decode(q, kv, sel, cnt, last, first_page_offset=pad)

@@ -34,7 +34,7 @@ class Gpu:
 
 def _both_ways(ops, pb, sink, local, what, must_split):
     cap = ops.sel_list_capacity(pb.topk, sink, local)
-    need = ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[1])
+    need = ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[2])
     assert (need > 0) == must_split, what
     a, b = Gpu(pb, cap), Gpu(pb, cap)
     ws = torch.full((max(need, 16),), 0x5A, dtype=torch.uint8, device=DEV)
