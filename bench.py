@@ -10,11 +10,22 @@ one layer on one GPU's share of the heads).  Sequence lengths stay fixed across
 steps, as in the reference harness whose metadata never changes.
 
 Prints ONE JSON line.  ``value`` is decode tokens/s per layer with every input
-already resident in HBM.  ``roofline`` describes the dominant kernel (the sparse
-paged attention), ``step_hbm`` the whole step against the algorithmic-bytes
-model, ``cpu_baseline`` the torch-CPU restatement of the reference path timed on
-this machine's host cores, ``dense_baseline`` the dense paged decode on the same
-tensors.
+already resident in HBM.  ``roofline`` describes the dominant kernel (the fused
+step kernel, or the sparse paged attention with --mode three); its ``achieved``
+is algorithmic bytes over the kernel's HIP-event time measured in this run,
+while ``traffic`` is NOT measured by this run: it is read from
+profiles/hbm_traffic.json, which holds the rocprofv3 --pmc FETCH_SIZE /
+WRITE_SIZE figures of an earlier run of the same kernel and workload
+(``traffic_source`` says so in the line).  ``step_hbm`` is the whole step
+against the algorithmic-bytes model, ``cpu_baseline`` the torch-CPU restatement
+of the reference path timed on this machine's host cores (a slice of the
+headline workload, and the tiny configuration in full), ``dense_baseline`` the
+dense paged decode on the same tensors.  For the headline workload the same
+line also carries ``workloads`` (the other BASELINE configurations, each
+measured the same way on its own cache), ``token_topk`` / ``strided_topk``
+(LiteSys' token-granular policies on the headline cache) and the figure in the
+reference's printed normalisation (divided by world_size * num_hidden_layers,
+benchmark/blocktopk.py:82).
 """
 from __future__ import annotations
 
@@ -146,7 +157,9 @@ def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2, ragged=False, 
 
 def cpu_baseline(torch, B_cpu, ctx, G, topk, budget_s=20.0):
     """The reference's torch path (oracle/torch_path.py) on the host cores, on a
-    slice of the workload: B_cpu sequences of the same context length."""
+    slice of the workload: B_cpu sequences of the same context length.  Scores in
+    bf16 as the reference computes them (benchmark/blocktopk_decoder.py:216), and
+    in fp32 beside it."""
     from oracle import torch_path
 
     cores = os.cpu_count() or 1
@@ -165,20 +178,28 @@ def cpu_baseline(torch, B_cpu, ctx, G, topk, budget_s=20.0):
     k = torch.randn(B_cpu, 1, D, generator=g).to(torch.bfloat16)
     v = torch.randn(B_cpu, 1, D, generator=g).to(torch.bfloat16)
     last = torch.ones(B_cpu, dtype=torch.int64)
-    times = []
-    for _ in range(3):
-        torch_path.blocktopk_decode_step(q, k, v, kv, kbar, table, last, topk)
-    t_end = time.perf_counter() + budget_s
-    while len(times) < 10 or (time.perf_counter() < t_end and len(times) < 200):
-        t0 = time.perf_counter()
-        torch_path.blocktopk_decode_step(q, k, v, kv, kbar, table, last, topk)
-        times.append(time.perf_counter() - t0)
-    med = statistics.median(times)
-    return dict(value=B_cpu / med, unit="tokens/s", cores=cores, kind="port",
+    med, count = {}, {}
+    for dt in (torch.bfloat16, torch.float32):
+        times = []
+        for _ in range(3):
+            torch_path.blocktopk_decode_step(q, k, v, kv, kbar, table, last, topk, compute_dtype=dt)
+        t_end = time.perf_counter() + budget_s / 2
+        while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 200):
+            t0 = time.perf_counter()
+            torch_path.blocktopk_decode_step(q, k, v, kv, kbar, table, last, topk, compute_dtype=dt)
+            times.append(time.perf_counter() - t0)
+        med[dt], count[dt] = statistics.median(times), len(times)
+    m = med[torch.bfloat16]
+    return dict(value=B_cpu / m, unit="tokens/s", cores=cores, cpu_model=cpu_model_name(), kind="port",
+                value_fp32_scores=B_cpu / med[torch.float32],
                 sample=f"torch-CPU restatement of the reference path (oracle/torch_path.py), {B_cpu} of the batch's "
-                       f"sequences at ctx={ctx}, k={topk}, median of {len(times)} steps after 3 warm-ups, "
-                       f"{med * 1e3:.2f} ms/step; tokens/s is linear in batch")
+                       f"sequences at ctx={ctx}, k={topk}, page scores in bf16 as the reference computes them "
+                       f"(value_fp32_scores: in fp32), median of {count[torch.bfloat16]} steps after 3 warm-ups, "
+                       f"{m * 1e3:.2f} ms/step; tokens/s is linear in batch")
 
+
+# (world_size, num_hidden_layers) the reference's printed figure is divided by (benchmark/blocktopk.py:82)
+REFERENCE_NORMALISATION = {"qwen3-8b-share": (8, 36), "qwen3-8b-readme": (8, 36), "qwen3-32b-share": (8, 64)}
 
 WHOLE_LAYER_MODEL = {"qwen3-8b-share": ("Qwen3-8B", 8), "qwen3-32b-share": ("Qwen3-32B", 8),
                      "qwen3-8b-readme": ("Qwen3-8B", 8)}
@@ -247,6 +268,142 @@ def whole_layer(torch, args, B, ctx, topk, device):
     return out
 
 
+def cpu_model_name():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def time_step(torch, ops, st, B, Hkv, topk, steps, warmup, mode="auto"):
+    """W untimed and K timed decode steps on the state ``st``; HIP events on the
+    launch stream bracket every kernel.  Returns (ms_per_step, elapsed_s,
+    {kernel: mean ms}, fused?)."""
+    device = st["q"].device
+    fused = mode == "fused" or (mode == "auto" and ops.prefer_fused_step(B, Hkv, st["max_pages_used"], topk))
+    # few long lists: the scoring of a list is shared by several workgroups that meet through this
+    sws = ops.step_workspace_bytes(B, Hkv, st["kbar"].shape[2])
+    step_ws = torch.empty(sws, dtype=torch.uint8, device=device) if sws else None
+    if fused:
+        kernels = [("fused_step", lambda: ops.blocktopk_decode_step(
+            st["q"], st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"], topk,
+            out=st["out"], workspace=step_ws))]
+    else:
+        kernels = [
+            ("append", lambda: ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"],
+                                                   st["last"])),
+            ("score_topk", lambda: ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], st["last"], topk,
+                                                        st["sel"], st["cnt"], workspace=step_ws)),
+            ("sparse_attention", lambda: ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"],
+                                                                 out=st["out"], workspace=st["ws"])),
+        ]
+    for _ in range(warmup):
+        for _, fn in kernels:
+            fn()
+    torch.cuda.synchronize()
+    K = steps
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(kernels) + 1)] for _ in range(K)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        ev[i][0].record()
+        for j, (_, fn) in enumerate(kernels):
+            fn()
+            ev[i][j + 1].record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kernel_ms = {name: statistics.fmean(e[j].elapsed_time(e[j + 1]) for e in ev) for j, (name, _) in enumerate(kernels)}
+    return elapsed / K * 1e3, elapsed, kernel_ms, fused
+
+
+def time_dense(torch, ops, st, nd):
+    """The dense baseline (benchmark/dense_decoder.py:211-219) on the same tensors: ms per step."""
+    for _ in range(2):
+        ops.dense_paged_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], st["max_pages_used"],
+                               out=st["out"], workspace=st["ws_dense"])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(nd):
+        ops.append_paged_kv(st["k"], st["v"], st["kv"], None, st["indices"], st["indptr"], st["last"])
+        ops.dense_paged_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], st["max_pages_used"],
+                               out=st["out"], workspace=st["ws_dense"])
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / nd * 1e3
+
+
+def time_token_policies(torch, ops, st, B, Hkv, G, topk, nt, traffic_of):
+    """LiteSys' token-granular policies on the same cache with the same token
+    budget (topk_pages * 16 tokens, 4 sink tokens, a 16-token window): every key of
+    the context is streamed once (256 B per token), then the listed tokens' K and V rows."""
+    device = st["q"].device
+    ntok, sink, window = topk * PS, 4, 16
+    res = {}
+    tok_bytes = sum(Hkv * (L * 256 + min(L, ntok + sink + window) * 512 + 512) + 2 * Hkv * G * 256 for L in st["lengths"])
+    ws_tok = torch.empty(max(16, ops.token_topk_workspace_bytes(B, Hkv, st["max_pages_used"])), dtype=torch.uint8, device=device)
+    ws_str = torch.empty(max(16, ops.strided_topk_workspace_bytes(B, Hkv, st["max_pages_used"])), dtype=torch.uint8, device=device)
+    calls = {
+        "token_topk": lambda: ops.token_topk_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], ntok,
+                                                     st["max_pages_used"], sink_tokens=sink, local_tokens=window,
+                                                     out=st["out"], workspace=ws_tok),
+        # strided overlapping blocks with the same budget: topk blocks of 16 tokens, a block every 8 tokens
+        "strided_topk": lambda: ops.strided_topk_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], topk,
+                                                         st["max_pages_used"], sink_tokens=sink, local_tokens=window,
+                                                         out=st["out"], workspace=ws_str),
+    }
+    for name, call in calls.items():
+        for _ in range(2):
+            call()
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nt)]
+        t0 = time.perf_counter()
+        for e0, e1 in evs:
+            ops.append_paged_kv(st["k"], st["v"], st["kv"], None, st["indices"], st["indptr"], st["last"])
+            e0.record()
+            call()
+            e1.record()
+        torch.cuda.synchronize()
+        tt = (time.perf_counter() - t0) / nt
+        tks = [e0.elapsed_time(e1) for e0, e1 in evs]
+        tk = statistics.fmean(tks) * 1e-3
+        res[name] = {"sink_tokens": sink, "local_tokens": window, "ms_per_step": tt * 1e3, "value": B / tt,
+                     "unit": "tokens/s", "steps": nt, "algorithmic_bytes_per_step": tok_bytes, "kernel_ms": tk * 1e3,
+                     "kernel_ms_min": min(tks), "kernel_ms_max": max(tks), "achieved_gbs": tok_bytes / tk / 1e9,
+                     "frac": tok_bytes / tk / 1e9 / HBM_PEAK_GBS, "traffic": traffic_of(name + "_kernel")}
+    res["token_topk"]["topk_tokens"] = ntok
+    res["strided_topk"].update(topk_blocks=topk, block_size=PS, stride=8)
+    return res
+
+
+def side_workload(torch, ops, name, steps, warmup, device, with_dense=True):
+    """One of the other BASELINE configurations, measured like the headline:
+    cache built, K steps timed, dense baseline on the same tensors, cache freed."""
+    B, ctx, Hkv, G, topk, desc = WORKLOADS[name]
+    st = build_state(torch, ops, B, ctx, Hkv, G, topk, device, ragged=name in RAGGED)
+    torch.cuda.synchronize()
+    ms_step, elapsed, kernel_ms, fused = time_step(torch, ops, st, B, Hkv, topk, steps, warmup)
+    ab = algorithmic_bytes(st["lengths"], Hkv, G, topk)
+    out = {"description": desc, "batch": B, "ctx": ctx, "num_kv_heads": Hkv, "num_q_heads": Hkv * G, "topk_pages": topk,
+           "page_table": "ragged, half fragmented" if name in RAGGED else "reference layout p*B+b",
+           "kv_resident_gb": round(st["kv"].numel() * 2 / 1e9, 2), "launches_per_step": len(kernel_ms),
+           "steps": steps, "warmup": warmup, "ms_per_step": ms_step, "value": B * steps / elapsed, "unit": "tokens/s",
+           "kernels_ms": kernel_ms, "algorithmic_bytes_per_step": ab["step"],
+           "achieved_gbs": ab["step"] / (ms_step * 1e-3) / 1e9, "frac": ab["step"] / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    if fused:
+        out["kernel_frac"] = ab["step"] / (kernel_ms["fused_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS
+    if with_dense:
+        td = time_dense(torch, ops, st, max(3, min(10, steps // 10)))
+        out["dense_ms_per_step"] = td
+        out["dense_frac"] = ab["dense"] / (td * 1e-3) / 1e9 / HBM_PEAK_GBS
+        out["sparse_over_dense"] = td / ms_step
+    del st
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -264,8 +421,11 @@ def main():
                     help="also time the whole decoder layer (norms, GEMMs, MLP around the attention path), "
                          "the quantity benchmark/blocktopk.py prints")
     ap.add_argument("--token-topk", action="store_true",
-                    help="also time token-level top-k decode (LiteSys' attn_topk policy) with the same token budget "
-                         "(topk_pages * 16 tokens, 4 sink tokens, a 16-token window)")
+                    help="also time token-level top-k and strided-block decode (LiteSys' attn_topk / attn_stride "
+                         "policies) with the same token budget; on by default for the headline workload")
+    ap.add_argument("--no-side-workloads", action="store_true",
+                    help="headline workload only: skip the `workloads` block (the other configurations) and the "
+                         "token-granular policies")
     # the reference's own command line (benchmark/blocktopk.py:6-19, benchmark/README.md): a context of
     # gen_len / 2 tokens, the model's heads divided by world_size
     ap.add_argument("--model", default=None, help="e.g. Qwen/Qwen3-8B: build the workload from the reference's arguments")
@@ -308,52 +468,16 @@ def main():
     B, ctx, Hkv, G, topk, desc = WORKLOADS[args.workload]
     if args.batch:
         B = args.batch
+    headline = args.workload == "qwen3-8b-share" and not args.batch
     t_setup = time.perf_counter()
     st = build_state(torch, ops, B, ctx, Hkv, G, topk, device, ragged=args.workload in RAGGED)
     torch.cuda.synchronize()
     print(f"[bench] {args.workload}: B={B} ctx={ctx} H_kv={Hkv} G={G} topk={topk}, "
           f"KV {st['kv'].numel() * 2 / 1e9:.1f} GB resident, setup {time.perf_counter() - t_setup:.1f}s", file=sys.stderr)
 
-    fused = args.mode == "fused" or (args.mode == "auto" and ops.prefer_fused_step(B, Hkv, st["max_pages_used"], topk))
-
-    # few long lists: the scoring of a list is shared by several workgroups that meet through this
-    sws = ops.step_workspace_bytes(B, Hkv, st["kbar"].shape[1])
-    step_ws = torch.empty(sws, dtype=torch.uint8, device=device) if sws else None
-
-    def launches():
-        """The step's kernel launches, in order, as (name, callable)."""
-        if fused:
-            return [("fused_step", lambda: ops.blocktopk_decode_step(
-                st["q"], st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"], topk,
-                out=st["out"], workspace=step_ws))]
-        return [
-            ("append", lambda: ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"],
-                                                   st["last"])),
-            ("score_topk", lambda: ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], st["last"], topk,
-                                                        st["sel"], st["cnt"], workspace=step_ws)),
-            ("sparse_attention", lambda: ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"],
-                                                                 out=st["out"], workspace=st["ws"])),
-        ]
-
-    kernels = launches()
-    for _ in range(args.warmup):
-        for _, fn in kernels:
-            fn()
-    torch.cuda.synchronize()
     # -- the timed region: K steps; HIP events on the launch stream bracket each kernel
     K = args.steps
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(kernels) + 1)] for _ in range(K)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(K):
-        ev[i][0].record()
-        for j, (_, fn) in enumerate(kernels):
-            fn()
-            ev[i][j + 1].record()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_step = elapsed / K * 1e3
-    kernel_ms = {name: statistics.fmean(e[j].elapsed_time(e[j + 1]) for e in ev) for j, (name, _) in enumerate(kernels)}
+    ms_step, elapsed, kernel_ms, fused = time_step(torch, ops, st, B, Hkv, topk, K, args.warmup, args.mode)
 
     ab = algorithmic_bytes(st["lengths"], Hkv, G, topk)
     step_gbs = ab["step"] / (ms_step * 1e-3) / 1e9
@@ -365,11 +489,13 @@ def main():
                                                    "paged_decode_kernel", ab["attention"], kernel_ms["sparse_attention"])
         kernel_ms["score_topk_gbs"] = ab["score_select"] / (kernel_ms["score_topk"] * 1e-3) / 1e9
     dom_gbs = dom_bytes / (dom_ms * 1e-3) / 1e9
-    traffic = None
+    traffic_table = {}
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get(f"{args.workload}:B={B}", {}).get(dom_kernel)
+            traffic_table = json.load(f).get(f"{args.workload}:B={B}", {})
+    traffic = traffic_table.get(dom_kernel)
+    world, layers = REFERENCE_NORMALISATION.get(args.workload, (None, None))
 
     result = {
         "metric": "decode tok/s per layer, Qwen3-8B 1-GPU share B=4096 ctx=32K; HBM GB/s % peak",
@@ -388,15 +514,25 @@ def main():
                    "num_q_heads": Hkv * G, "head_dim": D, "page_size": PS, "topk_pages": topk,
                    "page_table": "ragged, half fragmented" if args.workload in RAGGED else "reference layout p*B+b",
                    "kv_resident_gb": round(st["kv"].numel() * 2 / 1e9, 2),
-                   "launches_per_step": len(kernels)},
+                   "launches_per_step": len(kernel_ms) - (0 if fused else 1)},
         "roofline": {"bound": "hbm", "kernel": dom_name,
                      "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom_gbs / HBM_PEAK_GBS,
-                     "traffic": traffic, "algorithmic_bytes_per_launch": dom_bytes,
+                     "traffic": traffic,
+                     "traffic_source": ("profiles/hbm_traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run "
+                                        "of this kernel on this workload, scaled by a 1 GiB copy; not measured by this run")
+                     if traffic is not None else None,
+                     "algorithmic_bytes_per_launch": dom_bytes,
                      "avg_launch_ms": dom_ms},
         "step_hbm": {"algorithmic_bytes_per_step": ab["step"], "bytes_per_seq": ab["per_seq"], "achieved": step_gbs,
                      "unit": "GB/s", "frac": step_gbs / HBM_PEAK_GBS},
         "kernels_ms": kernel_ms,
     }
+    if world:
+        # the figure benchmark/blocktopk.py:82 prints divides the per-layer rate by world_size * num_hidden_layers;
+        # it is built from the attention step alone here (the whole layer: --whole-layer)
+        result["normalised_like_reference_print"] = {
+            "value": B * K / elapsed / (world * layers), "unit": "tokens/s", "world_size": world, "num_hidden_layers": layers,
+            "note": "attention step only / (world_size * num_hidden_layers), cf. benchmark/blocktopk.py:82"}
 
     if args.calibrate_copy:
         src = torch.empty(1 << 29, dtype=torch.bfloat16, device=device).normal_()
@@ -408,85 +544,28 @@ def main():
 
     if not args.no_dense:
         nd = max(3, min(10, K // 10))
-        for _ in range(2):
-            ops.dense_paged_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], st["max_pages_used"],
-                                   out=st["out"], workspace=st["ws_dense"])
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(nd):
-            ops.append_paged_kv(st["k"], st["v"], st["kv"], None, st["indices"], st["indptr"], st["last"])
-            ops.dense_paged_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], st["max_pages_used"],
-                                   out=st["out"], workspace=st["ws_dense"])
-        torch.cuda.synchronize()
-        td = (time.perf_counter() - t0) / nd
+        td = time_dense(torch, ops, st, nd) * 1e-3
         dense_bytes = ab["dense"]
         result["dense_baseline"] = {"value": B / td, "unit": "tokens/s", "ms_per_step": td * 1e3, "steps": nd,
                                     "achieved_gbs": dense_bytes / td / 1e9, "frac": dense_bytes / td / 1e9 / HBM_PEAK_GBS,
                                     "sparse_over_dense": (B * K / elapsed) / (B / td)}
-    if args.token_topk:
-        # every key of the context is streamed once (256 B per token), then the listed tokens' K and V rows
-        ntok, sink, window = topk * PS, 4, 16
-        ws_tok = torch.empty(max(16, ops.token_topk_workspace_bytes(B, Hkv, st["max_pages_used"])), dtype=torch.uint8,
-                             device=device)
-        nt = max(3, min(20, K // 5))
-
-        def token_step():
-            ops.append_paged_kv(st["k"], st["v"], st["kv"], None, st["indices"], st["indptr"], st["last"])
-            ops.token_topk_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], ntok, st["max_pages_used"],
-                                  sink_tokens=sink, local_tokens=window, out=st["out"], workspace=ws_tok)
-
-        for _ in range(2):
-            token_step()
-        torch.cuda.synchronize()
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nt)]
-        t0 = time.perf_counter()
-        for e0, e1 in evs:
-            ops.append_paged_kv(st["k"], st["v"], st["kv"], None, st["indices"], st["indptr"], st["last"])
-            e0.record()
-            ops.token_topk_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], ntok, st["max_pages_used"],
-                                  sink_tokens=sink, local_tokens=window, out=st["out"], workspace=ws_tok)
-            e1.record()
-        torch.cuda.synchronize()
-        tt = (time.perf_counter() - t0) / nt
-        tks = [e0.elapsed_time(e1) for e0, e1 in evs]
-        tk = statistics.fmean(tks) * 1e-3
-        tok_bytes = sum(Hkv * (L * 256 + min(L, ntok + sink + window) * 512 + 512) + 2 * Hkv * G * 256 for L in st["lengths"])
-        result["token_topk"] = {"topk_tokens": ntok, "sink_tokens": sink, "local_tokens": window, "ms_per_step": tt * 1e3,
-                                "value": B / tt, "unit": "tokens/s", "steps": nt, "algorithmic_bytes_per_step": tok_bytes,
-                                "kernel_ms": tk * 1e3, "kernel_ms_min": min(tks), "kernel_ms_max": max(tks), "achieved_gbs": tok_bytes / tk / 1e9,
-                                "frac": tok_bytes / tk / 1e9 / HBM_PEAK_GBS}
-        if os.path.exists(tpath):
-            with open(tpath) as f:
-                result["token_topk"]["traffic"] = json.load(f).get(f"{args.workload}:B={B}", {}).get("token_topk_kernel")
-        # strided overlapping blocks with the same budget: topk blocks of 16 tokens, a block every 8 tokens
-        ws_str = torch.empty(max(16, ops.strided_topk_workspace_bytes(B, Hkv, st["max_pages_used"])), dtype=torch.uint8,
-                             device=device)
-        for _ in range(2):
-            ops.strided_topk_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], topk, st["max_pages_used"],
-                                    sink_tokens=sink, local_tokens=window, out=st["out"], workspace=ws_str)
-        torch.cuda.synchronize()
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nt)]
-        for e0, e1 in evs:
-            e0.record()
-            ops.strided_topk_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], topk, st["max_pages_used"],
-                                    sink_tokens=sink, local_tokens=window, out=st["out"], workspace=ws_str)
-            e1.record()
-        torch.cuda.synchronize()
-        ts = statistics.fmean(e0.elapsed_time(e1) for e0, e1 in evs) * 1e-3
-        result["strided_topk"] = {"topk_blocks": topk, "block_size": PS, "stride": 8, "sink_tokens": sink,
-                                  "local_tokens": window, "kernel_ms": ts * 1e3, "algorithmic_bytes_per_step": tok_bytes,
-                                  "achieved_gbs": tok_bytes / ts / 1e9, "frac": tok_bytes / ts / 1e9 / HBM_PEAK_GBS}
-        if os.path.exists(tpath):
-            with open(tpath) as f:
-                result["strided_topk"]["traffic"] = json.load(f).get(f"{args.workload}:B={B}", {}).get("strided_topk_kernel")
-        del ws_str
-        del ws_tok
+    side = headline and not args.no_side_workloads
+    if args.token_topk or side:
+        result.update(time_token_policies(torch, ops, st, B, Hkv, G, topk, max(3, min(20, K // 5)), traffic_table.get))
     del st
     torch.cuda.empty_cache()
+    if side:
+        # every other BASELINE configuration in the same run, each on its own freshly built cache
+        ks, ws = max(5, K), max(3, min(args.warmup, 10))
+        result["workloads"] = {name: side_workload(torch, ops, name, ks, ws, device)
+                               for name in ("qwen3-32b-share", "qwen3-0.6b-mix", "qwen3-8b-readme", "qwen3-8b-tp1", "tiny")}
     if args.whole_layer and args.workload in WHOLE_LAYER_MODEL:
         result["whole_layer"] = whole_layer(torch, args, B, ctx, topk, device)
     if not args.no_cpu_baseline and Hkv == 1 and args.workload not in RAGGED:
         result["cpu_baseline"] = cpu_baseline(torch, min(args.cpu_batch, B), ctx, G, topk)
+        if side:
+            tb, tctx, _, tg, tk, _ = WORKLOADS["tiny"]
+            result["cpu_baseline"]["tiny_in_full"] = cpu_baseline(torch, tb, tctx, tg, tk, budget_s=3.0)
     print(json.dumps(result))
 
 

@@ -23,11 +23,17 @@ import torch
 
 
 @torch.inference_mode()
-def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_table, last_page_len, topk, compute_dtype=torch.float32):
+def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_table, last_page_len, topk, compute_dtype=torch.float32,
+                          return_scores=False):
     """q [B,G,D], k/v [B,1,D] bf16; kv_cache [P,2,ps,1,D] bf16; kbar [B,N,D] bf16
     with N = n_pages-1 candidates; page_table [B,n_pages] int64; last_page_len
     [B] int64 (cache state AFTER the append).  Returns (out [B,G,D] bf16,
-    topk logical indices [B,k])."""
+    topk logical indices [B,k]) and, with ``return_scores``, csim [B,N].
+    ``compute_dtype=torch.bfloat16`` is the reference's own score arithmetic: its q
+    and compressed_key_cache are bf16 tensors, so the einsum returns bf16, .mean(1)
+    returns bf16 and torch.topk ranks those bf16 values
+    (benchmark/blocktopk_decoder.py:216-217); float32 is the more exact restatement
+    that the HIP path follows."""
     B, G, D = q.shape
     ps = kv_cache.shape[2]
     n_pages = page_table.shape[1]
@@ -51,6 +57,8 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_table, last_page_len, to
     logits = logits.masked_fill(~valid[:, None, :], float("-inf"))
     p = torch.softmax(logits, dim=-1)
     out = torch.einsum("bgt,btd->bgd", p, V).to(torch.bfloat16)
+    if return_scores:
+        return out, idx, csim
     return out, idx
 
 
