@@ -80,3 +80,55 @@ def dense_decode_step(q, k, v, kv_cache, page_table, last_page_len):
     logits = logits.masked_fill(~valid[:, None, :], float("-inf"))
     p = torch.softmax(logits, dim=-1)
     return torch.einsum("bgt,btd->bgd", p, V).to(torch.bfloat16)
+
+
+@torch.inference_mode()
+def reference_bf16_scores(q, kbar):
+    """csim exactly as the reference forms it: bf16 tensors in, so the einsum's
+    [B,G,N] result is bf16 and .mean(1) is bf16 (benchmark/blocktopk_decoder.py:216).
+    q [B,G,D] bf16, kbar [B,N,D] bf16 -> [B,N] bf16."""
+    assert q.dtype == torch.bfloat16 and kbar.dtype == torch.bfloat16
+    return torch.einsum("bgd,bnd->bgn", q, kbar).mean(dim=1)
+
+
+def _bf16_ulp(x):
+    """Spacing of bfloat16 numbers (8 significant bits) around |x| (float64 tensor)."""
+    ax = x.abs().clamp_min(2.0 ** -126)
+    return torch.pow(2.0, torch.floor(torch.log2(ax)) - 7)
+
+
+@torch.inference_mode()
+def bf16_score_band(q, kbar):
+    """How far the reference's bf16 score of a page can lie from the exact one:
+    half a bf16 unit for each of the G per-head products the einsum rounds,
+    averaged, plus one unit of the mean itself (sum and division each round).
+    Returns (exact [B,N] float64, band [B,N] float64)."""
+    d = torch.einsum("bgd,bnd->bgn", q.double(), kbar.double())  # exact products of bf16 inputs (float64 holds them)
+    exact = d.mean(dim=1)
+    band = 0.5 * _bf16_ulp(d).mean(dim=1) + _bf16_ulp(exact)
+    return exact, band
+
+
+@torch.inference_mode()
+def compare_with_bf16_reference(q, kbar, got_idx, k):
+    """The page indices ``got_idx`` [B,k] (any order) of a selector that ranks by
+    exact / fp32 scores, against torch.topk on the reference's bf16 scores.
+    For every pair (p picked here but not by the reference, r picked by the
+    reference but not here) the reference's own scores must be tied within its
+    rounding: ref(r) - ref(p) <= band(r) + band(p).  Returns a dict with the
+    overlap fraction, the number of differing picks and the worst violation
+    (<= 0 means every disagreement is a tie at the reference's precision)."""
+    ref = reference_bf16_scores(q, kbar).double()
+    exact, band = bf16_score_band(q, kbar)
+    assert bool(((ref - exact).abs() <= band).all()), "the reference's bf16 score left its rounding band"
+    ref_idx = torch.topk(ref, k, dim=-1).indices
+    B = q.shape[0]
+    differing, worst = 0, -float("inf")
+    for b in range(B):
+        got, want = set(got_idx[b].tolist()), set(ref_idx[b].tolist())
+        only_got, only_ref = sorted(got - want), sorted(want - got)
+        differing += len(only_got)
+        for p in only_got:
+            for r in only_ref:
+                worst = max(worst, float(ref[b, r] - ref[b, p] - band[b, r] - band[b, p]))
+    return dict(overlap=1.0 - differing / float(B * k), differing=differing, picks=B * k, worst_violation=worst, ref_idx=ref_idx)

@@ -143,3 +143,25 @@ def int_tensor(a: np.ndarray, device="cpu"):
     import torch
 
     return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int32)).to(device)
+
+
+# Shapes on which the selection is compared with the reference's bf16-scored top-k.
+BF16_CASES = [
+    # seed, batch, context, topk, group, sigma of the per-page key offset (0: page scores barely separated)
+    (0, 8, 4096, 64, 4, 0.5),      # the tiny benchmark configuration
+    (1, 6, 32768, 128, 4, 0.5),    # headline shape, a slice of the batch
+    (2, 6, 32768, 256, 8, 0.5),    # Qwen3-32B share
+    (3, 12, 8192, 64, 3, 0.1),
+    (4, 6, 16384, 64, 4, 0.0),
+]
+
+
+def bf16_case(seed, B, L, topk, G, sigma):
+    """A uniform problem after its append, as torch tensors for oracle/torch_path.py."""
+    pb = make_problem(seed, [L + 1] * B, num_kv_heads=1, group=G, topk=topk, page_mean_sigma=sigma)
+    n = L // PAGE_SIZE
+    import torch
+
+    table = torch.from_numpy(pb.page_indices.astype(np.int64)).reshape(B, n + 1)
+    last = torch.from_numpy(pb.last_page_len.astype(np.int64))
+    return pb, n, table, last

@@ -442,6 +442,44 @@ def test_check_page_table_flags_bad_metadata(ops):
         ops.check_page_table(g.indices, bad_ptr, g.last, PS, pb.num_pages)
 
 
+@pytest.mark.parametrize("case", P.BF16_CASES, ids=lambda c: f"seed{c[0]}")
+def test_selection_vs_the_references_bf16_scoring(ops, case):
+    """The reference ranks pages by bf16 scores (benchmark/blocktopk_decoder.py:216-217),
+    the HIP path by fp32 scores.  Every page the HIP path picks differently must be a
+    tie at the reference's precision (its bf16 scores of the swapped pages lie within
+    the reference's rounding band of each other); sequences with the same page set
+    must give the same output within the contract."""
+    from oracle import torch_path
+
+    seed, B, L, topk, G, sigma = case
+    pb, n, table, last = P.bf16_case(*case)
+    g = Gpu(pb)
+    out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, topk, sel_pages=g.sel, sel_count=g.cnt)
+    sel2, cnt2 = torch.empty_like(g.sel), torch.empty_like(g.cnt)
+    ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, topk, sel2, cnt2, g.logical)
+    torch.cuda.synchronize()
+    assert torch.equal(sel2, g.sel) and torch.equal(cnt2, g.cnt)
+    got = g.logical[:, 0].cpu().long()
+    kv_t = P.to_torch(pb.kv_cache.copy())
+    kbar_after = g.kbar[:, 0, :n].cpu()
+    out_ref, idx_ref = torch_path.blocktopk_decode_step(P.to_torch(pb.q), P.to_torch(pb.k), P.to_torch(pb.v), kv_t, kbar_after, table,
+                                                        last, topk, compute_dtype=torch.bfloat16)
+    cmp = torch_path.compare_with_bf16_reference(P.to_torch(pb.q), kbar_after, got, topk)
+    same = (cmp["ref_idx"].sort(dim=1).values == got.sort(dim=1).values).all(dim=1).numpy()
+    diff = (out.float().cpu() - out_ref.float()).abs().numpy()
+    print(f"bf16-scored reference vs HIP, seed {seed} B={B} ctx={L} k={topk} G={G}: overlap {cmp['overlap']:.4f} "
+          f"({cmp['differing']} of {cmp['picks']} picks differ), worst violation {cmp['worst_violation']:.4g}, "
+          f"sequences with the same page set {int(same.sum())}/{B}, max |out diff| same set "
+          f"{diff[same].max() if same.any() else 0:.4g}, swapped {diff[~same].max() if (~same).any() else 0:.4g}")
+    assert cmp["worst_violation"] <= 1e-6, cmp
+    assert cmp["overlap"] >= 0.98, cmp
+    ref_abs = out_ref.float().abs().numpy()
+    tol = OUT_ATOL + OUT_RTOL * ref_abs
+    assert np.all(diff[same] <= tol[same])
+    if (~same).any():
+        assert diff[~same].max() <= 0.1
+
+
 # --------------------------------------------------------------------------- full benchmark sizes
 
 
@@ -522,6 +560,17 @@ def _check_full_size(ops, st, spot_rows):
     want, _ = O.sparse_paged_decode(q_np, kv_np, sel_sub, np.full((len(spot_rows), hkv), topk + 1, dtype=np.int32),
                                     np.ones(len(spot_rows), dtype=np.int32))
     assert_out_close(out[rows], want, "full-size spot check")
+    # the path that ships (bench.py and the layer objects default to it): one launch.  Same lists,
+    # same appended bytes, output against the oracle on the same rows.
+    kv_rows_before = st["kv"][pages].clone()
+    sel_f, cnt_f = torch.full_like(st["sel"], -5), torch.full_like(st["cnt"], -5)
+    out_f = ops.blocktopk_decode_step(st["q"], st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"],
+                                      topk, sel_pages=sel_f, sel_count=cnt_f)
+    torch.cuda.synchronize()
+    assert torch.equal(sel_f, st["sel"]) and torch.equal(cnt_f, st["cnt"]), "fused step: page lists differ"
+    assert torch.equal(st["kv"][pages], kv_rows_before), "fused step: cache rows differ"
+    assert_out_close(out_f[rows], want, "full-size spot check, fused step")
+    assert (out_f.float() - out.float()).abs().max().item() <= 1e-2
     return out
 
 
@@ -541,6 +590,14 @@ def test_full_size_qwen3_8b_share(ops):
     assert torch.equal(od, os_)
     # sparse output differs from dense (it really attends to a subset) but not wildly: same value range
     assert not torch.equal(od, out)
+    # three 2049-page rows of the dense output against the oracle
+    spot = [0, 1234, 4095]
+    rows = torch.tensor(spot, device=DEV)
+    n_pages = st["n_pages"]
+    kv_np = P.from_torch(st["kv"][st["table"][rows].reshape(-1).long()])
+    want_d, _ = O.dense_paged_decode(P.from_torch(st["q"][rows]), kv_np, np.arange(len(spot) * n_pages, dtype=np.int32),
+                                     (np.arange(len(spot) + 1) * n_pages).astype(np.int32), np.ones(len(spot), dtype=np.int32))
+    assert_out_close(od[rows], want_d, "full-size dense rows")
     del st
     torch.cuda.empty_cache()
 
@@ -630,6 +687,13 @@ def test_full_size_continuous_batching_mix(ops):
             sel_sub[j, h, c] = sub_ptr[j + 1] - 1
     want, _ = O.sparse_paged_decode(q_np, kv_np, sel_sub, got_cnt, last[rows])
     assert_out_close(out[rows], want, "mix spot check")
+    # the same step as one launch (the default path): same lists, output against the oracle on the same rows
+    sel_f, cnt_f = torch.full_like(sel, -5), torch.full_like(cnt, -5)
+    out_f = ops.blocktopk_decode_step(q, k, v, kv, kbar, indices, ptr, last_t, topk, sel_pages=sel_f, sel_count=cnt_f)
+    torch.cuda.synchronize()
+    assert torch.equal(sel_f, sel) and torch.equal(cnt_f, cnt), "fused step: page lists differ"
+    assert_out_close(out_f[rows], want, "mix spot check, fused step")
+    assert (out_f.float() - out.float()).abs().max().item() <= 1e-2
     # k >= candidates for the 1025-token sequence: sparse equals dense there
     od = ops.dense_paged_decode(q, kv, indices, ptr, last_t, max_pages)
     assert (od[0].float() - out[0].float()).abs().max().item() <= 1e-2
@@ -1265,21 +1329,15 @@ def test_fused_step_equals_three_calls(ops, case):
 
 
 def test_fused_step_full_size(ops):
-    """The headline workload through the single-launch path equals the
-    three-call path bit for bit."""
+    """The unsharded Qwen3-8B attention (B=512, 8 KV heads x 4 Q heads, context
+    32768, 128-page budget, about 69 GB of KV) through both paths: three launches
+    and the single-launch step, lists equal, four sequences (all heads) against
+    the oracle."""
     free, _ = torch.cuda.mem_get_info()
     if free < 90e9:
         pytest.skip("needs about 80 GB of free device memory")
-    st = _uniform_state(4096, 32768, 1, 4, 128, seed=2)
-    ops.build_kbar(st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
-    ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
-    ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], st["last"], 128, st["sel"], st["cnt"])
-    out_a = ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"], num_splits=1)
-    sel_b, cnt_b = torch.empty_like(st["sel"]), torch.empty_like(st["cnt"])
-    out_b = ops.blocktopk_decode_step(st["q"], st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"],
-                                      st["last"], 128, sel_pages=sel_b, sel_count=cnt_b)
-    torch.cuda.synchronize()
-    assert torch.equal(st["sel"], sel_b) and torch.equal(st["cnt"], cnt_b) and torch.equal(out_a, out_b)
+    st = _uniform_state(512, 32768, 8, 4, 128, seed=5)
+    _check_full_size(ops, st, [0, 77, 300, 511])
     del st
     torch.cuda.empty_cache()
 
