@@ -442,6 +442,60 @@ int kin_build_slot_page_table(const int32_t* slot_ids, const int32_t* seq_lens, 
                               int32_t* last_page_len, kin_stream_t stream);
 
 /*
+ * Page pool for a slot-based cache -- the paged replacement of LiteSys'
+ * per-slot contiguous caches that also gives memory back: LiteSys sizes
+ * [max_batch, H_kv, max_len, D] per layer up front and clear_cache zeroes a
+ * slot (ref: LiteSys/litesys/attention/batch_cache.py:40-62,147-152); here the
+ * slots draw 16-token pages from one pool of num_pool_pages pages through a
+ * free list that lives on the device, so the pool can be smaller than
+ * max_slots * pages_per_slot and a finished request returns its pages.  No host
+ * synchronisation anywhere; every call is a single small kernel.
+ *
+ * Caller-owned device arrays (int32):
+ *   free_stack  [num_pool_pages]  the free page ids; the top is the next to go
+ *   pool_state  [2]               [0] = pages on the stack, [1] = status bits:
+ *                                 1 = a reserve call wanted more pages than were
+ *                                     free (that call reserved nothing),
+ *                                 2 = a sequence wanted more than pages_per_slot
+ *                                     pages (it was cut there)
+ *   slot_table  [max_slots, pages_per_slot]  physical page of each logical page
+ *   slot_npages [max_slots]       pages the slot owns
+ * kin_page_pool_init fills the stack (pages are handed out 0, 1, 2, ...), and
+ * clears the state and the slot counts.
+ * kin_page_pool_reserve grows the slot of every sequence b (slot_ids[b], NULL =
+ * identity; distinct) to ceil(seq_lens[b] / page_size) pages, at most
+ * pages_per_slot; it never shrinks a slot, so sequences with seq_lens[b] <= 0
+ * are left alone and calling it again with the same lengths changes nothing.
+ * All or nothing: if the stack cannot cover the whole call it reserves nothing
+ * and raises status bit 1.  batch <= 65535.
+ * kin_page_pool_release pushes every page of the `count` listed slots back and
+ * empties them (clear_cache).
+ * kin_build_pool_page_table is kin_build_slot_page_table with page ids taken
+ * from slot_table; a sequence is cut to the pages its slot owns (so after a
+ * failed reserve no unowned entry is ever listed).
+ * The status word is for the host to poll when it is convenient
+ * (hipMemcpy of pool_state); kernels cannot raise.
+ */
+int kin_page_pool_init(int32_t* free_stack, int32_t* pool_state, int32_t* slot_npages,
+                       int num_pool_pages, int max_slots, kin_stream_t stream);
+
+int kin_page_pool_reserve(const int32_t* slot_ids, const int32_t* seq_lens, int batch,
+                          int pages_per_slot, int page_size,
+                          int32_t* slot_table, int32_t* slot_npages,
+                          const int32_t* free_stack, int32_t* pool_state, kin_stream_t stream);
+
+int kin_page_pool_release(const int32_t* slot_ids, int count, int pages_per_slot,
+                          const int32_t* slot_table, int32_t* slot_npages,
+                          int32_t* free_stack, int32_t* pool_state, int num_pool_pages,
+                          kin_stream_t stream);
+
+int kin_build_pool_page_table(const int32_t* slot_ids, const int32_t* seq_lens, int batch,
+                              int pages_per_slot, int page_size,
+                              const int32_t* slot_table, const int32_t* slot_npages,
+                              int32_t* page_indices, int32_t* page_indptr,
+                              int32_t* last_page_len, kin_stream_t stream);
+
+/*
  * Debugging aid, SYNCHRONOUS (waits for the stream): verifies on the device
  * that page_indptr is non-decreasing from 0 and never exceeds nnz (the length
  * of page_indices), every page id lies in [0, num_pages), and every

@@ -80,6 +80,10 @@ SIGNATURES = {
          c_int, c_int, c_int64, c_int, c_int, c_float, _P],
     ),
     "kin_build_slot_page_table": (c_int, [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P]),
+    "kin_page_pool_init": (c_int, [_P, _P, _P, c_int, c_int, _P]),
+    "kin_page_pool_reserve": (c_int, [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P, _P]),
+    "kin_page_pool_release": (c_int, [_P, c_int, c_int, _P, _P, _P, _P, c_int, _P]),
+    "kin_build_pool_page_table": (c_int, [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P]),
     "kin_check_page_table": (c_int, [_P, _P, _P, c_int, c_int, c_int64, c_int64, _P, _P]),
     "kin_rms_norm": (c_int, [_P, _P, _P, _P, c_int64, c_int, c_int64, c_int64, c_float, _P]),
     "kin_qkv_norm_split": (c_int, [_P, c_int64, _P, _P, c_float, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),

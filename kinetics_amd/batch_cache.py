@@ -4,8 +4,11 @@
 LiteSys keeps contiguous per-slot caches ``[max_batch, H_kv, max_len, D]`` and,
 for block-sparse decoding, computes full-context logits, masks all but the
 top-k blocks and runs softmax and P.V over the whole context
-(batch_cache.py:154-168, sparsity_utils.py:24-47).  Here every slot owns a fixed
-run of 16-token pages of one paged cache per layer; decode appends the token,
+(batch_cache.py:154-168, sparsity_utils.py:24-47).  Here every slot draws
+16-token pages of one paged cache per layer from a pool through a free list on
+the device (``kv_pool_pages`` pages, by default enough for every slot at
+``max_seq_len``; fewer saves memory and serves as many tokens as fit);
+``clear_cache`` returns a slot's pages to the pool.  Decode appends the token,
 scores the per-page mean keys, selects the top-k pages per KV head and attends
 only to those pages plus the pinned ones -- the same result as the mask
 formulation, without touching the rest of the context.
@@ -47,7 +50,7 @@ import math
 import torch
 import torch.nn.functional as F
 
-from . import ops
+from . import _lib, ops
 
 PAGE = 16
 
@@ -120,11 +123,18 @@ class PagedBatchKVManager:
         B, Hq, Hkv, D = max_batch_size, self.num_attention_heads, self.num_key_value_heads, self.head_dim
         self.pages_per_slot = P = (max_seq_len + self.pad + PAGE - 1) // PAGE
         dev = self.device
-        self.kv_cache = [torch.zeros(B * P, 2, PAGE, Hkv, D, dtype=dtype, device=dev) for _ in range(self.num_layers)]
+        # The page pool, shared by all layers (a token position occupies the same page id in every
+        # layer's cache): slots take pages as they grow and give them back in clear_cache.
+        self.num_pool_pages = int(kwargs.get("kv_pool_pages") or B * P)
+        if not 1 <= self.num_pool_pages <= B * P:
+            raise ValueError(f"kv_pool_pages must be in [1, max_batch_size * pages_per_slot = {B * P}]")
+        self.pool = ops.PagePool(self.num_pool_pages, B, P, PAGE, dev)
+        self.kv_cache = [torch.zeros(self.num_pool_pages, 2, PAGE, Hkv, D, dtype=dtype, device=dev)
+                         for _ in range(self.num_layers)]
         self.kbar = [torch.zeros(B, Hkv, P, D, dtype=dtype, device=dev) for _ in range(self.num_layers)]
         self.kv_offset = [torch.zeros(B, dtype=torch.int32, device=dev) for _ in range(self.num_layers)]
         # page-table metadata (rebuilt on the device each decode call) and full-batch staging buffers
-        self.page_indices = torch.zeros(B * P, dtype=torch.int32, device=dev)
+        self.page_indices = torch.zeros(self.num_pool_pages, dtype=torch.int32, device=dev)
         self.page_indptr = torch.zeros(B + 1, dtype=torch.int32, device=dev)
         self.last_page_len = torch.ones(B, dtype=torch.int32, device=dev)
         self._lens = torch.zeros(B, dtype=torch.int32, device=dev)
@@ -156,9 +166,13 @@ class PagedBatchKVManager:
         return out.reshape(bsz, seq_len, self.hidden_size)
 
     def clear_cache(self, batch_idx: int):
-        """batch_cache.py:147-152.  Pages need no zeroing: an empty page list hides them."""
+        """batch_cache.py:147-152.  The slot's pages go back to the pool; they need no
+        zeroing (an empty page list hides them).  Also the place where trouble that the
+        kernels could only flag is raised: an exhausted pool, a sequence beyond max_seq_len."""
         for i in range(self.num_layers):
             self.kv_offset[i][batch_idx] = 0
+        self.pool.release(torch.tensor([int(batch_idx)], dtype=torch.int32, device=self.device))
+        self.pool.raise_on_overflow()
 
     # ------------------------------------------------------------------ decode
     def decode(self, query, key, value, batch_idx, layer_idx):
@@ -169,7 +183,9 @@ class PagedBatchKVManager:
         # Sequence b of the kernels == slot b; inactive slots get an empty page list.
         self._lens.zero_()
         self._lens[slots] = off[slots] + self.pad
-        ops.build_slot_page_table(self._lens, self.pages_per_slot, PAGE, self.page_indices, self.page_indptr, self.last_page_len)
+        # a slot that crossed a page boundary takes a page from the pool (the first layer to get there does it)
+        self.pool.reserve(self._lens)
+        self.pool.build_page_table(self._lens, self.page_indices, self.page_indptr, self.last_page_len)
         self._q[slots] = query[:, :, 0, :]
         self._k[slots] = key[:, :, 0, :]
         self._v[slots] = value[:, :, 0, :]
@@ -216,19 +232,24 @@ class PagedBatchKVManager:
         pad = self.pad                                   # token t lives in cache slot t + pad
         if total + pad > self.pages_per_slot * PAGE:
             raise ValueError(f"sequence of {total} tokens exceeds max_seq_len")
-        P, Hkv, D = self.pages_per_slot, self.num_key_value_heads, self.head_dim
-        view = self.kv_cache[layer_idx].view(self.max_batch_size, P, 2, PAGE, Hkv, D)
+        Hkv, D = self.num_key_value_heads, self.head_dim
         self.kv_offset[layer_idx][slot] += seq_len
         n_pages = (total + pad + PAGE - 1) // PAGE
-        idx = (slot * P + torch.arange(n_pages, device=self.device, dtype=torch.int32)).contiguous()
+        self.pool.reserve(torch.tensor([total + pad], dtype=torch.int32, device=self.device),
+                          torch.tensor([slot], dtype=torch.int32, device=self.device))
+        free, bits = self.pool.status()
+        if bits & ops.PagePool.EXHAUSTED:
+            raise _lib.KineticsError(f"page pool exhausted ({free} pages free): cannot hold {total} tokens in slot {slot}")
+        idx = self.pool.slot_table[slot, :n_pages].contiguous()
         ptr = torch.tensor([0, n_pages], dtype=torch.int32, device=self.device)
         last = torch.tensor([total + pad - (n_pages - 1) * PAGE], dtype=torch.int32, device=self.device)
         # rows to their page slots, mean keys of the pages that are now full
         ops.append_paged_kv_ragged(key_states[0].transpose(0, 1).contiguous(), value_states[0].transpose(0, 1).contiguous(),
                                    torch.tensor([0, seq_len], dtype=torch.int32, device=self.device),
                                    self.kv_cache[layer_idx], self.kbar[layer_idx][slot:slot + 1], idx, ptr, last)
-        k_all = view[slot, :n_pages, 0].reshape(n_pages * PAGE, Hkv, D)[pad:total + pad].transpose(0, 1)  # [Hkv, total, D]
-        v_all = view[slot, :n_pages, 1].reshape(n_pages * PAGE, Hkv, D)[pad:total + pad].transpose(0, 1)
+        pages = self.kv_cache[layer_idx][idx.long()]                                           # [n_pages, 2, PAGE, Hkv, D]
+        k_all = pages[:, 0].reshape(n_pages * PAGE, Hkv, D)[pad:total + pad].transpose(0, 1)   # [Hkv, total, D]
+        v_all = pages[:, 1].reshape(n_pages * PAGE, Hkv, D)[pad:total + pad].transpose(0, 1)
         G = self.num_attention_heads // Hkv
         q = query_states[0]                                                                    # [Hq, s, D]
         pos_q = torch.arange(offset, total, device=self.device)[:, None]

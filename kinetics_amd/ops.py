@@ -538,6 +538,86 @@ def build_slot_page_table(seq_lens, pages_per_slot, page_size, page_indices, pag
         )
 
 
+class PagePool:
+    """Device-resident free list from which the slots of a slot-based cache draw
+    their pages (kin_page_pool_*): the paged answer to LiteSys' fixed
+    [max_batch, H_kv, max_len, D] caches and zeroing clear_cache
+    (LiteSys/litesys/attention/batch_cache.py:40-62,147-152).  The pool may hold
+    fewer pages than ``max_slots * pages_per_slot``; a finished slot returns its
+    pages.  No method synchronises except ``status()`` / ``raise_on_overflow()``."""
+
+    EXHAUSTED, SLOT_TOO_LONG = 1, 2
+
+    def __init__(self, num_pool_pages: int, max_slots: int, pages_per_slot: int, page_size: int, device):
+        self.num_pool_pages, self.max_slots = int(num_pool_pages), int(max_slots)
+        self.pages_per_slot, self.page_size = int(pages_per_slot), int(page_size)
+        self.free_stack = torch.empty(self.num_pool_pages, dtype=torch.int32, device=torch.device(device))
+        self.device = dev = self.free_stack.device   # with its index, as tensors report it
+        self.pool_state = torch.empty(2, dtype=torch.int32, device=dev)
+        self.slot_table = torch.full((self.max_slots, self.pages_per_slot), -1, dtype=torch.int32, device=dev)
+        self.slot_npages = torch.empty(self.max_slots, dtype=torch.int32, device=dev)
+        with _on(dev):
+            _lib.check(_lib.load().kin_page_pool_init(_ptr(self.free_stack), _ptr(self.pool_state), _ptr(self.slot_npages),
+                                                      self.num_pool_pages, self.max_slots, _stream(dev)))
+
+    def _lens(self, seq_lens, slot_ids):
+        _require(seq_lens, "seq_lens", torch.int32, 1, self.device)
+        if slot_ids is not None:
+            _require(slot_ids, "slot_ids", torch.int32, 1, self.device)
+            if slot_ids.numel() != seq_lens.numel():
+                raise ValueError("slot_ids must have one entry per sequence")
+        elif seq_lens.numel() > self.max_slots:
+            raise ValueError(f"{seq_lens.numel()} sequences but only {self.max_slots} slots")
+        return seq_lens.numel()
+
+    def reserve(self, seq_lens, slot_ids=None) -> None:
+        """Grow the slots to cover ``seq_lens`` tokens each (never shrinks; all or nothing)."""
+        batch = self._lens(seq_lens, slot_ids)
+        with _on(self.device):
+            _lib.check(_lib.load().kin_page_pool_reserve(
+                _ptr(slot_ids), _ptr(seq_lens), batch, self.pages_per_slot, self.page_size, _ptr(self.slot_table),
+                _ptr(self.slot_npages), _ptr(self.free_stack), _ptr(self.pool_state), _stream(self.device)))
+
+    def release(self, slot_ids) -> None:
+        """Return every page of the listed slots (int32 tensor of distinct slot ids) to the pool."""
+        _require(slot_ids, "slot_ids", torch.int32, 1, self.device)
+        with _on(self.device):
+            _lib.check(_lib.load().kin_page_pool_release(
+                _ptr(slot_ids), slot_ids.numel(), self.pages_per_slot, _ptr(self.slot_table), _ptr(self.slot_npages),
+                _ptr(self.free_stack), _ptr(self.pool_state), self.num_pool_pages, _stream(self.device)))
+
+    def build_page_table(self, seq_lens, page_indices, page_indptr, last_page_len, slot_ids=None) -> None:
+        """CSR page table of the sequences from the slots' page lists (kin_build_pool_page_table)."""
+        batch = self._lens(seq_lens, slot_ids)
+        dev = self.device
+        _require(page_indices, "page_indices", torch.int32, 1, dev)
+        _require(page_indptr, "page_indptr", torch.int32, 1, dev)
+        _require(last_page_len, "last_page_len", torch.int32, 1, dev)
+        if page_indptr.numel() != batch + 1 or last_page_len.numel() != batch:
+            raise ValueError("page_indptr needs batch+1 entries and last_page_len batch entries")
+        if page_indices.numel() < min(batch * self.pages_per_slot, self.num_pool_pages):
+            raise ValueError("page_indices needs room for min(batch*pages_per_slot, num_pool_pages) entries")
+        with _on(dev):
+            _lib.check(_lib.load().kin_build_pool_page_table(
+                _ptr(slot_ids), _ptr(seq_lens), batch, self.pages_per_slot, self.page_size, _ptr(self.slot_table),
+                _ptr(self.slot_npages), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), _stream(dev)))
+
+    def status(self):
+        """(free pages, status bits) -- copies two ints to the host (synchronises)."""
+        free, bits = self.pool_state.tolist()
+        return free, bits
+
+    def raise_on_overflow(self) -> None:
+        """Raise if any earlier reserve ran out of pages or met a sequence longer than a slot
+        can hold (synchronises; the kernels themselves cannot raise)."""
+        free, bits = self.status()
+        if bits & self.EXHAUSTED:
+            raise _lib.KineticsError(f"page pool exhausted: a reserve wanted more than the {free} free pages "
+                                     f"(pool of {self.num_pool_pages})")
+        if bits & self.SLOT_TOO_LONG:
+            raise ValueError(f"a sequence exceeds {self.pages_per_slot} pages of {self.page_size} tokens (max_seq_len)")
+
+
 def check_page_table(page_indices, page_indptr, last_page_len, page_size, num_pages) -> None:
     """Synchronous device-side validation of a page table (debugging aid);
     raises KineticsError on an invalid entry."""

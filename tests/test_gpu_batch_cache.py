@@ -20,11 +20,14 @@ def bf(x):
     return x.to(torch.bfloat16)
 
 
+def cfg_small():
+    return SimpleNamespace(num_attention_heads=4, num_key_value_heads=2, head_dim=D, hidden_size=512, num_hidden_layers=2)
+
+
 def make_manager(**sparse):
     from kinetics_amd.batch_cache import PagedBatchKVManager
 
-    cfg = SimpleNamespace(num_attention_heads=4, num_key_value_heads=2, head_dim=D, hidden_size=512, num_hidden_layers=2)
-    return PagedBatchKVManager(cfg, max_batch_size=6, max_seq_len=PS * 24, device=DEV, dtype=torch.bfloat16, **sparse)
+    return PagedBatchKVManager(cfg_small(), max_batch_size=6, max_seq_len=PS * 24, device=DEV, dtype=torch.bfloat16, **sparse)
 
 
 def test_rejects_what_it_does_not_implement():
@@ -116,13 +119,16 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
             assert out.shape == (bsz, 1, Hq * D)
             for i, slot in enumerate(batch_slots):
                 feed(layer, slot, k[i], v[i])
-            # the paged cache holds exactly the history that was fed
-            view = m.kv_cache[layer].view(6, m.pages_per_slot, 2, PS, Hkv, D)
+            # the paged cache holds exactly the history that was fed (pages through the slot's page list)
+            table = m.pool.slot_table.cpu().numpy()
+            owned = m.pool.slot_npages.cpu().numpy()
             for slot in batch_slots:
                 K, V = hist[(layer, slot)]
                 t = K.shape[0]
                 assert m.kv_offset[layer][slot].item() == t == off_before[slot] + 1
-                got_k = view[slot, :, 0].reshape(-1, Hkv, D)[pad:pad + t].float().cpu()
+                assert owned[slot] == (t + pad + PS - 1) // PS
+                pages = torch.from_numpy(table[slot, : owned[slot]]).long().to(DEV)
+                got_k = m.kv_cache[layer][pages, 0].reshape(-1, Hkv, D)[pad:pad + t].float().cpu()
                 assert torch.equal(got_k, K)
             # oracle on the manager's own state before the call
             lens = np.zeros(6, dtype=np.int64)
@@ -130,7 +136,7 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
             n_pages = (lens + PS - 1) // PS
             indptr = np.zeros(7, dtype=np.int32)
             indptr[1:] = np.cumsum(n_pages)
-            idx = np.concatenate([s * m.pages_per_slot + np.arange(n_pages[s]) for s in range(6)]).astype(np.int32)
+            idx = np.concatenate([table[s, : n_pages[s]] for s in range(6)]).astype(np.int32)
             last = np.where(lens > 0, lens - (n_pages - 1) * PS, 1).astype(np.int32)
             assert np.array_equal(m.page_indptr.cpu().numpy(), indptr)
             assert np.array_equal(m.page_indices.cpu().numpy()[: len(idx)], idx)
@@ -175,8 +181,11 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
     for _ in range(12):           # crosses page boundaries (mean keys refreshed) for every slot
         decode_round([0, 2, 5])
     decode_round([5, 0])          # a subset, in another order
-    m.clear_cache(2)              # recycle slot 2
+    free_before, _ = m.pool.status()
+    held = int(m.pool.slot_npages[2].item())
+    m.clear_cache(2)              # recycle slot 2: its pages go back to the pool
     assert m.kv_offset[1][2].item() == 0
+    assert m.pool.status() == (free_before + held, 0) and int(m.pool.slot_npages[2].item()) == 0
     for layer in range(L):
         hist.pop((layer, 2))
         q, k, v = bf(torch.randn(1, Hq, 20, D, device=DEV)), bf(torch.randn(1, Hkv, 20, D, device=DEV)), bf(torch.randn(1, Hkv, 20, D, device=DEV))
@@ -214,3 +223,103 @@ def test_slot_page_table_against_numpy(batch, with_slots):
     for b in range(batch):
         s = b if slots is None else int(slots[b])
         assert np.array_equal(got[want_ptr[b]: want_ptr[b + 1]], s * pps + np.arange(n[b]))
+
+
+def test_page_pool_against_a_python_free_list():
+    """kin_page_pool_init / reserve / release / kin_build_pool_page_table against a
+    Python model of the same free list on a random sequence of grow, release and
+    over-subscription steps: page lists, counts, free stack and status word."""
+    from kinetics_amd import ops
+
+    rng = np.random.default_rng(77)
+    slots, pps, pool_pages = 37, 9, 120
+    pool = ops.PagePool(pool_pages, slots, pps, PS, DEV)
+    stack = list(range(pool_pages - 1, -1, -1))
+    table = [[] for _ in range(slots)]
+    status = 0
+    idx = torch.empty(pool_pages, dtype=torch.int32, device=DEV)
+    ptr = torch.empty(slots + 1, dtype=torch.int32, device=DEV)
+    last = torch.empty(slots, dtype=torch.int32, device=DEV)
+    for step in range(60):
+        if step % 5 == 4:
+            rel = rng.permutation(slots)[: int(rng.integers(1, 6))].astype(np.int32)
+            pool.release(torch.from_numpy(rel).to(DEV))
+            for s in rel:
+                stack.extend(table[s])
+                table[s] = []
+        lens = np.where(rng.random(slots) < 0.4, rng.integers(0, PS * pps + 30, size=slots), 0).astype(np.int32)
+        if step == 20:
+            lens[:] = PS * pps       # more than the pool holds: nothing may be reserved
+        pool.reserve(torch.from_numpy(lens).to(DEV))
+        need = np.minimum((lens + PS - 1) // PS, pps)
+        extra = [max(0, int(need[s]) - len(table[s])) for s in range(slots)]
+        if (lens > PS * pps).any():
+            status |= 2
+        if sum(extra) > len(stack):
+            status |= 1
+        else:
+            top, first = len(stack), 0
+            for s in range(slots):
+                table[s] += [stack[top - 1 - (first + j)] for j in range(extra[s])]
+                first += extra[s]
+            del stack[top - first:]
+        free, bits = pool.status()
+        assert (free, bits) == (len(stack), status), f"step {step}"
+        assert pool.slot_npages.cpu().tolist() == [len(t) for t in table], f"step {step}"
+        got_table = pool.slot_table.cpu().numpy()
+        for s in range(slots):
+            assert got_table[s, : len(table[s])].tolist() == table[s], f"step {step} slot {s}"
+        assert sorted(pool.free_stack.cpu().numpy()[:free].tolist() + [p for t in table for p in t]) == list(range(pool_pages))
+        # the CSR table of these lengths: cut to what each slot owns
+        pool.build_page_table(torch.from_numpy(lens).to(DEV), idx, ptr, last)
+        n = np.array([min(int(need[s]), len(table[s])) for s in range(slots)])
+        want_ptr = np.concatenate([[0], np.cumsum(n)])
+        assert ptr.cpu().tolist() == want_ptr.tolist()
+        got = idx.cpu().numpy()
+        for s in range(slots):
+            assert got[want_ptr[s]: want_ptr[s + 1]].tolist() == table[s][: n[s]]
+    assert status == 3     # both conditions were met on the way
+    with pytest.raises(Exception):
+        pool.raise_on_overflow()
+
+
+def test_manager_with_a_small_pool_and_overlong_sequences():
+    """A pool smaller than max_batch x max_len serves what fits, reuses returned pages
+    (the recycled slot's table is fragmented) and reports exhaustion and sequences
+    past max_seq_len instead of silently overwriting the last slot."""
+    from kinetics_amd._lib import KineticsError
+
+    torch.manual_seed(9)
+    L, Hq, Hkv = 2, 4, 2
+    from kinetics_amd.batch_cache import PagedBatchKVManager
+
+    m = PagedBatchKVManager(cfg_small(), max_batch_size=4, max_seq_len=PS * 6, device=DEV, dtype=torch.bfloat16,
+                            kv_pool_pages=10)
+    assert m.kv_cache[0].shape[0] == 10
+
+    def prefill(slot, n):
+        for layer in range(L):
+            q, k, v = (bf(torch.randn(1, h, n, D, device=DEV)) for h in (Hq, Hkv, Hkv))
+            m.compute_attention(q, k, v, layer, torch.tensor([slot]))
+
+    prefill(0, PS * 4)            # 4 pages
+    prefill(1, PS * 3 + 1)        # 4 pages
+    assert m.pool.status() == (2, 0)
+    with pytest.raises(KineticsError):
+        prefill(2, PS * 3)        # wants 3, 2 are free
+    m.pool.pool_state[1] = 0      # (acknowledged)
+    m.kv_offset[0][2] = 0
+    m.clear_cache(0)              # 4 pages back
+    assert m.pool.status() == (6, 0)
+    prefill(2, PS * 5)            # takes 5 of the 6 free pages, most of them slot 0's old ones
+    pages2 = m.pool.slot_table[2, :5].cpu().tolist()
+    assert sorted(pages2) != pages2 or pages2[0] != 0   # not the fixed run a slot used to own
+    # decode slot 1 until it is past max_seq_len: flagged, not silently wrapped
+    m.clear_cache(2)
+    for _ in range(PS * 3 + 4):
+        for layer in range(L):
+            q, k, v = (bf(torch.randn(1, h, 1, D, device=DEV)) for h in (Hq, Hkv, Hkv))
+            m.compute_attention(q, k, v, layer, torch.tensor([1]))
+    assert m.kv_offset[0][1].item() > PS * 6
+    with pytest.raises(ValueError):
+        m.clear_cache(1)
