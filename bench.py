@@ -404,6 +404,29 @@ def side_workload(torch, ops, name, steps, warmup, device, with_dense=True):
     return out
 
 
+def placement_rounds(torch, ops, args, B, ctx, Hkv, G, topk, device):
+    """Same binary, same seeded inputs, several allocations of the cache in one
+    process: round 0 is the process's first large allocation; later rounds reuse
+    memory that was freed, behind a dummy allocation of varying size."""
+    dummy_gib = [0, 0, 3, 11, 0, 27, 0, 5]
+    rounds = []
+    for r in range(args.placement_rounds):
+        d = dummy_gib[r % len(dummy_gib)]
+        dummy = torch.empty(d << 30, dtype=torch.uint8, device=device) if d else None
+        st = build_state(torch, ops, B, ctx, Hkv, G, topk, device, ragged=args.workload in RAGGED)
+        ms_step, _, kernel_ms, _ = time_step(torch, ops, st, B, Hkv, topk, max(5, min(args.steps, 20)), 3, args.mode)
+        dense_ms = None if args.no_dense else time_dense(torch, ops, st, 3)
+        rounds.append({"round": r, "dummy_gib": d, "kv_ptr": hex(st["kv"].data_ptr()), "ms_per_step": ms_step,
+                       "kernels_ms": kernel_ms, "dense_ms_per_step": dense_ms})
+        print(f"[placement] round {r}: dummy {d} GiB, kv at {hex(st['kv'].data_ptr())}, step {ms_step:.4f} ms, "
+              f"dense {dense_ms if dense_ms is None else round(dense_ms, 3)} ms", file=sys.stderr, flush=True)
+        del st, dummy
+        torch.cuda.empty_cache()
+    steps = [x["ms_per_step"] for x in rounds]
+    return {"workload": args.workload, "batch": B, "placement_rounds": rounds,
+            "ms_per_step_min": min(steps), "ms_per_step_max": max(steps), "spread": max(steps) / min(steps) - 1.0}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -434,6 +457,10 @@ def main():
     ap.add_argument("--topk_page", type=int, default=64)
     ap.add_argument("--page_size", type=int, default=16)
     ap.add_argument("--world_size", type=int, default=8)
+    ap.add_argument("--placement-rounds", type=int, default=0,
+                    help="instead of the benchmark: build, time (step and dense) and free the workload's cache this many "
+                         "times in one process, with dummy allocations of varying size in front of it, to see how much "
+                         "the physical placement of the cache moves the kernels; prints one JSON line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) to scale profiler byte counters")
     args = ap.parse_args()
@@ -469,6 +496,9 @@ def main():
     if args.batch:
         B = args.batch
     headline = args.workload == "qwen3-8b-share" and not args.batch
+    if args.placement_rounds:
+        print(json.dumps(placement_rounds(torch, ops, args, B, ctx, Hkv, G, topk, device)))
+        return
     t_setup = time.perf_counter()
     st = build_state(torch, ops, B, ctx, Hkv, G, topk, device, ragged=args.workload in RAGGED)
     torch.cuda.synchronize()
