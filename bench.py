@@ -57,7 +57,7 @@ WORKLOADS = {
 RAGGED = {"qwen3-0.6b-mix"}
 
 
-def algorithmic_bytes(lengths, Hkv, G, topk):
+def algorithmic_bytes(lengths, Hkv, G, topk, PS=PS):
     """Bytes per step that the algorithm has to move (bf16 K/V, int32 indices),
     summed over sequences with post-append token counts ``lengths``."""
     Hq = Hkv * G
@@ -78,7 +78,7 @@ def algorithmic_bytes(lengths, Hkv, G, topk):
     return dict(step=step, attention=attn, score_select=score, dense=dense, per_seq=step / max(1, len(lengths)))
 
 
-def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2, ragged=False, kv_alloc=None):
+def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2, ragged=False, kv_alloc=None, PS=PS):
     """Paged cache, K ~ N(0,1) + per-page mean offset N(0,0.5), V ~ N(0,1); kbar =
     true page means.  Uniform workloads use the reference layout (page id =
     p*B + b, max_len = ctx+512, every context ``ctx`` tokens + the appended one).
@@ -146,6 +146,7 @@ def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2, ragged=False, 
         out=torch.empty(B, Hkv * G, D, dtype=torch.bfloat16, device=device),
         n_full=n_full, max_pages=max_pages, num_pages=num_pages,
     )
+    st["page_size"] = PS
     st["max_pages_used"] = max((L + PS - 1) // PS for L in st["lengths"])
     ops.build_kbar(st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"])
     ws = ops.decode_workspace_bytes(B, Hkv * G, Hkv, topk + 1)
@@ -297,7 +298,7 @@ def time_step(torch, ops, st, B, Hkv, topk, steps, warmup, mode="auto"):
             ("append", lambda: ops.append_paged_kv(st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"],
                                                    st["last"])),
             ("score_topk", lambda: ops.block_score_topk(st["q"], st["kbar"], st["indices"], st["indptr"], st["last"], topk,
-                                                        st["sel"], st["cnt"], workspace=step_ws)),
+                                                        st["sel"], st["cnt"], workspace=step_ws, page_size=st["page_size"])),
             ("sparse_attention", lambda: ops.sparse_paged_decode(st["q"], st["kv"], st["sel"], st["cnt"], st["last"],
                                                                  out=st["out"], workspace=st["ws"])),
         ]
@@ -455,7 +456,8 @@ def main():
     ap.add_argument("--gen_len", type=int, default=32768)
     ap.add_argument("--batch_size", type=int, default=256)
     ap.add_argument("--topk_page", type=int, default=64)
-    ap.add_argument("--page_size", type=int, default=16)
+    ap.add_argument("--page_size", type=int, default=16, choices=[16, 32, 64],
+                    help="tokens per page of the cache (any workload; the reference's flag, benchmark/blocktopk.py:13)")
     ap.add_argument("--world_size", type=int, default=8)
     ap.add_argument("--placement-rounds", type=int, default=0,
                     help="instead of the benchmark: build, time (step and dense) and free the workload's cache this many "
@@ -472,16 +474,13 @@ def main():
     if args.model:
         from kinetics_amd.decoder_layer import qwen3_config
 
-        if args.page_size != PS:
-            print(f"bench.py: the kernels are built for page_size {PS}", file=sys.stderr)
-            sys.exit(2)
         mcfg = qwen3_config(args.model)
         hq, hkv = mcfg.num_attention_heads // args.world_size, mcfg.num_key_value_heads // args.world_size
         if hq < 1 or hkv < 1:
             print("bench.py: world_size exceeds the number of heads", file=sys.stderr)
             sys.exit(2)
         args.workload = "custom"
-        WORKLOADS["custom"] = (args.batch_size, args.gen_len // 2, hkv, hq // hkv, args.topk_page,
+        WORKLOADS["custom"] = (args.batch_size, args.gen_len // 2 // args.page_size * args.page_size, hkv, hq // hkv, args.topk_page,
                                f"{args.model} at world_size {args.world_size}: {hkv} KV heads, {hq} Q heads")
         WHOLE_LAYER_MODEL["custom"] = (args.model, args.world_size)
 
@@ -500,7 +499,8 @@ def main():
         print(json.dumps(placement_rounds(torch, ops, args, B, ctx, Hkv, G, topk, device)))
         return
     t_setup = time.perf_counter()
-    st = build_state(torch, ops, B, ctx, Hkv, G, topk, device, ragged=args.workload in RAGGED)
+    page = args.page_size
+    st = build_state(torch, ops, B, ctx, Hkv, G, topk, device, ragged=args.workload in RAGGED, PS=page)
     torch.cuda.synchronize()
     print(f"[bench] {args.workload}: B={B} ctx={ctx} H_kv={Hkv} G={G} topk={topk}, "
           f"KV {st['kv'].numel() * 2 / 1e9:.1f} GB resident, setup {time.perf_counter() - t_setup:.1f}s", file=sys.stderr)
@@ -509,7 +509,7 @@ def main():
     K = args.steps
     ms_step, elapsed, kernel_ms, fused = time_step(torch, ops, st, B, Hkv, topk, K, args.warmup, args.mode)
 
-    ab = algorithmic_bytes(st["lengths"], Hkv, G, topk)
+    ab = algorithmic_bytes(st["lengths"], Hkv, G, topk, page)
     step_gbs = ab["step"] / (ms_step * 1e-3) / 1e9
     if fused:
         dom_name, dom_kernel, dom_bytes, dom_ms = ("blocktopk_step_kernel (append + score + select + attention, fused)",
@@ -541,7 +541,7 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": args.workload, "description": desc, "batch": B, "ctx": ctx, "num_kv_heads": Hkv,
-                   "num_q_heads": Hkv * G, "head_dim": D, "page_size": PS, "topk_pages": topk,
+                   "num_q_heads": Hkv * G, "head_dim": D, "page_size": page, "topk_pages": topk,
                    "page_table": "ragged, half fragmented" if args.workload in RAGGED else "reference layout p*B+b",
                    "kv_resident_gb": round(st["kv"].numel() * 2 / 1e9, 2),
                    "launches_per_step": len(kernel_ms) - (0 if fused else 1)},
@@ -579,8 +579,8 @@ def main():
         result["dense_baseline"] = {"value": B / td, "unit": "tokens/s", "ms_per_step": td * 1e3, "steps": nd,
                                     "achieved_gbs": dense_bytes / td / 1e9, "frac": dense_bytes / td / 1e9 / HBM_PEAK_GBS,
                                     "sparse_over_dense": (B * K / elapsed) / (B / td)}
-    side = headline and not args.no_side_workloads
-    if args.token_topk or side:
+    side = headline and page == PS and not args.no_side_workloads
+    if (args.token_topk or side) and page == PS:   # the token-granular policies are built for 16-token pages
         result.update(time_token_policies(torch, ops, st, B, Hkv, G, topk, max(3, min(20, K // 5)), traffic_table.get))
     del st
     torch.cuda.empty_cache()

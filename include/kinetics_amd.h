@@ -37,8 +37,11 @@
  *                 final entry is always the sequence's last page
  *                 (ref: benchmark/blocktopk_decoder.py:143,217-221).
  *
- * Supported shapes: head_dim == 128, page_size == 16,
+ * Supported shapes: head_dim == 128; page_size 16, 32 or 64 (the reference's
+ * --page_size, benchmark/blocktopk.py:13; the token-granular policies
+ * kin_token_topk_decode / kin_strided_topk_decode: 16 only);
  * num_q_heads % num_kv_heads == 0 and group size num_q_heads/num_kv_heads <= 8.
+ * Where a comment below says "16" for a page it means page_size.
  */
 #ifndef KINETICS_AMD_H
 #define KINETICS_AMD_H
@@ -187,14 +190,14 @@ int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
                          int topk, int sink_pages, int local_tokens,
                          int32_t* sel_pages, int32_t* sel_count,
                          int32_t* sel_logical, float* scores_out,
-                         int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                         int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
                          int kbar_pages, int sel_stride,
                          void* workspace, size_t workspace_bytes, kin_stream_t stream);
 
 /*
  * Longest page list the selector can write for these settings:
- * topk + sink_pages + 1 + ceil((local_tokens - 1) / 16).  0 for arguments out
- * of range.
+ * topk + sink_pages + 1 + ceil((local_tokens - 1) / 16) (the bound for 16-token
+ * pages; larger pages never need more).  0 for arguments out of range.
  */
 int kin_sel_list_capacity(int topk, int sink_pages, int local_tokens);
 
@@ -225,11 +228,11 @@ int kin_decode_auto_splits(int batch, int num_kv_heads, int max_pages_per_list);
  * 1/sqrt(head_dim).  num_splits: 0 = automatic, else the number of split-K
  * partitions per list (>1 needs workspace, see kin_decode_workspace_bytes).
  * An empty list yields out = 0, lse = -inf.
- * first_page_offset (0..15): the first that many token slots of the FIRST listed
+ * first_page_offset (0 .. page_size-1): the first that many token slots of the FIRST listed
  * page of every list hold no token and are skipped -- for caches that store
  * each sequence shifted into its first page so that pages line up with blocks
  * that do not start at token 0 (LiteSys' blocks start after 4 sink tokens,
- * sparsity_utils.py:24-35: offset 12).  The offset is applied to list entry 0,
+ * sparsity_utils.py:24-35: offset page_size - 4, i.e. 12 for its default blocks of 16).  The offset is applied to list entry 0,
  * which is the sequence's first page only if the list was made with
  * sink_pages >= 1 (kin_block_score_topk then lists the first page first) or
  * the sequence has a single page: a caller that passes first_page_offset > 0

@@ -39,8 +39,8 @@ SIGNATURES = {
     "kin_build_kbar": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int64, c_int, _P]),
     "kin_block_score_topk": (
         c_int,
-        [_P, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P, c_size_t,
-         _P],
+        [_P, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P,
+         c_size_t, _P],
     ),
     "kin_sel_list_capacity": (c_int, [c_int, c_int, c_int]),
     "kin_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),

@@ -15,7 +15,8 @@ formulation, without touching the rest of the context.
 
 Supported configurations (anything else raises at construction):
   * no sparsity arguments                      -> dense paged decode
-  * ``attn_block_topk=k`` (+ ``attn_local``)    -> block top-k with block size 16
+  * ``attn_block_topk=k`` (+ ``attn_local``)    -> block top-k with ``attn_block_size`` 16 (default),
+                                                  32 or 64: the pages are that size
   * ``attn_topk=k`` (+ ``attn_local``)          -> token-level top-k (topk_sparsity,
                                                   sparsity_utils.py:6-21), one launch that
                                                   reads every key of the context once
@@ -30,9 +31,10 @@ Supported configurations (anything else raises at construction):
 LiteSys always attends 4 hard-wired "sink" tokens, starts its 16-token blocks
 right after them and always attends the ``_local`` newest tokens that remain
 after the last whole block (sparsity_utils.py:24-35,240).  To keep that exact
-geometry on 16-token pages, a sparse manager stores every sequence 12 slots
-into its first page: the sink tokens are slots 12..15 of page 0, block j is
-page j+1, and the kernels are told to skip the 12 padding slots
+geometry on pages of one block each, a sparse manager stores every sequence
+block_size - 4 slots (12 for blocks of 16) into its first page: the sink tokens
+are the last 4 slots of page 0, block j is page j+1, and the kernels are told to
+skip the padding slots
 (``first_page_offset``), to pin one sink page and to keep the newest
 ``attn_local`` tokens out of the candidates (``local_tokens``).  The attended
 token set is then LiteSys' own, token for token.
@@ -101,8 +103,8 @@ class PagedBatchKVManager:
                         and 0 <= self.token_local <= 1024):
                     raise NotImplementedError("strided blocks: block size <= 64, budget <= 4096 tokens, attn_local <= 1024")
                 self.block_topk = None
-            elif kwargs.get("attn_block_size", PAGE) != PAGE:
-                raise NotImplementedError("block size must equal the page size (16)")
+            elif kwargs.get("attn_block_size", PAGE) not in (16, 32, 64):
+                raise NotImplementedError("attn_block_size must be 16, 32 or 64 (a block is one page)")
         elif kwargs.get("attn_stride") is not None:
             raise NotImplementedError("attn_stride needs attn_block_topk")
         if kwargs.get("attn_local") is not None and self.block_topk is None and self.strided is None and self.token_topk is None:
@@ -110,6 +112,8 @@ class PagedBatchKVManager:
             if not 0 <= int(kwargs["attn_local"]) <= 1024:
                 raise NotImplementedError("attn_local must be in [0, 1024]")
         self.sparse = self.block_topk is not None
+        # tokens per page: LiteSys' block size for the block policy, 16 otherwise
+        self.page = int(kwargs.get("attn_block_size", PAGE)) if self.sparse else PAGE
         if self.token_topk is not None:
             self.token_local = int(kwargs["attn_local"])
         self.layer_skip = list(kwargs.get("attn_layer_skip", [0]))
@@ -118,18 +122,18 @@ class PagedBatchKVManager:
         if self.sparse and not 1 <= self.local_tokens <= 1009:
             raise NotImplementedError("attn_local must be in [1, 1009]")
         # padding slots in front of every sequence: LiteSys' 4 sink tokens end page 0, its blocks are pages 1, 2, ...
-        self.pad = PAGE - 4 if self.sparse else 0
+        self.pad = self.page - 4 if self.sparse else 0
 
         B, Hq, Hkv, D = max_batch_size, self.num_attention_heads, self.num_key_value_heads, self.head_dim
-        self.pages_per_slot = P = (max_seq_len + self.pad + PAGE - 1) // PAGE
+        self.pages_per_slot = P = (max_seq_len + self.pad + self.page - 1) // self.page
         dev = self.device
         # The page pool, shared by all layers (a token position occupies the same page id in every
         # layer's cache): slots take pages as they grow and give them back in clear_cache.
         self.num_pool_pages = int(kwargs.get("kv_pool_pages") or B * P)
         if not 1 <= self.num_pool_pages <= B * P:
             raise ValueError(f"kv_pool_pages must be in [1, max_batch_size * pages_per_slot = {B * P}]")
-        self.pool = ops.PagePool(self.num_pool_pages, B, P, PAGE, dev)
-        self.kv_cache = [torch.zeros(self.num_pool_pages, 2, PAGE, Hkv, D, dtype=dtype, device=dev)
+        self.pool = ops.PagePool(self.num_pool_pages, B, P, self.page, dev)
+        self.kv_cache = [torch.zeros(self.num_pool_pages, 2, self.page, Hkv, D, dtype=dtype, device=dev)
                          for _ in range(self.num_layers)]
         self.kbar = [torch.zeros(B, Hkv, P, D, dtype=dtype, device=dev) for _ in range(self.num_layers)]
         self.kv_offset = [torch.zeros(B, dtype=torch.int32, device=dev) for _ in range(self.num_layers)]
@@ -211,7 +215,7 @@ class PagedBatchKVManager:
             if sparse:
                 ops.block_score_topk(self._q, kbar, self.page_indices, self.page_indptr, self.last_page_len,
                                      self.block_topk, self._sel, self._cnt, sink_pages=self.sink_pages,
-                                     local_tokens=self.local_tokens, workspace=self._ws)
+                                     local_tokens=self.local_tokens, workspace=self._ws, page_size=self.page)
                 ops.sparse_paged_decode(self._q, kv, self._sel, self._cnt, self.last_page_len, out=self._out,
                                         workspace=self._ws, first_page_offset=self.pad)
             else:
@@ -230,11 +234,11 @@ class PagedBatchKVManager:
         offset = int(self.kv_offset[layer_idx][slot].item())
         total = offset + seq_len
         pad = self.pad                                   # token t lives in cache slot t + pad
-        if total + pad > self.pages_per_slot * PAGE:
+        if total + pad > self.pages_per_slot * self.page:
             raise ValueError(f"sequence of {total} tokens exceeds max_seq_len")
         Hkv, D = self.num_key_value_heads, self.head_dim
         self.kv_offset[layer_idx][slot] += seq_len
-        n_pages = (total + pad + PAGE - 1) // PAGE
+        n_pages = (total + pad + self.page - 1) // self.page
         self.pool.reserve(torch.tensor([total + pad], dtype=torch.int32, device=self.device),
                           torch.tensor([slot], dtype=torch.int32, device=self.device))
         free, bits = self.pool.status()
@@ -242,14 +246,14 @@ class PagedBatchKVManager:
             raise _lib.KineticsError(f"page pool exhausted ({free} pages free): cannot hold {total} tokens in slot {slot}")
         idx = self.pool.slot_table[slot, :n_pages].contiguous()
         ptr = torch.tensor([0, n_pages], dtype=torch.int32, device=self.device)
-        last = torch.tensor([total + pad - (n_pages - 1) * PAGE], dtype=torch.int32, device=self.device)
+        last = torch.tensor([total + pad - (n_pages - 1) * self.page], dtype=torch.int32, device=self.device)
         # rows to their page slots, mean keys of the pages that are now full
         ops.append_paged_kv_ragged(key_states[0].transpose(0, 1).contiguous(), value_states[0].transpose(0, 1).contiguous(),
                                    torch.tensor([0, seq_len], dtype=torch.int32, device=self.device),
                                    self.kv_cache[layer_idx], self.kbar[layer_idx][slot:slot + 1], idx, ptr, last)
-        pages = self.kv_cache[layer_idx][idx.long()]                                           # [n_pages, 2, PAGE, Hkv, D]
-        k_all = pages[:, 0].reshape(n_pages * PAGE, Hkv, D)[pad:total + pad].transpose(0, 1)   # [Hkv, total, D]
-        v_all = pages[:, 1].reshape(n_pages * PAGE, Hkv, D)[pad:total + pad].transpose(0, 1)
+        pages = self.kv_cache[layer_idx][idx.long()]                                           # [n_pages, 2, self.page, Hkv, D]
+        k_all = pages[:, 0].reshape(n_pages * self.page, Hkv, D)[pad:total + pad].transpose(0, 1)   # [Hkv, total, D]
+        v_all = pages[:, 1].reshape(n_pages * self.page, Hkv, D)[pad:total + pad].transpose(0, 1)
         G = self.num_attention_heads // Hkv
         q = query_states[0]                                                                    # [Hq, s, D]
         pos_q = torch.arange(offset, total, device=self.device)[:, None]

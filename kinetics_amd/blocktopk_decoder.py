@@ -99,7 +99,7 @@ class BlockTopkPagedAttention:
         torch.ops.kinetics.block_score_topk(query_states, self.compressed_key_cache, self.paged_kv_indices,
                                             self.paged_kv_indptr, self.last_kv_lens, self.topk_page,
                                             self.topk_page_indices, self.topk_page_count, self.sink_pages,
-                                            self.local_tokens, self.step_workspace)
+                                            self.local_tokens, self.step_workspace, self.page_size)
 
     def decode(self, query_states: torch.Tensor) -> torch.Tensor:
         """benchmark/blocktopk_decoder.py:223-225."""

@@ -32,9 +32,8 @@ int check_common_dims(const char* fn, int batch, int num_q_heads, int num_kv_hea
     return fail(KIN_ERR_BAD_SHAPE, "%s: head_dim=%d and page_size=%d must be positive", fn, head_dim, page_size);
   if (head_dim != kHeadDim)
     return fail(KIN_ERR_UNSUPPORTED, "%s: head_dim=%d unsupported (kernels are built for %d)", fn, head_dim, kHeadDim);
-  if (page_size != kPageSize)
-    return fail(KIN_ERR_UNSUPPORTED, "%s: page_size=%d unsupported (kernels are built for %d)", fn, page_size,
-                kPageSize);
+  if (!supported_page_size(page_size))
+    return fail(KIN_ERR_UNSUPPORTED, "%s: page_size=%d unsupported (kernels are built for 16, 32 and 64)", fn, page_size);
   if (num_q_heads / num_kv_heads > kMaxGroup)
     return fail(KIN_ERR_UNSUPPORTED, "%s: GQA group %d unsupported (max %d)", fn, num_q_heads / num_kv_heads,
                 kMaxGroup);
@@ -48,9 +47,16 @@ int check_fixed_pages(const char* fn, int sink_pages, int local_tokens) {
   return KIN_OK;
 }
 
-int check_first_page_offset(const char* fn, int first_page_offset) {
-  if (first_page_offset < 0 || first_page_offset >= kPageSize)
-    return fail(KIN_ERR_BAD_SHAPE, "%s: first_page_offset=%d must be in [0, %d)", fn, first_page_offset, kPageSize);
+int check_first_page_offset(const char* fn, int first_page_offset, int page_size) {
+  if (first_page_offset < 0 || first_page_offset >= page_size)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: first_page_offset=%d must be in [0, page_size=%d)", fn, first_page_offset, page_size);
+  return KIN_OK;
+}
+
+int check_page_size_16(const char* fn, int page_size) {
+  if (page_size != kPageSize)
+    return fail(KIN_ERR_UNSUPPORTED, "%s: page_size=%d unsupported (the token-granular policies are built for %d)", fn,
+                page_size, kPageSize);
   return KIN_OK;
 }
 

@@ -13,7 +13,7 @@ struct AppendParams {
   const int32_t* page_indices;
   const int32_t* page_indptr;
   const int32_t* last_page_len;
-  int batch, num_kv_heads, kbar_pages;
+  int batch, num_kv_heads, kbar_pages, page_size;
   int64_t num_pages;
 };
 
@@ -29,7 +29,8 @@ __global__ __launch_bounds__(256) void append_kernel(AppendParams p) {
   uint32_t* kbar_row = p.kbar ? p.kbar + kbar_row_index(b, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2)
                               : nullptr;
   append_token_row(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2), p.kv_cache, kbar_row,
-                   p.page_indices[e - 1], p.last_page_len[b], n_pages, p.kbar_pages, h, p.num_kv_heads, p.num_pages, lane);
+                   p.page_indices[e - 1], p.last_page_len[b], n_pages, p.kbar_pages, h, p.num_kv_heads, p.num_pages, lane,
+                   p.page_size);
 }
 
 // grid = batch * Hkv * ceil(kbar_pages / 16) blocks (flat, so it is not bound by
@@ -45,14 +46,14 @@ __global__ __launch_bounds__(256) void build_kbar_kernel(AppendParams p, int pag
   const int s = p.page_indptr[b], e = p.page_indptr[b + 1];
   const int n_pages = e - s;
   if (n_pages <= 0) return;
-  const int n_full = (p.last_page_len[b] >= kPageSize) ? n_pages : n_pages - 1;
+  const int n_full = (p.last_page_len[b] >= p.page_size) ? n_pages : n_pages - 1;
   if (page >= n_full || page >= p.kbar_pages) return;
   const int64_t pid = p.page_indices[s + page];
   if (pid < 0 || pid >= p.num_pages) return;
   const int row_stride = p.num_kv_heads * (kHeadDim / 2);  // dwords per token row
-  const int64_t page_dwords = 2LL * kPageSize * row_stride;
+  const int64_t page_dwords = 2LL * p.page_size * row_stride;
   const u32x4* kplane = reinterpret_cast<const u32x4*>(p.kv_cache + pid * page_dwords + h * (kHeadDim / 2)) + c16;
-  const u32x4 m = page_mean_16B(kplane, row_stride / 4);
+  const u32x4 m = page_mean_16B(kplane, row_stride / 4, p.page_size);
   reinterpret_cast<u32x4*>(p.kbar + kbar_row_index(b, h, page, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2))[c16] = m;
 }
 
@@ -66,7 +67,7 @@ struct RaggedAppendParams {
   const int32_t* page_indices;
   const int32_t* page_indptr;
   const int32_t* last_page_len;
-  int batch, num_kv_heads, kbar_pages;
+  int batch, num_kv_heads, kbar_pages, page_size;
   int64_t nnz;
   int64_t num_pages;
 };
@@ -96,6 +97,7 @@ __global__ __launch_bounds__(256) void append_ragged_kernel(RaggedAppendParams p
   const int64_t row0 = (int64_t)blockIdx.x * kRaggedRows;
   const int rows_here = (int)min((int64_t)kRaggedRows, p.nnz - row0);
   const int cpr = p.num_kv_heads * (kHeadDim / 8);  // 16-byte chunks per token row (all heads)
+  const int P = p.page_size;
   if (tid < kRaggedRows) {
     int64_t dst = -1;
     const int64_t row = row0 + tid;
@@ -106,12 +108,12 @@ __global__ __launch_bounds__(256) void append_ragged_kernel(RaggedAppendParams p
       const int n_pages = e - s;
       const int last = p.last_page_len[b];
       // rows outside their sequence's range (malformed indptr) or contract are skipped
-      if (row >= a0 && row < a1 && n_pages > 0 && last >= 1 && last <= kPageSize) {
-        const int64_t kv_len = (int64_t)(n_pages - 1) * kPageSize + last;
+      if (row >= a0 && row < a1 && n_pages > 0 && last >= 1 && last <= P) {
+        const int64_t kv_len = (int64_t)(n_pages - 1) * P + last;
         const int64_t pos = kv_len - (a1 - a0) + (row - a0);
         if (pos >= 0) {
-          const int64_t pid = p.page_indices[s + (int)(pos / kPageSize)];
-          if (pid >= 0 && pid < p.num_pages) dst = (pid * 2 * kPageSize + (pos % kPageSize)) * cpr;
+          const int64_t pid = p.page_indices[s + (int)(pos / P)];
+          if (pid >= 0 && pid < p.num_pages) dst = (pid * 2 * P + (pos % P)) * cpr;
         }
       }
     }
@@ -121,7 +123,7 @@ __global__ __launch_bounds__(256) void append_ragged_kernel(RaggedAppendParams p
   const u32x4* ksrc = reinterpret_cast<const u32x4*>(p.k) + row0 * cpr;
   const u32x4* vsrc = reinterpret_cast<const u32x4*>(p.v) + row0 * cpr;
   u32x4* cache = reinterpret_cast<u32x4*>(p.kv_cache);
-  const int64_t v_plane = (int64_t)kPageSize * cpr;  // V plane of a page follows its K plane
+  const int64_t v_plane = (int64_t)P * cpr;  // V plane of a page follows its K plane
   const int total = rows_here * cpr;
   constexpr int kU = 4;
   for (int base = tid; base < total; base += 256 * kU) {
@@ -161,6 +163,7 @@ __global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p)
   const int64_t row0 = (int64_t)blockIdx.x * kRaggedRows;
   const int rows_here = (int)min((int64_t)kRaggedRows, p.nnz - row0);
   const int cpr = p.num_kv_heads * (kHeadDim / 8);
+  const int P = p.page_size;
   if (tid < kRaggedRows) {
     int64_t src = -1, dst = 0;
     const int64_t row = row0 + tid;
@@ -170,14 +173,14 @@ __global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p)
       const int s = p.page_indptr[b], e = p.page_indptr[b + 1];
       const int n_pages = e - s;
       const int last = p.last_page_len[b];
-      if (row >= a0 && row < a1 && n_pages > 0 && last >= 1 && last <= kPageSize) {
-        const int64_t kv_len = (int64_t)(n_pages - 1) * kPageSize + last;
+      if (row >= a0 && row < a1 && n_pages > 0 && last >= 1 && last <= P) {
+        const int64_t kv_len = (int64_t)(n_pages - 1) * P + last;
         const int64_t pos = kv_len - (a1 - a0) + (row - a0);
-        const int64_t page = pos / kPageSize;
-        if (pos >= 0 && pos % kPageSize == kPageSize - 1 && page < p.kbar_pages) {
+        const int64_t page = pos / P;
+        if (pos >= 0 && pos % P == P - 1 && page < p.kbar_pages) {
           const int64_t pid = p.page_indices[s + (int)page];
           if (pid >= 0 && pid < p.num_pages) {
-            src = pid * 2 * kPageSize * cpr;
+            src = pid * 2 * P * cpr;
             dst = kbar_row_index(b, 0, (int)page, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 8);
           }
         }
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p)
     const int r = pair / p.num_kv_heads, h = pair - r * p.num_kv_heads;
     const int64_t src = src16[r];
     if (src < 0) continue;
-    const u32x4 m = page_mean_16B(cache + src + h * (kHeadDim / 8) + c16, cpr);
+    const u32x4 m = page_mean_16B(cache + src + h * (kHeadDim / 8) + c16, cpr, P);
     kbar[dst16[r] + (int64_t)h * p.kbar_pages * (kHeadDim / 8) + c16] = m;
   }
 }
@@ -241,6 +244,7 @@ int kin_append_paged_kv(const kin_bf16_t* k, const kin_bf16_t* v, kin_bf16_t* kv
   p.batch = batch;
   p.num_kv_heads = num_kv_heads;
   p.kbar_pages = kbar_pages;
+  p.page_size = page_size;
   p.num_pages = num_pages;
   const int64_t items = (int64_t)batch * num_kv_heads;
   const unsigned blocks = (unsigned)((items + 3) / 4);
@@ -274,6 +278,7 @@ int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* 
   p.batch = batch;
   p.num_kv_heads = num_kv_heads;
   p.kbar_pages = kbar_pages;
+  p.page_size = page_size;
   p.num_pages = num_pages;
   build_kbar_kernel<<<(unsigned)(items * page_blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(p, page_blocks);
   return check_hip(hipGetLastError(), "build_kbar_kernel launch");
@@ -310,6 +315,7 @@ int kin_append_paged_kv_ragged(const kin_bf16_t* k, const kin_bf16_t* v, const i
   p.batch = batch;
   p.num_kv_heads = num_kv_heads;
   p.kbar_pages = kbar_pages;
+  p.page_size = page_size;
   p.nnz = nnz;
   p.num_pages = num_pages;
   hipStream_t s = static_cast<hipStream_t>(stream);

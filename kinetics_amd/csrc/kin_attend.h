@@ -4,9 +4,11 @@
 // lists have to fill the GPU).  Shared by the stand-alone paged decode kernel and the fused
 // decode-step kernel.
 //
-// Work decomposition: the workgroup's NW waves take the list's pages round-robin,
-// one 8 KiB page (16 keys + 16 values of 128 bf16) per wave per iteration, and
-// keep private online-softmax state that is merged once at the end.
+// Work decomposition: the workgroup's NW waves take the list's tiles round-robin,
+// one tile (16 keys + 16 values of 128 bf16: 8 KiB) per wave per iteration, and
+// keep private online-softmax state that is merged once at the end.  A page of
+// 16 tokens is one tile; pages of 32 or 64 tokens are 2 or 4 tiles, each a run of
+// 16 rows of the page's K plane and the matching 16 rows of its V plane.
 //
 // Per page and wave (lane l, row group kg = l/16, 16-byte column chunk c = l%16):
 //   K  4 x 16-byte LDS-direct buffer loads, each instruction covering 4 whole
@@ -118,15 +120,16 @@ struct AttendArgs {
   const uint16_t* q_bh;  // the group's G query rows (contiguous, 128 bf16 each)
   const char* kvb;       // kv_cache base + h * 256 bytes
   int row_bytes;         // bytes between token rows of a page (H_kv * 256)
-  int page_bytes;        // 2 * 16 * row_bytes
+  int page_bytes;        // 2 * page_size * row_bytes
   int span;              // bytes addressable from kvb within one page
+  int page_size;         // tokens per page: 16, 32 or 64
   int64_t num_pages;
   int G;
   float scale_log2;      // sm_scale * log2(e)
   int n;                 // list length
   int p0, p1;            // this workgroup's part of the list [p0, p1)
   int last_len;          // tokens in the list's final page
-  int first_skip;        // leading token slots of list entry 0 that hold no token (0..15)
+  int first_skip;        // leading token slots of list entry 0 that hold no token (0 .. page_size-1)
 };
 
 // K pages a wave keeps staged in LDS in attend_list(): the one being read and 1 or
@@ -248,9 +251,12 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
   const int page_bytes = a.page_bytes;
   const int span = a.span;
   const char* kvb = a.kvb;
+  // A tile's rows are addressed from its first K row: its V rows lie one K plane
+  // (page_size rows) further.
+  const int tshift = page_tile_shift(a.page_size), tmask = (1 << tshift) - 1;
   int voff[4];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) voff[c] = (kPageSize + 4 * kg + c) * row_bytes + c16 * 16;
+  for (int c = 0; c < 4; ++c) voff[c] = (a.page_size + 4 * kg + c) * row_bytes + c16 * 16;
   // K staging: KS 4 KiB stages per wave, filled by LDS-direct buffer loads
   // (no VGPRs while in flight).  Load c brings rows 4c..4c+3: lane (kg, c16)
   // lands at LDS row 4c+kg, position c16, and fetches the chunk that belongs
@@ -276,28 +282,36 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
     for (int u = 0; u < 8; ++u) O[half][u] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // This wave takes list entries my_first, my_first+NW, ...  The loop below is
-  // branch-free: a page past the end (or with an id outside the cache) is read
-  // through an empty buffer descriptor -- zeros, no memory traffic -- and all
-  // of its tokens are masked.
-  const int my_first = p0 + w;
-  const int iters = (p1 > my_first) ? (p1 - my_first + NW - 1) / NW : 0;
+  // This wave takes the tiles my_first, my_first+NW, ... of the list entries p0 .. p1-1
+  // (entry e owns the tiles e << tshift ..; of the list's final page only the tiles
+  // that hold tokens count).  The loop below is branch-free: a tile past the end (or
+  // of a page with an id outside the cache) is read through an empty buffer
+  // descriptor -- zeros, no memory traffic -- and all of its tokens are masked.
   const int n_last = n - 1;
+  const int n_tiles = n > 0 ? (n_last << tshift) + ((min(max(last_len, 1), a.page_size) + kPageSize - 1) >> 4) : 0;
+  const int t0 = p0 << tshift, t1 = min(p1 << tshift, n_tiles);
+  const int my_first = t0 + w;
+  const int iters = (t1 > my_first) ? (t1 - my_first + NW - 1) / NW : 0;
   // Page ids are fetched one half-step before they are needed.
   auto load_id = [&](int it) -> int {
     const int idx = my_first + NW * it;
-    return id_at(idx < p1 ? idx : p0);
+    return id_at((idx < t1 ? idx : t0) >> tshift);
   };
   const int first_skip = a.first_skip;
   auto page_rsrc = [&](int it, int id, int& valid_tokens) {
     const int idx = my_first + NW * it;
-    const bool ok = idx < p1 && id >= 0 && (int64_t)id < a.num_pages;
-    // The skipped slots of entry 0 are folded into one number: bits 8.. hold
-    // the first counted slot, bits 0..7 one past the last.
-    const int hi = idx == n_last ? last_len : kPageSize;
-    const int lo = idx == 0 ? min(first_skip, hi) : 0;
+    const int e = idx >> tshift, sub16 = (idx & tmask) * kPageSize;  // list entry, first token slot of the tile in its page
+    const bool ok = idx < t1 && id >= 0 && (int64_t)id < a.num_pages;
+    // The token slots of the page that count are [lo_p, hi_p); the tile's share of
+    // them is folded into one number: bits 8.. hold the first counted slot of the
+    // tile, bits 0..7 one past the last.
+    const int hi_p = e == n_last ? last_len : a.page_size;
+    const int lo_p = e == 0 ? min(first_skip, hi_p) : 0;
+    const int hi = min(max(hi_p - sub16, 0), kPageSize);
+    const int lo = min(max(lo_p - sub16, 0), hi);
     valid_tokens = ok ? (hi | (lo << 8)) : 0;
-    return make_rsrc(kvb + (int64_t)(ok ? id : 0) * page_bytes, ok ? span : 0);
+    const int tile_off = sub16 * row_bytes;
+    return make_rsrc(kvb + (int64_t)(ok ? id : 0) * page_bytes + tile_off, ok ? span - tile_off : 0);
   };
   auto issue_v = [&](__amdgpu_buffer_rsrc_t r, u32x4 (&vv)[4]) {
 #pragma unroll

@@ -9,7 +9,8 @@
 namespace kin {
 
 constexpr int kHeadDim = 128;    // elements per head row (256 B in bf16)
-constexpr int kPageSize = 16;    // tokens per page
+constexpr int kPageSize = 16;    // tokens of one attention tile (an MFMA tile is 16 keys); the smallest page
+constexpr int kMaxPageSize = 64; // pages hold 16, 32 or 64 tokens: 1, 2 or 4 tiles
 constexpr int kRowBytes = kHeadDim * 2;
 constexpr int kMaxGroup = 8;     // largest supported num_q_heads / num_kv_heads
 constexpr int kMaxTopk = 2048;
@@ -25,8 +26,13 @@ inline int64_t xcd_grid_size(int batch, int num_kv_heads) {
 constexpr int kMaxFixedPages = 64;  // most sink / local pages that can be pinned into every list
 constexpr int kMaxLocalTokens = (kMaxFixedPages - 1) * kPageSize + 1;
 
-// Most trailing pages that local_tokens always-attended trailing tokens can span.
+// Most trailing pages that local_tokens always-attended trailing tokens can span
+// (for 16-token pages; larger pages need no more).
 __host__ __device__ inline int max_local_pages(int local_tokens) { return 1 + (local_tokens + kPageSize - 2) / kPageSize; }
+
+inline bool supported_page_size(int ps) { return ps == 16 || ps == 32 || ps == 64; }
+// log2(page_size / 16): a page is 1 << page_tile_shift(ps) tiles of 16 tokens.
+__host__ __device__ inline int page_tile_shift(int ps) { return ps >= 64 ? 2 : (ps >= 32 ? 1 : 0); }
 
 // Cache-policy bits for buffer loads of read-once data (K/V pages, mean keys):
 // the non-temporal hint keeps streams from displacing each other in L2/MALL and
@@ -55,7 +61,9 @@ int check_common_dims(const char* fn, int batch, int num_q_heads, int num_kv_hea
 // Range rules for the always-attended parts of a page list.
 int check_fixed_pages(const char* fn, int sink_pages, int local_tokens);
 // first_page_offset: padding slots at the start of every sequence's first page.
-int check_first_page_offset(const char* fn, int first_page_offset);
+int check_first_page_offset(const char* fn, int first_page_offset, int page_size = kPageSize);
+// The token-granular policies address single token rows and are built for 16-token pages only.
+int check_page_size_16(const char* fn, int page_size);
 
 // Split scoring of the page selector (few, long lists): workgroups per list.  1
 // unless the lists are at most a quarter of the CUs and long, then enough to put

@@ -21,6 +21,7 @@ struct DecodeParams {
   int batch, num_q_heads, num_kv_heads, group;
   int list_stride, num_splits;
   int first_page_offset;  // padding slots at the start of list entry 0
+  int page_size;
   int64_t num_pages;
   float scale_log2;  // sm_scale * log2(e)
 };
@@ -54,8 +55,9 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
   a.q_bh = p.q + ((int64_t)b * p.num_q_heads + (int64_t)h * G) * kHeadDim;
   a.kvb = reinterpret_cast<const char*>(p.kv) + (int64_t)h * kRowBytes;
   a.row_bytes = p.num_kv_heads * kRowBytes;
-  a.page_bytes = 2 * kPageSize * a.row_bytes;
+  a.page_bytes = 2 * p.page_size * a.row_bytes;
   a.span = a.page_bytes - h * kRowBytes;
+  a.page_size = p.page_size;
   a.num_pages = p.num_pages;
   a.G = G;
   a.scale_log2 = p.scale_log2;
@@ -167,7 +169,7 @@ static int check_decode_args(const char* fn, const void* q, const void* kv_cache
   if (!q || !kv_cache || !last_page_len || !out) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size);
   if (st) return st;
-  st = check_first_page_offset(fn, first_page_offset);
+  st = check_first_page_offset(fn, first_page_offset, page_size);
   if (st) return st;
   if (num_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_pages=%lld must be >= 1", fn, (long long)num_pages);
   if (num_splits < 0) return fail(KIN_ERR_BAD_SHAPE, "%s: num_splits=%d is negative", fn, num_splits);
@@ -220,6 +222,7 @@ int kin_sparse_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, con
   p.list_stride = sel_stride;
   p.num_pages = num_pages;
   p.first_page_offset = first_page_offset;
+  p.page_size = page_size;
   const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
   p.scale_log2 = scale * 1.4426950408889634f;
   return launch_decode(fn, p, batch, workspace, workspace_bytes, sel_stride, num_splits,
@@ -255,6 +258,7 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, cons
   p.list_stride = 0;
   p.num_pages = num_pages;
   p.first_page_offset = first_page_offset;
+  p.page_size = page_size;
   const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
   p.scale_log2 = scale * 1.4426950408889634f;
   return launch_decode(fn, p, batch, workspace, workspace_bytes, max_pages_per_seq, num_splits,

@@ -18,7 +18,7 @@ struct ScoreTopkParams {
   int32_t* sel_logical;  // may be null
   float* scores_out;     // may be null
   int batch, num_q_heads, num_kv_heads, group;
-  int kbar_pages, sel_stride, topk, sink_pages, local_tokens;
+  int kbar_pages, sel_stride, topk, sink_pages, local_tokens, page_size;
   int sort_cap;
   int chunks;          // workgroups per list
   int32_t* ws_count;   // [lists] arrival counters, zero at launch and left zero
@@ -52,7 +52,7 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
   a.q_bh = p.q + ((int64_t)b * p.num_q_heads + (int64_t)h * p.group) * kHeadDim;
   a.G = p.group;
   a.n_pages = n_pages;
-  split_pages(n_pages, p.last_page_len[b], p.sink_pages, p.local_tokens, p.kbar_pages, a.n_sink, a.n_cand, a.n_local);
+  split_pages(n_pages, p.last_page_len[b], p.sink_pages, p.local_tokens, p.kbar_pages, p.page_size, a.n_sink, a.n_cand, a.n_local);
   a.kb = reinterpret_cast<const char*>(p.kbar) + kbar_row_index(b, h, a.n_sink, p.num_kv_heads, p.kbar_pages) * kRowBytes;
   a.topk = p.topk;
   a.table = p.page_indices + ps;
@@ -97,13 +97,13 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
                                     int sink_pages, int local_tokens,
                                     int32_t* sel_pages, int32_t* sel_count,
                                     int32_t* sel_logical, float* scores_out, int batch, int num_q_heads,
-                                    int num_kv_heads, int head_dim, int kbar_pages, int sel_stride,
+                                    int num_kv_heads, int head_dim, int page_size, int kbar_pages, int sel_stride,
                                     void* workspace, size_t workspace_bytes, kin_stream_t stream) {
   using namespace kin;
   const char* fn = "kin_block_score_topk";
   if (!q || !kbar || !page_indices || !page_indptr || !last_page_len || !sel_pages || !sel_count)
     return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
-  int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, kPageSize);
+  int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size);
   if (st) return st;
   if (topk < 0) return fail(KIN_ERR_BAD_SHAPE, "%s: topk=%d is negative", fn, topk);
   st = check_fixed_pages(fn, sink_pages, local_tokens);
@@ -138,6 +138,7 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
   p.topk = topk;
   p.sink_pages = sink_pages;
   p.local_tokens = local_tokens;
+  p.page_size = page_size;
   p.sort_cap = select_sort_cap(topk, kbar_pages);
   const size_t lds = select_lds_bytes(kbar_pages, p.sort_cap) + (size_t)list_cap * 4;
   const int64_t items = (int64_t)batch * num_kv_heads;

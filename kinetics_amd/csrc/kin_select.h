@@ -64,11 +64,11 @@ __host__ __device__ inline int select_sort_cap(int topk, int kbar_pages) {
 // pages and the newest local_tokens tokens, so the open page (local_tokens >= 1)
 // is always local.  kbar_pages bounds the logical pages that have a mean key.
 __host__ __device__ inline void split_pages(int n_pages, int last_len, int sink_pages, int local_tokens,
-                                            int kbar_pages, int& n_sink, int& n_cand, int& n_local) {
-  last_len = last_len < 1 ? 1 : (last_len > kPageSize ? kPageSize : last_len);
+                                            int kbar_pages, int page_size, int& n_sink, int& n_cand, int& n_local) {
+  last_len = last_len < 1 ? 1 : (last_len > page_size ? page_size : last_len);
   n_sink = sink_pages < n_pages - 1 ? sink_pages : n_pages - 1;
-  const int between = (n_pages - 1 - n_sink) * kPageSize + last_len - local_tokens;  // tokens after the sink, before the local part
-  n_cand = between > 0 ? between / kPageSize : 0;
+  const int between = (n_pages - 1 - n_sink) * page_size + last_len - local_tokens;  // tokens after the sink, before the local part
+  n_cand = between > 0 ? between / page_size : 0;
   n_local = n_pages - n_sink - n_cand;
   const int cap = kbar_pages - n_sink;
   if (n_cand > cap) n_cand = cap > 0 ? cap : 0;

@@ -32,7 +32,7 @@ struct StepParams {
   uint16_t* out;
   float* lse;  // optional
   int batch, num_q_heads, num_kv_heads, group;
-  int kbar_pages, sel_stride, topk, sink_pages, local_tokens, first_page_offset, sort_cap;
+  int kbar_pages, sel_stride, topk, sink_pages, local_tokens, first_page_offset, sort_cap, page_size;
   int region0_bytes;  // LDS: max(attend staging, select scratch); the page list follows it
   // Split scoring (few, long sequences): `chunks` workgroups per list score a slice of the
   // candidates each into ws_keys; the last one to finish selects and attends.
@@ -86,7 +86,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
           reinterpret_cast<uint32_t*>(p.kbar) + kbar_row_index(b, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2);
       append_token_row(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2),
                        reinterpret_cast<uint32_t*>(p.kv), kbar_row, p.page_indices[pe - 1], last_len, n_pages, p.kbar_pages, h,
-                       p.num_kv_heads, p.num_pages, tid);
+                       p.num_kv_heads, p.num_pages, tid, p.page_size);
       // The attention phase of this workgroup reads the row back: make the stores
       // visible before the barriers that separate the phases.
       __threadfence_block();
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   s.q_bh = p.q + hq0 * kHeadDim;
   s.G = G;
   s.n_pages = n_pages;
-  split_pages(n_pages, last_len, p.sink_pages, p.local_tokens, p.kbar_pages, s.n_sink, s.n_cand, s.n_local);
+  split_pages(n_pages, last_len, p.sink_pages, p.local_tokens, p.kbar_pages, p.page_size, s.n_sink, s.n_cand, s.n_local);
   s.kb = reinterpret_cast<const char*>(p.kbar) + kbar_row_index(b, h, s.n_sink, p.num_kv_heads, p.kbar_pages) * kRowBytes;
   s.topk = p.topk;
   s.table = p.page_indices + ps;
@@ -148,8 +148,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   a.q_bh = s.q_bh;
   a.kvb = reinterpret_cast<const char*>(p.kv) + (int64_t)h * kRowBytes;
   a.row_bytes = p.num_kv_heads * kRowBytes;
-  a.page_bytes = 2 * kPageSize * a.row_bytes;
+  a.page_bytes = 2 * p.page_size * a.row_bytes;
   a.span = a.page_bytes - h * kRowBytes;
+  a.page_size = p.page_size;
   a.num_pages = p.num_pages;
   a.G = G;
   a.scale_log2 = p.scale_log2;
@@ -197,7 +198,7 @@ static int launch_step(const char* fn, const kin_bf16_t* q, const kin_bf16_t* k,
   if (kbar_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: kbar_pages=%d must be >= 1", fn, kbar_pages);
   st = check_fixed_pages(fn, sink_pages, local_tokens);
   if (st) return st;
-  st = check_first_page_offset(fn, first_page_offset);
+  st = check_first_page_offset(fn, first_page_offset, page_size);
   if (st) return st;
   if (first_page_offset > 0 && sink_pages < 1)
     return fail(KIN_ERR_BAD_SHAPE, "%s: first_page_offset=%d needs sink_pages >= 1 (a padded page has no mean key)", fn,
@@ -238,6 +239,7 @@ static int launch_step(const char* fn, const kin_bf16_t* q, const kin_bf16_t* k,
   p.sink_pages = sink_pages;
   p.local_tokens = local_tokens;
   p.first_page_offset = first_page_offset;
+  p.page_size = page_size;
   p.sort_cap = select_sort_cap(topk, kbar_pages);
   // Waves per workgroup: aim for 16 waves per CU (8 with the two-pass kernel for
   // groups above 4, whose registers allow no more) when the lists are few.

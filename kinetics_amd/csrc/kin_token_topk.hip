@@ -149,6 +149,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
   a.p1 = n;
   a.last_len = kPageSize;
   a.first_skip = 0;
+  a.page_size = kPageSize;
   attend_tokens<NG, NW>(a, list, smem, sm_m, sm_l, [&](int g, int d, float o, float lse2) {
     p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_bf16(o);
     if (p.lse && d == 0) p.lse[hq0 + g] = lse2 * kLn2;
@@ -186,6 +187,8 @@ static int launch_token_policy(const char* fn, const kin_bf16_t* q, const kin_bf
   if (!q || !kv_cache || !page_indices || !page_indptr || !last_page_len || !out)
     return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size);
+  if (st) return st;
+  st = check_page_size_16(fn, page_size);
   if (st) return st;
   st = check_first_page_offset(fn, first_page_offset);
   if (st) return st;

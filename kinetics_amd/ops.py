@@ -210,7 +210,8 @@ def sel_list_capacity(topk: int, sink_pages: int = 0, local_tokens: int = 1) -> 
 
 
 def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sel_logical=None,
-                     scores_out=None, sink_pages: int = 0, local_tokens: int = 1, workspace=None) -> None:
+                     scores_out=None, sink_pages: int = 0, local_tokens: int = 1, workspace=None,
+                     page_size: int = PAGE_SIZE) -> None:
     """Score every candidate page with the group-mean query and write the
     top-``topk`` pages plus the last page into ``sel_pages`` / ``sel_count``
     (in place: fixed buffers, as the reference registers with its decode
@@ -222,7 +223,8 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
     LiteSys/litesys/attention/sparsity_utils.py:24-47).  List order: sink pages,
     selected pages by descending score, local pages.  ``workspace`` (uint8,
     ``step_workspace_bytes``; optional) lets few, long sequences spread their
-    scoring over the GPU."""
+    scoring over the GPU.  ``page_size``: tokens per page of the cache the table
+    describes (16, 32 or 64)."""
     _require(q, "q", torch.bfloat16, 3)
     dev = q.device
     batch, num_q_heads, head_dim = q.shape
@@ -252,8 +254,8 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
         _lib.check(
             lib.kin_block_score_topk(
                 _ptr(q), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), int(topk), int(sink_pages),
-                int(local_tokens), _ptr(sel_pages), _ptr(sel_count), _ptr(sel_logical), _ptr(scores_out), batch, num_q_heads, num_kv_heads, head_dim,
-                kbar_pages, sel_stride, _ptr(workspace), workspace.numel() if workspace is not None else 0, _stream(dev),
+                int(local_tokens), _ptr(sel_pages), _ptr(sel_count), _ptr(sel_logical), _ptr(scores_out), batch, num_q_heads,
+                num_kv_heads, head_dim, int(page_size), kbar_pages, sel_stride, _ptr(workspace), workspace.numel() if workspace is not None else 0, _stream(dev),
             )
         )
 
@@ -760,7 +762,8 @@ torch.library.define(
 torch.library.define(
     "kinetics::block_score_topk",
     "(Tensor q, Tensor kbar, Tensor page_indices, Tensor page_indptr, Tensor last_page_len, int topk, "
-    "Tensor(a!) sel_pages, Tensor(b!) sel_count, int sink_pages=0, int local_tokens=1, Tensor(c!)? workspace=None) -> ()",
+    "Tensor(a!) sel_pages, Tensor(b!) sel_count, int sink_pages=0, int local_tokens=1, Tensor(c!)? workspace=None, "
+    "int page_size=16) -> ()",
 )
 torch.library.define(
     "kinetics::sparse_paged_decode",
@@ -840,14 +843,14 @@ def _update_kv_fake(k, v, kv_append_indptr, kv_cache, kv_page_indices, kv_page_i
 
 @torch.library.impl("kinetics::block_score_topk", "cuda")
 def _select_impl(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sink_pages=0,
-                 local_tokens=1, workspace=None):
+                 local_tokens=1, workspace=None, page_size=PAGE_SIZE):
     block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count,
-                     sink_pages=sink_pages, local_tokens=local_tokens, workspace=workspace)
+                     sink_pages=sink_pages, local_tokens=local_tokens, workspace=workspace, page_size=page_size)
 
 
 @torch.library.register_fake("kinetics::block_score_topk")
 def _select_fake(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sink_pages=0,
-                 local_tokens=1, workspace=None):
+                 local_tokens=1, workspace=None, page_size=PAGE_SIZE):
     return None
 
 

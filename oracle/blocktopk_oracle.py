@@ -182,7 +182,7 @@ def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len):
 # ---------------------------------------------------------------------------
 
 
-def split_pages(n_pages, last_len, sink_pages, local_tokens, kbar_pages):
+def split_pages(n_pages, last_len, sink_pages, local_tokens, kbar_pages, page_size=16):
     """(n_sink, n_cand, n_local).  The first ``sink_pages`` pages (never the
     open page) and the pages that hold the newest ``local_tokens`` tokens are
     always attended; the candidates are the whole pages in between.  sink 0 /
@@ -191,16 +191,18 @@ def split_pages(n_pages, last_len, sink_pages, local_tokens, kbar_pages):
     ``local`` is LiteSys/litesys/attention/sparsity_utils.py:31-33:
     ``_n_dynamic = (seq_len - local - sink) // block_size * block_size`` with
     sink = 4, the rest of the tokens being the local part.  Candidates beyond
-    ``kbar_pages`` have no mean key and are dropped."""
+    ``kbar_pages`` have no mean key and are dropped.  ``page_size``: tokens per
+    page (the reference's --page_size, benchmark/blocktopk.py:13)."""
+    ps = int(page_size)
     n_sink = min(sink_pages, n_pages - 1)
-    kv_len = (n_pages - 1) * 16 + min(max(int(last_len), 1), 16)
-    n_cand = max(0, (kv_len - 16 * n_sink - local_tokens) // 16)
+    kv_len = (n_pages - 1) * ps + min(max(int(last_len), 1), ps)
+    n_cand = max(0, (kv_len - ps * n_sink - local_tokens) // ps)
     n_local = n_pages - n_sink - n_cand
     n_cand = max(0, min(n_cand, kbar_pages - n_sink))
     return n_sink, n_cand, n_local
 
 
-def block_scores(q, kbar, page_indptr, last_page_len, sink_pages=0, local_tokens=1):
+def block_scores(q, kbar, page_indptr, last_page_len, sink_pages=0, local_tokens=1, page_size=16):
     """score[b][h][n] = mean_g q[b, h*G+g, :] . kbar[b, h, n_sink + n, :] in
     float64 over the candidate pages.  Returns a list (b) of lists (h) of
     float64 arrays."""
@@ -214,7 +216,7 @@ def block_scores(q, kbar, page_indptr, last_page_len, sink_pages=0, local_tokens
         if n_pages <= 0:
             out.append([np.zeros(0) for _ in range(Hkv)])
             continue
-        n_sink, n_cand, _ = split_pages(n_pages, last_page_len[b], sink_pages, local_tokens, kbar.shape[2])
+        n_sink, n_cand, _ = split_pages(n_pages, last_page_len[b], sink_pages, local_tokens, kbar.shape[2], page_size)
         kb = bf16_to_f32(kbar[b, :, n_sink : n_sink + n_cand]).astype(np.float64)  # [Hkv, n, D]
         per_head = []
         for h in range(Hkv):
@@ -239,12 +241,12 @@ def select_topk(scores: np.ndarray, k: int) -> np.ndarray:
 
 
 def sel_list_capacity(topk, sink_pages=0, local_tokens=1):
-    """Longest list block_score_topk can produce."""
+    """Longest list block_score_topk can produce (for 16-token pages; larger pages need no more)."""
     return topk + sink_pages + 1 + (local_tokens + 14) // 16
 
 
 def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_stride=None, sink_pages=0,
-                     local_tokens=1):
+                     local_tokens=1, page_size=16):
     """Returns (sel_pages [B,Hkv,stride] int32 padded with -1, sel_count [B,Hkv],
     sel_logical list[b][h] of logical page index arrays, scores list[b][h] over
     the candidates).  List order: sink pages, winners (descending score), local
@@ -252,7 +254,7 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
     B = q.shape[0]
     Hkv = kbar.shape[1]
     stride = sel_list_capacity(topk, sink_pages, local_tokens) if sel_stride is None else sel_stride
-    scores = block_scores(q, kbar, page_indptr, last_page_len, sink_pages, local_tokens)
+    scores = block_scores(q, kbar, page_indptr, last_page_len, sink_pages, local_tokens, page_size)
     sel_pages = np.full((B, Hkv, stride), -1, dtype=np.int32)
     sel_count = np.zeros((B, Hkv), dtype=np.int32)
     sel_logical = []
@@ -263,7 +265,7 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
             if len(pages) == 0:
                 row.append(np.zeros(0, dtype=np.int64))
                 continue
-            n_sink, _, n_local = split_pages(len(pages), last_page_len[b], sink_pages, local_tokens, kbar.shape[2])
+            n_sink, _, n_local = split_pages(len(pages), last_page_len[b], sink_pages, local_tokens, kbar.shape[2], page_size)
             idx = n_sink + select_topk(scores[b][h], topk)
             full = np.concatenate([pages[:n_sink], pages[idx], pages[len(pages) - n_local :]])
             sel_pages[b, h, : len(full)] = full
@@ -367,7 +369,8 @@ def decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_le
     dict(out, lse, sel_pages, sel_count, sel_logical, scores)."""
     append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len)
     sel_pages, sel_count, sel_logical, scores = block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk,
-                                                                 sink_pages=sink_pages, local_tokens=local_tokens)
+                                                                 sink_pages=sink_pages, local_tokens=local_tokens,
+                                                                 page_size=kv_cache.shape[2])
     out, lse = sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, sm_scale, first_page_offset)
     return dict(out=out, lse=lse, sel_pages=sel_pages, sel_count=sel_count, sel_logical=sel_logical, scores=scores)
 

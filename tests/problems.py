@@ -60,7 +60,7 @@ def randn_bf16(rng, shape, scale=1.0, offset=None):
 
 def make_problem(seed: int, lengths, num_kv_heads: int = 1, group: int = 4, topk: int = 8,
                  table: str = "random", extra_pages: int = 3, kbar_slack: int = 2,
-                 page_mean_sigma: float = 0.5, build_kbar: bool = True) -> Problem:
+                 page_mean_sigma: float = 0.5, build_kbar: bool = True, page_size: int = PAGE_SIZE) -> Problem:
     """``lengths`` are token counts AFTER the append (>= 1 each; 0 = empty sequence).
 
     table: "random"     physical ids are a seeded permutation of all pages
@@ -70,7 +70,7 @@ def make_problem(seed: int, lengths, num_kv_heads: int = 1, group: int = 4, topk
     rng = np.random.default_rng(seed)
     lengths = np.asarray(lengths, dtype=np.int64)
     B = len(lengths)
-    ps, D = PAGE_SIZE, HEAD_DIM
+    ps, D = page_size, HEAD_DIM
     n_pages = (lengths + ps - 1) // ps
     total = int(n_pages.sum()) + extra_pages
     indptr = np.zeros(B + 1, dtype=np.int32)

@@ -52,7 +52,9 @@ def test_append_argument_errors(lib):
     assert append(lib, P=0) == _lib.KIN_ERR_BAD_SHAPE
     assert append(lib, kp=0) == _lib.KIN_ERR_BAD_SHAPE
     assert append(lib, D=64) == _lib.KIN_ERR_UNSUPPORTED
-    assert append(lib, ps=32) == _lib.KIN_ERR_UNSUPPORTED
+    assert append(lib, ps=24) == _lib.KIN_ERR_UNSUPPORTED
+    assert append(lib, ps=128) == _lib.KIN_ERR_UNSUPPORTED
+    assert append(lib, ps=32, B=0) == _lib.KIN_OK and append(lib, ps=64, B=0) == _lib.KIN_OK
     assert append(lib, kv=A + 2) == _lib.KIN_ERR_MISALIGNED
     assert b"kv_cache" in lib.kin_last_error()
     assert append(lib, B=0) == _lib.KIN_OK  # nothing to do, nothing launched
@@ -72,8 +74,8 @@ def test_ragged_append_argument_errors(lib):
 
 
 def select(lib, q=A, kbar=A, idx=A, ptr=A, last=A, topk=4, sel=A, cnt=A, B=2, Hq=4, Hkv=1, D=128, kp=64, stride=5, sink=0,
-           local=1):
-    return lib.kin_block_score_topk(q, kbar, idx, ptr, last, topk, sink, local, sel, cnt, None, None, B, Hq, Hkv, D, kp,
+           local=1, ps=16):
+    return lib.kin_block_score_topk(q, kbar, idx, ptr, last, topk, sink, local, sel, cnt, None, None, B, Hq, Hkv, D, ps, kp,
                                     stride, None, 0, None)
 
 
@@ -94,7 +96,8 @@ def test_select_argument_errors(lib):
     assert select(lib, topk=4096, stride=4097) == _lib.KIN_ERR_UNSUPPORTED
     assert select(lib, kp=20000) == _lib.KIN_ERR_UNSUPPORTED
     assert select(lib, kbar=A + 8) == _lib.KIN_ERR_MISALIGNED
-    assert select(lib, B=0) == _lib.KIN_OK
+    assert select(lib, ps=48) == _lib.KIN_ERR_UNSUPPORTED
+    assert select(lib, B=0) == _lib.KIN_OK and select(lib, B=0, ps=64) == _lib.KIN_OK
 
 
 def sparse(lib, q=A, kv=A, sel=A, cnt=A, last=A, out=A, ws=None, wsb=0, B=2, Hq=4, Hkv=1, D=128, ps=16, P=8,
@@ -241,7 +244,7 @@ def test_auto_splits_policy(lib):
 
 def test_python_wrapper_maps_status_to_exceptions():
     with pytest.raises(ValueError, match="KIN_ERR_BAD_SHAPE"):
-        _lib.check(_lib.load().kin_block_score_topk(A, A, A, A, A, -1, 0, 1, A, A, None, None, 2, 4, 1, 128, 64, 5, None, 0, None))
+        _lib.check(_lib.load().kin_block_score_topk(A, A, A, A, A, -1, 0, 1, A, A, None, None, 2, 4, 1, 128, 16, 64, 5, None, 0, None))
     with pytest.raises(_lib.KineticsError, match="KIN_ERR_WORKSPACE"):
         _lib.check(sparse(_lib.load(), splits=3))
 

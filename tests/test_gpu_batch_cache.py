@@ -27,7 +27,9 @@ def cfg_small():
 def make_manager(**sparse):
     from kinetics_amd.batch_cache import PagedBatchKVManager
 
-    return PagedBatchKVManager(cfg_small(), max_batch_size=6, max_seq_len=PS * 24, device=DEV, dtype=torch.bfloat16, **sparse)
+    block_policy = "attn_block_topk" in sparse and "attn_stride" not in sparse
+    page = sparse.get("attn_block_size", PS) if block_policy else PS
+    return PagedBatchKVManager(cfg_small(), max_batch_size=6, max_seq_len=page * 24, device=DEV, dtype=torch.bfloat16, **sparse)
 
 
 def test_rejects_what_it_does_not_implement():
@@ -43,12 +45,15 @@ def test_rejects_what_it_does_not_implement():
     with pytest.raises(AssertionError):
         PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_block_topk=2)          # LiteSys: local required
     with pytest.raises(NotImplementedError):
-        PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_block_topk=2, attn_local=4, attn_block_size=32)
+        PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_block_topk=2, attn_local=4, attn_block_size=24)
 
 
 @pytest.mark.parametrize("sparse,fused", [(dict(), None), (dict(attn_block_topk=3, attn_local=16), True),
                                           (dict(attn_block_topk=3, attn_local=16), False),
                                           (dict(attn_block_topk=2, attn_local=21), True),
+                                          (dict(attn_block_topk=2, attn_local=20, attn_block_size=32), True),
+                                          (dict(attn_block_topk=2, attn_local=33, attn_block_size=32), False),
+                                          (dict(attn_block_topk=1, attn_local=7, attn_block_size=64), True),
                                           (dict(attn_local=24), False),
                                           (dict(attn_topk=40, attn_local=10), None),
                                           (dict(attn_block_topk=2, attn_local=9, attn_stride=8), None),
@@ -56,6 +61,7 @@ def test_rejects_what_it_does_not_implement():
 def test_prefill_then_decode_like_litesys(sparse, fused):
     torch.manual_seed(5)
     m = make_manager(**sparse)
+    PS = m.page                   # tokens per page: LiteSys' block size for the block policy, else 16
     if fused is not None:
         m._fused = fused          # both routes of decode(): one launch, or append + select + attend
     L, Hq, Hkv = 2, 4, 2
@@ -66,7 +72,7 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
     token_policy = "attn_topk" in sparse or strided or window_only
     policy = "strided" if strided else ("topk" if token_policy else "block")
     block_size, stride = sparse.get("attn_block_size", 16), sparse.get("attn_stride", 8)
-    pad = 12 if sparse and not token_policy else 0
+    pad = PS - 4 if sparse and not token_policy else 0
     topk_block, local = sparse.get("attn_block_topk", sparse.get("attn_topk", 0)), sparse.get("attn_local")
     gen = torch.Generator().manual_seed(11)
     block_bias = torch.randn(64, Hkv, 1, generator=gen) * 0.5   # separates the block scores well beyond bf16 rounding
@@ -174,7 +180,7 @@ def test_prefill_then_decode_like_litesys(sparse, fused):
                 ref, keep = O.litesys_decode(q[i, :, 0].float().cpu().numpy(), K.numpy(), V.numpy(),
                                              topk_block if is_sparse else None, local, policy=policy,
                                              block_size=block_size, stride=stride)
-                if is_sparse and K.shape[0] > 100:
+                if is_sparse and K.shape[0] > 100 * max(block_size, 16) // 16:
                     assert not keep.all()
                 assert np.all(np.abs(got[i] - ref) <= 2e-2 + 2e-2 * np.abs(ref)), (layer, slot)
 

@@ -393,8 +393,11 @@ def test_properties_at_scale(ops):
 # --------------------------------------------------------------------------- layer objects + custom ops
 
 
+@pytest.mark.parametrize("PS", [16, 32, 64])
 @pytest.mark.parametrize("fused", [False, True])
-def test_layer_objects_follow_the_reference_call_order(ops, fused):
+def test_layer_objects_follow_the_reference_call_order(ops, fused, PS):
+    """The attention objects with the reference constructor's arguments, at each
+    --page_size the kernels support (benchmark/blocktopk.py:13)."""
     from kinetics_amd import BlockTopkPagedAttention, DensePagedAttention
 
     B, prefix, topk = 5, PS * 48, 8
@@ -478,6 +481,95 @@ def test_selection_vs_the_references_bf16_scoring(ops, case):
     assert np.all(diff[same] <= tol[same])
     if (~same).any():
         assert diff[~same].max() <= 0.1
+
+
+@pytest.mark.parametrize("page_size", [32, 64])
+@pytest.mark.parametrize("hkv,group", [(1, 4), (2, 8), (8, 2), (1, 3)])
+def test_pages_of_32_and_64_tokens(ops, page_size, hkv, group):
+    """Every entry point of the page path on caches with 32- and 64-token pages
+    (the reference's --page_size, benchmark/blocktopk.py:13): append and mean keys
+    bit-exact, selection against the oracle, sparse / dense / fused attention within
+    the contract, with and without sink pages, a local window and a padded first page."""
+    ps = page_size
+    lengths = [ps * 37 + 3, ps * 5 + ps, 1, 0, ps, ps * 64 + 17, ps * 9 + ps - 1, 7, ps * 2 + 1]
+    for sink, local, offset in ((0, 1, 0), (1, ps + 5, ps - 4), (2, 3 * ps, 0)):
+        topk = 6
+        pb = P.make_problem(700 + hkv + ps, lengths, num_kv_heads=hkv, group=group, topk=topk, page_size=ps)
+        cap = ops.sel_list_capacity(topk, sink, local)
+        what = f"ps={ps} hkv={hkv} G={group} sink={sink} local={local} offset={offset}"
+        kv_o, kbar_o = pb.kv_cache.copy(), pb.kbar.copy()
+        res = O.decode_step(pb.q, pb.k, pb.v, kv_o, kbar_o, pb.page_indices, pb.page_indptr, pb.last_page_len, topk,
+                            sink_pages=sink, local_tokens=local, first_page_offset=offset)
+        outs = {}
+        for path in ("three", "fused"):
+            g = Gpu(pb)
+            g.sel = torch.full((pb.B, hkv, cap), -7, dtype=torch.int32, device=DEV)
+            ops.check_page_table(g.indices, g.indptr, g.last, ps, pb.num_pages)
+            if path == "fused":
+                out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, topk, sel_pages=g.sel,
+                                                sel_count=g.cnt, sink_pages=sink, local_tokens=local, first_page_offset=offset)
+            else:
+                ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
+                ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, topk, g.sel, g.cnt, sink_pages=sink,
+                                     local_tokens=local, page_size=ps)
+                out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, first_page_offset=offset, num_splits=2)
+            torch.cuda.synchronize()
+            assert np.array_equal(P.from_torch(g.kv), kv_o), f"{what} {path}: cache bytes"
+            assert np.array_equal(P.from_torch(g.kbar), kbar_o), f"{what} {path}: mean keys"
+            assert np.array_equal(g.cnt.cpu().numpy(), res["sel_count"]), f"{what} {path}: list lengths"
+            sel = g.sel.cpu().numpy()
+            for b in range(pb.B):
+                pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+                lookup = {int(p): i for i, p in enumerate(pages)}
+                for h in range(hkv):
+                    c = int(res["sel_count"][b, h])
+                    if c == 0:
+                        continue
+                    n_sink, n_cand, n_local = O.split_pages(len(pages), pb.last_page_len[b], sink, local, pb.kbar.shape[2], ps)
+                    k_eff = min(topk, n_cand)
+                    assert c == n_sink + k_eff + n_local
+                    got_logical = np.array([lookup[int(x)] for x in sel[b, h, n_sink:n_sink + k_eff]]) - n_sink
+                    ok, msg = O.selection_matches(got_logical, res["scores"][b][h], topk)
+                    assert ok, f"{what} {path} b={b} h={h}: {msg}"
+                    assert sel[b, h, :n_sink].tolist() == pages[:n_sink].tolist()
+                    assert sel[b, h, n_sink + k_eff:c].tolist() == pages[len(pages) - n_local:].tolist()
+            want, _ = O.sparse_paged_decode(pb.q, kv_o, sel, res["sel_count"], pb.last_page_len, first_page_offset=offset)
+            assert_out_close(out, want, f"{what} {path}")
+            outs[path] = out
+            # dense over the same cache, one pass and split
+            for splits in (1, 3):
+                dense = ops.dense_paged_decode(g.q, g.kv, g.indices, g.indptr, g.last, pb.max_pages, first_page_offset=offset,
+                                               num_splits=splits)
+                wd, _ = O.dense_paged_decode(pb.q, kv_o, pb.page_indices, pb.page_indptr, pb.last_page_len,
+                                             first_page_offset=offset)
+                assert_out_close(dense, wd, f"{what} dense splits={splits}")
+    # bulk mean keys and the ragged (prefill) append on the larger pages
+    pb = P.make_problem(760 + ps, [ps * 37, ps * 5 + 3, 1, 0, ps, ps * 20 + ps], num_kv_heads=hkv, group=group, build_kbar=False,
+                        page_size=ps)
+    g = Gpu(pb)
+    g.kbar.fill_(float("nan"))
+    ops.build_kbar(g.kv, g.kbar, g.indices, g.indptr, g.last)
+    want = P.from_torch(torch.full_like(g.kbar, float("nan")))
+    O.build_kbar(pb.kv_cache, want, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    assert np.array_equal(P.from_torch(g.kbar), want)
+    rng = np.random.default_rng(ps + hkv)
+    new = np.array([min(int(L), int(rng.integers(0, 3 * ps))) for L in pb.lengths])
+    append_indptr = np.concatenate([[0], np.cumsum(new)]).astype(np.int32)
+    k_new, v_new = P.randn_bf16(rng, (int(new.sum()), hkv, D)), P.randn_bf16(rng, (int(new.sum()), hkv, D))
+    want_kv, want_kbar = pb.kv_cache.copy(), want.copy()
+    O.append_paged_kv_ragged(k_new, v_new, append_indptr, want_kv, want_kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
+    ops.append_paged_kv_ragged(P.to_torch(k_new, DEV), P.to_torch(v_new, DEV), P.int_tensor(append_indptr, DEV), g.kv, g.kbar,
+                               g.indices, g.indptr, g.last)
+    torch.cuda.synchronize()
+    assert np.array_equal(P.from_torch(g.kv), want_kv) and np.array_equal(P.from_torch(g.kbar), want_kbar)
+
+
+def test_token_policies_reject_larger_pages(ops):
+    pb = P.make_problem(790, [100, 40], num_kv_heads=1, group=4, page_size=32)
+    g = Gpu(pb)
+    ws = torch.empty(1 << 16, dtype=torch.uint8, device=DEV)
+    with pytest.raises(ValueError):
+        ops.token_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, 16, pb.max_pages, sink_tokens=4, local_tokens=8, workspace=ws)
 
 
 # --------------------------------------------------------------------------- full benchmark sizes

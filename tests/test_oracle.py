@@ -271,8 +271,10 @@ def _depaged(pb, b, h):
     return K.astype(np.float64), V.astype(np.float64)
 
 
-def test_dense_attention_equals_torch_sdpa():
-    pb = P.make_problem(41, [PS * 6 + 5, PS * 2, 9], num_kv_heads=2, group=4)
+@pytest.mark.parametrize("page_size", [16, 32, 64])
+def test_dense_attention_equals_torch_sdpa(page_size):
+    pb = P.make_problem(41, [PS * 6 + 5, PS * 2, 9], num_kv_heads=2, group=4, page_size=page_size)
+    assert pb.kv_cache.shape[2] == page_size
     out, lse = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len)
     qf = O.bf16_to_f32(pb.q).astype(np.float64)
     for b in range(pb.B):
@@ -285,6 +287,33 @@ def test_dense_attention_equals_torch_sdpa():
             assert np.allclose(out[b, 4 * h : 4 * h + 4], want, rtol=1e-9, atol=1e-9)
             logits = qf[b, 4 * h : 4 * h + 4] @ K.T / math.sqrt(D)
             assert np.allclose(lse[b, 4 * h : 4 * h + 4], logsumexp(logits, axis=1), rtol=1e-12)
+
+
+def test_repaging_leaves_dense_attention_unchanged():
+    """The same token rows stored in 16-, 32- and 64-token pages: dense attention
+    over them is the same function of the tokens, bit for bit in float64 up to
+    summation order."""
+    rng = np.random.default_rng(47)
+    lengths = [257, 64, 5]
+    Hkv, G = 2, 3
+    rows_k = [P.randn_bf16(rng, (L, Hkv, D)) for L in lengths]
+    rows_v = [P.randn_bf16(rng, (L, Hkv, D)) for L in lengths]
+    q = P.randn_bf16(rng, (len(lengths), Hkv * G, D))
+    outs = []
+    for ps in (16, 32, 64):
+        n_pages = [(L + ps - 1) // ps for L in lengths]
+        total = sum(n_pages) + 2
+        perm = rng.permutation(total).astype(np.int32)
+        kv = P.randn_bf16(rng, (total, 2, ps, Hkv, D))
+        indptr = np.concatenate([[0], np.cumsum(n_pages)]).astype(np.int32)
+        for b, L in enumerate(lengths):
+            for t in range(L):
+                pid = perm[indptr[b] + t // ps]
+                kv[pid, 0, t % ps], kv[pid, 1, t % ps] = rows_k[b][t], rows_v[b][t]
+        last = np.array([L - (n - 1) * ps for L, n in zip(lengths, n_pages)], dtype=np.int32)
+        outs.append(O.dense_paged_decode(q, kv, perm[: indptr[-1]], indptr, last))
+    for o, l in outs[1:]:
+        assert np.allclose(o, outs[0][0], rtol=1e-12, atol=1e-14) and np.allclose(l, outs[0][1], rtol=1e-12)
 
 
 def test_sparse_with_every_page_selected_equals_dense():
@@ -349,11 +378,14 @@ def test_attention_permutation_and_split_invariance():
         assert np.allclose(mo, out[0], rtol=1e-12, atol=1e-13) and np.allclose(ml, lse[0], rtol=1e-13)
 
 
-def test_decode_step_equals_masked_dense_formulation():
+@pytest.mark.parametrize("page_size", [16, 32, 64])
+def test_decode_step_equals_masked_dense_formulation(page_size):
     """LiteSys expresses block sparsity as a -inf mask on full-context logits
     (sparsity_utils.py:39-45) followed by softmax and P.V; the gather form must
-    give the same numbers."""
-    pb = P.make_problem(59, [PS * 10 + 5, PS * 7 + 16], num_kv_heads=2, group=2, topk=3)
+    give the same numbers, at every page size (the reference's --page_size,
+    benchmark/blocktopk.py:13)."""
+    PS = page_size
+    pb = P.make_problem(59, [PS * 10 + 5, PS * 7 + PS], num_kv_heads=2, group=2, topk=3, page_size=page_size)
     res = O.decode_step(pb.q, pb.k, pb.v, pb.kv_cache, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
     qf = O.bf16_to_f32(pb.q).astype(np.float64)
     for b in range(pb.B):
@@ -466,26 +498,28 @@ def test_sink_and_local_pages_are_pinned_not_candidates():
     assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
 
 
-def test_split_pages_against_token_level_definition():
+@pytest.mark.parametrize("page_size", [16, 32, 64])
+def test_split_pages_against_token_level_definition(page_size):
     """Brute force: a page is a candidate iff it comes after the sink pages and
     ends at or before the first of the newest ``local_tokens`` tokens."""
-    for kv_len in list(range(1, 200)) + [1000, 1009, 4096]:
+    PS = page_size
+    for kv_len in list(range(1, 300)) + [1000, 1009, 4096]:
         n_pages = (kv_len + PS - 1) // PS
         last = kv_len - (n_pages - 1) * PS
         for sink in (0, 1, 2, 5):
             for local in (1, 2, 15, 16, 17, 18, 33, 100):
-                n_sink, n_cand, n_local = O.split_pages(n_pages, last, sink, local, 10 ** 6)
+                n_sink, n_cand, n_local = O.split_pages(n_pages, last, sink, local, 10 ** 6, PS)
                 want_sink = min(sink, n_pages - 1)
                 cand = [p for p in range(want_sink, n_pages) if (p + 1) * PS <= kv_len - local]
                 assert (n_sink, n_cand) == (want_sink, len(cand)), (kv_len, sink, local)
                 assert cand == list(range(want_sink, want_sink + len(cand)))
                 assert n_sink + n_cand + n_local == n_pages and n_local >= 1
-                assert n_local <= 1 + (local + 14) // PS
+                assert n_local <= 1 + (local + PS - 2) // PS <= 1 + (local + 14) // 16
     # local_tokens = 16 (L - 1) + 1 pins exactly the last L pages whatever the open page holds
     for n_pages in range(1, 12):
         for last in range(1, PS + 1):
             for L in (1, 2, 3):
-                n_sink, n_cand, n_local = O.split_pages(n_pages, last, 0, PS * (L - 1) + 1, 10 ** 6)
+                n_sink, n_cand, n_local = O.split_pages(n_pages, last, 0, PS * (L - 1) + 1, 10 ** 6, PS)
                 assert n_local == min(L, n_pages) and n_cand == n_pages - n_local
     # mean keys exist for the first kbar_pages pages only
     assert O.split_pages(100, 3, 2, 1, 50) == (2, 48, 1)
@@ -512,17 +546,20 @@ def test_litesys_mask_hand_case():
     assert O.litesys_blockwise_topk_mask(np.arange(33.0), 33, 1, local).sum() == 4 + 16 + 13
 
 
-def test_page_lists_with_offset_12_equal_litesys_mask_formulation():
+@pytest.mark.parametrize("page_size", [16, 32, 64])
+def test_page_lists_with_offset_12_equal_litesys_mask_formulation(page_size):
     """The paged formulation (sink_pages=1, local_tokens=local, sequences stored
-    12 slots into their first page) and LiteSys' mask on full logits
+    page_size - 4 slots into their first page: 12 for LiteSys' default blocks of 16) and
+    LiteSys' mask on full logits with block_size = page_size
     (sparsity_utils.py:24-47, batch_cache.py:154-168) are the same function:
-    same kept tokens, same output.  Keys are multiples of 16 so that page means
+    same kept tokens, same output.  Keys are multiples of 64 so that page means
     are exact in bfloat16 and no score is perturbed by rounding."""
     rng = np.random.default_rng(123)
-    Hkv, G, pad = 2, 2, 12
+    PS = page_size
+    Hkv, G, pad = 2, 2, page_size - 4
     for seq_len, topk, local in [(300, 3, 20), (301, 3, 16), (52, 2, 5), (53, 2, 5), (40, 4, 7), (5, 2, 3), (4, 1, 1),
                                  (1, 1, 1), (1000, 10, 64), (999, 10, 1), (131, 1, 100), (307, 5, 33)]:
-        K = (rng.integers(-8, 9, size=(seq_len, Hkv, D)) * 16).astype(np.float32)
+        K = (rng.integers(-1, 2, size=(seq_len, Hkv, D)) * 64).astype(np.float32)
         V = O.bf16_to_f32(P.randn_bf16(rng, (seq_len, Hkv, D)))
         q = P.randn_bf16(rng, (1, Hkv * G, D))
         cache_len = seq_len + pad
@@ -539,9 +576,10 @@ def test_page_lists_with_offset_12_equal_litesys_mask_formulation():
         last = np.array([cache_len - (n_pages - 1) * PS], dtype=np.int32)
         kbar = np.zeros((1, Hkv, n_pages, D), dtype=np.uint16)
         O.build_kbar(kv, kbar, perm, indptr, last)
-        sel, cnt, logical, _ = O.block_score_topk(q, kbar, perm, indptr, last, topk, sink_pages=1, local_tokens=local)
+        sel, cnt, logical, _ = O.block_score_topk(q, kbar, perm, indptr, last, topk, sink_pages=1, local_tokens=local,
+                                                  page_size=PS)
         out, _ = O.sparse_paged_decode(q, kv, sel, cnt, last, first_page_offset=pad)
-        want, keep = O.litesys_decode(O.bf16_to_f32(q[0]), K, V, topk, local)
+        want, keep = O.litesys_decode(O.bf16_to_f32(q[0]), K, V, topk, local, block_size=PS)
         lookup = {int(p): i for i, p in enumerate(perm)}
         for h in range(Hkv):
             got_keep = np.zeros(n_pages * PS, dtype=bool)
