@@ -78,12 +78,13 @@ def algorithmic_bytes(lengths, Hkv, G, topk, PS=PS):
     return dict(step=step, attention=attn, score_select=score, dense=dense, per_seq=step / max(1, len(lengths)))
 
 
-def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2, ragged=False, kv_alloc=None, PS=PS):
+def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2, ragged=False, kv_alloc=None, PS=PS, dtype=None):
     """Paged cache, K ~ N(0,1) + per-page mean offset N(0,0.5), V ~ N(0,1); kbar =
     true page means.  Uniform workloads use the reference layout (page id =
     p*B + b, max_len = ctx+512, every context ``ctx`` tokens + the appended one).
     Ragged ones draw contexts uniformly from [1024, ctx] (seed 3); even
     sequences own contiguous page runs, odd ones pages from a shuffled free list."""
+    dtype = dtype or torch.bfloat16
     n_full = ctx // PS
     max_pages = (ctx + 512) // PS
     gen = torch.Generator(device=device).manual_seed(seed)
@@ -113,14 +114,14 @@ def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2, ragged=False, 
         num_pages = max_pages * B
         lengths = [ctx + 1] * B
     kv_shape = (num_pages, 2, PS, Hkv, D)
-    kv = kv_alloc(kv_shape) if kv_alloc else torch.empty(kv_shape, dtype=torch.bfloat16, device=device)
+    kv = kv_alloc(kv_shape) if kv_alloc else torch.empty(kv_shape, dtype=dtype, device=device)
     chunk = max(1, (1 << 28) // (2 * PS * Hkv * D))
     for s in range(0, num_pages, chunk):
         e = min(num_pages, s + chunk)
         x = torch.randn(e - s, 2, PS, Hkv, D, generator=gen, device=device, dtype=torch.float32)
         mu = torch.randn(e - s, 1, 1, Hkv, 1, generator=gen, device=device, dtype=torch.float32) * 0.5
         x[:, 0:1] += mu
-        kv[s:e] = x.to(torch.bfloat16)
+        kv[s:e] = x.to(dtype)
         del x, mu
     if ragged:
         indices = torch.from_numpy(ids.astype("int32")).to(device)
@@ -137,13 +138,13 @@ def build_state(torch, ops, B, ctx, Hkv, G, topk, device, seed=2, ragged=False, 
         indptr=indptr,
         last=last,
         lengths=[int(x) for x in lengths],
-        kbar=torch.zeros(B, Hkv, max_pages, D, dtype=torch.bfloat16, device=device),
+        kbar=torch.zeros(B, Hkv, max_pages, D, dtype=dtype, device=device),
         sel=torch.full((B, Hkv, topk + 1), -1, dtype=torch.int32, device=device),
         cnt=torch.zeros(B, Hkv, dtype=torch.int32, device=device),
-        q=torch.randn(B, Hkv * G, D, generator=gen, device=device, dtype=torch.float32).to(torch.bfloat16),
-        k=torch.randn(B, Hkv, D, generator=gen, device=device, dtype=torch.float32).to(torch.bfloat16),
-        v=torch.randn(B, Hkv, D, generator=gen, device=device, dtype=torch.float32).to(torch.bfloat16),
-        out=torch.empty(B, Hkv * G, D, dtype=torch.bfloat16, device=device),
+        q=torch.randn(B, Hkv * G, D, generator=gen, device=device, dtype=torch.float32).to(dtype),
+        k=torch.randn(B, Hkv, D, generator=gen, device=device, dtype=torch.float32).to(dtype),
+        v=torch.randn(B, Hkv, D, generator=gen, device=device, dtype=torch.float32).to(dtype),
+        out=torch.empty(B, Hkv * G, D, dtype=dtype, device=device),
         n_full=n_full, max_pages=max_pages, num_pages=num_pages,
     )
     st["page_size"] = PS
@@ -459,6 +460,9 @@ def main():
     ap.add_argument("--page_size", type=int, default=16, choices=[16, 32, 64],
                     help="tokens per page of the cache (any workload; the reference's flag, benchmark/blocktopk.py:13)")
     ap.add_argument("--world_size", type=int, default=8)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float16"],
+                    help="element type of q, the cache, the mean keys and the output (the reference's flag, "
+                         "benchmark/blocktopk.py:18)")
     ap.add_argument("--placement-rounds", type=int, default=0,
                     help="instead of the benchmark: build, time (step and dense) and free the workload's cache this many "
                          "times in one process, with dummy allocations of varying size in front of it, to see how much "
@@ -500,7 +504,8 @@ def main():
         return
     t_setup = time.perf_counter()
     page = args.page_size
-    st = build_state(torch, ops, B, ctx, Hkv, G, topk, device, ragged=args.workload in RAGGED, PS=page)
+    elem = torch.float16 if args.dtype == "float16" else torch.bfloat16
+    st = build_state(torch, ops, B, ctx, Hkv, G, topk, device, ragged=args.workload in RAGGED, PS=page, dtype=elem)
     torch.cuda.synchronize()
     print(f"[bench] {args.workload}: B={B} ctx={ctx} H_kv={Hkv} G={G} topk={topk}, "
           f"KV {st['kv'].numel() * 2 / 1e9:.1f} GB resident, setup {time.perf_counter() - t_setup:.1f}s", file=sys.stderr)
@@ -538,7 +543,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": "bf16" if elem is torch.bfloat16 else "f16",
         "data": "synthetic",
         "config": {"workload": args.workload, "description": desc, "batch": B, "ctx": ctx, "num_kv_heads": Hkv,
                    "num_q_heads": Hkv * G, "head_dim": D, "page_size": page, "topk_pages": topk,
@@ -579,8 +584,8 @@ def main():
         result["dense_baseline"] = {"value": B / td, "unit": "tokens/s", "ms_per_step": td * 1e3, "steps": nd,
                                     "achieved_gbs": dense_bytes / td / 1e9, "frac": dense_bytes / td / 1e9 / HBM_PEAK_GBS,
                                     "sparse_over_dense": (B * K / elapsed) / (B / td)}
-    side = headline and page == PS and not args.no_side_workloads
-    if (args.token_topk or side) and page == PS:   # the token-granular policies are built for 16-token pages
+    side = headline and page == PS and elem is torch.bfloat16 and not args.no_side_workloads
+    if (args.token_topk or side) and page == PS and elem is torch.bfloat16:   # token-granular policies: 16-token pages, bf16
         result.update(time_token_policies(torch, ops, st, B, Hkv, G, topk, max(3, min(20, K // 5)), traffic_table.get))
     del st
     torch.cuda.empty_cache()

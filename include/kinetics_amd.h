@@ -12,7 +12,8 @@
  * the reference interface each entry point stands in for.
  *
  * Tensor conventions (all device memory, densely packed, row-major):
- *   bf16 tensors are passed as uint16_t* (raw bfloat16 bit patterns).
+ *   bf16 tensors are passed as uint16_t* (raw bfloat16 bit patterns); the
+ *   *_f16 entry points near the end take IEEE binary16 bits the same way.
  *   q, out        [batch, num_q_heads, head_dim]                    bf16
  *   k, v          [batch, num_kv_heads, head_dim]                   bf16
  *   kv_cache      [num_pages, 2, page_size, num_kv_heads, head_dim] bf16
@@ -54,6 +55,7 @@ extern "C" {
 #endif
 
 typedef uint16_t kin_bf16_t;  /* raw bfloat16 bits */
+typedef uint16_t kin_f16_t;   /* raw IEEE binary16 bits */
 typedef void* kin_stream_t;   /* a hipStream_t */
 
 enum kin_status {
@@ -510,6 +512,82 @@ int kin_check_page_table(const int32_t* page_indices, const int32_t* page_indptr
                          const int32_t* last_page_len, int batch, int page_size,
                          int64_t num_pages, int64_t nnz, int32_t* scratch,
                          kin_stream_t stream);
+
+/* ---- float16 caches ----------------------------------------------------------
+ * The reference benchmark takes --dtype (benchmark/blocktopk.py:18,
+ * benchmark/dense.py) and allocates q, kv_cache and compressed_key_cache in it;
+ * LiteSys' manager takes a dtype too (LiteSys/litesys/attention/batch_cache.py:21).
+ * The entry points above are the bfloat16 path; each of the following is its
+ * float16 twin: same arguments, same meaning, same fp32 accumulation, with q, k,
+ * v, kv_cache, kbar and out holding IEEE binary16 (round-to-nearest-even on
+ * every store; the mean key is the fp32 sum times 1/page_size rounded to
+ * binary16).  The token-granular policies, the entry point with built-in scratch
+ * and the row-wise layer kernels are bfloat16 only.
+ */
+int kin_append_paged_kv_f16(const kin_f16_t* k, const kin_f16_t* v,
+                            kin_f16_t* kv_cache, kin_f16_t* kbar,
+                            const int32_t* page_indices, const int32_t* page_indptr,
+                            const int32_t* last_page_len,
+                            int batch, int num_kv_heads, int head_dim, int page_size,
+                            int64_t num_pages, int kbar_pages, kin_stream_t stream);
+
+int kin_build_kbar_f16(const kin_f16_t* kv_cache, kin_f16_t* kbar,
+                       const int32_t* page_indices, const int32_t* page_indptr,
+                       const int32_t* last_page_len,
+                       int batch, int num_kv_heads, int head_dim, int page_size,
+                       int64_t num_pages, int kbar_pages, kin_stream_t stream);
+
+int kin_append_paged_kv_ragged_f16(const kin_f16_t* k, const kin_f16_t* v,
+                                   const int32_t* append_indptr,
+                                   kin_f16_t* kv_cache, kin_f16_t* kbar,
+                                   const int32_t* page_indices, const int32_t* page_indptr,
+                                   const int32_t* last_page_len,
+                                   int batch, int64_t nnz, int max_append_len,
+                                   int num_kv_heads, int head_dim, int page_size,
+                                   int64_t num_pages, int kbar_pages, kin_stream_t stream);
+
+int kin_block_score_topk_f16(const kin_f16_t* q, const kin_f16_t* kbar,
+                             const int32_t* page_indices, const int32_t* page_indptr,
+                             const int32_t* last_page_len,
+                             int topk, int sink_pages, int local_tokens,
+                             int32_t* sel_pages, int32_t* sel_count,
+                             int32_t* sel_logical, float* scores_out,
+                             int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
+                             int kbar_pages, int sel_stride,
+                             void* workspace, size_t workspace_bytes, kin_stream_t stream);
+
+int kin_sparse_paged_decode_f16(const kin_f16_t* q, const kin_f16_t* kv_cache,
+                                const int32_t* sel_pages, const int32_t* sel_count,
+                                const int32_t* last_page_len,
+                                kin_f16_t* out, float* lse,
+                                void* workspace, size_t workspace_bytes,
+                                int batch, int num_q_heads, int num_kv_heads,
+                                int head_dim, int page_size, int64_t num_pages,
+                                int sel_stride, int first_page_offset,
+                                float sm_scale, int num_splits, kin_stream_t stream);
+
+int kin_dense_paged_decode_f16(const kin_f16_t* q, const kin_f16_t* kv_cache,
+                               const int32_t* page_indices, const int32_t* page_indptr,
+                               const int32_t* last_page_len,
+                               kin_f16_t* out, float* lse,
+                               void* workspace, size_t workspace_bytes,
+                               int batch, int num_q_heads, int num_kv_heads,
+                               int head_dim, int page_size, int64_t num_pages,
+                               int max_pages_per_seq, int first_page_offset,
+                               float sm_scale, int num_splits, kin_stream_t stream);
+
+int kin_blocktopk_decode_step_f16(const kin_f16_t* q, const kin_f16_t* k, const kin_f16_t* v,
+                                  kin_f16_t* kv_cache, kin_f16_t* kbar,
+                                  const int32_t* page_indices, const int32_t* page_indptr,
+                                  const int32_t* last_page_len, int topk,
+                                  int sink_pages, int local_tokens,
+                                  int32_t* sel_pages, int32_t* sel_count,
+                                  kin_f16_t* out, float* lse,
+                                  int batch, int num_q_heads, int num_kv_heads,
+                                  int head_dim, int page_size, int64_t num_pages,
+                                  int kbar_pages, int sel_stride, int first_page_offset,
+                                  float sm_scale, void* workspace, size_t workspace_bytes,
+                                  kin_stream_t stream);
 
 /* ---- row-wise layer kernels around the attention path ---------------------
  * The reference's decoder layer (benchmark/blocktopk_decoder.py:187-240) calls

@@ -90,6 +90,11 @@ SIGNATURES = {
     "kin_gated_act": (c_int, [_P, _P, _P, c_int64, c_int, c_int64, c_int64, c_int, _P]),
 }
 
+# the float16 twins have the signatures of their bfloat16 originals
+for _name in ("kin_append_paged_kv", "kin_build_kbar", "kin_append_paged_kv_ragged", "kin_block_score_topk",
+              "kin_sparse_paged_decode", "kin_dense_paged_decode", "kin_blocktopk_decode_step"):
+    SIGNATURES[_name + "_f16"] = SIGNATURES[_name]
+
 _lib = None
 
 

@@ -61,8 +61,11 @@ _UNSUPPORTED = ("attn_random_select", "attn_random_nsample")
 
 class PagedBatchKVManager:
     def __init__(self, config, max_batch_size: int, max_seq_len: int, device, dtype, **kwargs):
-        if dtype != torch.bfloat16:
-            raise ValueError("the HIP kernels are built for bfloat16")
+        if dtype not in (torch.bfloat16, torch.float16):
+            raise ValueError("the HIP kernels are built for bfloat16 and float16")
+        if dtype is torch.float16 and (kwargs.get("attn_topk") is not None or kwargs.get("attn_stride") is not None
+                                       or (kwargs.get("attn_local") is not None and kwargs.get("attn_block_topk") is None)):
+            raise NotImplementedError("the token-granular policies are built for bfloat16 only")
         self.config = config
         self.max_length = max_seq_len
         self.device = torch.device(device)

@@ -31,8 +31,8 @@ class BlockTopkPagedAttention:
                  max_len: int, page_size: int, topk_page: int, device="cuda", dtype=torch.bfloat16,
                  init_cache: str = "randn", seed: int = 0, fused: Optional[bool] = None, sink_pages: int = 0,
                  local_tokens: int = 1):
-        if dtype != torch.bfloat16:
-            raise ValueError("the HIP kernels are built for bfloat16")
+        if dtype not in (torch.bfloat16, torch.float16):
+            raise ValueError("the HIP kernels are built for bfloat16 and float16")
         if prefix_len % page_size != 0:
             raise ValueError("prefix_len must be a multiple of page_size (as in the reference benchmark)")
         if max_len < prefix_len + page_size:

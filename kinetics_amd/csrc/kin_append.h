@@ -10,16 +10,17 @@ namespace kin {
 // Mean of the page_size key rows of one page for one head, for this lane's
 // two columns.  `krow` points at slot 0 of the page's K plane for that head
 // (in dwords); `row_stride` is in dwords.  Sum order is slot 0, 1, ..., page_size-1.
+template <bool F16 = false>
 __device__ __forceinline__ uint32_t page_mean_dword(const uint32_t* krow, int row_stride, int lane, int page_size) {
   float s0 = 0.f, s1 = 0.f;
 #pragma unroll 16
   for (int t = 0; t < page_size; ++t) {
     const uint32_t w = krow[(int64_t)t * row_stride + lane];
-    s0 += bf16_lo(w);
-    s1 += bf16_hi(w);
+    s0 += elem_lo<F16>(w);
+    s1 += elem_hi<F16>(w);
   }
   const float inv = 1.0f / (float)page_size;
-  return f32_to_bf16(s0 * inv) | (f32_to_bf16(s1 * inv) << 16);
+  return f32_to_elem<F16>(s0 * inv) | (f32_to_elem<F16>(s1 * inv) << 16);
 }
 
 // The same mean for 8 columns at once: `kplane16` points at this lane's 16 bytes of
@@ -27,6 +28,7 @@ __device__ __forceinline__ uint32_t page_mean_dword(const uint32_t* krow, int ro
 // distance between token rows in 16-byte units.  16 loads are in flight
 // together (one tile of the page at a time); the sums run in slot order like
 // page_mean_dword(), so both give the same bits.
+template <bool F16 = false>
 __device__ __forceinline__ u32x4 page_mean_16B(const u32x4* kplane16, int row_stride16, int page_size) {
   float acc[8];
 #pragma unroll
@@ -37,18 +39,18 @@ __device__ __forceinline__ u32x4 page_mean_16B(const u32x4* kplane16, int row_st
     for (int t = 0; t < kPageSize; ++t) x[t] = __builtin_nontemporal_load(kplane16 + (int64_t)(t0 + t) * row_stride16);
 #pragma unroll
     for (int t = 0; t < kPageSize; ++t) {
-      acc[0] += bf16_lo(x[t].x); acc[1] += bf16_hi(x[t].x);
-      acc[2] += bf16_lo(x[t].y); acc[3] += bf16_hi(x[t].y);
-      acc[4] += bf16_lo(x[t].z); acc[5] += bf16_hi(x[t].z);
-      acc[6] += bf16_lo(x[t].w); acc[7] += bf16_hi(x[t].w);
+      acc[0] += elem_lo<F16>(x[t].x); acc[1] += elem_hi<F16>(x[t].x);
+      acc[2] += elem_lo<F16>(x[t].y); acc[3] += elem_hi<F16>(x[t].y);
+      acc[4] += elem_lo<F16>(x[t].z); acc[5] += elem_hi<F16>(x[t].z);
+      acc[6] += elem_lo<F16>(x[t].w); acc[7] += elem_hi<F16>(x[t].w);
     }
   }
   const float inv = 1.0f / (float)page_size;
   u32x4 m;
-  m.x = f32_to_bf16(acc[0] * inv) | (f32_to_bf16(acc[1] * inv) << 16);
-  m.y = f32_to_bf16(acc[2] * inv) | (f32_to_bf16(acc[3] * inv) << 16);
-  m.z = f32_to_bf16(acc[4] * inv) | (f32_to_bf16(acc[5] * inv) << 16);
-  m.w = f32_to_bf16(acc[6] * inv) | (f32_to_bf16(acc[7] * inv) << 16);
+  m.x = f32_to_elem<F16>(acc[0] * inv) | (f32_to_elem<F16>(acc[1] * inv) << 16);
+  m.y = f32_to_elem<F16>(acc[2] * inv) | (f32_to_elem<F16>(acc[3] * inv) << 16);
+  m.z = f32_to_elem<F16>(acc[4] * inv) | (f32_to_elem<F16>(acc[5] * inv) << 16);
+  m.w = f32_to_elem<F16>(acc[6] * inv) | (f32_to_elem<F16>(acc[7] * inv) << 16);
   return m;
 }
 
@@ -61,6 +63,7 @@ __device__ __forceinline__ u32x4 page_mean_16B(const u32x4* kplane16, int row_st
 // read from the cache, the last row is taken from the register, so the result does not
 // depend on store visibility.  Metadata outside its contract would write
 // outside the cache: the row is skipped.
+template <bool F16 = false>
 __device__ __forceinline__ void append_token_row(const uint32_t* k_row, const uint32_t* v_row, uint32_t* kv_cache,
                                                  uint32_t* kbar_page_row, int64_t last_pid, int last_len, int n_pages,
                                                  int kbar_pages, int h, int num_kv_heads, int64_t num_pages, int lane,
@@ -80,13 +83,13 @@ __device__ __forceinline__ void append_token_row(const uint32_t* k_row, const ui
 #pragma unroll 15
     for (int t = 0; t < page_size - 1; ++t) {
       const uint32_t w = kplane[(int64_t)t * row_stride + lane];
-      s0 += bf16_lo(w);
-      s1 += bf16_hi(w);
+      s0 += elem_lo<F16>(w);
+      s1 += elem_hi<F16>(w);
     }
-    s0 += bf16_lo(kw);
-    s1 += bf16_hi(kw);
+    s0 += elem_lo<F16>(kw);
+    s1 += elem_hi<F16>(kw);
     const float inv = 1.0f / (float)page_size;
-    kbar_page_row[lane] = f32_to_bf16(s0 * inv) | (f32_to_bf16(s1 * inv) << 16);
+    kbar_page_row[lane] = f32_to_elem<F16>(s0 * inv) | (f32_to_elem<F16>(s1 * inv) << 16);
   }
 }
 

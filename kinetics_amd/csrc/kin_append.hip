@@ -18,6 +18,7 @@ struct AppendParams {
 };
 
 // grid = ceil(batch*Hkv / 4) blocks of 256 threads; one wave per (sequence, head).
+template <bool F16>
 __global__ __launch_bounds__(256) void append_kernel(AppendParams p) {
   const int lane = threadIdx.x & 63;
   const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -28,7 +29,7 @@ __global__ __launch_bounds__(256) void append_kernel(AppendParams p) {
   if (n_pages <= 0) return;
   uint32_t* kbar_row = p.kbar ? p.kbar + kbar_row_index(b, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2)
                               : nullptr;
-  append_token_row(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2), p.kv_cache, kbar_row,
+  append_token_row<F16>(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2), p.kv_cache, kbar_row,
                    p.page_indices[e - 1], p.last_page_len[b], n_pages, p.kbar_pages, h, p.num_kv_heads, p.num_pages, lane,
                    p.page_size);
 }
@@ -38,6 +39,7 @@ __global__ __launch_bounds__(256) void append_kernel(AppendParams p) {
 // owns 8 columns of all 16 key rows: 16 loads of 16 B in flight per lane, and the
 // same fp32 sum in slot order that page_mean_dword() makes, so a page's mean key
 // is bit-identical whether it is built here or by the append that fills the page.
+template <bool F16>
 __global__ __launch_bounds__(256) void build_kbar_kernel(AppendParams p, int page_blocks) {
   const int sub = threadIdx.x >> 4, c16 = threadIdx.x & 15;
   const int item = blockIdx.x / page_blocks;
@@ -53,7 +55,7 @@ __global__ __launch_bounds__(256) void build_kbar_kernel(AppendParams p, int pag
   const int row_stride = p.num_kv_heads * (kHeadDim / 2);  // dwords per token row
   const int64_t page_dwords = 2LL * p.page_size * row_stride;
   const u32x4* kplane = reinterpret_cast<const u32x4*>(p.kv_cache + pid * page_dwords + h * (kHeadDim / 2)) + c16;
-  const u32x4 m = page_mean_16B(kplane, row_stride / 4, p.page_size);
+  const u32x4 m = page_mean_16B<F16>(kplane, row_stride / 4, p.page_size);
   reinterpret_cast<u32x4*>(p.kbar + kbar_row_index(b, h, page, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2))[c16] = m;
 }
 
@@ -156,6 +158,7 @@ __global__ __launch_bounds__(256) void append_ragged_kernel(RaggedAppendParams p
 // (so its cost follows the number of appended rows, whatever their split over the
 // sequences); 16 lanes per (completed page, head).  Runs after
 // append_ragged_kernel on the same stream.
+template <bool F16>
 __global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p) {
   __shared__ int64_t src16[kRaggedRows];  // K plane of the page a row completed, in 16-byte units; -1: none
   __shared__ int64_t dst16[kRaggedRows];  // its mean-key row for head 0, in 16-byte units (head h: + h * kbar_pages rows)
@@ -197,7 +200,7 @@ __global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p)
     const int r = pair / p.num_kv_heads, h = pair - r * p.num_kv_heads;
     const int64_t src = src16[r];
     if (src < 0) continue;
-    const u32x4 m = page_mean_16B(cache + src + h * (kHeadDim / 8) + c16, cpr, P);
+    const u32x4 m = page_mean_16B<F16>(cache + src + h * (kHeadDim / 8) + c16, cpr, P);
     kbar[dst16[r] + (int64_t)h * p.kbar_pages * (kHeadDim / 8) + c16] = m;
   }
 }
@@ -220,12 +223,11 @@ static int check_append_args(const char* fn, const void* kv_cache, const void* p
 
 extern "C" {
 
-int kin_append_paged_kv(const kin_bf16_t* k, const kin_bf16_t* v, kin_bf16_t* kv_cache, kin_bf16_t* kbar,
-                        const int32_t* page_indices, const int32_t* page_indptr, const int32_t* last_page_len,
-                        int batch, int num_kv_heads, int head_dim, int page_size, int64_t num_pages,
-                        int kbar_pages, kin_stream_t stream) {
+static int append_impl(const char* fn, bool f16, const uint16_t* k, const uint16_t* v, uint16_t* kv_cache, uint16_t* kbar,
+                       const int32_t* page_indices, const int32_t* page_indptr, const int32_t* last_page_len,
+                       int batch, int num_kv_heads, int head_dim, int page_size, int64_t num_pages,
+                       int kbar_pages, kin_stream_t stream) {
   using namespace kin;
-  const char* fn = "kin_append_paged_kv";
   if (!k || !v) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_append_args(fn, kv_cache, page_indices, page_indptr, last_page_len, batch, num_kv_heads,
                              head_dim, page_size, num_pages, kbar_pages, kbar != nullptr);
@@ -248,15 +250,31 @@ int kin_append_paged_kv(const kin_bf16_t* k, const kin_bf16_t* v, kin_bf16_t* kv
   p.num_pages = num_pages;
   const int64_t items = (int64_t)batch * num_kv_heads;
   const unsigned blocks = (unsigned)((items + 3) / 4);
-  append_kernel<<<blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(p);
+  if (f16) append_kernel<true><<<blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(p);
+  else append_kernel<false><<<blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(p);
   return check_hip(hipGetLastError(), "append_kernel launch");
 }
 
-int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
-                   const int32_t* page_indptr, const int32_t* last_page_len, int batch, int num_kv_heads,
-                   int head_dim, int page_size, int64_t num_pages, int kbar_pages, kin_stream_t stream) {
+int kin_append_paged_kv(const kin_bf16_t* k, const kin_bf16_t* v, kin_bf16_t* kv_cache, kin_bf16_t* kbar,
+                        const int32_t* page_indices, const int32_t* page_indptr, const int32_t* last_page_len,
+                        int batch, int num_kv_heads, int head_dim, int page_size, int64_t num_pages,
+                        int kbar_pages, kin_stream_t stream) {
+  return append_impl("kin_append_paged_kv", false, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, batch,
+                     num_kv_heads, head_dim, page_size, num_pages, kbar_pages, stream);
+}
+
+int kin_append_paged_kv_f16(const kin_f16_t* k, const kin_f16_t* v, kin_f16_t* kv_cache, kin_f16_t* kbar,
+                            const int32_t* page_indices, const int32_t* page_indptr, const int32_t* last_page_len,
+                            int batch, int num_kv_heads, int head_dim, int page_size, int64_t num_pages,
+                            int kbar_pages, kin_stream_t stream) {
+  return append_impl("kin_append_paged_kv_f16", true, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, batch,
+                     num_kv_heads, head_dim, page_size, num_pages, kbar_pages, stream);
+}
+
+static int build_kbar_impl(const char* fn, bool f16, const uint16_t* kv_cache, uint16_t* kbar, const int32_t* page_indices,
+                           const int32_t* page_indptr, const int32_t* last_page_len, int batch, int num_kv_heads,
+                           int head_dim, int page_size, int64_t num_pages, int kbar_pages, kin_stream_t stream) {
   using namespace kin;
-  const char* fn = "kin_build_kbar";
   if (!kbar) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_append_args(fn, kv_cache, page_indices, page_indptr, last_page_len, batch, num_kv_heads,
                              head_dim, page_size, num_pages, kbar_pages, true);
@@ -280,17 +298,31 @@ int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* 
   p.kbar_pages = kbar_pages;
   p.page_size = page_size;
   p.num_pages = num_pages;
-  build_kbar_kernel<<<(unsigned)(items * page_blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(p, page_blocks);
+  if (f16) build_kbar_kernel<true><<<(unsigned)(items * page_blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(p, page_blocks);
+  else build_kbar_kernel<false><<<(unsigned)(items * page_blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(p, page_blocks);
   return check_hip(hipGetLastError(), "build_kbar_kernel launch");
 }
 
-int kin_append_paged_kv_ragged(const kin_bf16_t* k, const kin_bf16_t* v, const int32_t* append_indptr,
-                               kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
-                               const int32_t* page_indptr, const int32_t* last_page_len, int batch, int64_t nnz,
-                               int max_append_len, int num_kv_heads, int head_dim, int page_size,
-                               int64_t num_pages, int kbar_pages, kin_stream_t stream) {
+int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
+                   const int32_t* page_indptr, const int32_t* last_page_len, int batch, int num_kv_heads,
+                   int head_dim, int page_size, int64_t num_pages, int kbar_pages, kin_stream_t stream) {
+  return build_kbar_impl("kin_build_kbar", false, kv_cache, kbar, page_indices, page_indptr, last_page_len, batch, num_kv_heads,
+                         head_dim, page_size, num_pages, kbar_pages, stream);
+}
+
+int kin_build_kbar_f16(const kin_f16_t* kv_cache, kin_f16_t* kbar, const int32_t* page_indices,
+                       const int32_t* page_indptr, const int32_t* last_page_len, int batch, int num_kv_heads,
+                       int head_dim, int page_size, int64_t num_pages, int kbar_pages, kin_stream_t stream) {
+  return build_kbar_impl("kin_build_kbar_f16", true, kv_cache, kbar, page_indices, page_indptr, last_page_len, batch,
+                         num_kv_heads, head_dim, page_size, num_pages, kbar_pages, stream);
+}
+
+static int append_ragged_impl(const char* fn, bool f16, const uint16_t* k, const uint16_t* v, const int32_t* append_indptr,
+                              uint16_t* kv_cache, uint16_t* kbar, const int32_t* page_indices,
+                              const int32_t* page_indptr, const int32_t* last_page_len, int batch, int64_t nnz,
+                              int max_append_len, int num_kv_heads, int head_dim, int page_size,
+                              int64_t num_pages, int kbar_pages, kin_stream_t stream) {
   using namespace kin;
-  const char* fn = "kin_append_paged_kv_ragged";
   if (!k || !v || !append_indptr) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_append_args(fn, kv_cache, page_indices, page_indptr, last_page_len, batch, num_kv_heads,
                              head_dim, page_size, num_pages, kbar_pages, kbar != nullptr);
@@ -322,8 +354,29 @@ int kin_append_paged_kv_ragged(const kin_bf16_t* k, const kin_bf16_t* v, const i
   append_ragged_kernel<<<(unsigned)blocks, 256, 0, s>>>(p);
   st = check_hip(hipGetLastError(), "append_ragged_kernel launch");
   if (st || !kbar) return st;
-  refresh_kbar_kernel<<<(unsigned)blocks, 256, 0, s>>>(p);
+  if (f16) refresh_kbar_kernel<true><<<(unsigned)blocks, 256, 0, s>>>(p);
+  else refresh_kbar_kernel<false><<<(unsigned)blocks, 256, 0, s>>>(p);
   return check_hip(hipGetLastError(), "refresh_kbar_kernel launch");
+}
+
+int kin_append_paged_kv_ragged(const kin_bf16_t* k, const kin_bf16_t* v, const int32_t* append_indptr,
+                               kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
+                               const int32_t* page_indptr, const int32_t* last_page_len, int batch, int64_t nnz,
+                               int max_append_len, int num_kv_heads, int head_dim, int page_size,
+                               int64_t num_pages, int kbar_pages, kin_stream_t stream) {
+  return append_ragged_impl("kin_append_paged_kv_ragged", false, k, v, append_indptr, kv_cache, kbar, page_indices, page_indptr,
+                            last_page_len, batch, nnz, max_append_len, num_kv_heads, head_dim, page_size, num_pages,
+                            kbar_pages, stream);
+}
+
+int kin_append_paged_kv_ragged_f16(const kin_f16_t* k, const kin_f16_t* v, const int32_t* append_indptr,
+                                   kin_f16_t* kv_cache, kin_f16_t* kbar, const int32_t* page_indices,
+                                   const int32_t* page_indptr, const int32_t* last_page_len, int batch, int64_t nnz,
+                                   int max_append_len, int num_kv_heads, int head_dim, int page_size,
+                                   int64_t num_pages, int kbar_pages, kin_stream_t stream) {
+  return append_ragged_impl("kin_append_paged_kv_ragged_f16", true, k, v, append_indptr, kv_cache, kbar, page_indices,
+                            page_indptr, last_page_len, batch, nnz, max_append_len, num_kv_heads, head_dim, page_size,
+                            num_pages, kbar_pages, stream);
 }
 
 }  // extern "C"

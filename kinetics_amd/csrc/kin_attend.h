@@ -14,7 +14,7 @@
 //   K  4 x 16-byte LDS-direct buffer loads, each instruction covering 4 whole
 //      256-byte rows, into a wave-private, XOR-swizzled staging area (two
 //      stages); read back in the MFMA operand layout "row = l%16".
-//   S  = K q^T with 4 x v_mfma_f32_16x16x32_bf16; the 16 output columns hold
+//   S  = K q^T with 4 x v_mfma_f32_16x16x32_bf16 (_f16 for half caches); the 16 output columns hold
 //      the (<=4) query heads of the group replicated 4x, so lane l ends up with
 //      S[g = l%4][t = 4*kg + r] (r = 0..3) and no cross-lane traffic is needed.
 //   softmax state (m, l) is kept per (row group, head): 4 independent partial
@@ -44,8 +44,8 @@ constexpr float kLn2 = 0.6931471805599453f;
 // ka: this lane's 4 K chunks in MFMA A layout.  Leaves the probabilities of
 // this lane's 4 tokens in pr.  Requires 0 <= first_token <= 16 and
 // 0 <= valid_tokens <= 16 (an empty range masks the whole page).
-template <int NG>
-__device__ __forceinline__ void page_scores(const uint4 (&ka)[4], const bf16x8 (&qB)[NG][4], float (&m_run)[NG],
+template <int NG, bool F16 = false>
+__device__ __forceinline__ void page_scores(const uint4 (&ka)[4], const uint4 (&qB)[NG][4], float (&m_run)[NG],
                                             float (&l_run)[NG], floatx4 (&O)[NG][8], float (&pr)[NG][4],
                                             float scale_log2, int first_token, int valid_tokens, int kg) {
   floatx4 S[NG];
@@ -53,10 +53,8 @@ __device__ __forceinline__ void page_scores(const uint4 (&ka)[4], const bf16x8 (
   for (int half = 0; half < NG; ++half) S[half] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
-    const bf16x8 a = __builtin_bit_cast(bf16x8, ka[c]);
 #pragma unroll
-    for (int half = 0; half < NG; ++half)
-      S[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qB[half][c], S[half], 0, 0, 0);
+    for (int half = 0; half < NG; ++half) S[half] = mfma_16x16x32<F16>(ka[c], qB[half][c], S[half]);
   }
 #pragma unroll
   for (int half = 0; half < NG; ++half) {
@@ -89,13 +87,13 @@ __device__ __forceinline__ void page_scores(const uint4 (&ka)[4], const bf16x8 (
 }
 
 // Second half: O += P V.  vr: this lane's 4 V rows (row 4*kg + r).
-template <int NG>
+template <int NG, bool F16 = false>
 __device__ __forceinline__ void page_pv(const u32x4 (&vr)[4], const float (&pr)[NG][4], floatx4 (&O)[NG][8]) {
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const u32x4 vv = vr[r];
-    const float vf[8] = {bf16_lo(vv.x), bf16_hi(vv.x), bf16_lo(vv.y), bf16_hi(vv.y),
-                         bf16_lo(vv.z), bf16_hi(vv.z), bf16_lo(vv.w), bf16_hi(vv.w)};
+    const float vf[8] = {elem_lo<F16>(vv.x), elem_hi<F16>(vv.x), elem_lo<F16>(vv.y), elem_hi<F16>(vv.y),
+                         elem_lo<F16>(vv.z), elem_hi<F16>(vv.z), elem_lo<F16>(vv.w), elem_hi<F16>(vv.w)};
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
 #pragma unroll
@@ -227,7 +225,7 @@ __device__ __forceinline__ void attend_finish(float (&m_run)[NG], float (&l_run)
 // lds: attend_lds_bytes(NW, attend_k_stages(NG)), 16-byte aligned; sm_m / sm_l: NW x
 // (4*NG) floats each.
 // Every one of the workgroup's NW*64 threads calls this.
-template <int NG, int NW, typename IdAt, typename Emit>
+template <int NG, int NW, bool F16 = false, typename IdAt, typename Emit>
 __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, unsigned char* lds,
                                             float (*sm_m)[4 * NG], float (*sm_l)[4 * NG], Emit emit) {
   const int tid = threadIdx.x;
@@ -237,14 +235,14 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
   const int n = a.n, p0 = a.p0, p1 = a.p1, last_len = a.last_len;
 
   // Query operands: B[k][j], j = l%16 -> head 4*half + l%4, k-chunk = l/16.
-  bf16x8 qB[NG][4];
+  uint4 qB[NG][4];
 #pragma unroll
   for (int half = 0; half < NG; ++half) {
     const int g = min(4 * half + gq, G - 1);
     const uint16_t* qp = a.q_bh + (int64_t)g * kHeadDim + 8 * kg;
 #pragma unroll
     for (int c = 0; c < 4; ++c)
-      qB[half][c] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(qp + 32 * c));
+      qB[half][c] = *reinterpret_cast<const uint4*>(qp + 32 * c);
   }
 
   const int row_bytes = a.row_bytes;
@@ -370,7 +368,7 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
           __builtin_amdgcn_sched_barrier(0);
           read_k(s3, ka);
           __builtin_amdgcn_sched_barrier(0);
-          page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, cur_valid >> 8, cur_valid & 255, kg);
+          page_scores<NG, F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, cur_valid >> 8, cur_valid & 255, kg);
           __builtin_amdgcn_sched_barrier(0);
           // The stage just read is refilled only now that the matrix unit has consumed
           // it: a load through an empty descriptor (a masked page) returns at once
@@ -380,7 +378,7 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
           __builtin_amdgcn_sched_barrier(0);
           id_next = load_id(it + s3 + 4);  // lands while the P V products run
           if (cur_valid != kPageSize) clear_unused_v_rows(v[s3], cur_valid >> 8, cur_valid & 255, kg);
-          page_pv<NG>(v[s3], pr, O);
+          page_pv<NG, F16>(v[s3], pr, O);
         }
       }
     }
@@ -408,11 +406,11 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
         __builtin_amdgcn_sched_barrier(0);
         issue_k(r1, 1);
         __builtin_amdgcn_sched_barrier(0);
-        page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validA >> 8, validA & 255, kg);
+        page_scores<NG, F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validA >> 8, validA & 255, kg);
         __builtin_amdgcn_sched_barrier(0);
         id_next = load_id(it + 2);  // lands while the P V products run
         if (validA != kPageSize) clear_unused_v_rows(vA, validA >> 8, validA & 255, kg);  // partial page: rare
-        page_pv<NG>(vA, pr, O);
+        page_pv<NG, F16>(vA, pr, O);
       }
       {
         const __amdgpu_buffer_rsrc_t r2 = page_rsrc(it + 2, id_next, validA);
@@ -425,11 +423,11 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
         __builtin_amdgcn_sched_barrier(0);
         issue_k(r2, 0);
         __builtin_amdgcn_sched_barrier(0);
-        page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validB >> 8, validB & 255, kg);
+        page_scores<NG, F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validB >> 8, validB & 255, kg);
         __builtin_amdgcn_sched_barrier(0);
         id_next = load_id(it + 3);
         if (validB != kPageSize) clear_unused_v_rows(vB, validB >> 8, validB & 255, kg);
-        page_pv<NG>(vB, pr, O);
+        page_pv<NG, F16>(vB, pr, O);
       }
     }
   }

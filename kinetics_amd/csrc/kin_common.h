@@ -125,6 +125,38 @@ __device__ __forceinline__ uint32_t f32_to_bf16(float f) {
   return u >> 16;
 }
 
+// ---- element formats --------------------------------------------------------
+// q, k, v, kv_cache, kbar and out hold bfloat16 (F16 = false) or IEEE half
+// (F16 = true, the reference's --dtype float16); everything is accumulated in fp32.
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+// The two elements packed in one dword, widened to fp32 (exact).
+template <bool F16>
+__device__ __forceinline__ float elem_lo(uint32_t w) {
+  if constexpr (F16) return (float)__builtin_bit_cast(f16x2, w).x;
+  else return bf16_lo(w);
+}
+template <bool F16>
+__device__ __forceinline__ float elem_hi(uint32_t w) {
+  if constexpr (F16) return (float)__builtin_bit_cast(f16x2, w).y;
+  else return bf16_hi(w);
+}
+// fp32 -> element bits (low 16 bits of the result), round-to-nearest-even.
+template <bool F16>
+__device__ __forceinline__ uint32_t f32_to_elem(float f) {
+  if constexpr (F16) return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+  else return f32_to_bf16(f);
+}
+// 16 keys x 32 columns times 32 columns x 16 queries on the matrix unit, 8 elements per lane and operand.
+template <bool F16>
+__device__ __forceinline__ floatx4 mfma_16x16x32(const uint4& a, const uint4& b, floatx4 c) {
+  if constexpr (F16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
 // DPP lane permutes inside a row of 16 lanes (no LDS traffic).
 template <int CTRL>
 __device__ __forceinline__ float dpp_f(float x) {

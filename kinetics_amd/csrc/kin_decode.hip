@@ -26,7 +26,7 @@ struct DecodeParams {
   float scale_log2;  // sm_scale * log2(e)
 };
 
-template <int NG>
+template <int NG, bool F16>
 __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
   __shared__ __attribute__((aligned(16))) unsigned char lds[attend_lds_bytes(4, attend_k_stages(NG))];
   __shared__ float sm_m[4][4 * NG];
@@ -73,12 +73,12 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
   const __attribute__((address_space(4))) int32_t* pl_c =
       reinterpret_cast<const __attribute__((address_space(4))) int32_t*>(reinterpret_cast<uintptr_t>(pl));
   const int64_t hq0 = (int64_t)b * p.num_q_heads + (int64_t)h * G;
-  attend_list<NG, 4>(
+  attend_list<NG, 4, F16>(
       a, [&](int i) -> int { return pl_c[i]; }, lds, sm_m, sm_l,
       [&](int g, int d, float o, float lse2) {
         const int64_t hq = hq0 + g;
         if (p.num_splits == 1) {
-          p.out[hq * kHeadDim + d] = (uint16_t)f32_to_bf16(o);
+          p.out[hq * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(o);
           if (p.lse && d == 0) p.lse[hq] = lse2 * kLn2;
         } else {
           p.ws_o[(hq * p.num_splits + split) * kHeadDim + d] = o;
@@ -88,6 +88,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
 }
 
 // Split-K merge: one 128-thread block per (sequence, query head).
+template <bool F16>
 __global__ __launch_bounds__(128) void merge_splits_kernel(const float* __restrict__ ws_o,
                                                            const float* __restrict__ ws_lse,
                                                            uint16_t* __restrict__ out, float* __restrict__ lse,
@@ -104,7 +105,7 @@ __global__ __launch_bounds__(128) void merge_splits_kernel(const float* __restri
     num += ws_o[(hq * num_splits + s) * kHeadDim + d] * wgt;
     den += wgt;
   }
-  out[hq * kHeadDim + d] = (uint16_t)f32_to_bf16(den > 0.f ? num / den : 0.f);
+  out[hq * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(den > 0.f ? num / den : 0.f);
   if (lse && d == 0) lse[hq] = (den > 0.f) ? (mm + fast_log2(den)) * kLn2 : kNegInf;
 }
 
@@ -129,7 +130,7 @@ static size_t workspace_bytes_for(int batch, int num_q_heads, int splits) {
 }
 
 static int launch_decode(const char* fn, DecodeParams& p, int batch, void* workspace, size_t workspace_bytes,
-                         int max_pages_per_list, int num_splits, hipStream_t stream) {
+                         int max_pages_per_list, int num_splits, bool f16, hipStream_t stream) {
   int splits = num_splits > 0 ? num_splits : auto_splits(batch, p.num_kv_heads, max_pages_per_list);
   if (splits > 65535) return fail(KIN_ERR_BAD_SHAPE, "%s: num_splits=%d exceeds 65535", fn, splits);
   p.num_splits = splits;
@@ -149,15 +150,19 @@ static int launch_decode(const char* fn, DecodeParams& p, int batch, void* works
   if (lists > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   p.batch = batch;
   dim3 grid((unsigned)lists, (unsigned)splits);
-  if (p.group <= 4)
-    paged_decode_kernel<1><<<grid, 256, 0, stream>>>(p);
-  else
-    paged_decode_kernel<2><<<grid, 256, 0, stream>>>(p);
+  if (p.group <= 4) {
+    if (f16) paged_decode_kernel<1, true><<<grid, 256, 0, stream>>>(p);
+    else paged_decode_kernel<1, false><<<grid, 256, 0, stream>>>(p);
+  } else {
+    if (f16) paged_decode_kernel<2, true><<<grid, 256, 0, stream>>>(p);
+    else paged_decode_kernel<2, false><<<grid, 256, 0, stream>>>(p);
+  }
   int st = check_hip(hipGetLastError(), "paged_decode_kernel launch");
   if (st) return st;
   if (splits > 1) {
-    merge_splits_kernel<<<(unsigned)((int64_t)batch * p.num_q_heads), 128, 0, stream>>>(p.ws_o, p.ws_lse, p.out,
-                                                                                         p.lse, splits);
+    const unsigned mgrid = (unsigned)((int64_t)batch * p.num_q_heads);
+    if (f16) merge_splits_kernel<true><<<mgrid, 128, 0, stream>>>(p.ws_o, p.ws_lse, p.out, p.lse, splits);
+    else merge_splits_kernel<false><<<mgrid, 128, 0, stream>>>(p.ws_o, p.ws_lse, p.out, p.lse, splits);
     st = check_hip(hipGetLastError(), "merge_splits_kernel launch");
   }
   return st;
@@ -194,13 +199,12 @@ size_t kin_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads, 
   return kin::workspace_bytes_for(batch, num_q_heads, splits);
 }
 
-int kin_sparse_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const int32_t* sel_pages,
-                            const int32_t* sel_count, const int32_t* last_page_len, kin_bf16_t* out, float* lse,
-                            void* workspace, size_t workspace_bytes, int batch, int num_q_heads, int num_kv_heads,
-                            int head_dim, int page_size, int64_t num_pages, int sel_stride, int first_page_offset,
-                            float sm_scale, int num_splits, kin_stream_t stream) {
+static int sparse_decode_impl(const char* fn, bool f16, const uint16_t* q, const uint16_t* kv_cache, const int32_t* sel_pages,
+                              const int32_t* sel_count, const int32_t* last_page_len, uint16_t* out, float* lse,
+                              void* workspace, size_t workspace_bytes, int batch, int num_q_heads, int num_kv_heads,
+                              int head_dim, int page_size, int64_t num_pages, int sel_stride, int first_page_offset,
+                              float sm_scale, int num_splits, kin_stream_t stream) {
   using namespace kin;
-  const char* fn = "kin_sparse_paged_decode";
   if (!sel_pages || !sel_count) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_decode_args(fn, q, kv_cache, last_page_len, out, batch, num_q_heads, num_kv_heads, head_dim,
                              page_size, num_pages, first_page_offset, num_splits);
@@ -225,17 +229,16 @@ int kin_sparse_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, con
   p.page_size = page_size;
   const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
   p.scale_log2 = scale * 1.4426950408889634f;
-  return launch_decode(fn, p, batch, workspace, workspace_bytes, sel_stride, num_splits,
+  return launch_decode(fn, p, batch, workspace, workspace_bytes, sel_stride, num_splits, f16,
                        static_cast<hipStream_t>(stream));
 }
 
-int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const int32_t* page_indices,
-                           const int32_t* page_indptr, const int32_t* last_page_len, kin_bf16_t* out, float* lse,
-                           void* workspace, size_t workspace_bytes, int batch, int num_q_heads, int num_kv_heads,
-                           int head_dim, int page_size, int64_t num_pages, int max_pages_per_seq,
-                           int first_page_offset, float sm_scale, int num_splits, kin_stream_t stream) {
+static int dense_decode_impl(const char* fn, bool f16, const uint16_t* q, const uint16_t* kv_cache, const int32_t* page_indices,
+                             const int32_t* page_indptr, const int32_t* last_page_len, uint16_t* out, float* lse,
+                             void* workspace, size_t workspace_bytes, int batch, int num_q_heads, int num_kv_heads,
+                             int head_dim, int page_size, int64_t num_pages, int max_pages_per_seq,
+                             int first_page_offset, float sm_scale, int num_splits, kin_stream_t stream) {
   using namespace kin;
-  const char* fn = "kin_dense_paged_decode";
   if (!page_indices || !page_indptr) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_decode_args(fn, q, kv_cache, last_page_len, out, batch, num_q_heads, num_kv_heads, head_dim,
                              page_size, num_pages, first_page_offset, num_splits);
@@ -261,8 +264,48 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, cons
   p.page_size = page_size;
   const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
   p.scale_log2 = scale * 1.4426950408889634f;
-  return launch_decode(fn, p, batch, workspace, workspace_bytes, max_pages_per_seq, num_splits,
+  return launch_decode(fn, p, batch, workspace, workspace_bytes, max_pages_per_seq, num_splits, f16,
                        static_cast<hipStream_t>(stream));
+}
+
+#define KIN_SPARSE_DECODE_ARGS                                                                                         \
+  sel_pages, sel_count, last_page_len, out, lse, workspace, workspace_bytes, batch, num_q_heads, num_kv_heads, head_dim, \
+      page_size, num_pages, sel_stride, first_page_offset, sm_scale, num_splits, stream
+
+int kin_sparse_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const int32_t* sel_pages,
+                            const int32_t* sel_count, const int32_t* last_page_len, kin_bf16_t* out, float* lse,
+                            void* workspace, size_t workspace_bytes, int batch, int num_q_heads, int num_kv_heads,
+                            int head_dim, int page_size, int64_t num_pages, int sel_stride, int first_page_offset,
+                            float sm_scale, int num_splits, kin_stream_t stream) {
+  return sparse_decode_impl("kin_sparse_paged_decode", false, q, kv_cache, KIN_SPARSE_DECODE_ARGS);
+}
+
+int kin_sparse_paged_decode_f16(const kin_f16_t* q, const kin_f16_t* kv_cache, const int32_t* sel_pages,
+                                const int32_t* sel_count, const int32_t* last_page_len, kin_f16_t* out, float* lse,
+                                void* workspace, size_t workspace_bytes, int batch, int num_q_heads, int num_kv_heads,
+                                int head_dim, int page_size, int64_t num_pages, int sel_stride, int first_page_offset,
+                                float sm_scale, int num_splits, kin_stream_t stream) {
+  return sparse_decode_impl("kin_sparse_paged_decode_f16", true, q, kv_cache, KIN_SPARSE_DECODE_ARGS);
+}
+
+#define KIN_DENSE_DECODE_ARGS                                                                                             \
+  page_indices, page_indptr, last_page_len, out, lse, workspace, workspace_bytes, batch, num_q_heads, num_kv_heads, head_dim, \
+      page_size, num_pages, max_pages_per_seq, first_page_offset, sm_scale, num_splits, stream
+
+int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const int32_t* page_indices,
+                           const int32_t* page_indptr, const int32_t* last_page_len, kin_bf16_t* out, float* lse,
+                           void* workspace, size_t workspace_bytes, int batch, int num_q_heads, int num_kv_heads,
+                           int head_dim, int page_size, int64_t num_pages, int max_pages_per_seq,
+                           int first_page_offset, float sm_scale, int num_splits, kin_stream_t stream) {
+  return dense_decode_impl("kin_dense_paged_decode", false, q, kv_cache, KIN_DENSE_DECODE_ARGS);
+}
+
+int kin_dense_paged_decode_f16(const kin_f16_t* q, const kin_f16_t* kv_cache, const int32_t* page_indices,
+                               const int32_t* page_indptr, const int32_t* last_page_len, kin_f16_t* out, float* lse,
+                               void* workspace, size_t workspace_bytes, int batch, int num_q_heads, int num_kv_heads,
+                               int head_dim, int page_size, int64_t num_pages, int max_pages_per_seq,
+                               int first_page_offset, float sm_scale, int num_splits, kin_stream_t stream) {
+  return dense_decode_impl("kin_dense_paged_decode_f16", true, q, kv_cache, KIN_DENSE_DECODE_ARGS);
 }
 
 }  // extern "C"

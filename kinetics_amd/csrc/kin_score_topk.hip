@@ -26,7 +26,7 @@ struct ScoreTopkParams {
 };
 
 // Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap] | int32 sel[sink + topk + local]
-template <int UNROLL>
+template <int UNROLL, bool F16>
 __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ int sh_last;
@@ -70,7 +70,7 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
     const int n_score = (min(a.topk, a.n_cand) > 0 || a.scores_out) ? a.n_cand : 0;
     const int per = ((n_score + p.chunks - 1) / p.chunks + 63) & ~63;
     const int r0 = min(chunk * per, n_score), r1 = min(r0 + per, n_score);
-    score_rows<UNROLL, kThreads, true>(a, r0, r1, gkeys);
+    score_rows<UNROLL, kThreads, true, F16>(a, r0, r1, gkeys);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (tid == 0)
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
     __syncthreads();
     n_list = select_from_keys<kThreads>(a, sel_lds);
   } else {
-    n_list = score_select<UNROLL>(a, sel_lds);
+    n_list = score_select<UNROLL, kThreads, F16>(a, sel_lds);
   }
 
   for (int i = tid; i < p.sel_stride; i += kThreads) sel[i] = (i < n_list) ? sel_lds[i] : -1;
@@ -92,15 +92,14 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
 
 }  // namespace kin
 
-extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar, const int32_t* page_indices,
-                                    const int32_t* page_indptr, const int32_t* last_page_len, int topk,
-                                    int sink_pages, int local_tokens,
-                                    int32_t* sel_pages, int32_t* sel_count,
-                                    int32_t* sel_logical, float* scores_out, int batch, int num_q_heads,
-                                    int num_kv_heads, int head_dim, int page_size, int kbar_pages, int sel_stride,
-                                    void* workspace, size_t workspace_bytes, kin_stream_t stream) {
-  using namespace kin;
-  const char* fn = "kin_block_score_topk";
+namespace kin {
+static int score_topk_impl(const char* fn, bool f16, const uint16_t* q, const uint16_t* kbar, const int32_t* page_indices,
+                           const int32_t* page_indptr, const int32_t* last_page_len, int topk,
+                           int sink_pages, int local_tokens,
+                           int32_t* sel_pages, int32_t* sel_count,
+                           int32_t* sel_logical, float* scores_out, int batch, int num_q_heads,
+                           int num_kv_heads, int head_dim, int page_size, int kbar_pages, int sel_stride,
+                           void* workspace, size_t workspace_bytes, kin_stream_t stream) {
   if (!q || !kbar || !page_indices || !page_indptr || !last_page_len || !sel_pages || !sel_count)
     return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size);
@@ -165,17 +164,42 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
   // Few workgroups cannot saturate HBM with 4 loads per lane in flight: give a
   // small grid 16 (more registers, which it can afford).
   const bool small_grid = items < 512;
-  const void* fn_ptr = small_grid ? reinterpret_cast<const void*>(&score_topk_kernel<16>)
-                                  : reinterpret_cast<const void*>(&score_topk_kernel<4>);
+  const void* fn_ptr;
+  if (f16)
+    fn_ptr = small_grid ? reinterpret_cast<const void*>(&score_topk_kernel<16, true>)
+                        : reinterpret_cast<const void*>(&score_topk_kernel<4, true>);
+  else
+    fn_ptr = small_grid ? reinterpret_cast<const void*>(&score_topk_kernel<16, false>)
+                        : reinterpret_cast<const void*>(&score_topk_kernel<4, false>);
   if (lds > 48 * 1024) {
     // Above the default dynamic-LDS allowance the runtime wants an explicit opt-in.
     st = check_hip(hipFuncSetAttribute(fn_ptr, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
                    "hipFuncSetAttribute(score_topk_kernel)");
     if (st) return st;
   }
-  if (small_grid)
-    score_topk_kernel<16><<<(unsigned)grid, kThreads, lds, hs>>>(p);
-  else
-    score_topk_kernel<4><<<(unsigned)grid, kThreads, lds, hs>>>(p);
-  return check_hip(hipGetLastError(), "score_topk_kernel launch");
+  void* args[] = {&p};
+  return check_hip(hipLaunchKernel(fn_ptr, dim3((unsigned)grid), dim3(kThreads), args, lds, hs), "score_topk_kernel launch");
+}
+}  // namespace kin
+
+extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar, const int32_t* page_indices,
+                                    const int32_t* page_indptr, const int32_t* last_page_len, int topk,
+                                    int sink_pages, int local_tokens, int32_t* sel_pages, int32_t* sel_count,
+                                    int32_t* sel_logical, float* scores_out, int batch, int num_q_heads,
+                                    int num_kv_heads, int head_dim, int page_size, int kbar_pages, int sel_stride,
+                                    void* workspace, size_t workspace_bytes, kin_stream_t stream) {
+  return kin::score_topk_impl("kin_block_score_topk", false, q, kbar, page_indices, page_indptr, last_page_len, topk,
+                              sink_pages, local_tokens, sel_pages, sel_count, sel_logical, scores_out, batch, num_q_heads,
+                              num_kv_heads, head_dim, page_size, kbar_pages, sel_stride, workspace, workspace_bytes, stream);
+}
+
+extern "C" int kin_block_score_topk_f16(const kin_f16_t* q, const kin_f16_t* kbar, const int32_t* page_indices,
+                                        const int32_t* page_indptr, const int32_t* last_page_len, int topk,
+                                        int sink_pages, int local_tokens, int32_t* sel_pages, int32_t* sel_count,
+                                        int32_t* sel_logical, float* scores_out, int batch, int num_q_heads,
+                                        int num_kv_heads, int head_dim, int page_size, int kbar_pages, int sel_stride,
+                                        void* workspace, size_t workspace_bytes, kin_stream_t stream) {
+  return kin::score_topk_impl("kin_block_score_topk_f16", true, q, kbar, page_indices, page_indptr, last_page_len, topk,
+                              sink_pages, local_tokens, sel_pages, sel_count, sel_logical, scores_out, batch, num_q_heads,
+                              num_kv_heads, head_dim, page_size, kbar_pages, sel_stride, workspace, workspace_bytes, stream);
 }

@@ -114,7 +114,7 @@ __device__ __forceinline__ void radix_pick_bin(const uint32_t* hist, uint32_t re
 // UNROLL: independent 16-byte loads each lane keeps in flight while streaming the
 // mean keys (4 saturates HBM when thousands of workgroups run; a small grid
 // needs more per workgroup).
-template <int UNROLL, int NT, bool DEVICE_VISIBLE = false>
+template <int UNROLL, int NT, bool DEVICE_VISIBLE = false, bool F16 = false>
 __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, uint32_t* keys_out) {
   constexpr int kUnroll = UNROLL;
   constexpr int kRows = NT / 16;  // mean keys one pass of the workgroup covers
@@ -129,10 +129,10 @@ __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, 
     const uint16_t* qp = a.q_bh + 8 * c16;
     for (int g = 0; g < a.G; ++g) {
       const uint4 w = *reinterpret_cast<const uint4*>(qp + (int64_t)g * kHeadDim);
-      qm[0] += bf16_lo(w.x); qm[1] += bf16_hi(w.x);
-      qm[2] += bf16_lo(w.y); qm[3] += bf16_hi(w.y);
-      qm[4] += bf16_lo(w.z); qm[5] += bf16_hi(w.z);
-      qm[6] += bf16_lo(w.w); qm[7] += bf16_hi(w.w);
+      qm[0] += elem_lo<F16>(w.x); qm[1] += elem_hi<F16>(w.x);
+      qm[2] += elem_lo<F16>(w.y); qm[3] += elem_hi<F16>(w.y);
+      qm[4] += elem_lo<F16>(w.z); qm[5] += elem_hi<F16>(w.z);
+      qm[6] += elem_lo<F16>(w.w); qm[7] += elem_hi<F16>(w.w);
     }
     const float inv = 1.0f / (float)a.G;
 #pragma unroll
@@ -165,10 +165,10 @@ __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, 
       const u32x4 x = w[j];
       w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, next_off + j * kRows * row_stride_b, 0, kStreamLoad);
       float acc = 0.f;
-      acc = fmaf(qm[0], bf16_lo(x.x), acc); acc = fmaf(qm[1], bf16_hi(x.x), acc);
-      acc = fmaf(qm[2], bf16_lo(x.y), acc); acc = fmaf(qm[3], bf16_hi(x.y), acc);
-      acc = fmaf(qm[4], bf16_lo(x.z), acc); acc = fmaf(qm[5], bf16_hi(x.z), acc);
-      acc = fmaf(qm[6], bf16_lo(x.w), acc); acc = fmaf(qm[7], bf16_hi(x.w), acc);
+      acc = fmaf(qm[0], elem_lo<F16>(x.x), acc); acc = fmaf(qm[1], elem_hi<F16>(x.x), acc);
+      acc = fmaf(qm[2], elem_lo<F16>(x.y), acc); acc = fmaf(qm[3], elem_hi<F16>(x.y), acc);
+      acc = fmaf(qm[4], elem_lo<F16>(x.z), acc); acc = fmaf(qm[5], elem_hi<F16>(x.z), acc);
+      acc = fmaf(qm[6], elem_lo<F16>(x.w), acc); acc = fmaf(qm[7], elem_hi<F16>(x.w), acc);
       acc = row16_sum(acc);
       const int row = base + j * kRows + sub;
       if (c16 == 0 && row < n) {
@@ -339,11 +339,11 @@ __device__ __forceinline__ int select_from_keys(const SelectArgs& a, int32_t* se
 }
 
 // score_rows() over every candidate into a.keys, then select_from_keys().
-template <int UNROLL = 4, int NT = kThreads>
+template <int UNROLL = 4, int NT = kThreads, bool F16 = false>
 __device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_lds) {
   // Nothing to choose (topk == 0) and nobody asked for the scores: stream nothing.
   const int n_score = (min(a.topk, a.n_cand) > 0 || a.scores_out) ? a.n_cand : 0;
-  score_rows<UNROLL, NT>(a, 0, n_score, a.keys);
+  score_rows<UNROLL, NT, false, F16>(a, 0, n_score, a.keys);
   __syncthreads();
   return select_from_keys<NT>(a, sel_lds);
 }

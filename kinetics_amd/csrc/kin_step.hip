@@ -43,7 +43,7 @@ struct StepParams {
   float scale_log2;
 };
 
-template <int NG, int NW>
+template <int NG, int NW, bool F16>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kernel(StepParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ float sm_m[NW][4 * NG];
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     if (p.k != nullptr && tid < 64) {
       uint32_t* kbar_row =
           reinterpret_cast<uint32_t*>(p.kbar) + kbar_row_index(b, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2);
-      append_token_row(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2),
+      append_token_row<F16>(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2),
                        reinterpret_cast<uint32_t*>(p.kv), kbar_row, p.page_indices[pe - 1], last_len, n_pages, p.kbar_pages, h,
                        p.num_kv_heads, p.num_pages, tid, p.page_size);
       // The attention phase of this workgroup reads the row back: make the stores
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     const int n_score = min(s.topk, s.n_cand) > 0 ? s.n_cand : 0;
     const int per = ((n_score + p.chunks - 1) / p.chunks + 63) & ~63;
     const int r0 = min(chunk * per, n_score), r1 = min(r0 + per, n_score);
-    score_rows<4, NT, true>(s, r0, r1, gkeys);
+    score_rows<4, NT, true, F16>(s, r0, r1, gkeys);
     // The slices meet through memory without cache maintenance: keys and the
     // arrival counter are written and read at device scope (they bypass the
     // XCD-private L2), and every wave waits for its own stores to be acknowledged
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     __syncthreads();
     n = select_from_keys<NT>(s, sel_lds);
   } else {
-    n = score_select<4, NT>(s, sel_lds);
+    n = score_select<4, NT, F16>(s, sel_lds);
   }
   if (p.sel_pages) {
     int32_t* sel = p.sel_pages + (int64_t)item * p.sel_stride;
@@ -159,10 +159,10 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   a.p1 = n;
   a.last_len = last_len;
   a.first_skip = p.first_page_offset;
-  attend_list<NG, NW>(
+  attend_list<NG, NW, F16>(
       a, [&](int i) -> int { return __builtin_amdgcn_readfirstlane(sel_lds[i]); }, smem, sm_m, sm_l,
       [&](int g, int d, float o, float lse2) {
-        p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_bf16(o);
+        p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(o);
         if (p.lse && d == 0) p.lse[hq0 + g] = lse2 * kLn2;
       });
 }
@@ -180,8 +180,8 @@ namespace kin {
 // Validation and launch shared by kin_blocktopk_decode_step (workspace from the
 // caller) and kin_blocktopk_decode_step_static (workspace = this library's own
 // device array).  fn: the entry point's name, for error messages.
-static int launch_step(const char* fn, const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
-                       kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
+static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                       uint16_t* kv_cache, uint16_t* kbar, const int32_t* page_indices,
                        const int32_t* page_indptr, const int32_t* last_page_len, int topk, int sink_pages,
                        int local_tokens, int32_t* sel_pages, int32_t* sel_count, kin_bf16_t* out, float* lse,
                        int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
@@ -273,13 +273,23 @@ static int launch_step(const char* fn, const kin_bf16_t* q, const kin_bf16_t* k,
   const size_t lds = region0 + (size_t)list_cap * 4;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const void* kernel;
-  if (p.group <= 4)
-    kernel = nw == 16  ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 16>)
-             : nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 8>)
-                       : reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 4>);
-  else
-    kernel = nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<2, 8>)
-                     : reinterpret_cast<const void*>(&blocktopk_step_kernel<2, 4>);
+  if (f16) {
+    if (p.group <= 4)
+      kernel = nw == 16  ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 16, true>)
+               : nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 8, true>)
+                         : reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 4, true>);
+    else
+      kernel = nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<2, 8, true>)
+                       : reinterpret_cast<const void*>(&blocktopk_step_kernel<2, 4, true>);
+  } else {
+    if (p.group <= 4)
+      kernel = nw == 16  ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 16, false>)
+               : nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 8, false>)
+                         : reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 4, false>);
+    else
+      kernel = nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<2, 8, false>)
+                       : reinterpret_cast<const void*>(&blocktopk_step_kernel<2, 4, false>);
+  }
   if (lds > 48 * 1024) {
     // Above the default dynamic-LDS allowance the runtime wants an explicit opt-in.
     st = check_hip(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
@@ -337,10 +347,24 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
                                          int head_dim, int page_size, int64_t num_pages, int kbar_pages,
                                          int sel_stride, int first_page_offset, float sm_scale, void* workspace,
                                          size_t workspace_bytes, kin_stream_t stream) {
-  return kin::launch_step("kin_blocktopk_decode_step", q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len,
-                          topk, sink_pages, local_tokens, sel_pages, sel_count, out, lse, batch, num_q_heads, num_kv_heads,
-                          head_dim, page_size, num_pages, kbar_pages, sel_stride, first_page_offset, sm_scale, workspace,
-                          workspace_bytes, stream);
+  return kin::launch_step("kin_blocktopk_decode_step", false, q, k, v, kv_cache, kbar, page_indices, page_indptr,
+                          last_page_len, topk, sink_pages, local_tokens, sel_pages, sel_count, out, lse, batch, num_q_heads,
+                          num_kv_heads, head_dim, page_size, num_pages, kbar_pages, sel_stride, first_page_offset, sm_scale,
+                          workspace, workspace_bytes, stream);
+}
+
+extern "C" int kin_blocktopk_decode_step_f16(const kin_f16_t* q, const kin_f16_t* k, const kin_f16_t* v,
+                                             kin_f16_t* kv_cache, kin_f16_t* kbar, const int32_t* page_indices,
+                                             const int32_t* page_indptr, const int32_t* last_page_len, int topk,
+                                             int sink_pages, int local_tokens, int32_t* sel_pages, int32_t* sel_count,
+                                             kin_f16_t* out, float* lse, int batch, int num_q_heads, int num_kv_heads,
+                                             int head_dim, int page_size, int64_t num_pages, int kbar_pages,
+                                             int sel_stride, int first_page_offset, float sm_scale, void* workspace,
+                                             size_t workspace_bytes, kin_stream_t stream) {
+  return kin::launch_step("kin_blocktopk_decode_step_f16", true, q, k, v, kv_cache, kbar, page_indices, page_indptr,
+                          last_page_len, topk, sink_pages, local_tokens, sel_pages, sel_count, out, lse, batch, num_q_heads,
+                          num_kv_heads, head_dim, page_size, num_pages, kbar_pages, sel_stride, first_page_offset, sm_scale,
+                          workspace, workspace_bytes, stream);
 }
 
 extern "C" size_t kin_static_scratch_bytes(void) { return kin::kStaticScratchBytes; }
@@ -369,7 +393,7 @@ extern "C" int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_b
     const int st = static_scratch_address(fn, &ws);
     if (st) return st;
   }
-  return launch_step(fn, q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sink_pages, local_tokens,
+  return launch_step(fn, false, q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sink_pages, local_tokens,
                      sel_pages, sel_count, out, lse, batch, num_q_heads, num_kv_heads, head_dim, page_size, num_pages,
                      kbar_pages, sel_stride, first_page_offset, sm_scale, ws, need > 0 ? kStaticScratchBytes : 0, stream);
 }

@@ -571,14 +571,14 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
   const int G = a.G;
   const int n = a.n;
 
-  bf16x8 qB[NG][4];
+  uint4 qB[NG][4];
 #pragma unroll
   for (int half = 0; half < NG; ++half) {
     const int g = min(4 * half + gq, G - 1);
     const uint16_t* qp = a.q_bh + (int64_t)g * kHeadDim + 8 * kg;
 #pragma unroll
     for (int c = 0; c < 4; ++c)
-      qB[half][c] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(qp + 32 * c));
+      qB[half][c] = *reinterpret_cast<const uint4*>(qp + 32 * c);
   }
 
   const int row_bytes = a.row_bytes;

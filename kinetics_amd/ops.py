@@ -59,7 +59,7 @@ def _require(t: torch.Tensor, name: str, dtype: torch.dtype, ndim=None, device=N
     # On the launch path of every call: the cheap tests first, messages built only on failure.
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
-    if t.dtype is not dtype:
+    if t.dtype is not dtype and (not isinstance(dtype, tuple) or t.dtype not in dtype):
         raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
     if not t.is_cuda:
         raise ValueError(f"{name} must live on the GPU (device 'cuda'), got {t.device}")
@@ -73,18 +73,27 @@ def _require(t: torch.Tensor, name: str, dtype: torch.dtype, ndim=None, device=N
             raise ValueError(f"{name} must have {ndim} dimensions, got shape {tuple(t.shape)}")
 
 
+# q, k, v, kv_cache, kbar and out hold bfloat16, or float16 (the reference's --dtype float16,
+# benchmark/blocktopk.py:18): one dtype per call, which picks the kin_* or kin_*_f16 entry point
+ELEM_DTYPES = (torch.bfloat16, torch.float16)
+
+
+def _entry(lib, name: str, dtype: torch.dtype):
+    return getattr(lib, name + "_f16" if dtype is torch.float16 else name)
+
+
 def _cache_dims(kv_cache: torch.Tensor):
-    _require(kv_cache, "kv_cache", torch.bfloat16, 5)
+    _require(kv_cache, "kv_cache", ELEM_DTYPES, 5)
     num_pages, two, page_size, num_kv_heads, head_dim = kv_cache.shape
     if two != 2:
         raise ValueError(f"kv_cache must be [num_pages, 2, page_size, num_kv_heads, head_dim], got {tuple(kv_cache.shape)}")
     return num_pages, page_size, num_kv_heads, head_dim
 
 
-def _kbar_pages(kbar: torch.Tensor, batch: int, num_kv_heads: int, head_dim: int) -> int:
+def _kbar_pages(kbar: torch.Tensor, batch: int, num_kv_heads: int, head_dim: int, dtype: torch.dtype) -> int:
     """kbar is [B, Hkv, pages, D] (head-major), or the reference's [B, pages, D]
     when Hkv == 1 (the same bytes)."""
-    _require(kbar, "kbar", torch.bfloat16, (3, 4))
+    _require(kbar, "kbar", dtype, (3, 4))
     if kbar.dim() == 3:
         ok = num_kv_heads == 1 and kbar.shape[0] == batch and kbar.shape[2] == head_dim
         pages = kbar.shape[1]
@@ -122,21 +131,22 @@ def append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_l
     the cache after the append.  ``kbar`` may be None."""
     num_pages, page_size, num_kv_heads, head_dim = _cache_dims(kv_cache)
     dev = kv_cache.device
-    _require(k, "k", torch.bfloat16, 3, dev)
-    _require(v, "v", torch.bfloat16, 3, dev)
+    dt = kv_cache.dtype
+    _require(k, "k", dt, 3, dev)
+    _require(v, "v", dt, 3, dev)
     batch = k.shape[0]
     if tuple(k.shape) != (batch, num_kv_heads, head_dim) or k.shape != v.shape:
         raise ValueError(f"k and v must be [batch, {num_kv_heads}, {head_dim}], got {tuple(k.shape)} and {tuple(v.shape)}")
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     kbar_pages = 0
     if kbar is not None:
-        kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim)
+        kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim, dt)
         if kbar.device != dev:
             raise ValueError("kbar must be on the same device as kv_cache")
     lib = _lib.load()
     with _on(dev):
         _lib.check(
-            lib.kin_append_paged_kv(
+            _entry(lib, "kin_append_paged_kv", dt)(
                 _ptr(k), _ptr(v), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
                 _ptr(last_page_len), batch, num_kv_heads, head_dim, page_size, num_pages, kbar_pages, _stream(dev),
             )
@@ -154,8 +164,9 @@ def append_paged_kv_ragged(k, v, append_indptr, kv_cache, kbar, page_indices, pa
     longest append (default: nnz; it is checked, the cost does not depend on it)."""
     num_pages, page_size, num_kv_heads, head_dim = _cache_dims(kv_cache)
     dev = kv_cache.device
-    _require(k, "k", torch.bfloat16, 3, dev)
-    _require(v, "v", torch.bfloat16, 3, dev)
+    dt = kv_cache.dtype
+    _require(k, "k", dt, 3, dev)
+    _require(v, "v", dt, 3, dev)
     nnz = k.shape[0]
     if tuple(k.shape) != (nnz, num_kv_heads, head_dim) or k.shape != v.shape:
         raise ValueError(f"k and v must be [nnz, {num_kv_heads}, {head_dim}], got {tuple(k.shape)} and {tuple(v.shape)}")
@@ -166,13 +177,13 @@ def append_paged_kv_ragged(k, v, append_indptr, kv_cache, kbar, page_indices, pa
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     kbar_pages = 0
     if kbar is not None:
-        kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim)
+        kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim, dt)
         if kbar.device != dev:
             raise ValueError("kbar must be on the same device as kv_cache")
     lib = _lib.load()
     with _on(dev):
         _lib.check(
-            lib.kin_append_paged_kv_ragged(
+            _entry(lib, "kin_append_paged_kv_ragged", dt)(
                 _ptr(k), _ptr(v), _ptr(append_indptr), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
                 _ptr(last_page_len), batch, nnz, nnz if max_append_len is None else int(max_append_len), num_kv_heads,
                 head_dim, page_size, num_pages, kbar_pages, _stream(dev),
@@ -188,11 +199,11 @@ def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len) -> None
     dev = kv_cache.device
     batch = page_indptr.numel() - 1
     _table(page_indices, page_indptr, last_page_len, batch, dev)
-    kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim)
+    kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim, kv_cache.dtype)
     lib = _lib.load()
     with _on(dev):
         _lib.check(
-            lib.kin_build_kbar(
+            _entry(lib, "kin_build_kbar", kv_cache.dtype)(
                 _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len),
                 batch, num_kv_heads, head_dim, page_size, num_pages, kbar_pages, _stream(dev),
             )
@@ -225,7 +236,7 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
     ``step_workspace_bytes``; optional) lets few, long sequences spread their
     scoring over the GPU.  ``page_size``: tokens per page of the cache the table
     describes (16, 32 or 64)."""
-    _require(q, "q", torch.bfloat16, 3)
+    _require(q, "q", ELEM_DTYPES, 3)
     dev = q.device
     batch, num_q_heads, head_dim = q.shape
     _require(sel_pages, "sel_pages", torch.int32, 3, dev)
@@ -235,7 +246,7 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
     _require(sel_count, "sel_count", torch.int32, 2, dev)
     if tuple(sel_count.shape) != (batch, num_kv_heads):
         raise ValueError(f"sel_count must be [{batch}, {num_kv_heads}], got {tuple(sel_count.shape)}")
-    kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim)
+    kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim, q.dtype)
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     if last_page_len is None:
         raise TypeError("last_page_len is required")
@@ -252,7 +263,7 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
     lib = _lib.load()
     with _on(dev):
         _lib.check(
-            lib.kin_block_score_topk(
+            _entry(lib, "kin_block_score_topk", q.dtype)(
                 _ptr(q), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), int(topk), int(sink_pages),
                 int(local_tokens), _ptr(sel_pages), _ptr(sel_count), _ptr(sel_logical), _ptr(scores_out), batch, num_q_heads,
                 num_kv_heads, head_dim, int(page_size), kbar_pages, sel_stride, _ptr(workspace), workspace.numel() if workspace is not None else 0, _stream(dev),
@@ -281,7 +292,7 @@ def decode_auto_splits(batch, num_kv_heads, max_pages_per_list) -> int:
 def _decode_common(q, kv_cache, last_page_len, out, lse, workspace):
     num_pages, page_size, num_kv_heads, head_dim = _cache_dims(kv_cache)
     dev = kv_cache.device
-    _require(q, "q", torch.bfloat16, 3, dev)
+    _require(q, "q", kv_cache.dtype, 3, dev)
     batch, num_q_heads, qd = q.shape
     if qd != head_dim:
         raise ValueError(f"q head_dim {qd} != kv_cache head_dim {head_dim}")
@@ -291,7 +302,7 @@ def _decode_common(q, kv_cache, last_page_len, out, lse, workspace):
     if out is None:
         out = torch.empty_like(q)
     else:
-        _require(out, "out", torch.bfloat16, 3, dev)
+        _require(out, "out", kv_cache.dtype, 3, dev)
         if out.shape != q.shape:
             raise ValueError(f"out shape {tuple(out.shape)} != q shape {tuple(q.shape)}")
     if lse is not None:
@@ -331,7 +342,7 @@ def sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, out=No
     lib = _lib.load()
     with _on(dev):
         _lib.check(
-            lib.kin_sparse_paged_decode(
+            _entry(lib, "kin_sparse_paged_decode", kv_cache.dtype)(
                 _ptr(q), _ptr(kv_cache), _ptr(sel_pages), _ptr(sel_count), _ptr(last_page_len), _ptr(out), _ptr(lse),
                 _ptr(workspace), ws_bytes, batch, hq, hkv, d, ps, num_pages, sel_pages.shape[2], int(first_page_offset),
                 float(sm_scale), int(num_splits), _stream(dev),
@@ -350,7 +361,7 @@ def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, ma
     lib = _lib.load()
     with _on(dev):
         _lib.check(
-            lib.kin_dense_paged_decode(
+            _entry(lib, "kin_dense_paged_decode", kv_cache.dtype)(
                 _ptr(q), _ptr(kv_cache), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), _ptr(out),
                 _ptr(lse), _ptr(workspace), ws_bytes, batch, hq, hkv, d, ps, num_pages, int(max_pages_per_seq),
                 int(first_page_offset), float(sm_scale), int(num_splits), _stream(dev),
@@ -389,12 +400,13 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
         raise ValueError("static_scratch=True needs a caller-provided out and takes no workspace")
     dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, workspace)
     _table(page_indices, page_indptr, last_page_len, batch, dev)
-    kbar_pages = _kbar_pages(kbar, batch, hkv, d)
+    dt = kv_cache.dtype
+    kbar_pages = _kbar_pages(kbar, batch, hkv, d, dt)
     if (k is None) != (v is None):
         raise ValueError("k and v must both be given or both be None")
     if k is not None:
-        _require(k, "k", torch.bfloat16, 3, dev)
-        _require(v, "v", torch.bfloat16, 3, dev)
+        _require(k, "k", dt, 3, dev)
+        _require(v, "v", dt, 3, dev)
         if tuple(k.shape) != (batch, hkv, d) or k.shape != v.shape:
             raise ValueError(f"k and v must be [{batch}, {hkv}, {d}], got {tuple(k.shape)} and {tuple(v.shape)}")
     sel_stride = 0
@@ -408,6 +420,8 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
         sel_stride = sel_pages.shape[2]
     lib = _lib.load()
     if static_scratch:
+        if dt is not torch.bfloat16:
+            raise ValueError("static_scratch=True is built for bfloat16 only")
         with _on(dev):
             _lib.check(
                 lib.kin_blocktopk_decode_step_static(
@@ -424,7 +438,7 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
             workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     with _on(dev):
         _lib.check(
-            lib.kin_blocktopk_decode_step(
+            _entry(lib, "kin_blocktopk_decode_step", dt)(
                 _ptr(q), _ptr(k), _ptr(v), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
                 _ptr(last_page_len), int(topk), int(sink_pages), int(local_tokens), _ptr(sel_pages), _ptr(sel_count),
                 _ptr(out), _ptr(lse), batch, hq, hkv, d, ps, num_pages, kbar_pages, sel_stride, int(first_page_offset),
@@ -440,6 +454,8 @@ def token_topk_workspace_bytes(batch: int, num_kv_heads: int, max_pages_per_seq:
 
 def _token_policy(q, kv_cache, page_indices, page_indptr, last_page_len, out, lse, sel_tokens, sel_count, workspace,
                   need_bytes):
+    if kv_cache.dtype is not torch.bfloat16:
+        raise ValueError("the token-granular policies are built for bfloat16 caches only")
     dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, None)
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     sel_stride = 0

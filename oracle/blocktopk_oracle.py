@@ -56,11 +56,48 @@ bfloat16 tensors are numpy uint16 arrays of raw bit patterns throughout.
 """
 from __future__ import annotations
 
+import contextlib
+
 import numpy as np
 
 # ---------------------------------------------------------------------------
 # bfloat16 <-> float32
 # ---------------------------------------------------------------------------
+
+
+# The page path (append, mean keys, scores, attention) works on one element
+# format per call: bfloat16, or IEEE binary16 (the reference's --dtype float16,
+# benchmark/blocktopk.py:18).  Tensors are uint16 bit arrays either way; the
+# format in force is chosen with ``element_format``.
+_ELEMENT_FORMAT = "bf16"
+
+
+@contextlib.contextmanager
+def element_format(name: str):
+    """``with element_format("f16"):`` -- the page-path functions below read and
+    write IEEE binary16 bit patterns inside the block (default: bfloat16)."""
+    global _ELEMENT_FORMAT
+    if name not in ("bf16", "f16"):
+        raise ValueError(name)
+    old, _ELEMENT_FORMAT = _ELEMENT_FORMAT, name
+    try:
+        yield
+    finally:
+        _ELEMENT_FORMAT = old
+
+
+def elem_to_f32(bits: np.ndarray) -> np.ndarray:
+    """Exact widening of the element format in force to float32."""
+    if _ELEMENT_FORMAT == "f16":
+        return np.ascontiguousarray(bits, dtype=np.uint16).view(np.float16).astype(np.float32)
+    return bf16_to_f32(bits)
+
+
+def f32_to_elem(x: np.ndarray) -> np.ndarray:
+    """float32 -> bits of the element format in force, round-to-nearest-even."""
+    if _ELEMENT_FORMAT == "f16":
+        return np.asarray(x, dtype=np.float32).astype(np.float16).view(np.uint16)
+    return f32_to_bf16(x)
 
 
 def bf16_to_f32(bits: np.ndarray) -> np.ndarray:
@@ -106,12 +143,12 @@ def page_mean_key(page_k_bits: np.ndarray) -> np.ndarray:
     reference leaves compressed_key_cache random
     (benchmark/blocktopk_decoder.py:166-168); the block mean is what LiteSys ranks
     blocks by (sparsity_utils.py:37) up to the query projection."""
-    rows = bf16_to_f32(page_k_bits)
+    rows = elem_to_f32(page_k_bits)
     ps = rows.shape[-2]
     acc = np.zeros(rows.shape[:-2] + rows.shape[-1:], dtype=np.float32)
     for t in range(ps):
         acc = (acc + rows[..., t, :]).astype(np.float32)
-    return f32_to_bf16(acc * np.float32(1.0 / ps))
+    return f32_to_elem(acc * np.float32(1.0 / ps))
 
 
 def append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len):
@@ -209,7 +246,7 @@ def block_scores(q, kbar, page_indptr, last_page_len, sink_pages=0, local_tokens
     B, Hq, D = q.shape
     Hkv = kbar.shape[1]
     G = Hq // Hkv
-    qf = bf16_to_f32(q).astype(np.float64)
+    qf = elem_to_f32(q).astype(np.float64)
     out = []
     for b in range(B):
         n_pages = int(page_indptr[b + 1]) - int(page_indptr[b])
@@ -217,7 +254,7 @@ def block_scores(q, kbar, page_indptr, last_page_len, sink_pages=0, local_tokens
             out.append([np.zeros(0) for _ in range(Hkv)])
             continue
         n_sink, n_cand, _ = split_pages(n_pages, last_page_len[b], sink_pages, local_tokens, kbar.shape[2], page_size)
-        kb = bf16_to_f32(kbar[b, :, n_sink : n_sink + n_cand]).astype(np.float64)  # [Hkv, n, D]
+        kb = elem_to_f32(kbar[b, :, n_sink : n_sink + n_cand]).astype(np.float64)  # [Hkv, n, D]
         per_head = []
         for h in range(Hkv):
             per_q = np.einsum("gd,nd->gn", qf[b, h * G : (h + 1) * G], kb[h])  # [G, n]
@@ -292,8 +329,8 @@ def attend_pages(q_bh, kv_cache, pages, h, last_len, sm_scale, first_skip=0):
     if len(pages) == 0:
         return np.zeros((G, D)), np.full(G, -np.inf)
     ps = kv_cache.shape[2]
-    K = bf16_to_f32(kv_cache[np.asarray(pages), 0, :, h, :]).astype(np.float64).reshape(-1, D)
-    V = bf16_to_f32(kv_cache[np.asarray(pages), 1, :, h, :]).astype(np.float64).reshape(-1, D)
+    K = elem_to_f32(kv_cache[np.asarray(pages), 0, :, h, :]).astype(np.float64).reshape(-1, D)
+    V = elem_to_f32(kv_cache[np.asarray(pages), 1, :, h, :]).astype(np.float64).reshape(-1, D)
     n_tok = (len(pages) - 1) * ps + int(last_len)
     K, V = K[first_skip:n_tok], V[first_skip:n_tok]
     if len(K) == 0:
@@ -312,7 +349,7 @@ def sparse_paged_decode(q, kv_cache, sel_pages, sel_count, last_page_len, sm_sca
     Hkv = kv_cache.shape[3]
     G = Hq // Hkv
     scale = 1.0 / np.sqrt(D) if sm_scale is None else sm_scale
-    qf = bf16_to_f32(q).astype(np.float64)
+    qf = elem_to_f32(q).astype(np.float64)
     out = np.zeros((B, Hq, D))
     lse = np.full((B, Hq), -np.inf)
     for b in range(B):
@@ -330,7 +367,7 @@ def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, sm
     Hkv = kv_cache.shape[3]
     G = Hq // Hkv
     scale = 1.0 / np.sqrt(D) if sm_scale is None else sm_scale
-    qf = bf16_to_f32(q).astype(np.float64)
+    qf = elem_to_f32(q).astype(np.float64)
     out = np.zeros((B, Hq, D))
     lse = np.full((B, Hq), -np.inf)
     for b in range(B):

@@ -55,7 +55,7 @@ def randn_bf16(rng, shape, scale=1.0, offset=None):
     x = rng.standard_normal(shape, dtype=np.float32) * np.float32(scale)
     if offset is not None:
         x = x + offset.astype(np.float32)
-    return O.f32_to_bf16(x)
+    return O.f32_to_elem(x)   # bfloat16 bits unless a test is inside O.element_format("f16")
 
 
 def make_problem(seed: int, lengths, num_kv_heads: int = 1, group: int = 4, topk: int = 8,
@@ -127,9 +127,11 @@ def make_problem(seed: int, lengths, num_kv_heads: int = 1, group: int = 4, topk
 
 
 def to_torch(bits: np.ndarray, device="cpu"):
+    """uint16 bit patterns -> a bfloat16 tensor (a float16 one inside O.element_format("f16"))."""
     import torch
 
-    t = torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).view(torch.bfloat16)
+    dt = torch.float16 if O._ELEMENT_FORMAT == "f16" else torch.bfloat16
+    t = torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).view(dt)
     return t.to(device)
 
 

@@ -329,3 +329,56 @@ def test_manager_with_a_small_pool_and_overlong_sequences():
     assert m.kv_offset[0][1].item() > PS * 6
     with pytest.raises(ValueError):
         m.clear_cache(1)
+
+
+@pytest.mark.parametrize("sparse", [dict(), dict(attn_block_topk=2, attn_local=18), dict(attn_block_topk=2, attn_local=18, attn_block_size=32)])
+def test_float16_manager(sparse):
+    """LiteSys' manager takes a dtype (batch_cache.py:21); in float16 the paged manager
+    must give LiteSys' own formulation (full logits, its mask, softmax, P.V) on the
+    history that was fed."""
+    from kinetics_amd.batch_cache import PagedBatchKVManager
+
+    torch.manual_seed(21)
+    L, Hq, Hkv = 2, 4, 2
+    block = sparse.get("attn_block_size", 16)
+    m = PagedBatchKVManager(cfg_small(), max_batch_size=3, max_seq_len=block * 30, device=DEV, dtype=torch.float16, **sparse)
+    hist = {}
+    gen = torch.Generator().manual_seed(3)
+    bias = torch.randn(64, Hkv, 1, generator=gen) * 0.5
+
+    def keys(start, n):
+        t = torch.arange(start, start + n)
+        blk = torch.clamp((t - 4) // block + 1, min=0)
+        return (torch.randn(1, Hkv, n, D) + bias[blk].permute(1, 0, 2)[None]).half().to(DEV)
+
+    def feed(layer, slot, k, v):
+        K, V = hist.get((layer, slot), (torch.zeros(0, Hkv, D), torch.zeros(0, Hkv, D)))
+        hist[(layer, slot)] = (torch.cat([K, k.float().cpu().transpose(0, 1)]), torch.cat([V, v.float().cpu().transpose(0, 1)]))
+
+    for slot, n in ((0, block * 9 + 3), (2, block * 5)):
+        for layer in range(L):
+            q, v = torch.randn(1, Hq, n, D, device=DEV).half(), torch.randn(1, Hkv, n, D, device=DEV).half()
+            k = keys(0, n)
+            feed(layer, slot, k[0], v[0])
+            out = m.compute_attention(q, k, v, layer, torch.tensor([slot]))
+            assert out.dtype is torch.float16 and out.shape == (1, n, Hq * D)
+    with pytest.raises(NotImplementedError):
+        PagedBatchKVManager(cfg_small(), 2, 64, DEV, torch.float16, attn_topk=8, attn_local=4)
+    for _ in range(block + 2):                     # crosses a page boundary: a float16 mean key is written
+        for layer in range(L):
+            slots = [0, 2]
+            q, v = torch.randn(2, Hq, 1, D, device=DEV).half(), torch.randn(2, Hkv, 1, D, device=DEV).half()
+            k = torch.cat([keys(int(m.kv_offset[layer][s].item()), 1) for s in slots])
+            out = m.compute_attention(q, k, v, layer, torch.tensor(slots))
+            torch.cuda.synchronize()
+            got = out.float().cpu().numpy().reshape(2, Hq, D)
+            for i, s in enumerate(slots):
+                feed(layer, s, k[i], v[i])
+                K, V = hist[(layer, s)]
+                is_sparse = bool(sparse) and layer != 0
+                ref, keep = O.litesys_decode(q[i, :, 0].float().cpu().numpy(), K.numpy(), V.numpy(),
+                                             sparse["attn_block_topk"] if is_sparse else None, sparse.get("attn_local"),
+                                             block_size=block)
+                assert np.all(np.abs(got[i] - ref) <= 2e-2 + 2e-2 * np.abs(ref)), (layer, s)
+                if is_sparse:
+                    assert not keep.all()

@@ -572,6 +572,84 @@ def test_token_policies_reject_larger_pages(ops):
         ops.token_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, 16, pb.max_pages, sink_tokens=4, local_tokens=8, workspace=ws)
 
 
+@pytest.mark.parametrize("page_size", [16, 64])
+@pytest.mark.parametrize("hkv,group", [(1, 4), (2, 8), (8, 2)])
+def test_float16_caches(ops, hkv, group, page_size):
+    """The reference's --dtype float16 (benchmark/blocktopk.py:18): q, k, v, the
+    cache, the mean keys and the output in IEEE half through the *_f16 entry
+    points -- append and mean keys bit-exact, selection against the oracle, sparse
+    / dense / fused attention within the contract."""
+    ps = page_size
+    with O.element_format("f16"):
+        lengths = [ps * 37 + 3, ps * 5 + ps, 1, 0, ps, ps * 70 + 9, 7, ps * 2 + 1]
+        topk, sink, local = 5, 1, ps + 3
+        pb = P.make_problem(900 + hkv + ps, lengths, num_kv_heads=hkv, group=group, topk=topk, page_size=ps)
+        cap = ops.sel_list_capacity(topk, sink, local)
+        kv_o, kbar_o = pb.kv_cache.copy(), pb.kbar.copy()
+        res = O.decode_step(pb.q, pb.k, pb.v, kv_o, kbar_o, pb.page_indices, pb.page_indptr, pb.last_page_len, topk,
+                            sink_pages=sink, local_tokens=local)
+        assert not np.array_equal(kbar_o, pb.kbar)          # some page filled up: a float16 mean key was written
+        for path in ("three", "fused"):
+            g = Gpu(pb)
+            assert g.kv.dtype is torch.float16 and g.q.dtype is torch.float16
+            g.sel = torch.full((pb.B, hkv, cap), -7, dtype=torch.int32, device=DEV)
+            what = f"float16 ps={ps} hkv={hkv} G={group} {path}"
+            if path == "fused":
+                out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, topk, sel_pages=g.sel,
+                                                sel_count=g.cnt, sink_pages=sink, local_tokens=local)
+            else:
+                ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
+                ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, topk, g.sel, g.cnt, sink_pages=sink,
+                                     local_tokens=local, page_size=ps)
+                out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, num_splits=2)
+            torch.cuda.synchronize()
+            assert out.dtype is torch.float16
+            assert np.array_equal(P.from_torch(g.kv), kv_o), f"{what}: cache bytes"
+            assert np.array_equal(P.from_torch(g.kbar), kbar_o), f"{what}: mean keys"
+            assert np.array_equal(g.cnt.cpu().numpy(), res["sel_count"]), what
+            sel = g.sel.cpu().numpy()
+            for b in range(pb.B):
+                pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
+                lookup = {int(p): i for i, p in enumerate(pages)}
+                for h in range(hkv):
+                    c = int(res["sel_count"][b, h])
+                    if c == 0:
+                        continue
+                    n_sink, n_cand, n_local = O.split_pages(len(pages), pb.last_page_len[b], sink, local, pb.kbar.shape[2], ps)
+                    k_eff = min(topk, n_cand)
+                    got_logical = np.array([lookup[int(x)] for x in sel[b, h, n_sink:n_sink + k_eff]]) - n_sink
+                    ok, msg = O.selection_matches(got_logical, res["scores"][b][h], topk)
+                    assert ok, f"{what} b={b} h={h}: {msg}"
+            want, _ = O.sparse_paged_decode(pb.q, kv_o, sel, res["sel_count"], pb.last_page_len)
+            assert_out_close(out, want, what)
+            dense = ops.dense_paged_decode(g.q, g.kv, g.indices, g.indptr, g.last, pb.max_pages, num_splits=3)
+            wd, _ = O.dense_paged_decode(pb.q, kv_o, pb.page_indices, pb.page_indptr, pb.last_page_len)
+            assert_out_close(dense, wd, what + " dense")
+        # bulk mean keys and the ragged append
+        g = Gpu(pb)
+        g.kbar.zero_()
+        pre_last = torch.clamp(g.last - 1, min=0)
+        ops.build_kbar(g.kv, g.kbar, g.indices, g.indptr, pre_last)
+        assert np.array_equal(P.from_torch(g.kbar), pb.kbar)
+        rng = np.random.default_rng(ps + hkv)
+        new = np.array([min(int(L), int(rng.integers(0, 3 * ps))) for L in pb.lengths])
+        append_indptr = np.concatenate([[0], np.cumsum(new)]).astype(np.int32)
+        k_new, v_new = P.randn_bf16(rng, (int(new.sum()), hkv, D)), P.randn_bf16(rng, (int(new.sum()), hkv, D))
+        want_kv, want_kbar = pb.kv_cache.copy(), pb.kbar.copy()
+        O.append_paged_kv_ragged(k_new, v_new, append_indptr, want_kv, want_kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
+        ops.append_paged_kv_ragged(P.to_torch(k_new, DEV), P.to_torch(v_new, DEV), P.int_tensor(append_indptr, DEV), g.kv, g.kbar,
+                                   g.indices, g.indptr, g.last)
+        torch.cuda.synchronize()
+        assert np.array_equal(P.from_torch(g.kv), want_kv) and np.array_equal(P.from_torch(g.kbar), want_kbar)
+    # mixed dtypes and float16 on the bfloat16-only paths are refused
+    pb = P.make_problem(990, [40, 9], num_kv_heads=hkv, group=group)
+    g = Gpu(pb)
+    with pytest.raises(TypeError):
+        ops.sparse_paged_decode(g.q.half(), g.kv, g.sel, g.cnt, g.last)
+    with pytest.raises(ValueError):
+        ops.token_topk_decode(g.q.half(), g.kv.half(), g.indices, g.indptr, g.last, 4, pb.max_pages)
+
+
 # --------------------------------------------------------------------------- full benchmark sizes
 
 

@@ -266,17 +266,40 @@ def test_selection_matches_rule():
 def _depaged(pb, b, h):
     pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
     L = int(pb.lengths[b])
-    K = O.bf16_to_f32(pb.kv_cache[pages, 0, :, h]).reshape(-1, D)[:L]
-    V = O.bf16_to_f32(pb.kv_cache[pages, 1, :, h]).reshape(-1, D)[:L]
+    K = O.elem_to_f32(pb.kv_cache[pages, 0, :, h]).reshape(-1, D)[:L]
+    V = O.elem_to_f32(pb.kv_cache[pages, 1, :, h]).reshape(-1, D)[:L]
     return K.astype(np.float64), V.astype(np.float64)
 
 
+def test_float16_element_format_is_ieee_half():
+    """The oracle's float16 conversions against torch's: bit patterns and values."""
+    x = np.random.default_rng(5).standard_normal(4096).astype(np.float32) * np.float32(300.0)
+    x[:4] = [0.0, -0.0, 65504.0, 1e-7]
+    with O.element_format("f16"):
+        bits = O.f32_to_elem(x)
+        back = O.elem_to_f32(bits)
+        mean = O.page_mean_key(bits.reshape(-1, 16, 16))          # [256 pages, 16 rows, 16 cols]
+    t = torch.from_numpy(x).half()
+    assert np.array_equal(bits, t.view(torch.int16).numpy().view(np.uint16))
+    assert np.array_equal(back, t.float().numpy())
+    want = (t.float().reshape(-1, 16, 16).sum(dim=1) * (1.0 / 16)).half()   # fp32 sum of 16 rows (exact order aside), one rounding
+    got = torch.from_numpy(mean.view(np.int16)).view(torch.float16)
+    assert torch.allclose(got.float(), want.float(), rtol=2 ** -10, atol=1e-6)
+    assert O._ELEMENT_FORMAT == "bf16"                            # the block restored the default
+
+
+@pytest.mark.parametrize("fmt", ["bf16", "f16"])
 @pytest.mark.parametrize("page_size", [16, 32, 64])
-def test_dense_attention_equals_torch_sdpa(page_size):
+def test_dense_attention_equals_torch_sdpa(page_size, fmt):
+    with O.element_format(fmt):
+        _dense_attention_equals_torch_sdpa(page_size)
+
+
+def _dense_attention_equals_torch_sdpa(page_size):
     pb = P.make_problem(41, [PS * 6 + 5, PS * 2, 9], num_kv_heads=2, group=4, page_size=page_size)
     assert pb.kv_cache.shape[2] == page_size
     out, lse = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len)
-    qf = O.bf16_to_f32(pb.q).astype(np.float64)
+    qf = O.elem_to_f32(pb.q).astype(np.float64)
     for b in range(pb.B):
         for h in range(2):
             K, V = _depaged(pb, b, h)
@@ -378,6 +401,11 @@ def test_attention_permutation_and_split_invariance():
         assert np.allclose(mo, out[0], rtol=1e-12, atol=1e-13) and np.allclose(ml, lse[0], rtol=1e-13)
 
 
+def test_decode_step_equals_masked_dense_formulation_float16():
+    with O.element_format("f16"):
+        test_decode_step_equals_masked_dense_formulation(32)
+
+
 @pytest.mark.parametrize("page_size", [16, 32, 64])
 def test_decode_step_equals_masked_dense_formulation(page_size):
     """LiteSys expresses block sparsity as a -inf mask on full-context logits
@@ -387,7 +415,7 @@ def test_decode_step_equals_masked_dense_formulation(page_size):
     PS = page_size
     pb = P.make_problem(59, [PS * 10 + 5, PS * 7 + PS], num_kv_heads=2, group=2, topk=3, page_size=page_size)
     res = O.decode_step(pb.q, pb.k, pb.v, pb.kv_cache, pb.kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
-    qf = O.bf16_to_f32(pb.q).astype(np.float64)
+    qf = O.elem_to_f32(pb.q).astype(np.float64)
     for b in range(pb.B):
         L = int(pb.lengths[b])
         n_pages = (L + PS - 1) // PS
