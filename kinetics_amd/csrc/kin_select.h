@@ -104,6 +104,41 @@ __device__ __forceinline__ void radix_pick_bin(const uint32_t* hist, uint32_t re
   }
 }
 
+// The same digit pick made by EVERY wave that calls it (all 64 lanes), with the
+// result in every lane: no shared variable, so no barrier after it.  exhausted:
+// the keys wanted from the threshold bin are all the keys in it (every key with the
+// digits fixed so far, this one included, is taken: no further digit is needed).
+__device__ __forceinline__ void radix_pick_bin_uniform(const uint32_t* hist, uint32_t remaining, int lane, uint32_t& bin_out,
+                                                       uint32_t& remaining_out, bool& exhausted) {
+  const int top = 255 - 4 * lane;
+  const uint32_t c0 = hist[top], c1 = hist[top - 1], c2 = hist[top - 2], c3 = hist[top - 3];
+  const uint32_t mine = c0 + c1 + c2 + c3;
+  uint32_t incl = mine;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t up = __shfl_up(incl, off);
+    if (lane >= off) incl += up;
+  }
+  uint32_t run = incl - mine;  // keys in bins above this lane's
+  const bool owner = run < remaining && remaining <= incl;
+  uint32_t bin = 0, rem = 0, cnt = 0;
+  if (owner) {
+    bin = top;
+    uint32_t c = c0;
+    if (run + c < remaining) { run += c; bin = top - 1; c = c1; }
+    if (run + c < remaining) { run += c; bin = top - 2; c = c2; }
+    if (run + c < remaining) { run += c; bin = top - 3; c = c3; }
+    rem = remaining - run;
+    cnt = c;
+  }
+  // exactly one lane owns the threshold bin (1 <= remaining <= number of counted keys)
+  const unsigned long long who = __ballot(owner);
+  const int src = who ? __builtin_ctzll(who) : 0;
+  bin_out = __shfl(bin, src);
+  remaining_out = __shfl(rem, src);
+  exhausted = __shfl(cnt, src) == remaining_out;
+}
+
 // Scores the candidates r0 <= r < r1 of one (sequence, KV head) with the
 // group-mean query and stores them as order-preserving keys in keys_out[r] (LDS
 // or global memory) and, if a.scores_out is set, as fp32 in scores_out[r].
@@ -210,9 +245,9 @@ __device__ __forceinline__ void load_shared_keys(const uint32_t* gkeys, int n, u
 // sel_lds is visible to every thread and keys / sortbuf are free for reuse.
 template <int NT>
 __device__ __forceinline__ int select_from_keys(const SelectArgs& a, int32_t* sel_lds) {
-  __shared__ uint32_t hist[256];
+  __shared__ uint32_t hist[4][256];  // one histogram per radix digit, all zeroed up front
   __shared__ uint32_t wave_tot[NT / 64];
-  __shared__ uint32_t sh_bin, sh_remaining, sh_count;
+  __shared__ uint32_t sh_count;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -222,28 +257,39 @@ __device__ __forceinline__ int select_from_keys(const SelectArgs& a, int32_t* se
   unsigned long long* sortbuf = a.sortbuf;
 
   // ---- phase 2: radix select of the k_eff-th largest key -------------------
+  // One barrier per digit: the histograms are separate arrays zeroed together, and
+  // every wave reads the digit's histogram for itself.  The loop stops as soon as the
+  // threshold bin is wanted whole (usually after two or three digits).
   uint32_t prefix = 0, mask = 0;
   uint32_t remaining = (uint32_t)k_eff;  // how many keys equal to the threshold are taken
+  uint32_t thr = 0;
   if (k_eff > 0 && k_eff < n_cand) {
-    for (int shift = 24; shift >= 0; shift -= 8) {
-      if (tid < 256) hist[tid] = 0;
-      __syncthreads();
+    for (int i = tid; i < 4 * 256; i += NT) (&hist[0][0])[i] = 0;
+    __syncthreads();
+    bool whole_bin = false;
+    for (int pass = 0; pass < 4 && !whole_bin; ++pass) {
+      const int shift = 24 - 8 * pass;
       for (int i = tid; i < n_cand; i += NT) {
         const uint32_t key = keys[i];
-        if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+        if ((key & mask) == prefix) atomicAdd(&hist[pass][(key >> shift) & 255u], 1u);
       }
       __syncthreads();
-      if (wave == 0) radix_pick_bin(hist, remaining, lane, &sh_bin, &sh_remaining);
-      __syncthreads();
-      prefix |= sh_bin << shift;
+      uint32_t bin;
+      radix_pick_bin_uniform(hist[pass], remaining, lane, bin, remaining, whole_bin);
+      prefix |= bin << shift;
       mask |= 255u << shift;
-      remaining = sh_remaining;
-      // The two barriers at the top of the next pass order these reads before
-      // the next write of sh_bin / sh_remaining.
+      if (shift == 0) whole_bin = false;  // all 32 bits fixed: `remaining` counts keys equal to the threshold
+    }
+    if (whole_bin && prefix != 0) {
+      // every key that starts with `prefix` is a winner: they all compare above prefix - 1,
+      // and nothing else does except the keys of higher bins
+      thr = prefix - 1u;
+      remaining = 0;
+    } else {
+      thr = prefix;
     }
   }
   const bool take_all = (k_eff >= n_cand);
-  const uint32_t thr = prefix;
 
   // ---- phase 3: gather, sort, translate --------------------------------------
   const bool rank_sort = (k_eff <= kRankSortMax);
