@@ -45,7 +45,7 @@ class Gpu:
 
 
 def check_table(ops, g: Gpu):
-    ops.check_page_table(g.indices, g.indptr, g.last, PS, g.pb.num_pages)
+    ops.check_page_table(g.indices, g.indptr, g.last, g.pb.kv_cache.shape[2], g.pb.num_pages)
 
 
 def assert_out_close(got_bf16: torch.Tensor, want: np.ndarray, what=""):
@@ -1679,13 +1679,20 @@ def test_topk_zero_is_sink_plus_local_window(ops):
 # --------------------------------------------------------------------------- seeded sweep over odd shapes
 
 
-def test_seeded_sweep_of_shapes(ops):
-    """40 seeded random configurations -- head counts, group sizes 1..8, ragged
+@pytest.mark.parametrize("page_size,fmt,trials", [(16, "bf16", 40), (32, "bf16", 15), (64, "bf16", 10), (16, "f16", 15), (64, "f16", 10)])
+def test_seeded_sweep_of_shapes(ops, page_size, fmt, trials):
+    """Seeded random configurations -- head counts, group sizes 1..8, ragged
     lengths with empty and one-token sequences, budgets above and below the
     candidate count, pinned pages, table layouts, split counts, both step
-    paths -- each checked end to end against the oracle."""
-    rng = np.random.default_rng(2024)
-    for trial in range(40):
+    paths -- each checked end to end against the oracle, at each page size and
+    element format."""
+    with O.element_format(fmt):
+        _sweep_of_shapes(ops, page_size, trials, 2024 + page_size + (7 if fmt == "f16" else 0))
+
+
+def _sweep_of_shapes(ops, PS, trials, seed):
+    rng = np.random.default_rng(seed)
+    for trial in range(trials):
         hkv = int(rng.choice([1, 1, 2, 3, 4, 8]))
         group = int(rng.integers(1, 9))
         B = int(rng.integers(1, 7))
@@ -1706,8 +1713,8 @@ def test_seeded_sweep_of_shapes(ops):
         table = str(rng.choice(["random", "fragmented"]))
         fused = bool(rng.integers(0, 2))
         splits = int(rng.choice([0, 1, 2, 5]))
-        what = f"trial {trial}: hkv={hkv} G={group} lengths={lengths} topk={topk} sink={sink} local={local} offset={offset} {table} fused={fused} splits={splits}"
-        pb = P.make_problem(3000 + trial, lengths, num_kv_heads=hkv, group=group, topk=topk, table=table)
+        what = f"ps={PS} trial {trial}: hkv={hkv} G={group} lengths={lengths} topk={topk} sink={sink} local={local} offset={offset} {table} fused={fused} splits={splits}"
+        pb = P.make_problem(3000 + trial, lengths, num_kv_heads=hkv, group=group, topk=topk, table=table, page_size=PS)
         g = Gpu(pb)
         g.sel = torch.full((pb.B, hkv, ops.sel_list_capacity(topk, sink, local)), -7, dtype=torch.int32, device=DEV)
         check_table(ops, g)
@@ -1719,7 +1726,7 @@ def test_seeded_sweep_of_shapes(ops):
         else:
             ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
             ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, topk, g.sel, g.cnt, sink_pages=sink,
-                                 local_tokens=local)
+                                 local_tokens=local, page_size=PS)
             out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, lse=lse, num_splits=splits,
                                           first_page_offset=offset)
         torch.cuda.synchronize()
@@ -1736,7 +1743,7 @@ def test_seeded_sweep_of_shapes(ops):
                 pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
                 if len(pages) == 0:
                     continue
-                n_sink = O.split_pages(len(pages), pb.last_page_len[b], sink, local, pb.kbar.shape[2])[0]
+                n_sink = O.split_pages(len(pages), pb.last_page_len[b], sink, local, pb.kbar.shape[2], PS)[0]
                 lookup = {int(p): i for i, p in enumerate(pages)}
                 for h in range(hkv):
                     k_eff = len(res["sel_logical"][b][h])
