@@ -396,6 +396,10 @@ def side_workload(torch, ops, name, steps, warmup, device, with_dense=True):
            "achieved_gbs": ab["step"] / (ms_step * 1e-3) / 1e9, "frac": ab["step"] / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
     if fused:
         out["kernel_frac"] = ab["step"] / (kernel_ms["fused_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS
+        tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+        if os.path.exists(tpath):   # rocprofv3 counters of an earlier run of the same kernel and workload, not of this run
+            with open(tpath) as f:
+                out["traffic"] = json.load(f).get(f"{name}:B={B}", {}).get("blocktopk_step_kernel")
     if with_dense:
         td = time_dense(torch, ops, st, max(3, min(10, steps // 10)))
         out["dense_ms_per_step"] = td
