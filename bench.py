@@ -30,6 +30,8 @@ benchmark/blocktopk.py:82).
 from __future__ import annotations
 
 import argparse
+import contextlib
+import gc
 import json
 import os
 import statistics
@@ -281,6 +283,24 @@ def cpu_model_name():
     return "unknown"
 
 
+LAST_LAUNCH_MS = []
+
+
+@contextlib.contextmanager
+def collector_paused():
+    """A timed loop without the interpreter's cyclic collector (as timeit does): a
+    full collection that lands between two launches stalls the host for tens of
+    milliseconds, and the GPU idles through it inside the timed K steps."""
+    was = gc.isenabled()
+    gc.collect()
+    gc.disable()
+    try:
+        yield
+    finally:
+        if was:
+            gc.enable()
+
+
 def time_step(torch, ops, st, B, Hkv, topk, steps, warmup, mode="auto"):
     """W untimed and K timed decode steps on the state ``st``; HIP events on the
     launch stream bracket every kernel.  Returns (ms_per_step, elapsed_s,
@@ -309,16 +329,19 @@ def time_step(torch, ops, st, B, Hkv, topk, steps, warmup, mode="auto"):
     torch.cuda.synchronize()
     K = steps
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(kernels) + 1)] for _ in range(K)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(K):
-        ev[i][0].record()
-        for j, (_, fn) in enumerate(kernels):
-            fn()
-            ev[i][j + 1].record()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    with collector_paused():
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(K):
+            ev[i][0].record()
+            for j, (_, fn) in enumerate(kernels):
+                fn()
+                ev[i][j + 1].record()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
     kernel_ms = {name: statistics.fmean(e[j].elapsed_time(e[j + 1]) for e in ev) for j, (name, _) in enumerate(kernels)}
+    global LAST_LAUNCH_MS
+    LAST_LAUNCH_MS = [round(sum(e[j].elapsed_time(e[j + 1]) for j in range(len(kernels))), 3) for e in ev]
     return elapsed / K * 1e3, elapsed, kernel_ms, fused
 
 
@@ -327,14 +350,15 @@ def time_dense(torch, ops, st, nd):
     for _ in range(2):
         ops.dense_paged_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], st["max_pages_used"],
                                out=st["out"], workspace=st["ws_dense"])
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(nd):
-        ops.append_paged_kv(st["k"], st["v"], st["kv"], None, st["indices"], st["indptr"], st["last"])
-        ops.dense_paged_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], st["max_pages_used"],
-                               out=st["out"], workspace=st["ws_dense"])
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) / nd * 1e3
+    with collector_paused():
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(nd):
+            ops.append_paged_kv(st["k"], st["v"], st["kv"], None, st["indices"], st["indptr"], st["last"])
+            ops.dense_paged_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], st["max_pages_used"],
+                                   out=st["out"], workspace=st["ws_dense"])
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / nd * 1e3
 
 
 def time_token_policies(torch, ops, st, B, Hkv, G, topk, nt, traffic_of):
@@ -361,14 +385,15 @@ def time_token_policies(torch, ops, st, B, Hkv, G, topk, nt, traffic_of):
             call()
         torch.cuda.synchronize()
         evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nt)]
-        t0 = time.perf_counter()
-        for e0, e1 in evs:
-            ops.append_paged_kv(st["k"], st["v"], st["kv"], None, st["indices"], st["indptr"], st["last"])
-            e0.record()
-            call()
-            e1.record()
-        torch.cuda.synchronize()
-        tt = (time.perf_counter() - t0) / nt
+        with collector_paused():
+            t0 = time.perf_counter()
+            for e0, e1 in evs:
+                ops.append_paged_kv(st["k"], st["v"], st["kv"], None, st["indices"], st["indptr"], st["last"])
+                e0.record()
+                call()
+                e1.record()
+            torch.cuda.synchronize()
+            tt = (time.perf_counter() - t0) / nt
         tks = [e0.elapsed_time(e1) for e0, e1 in evs]
         tk = statistics.fmean(tks) * 1e-3
         res[name] = {"sink_tokens": sink, "local_tokens": window, "ms_per_step": tt * 1e3, "value": B / tt,
@@ -387,6 +412,9 @@ def side_workload(torch, ops, name, steps, warmup, device, with_dense=True):
     st = build_state(torch, ops, B, ctx, Hkv, G, topk, device, ragged=name in RAGGED)
     torch.cuda.synchronize()
     ms_step, elapsed, kernel_ms, fused = time_step(torch, ops, st, B, Hkv, topk, steps, warmup)
+    print(f"[bench] {name}: kv at {hex(st['kv'].data_ptr())}, kbar at {hex(st['kbar'].data_ptr())}, "
+          f"{torch.cuda.memory_allocated() / 1e9:.1f} GB allocated, {torch.cuda.memory_reserved() / 1e9:.1f} GB reserved, "
+          f"step {ms_step:.4f} ms, launches {min(LAST_LAUNCH_MS):.3f}..{max(LAST_LAUNCH_MS):.3f} ms", file=sys.stderr, flush=True)
     ab = algorithmic_bytes(st["lengths"], Hkv, G, topk)
     out = {"description": desc, "batch": B, "ctx": ctx, "num_kv_heads": Hkv, "num_q_heads": Hkv * G, "topk_pages": topk,
            "page_table": "ragged, half fragmented" if name in RAGGED else "reference layout p*B+b",
@@ -405,8 +433,10 @@ def side_workload(torch, ops, name, steps, warmup, device, with_dense=True):
         out["dense_ms_per_step"] = td
         out["dense_frac"] = ab["dense"] / (td * 1e-3) / 1e9 / HBM_PEAK_GBS
         out["sparse_over_dense"] = td / ms_step
+    # No empty_cache() here: the allocator keeps the freed blocks, and the next workload's cache is
+    # carved from memory whose physical backing this process got first (returning it to the driver
+    # and allocating again lands on a slower backing, 3-9 % on these kernels).
     del st
-    torch.cuda.empty_cache()
     return out
 
 
@@ -512,7 +542,8 @@ def main():
     st = build_state(torch, ops, B, ctx, Hkv, G, topk, device, ragged=args.workload in RAGGED, PS=page, dtype=elem)
     torch.cuda.synchronize()
     print(f"[bench] {args.workload}: B={B} ctx={ctx} H_kv={Hkv} G={G} topk={topk}, "
-          f"KV {st['kv'].numel() * 2 / 1e9:.1f} GB resident, setup {time.perf_counter() - t_setup:.1f}s", file=sys.stderr)
+          f"KV {st['kv'].numel() * 2 / 1e9:.1f} GB resident at {hex(st['kv'].data_ptr())}, kbar at {hex(st['kbar'].data_ptr())}, "
+          f"setup {time.perf_counter() - t_setup:.1f}s", file=sys.stderr, flush=True)
 
     # -- the timed region: K steps; HIP events on the launch stream bracket each kernel
     K = args.steps
@@ -592,12 +623,15 @@ def main():
     if (args.token_topk or side) and page == PS and elem is torch.bfloat16:   # token-granular policies: 16-token pages, bf16
         result.update(time_token_policies(torch, ops, st, B, Hkv, G, topk, max(3, min(20, K // 5)), traffic_table.get))
     del st
-    torch.cuda.empty_cache()
+    if not side:
+        torch.cuda.empty_cache()
     if side:
         # every other BASELINE configuration in the same run, each on its own freshly built cache
+        # (carved from the blocks the headline cache has just left in the allocator)
         ks, ws = max(5, K), max(3, min(args.warmup, 10))
         result["workloads"] = {name: side_workload(torch, ops, name, ks, ws, device)
-                               for name in ("qwen3-32b-share", "qwen3-0.6b-mix", "qwen3-8b-readme", "qwen3-8b-tp1", "tiny")}
+                               for name in ("qwen3-8b-tp1", "qwen3-0.6b-mix", "qwen3-32b-share", "qwen3-8b-readme", "tiny")}
+        torch.cuda.empty_cache()
     if args.whole_layer and args.workload in WHOLE_LAYER_MODEL:
         result["whole_layer"] = whole_layer(torch, args, B, ctx, topk, device)
     if not args.no_cpu_baseline and Hkv == 1 and args.workload not in RAGGED:
