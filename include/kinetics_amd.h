@@ -41,7 +41,7 @@
  * Supported shapes: head_dim == 128; page_size 16, 32 or 64 (the reference's
  * --page_size, benchmark/blocktopk.py:13; the token-granular policies
  * kin_token_topk_decode / kin_strided_topk_decode: 16 only);
- * num_q_heads % num_kv_heads == 0 and group size num_q_heads/num_kv_heads <= 8.
+ * num_q_heads % num_kv_heads == 0 and group size num_q_heads/num_kv_heads <= 16.
  * Where a comment below says "16" for a page it means page_size.
  */
 #ifndef KINETICS_AMD_H

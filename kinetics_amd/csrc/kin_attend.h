@@ -24,7 +24,11 @@
 //      block = 4 lanes = one token row, A = p[g][t] (lane%4 = g), B = V[t][d]
 //      (d = 8*c + u), so values feed the matrix unit in the layout they were
 //      loaded in; P and V stay fp32.
-// Query groups larger than 4 run NG = 2 passes of the S / PV tiles per page.
+// Query groups larger than 4 run the "wide" form NG = 4 (up to 16 heads, see
+// page_scores_wide): the 16 columns of the S tile are 16 different heads and O += P V
+// runs on v_mfma_f32_16x16x4_f32, whose K dimension adds the wave's four row groups up
+// inside the matrix unit (same registers per lane as the narrow form, four times the
+// matrix cycles).
 #pragma once
 
 #include <cmath>
@@ -40,66 +44,54 @@ constexpr int kWaitVm4 = 4 | (7 << 4) | (15 << 8);
 constexpr float kNegInf = -INFINITY;
 constexpr float kLn2 = 0.6931471805599453f;
 
-// One page for one wave, first half: scores and the online softmax update.
+// One tile for one wave, first half: scores and the online softmax update, for
+// groups of up to 4 heads (NG = 1).
 // ka: this lane's 4 K chunks in MFMA A layout.  Leaves the probabilities of
 // this lane's 4 tokens in pr.  Requires 0 <= first_token <= 16 and
-// 0 <= valid_tokens <= 16 (an empty range masks the whole page).
-template <int NG, bool F16 = false>
-__device__ __forceinline__ void page_scores(const uint4 (&ka)[4], const uint4 (&qB)[NG][4], float (&m_run)[NG],
-                                            float (&l_run)[NG], floatx4 (&O)[NG][8], float (&pr)[NG][4],
-                                            float scale_log2, int first_token, int valid_tokens, int kg) {
-  floatx4 S[NG];
+// 0 <= valid_tokens <= 16 (an empty range masks the whole tile).
+template <bool F16 = false>
+__device__ __forceinline__ void page_scores(const uint4 (&ka)[4], const uint4 (&qB)[4], float& m_run, float& l_run,
+                                            floatx4 (&O)[8], float (&pr)[4], float scale_log2, int first_token,
+                                            int valid_tokens, int kg) {
+  floatx4 S = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int half = 0; half < NG; ++half) S[half] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int c = 0; c < 4; ++c) S = mfma_16x16x32<F16>(ka[c], qB[c], S);
+  float s[4];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
+  for (int r = 0; r < 4; ++r)  // token slots [first_token, valid_tokens) of the tile count
+    s[r] = ((unsigned)(4 * kg + r - first_token) < (unsigned)(valid_tokens - first_token)) ? S[r] * scale_log2 : kNegInf;
+  const float m_new = fmaxf(m_run, fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
+  if (__any(m_new > m_run)) {
+    const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
+    const float alpha = fast_exp2(m_run - m_safe);
+    l_run *= alpha;
+    const float a0 = quad_bcast<0>(alpha), a1 = quad_bcast<1>(alpha);
+    const float a2 = quad_bcast<2>(alpha), a3 = quad_bcast<3>(alpha);
 #pragma unroll
-    for (int half = 0; half < NG; ++half) S[half] = mfma_16x16x32<F16>(ka[c], qB[half][c], S[half]);
-  }
-#pragma unroll
-  for (int half = 0; half < NG; ++half) {
-    float s[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r)  // token slots [first_token, valid_tokens) of the page count
-      s[r] = ((unsigned)(4 * kg + r - first_token) < (unsigned)(valid_tokens - first_token)) ? S[half][r] * scale_log2
-                                                                                             : kNegInf;
-    const float m_new = fmaxf(m_run[half], fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
-    if (__any(m_new > m_run[half])) {
-      const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
-      const float alpha = fast_exp2(m_run[half] - m_safe);
-      l_run[half] *= alpha;
-      const float a0 = quad_bcast<0>(alpha), a1 = quad_bcast<1>(alpha);
-      const float a2 = quad_bcast<2>(alpha), a3 = quad_bcast<3>(alpha);
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        O[half][u][0] *= a0;
-        O[half][u][1] *= a1;
-        O[half][u][2] *= a2;
-        O[half][u][3] *= a3;
-      }
-      m_run[half] = m_new;
+    for (int u = 0; u < 8; ++u) {
+      O[u][0] *= a0;
+      O[u][1] *= a1;
+      O[u][2] *= a2;
+      O[u][3] *= a3;
     }
-    const float m_use = (m_run[half] == kNegInf) ? 0.f : m_run[half];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) pr[half][r] = fast_exp2(s[r] - m_use);
-    l_run[half] += (pr[half][0] + pr[half][1]) + (pr[half][2] + pr[half][3]);
+    m_run = m_new;
   }
+  const float m_use = (m_run == kNegInf) ? 0.f : m_run;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) pr[r] = fast_exp2(s[r] - m_use);
+  l_run += (pr[0] + pr[1]) + (pr[2] + pr[3]);
 }
 
 // Second half: O += P V.  vr: this lane's 4 V rows (row 4*kg + r).
-template <int NG, bool F16 = false>
-__device__ __forceinline__ void page_pv(const u32x4 (&vr)[4], const float (&pr)[NG][4], floatx4 (&O)[NG][8]) {
+template <bool F16 = false>
+__device__ __forceinline__ void page_pv(const u32x4 (&vr)[4], const float (&pr)[4], floatx4 (&O)[8]) {
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const u32x4 vv = vr[r];
     const float vf[8] = {elem_lo<F16>(vv.x), elem_hi<F16>(vv.x), elem_lo<F16>(vv.y), elem_hi<F16>(vv.y),
                          elem_lo<F16>(vv.z), elem_hi<F16>(vv.z), elem_lo<F16>(vv.w), elem_hi<F16>(vv.w)};
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-#pragma unroll
-      for (int half = 0; half < NG; ++half)
-        O[half][u] = __builtin_amdgcn_mfma_f32_4x4x1f32(pr[half][r], vf[u], O[half][u], 0, 0, 0);
-    }
+    for (int u = 0; u < 8; ++u) O[u] = __builtin_amdgcn_mfma_f32_4x4x1f32(pr[r], vf[u], O[u], 0, 0, 0);
   }
 }
 
@@ -111,6 +103,69 @@ __device__ __forceinline__ void clear_unused_v_rows(u32x4 (&vr)[4], int first_to
 #pragma unroll
   for (int r = 0; r < 4; ++r)
     if (!((unsigned)(4 * kg + r - first_token) < (unsigned)(valid_tokens - first_token))) vr[r] = u32x4{0u, 0u, 0u, 0u};
+}
+
+// NG names the kernel variant by the heads it holds, 4 * NG: 1 (narrow) or 4 (wide).
+template <int NG>
+constexpr bool attend_variant_ok() { return NG == 1 || NG == 4; }
+
+// The wide form of page_scores(): qB holds head min(l%16, G-1) in column l%16, so
+// lane (kg, c16) ends up with S[head c16][token 4*kg + r].  The running maximum of a
+// head is kept equal in the four lanes (kg = 0..3) that share it, because the P V
+// product below adds their tokens up inside one matrix instruction: it moves only
+// when some token of the tile exceeds it (rare once a list is under way), and only
+// then do the lanes exchange their maxima and rescale O.
+template <bool F16 = false>
+__device__ __forceinline__ void page_scores_wide(const uint4 (&ka)[4], const uint4 (&qB)[4], float& m_run, float& l_run,
+                                                 floatx4 (&O)[8], float (&pr)[4], float scale_log2, int first_token,
+                                                 int valid_tokens, int kg) {
+  floatx4 S = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int c = 0; c < 4; ++c) S = mfma_16x16x32<F16>(ka[c], qB[c], S);
+  float s[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    s[r] = ((unsigned)(4 * kg + r - first_token) < (unsigned)(valid_tokens - first_token)) ? S[r] * scale_log2 : kNegInf;
+  const float m_loc = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+  if (__any(m_loc > m_run)) {
+    float mt = fmaxf(m_loc, __shfl_xor(m_loc, 16));
+    mt = fmaxf(mt, __shfl_xor(mt, 32));
+    const float m_new = fmaxf(m_run, mt);
+    const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
+    const float alpha = fast_exp2(m_run - m_safe);
+    l_run *= alpha;
+    // This lane's O rows are heads 4*kg + 0..3; their factors sit in the lanes whose column is that head.
+    const int src = (threadIdx.x & 48) + 4 * kg;
+    const float a0 = __shfl(alpha, src), a1 = __shfl(alpha, src + 1);
+    const float a2 = __shfl(alpha, src + 2), a3 = __shfl(alpha, src + 3);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      O[u][0] *= a0;
+      O[u][1] *= a1;
+      O[u][2] *= a2;
+      O[u][3] *= a3;
+    }
+    m_run = m_new;
+  }
+  const float m_use = (m_run == kNegInf) ? 0.f : m_run;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) pr[r] = fast_exp2(s[r] - m_use);
+  l_run += (pr[0] + pr[1]) + (pr[2] + pr[3]);
+}
+
+// O += P V, wide form: A[i = head l%16][k = l/16] = p of token 4*kg + r, B[k = l/16][j = l%16] =
+// V[token 4*kg + r][8*(l%16) + u]; the instruction's K = 4 adds the four row groups, so lane
+// (kg, c16) accumulates O[head 4*kg + reg][d = 8*c16 + u] over all 16 tokens of the tile.
+template <bool F16 = false>
+__device__ __forceinline__ void page_pv_wide(const u32x4 (&vr)[4], const float (&pr)[4], floatx4 (&O)[8]) {
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const u32x4 vv = vr[r];
+    const float vf[8] = {elem_lo<F16>(vv.x), elem_hi<F16>(vv.x), elem_lo<F16>(vv.y), elem_hi<F16>(vv.y),
+                         elem_lo<F16>(vv.z), elem_hi<F16>(vv.z), elem_lo<F16>(vv.w), elem_hi<F16>(vv.w)};
+#pragma unroll
+    for (int u = 0; u < 8; ++u) O[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(pr[r], vf[u], O[u], 0, 0, 0);
+  }
 }
 
 // Wave-uniform description of one list for attend_list().
@@ -130,68 +185,76 @@ struct AttendArgs {
   int first_skip;        // leading token slots of list entry 0 that hold no token (0 .. page_size-1)
 };
 
-// K pages a wave keeps staged in LDS in attend_list(): the one being read and 1 or
-// 2 in flight.  The two-pass kernel for groups above 4 runs only 2 waves per SIMD
-// (200 registers), so it keeps one more page (and one more V register set) in
-// flight per wave to cover the memory latency.
-constexpr int attend_k_stages(int ng) { return ng == 1 ? 2 : 3; }
-// K staging for NW waves of `stages` 4 KiB stages each; also large enough for the
-// merge buffer [NW][4*NG][128] fp32 (NG <= 2).
-constexpr int attend_lds_bytes(int nw, int stages = 2) { return nw * stages * 4096; }
-// s_waitcnt immediate for "vmcnt <= 16" (vmcnt[3:0] = 0, vmcnt_hi[15:14] = 1).
-constexpr int kWaitVm16 = 0 | (7 << 4) | (15 << 8) | (1 << 14);
+// K tiles a wave keeps staged in LDS in attend_list(): the one being read and the one in flight.
+constexpr int kAttendStages = 2;
+// K staging for NW waves of kAttendStages 4 KiB stages each; the same 8 KiB per wave hold the
+// merge buffer [NW][4*NG][128] fp32 afterwards (2 KiB per wave for NG = 1, 8 KiB for the wide form).
+constexpr int attend_lds_bytes(int nw) { return nw * kAttendStages * 4096; }
 
 // Common tail of the attention loops: merges the wave's 4 row groups, then the
 // workgroup's NW waves through LDS, and hands out the normalised results.
 // m_run / l_run / O: this lane's online-softmax state (see page_scores).
 template <int NG, int NW, typename Emit>
-__device__ __forceinline__ void attend_finish(float (&m_run)[NG], float (&l_run)[NG], floatx4 (&O)[NG][8], int G,
-                                              unsigned char* lds, float (*sm_m)[4 * NG], float (*sm_l)[4 * NG],
-                                              Emit emit) {
+__device__ __forceinline__ void attend_finish(float m_run, float l_run, floatx4 (&O)[8], int G, unsigned char* lds,
+                                              float (*sm_m)[4 * NG], float (*sm_l)[4 * NG], Emit emit) {
+  static_assert(attend_variant_ok<NG>(), "NG is 1 (up to 4 heads) or 4 (up to 16)");
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l = tid & 63, kg = l >> 4, c16 = l & 15;
   // LDS-direct loads that are still in flight (masked tail pages) must land
   // before the staging area is reused below.
   __builtin_amdgcn_s_waitcnt(0);
+  float* ow = reinterpret_cast<float*>(lds);  // [NW waves][4*NG heads][128]
 
-  // ---- merge the 4 row groups of the wave (lanes l, l^16, l^32, l^48) --------
-  float m_w[NG], l_w[NG];
+  if constexpr (NG == 4) {
+    // Wide form: O is already summed over the row groups; the lanes of a head share m
+    // and hold partial sums l.
+    float ll = l_run;
+    ll += __shfl_xor(ll, 16);
+    ll += __shfl_xor(ll, 32);
+    __syncthreads();  // every wave is done with its K staging area
 #pragma unroll
-  for (int half = 0; half < NG; ++half) {
-    float mm = m_run[half];
+    for (int i = 0; i < 4; ++i) {
+      const int h = 4 * kg + i;
+      if (h < G) {
+        float* dst = ow + ((w * 16 + h) * kHeadDim + 8 * c16);
+        *reinterpret_cast<float4*>(dst) = make_float4(O[0][i], O[1][i], O[2][i], O[3][i]);
+        *reinterpret_cast<float4*>(dst + 4) = make_float4(O[4][i], O[5][i], O[6][i], O[7][i]);
+      }
+    }
+    if (l < 16) {
+      sm_m[w][l] = m_run;
+      sm_l[w][l] = ll;
+    }
+  } else {
+    // ---- merge the 4 row groups of the wave (lanes l, l^16, l^32, l^48) --------
+    float mm = m_run;
     mm = fmaxf(mm, __shfl_xor(mm, 16));
     mm = fmaxf(mm, __shfl_xor(mm, 32));
     const float m_safe = (mm == kNegInf) ? 0.f : mm;
-    const float sc = fast_exp2(m_run[half] - m_safe);
-    float ll = l_run[half] * sc;
+    const float sc = fast_exp2(m_run - m_safe);
+    float ll = l_run * sc;
     ll += __shfl_xor(ll, 16);
     ll += __shfl_xor(ll, 32);
-    m_w[half] = mm;
-    l_w[half] = ll;
     const float s0 = quad_bcast<0>(sc), s1 = quad_bcast<1>(sc), s2 = quad_bcast<2>(sc), s3 = quad_bcast<3>(sc);
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      float x0 = O[half][u][0] * s0, x1 = O[half][u][1] * s1, x2 = O[half][u][2] * s2, x3 = O[half][u][3] * s3;
+      float x0 = O[u][0] * s0, x1 = O[u][1] * s1, x2 = O[u][2] * s2, x3 = O[u][3] * s3;
       x0 += __shfl_xor(x0, 16); x1 += __shfl_xor(x1, 16); x2 += __shfl_xor(x2, 16); x3 += __shfl_xor(x3, 16);
       x0 += __shfl_xor(x0, 32); x1 += __shfl_xor(x1, 32); x2 += __shfl_xor(x2, 32); x3 += __shfl_xor(x3, 32);
-      O[half][u] = floatx4{x0, x1, x2, x3};
+      O[u] = floatx4{x0, x1, x2, x3};
     }
-  }
-  __syncthreads();  // every wave is done with its K staging area
-  float* ow = reinterpret_cast<float*>(lds);  // [NW waves][4*NG heads][128]
-  if (kg == 0) {
-#pragma unroll
-    for (int half = 0; half < NG; ++half) {
+    __syncthreads();  // every wave is done with its K staging area
+    if (kg == 0) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float* dst = ow + ((w * 4 * NG + 4 * half + i) * kHeadDim + 8 * c16);
-        *reinterpret_cast<float4*>(dst) = make_float4(O[half][0][i], O[half][1][i], O[half][2][i], O[half][3][i]);
-        *reinterpret_cast<float4*>(dst + 4) = make_float4(O[half][4][i], O[half][5][i], O[half][6][i], O[half][7][i]);
+        float* dst = ow + ((w * 4 + i) * kHeadDim + 8 * c16);
+        *reinterpret_cast<float4*>(dst) = make_float4(O[0][i], O[1][i], O[2][i], O[3][i]);
+        *reinterpret_cast<float4*>(dst + 4) = make_float4(O[4][i], O[5][i], O[6][i], O[7][i]);
       }
       if (l < 4) {
-        sm_m[w][4 * half + l] = m_w[half];
-        sm_l[w][4 * half + l] = l_w[half];
+        sm_m[w][l] = mm;
+        sm_l[w][l] = ll;
       }
     }
   }
@@ -222,7 +285,7 @@ __device__ __forceinline__ void attend_finish(float (&m_run)[NG], float (&l_run)
 // id_at(i) returns the (wave-uniform) physical page id of list entry i, 0 <= i < n.
 // emit(g, d, o, lse2) receives, once per (head g < G, column d), the normalised
 // output and the base-2 log-sum-exp (-inf and o = 0 for an empty part).
-// lds: attend_lds_bytes(NW, attend_k_stages(NG)), 16-byte aligned; sm_m / sm_l: NW x
+// lds: attend_lds_bytes(NW), 16-byte aligned; sm_m / sm_l: NW x
 // (4*NG) floats each.
 // Every one of the workgroup's NW*64 threads calls this.
 template <int NG, int NW, bool F16 = false, typename IdAt, typename Emit>
@@ -234,15 +297,13 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
   const int G = a.G;
   const int n = a.n, p0 = a.p0, p1 = a.p1, last_len = a.last_len;
 
-  // Query operands: B[k][j], j = l%16 -> head 4*half + l%4, k-chunk = l/16.
-  uint4 qB[NG][4];
-#pragma unroll
-  for (int half = 0; half < NG; ++half) {
-    const int g = min(4 * half + gq, G - 1);
+  // Query operands: B[k][j], j = l%16 -> head l%4 (wide form: head l%16), k-chunk = l/16.
+  uint4 qB[4];
+  {
+    const int g = min(NG == 4 ? c16 : gq, G - 1);
     const uint16_t* qp = a.q_bh + (int64_t)g * kHeadDim + 8 * kg;
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
-      qB[half][c] = *reinterpret_cast<const uint4*>(qp + 32 * c);
+    for (int c = 0; c < 4; ++c) qB[c] = *reinterpret_cast<const uint4*>(qp + 32 * c);
   }
 
   const int row_bytes = a.row_bytes;
@@ -255,12 +316,11 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
   int voff[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c) voff[c] = (a.page_size + 4 * kg + c) * row_bytes + c16 * 16;
-  // K staging: KS 4 KiB stages per wave, filled by LDS-direct buffer loads
+  // K staging: kAttendStages 4 KiB stages per wave, filled by LDS-direct buffer loads
   // (no VGPRs while in flight).  Load c brings rows 4c..4c+3: lane (kg, c16)
   // lands at LDS row 4c+kg, position c16, and fetches the chunk that belongs
   // there under the XOR swizzle (position p of row R holds chunk p ^ R).
-  constexpr int KS = attend_k_stages(NG);
-  unsigned char* kl = lds + w * (KS * 4096);
+  unsigned char* kl = lds + w * (kAttendStages * 4096);
   int kdma_off[4], lds_r[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
@@ -270,15 +330,22 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
     lds_r[c] = c16 * 256 + ((chunk_r ^ c16) & 15) * 16;
   }
 
-  float m_run[NG], l_run[NG];
-  floatx4 O[NG][8];
+  float m_run = kNegInf, l_run = 0.f;
+  floatx4 O[8];
 #pragma unroll
-  for (int half = 0; half < NG; ++half) {
-    m_run[half] = kNegInf;
-    l_run[half] = 0.f;
-#pragma unroll
-    for (int u = 0; u < 8; ++u) O[half][u] = floatx4{0.f, 0.f, 0.f, 0.f};
-  }
+  for (int u = 0; u < 8; ++u) O[u] = floatx4{0.f, 0.f, 0.f, 0.f};
+  auto scores = [&](const uint4 (&ka)[4], float (&pr)[4], int valid) {
+    if constexpr (NG == 4)
+      page_scores_wide<F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, valid >> 8, valid & 255, kg);
+    else
+      page_scores<F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, valid >> 8, valid & 255, kg);
+  };
+  auto pv = [&](const u32x4 (&vr)[4], const float (&pr)[4]) {
+    if constexpr (NG == 4)
+      page_pv_wide<F16>(vr, pr, O);
+    else
+      page_pv<F16>(vr, pr, O);
+  };
 
   // This wave takes the tiles my_first, my_first+NW, ... of the list entries p0 .. p1-1
   // (entry e owns the tiles e << tshift ..; of the list's final page only the tiles
@@ -332,61 +399,10 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
   // before it are allowed to be outstanding, which means the K stage about to
   // be read (and the V registers about to be used) have landed.  The scheduling
   // fences keep the instruction order this count relies on.
-  if constexpr (KS == 3) {
-    // Three stages: K runs three pages ahead of the one being read, V two.  Issue
-    // order in steady state is ... V(p+1), K(p+2), V(p+2) | wait | read K(p), scores,
-    // K(p+3) ..., so at the wait the loads allowed to be outstanding are K and V of
-    // pages p+1 and p+2: 16 of them; everything older (page p) has landed.  (The
-    // compiler, which sees the LDS reads, tightens this wait to "every LDS-direct
-    // load issued so far", i.e. vmcnt(4); hiding the reads from it in inline
-    // assembly restores vmcnt(16) but was not measurably faster.)
-    if (iters > 0 && n > 0) {
-      u32x4 v[3][4];
-      uint4 ka[4];
-      float pr[NG][4];
-      int valid[3];
-      __amdgpu_buffer_rsrc_t r_v;  // descriptor of the page whose V is issued next
-      {
-        const __amdgpu_buffer_rsrc_t r0 = page_rsrc(0, load_id(0), valid[0]);
-        issue_k(r0, 0);
-        issue_v(r0, v[0]);
-        const __amdgpu_buffer_rsrc_t r1 = page_rsrc(1, load_id(1), valid[1]);
-        issue_k(r1, 1);
-        issue_v(r1, v[1]);
-        r_v = page_rsrc(2, load_id(2), valid[2]);
-        issue_k(r_v, 2);
-      }
-      int id_next = load_id(3);
-      for (int it = 0; it < iters; it += 3) {
-#pragma unroll
-        for (int s3 = 0; s3 < 3; ++s3) {
-          const int cur_valid = valid[s3];
-          __builtin_amdgcn_sched_barrier(0);
-          issue_v(r_v, v[(s3 + 2) % 3]);
-          __builtin_amdgcn_sched_barrier(0);
-          __builtin_amdgcn_s_waitcnt(kWaitVm16);
-          __builtin_amdgcn_sched_barrier(0);
-          read_k(s3, ka);
-          __builtin_amdgcn_sched_barrier(0);
-          page_scores<NG, F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, cur_valid >> 8, cur_valid & 255, kg);
-          __builtin_amdgcn_sched_barrier(0);
-          // The stage just read is refilled only now that the matrix unit has consumed
-          // it: a load through an empty descriptor (a masked page) returns at once
-          // and would otherwise overtake LDS reads that are still queued.
-          r_v = page_rsrc(it + s3 + 3, id_next, valid[s3]);
-          issue_k(r_v, s3);
-          __builtin_amdgcn_sched_barrier(0);
-          id_next = load_id(it + s3 + 4);  // lands while the P V products run
-          if (cur_valid != kPageSize) clear_unused_v_rows(v[s3], cur_valid >> 8, cur_valid & 255, kg);
-          page_pv<NG, F16>(v[s3], pr, O);
-        }
-      }
-    }
-  } else
   if (iters > 0 && n > 0) {
     u32x4 vA[4], vB[4];
     uint4 ka[4];
-    float pr[NG][4];
+    float pr[4];
     int validA, validB;
     {
       const __amdgpu_buffer_rsrc_t r0 = page_rsrc(0, load_id(0), validA);
@@ -406,11 +422,11 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
         __builtin_amdgcn_sched_barrier(0);
         issue_k(r1, 1);
         __builtin_amdgcn_sched_barrier(0);
-        page_scores<NG, F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validA >> 8, validA & 255, kg);
+        scores(ka, pr, validA);
         __builtin_amdgcn_sched_barrier(0);
         id_next = load_id(it + 2);  // lands while the P V products run
         if (validA != kPageSize) clear_unused_v_rows(vA, validA >> 8, validA & 255, kg);  // partial page: rare
-        page_pv<NG, F16>(vA, pr, O);
+        pv(vA, pr);
       }
       {
         const __amdgpu_buffer_rsrc_t r2 = page_rsrc(it + 2, id_next, validA);
@@ -423,11 +439,11 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
         __builtin_amdgcn_sched_barrier(0);
         issue_k(r2, 0);
         __builtin_amdgcn_sched_barrier(0);
-        page_scores<NG, F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, validB >> 8, validB & 255, kg);
+        scores(ka, pr, validB);
         __builtin_amdgcn_sched_barrier(0);
         id_next = load_id(it + 3);
         if (validB != kPageSize) clear_unused_v_rows(vB, validB >> 8, validB & 255, kg);
-        page_pv<NG, F16>(vB, pr, O);
+        pv(vB, pr);
       }
     }
   }

@@ -12,7 +12,7 @@ constexpr int kHeadDim = 128;    // elements per head row (256 B in bf16)
 constexpr int kPageSize = 16;    // tokens of one attention tile (an MFMA tile is 16 keys); the smallest page
 constexpr int kMaxPageSize = 64; // pages hold 16, 32 or 64 tokens: 1, 2 or 4 tiles
 constexpr int kRowBytes = kHeadDim * 2;
-constexpr int kMaxGroup = 8;     // largest supported num_q_heads / num_kv_heads
+constexpr int kMaxGroup = 16;    // largest supported num_q_heads / num_kv_heads
 constexpr int kMaxTopk = 2048;
 constexpr int kMaxCandidates = 16384;
 constexpr int kNumCus = 256;     // compute units of the target GPU (MI355X)

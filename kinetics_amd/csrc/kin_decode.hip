@@ -28,7 +28,7 @@ struct DecodeParams {
 
 template <int NG, bool F16>
 __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
-  __shared__ __attribute__((aligned(16))) unsigned char lds[attend_lds_bytes(4, attend_k_stages(NG))];
+  __shared__ __attribute__((aligned(16))) unsigned char lds[attend_lds_bytes(4)];
   __shared__ float sm_m[4][4 * NG];
   __shared__ float sm_l[4][4 * NG];
 
@@ -154,8 +154,8 @@ static int launch_decode(const char* fn, DecodeParams& p, int batch, void* works
     if (f16) paged_decode_kernel<1, true><<<grid, 256, 0, stream>>>(p);
     else paged_decode_kernel<1, false><<<grid, 256, 0, stream>>>(p);
   } else {
-    if (f16) paged_decode_kernel<2, true><<<grid, 256, 0, stream>>>(p);
-    else paged_decode_kernel<2, false><<<grid, 256, 0, stream>>>(p);
+    if (f16) paged_decode_kernel<4, true><<<grid, 256, 0, stream>>>(p);
+    else paged_decode_kernel<4, false><<<grid, 256, 0, stream>>>(p);
   }
   int st = check_hip(hipGetLastError(), "paged_decode_kernel launch");
   if (st) return st;

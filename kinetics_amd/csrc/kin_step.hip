@@ -241,8 +241,8 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
   p.first_page_offset = first_page_offset;
   p.page_size = page_size;
   p.sort_cap = select_sort_cap(topk, kbar_pages);
-  // Waves per workgroup: aim for 16 waves per CU (8 with the two-pass kernel for
-  // groups above 4, whose registers allow no more) when the lists are few.
+  // Waves per workgroup: aim for 16 waves per CU (8 with the wide kernel for groups
+  // above 4, which holds a few registers too many for 16) when the lists are few.
   const int64_t items = (int64_t)batch * num_kv_heads;
   if (xcd_grid_size(batch, num_kv_heads) > 0x7fffffffLL)
     return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
@@ -263,7 +263,7 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
     p.ws_keys = nullptr;
   }
   const size_t sel_scratch = select_lds_bytes(kbar_pages, p.sort_cap);
-  const size_t attend_bytes = (size_t)attend_lds_bytes(nw, attend_k_stages(p.group <= 4 ? 1 : 2));
+  const size_t attend_bytes = (size_t)attend_lds_bytes(nw);
   size_t region0 = sel_scratch > attend_bytes ? sel_scratch : attend_bytes;
   region0 = (region0 + 15) & ~(size_t)15;
   p.region0_bytes = (int)region0;
@@ -279,16 +279,16 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
                : nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 8, true>)
                          : reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 4, true>);
     else
-      kernel = nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<2, 8, true>)
-                       : reinterpret_cast<const void*>(&blocktopk_step_kernel<2, 4, true>);
+      kernel = nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<4, 8, true>)
+                       : reinterpret_cast<const void*>(&blocktopk_step_kernel<4, 4, true>);
   } else {
     if (p.group <= 4)
       kernel = nw == 16  ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 16, false>)
                : nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 8, false>)
                          : reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 4, false>);
     else
-      kernel = nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<2, 8, false>)
-                       : reinterpret_cast<const void*>(&blocktopk_step_kernel<2, 4, false>);
+      kernel = nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<4, 8, false>)
+                       : reinterpret_cast<const void*>(&blocktopk_step_kernel<4, 4, false>);
   }
   if (lds > 48 * 1024) {
     // Above the default dynamic-LDS allowance the runtime wants an explicit opt-in.

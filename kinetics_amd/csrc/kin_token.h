@@ -6,7 +6,8 @@
 //       q_g . k_t is (mean_g q_g) . k_t, one fp32 dot product per token) and
 //       turns the score of every token of the "dynamic" part (after the sink
 //       tokens, before the local window) into an order-preserving 32-bit key in
-//       an HBM scratch array;
+//       a key array: in LDS when the sequence's keys fit there beside the token
+//       list (LDSK = true; up to ~34 K tokens), else in an HBM scratch array;
 //   token_select_list()   radix-selects the k-th largest key and compacts the
 //       winners, in ascending token order, into a token list in LDS: sink
 //       tokens, winners, local-window tokens;
@@ -16,8 +17,10 @@
 //       attend_list() with one address per token row instead of one per page.
 //
 // HBM-bound on the key stream: 256 B per context token, plus 512 B per listed
-// token; the scratch keys (4 B per token, written and read back at device scope
-// so that several workgroups can share the scoring of one sequence) add about 5 %.
+// token.  Keys in HBM (4 B per token, written and read back at device scope so
+// that several workgroups can share the scoring of one sequence) add 5 % of traffic
+// and, interleaved with a saturated read stream, up to 14 % of time; keys in LDS
+// cost neither.
 #pragma once
 
 #include "kin_attend.h"
@@ -44,6 +47,7 @@ struct TokenArgs {
   int n_sink, n_dyn, n_local;  // tokens: always attended / candidates / always attended
   int topk;
   uint32_t* keys;        // HBM scratch, n_pages * 16 entries, 16-byte aligned
+  uint32_t* lds_keys;    // LDSK kernels: the same array in LDS, n_pages * 16 + 4 entries (the last 4: a dump slot)
   int32_t* list;         // LDS, >= n_sink + min(topk, n_dyn) + n_local entries
   int32_t* sel_tokens;   // HBM, the listed tokens' positions in the sequence, or null
   unsigned rotate;       // where in its page range this list starts streaming (any value)
@@ -83,20 +87,36 @@ constexpr int kSelLoads = 16;
 
 // Chunk c0 of the key array -> registers: wave w holds the 1024 * kSelLoads / 4
 // consecutive keys from c0 + w * 256 * kSelLoads, load u the keys 256 * u + 4 * lane
-// + 0..3 of them (so wave, u, lane, j ascending is index ascending).  keys covers
-// exactly the n_keys (a multiple of 4) keys: entries past them read as 0, "not a
-// candidate".  Device-scope loads: the keys may come from workgroups on other XCDs.
-template <int NW>
-__device__ __forceinline__ void load_key_chunk(__amdgpu_buffer_rsrc_t keys, int c0, u32x4 (&kk)[kSelLoads]) {
+// + 0..3 of them (so wave, u, lane, j ascending is index ascending).  keys (GlobalKeys
+// or LdsKeys below) covers exactly the n_keys (a multiple of 4) keys: entries past
+// them read as 0, "not a candidate".
+template <int NW, typename Keys>
+__device__ __forceinline__ void load_key_chunk(const Keys& keys, int c0, u32x4 (&kk)[kSelLoads]) {
   const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), l = threadIdx.x & 63;
   const int base = c0 + w * (256 * kSelLoads) + 4 * l;
 #pragma unroll
-  for (int u = 0; u < kSelLoads; ++u) kk[u] = __builtin_amdgcn_raw_buffer_load_b128(keys, (base + u * 256) * 4, 0, kDeviceScope);
+  for (int u = 0; u < kSelLoads; ++u) kk[u] = keys(base + u * 256);
 }
 
+// Where the select reads its keys: four consecutive keys from index i (a multiple
+// of 4), zeros past the end.
+struct GlobalKeys {  // device-scope loads through a descriptor over exactly the keys
+  __amdgpu_buffer_rsrc_t rsrc;
+  __device__ __forceinline__ u32x4 operator()(int i) const {
+    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, i * 4, 0, kDeviceScope);
+  }
+};
+struct LdsKeys {  // 16-byte aligned LDS array of n (a multiple of 4) keys
+  const uint32_t* keys;
+  int n;
+  __device__ __forceinline__ u32x4 operator()(int i) const {
+    return i < n ? *reinterpret_cast<const u32x4*>(keys + i) : u32x4{0u, 0u, 0u, 0u};
+  }
+};
+
 // Most-significant-digit-first radix select over n_keys (a multiple of 16) 32-bit
-// keys in global memory (a descriptor over exactly those keys, written at device
-// scope), run by a workgroup of NW waves, followed by the ordered
+// keys in global memory (GlobalKeys: a descriptor over exactly those keys, written at
+// device scope) or in LDS (LdsKeys), run by a workgroup of NW waves, followed by the ordered
 // compaction of the winners: finds the k-th largest non-zero key (zero keys are
 // "not a candidate"; at least k >= 1 keys are non-zero), then calls emit(pos, index)
 // for every key above it and for the lowest-indexed keys equal to it that complete
@@ -106,8 +126,8 @@ __device__ __forceinline__ void load_key_chunk(__amdgpu_buffer_rsrc_t keys, int 
 // have completed (s_waitcnt + barrier, or the arrival counter of split scoring).
 // Up to NW * 4096 keys are loaded once and stay in registers through all passes;
 // longer arrays are walked in chunks of that size, one trip per chunk and pass.
-template <int NW, typename Emit>
-__device__ __forceinline__ void radix_select_emit(__amdgpu_buffer_rsrc_t keys, int n_keys, uint32_t k,
+template <int NW, typename Keys, typename Emit>
+__device__ __forceinline__ void radix_select_emit(const Keys& keys, int n_keys, uint32_t k,
                                                   bool first_digit_counted, KeySelectShared* sh, Emit emit) {
   constexpr int kChunk = NW * 256 * kSelLoads;
   const int tid = threadIdx.x;
@@ -357,18 +377,22 @@ __device__ __forceinline__ bool token_needs_scores(const TokenArgs& a) {
   return k_eff > 0 && k_eff < a.n_dyn;
 }
 
-// Scores the tokens of the pages pg0 <= p < pg1 into a.keys (device-scope stores;
-// 0 marks "not a candidate", order_key is never 0 for a finite score).  hist:
-// 256 zeroed LDS counters that receive the histogram of the keys' top byte, or
-// null.  No barrier inside; the stores are complete after s_waitcnt(0).
-template <int NW>
+// Scores the tokens of the pages pg0 <= p < pg1 into a.keys (device-scope stores) or,
+// LDSK, into a.lds_keys; 0 marks "not a candidate", order_key is never 0 for a finite
+// score.  hist: 256 zeroed LDS counters that receive the histogram of the keys' top
+// byte, or null.  No barrier inside; the stores are complete after s_waitcnt(0).
+template <int NW, bool LDSK = false>
 __device__ __forceinline__ void token_score_keys(const TokenArgs& a, int pg0, int pg1, uint32_t* hist) {
   const int dyn_lo = a.pad + a.n_sink, dyn_hi = dyn_lo + a.n_dyn;  // cache slots of the candidates
-  const __amdgpu_buffer_rsrc_t keys_rsrc = make_rsrc(a.keys, a.n_pages * kPageSize * 4);
+  const __amdgpu_buffer_rsrc_t keys_rsrc = make_rsrc(a.keys, LDSK ? 0 : a.n_pages * kPageSize * 4);
+  uint32_t* lds_keys = a.lds_keys;
+  const int dump = a.n_pages * kPageSize;  // lanes without a row write here
   stream_token_scores<NW>(a, pg0, pg1, [&](int c, float score, bool valid) {
     const uint32_t key = (c >= dyn_lo && c < dyn_hi) ? order_key(score) : 0u;
-    // lanes without a row store at an offset outside the descriptor: dropped by the hardware
-    __builtin_amdgcn_raw_buffer_store_b32(key, keys_rsrc, valid ? c * 4 : -1, 0, kDeviceScope);
+    if constexpr (LDSK)
+      lds_keys[valid ? c : dump] = key;
+    else  // lanes without a row store at an offset outside the descriptor: dropped by the hardware
+      __builtin_amdgcn_raw_buffer_store_b32(key, keys_rsrc, valid ? c * 4 : -1, 0, kDeviceScope);
     if (hist && valid && key) atomicAdd(&hist[key >> 24], 1u);
   });
 }
@@ -378,7 +402,7 @@ __device__ __forceinline__ void token_score_keys(const TokenArgs& a, int pg0, in
 // its length.  When token_needs_scores(), a.keys is complete and, if
 // first_digit_counted, sh->hist holds the histogram of the keys' top byte.  Every
 // thread of the workgroup calls this; it ends with a workgroup barrier.
-template <int NG, int NW>
+template <int NG, int NW, bool LDSK = false>
 __device__ __forceinline__ int token_select_list(const TokenArgs& a, KeySelectShared* sh, bool first_digit_counted) {
   constexpr int NT = NW * 64;
   const int tid = threadIdx.x;
@@ -389,8 +413,11 @@ __device__ __forceinline__ int token_select_list(const TokenArgs& a, KeySelectSh
   const int32_t* table = a.table;
 
   if (token_needs_scores(a)) {
-    radix_select_emit<NW>(make_rsrc(a.keys, n_keys * 4), n_keys, (uint32_t)k_eff, first_digit_counted, sh,
-                          [&](int pos, int c) { list[a.n_sink + pos] = c; });
+    auto put = [&](int pos, int c) { list[a.n_sink + pos] = c; };
+    if constexpr (LDSK)
+      radix_select_emit<NW>(LdsKeys{a.lds_keys, n_keys}, n_keys, (uint32_t)k_eff, first_digit_counted, sh, put);
+    else
+      radix_select_emit<NW>(GlobalKeys{make_rsrc(a.keys, n_keys * 4)}, n_keys, (uint32_t)k_eff, first_digit_counted, sh, put);
     __syncthreads();
     translate_slots<NT>(list, a.n_sink, k_eff, table, a.pad, a.sel_tokens);
   } else if (k_eff > 0) {
@@ -417,7 +444,7 @@ struct StridedArgs {
   int block;             // tokens per block
   int stride;            // tokens between block starts
   int topk_blocks;       // budget: 2 * topk_blocks blocks are chosen, at most topk_blocks * block tokens kept
-  float* scores;         // HBM scratch, n_pages * 16 entries
+  float* scores;         // HBM scratch, n_pages * 16 entries (LDSK kernels: TokenArgs::lds_keys holds them instead)
   uint32_t* block_keys;  // HBM scratch, >= n_pages * 16 entries, 16-byte aligned
   uint32_t* bitmap;      // LDS, one bit per candidate token: (n_dyn + 31) / 32 words
   int32_t* winners;      // LDS, room for 2 * topk_blocks block numbers
@@ -436,19 +463,26 @@ __device__ __forceinline__ bool strided_needs_scores(const TokenArgs& a, const S
   return 2 * sa.topk_blocks < num_blocks;  // otherwise every block is chosen
 }
 
-// fp32 scores of the tokens of the pages pg0 <= p < pg1 -> sa.scores (device-scope stores).
-template <int NW>
+// fp32 scores of the tokens of the pages pg0 <= p < pg1 -> sa.scores (device-scope
+// stores) or, LDSK, -> a.lds_keys (as bit patterns).
+template <int NW, bool LDSK = false>
 __device__ __forceinline__ void strided_score_tokens(const TokenArgs& a, const StridedArgs& sa, int pg0, int pg1) {
-  const __amdgpu_buffer_rsrc_t scores_rsrc = make_rsrc(sa.scores, a.n_pages * kPageSize * 4);
+  const __amdgpu_buffer_rsrc_t scores_rsrc = make_rsrc(sa.scores, LDSK ? 0 : a.n_pages * kPageSize * 4);
+  uint32_t* lds_scores = a.lds_keys;
+  const int dump = a.n_pages * kPageSize;
   stream_token_scores<NW>(a, pg0, pg1, [&](int c, float score, bool valid) {
-    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(score), scores_rsrc, valid ? c * 4 : -1, 0, kDeviceScope);
+    if constexpr (LDSK)
+      lds_scores[valid ? c : dump] = __float_as_uint(score);
+    else
+      __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(score), scores_rsrc, valid ? c * 4 : -1, 0, kDeviceScope);
   });
 }
 
 // Writes the token list to a.list (sink tokens, kept tokens in ascending order,
-// local tokens) and returns its length; sa.scores is complete when
-// strided_needs_scores().  Ends with a barrier.
-template <int NG, int NW>
+// local tokens) and returns its length; sa.scores (LDSK: a.lds_keys) is complete when
+// strided_needs_scores().  sa.winners may overlap the LDS scores: they are dead by the
+// time the winners are written.  Ends with a barrier.
+template <int NG, int NW, bool LDSK = false>
 __device__ __forceinline__ int strided_select_list(const TokenArgs& a, const StridedArgs& sa, KeySelectShared* sh) {
   constexpr int NT = NW * 64;
   __shared__ uint32_t wave_cnt[NW];
@@ -500,7 +534,8 @@ __device__ __forceinline__ int strided_select_list(const TokenArgs& a, const Str
           const int off = (dyn_lo + i * sa.stride) * 4;
           float sum = 0.f;
           for (int t = 0; t < sa.block; ++t)
-            sum += __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(scores_rsrc, off + t * 4, 0, kDeviceScope));
+            sum += LDSK ? __uint_as_float(a.lds_keys[(off >> 2) + t])
+                        : __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(scores_rsrc, off + t * 4, 0, kDeviceScope));
           key = order_key(sum * inv);
           atomicAdd(&hist[key >> 24], 1u);
         }
@@ -508,7 +543,7 @@ __device__ __forceinline__ int strided_select_list(const TokenArgs& a, const Str
       }
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
-      radix_select_emit<NW>(bkeys_rsrc, nb_pad, (uint32_t)k_blocks, true, sh, [&](int pos, int i) { sa.winners[pos] = i; });
+      radix_select_emit<NW>(GlobalKeys{bkeys_rsrc}, nb_pad, (uint32_t)k_blocks, true, sh, [&](int pos, int i) { sa.winners[pos] = i; });
       __syncthreads();
       for (int i = tid; i < k_blocks; i += NT) mark_block(sa.winners[i]);
     } else {
@@ -571,14 +606,12 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
   const int G = a.G;
   const int n = a.n;
 
-  uint4 qB[NG][4];
-#pragma unroll
-  for (int half = 0; half < NG; ++half) {
-    const int g = min(4 * half + gq, G - 1);
+  uint4 qB[4];
+  {
+    const int g = min(NG == 4 ? c16 : gq, G - 1);
     const uint16_t* qp = a.q_bh + (int64_t)g * kHeadDim + 8 * kg;
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
-      qB[half][c] = *reinterpret_cast<const uint4*>(qp + 32 * c);
+    for (int c = 0; c < 4; ++c) qB[c] = *reinterpret_cast<const uint4*>(qp + 32 * c);
   }
 
   const int row_bytes = a.row_bytes;
@@ -595,15 +628,22 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
   }
   const int vchunk = kPageSize * row_bytes + c16 * 16;  // V plane of the page, this lane's columns
 
-  float m_run[NG], l_run[NG];
-  floatx4 O[NG][8];
+  float m_run = kNegInf, l_run = 0.f;
+  floatx4 O[8];
 #pragma unroll
-  for (int half = 0; half < NG; ++half) {
-    m_run[half] = kNegInf;
-    l_run[half] = 0.f;
-#pragma unroll
-    for (int u = 0; u < 8; ++u) O[half][u] = floatx4{0.f, 0.f, 0.f, 0.f};
-  }
+  for (int u = 0; u < 8; ++u) O[u] = floatx4{0.f, 0.f, 0.f, 0.f};
+  auto scores = [&](const uint4 (&ka)[4], float (&pr)[4], int valid) {
+    if constexpr (NG == 4)
+      page_scores_wide<false>(ka, qB, m_run, l_run, O, pr, a.scale_log2, 0, valid, kg);
+    else
+      page_scores<false>(ka, qB, m_run, l_run, O, pr, a.scale_log2, 0, valid, kg);
+  };
+  auto pv = [&](const u32x4 (&vr)[4], const float (&pr)[4]) {
+    if constexpr (NG == 4)
+      page_pv_wide<false>(vr, pr, O);
+    else
+      page_pv<false>(vr, pr, O);
+  };
 
   // This wave takes the 16-entry groups w, w+NW, ...  Entries past the end (and
   // ids outside the cache) read token 0 of the cache and are masked.
@@ -656,7 +696,7 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
   if (iters > 0) {
     u32x4 vA[4], vB[4];
     uint4 ka[4];
-    float pr[NG][4];
+    float pr[4];
     Ids idA = fetch_ids(0), idB;
     issue_k(idA, 0);
     issue_v(idA, vA);
@@ -672,9 +712,9 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
         __builtin_amdgcn_sched_barrier(0);
         issue_k(idB, 1);
         __builtin_amdgcn_sched_barrier(0);
-        page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, 0, idA.valid, kg);
+        scores(ka, pr, idA.valid);
         if (idA.valid != kPageSize) clear_unused_v_rows(vA, 0, idA.valid, kg);
-        page_pv<NG>(vA, pr, O);
+        pv(vA, pr);
       }
       {
         idA = fetch_ids(it + 2);
@@ -687,9 +727,9 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
         __builtin_amdgcn_sched_barrier(0);
         issue_k(idA, 0);
         __builtin_amdgcn_sched_barrier(0);
-        page_scores<NG>(ka, qB, m_run, l_run, O, pr, a.scale_log2, 0, idB.valid, kg);
+        scores(ka, pr, idB.valid);
         if (idB.valid != kPageSize) clear_unused_v_rows(vB, 0, idB.valid, kg);
-        page_pv<NG>(vB, pr, O);
+        pv(vB, pr);
       }
     }
   }

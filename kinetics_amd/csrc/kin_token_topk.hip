@@ -25,6 +25,7 @@ struct TokenTopkParams {
   float* scores;        // workspace, strided blocks only: [lists, max_pages_per_seq * 16]
   int block, stride;    // strided blocks only
   int list_cap;         // entries of the LDS token list
+  int region0_bytes;    // K staging (and, LDSK, the key array under it) in front of the token list
   int batch, num_q_heads, num_kv_heads, group;
   int topk, sink_tokens, local_tokens, first_page_offset;
   int max_pages_per_seq, sel_stride;
@@ -33,9 +34,12 @@ struct TokenTopkParams {
 };
 
 // STRIDED = false: token-level top-k (p.topk tokens); true: strided overlapping
-// blocks (p.topk blocks).
-// Dynamic LDS: K staging attend_lds_bytes(NW) | int32 list[list_cap] | uint32 bitmap[] (strided only)
-template <int NG, int NW, bool STRIDED>
+// blocks (p.topk blocks).  LDSK: the per-token keys / scores live in LDS instead of
+// the HBM workspace (one workgroup per list, the sequence short enough).
+// Dynamic LDS: region 0 (p.region0_bytes: K staging attend_lds_bytes(NW), which the keys
+// of an LDSK kernel share: they are dead when the attention starts) | int32 list[list_cap]
+// | uint32 bitmap[] (strided only)
+template <int NG, int NW, bool STRIDED, bool LDSK>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(TokenTopkParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ float sm_m[NW][4 * NG];
@@ -70,7 +74,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
     return;
   }
 
-  int32_t* list = reinterpret_cast<int32_t*>(smem + attend_lds_bytes(NW));
+  int32_t* list = reinterpret_cast<int32_t*>(smem + p.region0_bytes);
   TokenArgs t;
   t.q_bh = p.q + hq0 * kHeadDim;
   t.kvb = reinterpret_cast<const char*>(p.kv) + (int64_t)h * kRowBytes;
@@ -87,6 +91,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
   t.n_dyn = seq_len - t.n_sink - t.n_local;
   t.topk = p.topk;
   t.keys = p.keys + (int64_t)item * p.max_pages_per_seq * kPageSize;
+  t.lds_keys = reinterpret_cast<uint32_t*>(smem);
   t.list = list;
   t.sel_tokens = sel_out;
   t.rotate = (unsigned)item * 2654435761u >> 12;  // a different starting point for every list
@@ -98,8 +103,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
     sa.scores = p.scores + (int64_t)item * p.max_pages_per_seq * kPageSize;
     sa.block_keys = t.keys;
     sa.bitmap = reinterpret_cast<uint32_t*>(list + p.list_cap);
-    // the K staging area is idle until the attention starts: 2 * topk_blocks <= 2 * kMaxTopkTokens
-    // block numbers fit its attend_lds_bytes(4) = 32 KiB
+    // the K staging area is idle until the attention starts (and the LDS scores are dead once the
+    // block keys exist): 2 * topk_blocks <= 2 * kMaxTopkTokens block numbers fit its
+    // attend_lds_bytes(4) = 32 KiB
     sa.winners = reinterpret_cast<int32_t*>(smem);
   }
   const bool scored = STRIDED ? strided_needs_scores(t, sa) : token_needs_scores(t);
@@ -112,8 +118,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
       if (tid < 256) sh.hist[tid] = 0;
       __syncthreads();
     }
-    if (STRIDED) strided_score_tokens<NW>(t, sa, pg0, pg1);
-    else token_score_keys<NW>(t, pg0, pg1, hist_on_the_fly ? sh.hist : nullptr);
+    if (STRIDED) strided_score_tokens<NW, LDSK>(t, sa, pg0, pg1);
+    else token_score_keys<NW, LDSK>(t, pg0, pg1, hist_on_the_fly ? sh.hist : nullptr);
     // Every wave waits for its own stores to be acknowledged; after the barrier the
     // workgroup's scores are in memory.
     __builtin_amdgcn_s_waitcnt(0);
@@ -130,7 +136,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
       if (tid == 0) __hip_atomic_store(&p.count[item], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
     }
   }
-  const int n = STRIDED ? strided_select_list<NG, NW>(t, sa, &sh) : token_select_list<NG, NW>(t, &sh, hist_on_the_fly);
+  const int n = STRIDED ? strided_select_list<NG, NW, LDSK>(t, sa, &sh) : token_select_list<NG, NW, LDSK>(t, &sh, hist_on_the_fly);
   if (sel_out)
     for (int i = n + tid; i < p.sel_stride; i += NT) sel_out[i] = -1;
   if (p.sel_count && tid == 0) p.sel_count[item] = n;
@@ -267,28 +273,42 @@ static int launch_token_policy(const char* fn, const kin_bf16_t* q, const kin_bf
   // workgroups -- whatever the number of chunks: selection and attention are done by
   // one workgroup per list (the per-token addressing needs ~140 registers, so 16 waves
   // do not fit).
-  const int nw = items <= 2 * kNumCus ? 8 : 4;
+  int nw = items <= 2 * kNumCus ? 8 : 4;
   const size_t bitmap_bytes = strided ? ((size_t)max_pages_per_seq * kPageSize / 32 + 1) * 4 : 0;
-  const size_t lds = (size_t)attend_lds_bytes(nw) + (size_t)p.list_cap * 4 + bitmap_bytes;
-  if (lds > 150 * 1024)
+  const size_t tail_bytes = (size_t)p.list_cap * 4 + bitmap_bytes;
+  // With the GPU full of whole lists, the keys stay in LDS when they fit: three 4-wave
+  // workgroups per CU for short sequences, else one of 12 waves (the same 12 waves per CU).
+  // Key stores to HBM between the loads of a saturated stream cost far more than their bytes.
+  const size_t key_lds = ((size_t)max_pages_per_seq * kPageSize + 4) * sizeof(uint32_t);
+  bool ldsk = false;
+  if (p.chunks == 1 && nw == 4) {
+    const size_t small = (key_lds > (size_t)attend_lds_bytes(4) ? key_lds : (size_t)attend_lds_bytes(4)) + tail_bytes;
+    const size_t big = (key_lds > (size_t)attend_lds_bytes(12) ? key_lds : (size_t)attend_lds_bytes(12)) + tail_bytes;
+    if (small <= 50 * 1024) {
+      ldsk = true;
+    } else if (big <= 156 * 1024) {
+      ldsk = true;
+      nw = 12;
+    }
+  }
+  size_t region0 = (size_t)attend_lds_bytes(nw);
+  if (ldsk && key_lds > region0) region0 = (key_lds + 15) & ~(size_t)15;
+  p.region0_bytes = (int)region0;
+  const size_t lds = region0 + tail_bytes;
+  if (lds > 150 * 1024 && !ldsk)
     return fail(KIN_ERR_UNSUPPORTED, "%s: max_pages_per_seq=%d is too long for the strided policy's token bitmap", fn,
                 max_pages_per_seq);
+#define KIN_TOKEN_KERNEL(NG_, NW_, S_, L_) reinterpret_cast<const void*>(&token_topk_kernel<NG_, NW_, S_, L_>)
+#define KIN_TOKEN_PICK(NG_, S_)                                                             \
+  (ldsk ? (nw == 12 ? KIN_TOKEN_KERNEL(NG_, 12, S_, true) : KIN_TOKEN_KERNEL(NG_, 4, S_, true)) \
+        : (nw == 8 ? KIN_TOKEN_KERNEL(NG_, 8, S_, false) : KIN_TOKEN_KERNEL(NG_, 4, S_, false)))
   const void* kernel;
-  if (strided) {
-    if (p.group <= 4)
-      kernel = nw == 8 ? reinterpret_cast<const void*>(&token_topk_kernel<1, 8, true>)
-                       : reinterpret_cast<const void*>(&token_topk_kernel<1, 4, true>);
-    else
-      kernel = nw == 8 ? reinterpret_cast<const void*>(&token_topk_kernel<2, 8, true>)
-                       : reinterpret_cast<const void*>(&token_topk_kernel<2, 4, true>);
-  } else {
-    if (p.group <= 4)
-      kernel = nw == 8 ? reinterpret_cast<const void*>(&token_topk_kernel<1, 8, false>)
-                       : reinterpret_cast<const void*>(&token_topk_kernel<1, 4, false>);
-    else
-      kernel = nw == 8 ? reinterpret_cast<const void*>(&token_topk_kernel<2, 8, false>)
-                       : reinterpret_cast<const void*>(&token_topk_kernel<2, 4, false>);
-  }
+  if (strided)
+    kernel = p.group <= 4 ? KIN_TOKEN_PICK(1, true) : KIN_TOKEN_PICK(4, true);
+  else
+    kernel = p.group <= 4 ? KIN_TOKEN_PICK(1, false) : KIN_TOKEN_PICK(4, false);
+#undef KIN_TOKEN_PICK
+#undef KIN_TOKEN_KERNEL
   if (lds > 48 * 1024) {
     st = check_hip(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
                    "hipFuncSetAttribute(token_topk_kernel)");

@@ -92,7 +92,7 @@ def test_select_argument_errors(lib):
     assert select(lib, sink=-1) == _lib.KIN_ERR_BAD_SHAPE
     assert select(lib, stride=200, local=1010) == _lib.KIN_ERR_BAD_SHAPE
     assert select(lib, Hq=5, Hkv=2) == _lib.KIN_ERR_BAD_SHAPE
-    assert select(lib, Hq=16, Hkv=1) == _lib.KIN_ERR_UNSUPPORTED    # group 16 > 8
+    assert select(lib, Hq=32, Hkv=1) == _lib.KIN_ERR_UNSUPPORTED    # group 32 > 16
     assert select(lib, topk=4096, stride=4097) == _lib.KIN_ERR_UNSUPPORTED
     assert select(lib, kp=20000) == _lib.KIN_ERR_UNSUPPORTED
     assert select(lib, kbar=A + 8) == _lib.KIN_ERR_MISALIGNED

@@ -133,7 +133,7 @@ def check_selection(pb, sel, cnt, logical, scores, exact=False):
             assert np.all(sel[b, h, c:] == -1)
 
 
-@pytest.mark.parametrize("hkv,group,topk", [(1, 4, 8), (2, 2, 5), (8, 2, 16), (1, 8, 64), (1, 1, 3)])
+@pytest.mark.parametrize("hkv,group,topk", [(1, 4, 8), (2, 2, 5), (8, 2, 16), (1, 8, 64), (1, 1, 3), (2, 16, 7), (1, 11, 20)])
 def test_score_topk_small(ops, hkv, group, topk):
     lengths = [PS * 40 + 3, PS * 9, 1, 0, PS * 3 + 1, PS * 130 + 16, PS * topk + 1, PS * (topk + 1) + 1]
     pb = P.make_problem(300 + hkv + topk, lengths, num_kv_heads=hkv, group=group, topk=topk)
@@ -181,7 +181,7 @@ def oracle_sparse(pb, kv=None):
     return sel, cnt, out, lse
 
 
-@pytest.mark.parametrize("hkv,group", [(1, 4), (1, 8), (8, 2), (2, 1), (1, 3), (2, 6)])
+@pytest.mark.parametrize("hkv,group", [(1, 4), (1, 8), (8, 2), (2, 1), (1, 3), (2, 6), (1, 5), (2, 12), (1, 16), (4, 9)])
 @pytest.mark.parametrize("splits", [1, 3, 0])
 def test_sparse_decode_matches_oracle(ops, hkv, group, splits):
     lengths = [PS * 30 + r for r in (1, 2, 7, 15, 16)] + [1, 0, PS, PS * 3 + 4, PS * 100 + 9]
@@ -200,7 +200,7 @@ def test_sparse_decode_matches_oracle(ops, hkv, group, splits):
     assert np.allclose(got_lse[fin], want_lse[fin], rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("hkv,group", [(1, 4), (8, 2), (1, 8)])
+@pytest.mark.parametrize("hkv,group", [(1, 4), (8, 2), (1, 8), (2, 16), (1, 13)])
 @pytest.mark.parametrize("splits", [1, 4, 0])
 def test_dense_decode_matches_oracle(ops, hkv, group, splits):
     lengths = [PS * 70 + 5, PS * 33, 1, 0, 17, PS * 257 + 16]
@@ -976,7 +976,7 @@ def test_seeded_sweep_of_split_scoring(ops):
     rng = np.random.default_rng(61)
     for trial in range(6):
         hkv = int(rng.choice([1, 1, 2, 4]))
-        group = int(rng.integers(1, 9))
+        group = int(rng.integers(1, 17))
         B = int(rng.integers(1, 5))
         lengths = [int(rng.choice([0, 5, PS * 7, int(rng.integers(PS * 2048, PS * 6000)), int(rng.integers(PS * 100, PS * 3000))]))
                    for _ in range(B)]
@@ -1067,15 +1067,16 @@ def test_ragged_append_bit_exact(ops, hkv):
 # --------------------------------------------------------------------------- token-level top-k
 
 
-def _check_token_topk(ops, pb, topk, sink, local, offset, what):
+def _check_token_topk(ops, pb, topk, sink, local, offset, what, max_pages=None):
     g = Gpu(pb)
     ops.append_paged_kv(g.k, g.v, g.kv, None, g.indices, g.indptr, g.last)
     stride = topk + sink + local
     sel = torch.full((pb.B, pb.Hkv, stride), -7, dtype=torch.int32, device=DEV)
     cnt = torch.full((pb.B, pb.Hkv), -7, dtype=torch.int32, device=DEV)
     lse = torch.full((pb.B, pb.Hq), float("nan"), dtype=torch.float32, device=DEV)
-    out = ops.token_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, topk, max(pb.max_pages, 1), sink_tokens=sink,
-                                local_tokens=local, first_page_offset=offset, lse=lse, sel_tokens=sel, sel_count=cnt)
+    out = ops.token_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, topk, max_pages or max(pb.max_pages, 1),
+                                sink_tokens=sink, local_tokens=local, first_page_offset=offset, lse=lse, sel_tokens=sel,
+                                sel_count=cnt)
     torch.cuda.synchronize()
     kv = pb.kv_cache.copy()
     O.append_paged_kv(pb.k, pb.v, kv, None, pb.page_indices, pb.page_indptr, pb.last_page_len)
@@ -1118,7 +1119,8 @@ def _check_token_topk(ops, pb, topk, sink, local, offset, what):
     return lse.cpu().numpy()
 
 
-@pytest.mark.parametrize("case", ["mixed", "hkv8", "g8", "g7", "many", "offset", "all", "window_only", "split", "split_many"])
+@pytest.mark.parametrize("case", ["mixed", "hkv8", "g8", "g7", "many", "many_12_waves", "many_g16", "offset", "all",
+                                  "window_only", "split", "split_many"])
 def test_token_topk_decode(ops, case):
     """LiteSys' token-level top-k (sparsity_utils.py:6-21): sink tokens, the
     top-k tokens of the middle by group-mean logit, the local window."""
@@ -1134,10 +1136,21 @@ def test_token_topk_decode(ops, case):
     elif case == "g7":       # a group that fills the second head tile only partly
         pb = P.make_problem(1309, [PS * 50 + 9, PS * 3, 40], num_kv_heads=2, group=7)
         args = (200, 4, 12, 0)
-    elif case == "many":     # > 512 lists: 4 waves per list
+    elif case == "many":     # > 512 lists: 4 waves per list, keys in LDS
         rng = np.random.default_rng(1303)
         pb = P.make_problem(1303, [int(x) for x in rng.integers(1, PS * 30, size=600)], num_kv_heads=1, group=3)
         args = (48, 4, 8, 0)
+    elif case == "many_12_waves":  # > 512 lists and room asked for long sequences: keys in LDS, one 12-wave workgroup per list
+        rng = np.random.default_rng(1310)
+        pb = P.make_problem(1310, [PS * 200 + 5, 0, 3] + [int(x) for x in rng.integers(1, PS * 40, size=530)], num_kv_heads=1,
+                            group=4)
+        args = (56, 4, 24, 0)
+        max_pages = 1500
+    elif case == "many_g16":  # the same with 16 query heads per KV head and an offset
+        rng = np.random.default_rng(1311)
+        pb = P.make_problem(1311, [int(x) for x in rng.integers(13, PS * 25, size=270)], num_kv_heads=2, group=16)
+        args = (30, 4, 9, 12)
+        max_pages = 2049
     elif case == "offset":   # sequences stored 12 slots into their first page
         pb = P.make_problem(1304, [PS * 25 + 2, PS * 2, 13, 12, 30], num_kv_heads=2, group=4)
         args = (32, 4, 10, 12)
@@ -1158,7 +1171,8 @@ def test_token_topk_decode(ops, case):
         pb = P.make_problem(1306, [PS * 20 + 2, 40], num_kv_heads=2, group=1)
         args = (0, 4, 33, 0)
     topk, sink, local, offset = args
-    lse = _check_token_topk(ops, pb, topk, sink, local, offset, f"token top-k {case}")
+    lse = _check_token_topk(ops, pb, topk, sink, local, offset, f"token top-k {case}",
+                            max_pages=max_pages if case in ("many_12_waves", "many_g16") else None)
     assert not np.isnan(lse).any()
     if case == "all":
         kv = pb.kv_cache.copy()
@@ -1167,14 +1181,14 @@ def test_token_topk_decode(ops, case):
         assert np.allclose(lse, want_lse, rtol=1e-4, atol=1e-4)
 
 
-def _check_strided(ops, pb, topk, sink, local, block, stride, offset, what, need_sparse=True):
+def _check_strided(ops, pb, topk, sink, local, block, stride, offset, what, need_sparse=True, max_pages=None):
     g = Gpu(pb)
     ops.append_paged_kv(g.k, g.v, g.kv, None, g.indices, g.indptr, g.last)
     cap = max(topk, 1) * block + sink + local
     sel = torch.full((pb.B, pb.Hkv, cap), -7, dtype=torch.int32, device=DEV)
     cnt = torch.full((pb.B, pb.Hkv), -7, dtype=torch.int32, device=DEV)
     lse = torch.full((pb.B, pb.Hq), float("nan"), dtype=torch.float32, device=DEV)
-    out = ops.strided_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, topk, max(pb.max_pages, 1), block_size=block,
+    out = ops.strided_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, topk, max_pages or max(pb.max_pages, 1), block_size=block,
                                   stride=stride, sink_tokens=sink, local_tokens=local, first_page_offset=offset, lse=lse,
                                   sel_tokens=sel, sel_count=cnt)
     torch.cuda.synchronize()
@@ -1213,7 +1227,7 @@ def _check_strided(ops, pb, topk, sink, local, block, stride, offset, what, need
     assert not np.isnan(lse.cpu().numpy()).any()
 
 
-@pytest.mark.parametrize("case", ["mixed", "hkv8_stride4", "g8", "g5", "many", "offset", "stride16", "split", "block8_stride3"])
+@pytest.mark.parametrize("case", ["mixed", "hkv8_stride4", "g8", "g5", "many", "many_12_waves", "offset", "stride16", "split", "block8_stride3"])
 def test_strided_topk_decode(ops, case):
     """LiteSys' strided overlapping-block policy (sparsity_utils.py:49-105)."""
     block, stride, offset = 16, 8, 0
@@ -1229,10 +1243,16 @@ def test_strided_topk_decode(ops, case):
     elif case == "g5":
         pb = P.make_problem(1508, [PS * 50 + 9, PS * 3, 40], num_kv_heads=2, group=5)
         topk, sink, local = 6, 4, 12
-    elif case == "many":     # > 512 lists: 4 waves per list
+    elif case == "many":     # > 512 lists: 4 waves per list, scores in LDS
         rng = np.random.default_rng(1503)
         pb = P.make_problem(1503, [int(x) for x in rng.integers(1, PS * 30, size=600)], num_kv_heads=1, group=3)
         topk, sink, local = 3, 4, 8
+    elif case == "many_12_waves":  # > 512 lists and room asked for long sequences: scores in LDS, 12 waves per list
+        rng = np.random.default_rng(1509)
+        pb = P.make_problem(1509, [PS * 180 + 5, 0, 3] + [int(x) for x in rng.integers(1, PS * 40, size=530)], num_kv_heads=1,
+                            group=4)
+        topk, sink, local, stride = 5, 4, 24, 4
+        max_pages = 2049
     elif case == "offset":
         pb = P.make_problem(1504, [PS * 25 + 2, PS * 2, 13, 12, 30], num_kv_heads=2, group=4)
         topk, sink, local, offset = 2, 4, 10, 12
@@ -1245,7 +1265,8 @@ def test_strided_topk_decode(ops, case):
     else:
         pb = P.make_problem(1506, [PS * 33 + 1, 40, 19], num_kv_heads=2, group=1)
         topk, sink, local, block, stride = 9, 2, 5, 8, 3
-    _check_strided(ops, pb, topk, sink, local, block, stride, offset, f"strided {case}")
+    _check_strided(ops, pb, topk, sink, local, block, stride, offset, f"strided {case}",
+                   max_pages=max_pages if case == "many_12_waves" else None)
 
 
 @pytest.mark.parametrize("lists", [1, 2])
@@ -1298,7 +1319,7 @@ def test_seeded_sweep_of_token_policies(ops):
     rng = np.random.default_rng(777)
     for trial in range(30):
         hkv = int(rng.choice([1, 1, 2, 4, 8]))
-        group = int(rng.integers(1, 9))
+        group = int(rng.integers(1, 17))
         B = int(rng.integers(1, 6))
         lengths = []
         for _ in range(B):
@@ -1694,7 +1715,7 @@ def _sweep_of_shapes(ops, PS, trials, seed):
     rng = np.random.default_rng(seed)
     for trial in range(trials):
         hkv = int(rng.choice([1, 1, 2, 3, 4, 8]))
-        group = int(rng.integers(1, 9))
+        group = int(rng.integers(1, 17))
         B = int(rng.integers(1, 7))
         lengths = []
         for _ in range(B):
