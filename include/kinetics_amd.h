@@ -373,8 +373,10 @@ int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_bf16_t* k, c
  * (-1 for a sequence with more than max_pages_per_seq pages, which is skipped:
  * out = 0).  workspace: kin_token_topk_workspace_bytes(...) bytes of scratch
  * (4 bytes per cache slot and KV head, plus an arrival counter per list; any
- * contents, 16-byte aligned).  Reads every key of the context once: HBM
- * traffic is about half of dense decode's.  When the lists are fewer than
+ * contents, 16-byte aligned; with more than 512 lists and max_pages_per_seq up
+ * to ~2100 the per-token keys stay in on-chip memory and the scratch is not
+ * touched, but its size is still checked).  Reads every key of the context
+ * once: HBM traffic is about half of dense decode's.  When the lists are fewer than
  * the GPU's compute units, several workgroups share the scoring of a list;
  * a small kernel that zeroes the counters is then launched first on the
  * same stream (no memset, so the call can be captured in a HIP graph).
