@@ -1269,6 +1269,40 @@ def test_strided_topk_decode(ops, case):
                    max_pages=max_pages if case == "many_12_waves" else None)
 
 
+@pytest.mark.parametrize("policy", ["token", "strided"])
+def test_token_policies_with_the_gpu_full_of_lists(ops, policy):
+    """More than 512 lists: one workgroup per list, and the per-token keys (scores,
+    for the strided policy) stay in LDS when ``max_pages_per_seq`` lets them fit --
+    in 4-wave workgroups for short sequences, one 12-wave workgroup per list for long
+    ones -- or go through the HBM workspace when it does not.  Seeded shapes with
+    groups up to 16, pinned tokens, offsets and empty sequences, each against the oracle."""
+    rng = np.random.default_rng(8100 if policy == "token" else 8200)
+    for trial in range(5):
+        hkv = int(rng.choice([1, 1, 2, 4]))
+        group = int(rng.choice([1, 2, 4, 5, 8, 12, 16]))
+        lists = int(rng.integers(513, 620))
+        B = (lists + hkv - 1) // hkv
+        longest = int(rng.choice([PS * 30, PS * 60, PS * 150]))
+        lengths = [int(x) for x in rng.integers(0, longest, size=B)]
+        lengths[int(rng.integers(0, B))] = longest + int(rng.integers(1, 16))
+        sink, local = int(rng.choice([0, 4, 4, 9])), int(rng.choice([1, 1, 16, 33]))
+        offset = int(rng.integers(0, PS)) if rng.integers(0, 2) else 0
+        lengths = [L + offset if L else 0 for L in lengths]
+        # 0: exactly the longest sequence; 700 / 2049: keys in LDS (4 / 12 waves); 2600: too long for LDS
+        max_pages = [0, 700, 2049, 2600, 1500][trial]
+        pb = P.make_problem(8300 + 10 * trial + (1 if policy == "token" else 2), lengths, num_kv_heads=hkv, group=group)
+        mp = max(max_pages, pb.max_pages) if max_pages else None
+        if policy == "token":
+            topk = int(rng.choice([0, 5, 40, 300]))
+            what = f"trial {trial}: hkv={hkv} G={group} B={B} longest={longest} topk={topk} sink={sink} local={local} offset={offset} max_pages={mp}"
+            _check_token_topk(ops, pb, topk, sink, local, offset, what, max_pages=mp)
+        else:
+            topk, block, stride = int(rng.choice([1, 3, 10])), int(rng.choice([8, 16, 32])), int(rng.choice([1, 4, 8, 16]))
+            what = (f"trial {trial}: hkv={hkv} G={group} B={B} longest={longest} topk={topk} block={block} stride={stride} "
+                    f"sink={sink} local={local} offset={offset} max_pages={mp}")
+            _check_strided(ops, pb, topk, sink, local, block, stride, offset, what, need_sparse=False, max_pages=mp)
+
+
 @pytest.mark.parametrize("lists", [1, 2])
 def test_token_topk_ties_pick_the_lowest_positions(ops, lists):
     """Equal scores are taken in ascending token position, also across the
