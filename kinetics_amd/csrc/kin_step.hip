@@ -41,6 +41,7 @@ struct StepParams {
   uint32_t* ws_keys;   // [lists, score_key_stride(kbar_pages)]
   int64_t num_pages;
   float scale_log2;
+  int deep_score;      // few lists: more mean-key loads in flight per lane (see the kernel)
 };
 
 template <int NG, int NW, bool F16>
@@ -135,7 +136,16 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     __syncthreads();
     n = select_from_keys<NT>(s, sel_lds);
   } else {
-    n = score_select<4, NT, F16>(s, sel_lds);
+    // Mean-key loads in flight per lane.  4 saturate HBM while several rounds of workgroups overlap
+    // (4096 lists; more only lengthens the last pass of short lists).  With fewer lists the workgroups
+    // score in step and each has to keep 64 KiB in flight: 16 / 8 / 4 loads at 4 / 8 / 16 waves
+    // (1024 lists of 2048 pages: 5 % faster than with 4).
+    if (p.deep_score) {
+      constexpr int kDeep = NW <= 4 ? 16 : (NW <= 8 ? 8 : 4);
+      n = score_select<kDeep, NT, F16>(s, sel_lds);
+    } else {
+      n = score_select<4, NT, F16>(s, sel_lds);
+    }
   }
   if (p.sel_pages) {
     int32_t* sel = p.sel_pages + (int64_t)item * p.sel_stride;
@@ -262,6 +272,7 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
     p.ws_count = nullptr;
     p.ws_keys = nullptr;
   }
+  p.deep_score = items < 4096 ? 1 : 0;
   const size_t sel_scratch = select_lds_bytes(kbar_pages, p.sort_cap);
   const size_t attend_bytes = (size_t)attend_lds_bytes(nw);
   size_t region0 = sel_scratch > attend_bytes ? sel_scratch : attend_bytes;
