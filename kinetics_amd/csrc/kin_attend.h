@@ -183,7 +183,22 @@ struct AttendArgs {
   int p0, p1;            // this workgroup's part of the list [p0, p1)
   int last_len;          // tokens in the list's final page
   int first_skip;        // leading token slots of list entry 0 that hold no token (0 .. page_size-1)
+  unsigned rotate;       // long parts start at tile (rotate mod tiles) and wrap around; 0: in list order
 };
+
+// Long lists that many workgroups walk in step -- dense decode over a cache whose pages are numbered
+// p * batch + b, as the reference lays them out -- are all at the same page at the same time and
+// read one narrow window of the cache (1024 sequences: 81 % of peak against 85-87 % for any other
+// numbering).  Every list therefore starts at its own tile and wraps around; the sum over tiles does
+// not care about the order.  Only with more lists than fill the GPU twice over (with fewer, neighbours
+// reading neighbouring pages helps: 256 lists lose 4 % when rotated) and only parts of at least
+// kRotateMinTiles tiles.  The rule depends on the batch alone, so the fused step and the stand-alone
+// kernel visit a list's tiles in the same order.
+constexpr int kRotateMinTiles = 512;
+__host__ __device__ inline bool attend_rotates(int64_t lists) { return lists > 2 * kNumCus; }
+__device__ __forceinline__ unsigned attend_rotation(int list, int split) {
+  return ((unsigned)list * 2654435761u >> 8) + 977u * (unsigned)split;
+}
 
 // K tiles a wave keeps staged in LDS in attend_list(): the one being read and the one in flight.
 constexpr int kAttendStages = 2;
@@ -357,14 +372,23 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
   const int t0 = p0 << tshift, t1 = min(p1 << tshift, n_tiles);
   const int my_first = t0 + w;
   const int iters = (t1 > my_first) ? (t1 - my_first + NW - 1) / NW : 0;
+  // The it-th tile of this wave: my_first + NW * it, shifted by the part's rotation (see attend_rotates()).
+  const int span_t = t1 - t0;
+  const int rot = span_t >= kRotateMinTiles ? (int)(a.rotate % (unsigned)span_t) : 0;
+  auto tile_at = [&](int it) -> int {
+    const int i = my_first + NW * it;
+    if (i >= t1) return i;  // past the end: stays past the end
+    const int r = i - t0 + rot;
+    return t0 + (r >= span_t ? r - span_t : r);
+  };
   // Page ids are fetched one half-step before they are needed.
   auto load_id = [&](int it) -> int {
-    const int idx = my_first + NW * it;
+    const int idx = tile_at(it);
     return id_at((idx < t1 ? idx : t0) >> tshift);
   };
   const int first_skip = a.first_skip;
   auto page_rsrc = [&](int it, int id, int& valid_tokens) {
-    const int idx = my_first + NW * it;
+    const int idx = tile_at(it);
     const int e = idx >> tshift, sub16 = (idx & tmask) * kPageSize;  // list entry, first token slot of the tile in its page
     const bool ok = idx < t1 && id >= 0 && (int64_t)id < a.num_pages;
     // The token slots of the page that count are [lo_p, hi_p); the tile's share of

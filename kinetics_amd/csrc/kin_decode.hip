@@ -22,6 +22,7 @@ struct DecodeParams {
   int list_stride, num_splits;
   int first_page_offset;  // padding slots at the start of list entry 0
   int page_size;
+  int rotate;  // attend_rotates(lists)
   int64_t num_pages;
   float scale_log2;  // sm_scale * log2(e)
 };
@@ -66,6 +67,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
   a.p1 = min(n, a.p0 + per_split);
   a.last_len = p.last_page_len[b];
   a.first_skip = p.first_page_offset;
+  a.rotate = p.rotate ? attend_rotation(list, split) : 0u;
 
   // The list is read-only for the whole kernel; the constant address space
   // makes the uniform id load a scalar one (off the vector-memory counter that
@@ -149,6 +151,7 @@ static int launch_decode(const char* fn, DecodeParams& p, int batch, void* works
   const int64_t lists = xcd_grid_size(batch, p.num_kv_heads);
   if (lists > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   p.batch = batch;
+  p.rotate = attend_rotates((int64_t)batch * p.num_kv_heads) ? 1 : 0;
   dim3 grid((unsigned)lists, (unsigned)splits);
   if (p.group <= 4) {
     if (f16) paged_decode_kernel<1, true><<<grid, 256, 0, stream>>>(p);

@@ -42,6 +42,7 @@ struct StepParams {
   int64_t num_pages;
   float scale_log2;
   int deep_score;      // few lists: more mean-key loads in flight per lane (see the kernel)
+  int rotate;          // attend_rotates(lists)
 };
 
 template <int NG, int NW, bool F16>
@@ -169,6 +170,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   a.p1 = n;
   a.last_len = last_len;
   a.first_skip = p.first_page_offset;
+  a.rotate = p.rotate ? attend_rotation(item, 0) : 0u;
   attend_list<NG, NW, F16>(
       a, [&](int i) -> int { return __builtin_amdgcn_readfirstlane(sel_lds[i]); }, smem, sm_m, sm_l,
       [&](int g, int d, float o, float lse2) {
@@ -273,6 +275,7 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
     p.ws_keys = nullptr;
   }
   p.deep_score = items < 4096 ? 1 : 0;
+  p.rotate = attend_rotates(items) ? 1 : 0;
   const size_t sel_scratch = select_lds_bytes(kbar_pages, p.sort_cap);
   const size_t attend_bytes = (size_t)attend_lds_bytes(nw);
   size_t region0 = sel_scratch > attend_bytes ? sel_scratch : attend_bytes;

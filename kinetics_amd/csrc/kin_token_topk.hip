@@ -155,6 +155,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
   a.p1 = n;
   a.last_len = kPageSize;
   a.first_skip = 0;
+  a.rotate = 0;
   a.page_size = kPageSize;
   attend_tokens<NG, NW>(a, list, smem, sm_m, sm_l, [&](int g, int d, float o, float lse2) {
     p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_bf16(o);
