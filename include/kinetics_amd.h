@@ -69,7 +69,11 @@ enum kin_status {
   KIN_ERR_MISALIGNED = 7     /* a tensor pointer is not 16-byte aligned */
 };
 
-/* Library version (major*10000 + minor*100 + patch). */
+/* Library version (major*10000 + minor*100 + patch).  2.0.0: mean keys are stored
+ * head-major ([batch, num_kv_heads, kbar_pages, 128]; 1.x had [batch, kbar_pages,
+ * num_kv_heads, 128]), kin_block_score_topk takes the page size, pages of 32 and 64
+ * tokens, float16 twins (kin_*_f16), groups of up to 16 query heads per KV head,
+ * the page pool and kin_blocktopk_decode_step_static. */
 int kin_version(void);
 
 /* Human-readable text of the last non-OK status on the calling thread
