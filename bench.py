@@ -217,10 +217,11 @@ def whole_layer(torch, args, B, ctx, topk, device):
 
     name, world = WHOLE_LAYER_MODEL[args.workload]
     cfg = qwen3_config(name)
-    layer = BlockTopkDecoderLayer(cfg, world, B, ctx, ctx + 512, PS, topk, device, torch.bfloat16)
+    elem = torch.float16 if args.dtype == "float16" else torch.bfloat16   # the whole layer moves to --dtype, as in the reference
+    layer = BlockTopkDecoderLayer(cfg, world, B, ctx, ctx + 512, PS, topk, device, elem)
     layer.apply(init_weights)
-    layer.eval().to(device, dtype=torch.bfloat16)
-    hidden = torch.randn(B, 1, cfg.hidden_size, device=device, dtype=torch.bfloat16)
+    layer.eval().to(device, dtype=elem)
+    hidden = torch.randn(B, 1, cfg.hidden_size, device=device, dtype=elem)
     for _ in range(args.warmup):
         layer(hidden.clone())
     torch.cuda.synchronize()
@@ -251,9 +252,9 @@ def whole_layer(torch, args, B, ctx, topk, device):
         # the reference's dense layer (benchmark/dense.py, dense_decoder.py) on the same shape
         from kinetics_amd.decoder_layer import DenseDecoderLayer
 
-        dense = DenseDecoderLayer(cfg, world, B, ctx, ctx + 512, PS, device, torch.bfloat16)
+        dense = DenseDecoderLayer(cfg, world, B, ctx, ctx + 512, PS, device, elem)
         dense.apply(init_weights)
-        dense.eval().to(device, dtype=torch.bfloat16)
+        dense.eval().to(device, dtype=elem)
         dense.prepare_wrapper()
         nd = max(3, min(args.steps, 20))
         for _ in range(2):

@@ -527,8 +527,9 @@ int kin_check_page_table(const int32_t* page_indices, const int32_t* page_indptr
  * float16 twin: same arguments, same meaning, same fp32 accumulation, with q, k,
  * v, kv_cache, kbar and out holding IEEE binary16 (round-to-nearest-even on
  * every store; the mean key is the fp32 sum times 1/page_size rounded to
- * binary16).  The token-granular policies, the entry point with built-in scratch
- * and the row-wise layer kernels are bfloat16 only.
+ * binary16).  The row-wise layer kernels further down have float16 twins too
+ * (the reference moves the whole layer to --dtype).  The token-granular policies
+ * and the entry point with built-in scratch are bfloat16 only.
  */
 int kin_append_paged_kv_f16(const kin_f16_t* k, const kin_f16_t* v,
                             kin_f16_t* kv_cache, kin_f16_t* kbar,
@@ -600,7 +601,9 @@ int kin_blocktopk_decode_step_f16(const kin_f16_t* q, const kin_f16_t* k, const 
  * flashinfer's RMSNorm through its custom ops layer_norm and qk_norm
  * (benchmark/model_utils.py:4-25) and leaves the residual adds, the q/k/v split
  * and act(gate)*up to PyTorch.  These three entry points cover the same steps
- * with one pass over the data each.  All tensors are bf16; statistics are fp32.
+ * with one pass over the data each.  All tensors are bf16 (float16 for the
+ * kin_*_f16 twins, whose roundings are to float16 wherever the text below says
+ * bf16); statistics are fp32.
  */
 
 /*
@@ -623,6 +626,9 @@ int kin_blocktopk_decode_step_f16(const kin_f16_t* q, const kin_f16_t* k, const 
 int kin_rms_norm(const void* x, void* residual, const void* weight, void* out,
                  int64_t rows, int hidden, int64_t x_row_stride, int64_t out_row_stride,
                  float eps, kin_stream_t stream);
+int kin_rms_norm_f16(const void* x, void* residual, const void* weight, void* out,
+                     int64_t rows, int hidden, int64_t x_row_stride, int64_t out_row_stride,
+                     float eps, kin_stream_t stream);
 
 /*
  * The steps between the fused QKV projection and the attention path
@@ -637,6 +643,10 @@ int kin_qkv_norm_split(const void* qkv, int64_t qkv_row_stride, const void* q_we
                        const void* k_weight, float eps, void* q, void* k, void* v,
                        int batch, int num_q_heads, int num_kv_heads, int head_dim,
                        kin_stream_t stream);
+int kin_qkv_norm_split_f16(const void* qkv, int64_t qkv_row_stride, const void* q_weight,
+                           const void* k_weight, float eps, void* q, void* k, void* v,
+                           int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                           kin_stream_t stream);
 
 #define KIN_ACT_SILU 0
 #define KIN_ACT_GELU 1 /* erf form */
@@ -652,6 +662,9 @@ int kin_qkv_norm_split(const void* qkv, int64_t qkv_row_stride, const void* q_we
 int kin_gated_act(const void* gate, const void* up, void* out, int64_t rows, int inter,
                   int64_t gate_row_stride, int64_t up_row_stride, int act,
                   kin_stream_t stream);
+int kin_gated_act_f16(const void* gate, const void* up, void* out, int64_t rows, int inter,
+                      int64_t gate_row_stride, int64_t up_row_stride, int act,
+                      kin_stream_t stream);
 
 #ifdef __cplusplus
 }

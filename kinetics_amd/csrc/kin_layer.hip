@@ -4,6 +4,7 @@
 // element is read once and written once with 16-byte accesses, statistics are
 // taken in fp32 inside lane groups (no LDS), and each replaces a chain of
 // elementwise launches that would move the same rows through HBM several times.
+// F16 = false: bfloat16 tensors; true: float16 (the kin_*_f16 entry points).
 #include "kin_common.h"
 
 namespace kin {
@@ -22,26 +23,30 @@ struct NormParams {
   float eps, inv_hidden;
 };
 
+template <bool F16>
 __device__ __forceinline__ float sum_sq8(const u32x4& v) {
   float s = 0.f;
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const float a = bf16_lo(w[i]), b = bf16_hi(w[i]);
+    const float a = elem_lo<F16>(w[i]), b = elem_hi<F16>(w[i]);
     s = fmaf(a, a, s);
     s = fmaf(b, b, s);
   }
   return s;
 }
 
-// bf16(a + b) per element, as a bf16 tensor add computes it.
-__device__ __forceinline__ uint32_t add_bf16x2(uint32_t a, uint32_t b) {
-  return f32_to_bf16(bf16_lo(a) + bf16_lo(b)) | (f32_to_bf16(bf16_hi(a) + bf16_hi(b)) << 16);
+// round(a + b) per element, as a 16-bit tensor add computes it.
+template <bool F16>
+__device__ __forceinline__ uint32_t add_x2(uint32_t a, uint32_t b) {
+  return f32_to_elem<F16>(elem_lo<F16>(a) + elem_lo<F16>(b)) | (f32_to_elem<F16>(elem_hi<F16>(a) + elem_hi<F16>(b)) << 16);
 }
 
-// bf16((x * r) * w) per element.
-__device__ __forceinline__ uint32_t scale_bf16x2(uint32_t x, float r, uint32_t w) {
-  return f32_to_bf16(bf16_lo(x) * r * bf16_lo(w)) | (f32_to_bf16(bf16_hi(x) * r * bf16_hi(w)) << 16);
+// round((x * r) * w) per element.
+template <bool F16>
+__device__ __forceinline__ uint32_t scale_x2(uint32_t x, float r, uint32_t w) {
+  return f32_to_elem<F16>(elem_lo<F16>(x) * r * elem_lo<F16>(w)) |
+         (f32_to_elem<F16>(elem_hi<F16>(x) * r * elem_hi<F16>(w)) << 16);
 }
 
 template <int LPR>
@@ -60,7 +65,7 @@ __device__ __forceinline__ float group_sum(float x) {
 // (the row stays in registers between the two passes): the smaller
 // instantiations need fewer registers, so that a grid of a few thousand rows is
 // resident at once instead of running a nearly empty second round.
-template <int LPR, int MAXC, bool RES>
+template <int LPR, int MAXC, bool RES, bool F16>
 __global__ __launch_bounds__(256) void rms_norm_kernel(NormParams p) {
   const int sub = threadIdx.x / LPR, l = threadIdx.x % LPR;
   const int64_t row = (int64_t)blockIdx.x * (256 / LPR) + sub;
@@ -80,13 +85,13 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(NormParams p) {
   for (int c = 0; c < MAXC; ++c) {
     if (c < p.chunks) {
       if (RES) {
-        v[c].x = add_bf16x2(v[c].x, r[c].x);
-        v[c].y = add_bf16x2(v[c].y, r[c].y);
-        v[c].z = add_bf16x2(v[c].z, r[c].z);
-        v[c].w = add_bf16x2(v[c].w, r[c].w);
+        v[c].x = add_x2<F16>(v[c].x, r[c].x);
+        v[c].y = add_x2<F16>(v[c].y, r[c].y);
+        v[c].z = add_x2<F16>(v[c].z, r[c].z);
+        v[c].w = add_x2<F16>(v[c].w, r[c].w);
         rr[c * LPR + l] = v[c];
       }
-      ss += sum_sq8(v[c]);
+      ss += sum_sq8<F16>(v[c]);
     }
   }
   ss = group_sum<LPR>(ss);
@@ -97,10 +102,10 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(NormParams p) {
     if (c < p.chunks) {
       const u32x4 w = p.weight[c * LPR + l];
       u32x4 o;
-      o.x = scale_bf16x2(v[c].x, rinv, w.x);
-      o.y = scale_bf16x2(v[c].y, rinv, w.y);
-      o.z = scale_bf16x2(v[c].z, rinv, w.z);
-      o.w = scale_bf16x2(v[c].w, rinv, w.w);
+      o.x = scale_x2<F16>(v[c].x, rinv, w.x);
+      o.y = scale_x2<F16>(v[c].y, rinv, w.y);
+      o.z = scale_x2<F16>(v[c].z, rinv, w.z);
+      o.w = scale_x2<F16>(v[c].w, rinv, w.w);
       orow[c * LPR + l] = o;
     }
   }
@@ -117,6 +122,7 @@ struct QkvParams {
 
 // 16 lanes per head row of 128 elements: q and k heads are normalised, v heads
 // copied, each to its own contiguous [batch, heads, 128] tensor.
+template <bool F16>
 __global__ __launch_bounds__(256) void qkv_norm_split_kernel(QkvParams p) {
   const int heads = p.hq + 2 * p.hkv;
   const int64_t g = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
@@ -128,13 +134,13 @@ __global__ __launch_bounds__(256) void qkv_norm_split_kernel(QkvParams p) {
   u32x4* dst;
   if (j < p.hq + p.hkv) {
     const bool is_q = j < p.hq;
-    const float ss = row16_sum(sum_sq8(x));
+    const float ss = row16_sum(sum_sq8<F16>(x));
     const float rinv = rsqrtf(ss * (1.0f / kHeadDim) + p.eps);
     const u32x4 w = (is_q ? p.q_weight : p.k_weight)[l];
-    x.x = scale_bf16x2(x.x, rinv, w.x);
-    x.y = scale_bf16x2(x.y, rinv, w.y);
-    x.z = scale_bf16x2(x.z, rinv, w.z);
-    x.w = scale_bf16x2(x.w, rinv, w.w);
+    x.x = scale_x2<F16>(x.x, rinv, w.x);
+    x.y = scale_x2<F16>(x.y, rinv, w.y);
+    x.z = scale_x2<F16>(x.z, rinv, w.z);
+    x.w = scale_x2<F16>(x.w, rinv, w.w);
     dst = is_q ? p.q + (b * p.hq + j) * 16 : p.k + (b * p.hkv + (j - p.hq)) * 16;
   } else {
     dst = p.v + (b * p.hkv + (j - p.hq - p.hkv)) * 16;
@@ -150,23 +156,24 @@ struct GateParams {
   int row_chunks;                  // inter / 8
 };
 
-// Each activation is rounded to bf16 before the product, as the chain
-// act(gate) * up over bf16 tensors rounds it.
-template <int ACT>
-__device__ __forceinline__ float act_bf16(float x) {
+// Each activation is rounded to the element format before the product, as the chain
+// act(gate) * up over 16-bit tensors rounds it.
+template <int ACT, bool F16>
+__device__ __forceinline__ float act_rounded(float x) {
   float y;
   if (ACT == KIN_ACT_SILU) y = x / (1.0f + expf(-x));
-  else if (ACT == KIN_ACT_GELU) y = 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+  else if (ACT == KIN_ACT_GELU) y = 0.5f * x * erfcf(-x * 0.70710678118654752440f);  // = 1 + erf(x / sqrt 2), without its cancellation for x < 0
   else y = fmaxf(x, 0.f);
-  return __uint_as_float(f32_to_bf16(y) << 16);
+  return elem_lo<F16>(f32_to_elem<F16>(y));
 }
 
-template <int ACT>
-__device__ __forceinline__ uint32_t gate_bf16x2(uint32_t g, uint32_t u) {
-  return f32_to_bf16(act_bf16<ACT>(bf16_lo(g)) * bf16_lo(u)) | (f32_to_bf16(act_bf16<ACT>(bf16_hi(g)) * bf16_hi(u)) << 16);
+template <int ACT, bool F16>
+__device__ __forceinline__ uint32_t gate_x2(uint32_t g, uint32_t u) {
+  return f32_to_elem<F16>(act_rounded<ACT, F16>(elem_lo<F16>(g)) * elem_lo<F16>(u)) |
+         (f32_to_elem<F16>(act_rounded<ACT, F16>(elem_hi<F16>(g)) * elem_hi<F16>(u)) << 16);
 }
 
-template <int ACT>
+template <int ACT, bool F16>
 __global__ __launch_bounds__(256) void gated_act_kernel(GateParams p) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= p.rows * p.row_chunks) return;
@@ -175,10 +182,10 @@ __global__ __launch_bounds__(256) void gated_act_kernel(GateParams p) {
   const u32x4 g = __builtin_nontemporal_load(p.gate + row * p.gate_stride + c);
   const u32x4 u = __builtin_nontemporal_load(p.up + row * p.up_stride + c);
   u32x4 o;
-  o.x = gate_bf16x2<ACT>(g.x, u.x);
-  o.y = gate_bf16x2<ACT>(g.y, u.y);
-  o.z = gate_bf16x2<ACT>(g.z, u.z);
-  o.w = gate_bf16x2<ACT>(g.w, u.w);
+  o.x = gate_x2<ACT, F16>(g.x, u.x);
+  o.y = gate_x2<ACT, F16>(g.y, u.y);
+  o.z = gate_x2<ACT, F16>(g.z, u.z);
+  o.w = gate_x2<ACT, F16>(g.w, u.w);
   p.out[idx] = o;
 }
 
@@ -191,10 +198,9 @@ static int check_row_stride(const char* fn, const char* name, int64_t stride, in
 
 }  // namespace kin
 
-extern "C" int kin_rms_norm(const void* x, void* residual, const void* weight, void* out, int64_t rows, int hidden,
-                            int64_t x_row_stride, int64_t out_row_stride, float eps, kin_stream_t stream) {
-  using namespace kin;
-  const char* fn = "kin_rms_norm";
+namespace kin {
+static int rms_norm_impl(const char* fn, bool f16, const void* x, void* residual, const void* weight, void* out, int64_t rows,
+                         int hidden, int64_t x_row_stride, int64_t out_row_stride, float eps, kin_stream_t stream) {
   if (!x || !weight || !out) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   if (rows < 0 || hidden < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: rows=%lld hidden=%d", fn, (long long)rows, hidden);
   int lpr;
@@ -225,10 +231,15 @@ extern "C" int kin_rms_norm(const void* x, void* residual, const void* weight, v
   p.inv_hidden = 1.0f / (float)hidden;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const unsigned g = (unsigned)grid;
-#define KIN_NORM_LAUNCH(LPR, MAXC)                                            \
-  do {                                                                        \
-    if (residual) rms_norm_kernel<LPR, MAXC, true><<<g, 256, 0, s>>>(p);      \
-    else rms_norm_kernel<LPR, MAXC, false><<<g, 256, 0, s>>>(p);              \
+#define KIN_NORM_LAUNCH(LPR, MAXC)                                                          \
+  do {                                                                                      \
+    if (f16) {                                                                              \
+      if (residual) rms_norm_kernel<LPR, MAXC, true, true><<<g, 256, 0, s>>>(p);            \
+      else rms_norm_kernel<LPR, MAXC, false, true><<<g, 256, 0, s>>>(p);                    \
+    } else {                                                                                \
+      if (residual) rms_norm_kernel<LPR, MAXC, true, false><<<g, 256, 0, s>>>(p);           \
+      else rms_norm_kernel<LPR, MAXC, false, false><<<g, 256, 0, s>>>(p);                   \
+    }                                                                                       \
   } while (0)
   if (lpr == 64) {
     if (p.chunks <= 4) KIN_NORM_LAUNCH(64, 4);
@@ -243,11 +254,9 @@ extern "C" int kin_rms_norm(const void* x, void* residual, const void* weight, v
   return check_hip(hipGetLastError(), "rms_norm_kernel launch");
 }
 
-extern "C" int kin_qkv_norm_split(const void* qkv, int64_t qkv_row_stride, const void* q_weight, const void* k_weight,
-                                  float eps, void* q, void* k, void* v, int batch, int num_q_heads, int num_kv_heads,
-                                  int head_dim, kin_stream_t stream) {
-  using namespace kin;
-  const char* fn = "kin_qkv_norm_split";
+static int qkv_norm_split_impl(const char* fn, bool f16, const void* qkv, int64_t qkv_row_stride, const void* q_weight,
+                               const void* k_weight, float eps, void* q, void* k, void* v, int batch, int num_q_heads,
+                               int num_kv_heads, int head_dim, kin_stream_t stream) {
   if (!qkv || !q_weight || !k_weight || !q || !k || !v) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   if (batch < 0 || num_q_heads < 1 || num_kv_heads < 1)
     return fail(KIN_ERR_BAD_SHAPE, "%s: batch=%d num_q_heads=%d num_kv_heads=%d", fn, batch, num_q_heads, num_kv_heads);
@@ -273,14 +282,13 @@ extern "C" int kin_qkv_norm_split(const void* qkv, int64_t qkv_row_stride, const
   p.hq = num_q_heads;
   p.hkv = num_kv_heads;
   p.eps = eps;
-  qkv_norm_split_kernel<<<(unsigned)grid, 256, 0, static_cast<hipStream_t>(stream)>>>(p);
+  if (f16) qkv_norm_split_kernel<true><<<(unsigned)grid, 256, 0, static_cast<hipStream_t>(stream)>>>(p);
+  else qkv_norm_split_kernel<false><<<(unsigned)grid, 256, 0, static_cast<hipStream_t>(stream)>>>(p);
   return check_hip(hipGetLastError(), "qkv_norm_split_kernel launch");
 }
 
-extern "C" int kin_gated_act(const void* gate, const void* up, void* out, int64_t rows, int inter,
-                             int64_t gate_row_stride, int64_t up_row_stride, int act, kin_stream_t stream) {
-  using namespace kin;
-  const char* fn = "kin_gated_act";
+static int gated_act_impl(const char* fn, bool f16, const void* gate, const void* up, void* out, int64_t rows, int inter,
+                          int64_t gate_row_stride, int64_t up_row_stride, int act, kin_stream_t stream) {
   if (!gate || !up || !out) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   if (rows < 0 || inter < 1 || inter % 8 != 0)
     return fail(KIN_ERR_BAD_SHAPE, "%s: rows=%lld inter=%d (inter must be a positive multiple of 8)", fn, (long long)rows, inter);
@@ -302,8 +310,51 @@ extern "C" int kin_gated_act(const void* gate, const void* up, void* out, int64_
   if (grid > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: rows*inter is too large", fn);
   if (rows == 0) return KIN_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (act == KIN_ACT_SILU) gated_act_kernel<KIN_ACT_SILU><<<(unsigned)grid, 256, 0, s>>>(p);
-  else if (act == KIN_ACT_GELU) gated_act_kernel<KIN_ACT_GELU><<<(unsigned)grid, 256, 0, s>>>(p);
-  else gated_act_kernel<KIN_ACT_RELU><<<(unsigned)grid, 256, 0, s>>>(p);
+#define KIN_GATE_LAUNCH(ACT)                                                       \
+  do {                                                                             \
+    if (f16) gated_act_kernel<ACT, true><<<(unsigned)grid, 256, 0, s>>>(p);        \
+    else gated_act_kernel<ACT, false><<<(unsigned)grid, 256, 0, s>>>(p);           \
+  } while (0)
+  if (act == KIN_ACT_SILU) KIN_GATE_LAUNCH(KIN_ACT_SILU);
+  else if (act == KIN_ACT_GELU) KIN_GATE_LAUNCH(KIN_ACT_GELU);
+  else KIN_GATE_LAUNCH(KIN_ACT_RELU);
+#undef KIN_GATE_LAUNCH
   return check_hip(hipGetLastError(), "gated_act_kernel launch");
 }
+}  // namespace kin
+
+extern "C" {
+
+int kin_rms_norm(const void* x, void* residual, const void* weight, void* out, int64_t rows, int hidden,
+                 int64_t x_row_stride, int64_t out_row_stride, float eps, kin_stream_t stream) {
+  return kin::rms_norm_impl("kin_rms_norm", false, x, residual, weight, out, rows, hidden, x_row_stride, out_row_stride, eps,
+                            stream);
+}
+int kin_rms_norm_f16(const void* x, void* residual, const void* weight, void* out, int64_t rows, int hidden,
+                     int64_t x_row_stride, int64_t out_row_stride, float eps, kin_stream_t stream) {
+  return kin::rms_norm_impl("kin_rms_norm_f16", true, x, residual, weight, out, rows, hidden, x_row_stride, out_row_stride,
+                            eps, stream);
+}
+int kin_qkv_norm_split(const void* qkv, int64_t qkv_row_stride, const void* q_weight, const void* k_weight, float eps,
+                       void* q, void* k, void* v, int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                       kin_stream_t stream) {
+  return kin::qkv_norm_split_impl("kin_qkv_norm_split", false, qkv, qkv_row_stride, q_weight, k_weight, eps, q, k, v, batch,
+                                  num_q_heads, num_kv_heads, head_dim, stream);
+}
+int kin_qkv_norm_split_f16(const void* qkv, int64_t qkv_row_stride, const void* q_weight, const void* k_weight, float eps,
+                           void* q, void* k, void* v, int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                           kin_stream_t stream) {
+  return kin::qkv_norm_split_impl("kin_qkv_norm_split_f16", true, qkv, qkv_row_stride, q_weight, k_weight, eps, q, k, v, batch,
+                                  num_q_heads, num_kv_heads, head_dim, stream);
+}
+int kin_gated_act(const void* gate, const void* up, void* out, int64_t rows, int inter, int64_t gate_row_stride,
+                  int64_t up_row_stride, int act, kin_stream_t stream) {
+  return kin::gated_act_impl("kin_gated_act", false, gate, up, out, rows, inter, gate_row_stride, up_row_stride, act, stream);
+}
+int kin_gated_act_f16(const void* gate, const void* up, void* out, int64_t rows, int inter, int64_t gate_row_stride,
+                      int64_t up_row_stride, int act, kin_stream_t stream) {
+  return kin::gated_act_impl("kin_gated_act_f16", true, gate, up, out, rows, inter, gate_row_stride, up_row_stride, act,
+                             stream);
+}
+
+}  // extern "C"

@@ -661,14 +661,15 @@ def check_page_table(page_indices, page_indptr, last_page_len, page_size, num_pa
 ACTIVATIONS = {"silu": 0, "gelu": 1, "relu": 2}
 
 
-def _row_view(t: torch.Tensor, name: str, device=None):
-    """(rows, width, row stride in elements) of a bf16 tensor whose rows are its
-    last dimension: any contiguous shape, or a 2-D view with a row stride (a
-    slice of a wider projection)."""
+def _row_view(t: torch.Tensor, name: str, device=None, dtype=None):
+    """(rows, width, row stride in elements) of a bf16 / fp16 tensor (``dtype``: that
+    very type) whose rows are its last dimension: any contiguous shape, or a 2-D view
+    with a row stride (a slice of a wider projection)."""
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
-    if t.dtype != torch.bfloat16:
-        raise TypeError(f"{name} must be torch.bfloat16, got {t.dtype}")
+    if t.dtype not in ELEM_DTYPES or (dtype is not None and t.dtype != dtype):
+        want = dtype if dtype is not None else "torch.bfloat16 or torch.float16"
+        raise TypeError(f"{name} must be {want}, got {t.dtype}")
     if t.device.type != "cuda":
         raise ValueError(f"{name} must live on the GPU (device 'cuda'), got {t.device}")
     if device is not None and t.device != device:
@@ -691,23 +692,23 @@ def rms_norm(x, weight, eps: float, residual=None, out=None) -> torch.Tensor:
     (benchmark/model_utils.py:27-41): ``residual`` becomes ``x + residual`` and
     the norm of that sum is returned."""
     rows, hidden, x_stride = _row_view(x, "x")
-    dev = x.device
-    _require(weight, "weight", torch.bfloat16, 1, dev)
+    dev, dt = x.device, x.dtype
+    _require(weight, "weight", dt, 1, dev)
     if weight.numel() != hidden:
         raise ValueError(f"weight has {weight.numel()} entries for rows of {hidden}")
     if out is None:
         out = torch.empty(x.shape, dtype=x.dtype, device=dev)
-    orows, owidth, out_stride = _row_view(out, "out", dev)
+    orows, owidth, out_stride = _row_view(out, "out", dev, dt)
     if (orows, owidth) != (rows, hidden):
         raise ValueError(f"out shape {tuple(out.shape)} does not match x {tuple(x.shape)}")
     if residual is not None:
-        _require(residual, "residual", torch.bfloat16, None, dev)
+        _require(residual, "residual", dt, None, dev)
         if residual.numel() != rows * hidden or residual.shape[-1] != hidden:
             raise ValueError(f"residual shape {tuple(residual.shape)} does not match x {tuple(x.shape)}")
     lib = _lib.load()
     with _on(dev):
-        _lib.check(lib.kin_rms_norm(_ptr(x), _ptr(residual), _ptr(weight), _ptr(out), rows, hidden, x_stride, out_stride,
-                                    float(eps), _stream(dev)))
+        _lib.check(_entry(lib, "kin_rms_norm", dt)(_ptr(x), _ptr(residual), _ptr(weight), _ptr(out), rows, hidden, x_stride,
+                                                   out_stride, float(eps), _stream(dev)))
     return out
 
 
@@ -717,45 +718,46 @@ def qkv_norm_split(qkv, q_weight, k_weight, eps: float, num_q_heads: int, num_kv
     q and k heads RMS-normalised: the split, qk_norm calls and reshapes of
     benchmark/blocktopk_decoder.py:196-207 in one pass."""
     batch, width, stride = _row_view(qkv, "qkv")
-    dev = qkv.device
+    dev, dt = qkv.device, qkv.dtype
     if width != (num_q_heads + 2 * num_kv_heads) * HEAD_DIM:
         raise ValueError(f"qkv rows have {width} elements, expected (Hq + 2*Hkv) * {HEAD_DIM} = "
                          f"{(num_q_heads + 2 * num_kv_heads) * HEAD_DIM}")
-    _require(q_weight, "q_weight", torch.bfloat16, 1, dev)
-    _require(k_weight, "k_weight", torch.bfloat16, 1, dev)
+    _require(q_weight, "q_weight", dt, 1, dev)
+    _require(k_weight, "k_weight", dt, 1, dev)
     if q_weight.numel() != HEAD_DIM or k_weight.numel() != HEAD_DIM:
         raise ValueError(f"q_weight and k_weight must have {HEAD_DIM} entries")
-    q = torch.empty(batch, num_q_heads, HEAD_DIM, dtype=torch.bfloat16, device=dev)
-    k = torch.empty(batch, num_kv_heads, HEAD_DIM, dtype=torch.bfloat16, device=dev)
-    v = torch.empty(batch, num_kv_heads, HEAD_DIM, dtype=torch.bfloat16, device=dev)
+    q = torch.empty(batch, num_q_heads, HEAD_DIM, dtype=dt, device=dev)
+    k = torch.empty(batch, num_kv_heads, HEAD_DIM, dtype=dt, device=dev)
+    v = torch.empty(batch, num_kv_heads, HEAD_DIM, dtype=dt, device=dev)
     lib = _lib.load()
     with _on(dev):
-        _lib.check(lib.kin_qkv_norm_split(_ptr(qkv), stride, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(q), _ptr(k),
-                                          _ptr(v), batch, int(num_q_heads), int(num_kv_heads), HEAD_DIM, _stream(dev)))
+        _lib.check(_entry(lib, "kin_qkv_norm_split", dt)(_ptr(qkv), stride, _ptr(q_weight), _ptr(k_weight), float(eps),
+                                                         _ptr(q), _ptr(k), _ptr(v), batch, int(num_q_heads),
+                                                         int(num_kv_heads), HEAD_DIM, _stream(dev)))
     return q, k, v
 
 
 def gated_act(gate, up, act: str = "silu", out=None) -> torch.Tensor:
     """``act(gate) * up`` of the gated MLP (benchmark/blocktopk_decoder.py:234-237),
     rounded to bf16 after the activation and after the product as the two tensor
-    operations round.  ``gate`` and ``up`` may be column slices of one fused
+    operations round (bf16 or fp16, whichever the tensors are).  ``gate`` and ``up`` may be column slices of one fused
     projection (2-D views with a row stride)."""
     if act not in ACTIVATIONS:
         raise ValueError(f"act must be one of {sorted(ACTIVATIONS)}, got {act!r}")
     rows, inter, g_stride = _row_view(gate, "gate")
-    dev = gate.device
-    urows, uwidth, u_stride = _row_view(up, "up", dev)
+    dev, dt = gate.device, gate.dtype
+    urows, uwidth, u_stride = _row_view(up, "up", dev, dt)
     if (urows, uwidth) != (rows, inter):
         raise ValueError(f"up shape {tuple(up.shape)} does not match gate {tuple(gate.shape)}")
     if out is None:
-        out = torch.empty(gate.shape, dtype=torch.bfloat16, device=dev)
-    _require(out, "out", torch.bfloat16, None, dev)
+        out = torch.empty(gate.shape, dtype=dt, device=dev)
+    _require(out, "out", dt, None, dev)
     if out.numel() != rows * inter or out.shape[-1] != inter:
         raise ValueError(f"out shape {tuple(out.shape)} does not match gate {tuple(gate.shape)}")
     lib = _lib.load()
     with _on(dev):
-        _lib.check(lib.kin_gated_act(_ptr(gate), _ptr(up), _ptr(out), rows, inter, g_stride, u_stride, ACTIVATIONS[act],
-                                     _stream(dev)))
+        _lib.check(_entry(lib, "kin_gated_act", dt)(_ptr(gate), _ptr(up), _ptr(out), rows, inter, g_stride, u_stride,
+                                                    ACTIVATIONS[act], _stream(dev)))
     return out
 
 

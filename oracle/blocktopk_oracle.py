@@ -571,21 +571,22 @@ def litesys_decode(q, K, V, topk_block, local, sink=4, block_size=16, sm_scale=N
 
 
 def rms_norm(x, weight, eps, residual=None):
-    """RMSNorm over the last axis, bf16 bits in and out: x * rsqrt(mean(x^2) + eps)
+    """RMSNorm over the last axis, element bits in and out (bf16, or fp16 inside
+    ``element_format("f16")``; "bf16" below then reads "fp16"): x * rsqrt(mean(x^2) + eps)
     * weight, which is flashinfer.rmsnorm as the reference's layer_norm and
     qk_norm call it (benchmark/model_utils.py:4-25).  With ``residual`` the sum
     x + residual, rounded to bf16 as a bf16 tensor add rounds it
     (benchmark/blocktopk_decoder.py:229-232; fused_layer_norm,
     benchmark/model_utils.py:27-41), is normalised instead.  Returns
     (out_bits, new_residual_bits or None)."""
-    xf = bf16_to_f32(x).astype(np.float64)
+    xf = elem_to_f32(x).astype(np.float64)
     new_res = None
     if residual is not None:
-        new_res = f32_to_bf16((xf + bf16_to_f32(residual).astype(np.float64)).astype(np.float32))
-        xf = bf16_to_f32(new_res).astype(np.float64)
-    w = bf16_to_f32(weight).astype(np.float64)
+        new_res = f32_to_elem((xf + elem_to_f32(residual).astype(np.float64)).astype(np.float32))
+        xf = elem_to_f32(new_res).astype(np.float64)
+    w = elem_to_f32(weight).astype(np.float64)
     r = 1.0 / np.sqrt(np.mean(xf * xf, axis=-1, keepdims=True) + float(eps))
-    return f32_to_bf16((xf * r * w).astype(np.float32)), new_res
+    return f32_to_elem((xf * r * w).astype(np.float32)), new_res
 
 
 def qkv_norm_split(qkv, q_weight, k_weight, eps, num_q_heads, num_kv_heads, head_dim=128):
@@ -606,7 +607,7 @@ def gated_act(gate, up, act="silu"):
     tensor operations.  gelu is the erf form."""
     from math import erf
 
-    g = bf16_to_f32(gate).astype(np.float64)
+    g = elem_to_f32(gate).astype(np.float64)
     if act == "silu":
         a = g / (1.0 + np.exp(-g))
     elif act == "gelu":
@@ -615,8 +616,8 @@ def gated_act(gate, up, act="silu"):
         a = np.maximum(g, 0.0)
     else:
         raise ValueError(f"unknown activation {act!r}")
-    a = bf16_to_f32(f32_to_bf16(a.astype(np.float32))).astype(np.float64)
-    return f32_to_bf16((a * bf16_to_f32(up).astype(np.float64)).astype(np.float32))
+    a = elem_to_f32(f32_to_elem(a.astype(np.float32))).astype(np.float64)
+    return f32_to_elem((a * elem_to_f32(up).astype(np.float64)).astype(np.float32))
 
 
 # ---------------------------------------------------------------------------

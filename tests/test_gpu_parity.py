@@ -1570,11 +1570,18 @@ def test_fused_step_full_size(ops):
 # --------------------------------------------------------------------------- whole decoder layer
 
 
+@pytest.mark.parametrize("fmt", ["bf16", "f16"])
 @pytest.mark.parametrize("dense", [False, True])
-def test_decoder_layer_matches_fp32_reference(ops, dense):
+def test_decoder_layer_matches_fp32_reference(ops, dense, fmt):
     """The drop-in layers: norms/GEMMs in PyTorch around the HIP attention.  The
     attention inside is checked against the oracle on the layer's own q, k, v;
-    the rest against an fp32 restatement of the same layer."""
+    the rest against an fp32 restatement of the same layer.  In bfloat16 and in
+    float16 (the reference moves the whole layer to --dtype, benchmark/blocktopk.py:18,37-40)."""
+    with O.element_format(fmt):
+        _decoder_layer_case(ops, dense, torch.float16 if fmt == "f16" else torch.bfloat16)
+
+
+def _decoder_layer_case(ops, dense, dt):
     from types import SimpleNamespace
 
     from kinetics_amd.decoder_layer import BlockTopkDecoderLayer, DenseDecoderLayer, init_weights, qwen3_config, rms_norm
@@ -1585,14 +1592,14 @@ def test_decoder_layer_matches_fp32_reference(ops, dense):
     B, prefix, topk = 6, PS * 40, 8
     torch.manual_seed(11)
     if dense:
-        layer = DenseDecoderLayer(cfg, 2, B, prefix, prefix + 512, PS, DEV, torch.bfloat16, seed=5)
+        layer = DenseDecoderLayer(cfg, 2, B, prefix, prefix + 512, PS, DEV, dt, seed=5)
     else:
-        layer = BlockTopkDecoderLayer(cfg, 2, B, prefix, prefix + 512, PS, topk, DEV, torch.bfloat16, seed=5)
+        layer = BlockTopkDecoderLayer(cfg, 2, B, prefix, prefix + 512, PS, topk, DEV, dt, seed=5)
     layer.apply(init_weights)
-    layer.eval().to(DEV, dtype=torch.bfloat16)
+    layer.eval().to(DEV, dtype=dt)
     assert (layer.num_heads, layer.num_kv_heads) == (4, 1)  # world_size 2 shard
     layer.prepare_wrapper() if dense else layer.prepare_wrapper(prefix)
-    hidden = torch.randn(B, 1, 512, device=DEV).to(torch.bfloat16)
+    hidden = torch.randn(B, 1, 512, device=DEV).to(dt)
     st = layer.attn.state if dense else layer.attn
     kv_before = P.from_torch(st.kv_cache)
     kbar_before = P.from_torch(st.compressed_key_cache)
@@ -1600,7 +1607,7 @@ def test_decoder_layer_matches_fp32_reference(ops, dense):
         q, k, v = layer._qkv(hidden)
     out = layer(hidden.clone())
     torch.cuda.synchronize()
-    assert out.shape == hidden.shape and out.dtype == torch.bfloat16
+    assert out.shape == hidden.shape and out.dtype == dt
     # q, k, v against fp32
     W = {n: p.detach().float().cpu() for n, p in layer.named_parameters()}
     h32 = hidden.float().cpu()
@@ -1608,7 +1615,7 @@ def test_decoder_layer_matches_fp32_reference(ops, dense):
     def rn(x, w):
         return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * w
 
-    x = rn(h32, W["input_layernorm_weight"]).to(torch.bfloat16).float()
+    x = rn(h32, W["input_layernorm_weight"]).to(dt).float()
     qkv = x @ W["wqkv.weight"].T + W["wqkv.bias"]
     q32, k32, v32 = qkv.split((512, 128, 128), dim=-1)
     q32 = rn(q32.reshape(B, 4, D), W["qnorm_weight"])
@@ -1627,17 +1634,17 @@ def test_decoder_layer_matches_fp32_reference(ops, dense):
         assert np.array_equal(layer.attn.topk_page_indices.cpu().numpy(), res["sel_pages"])
     assert np.array_equal(P.from_torch(st.kv_cache), kv_before)
     # the rest of the layer in fp32
-    o32 = torch.from_numpy(attn).float().to(torch.bfloat16).float().reshape(B, 1, 512)
+    o32 = torch.from_numpy(attn).float().to(dt).float().reshape(B, 1, 512)
     h1 = h32 + o32 @ W["wo.weight"].T
     y = rn(h1, W["post_attention_layernorm_weight"])
     want = h1 + (torch.nn.functional.silu(y @ W["gate_proj.weight"].T) * (y @ W["up_proj.weight"].T)) @ W["down_proj.weight"].T
     got = out.float().cpu()
     assert torch.allclose(got, want, rtol=5e-2, atol=5e-2), (got - want).abs().max()
-    assert rms_norm(hidden, 1e-6, layer.input_layernorm_weight).dtype == torch.bfloat16
+    assert rms_norm(hidden, 1e-6, layer.input_layernorm_weight).dtype == dt
     # the whole forward traces without a graph break (the reference compiles it with fullgraph=True,
     # benchmark/blocktopk.py:41-43); backend "eager": no code generation, the same kernels run
     compiled = torch.compile(layer.forward, backend="eager", fullgraph=True)
-    h_c = torch.randn(B, 1, 512, device=DEV).to(torch.bfloat16)
+    h_c = torch.randn(B, 1, 512, device=DEV).to(dt)
     want_c = layer(h_c.clone()).clone()
     got_c = compiled(h_c.clone())
     torch.cuda.synchronize()
@@ -1646,7 +1653,7 @@ def test_decoder_layer_matches_fp32_reference(ops, dense):
     # with eager work and synchronisations between the replays
     graphed = layer.graphed(hidden)
     for i in range(4):
-        h_i = torch.randn(B, 1, 512, device=DEV).to(torch.bfloat16)
+        h_i = torch.randn(B, 1, 512, device=DEV).to(dt)
         eager = layer(h_i.clone()).clone()
         torch.cuda.synchronize()
         replay = graphed(h_i)

@@ -796,3 +796,43 @@ def test_gated_act_against_torch_bf16_ops(act):
     assert np.array_equal(O.gated_act(big, u[:1, :8], act), O.f32_to_bf16(32.0 * O.bf16_to_f32(u[:1, :8])))
     with pytest.raises(ValueError):
         O.gated_act(g, u, "tanh")
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu", "relu"])
+def test_layer_rows_in_float16_against_torch(act):
+    """The same three functions inside element_format("f16"): torch's own float16
+    tensor operations (computed in fp32, rounded once per operation) are the pin."""
+    rng = np.random.default_rng(25)
+    with O.element_format("f16"):
+        x = O.f32_to_elem(rng.standard_normal((6, 256)).astype(np.float32) * 3)
+        r = O.f32_to_elem(rng.standard_normal((6, 256)).astype(np.float32) * 2)
+        w = O.f32_to_elem(1 + 0.2 * rng.standard_normal(256).astype(np.float32))
+        assert P.to_torch(x).dtype == torch.float16
+        got, new_r = O.rms_norm(x, w, 1e-6, residual=r)
+        want_r = P.to_torch(x) + P.to_torch(r)              # one float16 tensor add
+        assert np.array_equal(new_r, P.from_torch(want_r))
+        want = torch.nn.functional.rms_norm(want_r.double(), (256,), P.to_torch(w).double(), 1e-6)
+        assert _ulps_elem(got, P.from_torch(want.float().to(torch.float16))) <= 1
+        g = O.f32_to_elem(rng.standard_normal((4, 64)).astype(np.float32) * 3)
+        u = O.f32_to_elem(rng.standard_normal((4, 64)).astype(np.float32) * 2)
+        fn = {"silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu, "relu": torch.relu}[act]
+        want_g = fn(P.to_torch(g)) * P.to_torch(u)          # two float16 tensor operations
+        # torch evaluates gelu in fp32, where 1 + erf(g / sqrt 2) cancels for g < -2: its own error (1e-4
+        # relative) shows at float16's 11 bits, the oracle's float64 does not have it
+        assert _ulps_elem(O.gated_act(g, u, act), P.from_torch(want_g)) <= (2 if act == "gelu" else 1)
+        # the format matters: the same bits read as bf16 give another answer
+        assert not np.array_equal(O.rms_norm(x, w, 1e-6)[0], _as_bf16(lambda: O.rms_norm(x, w, 1e-6)[0]))
+
+
+def _as_bf16(fn):
+    with O.element_format("bf16"):
+        return fn()
+
+
+def _ulps_elem(a_bits, b_bits):
+    def key(b):
+        b = b.astype(np.int32)
+        return np.where(b & 0x8000, 0x8000 - b, b)
+
+    near = np.abs(O.elem_to_f32(a_bits).astype(np.float64) - O.elem_to_f32(b_bits)) <= 1e-6
+    return int(np.where(near, 0, np.abs(key(a_bits) - key(b_bits))).max())
