@@ -400,6 +400,18 @@ int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
                           int head_dim, int page_size, int64_t num_pages,
                           int max_pages_per_seq, int sel_stride, float sm_scale,
                           kin_stream_t stream);
+int kin_token_topk_decode_f16(const kin_f16_t* q, const kin_f16_t* kv_cache,
+                              const int32_t* page_indices, const int32_t* page_indptr,
+                              const int32_t* last_page_len,
+                              int topk_tokens, int sink_tokens, int local_tokens,
+                              int first_page_offset,
+                              int32_t* sel_tokens, int32_t* sel_count,
+                              kin_f16_t* out, float* lse,
+                              void* workspace, size_t workspace_bytes,
+                              int batch, int num_q_heads, int num_kv_heads,
+                              int head_dim, int page_size, int64_t num_pages,
+                              int max_pages_per_seq, int sel_stride, float sm_scale,
+                              kin_stream_t stream);
 
 /*
  * Strided overlapping-block top-k decode attention in one launch -- LiteSys'
@@ -432,6 +444,18 @@ int kin_strided_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
                             int head_dim, int page_size, int64_t num_pages,
                             int max_pages_per_seq, int sel_stride, float sm_scale,
                             kin_stream_t stream);
+int kin_strided_topk_decode_f16(const kin_f16_t* q, const kin_f16_t* kv_cache,
+                                const int32_t* page_indices, const int32_t* page_indptr,
+                                const int32_t* last_page_len,
+                                int topk_blocks, int block_size, int stride,
+                                int sink_tokens, int local_tokens, int first_page_offset,
+                                int32_t* sel_tokens, int32_t* sel_count,
+                                kin_f16_t* out, float* lse,
+                                void* workspace, size_t workspace_bytes,
+                                int batch, int num_q_heads, int num_kv_heads,
+                                int head_dim, int page_size, int64_t num_pages,
+                                int max_pages_per_seq, int sel_stride, float sm_scale,
+                                kin_stream_t stream);
 
 /*
  * Page-table metadata for a slot-based cache -- the paged replacement of
@@ -527,9 +551,9 @@ int kin_check_page_table(const int32_t* page_indices, const int32_t* page_indptr
  * float16 twin: same arguments, same meaning, same fp32 accumulation, with q, k,
  * v, kv_cache, kbar and out holding IEEE binary16 (round-to-nearest-even on
  * every store; the mean key is the fp32 sum times 1/page_size rounded to
- * binary16).  The row-wise layer kernels further down have float16 twins too
- * (the reference moves the whole layer to --dtype).  The token-granular policies
- * and the entry point with built-in scratch are bfloat16 only.
+ * binary16).  The token-granular policies above and the row-wise layer kernels
+ * further down have float16 twins too (the reference moves the whole layer to
+ * --dtype).  Only the entry point with built-in scratch is bfloat16 only.
  */
 int kin_append_paged_kv_f16(const kin_f16_t* k, const kin_f16_t* v,
                             kin_f16_t* kv_cache, kin_f16_t* kbar,

@@ -93,7 +93,7 @@ SIGNATURES = {
 # the float16 twins have the signatures of their bfloat16 originals
 for _name in ("kin_append_paged_kv", "kin_build_kbar", "kin_append_paged_kv_ragged", "kin_block_score_topk",
               "kin_sparse_paged_decode", "kin_dense_paged_decode", "kin_blocktopk_decode_step", "kin_rms_norm",
-              "kin_qkv_norm_split", "kin_gated_act"):
+              "kin_qkv_norm_split", "kin_gated_act", "kin_token_topk_decode", "kin_strided_topk_decode"):
     SIGNATURES[_name + "_f16"] = SIGNATURES[_name]
 
 _lib = None

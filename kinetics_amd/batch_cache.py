@@ -63,9 +63,6 @@ class PagedBatchKVManager:
     def __init__(self, config, max_batch_size: int, max_seq_len: int, device, dtype, **kwargs):
         if dtype not in (torch.bfloat16, torch.float16):
             raise ValueError("the HIP kernels are built for bfloat16 and float16")
-        if dtype is torch.float16 and (kwargs.get("attn_topk") is not None or kwargs.get("attn_stride") is not None
-                                       or (kwargs.get("attn_local") is not None and kwargs.get("attn_block_topk") is None)):
-            raise NotImplementedError("the token-granular policies are built for bfloat16 only")
         self.config = config
         self.max_length = max_seq_len
         self.device = torch.device(device)

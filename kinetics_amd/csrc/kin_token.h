@@ -265,7 +265,7 @@ __device__ __forceinline__ void radix_select_emit(const Keys& keys, int n_keys, 
 // those pages (slots past the last token included).  emit must not branch around
 // vector memory operations (store through a descriptor, out of range when !valid).  16-byte loads straight to registers, 16 of them in flight per
 // lane; no LDS, no barrier.
-template <int NW, typename Emit>
+template <int NW, bool F16 = false, typename Emit>
 __device__ __forceinline__ void stream_token_scores(const TokenArgs& a, int pg0, int pg1, Emit emit) {
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -282,10 +282,10 @@ __device__ __forceinline__ void stream_token_scores(const TokenArgs& a, int pg0,
     const uint16_t* qp = a.q_bh + 8 * c16;
     for (int g = 0; g < G; ++g) {
       const uint4 x = *reinterpret_cast<const uint4*>(qp + (int64_t)g * kHeadDim);
-      qm[0] += bf16_lo(x.x); qm[1] += bf16_hi(x.x);
-      qm[2] += bf16_lo(x.y); qm[3] += bf16_hi(x.y);
-      qm[4] += bf16_lo(x.z); qm[5] += bf16_hi(x.z);
-      qm[6] += bf16_lo(x.w); qm[7] += bf16_hi(x.w);
+      qm[0] += elem_lo<F16>(x.x); qm[1] += elem_hi<F16>(x.x);
+      qm[2] += elem_lo<F16>(x.y); qm[3] += elem_hi<F16>(x.y);
+      qm[4] += elem_lo<F16>(x.z); qm[5] += elem_hi<F16>(x.z);
+      qm[6] += elem_lo<F16>(x.w); qm[7] += elem_hi<F16>(x.w);
     }
     const float inv = 1.0f / (float)G;
 #pragma unroll
@@ -350,10 +350,10 @@ __device__ __forceinline__ void stream_token_scores(const TokenArgs& a, int pg0,
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float s = 0.f;
-        s = fmaf(qm[0], bf16_lo(kx[i].x), s); s = fmaf(qm[1], bf16_hi(kx[i].x), s);
-        s = fmaf(qm[2], bf16_lo(kx[i].y), s); s = fmaf(qm[3], bf16_hi(kx[i].y), s);
-        s = fmaf(qm[4], bf16_lo(kx[i].z), s); s = fmaf(qm[5], bf16_hi(kx[i].z), s);
-        s = fmaf(qm[6], bf16_lo(kx[i].w), s); s = fmaf(qm[7], bf16_hi(kx[i].w), s);
+        s = fmaf(qm[0], elem_lo<F16>(kx[i].x), s); s = fmaf(qm[1], elem_hi<F16>(kx[i].x), s);
+        s = fmaf(qm[2], elem_lo<F16>(kx[i].y), s); s = fmaf(qm[3], elem_hi<F16>(kx[i].y), s);
+        s = fmaf(qm[4], elem_lo<F16>(kx[i].z), s); s = fmaf(qm[5], elem_hi<F16>(kx[i].z), s);
+        s = fmaf(qm[6], elem_lo<F16>(kx[i].w), s); s = fmaf(qm[7], elem_hi<F16>(kx[i].w), s);
         acc[i] = row16_sum(s);
       }
       const int i_mine = c16 & 3;
@@ -381,13 +381,13 @@ __device__ __forceinline__ bool token_needs_scores(const TokenArgs& a) {
 // LDSK, into a.lds_keys; 0 marks "not a candidate", order_key is never 0 for a finite
 // score.  hist: 256 zeroed LDS counters that receive the histogram of the keys' top
 // byte, or null.  No barrier inside; the stores are complete after s_waitcnt(0).
-template <int NW, bool LDSK = false>
+template <int NW, bool LDSK = false, bool F16 = false>
 __device__ __forceinline__ void token_score_keys(const TokenArgs& a, int pg0, int pg1, uint32_t* hist) {
   const int dyn_lo = a.pad + a.n_sink, dyn_hi = dyn_lo + a.n_dyn;  // cache slots of the candidates
   const __amdgpu_buffer_rsrc_t keys_rsrc = make_rsrc(a.keys, LDSK ? 0 : a.n_pages * kPageSize * 4);
   uint32_t* lds_keys = a.lds_keys;
   const int dump = a.n_pages * kPageSize;  // lanes without a row write here
-  stream_token_scores<NW>(a, pg0, pg1, [&](int c, float score, bool valid) {
+  stream_token_scores<NW, F16>(a, pg0, pg1, [&](int c, float score, bool valid) {
     const uint32_t key = (c >= dyn_lo && c < dyn_hi) ? order_key(score) : 0u;
     if constexpr (LDSK)
       lds_keys[valid ? c : dump] = key;
@@ -465,12 +465,12 @@ __device__ __forceinline__ bool strided_needs_scores(const TokenArgs& a, const S
 
 // fp32 scores of the tokens of the pages pg0 <= p < pg1 -> sa.scores (device-scope
 // stores) or, LDSK, -> a.lds_keys (as bit patterns).
-template <int NW, bool LDSK = false>
+template <int NW, bool LDSK = false, bool F16 = false>
 __device__ __forceinline__ void strided_score_tokens(const TokenArgs& a, const StridedArgs& sa, int pg0, int pg1) {
   const __amdgpu_buffer_rsrc_t scores_rsrc = make_rsrc(sa.scores, LDSK ? 0 : a.n_pages * kPageSize * 4);
   uint32_t* lds_scores = a.lds_keys;
   const int dump = a.n_pages * kPageSize;
-  stream_token_scores<NW>(a, pg0, pg1, [&](int c, float score, bool valid) {
+  stream_token_scores<NW, F16>(a, pg0, pg1, [&](int c, float score, bool valid) {
     if constexpr (LDSK)
       lds_scores[valid ? c : dump] = __float_as_uint(score);
     else
@@ -597,7 +597,7 @@ __device__ __forceinline__ int strided_select_list(const TokenArgs& a, const Str
 // and online softmax as attend_list(); a "page" is any 16 consecutive list
 // entries, each K and V row fetched from its own address.
 // lds: attend_lds_bytes(NW); sm_m / sm_l: NW x (4*NG) floats each.
-template <int NG, int NW, typename Emit>
+template <int NG, int NW, bool F16 = false, typename Emit>
 __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t* list, unsigned char* lds,
                                               float (*sm_m)[4 * NG], float (*sm_l)[4 * NG], Emit emit) {
   const int tid = threadIdx.x;
@@ -634,15 +634,15 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
   for (int u = 0; u < 8; ++u) O[u] = floatx4{0.f, 0.f, 0.f, 0.f};
   auto scores = [&](const uint4 (&ka)[4], float (&pr)[4], int valid) {
     if constexpr (NG == 4)
-      page_scores_wide<false>(ka, qB, m_run, l_run, O, pr, a.scale_log2, 0, valid, kg);
+      page_scores_wide<F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, 0, valid, kg);
     else
-      page_scores<false>(ka, qB, m_run, l_run, O, pr, a.scale_log2, 0, valid, kg);
+      page_scores<F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, 0, valid, kg);
   };
   auto pv = [&](const u32x4 (&vr)[4], const float (&pr)[4]) {
     if constexpr (NG == 4)
-      page_pv_wide<false>(vr, pr, O);
+      page_pv_wide<F16>(vr, pr, O);
     else
-      page_pv<false>(vr, pr, O);
+      page_pv<F16>(vr, pr, O);
   };
 
   // This wave takes the 16-entry groups w, w+NW, ...  Entries past the end (and

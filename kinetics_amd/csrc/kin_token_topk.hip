@@ -35,11 +35,11 @@ struct TokenTopkParams {
 
 // STRIDED = false: token-level top-k (p.topk tokens); true: strided overlapping
 // blocks (p.topk blocks).  LDSK: the per-token keys / scores live in LDS instead of
-// the HBM workspace (one workgroup per list, the sequence short enough).
+// the HBM workspace (one workgroup per list, the sequence short enough).  F16: float16 tensors.
 // Dynamic LDS: region 0 (p.region0_bytes: K staging attend_lds_bytes(NW), which the keys
 // of an LDSK kernel share: they are dead when the attention starts) | int32 list[list_cap]
 // | uint32 bitmap[] (strided only)
-template <int NG, int NW, bool STRIDED, bool LDSK>
+template <int NG, int NW, bool STRIDED, bool LDSK, bool F16>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(TokenTopkParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ float sm_m[NW][4 * NG];
@@ -118,8 +118,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
       if (tid < 256) sh.hist[tid] = 0;
       __syncthreads();
     }
-    if (STRIDED) strided_score_tokens<NW, LDSK>(t, sa, pg0, pg1);
-    else token_score_keys<NW, LDSK>(t, pg0, pg1, hist_on_the_fly ? sh.hist : nullptr);
+    if (STRIDED) strided_score_tokens<NW, LDSK, F16>(t, sa, pg0, pg1);
+    else token_score_keys<NW, LDSK, F16>(t, pg0, pg1, hist_on_the_fly ? sh.hist : nullptr);
     // Every wave waits for its own stores to be acknowledged; after the barrier the
     // workgroup's scores are in memory.
     __builtin_amdgcn_s_waitcnt(0);
@@ -157,8 +157,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
   a.first_skip = 0;
   a.rotate = 0;
   a.page_size = kPageSize;
-  attend_tokens<NG, NW>(a, list, smem, sm_m, sm_l, [&](int g, int d, float o, float lse2) {
-    p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_bf16(o);
+  attend_tokens<NG, NW, F16>(a, list, smem, sm_m, sm_l, [&](int g, int d, float o, float lse2) {
+    p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(o);
     if (p.lse && d == 0) p.lse[hq0 + g] = lse2 * kLn2;
   });
 }
@@ -183,7 +183,7 @@ static int token_score_chunks(int64_t lists, int max_pages_per_seq) {
 }
 
 // Shared by the two entry points.  topk counts tokens (block == 0) or blocks.
-static int launch_token_policy(const char* fn, const kin_bf16_t* q, const kin_bf16_t* kv_cache,
+static int launch_token_policy(const char* fn, bool f16, const kin_bf16_t* q, const kin_bf16_t* kv_cache,
                                const int32_t* page_indices, const int32_t* page_indptr, const int32_t* last_page_len,
                                int topk, int block, int stride, int sink_tokens, int local_tokens,
                                int first_page_offset, int32_t* sel_tokens, int32_t* sel_count, kin_bf16_t* out,
@@ -299,7 +299,9 @@ static int launch_token_policy(const char* fn, const kin_bf16_t* q, const kin_bf
   if (lds > 150 * 1024 && !ldsk)
     return fail(KIN_ERR_UNSUPPORTED, "%s: max_pages_per_seq=%d is too long for the strided policy's token bitmap", fn,
                 max_pages_per_seq);
-#define KIN_TOKEN_KERNEL(NG_, NW_, S_, L_) reinterpret_cast<const void*>(&token_topk_kernel<NG_, NW_, S_, L_>)
+#define KIN_TOKEN_KERNEL(NG_, NW_, S_, L_)                                                   \
+  (f16 ? reinterpret_cast<const void*>(&token_topk_kernel<NG_, NW_, S_, L_, true>)           \
+       : reinterpret_cast<const void*>(&token_topk_kernel<NG_, NW_, S_, L_, false>))
 #define KIN_TOKEN_PICK(NG_, S_)                                                             \
   (ldsk ? (nw == 12 ? KIN_TOKEN_KERNEL(NG_, 12, S_, true) : KIN_TOKEN_KERNEL(NG_, 4, S_, true)) \
         : (nw == 8 ? KIN_TOKEN_KERNEL(NG_, 8, S_, false) : KIN_TOKEN_KERNEL(NG_, 4, S_, false)))
@@ -349,7 +351,20 @@ int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const
                           int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
                           int64_t num_pages, int max_pages_per_seq, int sel_stride, float sm_scale,
                           kin_stream_t stream) {
-  return kin::launch_token_policy("kin_token_topk_decode", q, kv_cache, page_indices, page_indptr, last_page_len,
+  return kin::launch_token_policy("kin_token_topk_decode", false, q, kv_cache, page_indices, page_indptr, last_page_len,
+                                  topk_tokens, 0, 0, sink_tokens, local_tokens, first_page_offset, sel_tokens,
+                                  sel_count, out, lse, workspace, workspace_bytes, batch, num_q_heads, num_kv_heads,
+                                  head_dim, page_size, num_pages, max_pages_per_seq, sel_stride, sm_scale, stream);
+}
+
+int kin_token_topk_decode_f16(const kin_f16_t* q, const kin_f16_t* kv_cache, const int32_t* page_indices,
+                              const int32_t* page_indptr, const int32_t* last_page_len, int topk_tokens,
+                              int sink_tokens, int local_tokens, int first_page_offset, int32_t* sel_tokens,
+                              int32_t* sel_count, kin_f16_t* out, float* lse, void* workspace, size_t workspace_bytes,
+                              int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
+                              int64_t num_pages, int max_pages_per_seq, int sel_stride, float sm_scale,
+                              kin_stream_t stream) {
+  return kin::launch_token_policy("kin_token_topk_decode_f16", true, q, kv_cache, page_indices, page_indptr, last_page_len,
                                   topk_tokens, 0, 0, sink_tokens, local_tokens, first_page_offset, sel_tokens,
                                   sel_count, out, lse, workspace, workspace_bytes, batch, num_q_heads, num_kv_heads,
                                   head_dim, page_size, num_pages, max_pages_per_seq, sel_stride, sm_scale, stream);
@@ -364,11 +379,27 @@ int kin_strided_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, con
                             kin_stream_t stream) {
   if (block_size < 1)
     return kin::fail(KIN_ERR_BAD_SHAPE, "kin_strided_topk_decode: block_size=%d must be in [1, 64]", block_size);
-  return kin::launch_token_policy("kin_strided_topk_decode", q, kv_cache, page_indices, page_indptr, last_page_len,
+  return kin::launch_token_policy("kin_strided_topk_decode", false, q, kv_cache, page_indices, page_indptr, last_page_len,
                                   topk_blocks, block_size, stride, sink_tokens, local_tokens, first_page_offset,
                                   sel_tokens, sel_count, out, lse, workspace, workspace_bytes, batch, num_q_heads,
                                   num_kv_heads, head_dim, page_size, num_pages, max_pages_per_seq, sel_stride,
                                   sm_scale, stream);
+}
+
+int kin_strided_topk_decode_f16(const kin_f16_t* q, const kin_f16_t* kv_cache, const int32_t* page_indices,
+                                const int32_t* page_indptr, const int32_t* last_page_len, int topk_blocks,
+                                int block_size, int stride, int sink_tokens, int local_tokens, int first_page_offset,
+                                int32_t* sel_tokens, int32_t* sel_count, kin_f16_t* out, float* lse, void* workspace,
+                                size_t workspace_bytes, int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                                int page_size, int64_t num_pages, int max_pages_per_seq, int sel_stride,
+                                float sm_scale, kin_stream_t stream) {
+  if (block_size < 1)
+    return kin::fail(KIN_ERR_BAD_SHAPE, "kin_strided_topk_decode_f16: block_size=%d must be in [1, 64]", block_size);
+  return kin::launch_token_policy("kin_strided_topk_decode_f16", true, q, kv_cache, page_indices, page_indptr,
+                                  last_page_len, topk_blocks, block_size, stride, sink_tokens, local_tokens,
+                                  first_page_offset, sel_tokens, sel_count, out, lse, workspace, workspace_bytes, batch,
+                                  num_q_heads, num_kv_heads, head_dim, page_size, num_pages, max_pages_per_seq,
+                                  sel_stride, sm_scale, stream);
 }
 
 }  // extern "C"

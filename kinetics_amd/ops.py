@@ -454,8 +454,6 @@ def token_topk_workspace_bytes(batch: int, num_kv_heads: int, max_pages_per_seq:
 
 def _token_policy(q, kv_cache, page_indices, page_indptr, last_page_len, out, lse, sel_tokens, sel_count, workspace,
                   need_bytes):
-    if kv_cache.dtype is not torch.bfloat16:
-        raise ValueError("the token-granular policies are built for bfloat16 caches only")
     dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, None)
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     sel_stride = 0
@@ -489,7 +487,7 @@ def token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, top
     lib = _lib.load()
     with _on(dev):
         _lib.check(
-            lib.kin_token_topk_decode(
+            _entry(lib, "kin_token_topk_decode", kv_cache.dtype)(
                 _ptr(q), _ptr(kv_cache), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), int(topk_tokens),
                 int(sink_tokens), int(local_tokens), int(first_page_offset), _ptr(sel_tokens), _ptr(sel_count), _ptr(out),
                 _ptr(lse), _ptr(workspace), workspace.numel(), batch, hq, hkv, d, ps, num_pages, int(max_pages_per_seq),
@@ -519,7 +517,7 @@ def strided_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, t
     lib = _lib.load()
     with _on(dev):
         _lib.check(
-            lib.kin_strided_topk_decode(
+            _entry(lib, "kin_strided_topk_decode", kv_cache.dtype)(
                 _ptr(q), _ptr(kv_cache), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), int(topk_blocks),
                 int(block_size), int(stride), int(sink_tokens), int(local_tokens), int(first_page_offset),
                 _ptr(sel_tokens), _ptr(sel_count), _ptr(out), _ptr(lse), _ptr(workspace), workspace.numel(), batch, hq,

@@ -504,7 +504,7 @@ def token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, top
     ps = kv_cache.shape[2]
     out = np.zeros((B, Hq, D))
     keeps, means = [], []
-    qf = bf16_to_f32(q).astype(np.float64)
+    qf = elem_to_f32(q).astype(np.float64)
     for b in range(B):
         pages = seq_pages(page_indices, page_indptr, b)
         kv_len = (len(pages) - 1) * ps + int(last_page_len[b]) if len(pages) else 0
@@ -512,8 +512,8 @@ def token_topk_decode(q, kv_cache, page_indices, page_indptr, last_page_len, top
             keeps.append(None)
             means.append(None)
             continue
-        K = bf16_to_f32(kv_cache[pages, 0]).reshape(len(pages) * ps, -1, D)[first_page_offset:kv_len]
-        V = bf16_to_f32(kv_cache[pages, 1]).reshape(len(pages) * ps, -1, D)[first_page_offset:kv_len]
+        K = elem_to_f32(kv_cache[pages, 0]).reshape(len(pages) * ps, -1, D)[first_page_offset:kv_len]
+        V = elem_to_f32(kv_cache[pages, 1]).reshape(len(pages) * ps, -1, D)[first_page_offset:kv_len]
         o, keep, mean = litesys_decode(qf[b], K, V, topk, local, sink=sink, sm_scale=sm_scale, policy=policy,
                                        block_size=block_size, stride=stride, return_mean_logits=True)
         out[b] = o

@@ -16,8 +16,11 @@ DEV = "cuda"
 D, PS = P.HEAD_DIM, P.PAGE_SIZE
 
 
+_DT = [torch.bfloat16]   # element type of the test that is running (test_prefill_then_decode_like_litesys switches it)
+
+
 def bf(x):
-    return x.to(torch.bfloat16)
+    return x.to(_DT[0])
 
 
 def cfg_small():
@@ -29,7 +32,7 @@ def make_manager(**sparse):
 
     block_policy = "attn_block_topk" in sparse and "attn_stride" not in sparse
     page = sparse.get("attn_block_size", PS) if block_policy else PS
-    return PagedBatchKVManager(cfg_small(), max_batch_size=6, max_seq_len=page * 24, device=DEV, dtype=torch.bfloat16, **sparse)
+    return PagedBatchKVManager(cfg_small(), max_batch_size=6, max_seq_len=page * 24, device=DEV, dtype=_DT[0], **sparse)
 
 
 def test_rejects_what_it_does_not_implement():
@@ -58,7 +61,17 @@ def test_rejects_what_it_does_not_implement():
                                           (dict(attn_topk=40, attn_local=10), None),
                                           (dict(attn_block_topk=2, attn_local=9, attn_stride=8), None),
                                           (dict(attn_block_topk=3, attn_local=5, attn_stride=4, attn_block_size=8), None)])
-def test_prefill_then_decode_like_litesys(sparse, fused):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_prefill_then_decode_like_litesys(sparse, fused, dtype):
+    _DT[0] = dtype
+    try:
+        with O.element_format("f16" if dtype is torch.float16 else "bf16"):   # how the oracle reads the cache bits
+            _prefill_then_decode_like_litesys(sparse, fused)
+    finally:
+        _DT[0] = torch.bfloat16
+
+
+def _prefill_then_decode_like_litesys(sparse, fused):
     torch.manual_seed(5)
     m = make_manager(**sparse)
     PS = m.page                   # tokens per page: LiteSys' block size for the block policy, else 16
@@ -362,8 +375,6 @@ def test_float16_manager(sparse):
             feed(layer, slot, k[0], v[0])
             out = m.compute_attention(q, k, v, layer, torch.tensor([slot]))
             assert out.dtype is torch.float16 and out.shape == (1, n, Hq * D)
-    with pytest.raises(NotImplementedError):
-        PagedBatchKVManager(cfg_small(), 2, 64, DEV, torch.float16, attn_topk=8, attn_local=4)
     for _ in range(block + 2):                     # crosses a page boundary: a float16 mean key is written
         for layer in range(L):
             slots = [0, 2]

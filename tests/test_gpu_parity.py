@@ -641,13 +641,13 @@ def test_float16_caches(ops, hkv, group, page_size):
                                    g.indices, g.indptr, g.last)
         torch.cuda.synchronize()
         assert np.array_equal(P.from_torch(g.kv), want_kv) and np.array_equal(P.from_torch(g.kbar), want_kbar)
-    # mixed dtypes and float16 on the bfloat16-only paths are refused
+    # mixed dtypes are refused
     pb = P.make_problem(990, [40, 9], num_kv_heads=hkv, group=group)
     g = Gpu(pb)
     with pytest.raises(TypeError):
         ops.sparse_paged_decode(g.q.half(), g.kv, g.sel, g.cnt, g.last)
-    with pytest.raises(ValueError):
-        ops.token_topk_decode(g.q.half(), g.kv.half(), g.indices, g.indptr, g.last, 4, pb.max_pages)
+    with pytest.raises(TypeError):
+        ops.token_topk_decode(g.q.half(), g.kv, g.indices, g.indptr, g.last, 4, pb.max_pages)
 
 
 # --------------------------------------------------------------------------- full benchmark sizes
@@ -1084,7 +1084,7 @@ def _check_token_topk(ops, pb, topk, sink, local, offset, what, max_pages=None):
                                              local=local, first_page_offset=offset)
     sel, cnt, got = sel.cpu().numpy(), cnt.cpu().numpy(), out.float().cpu().numpy()
     G = pb.Hq // pb.Hkv
-    qf = O.bf16_to_f32(pb.q).astype(np.float64)
+    qf = O.elem_to_f32(pb.q).astype(np.float64)
     for b in range(pb.B):
         if keeps[b] is None:
             assert (cnt[b] == 0).all() and (sel[b] == -1).all() and (got[b] == 0).all(), what
@@ -1095,8 +1095,8 @@ def _check_token_topk(ops, pb, topk, sink, local, offset, what, max_pages=None):
         n_dyn = S - n_sink - n_local
         k_eff = min(topk, n_dyn)
         pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
-        K = O.bf16_to_f32(kv[pages, 0]).reshape(-1, pb.Hkv, D)[offset : offset + S]
-        V = O.bf16_to_f32(kv[pages, 1]).reshape(-1, pb.Hkv, D)[offset : offset + S]
+        K = O.elem_to_f32(kv[pages, 0]).reshape(-1, pb.Hkv, D)[offset : offset + S]
+        V = O.elem_to_f32(kv[pages, 1]).reshape(-1, pb.Hkv, D)[offset : offset + S]
         got_keep = np.zeros((pb.Hkv, S), dtype=bool)
         for h in range(pb.Hkv):
             n = cnt[b, h]
@@ -1198,7 +1198,7 @@ def _check_strided(ops, pb, topk, sink, local, block, stride, offset, what, need
                                              local=local, first_page_offset=offset, policy="strided", block_size=block,
                                              stride=stride)
     sel, cnt, got = sel.cpu().numpy(), cnt.cpu().numpy(), out.float().cpu().numpy()
-    qf = O.bf16_to_f32(pb.q).astype(np.float64)
+    qf = O.elem_to_f32(pb.q).astype(np.float64)
     sparse_rows = 0
     for b in range(pb.B):
         if keeps[b] is None:
@@ -1206,8 +1206,8 @@ def _check_strided(ops, pb, topk, sink, local, block, stride, offset, what, need
             continue
         S = keeps[b].shape[1]
         pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
-        K = O.bf16_to_f32(kv[pages, 0]).reshape(-1, pb.Hkv, D)[offset : offset + S]
-        V = O.bf16_to_f32(kv[pages, 1]).reshape(-1, pb.Hkv, D)[offset : offset + S]
+        K = O.elem_to_f32(kv[pages, 0]).reshape(-1, pb.Hkv, D)[offset : offset + S]
+        V = O.elem_to_f32(kv[pages, 1]).reshape(-1, pb.Hkv, D)[offset : offset + S]
         got_keep = np.zeros((pb.Hkv, S), dtype=bool)
         for h in range(pb.Hkv):
             n = cnt[b, h]
@@ -1267,6 +1267,26 @@ def test_strided_topk_decode(ops, case):
         topk, sink, local, block, stride = 9, 2, 5, 8, 3
     _check_strided(ops, pb, topk, sink, local, block, stride, offset, f"strided {case}",
                    max_pages=max_pages if case == "many_12_waves" else None)
+
+
+@pytest.mark.parametrize("policy", ["token", "strided"])
+def test_token_policies_in_float16(ops, policy):
+    """The kin_*_f16 twins of the token-granular policies: few long lists (shared
+    scoring through HBM keys), and many lists (keys in LDS), against the oracle
+    reading the same bits as float16."""
+    with O.element_format("f16"):
+        rng = np.random.default_rng(8400)
+        problems = [
+            (P.make_problem(8401, [PS * 40 + 3, PS * 9, 1, 0, PS * 3 + 1, PS * 130 + 16, 17, 5], num_kv_heads=2, group=4), None),
+            (P.make_problem(8402, [PS * 1300 + 7, PS * 300 + 1, 17], num_kv_heads=1, group=8), None),
+            (P.make_problem(8403, [int(x) for x in rng.integers(1, PS * 30, size=560)], num_kv_heads=1, group=3), 1200),
+        ]
+        for i, (pb, mp) in enumerate(problems):
+            assert Gpu(pb).kv.dtype is torch.float16
+            if policy == "token":
+                _check_token_topk(ops, pb, 48, 4, 16, 0, f"float16 token top-k {i}", max_pages=mp)
+            else:
+                _check_strided(ops, pb, 4, 4, 16, 16, 8, 0, f"float16 strided {i}", need_sparse=False, max_pages=mp)
 
 
 @pytest.mark.parametrize("policy", ["token", "strided"])
