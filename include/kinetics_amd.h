@@ -377,8 +377,8 @@ int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_bf16_t* k, c
  * (-1 for a sequence with more than max_pages_per_seq pages, which is skipped:
  * out = 0).  workspace: kin_token_topk_workspace_bytes(...) bytes of scratch
  * (4 bytes per cache slot and KV head, plus an arrival counter per list; any
- * contents, 16-byte aligned; with more than 512 lists and max_pages_per_seq up
- * to ~2100 the per-token keys stay in on-chip memory and the scratch is not
+ * contents, 16-byte aligned; with 128 lists or more and max_pages_per_seq up
+ * to ~2300 the per-token keys stay in on-chip memory and the scratch is not
  * touched, but its size is still checked).  Reads every key of the context
  * once: HBM traffic is about half of dense decode's.  When the lists are fewer than
  * the GPU's compute units, several workgroups share the scoring of a list;

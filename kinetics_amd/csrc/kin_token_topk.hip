@@ -250,7 +250,6 @@ static int launch_token_policy(const char* fn, bool f16, const kin_bf16_t* q, co
   p.count = static_cast<int32_t*>(workspace);
   p.keys = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + count_bytes);
   p.scores = strided ? reinterpret_cast<float*>(static_cast<char*>(workspace) + count_bytes + key_bytes) : nullptr;
-  p.chunks = token_score_chunks(items, max_pages_per_seq);
   p.block = block;
   p.stride = stride;
   p.list_cap = list_cap > 0 ? list_cap : 1;
@@ -268,30 +267,29 @@ static int launch_token_policy(const char* fn, bool f16, const kin_bf16_t* q, co
   const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
   p.scale_log2 = scale * 1.4426950408889634f;
 
-  const int64_t grid = xcd_grid_size(batch, num_kv_heads) * p.chunks;
-  if (grid > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
-  // Waves per workgroup: 8 when the lists are too few to fill the GPU with 4-wave
-  // workgroups -- whatever the number of chunks: selection and attention are done by
-  // one workgroup per list (the per-token addressing needs ~140 registers, so 16 waves
-  // do not fit).
-  int nw = items <= 2 * kNumCus ? 8 : 4;
+  // How a list's token keys travel from scoring to selection.  Kept in LDS when they fit
+  // and the lists alone occupy at least half the CUs: key stores to HBM between the loads
+  // of a saturated stream cost far more than their bytes.  One 12-wave workgroup per CU
+  // while the lists are no more than the CUs or the keys need the room, else three 4-wave
+  // workgroups per CU (the same 12 waves).  Otherwise the keys go through the workspace:
+  // few lists split their scoring into chunks, and workgroups have 8 waves until 4-wave
+  // ones fill the GPU (the per-token addressing needs ~140 registers, so 16 do not fit).
   const size_t bitmap_bytes = strided ? ((size_t)max_pages_per_seq * kPageSize / 32 + 1) * 4 : 0;
   const size_t tail_bytes = (size_t)p.list_cap * 4 + bitmap_bytes;
-  // With the GPU full of whole lists, the keys stay in LDS when they fit: three 4-wave
-  // workgroups per CU for short sequences, else one of 12 waves (the same 12 waves per CU).
-  // Key stores to HBM between the loads of a saturated stream cost far more than their bytes.
   const size_t key_lds = ((size_t)max_pages_per_seq * kPageSize + 4) * sizeof(uint32_t);
-  bool ldsk = false;
-  if (p.chunks == 1 && nw == 4) {
-    const size_t small = (key_lds > (size_t)attend_lds_bytes(4) ? key_lds : (size_t)attend_lds_bytes(4)) + tail_bytes;
-    const size_t big = (key_lds > (size_t)attend_lds_bytes(12) ? key_lds : (size_t)attend_lds_bytes(12)) + tail_bytes;
-    if (small <= 50 * 1024) {
-      ldsk = true;
-    } else if (big <= 156 * 1024) {
-      ldsk = true;
-      nw = 12;
-    }
+  const size_t small = (key_lds > (size_t)attend_lds_bytes(4) ? key_lds : (size_t)attend_lds_bytes(4)) + tail_bytes;
+  const size_t big = (key_lds > (size_t)attend_lds_bytes(12) ? key_lds : (size_t)attend_lds_bytes(12)) + tail_bytes;
+  const bool ldsk = items >= kNumCus / 2 && big <= 156 * 1024;
+  int nw;
+  if (ldsk) {
+    p.chunks = 1;
+    nw = items > kNumCus && small <= 50 * 1024 ? 4 : 12;
+  } else {
+    p.chunks = token_score_chunks(items, max_pages_per_seq);
+    nw = items <= 2 * kNumCus ? 8 : 4;
   }
+  const int64_t grid = xcd_grid_size(batch, num_kv_heads) * p.chunks;
+  if (grid > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   size_t region0 = (size_t)attend_lds_bytes(nw);
   if (ldsk && key_lds > region0) region0 = (key_lds + 15) & ~(size_t)15;
   p.region0_bytes = (int)region0;

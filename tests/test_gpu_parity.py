@@ -1136,11 +1136,11 @@ def test_token_topk_decode(ops, case):
     elif case == "g7":       # a group that fills the second head tile only partly
         pb = P.make_problem(1309, [PS * 50 + 9, PS * 3, 40], num_kv_heads=2, group=7)
         args = (200, 4, 12, 0)
-    elif case == "many":     # > 512 lists: 4 waves per list, keys in LDS
+    elif case == "many":     # > 256 lists: 4 waves per list, keys in LDS
         rng = np.random.default_rng(1303)
         pb = P.make_problem(1303, [int(x) for x in rng.integers(1, PS * 30, size=600)], num_kv_heads=1, group=3)
         args = (48, 4, 8, 0)
-    elif case == "many_12_waves":  # > 512 lists and room asked for long sequences: keys in LDS, one 12-wave workgroup per list
+    elif case == "many_12_waves":  # many lists and room asked for long sequences: keys in LDS, one 12-wave workgroup per list
         rng = np.random.default_rng(1310)
         pb = P.make_problem(1310, [PS * 200 + 5, 0, 3] + [int(x) for x in rng.integers(1, PS * 40, size=530)], num_kv_heads=1,
                             group=4)
@@ -1161,7 +1161,7 @@ def test_token_topk_decode(ops, case):
         # ones), 8 waves; the longest has more keys than the selecting workgroup holds in registers at once
         pb = P.make_problem(1307, [PS * 2100 + 7, PS * 1030 + 16, PS * 300 + 1, 17], num_kv_heads=1, group=4)
         args = (700, 4, 16, 0)
-    elif case == "split_many":  # > 512 lists (4 waves, no splitting), one of them with more keys than the
+    elif case == "split_many":  # many lists (no splitting, keys in LDS), one of them with more keys than the
         # selecting workgroup holds in registers at once
         rng = np.random.default_rng(1308)
         pb = P.make_problem(1308, [PS * 1100 + 3] + [int(x) for x in rng.integers(1, PS * 20, size=519)], num_kv_heads=1,
@@ -1243,11 +1243,11 @@ def test_strided_topk_decode(ops, case):
     elif case == "g5":
         pb = P.make_problem(1508, [PS * 50 + 9, PS * 3, 40], num_kv_heads=2, group=5)
         topk, sink, local = 6, 4, 12
-    elif case == "many":     # > 512 lists: 4 waves per list, scores in LDS
+    elif case == "many":     # > 256 lists: 4 waves per list, scores in LDS
         rng = np.random.default_rng(1503)
         pb = P.make_problem(1503, [int(x) for x in rng.integers(1, PS * 30, size=600)], num_kv_heads=1, group=3)
         topk, sink, local = 3, 4, 8
-    elif case == "many_12_waves":  # > 512 lists and room asked for long sequences: scores in LDS, 12 waves per list
+    elif case == "many_12_waves":  # many lists and room asked for long sequences: scores in LDS, 12 waves per list
         rng = np.random.default_rng(1509)
         pb = P.make_problem(1509, [PS * 180 + 5, 0, 3] + [int(x) for x in rng.integers(1, PS * 40, size=530)], num_kv_heads=1,
                             group=4)
@@ -1291,16 +1291,17 @@ def test_token_policies_in_float16(ops, policy):
 
 @pytest.mark.parametrize("policy", ["token", "strided"])
 def test_token_policies_with_the_gpu_full_of_lists(ops, policy):
-    """More than 512 lists: one workgroup per list, and the per-token keys (scores,
+    """128 lists or more: one workgroup per list, and the per-token keys (scores,
     for the strided policy) stay in LDS when ``max_pages_per_seq`` lets them fit --
-    in 4-wave workgroups for short sequences, one 12-wave workgroup per list for long
-    ones -- or go through the HBM workspace when it does not.  Seeded shapes with
-    groups up to 16, pinned tokens, offsets and empty sequences, each against the oracle."""
+    one 12-wave workgroup per list up to 256 lists or for long sequences, 4-wave
+    workgroups for more lists of short sequences -- or go through the HBM workspace
+    when it does not (8 waves up to 512 lists, then 4).  Seeded shapes with groups up
+    to 16, pinned tokens, offsets and empty sequences, each against the oracle."""
     rng = np.random.default_rng(8100 if policy == "token" else 8200)
-    for trial in range(5):
+    for trial in range(9):
         hkv = int(rng.choice([1, 1, 2, 4]))
         group = int(rng.choice([1, 2, 4, 5, 8, 12, 16]))
-        lists = int(rng.integers(513, 620))
+        lists = int(rng.integers(513, 620)) if trial < 5 else [128, 256, 260, 500][trial - 5] + 4 * int(rng.integers(0, 3))
         B = (lists + hkv - 1) // hkv
         longest = int(rng.choice([PS * 30, PS * 60, PS * 150]))
         lengths = [int(x) for x in rng.integers(0, longest, size=B)]
@@ -1309,7 +1310,7 @@ def test_token_policies_with_the_gpu_full_of_lists(ops, policy):
         offset = int(rng.integers(0, PS)) if rng.integers(0, 2) else 0
         lengths = [L + offset if L else 0 for L in lengths]
         # 0: exactly the longest sequence; 700 / 2049: keys in LDS (4 / 12 waves); 2600: too long for LDS
-        max_pages = [0, 700, 2049, 2600, 1500][trial]
+        max_pages = [0, 700, 2049, 2600, 1500, 0, 2600, 700, 2049][trial]
         pb = P.make_problem(8300 + 10 * trial + (1 if policy == "token" else 2), lengths, num_kv_heads=hkv, group=group)
         mp = max(max_pages, pb.max_pages) if max_pages else None
         if policy == "token":
