@@ -288,7 +288,7 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  * kin_block_score_topk, first_page_offset as in kin_sparse_paged_decode (a
  * non-zero offset requires sink_pages >= 1: a padded page has no valid mean
  * key); lse is optional.  Needs no workspace.  One workgroup walks a whole
- * list (no split-K); with few lists it runs 8 or 16 waves instead of 4, which
+ * list (no split-K); with 256 lists or fewer it runs 8 waves instead of 4, which
  * changes the fp32 summation order of the output (not the page lists or cache
  * bytes).  Faster than the three calls except for few (< 256) and very long
  * (topk > 512) lists.  workspace: optional, see kin_step_workspace_bytes.

@@ -139,10 +139,10 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   } else {
     // Mean-key loads in flight per lane.  4 saturate HBM while several rounds of workgroups overlap
     // (4096 lists; more only lengthens the last pass of short lists).  With fewer lists the workgroups
-    // score in step and each has to keep 64 KiB in flight: 16 / 8 / 4 loads at 4 / 8 / 16 waves
+    // score in step and each has to keep 64 KiB in flight: 16 / 8 loads at 4 / 8 waves
     // (1024 lists of 2048 pages: 5 % faster than with 4).
     if (p.deep_score) {
-      constexpr int kDeep = NW <= 4 ? 16 : (NW <= 8 ? 8 : 4);
+      constexpr int kDeep = NW <= 4 ? 16 : 8;
       n = score_select<kDeep, NT, F16>(s, sel_lds);
     } else {
       n = score_select<4, NT, F16>(s, sel_lds);
@@ -253,16 +253,14 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
   p.first_page_offset = first_page_offset;
   p.page_size = page_size;
   p.sort_cap = select_sort_cap(topk, kbar_pages);
-  // Waves per workgroup: aim for 16 waves per CU (8 with the wide kernel for groups
-  // above 4, which holds a few registers too many for 16) when the lists are few.
+  // Waves per workgroup.  The kernels hold 140-145 registers, so a CU runs 12 waves: three
+  // 4-wave workgroups, or one of 8 while the lists are no more than the CUs (measured: 8 waves
+  // beat 4, 6, 12 and a 16-wave build that spills, by 2-20 %; from 257 lists on, 8-wave
+  // workgroups would take two rounds and 4 waves win by 3-25 %).
   const int64_t items = (int64_t)batch * num_kv_heads;
   if (xcd_grid_size(batch, num_kv_heads) > 0x7fffffffLL)
     return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
-  int nw = 4;
-  if (p.group <= 4)
-    nw = items <= kNumCus ? 16 : (items <= 2 * kNumCus ? 8 : 4);
-  else
-    nw = items <= kNumCus ? 8 : 4;
+  const int nw = items <= kNumCus ? 8 : 4;
   // Few long sequences: spread the scoring of each list over several workgroups.
   p.chunks = score_chunks(batch, num_kv_heads, kbar_pages);
   if (p.chunks > 1 && workspace && aligned16(workspace) &&
@@ -287,23 +285,14 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
   const size_t lds = region0 + (size_t)list_cap * 4;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const void* kernel;
-  if (f16) {
-    if (p.group <= 4)
-      kernel = nw == 16  ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 16, true>)
-               : nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 8, true>)
-                         : reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 4, true>);
-    else
-      kernel = nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<4, 8, true>)
-                       : reinterpret_cast<const void*>(&blocktopk_step_kernel<4, 4, true>);
-  } else {
-    if (p.group <= 4)
-      kernel = nw == 16  ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 16, false>)
-               : nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 8, false>)
-                         : reinterpret_cast<const void*>(&blocktopk_step_kernel<1, 4, false>);
-    else
-      kernel = nw == 8 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<4, 8, false>)
-                       : reinterpret_cast<const void*>(&blocktopk_step_kernel<4, 4, false>);
-  }
+#define KIN_STEP_KERNEL(NG_, NW_)                                                        \
+  (f16 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<NG_, NW_, true>)           \
+       : reinterpret_cast<const void*>(&blocktopk_step_kernel<NG_, NW_, false>))
+  if (p.group <= 4)
+    kernel = nw == 8 ? KIN_STEP_KERNEL(1, 8) : KIN_STEP_KERNEL(1, 4);
+  else
+    kernel = nw == 8 ? KIN_STEP_KERNEL(4, 8) : KIN_STEP_KERNEL(4, 4);
+#undef KIN_STEP_KERNEL
   if (lds > 48 * 1024) {
     // Above the default dynamic-LDS allowance the runtime wants an explicit opt-in.
     st = check_hip(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),

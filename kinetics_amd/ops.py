@@ -374,7 +374,7 @@ def prefer_fused_step(batch: int, num_kv_heads: int, max_pages_per_seq: int, top
     """Which of the two equivalent decode-step paths to use.  The single-launch
     kernel saves two dependent dispatches, the selector's drain and the attention
     ramp-up (3-30 % per step on MI355X, the more the smaller the step), and
-    widens its workgroups to 8 or 16 waves when there are few lists; but one
+    widens its workgroups to 8 waves when there are few lists; but one
     workgroup walks a whole list: it has no split-K.  Measured on MI355X it wins
     from 256 (sequence, KV head) lists up at every top-k, and for top-k up to 512
     at every batch size; only few lists that are also very long (64 sequences

@@ -1514,7 +1514,7 @@ def test_fused_step_equals_three_calls(ops, case):
     """kin_blocktopk_decode_step must give what append + score/select + attend
     give and match the oracle: cache bytes, mean keys and page lists bit for bit;
     the output bit for bit when the fused kernel runs 4 waves per list like the
-    stand-alone one (more than 512 lists), else to fp32 summation order (wider
+    stand-alone one (more than 256 lists), else to fp32 summation order (wider
     workgroups deal the pages to more waves)."""
     if case == "mixed":
         pb = P.make_problem(900, [PS * 40 + 3, PS * 9, 1, 0, PS * 3 + 1, PS * 130 + 16, 17], num_kv_heads=1, group=4, topk=8)
@@ -1535,7 +1535,7 @@ def test_fused_step_equals_three_calls(ops, case):
     elif case == "many_g8":    # > 256 lists with a group above 4: 4 waves per list
         rng = np.random.default_rng(907)
         pb = P.make_problem(907, [int(x) for x in rng.integers(1, PS * 30, size=300)], num_kv_heads=1, group=8, topk=6)
-    else:                      # 257..512 lists: 8 waves per list
+    else:                      # 257..512 lists: 4 waves per list, not every CU with three workgroups
         rng = np.random.default_rng(908)
         pb = P.make_problem(908, [int(x) for x in rng.integers(1, PS * 40, size=150)], num_kv_heads=2, group=3, topk=9)
     a, b = Gpu(pb), Gpu(pb)
@@ -1550,7 +1550,7 @@ def test_fused_step_equals_three_calls(ops, case):
     torch.cuda.synchronize()
     assert torch.equal(a.kv, b.kv) and torch.equal(a.kbar, b.kbar)
     assert torch.equal(a.cnt, b.cnt) and torch.equal(a.sel, b.sel)
-    if case in ("many", "many_g8"):
+    if case in ("many", "many_g8", "mid"):
         assert torch.equal(out_a, out_b)
         assert torch.equal(lse_a, lse_b)
     else:
