@@ -290,8 +290,9 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  * key); lse is optional.  Needs no workspace.  One workgroup walks a whole
  * list (no split-K); with 256 lists or fewer it runs 8 waves instead of 4, which
  * changes the fp32 summation order of the output (not the page lists or cache
- * bytes).  Faster than the three calls except for few (< 256) and very long
- * (topk > 512) lists.  workspace: optional, see kin_step_workspace_bytes.
+ * bytes).  Faster than the three calls from about 160 lists on and for topk up
+ * to 128 at any batch; fewer lists with longer page lists are served better by
+ * the three calls, whose decode splits each list across workgroups.  workspace: optional, see kin_step_workspace_bytes.
  */
 int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
                               kin_bf16_t* kv_cache, kin_bf16_t* kbar,

@@ -373,15 +373,23 @@ def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, ma
 def prefer_fused_step(batch: int, num_kv_heads: int, max_pages_per_seq: int, topk: int) -> bool:
     """Which of the two equivalent decode-step paths to use.  The single-launch
     kernel saves two dependent dispatches, the selector's drain and the attention
-    ramp-up (3-30 % per step on MI355X, the more the smaller the step), and
-    widens its workgroups to 8 waves when there are few lists; but one
-    workgroup walks a whole list: it has no split-K.  Measured on MI355X it wins
-    from 256 (sequence, KV head) lists up at every top-k, and for top-k up to 512
-    at every batch size; only few lists that are also very long (64 sequences
-    with top-k 2048: 377 vs 268 us) are served better by the three-launch path,
-    which splits each list across workgroups."""
+    ramp-up, but one workgroup walks a whole list: it has no split-K.  Measured on
+    MI355X against the three launches queued back to back (fused / three): 8 lists
+    k=128 0.87, k=256 1.31, k=512 1.87; 64 lists k=128 1.02, k=512 1.36; 100 lists
+    k=512 1.03, k=1024 1.18; 128 lists k=768..2048 1.01..1.04; 200..256 lists
+    0.95..0.98; 260..300 lists k<=768 0.96..0.98, k=1024 1.17..1.20 (some CUs hold
+    two long lists, the others one); 350 lists and more 0.96..1.00 (600 lists with
+    k>=1024: 1.05).  Hence: fused for k <= 128 at any batch, up to k = 512 from 96
+    lists, everything from 160 lists -- except 257..349 lists with k > 768."""
     del max_pages_per_seq
-    return batch * num_kv_heads >= 256 or topk <= 512
+    lists = batch * num_kv_heads
+    if lists < 96:
+        return topk <= 128
+    if lists < 160:
+        return topk <= 512
+    if 256 < lists < 350:
+        return topk <= 768
+    return True
 
 
 def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, out=None, lse=None,

@@ -242,6 +242,32 @@ def test_auto_splits_policy(lib):
     assert lib.kin_decode_workspace_bytes(4096, 4, 1, 128, 129, 0) == 0
 
 
+def test_auto_splits_policy_follows_the_lists(lib):
+    """Few lists: about one workgroup per CU in total; just above 256 lists only
+    long lists are split; from 768 lists on none; never fewer than 4 pages a split."""
+    assert lib.kin_decode_auto_splits(8, 1, 2049) == 28
+    assert lib.kin_decode_auto_splits(64, 1, 2049) == 4
+    assert lib.kin_decode_auto_splits(4, 8, 257) == 7
+    assert lib.kin_decode_auto_splits(256, 1, 2049) == 1
+    assert lib.kin_decode_auto_splits(300, 1, 2049) == 4
+    assert lib.kin_decode_auto_splits(300, 1, 513) == 1
+    assert lib.kin_decode_auto_splits(768, 1, 2049) == 1
+    assert lib.kin_decode_auto_splits(1, 1, 1 << 20) == 64
+    assert lib.kin_decode_auto_splits(8, 1, 17) == 4
+
+
+def test_path_preference_rule():
+    """prefer_fused_step: the single launch for short page lists at any batch and for
+    everything from 160 lists on, except long lists just above one list per CU."""
+    from kinetics_amd import ops
+    assert ops.prefer_fused_step(8, 1, 257, 64) and ops.prefer_fused_step(1, 8, 2049, 128)
+    assert not ops.prefer_fused_step(8, 1, 2049, 256) and not ops.prefer_fused_step(64, 1, 2049, 512)
+    assert ops.prefer_fused_step(100, 1, 2049, 512) and not ops.prefer_fused_step(100, 1, 2049, 1024)
+    assert ops.prefer_fused_step(256, 1, 1025, 64) and ops.prefer_fused_step(200, 1, 4097, 2048)
+    assert ops.prefer_fused_step(300, 1, 2049, 768) and not ops.prefer_fused_step(300, 1, 2049, 1024)
+    assert ops.prefer_fused_step(512, 8, 2049, 64) and ops.prefer_fused_step(4096, 1, 2049, 128)
+
+
 def test_python_wrapper_maps_status_to_exceptions():
     with pytest.raises(ValueError, match="KIN_ERR_BAD_SHAPE"):
         _lib.check(_lib.load().kin_block_score_topk(A, A, A, A, A, -1, 0, 1, A, A, None, None, 2, 4, 1, 128, 16, 64, 5, None, 0, None))
