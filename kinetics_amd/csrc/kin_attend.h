@@ -190,12 +190,13 @@ struct AttendArgs {
 // p * batch + b, as the reference lays them out -- are all at the same page at the same time and
 // read one narrow window of the cache (1024 sequences: 81 % of peak against 85-87 % for any other
 // numbering).  Every list therefore starts at its own tile and wraps around; the sum over tiles does
-// not care about the order.  Only with more lists than fill the GPU twice over (with fewer, neighbours
-// reading neighbouring pages helps: 256 lists lose 4 % when rotated) and only parts of at least
+// not care about the order.  Only with at least two lists per CU (512 sequences: 74 % in list order,
+// 82 % rotated; with fewer, neighbours reading neighbouring pages helps: 256 lists lose 3 % when
+// rotated, 384 lists 1 %) and only parts of at least
 // kRotateMinTiles tiles.  The rule depends on the batch alone, so the fused step and the stand-alone
 // kernel visit a list's tiles in the same order.
 constexpr int kRotateMinTiles = 512;
-__host__ __device__ inline bool attend_rotates(int64_t lists) { return lists > 2 * kNumCus; }
+__host__ __device__ inline bool attend_rotates(int64_t lists) { return lists >= 2 * kNumCus; }
 __device__ __forceinline__ unsigned attend_rotation(int list, int split) {
   return ((unsigned)list * 2654435761u >> 8) + 977u * (unsigned)split;
 }

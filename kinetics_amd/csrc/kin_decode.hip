@@ -116,15 +116,16 @@ static int auto_splits(int batch, int num_kv_heads, int max_pages_per_list) {
   // up to 256 lists, a little under one workgroup per CU is best (more splits only add
   // partial results and merge work), never below 4 pages -- one per wave -- a split;
   // between 256 and 768 lists only long lists gain from splitting (300 lists of 2049
-  // pages: 0.94 ms whole, 0.77 ms in four parts -- whole lists cannot be balanced over
-  // the CUs), and from 768 lists on every CU holds its three workgroups anyway.
+  // pages: 0.94 ms whole, 0.77 ms in four to eight parts; 513 lists: 1.51 ms whole, 1.36
+  // in four -- whole lists cannot be balanced over the CUs), and from 768 lists on every
+  // CU holds its three workgroups anyway.
   const int64_t lists = (int64_t)batch * num_kv_heads;
   if (lists <= 0) return 1;
   int64_t want = 1;
   if (lists <= kNumCus)
     want = (kNumCus - kNumCus / 8 + lists / 2) / lists;
   else if (lists < 3 * kNumCus && max_pages_per_list >= 1024)
-    want = (4 * kNumCus + lists - 1) / lists;
+    want = (8 * kNumCus + lists - 1) / lists;
   int64_t cap = max_pages_per_list / 4;
   if (want > cap) want = cap;
   if (want > 64) want = 64;

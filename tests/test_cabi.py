@@ -249,7 +249,7 @@ def test_auto_splits_policy_follows_the_lists(lib):
     assert lib.kin_decode_auto_splits(64, 1, 2049) == 4
     assert lib.kin_decode_auto_splits(4, 8, 257) == 7
     assert lib.kin_decode_auto_splits(256, 1, 2049) == 1
-    assert lib.kin_decode_auto_splits(300, 1, 2049) == 4
+    assert lib.kin_decode_auto_splits(300, 1, 2049) == 7
     assert lib.kin_decode_auto_splits(300, 1, 513) == 1
     assert lib.kin_decode_auto_splits(768, 1, 2049) == 1
     assert lib.kin_decode_auto_splits(1, 1, 1 << 20) == 64
