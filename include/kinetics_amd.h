@@ -73,7 +73,9 @@ enum kin_status {
  * head-major ([batch, num_kv_heads, kbar_pages, 128]; 1.x had [batch, kbar_pages,
  * num_kv_heads, 128]), kin_block_score_topk takes the page size, pages of 32 and 64
  * tokens, float16 twins (kin_*_f16), groups of up to 16 query heads per KV head,
- * the page pool and kin_blocktopk_decode_step_static. */
+ * the page pool and kin_blocktopk_decode_step_static.  2.1.0: the decode step
+ * attends few lists in parts (kin_step_workspace_bytes grows to up to 2.1 MB for
+ * up to 112 lists; KIN_STATIC_SCRATCH_BYTES grows by 32 KiB less 256 B). */
 int kin_version(void);
 
 /* Human-readable text of the last non-OK status on the calling thread
@@ -287,12 +289,15 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  * kin_sel_list_capacity(...)); topk / sink_pages / local_tokens as in
  * kin_block_score_topk, first_page_offset as in kin_sparse_paged_decode (a
  * non-zero offset requires sink_pages >= 1: a padded page has no valid mean
- * key); lse is optional.  Needs no workspace.  One workgroup walks a whole
- * list (no split-K); with 256 lists or fewer it runs 8 waves instead of 4, which
- * changes the fp32 summation order of the output (not the page lists or cache
- * bytes).  Faster than the three calls from about 160 lists on and for topk up
- * to 128 at any batch; fewer lists with longer page lists are served better by
- * the three calls, whose decode splits each list across workgroups.  workspace: optional, see kin_step_workspace_bytes.
+ * key); lse is optional.  One workgroup walks a whole list, of 8 waves instead
+ * of 4 with 256 lists or fewer; with lists for under half the GPU's compute
+ * units and a workspace (optional, see kin_step_workspace_bytes), several
+ * workgroups share a list: each attends a part of the listed pages and the last
+ * to finish merges the partial results, or -- very long sequences -- each
+ * scores a part of the candidates.  Any of this changes only the fp32 summation
+ * order of the output, not the page lists or cache bytes.  At least as fast as
+ * the three calls except for few lists of more than 4096 pages with topk >= 512
+ * and for 257..349 lists with topk > 768 (up to 1.6x and 1.2x slower).
  */
 int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
                               kin_bf16_t* kv_cache, kin_bf16_t* kbar,
@@ -309,13 +314,15 @@ int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const ki
 
 /*
  * Workspace kin_blocktopk_decode_step and kin_block_score_topk can use for the
- * given problem: 0 unless
- * the lists are few (batch * num_kv_heads <= 64) and long (kbar_pages >= 2048),
- * where the step spreads the scoring of each list over several workgroups that
- * meet through this memory (4 bytes per candidate page and an arrival counter
- * per list; contents need no initialisation and are of no use afterwards).
- * Passing NULL or too little is allowed: the step then scores each list with a
- * single workgroup, as it does for every other shape.
+ * given problem: 0 unless the lists are few.  Up to 112 lists (batch *
+ * num_kv_heads) the step may attend a list in parts, by several workgroups that
+ * leave partial results here (up to 256 workgroups x 16 heads x 129 floats:
+ * 2.1 MB at most); up to 64 lists of 2048 candidate pages or more, the step and
+ * the selector may instead spread the scoring of a list over several workgroups
+ * that meet through this memory (4 bytes per candidate page).  An arrival
+ * counter per list comes first; contents need no initialisation and are of no
+ * use afterwards.  Passing NULL or too little is allowed: a list is then shared
+ * by fewer workgroups, or walked by a single one as for every other shape.
  */
 size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages);
 
@@ -324,7 +331,7 @@ size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages);
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
  * no counterpart in the reference (which sizes a 128 MiB workspace up front,
  * benchmark/blocktopk_decoder.py:152).  Same arguments, arithmetic and results as
- * kin_blocktopk_decode_step given a full workspace, but the split-scoring
+ * kin_blocktopk_decode_step given a full workspace, but the
  * workspace is an array of KIN_STATIC_SCRATCH_BYTES bytes inside the library's
  * device code: each GPU the library runs on holds its own copy until the
  * process ends.  The call allocates and frees nothing (no hipMalloc, no
@@ -333,16 +340,17 @@ size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages);
  * the array's address up (hipGetSymbolAddress, with that device current; make
  * that call outside graph capture); the stream must belong to the current
  * device.
- * Limit: shapes whose kin_step_workspace_bytes() exceeds
- * KIN_STATIC_SCRATCH_BYTES are rejected with KIN_ERR_WORKSPACE -- the array
- * covers up to 524288 candidate pages in total over all lists that split, e.g.
- * 64 lists of 8192 pages or 32 of 16384; shapes that do not split (that function
- * returns 0) never touch the array and are always accepted.
+ * Limit: shapes that split their scoring and would need more than
+ * KIN_STATIC_SCRATCH_BYTES for it are rejected with KIN_ERR_WORKSPACE -- the
+ * array covers up to 524288 candidate pages in total over all such lists, e.g.
+ * 64 lists of 8192 pages or 32 of 16384; split attention always fits; shapes
+ * that share no list between workgroups (kin_step_workspace_bytes() returns 0)
+ * never touch the array.
  * All calls on one GPU share the array: calls that overlap in time on the same
  * GPU (different streams, or different threads) race and must be serialised by
  * the caller; calls in one stream are ordered by the stream.
  */
-#define KIN_STATIC_SCRATCH_BYTES (2u * 1024u * 1024u + 256u)
+#define KIN_STATIC_SCRATCH_BYTES (2u * 1024u * 1024u + 32u * 1024u)
 
 size_t kin_static_scratch_bytes(void);
 

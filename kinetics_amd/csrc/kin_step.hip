@@ -1,7 +1,7 @@
 // Fused decode step: append -> score -> select -> attend in ONE launch, one
 // workgroup of NW waves per (sequence, KV head): 4 waves when there are enough
-// lists to fill the GPU, 8 or 16 when there are few (one wide workgroup per CU
-// then keeps as many loads in flight as four narrow ones would).
+// lists to fill the GPU, 8 when there are few (one workgroup per CU).  With lists
+// for at most half the CUs, several workgroups share a list (see StepParams).
 //
 // Compared with the three stand-alone kernels this removes two dependent
 // dispatches, the selector's drain (its last workgroups finish their LDS-only
@@ -39,6 +39,12 @@ struct StepParams {
   int chunks;
   int32_t* ws_count;   // [lists], zero at launch and left zero
   uint32_t* ws_keys;   // [lists, score_key_stride(kbar_pages)]
+  // Split attention (lists for at most half the CUs): `parts` workgroups per list.  Each scores
+  // and selects the whole list for itself (identical results), attends its share of the listed
+  // pages and leaves a partial result; the last one to finish merges them.
+  int parts;
+  uint32_t* ws_po;    // [lists, parts, group, 128] fp32 bits: normalised partial outputs
+  uint32_t* ws_plse;  // [lists, parts, group] fp32 bits: base-2 log-sum-exp of the parts
   int64_t num_pages;
   float scale_log2;
   int deep_score;      // few lists: more mean-key loads in flight per lane (see the kernel)
@@ -54,10 +60,12 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
 
   __shared__ int sh_last;
   const int tid = threadIdx.x;
-  int b, h, chunk = 0;
-  if (p.chunks > 1) {
-    const int list = blockIdx.x / p.chunks;
-    chunk = blockIdx.x - list * p.chunks;
+  int b, h, chunk = 0, part = 0;
+  if (p.chunks > 1 || p.parts > 1) {
+    const int per_list = p.chunks > 1 ? p.chunks : p.parts;
+    const int list = blockIdx.x / per_list;
+    const int sub = blockIdx.x - list * per_list;
+    if (p.chunks > 1) chunk = sub; else part = sub;
     b = list / p.num_kv_heads;
     h = list - b * p.num_kv_heads;
   } else if (!xcd_list_of(blockIdx.x, p.batch, p.num_kv_heads, b, h)) {
@@ -70,7 +78,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   const int ps = p.page_indptr[b], pe = p.page_indptr[b + 1];
   const int n_pages = pe - ps;
   if (n_pages <= 0) {  // empty sequence: nothing to append, select or attend
-    if (chunk != 0) return;
+    if (chunk != 0 || part != 0) return;
     if (p.sel_pages)
       for (int i = tid; i < p.sel_stride; i += NT) p.sel_pages[(int64_t)item * p.sel_stride + i] = -1;
     if (p.sel_count && tid == 0) p.sel_count[item] = 0;
@@ -94,7 +102,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
       __threadfence_block();
     }
   };
-  if (p.chunks <= 1) append_token();
+  if (p.chunks <= 1 && p.parts <= 1) append_token();
 
   // ---- score + select: page list into LDS -------------------------------------
   int32_t* sel_lds = reinterpret_cast<int32_t*>(smem + p.region0_bytes);
@@ -148,11 +156,23 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
       n = score_select<4, NT, F16>(s, sel_lds);
     }
   }
-  if (p.sel_pages) {
+  if (p.sel_pages && part == 0) {
     int32_t* sel = p.sel_pages + (int64_t)item * p.sel_stride;
     for (int i = tid; i < p.sel_stride; i += NT) sel[i] = (i < n) ? sel_lds[i] : -1;
   }
-  if (p.sel_count && tid == 0) p.sel_count[item] = n;
+  if (p.sel_count && tid == 0 && part == 0) p.sel_count[item] = n;
+  int p0 = 0, p1 = n;
+  if (p.parts > 1) {
+    const int per = (n + p.parts - 1) / p.parts;
+    p0 = min(part * per, n);
+    p1 = min(p0 + per, n);
+    // The new token goes into the sequence's last page, which closes every list and is
+    // nobody's candidate (local_tokens >= 1): the part that attends it appends it first.
+    if (p1 == n && p1 > p0) {
+      append_token();
+      __syncthreads();
+    }
+  }
 
   // ---- attend over the listed pages (select scratch is dead: reuse as staging) ---
   AttendArgs a;
@@ -166,25 +186,123 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   a.G = G;
   a.scale_log2 = p.scale_log2;
   a.n = n;
-  a.p0 = 0;
-  a.p1 = n;
+  a.p0 = p0;
+  a.p1 = p1;
   a.last_len = last_len;
   a.first_skip = p.first_page_offset;
-  a.rotate = p.rotate ? attend_rotation(item, 0) : 0u;
+  a.rotate = p.rotate ? attend_rotation(item, part) : 0u;
   attend_list<NG, NW, F16>(
       a, [&](int i) -> int { return __builtin_amdgcn_readfirstlane(sel_lds[i]); }, smem, sm_m, sm_l,
       [&](int g, int d, float o, float lse2) {
-        p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(o);
-        if (p.lse && d == 0) p.lse[hq0 + g] = lse2 * kLn2;
+        if (p.parts > 1) {
+          // partial result, read by a workgroup that may sit on another XCD: device-scope stores
+          const int64_t row = ((int64_t)item * p.parts + part) * G + g;
+          __hip_atomic_store(p.ws_po + row * kHeadDim + d, __float_as_uint(o), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (d == 0) __hip_atomic_store(p.ws_plse + row, __float_as_uint(lse2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+          p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(o);
+          if (p.lse && d == 0) p.lse[hq0 + g] = lse2 * kLn2;
+        }
       });
+  if (p.parts <= 1) return;
+  // Every wave waits for its partial stores to be acknowledged, then the workgroup counts in;
+  // whoever counts in last sees all parts and merges them (as merge_splits_kernel does).
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (tid == 0)
+    sh_last = (__hip_atomic_fetch_add(&p.ws_count[item], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.parts - 1) ? 1 : 0;
+  __syncthreads();
+  if (!sh_last) return;
+  if (tid == 0) __hip_atomic_store(&p.ws_count[item], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+  for (int idx = tid; idx < G * kHeadDim; idx += NT) {
+    const int g = idx >> 7, d = idx & (kHeadDim - 1);
+    const int64_t row0 = (int64_t)item * p.parts * G + g;
+    float mm = kNegInf;
+    for (int sp = 0; sp < p.parts; ++sp)
+      mm = fmaxf(mm, __uint_as_float(__hip_atomic_load(p.ws_plse + row0 + (int64_t)sp * G, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
+    const float m_safe = (mm == kNegInf) ? 0.f : mm;
+    float num = 0.f, den = 0.f;
+    for (int sp = 0; sp < p.parts; ++sp) {
+      const int64_t row = row0 + (int64_t)sp * G;
+      const float wgt = fast_exp2(__uint_as_float(__hip_atomic_load(p.ws_plse + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) - m_safe);
+      num += __uint_as_float(__hip_atomic_load(p.ws_po + row * kHeadDim + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) * wgt;
+      den += wgt;
+    }
+    p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(den > 0.f ? num / den : 0.f);
+    if (p.lse && d == 0) p.lse[hq0 + g] = (den > 0.f) ? (mm + fast_log2(den)) * kLn2 : kNegInf;
+  }
+}
+
+}  // namespace kin
+
+namespace kin {
+
+// How the workgroups of a launch share the lists.  chunks > 1: split scoring (few lists
+// with many candidates); parts > 1: split attention (lists for at most half the CUs);
+// never both.  need: workspace bytes of the mode chosen (arrival counters first).
+struct StepPlan {
+  int chunks, parts;
+  size_t need;
+};
+
+constexpr int kMaxParts = 64;
+
+static size_t parts_workspace_bytes(int64_t items, int parts, int group) {
+  return score_count_bytes(items) + (size_t)items * parts * group * (kHeadDim + 1) * sizeof(float);
+}
+
+// list_tiles: upper bound of the 16-token tiles a page list holds.  avail: bytes the caller's
+// workspace has (a smaller one gets fewer parts, or none, never an error).
+//
+// Split attention: as many parts as keep the launch at one workgroup per CU, each with at
+// least four tiles for each of its 8 waves (below that the merge costs more than it saves;
+// 64 lists x 4 parts of k = 128 pages: 48 us against 46 in 2 parts and 47 whole).  Every part
+// scores the whole list for itself, ~7 ns per mean key on one CU, where split scoring takes a
+// few us for any length; a tile costs the lone attending workgroup ~0.15 us.  So where the
+// shape could split its scoring instead, parts are taken only if they save more attention
+// than the repeated scoring costs (8 lists of 4097 pages, k = 512: 63 us in parts, 103 us
+// with split scoring; k = 128: 49 against 42).
+static StepPlan plan_step(int batch, int num_kv_heads, int group, int kbar_pages, int64_t list_tiles, size_t avail) {
+  const int64_t items = (int64_t)batch * num_kv_heads;
+  StepPlan plan{1, 1, 0};
+  if (items <= 0) return plan;
+  const int chunks = score_chunks(batch, num_kv_heads, kbar_pages);
+  int64_t parts = 1;
+  if (items * 2 <= kNumCus - 32 && list_tiles >= 96) {
+    parts = kNumCus / items;
+    const int64_t by_work = list_tiles / 32;
+    if (parts > by_work) parts = by_work;
+    if (parts > kMaxParts) parts = kMaxParts;
+    while (parts > 1 && parts_workspace_bytes(items, (int)parts, group) > avail) parts /= 2;
+    if (parts < 1) parts = 1;
+  }
+  const bool chunks_fit = chunks > 1 && score_workspace_bytes(items, kbar_pages) <= avail;
+  if (parts > 1 && chunks_fit && 12 * (list_tiles - list_tiles / parts) <= kbar_pages) parts = 1;
+  if (parts > 1) {
+    plan.parts = (int)parts;
+    plan.need = parts_workspace_bytes(items, plan.parts, group);
+  } else if (chunks_fit) {
+    plan.chunks = chunks;
+    plan.need = score_workspace_bytes(items, kbar_pages);
+  }
+  return plan;
 }
 
 }  // namespace kin
 
 extern "C" size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages) {
-  if (kin::score_chunks(batch, num_kv_heads, kbar_pages) <= 1) return 0;
+  // Enough for whichever mode the launch picks, whatever the group size and page budget.
   const int64_t items = (int64_t)batch * num_kv_heads;
-  return kin::score_workspace_bytes(items, kbar_pages);
+  if (items <= 0) return 0;
+  size_t need = 0;
+  if (kin::score_chunks(batch, num_kv_heads, kbar_pages) > 1) need = kin::score_workspace_bytes(items, kbar_pages);
+  if (items * 2 <= kin::kNumCus - 32) {
+    int64_t parts = kin::kNumCus / items;
+    if (parts > kin::kMaxParts) parts = kin::kMaxParts;
+    const size_t split = kin::parts_workspace_bytes(items, (int)parts, kin::kMaxGroup);
+    if (split > need) need = split;
+  }
+  return need;
 }
 
 namespace kin {
@@ -261,16 +379,24 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
   if (xcd_grid_size(batch, num_kv_heads) > 0x7fffffffLL)
     return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
   const int nw = items <= kNumCus ? 8 : 4;
-  // Few long sequences: spread the scoring of each list over several workgroups.
-  p.chunks = score_chunks(batch, num_kv_heads, kbar_pages);
-  if (p.chunks > 1 && workspace && aligned16(workspace) &&
-      workspace_bytes >= kin_step_workspace_bytes(batch, num_kv_heads, kbar_pages)) {
+  // Few lists: several workgroups share one (split attention, or split scoring for very long sequences).
+  const StepPlan plan = plan_step(batch, num_kv_heads, p.group, kbar_pages, (int64_t)list_cap << page_tile_shift(page_size),
+                                  workspace && aligned16(workspace) ? workspace_bytes : 0);
+  p.chunks = plan.chunks;
+  p.parts = plan.parts;
+  p.ws_count = nullptr;
+  p.ws_keys = nullptr;
+  p.ws_po = nullptr;
+  p.ws_plse = nullptr;
+  if (plan.chunks > 1 || plan.parts > 1) {
+    char* after_counters = static_cast<char*>(workspace) + score_count_bytes(items);
     p.ws_count = static_cast<int32_t*>(workspace);
-    p.ws_keys = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + score_count_bytes(items));
-  } else {
-    p.chunks = 1;
-    p.ws_count = nullptr;
-    p.ws_keys = nullptr;
+    if (plan.chunks > 1) {
+      p.ws_keys = reinterpret_cast<uint32_t*>(after_counters);
+    } else {
+      p.ws_po = reinterpret_cast<uint32_t*>(after_counters);
+      p.ws_plse = p.ws_po + (size_t)items * plan.parts * p.group * kHeadDim;
+    }
   }
   p.deep_score = items < 4096 ? 1 : 0;
   p.rotate = attend_rotates(items) ? 1 : 0;
@@ -300,12 +426,12 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
     if (st) return st;
   }
   unsigned grid = (unsigned)xcd_grid_size(batch, num_kv_heads);
-  if (p.chunks > 1) {
+  if (p.chunks > 1 || p.parts > 1) {
     // the arrival counters start at zero (a fill kernel, so that the launch pair can be captured in a graph)
     fill_zero_i32_kernel<<<(unsigned)((items + 255) / 256), 256, 0, s>>>(p.ws_count, (int)items);
     st = check_hip(hipGetLastError(), "fill_zero_i32_kernel launch");
     if (st) return st;
-    grid = (unsigned)(items * p.chunks);
+    grid = (unsigned)(items * (p.chunks > 1 ? p.chunks : p.parts));
   }
   void* args[] = {&p};
   st = check_hip(hipLaunchKernel(kernel, dim3(grid), dim3(nw * 64), args, lds, s), "blocktopk_step_kernel launch");
@@ -313,8 +439,8 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
 }
 
 // ---- device memory of the entry point that allocates nothing -------------------
-// Split-scoring workspace (arrival counters, then keys) for callers that cannot
-// bring one.  Every GPU the library's code object is loaded on holds its own copy
+// Workspace of the launches that share lists between workgroups (arrival counters,
+// then keys or partial results) for callers that cannot bring one.  Every GPU the library's code object is loaded on holds its own copy
 // until the process ends.  In host code the array's name is only a handle for
 // hipGetSymbolAddress; kernels get the address that call returns.
 constexpr size_t kStaticScratchBytes = KIN_STATIC_SCRATCH_BYTES;
@@ -382,10 +508,16 @@ extern "C" int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_b
                                                 int first_page_offset, float sm_scale, kin_stream_t stream) {
   using namespace kin;
   const char* fn = "kin_blocktopk_decode_step_static";
-  // What the split scoring of this shape needs (0: the shape does not split and
-  // no scratch is touched).  Sizes beyond the array are an error, not a silent
-  // fall-back to the slower single-workgroup scoring.
-  const size_t need = kin_step_workspace_bytes(batch, num_kv_heads, kbar_pages);
+  // What this shape's way of sharing lists between workgroups needs, from the dimensions
+  // alone.  Split scoring beyond the array is an error, not a silent fall-back to the
+  // slower single-workgroup scoring; split attention always fits (kMaxGroup heads included).
+  size_t need = 0;
+  if (batch > 0 && num_kv_heads > 0 && num_q_heads >= num_kv_heads && kbar_pages > 0 && topk >= 0 && sink_pages >= 0 &&
+      local_tokens >= 1 && page_size >= kPageSize) {
+    const int64_t list_cap = (int64_t)topk + sink_pages + max_local_pages(local_tokens);
+    need = plan_step(batch, num_kv_heads, num_q_heads / num_kv_heads, kbar_pages, list_cap << page_tile_shift(page_size),
+                     ~(size_t)0).need;
+  }
   if (need > kStaticScratchBytes)
     return fail(KIN_ERR_WORKSPACE,
                 "%s: batch=%d x num_kv_heads=%d lists of kbar_pages=%d need %zu bytes of scratch, the built-in array has %zu "
@@ -398,5 +530,5 @@ extern "C" int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_b
   }
   return launch_step(fn, false, q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sink_pages, local_tokens,
                      sel_pages, sel_count, out, lse, batch, num_q_heads, num_kv_heads, head_dim, page_size, num_pages,
-                     kbar_pages, sel_stride, first_page_offset, sm_scale, ws, need > 0 ? kStaticScratchBytes : 0, stream);
+                     kbar_pages, sel_stride, first_page_offset, sm_scale, ws, ws ? kStaticScratchBytes : 0, stream);
 }

@@ -373,20 +373,20 @@ def dense_paged_decode(q, kv_cache, page_indices, page_indptr, last_page_len, ma
 def prefer_fused_step(batch: int, num_kv_heads: int, max_pages_per_seq: int, topk: int) -> bool:
     """Which of the two equivalent decode-step paths to use.  The single-launch
     kernel saves two dependent dispatches, the selector's drain and the attention
-    ramp-up, but one workgroup walks a whole list: it has no split-K.  Measured on
-    MI355X against the three launches queued back to back (fused / three): 8 lists
-    k=128 0.87, k=256 1.31, k=512 1.87; 64 lists k=128 1.02, k=512 1.36; 100 lists
-    k=512 1.03, k=1024 1.18; 128 lists k=768..2048 1.01..1.04; 200..256 lists
-    0.95..0.98; 260..300 lists k<=768 0.96..0.98, k=1024 1.17..1.20 (some CUs hold
-    two long lists, the others one); 350 lists and more 0.96..1.00 (600 lists with
-    k>=1024: 1.05).  Hence: fused for k <= 128 at any batch, up to k = 512 from 96
-    lists, everything from 160 lists -- except 257..349 lists with k > 768."""
-    del max_pages_per_seq
+    ramp-up; given its workspace it shares a list between workgroups when the lists
+    are few (split attention up to 112 lists, split scoring for very long
+    sequences).  Measured on MI355X against the three launches queued back to back
+    (fused / three): 1..112 lists of 2049 pages, k = 128..2048: 0.84..1.04; of 257
+    pages: 0.5; 8..32 lists of 8193 pages: k = 128 0.94, k = 512 1.3..1.6, k = 2048
+    1.05..1.15 (every part would score 2 MiB of mean keys for itself, so the step
+    splits the scoring instead and one workgroup attends alone); 128..256 lists
+    0.95..1.04; 260..300 lists k <= 768 0.96..0.98, k = 1024 1.17..1.20 (some CUs hold
+    two long lists, the others one); 350 lists and more 0.96..1.00.  Hence: fused,
+    except few lists of more than 4096 pages with k >= 512, and 257..349 lists with
+    k > 768."""
     lists = batch * num_kv_heads
-    if lists < 96:
-        return topk <= 128
     if lists < 160:
-        return topk <= 512
+        return not (max_pages_per_seq > 4096 and topk >= 512)
     if 256 < lists < 350:
         return topk <= 768
     return True
@@ -399,8 +399,8 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
     reference layer's forward (benchmark/blocktopk_decoder.py) as a single
     kernel.  ``k``/``v`` may be None (no append); ``sel_pages``/``sel_count`` are
     optional outputs.  ``workspace`` (``step_workspace_bytes``; allocated here when
-    None and the shape profits) lets few, long sequences spread their scoring over
-    the GPU.  ``static_scratch=True`` calls ``kin_blocktopk_decode_step_static``
+    None and the shape profits) lets several workgroups share a list when the lists
+    are few: split attention, or split scoring for very long sequences.  ``static_scratch=True`` calls ``kin_blocktopk_decode_step_static``
     instead: the library's built-in device array is the workspace and nothing is
     allocated (``out`` must then be given; ``workspace`` must be None).
     Returns ``out`` [batch, num_q_heads, head_dim] bf16."""

@@ -257,12 +257,13 @@ def test_auto_splits_policy_follows_the_lists(lib):
 
 
 def test_path_preference_rule():
-    """prefer_fused_step: the single launch for short page lists at any batch and for
-    everything from 160 lists on, except long lists just above one list per CU."""
+    """prefer_fused_step: the single launch, except few lists of very long sequences with
+    long page lists and long lists just above one list per CU."""
     from kinetics_amd import ops
-    assert ops.prefer_fused_step(8, 1, 257, 64) and ops.prefer_fused_step(1, 8, 2049, 128)
-    assert not ops.prefer_fused_step(8, 1, 2049, 256) and not ops.prefer_fused_step(64, 1, 2049, 512)
-    assert ops.prefer_fused_step(100, 1, 2049, 512) and not ops.prefer_fused_step(100, 1, 2049, 1024)
+    assert ops.prefer_fused_step(8, 1, 257, 64) and ops.prefer_fused_step(1, 8, 2049, 2048)
+    assert ops.prefer_fused_step(64, 1, 2049, 512) and ops.prefer_fused_step(100, 1, 2049, 1024)
+    assert ops.prefer_fused_step(8, 1, 8193, 128) and not ops.prefer_fused_step(8, 1, 8193, 512)
+    assert not ops.prefer_fused_step(32, 1, 4097, 2048)
     assert ops.prefer_fused_step(256, 1, 1025, 64) and ops.prefer_fused_step(200, 1, 4097, 2048)
     assert ops.prefer_fused_step(300, 1, 2049, 768) and not ops.prefer_fused_step(300, 1, 2049, 1024)
     assert ops.prefer_fused_step(512, 8, 2049, 64) and ops.prefer_fused_step(4096, 1, 2049, 128)
@@ -349,7 +350,7 @@ def test_header_is_plain_c_and_links_from_c(tmp_path):
 def test_static_scratch_step_size_limit_is_checked_before_anything_else(lib):
     """The entry point that allocates nothing rejects shapes whose split-scoring
     scratch exceeds its built-in array, from the dimensions alone."""
-    assert lib.kin_static_scratch_bytes() == 2 * 1024 * 1024 + 256
+    assert lib.kin_static_scratch_bytes() == 2 * 1024 * 1024 + 32 * 1024
     assert 0 < lib.kin_step_workspace_bytes(64, 1, 8192) <= lib.kin_static_scratch_bytes()
     assert lib.kin_step_workspace_bytes(64, 1, 16384) > lib.kin_static_scratch_bytes()
     st = lib.kin_blocktopk_decode_step_static(None, None, None, None, None, None, None, None, 128, 0, 1, None, None, None,

@@ -1,6 +1,6 @@
 """The decode step's entry point that allocates nothing
-(kin_blocktopk_decode_step_static: split-scoring workspace = an array inside the
-library's device code) against the existing entry point it is a variant of
+(kin_blocktopk_decode_step_static: the workspace through which workgroups share a
+list = an array inside the library's device code) against the existing entry point it is a variant of
 (kin_blocktopk_decode_step with a caller workspace), through the C ABI: cache
 bytes, page lists and attention output bit-equal, on calls in a row that share
 the array -- the second with a smaller input, so the first call's keys are still
@@ -63,18 +63,24 @@ def test_static_scratch_step_equals_workspace_step():
     from kinetics_amd import _lib, ops
 
     lib = _lib.load()
-    assert lib.kin_static_scratch_bytes() == 2 * 1024 * 1024 + 256
+    assert lib.kin_static_scratch_bytes() == 2 * 1024 * 1024 + 32 * 1024
     # two calls in a row on the same array, the second smaller (fewer and shorter lists): the
     # first call's keys and counters are what the second finds there
     big = P.make_problem(9101, [PS * 2500 + 3, PS * 2100 + 16, 5, 0, PS * 300 + 1], num_kv_heads=2, group=4, topk=40)
     _both_ways(ops, big, sink=1, local=17, what="first call (5 sequences x 2 KV heads, up to 2501 pages)", must_split=True)
     small = P.make_problem(9102, [PS * 2048 + 9, 70], num_kv_heads=1, group=8, topk=64)
     _both_ways(ops, small, sink=0, local=1, what="second call (2 sequences, up to 2049 pages)", must_split=True)
-    # a shape that does not split never touches the array
-    plain = P.make_problem(9103, [PS * 40 + 1] * 6 + [3], num_kv_heads=2, group=2, topk=8)
-    _both_ways(ops, plain, sink=0, local=1, what="third call (no split scoring)", must_split=False)
+    # a shape with lists for more than half the CUs shares nothing between workgroups and never touches the array
+    plain = P.make_problem(9103, [PS * 40 + 1] * 59 + [3], num_kv_heads=2, group=2, topk=8)
+    _both_ways(ops, plain, sink=0, local=1, what="third call (one workgroup per list)", must_split=False)
+    # few lists with long page lists: split attention, the partial results lie where the keys lay;
+    # 8 lists x 32 parts x 16 heads fill the array to the last kilobytes
+    parts = P.make_problem(9104, [PS * 400 + 1, PS * 300 + 16, 9], num_kv_heads=2, group=4, topk=150)
+    _both_ways(ops, parts, sink=1, local=20, what="fourth call (split attention)", must_split=True)
+    full = P.make_problem(9105, [PS * 1300 + 5] * 4, num_kv_heads=2, group=16, topk=1100)
+    _both_ways(ops, full, sink=0, local=1, what="fifth call (split attention, 16 heads per list)", must_split=True)
     # and the first shape once more after them
-    _both_ways(ops, big, sink=0, local=33, what="fourth call (first shape again)", must_split=True)
+    _both_ways(ops, big, sink=0, local=33, what="sixth call (first shape again)", must_split=True)
 
 
 def test_static_scratch_step_rejects_sizes_beyond_the_array():
