@@ -1480,14 +1480,16 @@ def test_token_topk_rejects_short_workspace_and_long_sequences(ops):
 # --------------------------------------------------------------------------- graph capture / tracing
 
 
-@pytest.mark.parametrize("path", ["three", "three_split", "fused", "fused_split", "token", "strided", "token_split",
-                                  "strided_split"])
+@pytest.mark.parametrize("path", ["three", "three_split", "fused", "fused_split", "fused_parts", "token", "strided",
+                                  "token_split", "strided_split"])
 def test_step_replays_under_hip_graph(ops, path):
     """No allocation, no host sync, fixed buffers: every launch sequence can be
     captured once and replayed.  Every replay (with eager work and syncs in
     between) must equal the eager result for the inputs current at replay time."""
     if path.endswith("_split"):   # few long sequences: fill kernel + several workgroups per list
         pb = P.make_problem(801, [PS * 2300 + 3, PS * 2100 + 9], num_kv_heads=1, group=4, topk=32)
+    elif path == "fused_parts":   # few lists with long page lists: fill kernel + several workgroups attend each list
+        pb = P.make_problem(802, [PS * 400 + 3] * 5 + [PS * 90], num_kv_heads=2, group=4, topk=200)
     else:
         pb = P.make_problem(800, [PS * 200 + 3] * 64, num_kv_heads=2, group=4, topk=32)
     g = Gpu(pb)
@@ -1496,14 +1498,14 @@ def test_step_replays_under_hip_graph(ops, path):
     step_ws = torch.empty(max(16, ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[2])), dtype=torch.uint8, device=DEV)
     tok_ws = torch.empty(max(16, ops.strided_topk_workspace_bytes(pb.B, pb.Hkv, pb.max_pages)), dtype=torch.uint8, device=DEV)
     tok_sel = torch.full((pb.B, pb.Hkv, 64 * 16 + 4 + 16), -1, dtype=torch.int32, device=DEV)
-    assert path.endswith("_split") == (ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[2]) > 0)
+    assert path.endswith(("_split", "_parts")) == (ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[2]) > 0)
 
     def step():
         if path in ("three", "three_split"):
             ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
             ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, pb.topk, g.sel, g.cnt, workspace=step_ws)
             ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, out=out, workspace=ws)
-        elif path in ("fused", "fused_split"):
+        elif path in ("fused", "fused_split", "fused_parts"):
             ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, pb.topk, out=out,
                                       sel_pages=g.sel, sel_count=g.cnt, workspace=step_ws)
         else:
