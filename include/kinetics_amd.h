@@ -75,7 +75,7 @@ enum kin_status {
  * tokens, float16 twins (kin_*_f16), groups of up to 16 query heads per KV head,
  * the page pool and kin_blocktopk_decode_step_static.  2.1.0: the decode step
  * attends few lists in parts (kin_step_workspace_bytes grows to up to 2.1 MB for
- * up to 112 lists; KIN_STATIC_SCRATCH_BYTES grows by 32 KiB less 256 B). */
+ * up to 128 lists; KIN_STATIC_SCRATCH_BYTES grows by 32 KiB less 256 B). */
 int kin_version(void);
 
 /* Human-readable text of the last non-OK status on the calling thread
@@ -314,7 +314,7 @@ int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const ki
 
 /*
  * Workspace kin_blocktopk_decode_step and kin_block_score_topk can use for the
- * given problem: 0 unless the lists are few.  Up to 112 lists (batch *
+ * given problem: 0 unless the lists are few.  Up to 128 lists (batch *
  * num_kv_heads) the step may attend a list in parts, by several workgroups that
  * leave partial results here (up to 256 workgroups x 16 heads x 129 floats:
  * 2.1 MB at most); up to 64 lists of 2048 candidate pages or more, the step and

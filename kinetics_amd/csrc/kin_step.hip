@@ -256,7 +256,9 @@ static size_t parts_workspace_bytes(int64_t items, int parts, int group) {
 //
 // Split attention: as many parts as keep the launch at one workgroup per CU, each with at
 // least four tiles for each of its 8 waves (below that the merge costs more than it saves;
-// 64 lists x 4 parts of k = 128 pages: 48 us against 46 in 2 parts and 47 whole).  Every part
+// 64 lists x 4 parts of k = 128 pages: 48 us against 46 in 2 parts and 47 whole; a launch
+// that fills every CU wants longer lists still: 128 lists x 2 parts lose 6 % at k = 128
+// and gain 5 % at k = 512).  Every part
 // scores the whole list for itself, ~7 ns per mean key on one CU, where split scoring takes a
 // few us for any length; a tile costs the lone attending workgroup ~0.15 us.  So where the
 // shape could split its scoring instead, parts are taken only if they save more attention
@@ -268,7 +270,7 @@ static StepPlan plan_step(int batch, int num_kv_heads, int group, int kbar_pages
   if (items <= 0) return plan;
   const int chunks = score_chunks(batch, num_kv_heads, kbar_pages);
   int64_t parts = 1;
-  if (items * 2 <= kNumCus - 32 && list_tiles >= 96) {
+  if (items * 2 <= kNumCus && list_tiles >= (items * 2 <= kNumCus - 32 ? 96 : 384)) {
     parts = kNumCus / items;
     const int64_t by_work = list_tiles / 32;
     if (parts > by_work) parts = by_work;
@@ -296,7 +298,7 @@ extern "C" size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar
   if (items <= 0) return 0;
   size_t need = 0;
   if (kin::score_chunks(batch, num_kv_heads, kbar_pages) > 1) need = kin::score_workspace_bytes(items, kbar_pages);
-  if (items * 2 <= kin::kNumCus - 32) {
+  if (items * 2 <= kin::kNumCus) {
     int64_t parts = kin::kNumCus / items;
     if (parts > kin::kMaxParts) parts = kin::kMaxParts;
     const size_t split = kin::parts_workspace_bytes(items, (int)parts, kin::kMaxGroup);

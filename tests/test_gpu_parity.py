@@ -1491,7 +1491,7 @@ def test_step_replays_under_hip_graph(ops, path):
     elif path == "fused_parts":   # few lists with long page lists: fill kernel + several workgroups attend each list
         pb = P.make_problem(802, [PS * 400 + 3] * 5 + [PS * 90], num_kv_heads=2, group=4, topk=200)
     else:
-        pb = P.make_problem(800, [PS * 200 + 3] * 64, num_kv_heads=2, group=4, topk=32)
+        pb = P.make_problem(800, [PS * 200 + 3] * 66, num_kv_heads=2, group=4, topk=32)
     g = Gpu(pb)
     out = torch.empty_like(g.q)
     ws = workspace(ops, pb, pb.topk + 1, 0)

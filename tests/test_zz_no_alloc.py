@@ -71,7 +71,7 @@ def test_static_scratch_step_equals_workspace_step():
     small = P.make_problem(9102, [PS * 2048 + 9, 70], num_kv_heads=1, group=8, topk=64)
     _both_ways(ops, small, sink=0, local=1, what="second call (2 sequences, up to 2049 pages)", must_split=True)
     # a shape with lists for more than half the CUs shares nothing between workgroups and never touches the array
-    plain = P.make_problem(9103, [PS * 40 + 1] * 59 + [3], num_kv_heads=2, group=2, topk=8)
+    plain = P.make_problem(9103, [PS * 40 + 1] * 69 + [3], num_kv_heads=2, group=2, topk=8)
     _both_ways(ops, plain, sink=0, local=1, what="third call (one workgroup per list)", must_split=False)
     # few lists with long page lists: split attention, the partial results lie where the keys lay;
     # 8 lists x 32 parts x 16 heads fill the array to the last kilobytes
