@@ -968,57 +968,58 @@ def test_fused_step_split_scoring_for_few_long_sequences(ops, hkv, group):
     assert torch.equal(one.sel, a.sel)
 
 
-@pytest.mark.parametrize("ps", [16, 32, 64])
-def test_fused_step_split_attention_for_few_lists(ops, ps):
+@pytest.mark.parametrize("ps,fmt", [(16, "bf16"), (32, "bf16"), (64, "bf16"), (16, "f16")])
+def test_fused_step_split_attention_for_few_lists(ops, ps, fmt):
     """Lists for at most half the CUs with long page lists: several workgroups per
     list, each scoring and selecting for itself and attending a share of the pages,
     the last to finish merging the partial results through the workspace.  Same
     cache bytes and page lists as one workgroup per list, outputs equal to fp32
     summation order, call after call on a workspace that was never initialised;
-    groups of 1 to 16 heads, an offset, an empty and a one-page sequence."""
-    rng = np.random.default_rng(7700 + ps)
-    for trial, (hkv, group, topk, sink, local, offset) in enumerate(
-            [(1, 4, 200, 0, 1, 0), (2, 8, 120, 1, 40, 5), (1, 16, 300, 2, 17, 0), (4, 1, 96, 1, 1, 3), (1, 5, 700, 0, 33, 0)]):
-        lengths = [ps * 900 + 3, ps * 400 + ps, 5, 0, ps * 150 + 1, ps * 1000 + 7, ps * 2 + 2][: max(3, 7 - trial)]
-        lengths = [L + offset if L else 0 for L in lengths]
-        what = f"ps={ps} trial {trial}: hkv={hkv} G={group} topk={topk} sink={sink} local={local} offset={offset}"
-        pb = P.make_problem(7700 + 10 * trial + ps, lengths, num_kv_heads=hkv, group=group, topk=topk, page_size=ps)
-        need = ops.step_workspace_bytes(pb.B, hkv, pb.kbar.shape[2])
-        assert need > 0, what
-        ws = torch.full((need,), 0xAB, dtype=torch.uint8, device=DEV)
-        cap = ops.sel_list_capacity(topk, sink, local)
-        plain = Gpu(pb)
-        plain.sel = torch.full((pb.B, hkv, cap), -7, dtype=torch.int32, device=DEV)
-        lse_plain = torch.empty(pb.B, pb.Hq, dtype=torch.float32, device=DEV)
-        out_plain = ops.blocktopk_decode_step(plain.q, plain.k, plain.v, plain.kv, plain.kbar, plain.indices, plain.indptr,
-                                              plain.last, topk, sel_pages=plain.sel, sel_count=plain.cnt, lse=lse_plain,
-                                              sink_pages=sink, local_tokens=local, first_page_offset=offset,
-                                              workspace=torch.empty(0, dtype=torch.uint8, device=DEV))
-        first = None
-        for call in range(3):
-            g = Gpu(pb)
-            g.sel = torch.full((pb.B, hkv, cap), -7, dtype=torch.int32, device=DEV)
-            lse = torch.full((pb.B, pb.Hq), float("nan"), dtype=torch.float32, device=DEV)
-            out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, topk, sel_pages=g.sel,
-                                            sel_count=g.cnt, lse=lse, sink_pages=sink, local_tokens=local,
-                                            first_page_offset=offset, workspace=ws)
-            torch.cuda.synchronize()
-            assert torch.equal(g.kv, plain.kv) and torch.equal(g.kbar, plain.kbar), f"{what}: cache differs (call {call})"
-            assert torch.equal(g.sel, plain.sel) and torch.equal(g.cnt, plain.cnt), f"{what}: lists differ (call {call})"
-            assert torch.allclose(out.float(), out_plain.float(), rtol=1e-2, atol=1e-2), what
-            assert torch.allclose(lse, lse_plain, rtol=1e-5, atol=1e-5), what
-            if first is None:
-                first = (out.clone(), lse.clone())
-            else:
-                assert torch.equal(out, first[0]) and torch.equal(lse, first[1]), f"{what}: call {call} differs from the first"
-        kv, kbar = pb.kv_cache.copy(), pb.kbar.copy()
-        O.append_paged_kv(pb.k, pb.v, kv, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
-        assert np.array_equal(P.from_torch(plain.kv), kv) and np.array_equal(P.from_torch(plain.kbar), kbar), what
-        want, want_lse = O.sparse_paged_decode(pb.q, kv, plain.sel.cpu().numpy(), plain.cnt.cpu().numpy(), pb.last_page_len,
-                                               first_page_offset=offset)
-        assert_out_close(first[0], want, what)
-        live = np.isfinite(want_lse)
-        assert np.allclose(first[1].cpu().numpy()[live], want_lse[live], rtol=1e-4, atol=1e-4), what
+    groups of 1 to 16 heads, an offset, an empty and a one-page sequence; bfloat16 and float16."""
+    with O.element_format(fmt):
+        rng = np.random.default_rng(7700 + ps)
+        for trial, (hkv, group, topk, sink, local, offset) in enumerate(
+                [(1, 4, 200, 0, 1, 0), (2, 8, 120, 1, 40, 5), (1, 16, 300, 2, 17, 0), (4, 1, 96, 1, 1, 3), (1, 5, 700, 0, 33, 0)]):
+            lengths = [ps * 900 + 3, ps * 400 + ps, 5, 0, ps * 150 + 1, ps * 1000 + 7, ps * 2 + 2][: max(3, 7 - trial)]
+            lengths = [L + offset if L else 0 for L in lengths]
+            what = f"ps={ps} trial {trial}: hkv={hkv} G={group} topk={topk} sink={sink} local={local} offset={offset}"
+            pb = P.make_problem(7700 + 10 * trial + ps, lengths, num_kv_heads=hkv, group=group, topk=topk, page_size=ps)
+            need = ops.step_workspace_bytes(pb.B, hkv, pb.kbar.shape[2])
+            assert need > 0, what
+            ws = torch.full((need,), 0xAB, dtype=torch.uint8, device=DEV)
+            cap = ops.sel_list_capacity(topk, sink, local)
+            plain = Gpu(pb)
+            plain.sel = torch.full((pb.B, hkv, cap), -7, dtype=torch.int32, device=DEV)
+            lse_plain = torch.empty(pb.B, pb.Hq, dtype=torch.float32, device=DEV)
+            out_plain = ops.blocktopk_decode_step(plain.q, plain.k, plain.v, plain.kv, plain.kbar, plain.indices, plain.indptr,
+                                                  plain.last, topk, sel_pages=plain.sel, sel_count=plain.cnt, lse=lse_plain,
+                                                  sink_pages=sink, local_tokens=local, first_page_offset=offset,
+                                                  workspace=torch.empty(0, dtype=torch.uint8, device=DEV))
+            first = None
+            for call in range(3):
+                g = Gpu(pb)
+                g.sel = torch.full((pb.B, hkv, cap), -7, dtype=torch.int32, device=DEV)
+                lse = torch.full((pb.B, pb.Hq), float("nan"), dtype=torch.float32, device=DEV)
+                out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, topk, sel_pages=g.sel,
+                                                sel_count=g.cnt, lse=lse, sink_pages=sink, local_tokens=local,
+                                                first_page_offset=offset, workspace=ws)
+                torch.cuda.synchronize()
+                assert torch.equal(g.kv, plain.kv) and torch.equal(g.kbar, plain.kbar), f"{what}: cache differs (call {call})"
+                assert torch.equal(g.sel, plain.sel) and torch.equal(g.cnt, plain.cnt), f"{what}: lists differ (call {call})"
+                assert torch.allclose(out.float(), out_plain.float(), rtol=1e-2, atol=1e-2), what
+                assert torch.allclose(lse, lse_plain, rtol=1e-5, atol=1e-5), what
+                if first is None:
+                    first = (out.clone(), lse.clone())
+                else:
+                    assert torch.equal(out, first[0]) and torch.equal(lse, first[1]), f"{what}: call {call} differs from the first"
+            kv, kbar = pb.kv_cache.copy(), pb.kbar.copy()
+            O.append_paged_kv(pb.k, pb.v, kv, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
+            assert np.array_equal(P.from_torch(plain.kv), kv) and np.array_equal(P.from_torch(plain.kbar), kbar), what
+            want, want_lse = O.sparse_paged_decode(pb.q, kv, plain.sel.cpu().numpy(), plain.cnt.cpu().numpy(), pb.last_page_len,
+                                                   first_page_offset=offset)
+            assert_out_close(first[0], want, what)
+            live = np.isfinite(want_lse)
+            assert np.allclose(first[1].cpu().numpy()[live], want_lse[live], rtol=1e-4, atol=1e-4), what
 
 
 def test_seeded_sweep_of_split_scoring(ops):
