@@ -170,13 +170,14 @@ namespace kin {
 // Bytes of the arrival counters in front of the score arrays.
 static size_t token_count_bytes(int64_t lists) { return ((size_t)lists * sizeof(int32_t) + 255) & ~(size_t)255; }
 
-// Workgroups that share the scoring of one list (each at least 256 pages = 1 MiB
-// of keys): as many as it takes to give every CU one when the lists are fewer than
-// the CUs, otherwise one -- with the GPU already full, splitting only adds
+// Workgroups that share the scoring of one list (each at least 64 pages = 256 KiB
+// of keys; with 256 the 8 lists of a small batch occupied 64 CUs: 109 against 97 us
+// at 32 K tokens): as many as it takes to give every CU one when the lists are fewer
+// than the CUs, otherwise one -- with the GPU already full, splitting only adds
 // workgroups, the extra pass that recounts the first radix digit and a second
 // round of launches (measured: 6.35 -> 7.1 ms at 4096 lists of 32 K tokens).
 static int token_score_chunks(int64_t lists, int max_pages_per_seq) {
-  const int by_len = max_pages_per_seq / 256;
+  const int by_len = max_pages_per_seq / 64;
   const int64_t want = kNumCus / lists;
   if (by_len < 2 || want < 2) return 1;
   return (int)(want < by_len ? want : by_len);
@@ -286,7 +287,10 @@ static int launch_token_policy(const char* fn, bool f16, const kin_bf16_t* q, co
     nw = items > kNumCus && small <= 50 * 1024 ? 4 : 12;
   } else {
     p.chunks = token_score_chunks(items, max_pages_per_seq);
-    nw = items <= 2 * kNumCus ? 8 : 4;
+    // Up to one list per CU: 12 waves once a sequence may have more keys than 8 waves hold in
+    // registers through the select's passes (32 K; 8 lists of 32 K tokens: 97 -> 83 us), else 8.
+    nw = items <= kNumCus && (int64_t)max_pages_per_seq * kPageSize > 8 * 4096 ? 12 : (items <= 2 * kNumCus ? 8 : 4);
+    if (nw == 12 && (size_t)attend_lds_bytes(12) + tail_bytes > 150 * 1024) nw = 8;  // room for the strided policy's bitmap
   }
   const int64_t grid = xcd_grid_size(batch, num_kv_heads) * p.chunks;
   if (grid > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
@@ -302,7 +306,7 @@ static int launch_token_policy(const char* fn, bool f16, const kin_bf16_t* q, co
        : reinterpret_cast<const void*>(&token_topk_kernel<NG_, NW_, S_, L_, false>))
 #define KIN_TOKEN_PICK(NG_, S_)                                                             \
   (ldsk ? (nw == 12 ? KIN_TOKEN_KERNEL(NG_, 12, S_, true) : KIN_TOKEN_KERNEL(NG_, 4, S_, true)) \
-        : (nw == 8 ? KIN_TOKEN_KERNEL(NG_, 8, S_, false) : KIN_TOKEN_KERNEL(NG_, 4, S_, false)))
+        : (nw == 12 ? KIN_TOKEN_KERNEL(NG_, 12, S_, false) : nw == 8 ? KIN_TOKEN_KERNEL(NG_, 8, S_, false) : KIN_TOKEN_KERNEL(NG_, 4, S_, false)))
   const void* kernel;
   if (strided)
     kernel = p.group <= 4 ? KIN_TOKEN_PICK(1, true) : KIN_TOKEN_PICK(4, true);
