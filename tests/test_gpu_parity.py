@@ -1012,6 +1012,14 @@ def test_fused_step_split_attention_for_few_lists(ops, ps, fmt):
                     first = (out.clone(), lse.clone())
                 else:
                     assert torch.equal(out, first[0]) and torch.equal(lse, first[1]), f"{what}: call {call} differs from the first"
+            # a workspace too small for all the parts gets fewer of them, never an error
+            for frac in (3, 17):
+                g = Gpu(pb)
+                out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, topk, sink_pages=sink,
+                                                local_tokens=local, first_page_offset=offset, workspace=ws[: need // frac])
+                torch.cuda.synchronize()
+                assert torch.equal(g.kv, plain.kv) and torch.equal(g.kbar, plain.kbar), f"{what}: cache differs (1/{frac} workspace)"
+                assert torch.allclose(out.float(), out_plain.float(), rtol=1e-2, atol=1e-2), f"{what} (1/{frac} workspace)"
             kv, kbar = pb.kv_cache.copy(), pb.kbar.copy()
             O.append_paged_kv(pb.k, pb.v, kv, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
             assert np.array_equal(P.from_torch(plain.kv), kv) and np.array_equal(P.from_torch(plain.kbar), kbar), what
