@@ -99,9 +99,11 @@ __global__ __launch_bounds__(128) void merge_splits_kernel(const float* __restri
   const int d = threadIdx.x;
   const float* l2 = ws_lse + hq * num_splits;
   float mm = kNegInf;
+#pragma unroll 8
   for (int s = 0; s < num_splits; ++s) mm = fmaxf(mm, l2[s]);
   const float m_safe = (mm == kNegInf) ? 0.f : mm;
   float num = 0.f, den = 0.f;
+#pragma unroll 8
   for (int s = 0; s < num_splits; ++s) {
     const float wgt = fast_exp2(l2[s] - m_safe);
     num += ws_o[(hq * num_splits + s) * kHeadDim + d] * wgt;

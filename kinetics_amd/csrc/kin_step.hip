@@ -214,22 +214,39 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   __syncthreads();
   if (!sh_last) return;
   if (tid == 0) __hip_atomic_store(&p.ws_count[item], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
-  for (int idx = tid; idx < G * kHeadDim; idx += NT) {
-    const int g = idx >> 7, d = idx & (kHeadDim - 1);
-    const int64_t row0 = (int64_t)item * p.parts * G + g;
+  // The parts' log-sum-exps become weights in LDS (the attention's staging area is dead), then every
+  // thread sums its output element over the parts with independent device-scope loads.
+  float* wl = reinterpret_cast<float*>(smem);  // [parts][G] weights, then [G] denominators
+  float* den_g = wl + p.parts * G;
+  const int64_t first_row = (int64_t)item * p.parts * G;
+  const __amdgpu_buffer_rsrc_t rl = make_rsrc(p.ws_plse + first_row, p.parts * G * (int)sizeof(float));
+  for (int i = tid; i < p.parts * G; i += NT)
+    wl[i] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rl, i * 4, 0, kDeviceScope));
+  __syncthreads();
+  if (tid < G) {
     float mm = kNegInf;
-    for (int sp = 0; sp < p.parts; ++sp)
-      mm = fmaxf(mm, __uint_as_float(__hip_atomic_load(p.ws_plse + row0 + (int64_t)sp * G, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
+    for (int sp = 0; sp < p.parts; ++sp) mm = fmaxf(mm, wl[sp * G + tid]);
     const float m_safe = (mm == kNegInf) ? 0.f : mm;
-    float num = 0.f, den = 0.f;
+    float den = 0.f;
     for (int sp = 0; sp < p.parts; ++sp) {
-      const int64_t row = row0 + (int64_t)sp * G;
-      const float wgt = fast_exp2(__uint_as_float(__hip_atomic_load(p.ws_plse + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) - m_safe);
-      num += __uint_as_float(__hip_atomic_load(p.ws_po + row * kHeadDim + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) * wgt;
+      const float wgt = fast_exp2(wl[sp * G + tid] - m_safe);
+      wl[sp * G + tid] = wgt;
       den += wgt;
     }
+    den_g[tid] = den;
+    if (p.lse) p.lse[hq0 + tid] = (den > 0.f) ? (mm + fast_log2(den)) * kLn2 : kNegInf;
+  }
+  __syncthreads();
+  const __amdgpu_buffer_rsrc_t ro = make_rsrc(p.ws_po + first_row * kHeadDim, p.parts * G * kHeadDim * (int)sizeof(float));
+  for (int idx = tid; idx < G * kHeadDim; idx += NT) {
+    const int g = idx >> 7, d = idx & (kHeadDim - 1);
+    float num = 0.f;
+#pragma unroll 8
+    for (int sp = 0; sp < p.parts; ++sp)
+      num += __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ro, ((sp * G + g) * kHeadDim + d) * 4, 0, kDeviceScope)) *
+             wl[sp * G + g];
+    const float den = den_g[g];
     p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(den > 0.f ? num / den : 0.f);
-    if (p.lse && d == 0) p.lse[hq0 + g] = (den > 0.f) ? (mm + fast_log2(den)) * kLn2 : kNegInf;
   }
 }
 
