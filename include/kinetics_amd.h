@@ -296,8 +296,8 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  * to finish merges the partial results, or -- very long sequences -- each
  * scores a part of the candidates.  Any of this changes only the fp32 summation
  * order of the output, not the page lists or cache bytes.  At least as fast as
- * the three calls except for few lists of more than 4096 pages with topk >= 512
- * and for 257..349 lists with topk > 768 (up to 1.6x and 1.2x slower).
+ * the three calls except for few lists of more than 4096 pages with topk >= 256
+ * and for 257..349 lists with topk > 768 (up to 1.3x and 1.2x slower).
  */
 int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
                               kin_bf16_t* kv_cache, kin_bf16_t* kbar,

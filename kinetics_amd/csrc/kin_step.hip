@@ -276,11 +276,12 @@ static size_t parts_workspace_bytes(int64_t items, int parts, int group) {
 // 64 lists x 4 parts of k = 128 pages: 48 us against 46 in 2 parts and 47 whole; a launch
 // that fills every CU wants longer lists still: 128 lists x 2 parts lose 6 % at k = 128
 // and gain 5 % at k = 512).  Every part
-// scores the whole list for itself, ~7 ns per mean key on one CU, where split scoring takes a
+// scores the whole list for itself, ~7 ns per mean key on one CU (more once over 128
+// workgroups pull whole lists through HBM at the same time), where split scoring takes a
 // few us for any length; a tile costs the lone attending workgroup ~0.15 us.  So where the
 // shape could split its scoring instead, parts are taken only if they save more attention
-// than the repeated scoring costs (8 lists of 4097 pages, k = 512: 63 us in parts, 103 us
-// with split scoring; k = 128: 49 against 42).
+// than the repeated scoring costs (8 lists of 4097 pages, k = 512: 59 us in parts, 103 us
+// with split scoring; k = 128: 49 against 43; one list of 2049 pages, k = 128: 30 against 37).
 static StepPlan plan_step(int batch, int num_kv_heads, int group, int kbar_pages, int64_t list_tiles, size_t avail) {
   const int64_t items = (int64_t)batch * num_kv_heads;
   StepPlan plan{1, 1, 0};
@@ -296,7 +297,10 @@ static StepPlan plan_step(int batch, int num_kv_heads, int group, int kbar_pages
     if (parts < 1) parts = 1;
   }
   const bool chunks_fit = chunks > 1 && score_workspace_bytes(items, kbar_pages) <= avail;
-  if (parts > 1 && chunks_fit && 12 * (list_tiles - list_tiles / parts) <= kbar_pages) parts = 1;
+  if (parts > 1 && chunks_fit) {
+    const int64_t groups = items * parts;  // workgroups that would each score a whole list
+    if (24 * (list_tiles - list_tiles / parts) * 128 <= (int64_t)kbar_pages * (groups > 128 ? groups : 128)) parts = 1;
+  }
   if (parts > 1) {
     plan.parts = (int)parts;
     plan.need = parts_workspace_bytes(items, plan.parts, group);

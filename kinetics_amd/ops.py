@@ -377,16 +377,16 @@ def prefer_fused_step(batch: int, num_kv_heads: int, max_pages_per_seq: int, top
     are few (split attention up to 128 lists, split scoring for very long
     sequences).  Measured on MI355X against the three launches queued back to back
     (fused / three): 1..128 lists of 2049 pages, k = 128..2048: 0.84..1.04; of 257
-    pages: 0.5; 8..32 lists of 8193 pages: k = 128 0.94, k = 512 1.3..1.6, k = 2048
-    1.05..1.15 (every part would score 2 MiB of mean keys for itself, so the step
-    splits the scoring instead and one workgroup attends alone); 200..256 lists
+    pages: 0.5; 8..32 lists of 4097..8193 pages: k = 128 0.96..1.02, k = 256..512
+    1.1..1.3, k = 2048 1.13 (scoring a whole list in every part costs as much as
+    the parts save); 200..256 lists
     0.95..0.98; 260..300 lists k <= 768 0.96..0.98, k = 1024 1.17..1.20 (some CUs hold
     two long lists, the others one); 350 lists and more 0.96..1.00.  Hence: fused,
-    except few lists of more than 4096 pages with k >= 512, and 257..349 lists with
+    except few lists of more than 4096 pages with k >= 256, and 257..349 lists with
     k > 768."""
     lists = batch * num_kv_heads
     if lists < 160:
-        return not (max_pages_per_seq > 4096 and topk >= 512)
+        return not (max_pages_per_seq > 4096 and topk >= 256)
     if 256 < lists < 350:
         return topk <= 768
     return True

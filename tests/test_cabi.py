@@ -262,7 +262,7 @@ def test_path_preference_rule():
     from kinetics_amd import ops
     assert ops.prefer_fused_step(8, 1, 257, 64) and ops.prefer_fused_step(1, 8, 2049, 2048)
     assert ops.prefer_fused_step(64, 1, 2049, 512) and ops.prefer_fused_step(100, 1, 2049, 1024)
-    assert ops.prefer_fused_step(8, 1, 8193, 128) and not ops.prefer_fused_step(8, 1, 8193, 512)
+    assert ops.prefer_fused_step(8, 1, 8193, 128) and not ops.prefer_fused_step(8, 1, 8193, 256)
     assert not ops.prefer_fused_step(32, 1, 4097, 2048)
     assert ops.prefer_fused_step(256, 1, 1025, 64) and ops.prefer_fused_step(200, 1, 4097, 2048)
     assert ops.prefer_fused_step(300, 1, 2049, 768) and not ops.prefer_fused_step(300, 1, 2049, 1024)
