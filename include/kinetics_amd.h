@@ -321,8 +321,9 @@ int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const ki
  * the selector may instead spread the scoring of a list over several workgroups
  * that meet through this memory (4 bytes per candidate page).  An arrival
  * counter per list comes first; contents need no initialisation and are of no
- * use afterwards.  Passing NULL or too little is allowed: a list is then shared
- * by fewer workgroups, or walked by a single one as for every other shape.
+ * use afterwards; launches that overlap in time must not share a workspace.
+ * Passing NULL or too little is allowed: a list is then shared by fewer
+ * workgroups, or walked by a single one as for every other shape.
  */
 size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages);
 
