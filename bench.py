@@ -285,6 +285,7 @@ def cpu_model_name():
 
 
 LAST_LAUNCH_MS = []
+LAST_GRAPH_REPLAY_MS = None
 
 
 @contextlib.contextmanager
@@ -302,10 +303,44 @@ def collector_paused():
             gc.enable()
 
 
+GRAPH_REPLAY_BELOW_MS = 0.1   # steps shorter than this are host-bound when launched eagerly
+
+
+def time_graph_replay(torch, step, steps, warmup):
+    """The step captured once as a HIP graph and replayed: what the GPU does when
+    the host is out of the way (the launch-overhead half of the reference's
+    torch.compile(mode="max-autotune"), benchmark/blocktopk.py:41-43).  All ``steps``
+    replays are queued back to back between two synchronisations; ms per step."""
+    cur = torch.cuda.current_stream()
+    side = torch.cuda.Stream()
+    side.wait_stream(cur)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        step()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    cur.wait_stream(side)
+    torch.cuda.synchronize()
+    with collector_paused():
+        for _ in range(warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+    del graph
+    return dt * 1e3
+
+
 def time_step(torch, ops, st, B, Hkv, topk, steps, warmup, mode="auto"):
     """W untimed and K timed decode steps on the state ``st``; HIP events on the
     launch stream bracket every kernel.  Returns (ms_per_step, elapsed_s,
-    {kernel: mean ms}, fused?)."""
+    {kernel: mean ms}, fused?).  When the eager step is shorter than
+    GRAPH_REPLAY_BELOW_MS, LAST_GRAPH_REPLAY_MS also holds the same step replayed
+    as a HIP graph (None otherwise)."""
     device = st["q"].device
     fused = mode == "fused" or (mode == "auto" and ops.prefer_fused_step(B, Hkv, st["max_pages_used"], topk))
     # few long lists: the scoring of a list is shared by several workgroups that meet through this
@@ -343,8 +378,14 @@ def time_step(torch, ops, st, B, Hkv, topk, steps, warmup, mode="auto"):
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
     kernel_ms = {name: statistics.fmean(e[j].elapsed_time(e[j + 1]) for e in ev) for j, (name, _) in enumerate(kernels)}
-    global LAST_LAUNCH_MS
+    global LAST_LAUNCH_MS, LAST_GRAPH_REPLAY_MS
     LAST_LAUNCH_MS = [round(sum(e[j].elapsed_time(e[j + 1]) for j in range(len(kernels))), 3) for e in ev]
+    LAST_GRAPH_REPLAY_MS = None
+    if elapsed / K * 1e3 < GRAPH_REPLAY_BELOW_MS:
+        def whole_step():
+            for _, fn in kernels:
+                fn()
+        LAST_GRAPH_REPLAY_MS = time_graph_replay(torch, whole_step, K, warmup)
     return elapsed / K * 1e3, elapsed, kernel_ms, fused
 
 
@@ -417,7 +458,8 @@ def side_workload(torch, ops, name, steps, warmup, device, with_dense=True):
     ms_step, elapsed, kernel_ms, fused = time_step(torch, ops, st, B, Hkv, topk, steps, warmup)
     print(f"[bench] {name}: kv at {hex(st['kv'].data_ptr())}, kbar at {hex(st['kbar'].data_ptr())}, "
           f"{torch.cuda.memory_allocated() / 1e9:.1f} GB allocated, {torch.cuda.memory_reserved() / 1e9:.1f} GB reserved, "
-          f"step {ms_step:.4f} ms, launches {min(LAST_LAUNCH_MS):.3f}..{max(LAST_LAUNCH_MS):.3f} ms", file=sys.stderr, flush=True)
+          f"step {ms_step:.4f} ms, launches {min(LAST_LAUNCH_MS):.3f}..{max(LAST_LAUNCH_MS):.3f} ms "
+          f"(first five {LAST_LAUNCH_MS[:5]}, last five {LAST_LAUNCH_MS[-5:]})", file=sys.stderr, flush=True)
     ab = algorithmic_bytes(st["lengths"], Hkv, G, topk)
     out = {"description": desc, "batch": B, "ctx": ctx, "num_kv_heads": Hkv, "num_q_heads": Hkv * G, "topk_pages": topk,
            "page_table": "ragged, half fragmented" if name in RAGGED else "reference layout p*B+b",
@@ -425,6 +467,10 @@ def side_workload(torch, ops, name, steps, warmup, device, with_dense=True):
            "steps": steps, "warmup": warmup, "ms_per_step": ms_step, "value": B * steps / elapsed, "unit": "tokens/s",
            "kernels_ms": kernel_ms, "algorithmic_bytes_per_step": ab["step"],
            "achieved_gbs": ab["step"] / (ms_step * 1e-3) / 1e9, "frac": ab["step"] / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    if LAST_GRAPH_REPLAY_MS is not None:
+        # a step this short is host-bound when launched eagerly: the same launches replayed as one HIP graph
+        out["graph_replay_ms_per_step"] = LAST_GRAPH_REPLAY_MS
+        out["graph_replay_frac"] = ab["step"] / (LAST_GRAPH_REPLAY_MS * 1e-3) / 1e9 / HBM_PEAK_GBS
     if fused:
         out["kernel_frac"] = ab["step"] / (kernel_ms["fused_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS
         tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
@@ -600,6 +646,9 @@ def main():
                      "unit": "GB/s", "frac": step_gbs / HBM_PEAK_GBS},
         "kernels_ms": kernel_ms,
     }
+    if LAST_GRAPH_REPLAY_MS is not None:
+        result["graph_replay_ms_per_step"] = LAST_GRAPH_REPLAY_MS
+        result["graph_replay_frac"] = ab["step"] / (LAST_GRAPH_REPLAY_MS * 1e-3) / 1e9 / HBM_PEAK_GBS
     if world:
         # the figure benchmark/blocktopk.py:82 prints divides the per-layer rate by world_size * num_hidden_layers;
         # it is built from the attention step alone here (the whole layer: --whole-layer)
@@ -631,7 +680,10 @@ def main():
     if side:
         # every other BASELINE configuration in the same run, each on its own freshly built cache
         # (carved from the blocks the headline cache has just left in the allocator)
-        ks, ws = max(5, K), max(3, min(args.warmup, 10))
+        # whatever --steps / --warmup the headline was given: at least 100 timed steps after at least 20
+        # warm-ups each (they cost under 0.1 s per workload; the reference warms up 200 times,
+        # benchmark/blocktopk.py:49)
+        ks, ws = max(100, K), max(20, args.warmup)
         result["workloads"] = {name: side_workload(torch, ops, name, ks, ws, device)
                                for name in ("qwen3-8b-tp1", "qwen3-0.6b-mix", "qwen3-32b-share", "qwen3-8b-readme", "tiny")}
         torch.cuda.empty_cache()
