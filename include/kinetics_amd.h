@@ -75,7 +75,11 @@ enum kin_status {
  * tokens, float16 twins (kin_*_f16), groups of up to 16 query heads per KV head,
  * the page pool and kin_blocktopk_decode_step_static.  2.1.0: the decode step
  * attends few lists in parts (kin_step_workspace_bytes grows to up to 2.1 MB for
- * up to 128 lists; KIN_STATIC_SCRATCH_BYTES grows by 32 KiB less 256 B). */
+ * up to 128 lists; KIN_STATIC_SCRATCH_BYTES grows by 32 KiB less 256 B).  2.2.0:
+ * few lists are handled by teams of workgroups that share the scoring and the
+ * attention (kin_step_workspace_bytes covers keys and partial results;
+ * KIN_STATIC_SCRATCH_BYTES doubles); without sel_pages the step attends the
+ * winners in index order. */
 int kin_version(void);
 
 /* Human-readable text of the last non-OK status on the calling thread
@@ -290,14 +294,20 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  * kin_block_score_topk, first_page_offset as in kin_sparse_paged_decode (a
  * non-zero offset requires sink_pages >= 1: a padded page has no valid mean
  * key); lse is optional.  One workgroup walks a whole list, of 8 waves instead
- * of 4 with 256 lists or fewer; with lists for under half the GPU's compute
- * units and a workspace (optional, see kin_step_workspace_bytes), several
- * workgroups share a list: each attends a part of the listed pages and the last
- * to finish merges the partial results, or -- very long sequences -- each
- * scores a part of the candidates.  Any of this changes only the fp32 summation
- * order of the output, not the page lists or cache bytes.  At least as fast as
- * the three calls except for few lists of more than 4096 pages with topk >= 256
- * and for 257..349 lists with topk > 768 (up to 1.3x and 1.2x slower).
+ * of 4 with 256 lists or fewer; with lists for at most a third of the GPU's
+ * compute units (half, for page lists of 384 tiles of 16 tokens or more) and a
+ * workspace (optional, see kin_step_workspace_bytes), a team of workgroups
+ * shares a list: each scores a slice of the candidates, the keys meet in the
+ * workspace, and the members each select for themselves (identical results),
+ * attend a part of the listed pages and leave a partial result that the last to
+ * finish merges.  A member waits for its team's keys for a bounded time only
+ * and then scores the list alone, so the launch never depends on which
+ * workgroups run at the same time.  Without sel_pages the winners are attended
+ * in index order instead of score order (no sort).  Any of this changes only the
+ * fp32 summation order of the output, not the page lists or cache bytes.  At
+ * least as fast as the three calls except for few lists of more than 4096 pages
+ * with topk >= 256 and for 257..349 lists with topk > 768 (up to 1.3x and 1.2x
+ * slower).
  */
 int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
                               kin_bf16_t* kv_cache, kin_bf16_t* kbar,
@@ -315,13 +325,14 @@ int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const ki
 /*
  * Workspace kin_blocktopk_decode_step and kin_block_score_topk can use for the
  * given problem: 0 unless the lists are few.  Up to 128 lists (batch *
- * num_kv_heads) the step may attend a list in parts, by several workgroups that
- * leave partial results here (up to 256 workgroups x 16 heads x 129 floats:
- * 2.1 MB at most); up to 64 lists of 2048 candidate pages or more, the step and
- * the selector may instead spread the scoring of a list over several workgroups
- * that meet through this memory (4 bytes per candidate page).  An arrival
- * counter per list comes first; contents need no initialisation and are of no
- * use afterwards; launches that overlap in time must not share a workspace.
+ * num_kv_heads) the step may hand a list to a team of workgroups that meet
+ * through this memory: two arrival counters per list, 4 bytes per candidate
+ * page and list for the keys, and the partial results of the members that
+ * attend (up to 256 workgroups x 16 heads x 129 floats: 2.1 MB at most); the
+ * figure returned covers any group size and page budget.  Up to 64 lists of
+ * 2048 candidate pages or more the selector spreads the scoring of a list over
+ * several workgroups the same way.  Contents need no initialisation and are of
+ * no use afterwards; launches that overlap in time must not share a workspace.
  * Passing NULL or too little is allowed: a list is then shared by fewer
  * workgroups, or walked by a single one as for every other shape.
  */
@@ -341,17 +352,17 @@ size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages);
  * the array's address up (hipGetSymbolAddress, with that device current; make
  * that call outside graph capture); the stream must belong to the current
  * device.
- * Limit: shapes that split their scoring and would need more than
- * KIN_STATIC_SCRATCH_BYTES for it are rejected with KIN_ERR_WORKSPACE -- the
- * array covers up to 524288 candidate pages in total over all such lists, e.g.
- * 64 lists of 8192 pages or 32 of 16384; split attention always fits; shapes
- * that share no list between workgroups (kin_step_workspace_bytes() returns 0)
- * never touch the array.
+ * Limit: shapes whose teams would need more than KIN_STATIC_SCRATCH_BYTES are
+ * rejected with KIN_ERR_WORKSPACE -- besides the partial results (2.1 MB at
+ * most) the array covers the keys of up to 524288 candidate pages in total over
+ * all lists, e.g. 64 lists of 8192 pages or 32 of 16384; shapes that share no
+ * list between workgroups (kin_step_workspace_bytes() returns 0) never touch
+ * the array.
  * All calls on one GPU share the array: calls that overlap in time on the same
  * GPU (different streams, or different threads) race and must be serialised by
  * the caller; calls in one stream are ordered by the stream.
  */
-#define KIN_STATIC_SCRATCH_BYTES (2u * 1024u * 1024u + 32u * 1024u)
+#define KIN_STATIC_SCRATCH_BYTES (4u * 1024u * 1024u + 64u * 1024u)
 
 size_t kin_static_scratch_bytes(void);
 

@@ -475,4 +475,49 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
   attend_finish<NG, NW>(m_run, l_run, O, G, lds, sm_m, sm_l, emit);
 }
 
+// Merges the `parts` partial results that the workgroups sharing one list left in
+// global memory (ws_po [lists, parts, G, 128] normalised outputs, ws_plse [lists, parts, G]
+// base-2 log-sum-exps, both fp32 bits written at device scope) and writes the list's G output
+// rows (out_bh) and, if lse_bh is set, their natural-log log-sum-exps.  Run by the workgroup
+// that counted in last, all NT threads; lds: room for (parts + 1) * G floats, free for reuse.
+// The log-sum-exps first become weights in LDS, then every thread sums its output element over
+// the parts with independent device-scope loads (the arithmetic of merge_splits_kernel).
+template <int NT, bool F16>
+__device__ __forceinline__ void merge_list_parts(unsigned char* lds, const uint32_t* ws_po, const uint32_t* ws_plse, int item,
+                                                 int parts, int G, uint16_t* out_bh, float* lse_bh) {
+  const int tid = threadIdx.x;
+  float* wl = reinterpret_cast<float*>(lds);  // [parts][G] weights, then [G] denominators
+  float* den_g = wl + parts * G;
+  const int64_t first_row = (int64_t)item * parts * G;
+  const __amdgpu_buffer_rsrc_t rl = make_rsrc(ws_plse + first_row, parts * G * (int)sizeof(float));
+  for (int i = tid; i < parts * G; i += NT)
+    wl[i] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rl, i * 4, 0, kDeviceScope));
+  __syncthreads();
+  if (tid < G) {
+    float mm = kNegInf;
+    for (int sp = 0; sp < parts; ++sp) mm = fmaxf(mm, wl[sp * G + tid]);
+    const float m_safe = (mm == kNegInf) ? 0.f : mm;
+    float den = 0.f;
+    for (int sp = 0; sp < parts; ++sp) {
+      const float wgt = fast_exp2(wl[sp * G + tid] - m_safe);
+      wl[sp * G + tid] = wgt;
+      den += wgt;
+    }
+    den_g[tid] = den;
+    if (lse_bh) lse_bh[tid] = (den > 0.f) ? (mm + fast_log2(den)) * kLn2 : kNegInf;
+  }
+  __syncthreads();
+  const __amdgpu_buffer_rsrc_t ro = make_rsrc(ws_po + first_row * kHeadDim, parts * G * kHeadDim * (int)sizeof(float));
+  for (int idx = tid; idx < G * kHeadDim; idx += NT) {
+    const int g = idx >> 7, d = idx & (kHeadDim - 1);
+    float num = 0.f;
+#pragma unroll 8
+    for (int sp = 0; sp < parts; ++sp)
+      num += __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ro, ((sp * G + g) * kHeadDim + d) * 4, 0, kDeviceScope)) *
+             wl[sp * G + g];
+    const float den = den_g[g];
+    out_bh[g * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(den > 0.f ? num / den : 0.f);
+  }
+}
+
 }  // namespace kin

@@ -176,6 +176,23 @@ __device__ __forceinline__ float row16_sum(float x) {
   return x;
 }
 
+// Inclusive prefix sum over the 64 lanes of a wave on the DPP path (no LDS crossbar: about a
+// tenth of the latency of six ds_bpermute steps): inside each row of 16 lanes by shifts of
+// 1, 2, 3, then 4 and 8, then lane 15 of rows 0 and 2 is added to rows 1 and 3, and lane 31
+// to rows 2 and 3.  A lane without a source takes 0.
+template <int CTRL, int ROW_MASK, int BANK_MASK>
+__device__ __forceinline__ uint32_t dpp_or_zero(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, ROW_MASK, BANK_MASK, false);
+}
+__device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t x) {
+  uint32_t s = x + dpp_or_zero<0x111, 0xf, 0xf>(x) + dpp_or_zero<0x112, 0xf, 0xf>(x) + dpp_or_zero<0x113, 0xf, 0xf>(x);  // row_shr:1..3
+  s += dpp_or_zero<0x114, 0xf, 0xe>(s);  // row_shr:4 into lanes 4..15 of each row
+  s += dpp_or_zero<0x118, 0xf, 0xc>(s);  // row_shr:8 into lanes 8..15
+  s += dpp_or_zero<0x142, 0xa, 0xf>(s);  // row_bcast:15 into rows 1 and 3
+  s += dpp_or_zero<0x143, 0xc, 0xf>(s);  // row_bcast:31 into rows 2 and 3
+  return s;
+}
+
 // Value of lane (quad base + I) broadcast to the 4 lanes of each quad.
 template <int I>
 __device__ __forceinline__ float quad_bcast(float x) {
@@ -195,6 +212,38 @@ static __global__ __attribute__((unused)) void fill_zero_i32_kernel(int32_t* p, 
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0;
 }
+
+#ifdef KIN_TUNE
+// Phase stamps of experimental builds: per workgroup up to 64 (tag, 100 MHz clock) pairs, in arrays
+// private to the translation unit.
+static __device__ long long g_stamps[1024 * 64 * 2];
+static __device__ int g_nstamps[1024];
+#define KIN_STAMP(tag)                                                          \
+  do {                                                                          \
+    if (threadIdx.x == 0 && blockIdx.x < 1024) {                                \
+      const int k_ = g_nstamps[blockIdx.x];                                     \
+      if (k_ < 64) {                                                            \
+        g_stamps[(blockIdx.x * 64 + k_) * 2] = (tag);                           \
+        g_stamps[(blockIdx.x * 64 + k_) * 2 + 1] = wall_clock64();              \
+        g_nstamps[blockIdx.x] = k_ + 1;                                         \
+      }                                                                         \
+    }                                                                           \
+  } while (0)
+#define KIN_STAMP_RESET()                                                       \
+  do {                                                                          \
+    if (threadIdx.x == 0 && blockIdx.x < 1024) g_nstamps[blockIdx.x] = 0;       \
+  } while (0)
+#define KIN_STAMP_ACCESSOR(fn_name)                                                                                          \
+  extern "C" int fn_name(long long* stamps, int* counts) {                                                                  \
+    if (hipDeviceSynchronize() != hipSuccess) return 1;                                                                      \
+    if (hipMemcpyFromSymbol(stamps, HIP_SYMBOL(kin::g_stamps), sizeof(long long) * 1024 * 64 * 2) != hipSuccess) return 2;   \
+    if (hipMemcpyFromSymbol(counts, HIP_SYMBOL(kin::g_nstamps), sizeof(int) * 1024) != hipSuccess) return 3;                 \
+    return 0;                                                                                                                \
+  }
+#else
+#define KIN_STAMP(tag) do { } while (0)
+#define KIN_STAMP_RESET() do { } while (0)
+#endif
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }

@@ -20,17 +20,21 @@ struct ScoreTopkParams {
   int batch, num_q_heads, num_kv_heads, group;
   int kbar_pages, sel_stride, topk, sink_pages, local_tokens, page_size;
   int sort_cap;
+  int table_cap;       // LDS entries for the copy of a sequence's page table (0: none)
   int chunks;          // workgroups per list
   int32_t* ws_count;   // [lists] arrival counters, zero at launch and left zero
   uint32_t* ws_keys;   // [lists, score_key_stride(kbar_pages)]
 };
 
-// Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap] | int32 sel[sink + topk + local]
+// Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap] | int32 table[table_cap] |
+// int32 sel[sink + topk + local]
 template <int UNROLL, bool F16>
 __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ int sh_last;
+  __shared__ SelectScratch ss;
   const int tid = threadIdx.x;
+  clear_select_scratch<kThreads>(&ss);
   const int list_id = blockIdx.x / p.chunks, chunk = blockIdx.x - list_id * p.chunks;
   int b, h;
   if (!xcd_list_of(list_id, p.batch, p.num_kv_heads, b, h)) return;
@@ -45,8 +49,9 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
     if (tid == 0) p.sel_count[item] = 0;
     return;
   }
-  const size_t sel_off = select_lds_bytes(p.kbar_pages, p.sort_cap);
+  const size_t sel_off = select_lds_bytes(p.kbar_pages, p.sort_cap, p.table_cap);
   int32_t* sel_lds = reinterpret_cast<int32_t*>(smem + sel_off);
+  int32_t* table_lds = reinterpret_cast<int32_t*>(smem + select_table_offset(p.kbar_pages, p.sort_cap));
 
   SelectArgs a;
   a.q_bh = p.q + ((int64_t)b * p.num_q_heads + (int64_t)h * p.group) * kHeadDim;
@@ -61,6 +66,10 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
   a.keys = reinterpret_cast<uint32_t*>(smem);
   a.sortbuf = reinterpret_cast<unsigned long long*>(smem + (size_t)((p.kbar_pages + 3) & ~3) * 4);
   a.sort_cap = p.sort_cap;
+  a.ss = &ss;
+  a.table_lds = nullptr;
+  a.digit0_counted = false;
+  a.sorted = true;
   int n_list;
   if (p.chunks > 1) {
     // This workgroup's slice of the candidates -> keys in global memory, written and
@@ -79,10 +88,14 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
     __syncthreads();
     if (!sh_last) return;
     if (tid == 0) __hip_atomic_store(&p.ws_count[item], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+    a.table_lds = prefetch_table<kThreads>(a.table, n_pages, table_lds, p.table_cap);
     load_shared_keys<kThreads>(gkeys, n_score, a.keys);
+    __builtin_amdgcn_s_waitcnt(0);  // the table copy has landed too
     __syncthreads();
     n_list = select_from_keys<kThreads>(a, sel_lds);
   } else {
+    a.table_lds = prefetch_table<kThreads>(a.table, n_pages, table_lds, p.table_cap);
+    __syncthreads();  // histograms zeroed
     n_list = score_select<UNROLL, kThreads, F16>(a, sel_lds);
   }
 
@@ -139,7 +152,8 @@ static int score_topk_impl(const char* fn, bool f16, const uint16_t* q, const ui
   p.local_tokens = local_tokens;
   p.page_size = page_size;
   p.sort_cap = select_sort_cap(topk, kbar_pages);
-  const size_t lds = select_lds_bytes(kbar_pages, p.sort_cap) + (size_t)list_cap * 4;
+  p.table_cap = select_table_cap(kbar_pages + max_local_pages(local_tokens) + 1);
+  const size_t lds = select_lds_bytes(kbar_pages, p.sort_cap, p.table_cap) + (size_t)list_cap * 4;
   const int64_t items = (int64_t)batch * num_kv_heads;
   if (xcd_grid_size(batch, num_kv_heads) > 0x7fffffffLL)
     return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);

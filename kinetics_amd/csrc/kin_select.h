@@ -6,11 +6,15 @@
 //            16 lanes per key with 16-byte loads, fp32 dot with the group-mean
 //            query, DPP reduction inside each 16-lane row; scores stay in LDS
 //            as order-preserving 32-bit keys (never written to HBM);
-//   phase 2  4-pass 8-bit radix select in LDS for the k-th largest key;
+//   phase 2  8-bit radix select in LDS for the k-th largest key (the first digit
+//            is counted while the scores are produced);
 //   phase 3  gather the winners (ties at the threshold by lowest index), order
 //            them (score descending, index ascending) in LDS -- by counting for
 //            k <= 512, by bitonic sort above -- translate logical -> physical
-//            page ids and append the last page.
+//            page ids and append the last page.  The sequence's page table is
+//            copied to LDS while the mean keys stream, so the translation costs
+//            no memory round trip (under a saturated read stream a dependent
+//            global load takes microseconds).
 // HBM-bound on phase 1: n_cand * 256 B per workgroup.
 #pragma once
 
@@ -29,6 +33,21 @@ __device__ __forceinline__ uint32_t order_key(float f) {
 constexpr int kThreads = 256;  // workgroup size of the stand-alone selector
 constexpr int kRankSortMax = 512;   // up to here winners are ordered by counting, above by bitonic sort
 
+// Statically allocated LDS of one selection problem (one per workgroup).
+struct SelectScratch {
+  uint32_t hist[4][256];  // one histogram per radix digit; all zero when a selection starts (see clear_select_scratch)
+  uint32_t wave_tot[16];
+  uint32_t count;
+  uint32_t run_cnt[kMaxCandidates / 64];  // winners in each run of 64 candidates (index-ordered listing)
+};
+
+// Zeroes the histograms.  Every thread of the workgroup calls it; the caller puts a
+// barrier between this and the first score_rows<..., COUNT0 = true> / select_from_keys().
+template <int NT>
+__device__ __forceinline__ void clear_select_scratch(SelectScratch* ss) {
+  for (int i = threadIdx.x; i < 4 * 256; i += NT) (&ss->hist[0][0])[i] = 0;
+}
+
 // Wave-uniform description of one selection problem.
 struct SelectArgs {
   const uint16_t* q_bh;       // the group's G query rows
@@ -45,10 +64,47 @@ struct SelectArgs {
   uint32_t* keys;             // LDS, >= n_cand entries
   unsigned long long* sortbuf;  // LDS, sort_cap entries
   int sort_cap;               // power of two >= min(topk, capacity)
+  SelectScratch* ss;          // LDS, histograms zeroed
+  bool sorted;                // list the winners by descending score (ties: ascending index) as torch.topk does; else by
+                              // ascending index, which needs no sort (the attention's sum does not care)
+  const int32_t* table_lds;   // LDS copy of table[0 .. n_pages) (see prefetch_table), or null: look up in global memory
+  bool digit0_counted;        // ss->hist[0] already holds the first digit of every candidate's key
 };
 
-__host__ __device__ inline size_t select_lds_bytes(int kbar_pages, int sort_cap) {
+// table_cap: entries reserved for the LDS copy of a page table (a multiple of 64, 0: none);
+// it follows the sort buffer.
+__host__ __device__ inline size_t select_lds_bytes(int kbar_pages, int sort_cap, int table_cap = 0) {
+  return (size_t)((kbar_pages + 3) & ~3) * 4 + (size_t)sort_cap * 8 + (size_t)table_cap * 4;
+}
+__host__ __device__ inline size_t select_table_offset(int kbar_pages, int sort_cap) {
   return (size_t)((kbar_pages + 3) & ~3) * 4 + (size_t)sort_cap * 8;
+}
+
+// Largest page table that is copied to LDS (16 KiB); longer sequences translate through global memory.
+constexpr int kMaxTableLds = 4096;
+// Entries to reserve so that every sequence of up to max_pages pages gets the copy, capped at
+// kMaxTableLds: a multiple of 64 (whole wave loads).  Whether a sequence fits is decided per sequence.
+__host__ __device__ inline int select_table_cap(int max_pages) {
+  const int want = (max_pages + 63) & ~63;
+  return want < kMaxTableLds ? want : kMaxTableLds;
+}
+
+// Starts the copy of table[0 .. n_pages) to dst (LDS, room for table_cap entries) with LDS-direct
+// loads (no registers are held while they are in flight) when n_pages fits; returns dst then, else
+// null.  Every thread of the workgroup calls it.  The data may be read after
+// every wave has waited for its loads (s_waitcnt vmcnt(0)) and a workgroup barrier.
+template <int NT>
+__device__ __forceinline__ const int32_t* prefetch_table(const int32_t* table, int n_pages, int32_t* dst, int table_cap) {
+  if (n_pages > table_cap || n_pages <= 0) return nullptr;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const __amdgpu_buffer_rsrc_t r = make_rsrc(table, n_pages * 4);   // past the end: zeros, no traffic
+  const int chunks = (n_pages + 63) >> 6;                            // 64 entries = 256 B per wave load
+  for (int c = wave; c < chunks; c += NT / 64) {
+    __attribute__((address_space(3))) unsigned char* d =
+        (__attribute__((address_space(3))) unsigned char*)(dst + c * 64);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, d, 4, (c * 64 + lane) * 4, 0, 0, 0);
+  }
+  return dst;
 }
 
 __host__ __device__ inline int select_sort_cap(int topk, int kbar_pages) {
@@ -113,12 +169,7 @@ __device__ __forceinline__ void radix_pick_bin_uniform(const uint32_t* hist, uin
   const int top = 255 - 4 * lane;
   const uint32_t c0 = hist[top], c1 = hist[top - 1], c2 = hist[top - 2], c3 = hist[top - 3];
   const uint32_t mine = c0 + c1 + c2 + c3;
-  uint32_t incl = mine;
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const uint32_t up = __shfl_up(incl, off);
-    if (lane >= off) incl += up;
-  }
+  const uint32_t incl = wave_inclusive_sum(mine);
   uint32_t run = incl - mine;  // keys in bins above this lane's
   const bool owner = run < remaining && remaining <= incl;
   uint32_t bin = 0, rem = 0, cnt = 0;
@@ -134,9 +185,9 @@ __device__ __forceinline__ void radix_pick_bin_uniform(const uint32_t* hist, uin
   // exactly one lane owns the threshold bin (1 <= remaining <= number of counted keys)
   const unsigned long long who = __ballot(owner);
   const int src = who ? __builtin_ctzll(who) : 0;
-  bin_out = __shfl(bin, src);
-  remaining_out = __shfl(rem, src);
-  exhausted = __shfl(cnt, src) == remaining_out;
+  bin_out = (uint32_t)__builtin_amdgcn_readlane((int)bin, src);
+  remaining_out = (uint32_t)__builtin_amdgcn_readlane((int)rem, src);
+  exhausted = (uint32_t)__builtin_amdgcn_readlane((int)cnt, src) == remaining_out;
 }
 
 // Scores the candidates r0 <= r < r1 of one (sequence, KV head) with the
@@ -149,7 +200,9 @@ __device__ __forceinline__ void radix_pick_bin_uniform(const uint32_t* hist, uin
 // UNROLL: independent 16-byte loads each lane keeps in flight while streaming the
 // mean keys (4 saturates HBM when thousands of workgroups run; a small grid
 // needs more per workgroup).
-template <int UNROLL, int NT, bool DEVICE_VISIBLE = false, bool F16 = false>
+// COUNT0: also count every key's first radix digit in a.ss->hist[0] (LDS atomics spread
+// over the streaming, instead of a pass over the keys afterwards).
+template <int UNROLL, int NT, bool DEVICE_VISIBLE = false, bool F16 = false, bool COUNT0 = false>
 __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, uint32_t* keys_out) {
   constexpr int kUnroll = UNROLL;
   constexpr int kRows = NT / 16;  // mean keys one pass of the workgroup covers
@@ -207,10 +260,12 @@ __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, 
       acc = row16_sum(acc);
       const int row = base + j * kRows + sub;
       if (c16 == 0 && row < n) {
+        const uint32_t key = order_key(acc);
         if (DEVICE_VISIBLE)
-          __hip_atomic_store(keys_out + r0 + row, order_key(acc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(keys_out + r0 + row, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         else
-          keys_out[r0 + row] = order_key(acc);
+          keys_out[r0 + row] = key;
+        if (COUNT0) atomicAdd(&a.ss->hist[0][key >> 24], 1u);
         if (sc_out) sc_out[r0 + row] = acc;
       }
     }
@@ -241,14 +296,13 @@ __device__ __forceinline__ void load_shared_keys(const uint32_t* gkeys, int n, u
 // page list to sel_lds (LDS, >= n_sink + topk + n_local entries): the sink
 // pages, then the ordered physical ids of the k_eff winners, then the local
 // pages (the open page last).  Returns the list length.  The caller has put a
-// workgroup barrier between the last key write and this call; it ends with one:
+// workgroup barrier between the last key write (and the last count into
+// a.ss->hist[0], and the arrival of a.table_lds) and this call; it ends with one:
 // sel_lds is visible to every thread and keys / sortbuf are free for reuse.
+// a.ss->hist is left dirty: clear_select_scratch() before the next selection.
 template <int NT>
 __device__ __forceinline__ int select_from_keys(const SelectArgs& a, int32_t* sel_lds) {
-  __shared__ uint32_t hist[4][256];  // one histogram per radix digit, all zeroed up front
-  __shared__ uint32_t wave_tot[NT / 64];
-  __shared__ uint32_t sh_count;
-
+  SelectScratch& ss = *a.ss;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int n_cand = a.n_cand, n_pages = a.n_pages;
@@ -263,22 +317,23 @@ __device__ __forceinline__ int select_from_keys(const SelectArgs& a, int32_t* se
   uint32_t prefix = 0, mask = 0;
   uint32_t remaining = (uint32_t)k_eff;  // how many keys equal to the threshold are taken
   uint32_t thr = 0;
+  KIN_STAMP(20);  // select starts
   if (k_eff > 0 && k_eff < n_cand) {
-    for (int i = tid; i < 4 * 256; i += NT) (&hist[0][0])[i] = 0;
-    __syncthreads();
     bool whole_bin = false;
     for (int pass = 0; pass < 4 && !whole_bin; ++pass) {
       const int shift = 24 - 8 * pass;
-      for (int i = tid; i < n_cand; i += NT) {
-        const uint32_t key = keys[i];
-        if ((key & mask) == prefix) atomicAdd(&hist[pass][(key >> shift) & 255u], 1u);
+      if (pass > 0 || !a.digit0_counted) {
+        for (int i = tid; i < n_cand; i += NT) {
+          const uint32_t key = keys[i];
+          if ((key & mask) == prefix) atomicAdd(&ss.hist[pass][(key >> shift) & 255u], 1u);
+        }
+        __syncthreads();
       }
-      __syncthreads();
       uint32_t bin;
-      radix_pick_bin_uniform(hist[pass], remaining, lane, bin, remaining, whole_bin);
+      radix_pick_bin_uniform(ss.hist[pass], remaining, lane, bin, remaining, whole_bin);
       prefix |= bin << shift;
       mask |= 255u << shift;
-      if (shift == 0) whole_bin = false;  // all 32 bits fixed: `remaining` counts keys equal to the threshold
+      KIN_STAMP(21 + pass);  // digit fixed
     }
     if (whole_bin && prefix != 0) {
       // every key that starts with `prefix` is a winner: they all compare above prefix - 1,
@@ -286,49 +341,118 @@ __device__ __forceinline__ int select_from_keys(const SelectArgs& a, int32_t* se
       thr = prefix - 1u;
       remaining = 0;
     } else {
-      thr = prefix;
+      thr = prefix;  // all 32 bits fixed (or prefix 0): `remaining` of the keys equal to thr are taken
     }
   }
   const bool take_all = (k_eff >= n_cand);
+  // Logical -> physical page id: from the LDS copy of the table when there is one.  The copy is read
+  // through a pointer typed as LDS: through a generic pointer the loads would be flat instructions,
+  // which queue up behind the CU's global loads (microseconds under a saturated read stream).
+  typedef const __attribute__((address_space(3))) int32_t* lds_table_t;
+  const lds_table_t table_lds = (lds_table_t)a.table_lds;
+  const bool have_lds_table = a.table_lds != nullptr;
+  auto table = [&](int i) -> int32_t { return have_lds_table ? table_lds[i] : a.table[i]; };
+
+  if (!a.sorted) {
+    // ---- phase 3, listing by ascending index: an ordered compaction, no sort -------
+    // Wave w owns the runs of 64 consecutive candidates w, w + NT/64, ...; it counts each run's
+    // winners (low half: keys above the threshold; high half: keys equal to it), one wave turns
+    // the counts into offsets, and every wave writes its winners in place.  Of the keys equal
+    // to the threshold the `remaining` lowest-indexed count.
+    const int runs = (n_cand + 63) >> 6;
+    auto classify = [&](int i, bool& gt, bool& eq) {
+      const uint32_t key = i < n_cand ? keys[i] : 0u;
+      gt = i < n_cand && (take_all || key > thr);
+      eq = i < n_cand && !take_all && remaining > 0 && key == thr;
+    };
+    if (k_eff > 0) {
+      for (int r = wave; r < runs; r += NT / 64) {
+        bool gt, eq;
+        classify(r * 64 + lane, gt, eq);
+        const uint32_t c = (uint32_t)__popcll(__ballot(gt)) | ((uint32_t)__popcll(__ballot(eq)) << 16);
+        if (lane == 0) ss.run_cnt[r] = c;
+      }
+    }
+    __syncthreads();
+    if (k_eff > 0 && wave == 0) {
+      // exclusive prefix over the runs, 64 at a time (halves add without carry: at most 16384 candidates)
+      uint32_t carry = 0;
+      for (int r0 = 0; r0 < runs; r0 += 64) {
+        const uint32_t c = r0 + lane < runs ? ss.run_cnt[r0 + lane] : 0u;
+        const uint32_t incl = wave_inclusive_sum(c);
+        if (r0 + lane < runs) ss.run_cnt[r0 + lane] = carry + incl - c;
+        carry += (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+      }
+    }
+    __syncthreads();
+    if (k_eff > 0) {
+      for (int r = wave; r < runs; r += NT / 64) {
+        bool gt, eq;
+        const int i = r * 64 + lane;
+        classify(i, gt, eq);
+        const unsigned long long bg = __ballot(gt), be = __ballot(eq);
+        const uint32_t before = ss.run_cnt[r];
+        const uint32_t gt_before = (before & 0xffffu) + __builtin_amdgcn_mbcnt_hi((uint32_t)(bg >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bg, 0u));
+        const uint32_t eq_before = (before >> 16) + __builtin_amdgcn_mbcnt_hi((uint32_t)(be >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)be, 0u));
+        if (gt || (eq && eq_before < remaining))
+          sel_lds[a.n_sink + gt_before + min(eq_before, remaining)] = table(a.n_sink + i);
+      }
+    }
+    for (int i = tid; i < a.n_sink + a.n_local; i += NT) {
+      if (i < a.n_sink)
+        sel_lds[i] = table(i);
+      else
+        sel_lds[k_eff + i] = table(n_pages - a.n_local + (i - a.n_sink));
+    }
+    __syncthreads();
+    return k_eff + a.n_sink + a.n_local;
+  }
 
   // ---- phase 3: gather, sort, translate --------------------------------------
   const bool rank_sort = (k_eff <= kRankSortMax);
   if (!rank_sort)
     for (int i = tid; i < a.sort_cap; i += NT) sortbuf[i] = 0ull;
-  if (tid == 0) sh_count = 0;
+  if (tid == 0) ss.count = 0;
   __syncthreads();
   if (k_eff > 0) {
-    // Keys above the threshold: any order (the sort fixes it).
-    // Keys equal to it: the `remaining` lowest indices, found by an ordered count.
-    const int per = (n_cand + NT - 1) / NT;
-    const int lo = min(tid * per, n_cand), hi = min(lo + per, n_cand);
-    uint32_t eq_cnt = 0;
-    for (int i = lo; i < hi; ++i) {
-      const uint32_t key = keys[i];
-      if (take_all || key > thr) {
-        const uint32_t slot = atomicAdd(&sh_count, 1u);
-        sortbuf[slot] = ((unsigned long long)key << 32) | (uint32_t)(0xffffffffu - (uint32_t)i);
-      } else if (key == thr) {
-        eq_cnt++;
+    // Keys above the threshold (or all of them): any order, the sort fixes it.  One slot
+    // allocation per wave and step.
+    for (int base = 0; base < n_cand; base += NT) {
+      const int i = base + tid;
+      const uint32_t key = i < n_cand ? keys[i] : 0u;
+      const bool win = i < n_cand && (take_all || key > thr);
+      const unsigned long long bal = __ballot(win);
+      if (bal) {  // wave-uniform
+        uint32_t slot0 = 0;
+        if (lane == 0) slot0 = atomicAdd(&ss.count, (uint32_t)__popcll(bal));
+        slot0 = __shfl(slot0, 0);
+        const uint32_t before = __builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u));
+        if (win) sortbuf[slot0 + before] = ((unsigned long long)key << 32) | (uint32_t)(0xffffffffu - (uint32_t)i);
       }
     }
-    if (!take_all) {
-      // exclusive block scan of eq_cnt in thread order (== index order)
+    if (!take_all && remaining > 0) {
+      // Keys equal to the threshold: the `remaining` lowest indices, found by an ordered
+      // count (every thread owns a run of consecutive candidates).  Only reached when the
+      // threshold bin could not be taken whole, i.e. with exact ties at the threshold.
+      const int per = (n_cand + NT - 1) / NT;
+      const int lo = min(tid * per, n_cand), hi = min(lo + per, n_cand);
+      uint32_t eq_cnt = 0;
+      for (int i = lo; i < hi; ++i) eq_cnt += (keys[i] == thr) ? 1u : 0u;
       uint32_t incl = eq_cnt;
 #pragma unroll
       for (int off = 1; off < 64; off <<= 1) {
         const uint32_t up = __shfl_up(incl, off);
         if (lane >= off) incl += up;
       }
-      if (lane == 63) wave_tot[wave] = incl;
+      if (lane == 63) ss.wave_tot[wave] = incl;
       __syncthreads();
       uint32_t before = 0;
-      for (int wv = 0; wv < wave; ++wv) before += wave_tot[wv];
+      for (int wv = 0; wv < wave; ++wv) before += ss.wave_tot[wv];
       uint32_t rank = incl - eq_cnt + before;
       for (int i = lo; i < hi && rank < remaining; ++i) {
         const uint32_t key = keys[i];
         if (key == thr) {
-          const uint32_t slot = atomicAdd(&sh_count, 1u);
+          const uint32_t slot = atomicAdd(&ss.count, 1u);
           sortbuf[slot] = ((unsigned long long)key << 32) | (uint32_t)(0xffffffffu - (uint32_t)i);
           rank++;
         }
@@ -336,7 +460,7 @@ __device__ __forceinline__ int select_from_keys(const SelectArgs& a, int32_t* se
     }
   }
   __syncthreads();
-  const int32_t* table = a.table;
+  KIN_STAMP(25);  // winners gathered
   if (rank_sort) {
     // Small k: every winner counts the winners that beat it (entries are
     // distinct, so the counts are a permutation) and writes itself to that slot.
@@ -347,7 +471,7 @@ __device__ __forceinline__ int select_from_keys(const SelectArgs& a, int32_t* se
 #pragma unroll 8
       for (int j = 0; j < k_eff; ++j) rank += (sortbuf[j] > mine) ? 1 : 0;
       const uint32_t logical = 0xffffffffu - (uint32_t)(mine & 0xffffffffull);
-      sel_lds[a.n_sink + rank] = table[a.n_sink + logical];
+      sel_lds[a.n_sink + rank] = table(a.n_sink + logical);
       if (a.sel_logical) a.sel_logical[rank] = (int32_t)(a.n_sink + logical);
     }
   } else {
@@ -370,26 +494,33 @@ __device__ __forceinline__ int select_from_keys(const SelectArgs& a, int32_t* se
     }
     for (int i = tid; i < k_eff; i += NT) {
       const uint32_t logical = 0xffffffffu - (uint32_t)(sortbuf[i] & 0xffffffffull);
-      sel_lds[a.n_sink + i] = table[a.n_sink + logical];
+      sel_lds[a.n_sink + i] = table(a.n_sink + logical);
       if (a.sel_logical) a.sel_logical[i] = (int32_t)(a.n_sink + logical);
     }
   }
   for (int i = tid; i < a.n_sink + a.n_local; i += NT) {
     if (i < a.n_sink)
-      sel_lds[i] = table[i];
+      sel_lds[i] = table(i);
     else
-      sel_lds[k_eff + i] = table[n_pages - a.n_local + (i - a.n_sink)];
+      sel_lds[k_eff + i] = table(n_pages - a.n_local + (i - a.n_sink));
   }
   __syncthreads();
   return k_eff + a.n_sink + a.n_local;
 }
 
 // score_rows() over every candidate into a.keys, then select_from_keys().
+// a.ss->hist is zero and visible (clear_select_scratch + barrier); a.digit0_counted is
+// ignored: the first digit is always counted on the fly here.
 template <int UNROLL = 4, int NT = kThreads, bool F16 = false>
-__device__ __forceinline__ int score_select(const SelectArgs& a, int32_t* sel_lds) {
+__device__ __forceinline__ int score_select(SelectArgs& a, int32_t* sel_lds) {
   // Nothing to choose (topk == 0) and nobody asked for the scores: stream nothing.
   const int n_score = (min(a.topk, a.n_cand) > 0 || a.scores_out) ? a.n_cand : 0;
-  score_rows<UNROLL, NT, false, F16>(a, 0, n_score, a.keys);
+  score_rows<UNROLL, NT, false, F16, true>(a, 0, n_score, a.keys);
+  a.digit0_counted = true;
+  // the page-table copy (LDS-direct loads) has landed in every wave before anyone reads it
+  KIN_STAMP(18);  // this wave's scores are issued
+  __builtin_amdgcn_s_waitcnt(0);
+  KIN_STAMP(19);  // ... and have landed
   __syncthreads();
   return select_from_keys<NT>(a, sel_lds);
 }

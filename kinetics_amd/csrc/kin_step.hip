@@ -1,7 +1,9 @@
 // Fused decode step: append -> score -> select -> attend in ONE launch, one
 // workgroup of NW waves per (sequence, KV head): 4 waves when there are enough
-// lists to fill the GPU, 8 when there are few (one workgroup per CU).  With lists
-// for at most half the CUs, several workgroups share a list (see StepParams).
+// lists to fill the GPU, 8 when there are few (one workgroup per CU).  Lists that
+// would leave CUs idle -- few lists, a batch just above one list per CU, the last
+// lists of a batch a little larger than the GPU holds at once -- are handled by a
+// *team* of workgroups each (see StepParams).
 //
 // Compared with the three stand-alone kernels this removes two dependent
 // dispatches, the selector's drain (its last workgroups finish their LDS-only
@@ -11,45 +13,15 @@
 // optional outputs).  Same building blocks and arithmetic as the stand-alone
 // kernels: score_select() (kin_select.h) and attend_list() (kin_attend.h).
 #include <atomic>
+#include <cstdio>
+#include <cstdlib>
 
 #include "kin_append.h"
 #include "kin_attend.h"
 #include "kin_select.h"
+#include "kin_step.h"
 
 namespace kin {
-
-struct StepParams {
-  const uint16_t* q;
-  const uint32_t* k;  // new token's K/V rows as dwords; null = no append
-  const uint32_t* v;
-  uint16_t* kv;
-  uint16_t* kbar;
-  const int32_t* page_indices;
-  const int32_t* page_indptr;
-  const int32_t* last_page_len;
-  int32_t* sel_pages;  // optional HBM copy of the page lists
-  int32_t* sel_count;  // optional
-  uint16_t* out;
-  float* lse;  // optional
-  int batch, num_q_heads, num_kv_heads, group;
-  int kbar_pages, sel_stride, topk, sink_pages, local_tokens, first_page_offset, sort_cap, page_size;
-  int region0_bytes;  // LDS: max(attend staging, select scratch); the page list follows it
-  // Split scoring (few, long sequences): `chunks` workgroups per list score a slice of the
-  // candidates each into ws_keys; the last one to finish selects and attends.
-  int chunks;
-  int32_t* ws_count;   // [lists], zero at launch and left zero
-  uint32_t* ws_keys;   // [lists, score_key_stride(kbar_pages)]
-  // Split attention (lists for at most half the CUs): `parts` workgroups per list.  Each scores
-  // and selects the whole list for itself (identical results), attends its share of the listed
-  // pages and leaves a partial result; the last one to finish merges them.
-  int parts;
-  uint32_t* ws_po;    // [lists, parts, group, 128] fp32 bits: normalised partial outputs
-  uint32_t* ws_plse;  // [lists, parts, group] fp32 bits: base-2 log-sum-exp of the parts
-  int64_t num_pages;
-  float scale_log2;
-  int deep_score;      // few lists: more mean-key loads in flight per lane (see the kernel)
-  int rotate;          // attend_rotates(lists)
-};
 
 template <int NG, int NW, bool F16>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kernel(StepParams p) {
@@ -59,26 +31,37 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   constexpr int NT = NW * 64;
 
   __shared__ int sh_last;
+  __shared__ SelectScratch ss;
   const int tid = threadIdx.x;
-  int b, h, chunk = 0, part = 0;
-  if (p.chunks > 1 || p.parts > 1) {
-    const int per_list = p.chunks > 1 ? p.chunks : p.parts;
-    const int list = blockIdx.x / per_list;
-    const int sub = blockIdx.x - list * per_list;
-    if (p.chunks > 1) chunk = sub; else part = sub;
+  clear_select_scratch<NT>(&ss);
+  KIN_STAMP_RESET();
+  KIN_STAMP(0);
+  // The first head_blocks workgroups own a list each; behind them come the teams, `team`
+  // consecutive workgroups per list from list head_lists on.
+  int b, h, member = 0, team = 1, parts = 1;
+  if ((int)blockIdx.x >= p.head_blocks) {
+    const int i = blockIdx.x - p.head_blocks;
+    const int list = p.head_lists + i / p.team;
+    member = i - (i / p.team) * p.team;
+    team = p.team;
+    parts = p.parts;
     b = list / p.num_kv_heads;
     h = list - b * p.num_kv_heads;
-  } else if (!xcd_list_of(blockIdx.x, p.batch, p.num_kv_heads, b, h)) {
-    return;
+  } else if (p.head_lists == p.batch * p.num_kv_heads) {
+    if (!xcd_list_of(blockIdx.x, p.batch, p.num_kv_heads, b, h)) return;
+  } else {
+    b = blockIdx.x / p.num_kv_heads;
+    h = blockIdx.x - b * p.num_kv_heads;
   }
+  const int part = member;  // members 0 .. parts-1 also select and attend a share of the page list
   const int item = b * p.num_kv_heads + h;
   const int G = p.group;
   const int64_t hq0 = (int64_t)b * p.num_q_heads + (int64_t)h * G;
 
   const int ps = p.page_indptr[b], pe = p.page_indptr[b + 1];
   const int n_pages = pe - ps;
-  if (n_pages <= 0) {  // empty sequence: nothing to append, select or attend
-    if (chunk != 0 || part != 0) return;
+  if (n_pages <= 0) {  // empty sequence: nothing to append, select or attend (every member sees that)
+    if (member != 0) return;
     if (p.sel_pages)
       for (int i = tid; i < p.sel_stride; i += NT) p.sel_pages[(int64_t)item * p.sel_stride + i] = -1;
     if (p.sel_count && tid == 0) p.sel_count[item] = 0;
@@ -89,7 +72,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   const int last_len = p.last_page_len[b];
 
   // ---- append (wave 0): same byte moves and mean-key update as append_kernel ----
-  // With split scoring the workgroup that ends up attending does it (see below).
+  // In a team the member that attends the sequence's last page does it (see below).
   auto append_token = [&]() {
     if (p.k != nullptr && tid < 64) {
       uint32_t* kbar_row =
@@ -102,7 +85,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
       __threadfence_block();
     }
   };
-  if (p.chunks <= 1 && p.parts <= 1) append_token();
+  if (team == 1) append_token();
 
   // ---- score + select: page list into LDS -------------------------------------
   int32_t* sel_lds = reinterpret_cast<int32_t*>(smem + p.region0_bytes);
@@ -119,32 +102,59 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   s.keys = reinterpret_cast<uint32_t*>(smem);
   s.sortbuf = reinterpret_cast<unsigned long long*>(smem + (size_t)((p.kbar_pages + 3) & ~3) * 4);
   s.sort_cap = p.sort_cap;
+  s.ss = &ss;
+  s.table_lds = nullptr;
+  s.digit0_counted = false;
+  s.sorted = p.sel_pages != nullptr;
+  int32_t* table_lds = reinterpret_cast<int32_t*>(smem + select_table_offset(p.kbar_pages, p.sort_cap));
   int n;
-  if (p.chunks > 1) {
-    // This workgroup's slice of the candidates -> keys in HBM.
-    uint32_t* gkeys = p.ws_keys + (int64_t)item * score_key_stride(p.kbar_pages);
+  if (team > 1) {
+    // This member's slice of the candidates -> keys in HBM.
+    const int titem = item - p.head_lists;
+    uint32_t* gkeys = p.ws_keys + (int64_t)titem * score_key_stride(p.kbar_pages);
     const int n_score = min(s.topk, s.n_cand) > 0 ? s.n_cand : 0;
-    const int per = ((n_score + p.chunks - 1) / p.chunks + 63) & ~63;
-    const int r0 = min(chunk * per, n_score), r1 = min(r0 + per, n_score);
-    score_rows<4, NT, true, F16>(s, r0, r1, gkeys);
+    const int per = ((n_score + team - 1) / team + 63) & ~63;
+    const int r0 = min(member * per, n_score), r1 = min(r0 + per, n_score);
+    constexpr int kDeep = NW <= 4 ? 16 : 8;
+    score_rows<kDeep, NT, true, F16>(s, r0, r1, gkeys);
     // The slices meet through memory without cache maintenance: keys and the
     // arrival counter are written and read at device scope (they bypass the
     // XCD-private L2), and every wave waits for its own stores to be acknowledged
-    // before the workgroup counts in.  Whoever counts in last sees everybody's
-    // keys and carries on alone; the others are done.
+    // before the workgroup counts in.
+    KIN_STAMP(40);  // slice issued
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    if (tid == 0)
-      sh_last = (__hip_atomic_fetch_add(&p.ws_count[item], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.chunks - 1)
-                    ? 1 : 0;
+    KIN_STAMP(41);  // slice scored, keys stored
+    if (tid == 0) __hip_atomic_fetch_add(&p.ws_count[titem], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (member >= parts) return;  // a member that only scores is done
+    // The members that go on need everybody's keys.  The others are running or about to be
+    // dispatched (a team's workgroups are neighbours in the grid), so the wait is short; it is
+    // bounded all the same, and a member whose patience runs out -- whatever keeps its team-mates:
+    // a GPU shared with another job, a dispatch order that is no one's promise -- scores the whole
+    // list for itself and gets the same keys.  The wait is an optimisation, never a dependency.
+    s.table_lds = prefetch_table<NT>(s.table, n_pages, table_lds, p.table_cap);
+    if (tid == 0) {
+      int seen = __hip_atomic_load(&p.ws_count[titem], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int spins = 0; seen < team && spins < p.spin_limit; ++spins) {
+        __builtin_amdgcn_s_sleep(4);
+        seen = __hip_atomic_load(&p.ws_count[titem], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      sh_last = seen >= team ? 1 : 0;
+    }
     __syncthreads();
-    if (!sh_last) return;
-    if (tid == 0) __hip_atomic_store(&p.ws_count[item], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
-    append_token();
-    load_shared_keys<NT>(gkeys, n_score, s.keys);
+    KIN_STAMP(42);  // team complete (or patience over)
+    if (__builtin_amdgcn_readfirstlane(sh_last)) {
+      load_shared_keys<NT>(gkeys, n_score, s.keys);
+    } else {
+      score_rows<kDeep, NT, false, F16>(s, 0, n_score, s.keys);
+    }
+    __builtin_amdgcn_s_waitcnt(0);  // the table copy has landed too
     __syncthreads();
+    KIN_STAMP(43);  // keys in LDS
     n = select_from_keys<NT>(s, sel_lds);
   } else {
+    s.table_lds = prefetch_table<NT>(s.table, n_pages, table_lds, p.table_cap);
+    __syncthreads();  // histograms zeroed
     // Mean-key loads in flight per lane.  4 saturate HBM while several rounds of workgroups overlap
     // (4096 lists; more only lengthens the last pass of short lists).  With fewer lists the workgroups
     // score in step and each has to keep 64 KiB in flight: 16 / 8 loads at 4 / 8 waves
@@ -156,14 +166,15 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
       n = score_select<4, NT, F16>(s, sel_lds);
     }
   }
+  KIN_STAMP(30);  // list ready
   if (p.sel_pages && part == 0) {
     int32_t* sel = p.sel_pages + (int64_t)item * p.sel_stride;
     for (int i = tid; i < p.sel_stride; i += NT) sel[i] = (i < n) ? sel_lds[i] : -1;
   }
   if (p.sel_count && tid == 0 && part == 0) p.sel_count[item] = n;
   int p0 = 0, p1 = n;
-  if (p.parts > 1) {
-    const int per = (n + p.parts - 1) / p.parts;
+  if (team > 1) {
+    const int per = (n + parts - 1) / parts;
     p0 = min(part * per, n);
     p1 = min(p0 + per, n);
     // The new token goes into the sequence's last page, which closes every list and is
@@ -194,9 +205,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   attend_list<NG, NW, F16>(
       a, [&](int i) -> int { return __builtin_amdgcn_readfirstlane(sel_lds[i]); }, smem, sm_m, sm_l,
       [&](int g, int d, float o, float lse2) {
-        if (p.parts > 1) {
+        if (parts > 1) {
           // partial result, read by a workgroup that may sit on another XCD: device-scope stores
-          const int64_t row = ((int64_t)item * p.parts + part) * G + g;
+          const int64_t row = ((int64_t)(item - p.head_lists) * parts + part) * G + g;
           __hip_atomic_store(p.ws_po + row * kHeadDim + d, __float_as_uint(o), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           if (d == 0) __hip_atomic_store(p.ws_plse + row, __float_as_uint(lse2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         } else {
@@ -204,127 +215,128 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
           if (p.lse && d == 0) p.lse[hq0 + g] = lse2 * kLn2;
         }
       });
-  if (p.parts <= 1) return;
+  KIN_STAMP(31);  // attended
+  if (parts <= 1) return;
   // Every wave waits for its partial stores to be acknowledged, then the workgroup counts in;
   // whoever counts in last sees all parts and merges them (as merge_splits_kernel does).
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   if (tid == 0)
-    sh_last = (__hip_atomic_fetch_add(&p.ws_count[item], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.parts - 1) ? 1 : 0;
+    sh_last = (__hip_atomic_fetch_add(&p.ws_count2[item - p.head_lists], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == parts - 1) ? 1 : 0;
   __syncthreads();
-  if (!sh_last) return;
-  if (tid == 0) __hip_atomic_store(&p.ws_count[item], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
-  // The parts' log-sum-exps become weights in LDS (the attention's staging area is dead), then every
-  // thread sums its output element over the parts with independent device-scope loads.
-  float* wl = reinterpret_cast<float*>(smem);  // [parts][G] weights, then [G] denominators
-  float* den_g = wl + p.parts * G;
-  const int64_t first_row = (int64_t)item * p.parts * G;
-  const __amdgpu_buffer_rsrc_t rl = make_rsrc(p.ws_plse + first_row, p.parts * G * (int)sizeof(float));
-  for (int i = tid; i < p.parts * G; i += NT)
-    wl[i] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rl, i * 4, 0, kDeviceScope));
-  __syncthreads();
-  if (tid < G) {
-    float mm = kNegInf;
-    for (int sp = 0; sp < p.parts; ++sp) mm = fmaxf(mm, wl[sp * G + tid]);
-    const float m_safe = (mm == kNegInf) ? 0.f : mm;
-    float den = 0.f;
-    for (int sp = 0; sp < p.parts; ++sp) {
-      const float wgt = fast_exp2(wl[sp * G + tid] - m_safe);
-      wl[sp * G + tid] = wgt;
-      den += wgt;
-    }
-    den_g[tid] = den;
-    if (p.lse) p.lse[hq0 + tid] = (den > 0.f) ? (mm + fast_log2(den)) * kLn2 : kNegInf;
-  }
-  __syncthreads();
-  const __amdgpu_buffer_rsrc_t ro = make_rsrc(p.ws_po + first_row * kHeadDim, p.parts * G * kHeadDim * (int)sizeof(float));
-  for (int idx = tid; idx < G * kHeadDim; idx += NT) {
-    const int g = idx >> 7, d = idx & (kHeadDim - 1);
-    float num = 0.f;
-#pragma unroll 8
-    for (int sp = 0; sp < p.parts; ++sp)
-      num += __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ro, ((sp * G + g) * kHeadDim + d) * 4, 0, kDeviceScope)) *
-             wl[sp * G + g];
-    const float den = den_g[g];
-    p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(den > 0.f ? num / den : 0.f);
-  }
+  KIN_STAMP(44);  // partial stored, counted in
+  if (!__builtin_amdgcn_readfirstlane(sh_last)) return;
+  merge_list_parts<NT, F16>(smem, p.ws_po, p.ws_plse, item - p.head_lists, parts, G, p.out + hq0 * kHeadDim, p.lse ? p.lse + hq0 : nullptr);
+  KIN_STAMP(45);  // merged
 }
 
 }  // namespace kin
 
 namespace kin {
 
-// How the workgroups of a launch share the lists.  chunks > 1: split scoring (few lists
-// with many candidates); parts > 1: split attention (lists for at most half the CUs);
-// never both.  need: workspace bytes of the mode chosen (arrival counters first).
+// How the workgroups of a launch share the lists: the first head_lists lists have a workgroup
+// each, every later list a team of `team` workgroups of which `parts` also attend (see
+// StepParams).  nw: waves per workgroup.  need: workspace bytes.
 struct StepPlan {
-  int chunks, parts;
+  int head_lists, team, parts, nw;
   size_t need;
 };
 
-constexpr int kMaxParts = 64;
+constexpr int kMaxTeam = 64;
 
-static size_t parts_workspace_bytes(int64_t items, int parts, int group) {
-  return score_count_bytes(items) + (size_t)items * parts * group * (kHeadDim + 1) * sizeof(float);
+static size_t round256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+// Workspace of `team_lists` lists handled by teams: two arrival counters per list, the shared
+// keys, the partial results.
+static size_t team_workspace_bytes(int64_t team_lists, int parts, int group, int kbar_pages) {
+  if (team_lists <= 0) return 0;
+  size_t need = round256((size_t)team_lists * 2 * sizeof(int32_t));
+  need += round256((size_t)team_lists * score_key_stride(kbar_pages) * sizeof(uint32_t));
+  if (parts > 1) need += (size_t)team_lists * parts * group * (kHeadDim + 1) * sizeof(float);
+  return need;
 }
 
 // list_tiles: upper bound of the 16-token tiles a page list holds.  avail: bytes the caller's
-// workspace has (a smaller one gets fewer parts, or none, never an error).
+// workspace has (a smaller one gets smaller teams, or none, never an error).
 //
-// Split attention: as many parts as keep the launch at one workgroup per CU, each with at
-// least four tiles for each of its 8 waves (below that the merge costs more than it saves;
-// 64 lists x 4 parts of k = 128 pages: 48 us against 46 in 2 parts and 47 whole; a launch
-// that fills every CU wants longer lists still: 128 lists x 2 parts lose 6 % at k = 128
-// and gain 5 % at k = 512).  Every part
-// scores the whole list for itself, ~7 ns per mean key on one CU (more once over 128
-// workgroups pull whole lists through HBM at the same time), where split scoring takes a
-// few us for any length; a tile costs the lone attending workgroup ~0.15 us.  So where the
-// shape could split its scoring instead, parts are taken only if they save more attention
-// than the repeated scoring costs (8 lists of 4097 pages, k = 512: 59 us in parts, 103 us
-// with split scoring; k = 128: 49 against 43; one list of 2049 pages, k = 128: 30 against 37).
-static StepPlan plan_step(int batch, int num_kv_heads, int group, int kbar_pages, int64_t list_tiles, size_t avail) {
-  const int64_t items = (int64_t)batch * num_kv_heads;
-  StepPlan plan{1, 1, 0};
+// Teams are formed when the lists are at most a third of the CUs (or half of them, for page lists
+// of 384 tiles or more): as many members as put one 8-wave workgroup on every CU, no more than
+// give every scoring slice 64 KiB of mean keys or every attending member 16 tiles (below that the
+// exchange and the merge cost more than they save), and of them as many attend as have 16 tiles
+// each.  Measured on MI355X (ctx 32 K, k = 128, G = 4, us per step; one workgroup per list |
+// teams | the earlier scheme, in which every part scored the whole list for itself): 8 lists
+// 38 | 30 | 35; 32 lists 45 | 35 | 45; 64 lists 48 | 42 | 50; 128 lists 54 | 56 | 56.
+// Tried and not kept, because one workgroup per list is faster there: teams of two or three for
+// 129 .. 400 lists (160 lists 53 | 73; 256 lists 74 | 92; 300 lists 102 | 109: the streaming
+// phases are bound by HBM either way, and the exchange, the second select and the merge add
+// 9 us to every list's critical path, a fill launch in front 4 more), and teams for the lists
+// of the second round of a batch a little larger than the GPU holds at once (1024 lists of
+// 8 heads, k = 256: 428 | 452).
+static StepPlan plan_step(int64_t items, int group, int kbar_pages, int64_t list_tiles, size_t avail) {
+  StepPlan plan{(int)items, 1, 1, items <= kNumCus ? 8 : 4, 0};
   if (items <= 0) return plan;
-  const int chunks = score_chunks(batch, num_kv_heads, kbar_pages);
-  int64_t parts = 1;
-  if (items * 2 <= kNumCus && list_tiles >= (items * 2 <= kNumCus - 32 ? 96 : 384)) {
-    parts = kNumCus / items;
-    const int64_t by_work = list_tiles / 32;
-    if (parts > by_work) parts = by_work;
-    if (parts > kMaxParts) parts = kMaxParts;
-    while (parts > 1 && parts_workspace_bytes(items, (int)parts, group) > avail) parts /= 2;
-    if (parts < 1) parts = 1;
+  int64_t head = items, team = 1, parts = 1;
+  const int64_t by_attend = list_tiles / 16;
+  const int64_t by_score = kbar_pages / 256;
+  // (short lists -- under 96 tiles to attend and under 1024 mean keys to score -- are quicker in one workgroup:
+  // 8 .. 64 lists of 8 K tokens, k = 64: 25 .. 28 us against 26 .. 29)
+  if ((items * 3 <= kNumCus && (list_tiles >= 96 || kbar_pages >= 1024)) || (items * 2 <= kNumCus && list_tiles >= 384)) {
+    team = kNumCus / items;
+    const int64_t useful = by_attend > by_score ? by_attend : by_score;
+    if (team > useful) team = useful;
+    if (team > kMaxTeam) team = kMaxTeam;
+    parts = team < by_attend ? team : by_attend;
+    head = 0;
   }
-  const bool chunks_fit = chunks > 1 && score_workspace_bytes(items, kbar_pages) <= avail;
-  if (parts > 1 && chunks_fit) {
-    const int64_t groups = items * parts;  // workgroups that would each score a whole list
-    if (24 * (list_tiles - list_tiles / parts) * 128 <= (int64_t)kbar_pages * (groups > 128 ? groups : 128)) parts = 1;
+  if (parts < 1) parts = 1;
+  if (team < 2) {
+    team = parts = 1;
+    head = items;
   }
-  if (parts > 1) {
-    plan.parts = (int)parts;
-    plan.need = parts_workspace_bytes(items, plan.parts, group);
-  } else if (chunks_fit) {
-    plan.chunks = chunks;
-    plan.need = score_workspace_bytes(items, kbar_pages);
+#ifdef KIN_TUNE
+  // experiments only: KIN_TEAM=head_lists,team,parts,nw
+  int env_nw = 0;
+  if (const char* e = getenv("KIN_TEAM")) {
+    long long eh = 0;
+    int et = 1, ep = 1;
+    if (sscanf(e, "%lld,%d,%d,%d", &eh, &et, &ep, &env_nw) >= 3 && et >= 1 && ep >= 1 && ep <= et && eh >= 0 && eh <= items) {
+      head = et > 1 && eh < items ? eh : items;
+      team = head < items ? et : 1;
+      parts = head < items ? ep : 1;
+    }
   }
+#endif
+  // a workspace too small: fewer parts, then no teams
+  while (team > 1 && team_workspace_bytes(items - head, (int)parts, group, kbar_pages) > avail) {
+    if (parts > 1) {
+      parts /= 2;
+    } else {
+      team = 1;
+      head = items;
+    }
+  }
+  plan.head_lists = (int)head;
+  plan.team = (int)team;
+  plan.parts = (int)parts;
+  const int64_t wgs = head + (items - head) * team;
+  plan.nw = wgs <= kNumCus ? 8 : 4;
+#ifdef KIN_TUNE
+  if (env_nw == 4 || env_nw == 8) plan.nw = env_nw;
+#endif
+  plan.need = team > 1 ? team_workspace_bytes(items - head, plan.parts, group, kbar_pages) : 0;
   return plan;
 }
 
 }  // namespace kin
 
 extern "C" size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages) {
-  // Enough for whichever mode the launch picks, whatever the group size and page budget.
+  // Enough for whichever teams the launch forms, whatever the group size and page budget.
   const int64_t items = (int64_t)batch * num_kv_heads;
   if (items <= 0) return 0;
-  size_t need = 0;
-  if (kin::score_chunks(batch, num_kv_heads, kbar_pages) > 1) need = kin::score_workspace_bytes(items, kbar_pages);
-  if (items * 2 <= kin::kNumCus) {
-    int64_t parts = kin::kNumCus / items;
-    if (parts > kin::kMaxParts) parts = kin::kMaxParts;
-    const size_t split = kin::parts_workspace_bytes(items, (int)parts, kin::kMaxGroup);
-    if (split > need) need = split;
-  }
+  size_t need = kin::plan_step(items, kin::kMaxGroup, kbar_pages, kin::kMaxTopk + 2 * kin::kMaxFixedPages, ~(size_t)0).need;
+#ifdef KIN_TUNE
+  if (need < ((size_t)192 << 20)) need = (size_t)192 << 20;
+#endif
   return need;
 }
 
@@ -394,43 +406,48 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
   p.first_page_offset = first_page_offset;
   p.page_size = page_size;
   p.sort_cap = select_sort_cap(topk, kbar_pages);
-  // Waves per workgroup.  The kernels hold 140-145 registers, so a CU runs 12 waves: three
-  // 4-wave workgroups, or one of 8 while the lists are no more than the CUs (measured: 8 waves
-  // beat 4, 6, 12 and a 16-wave build that spills, by 2-20 %; from 257 lists on, 8-wave
-  // workgroups would take two rounds and 4 waves win by 3-25 %).
+  p.table_cap = select_table_cap(kbar_pages + max_local_pages(local_tokens) + 1);
   const int64_t items = (int64_t)batch * num_kv_heads;
-  if (xcd_grid_size(batch, num_kv_heads) > 0x7fffffffLL)
+  if (xcd_grid_size(batch, num_kv_heads) > 0x7fffffffLL || items * kMaxTeam > 0x7fffffffLL)
     return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads too large", fn);
-  const int nw = items <= kNumCus ? 8 : 4;
-  // Few lists: several workgroups share one (split attention, or split scoring for very long sequences).
-  const StepPlan plan = plan_step(batch, num_kv_heads, p.group, kbar_pages, (int64_t)list_cap << page_tile_shift(page_size),
+  p.num_pages = num_pages;
+  const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
+  p.scale_log2 = scale * 1.4426950408889634f;
+  p.deep_score = items < 4096 ? 1 : 0;
+  p.rotate = attend_rotates(items) ? 1 : 0;
+  // Lists that would leave CUs idle get teams of workgroups (given a workspace).
+  const StepPlan plan = plan_step(items, p.group, kbar_pages, (int64_t)list_cap << page_tile_shift(page_size),
                                   workspace && aligned16(workspace) ? workspace_bytes : 0);
-  p.chunks = plan.chunks;
+  // Waves per workgroup.  The kernels hold 140-145 registers, so a CU runs 12 waves: three
+  // 4-wave workgroups, or one of 8 while the workgroups are no more than the CUs (measured: 8 waves
+  // beat 4, 6, 12 and a 16-wave build that spills, by 2-20 %; from 257 workgroups on, 8-wave
+  // workgroups would take two rounds and 4 waves win by 3-25 %).
+  const int nw = plan.nw;
+  p.head_lists = plan.head_lists;
+  p.team = plan.team;
   p.parts = plan.parts;
-  p.ws_count = nullptr;
+  p.head_blocks = plan.head_lists == items ? (int)xcd_grid_size(batch, num_kv_heads) : plan.head_lists;
+  p.spin_limit = kTeamSpinLimit;
+  p.ws_count = p.ws_count2 = nullptr;
   p.ws_keys = nullptr;
   p.ws_po = nullptr;
   p.ws_plse = nullptr;
-  if (plan.chunks > 1 || plan.parts > 1) {
-    char* after_counters = static_cast<char*>(workspace) + score_count_bytes(items);
-    p.ws_count = static_cast<int32_t*>(workspace);
-    if (plan.chunks > 1) {
-      p.ws_keys = reinterpret_cast<uint32_t*>(after_counters);
-    } else {
-      p.ws_po = reinterpret_cast<uint32_t*>(after_counters);
-      p.ws_plse = p.ws_po + (size_t)items * plan.parts * p.group * kHeadDim;
-    }
+  const int64_t team_lists = items - plan.head_lists;
+  if (plan.team > 1) {
+    char* w = static_cast<char*>(workspace);
+    p.ws_count = reinterpret_cast<int32_t*>(w);
+    p.ws_count2 = p.ws_count + team_lists;
+    w += round256((size_t)team_lists * 2 * sizeof(int32_t));
+    p.ws_keys = reinterpret_cast<uint32_t*>(w);
+    w += round256((size_t)team_lists * score_key_stride(kbar_pages) * sizeof(uint32_t));
+    p.ws_po = reinterpret_cast<uint32_t*>(w);
+    p.ws_plse = p.ws_po + (size_t)team_lists * plan.parts * p.group * kHeadDim;
   }
-  p.deep_score = items < 4096 ? 1 : 0;
-  p.rotate = attend_rotates(items) ? 1 : 0;
-  const size_t sel_scratch = select_lds_bytes(kbar_pages, p.sort_cap);
+  const size_t sel_scratch = select_lds_bytes(kbar_pages, p.sort_cap, p.table_cap);
   const size_t attend_bytes = (size_t)attend_lds_bytes(nw);
   size_t region0 = sel_scratch > attend_bytes ? sel_scratch : attend_bytes;
   region0 = (region0 + 15) & ~(size_t)15;
   p.region0_bytes = (int)region0;
-  p.num_pages = num_pages;
-  const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
-  p.scale_log2 = scale * 1.4426950408889634f;
   const size_t lds = region0 + (size_t)list_cap * 4;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const void* kernel;
@@ -448,13 +465,12 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
                    "hipFuncSetAttribute(blocktopk_step_kernel)");
     if (st) return st;
   }
-  unsigned grid = (unsigned)xcd_grid_size(batch, num_kv_heads);
-  if (p.chunks > 1 || p.parts > 1) {
+  const unsigned grid = (unsigned)(p.head_blocks + team_lists * plan.team);
+  if (plan.team > 1) {
     // the arrival counters start at zero (a fill kernel, so that the launch pair can be captured in a graph)
-    fill_zero_i32_kernel<<<(unsigned)((items + 255) / 256), 256, 0, s>>>(p.ws_count, (int)items);
+    fill_zero_i32_kernel<<<(unsigned)((2 * team_lists + 255) / 256), 256, 0, s>>>(p.ws_count, (int)(2 * team_lists));
     st = check_hip(hipGetLastError(), "fill_zero_i32_kernel launch");
     if (st) return st;
-    grid = (unsigned)(items * (p.chunks > 1 ? p.chunks : p.parts));
   }
   void* args[] = {&p};
   st = check_hip(hipLaunchKernel(kernel, dim3(grid), dim3(nw * 64), args, lds, s), "blocktopk_step_kernel launch");
@@ -519,6 +535,10 @@ extern "C" int kin_blocktopk_decode_step_f16(const kin_f16_t* q, const kin_f16_t
                           workspace, workspace_bytes, stream);
 }
 
+#ifdef KIN_TUNE
+KIN_STAMP_ACCESSOR(kin_debug_stamps_step)
+#endif
+
 extern "C" size_t kin_static_scratch_bytes(void) { return kin::kStaticScratchBytes; }
 
 extern "C" int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,
@@ -531,15 +551,18 @@ extern "C" int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_b
                                                 int first_page_offset, float sm_scale, kin_stream_t stream) {
   using namespace kin;
   const char* fn = "kin_blocktopk_decode_step_static";
-  // What this shape's way of sharing lists between workgroups needs, from the dimensions
-  // alone.  Split scoring beyond the array is an error, not a silent fall-back to the
-  // slower single-workgroup scoring; split attention always fits (kMaxGroup heads included).
+  // What the teams of this shape need, from the dimensions alone.  With few lists (up to one for
+  // every other CU) the teams are what keeps the GPU busy at all: if theirs do not fit the array
+  // (long sequences: 4 bytes per candidate page and list), that is an error, not a silent
+  // fall-back to one workgroup per list.  Larger batches take the teams that fit, or none.
   size_t need = 0;
   if (batch > 0 && num_kv_heads > 0 && num_q_heads >= num_kv_heads && kbar_pages > 0 && topk >= 0 && sink_pages >= 0 &&
       local_tokens >= 1 && page_size >= kPageSize) {
     const int64_t list_cap = (int64_t)topk + sink_pages + max_local_pages(local_tokens);
-    need = plan_step(batch, num_kv_heads, num_q_heads / num_kv_heads, kbar_pages, list_cap << page_tile_shift(page_size),
-                     ~(size_t)0).need;
+    const int64_t lists = (int64_t)batch * num_kv_heads;
+    need = plan_step(lists, num_q_heads / num_kv_heads, kbar_pages, list_cap << page_tile_shift(page_size), ~(size_t)0).need;
+    if (lists * 2 > kNumCus && need > kStaticScratchBytes)
+      need = plan_step(lists, num_q_heads / num_kv_heads, kbar_pages, list_cap << page_tile_shift(page_size), kStaticScratchBytes).need;
   }
   if (need > kStaticScratchBytes)
     return fail(KIN_ERR_WORKSPACE,

@@ -348,9 +348,9 @@ def test_header_is_plain_c_and_links_from_c(tmp_path):
 
 
 def test_static_scratch_step_size_limit_is_checked_before_anything_else(lib):
-    """The entry point that allocates nothing rejects shapes whose split-scoring
-    scratch exceeds its built-in array, from the dimensions alone."""
-    assert lib.kin_static_scratch_bytes() == 2 * 1024 * 1024 + 32 * 1024
+    """The entry point that allocates nothing rejects shapes whose teams' scratch
+    (shared keys and partial results) exceeds its built-in array, from the dimensions alone."""
+    assert lib.kin_static_scratch_bytes() == 4 * 1024 * 1024 + 64 * 1024
     assert 0 < lib.kin_step_workspace_bytes(64, 1, 8192) <= lib.kin_static_scratch_bytes()
     assert lib.kin_step_workspace_bytes(64, 1, 16384) > lib.kin_static_scratch_bytes()
     st = lib.kin_blocktopk_decode_step_static(None, None, None, None, None, None, None, None, 128, 0, 1, None, None, None,

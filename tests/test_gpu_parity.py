@@ -916,9 +916,10 @@ def test_unused_cache_slots_may_hold_nan(ops):
 
 @pytest.mark.parametrize("hkv,group", [(1, 4), (2, 8), (8, 1)])
 def test_fused_step_split_scoring_for_few_long_sequences(ops, hkv, group):
-    """Few lists with thousands of candidate pages: the step spreads the scoring
-    of each list over several workgroups that meet through the workspace; same
-    cache bytes, page lists and output as without it, call after call."""
+    """Few lists with thousands of candidate pages: a team of workgroups per list shares
+    the scoring (and the attention) and meets through the workspace; same cache bytes and
+    page lists as without it, outputs equal to fp32 summation order and identical call
+    after call."""
     lengths = [PS * 2500 + 3, PS * 2100 + 16, 5, 0, PS * 300 + 1][: max(2, 10 // hkv)]
     pb = P.make_problem(1400 + hkv, lengths, num_kv_heads=hkv, group=group, topk=40)
     kbar_pages = pb.kbar.shape[2]
@@ -936,20 +937,24 @@ def test_fused_step_split_scoring_for_few_long_sequences(ops, hkv, group):
         torch.cuda.synchronize()
         assert torch.equal(a.kv, b2.kv) and torch.equal(a.kbar, b2.kbar)
         assert torch.equal(a.cnt, b2.cnt) and torch.equal(a.sel, b2.sel)
-        assert torch.equal(out_a, outs[-1])
+        assert torch.allclose(out_a.float(), outs[-1].float(), rtol=1e-2, atol=1e-2)
+        assert torch.equal(outs[0], outs[-1])
     kv, kbar = pb.kv_cache.copy(), pb.kbar.copy()
     res = O.decode_step(pb.q, pb.k, pb.v, kv, kbar, pb.page_indices, pb.page_indptr, pb.last_page_len, pb.topk)
     assert np.array_equal(P.from_torch(a.kv), kv) and np.array_equal(P.from_torch(a.kbar), kbar)
     assert np.array_equal(a.cnt.cpu().numpy(), res["sel_count"])
     sel = a.sel.cpu().numpy()
     want, _ = O.sparse_paged_decode(pb.q, kv, sel, res["sel_count"], pb.last_page_len)
-    assert_out_close(out_a, want, "split scoring")
+    assert_out_close(out_a, want, "one workgroup per list")
+    assert_out_close(outs[0], want, "teams")
     if np.array_equal(sel, res["sel_pages"]):
-        assert_out_close(out_a, res["out"], "split scoring vs oracle end to end")
+        assert_out_close(outs[0], res["out"], "teams vs oracle end to end")
     # the wrapper allocates the workspace itself when none is given
     c = Gpu(pb)
     out_c = ops.blocktopk_decode_step(c.q, c.k, c.v, c.kv, c.kbar, c.indices, c.indptr, c.last, pb.topk)
-    assert torch.equal(out_c, out_a)
+    # (no page-list output: winners attended in index order, another fp32 summation order)
+    assert torch.allclose(out_c.float(), out_a.float(), rtol=1e-2, atol=1e-2)
+    assert_out_close(out_c, want, "split scoring, no page-list output")
     # the stand-alone selector splits the same way when it is given the workspace: same lists,
     # same logical indices and scores as alone, call after call
     one, two = Gpu(pb), Gpu(pb)
@@ -1638,7 +1643,10 @@ def test_fused_step_equals_three_calls(ops, case):
     c = Gpu(pb)
     ops.append_paged_kv(c.k, c.v, c.kv, c.kbar, c.indices, c.indptr, c.last)
     out_c = ops.blocktopk_decode_step(c.q, None, None, c.kv, c.kbar, c.indices, c.indptr, c.last, pb.topk)
-    assert torch.equal(out_c, out_b)
+    # without the page-list output the winners are attended in index order rather than score order
+    # (no sort): the same pages, another fp32 summation order
+    assert torch.allclose(out_c.float(), out_b.float(), rtol=1e-2, atol=1e-2)
+    assert_out_close(out_c, want, f"fused {case}, no page-list output")
 
 
 def test_fused_step_full_size(ops):

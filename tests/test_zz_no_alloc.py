@@ -63,7 +63,7 @@ def test_static_scratch_step_equals_workspace_step():
     from kinetics_amd import _lib, ops
 
     lib = _lib.load()
-    assert lib.kin_static_scratch_bytes() == 2 * 1024 * 1024 + 32 * 1024
+    assert lib.kin_static_scratch_bytes() == 4 * 1024 * 1024 + 64 * 1024
     # two calls in a row on the same array, the second smaller (fewer and shorter lists): the
     # first call's keys and counters are what the second finds there
     big = P.make_problem(9101, [PS * 2500 + 3, PS * 2100 + 16, 5, 0, PS * 300 + 1], num_kv_heads=2, group=4, topk=40)
@@ -73,8 +73,7 @@ def test_static_scratch_step_equals_workspace_step():
     # a shape with lists for more than half the CUs shares nothing between workgroups and never touches the array
     plain = P.make_problem(9103, [PS * 40 + 1] * 69 + [3], num_kv_heads=2, group=2, topk=8)
     _both_ways(ops, plain, sink=0, local=1, what="third call (one workgroup per list)", must_split=False)
-    # few lists with long page lists: split attention, the partial results lie where the keys lay;
-    # 8 lists x 32 parts x 16 heads fill the array to the last kilobytes
+    # few lists with long page lists: larger teams, more partial results (8 lists x 32 parts x 16 heads: 2.1 MB)
     parts = P.make_problem(9104, [PS * 400 + 1, PS * 300 + 16, 9], num_kv_heads=2, group=4, topk=150)
     _both_ways(ops, parts, sink=1, local=20, what="fourth call (split attention)", must_split=True)
     full = P.make_problem(9105, [PS * 1300 + 5] * 4, num_kv_heads=2, group=16, topk=1100)
@@ -87,7 +86,7 @@ def test_static_scratch_step_rejects_sizes_beyond_the_array():
     from kinetics_amd import _lib
 
     lib = _lib.load()
-    # 64 lists of 16384 candidate pages want 4 MiB of keys: more than the array holds.  The size
+    # 64 lists of 16384 candidate pages want 4 MiB of keys and 0.5 MB of partial results: more than the array holds.  The size
     # test comes first, from the dimensions alone: no pointer is looked at.
     assert lib.kin_step_workspace_bytes(64, 1, 16384) > lib.kin_static_scratch_bytes()
     null = ctypes.c_void_p(None)
