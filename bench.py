@@ -489,6 +489,88 @@ def side_workload(torch, ops, name, steps, warmup, device, with_dense=True):
     return out
 
 
+def manager_bench(torch, ops, steps, warmup, device):
+    """The LiteSys-style KV manager (kinetics_amd/batch_cache.py, the paged stand-in for
+    LiteSys/litesys/attention/batch_cache.py:86-168) around the fused step: wall time of one
+    compute_attention call per layer -- offsets, page reservation and page table once per step,
+    the kernels planned for the active sequences -- against the bare fused step on the same
+    tensors.  Every slot is active; the block policy on every layer (attn_layer_skip=[])."""
+    from types import SimpleNamespace
+
+    from kinetics_amd.batch_cache import PagedBatchKVManager
+
+    out = {}
+    Hq, Hkv, topk, local = 4, 1, 64, 16
+    # (layers: what fits beside the caches; the page table is built once per step, whatever their number)
+    for B, ctx, L in ((32, 32768, 8), (256, 16384, 8), (4096, 8192, 4)):
+        cfg = SimpleNamespace(num_attention_heads=Hq, num_key_value_heads=Hkv, head_dim=D, hidden_size=Hq * D, num_hidden_layers=L)
+        m = PagedBatchKVManager(cfg, B, ctx + 1024, device, torch.bfloat16, attn_block_topk=topk, attn_local=local, attn_layer_skip=[])
+        # state as after a prefill of ctx tokens per slot, written directly: offsets, pages, random K/V, mean keys
+        gen = torch.Generator(device=device).manual_seed(7)
+        lens = torch.full((B,), ctx + m.pad, dtype=torch.int32, device=device)
+        m.pool.reserve(lens)
+        idx = torch.empty(m.num_pool_pages, dtype=torch.int32, device=device)
+        ptr = torch.empty(B + 1, dtype=torch.int32, device=device)
+        last = torch.empty(B, dtype=torch.int32, device=device)
+        m.pool.build_page_table(lens, idx, ptr, last)
+        for layer in range(L):
+            m.kv_offset[layer].fill_(ctx)
+            kv = m.kv_cache[layer]
+            chunk = max(1, (1 << 27) // (2 * m.page * Hkv * D))
+            for s0 in range(0, kv.shape[0], chunk):
+                e0 = min(kv.shape[0], s0 + chunk)
+                kv[s0:e0] = torch.randn(e0 - s0, 2, m.page, Hkv, D, generator=gen, device=device).bfloat16()
+            ops.build_kbar(kv, m.kbar[layer], idx, ptr, last)
+        batch_idx = torch.arange(B, device=device)
+        qs, ks, vs = (torch.randn(B, h, 1, D, generator=gen, device=device).bfloat16() for h in (Hq, Hkv, Hkv))
+
+        def step():
+            for layer in range(L):
+                m.compute_attention(qs, ks, vs, layer, batch_idx)
+
+        with collector_paused():
+            for _ in range(warmup):
+                step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                step()
+            torch.cuda.synchronize()
+            per_call = (time.perf_counter() - t0) / (steps * L)
+        # the bare fused step on the manager's own tensors (table of the last step), layer after layer
+        # like the manager (one layer's cache over and over would sit in the 256 MB last-level cache)
+        n, slots, indptr, lastp = B, m._slots32[:B], m._indptr[: B + 1], m._last[:B]
+        q3, k3, v3 = qs[:, :, 0, :], ks[:, :, 0, :], vs[:, :, 0, :]
+        o3 = torch.empty_like(q3)
+
+        def bare(layer):
+            ops.blocktopk_decode_step(q3, k3, v3, m.kv_cache[layer], m.kbar[layer], m.page_indices, indptr, lastp, topk, out=o3,
+                                      sink_pages=m.sink_pages, local_tokens=m.local_tokens, first_page_offset=m.pad,
+                                      workspace=m._ws, slot_ids=slots)
+
+        with collector_paused():
+            for i in range(warmup):
+                bare(i % L)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(steps * L):
+                bare(i % L)
+            torch.cuda.synchronize()
+            per_bare = (time.perf_counter() - t0) / (steps * L)
+        graph_ms = time_graph_replay(torch, step, steps, warmup) / L if per_call * 1e3 < GRAPH_REPLAY_BELOW_MS * 2 else None
+        free, bits = m.pool.status()
+        out[f"B={B}"] = {"batch": B, "ctx": ctx, "layers": L, "topk_pages": topk, "local_tokens": local,
+                         "ms_per_layer_call": per_call * 1e3, "ms_bare_fused_step": per_bare * 1e3,
+                         "glue_fraction": 1.0 - per_bare / per_call, "ms_per_layer_call_hip_graph": graph_ms,
+                         "tokens_per_s_per_layer": B / per_call, "pool_status_bits": bits}
+        print(f"[bench] manager B={B} ctx={ctx}: {per_call * 1e6:.1f} us per layer call, bare step {per_bare * 1e6:.1f} us, "
+              f"glue {100 * (1 - per_bare / per_call):.1f} %" + (f", replayed as a graph {graph_ms * 1e3:.1f} us" if graph_ms else ""),
+              file=sys.stderr, flush=True)
+        del m, idx, ptr, last, qs, ks, vs
+        torch.cuda.empty_cache()
+    return out
+
+
 def placement_rounds(torch, ops, args, B, ctx, Hkv, G, topk, device):
     """Same binary, same seeded inputs, several allocations of the cache in one
     process: round 0 is the process's first large allocation; later rounds reuse
@@ -550,6 +632,9 @@ def main():
                     help="instead of the benchmark: build, time (step and dense) and free the workload's cache this many "
                          "times in one process, with dummy allocations of varying size in front of it, to see how much "
                          "the physical placement of the cache moves the kernels; prints one JSON line")
+    ap.add_argument("--manager", action="store_true",
+                    help="instead of the benchmark: time the LiteSys-style KV manager's decode call per layer at 32 / 256 / 4096 "
+                         "active slots against the bare fused step on the same tensors; prints one JSON line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) to scale profiler byte counters")
     args = ap.parse_args()
@@ -584,6 +669,9 @@ def main():
     headline = args.workload == "qwen3-8b-share" and not args.batch
     if args.placement_rounds:
         print(json.dumps(placement_rounds(torch, ops, args, B, ctx, Hkv, G, topk, device)))
+        return
+    if args.manager:
+        print(json.dumps({"manager": manager_bench(torch, ops, max(args.steps, 50), max(args.warmup, 10), device)}))
         return
     t_setup = time.perf_counter()
     page = args.page_size

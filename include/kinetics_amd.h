@@ -79,7 +79,8 @@ enum kin_status {
  * few lists are handled by teams of workgroups that share the scoring and the
  * attention (kin_step_workspace_bytes covers keys and partial results;
  * KIN_STATIC_SCRATCH_BYTES doubles); without sel_pages the step attends the
- * winners in index order. */
+ * winners in index order.  3.0.0: every entry point that touches kbar takes
+ * slot_ids / num_slots in front of the stream (kbar laid out by cache slot). */
 int kin_version(void);
 
 /* Human-readable text of the last non-OK status on the calling thread
@@ -101,13 +102,26 @@ const char* kin_status_string(int status);
  * kbar[b, h, n_pages-1, :] is set to the mean of the page's page_size keys
  * (fp32 sum in slot order, times 1/page_size, round-to-nearest-even to bf16).
  * Sequences with an empty page list are skipped.  kbar may be NULL.
+ *
+ * slot_ids / num_slots (here and in every entry point that touches kbar): the
+ * reference's kernels take batch_idx and index the cache by slot while q, k, v
+ * and the output follow the position in the active batch
+ * (ref: LiteSys/litesys/attention/cache_utils.py:40-51,67-70,
+ * LiteSys/litesys/attention/batch_cache.py:76-110).  Here the page table is
+ * already per active sequence, so the one tensor left that is laid out by slot is
+ * kbar: with slot_ids != NULL (int32 [batch], on the device), sequence b's mean
+ * keys are kbar[slot_ids[b], ...] and kbar has num_slots row blocks; a sequence
+ * whose id lies outside [0, num_slots) has no mean keys (nothing is written for
+ * it, and it has no candidate pages).  slot_ids == NULL: kbar[b, ...], num_slots
+ * is ignored.  Two sequences of one call must not share a slot.
  */
 int kin_append_paged_kv(const kin_bf16_t* k, const kin_bf16_t* v,
                         kin_bf16_t* kv_cache, kin_bf16_t* kbar,
                         const int32_t* page_indices, const int32_t* page_indptr,
                         const int32_t* last_page_len,
                         int batch, int num_kv_heads, int head_dim, int page_size,
-                        int64_t num_pages, int kbar_pages, kin_stream_t stream);
+                        int64_t num_pages, int kbar_pages,
+                        const int32_t* slot_ids, int num_slots, kin_stream_t stream);
 
 /*
  * Representative keys for every FULL page of every sequence (what a prefill
@@ -120,7 +134,8 @@ int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar,
                    const int32_t* page_indices, const int32_t* page_indptr,
                    const int32_t* last_page_len,
                    int batch, int num_kv_heads, int head_dim, int page_size,
-                   int64_t num_pages, int kbar_pages, kin_stream_t stream);
+                   int64_t num_pages, int kbar_pages,
+                   const int32_t* slot_ids, int num_slots, kin_stream_t stream);
 
 /*
  * Ragged multi-token append -- the general form of
@@ -146,7 +161,8 @@ int kin_append_paged_kv_ragged(const kin_bf16_t* k, const kin_bf16_t* v,
                                const int32_t* last_page_len,
                                int batch, int64_t nnz, int max_append_len,
                                int num_kv_heads, int head_dim, int page_size,
-                               int64_t num_pages, int kbar_pages, kin_stream_t stream);
+                               int64_t num_pages, int kbar_pages,
+                               const int32_t* slot_ids, int num_slots, kin_stream_t stream);
 
 /*
  * (2)+(3) Page scoring and top-k page selection, fused -- replaces
@@ -204,7 +220,8 @@ int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
                          int32_t* sel_logical, float* scores_out,
                          int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
                          int kbar_pages, int sel_stride,
-                         void* workspace, size_t workspace_bytes, kin_stream_t stream);
+                         void* workspace, size_t workspace_bytes,
+                         const int32_t* slot_ids, int num_slots, kin_stream_t stream);
 
 /*
  * Longest page list the selector can write for these settings:
@@ -303,7 +320,12 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  * finish merges.  A member waits for its team's keys for a bounded time only
  * and then scores the list alone, so the launch never depends on which
  * workgroups run at the same time.  Without sel_pages the winners are attended
- * in index order instead of score order (no sort).  Any of this changes only the
+ * in index order instead of score order (no sort).  slot_lens (optional, int32
+ * [num_slots], by slot like kbar; [batch] without slot_ids): a per-slot token
+ * counter that the kernel advances by one for every sequence of the call when
+ * k and v are given -- the reference's kv_offset[batch_idx] += 1 after its copy
+ * (ref: LiteSys/litesys/attention/batch_cache.py:76-84) without a launch of its
+ * own.  Any of this changes only the
  * fp32 summation order of the output, not the page lists or cache bytes.  At
  * least as fast as the three calls except for few lists of more than 4096 pages
  * with topk >= 256 and for 257..349 lists with topk > 768 (up to 1.3x and 1.2x
@@ -320,6 +342,7 @@ int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const ki
                               int head_dim, int page_size, int64_t num_pages,
                               int kbar_pages, int sel_stride, int first_page_offset,
                               float sm_scale, void* workspace, size_t workspace_bytes,
+                              const int32_t* slot_ids, int num_slots, int32_t* slot_lens,
                               kin_stream_t stream);
 
 /*
@@ -376,7 +399,9 @@ int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_bf16_t* k, c
                                      int batch, int num_q_heads, int num_kv_heads,
                                      int head_dim, int page_size, int64_t num_pages,
                                      int kbar_pages, int sel_stride, int first_page_offset,
-                                     float sm_scale, kin_stream_t stream);
+                                     float sm_scale,
+                                     const int32_t* slot_ids, int num_slots, int32_t* slot_lens,
+                                     kin_stream_t stream);
 
 /*
  * Token-level top-k sparse decode attention in one launch -- LiteSys'
@@ -484,8 +509,11 @@ int kin_strided_topk_decode_f16(const kin_f16_t* q, const kin_f16_t* kv_cache,
  * (ref: LiteSys/litesys/attention/batch_cache.py:40-62,76-84).  Slot s owns the
  * physical pages s*pages_per_slot .. (s+1)*pages_per_slot-1.  For sequence b
  * living in slot slot_ids[b] (NULL = identity) with seq_lens[b] tokens, writes
- *   page_indptr[0..batch]   CSR offsets (n_pages = ceil(len / page_size),
- *                           clamped to pages_per_slot; 0 pages for len <= 0)
+ *   page_indptr[0..batch]   CSR offsets (n_pages = ceil(len / page_size); 0
+ *                           pages for len <= 0, and for a sequence longer than
+ *                           its slot -- pages_per_slot pages -- can hold: the
+ *                           kernels then write nothing for it and return
+ *                           zeros, rather than append into a cut list)
  *   page_indices[...]       slot*pages_per_slot + p, packed per sequence
  *                           (capacity batch*pages_per_slot entries)
  *   last_page_len[b]        tokens in the final page (1 for empty sequences)
@@ -502,7 +530,7 @@ int kin_build_slot_page_table(const int32_t* slot_ids, const int32_t* seq_lens, 
  * per-slot contiguous caches that also gives memory back: LiteSys sizes
  * [max_batch, H_kv, max_len, D] per layer up front and clear_cache zeroes a
  * slot (ref: LiteSys/litesys/attention/batch_cache.py:40-62,147-152); here the
- * slots draw 16-token pages from one pool of num_pool_pages pages through a
+ * slots draw pages (of 16, 32 or 64 tokens) from one pool of num_pool_pages pages through a
  * free list that lives on the device, so the pool can be smaller than
  * max_slots * pages_per_slot and a finished request returns its pages.  No host
  * synchronisation anywhere; every call is a single small kernel.
@@ -513,13 +541,17 @@ int kin_build_slot_page_table(const int32_t* slot_ids, const int32_t* seq_lens, 
  *                                 1 = a reserve call wanted more pages than were
  *                                     free (that call reserved nothing),
  *                                 2 = a sequence wanted more than pages_per_slot
- *                                     pages (it was cut there)
+ *                                     pages (its slot got pages_per_slot),
+ *                                 4 = a slot id outside [0, max_slots), or one
+ *                                     that an earlier entry of the same call
+ *                                     named (that entry was skipped)
  *   slot_table  [max_slots, pages_per_slot]  physical page of each logical page
  *   slot_npages [max_slots]       pages the slot owns
  * kin_page_pool_init fills the stack (pages are handed out 0, 1, 2, ...), and
  * clears the state and the slot counts.
  * kin_page_pool_reserve grows the slot of every sequence b (slot_ids[b], NULL =
- * identity; distinct) to ceil(seq_lens[b] / page_size) pages, at most
+ * identity; distinct and below max_slots: other entries are skipped and raise
+ * status bit 4) to ceil(seq_lens[b] / page_size) pages, at most
  * pages_per_slot; it never shrinks a slot, so sequences with seq_lens[b] <= 0
  * are left alone and calling it again with the same lengths changes nothing.
  * All or nothing: if the stack cannot cover the whole call it reserves nothing
@@ -527,10 +559,12 @@ int kin_build_slot_page_table(const int32_t* slot_ids, const int32_t* seq_lens, 
  * kin_page_pool_release pushes every page of the `count` listed slots back and
  * empties them (clear_cache).
  * kin_build_pool_page_table is kin_build_slot_page_table with page ids taken
- * from slot_table; a sequence is cut to the pages its slot owns (so after a
- * failed reserve no unowned entry is ever listed).
+ * from slot_table; a sequence that needs more pages than its slot owns (a
+ * reserve failed, or it outgrew pages_per_slot) gets an empty page list, so no
+ * unowned entry is ever listed and nothing is appended into a cut list.
  * The status word is for the host to poll when it is convenient
- * (hipMemcpy of pool_state); kernels cannot raise.
+ * (hipMemcpy of pool_state) and to clear once it has seen it (a store of 0 to
+ * pool_state[1]); kernels cannot raise.
  */
 int kin_page_pool_init(int32_t* free_stack, int32_t* pool_state, int32_t* slot_npages,
                        int num_pool_pages, int max_slots, kin_stream_t stream);
@@ -538,18 +572,19 @@ int kin_page_pool_init(int32_t* free_stack, int32_t* pool_state, int32_t* slot_n
 int kin_page_pool_reserve(const int32_t* slot_ids, const int32_t* seq_lens, int batch,
                           int pages_per_slot, int page_size,
                           int32_t* slot_table, int32_t* slot_npages,
-                          const int32_t* free_stack, int32_t* pool_state, kin_stream_t stream);
+                          const int32_t* free_stack, int32_t* pool_state, int max_slots,
+                          kin_stream_t stream);
 
 int kin_page_pool_release(const int32_t* slot_ids, int count, int pages_per_slot,
                           const int32_t* slot_table, int32_t* slot_npages,
                           int32_t* free_stack, int32_t* pool_state, int num_pool_pages,
-                          kin_stream_t stream);
+                          int max_slots, kin_stream_t stream);
 
 int kin_build_pool_page_table(const int32_t* slot_ids, const int32_t* seq_lens, int batch,
                               int pages_per_slot, int page_size,
                               const int32_t* slot_table, const int32_t* slot_npages,
                               int32_t* page_indices, int32_t* page_indptr,
-                              int32_t* last_page_len, kin_stream_t stream);
+                              int32_t* last_page_len, int max_slots, kin_stream_t stream);
 
 /*
  * Debugging aid, SYNCHRONOUS (waits for the stream): verifies on the device
@@ -581,13 +616,15 @@ int kin_append_paged_kv_f16(const kin_f16_t* k, const kin_f16_t* v,
                             const int32_t* page_indices, const int32_t* page_indptr,
                             const int32_t* last_page_len,
                             int batch, int num_kv_heads, int head_dim, int page_size,
-                            int64_t num_pages, int kbar_pages, kin_stream_t stream);
+                            int64_t num_pages, int kbar_pages,
+                            const int32_t* slot_ids, int num_slots, kin_stream_t stream);
 
 int kin_build_kbar_f16(const kin_f16_t* kv_cache, kin_f16_t* kbar,
                        const int32_t* page_indices, const int32_t* page_indptr,
                        const int32_t* last_page_len,
                        int batch, int num_kv_heads, int head_dim, int page_size,
-                       int64_t num_pages, int kbar_pages, kin_stream_t stream);
+                       int64_t num_pages, int kbar_pages,
+                       const int32_t* slot_ids, int num_slots, kin_stream_t stream);
 
 int kin_append_paged_kv_ragged_f16(const kin_f16_t* k, const kin_f16_t* v,
                                    const int32_t* append_indptr,
@@ -596,7 +633,8 @@ int kin_append_paged_kv_ragged_f16(const kin_f16_t* k, const kin_f16_t* v,
                                    const int32_t* last_page_len,
                                    int batch, int64_t nnz, int max_append_len,
                                    int num_kv_heads, int head_dim, int page_size,
-                                   int64_t num_pages, int kbar_pages, kin_stream_t stream);
+                                   int64_t num_pages, int kbar_pages,
+                                   const int32_t* slot_ids, int num_slots, kin_stream_t stream);
 
 int kin_block_score_topk_f16(const kin_f16_t* q, const kin_f16_t* kbar,
                              const int32_t* page_indices, const int32_t* page_indptr,
@@ -606,7 +644,8 @@ int kin_block_score_topk_f16(const kin_f16_t* q, const kin_f16_t* kbar,
                              int32_t* sel_logical, float* scores_out,
                              int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
                              int kbar_pages, int sel_stride,
-                             void* workspace, size_t workspace_bytes, kin_stream_t stream);
+                             void* workspace, size_t workspace_bytes,
+                             const int32_t* slot_ids, int num_slots, kin_stream_t stream);
 
 int kin_sparse_paged_decode_f16(const kin_f16_t* q, const kin_f16_t* kv_cache,
                                 const int32_t* sel_pages, const int32_t* sel_count,
@@ -639,6 +678,7 @@ int kin_blocktopk_decode_step_f16(const kin_f16_t* q, const kin_f16_t* k, const 
                                   int head_dim, int page_size, int64_t num_pages,
                                   int kbar_pages, int sel_stride, int first_page_offset,
                                   float sm_scale, void* workspace, size_t workspace_bytes,
+                                  const int32_t* slot_ids, int num_slots, int32_t* slot_lens,
                                   kin_stream_t stream);
 
 /* ---- row-wise layer kernels around the attention path ---------------------

@@ -31,16 +31,16 @@ SIGNATURES = {
     "kin_version": (c_int, []),
     "kin_last_error": (c_char_p, []),
     "kin_status_string": (c_char_p, [c_int]),
-    "kin_append_paged_kv": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int64, c_int, _P]),
+    "kin_append_paged_kv": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int64, c_int, _P, c_int, _P]),
     "kin_append_paged_kv_ragged": (
         c_int,
-        [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int64, c_int, c_int, c_int, c_int, c_int64, c_int, _P],
+        [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int64, c_int, c_int, c_int, c_int, c_int64, c_int, _P, c_int, _P],
     ),
-    "kin_build_kbar": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int64, c_int, _P]),
+    "kin_build_kbar": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int64, c_int, _P, c_int, _P]),
     "kin_block_score_topk": (
         c_int,
         [_P, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P,
-         c_size_t, _P],
+         c_size_t, _P, c_int, _P],
     ),
     "kin_sel_list_capacity": (c_int, [c_int, c_int, c_int]),
     "kin_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
@@ -58,14 +58,14 @@ SIGNATURES = {
     "kin_blocktopk_decode_step": (
         c_int,
         [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int64,
-         c_int, c_int, c_int, c_float, _P, c_size_t, _P],
+         c_int, c_int, c_int, c_float, _P, c_size_t, _P, c_int, _P, _P],
     ),
     "kin_step_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "kin_static_scratch_bytes": (c_size_t, []),
     "kin_blocktopk_decode_step_static": (
         c_int,
         [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int64,
-         c_int, c_int, c_int, c_float, _P],
+         c_int, c_int, c_int, c_float, _P, c_int, _P, _P],
     ),
     "kin_token_topk_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "kin_token_topk_decode": (
@@ -81,9 +81,9 @@ SIGNATURES = {
     ),
     "kin_build_slot_page_table": (c_int, [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P]),
     "kin_page_pool_init": (c_int, [_P, _P, _P, c_int, c_int, _P]),
-    "kin_page_pool_reserve": (c_int, [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P, _P]),
-    "kin_page_pool_release": (c_int, [_P, c_int, c_int, _P, _P, _P, _P, c_int, _P]),
-    "kin_build_pool_page_table": (c_int, [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P]),
+    "kin_page_pool_reserve": (c_int, [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P, c_int, _P]),
+    "kin_page_pool_release": (c_int, [_P, c_int, c_int, _P, _P, _P, _P, c_int, c_int, _P]),
+    "kin_build_pool_page_table": (c_int, [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P, _P, c_int, _P]),
     "kin_check_page_table": (c_int, [_P, _P, _P, c_int, c_int, c_int64, c_int64, _P, _P]),
     "kin_rms_norm": (c_int, [_P, _P, _P, _P, c_int64, c_int, c_int64, c_int64, c_float, _P]),
     "kin_qkv_norm_split": (c_int, [_P, c_int64, _P, _P, c_float, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),

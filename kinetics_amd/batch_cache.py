@@ -135,29 +135,40 @@ class PagedBatchKVManager:
         self.pool = ops.PagePool(self.num_pool_pages, B, P, self.page, dev)
         self.kv_cache = [torch.zeros(self.num_pool_pages, 2, self.page, Hkv, D, dtype=dtype, device=dev)
                          for _ in range(self.num_layers)]
+        # mean keys by SLOT; the kernels find a sequence's row block through slot_ids
         self.kbar = [torch.zeros(B, Hkv, P, D, dtype=dtype, device=dev) for _ in range(self.num_layers)]
         self.kv_offset = [torch.zeros(B, dtype=torch.int32, device=dev) for _ in range(self.num_layers)]
-        # page-table metadata (rebuilt on the device each decode call) and full-batch staging buffers
+        # Page-table metadata of the ACTIVE batch (sequence b of a launch = the b-th entry of batch_idx),
+        # built on the device by the first layer of a decode step and reused by the other layers.
         self.page_indices = torch.zeros(self.num_pool_pages, dtype=torch.int32, device=dev)
-        self.page_indptr = torch.zeros(B + 1, dtype=torch.int32, device=dev)
-        self.last_page_len = torch.ones(B, dtype=torch.int32, device=dev)
-        self._lens = torch.zeros(B, dtype=torch.int32, device=dev)
-        self._q = torch.zeros(B, Hq, D, dtype=dtype, device=dev)
-        self._k = torch.zeros(B, Hkv, D, dtype=dtype, device=dev)
-        self._v = torch.zeros(B, Hkv, D, dtype=dtype, device=dev)
-        self._out = torch.zeros(B, Hq, D, dtype=dtype, device=dev)
+        self._indptr = torch.zeros(B + 1, dtype=torch.int32, device=dev)
+        self._last = torch.ones(B, dtype=torch.int32, device=dev)
+        self._one = torch.ones(B, dtype=torch.int32, device=dev)
+        self._slots32 = torch.zeros(B, dtype=torch.int32, device=dev)   # the active slots (fixed address: launch plans keep it)
+        self._slots64 = torch.zeros(B, dtype=torch.int64, device=dev)
+        self._step_batch_idx = None      # the batch_idx object the current table was built for
+        self._step = None                # (n, slots int32, slots int64, indptr view, last view, ones view)
+        self._plans = {}                 # (layer, n) -> ops.DecodeStepPlan of the fused step
+        self._last_layer = -1
         k = self.block_topk or 0
         self._sel = torch.full((B, Hkv, ops.sel_list_capacity(k, self.sink_pages, self.local_tokens)), -1,
                                dtype=torch.int32, device=dev)
         self._cnt = torch.zeros(B, Hkv, dtype=torch.int32, device=dev)
-        self._fused = ops.prefer_fused_step(B, Hkv, P, k)
-        ws = max(ops.decode_workspace_bytes(B, Hq, Hkv, P), ops.decode_workspace_bytes(B, Hq, Hkv, self._sel.shape[2]), 16)
-        if self.token_topk is not None:
-            ws = max(ws, ops.token_topk_workspace_bytes(B, Hkv, P))
-        if self.strided is not None:
-            ws = max(ws, ops.strided_topk_workspace_bytes(B, Hkv, P))
-        ws = max(ws, ops.step_workspace_bytes(B, Hkv, P))
+        # one workspace for every kernel and every number of active sequences
+        sizes = sorted({1 << i for i in range(B.bit_length())} | {B} | set(range(1, min(B, 128) + 1)))
+        ws = 16
+        for n in sizes:
+            ws = max(ws, ops.decode_workspace_bytes(n, Hq, Hkv, P), ops.decode_workspace_bytes(n, Hq, Hkv, self._sel.shape[2]),
+                     ops.step_workspace_bytes(n, Hkv, P))
+            if self.token_topk is not None:
+                ws = max(ws, ops.token_topk_workspace_bytes(n, Hkv, P))
+            if self.strided is not None:
+                ws = max(ws, ops.strided_topk_workspace_bytes(n, Hkv, P))
         self._ws = torch.empty(ws, dtype=torch.uint8, device=dev)
+        # raise at the next decode call, not only in clear_cache, when the pool has flagged trouble (costs a
+        # device-to-host copy per decode step)
+        self.check_overflow_every_step = bool(kwargs.get("check_overflow_every_step", False))
+        self._force_fused = None   # tests: True / False pins the route of the block policy (one launch, or three)
 
     # ------------------------------------------------------------------ LiteSys interface
     def compute_attention(self, query_states, key_states, value_states, layer_idx, batch_idx):
@@ -172,57 +183,92 @@ class PagedBatchKVManager:
     def clear_cache(self, batch_idx: int):
         """batch_cache.py:147-152.  The slot's pages go back to the pool; they need no
         zeroing (an empty page list hides them).  Also the place where trouble that the
-        kernels could only flag is raised: an exhausted pool, a sequence beyond max_seq_len."""
+        kernels could only flag is raised, once: an exhausted pool, a sequence beyond
+        max_seq_len (such a sequence had an empty page list from then on: nothing was
+        written for it and its output was zero)."""
         for i in range(self.num_layers):
             self.kv_offset[i][batch_idx] = 0
         self.pool.release(torch.tensor([int(batch_idx)], dtype=torch.int32, device=self.device))
+        self._step_batch_idx = None
         self.pool.raise_on_overflow()
 
     # ------------------------------------------------------------------ decode
+    def _begin_step(self, batch_idx, layer_idx):
+        """Page table of the active sequences.  The first layer of a decode step grows the slots
+        and builds it (four small launches, no host synchronisation); the other layers of the step
+        -- called in increasing order with the same batch_idx object, as LiteSys' layer loop does
+        (LiteSys/litesys/models/qwen3.py:134-135) -- find every layer's kv_offset at the same value
+        and reuse it."""
+        fresh = (self._step_batch_idx is not batch_idx) or layer_idx <= self._last_layer
+        self._last_layer = layer_idx
+        if fresh:
+            n = batch_idx.numel()
+            self._step_batch_idx = batch_idx
+            self._slots32[:n].copy_(batch_idx, non_blocking=True)
+            self._slots64[:n].copy_(batch_idx, non_blocking=True)
+            self._step = (n, self._slots32[:n], self._slots64[:n], self._indptr[: n + 1], self._last[:n], self._one[:n])
+        n, slots, slots_long, indptr, last, ones = self._step
+        if fresh:
+            if self.check_overflow_every_step:
+                self.pool.raise_on_overflow()
+            lens = self.kv_offset[layer_idx][slots_long] + (self.pad + 1)   # after this step's append
+            # a slot that crossed a page boundary takes a page from the pool
+            self.pool.reserve(lens, slots)
+            self.pool.build_page_table(lens, self.page_indices, indptr, last, slots)
+        return n, slots, indptr, last
+
+    def _advance(self, layer_idx):
+        """kv_offset[layer][batch_idx] += 1 (batch_cache.py:83) for the routes whose kernels do not do it themselves."""
+        self.kv_offset[layer_idx].index_add_(0, self._step[2], self._step[5])
+
     def decode(self, query, key, value, batch_idx, layer_idx):
-        """append -> (select ->) attend for the active slots (batch_cache.py:154-168)."""
-        slots = batch_idx.to(self.device, torch.long)
-        off = self.kv_offset[layer_idx]
-        off[slots] += 1
-        # Sequence b of the kernels == slot b; inactive slots get an empty page list.
-        self._lens.zero_()
-        self._lens[slots] = off[slots] + self.pad
-        # a slot that crossed a page boundary takes a page from the pool (the first layer to get there does it)
-        self.pool.reserve(self._lens)
-        self.pool.build_page_table(self._lens, self.page_indices, self.page_indptr, self.last_page_len)
-        self._q[slots] = query[:, :, 0, :]
-        self._k[slots] = key[:, :, 0, :]
-        self._v[slots] = value[:, :, 0, :]
+        """append -> (select ->) attend for the active slots (batch_cache.py:154-168): q, k, v and
+        the output are indexed by position in the active batch, the caches by slot (through the
+        page table, and slot_ids for the mean keys), as in the reference's kernels
+        (LiteSys/litesys/attention/cache_utils.py:40-51,67-70).  Launches are planned for the active
+        sequences, whatever max_batch_size is."""
+        n, slots, indptr, last = self._begin_step(batch_idx, layer_idx)
+        Hkv = self.num_key_value_heads
+        q, k, v = query[:, :, 0, :], key[:, :, 0, :], value[:, :, 0, :]
+        if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
+            q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        out = torch.empty_like(q)
+        idx = self.page_indices
         kv, kbar = self.kv_cache[layer_idx], self.kbar[layer_idx]
         sparse = self.sparse and layer_idx not in self.layer_skip
         if self.token_topk is not None and layer_idx not in self.layer_skip:
             # token-level top-k: LiteSys' 4 sink tokens, the top tokens of the middle, the newest attn_local tokens
-            ops.append_paged_kv(self._k, self._v, kv, None, self.page_indices, self.page_indptr, self.last_page_len)
-            ops.token_topk_decode(self._q, kv, self.page_indices, self.page_indptr, self.last_page_len, self.token_topk,
-                                  self.pages_per_slot, sink_tokens=4, local_tokens=self.token_local, out=self._out,
-                                  workspace=self._ws)
+            self._advance(layer_idx)
+            ops.append_paged_kv(k, v, kv, None, idx, indptr, last)
+            ops.token_topk_decode(q, kv, idx, indptr, last, self.token_topk, self.pages_per_slot, sink_tokens=4,
+                                  local_tokens=self.token_local, out=out, workspace=self._ws)
         elif self.strided is not None and layer_idx not in self.layer_skip:
-            ops.append_paged_kv(self._k, self._v, kv, None, self.page_indices, self.page_indptr, self.last_page_len)
-            ops.strided_topk_decode(self._q, kv, self.page_indices, self.page_indptr, self.last_page_len, self.strided[0],
-                                    self.pages_per_slot, block_size=self.strided[1], stride=self.strided[2], sink_tokens=4,
-                                    local_tokens=self.token_local, out=self._out, workspace=self._ws)
-        elif sparse and self._fused:
-            ops.blocktopk_decode_step(self._q, self._k, self._v, kv, kbar, self.page_indices, self.page_indptr,
-                                      self.last_page_len, self.block_topk, out=self._out, sink_pages=self.sink_pages,
-                                      local_tokens=self.local_tokens, first_page_offset=self.pad, workspace=self._ws)
+            self._advance(layer_idx)
+            ops.append_paged_kv(k, v, kv, None, idx, indptr, last)
+            ops.strided_topk_decode(q, kv, idx, indptr, last, self.strided[0], self.pages_per_slot,
+                                    block_size=self.strided[1], stride=self.strided[2], sink_tokens=4,
+                                    local_tokens=self.token_local, out=out, workspace=self._ws)
+        elif sparse and (self._force_fused if self._force_fused is not None
+                         else ops.prefer_fused_step(n, Hkv, self.pages_per_slot, self.block_topk)):
+            plan = self._plans.get((layer_idx, n))
+            if plan is None:   # everything but q, k, v, out is the manager's own and stays where it is: bound once
+                plan = self._plans[(layer_idx, n)] = ops.DecodeStepPlan(
+                    kv, kbar, idx, indptr, last, self.block_topk, self.num_attention_heads, sink_pages=self.sink_pages,
+                    local_tokens=self.local_tokens, first_page_offset=self.pad, workspace=self._ws, slot_ids=slots,
+                    slot_lens=self.kv_offset[layer_idx])     # the kernel advances the slots' offsets itself
+            plan(q, k, v, out)
         else:
-            ops.append_paged_kv(self._k, self._v, kv, kbar, self.page_indices, self.page_indptr, self.last_page_len)
+            self._advance(layer_idx)
+            ops.append_paged_kv(k, v, kv, kbar, idx, indptr, last, slot_ids=slots)
             if sparse:
-                ops.block_score_topk(self._q, kbar, self.page_indices, self.page_indptr, self.last_page_len,
-                                     self.block_topk, self._sel, self._cnt, sink_pages=self.sink_pages,
-                                     local_tokens=self.local_tokens, workspace=self._ws, page_size=self.page)
-                ops.sparse_paged_decode(self._q, kv, self._sel, self._cnt, self.last_page_len, out=self._out,
-                                        workspace=self._ws, first_page_offset=self.pad)
+                sel, cnt = self._sel[:n], self._cnt[:n]
+                ops.block_score_topk(q, kbar, idx, indptr, last, self.block_topk, sel, cnt, sink_pages=self.sink_pages,
+                                     local_tokens=self.local_tokens, workspace=self._ws, page_size=self.page, slot_ids=slots)
+                ops.sparse_paged_decode(q, kv, sel, cnt, last, out=out, workspace=self._ws, first_page_offset=self.pad)
             else:
-                ops.dense_paged_decode(self._q, kv, self.page_indices, self.page_indptr, self.last_page_len,
-                                       self.pages_per_slot, out=self._out, workspace=self._ws,
+                ops.dense_paged_decode(q, kv, idx, indptr, last, self.pages_per_slot, out=out, workspace=self._ws,
                                        first_page_offset=self.pad)
-        return self._out[slots]
+        return out
 
     # ------------------------------------------------------------------ prefill (not the accelerated path)
     def prefill_or_append(self, query_states, key_states, value_states, layer_idx, batch_idx):
@@ -237,13 +283,16 @@ class PagedBatchKVManager:
         if total + pad > self.pages_per_slot * self.page:
             raise ValueError(f"sequence of {total} tokens exceeds max_seq_len")
         Hkv, D = self.num_key_value_heads, self.head_dim
-        self.kv_offset[layer_idx][slot] += seq_len
         n_pages = (total + pad + self.page - 1) // self.page
+        self._step_batch_idx = None   # the next decode step builds its table afresh
         self.pool.reserve(torch.tensor([total + pad], dtype=torch.int32, device=self.device),
                           torch.tensor([slot], dtype=torch.int32, device=self.device))
         free, bits = self.pool.status()
         if bits & ops.PagePool.EXHAUSTED:
+            # nothing was reserved and nothing is recorded: the request can be retried after a clear_cache
+            self.pool.acknowledge()
             raise _lib.KineticsError(f"page pool exhausted ({free} pages free): cannot hold {total} tokens in slot {slot}")
+        self.kv_offset[layer_idx][slot] += seq_len
         idx = self.pool.slot_table[slot, :n_pages].contiguous()
         ptr = torch.tensor([0, n_pages], dtype=torch.int32, device=self.device)
         last = torch.tensor([total + pad - (n_pages - 1) * self.page], dtype=torch.int32, device=self.device)

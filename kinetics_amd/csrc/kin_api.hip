@@ -89,7 +89,7 @@ __global__ void check_page_table_kernel(const int32_t* __restrict__ page_indices
 
 extern "C" {
 
-int kin_version(void) { return 20200; }
+int kin_version(void) { return 30000; }
 
 int kin_sel_list_capacity(int topk, int sink_pages, int local_tokens) {
   if (topk < 0 || sink_pages < 0 || local_tokens < 1) return 0;

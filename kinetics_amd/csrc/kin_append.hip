@@ -15,6 +15,8 @@ struct AppendParams {
   const int32_t* last_page_len;
   int batch, num_kv_heads, kbar_pages, page_size;
   int64_t num_pages;
+  const int32_t* slot_ids;  // kbar row block of each sequence (null: the sequence's own index)
+  int num_slots;
 };
 
 // grid = ceil(batch*Hkv / 4) blocks of 256 threads; one wave per (sequence, head).
@@ -27,8 +29,9 @@ __global__ __launch_bounds__(256) void append_kernel(AppendParams p) {
   const int s = p.page_indptr[b], e = p.page_indptr[b + 1];
   const int n_pages = e - s;
   if (n_pages <= 0) return;
-  uint32_t* kbar_row = p.kbar ? p.kbar + kbar_row_index(b, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2)
-                              : nullptr;
+  const int kb = kbar_block_of(p.slot_ids, p.num_slots, b);
+  uint32_t* kbar_row = (p.kbar && kb >= 0) ? p.kbar + kbar_row_index(kb, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2)
+                                           : nullptr;
   append_token_row<F16>(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2), p.kv_cache, kbar_row,
                    p.page_indices[e - 1], p.last_page_len[b], n_pages, p.kbar_pages, h, p.num_kv_heads, p.num_pages, lane,
                    p.page_size);
@@ -52,6 +55,8 @@ __global__ __launch_bounds__(256) void build_kbar_kernel(AppendParams p, int pag
   if (page >= n_full || page >= p.kbar_pages) return;
   const int64_t pid = p.page_indices[s + page];
   if (pid < 0 || pid >= p.num_pages) return;
+  const int kb = kbar_block_of(p.slot_ids, p.num_slots, b);
+  if (kb < 0) return;
   const int row_stride = p.num_kv_heads * (kHeadDim / 2);  // dwords per token row
   const int64_t page_dwords = 2LL * p.page_size * row_stride;
   const u32x4* kplane = reinterpret_cast<const u32x4*>(p.kv_cache + pid * page_dwords + h * (kHeadDim / 2)) + c16;
@@ -59,7 +64,7 @@ __global__ __launch_bounds__(256) void build_kbar_kernel(AppendParams p, int pag
   // Streaming store: the mean keys are not read again by this launch.  (Stores that leave the caches while the
   // read stream is saturated cost about five times their bytes: 2.1 GB of them take the config-1 build from
   // 4.95 to 6.97 ms with a plain store, 6.55 ms with this one; writing them in 64 KiB bursts changes nothing.)
-  __builtin_nontemporal_store(m, reinterpret_cast<u32x4*>(p.kbar + kbar_row_index(b, h, page, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2)) + c16);
+  __builtin_nontemporal_store(m, reinterpret_cast<u32x4*>(p.kbar + kbar_row_index(kb, h, page, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2)) + c16);
 }
 
 // ---- ragged multi-token append ------------------------------------------------
@@ -75,6 +80,8 @@ struct RaggedAppendParams {
   int batch, num_kv_heads, kbar_pages, page_size;
   int64_t nnz;
   int64_t num_pages;
+  const int32_t* slot_ids;  // kbar row block of each sequence (null: the sequence's own index)
+  int num_slots;
 };
 
 // Sequence that owns appended row `row`: the last b with append_indptr[b] <= row.
@@ -185,9 +192,10 @@ __global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p)
         const int64_t page = pos / P;
         if (pos >= 0 && pos % P == P - 1 && page < p.kbar_pages) {
           const int64_t pid = p.page_indices[s + (int)page];
-          if (pid >= 0 && pid < p.num_pages) {
+          const int kb = kbar_block_of(p.slot_ids, p.num_slots, b);
+          if (pid >= 0 && pid < p.num_pages && kb >= 0) {
             src = pid * 2 * P * cpr;
-            dst = kbar_row_index(b, 0, (int)page, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 8);
+            dst = kbar_row_index(kb, 0, (int)page, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 8);
           }
         }
       }
@@ -210,7 +218,9 @@ __global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p)
 
 static int check_append_args(const char* fn, const void* kv_cache, const void* page_indices,
                              const void* page_indptr, const void* last_page_len, int batch, int num_kv_heads,
-                             int head_dim, int page_size, int64_t num_pages, int kbar_pages, bool has_kbar) {
+                             int head_dim, int page_size, int64_t num_pages, int kbar_pages, bool has_kbar,
+                             const int32_t* slot_ids, int num_slots) {
+  if (slot_ids && num_slots < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_slots=%d must be >= 1 when slot_ids is given", fn, num_slots);
   if (!kv_cache || !page_indices || !page_indptr || !last_page_len)
     return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_common_dims(fn, batch, num_kv_heads, num_kv_heads, head_dim, page_size);
@@ -229,11 +239,11 @@ extern "C" {
 static int append_impl(const char* fn, bool f16, const uint16_t* k, const uint16_t* v, uint16_t* kv_cache, uint16_t* kbar,
                        const int32_t* page_indices, const int32_t* page_indptr, const int32_t* last_page_len,
                        int batch, int num_kv_heads, int head_dim, int page_size, int64_t num_pages,
-                       int kbar_pages, kin_stream_t stream) {
+                       int kbar_pages, const int32_t* slot_ids, int num_slots, kin_stream_t stream) {
   using namespace kin;
   if (!k || !v) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_append_args(fn, kv_cache, page_indices, page_indptr, last_page_len, batch, num_kv_heads,
-                             head_dim, page_size, num_pages, kbar_pages, kbar != nullptr);
+                             head_dim, page_size, num_pages, kbar_pages, kbar != nullptr, slot_ids, num_slots);
   if (st) return st;
   if (!aligned16(k) || !aligned16(v) || (kbar && !aligned16(kbar)))
     return fail(KIN_ERR_MISALIGNED, "%s: k, v and kbar must be 16-byte aligned", fn);
@@ -251,6 +261,8 @@ static int append_impl(const char* fn, bool f16, const uint16_t* k, const uint16
   p.kbar_pages = kbar_pages;
   p.page_size = page_size;
   p.num_pages = num_pages;
+  p.slot_ids = slot_ids;
+  p.num_slots = slot_ids ? num_slots : batch;
   const int64_t items = (int64_t)batch * num_kv_heads;
   const unsigned blocks = (unsigned)((items + 3) / 4);
   if (f16) append_kernel<true><<<blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(p);
@@ -261,26 +273,26 @@ static int append_impl(const char* fn, bool f16, const uint16_t* k, const uint16
 int kin_append_paged_kv(const kin_bf16_t* k, const kin_bf16_t* v, kin_bf16_t* kv_cache, kin_bf16_t* kbar,
                         const int32_t* page_indices, const int32_t* page_indptr, const int32_t* last_page_len,
                         int batch, int num_kv_heads, int head_dim, int page_size, int64_t num_pages,
-                        int kbar_pages, kin_stream_t stream) {
+                        int kbar_pages, const int32_t* slot_ids, int num_slots, kin_stream_t stream) {
   return append_impl("kin_append_paged_kv", false, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, batch,
-                     num_kv_heads, head_dim, page_size, num_pages, kbar_pages, stream);
+                     num_kv_heads, head_dim, page_size, num_pages, kbar_pages, slot_ids, num_slots, stream);
 }
 
 int kin_append_paged_kv_f16(const kin_f16_t* k, const kin_f16_t* v, kin_f16_t* kv_cache, kin_f16_t* kbar,
                             const int32_t* page_indices, const int32_t* page_indptr, const int32_t* last_page_len,
                             int batch, int num_kv_heads, int head_dim, int page_size, int64_t num_pages,
-                            int kbar_pages, kin_stream_t stream) {
+                            int kbar_pages, const int32_t* slot_ids, int num_slots, kin_stream_t stream) {
   return append_impl("kin_append_paged_kv_f16", true, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, batch,
-                     num_kv_heads, head_dim, page_size, num_pages, kbar_pages, stream);
+                     num_kv_heads, head_dim, page_size, num_pages, kbar_pages, slot_ids, num_slots, stream);
 }
 
 static int build_kbar_impl(const char* fn, bool f16, const uint16_t* kv_cache, uint16_t* kbar, const int32_t* page_indices,
                            const int32_t* page_indptr, const int32_t* last_page_len, int batch, int num_kv_heads,
-                           int head_dim, int page_size, int64_t num_pages, int kbar_pages, kin_stream_t stream) {
+                           int head_dim, int page_size, int64_t num_pages, int kbar_pages, const int32_t* slot_ids, int num_slots, kin_stream_t stream) {
   using namespace kin;
   if (!kbar) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_append_args(fn, kv_cache, page_indices, page_indptr, last_page_len, batch, num_kv_heads,
-                             head_dim, page_size, num_pages, kbar_pages, true);
+                             head_dim, page_size, num_pages, kbar_pages, true, slot_ids, num_slots);
   if (st) return st;
   if (!aligned16(kbar)) return fail(KIN_ERR_MISALIGNED, "%s: kbar must be 16-byte aligned", fn);
   if (batch == 0) return KIN_OK;
@@ -301,6 +313,8 @@ static int build_kbar_impl(const char* fn, bool f16, const uint16_t* kv_cache, u
   p.kbar_pages = kbar_pages;
   p.page_size = page_size;
   p.num_pages = num_pages;
+  p.slot_ids = slot_ids;
+  p.num_slots = slot_ids ? num_slots : batch;
   if (f16) build_kbar_kernel<true><<<(unsigned)(items * page_blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(p, page_blocks);
   else build_kbar_kernel<false><<<(unsigned)(items * page_blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(p, page_blocks);
   return check_hip(hipGetLastError(), "build_kbar_kernel launch");
@@ -308,27 +322,27 @@ static int build_kbar_impl(const char* fn, bool f16, const uint16_t* kv_cache, u
 
 int kin_build_kbar(const kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
                    const int32_t* page_indptr, const int32_t* last_page_len, int batch, int num_kv_heads,
-                   int head_dim, int page_size, int64_t num_pages, int kbar_pages, kin_stream_t stream) {
+                   int head_dim, int page_size, int64_t num_pages, int kbar_pages, const int32_t* slot_ids, int num_slots, kin_stream_t stream) {
   return build_kbar_impl("kin_build_kbar", false, kv_cache, kbar, page_indices, page_indptr, last_page_len, batch, num_kv_heads,
-                         head_dim, page_size, num_pages, kbar_pages, stream);
+                         head_dim, page_size, num_pages, kbar_pages, slot_ids, num_slots, stream);
 }
 
 int kin_build_kbar_f16(const kin_f16_t* kv_cache, kin_f16_t* kbar, const int32_t* page_indices,
                        const int32_t* page_indptr, const int32_t* last_page_len, int batch, int num_kv_heads,
-                       int head_dim, int page_size, int64_t num_pages, int kbar_pages, kin_stream_t stream) {
+                       int head_dim, int page_size, int64_t num_pages, int kbar_pages, const int32_t* slot_ids, int num_slots, kin_stream_t stream) {
   return build_kbar_impl("kin_build_kbar_f16", true, kv_cache, kbar, page_indices, page_indptr, last_page_len, batch,
-                         num_kv_heads, head_dim, page_size, num_pages, kbar_pages, stream);
+                         num_kv_heads, head_dim, page_size, num_pages, kbar_pages, slot_ids, num_slots, stream);
 }
 
 static int append_ragged_impl(const char* fn, bool f16, const uint16_t* k, const uint16_t* v, const int32_t* append_indptr,
                               uint16_t* kv_cache, uint16_t* kbar, const int32_t* page_indices,
                               const int32_t* page_indptr, const int32_t* last_page_len, int batch, int64_t nnz,
                               int max_append_len, int num_kv_heads, int head_dim, int page_size,
-                              int64_t num_pages, int kbar_pages, kin_stream_t stream) {
+                              int64_t num_pages, int kbar_pages, const int32_t* slot_ids, int num_slots, kin_stream_t stream) {
   using namespace kin;
   if (!k || !v || !append_indptr) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_append_args(fn, kv_cache, page_indices, page_indptr, last_page_len, batch, num_kv_heads,
-                             head_dim, page_size, num_pages, kbar_pages, kbar != nullptr);
+                             head_dim, page_size, num_pages, kbar_pages, kbar != nullptr, slot_ids, num_slots);
   if (st) return st;
   if (nnz < 0 || max_append_len < 0 || max_append_len > nnz)
     return fail(KIN_ERR_BAD_SHAPE, "%s: nnz=%lld and max_append_len=%d must satisfy 0 <= max_append_len <= nnz", fn,
@@ -353,6 +367,8 @@ static int append_ragged_impl(const char* fn, bool f16, const uint16_t* k, const
   p.page_size = page_size;
   p.nnz = nnz;
   p.num_pages = num_pages;
+  p.slot_ids = slot_ids;
+  p.num_slots = slot_ids ? num_slots : batch;
   hipStream_t s = static_cast<hipStream_t>(stream);
   append_ragged_kernel<<<(unsigned)blocks, 256, 0, s>>>(p);
   st = check_hip(hipGetLastError(), "append_ragged_kernel launch");
@@ -366,20 +382,20 @@ int kin_append_paged_kv_ragged(const kin_bf16_t* k, const kin_bf16_t* v, const i
                                kin_bf16_t* kv_cache, kin_bf16_t* kbar, const int32_t* page_indices,
                                const int32_t* page_indptr, const int32_t* last_page_len, int batch, int64_t nnz,
                                int max_append_len, int num_kv_heads, int head_dim, int page_size,
-                               int64_t num_pages, int kbar_pages, kin_stream_t stream) {
+                               int64_t num_pages, int kbar_pages, const int32_t* slot_ids, int num_slots, kin_stream_t stream) {
   return append_ragged_impl("kin_append_paged_kv_ragged", false, k, v, append_indptr, kv_cache, kbar, page_indices, page_indptr,
                             last_page_len, batch, nnz, max_append_len, num_kv_heads, head_dim, page_size, num_pages,
-                            kbar_pages, stream);
+                            kbar_pages, slot_ids, num_slots, stream);
 }
 
 int kin_append_paged_kv_ragged_f16(const kin_f16_t* k, const kin_f16_t* v, const int32_t* append_indptr,
                                    kin_f16_t* kv_cache, kin_f16_t* kbar, const int32_t* page_indices,
                                    const int32_t* page_indptr, const int32_t* last_page_len, int batch, int64_t nnz,
                                    int max_append_len, int num_kv_heads, int head_dim, int page_size,
-                                   int64_t num_pages, int kbar_pages, kin_stream_t stream) {
+                                   int64_t num_pages, int kbar_pages, const int32_t* slot_ids, int num_slots, kin_stream_t stream) {
   return append_ragged_impl("kin_append_paged_kv_ragged_f16", true, k, v, append_indptr, kv_cache, kbar, page_indices,
                             page_indptr, last_page_len, batch, nnz, max_append_len, num_kv_heads, head_dim, page_size,
-                            num_pages, kbar_pages, stream);
+                            num_pages, kbar_pages, slot_ids, num_slots, stream);
 }
 
 }  // extern "C"

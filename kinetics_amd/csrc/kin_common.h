@@ -95,6 +95,15 @@ __host__ __device__ inline int64_t kbar_row_index(int b, int h, int page, int nu
 // ---- device side -----------------------------------------------------------
 #if defined(__HIPCC__)
 
+// Row block of kbar that holds the mean keys of sequence b: b itself, or slot_ids[b] when the
+// caller keeps kbar by cache slot (a serving engine's active batch is a changing subset of its
+// slots, and q, k, v, out and the page table follow the batch while the mean keys stay with
+// the slot).  -1 for an id outside [0, num_slots): such a sequence has no mean keys.
+__device__ __forceinline__ int kbar_block_of(const int32_t* slot_ids, int num_slots, int b) {
+  const int s = slot_ids ? slot_ids[b] : b;
+  return (unsigned)s < (unsigned)num_slots ? s : -1;
+}
+
 // Workgroups are handed to the GPU's 8 XCDs round-robin by index; every XCD has
 // its own L2 and address-translation caches.  The lists of one sequence's KV
 // heads read different parts of the same KV pages and the same page-table

@@ -24,6 +24,8 @@ struct ScoreTopkParams {
   int chunks;          // workgroups per list
   int32_t* ws_count;   // [lists] arrival counters, zero at launch and left zero
   uint32_t* ws_keys;   // [lists, score_key_stride(kbar_pages)]
+  const int32_t* slot_ids;  // kbar row block of each sequence (null: the sequence's own index)
+  int num_slots;
 };
 
 // Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap] | int32 table[table_cap] |
@@ -57,8 +59,10 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
   a.q_bh = p.q + ((int64_t)b * p.num_q_heads + (int64_t)h * p.group) * kHeadDim;
   a.G = p.group;
   a.n_pages = n_pages;
-  split_pages(n_pages, p.last_page_len[b], p.sink_pages, p.local_tokens, p.kbar_pages, p.page_size, a.n_sink, a.n_cand, a.n_local);
-  a.kb = reinterpret_cast<const char*>(p.kbar) + kbar_row_index(b, h, a.n_sink, p.num_kv_heads, p.kbar_pages) * kRowBytes;
+  const int kb = kbar_block_of(p.slot_ids, p.num_slots, b);  // (a sequence without mean keys has no candidates)
+  split_pages(n_pages, p.last_page_len[b], p.sink_pages, p.local_tokens, kb >= 0 ? p.kbar_pages : 0, p.page_size, a.n_sink, a.n_cand,
+              a.n_local);
+  a.kb = reinterpret_cast<const char*>(p.kbar) + kbar_row_index(max(kb, 0), h, a.n_sink, p.num_kv_heads, p.kbar_pages) * kRowBytes;
   a.topk = p.topk;
   a.table = p.page_indices + ps;
   a.sel_logical = p.sel_logical ? p.sel_logical + (int64_t)item * p.topk : nullptr;
@@ -112,7 +116,8 @@ static int score_topk_impl(const char* fn, bool f16, const uint16_t* q, const ui
                            int32_t* sel_pages, int32_t* sel_count,
                            int32_t* sel_logical, float* scores_out, int batch, int num_q_heads,
                            int num_kv_heads, int head_dim, int page_size, int kbar_pages, int sel_stride,
-                           void* workspace, size_t workspace_bytes, kin_stream_t stream) {
+                           void* workspace, size_t workspace_bytes, const int32_t* slot_ids, int num_slots,
+                           kin_stream_t stream) {
   if (!q || !kbar || !page_indices || !page_indptr || !last_page_len || !sel_pages || !sel_count)
     return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size);
@@ -125,6 +130,7 @@ static int score_topk_impl(const char* fn, bool f16, const uint16_t* q, const ui
     return fail(KIN_ERR_BAD_SHAPE, "%s: sel_stride=%d must be at least kin_sel_list_capacity(topk, sink_pages, local_tokens) = %d",
                 fn, sel_stride, list_cap);
   if (kbar_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: kbar_pages=%d must be >= 1", fn, kbar_pages);
+  if (slot_ids && num_slots < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_slots=%d must be >= 1 when slot_ids is given", fn, num_slots);
   if (topk > kMaxTopk) return fail(KIN_ERR_UNSUPPORTED, "%s: topk=%d exceeds the limit %d", fn, topk, kMaxTopk);
   if (kbar_pages > kMaxCandidates)
     return fail(KIN_ERR_UNSUPPORTED, "%s: kbar_pages=%d exceeds the limit %d", fn, kbar_pages, kMaxCandidates);
@@ -151,6 +157,8 @@ static int score_topk_impl(const char* fn, bool f16, const uint16_t* q, const ui
   p.sink_pages = sink_pages;
   p.local_tokens = local_tokens;
   p.page_size = page_size;
+  p.slot_ids = slot_ids;
+  p.num_slots = slot_ids ? num_slots : batch;
   p.sort_cap = select_sort_cap(topk, kbar_pages);
   p.table_cap = select_table_cap(kbar_pages + max_local_pages(local_tokens) + 1);
   const size_t lds = select_lds_bytes(kbar_pages, p.sort_cap, p.table_cap) + (size_t)list_cap * 4;
@@ -201,10 +209,11 @@ extern "C" int kin_block_score_topk(const kin_bf16_t* q, const kin_bf16_t* kbar,
                                     int sink_pages, int local_tokens, int32_t* sel_pages, int32_t* sel_count,
                                     int32_t* sel_logical, float* scores_out, int batch, int num_q_heads,
                                     int num_kv_heads, int head_dim, int page_size, int kbar_pages, int sel_stride,
-                                    void* workspace, size_t workspace_bytes, kin_stream_t stream) {
+                                    void* workspace, size_t workspace_bytes, const int32_t* slot_ids, int num_slots,
+                                    kin_stream_t stream) {
   return kin::score_topk_impl("kin_block_score_topk", false, q, kbar, page_indices, page_indptr, last_page_len, topk,
                               sink_pages, local_tokens, sel_pages, sel_count, sel_logical, scores_out, batch, num_q_heads,
-                              num_kv_heads, head_dim, page_size, kbar_pages, sel_stride, workspace, workspace_bytes, stream);
+                              num_kv_heads, head_dim, page_size, kbar_pages, sel_stride, workspace, workspace_bytes, slot_ids, num_slots, stream);
 }
 
 extern "C" int kin_block_score_topk_f16(const kin_f16_t* q, const kin_f16_t* kbar, const int32_t* page_indices,
@@ -212,8 +221,9 @@ extern "C" int kin_block_score_topk_f16(const kin_f16_t* q, const kin_f16_t* kba
                                         int sink_pages, int local_tokens, int32_t* sel_pages, int32_t* sel_count,
                                         int32_t* sel_logical, float* scores_out, int batch, int num_q_heads,
                                         int num_kv_heads, int head_dim, int page_size, int kbar_pages, int sel_stride,
-                                        void* workspace, size_t workspace_bytes, kin_stream_t stream) {
+                                        void* workspace, size_t workspace_bytes, const int32_t* slot_ids, int num_slots,
+                                        kin_stream_t stream) {
   return kin::score_topk_impl("kin_block_score_topk_f16", true, q, kbar, page_indices, page_indptr, last_page_len, topk,
                               sink_pages, local_tokens, sel_pages, sel_count, sel_logical, scores_out, batch, num_q_heads,
-                              num_kv_heads, head_dim, page_size, kbar_pages, sel_stride, workspace, workspace_bytes, stream);
+                              num_kv_heads, head_dim, page_size, kbar_pages, sel_stride, workspace, workspace_bytes, slot_ids, num_slots, stream);
 }

@@ -37,6 +37,9 @@ struct StepParams {
   uint32_t* ws_keys;   // [team lists, score_key_stride(kbar_pages)]
   uint32_t* ws_po;     // [team lists, parts, group, 128] fp32 bits: normalised partial outputs
   uint32_t* ws_plse;   // [team lists, parts, group] fp32 bits: base-2 log-sum-exp of the parts
+  const int32_t* slot_ids;  // kbar row block of each sequence (null: the sequence's own index)
+  int num_slots;
+  int32_t* slot_lens;       // optional [num_slots]: token count of each slot, advanced by one per appended token
   int64_t num_pages;
   float scale_log2;
   int deep_score;      // few lists: more mean-key loads in flight per lane (see the kernel)

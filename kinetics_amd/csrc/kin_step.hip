@@ -58,6 +58,11 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   const int G = p.group;
   const int64_t hq0 = (int64_t)b * p.num_q_heads + (int64_t)h * G;
 
+  // The caller's per-slot token counter (a KV manager's kv_offset) follows the append: one thread per sequence.
+  if (p.slot_lens && p.k && h == 0 && member == 0 && tid == 0) {
+    const int sl = p.slot_ids ? p.slot_ids[b] : b;
+    if ((unsigned)sl < (unsigned)p.num_slots) p.slot_lens[sl] += 1;
+  }
   const int ps = p.page_indptr[b], pe = p.page_indptr[b + 1];
   const int n_pages = pe - ps;
   if (n_pages <= 0) {  // empty sequence: nothing to append, select or attend (every member sees that)
@@ -70,13 +75,15 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     return;
   }
   const int last_len = p.last_page_len[b];
+  const int kb = kbar_block_of(p.slot_ids, p.num_slots, b);  // (a sequence without mean keys has no candidates)
 
   // ---- append (wave 0): same byte moves and mean-key update as append_kernel ----
   // In a team the member that attends the sequence's last page does it (see below).
   auto append_token = [&]() {
     if (p.k != nullptr && tid < 64) {
-      uint32_t* kbar_row =
-          reinterpret_cast<uint32_t*>(p.kbar) + kbar_row_index(b, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2);
+      uint32_t* kbar_row = kb < 0 ? nullptr
+                                  : reinterpret_cast<uint32_t*>(p.kbar) +
+                                        kbar_row_index(kb, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2);
       append_token_row<F16>(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2),
                        reinterpret_cast<uint32_t*>(p.kv), kbar_row, p.page_indices[pe - 1], last_len, n_pages, p.kbar_pages, h,
                        p.num_kv_heads, p.num_pages, tid, p.page_size);
@@ -93,8 +100,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   s.q_bh = p.q + hq0 * kHeadDim;
   s.G = G;
   s.n_pages = n_pages;
-  split_pages(n_pages, last_len, p.sink_pages, p.local_tokens, p.kbar_pages, p.page_size, s.n_sink, s.n_cand, s.n_local);
-  s.kb = reinterpret_cast<const char*>(p.kbar) + kbar_row_index(b, h, s.n_sink, p.num_kv_heads, p.kbar_pages) * kRowBytes;
+  split_pages(n_pages, last_len, p.sink_pages, p.local_tokens, kb >= 0 ? p.kbar_pages : 0, p.page_size, s.n_sink, s.n_cand, s.n_local);
+  s.kb = reinterpret_cast<const char*>(p.kbar) + kbar_row_index(max(kb, 0), h, s.n_sink, p.num_kv_heads, p.kbar_pages) * kRowBytes;
   s.topk = p.topk;
   s.table = p.page_indices + ps;
   s.sel_logical = nullptr;
@@ -351,7 +358,8 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
                        int local_tokens, int32_t* sel_pages, int32_t* sel_count, kin_bf16_t* out, float* lse,
                        int batch, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
                        int64_t num_pages, int kbar_pages, int sel_stride, int first_page_offset, float sm_scale,
-                       void* workspace, size_t workspace_bytes, kin_stream_t stream) {
+                       void* workspace, size_t workspace_bytes, const int32_t* slot_ids, int num_slots, int32_t* slot_lens,
+                       kin_stream_t stream) {
   if (!q || !kv_cache || !kbar || !page_indices || !page_indptr || !last_page_len || !out)
     return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   if ((k == nullptr) != (v == nullptr))
@@ -361,6 +369,7 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
   if (num_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_pages=%lld must be >= 1", fn, (long long)num_pages);
   if (topk < 0) return fail(KIN_ERR_BAD_SHAPE, "%s: topk=%d is negative", fn, topk);
   if (kbar_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: kbar_pages=%d must be >= 1", fn, kbar_pages);
+  if (slot_ids && num_slots < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_slots=%d must be >= 1 when slot_ids is given", fn, num_slots);
   st = check_fixed_pages(fn, sink_pages, local_tokens);
   if (st) return st;
   st = check_first_page_offset(fn, first_page_offset, page_size);
@@ -405,6 +414,9 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
   p.local_tokens = local_tokens;
   p.first_page_offset = first_page_offset;
   p.page_size = page_size;
+  p.slot_ids = slot_ids;
+  p.num_slots = slot_ids ? num_slots : batch;
+  p.slot_lens = slot_lens;
   p.sort_cap = select_sort_cap(topk, kbar_pages);
   p.table_cap = select_table_cap(kbar_pages + max_local_pages(local_tokens) + 1);
   const int64_t items = (int64_t)batch * num_kv_heads;
@@ -514,11 +526,12 @@ extern "C" int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* 
                                          kin_bf16_t* out, float* lse, int batch, int num_q_heads, int num_kv_heads,
                                          int head_dim, int page_size, int64_t num_pages, int kbar_pages,
                                          int sel_stride, int first_page_offset, float sm_scale, void* workspace,
-                                         size_t workspace_bytes, kin_stream_t stream) {
+                                         size_t workspace_bytes, const int32_t* slot_ids, int num_slots,
+                                         int32_t* slot_lens, kin_stream_t stream) {
   return kin::launch_step("kin_blocktopk_decode_step", false, q, k, v, kv_cache, kbar, page_indices, page_indptr,
                           last_page_len, topk, sink_pages, local_tokens, sel_pages, sel_count, out, lse, batch, num_q_heads,
                           num_kv_heads, head_dim, page_size, num_pages, kbar_pages, sel_stride, first_page_offset, sm_scale,
-                          workspace, workspace_bytes, stream);
+                          workspace, workspace_bytes, slot_ids, num_slots, slot_lens, stream);
 }
 
 extern "C" int kin_blocktopk_decode_step_f16(const kin_f16_t* q, const kin_f16_t* k, const kin_f16_t* v,
@@ -528,11 +541,12 @@ extern "C" int kin_blocktopk_decode_step_f16(const kin_f16_t* q, const kin_f16_t
                                              kin_f16_t* out, float* lse, int batch, int num_q_heads, int num_kv_heads,
                                              int head_dim, int page_size, int64_t num_pages, int kbar_pages,
                                              int sel_stride, int first_page_offset, float sm_scale, void* workspace,
-                                             size_t workspace_bytes, kin_stream_t stream) {
+                                             size_t workspace_bytes, const int32_t* slot_ids, int num_slots,
+                                             int32_t* slot_lens, kin_stream_t stream) {
   return kin::launch_step("kin_blocktopk_decode_step_f16", true, q, k, v, kv_cache, kbar, page_indices, page_indptr,
                           last_page_len, topk, sink_pages, local_tokens, sel_pages, sel_count, out, lse, batch, num_q_heads,
                           num_kv_heads, head_dim, page_size, num_pages, kbar_pages, sel_stride, first_page_offset, sm_scale,
-                          workspace, workspace_bytes, stream);
+                          workspace, workspace_bytes, slot_ids, num_slots, slot_lens, stream);
 }
 
 #ifdef KIN_TUNE
@@ -548,7 +562,8 @@ extern "C" int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_b
                                                 int32_t* sel_count, kin_bf16_t* out, float* lse, int batch,
                                                 int num_q_heads, int num_kv_heads, int head_dim, int page_size,
                                                 int64_t num_pages, int kbar_pages, int sel_stride,
-                                                int first_page_offset, float sm_scale, kin_stream_t stream) {
+                                                int first_page_offset, float sm_scale, const int32_t* slot_ids,
+                                                int num_slots, int32_t* slot_lens, kin_stream_t stream) {
   using namespace kin;
   const char* fn = "kin_blocktopk_decode_step_static";
   // What the teams of this shape need, from the dimensions alone.  With few lists (up to one for
@@ -576,5 +591,6 @@ extern "C" int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_b
   }
   return launch_step(fn, false, q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sink_pages, local_tokens,
                      sel_pages, sel_count, out, lse, batch, num_q_heads, num_kv_heads, head_dim, page_size, num_pages,
-                     kbar_pages, sel_stride, first_page_offset, sm_scale, ws, ws ? kStaticScratchBytes : 0, stream);
+                     kbar_pages, sel_stride, first_page_offset, sm_scale, ws, ws ? kStaticScratchBytes : 0, slot_ids, num_slots,
+                     slot_lens, stream);
 }

@@ -8,13 +8,18 @@
 namespace kin {
 
 // One 1024-thread workgroup: n_pages, last_page_len and the exclusive scan.
-// slot_npages (may be null): pages slot s really owns; a sequence is cut to them.
+// slot_npages (may be null): pages slot s really owns.  A sequence that its slot cannot hold
+// -- longer than pages_per_slot pages, or than the pages the slot owns because a reserve
+// failed -- gets an EMPTY page list: the kernels then write nothing for it and return
+// zeros, instead of appending into the wrong token slot of a truncated list.  So does a
+// sequence whose slot id lies outside [0, max_slots).
 __global__ __launch_bounds__(1024) void slot_table_scan_kernel(const int32_t* __restrict__ seq_lens, int batch,
                                                                int pages_per_slot, int page_size,
                                                                int32_t* __restrict__ page_indptr,
                                                                int32_t* __restrict__ last_page_len,
                                                                const int32_t* __restrict__ slot_ids = nullptr,
-                                                               const int32_t* __restrict__ slot_npages = nullptr) {
+                                                               const int32_t* __restrict__ slot_npages = nullptr,
+                                                               int max_slots = 0x7fffffff) {
   __shared__ int wave_sum[16];
   __shared__ int carry_sh;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -28,10 +33,12 @@ __global__ __launch_bounds__(1024) void slot_table_scan_kernel(const int32_t* __
     int n = 0;
     if (b < batch) {
       const int len = max(seq_lens[b], 0);
-      n = min((len + page_size - 1) / page_size, pages_per_slot);
-      if (slot_npages) n = min(n, slot_npages[slot_ids ? slot_ids[b] : b]);
-      const int tokens = min(len, n * page_size);
-      last_page_len[b] = (n > 0) ? tokens - (n - 1) * page_size : 1;
+      n = (len + page_size - 1) / page_size;
+      const int slot = slot_ids ? slot_ids[b] : b;
+      const bool slot_ok = (unsigned)slot < (unsigned)max_slots;
+      const int owned = !slot_ok ? 0 : (slot_npages ? min(slot_npages[slot], pages_per_slot) : pages_per_slot);
+      if (n > owned) n = 0;
+      last_page_len[b] = (n > 0) ? len - (n - 1) * page_size : 1;
     }
     int incl = n;
 #pragma unroll
@@ -60,7 +67,7 @@ __global__ __launch_bounds__(256) void slot_table_fill_kernel(const int32_t* __r
   const int p = blockIdx.x * 256 + threadIdx.x;
   const int s = page_indptr[b], n = page_indptr[b + 1] - s;
   if (p >= n) return;
-  const int slot = slot_ids ? slot_ids[b] : b;
+  const int slot = slot_ids ? slot_ids[b] : b;  // (in range: the scan gave other sequences an empty list)
   const int64_t e = (int64_t)slot * pages_per_slot + p;
   page_indices[s + p] = slot_table ? slot_table[e] : (int32_t)e;
 }
@@ -68,7 +75,9 @@ __global__ __launch_bounds__(256) void slot_table_fill_kernel(const int32_t* __r
 // ---- page pool: a free list on the device -------------------------------------
 // pool_state[0] = pages on the free stack, pool_state[1] = status bits.
 constexpr int kPoolExhausted = 1;   // a reserve call wanted more pages than were free: it reserved nothing
-constexpr int kPoolSlotTooLong = 2; // a sequence wanted more than pages_per_slot pages: clamped
+constexpr int kPoolSlotTooLong = 2; // a sequence wanted more than pages_per_slot pages: its slot got pages_per_slot
+constexpr int kPoolBadSlot = 4;     // a slot id outside [0, max_slots), or listed twice in one call: that entry was skipped
+constexpr int kPoolMark = 1 << 24;  // added to slot_npages[s] while a reserve call checks its ids for repeats
 
 __global__ __launch_bounds__(256) void pool_init_kernel(int32_t* __restrict__ free_stack, int32_t* __restrict__ pool_state,
                                                         int32_t* __restrict__ slot_npages, int num_pool_pages,
@@ -97,21 +106,43 @@ __device__ __forceinline__ int block_sum_1024(int x, int* red) {
 
 // One 1024-thread workgroup grows every listed slot to ceil(seq_lens[b] / page_size)
 // pages (never shrinks one), all or nothing: if the free stack cannot cover the
-// whole call, nothing is reserved and kPoolExhausted is raised.
+// whole call, nothing is reserved and kPoolExhausted is raised.  Entries whose slot id is
+// out of range, or that name a slot an earlier entry of the same call named, are skipped
+// (kPoolBadSlot): every entry first adds kPoolMark to its slot's page count, and whoever
+// finds the mark already there is a repeat.
 __global__ __launch_bounds__(1024) void pool_reserve_kernel(const int32_t* __restrict__ slot_ids,
                                                             const int32_t* __restrict__ seq_lens, int batch,
                                                             int pages_per_slot, int page_size,
                                                             int32_t* __restrict__ slot_table,
                                                             int32_t* __restrict__ slot_npages,
                                                             const int32_t* __restrict__ free_stack,
-                                                            int32_t* __restrict__ pool_state) {
+                                                            int32_t* __restrict__ pool_state, int max_slots) {
   __shared__ int red[16];
   __shared__ int wave_sum[16];
   __shared__ int carry_sh;
+  __shared__ uint32_t skip_bits[2048];  // one bit per entry of the call (batch <= 65535)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < 2048; i += 1024) skip_bits[i] = 0;
+  __syncthreads();
+  int bad = 0;
+  for (int b = tid; b < batch; b += 1024) {
+    const int slot = slot_ids ? slot_ids[b] : b;
+    bool skip = (unsigned)slot >= (unsigned)max_slots;
+    if (!skip) skip = atomicAdd(&slot_npages[slot], kPoolMark) >= kPoolMark;
+    if (skip) {
+      atomicOr(&skip_bits[b >> 5], 1u << (b & 31));
+      bad = 1;
+    }
+  }
+  __syncthreads();
+  auto skipped = [&](int b) -> bool { return (skip_bits[b >> 5] >> (b & 31)) & 1u; };
   auto demand = [&](int b, int& slot, int& have) -> int {
     slot = slot_ids ? slot_ids[b] : b;
-    have = slot_npages[slot];
+    if (skipped(b)) {
+      have = 0;
+      return 0;
+    }
+    have = slot_npages[slot] & (kPoolMark - 1);
     const int len = max(seq_lens[b], 0);
     const int need = min((len + page_size - 1) / page_size, pages_per_slot);
     return max(need - have, 0);
@@ -124,17 +155,20 @@ __global__ __launch_bounds__(1024) void pool_reserve_kernel(const int32_t* __res
   }
   const int total = block_sum_1024(mine, red);
   const int any_long = block_sum_1024(too_long, red);
+  const int any_bad = block_sum_1024(bad, red);
   const int free_top = pool_state[0];
   __syncthreads();  // everybody has read free_top before thread 0 may change it
-  if (tid == 0 && (any_long || total > free_top))
-    pool_state[1] |= (any_long ? kPoolSlotTooLong : 0) | (total > free_top ? kPoolExhausted : 0);
-  if (total > free_top || total == 0) return;
+  if (tid == 0 && (any_long || any_bad || total > free_top))
+    pool_state[1] |= (any_long ? kPoolSlotTooLong : 0) | (any_bad ? kPoolBadSlot : 0) | (total > free_top ? kPoolExhausted : 0);
+  const bool grow = total <= free_top && total > 0;
   if (tid == 0) carry_sh = 0;
   __syncthreads();
   for (int base = 0; base < batch; base += 1024) {
     const int b = base + tid;
     int slot = 0, have = 0, extra = 0;
+    const bool live = b < batch && !skipped(b);
     if (b < batch) extra = demand(b, slot, have);
+    if (!grow) extra = 0;
     int incl = extra;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
@@ -148,12 +182,12 @@ __global__ __launch_bounds__(1024) void pool_reserve_kernel(const int32_t* __res
     const int first = before + incl - extra;  // this slot takes entries first .. first+extra-1 from the top
     for (int j = 0; j < extra; ++j)
       slot_table[(int64_t)slot * pages_per_slot + have + j] = free_stack[free_top - 1 - (first + j)];
-    if (extra > 0) slot_npages[slot] = have + extra;
+    if (live) slot_npages[slot] = have + extra;  // (also takes the mark off)
     __syncthreads();
     if (tid == 1023) carry_sh = before + incl;
     __syncthreads();
   }
-  if (tid == 0) pool_state[0] = free_top - total;
+  if (tid == 0 && grow) pool_state[0] = free_top - total;
 }
 
 // One 256-thread workgroup pushes the pages of the listed slots back, slot after slot.
@@ -161,10 +195,15 @@ __global__ __launch_bounds__(256) void pool_release_kernel(const int32_t* __rest
                                                            int pages_per_slot, const int32_t* __restrict__ slot_table,
                                                            int32_t* __restrict__ slot_npages,
                                                            int32_t* __restrict__ free_stack,
-                                                           int32_t* __restrict__ pool_state, int num_pool_pages) {
+                                                           int32_t* __restrict__ pool_state, int num_pool_pages,
+                                                           int max_slots) {
   int top = pool_state[0];
   for (int i = 0; i < count; ++i) {
     const int slot = slot_ids[i];
+    if ((unsigned)slot >= (unsigned)max_slots) {  // (uniform: every thread reads the same id)
+      if (threadIdx.x == 0) pool_state[1] |= kPoolBadSlot;
+      continue;
+    }
     const int n = slot_npages[slot];
     __syncthreads();  // everybody has read n before it is cleared
     for (int j = threadIdx.x; j < n; j += 256)
@@ -221,7 +260,8 @@ extern "C" int kin_page_pool_init(int32_t* free_stack, int32_t* pool_state, int3
 
 extern "C" int kin_page_pool_reserve(const int32_t* slot_ids, const int32_t* seq_lens, int batch,
                                      int pages_per_slot, int page_size, int32_t* slot_table, int32_t* slot_npages,
-                                     const int32_t* free_stack, int32_t* pool_state, kin_stream_t stream) {
+                                     const int32_t* free_stack, int32_t* pool_state, int max_slots,
+                                     kin_stream_t stream) {
   using namespace kin;
   const char* fn = "kin_page_pool_reserve";
   if (!seq_lens || !slot_table || !slot_npages || !free_stack || !pool_state)
@@ -229,15 +269,19 @@ extern "C" int kin_page_pool_reserve(const int32_t* slot_ids, const int32_t* seq
   if (batch < 0 || pages_per_slot < 1 || page_size < 1)
     return fail(KIN_ERR_BAD_SHAPE, "%s: batch=%d pages_per_slot=%d page_size=%d", fn, batch, pages_per_slot, page_size);
   if (batch > 65535) return fail(KIN_ERR_UNSUPPORTED, "%s: batch=%d exceeds 65535", fn, batch);
+  if (max_slots < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: max_slots=%d must be >= 1", fn, max_slots);
+  if (pages_per_slot >= kPoolMark) return fail(KIN_ERR_UNSUPPORTED, "%s: pages_per_slot=%d exceeds %d", fn, pages_per_slot, kPoolMark - 1);
+  if (!slot_ids && batch > max_slots)
+    return fail(KIN_ERR_BAD_SHAPE, "%s: batch=%d sequences but only max_slots=%d slots", fn, batch, max_slots);
   if (batch == 0) return KIN_OK;
   pool_reserve_kernel<<<1, 1024, 0, static_cast<hipStream_t>(stream)>>>(slot_ids, seq_lens, batch, pages_per_slot, page_size,
-                                                                       slot_table, slot_npages, free_stack, pool_state);
+                                                                       slot_table, slot_npages, free_stack, pool_state, max_slots);
   return check_hip(hipGetLastError(), "pool_reserve_kernel launch");
 }
 
 extern "C" int kin_page_pool_release(const int32_t* slot_ids, int count, int pages_per_slot,
                                      const int32_t* slot_table, int32_t* slot_npages, int32_t* free_stack,
-                                     int32_t* pool_state, int num_pool_pages, kin_stream_t stream) {
+                                     int32_t* pool_state, int num_pool_pages, int max_slots, kin_stream_t stream) {
   using namespace kin;
   const char* fn = "kin_page_pool_release";
   if (!slot_ids || !slot_table || !slot_npages || !free_stack || !pool_state)
@@ -245,16 +289,18 @@ extern "C" int kin_page_pool_release(const int32_t* slot_ids, int count, int pag
   if (count < 0 || pages_per_slot < 1 || num_pool_pages < 1)
     return fail(KIN_ERR_BAD_SHAPE, "%s: count=%d pages_per_slot=%d num_pool_pages=%d", fn, count, pages_per_slot,
                 num_pool_pages);
+  if (max_slots < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: max_slots=%d must be >= 1", fn, max_slots);
   if (count == 0) return KIN_OK;
   pool_release_kernel<<<1, 256, 0, static_cast<hipStream_t>(stream)>>>(slot_ids, count, pages_per_slot, slot_table,
-                                                                      slot_npages, free_stack, pool_state, num_pool_pages);
+                                                                      slot_npages, free_stack, pool_state, num_pool_pages,
+                                                                      max_slots);
   return check_hip(hipGetLastError(), "pool_release_kernel launch");
 }
 
 extern "C" int kin_build_pool_page_table(const int32_t* slot_ids, const int32_t* seq_lens, int batch,
                                          int pages_per_slot, int page_size, const int32_t* slot_table,
                                          const int32_t* slot_npages, int32_t* page_indices, int32_t* page_indptr,
-                                         int32_t* last_page_len, kin_stream_t stream) {
+                                         int32_t* last_page_len, int max_slots, kin_stream_t stream) {
   using namespace kin;
   const char* fn = "kin_build_pool_page_table";
   if (!seq_lens || !slot_table || !slot_npages || !page_indices || !page_indptr || !last_page_len)
@@ -267,8 +313,9 @@ extern "C" int kin_build_pool_page_table(const int32_t* slot_ids, const int32_t*
     fill_zero_i32_kernel<<<1, 64, 0, s>>>(page_indptr, 1);
     return check_hip(hipGetLastError(), "fill_zero_i32_kernel launch");
   }
+  if (max_slots < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: max_slots=%d must be >= 1", fn, max_slots);
   slot_table_scan_kernel<<<1, 1024, 0, s>>>(seq_lens, batch, pages_per_slot, page_size, page_indptr, last_page_len, slot_ids,
-                                            slot_npages);
+                                            slot_npages, max_slots);
   int st = check_hip(hipGetLastError(), "slot_table_scan_kernel launch");
   if (st) return st;
   dim3 grid((unsigned)((pages_per_slot + 255) / 256), (unsigned)batch);

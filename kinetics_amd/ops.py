@@ -90,22 +90,37 @@ def _cache_dims(kv_cache: torch.Tensor):
     return num_pages, page_size, num_kv_heads, head_dim
 
 
-def _kbar_pages(kbar: torch.Tensor, batch: int, num_kv_heads: int, head_dim: int, dtype: torch.dtype) -> int:
+def _kbar_pages(kbar: torch.Tensor, batch: int, num_kv_heads: int, head_dim: int, dtype: torch.dtype, slot_ids=None) -> int:
     """kbar is [B, Hkv, pages, D] (head-major), or the reference's [B, pages, D]
-    when Hkv == 1 (the same bytes)."""
+    when Hkv == 1 (the same bytes).  With ``slot_ids`` its first dimension counts
+    cache slots, not sequences."""
     _require(kbar, "kbar", dtype, (3, 4))
+    rows_ok = kbar.shape[0] == batch or (slot_ids is not None and kbar.shape[0] >= 1)
     if kbar.dim() == 3:
-        ok = num_kv_heads == 1 and kbar.shape[0] == batch and kbar.shape[2] == head_dim
+        ok = num_kv_heads == 1 and rows_ok and kbar.shape[2] == head_dim
         pages = kbar.shape[1]
     else:
-        ok = kbar.shape[0] == batch and kbar.shape[1] == num_kv_heads and kbar.shape[3] == head_dim
+        ok = rows_ok and kbar.shape[1] == num_kv_heads and kbar.shape[3] == head_dim
         pages = kbar.shape[2]
     if not ok:
         raise ValueError(
             f"kbar shape {tuple(kbar.shape)} does not match batch={batch}, num_kv_heads={num_kv_heads}, head_dim={head_dim} "
-            "(expected [batch, num_kv_heads, pages, head_dim])"
+            "(expected [batch, num_kv_heads, pages, head_dim]; [slots, ...] with slot_ids)"
         )
     return pages
+
+
+def _slots(slot_ids, kbar, batch: int, device):
+    """(pointer, num_slots) of the optional ``slot_ids`` [batch] int32: sequence b's mean
+    keys are ``kbar[slot_ids[b]]`` (the reference's kernels index the cache by slot and
+    q, k, v, out by position in the active batch,
+    LiteSys/litesys/attention/cache_utils.py:40-51,67-70)."""
+    if slot_ids is None:
+        return None, 0
+    _require(slot_ids, "slot_ids", torch.int32, 1, device)
+    if slot_ids.numel() != batch:
+        raise ValueError(f"slot_ids must have batch={batch} entries, got {slot_ids.numel()}")
+    return _ptr(slot_ids), (0 if kbar is None else kbar.shape[0])
 
 
 def _table(page_indices, page_indptr, last_page_len, batch, device):
@@ -124,11 +139,13 @@ def _table(page_indices, page_indptr, last_page_len, batch, device):
 # ---------------------------------------------------------------------------
 
 
-def append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len) -> None:
+def append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, slot_ids=None) -> None:
     """Write one new token per sequence into the paged cache (and refresh the
     mean key of a page that becomes full).  Stands in for ``mylib::update_kv``
     (benchmark/blocktopk_decoder.py:23-46,209-213).  The page table describes
-    the cache after the append.  ``kbar`` may be None."""
+    the cache after the append.  ``kbar`` may be None.  ``slot_ids`` (int32
+    [batch], optional): ``kbar`` is laid out by cache slot and sequence b uses
+    ``kbar[slot_ids[b]]``."""
     num_pages, page_size, num_kv_heads, head_dim = _cache_dims(kv_cache)
     dev = kv_cache.device
     dt = kv_cache.dtype
@@ -140,21 +157,22 @@ def append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_l
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     kbar_pages = 0
     if kbar is not None:
-        kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim, dt)
+        kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim, dt, slot_ids)
         if kbar.device != dev:
             raise ValueError("kbar must be on the same device as kv_cache")
+    sp, ns = _slots(slot_ids, kbar, batch, dev)
     lib = _lib.load()
     with _on(dev):
         _lib.check(
             _entry(lib, "kin_append_paged_kv", dt)(
                 _ptr(k), _ptr(v), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
-                _ptr(last_page_len), batch, num_kv_heads, head_dim, page_size, num_pages, kbar_pages, _stream(dev),
+                _ptr(last_page_len), batch, num_kv_heads, head_dim, page_size, num_pages, kbar_pages, sp, ns, _stream(dev),
             )
         )
 
 
 def append_paged_kv_ragged(k, v, append_indptr, kv_cache, kbar, page_indices, page_indptr, last_page_len,
-                           max_append_len: Optional[int] = None) -> None:
+                           max_append_len: Optional[int] = None, slot_ids=None) -> None:
     """Write ``append_indptr[b+1] - append_indptr[b]`` new tokens per sequence
     (rows of ``k`` / ``v`` [nnz, num_kv_heads, head_dim]) into the paged cache and
     refresh the mean key of every page that becomes full: the general form of
@@ -177,21 +195,22 @@ def append_paged_kv_ragged(k, v, append_indptr, kv_cache, kbar, page_indices, pa
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     kbar_pages = 0
     if kbar is not None:
-        kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim, dt)
+        kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim, dt, slot_ids)
         if kbar.device != dev:
             raise ValueError("kbar must be on the same device as kv_cache")
+    sp, ns = _slots(slot_ids, kbar, batch, dev)
     lib = _lib.load()
     with _on(dev):
         _lib.check(
             _entry(lib, "kin_append_paged_kv_ragged", dt)(
                 _ptr(k), _ptr(v), _ptr(append_indptr), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
                 _ptr(last_page_len), batch, nnz, nnz if max_append_len is None else int(max_append_len), num_kv_heads,
-                head_dim, page_size, num_pages, kbar_pages, _stream(dev),
+                head_dim, page_size, num_pages, kbar_pages, sp, ns, _stream(dev),
             )
         )
 
 
-def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len) -> None:
+def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len, slot_ids=None) -> None:
     """Fill ``kbar`` with the mean key of every full page (prefill-side producer
     of what the reference calls compressed_key_cache,
     benchmark/blocktopk_decoder.py:166-168)."""
@@ -199,13 +218,14 @@ def build_kbar(kv_cache, kbar, page_indices, page_indptr, last_page_len) -> None
     dev = kv_cache.device
     batch = page_indptr.numel() - 1
     _table(page_indices, page_indptr, last_page_len, batch, dev)
-    kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim, kv_cache.dtype)
+    kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim, kv_cache.dtype, slot_ids)
+    sp, ns = _slots(slot_ids, kbar, batch, dev)
     lib = _lib.load()
     with _on(dev):
         _lib.check(
             _entry(lib, "kin_build_kbar", kv_cache.dtype)(
                 _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len),
-                batch, num_kv_heads, head_dim, page_size, num_pages, kbar_pages, _stream(dev),
+                batch, num_kv_heads, head_dim, page_size, num_pages, kbar_pages, sp, ns, _stream(dev),
             )
         )
 
@@ -222,7 +242,7 @@ def sel_list_capacity(topk: int, sink_pages: int = 0, local_tokens: int = 1) -> 
 
 def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sel_logical=None,
                      scores_out=None, sink_pages: int = 0, local_tokens: int = 1, workspace=None,
-                     page_size: int = PAGE_SIZE) -> None:
+                     page_size: int = PAGE_SIZE, slot_ids=None) -> None:
     """Score every candidate page with the group-mean query and write the
     top-``topk`` pages plus the last page into ``sel_pages`` / ``sel_count``
     (in place: fixed buffers, as the reference registers with its decode
@@ -246,7 +266,8 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
     _require(sel_count, "sel_count", torch.int32, 2, dev)
     if tuple(sel_count.shape) != (batch, num_kv_heads):
         raise ValueError(f"sel_count must be [{batch}, {num_kv_heads}], got {tuple(sel_count.shape)}")
-    kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim, q.dtype)
+    kbar_pages = _kbar_pages(kbar, batch, num_kv_heads, head_dim, q.dtype, slot_ids)
+    sp, ns = _slots(slot_ids, kbar, batch, dev)
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     if last_page_len is None:
         raise TypeError("last_page_len is required")
@@ -266,7 +287,8 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
             _entry(lib, "kin_block_score_topk", q.dtype)(
                 _ptr(q), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), int(topk), int(sink_pages),
                 int(local_tokens), _ptr(sel_pages), _ptr(sel_count), _ptr(sel_logical), _ptr(scores_out), batch, num_q_heads,
-                num_kv_heads, head_dim, int(page_size), kbar_pages, sel_stride, _ptr(workspace), workspace.numel() if workspace is not None else 0, _stream(dev),
+                num_kv_heads, head_dim, int(page_size), kbar_pages, sel_stride, _ptr(workspace),
+                workspace.numel() if workspace is not None else 0, sp, ns, _stream(dev),
             )
         )
 
@@ -394,7 +416,8 @@ def prefer_fused_step(batch: int, num_kv_heads: int, max_pages_per_seq: int, top
 
 def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, out=None, lse=None,
                           sel_pages=None, sel_count=None, sm_scale: float = 0.0, sink_pages: int = 0,
-                          local_tokens: int = 1, first_page_offset: int = 0, workspace=None, static_scratch: bool = False):
+                          local_tokens: int = 1, first_page_offset: int = 0, workspace=None, static_scratch: bool = False,
+                          slot_ids=None, slot_lens=None):
     """append -> score -> select -> attend in one launch: lines 209-225 of the
     reference layer's forward (benchmark/blocktopk_decoder.py) as a single
     kernel.  ``k``/``v`` may be None (no append); ``sel_pages``/``sel_count`` are
@@ -402,14 +425,21 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
     None and the shape profits) lets several workgroups share a list when the lists
     are few: split attention, or split scoring for very long sequences.  ``static_scratch=True`` calls ``kin_blocktopk_decode_step_static``
     instead: the library's built-in device array is the workspace and nothing is
-    allocated (``out`` must then be given; ``workspace`` must be None).
+    allocated (``out`` must then be given; ``workspace`` must be None).  ``slot_ids``: ``kbar`` is laid
+    out by cache slot; ``slot_lens`` (int32, one entry per row block of ``kbar``): a token counter
+    per slot that the kernel advances by one for every sequence it appends to.
     Returns ``out`` [batch, num_q_heads, head_dim] bf16."""
     if static_scratch and (out is None or workspace is not None):
         raise ValueError("static_scratch=True needs a caller-provided out and takes no workspace")
     dev, batch, hq, hkv, d, ps, num_pages, out = _decode_common(q, kv_cache, last_page_len, out, lse, workspace)
     _table(page_indices, page_indptr, last_page_len, batch, dev)
     dt = kv_cache.dtype
-    kbar_pages = _kbar_pages(kbar, batch, hkv, d, dt)
+    kbar_pages = _kbar_pages(kbar, batch, hkv, d, dt, slot_ids)
+    sp, ns = _slots(slot_ids, kbar, batch, dev)
+    if slot_lens is not None:
+        _require(slot_lens, "slot_lens", torch.int32, 1, dev)
+        if slot_lens.numel() != kbar.shape[0]:
+            raise ValueError(f"slot_lens must have one entry per row block of kbar ({kbar.shape[0]}), got {slot_lens.numel()}")
     if (k is None) != (v is None):
         raise ValueError("k and v must both be given or both be None")
     if k is not None:
@@ -436,7 +466,7 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
                     _ptr(q), _ptr(k), _ptr(v), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
                     _ptr(last_page_len), int(topk), int(sink_pages), int(local_tokens), _ptr(sel_pages), _ptr(sel_count),
                     _ptr(out), _ptr(lse), batch, hq, hkv, d, ps, num_pages, kbar_pages, sel_stride, int(first_page_offset),
-                    float(sm_scale), _stream(dev),
+                    float(sm_scale), sp, ns, _ptr(slot_lens), _stream(dev),
                 )
             )
         return out
@@ -450,10 +480,55 @@ def blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, la
                 _ptr(q), _ptr(k), _ptr(v), _ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr),
                 _ptr(last_page_len), int(topk), int(sink_pages), int(local_tokens), _ptr(sel_pages), _ptr(sel_count),
                 _ptr(out), _ptr(lse), batch, hq, hkv, d, ps, num_pages, kbar_pages, sel_stride, int(first_page_offset),
-                float(sm_scale), _ptr(workspace), 0 if workspace is None else workspace.numel(), _stream(dev),
+                float(sm_scale), _ptr(workspace), 0 if workspace is None else workspace.numel(), sp, ns, _ptr(slot_lens),
+                _stream(dev),
             )
         )
     return out
+
+
+class DecodeStepPlan:
+    """``blocktopk_decode_step`` with everything but q, k, v and out checked and bound once, for
+    callers that make the same call again and again on buffers they own (a KV manager: every layer
+    of every decode step).  The tensors given here must stay alive and in place; a call checks only
+    the four tensors it is given and hands their pointers to the C ABI (a few microseconds of host
+    time instead of ~20)."""
+
+    def __init__(self, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk: int, num_q_heads: int,
+                 sm_scale: float = 0.0, sink_pages: int = 0, local_tokens: int = 1, first_page_offset: int = 0,
+                 workspace=None, slot_ids=None, slot_lens=None):
+        num_pages, page_size, hkv, d = _cache_dims(kv_cache)
+        dev, dt = kv_cache.device, kv_cache.dtype
+        batch = page_indptr.numel() - 1
+        _table(page_indices, page_indptr, last_page_len, batch, dev)
+        kbar_pages = _kbar_pages(kbar, batch, hkv, d, dt, slot_ids)
+        sp, ns = _slots(slot_ids, kbar, batch, dev)
+        if workspace is not None:
+            _require(workspace, "workspace", torch.uint8, 1, dev)
+        if num_q_heads % hkv:
+            raise ValueError(f"num_q_heads={num_q_heads} is not a multiple of num_kv_heads={hkv}")
+        if slot_lens is not None:
+            _require(slot_lens, "slot_lens", torch.int32, 1, dev)
+            if slot_lens.numel() != kbar.shape[0]:
+                raise ValueError("slot_lens must have one entry per row block of kbar")
+        self._keep = (kv_cache, kbar, page_indices, page_indptr, last_page_len, workspace, slot_ids, slot_lens)
+        self._fn = _entry(_lib.load(), "kin_blocktopk_decode_step", dt)
+        self._dev, self._dt = dev, dt
+        self._q_shape, self._k_shape = (batch, int(num_q_heads), d), (batch, hkv, d)
+        self._head = (_ptr(kv_cache), _ptr(kbar), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), int(topk),
+                      int(sink_pages), int(local_tokens), None, None)
+        self._tail = (batch, int(num_q_heads), hkv, d, page_size, num_pages, kbar_pages, 0, int(first_page_offset), float(sm_scale),
+                      _ptr(workspace), 0 if workspace is None else workspace.numel(), sp, ns, _ptr(slot_lens))
+
+    def __call__(self, q, k, v, out):
+        for t, shape in ((q, self._q_shape), (k, self._k_shape), (v, self._k_shape), (out, self._q_shape)):
+            if t.dtype is not self._dt or t.device != self._dev or tuple(t.shape) != shape or not t.is_contiguous():
+                raise ValueError(f"DecodeStepPlan: expected a contiguous {self._dt} tensor of shape {shape} on {self._dev}, "
+                                 f"got {t.dtype} {tuple(t.shape)} on {t.device}")
+        with _on(self._dev):
+            _lib.check(self._fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), *self._head, out.data_ptr(), None, *self._tail,
+                                _stream(self._dev)))
+        return out
 
 
 def token_topk_workspace_bytes(batch: int, num_kv_heads: int, max_pages_per_seq: int) -> int:
@@ -570,7 +645,7 @@ class PagePool:
     fewer pages than ``max_slots * pages_per_slot``; a finished slot returns its
     pages.  No method synchronises except ``status()`` / ``raise_on_overflow()``."""
 
-    EXHAUSTED, SLOT_TOO_LONG = 1, 2
+    EXHAUSTED, SLOT_TOO_LONG, BAD_SLOT = 1, 2, 4
 
     def __init__(self, num_pool_pages: int, max_slots: int, pages_per_slot: int, page_size: int, device):
         self.num_pool_pages, self.max_slots = int(num_pool_pages), int(max_slots)
@@ -600,15 +675,15 @@ class PagePool:
         with _on(self.device):
             _lib.check(_lib.load().kin_page_pool_reserve(
                 _ptr(slot_ids), _ptr(seq_lens), batch, self.pages_per_slot, self.page_size, _ptr(self.slot_table),
-                _ptr(self.slot_npages), _ptr(self.free_stack), _ptr(self.pool_state), _stream(self.device)))
+                _ptr(self.slot_npages), _ptr(self.free_stack), _ptr(self.pool_state), self.max_slots, _stream(self.device)))
 
     def release(self, slot_ids) -> None:
-        """Return every page of the listed slots (int32 tensor of distinct slot ids) to the pool."""
+        """Return every page of the listed slots (int32 tensor of slot ids) to the pool."""
         _require(slot_ids, "slot_ids", torch.int32, 1, self.device)
         with _on(self.device):
             _lib.check(_lib.load().kin_page_pool_release(
                 _ptr(slot_ids), slot_ids.numel(), self.pages_per_slot, _ptr(self.slot_table), _ptr(self.slot_npages),
-                _ptr(self.free_stack), _ptr(self.pool_state), self.num_pool_pages, _stream(self.device)))
+                _ptr(self.free_stack), _ptr(self.pool_state), self.num_pool_pages, self.max_slots, _stream(self.device)))
 
     def build_page_table(self, seq_lens, page_indices, page_indptr, last_page_len, slot_ids=None) -> None:
         """CSR page table of the sequences from the slots' page lists (kin_build_pool_page_table)."""
@@ -624,22 +699,34 @@ class PagePool:
         with _on(dev):
             _lib.check(_lib.load().kin_build_pool_page_table(
                 _ptr(slot_ids), _ptr(seq_lens), batch, self.pages_per_slot, self.page_size, _ptr(self.slot_table),
-                _ptr(self.slot_npages), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), _stream(dev)))
+                _ptr(self.slot_npages), _ptr(page_indices), _ptr(page_indptr), _ptr(last_page_len), self.max_slots,
+                _stream(dev)))
 
     def status(self):
         """(free pages, status bits) -- copies two ints to the host (synchronises)."""
         free, bits = self.pool_state.tolist()
         return free, bits
 
+    def acknowledge(self) -> None:
+        """Clear the status bits (the condition has been seen and dealt with)."""
+        self.pool_state[1:2].zero_()
+
     def raise_on_overflow(self) -> None:
-        """Raise if any earlier reserve ran out of pages or met a sequence longer than a slot
-        can hold (synchronises; the kernels themselves cannot raise)."""
+        """Raise if any earlier call ran out of pages, met a sequence longer than a slot can
+        hold, or was given a slot id it could not use (synchronises; the kernels themselves
+        cannot raise).  The bits are cleared first: the condition is reported once."""
         free, bits = self.status()
+        if not bits:
+            return
+        self.acknowledge()
         if bits & self.EXHAUSTED:
             raise _lib.KineticsError(f"page pool exhausted: a reserve wanted more than the {free} free pages "
-                                     f"(pool of {self.num_pool_pages})")
+                                     f"(pool of {self.num_pool_pages}); the sequences it could not serve have an empty "
+                                     "page list (nothing was written for them, their output is zero)")
         if bits & self.SLOT_TOO_LONG:
-            raise ValueError(f"a sequence exceeds {self.pages_per_slot} pages of {self.page_size} tokens (max_seq_len)")
+            raise ValueError(f"a sequence exceeds {self.pages_per_slot} pages of {self.page_size} tokens (max_seq_len); "
+                             "it has an empty page list (nothing was written for it, its output is zero)")
+        raise ValueError(f"a slot id outside [0, {self.max_slots}) or listed twice in one call was skipped")
 
 
 def check_page_table(page_indices, page_indptr, last_page_len, page_size, num_pages) -> None:
@@ -774,20 +861,20 @@ def gated_act(gate, up, act: str = "silu", out=None) -> torch.Tensor:
 torch.library.define(
     "kinetics::append_paged_kv",
     "(Tensor k, Tensor v, Tensor(a!) kv_cache, Tensor(b!)? kbar, Tensor page_indices, Tensor page_indptr, "
-    "Tensor last_page_len) -> ()",
+    "Tensor last_page_len, Tensor? slot_ids=None) -> ()",
 )
 # Same argument order as the reference's mylib::update_kv
 # (benchmark/blocktopk_decoder.py:23-26), plus the mean-key cache it has to keep current.
 torch.library.define(
     "kinetics::update_kv",
     "(Tensor k, Tensor v, Tensor kv_append_indptr, Tensor(a!) kv_cache, Tensor kv_page_indices, Tensor kv_page_indptr, "
-    "Tensor cachelen, Tensor(b!)? kbar=None) -> ()",
+    "Tensor cachelen, Tensor(b!)? kbar=None, Tensor? slot_ids=None) -> ()",
 )
 torch.library.define(
     "kinetics::block_score_topk",
     "(Tensor q, Tensor kbar, Tensor page_indices, Tensor page_indptr, Tensor last_page_len, int topk, "
     "Tensor(a!) sel_pages, Tensor(b!) sel_count, int sink_pages=0, int local_tokens=1, Tensor(c!)? workspace=None, "
-    "int page_size=16) -> ()",
+    "int page_size=16, Tensor? slot_ids=None) -> ()",
 )
 torch.library.define(
     "kinetics::sparse_paged_decode",
@@ -827,54 +914,57 @@ torch.library.define(
     "kinetics::blocktopk_decode_step",
     "(Tensor q, Tensor k, Tensor v, Tensor(a!) kv_cache, Tensor(b!) kbar, Tensor page_indices, Tensor page_indptr, "
     "Tensor last_page_len, int topk, Tensor(c!)? sel_pages, Tensor(d!)? sel_count, float sm_scale, "
-    "int sink_pages=0, int local_tokens=1, int first_page_offset=0, Tensor(e!)? workspace=None) -> Tensor",
+    "int sink_pages=0, int local_tokens=1, int first_page_offset=0, Tensor(e!)? workspace=None, "
+    "Tensor? slot_ids=None) -> Tensor",
 )
 
 
 @torch.library.impl("kinetics::blocktopk_decode_step", "cuda")
 def _step_impl(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sm_scale,
-               sink_pages=0, local_tokens=1, first_page_offset=0, workspace=None):
+               sink_pages=0, local_tokens=1, first_page_offset=0, workspace=None, slot_ids=None):
     return blocktopk_decode_step(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk,
                                  sel_pages=sel_pages, sel_count=sel_count, sm_scale=sm_scale, sink_pages=sink_pages,
-                                 local_tokens=local_tokens, first_page_offset=first_page_offset, workspace=workspace)
+                                 local_tokens=local_tokens, first_page_offset=first_page_offset, workspace=workspace,
+                                 slot_ids=slot_ids)
 
 
 @torch.library.register_fake("kinetics::blocktopk_decode_step")
 def _step_fake(q, k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sm_scale,
-               sink_pages=0, local_tokens=1, first_page_offset=0, workspace=None):
+               sink_pages=0, local_tokens=1, first_page_offset=0, workspace=None, slot_ids=None):
     return torch.empty_like(q)
 
 
 @torch.library.impl("kinetics::append_paged_kv", "cuda")
-def _append_impl(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len):
-    append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len)
+def _append_impl(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, slot_ids=None):
+    append_paged_kv(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, slot_ids=slot_ids)
 
 
 @torch.library.register_fake("kinetics::append_paged_kv")
-def _append_fake(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len):
+def _append_fake(k, v, kv_cache, kbar, page_indices, page_indptr, last_page_len, slot_ids=None):
     return None
 
 
 @torch.library.impl("kinetics::update_kv", "cuda")
-def _update_kv_impl(k, v, kv_append_indptr, kv_cache, kv_page_indices, kv_page_indptr, cachelen, kbar=None):
-    append_paged_kv_ragged(k, v, kv_append_indptr, kv_cache, kbar, kv_page_indices, kv_page_indptr, cachelen)
+def _update_kv_impl(k, v, kv_append_indptr, kv_cache, kv_page_indices, kv_page_indptr, cachelen, kbar=None, slot_ids=None):
+    append_paged_kv_ragged(k, v, kv_append_indptr, kv_cache, kbar, kv_page_indices, kv_page_indptr, cachelen, slot_ids=slot_ids)
 
 
 @torch.library.register_fake("kinetics::update_kv")
-def _update_kv_fake(k, v, kv_append_indptr, kv_cache, kv_page_indices, kv_page_indptr, cachelen, kbar=None):
+def _update_kv_fake(k, v, kv_append_indptr, kv_cache, kv_page_indices, kv_page_indptr, cachelen, kbar=None, slot_ids=None):
     return None
 
 
 @torch.library.impl("kinetics::block_score_topk", "cuda")
 def _select_impl(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sink_pages=0,
-                 local_tokens=1, workspace=None, page_size=PAGE_SIZE):
+                 local_tokens=1, workspace=None, page_size=PAGE_SIZE, slot_ids=None):
     block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count,
-                     sink_pages=sink_pages, local_tokens=local_tokens, workspace=workspace, page_size=page_size)
+                     sink_pages=sink_pages, local_tokens=local_tokens, workspace=workspace, page_size=page_size,
+                     slot_ids=slot_ids)
 
 
 @torch.library.register_fake("kinetics::block_score_topk")
 def _select_fake(q, kbar, page_indices, page_indptr, last_page_len, topk, sel_pages, sel_count, sink_pages=0,
-                 local_tokens=1, workspace=None, page_size=PAGE_SIZE):
+                 local_tokens=1, workspace=None, page_size=PAGE_SIZE, slot_ids=None):
     return None
 
 

@@ -18,7 +18,7 @@ int main(void) {
   printf("kin_rms_norm(NULL...) -> %s: %s\n", kin_status_string(st), kin_last_error());
   if (st != KIN_ERR_NULL_POINTER || strlen(kin_last_error()) == 0) ++fails;
   st = kin_blocktopk_decode_step(NULL, NULL, NULL, NULL, NULL, NULL, NULL, NULL, 8, 0, 1, NULL, NULL, NULL, NULL, 2, 4, 1,
-                                 128, 16, 8, 4, 0, 0, 0.0f, NULL, 0, NULL);
+                                 128, 16, 8, 4, 0, 0, 0.0f, NULL, 0, NULL, 0, NULL, NULL);
   printf("kin_blocktopk_decode_step(NULL...) -> %s\n", kin_status_string(st));
   if (st != KIN_ERR_NULL_POINTER) ++fails;
   if (kin_step_workspace_bytes(4096, 1, 2048) != 0) ++fails;

@@ -40,8 +40,8 @@ def test_version_and_status_strings(lib):
     assert lib.kin_status_string(99) == b"KIN_ERR_UNKNOWN"
 
 
-def append(lib, k=A, v=A, kv=A, kbar=A, idx=A, ptr=A, last=A, B=2, Hkv=1, D=128, ps=16, P=8, kp=4):
-    return lib.kin_append_paged_kv(k, v, kv, kbar, idx, ptr, last, B, Hkv, D, ps, P, kp, None)
+def append(lib, k=A, v=A, kv=A, kbar=A, idx=A, ptr=A, last=A, B=2, Hkv=1, D=128, ps=16, P=8, kp=4, slots=None, ns=0):
+    return lib.kin_append_paged_kv(k, v, kv, kbar, idx, ptr, last, B, Hkv, D, ps, P, kp, slots, ns, None)
 
 
 def test_append_argument_errors(lib):
@@ -58,11 +58,14 @@ def test_append_argument_errors(lib):
     assert append(lib, kv=A + 2) == _lib.KIN_ERR_MISALIGNED
     assert b"kv_cache" in lib.kin_last_error()
     assert append(lib, B=0) == _lib.KIN_OK  # nothing to do, nothing launched
+    assert append(lib, slots=A, ns=0) == _lib.KIN_ERR_BAD_SHAPE       # a slot table without slots
+    assert b"num_slots" in lib.kin_last_error()
+    assert append(lib, slots=A, ns=4, B=0) == _lib.KIN_OK
 
 
 def test_ragged_append_argument_errors(lib):
     def ragged(k=A, ind=A, B=2, nnz=10, mx=10, kv=A):
-        return lib.kin_append_paged_kv_ragged(k, A, ind, kv, A, A, A, A, B, nnz, mx, 1, 128, 16, 8, 4, None)
+        return lib.kin_append_paged_kv_ragged(k, A, ind, kv, A, A, A, A, B, nnz, mx, 1, 128, 16, 8, 4, None, 0, None)
 
     assert ragged(k=None) == _lib.KIN_ERR_NULL_POINTER
     assert ragged(ind=None) == _lib.KIN_ERR_NULL_POINTER
@@ -74,9 +77,9 @@ def test_ragged_append_argument_errors(lib):
 
 
 def select(lib, q=A, kbar=A, idx=A, ptr=A, last=A, topk=4, sel=A, cnt=A, B=2, Hq=4, Hkv=1, D=128, kp=64, stride=5, sink=0,
-           local=1, ps=16):
+           local=1, ps=16, slots=None, ns=0):
     return lib.kin_block_score_topk(q, kbar, idx, ptr, last, topk, sink, local, sel, cnt, None, None, B, Hq, Hkv, D, ps, kp,
-                                    stride, None, 0, None)
+                                    stride, None, 0, slots, ns, None)
 
 
 def test_select_argument_errors(lib):
@@ -98,6 +101,7 @@ def test_select_argument_errors(lib):
     assert select(lib, kbar=A + 8) == _lib.KIN_ERR_MISALIGNED
     assert select(lib, ps=48) == _lib.KIN_ERR_UNSUPPORTED
     assert select(lib, B=0) == _lib.KIN_OK and select(lib, B=0, ps=64) == _lib.KIN_OK
+    assert select(lib, slots=A, ns=-1) == _lib.KIN_ERR_BAD_SHAPE
 
 
 def sparse(lib, q=A, kv=A, sel=A, cnt=A, last=A, out=A, ws=None, wsb=0, B=2, Hq=4, Hkv=1, D=128, ps=16, P=8,
@@ -131,9 +135,9 @@ def test_decode_argument_errors(lib):
 
 
 def step(lib, q=A, k=A, v=A, kv=A, kbar=A, idx=A, ptr=A, last=A, topk=4, sink=0, local=1, sel=None, cnt=None, out=A, B=2,
-         Hq=4, Hkv=1, D=128, ps=16, P=8, kp=64, stride=0, offset=0):
+         Hq=4, Hkv=1, D=128, ps=16, P=8, kp=64, stride=0, offset=0, slots=None, ns=0):
     return lib.kin_blocktopk_decode_step(q, k, v, kv, kbar, idx, ptr, last, topk, sink, local, sel, cnt, out, None, B, Hq, Hkv,
-                                         D, ps, P, kp, stride, offset, 0.0, None, 0, None)
+                                         D, ps, P, kp, stride, offset, 0.0, None, 0, slots, ns, None, None)
 
 
 def test_step_argument_errors(lib):
@@ -149,6 +153,7 @@ def test_step_argument_errors(lib):
     assert step(lib, topk=4096) == _lib.KIN_ERR_UNSUPPORTED
     assert step(lib, out=A + 2) == _lib.KIN_ERR_MISALIGNED
     assert step(lib, B=0, sink=1, offset=12) == _lib.KIN_OK
+    assert step(lib, slots=A, ns=0) == _lib.KIN_ERR_BAD_SHAPE
 
 
 def test_token_topk_argument_errors(lib):
@@ -271,7 +276,7 @@ def test_path_preference_rule():
 
 def test_python_wrapper_maps_status_to_exceptions():
     with pytest.raises(ValueError, match="KIN_ERR_BAD_SHAPE"):
-        _lib.check(_lib.load().kin_block_score_topk(A, A, A, A, A, -1, 0, 1, A, A, None, None, 2, 4, 1, 128, 16, 64, 5, None, 0, None))
+        _lib.check(_lib.load().kin_block_score_topk(A, A, A, A, A, -1, 0, 1, A, A, None, None, 2, 4, 1, 128, 16, 64, 5, None, 0, None, 0, None))
     with pytest.raises(_lib.KineticsError, match="KIN_ERR_WORKSPACE"):
         _lib.check(sparse(_lib.load(), splits=3))
 
@@ -354,10 +359,10 @@ def test_static_scratch_step_size_limit_is_checked_before_anything_else(lib):
     assert 0 < lib.kin_step_workspace_bytes(64, 1, 8192) <= lib.kin_static_scratch_bytes()
     assert lib.kin_step_workspace_bytes(64, 1, 16384) > lib.kin_static_scratch_bytes()
     st = lib.kin_blocktopk_decode_step_static(None, None, None, None, None, None, None, None, 128, 0, 1, None, None, None,
-                                              None, 64, 4, 1, 128, 16, 1 << 20, 16384, 0, 0, 0.0, None)
+                                              None, 64, 4, 1, 128, 16, 1 << 20, 16384, 0, 0, 0.0, None, 0, None, None)
     assert st == _lib.KIN_ERR_WORKSPACE
     assert b"kin_blocktopk_decode_step_static" in lib.kin_last_error()
     # a shape that does not split needs no scratch: ordinary argument checking applies
     st = lib.kin_blocktopk_decode_step_static(None, None, None, None, None, None, None, None, 128, 0, 1, None, None, None,
-                                              None, 4096, 4, 1, 128, 16, 1 << 20, 2048, 0, 0, 0.0, None)
+                                              None, 4096, 4, 1, 128, 16, 1 << 20, 2048, 0, 0, 0.0, None, 0, None, None)
     assert st == _lib.KIN_ERR_NULL_POINTER

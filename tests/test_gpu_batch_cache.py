@@ -75,8 +75,7 @@ def _prefill_then_decode_like_litesys(sparse, fused):
     torch.manual_seed(5)
     m = make_manager(**sparse)
     PS = m.page                   # tokens per page: LiteSys' block size for the block policy, else 16
-    if fused is not None:
-        m._fused = fused          # both routes of decode(): one launch, or append + select + attend
+    m._force_fused = fused        # both routes of decode(): one launch, or append + select + attend (None: the manager's choice)
     L, Hq, Hkv = 2, 4, 2
     hist = {}  # (layer, slot) -> (K [t, Hkv, D], V) float32 of the bf16 values fed so far
 
@@ -149,43 +148,44 @@ def _prefill_then_decode_like_litesys(sparse, fused):
                 pages = torch.from_numpy(table[slot, : owned[slot]]).long().to(DEV)
                 got_k = m.kv_cache[layer][pages, 0].reshape(-1, Hkv, D)[pad:pad + t].float().cpu()
                 assert torch.equal(got_k, K)
-            # oracle on the manager's own state before the call
-            lens = np.zeros(6, dtype=np.int64)
-            lens[batch_slots] = off_before[batch_slots] + 1 + pad
+            # oracle on the manager's own state before the call: the page table lists the ACTIVE
+            # sequences in batch order, the mean keys stay with their slots
+            lens = (off_before[batch_slots] + 1 + pad).astype(np.int64)
             n_pages = (lens + PS - 1) // PS
-            indptr = np.zeros(7, dtype=np.int32)
+            indptr = np.zeros(bsz + 1, dtype=np.int32)
             indptr[1:] = np.cumsum(n_pages)
-            idx = np.concatenate([table[s, : n_pages[s]] for s in range(6)]).astype(np.int32)
-            last = np.where(lens > 0, lens - (n_pages - 1) * PS, 1).astype(np.int32)
-            assert np.array_equal(m.page_indptr.cpu().numpy(), indptr)
+            idx = np.concatenate([table[s, : n_pages[i]] for i, s in enumerate(batch_slots)]).astype(np.int32)
+            last = (lens - (n_pages - 1) * PS).astype(np.int32)
+            assert np.array_equal(m._indptr.cpu().numpy()[: bsz + 1], indptr)
             assert np.array_equal(m.page_indices.cpu().numpy()[: len(idx)], idx)
-            assert np.array_equal(m.last_page_len.cpu().numpy(), last)
-            qf = np.zeros((6, Hq, D), dtype=np.uint16)
-            kf = np.zeros((6, Hkv, D), dtype=np.uint16)
-            vf = np.zeros((6, Hkv, D), dtype=np.uint16)
-            qf[batch_slots], kf[batch_slots], vf[batch_slots] = P.from_torch(q[:, :, 0]), P.from_torch(k[:, :, 0]), P.from_torch(v[:, :, 0])
+            assert np.array_equal(m._last.cpu().numpy()[:bsz], last)
+            qf, kf, vf = P.from_torch(q[:, :, 0]), P.from_torch(k[:, :, 0]), P.from_torch(v[:, :, 0])
+            kbar_slots_before = kbar_before
+            kbar_before = np.ascontiguousarray(kbar_slots_before[batch_slots])   # the oracle indexes mean keys by sequence
             is_sparse = bool(sparse) and layer not in (0,)   # layer 0 stays dense (attn_layer_skip default)
             if is_sparse and token_policy:
                 O.append_paged_kv(kf, vf, kv_before, None, idx, indptr, last)
                 want, keeps, _ = O.token_topk_decode(qf, kv_before, idx, indptr, last, topk_block, sink=4, local=local,
                                                      policy=policy, block_size=block_size, stride=stride)
-                assert strided or not keeps[batch_slots[0]].all() or lens[batch_slots[0]] <= 4 + topk_block + local
+                assert strided or not keeps[0].all() or lens[0] <= 4 + topk_block + local
             elif is_sparse:
                 # the paged oracle on the manager's own state: one sink page, `local` newest tokens, 12 padding slots
                 res = O.decode_step(qf, kf, vf, kv_before, kbar_before, idx, indptr, last, topk_block,
                                     sink_pages=1, local_tokens=local, first_page_offset=pad)
                 want = res["out"]
                 # really sparse for the long sequences: fewer pages than the context has
-                assert res["sel_count"][batch_slots].max() < n_pages[batch_slots].max()
+                assert res["sel_count"].max() < n_pages.max()
             else:
                 O.append_paged_kv(kf, vf, kv_before, kbar_before, idx, indptr, last)
                 want, _ = O.dense_paged_decode(qf, kv_before, idx, indptr, last, first_page_offset=pad)
             assert np.array_equal(P.from_torch(m.kv_cache[layer]), kv_before)
             if not token_policy:   # (that policy has no use for mean keys and does not maintain them)
-                assert np.array_equal(P.from_torch(m.kbar[layer]), kbar_before)
+                want_kbar = kbar_slots_before.copy()
+                want_kbar[batch_slots] = kbar_before        # the active slots' rows, and nobody else's
+                assert np.array_equal(P.from_torch(m.kbar[layer]), want_kbar)
             got = out.float().cpu().numpy().reshape(bsz, Hq, D)
-            err = np.abs(got - want[batch_slots])
-            assert np.all(err <= 2e-2 + 2e-2 * np.abs(want[batch_slots]))
+            err = np.abs(got - want)
+            assert np.all(err <= 2e-2 + 2e-2 * np.abs(want))
             # and LiteSys' own formulation on the contiguous history that was fed: full logits, its mask
             # (4 sink tokens, blocks from token 4, `local` newest tokens), softmax, P.V
             for i, slot in enumerate(batch_slots):
@@ -215,9 +215,9 @@ def _prefill_then_decode_like_litesys(sparse, fused):
 
 @pytest.mark.parametrize("batch,with_slots", [(0, False), (1, False), (7, True), (1500, True), (3000, False)])
 def test_slot_page_table_against_numpy(batch, with_slots):
-    """CSR page table of a slot-based cache (kin_build_slot_page_table): page
-    counts clamped to the slot's run, empty and over-long sequences, more
-    sequences than one scan pass, an empty batch."""
+    """CSR page table of a slot-based cache (kin_build_slot_page_table): empty
+    sequences, sequences longer than a slot's run (they get an empty list: nothing
+    may be appended into a cut one), more sequences than one scan pass, an empty batch."""
     from kinetics_amd import ops
 
     rng = np.random.default_rng(batch + 1)
@@ -232,11 +232,11 @@ def test_slot_page_table_against_numpy(batch, with_slots):
     ops.build_slot_page_table(torch.from_numpy(lens).to(DEV), pps, PS, idx, ptr, last,
                               slot_ids=None if slots is None else torch.from_numpy(slots).to(DEV))
     torch.cuda.synchronize()
-    n = np.minimum((np.maximum(lens, 0) + PS - 1) // PS, pps)
+    n = (np.maximum(lens, 0) + PS - 1) // PS
+    n = np.where(n > pps, 0, n)
     want_ptr = np.concatenate([[0], np.cumsum(n)]).astype(np.int32)
     assert np.array_equal(ptr.cpu().numpy(), want_ptr)
-    tokens = np.minimum(np.maximum(lens, 0), n * PS)
-    want_last = np.where(n > 0, tokens - (n - 1) * PS, 1).astype(np.int32)
+    want_last = np.where(n > 0, np.maximum(lens, 0) - (n - 1) * PS, 1).astype(np.int32)
     assert np.array_equal(last.cpu().numpy(), want_last)
     got = idx.cpu().numpy()
     for b in range(batch):
@@ -289,9 +289,11 @@ def test_page_pool_against_a_python_free_list():
         for s in range(slots):
             assert got_table[s, : len(table[s])].tolist() == table[s], f"step {step} slot {s}"
         assert sorted(pool.free_stack.cpu().numpy()[:free].tolist() + [p for t in table for p in t]) == list(range(pool_pages))
-        # the CSR table of these lengths: cut to what each slot owns
+        # the CSR table of these lengths: a sequence its slot cannot hold (a failed reserve, or longer
+        # than a slot may grow) has an empty list
         pool.build_page_table(torch.from_numpy(lens).to(DEV), idx, ptr, last)
-        n = np.array([min(int(need[s]), len(table[s])) for s in range(slots)])
+        full = (np.maximum(lens, 0) + PS - 1) // PS
+        n = np.array([int(full[s]) if int(full[s]) <= len(table[s]) else 0 for s in range(slots)])
         want_ptr = np.concatenate([[0], np.cumsum(n)])
         assert ptr.cpu().tolist() == want_ptr.tolist()
         got = idx.cpu().numpy()
@@ -300,6 +302,42 @@ def test_page_pool_against_a_python_free_list():
     assert status == 3     # both conditions were met on the way
     with pytest.raises(Exception):
         pool.raise_on_overflow()
+    pool.raise_on_overflow()   # reported once: the bits were cleared
+    assert pool.status()[1] == 0
+
+
+def test_page_pool_skips_bad_and_repeated_slot_ids():
+    """Slot ids outside the pool, or named twice in one call, are skipped and flagged; the
+    free list stays whole (free pages + owned pages = every page, once)."""
+    from kinetics_amd import ops
+
+    slots, pps, pool_pages = 8, 6, 40
+    pool = ops.PagePool(pool_pages, slots, pps, PS, DEV)
+
+    def whole():
+        free, _ = pool.status()
+        owned = pool.slot_npages.cpu().tolist()
+        table = pool.slot_table.cpu().numpy()
+        pages = pool.free_stack.cpu().numpy()[:free].tolist() + [int(p) for s in range(slots) for p in table[s, : owned[s]]]
+        return sorted(pages) == list(range(pool_pages)), owned
+
+    ids = torch.tensor([3, 9, 3, -1, 5, 3], dtype=torch.int32, device=DEV)       # 9 and -1 do not exist, 3 comes three times
+    lens = torch.tensor([PS * 2, PS, PS * 2, PS, PS * 3 + 1, PS * 2], dtype=torch.int32, device=DEV)
+    pool.reserve(lens, ids)
+    ok, owned = whole()
+    assert ok and owned == [0, 0, 0, 2, 0, 4, 0, 0]                              # one entry of slot 3 counts, not three
+    assert pool.status()[1] == ops.PagePool.BAD_SLOT
+    idx = torch.full((pool_pages,), -1, dtype=torch.int32, device=DEV)
+    ptr = torch.empty(7, dtype=torch.int32, device=DEV)
+    last = torch.empty(6, dtype=torch.int32, device=DEV)
+    pool.build_page_table(lens, idx, ptr, last, ids)
+    # sequences with an unusable id have an empty list (the table itself does not look for repeats)
+    assert ptr.cpu().tolist() == [0, 2, 2, 4, 4, 8, 10]
+    with pytest.raises(ValueError):
+        pool.raise_on_overflow()
+    pool.release(torch.tensor([3, 3, 11, 5], dtype=torch.int32, device=DEV))    # a repeat and a stranger
+    ok, owned = whole()
+    assert ok and owned == [0] * 8 and pool.status() == (pool_pages, ops.PagePool.BAD_SLOT)
 
 
 def test_manager_with_a_small_pool_and_overlong_sequences():
@@ -326,22 +364,37 @@ def test_manager_with_a_small_pool_and_overlong_sequences():
     assert m.pool.status() == (2, 0)
     with pytest.raises(KineticsError):
         prefill(2, PS * 3)        # wants 3, 2 are free
-    m.pool.pool_state[1] = 0      # (acknowledged)
-    m.kv_offset[0][2] = 0
+    # the failed request left nothing behind: no pages, no offset, no status bit to trip over later
+    assert m.pool.status() == (2, 0) and m.kv_offset[0][2].item() == 0 and int(m.pool.slot_npages[2].item()) == 0
     m.clear_cache(0)              # 4 pages back
     assert m.pool.status() == (6, 0)
     prefill(2, PS * 5)            # takes 5 of the 6 free pages, most of them slot 0's old ones
     pages2 = m.pool.slot_table[2, :5].cpu().tolist()
     assert sorted(pages2) != pages2 or pages2[0] != 0   # not the fixed run a slot used to own
-    # decode slot 1 until it is past max_seq_len: flagged, not silently wrapped
+    # decode slot 1 until it is past max_seq_len: flagged, and from then on inert -- its pages and mean
+    # keys are never written again (it used to be cut to the pages it owned, and every further token
+    # overwrote the last slot of its last page)
     m.clear_cache(2)
-    for _ in range(PS * 3 + 4):
+    snap, outs = None, []
+    for step in range(PS * 3 + 4):
+        if int(m.kv_offset[0][1].item()) == PS * 6:        # the slot is full: what it holds now must stay
+            pages1 = m.pool.slot_table[1, : int(m.pool.slot_npages[1].item())].long()
+            snap = [(c[pages1].clone(), kb[1].clone()) for c, kb in zip(m.kv_cache, m.kbar)]
         for layer in range(L):
             q, k, v = (bf(torch.randn(1, h, 1, D, device=DEV)) for h in (Hq, Hkv, Hkv))
-            m.compute_attention(q, k, v, layer, torch.tensor([1]))
-    assert m.kv_offset[0][1].item() > PS * 6
+            out = m.compute_attention(q, k, v, layer, torch.tensor([1]))
+            if snap is not None:
+                outs.append(out)
+    assert m.kv_offset[0][1].item() > PS * 6 and snap is not None and len(outs) >= 8
+    for layer in range(L):
+        assert torch.equal(m.kv_cache[layer][pages1], snap[layer][0]) and torch.equal(m.kbar[layer][1], snap[layer][1])
+    assert all(bool((o == 0).all()) for o in outs)         # an empty page list attends nothing
     with pytest.raises(ValueError):
         m.clear_cache(1)
+    assert m.pool.status()[1] == 0
+    m.clear_cache(1)                                       # reported once; the slot is usable again
+    prefill(1, PS * 2)
+    assert m.pool.status()[1] == 0 and int(m.pool.slot_npages[1].item()) == 2
 
 
 @pytest.mark.parametrize("sparse", [dict(), dict(attn_block_topk=2, attn_local=18), dict(attn_block_topk=2, attn_local=18, attn_block_size=32)])
@@ -393,3 +446,109 @@ def test_float16_manager(sparse):
                 assert np.all(np.abs(got[i] - ref) <= 2e-2 + 2e-2 * np.abs(ref)), (layer, s)
                 if is_sparse:
                     assert not keep.all()
+
+
+def _fed_manager(max_batch, sparse, seed, prefill_lens):
+    """A manager after seeded prefills; returns it with the fp32 history per (layer, slot)."""
+    from kinetics_amd.batch_cache import PagedBatchKVManager
+
+    L, Hq, Hkv = 2, 4, 2
+    m = PagedBatchKVManager(cfg_small(), max_batch_size=max_batch, max_seq_len=PS * 24, device=DEV, dtype=torch.bfloat16, **sparse)
+    gen = torch.Generator().manual_seed(seed)
+    hist = {}
+    for slot, n in prefill_lens:
+        for layer in range(L):
+            q, k, v = (torch.randn(1, h, n, D, generator=gen).bfloat16().to(DEV) for h in (Hq, Hkv, Hkv))
+            hist[(layer, slot)] = (k[0].float().cpu().transpose(0, 1), v[0].float().cpu().transpose(0, 1))
+            m.compute_attention(q, k, v, layer, torch.tensor([slot]))
+    return m, hist
+
+
+@pytest.mark.parametrize("sparse", [dict(), dict(attn_block_topk=3, attn_local=16)])
+def test_manager_few_active_slots_in_any_order(sparse):
+    """Five active slots of a 40-slot manager, in an order that is not the slots': q, k, v and the
+    output follow the batch, the caches the slots.  The page table built by the first layer of a
+    step is reused by the second (same batch_idx object) -- same bits as rebuilding it -- and the
+    outputs are LiteSys' own formulation on the fed history."""
+    L, Hq, Hkv = 2, 4, 2
+    slots = [33, 4, 17, 29, 8]
+    pre = [(s, PS * (3 + i) + 2 * i + 1) for i, s in enumerate(slots)]
+    a, hist = _fed_manager(40, sparse, 31, pre)
+    b, _ = _fed_manager(40, sparse, 31, pre)
+    gen = torch.Generator().manual_seed(32)
+    same = torch.tensor(slots)
+    for step in range(PS + 3):                                   # every slot crosses a page boundary
+        order = slots if step % 2 == 0 else slots[::-1][:3]      # a subset in another order now and then
+        batch_a = same if order is slots else torch.tensor(order)
+        for layer in range(L):
+            q, k, v = (torch.randn(len(order), h, 1, D, generator=gen).bfloat16().to(DEV) for h in (Hq, Hkv, Hkv))
+            out_a = a.compute_attention(q, k, v, layer, batch_a)                 # one object for the whole step
+            out_b = b.compute_attention(q, k, v, layer, torch.tensor(order))     # a new one per layer: rebuilt each time
+            torch.cuda.synchronize()
+            assert torch.equal(out_a, out_b), (step, layer)
+            got = out_a.float().cpu().numpy().reshape(len(order), Hq, D)
+            for i, s in enumerate(order):
+                K, V = hist[(layer, s)]
+                K, V = torch.cat([K, k[i].float().cpu().transpose(0, 1)]), torch.cat([V, v[i].float().cpu().transpose(0, 1)])
+                hist[(layer, s)] = (K, V)
+                is_sparse = bool(sparse) and layer != 0
+                ref, _ = O.litesys_decode(q[i, :, 0].float().cpu().numpy(), K.numpy(), V.numpy(),
+                                          sparse["attn_block_topk"] if is_sparse else None, sparse.get("attn_local"))
+                assert np.all(np.abs(got[i] - ref) <= 2e-2 + 2e-2 * np.abs(ref)), (step, layer, s)
+    for layer in range(L):
+        assert torch.equal(a.kv_cache[layer], b.kv_cache[layer]) and torch.equal(a.kbar[layer], b.kbar[layer])
+        assert torch.equal(a.kv_offset[layer], b.kv_offset[layer])
+    assert a.pool.status() == b.pool.status() and a.pool.status()[1] == 0
+
+
+def test_manager_decode_step_replays_under_hip_graph():
+    """A whole decode step of the manager (every layer: offsets, page reservation, page table, the
+    attention kernels) recorded once as a HIP graph: every replay, with the program's own eager work
+    and synchronisations in between, equals an eager twin fed the same inputs."""
+    L, Hq, Hkv = 2, 4, 2
+    sparse = dict(attn_block_topk=3, attn_local=16)
+    slots = [6, 1, 9]
+    pre = [(6, PS * 5 + 3), (1, PS * 8), (9, PS * 3 + 15)]
+    g, _ = _fed_manager(12, sparse, 41, pre)
+    e, _ = _fed_manager(12, sparse, 41, pre)
+    batch_idx = torch.tensor(slots, device=DEV)
+    qs = [torch.zeros(3, Hq, 1, D, dtype=torch.bfloat16, device=DEV) for _ in range(L)]
+    ks = [torch.zeros(3, Hkv, 1, D, dtype=torch.bfloat16, device=DEV) for _ in range(L)]
+    vs = [torch.zeros(3, Hkv, 1, D, dtype=torch.bfloat16, device=DEV) for _ in range(L)]
+
+    def step(m):
+        return [m.compute_attention(qs[layer], ks[layer], vs[layer], layer, batch_idx) for layer in range(L)]
+
+    gen = torch.Generator(device=DEV).manual_seed(42)
+
+    def new_inputs():
+        for t in qs + ks + vs:
+            t.copy_(torch.randn(t.shape, generator=gen, device=DEV).bfloat16())
+
+    new_inputs()
+    step(g), step(e)                                  # warm-up on both (one token each)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    new_inputs()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            outs_g = step(g)                          # (capture runs nothing: the first replay is this step)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for trial in range(PS + 2):                       # page boundaries are crossed inside replays
+        if trial:
+            new_inputs()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs_g]
+        want = step(e)
+        torch.cuda.synchronize()
+        for layer in range(L):
+            assert torch.equal(got[layer], want[layer]), f"replay {trial}, layer {layer}"
+    for layer in range(L):
+        assert torch.equal(g.kv_offset[layer], e.kv_offset[layer])
+        assert torch.equal(g.kbar[layer], e.kbar[layer])
+    assert g.pool.status() == e.pool.status() and g.pool.slot_npages.tolist() == e.pool.slot_npages.tolist()

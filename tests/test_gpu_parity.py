@@ -1663,6 +1663,110 @@ def test_fused_step_full_size(ops):
     torch.cuda.empty_cache()
 
 
+# --------------------------------------------------------------------------- mean keys laid out by cache slot
+
+
+@pytest.mark.parametrize("fmt", ["bf16", "f16"])
+def test_slot_ids_put_the_mean_keys_with_the_cache_slot(ops, fmt):
+    """The reference's kernels index q, k, v and the output by position in the active
+    batch and the cache by slot (LiteSys/litesys/attention/cache_utils.py:40-51,67-70).
+    Here the page table is per active sequence already; slot_ids does the same for kbar:
+    a permuted, sparse set of slots gives the cache bytes, page lists and outputs of the
+    plain call, the mean keys land in the slots' rows and nobody else's, through every
+    entry point that touches kbar; an id outside the slots means "no mean keys"."""
+    with O.element_format(fmt):
+        lengths = [PS * 40 + 3, PS * 9, 1, 0, PS * 21, PS * 130 + 16, PS * 17 + 1]      # two appends fill a page
+        pb = P.make_problem(1700, lengths, num_kv_heads=2, group=4, topk=8, build_kbar=False)
+        S = 23
+        slots = np.array([5, 22, 0, 9, 17, 3, 11], dtype=np.int32)
+        slot_t = P.int_tensor(slots, DEV)
+        plain = Gpu(pb)
+        ops.build_kbar(plain.kv, plain.kbar, plain.indices, plain.indptr, plain.last)
+        kbar0 = plain.kbar.clone()
+
+        def by_slot(kbar_seq):
+            big = torch.full((S,) + tuple(kbar_seq.shape[1:]), 0x7b7b, dtype=torch.int16, device=DEV).view(kbar_seq.dtype)
+            return big
+
+        # build_kbar
+        g = Gpu(pb)
+        big = by_slot(g.kbar)
+        marker = big.clone()
+        ops.build_kbar(g.kv, big, g.indices, g.indptr, g.last, slot_ids=slot_t)
+        torch.cuda.synchronize()
+        n_pages = np.diff(pb.page_indptr)
+        for b, s in enumerate(slots):
+            full = n_pages[b] - (0 if pb.last_page_len[b] == PS and n_pages[b] > 0 else 1)
+            full = max(int(full), 0)
+            assert torch.equal(big[s, :, :full].view(torch.int16), kbar0[b, :, :full].view(torch.int16)), f"build_kbar slot {s}"
+            assert torch.equal(big[s, :, full:].view(torch.int16), marker[s, :, full:].view(torch.int16))
+        others = [s for s in range(S) if s not in slots.tolist()]
+        assert torch.equal(big[others].view(torch.int16), marker[others].view(torch.int16))
+
+        def scatter(kbar_seq):
+            big = by_slot(kbar_seq)
+            big[slot_t.long()] = kbar_seq
+            return big
+
+        # three launches, plain and by slot
+        cap = pb.topk + 1
+        ops.append_paged_kv(plain.k, plain.v, plain.kv, plain.kbar, plain.indices, plain.indptr, plain.last)
+        ops.block_score_topk(plain.q, plain.kbar, plain.indices, plain.indptr, plain.last, pb.topk, plain.sel, plain.cnt)
+        out_plain = ops.sparse_paged_decode(plain.q, plain.kv, plain.sel, plain.cnt, plain.last, num_splits=1)
+        g = Gpu(pb)
+        big = scatter(kbar0)
+        before = big.clone()
+        ops.append_paged_kv(g.k, g.v, g.kv, big, g.indices, g.indptr, g.last, slot_ids=slot_t)
+        ops.block_score_topk(g.q, big, g.indices, g.indptr, g.last, pb.topk, g.sel, g.cnt, slot_ids=slot_t)
+        out = ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, num_splits=1)
+        torch.cuda.synchronize()
+        assert torch.equal(g.kv, plain.kv) and torch.equal(g.sel, plain.sel) and torch.equal(g.cnt, plain.cnt)
+        assert torch.equal(out, out_plain)
+        assert torch.equal(big[slot_t.long()].view(torch.int16), plain.kbar.view(torch.int16))
+        assert torch.equal(big[others].view(torch.int16), before[others].view(torch.int16))
+        assert not torch.equal(plain.kbar, kbar0)      # a page did fill up: a mean key was written through the indirection
+        # the fused step (with and without the team workspace), and the ragged append
+        for ws in (None, torch.empty(0, dtype=torch.uint8, device=DEV)):
+            g = Gpu(pb)
+            big = scatter(kbar0)
+            out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, big, g.indices, g.indptr, g.last, pb.topk, sel_pages=g.sel,
+                                            sel_count=g.cnt, slot_ids=slot_t, workspace=ws)
+            torch.cuda.synchronize()
+            assert torch.equal(g.kv, plain.kv) and torch.equal(g.sel, plain.sel) and torch.equal(g.cnt, plain.cnt)
+            assert torch.allclose(out.float(), out_plain.float(), rtol=1e-2, atol=1e-2)
+            assert torch.equal(big[slot_t.long()].view(torch.int16), plain.kbar.view(torch.int16))
+            assert torch.equal(big[others].view(torch.int16), before[others].view(torch.int16))
+        g = Gpu(pb)
+        big = scatter(kbar0)
+        ptr1 = torch.arange(pb.B + 1, dtype=torch.int32, device=DEV)
+        live = torch.tensor([L > 0 for L in lengths], device=DEV)
+        # (one new row per non-empty sequence: the ragged form of the same append)
+        rows = torch.cumsum(live.to(torch.int32), 0)
+        ptr1 = torch.cat([torch.zeros(1, dtype=torch.int32, device=DEV), rows.to(torch.int32)])
+        ops.append_paged_kv_ragged(g.k[live].contiguous(), g.v[live].contiguous(), ptr1, g.kv, big, g.indices, g.indptr, g.last,
+                                   slot_ids=slot_t)
+        torch.cuda.synchronize()
+        assert torch.equal(g.kv, plain.kv)
+        assert torch.equal(big[slot_t.long()].view(torch.int16), plain.kbar.view(torch.int16))
+        # an id outside the slots: that sequence has no mean keys -- nothing written, no candidates, still attended
+        bad = slots.copy()
+        bad[0], bad[5] = S + 4, -2
+        bad_t = P.int_tensor(bad, DEV)
+        g = Gpu(pb)
+        big = scatter(kbar0)
+        before = big.clone()
+        out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, big, g.indices, g.indptr, g.last, pb.topk, sel_pages=g.sel,
+                                        sel_count=g.cnt, slot_ids=bad_t)
+        torch.cuda.synchronize()
+        assert torch.equal(g.kv, plain.kv)
+        cnt = g.cnt.cpu().numpy()
+        assert (cnt[0] == 1).all() and (cnt[5] == 1).all()                  # the open page only
+        assert torch.equal(g.cnt[1:5], plain.cnt[1:5]) and torch.equal(g.sel[1:5], plain.sel[1:5])
+        assert torch.equal(big[[5, 3]].view(torch.int16), before[[5, 3]].view(torch.int16))   # their slots' rows were left alone
+        want, _ = O.sparse_paged_decode(pb.q, P.from_torch(plain.kv), g.sel.cpu().numpy(), cnt, pb.last_page_len)
+        assert_out_close(out, want, "sequences without mean keys")
+
+
 # --------------------------------------------------------------------------- whole decoder layer
 
 

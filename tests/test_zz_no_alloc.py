@@ -91,7 +91,7 @@ def test_static_scratch_step_rejects_sizes_beyond_the_array():
     assert lib.kin_step_workspace_bytes(64, 1, 16384) > lib.kin_static_scratch_bytes()
     null = ctypes.c_void_p(None)
     st = lib.kin_blocktopk_decode_step_static(null, null, null, null, null, null, null, null, 128, 0, 1, null, null, null, null,
-                                              64, 4, 1, 128, 16, 1 << 20, 16384, 0, 0, 0.0, null)
+                                              64, 4, 1, 128, 16, 1 << 20, 16384, 0, 0, 0.0, null, 0, null, null)
     assert st == _lib.KIN_ERR_WORKSPACE
     msg = lib.kin_last_error().decode()
     assert "kin_blocktopk_decode_step_static" in msg and "scratch" in msg
