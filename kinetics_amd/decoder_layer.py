@@ -187,7 +187,11 @@ class BlockTopkDecoderLayer(_LayerBase):
         self._gate_up_weight()
         return None
 
-    @torch.inference_mode()
+    # no_grad where the reference has inference_mode (benchmark/blocktopk_decoder.py:186): with
+    # inference mode on, AOT functionalisation cannot wrap an op result that is a view of an
+    # intermediate it never saw (nn.Linear on a 3-D input returns one), so the layer would not
+    # compile beyond Dynamo's tracing.
+    @torch.no_grad()
     def forward(self, hidden_states):
         q, k, v = self._qkv(hidden_states)
         o = self.attn(q, k, v)
@@ -206,7 +210,7 @@ class DenseDecoderLayer(_LayerBase):
         self._gate_up_weight()
         return None
 
-    @torch.inference_mode()
+    @torch.no_grad()  # see BlockTopkDecoderLayer.forward
     def forward(self, hidden_states):
         q, k, v = self._qkv(hidden_states)
         o = self.attn(q, k, v)

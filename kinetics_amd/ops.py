@@ -878,13 +878,13 @@ torch.library.define(
 )
 torch.library.define(
     "kinetics::sparse_paged_decode",
-    "(Tensor q, Tensor kv_cache, Tensor sel_pages, Tensor sel_count, Tensor last_page_len, Tensor? workspace, "
+    "(Tensor q, Tensor kv_cache, Tensor sel_pages, Tensor sel_count, Tensor last_page_len, Tensor(a!)? workspace, "
     "float sm_scale, int num_splits, int first_page_offset=0) -> Tensor",
 )
 torch.library.define(
     "kinetics::dense_paged_decode",
     "(Tensor q, Tensor kv_cache, Tensor page_indices, Tensor page_indptr, Tensor last_page_len, "
-    "int max_pages_per_seq, Tensor? workspace, float sm_scale, int num_splits, int first_page_offset=0) -> Tensor",
+    "int max_pages_per_seq, Tensor(a!)? workspace, float sm_scale, int num_splits, int first_page_offset=0) -> Tensor",
 )
 
 
