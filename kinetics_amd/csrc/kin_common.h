@@ -223,8 +223,8 @@ static __global__ __attribute__((unused)) void fill_zero_i32_kernel(int32_t* p, 
 }
 
 #ifdef KIN_TUNE
-// Phase stamps of experimental builds: per workgroup up to 64 (tag, 100 MHz clock) pairs, in arrays
-// private to the translation unit.
+// Phase stamps of the diagnostic build (-DKIN_TUNE): per workgroup up to 64 (tag, 100 MHz clock) pairs, in
+// arrays private to the translation unit; the accessor copies them out and empties them.
 static __device__ long long g_stamps[1024 * 64 * 2];
 static __device__ int g_nstamps[1024];
 #define KIN_STAMP(tag)                                                          \
@@ -247,6 +247,8 @@ static __device__ int g_nstamps[1024];
     if (hipDeviceSynchronize() != hipSuccess) return 1;                                                                      \
     if (hipMemcpyFromSymbol(stamps, HIP_SYMBOL(kin::g_stamps), sizeof(long long) * 1024 * 64 * 2) != hipSuccess) return 2;   \
     if (hipMemcpyFromSymbol(counts, HIP_SYMBOL(kin::g_nstamps), sizeof(int) * 1024) != hipSuccess) return 3;                 \
+    static const int zeros_[1024] = {};  /* the next reading starts empty, whatever grid wrote this one */                   \
+    if (hipMemcpyToSymbol(HIP_SYMBOL(kin::g_nstamps), zeros_, sizeof(zeros_)) != hipSuccess) return 4;                       \
     return 0;                                                                                                                \
   }
 #else

@@ -210,22 +210,28 @@ __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, 
   const int lane = tid & 63;
   // Lane owns columns d = 8*(lane%16) .. +7 of the mean query.
   const int c16 = lane & 15;
-  float qm[8];
-  {
+  // The group's query rows are requested four at a time (a loop of single loads would pay one memory
+  // round trip per head), the first four before the first mean keys and averaged after those are
+  // under way, so that the stream starts one round trip after the call.
+  const uint16_t* qp = a.q_bh + 8 * c16;
+  auto load_q_rows = [&](uint4 (&qv)[4], int g0) {
 #pragma unroll
-    for (int u = 0; u < 8; ++u) qm[u] = 0.f;
-    const uint16_t* qp = a.q_bh + 8 * c16;
-    for (int g = 0; g < a.G; ++g) {
-      const uint4 w = *reinterpret_cast<const uint4*>(qp + (int64_t)g * kHeadDim);
-      qm[0] += elem_lo<F16>(w.x); qm[1] += elem_hi<F16>(w.x);
-      qm[2] += elem_lo<F16>(w.y); qm[3] += elem_hi<F16>(w.y);
-      qm[4] += elem_lo<F16>(w.z); qm[5] += elem_hi<F16>(w.z);
-      qm[6] += elem_lo<F16>(w.w); qm[7] += elem_hi<F16>(w.w);
+    for (int i = 0; i < 4; ++i) qv[i] = *reinterpret_cast<const uint4*>(qp + (int64_t)min(g0 + i, a.G - 1) * kHeadDim);
+  };
+  auto add_q_rows = [&](float (&qm)[8], const uint4 (&qv)[4], int g0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (g0 + i < a.G) {
+        const uint4 w = qv[i];
+        qm[0] += elem_lo<F16>(w.x); qm[1] += elem_hi<F16>(w.x);
+        qm[2] += elem_lo<F16>(w.y); qm[3] += elem_hi<F16>(w.y);
+        qm[4] += elem_lo<F16>(w.z); qm[5] += elem_hi<F16>(w.z);
+        qm[6] += elem_lo<F16>(w.w); qm[7] += elem_hi<F16>(w.w);
+      }
     }
-    const float inv = 1.0f / (float)a.G;
-#pragma unroll
-    for (int u = 0; u < 8; ++u) qm[u] *= inv;
-  }
+  };
+  uint4 qv0[4];
+  load_q_rows(qv0, 0);
   // The candidates of (b, h) are contiguous rows of 256 B.  They are read
   // through a buffer descriptor that ends after the last wanted row, so loads past
   // the end return zeros without touching memory and the loop needs no branches:
@@ -246,6 +252,21 @@ __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, 
 #pragma unroll
   for (int j = 0; j < kUnroll; ++j)
     w[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + j * kRows * row_stride_b, 0, kStreamLoad);
+  float qm[8];
+  {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) qm[u] = 0.f;
+    add_q_rows(qm, qv0, 0);
+    for (int g0 = 4; g0 < a.G; g0 += 4) {
+      uint4 qv[4];
+      load_q_rows(qv, g0);
+      add_q_rows(qm, qv, g0);
+    }
+    const float inv = 1.0f / (float)a.G;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) qm[u] *= inv;
+  }
+  KIN_STAMP(16);  // mean query in registers
   for (int base = 0; base < n; base += kRows * kUnroll) {
     const int next_off = lane_off + (base + kRows * kUnroll) * row_stride_b;
 #pragma unroll
@@ -515,10 +536,11 @@ template <int UNROLL = 4, int NT = kThreads, bool F16 = false>
 __device__ __forceinline__ int score_select(SelectArgs& a, int32_t* sel_lds) {
   // Nothing to choose (topk == 0) and nobody asked for the scores: stream nothing.
   const int n_score = (min(a.topk, a.n_cand) > 0 || a.scores_out) ? a.n_cand : 0;
+  KIN_STAMP(17);  // prologue over: the stream of mean keys starts
   score_rows<UNROLL, NT, false, F16, true>(a, 0, n_score, a.keys);
   a.digit0_counted = true;
   // the page-table copy (LDS-direct loads) has landed in every wave before anyone reads it
-  KIN_STAMP(18);  // this wave's scores are issued
+  KIN_STAMP(18);  // this wave has consumed its last mean key
   __builtin_amdgcn_s_waitcnt(0);
   KIN_STAMP(19);  // ... and have landed
   __syncthreads();

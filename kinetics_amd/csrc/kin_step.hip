@@ -76,6 +76,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   }
   const int last_len = p.last_page_len[b];
   const int kb = kbar_block_of(p.slot_ids, p.num_slots, b);  // (a sequence without mean keys has no candidates)
+  KIN_STAMP(1);  // the sequence's table entries are known
 
   // ---- append (wave 0): same byte moves and mean-key update as append_kernel ----
   // In a team the member that attends the sequence's last page does it (see below).
@@ -93,6 +94,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     }
   };
   if (team == 1) append_token();
+  KIN_STAMP(2);  // appended (one workgroup per list)
 
   // ---- score + select: page list into LDS -------------------------------------
   int32_t* sel_lds = reinterpret_cast<int32_t*>(smem + p.region0_bytes);
