@@ -82,6 +82,32 @@ def test_static_scratch_step_equals_workspace_step():
     _both_ways(ops, big, sink=0, local=33, what="sixth call (first shape again)", must_split=True)
 
 
+def test_static_scratch_step_takes_no_device_memory():
+    """Free device memory as the driver reports it is the same before and after calls of the entry point,
+    with torch's caching allocator out of the picture: every tensor exists before the first reading.
+    (One call comes before the first reading: the runtime loads a kernel's code the first time it is
+    launched, which is the runtime's memory, not the entry point's.)"""
+    from kinetics_amd import ops
+
+    pb = P.make_problem(9106, [PS * 2200 + 3, PS * 900 + 16, 5], num_kv_heads=2, group=4, topk=40)
+    g = Gpu(pb, ops.sel_list_capacity(pb.topk, 0, 1))
+
+    def call():
+        ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, pb.topk, out=g.out, lse=g.lse,
+                                  sel_pages=g.sel, sel_count=g.cnt, static_scratch=True)
+
+    call()
+    torch.cuda.synchronize()
+    reserved0 = torch.cuda.memory_reserved()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(5):
+        call()
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert torch.cuda.memory_reserved() == reserved0, "torch allocated device memory during the calls"
+    assert free1 == free0, f"free device memory went from {free0} to {free1} bytes across kin_blocktopk_decode_step_static"
+
+
 def test_static_scratch_step_rejects_sizes_beyond_the_array():
     from kinetics_amd import _lib
 
