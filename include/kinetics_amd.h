@@ -38,9 +38,11 @@
  *                 final entry is always the sequence's last page
  *                 (ref: benchmark/blocktopk_decoder.py:143,217-221).
  *
- * Supported shapes: head_dim == 128; page_size 16, 32 or 64 (the reference's
- * --page_size, benchmark/blocktopk.py:13; the token-granular policies
- * kin_token_topk_decode / kin_strided_topk_decode: 16 only);
+ * Supported shapes: head_dim 128 or 64 (the reference reads it from the model
+ * config, benchmark/blocktopk_decoder.py:104; the token-granular policies
+ * kin_token_topk_decode / kin_strided_topk_decode: 128 only); page_size 16, 32 or 64
+ * (the reference's --page_size, benchmark/blocktopk.py:13; the token-granular
+ * policies: 16 only);
  * num_q_heads % num_kv_heads == 0 and group size num_q_heads/num_kv_heads <= 16.
  * Where a comment below says "16" for a page it means page_size.
  */
@@ -80,7 +82,10 @@ enum kin_status {
  * attention (kin_step_workspace_bytes covers keys and partial results;
  * KIN_STATIC_SCRATCH_BYTES doubles); without sel_pages the step attends the
  * winners in index order.  3.0.0: every entry point that touches kbar takes
- * slot_ids / num_slots in front of the stream (kbar laid out by cache slot). */
+ * slot_ids / num_slots in front of the stream (kbar laid out by cache slot).
+ * 3.1.0: head_dim 64 in the page path (append, mean keys, selector, sparse and
+ * dense decode, the fused step), in kin_qkv_norm_split and, for rows of 64
+ * elements, in kin_rms_norm. */
 int kin_version(void);
 
 /* Human-readable text of the last non-OK status on the calling thread
@@ -705,8 +710,8 @@ int kin_blocktopk_decode_step_f16(const kin_f16_t* q, const kin_f16_t* k, const 
  * (benchmark/model_utils.py:27-41), which is understood to keep the fp32 sum
  * for the statistics: the two can differ in the last bf16 place.
  * Row strides are in elements (multiples of 8, >= hidden); out may alias x.
- * hidden: a multiple of 512 up to 8192, or a multiple of 128 up to 2048
- * (head_dim 128 rows for qk_norm).
+ * hidden: a multiple of 512 up to 8192, a multiple of 128 up to 2048
+ * (head_dim 128 rows for qk_norm), or 64 (head_dim 64 rows for qk_norm).
  */
 int kin_rms_norm(const void* x, void* residual, const void* weight, void* out,
                  int64_t rows, int hidden, int64_t x_row_stride, int64_t out_row_stride,
@@ -722,7 +727,7 @@ int kin_rms_norm_f16(const void* x, void* residual, const void* weight, void* ou
  * head with q_weight[D] and every k head with k_weight[D] (qk_norm,
  * benchmark/model_utils.py:15-25), copy the v heads, and write contiguous
  * q[batch, num_q_heads, D], k[batch, num_kv_heads, D], v[batch, num_kv_heads, D].
- * qkv_row_stride in elements (multiple of 8).  head_dim must be 128.
+ * qkv_row_stride in elements (multiple of 8).  head_dim (D) must be 128 or 64.
  */
 int kin_qkv_norm_split(const void* qkv, int64_t qkv_row_stride, const void* q_weight,
                        const void* k_weight, float eps, void* q, void* k, void* v,

@@ -22,7 +22,7 @@ int check_hip(hipError_t e, const char* what) {
 }
 
 int check_common_dims(const char* fn, int batch, int num_q_heads, int num_kv_heads,
-                      int head_dim, int page_size) {
+                      int head_dim, int page_size, bool small_head_dim_built) {
   if (batch < 0) return fail(KIN_ERR_BAD_SHAPE, "%s: batch=%d is negative", fn, batch);
   if (num_kv_heads < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_kv_heads=%d must be >= 1", fn, num_kv_heads);
   if (num_q_heads < 1 || num_q_heads % num_kv_heads != 0)
@@ -30,8 +30,9 @@ int check_common_dims(const char* fn, int batch, int num_q_heads, int num_kv_hea
                 num_q_heads, num_kv_heads);
   if (head_dim <= 0 || page_size <= 0)
     return fail(KIN_ERR_BAD_SHAPE, "%s: head_dim=%d and page_size=%d must be positive", fn, head_dim, page_size);
-  if (head_dim != kHeadDim)
-    return fail(KIN_ERR_UNSUPPORTED, "%s: head_dim=%d unsupported (kernels are built for %d)", fn, head_dim, kHeadDim);
+  if (head_dim != kHeadDim && !(small_head_dim_built && head_dim == kHeadDimSmall))
+    return fail(KIN_ERR_UNSUPPORTED, "%s: head_dim=%d unsupported (kernels are built for %s%d)", fn, head_dim,
+                small_head_dim_built ? "64 and " : "", kHeadDim);
   if (!supported_page_size(page_size))
     return fail(KIN_ERR_UNSUPPORTED, "%s: page_size=%d unsupported (kernels are built for 16, 32 and 64)", fn, page_size);
   if (num_q_heads / num_kv_heads > kMaxGroup)
@@ -89,7 +90,7 @@ __global__ void check_page_table_kernel(const int32_t* __restrict__ page_indices
 
 extern "C" {
 
-int kin_version(void) { return 30000; }
+int kin_version(void) { return 30100; }
 
 int kin_sel_list_capacity(int topk, int sink_pages, int local_tokens) {
   if (topk < 0 || sink_pages < 0 || local_tokens < 1) return 0;

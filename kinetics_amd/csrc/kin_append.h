@@ -54,7 +54,8 @@ __device__ __forceinline__ u32x4 page_mean_16B(const u32x4* kplane16, int row_st
   return m;
 }
 
-// Run by the 64 lanes of one wave (lane = 0..63, 4 bytes each = one 256-byte row).
+// Run by the 64 lanes of one wave (lane = 0..63, 4 bytes each = one 256-byte row; with HD = 64 the
+// first 32 lanes move the 128-byte row and the others do nothing).
 // k_row / v_row: the new token's rows for this (sequence, head), in dwords.
 // The row lands in slot last_len-1 of the sequence's last page (physical id
 // last_pid).  If that fills the page and the page has a slot in kbar
@@ -63,16 +64,17 @@ __device__ __forceinline__ u32x4 page_mean_16B(const u32x4* kplane16, int row_st
 // read from the cache, the last row is taken from the register, so the result does not
 // depend on store visibility.  Metadata outside its contract would write
 // outside the cache: the row is skipped.
-template <bool F16 = false>
+template <bool F16 = false, int HD = kHeadDim>
 __device__ __forceinline__ void append_token_row(const uint32_t* k_row, const uint32_t* v_row, uint32_t* kv_cache,
                                                  uint32_t* kbar_page_row, int64_t last_pid, int last_len, int n_pages,
                                                  int kbar_pages, int h, int num_kv_heads, int64_t num_pages, int lane,
                                                  int page_size) {
   const int pos = last_len - 1;
   if (pos < 0 || pos >= page_size || last_pid < 0 || last_pid >= num_pages) return;
-  const int row_stride = num_kv_heads * (kHeadDim / 2);      // dwords per token row
+  if (HD < 128 && lane >= HD / 2) return;
+  const int row_stride = num_kv_heads * (HD / 2);            // dwords per token row
   const int64_t page_dwords = 2LL * page_size * row_stride;  // K plane + V plane
-  uint32_t* kplane = kv_cache + last_pid * page_dwords + h * (kHeadDim / 2);
+  uint32_t* kplane = kv_cache + last_pid * page_dwords + h * (HD / 2);
   uint32_t* vplane = kplane + (int64_t)page_size * row_stride;
   const uint32_t kw = k_row[lane];
   const uint32_t vw = v_row[lane];

@@ -14,6 +14,7 @@ struct AppendParams {
   const int32_t* page_indptr;
   const int32_t* last_page_len;
   int batch, num_kv_heads, kbar_pages, page_size;
+  int head_dim;  // 128 or 64: these kernels move bytes and take it at run time
   int64_t num_pages;
   const int32_t* slot_ids;  // kbar row block of each sequence (null: the sequence's own index)
   int num_slots;
@@ -30,23 +31,31 @@ __global__ __launch_bounds__(256) void append_kernel(AppendParams p) {
   const int n_pages = e - s;
   if (n_pages <= 0) return;
   const int kb = kbar_block_of(p.slot_ids, p.num_slots, b);
-  uint32_t* kbar_row = (p.kbar && kb >= 0) ? p.kbar + kbar_row_index(kb, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2)
+  const int row_dwords = p.head_dim / 2;
+  uint32_t* kbar_row = (p.kbar && kb >= 0) ? p.kbar + kbar_row_index(kb, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * row_dwords
                                            : nullptr;
-  append_token_row<F16>(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2), p.kv_cache, kbar_row,
-                   p.page_indices[e - 1], p.last_page_len[b], n_pages, p.kbar_pages, h, p.num_kv_heads, p.num_pages, lane,
-                   p.page_size);
+  const uint32_t* k_row = p.k + (int64_t)item * row_dwords;
+  const uint32_t* v_row = p.v + (int64_t)item * row_dwords;
+  if (p.head_dim == kHeadDimSmall)
+    append_token_row<F16, kHeadDimSmall>(k_row, v_row, p.kv_cache, kbar_row, p.page_indices[e - 1], p.last_page_len[b], n_pages,
+                                         p.kbar_pages, h, p.num_kv_heads, p.num_pages, lane, p.page_size);
+  else
+    append_token_row<F16, kHeadDim>(k_row, v_row, p.kv_cache, kbar_row, p.page_indices[e - 1], p.last_page_len[b], n_pages,
+                                    p.kbar_pages, h, p.num_kv_heads, p.num_pages, lane, p.page_size);
 }
 
-// grid = batch * Hkv * ceil(kbar_pages / 16) blocks (flat, so it is not bound by
-// the 65535 limit of grid.y); 16 lanes per (sequence, head, logical page), a lane
+// grid = batch * Hkv * page_blocks blocks (flat, so it is not bound by
+// the 65535 limit of grid.y); head_dim / 8 lanes (16 or 8) per (sequence, head, logical page), so a
+// block covers 16 or 32 pages; a lane
 // owns 8 columns of all 16 key rows: 16 loads of 16 B in flight per lane, and the
 // same fp32 sum in slot order that page_mean_dword() makes, so a page's mean key
 // is bit-identical whether it is built here or by the append that fills the page.
 template <bool F16>
 __global__ __launch_bounds__(256) void build_kbar_kernel(AppendParams p, int page_blocks) {
-  const int sub = threadIdx.x >> 4, c16 = threadIdx.x & 15;
+  const int lpp = p.head_dim / 8;  // lanes per page = 16-byte chunks of a head row
+  const int sub = threadIdx.x / lpp, c16 = threadIdx.x - sub * lpp;
   const int item = blockIdx.x / page_blocks;
-  const int page = (blockIdx.x - item * page_blocks) * 16 + sub;
+  const int page = (blockIdx.x - item * page_blocks) * (256 / lpp) + sub;
   const int b = item / p.num_kv_heads, h = item - b * p.num_kv_heads;
   const int s = p.page_indptr[b], e = p.page_indptr[b + 1];
   const int n_pages = e - s;
@@ -57,14 +66,14 @@ __global__ __launch_bounds__(256) void build_kbar_kernel(AppendParams p, int pag
   if (pid < 0 || pid >= p.num_pages) return;
   const int kb = kbar_block_of(p.slot_ids, p.num_slots, b);
   if (kb < 0) return;
-  const int row_stride = p.num_kv_heads * (kHeadDim / 2);  // dwords per token row
+  const int row_stride = p.num_kv_heads * (p.head_dim / 2);  // dwords per token row
   const int64_t page_dwords = 2LL * p.page_size * row_stride;
-  const u32x4* kplane = reinterpret_cast<const u32x4*>(p.kv_cache + pid * page_dwords + h * (kHeadDim / 2)) + c16;
+  const u32x4* kplane = reinterpret_cast<const u32x4*>(p.kv_cache + pid * page_dwords + h * (p.head_dim / 2)) + c16;
   const u32x4 m = page_mean_16B<F16>(kplane, row_stride / 4, p.page_size);
   // Streaming store: the mean keys are not read again by this launch.  (Stores that leave the caches while the
   // read stream is saturated cost about five times their bytes: 2.1 GB of them take the config-1 build from
   // 4.95 to 6.97 ms with a plain store, 6.55 ms with this one; writing them in 64 KiB bursts changes nothing.)
-  __builtin_nontemporal_store(m, reinterpret_cast<u32x4*>(p.kbar + kbar_row_index(kb, h, page, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2)) + c16);
+  __builtin_nontemporal_store(m, reinterpret_cast<u32x4*>(p.kbar + kbar_row_index(kb, h, page, p.num_kv_heads, p.kbar_pages) * (p.head_dim / 2)) + c16);
 }
 
 // ---- ragged multi-token append ------------------------------------------------
@@ -78,6 +87,7 @@ struct RaggedAppendParams {
   const int32_t* page_indptr;
   const int32_t* last_page_len;
   int batch, num_kv_heads, kbar_pages, page_size;
+  int head_dim;  // 128 or 64
   int64_t nnz;
   int64_t num_pages;
   const int32_t* slot_ids;  // kbar row block of each sequence (null: the sequence's own index)
@@ -97,7 +107,7 @@ __device__ __forceinline__ int owner_of_row(const int32_t* indptr, int batch, in
 constexpr int kRaggedRows = 32;  // appended token rows one workgroup moves
 
 // grid = ceil(nnz / kRaggedRows) blocks of 256 threads.  A token's K row over all
-// heads is one contiguous run of Hkv*256 bytes in k[] and in its page slot (and
+// heads is one contiguous run of Hkv * head_dim * 2 bytes in k[] and in its page slot (and
 // likewise V), so the workgroup's rows are moved as 16-byte chunks, several in
 // flight per thread; where each row goes is worked out once per row (threads
 // 0..31) and handed over in LDS.  The page table describes the cache after the
@@ -108,7 +118,7 @@ __global__ __launch_bounds__(256) void append_ragged_kernel(RaggedAppendParams p
   const int tid = threadIdx.x;
   const int64_t row0 = (int64_t)blockIdx.x * kRaggedRows;
   const int rows_here = (int)min((int64_t)kRaggedRows, p.nnz - row0);
-  const int cpr = p.num_kv_heads * (kHeadDim / 8);  // 16-byte chunks per token row (all heads)
+  const int cpr = p.num_kv_heads * (p.head_dim / 8);  // 16-byte chunks per token row (all heads)
   const int P = p.page_size;
   if (tid < kRaggedRows) {
     int64_t dst = -1;
@@ -175,7 +185,7 @@ __global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p)
   const int tid = threadIdx.x;
   const int64_t row0 = (int64_t)blockIdx.x * kRaggedRows;
   const int rows_here = (int)min((int64_t)kRaggedRows, p.nnz - row0);
-  const int cpr = p.num_kv_heads * (kHeadDim / 8);
+  const int cpr = p.num_kv_heads * (p.head_dim / 8);
   const int P = p.page_size;
   if (tid < kRaggedRows) {
     int64_t src = -1, dst = 0;
@@ -195,7 +205,7 @@ __global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p)
           const int kb = kbar_block_of(p.slot_ids, p.num_slots, b);
           if (pid >= 0 && pid < p.num_pages && kb >= 0) {
             src = pid * 2 * P * cpr;
-            dst = kbar_row_index(kb, 0, (int)page, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 8);
+            dst = kbar_row_index(kb, 0, (int)page, p.num_kv_heads, p.kbar_pages) * (p.head_dim / 8);
           }
         }
       }
@@ -204,15 +214,16 @@ __global__ __launch_bounds__(256) void refresh_kbar_kernel(RaggedAppendParams p)
     dst16[tid] = dst;
   }
   __syncthreads();
-  const int sub = tid >> 4, c16 = tid & 15;
+  const int lpp = p.head_dim / 8;  // lanes per (completed page, head) = 16-byte chunks of a head row
+  const int sub = tid / lpp, c16 = tid - sub * lpp;
   const u32x4* cache = reinterpret_cast<const u32x4*>(p.kv_cache);
   u32x4* kbar = reinterpret_cast<u32x4*>(p.kbar);
-  for (int pair = sub; pair < rows_here * p.num_kv_heads; pair += 16) {
+  for (int pair = sub; pair < rows_here * p.num_kv_heads; pair += 256 / lpp) {
     const int r = pair / p.num_kv_heads, h = pair - r * p.num_kv_heads;
     const int64_t src = src16[r];
     if (src < 0) continue;
-    const u32x4 m = page_mean_16B<F16>(cache + src + h * (kHeadDim / 8) + c16, cpr, P);
-    kbar[dst16[r] + (int64_t)h * p.kbar_pages * (kHeadDim / 8) + c16] = m;
+    const u32x4 m = page_mean_16B<F16>(cache + src + h * lpp + c16, cpr, P);
+    kbar[dst16[r] + (int64_t)h * p.kbar_pages * lpp + c16] = m;
   }
 }
 
@@ -223,7 +234,7 @@ static int check_append_args(const char* fn, const void* kv_cache, const void* p
   if (slot_ids && num_slots < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_slots=%d must be >= 1 when slot_ids is given", fn, num_slots);
   if (!kv_cache || !page_indices || !page_indptr || !last_page_len)
     return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
-  int st = check_common_dims(fn, batch, num_kv_heads, num_kv_heads, head_dim, page_size);
+  int st = check_common_dims(fn, batch, num_kv_heads, num_kv_heads, head_dim, page_size, true);
   if (st) return st;
   if (num_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_pages=%lld must be >= 1", fn, (long long)num_pages);
   if (has_kbar && kbar_pages < 1)
@@ -260,6 +271,7 @@ static int append_impl(const char* fn, bool f16, const uint16_t* k, const uint16
   p.num_kv_heads = num_kv_heads;
   p.kbar_pages = kbar_pages;
   p.page_size = page_size;
+  p.head_dim = head_dim;
   p.num_pages = num_pages;
   p.slot_ids = slot_ids;
   p.num_slots = slot_ids ? num_slots : batch;
@@ -297,7 +309,8 @@ static int build_kbar_impl(const char* fn, bool f16, const uint16_t* kv_cache, u
   if (!aligned16(kbar)) return fail(KIN_ERR_MISALIGNED, "%s: kbar must be 16-byte aligned", fn);
   if (batch == 0) return KIN_OK;
   const int64_t items = (int64_t)batch * num_kv_heads;
-  const int page_blocks = (kbar_pages + 15) / 16;
+  const int pages_per_block = 256 / (head_dim / 8);
+  const int page_blocks = (kbar_pages + pages_per_block - 1) / pages_per_block;
   if (items * page_blocks > 0x7fffffffLL)
     return fail(KIN_ERR_UNSUPPORTED, "%s: batch*num_kv_heads*kbar_pages too large for one launch", fn);
   AppendParams p;
@@ -312,6 +325,7 @@ static int build_kbar_impl(const char* fn, bool f16, const uint16_t* kv_cache, u
   p.num_kv_heads = num_kv_heads;
   p.kbar_pages = kbar_pages;
   p.page_size = page_size;
+  p.head_dim = head_dim;
   p.num_pages = num_pages;
   p.slot_ids = slot_ids;
   p.num_slots = slot_ids ? num_slots : batch;
@@ -365,6 +379,7 @@ static int append_ragged_impl(const char* fn, bool f16, const uint16_t* k, const
   p.num_kv_heads = num_kv_heads;
   p.kbar_pages = kbar_pages;
   p.page_size = page_size;
+  p.head_dim = head_dim;
   p.nnz = nnz;
   p.num_pages = num_pages;
   p.slot_ids = slot_ids;

@@ -29,6 +29,13 @@
 // runs on v_mfma_f32_16x16x4_f32, whose K dimension adds the wave's four row groups up
 // inside the matrix unit (same registers per lane as the narrow form, four times the
 // matrix cycles).
+//
+// Head rows of 64 elements (HD = 64, 128 bytes): a tile is 2 KiB of keys and 2 KiB of values.  K arrives in
+// 2 LDS-direct loads of 8 rows each and S takes 2 matrix instructions.  In the narrow form a lane fetches
+// 2 V rows -- the 16 lanes of a row group split into two halves of 8 chunks, the lower half taking tokens
+// 4*kg + 0..1 and the upper half 4*kg + 2..3 -- and the two halves' partial outputs are added at the end;
+// the wide form keeps 4 V rows per lane with both halves fetching the same chunks (its P V instruction
+// shares one probability between all 16 columns), so its columns 8..15 repeat columns 0..7.
 #pragma once
 
 #include <cmath>
@@ -37,9 +44,21 @@
 
 namespace kin {
 
-// s_waitcnt immediate for "vmcnt <= 4, no wait on expcnt / lgkmcnt" (gfx9 encoding:
+// s_waitcnt immediate for "vmcnt <= n (n < 16), no wait on expcnt / lgkmcnt" (gfx9 encoding:
 // vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]).
-constexpr int kWaitVm4 = 4 | (7 << 4) | (15 << 8);
+constexpr int wait_vm_imm(int n) { return n | (7 << 4) | (15 << 8); }
+
+// XOR swizzle of the K staging area: position p of row R holds the row's 16-byte chunk p ^ attend_swizzle(R),
+// so that the 16 lanes that read one chunk column of 16 different rows hit different banks.  Rows of
+// 256 bytes: R itself; rows of 128 bytes (two rows per 64 banks): rows 8..15 get the odd patterns.
+template <int HD>
+__device__ __forceinline__ int attend_swizzle(int row) {
+  if constexpr (HD == 128) return row & 15;
+  else return (row ^ (row >> 3)) & 7;
+}
+// V rows a lane fetches per tile: 4, or 2 in the narrow form with 128-byte rows.
+template <int NG, int HD>
+constexpr int attend_v_loads() { return (NG == 1 && HD == 64) ? 2 : 4; }
 
 constexpr float kNegInf = -INFINITY;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -49,13 +68,13 @@ constexpr float kLn2 = 0.6931471805599453f;
 // ka: this lane's 4 K chunks in MFMA A layout.  Leaves the probabilities of
 // this lane's 4 tokens in pr.  Requires 0 <= first_token <= 16 and
 // 0 <= valid_tokens <= 16 (an empty range masks the whole tile).
-template <bool F16 = false>
-__device__ __forceinline__ void page_scores(const uint4 (&ka)[4], const uint4 (&qB)[4], float& m_run, float& l_run,
+template <bool F16 = false, int KC = 4>
+__device__ __forceinline__ void page_scores(const uint4 (&ka)[KC], const uint4 (&qB)[KC], float& m_run, float& l_run,
                                             floatx4 (&O)[8], float (&pr)[4], float scale_log2, int first_token,
                                             int valid_tokens, int kg) {
   floatx4 S = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int c = 0; c < 4; ++c) S = mfma_16x16x32<F16>(ka[c], qB[c], S);
+  for (int c = 0; c < KC; ++c) S = mfma_16x16x32<F16>(ka[c], qB[c], S);
   float s[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r)  // token slots [first_token, valid_tokens) of the tile count
@@ -82,11 +101,20 @@ __device__ __forceinline__ void page_scores(const uint4 (&ka)[4], const uint4 (&
   l_run += (pr[0] + pr[1]) + (pr[2] + pr[3]);
 }
 
-// Second half: O += P V.  vr: this lane's 4 V rows (row 4*kg + r).
-template <bool F16 = false>
-__device__ __forceinline__ void page_pv(const u32x4 (&vr)[4], const float (&pr)[4], floatx4 (&O)[8]) {
+// Second half: O += P V.  vr: this lane's NV V rows (row 4*kg + r; with NV = 2: row 4*kg + 2*half + r, where
+// half says which of the two 8-chunk halves of its row group the lane is in).
+template <bool F16 = false, int NV = 4>
+__device__ __forceinline__ void page_pv(const u32x4 (&vr)[NV], const float (&pr4)[4], floatx4 (&O)[8], int half) {
+  float pr[NV];
+  if constexpr (NV == 4) {
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
+    for (int r = 0; r < 4; ++r) pr[r] = pr4[r];
+  } else {
+    pr[0] = half ? pr4[2] : pr4[0];
+    pr[1] = half ? pr4[3] : pr4[1];
+  }
+#pragma unroll
+  for (int r = 0; r < NV; ++r) {
     const u32x4 vv = vr[r];
     const float vf[8] = {elem_lo<F16>(vv.x), elem_hi<F16>(vv.x), elem_lo<F16>(vv.y), elem_hi<F16>(vv.y),
                          elem_lo<F16>(vv.z), elem_hi<F16>(vv.z), elem_lo<F16>(vv.w), elem_hi<F16>(vv.w)};
@@ -99,10 +127,12 @@ __device__ __forceinline__ void page_pv(const u32x4 (&vr)[4], const float (&pr)[
 // Zeroes the V rows of token slots outside [first_token, valid_tokens): their
 // probabilities are 0, but 0 * NaN would still poison the accumulator when an
 // unused cache slot happens to hold a NaN or Inf bit pattern.
-__device__ __forceinline__ void clear_unused_v_rows(u32x4 (&vr)[4], int first_token, int valid_tokens, int kg) {
+// row0: the tile row of vr[0] (4*kg, or 4*kg + 2*half with two rows per lane).
+template <int NV>
+__device__ __forceinline__ void clear_unused_v_rows(u32x4 (&vr)[NV], int first_token, int valid_tokens, int row0) {
 #pragma unroll
-  for (int r = 0; r < 4; ++r)
-    if (!((unsigned)(4 * kg + r - first_token) < (unsigned)(valid_tokens - first_token))) vr[r] = u32x4{0u, 0u, 0u, 0u};
+  for (int r = 0; r < NV; ++r)
+    if (!((unsigned)(row0 + r - first_token) < (unsigned)(valid_tokens - first_token))) vr[r] = u32x4{0u, 0u, 0u, 0u};
 }
 
 // NG names the kernel variant by the heads it holds, 4 * NG: 1 (narrow) or 4 (wide).
@@ -115,13 +145,13 @@ constexpr bool attend_variant_ok() { return NG == 1 || NG == 4; }
 // product below adds their tokens up inside one matrix instruction: it moves only
 // when some token of the tile exceeds it (rare once a list is under way), and only
 // then do the lanes exchange their maxima and rescale O.
-template <bool F16 = false>
-__device__ __forceinline__ void page_scores_wide(const uint4 (&ka)[4], const uint4 (&qB)[4], float& m_run, float& l_run,
+template <bool F16 = false, int KC = 4>
+__device__ __forceinline__ void page_scores_wide(const uint4 (&ka)[KC], const uint4 (&qB)[KC], float& m_run, float& l_run,
                                                  floatx4 (&O)[8], float (&pr)[4], float scale_log2, int first_token,
                                                  int valid_tokens, int kg) {
   floatx4 S = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int c = 0; c < 4; ++c) S = mfma_16x16x32<F16>(ka[c], qB[c], S);
+  for (int c = 0; c < KC; ++c) S = mfma_16x16x32<F16>(ka[c], qB[c], S);
   float s[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r)
@@ -170,9 +200,9 @@ __device__ __forceinline__ void page_pv_wide(const u32x4 (&vr)[4], const float (
 
 // Wave-uniform description of one list for attend_list().
 struct AttendArgs {
-  const uint16_t* q_bh;  // the group's G query rows (contiguous, 128 bf16 each)
-  const char* kvb;       // kv_cache base + h * 256 bytes
-  int row_bytes;         // bytes between token rows of a page (H_kv * 256)
+  const uint16_t* q_bh;  // the group's G query rows (contiguous, HD elements each)
+  const char* kvb;       // kv_cache base + h * HD * 2 bytes
+  int row_bytes;         // bytes between token rows of a page (H_kv * HD * 2)
   int page_bytes;        // 2 * page_size * row_bytes
   int span;              // bytes addressable from kvb within one page
   int page_size;         // tokens per page: 16, 32 or 64
@@ -203,28 +233,30 @@ __device__ __forceinline__ unsigned attend_rotation(int list, int split) {
 
 // K tiles a wave keeps staged in LDS in attend_list(): the one being read and the one in flight.
 constexpr int kAttendStages = 2;
-// K staging for NW waves of kAttendStages 4 KiB stages each; the same 8 KiB per wave hold the
-// merge buffer [NW][4*NG][128] fp32 afterwards (2 KiB per wave for NG = 1, 8 KiB for the wide form).
+// K staging for NW waves of kAttendStages stages of 4 KiB each (2 KiB with 64-element rows); the same 8 KiB per wave hold the
+// merge buffer [NW][4*NG][HD] fp32 afterwards (up to 2 KiB per wave for NG = 1, 8 KiB for the wide form).
 constexpr int attend_lds_bytes(int nw) { return nw * kAttendStages * 4096; }
 
 // Common tail of the attention loops: merges the wave's 4 row groups, then the
 // workgroup's NW waves through LDS, and hands out the normalised results.
 // m_run / l_run / O: this lane's online-softmax state (see page_scores).
-template <int NG, int NW, typename Emit>
+template <int NG, int NW, int HD, typename Emit>
 __device__ __forceinline__ void attend_finish(float m_run, float l_run, floatx4 (&O)[8], int G, unsigned char* lds,
                                               float (*sm_m)[4 * NG], float (*sm_l)[4 * NG], Emit emit) {
   static_assert(attend_variant_ok<NG>(), "NG is 1 (up to 4 heads) or 4 (up to 16)");
+  static_assert(HD == 128 || HD == 64, "head rows of 128 or 64 elements");
+  constexpr int CPR = HD / 8;  // 16-byte chunks of a head row
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int l = tid & 63, kg = l >> 4, c16 = l & 15;
+  const int l = tid & 63, kg = l >> 4, c16 = l & 15, cc = c16 & (CPR - 1);
   // LDS-direct loads that are still in flight (masked tail pages) must land
   // before the staging area is reused below.
   __builtin_amdgcn_s_waitcnt(0);
-  float* ow = reinterpret_cast<float*>(lds);  // [NW waves][4*NG heads][128]
+  float* ow = reinterpret_cast<float*>(lds);  // [NW waves][4*NG heads][HD]
 
   if constexpr (NG == 4) {
     // Wide form: O is already summed over the row groups; the lanes of a head share m
-    // and hold partial sums l.
+    // and hold partial sums l.  (HD = 64: lanes c16 >= 8 hold copies of lanes c16 - 8.)
     float ll = l_run;
     ll += __shfl_xor(ll, 16);
     ll += __shfl_xor(ll, 32);
@@ -232,8 +264,8 @@ __device__ __forceinline__ void attend_finish(float m_run, float l_run, floatx4 
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int h = 4 * kg + i;
-      if (h < G) {
-        float* dst = ow + ((w * 16 + h) * kHeadDim + 8 * c16);
+      if (h < G && c16 < CPR) {
+        float* dst = ow + ((w * 16 + h) * HD + 8 * cc);
         *reinterpret_cast<float4*>(dst) = make_float4(O[0][i], O[1][i], O[2][i], O[3][i]);
         *reinterpret_cast<float4*>(dst + 4) = make_float4(O[4][i], O[5][i], O[6][i], O[7][i]);
       }
@@ -256,15 +288,18 @@ __device__ __forceinline__ void attend_finish(float m_run, float l_run, floatx4 
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       float x0 = O[u][0] * s0, x1 = O[u][1] * s1, x2 = O[u][2] * s2, x3 = O[u][3] * s3;
+      if constexpr (HD == 64) {  // the two halves of a row group took different tokens of it
+        x0 += __shfl_xor(x0, 8); x1 += __shfl_xor(x1, 8); x2 += __shfl_xor(x2, 8); x3 += __shfl_xor(x3, 8);
+      }
       x0 += __shfl_xor(x0, 16); x1 += __shfl_xor(x1, 16); x2 += __shfl_xor(x2, 16); x3 += __shfl_xor(x3, 16);
       x0 += __shfl_xor(x0, 32); x1 += __shfl_xor(x1, 32); x2 += __shfl_xor(x2, 32); x3 += __shfl_xor(x3, 32);
       O[u] = floatx4{x0, x1, x2, x3};
     }
     __syncthreads();  // every wave is done with its K staging area
-    if (kg == 0) {
+    if (kg == 0 && c16 < CPR) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float* dst = ow + ((w * 4 + i) * kHeadDim + 8 * c16);
+        float* dst = ow + ((w * 4 + i) * HD + 8 * cc);
         *reinterpret_cast<float4*>(dst) = make_float4(O[0][i], O[1][i], O[2][i], O[3][i]);
         *reinterpret_cast<float4*>(dst + 4) = make_float4(O[4][i], O[5][i], O[6][i], O[7][i]);
       }
@@ -277,8 +312,8 @@ __device__ __forceinline__ void attend_finish(float m_run, float l_run, floatx4 
   __syncthreads();
 
   // ---- merge the NW waves and hand the results out ------------------------------
-  for (int idx = tid; idx < 4 * NG * kHeadDim; idx += NW * 64) {
-    const int g = idx >> 7, d = idx & 127;
+  for (int idx = tid; idx < 4 * NG * HD; idx += NW * 64) {
+    const int g = idx / HD, d = idx & (HD - 1);
     if (g < G) {
       float mm = kNegInf;
 #pragma unroll
@@ -288,7 +323,7 @@ __device__ __forceinline__ void attend_finish(float m_run, float l_run, floatx4 
 #pragma unroll
       for (int wv = 0; wv < NW; ++wv) {
         const float sc = fast_exp2(sm_m[wv][g] - m_safe);
-        num += ow[(wv * 4 * NG + g) * kHeadDim + d] * sc;
+        num += ow[(wv * 4 * NG + g) * HD + d] * sc;
         den += sm_l[wv][g] * sc;
       }
       const float o = (den > 0.f) ? num / den : 0.f;
@@ -304,22 +339,30 @@ __device__ __forceinline__ void attend_finish(float m_run, float l_run, floatx4 
 // lds: attend_lds_bytes(NW), 16-byte aligned; sm_m / sm_l: NW x
 // (4*NG) floats each.
 // Every one of the workgroup's NW*64 threads calls this.
-template <int NG, int NW, bool F16 = false, typename IdAt, typename Emit>
+template <int NG, int NW, bool F16 = false, int HD = kHeadDim, typename IdAt, typename Emit>
 __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, unsigned char* lds,
                                             float (*sm_m)[4 * NG], float (*sm_l)[4 * NG], Emit emit) {
+  static_assert(HD == 128 || HD == 64, "head rows of 128 or 64 elements");
+  constexpr int CPR = HD / 8;                      // 16-byte chunks of a head row: 16 or 8
+  constexpr int KC = HD / 32;                      // matrix steps over the head dimension = LDS-direct loads per K tile: 4 or 2
+  constexpr int RPI = 64 / CPR;                    // K rows one LDS-direct load brings: 4 or 8
+  constexpr int NV = attend_v_loads<NG, HD>();     // V rows per lane and tile
+  constexpr int kStage = kPageSize * HD * 2;       // bytes of one K stage (a tile's keys)
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int l = tid & 63, kg = l >> 4, c16 = l & 15, gq = l & 3;
+  const int l = tid & 63, kg = l >> 4, c16 = l & 15, gq = l & 3, cc = c16 & (CPR - 1);
+  const int half = NV == 2 ? (c16 >> 3) : 0;       // which half of its row group's tokens this lane's V rows cover
+  const int vrow0 = 4 * kg + 2 * half;             // tile row of this lane's first V row
   const int G = a.G;
   const int n = a.n, p0 = a.p0, p1 = a.p1, last_len = a.last_len;
 
   // Query operands: B[k][j], j = l%16 -> head l%4 (wide form: head l%16), k-chunk = l/16.
-  uint4 qB[4];
+  uint4 qB[KC];
   {
     const int g = min(NG == 4 ? c16 : gq, G - 1);
-    const uint16_t* qp = a.q_bh + (int64_t)g * kHeadDim + 8 * kg;
+    const uint16_t* qp = a.q_bh + (int64_t)g * HD + 8 * kg;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) qB[c] = *reinterpret_cast<const uint4*>(qp + 32 * c);
+    for (int c = 0; c < KC; ++c) qB[c] = *reinterpret_cast<const uint4*>(qp + 32 * c);
   }
 
   const int row_bytes = a.row_bytes;
@@ -329,38 +372,38 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
   // A tile's rows are addressed from its first K row: its V rows lie one K plane
   // (page_size rows) further.
   const int tshift = page_tile_shift(a.page_size), tmask = (1 << tshift) - 1;
-  int voff[4];
+  int voff[NV];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) voff[c] = (a.page_size + 4 * kg + c) * row_bytes + c16 * 16;
-  // K staging: kAttendStages 4 KiB stages per wave, filled by LDS-direct buffer loads
-  // (no VGPRs while in flight).  Load c brings rows 4c..4c+3: lane (kg, c16)
-  // lands at LDS row 4c+kg, position c16, and fetches the chunk that belongs
-  // there under the XOR swizzle (position p of row R holds chunk p ^ R).
-  unsigned char* kl = lds + w * (kAttendStages * 4096);
-  int kdma_off[4], lds_r[4];
+  for (int r = 0; r < NV; ++r) voff[r] = (a.page_size + vrow0 + r) * row_bytes + cc * 16;
+  // K staging: kAttendStages stages of one tile's keys per wave, filled by LDS-direct buffer loads
+  // (no VGPRs while in flight).  Load c brings rows RPI*c .. RPI*c + RPI-1, one kilobyte: lane l
+  // lands at LDS row RPI*c + l / CPR, position l % CPR, and fetches the chunk that belongs
+  // there under the XOR swizzle (see attend_swizzle).
+  unsigned char* kl = lds + w * (kAttendStages * kStage);
+  int kdma_off[KC], lds_r[KC];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    const int row = 4 * c + kg;
-    kdma_off[c] = row * row_bytes + ((c16 ^ row) & 15) * 16;
+  for (int c = 0; c < KC; ++c) {
+    const int row = RPI * c + l / CPR;
+    kdma_off[c] = row * row_bytes + ((cc ^ attend_swizzle<HD>(row)) & (CPR - 1)) * 16;
     const int chunk_r = 4 * c + kg;  // chunk of row c16 that MFMA c wants from this lane
-    lds_r[c] = c16 * 256 + ((chunk_r ^ c16) & 15) * 16;
+    lds_r[c] = c16 * (HD * 2) + ((chunk_r ^ attend_swizzle<HD>(c16)) & (CPR - 1)) * 16;
   }
 
   float m_run = kNegInf, l_run = 0.f;
   floatx4 O[8];
 #pragma unroll
   for (int u = 0; u < 8; ++u) O[u] = floatx4{0.f, 0.f, 0.f, 0.f};
-  auto scores = [&](const uint4 (&ka)[4], float (&pr)[4], int valid) {
+  auto scores = [&](const uint4 (&ka)[KC], float (&pr)[4], int valid) {
     if constexpr (NG == 4)
-      page_scores_wide<F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, valid >> 8, valid & 255, kg);
+      page_scores_wide<F16, KC>(ka, qB, m_run, l_run, O, pr, a.scale_log2, valid >> 8, valid & 255, kg);
     else
-      page_scores<F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, valid >> 8, valid & 255, kg);
+      page_scores<F16, KC>(ka, qB, m_run, l_run, O, pr, a.scale_log2, valid >> 8, valid & 255, kg);
   };
-  auto pv = [&](const u32x4 (&vr)[4], const float (&pr)[4]) {
+  auto pv = [&](const u32x4 (&vr)[NV], const float (&pr)[4]) {
     if constexpr (NG == 4)
       page_pv_wide<F16>(vr, pr, O);
     else
-      page_pv<F16>(vr, pr, O);
+      page_pv<F16, NV>(vr, pr, O, half);
   };
 
   // This wave takes the tiles my_first, my_first+NW, ... of the list entries p0 .. p1-1
@@ -403,30 +446,30 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
     const int tile_off = sub16 * row_bytes;
     return make_rsrc(kvb + (int64_t)(ok ? id : 0) * page_bytes + tile_off, ok ? span - tile_off : 0);
   };
-  auto issue_v = [&](__amdgpu_buffer_rsrc_t r, u32x4 (&vv)[4]) {
+  auto issue_v = [&](__amdgpu_buffer_rsrc_t r, u32x4 (&vv)[NV]) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) vv[c] = __builtin_amdgcn_raw_buffer_load_b128(r, voff[c], 0, kStreamLoad);
+    for (int c = 0; c < NV; ++c) vv[c] = __builtin_amdgcn_raw_buffer_load_b128(r, voff[c], 0, kStreamLoad);
   };
   auto issue_k = [&](__amdgpu_buffer_rsrc_t r, int stage) {
     __attribute__((address_space(3))) unsigned char* dst =
-        (__attribute__((address_space(3))) unsigned char*)(kl + stage * 4096);
+        (__attribute__((address_space(3))) unsigned char*)(kl + stage * kStage);
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
+    for (int c = 0; c < KC; ++c)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(r, dst + c * 1024, 16, kdma_off[c], 0, 0, kStreamLoad);
   };
-  auto read_k = [&](int stage, uint4 (&ka)[4]) {
+  auto read_k = [&](int stage, uint4 (&ka)[KC]) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) ka[c] = *reinterpret_cast<const uint4*>(kl + stage * 4096 + lds_r[c]);
+    for (int c = 0; c < KC; ++c) ka[c] = *reinterpret_cast<const uint4*>(kl + stage * kStage + lds_r[c]);
   };
 
   // The compiler does not order LDS reads after LDS-direct loads by itself, so
-  // the wait is explicit: when it executes, exactly the 4 V loads issued just
+  // the wait is explicit: when it executes, exactly the NV V loads issued just
   // before it are allowed to be outstanding, which means the K stage about to
   // be read (and the V registers about to be used) have landed.  The scheduling
   // fences keep the instruction order this count relies on.
   if (iters > 0 && n > 0) {
-    u32x4 vA[4], vB[4];
-    uint4 ka[4];
+    u32x4 vA[NV], vB[NV];
+    uint4 ka[KC];
     float pr[4];
     int validA, validB;
     {
@@ -441,7 +484,7 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
         __builtin_amdgcn_sched_barrier(0);
         issue_v(r1, vB);
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(kWaitVm4);
+        __builtin_amdgcn_s_waitcnt(wait_vm_imm(NV));
         __builtin_amdgcn_sched_barrier(0);
         read_k(0, ka);
         __builtin_amdgcn_sched_barrier(0);
@@ -450,7 +493,7 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
         scores(ka, pr, validA);
         __builtin_amdgcn_sched_barrier(0);
         id_next = load_id(it + 2);  // lands while the P V products run
-        if (validA != kPageSize) clear_unused_v_rows(vA, validA >> 8, validA & 255, kg);  // partial page: rare
+        if (validA != kPageSize) clear_unused_v_rows<NV>(vA, validA >> 8, validA & 255, vrow0);  // partial page: rare
         pv(vA, pr);
       }
       {
@@ -458,7 +501,7 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
         __builtin_amdgcn_sched_barrier(0);
         issue_v(r2, vA);
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(kWaitVm4);
+        __builtin_amdgcn_s_waitcnt(wait_vm_imm(NV));
         __builtin_amdgcn_sched_barrier(0);
         read_k(1, ka);
         __builtin_amdgcn_sched_barrier(0);
@@ -467,22 +510,22 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
         scores(ka, pr, validB);
         __builtin_amdgcn_sched_barrier(0);
         id_next = load_id(it + 3);
-        if (validB != kPageSize) clear_unused_v_rows(vB, validB >> 8, validB & 255, kg);
+        if (validB != kPageSize) clear_unused_v_rows<NV>(vB, validB >> 8, validB & 255, vrow0);
         pv(vB, pr);
       }
     }
   }
-  attend_finish<NG, NW>(m_run, l_run, O, G, lds, sm_m, sm_l, emit);
+  attend_finish<NG, NW, HD>(m_run, l_run, O, G, lds, sm_m, sm_l, emit);
 }
 
 // Merges the `parts` partial results that the workgroups sharing one list left in
-// global memory (ws_po [lists, parts, G, 128] normalised outputs, ws_plse [lists, parts, G]
+// global memory (ws_po [lists, parts, G, HD] normalised outputs, ws_plse [lists, parts, G]
 // base-2 log-sum-exps, both fp32 bits written at device scope) and writes the list's G output
 // rows (out_bh) and, if lse_bh is set, their natural-log log-sum-exps.  Run by the workgroup
 // that counted in last, all NT threads; lds: room for (parts + 1) * G floats, free for reuse.
 // The log-sum-exps first become weights in LDS, then every thread sums its output element over
 // the parts with independent device-scope loads (the arithmetic of merge_splits_kernel).
-template <int NT, bool F16>
+template <int NT, bool F16, int HD = kHeadDim>
 __device__ __forceinline__ void merge_list_parts(unsigned char* lds, const uint32_t* ws_po, const uint32_t* ws_plse, int item,
                                                  int parts, int G, uint16_t* out_bh, float* lse_bh) {
   const int tid = threadIdx.x;
@@ -507,16 +550,16 @@ __device__ __forceinline__ void merge_list_parts(unsigned char* lds, const uint3
     if (lse_bh) lse_bh[tid] = (den > 0.f) ? (mm + fast_log2(den)) * kLn2 : kNegInf;
   }
   __syncthreads();
-  const __amdgpu_buffer_rsrc_t ro = make_rsrc(ws_po + first_row * kHeadDim, parts * G * kHeadDim * (int)sizeof(float));
-  for (int idx = tid; idx < G * kHeadDim; idx += NT) {
-    const int g = idx >> 7, d = idx & (kHeadDim - 1);
+  const __amdgpu_buffer_rsrc_t ro = make_rsrc(ws_po + first_row * HD, parts * G * HD * (int)sizeof(float));
+  for (int idx = tid; idx < G * HD; idx += NT) {
+    const int g = idx / HD, d = idx & (HD - 1);
     float num = 0.f;
 #pragma unroll 8
     for (int sp = 0; sp < parts; ++sp)
-      num += __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ro, ((sp * G + g) * kHeadDim + d) * 4, 0, kDeviceScope)) *
+      num += __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ro, ((sp * G + g) * HD + d) * 4, 0, kDeviceScope)) *
              wl[sp * G + g];
     const float den = den_g[g];
-    out_bh[g * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(den > 0.f ? num / den : 0.f);
+    out_bh[g * HD + d] = (uint16_t)f32_to_elem<F16>(den > 0.f ? num / den : 0.f);
   }
 }
 

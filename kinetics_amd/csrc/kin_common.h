@@ -8,7 +8,8 @@
 
 namespace kin {
 
-constexpr int kHeadDim = 128;    // elements per head row (256 B in bf16)
+constexpr int kHeadDim = 128;    // elements per head row (256 B in bf16): the default, and the largest, head dimension
+constexpr int kHeadDimSmall = 64;  // the second head dimension the page path is built for (128-byte rows)
 constexpr int kPageSize = 16;    // tokens of one attention tile (an MFMA tile is 16 keys); the smallest page
 constexpr int kMaxPageSize = 64; // pages hold 16, 32 or 64 tokens: 1, 2 or 4 tiles
 constexpr int kRowBytes = kHeadDim * 2;
@@ -31,6 +32,7 @@ constexpr int kMaxLocalTokens = (kMaxFixedPages - 1) * kPageSize + 1;
 __host__ __device__ inline int max_local_pages(int local_tokens) { return 1 + (local_tokens + kPageSize - 2) / kPageSize; }
 
 inline bool supported_page_size(int ps) { return ps == 16 || ps == 32 || ps == 64; }
+inline bool supported_head_dim(int hd) { return hd == kHeadDim || hd == kHeadDimSmall; }
 // log2(page_size / 16): a page is 1 << page_tile_shift(ps) tiles of 16 tokens.
 __host__ __device__ inline int page_tile_shift(int ps) { return ps >= 64 ? 2 : (ps >= 32 ? 1 : 0); }
 
@@ -56,8 +58,10 @@ int check_hip(hipError_t e, const char* what);
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Shape rules every entry point shares.  Returns KIN_OK or records an error.
+// small_head_dim_built: the entry point also has kernels for head_dim 64 (the page path has, the
+// token-granular policies and the layer's row kernels have not).
 int check_common_dims(const char* fn, int batch, int num_q_heads, int num_kv_heads,
-                      int head_dim, int page_size);
+                      int head_dim, int page_size, bool small_head_dim_built = false);
 // Range rules for the always-attended parts of a page list.
 int check_fixed_pages(const char* fn, int sink_pages, int local_tokens);
 // first_page_offset: padding slots at the start of every sequence's first page.
@@ -182,6 +186,16 @@ __device__ __forceinline__ float row16_sum(float x) {
   x += dpp_f<kDppQuadXor2>(x);
   x += dpp_f<kDppHalfMirror>(x);
   x += dpp_f<kDppMirror>(x);
+  return x;
+}
+// Sum over each aligned group of LANES (8 or 16) lanes: the lanes that share one head row of LANES * 8 elements.
+template <int LANES>
+__device__ __forceinline__ float row_sum(float x) {
+  static_assert(LANES == 8 || LANES == 16, "a head row is 8 or 16 chunks of 16 bytes");
+  x += dpp_f<kDppQuadXor1>(x);
+  x += dpp_f<kDppQuadXor2>(x);
+  x += dpp_f<kDppHalfMirror>(x);
+  if constexpr (LANES == 16) x += dpp_f<kDppMirror>(x);
   return x;
 }
 

@@ -27,8 +27,9 @@ struct DecodeParams {
   float scale_log2;  // sm_scale * log2(e)
 };
 
-template <int NG, bool F16>
+template <int NG, bool F16, int HD = kHeadDim>
 __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
+  constexpr int kRowB = HD * 2;  // bytes of a head row
   __shared__ __attribute__((aligned(16))) unsigned char lds[attend_lds_bytes(4)];
   __shared__ float sm_m[4][4 * NG];
   __shared__ float sm_l[4][4 * NG];
@@ -53,11 +54,11 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
   const int per_split = (n + p.num_splits - 1) / p.num_splits;
 
   AttendArgs a;
-  a.q_bh = p.q + ((int64_t)b * p.num_q_heads + (int64_t)h * G) * kHeadDim;
-  a.kvb = reinterpret_cast<const char*>(p.kv) + (int64_t)h * kRowBytes;
-  a.row_bytes = p.num_kv_heads * kRowBytes;
+  a.q_bh = p.q + ((int64_t)b * p.num_q_heads + (int64_t)h * G) * HD;
+  a.kvb = reinterpret_cast<const char*>(p.kv) + (int64_t)h * kRowB;
+  a.row_bytes = p.num_kv_heads * kRowB;
   a.page_bytes = 2 * p.page_size * a.row_bytes;
-  a.span = a.page_bytes - h * kRowBytes;
+  a.span = a.page_bytes - h * kRowB;
   a.page_size = p.page_size;
   a.num_pages = p.num_pages;
   a.G = G;
@@ -75,21 +76,21 @@ __global__ __launch_bounds__(256, 2) void paged_decode_kernel(DecodeParams p) {
   const __attribute__((address_space(4))) int32_t* pl_c =
       reinterpret_cast<const __attribute__((address_space(4))) int32_t*>(reinterpret_cast<uintptr_t>(pl));
   const int64_t hq0 = (int64_t)b * p.num_q_heads + (int64_t)h * G;
-  attend_list<NG, 4, F16>(
+  attend_list<NG, 4, F16, HD>(
       a, [&](int i) -> int { return pl_c[i]; }, lds, sm_m, sm_l,
       [&](int g, int d, float o, float lse2) {
         const int64_t hq = hq0 + g;
         if (p.num_splits == 1) {
-          p.out[hq * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(o);
+          p.out[hq * HD + d] = (uint16_t)f32_to_elem<F16>(o);
           if (p.lse && d == 0) p.lse[hq] = lse2 * kLn2;
         } else {
-          p.ws_o[(hq * p.num_splits + split) * kHeadDim + d] = o;
+          p.ws_o[(hq * p.num_splits + split) * HD + d] = o;
           if (d == 0) p.ws_lse[hq * p.num_splits + split] = lse2;
         }
       });
 }
 
-// Split-K merge: one 128-thread block per (sequence, query head).
+// Split-K merge: one block of head_dim threads per (sequence, query head).
 template <bool F16>
 __global__ __launch_bounds__(128) void merge_splits_kernel(const float* __restrict__ ws_o,
                                                            const float* __restrict__ ws_lse,
@@ -97,6 +98,7 @@ __global__ __launch_bounds__(128) void merge_splits_kernel(const float* __restri
                                                            int num_splits) {
   const int64_t hq = blockIdx.x;
   const int d = threadIdx.x;
+  const int hd = blockDim.x;
   const float* l2 = ws_lse + hq * num_splits;
   float mm = kNegInf;
 #pragma unroll 8
@@ -106,10 +108,10 @@ __global__ __launch_bounds__(128) void merge_splits_kernel(const float* __restri
 #pragma unroll 8
   for (int s = 0; s < num_splits; ++s) {
     const float wgt = fast_exp2(l2[s] - m_safe);
-    num += ws_o[(hq * num_splits + s) * kHeadDim + d] * wgt;
+    num += ws_o[(hq * num_splits + s) * hd + d] * wgt;
     den += wgt;
   }
-  out[hq * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(den > 0.f ? num / den : 0.f);
+  out[hq * hd + d] = (uint16_t)f32_to_elem<F16>(den > 0.f ? num / den : 0.f);
   if (lse && d == 0) lse[hq] = (den > 0.f) ? (mm + fast_log2(den)) * kLn2 : kNegInf;
 }
 
@@ -141,7 +143,7 @@ static size_t workspace_bytes_for(int batch, int num_q_heads, int splits) {
 }
 
 static int launch_decode(const char* fn, DecodeParams& p, int batch, void* workspace, size_t workspace_bytes,
-                         int max_pages_per_list, int num_splits, bool f16, hipStream_t stream) {
+                         int max_pages_per_list, int num_splits, bool f16, int head_dim, hipStream_t stream) {
   int splits = num_splits > 0 ? num_splits : auto_splits(batch, p.num_kv_heads, max_pages_per_list);
   if (splits > 65535) return fail(KIN_ERR_BAD_SHAPE, "%s: num_splits=%d exceeds 65535", fn, splits);
   p.num_splits = splits;
@@ -152,7 +154,7 @@ static int launch_decode(const char* fn, DecodeParams& p, int batch, void* works
                   workspace ? workspace_bytes : (size_t)0);
     if (!aligned16(workspace)) return fail(KIN_ERR_MISALIGNED, "%s: workspace must be 16-byte aligned", fn);
     p.ws_o = static_cast<float*>(workspace);
-    p.ws_lse = p.ws_o + (size_t)batch * p.num_q_heads * splits * kHeadDim;
+    p.ws_lse = p.ws_o + (size_t)batch * p.num_q_heads * splits * head_dim;
   } else {
     p.ws_o = nullptr;
     p.ws_lse = nullptr;
@@ -162,7 +164,15 @@ static int launch_decode(const char* fn, DecodeParams& p, int batch, void* works
   p.batch = batch;
   p.rotate = attend_rotates((int64_t)batch * p.num_kv_heads) ? 1 : 0;
   dim3 grid((unsigned)lists, (unsigned)splits);
-  if (p.group <= 4) {
+  if (head_dim == kHeadDimSmall) {
+    if (p.group <= 4) {
+      if (f16) paged_decode_kernel<1, true, kHeadDimSmall><<<grid, 256, 0, stream>>>(p);
+      else paged_decode_kernel<1, false, kHeadDimSmall><<<grid, 256, 0, stream>>>(p);
+    } else {
+      if (f16) paged_decode_kernel<4, true, kHeadDimSmall><<<grid, 256, 0, stream>>>(p);
+      else paged_decode_kernel<4, false, kHeadDimSmall><<<grid, 256, 0, stream>>>(p);
+    }
+  } else if (p.group <= 4) {
     if (f16) paged_decode_kernel<1, true><<<grid, 256, 0, stream>>>(p);
     else paged_decode_kernel<1, false><<<grid, 256, 0, stream>>>(p);
   } else {
@@ -173,8 +183,8 @@ static int launch_decode(const char* fn, DecodeParams& p, int batch, void* works
   if (st) return st;
   if (splits > 1) {
     const unsigned mgrid = (unsigned)((int64_t)batch * p.num_q_heads);
-    if (f16) merge_splits_kernel<true><<<mgrid, 128, 0, stream>>>(p.ws_o, p.ws_lse, p.out, p.lse, splits);
-    else merge_splits_kernel<false><<<mgrid, 128, 0, stream>>>(p.ws_o, p.ws_lse, p.out, p.lse, splits);
+    if (f16) merge_splits_kernel<true><<<mgrid, head_dim, 0, stream>>>(p.ws_o, p.ws_lse, p.out, p.lse, splits);
+    else merge_splits_kernel<false><<<mgrid, head_dim, 0, stream>>>(p.ws_o, p.ws_lse, p.out, p.lse, splits);
     st = check_hip(hipGetLastError(), "merge_splits_kernel launch");
   }
   return st;
@@ -184,7 +194,7 @@ static int check_decode_args(const char* fn, const void* q, const void* kv_cache
                              const void* out, int batch, int num_q_heads, int num_kv_heads, int head_dim,
                              int page_size, int64_t num_pages, int first_page_offset, int num_splits) {
   if (!q || !kv_cache || !last_page_len || !out) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
-  int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size);
+  int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size, true);
   if (st) return st;
   st = check_first_page_offset(fn, first_page_offset, page_size);
   if (st) return st;
@@ -241,7 +251,7 @@ static int sparse_decode_impl(const char* fn, bool f16, const uint16_t* q, const
   p.page_size = page_size;
   const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
   p.scale_log2 = scale * 1.4426950408889634f;
-  return launch_decode(fn, p, batch, workspace, workspace_bytes, sel_stride, num_splits, f16,
+  return launch_decode(fn, p, batch, workspace, workspace_bytes, sel_stride, num_splits, f16, head_dim,
                        static_cast<hipStream_t>(stream));
 }
 
@@ -276,7 +286,7 @@ static int dense_decode_impl(const char* fn, bool f16, const uint16_t* q, const 
   p.page_size = page_size;
   const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim);
   p.scale_log2 = scale * 1.4426950408889634f;
-  return launch_decode(fn, p, batch, workspace, workspace_bytes, max_pages_per_seq, num_splits, f16,
+  return launch_decode(fn, p, batch, workspace, workspace_bytes, max_pages_per_seq, num_splits, f16, head_dim,
                        static_cast<hipStream_t>(stream));
 }
 

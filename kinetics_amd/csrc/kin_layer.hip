@@ -51,6 +51,7 @@ __device__ __forceinline__ uint32_t scale_x2(uint32_t x, float r, uint32_t w) {
 
 template <int LPR>
 __device__ __forceinline__ float group_sum(float x) {
+  if constexpr (LPR == 8) return row_sum<8>(x);
   x = row16_sum(x);
   if (LPR == 64) {
     x += __shfl_xor(x, 16);
@@ -59,7 +60,7 @@ __device__ __forceinline__ float group_sum(float x) {
   return x;
 }
 
-// LPR lanes (16 or 64) own one row; a 256-thread workgroup covers 256 / LPR rows.
+// LPR lanes (8, 16 or 64) own one row; a 256-thread workgroup covers 256 / LPR rows.
 // Lane l holds the 16-byte chunks c * LPR + l, so every load instruction of a
 // lane group covers LPR * 16 contiguous bytes.  MAXC bounds the chunks per lane
 // (the row stays in registers between the two passes): the smaller
@@ -120,30 +121,30 @@ struct QkvParams {
   float eps;
 };
 
-// 16 lanes per head row of 128 elements: q and k heads are normalised, v heads
-// copied, each to its own contiguous [batch, heads, 128] tensor.
-template <bool F16>
+// LPR lanes per head row of LPR * 8 elements (16 lanes for 128, 8 for 64): q and k heads are normalised, v heads
+// copied, each to its own contiguous [batch, heads, head_dim] tensor.
+template <bool F16, int LPR>
 __global__ __launch_bounds__(256) void qkv_norm_split_kernel(QkvParams p) {
   const int heads = p.hq + 2 * p.hkv;
-  const int64_t g = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
-  const int l = threadIdx.x & 15;
+  const int64_t g = (int64_t)blockIdx.x * (256 / LPR) + (threadIdx.x / LPR);
+  const int l = threadIdx.x & (LPR - 1);
   if (g >= (int64_t)p.batch * heads) return;
   const int64_t b = g / heads;
   const int j = (int)(g - b * heads);
-  u32x4 x = __builtin_nontemporal_load(p.qkv + b * p.row_stride + j * 16 + l);
+  u32x4 x = __builtin_nontemporal_load(p.qkv + b * p.row_stride + j * LPR + l);
   u32x4* dst;
   if (j < p.hq + p.hkv) {
     const bool is_q = j < p.hq;
-    const float ss = row16_sum(sum_sq8<F16>(x));
-    const float rinv = rsqrtf(ss * (1.0f / kHeadDim) + p.eps);
+    const float ss = row_sum<LPR>(sum_sq8<F16>(x));
+    const float rinv = rsqrtf(ss * (1.0f / (LPR * 8)) + p.eps);
     const u32x4 w = (is_q ? p.q_weight : p.k_weight)[l];
     x.x = scale_x2<F16>(x.x, rinv, w.x);
     x.y = scale_x2<F16>(x.y, rinv, w.y);
     x.z = scale_x2<F16>(x.z, rinv, w.z);
     x.w = scale_x2<F16>(x.w, rinv, w.w);
-    dst = is_q ? p.q + (b * p.hq + j) * 16 : p.k + (b * p.hkv + (j - p.hq)) * 16;
+    dst = is_q ? p.q + (b * p.hq + j) * LPR : p.k + (b * p.hkv + (j - p.hq)) * LPR;
   } else {
-    dst = p.v + (b * p.hkv + (j - p.hq - p.hkv)) * 16;
+    dst = p.v + (b * p.hkv + (j - p.hq - p.hkv)) * LPR;
   }
   dst[l] = x;
 }
@@ -206,8 +207,9 @@ static int rms_norm_impl(const char* fn, bool f16, const void* x, void* residual
   int lpr;
   if (hidden % 512 == 0 && hidden <= 512 * kNormMaxChunks) lpr = 64;
   else if (hidden % 128 == 0 && hidden <= 128 * kNormMaxChunks) lpr = 16;
+  else if (hidden == 64) lpr = 8;  // qk_norm over head rows of 64 elements
   else
-    return fail(KIN_ERR_UNSUPPORTED, "%s: hidden=%d must be a multiple of 128 up to %d or of 512 up to %d", fn, hidden,
+    return fail(KIN_ERR_UNSUPPORTED, "%s: hidden=%d must be 64, a multiple of 128 up to %d or of 512 up to %d", fn, hidden,
                 128 * kNormMaxChunks, 512 * kNormMaxChunks);
   if (int st = check_row_stride(fn, "x_row_stride", x_row_stride, hidden)) return st;
   if (int st = check_row_stride(fn, "out_row_stride", out_row_stride, hidden)) return st;
@@ -245,6 +247,8 @@ static int rms_norm_impl(const char* fn, bool f16, const void* x, void* residual
     if (p.chunks <= 4) KIN_NORM_LAUNCH(64, 4);
     else if (p.chunks <= 8) KIN_NORM_LAUNCH(64, 8);
     else KIN_NORM_LAUNCH(64, 16);
+  } else if (lpr == 8) {
+    KIN_NORM_LAUNCH(8, 1);
   } else {
     if (p.chunks <= 1) KIN_NORM_LAUNCH(16, 1);
     else if (p.chunks <= 4) KIN_NORM_LAUNCH(16, 4);
@@ -260,14 +264,16 @@ static int qkv_norm_split_impl(const char* fn, bool f16, const void* qkv, int64_
   if (!qkv || !q_weight || !k_weight || !q || !k || !v) return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   if (batch < 0 || num_q_heads < 1 || num_kv_heads < 1)
     return fail(KIN_ERR_BAD_SHAPE, "%s: batch=%d num_q_heads=%d num_kv_heads=%d", fn, batch, num_q_heads, num_kv_heads);
-  if (head_dim != kHeadDim) return fail(KIN_ERR_UNSUPPORTED, "%s: head_dim=%d, only %d is built", fn, head_dim, kHeadDim);
+  if (!supported_head_dim(head_dim))
+    return fail(KIN_ERR_UNSUPPORTED, "%s: head_dim=%d, only %d and %d are built", fn, head_dim, kHeadDimSmall, kHeadDim);
   const int64_t heads = (int64_t)num_q_heads + 2 * (int64_t)num_kv_heads;
-  if (heads * kHeadDim > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: too many heads", fn);
-  if (int st = check_row_stride(fn, "qkv_row_stride", qkv_row_stride, (int)(heads * kHeadDim))) return st;
+  if (heads * head_dim > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: too many heads", fn);
+  if (int st = check_row_stride(fn, "qkv_row_stride", qkv_row_stride, (int)(heads * head_dim))) return st;
   if (!aligned16(qkv) || !aligned16(q_weight) || !aligned16(k_weight) || !aligned16(q) || !aligned16(k) || !aligned16(v))
     return fail(KIN_ERR_MISALIGNED, "%s: pointers must be 16-byte aligned", fn);
   if (!(eps >= 0.f)) return fail(KIN_ERR_BAD_SHAPE, "%s: eps must be non-negative", fn);
-  const int64_t grid = ((int64_t)batch * heads + 15) / 16;
+  const int rows_per_block = 256 / (head_dim / 8);
+  const int64_t grid = ((int64_t)batch * heads + rows_per_block - 1) / rows_per_block;
   if (grid > 0x7fffffffLL) return fail(KIN_ERR_UNSUPPORTED, "%s: batch*heads is too large", fn);
   if (batch == 0) return KIN_OK;
   QkvParams p;
@@ -282,8 +288,14 @@ static int qkv_norm_split_impl(const char* fn, bool f16, const void* qkv, int64_
   p.hq = num_q_heads;
   p.hkv = num_kv_heads;
   p.eps = eps;
-  if (f16) qkv_norm_split_kernel<true><<<(unsigned)grid, 256, 0, static_cast<hipStream_t>(stream)>>>(p);
-  else qkv_norm_split_kernel<false><<<(unsigned)grid, 256, 0, static_cast<hipStream_t>(stream)>>>(p);
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  if (head_dim == kHeadDimSmall) {
+    if (f16) qkv_norm_split_kernel<true, 8><<<(unsigned)grid, 256, 0, hs>>>(p);
+    else qkv_norm_split_kernel<false, 8><<<(unsigned)grid, 256, 0, hs>>>(p);
+  } else {
+    if (f16) qkv_norm_split_kernel<true, 16><<<(unsigned)grid, 256, 0, hs>>>(p);
+    else qkv_norm_split_kernel<false, 16><<<(unsigned)grid, 256, 0, hs>>>(p);
+  }
   return check_hip(hipGetLastError(), "qkv_norm_split_kernel launch");
 }
 

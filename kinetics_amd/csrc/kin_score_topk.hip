@@ -30,7 +30,7 @@ struct ScoreTopkParams {
 
 // Dynamic LDS layout: uint32 keys[kbar_pages_padded] | uint64 sortbuf[sort_cap] | int32 table[table_cap] |
 // int32 sel[sink + topk + local]
-template <int UNROLL, bool F16>
+template <int UNROLL, bool F16, int HD = kHeadDim>
 __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ int sh_last;
@@ -56,13 +56,13 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
   int32_t* table_lds = reinterpret_cast<int32_t*>(smem + select_table_offset(p.kbar_pages, p.sort_cap));
 
   SelectArgs a;
-  a.q_bh = p.q + ((int64_t)b * p.num_q_heads + (int64_t)h * p.group) * kHeadDim;
+  a.q_bh = p.q + ((int64_t)b * p.num_q_heads + (int64_t)h * p.group) * HD;
   a.G = p.group;
   a.n_pages = n_pages;
   const int kb = kbar_block_of(p.slot_ids, p.num_slots, b);  // (a sequence without mean keys has no candidates)
   split_pages(n_pages, p.last_page_len[b], p.sink_pages, p.local_tokens, kb >= 0 ? p.kbar_pages : 0, p.page_size, a.n_sink, a.n_cand,
               a.n_local);
-  a.kb = reinterpret_cast<const char*>(p.kbar) + kbar_row_index(max(kb, 0), h, a.n_sink, p.num_kv_heads, p.kbar_pages) * kRowBytes;
+  a.kb = reinterpret_cast<const char*>(p.kbar) + kbar_row_index(max(kb, 0), h, a.n_sink, p.num_kv_heads, p.kbar_pages) * (HD * 2);
   a.topk = p.topk;
   a.table = p.page_indices + ps;
   a.sel_logical = p.sel_logical ? p.sel_logical + (int64_t)item * p.topk : nullptr;
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
     const int n_score = (min(a.topk, a.n_cand) > 0 || a.scores_out) ? a.n_cand : 0;
     const int per = ((n_score + p.chunks - 1) / p.chunks + 63) & ~63;
     const int r0 = min(chunk * per, n_score), r1 = min(r0 + per, n_score);
-    score_rows<UNROLL, kThreads, true, F16>(a, r0, r1, gkeys);
+    score_rows<UNROLL, kThreads, true, F16, false, HD>(a, r0, r1, gkeys);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (tid == 0)
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(kThreads) void score_topk_kernel(ScoreTopkParams p)
   } else {
     a.table_lds = prefetch_table<kThreads>(a.table, n_pages, table_lds, p.table_cap);
     __syncthreads();  // histograms zeroed
-    n_list = score_select<UNROLL, kThreads, F16>(a, sel_lds);
+    n_list = score_select<UNROLL, kThreads, F16, HD>(a, sel_lds);
   }
 
   for (int i = tid; i < p.sel_stride; i += kThreads) sel[i] = (i < n_list) ? sel_lds[i] : -1;
@@ -120,7 +120,7 @@ static int score_topk_impl(const char* fn, bool f16, const uint16_t* q, const ui
                            kin_stream_t stream) {
   if (!q || !kbar || !page_indices || !page_indptr || !last_page_len || !sel_pages || !sel_count)
     return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
-  int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size);
+  int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size, true);
   if (st) return st;
   if (topk < 0) return fail(KIN_ERR_BAD_SHAPE, "%s: topk=%d is negative", fn, topk);
   st = check_fixed_pages(fn, sink_pages, local_tokens);
@@ -187,12 +187,13 @@ static int score_topk_impl(const char* fn, bool f16, const uint16_t* q, const ui
   // small grid 16 (more registers, which it can afford).
   const bool small_grid = items < 512;
   const void* fn_ptr;
-  if (f16)
-    fn_ptr = small_grid ? reinterpret_cast<const void*>(&score_topk_kernel<16, true>)
-                        : reinterpret_cast<const void*>(&score_topk_kernel<4, true>);
-  else
-    fn_ptr = small_grid ? reinterpret_cast<const void*>(&score_topk_kernel<16, false>)
-                        : reinterpret_cast<const void*>(&score_topk_kernel<4, false>);
+#define KIN_SCORE_KERNEL(HD_)                                                                      \
+  (f16 ? (small_grid ? reinterpret_cast<const void*>(&score_topk_kernel<16, true, HD_>)            \
+                     : reinterpret_cast<const void*>(&score_topk_kernel<4, true, HD_>))            \
+       : (small_grid ? reinterpret_cast<const void*>(&score_topk_kernel<16, false, HD_>)           \
+                     : reinterpret_cast<const void*>(&score_topk_kernel<4, false, HD_>)))
+  fn_ptr = head_dim == kHeadDimSmall ? KIN_SCORE_KERNEL(kHeadDimSmall) : KIN_SCORE_KERNEL(kHeadDim);
+#undef KIN_SCORE_KERNEL
   if (lds > 48 * 1024) {
     // Above the default dynamic-LDS allowance the runtime wants an explicit opt-in.
     st = check_hip(hipFuncSetAttribute(fn_ptr, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),

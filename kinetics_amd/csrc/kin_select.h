@@ -202,21 +202,23 @@ __device__ __forceinline__ void radix_pick_bin_uniform(const uint32_t* hist, uin
 // needs more per workgroup).
 // COUNT0: also count every key's first radix digit in a.ss->hist[0] (LDS atomics spread
 // over the streaming, instead of a pass over the keys afterwards).
-template <int UNROLL, int NT, bool DEVICE_VISIBLE = false, bool F16 = false, bool COUNT0 = false>
+// HD: elements of a head row (128 or 64): HD / 8 lanes share a mean key, 16 bytes each.
+template <int UNROLL, int NT, bool DEVICE_VISIBLE = false, bool F16 = false, bool COUNT0 = false, int HD = kHeadDim>
 __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, uint32_t* keys_out) {
   constexpr int kUnroll = UNROLL;
-  constexpr int kRows = NT / 16;  // mean keys one pass of the workgroup covers
+  constexpr int kLanes = HD / 8;      // lanes per mean key
+  constexpr int kRows = NT / kLanes;  // mean keys one pass of the workgroup covers
+  constexpr int kRowB = HD * 2;       // bytes of a mean key
   const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  // Lane owns columns d = 8*(lane%16) .. +7 of the mean query.
-  const int c16 = lane & 15;
+  // Lane owns columns d = 8*c16 .. +7 of the mean query.
+  const int c16 = tid & (kLanes - 1);
   // The group's query rows are requested four at a time (a loop of single loads would pay one memory
   // round trip per head), the first four before the first mean keys and averaged after those are
   // under way, so that the stream starts one round trip after the call.
   const uint16_t* qp = a.q_bh + 8 * c16;
   auto load_q_rows = [&](uint4 (&qv)[4], int g0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) qv[i] = *reinterpret_cast<const uint4*>(qp + (int64_t)min(g0 + i, a.G - 1) * kHeadDim);
+    for (int i = 0; i < 4; ++i) qv[i] = *reinterpret_cast<const uint4*>(qp + (int64_t)min(g0 + i, a.G - 1) * HD);
   };
   auto add_q_rows = [&](float (&qm)[8], const uint4 (&qv)[4], int g0) {
 #pragma unroll
@@ -232,7 +234,7 @@ __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, 
   };
   uint4 qv0[4];
   load_q_rows(qv0, 0);
-  // The candidates of (b, h) are contiguous rows of 256 B.  They are read
+  // The candidates of (b, h) are contiguous rows of 256 B (128 B for HD = 64).  They are read
   // through a buffer descriptor that ends after the last wanted row, so loads past
   // the end return zeros without touching memory and the loop needs no branches:
   // each lane keeps kUnroll 16-byte loads in flight, re-issuing slot j for the
@@ -240,13 +242,13 @@ __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, 
   // per-lane (VGPR) offset with the descriptor's size -- the scalar offset operand
   // is added after the range check -- so the whole offset travels in the VGPR and
   // the scalar operand stays 0.
-  constexpr int row_stride_b = kRowBytes;  // the list's mean keys are contiguous rows (head-major kbar)
+  constexpr int row_stride_b = kRowB;  // the list's mean keys are contiguous rows (head-major kbar)
   const int n = r1 > r0 ? r1 - r0 : 0;
   const char* kb = a.kb + (int64_t)r0 * row_stride_b;
   float* sc_out = a.scores_out;
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<char*>(kb), 0, n > 0 ? (n - 1) * row_stride_b + kRowBytes : 0, 0x00020000);
-  const int sub = tid >> 4;  // which of the kRows rows of a slot this lane helps with
+      const_cast<char*>(kb), 0, n > 0 ? (n - 1) * row_stride_b + kRowB : 0, 0x00020000);
+  const int sub = tid / kLanes;  // which of the kRows rows of a slot this lane helps with
   const int lane_off = sub * row_stride_b + c16 * 16;
   u32x4 w[kUnroll];
 #pragma unroll
@@ -278,7 +280,7 @@ __device__ __forceinline__ void score_rows(const SelectArgs& a, int r0, int r1, 
       acc = fmaf(qm[2], elem_lo<F16>(x.y), acc); acc = fmaf(qm[3], elem_hi<F16>(x.y), acc);
       acc = fmaf(qm[4], elem_lo<F16>(x.z), acc); acc = fmaf(qm[5], elem_hi<F16>(x.z), acc);
       acc = fmaf(qm[6], elem_lo<F16>(x.w), acc); acc = fmaf(qm[7], elem_hi<F16>(x.w), acc);
-      acc = row16_sum(acc);
+      acc = row_sum<kLanes>(acc);
       const int row = base + j * kRows + sub;
       if (c16 == 0 && row < n) {
         const uint32_t key = order_key(acc);
@@ -532,12 +534,12 @@ __device__ __forceinline__ int select_from_keys(const SelectArgs& a, int32_t* se
 // score_rows() over every candidate into a.keys, then select_from_keys().
 // a.ss->hist is zero and visible (clear_select_scratch + barrier); a.digit0_counted is
 // ignored: the first digit is always counted on the fly here.
-template <int UNROLL = 4, int NT = kThreads, bool F16 = false>
+template <int UNROLL = 4, int NT = kThreads, bool F16 = false, int HD = kHeadDim>
 __device__ __forceinline__ int score_select(SelectArgs& a, int32_t* sel_lds) {
   // Nothing to choose (topk == 0) and nobody asked for the scores: stream nothing.
   const int n_score = (min(a.topk, a.n_cand) > 0 || a.scores_out) ? a.n_cand : 0;
   KIN_STAMP(17);  // prologue over: the stream of mean keys starts
-  score_rows<UNROLL, NT, false, F16, true>(a, 0, n_score, a.keys);
+  score_rows<UNROLL, NT, false, F16, true, HD>(a, 0, n_score, a.keys);
   a.digit0_counted = true;
   // the page-table copy (LDS-direct loads) has landed in every wave before anyone reads it
   KIN_STAMP(18);  // this wave has consumed its last mean key

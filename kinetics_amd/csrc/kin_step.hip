@@ -23,8 +23,10 @@
 
 namespace kin {
 
-template <int NG, int NW, bool F16>
+// HD: elements of a head row, 128 or 64.
+template <int NG, int NW, bool F16, int HD = kHeadDim>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kernel(StepParams p) {
+  constexpr int kRowB = HD * 2;  // bytes of a head row
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ float sm_m[NW][4 * NG];
   __shared__ float sm_l[NW][4 * NG];
@@ -70,7 +72,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     if (p.sel_pages)
       for (int i = tid; i < p.sel_stride; i += NT) p.sel_pages[(int64_t)item * p.sel_stride + i] = -1;
     if (p.sel_count && tid == 0) p.sel_count[item] = 0;
-    for (int i = tid; i < G * kHeadDim; i += NT) p.out[hq0 * kHeadDim + i] = 0;
+    for (int i = tid; i < G * HD; i += NT) p.out[hq0 * HD + i] = 0;
     if (p.lse && tid < G) p.lse[hq0 + tid] = kNegInf;
     return;
   }
@@ -84,8 +86,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     if (p.k != nullptr && tid < 64) {
       uint32_t* kbar_row = kb < 0 ? nullptr
                                   : reinterpret_cast<uint32_t*>(p.kbar) +
-                                        kbar_row_index(kb, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * (kHeadDim / 2);
-      append_token_row<F16>(p.k + (int64_t)item * (kHeadDim / 2), p.v + (int64_t)item * (kHeadDim / 2),
+                                        kbar_row_index(kb, h, n_pages - 1, p.num_kv_heads, p.kbar_pages) * (HD / 2);
+      append_token_row<F16, HD>(p.k + (int64_t)item * (HD / 2), p.v + (int64_t)item * (HD / 2),
                        reinterpret_cast<uint32_t*>(p.kv), kbar_row, p.page_indices[pe - 1], last_len, n_pages, p.kbar_pages, h,
                        p.num_kv_heads, p.num_pages, tid, p.page_size);
       // The attention phase of this workgroup reads the row back: make the stores
@@ -99,11 +101,11 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   // ---- score + select: page list into LDS -------------------------------------
   int32_t* sel_lds = reinterpret_cast<int32_t*>(smem + p.region0_bytes);
   SelectArgs s;
-  s.q_bh = p.q + hq0 * kHeadDim;
+  s.q_bh = p.q + hq0 * HD;
   s.G = G;
   s.n_pages = n_pages;
   split_pages(n_pages, last_len, p.sink_pages, p.local_tokens, kb >= 0 ? p.kbar_pages : 0, p.page_size, s.n_sink, s.n_cand, s.n_local);
-  s.kb = reinterpret_cast<const char*>(p.kbar) + kbar_row_index(max(kb, 0), h, s.n_sink, p.num_kv_heads, p.kbar_pages) * kRowBytes;
+  s.kb = reinterpret_cast<const char*>(p.kbar) + kbar_row_index(max(kb, 0), h, s.n_sink, p.num_kv_heads, p.kbar_pages) * kRowB;
   s.topk = p.topk;
   s.table = p.page_indices + ps;
   s.sel_logical = nullptr;
@@ -125,7 +127,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     const int per = ((n_score + team - 1) / team + 63) & ~63;
     const int r0 = min(member * per, n_score), r1 = min(r0 + per, n_score);
     constexpr int kDeep = NW <= 4 ? 16 : 8;
-    score_rows<kDeep, NT, true, F16>(s, r0, r1, gkeys);
+    score_rows<kDeep, NT, true, F16, false, HD>(s, r0, r1, gkeys);
     // The slices meet through memory without cache maintenance: keys and the
     // arrival counter are written and read at device scope (they bypass the
     // XCD-private L2), and every wave waits for its own stores to be acknowledged
@@ -155,7 +157,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     if (__builtin_amdgcn_readfirstlane(sh_last)) {
       load_shared_keys<NT>(gkeys, n_score, s.keys);
     } else {
-      score_rows<kDeep, NT, false, F16>(s, 0, n_score, s.keys);
+      score_rows<kDeep, NT, false, F16, false, HD>(s, 0, n_score, s.keys);
     }
     __builtin_amdgcn_s_waitcnt(0);  // the table copy has landed too
     __syncthreads();
@@ -170,9 +172,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     // (1024 lists of 2048 pages: 5 % faster than with 4).
     if (p.deep_score) {
       constexpr int kDeep = NW <= 4 ? 16 : 8;
-      n = score_select<kDeep, NT, F16>(s, sel_lds);
+      n = score_select<kDeep, NT, F16, HD>(s, sel_lds);
     } else {
-      n = score_select<4, NT, F16>(s, sel_lds);
+      n = score_select<4, NT, F16, HD>(s, sel_lds);
     }
   }
   KIN_STAMP(30);  // list ready
@@ -197,10 +199,10 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   // ---- attend over the listed pages (select scratch is dead: reuse as staging) ---
   AttendArgs a;
   a.q_bh = s.q_bh;
-  a.kvb = reinterpret_cast<const char*>(p.kv) + (int64_t)h * kRowBytes;
-  a.row_bytes = p.num_kv_heads * kRowBytes;
+  a.kvb = reinterpret_cast<const char*>(p.kv) + (int64_t)h * kRowB;
+  a.row_bytes = p.num_kv_heads * kRowB;
   a.page_bytes = 2 * p.page_size * a.row_bytes;
-  a.span = a.page_bytes - h * kRowBytes;
+  a.span = a.page_bytes - h * kRowB;
   a.page_size = p.page_size;
   a.num_pages = p.num_pages;
   a.G = G;
@@ -211,16 +213,16 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   a.last_len = last_len;
   a.first_skip = p.first_page_offset;
   a.rotate = p.rotate ? attend_rotation(item, part) : 0u;
-  attend_list<NG, NW, F16>(
+  attend_list<NG, NW, F16, HD>(
       a, [&](int i) -> int { return __builtin_amdgcn_readfirstlane(sel_lds[i]); }, smem, sm_m, sm_l,
       [&](int g, int d, float o, float lse2) {
         if (parts > 1) {
           // partial result, read by a workgroup that may sit on another XCD: device-scope stores
           const int64_t row = ((int64_t)(item - p.head_lists) * parts + part) * G + g;
-          __hip_atomic_store(p.ws_po + row * kHeadDim + d, __float_as_uint(o), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(p.ws_po + row * HD + d, __float_as_uint(o), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           if (d == 0) __hip_atomic_store(p.ws_plse + row, __float_as_uint(lse2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         } else {
-          p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(o);
+          p.out[(hq0 + g) * HD + d] = (uint16_t)f32_to_elem<F16>(o);
           if (p.lse && d == 0) p.lse[hq0 + g] = lse2 * kLn2;
         }
       });
@@ -235,7 +237,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   __syncthreads();
   KIN_STAMP(44);  // partial stored, counted in
   if (!__builtin_amdgcn_readfirstlane(sh_last)) return;
-  merge_list_parts<NT, F16>(smem, p.ws_po, p.ws_plse, item - p.head_lists, parts, G, p.out + hq0 * kHeadDim, p.lse ? p.lse + hq0 : nullptr);
+  merge_list_parts<NT, F16, HD>(smem, p.ws_po, p.ws_plse, item - p.head_lists, parts, G, p.out + hq0 * HD, p.lse ? p.lse + hq0 : nullptr);
   KIN_STAMP(45);  // merged
 }
 
@@ -366,7 +368,7 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
     return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
   if ((k == nullptr) != (v == nullptr))
     return fail(KIN_ERR_NULL_POINTER, "%s: k and v must both be given or both be null", fn);
-  int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size);
+  int st = check_common_dims(fn, batch, num_q_heads, num_kv_heads, head_dim, page_size, true);
   if (st) return st;
   if (num_pages < 1) return fail(KIN_ERR_BAD_SHAPE, "%s: num_pages=%lld must be >= 1", fn, (long long)num_pages);
   if (topk < 0) return fail(KIN_ERR_BAD_SHAPE, "%s: topk=%d is negative", fn, topk);
@@ -455,7 +457,7 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
     p.ws_keys = reinterpret_cast<uint32_t*>(w);
     w += round256((size_t)team_lists * score_key_stride(kbar_pages) * sizeof(uint32_t));
     p.ws_po = reinterpret_cast<uint32_t*>(w);
-    p.ws_plse = p.ws_po + (size_t)team_lists * plan.parts * p.group * kHeadDim;
+    p.ws_plse = p.ws_po + (size_t)team_lists * plan.parts * p.group * head_dim;
   }
   const size_t sel_scratch = select_lds_bytes(kbar_pages, p.sort_cap, p.table_cap);
   const size_t attend_bytes = (size_t)attend_lds_bytes(nw);
@@ -465,9 +467,12 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
   const size_t lds = region0 + (size_t)list_cap * 4;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const void* kernel;
-#define KIN_STEP_KERNEL(NG_, NW_)                                                        \
-  (f16 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<NG_, NW_, true>)           \
-       : reinterpret_cast<const void*>(&blocktopk_step_kernel<NG_, NW_, false>))
+#define KIN_STEP_KERNEL(NG_, NW_)                                                                              \
+  (head_dim == kHeadDimSmall                                                                                   \
+       ? (f16 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<NG_, NW_, true, kHeadDimSmall>)           \
+              : reinterpret_cast<const void*>(&blocktopk_step_kernel<NG_, NW_, false, kHeadDimSmall>))         \
+       : (f16 ? reinterpret_cast<const void*>(&blocktopk_step_kernel<NG_, NW_, true, kHeadDim>)                \
+              : reinterpret_cast<const void*>(&blocktopk_step_kernel<NG_, NW_, false, kHeadDim>)))
   if (p.group <= 4)
     kernel = nw == 8 ? KIN_STEP_KERNEL(1, 8) : KIN_STEP_KERNEL(1, 4);
   else

@@ -642,7 +642,7 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
     if constexpr (NG == 4)
       page_pv_wide<F16>(vr, pr, O);
     else
-      page_pv<F16>(vr, pr, O);
+      page_pv<F16>(vr, pr, O, 0);
   };
 
   // This wave takes the 16-entry groups w, w+NW, ...  Entries past the end (and
@@ -706,14 +706,14 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
         __builtin_amdgcn_sched_barrier(0);
         issue_v(idB, vB);
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(kWaitVm4);
+        __builtin_amdgcn_s_waitcnt(wait_vm_imm(4));
         __builtin_amdgcn_sched_barrier(0);
         read_k(0, ka);
         __builtin_amdgcn_sched_barrier(0);
         issue_k(idB, 1);
         __builtin_amdgcn_sched_barrier(0);
         scores(ka, pr, idA.valid);
-        if (idA.valid != kPageSize) clear_unused_v_rows(vA, 0, idA.valid, kg);
+        if (idA.valid != kPageSize) clear_unused_v_rows<4>(vA, 0, idA.valid, 4 * kg);
         pv(vA, pr);
       }
       {
@@ -721,19 +721,19 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
         __builtin_amdgcn_sched_barrier(0);
         issue_v(idA, vA);
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(kWaitVm4);
+        __builtin_amdgcn_s_waitcnt(wait_vm_imm(4));
         __builtin_amdgcn_sched_barrier(0);
         read_k(1, ka);
         __builtin_amdgcn_sched_barrier(0);
         issue_k(idA, 0);
         __builtin_amdgcn_sched_barrier(0);
         scores(ka, pr, idB.valid);
-        if (idB.valid != kPageSize) clear_unused_v_rows(vB, 0, idB.valid, kg);
+        if (idB.valid != kPageSize) clear_unused_v_rows<4>(vB, 0, idB.valid, 4 * kg);
         pv(vB, pr);
       }
     }
   }
-  attend_finish<NG, NW>(m_run, l_run, O, G, lds, sm_m, sm_l, emit);
+  attend_finish<NG, NW, kHeadDim>(m_run, l_run, O, G, lds, sm_m, sm_l, emit);
 }
 
 }  // namespace kin

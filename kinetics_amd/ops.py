@@ -20,6 +20,7 @@ import torch
 from . import _lib
 
 HEAD_DIM = 128
+HEAD_DIMS = (64, 128)  # head dimensions the page path and the layer's row kernels are built for
 PAGE_SIZE = 16
 
 
@@ -806,27 +807,30 @@ def rms_norm(x, weight, eps: float, residual=None, out=None) -> torch.Tensor:
 
 
 def qkv_norm_split(qkv, q_weight, k_weight, eps: float, num_q_heads: int, num_kv_heads: int):
-    """From the fused projection ``qkv[batch, (Hq + 2*Hkv) * 128]`` to contiguous
-    ``q[batch, Hq, 128]``, ``k[batch, Hkv, 128]``, ``v[batch, Hkv, 128]`` with the
+    """From the fused projection ``qkv[batch, (Hq + 2*Hkv) * D]`` to contiguous
+    ``q[batch, Hq, D]``, ``k[batch, Hkv, D]``, ``v[batch, Hkv, D]`` with the
     q and k heads RMS-normalised: the split, qk_norm calls and reshapes of
-    benchmark/blocktopk_decoder.py:196-207 in one pass."""
+    benchmark/blocktopk_decoder.py:196-207 in one pass.  The head dimension D is the
+    length of the norm weights (128 or 64)."""
     batch, width, stride = _row_view(qkv, "qkv")
     dev, dt = qkv.device, qkv.dtype
-    if width != (num_q_heads + 2 * num_kv_heads) * HEAD_DIM:
-        raise ValueError(f"qkv rows have {width} elements, expected (Hq + 2*Hkv) * {HEAD_DIM} = "
-                         f"{(num_q_heads + 2 * num_kv_heads) * HEAD_DIM}")
     _require(q_weight, "q_weight", dt, 1, dev)
     _require(k_weight, "k_weight", dt, 1, dev)
-    if q_weight.numel() != HEAD_DIM or k_weight.numel() != HEAD_DIM:
-        raise ValueError(f"q_weight and k_weight must have {HEAD_DIM} entries")
-    q = torch.empty(batch, num_q_heads, HEAD_DIM, dtype=dt, device=dev)
-    k = torch.empty(batch, num_kv_heads, HEAD_DIM, dtype=dt, device=dev)
-    v = torch.empty(batch, num_kv_heads, HEAD_DIM, dtype=dt, device=dev)
+    head_dim = q_weight.numel()
+    if head_dim not in HEAD_DIMS or k_weight.numel() != head_dim:
+        raise ValueError(f"q_weight and k_weight must have the same number of entries, one of {HEAD_DIMS}; "
+                         f"got {q_weight.numel()} and {k_weight.numel()}")
+    if width != (num_q_heads + 2 * num_kv_heads) * head_dim:
+        raise ValueError(f"qkv rows have {width} elements, expected (Hq + 2*Hkv) * {head_dim} = "
+                         f"{(num_q_heads + 2 * num_kv_heads) * head_dim}")
+    q = torch.empty(batch, num_q_heads, head_dim, dtype=dt, device=dev)
+    k = torch.empty(batch, num_kv_heads, head_dim, dtype=dt, device=dev)
+    v = torch.empty(batch, num_kv_heads, head_dim, dtype=dt, device=dev)
     lib = _lib.load()
     with _on(dev):
         _lib.check(_entry(lib, "kin_qkv_norm_split", dt)(_ptr(qkv), stride, _ptr(q_weight), _ptr(k_weight), float(eps),
                                                          _ptr(q), _ptr(k), _ptr(v), batch, int(num_q_heads),
-                                                         int(num_kv_heads), HEAD_DIM, _stream(dev)))
+                                                         int(num_kv_heads), head_dim, _stream(dev)))
     return q, k, v
 
 
@@ -1044,8 +1048,9 @@ def _qkv_norm_split_impl(qkv, q_weight, k_weight, eps, num_q_heads, num_kv_heads
 @torch.library.register_fake("kinetics::qkv_norm_split")
 def _qkv_norm_split_fake(qkv, q_weight, k_weight, eps, num_q_heads, num_kv_heads):
     batch = qkv.numel() // qkv.shape[-1]
-    return (qkv.new_empty(batch, num_q_heads, HEAD_DIM), qkv.new_empty(batch, num_kv_heads, HEAD_DIM),
-            qkv.new_empty(batch, num_kv_heads, HEAD_DIM))
+    head_dim = q_weight.numel()
+    return (qkv.new_empty(batch, num_q_heads, head_dim), qkv.new_empty(batch, num_kv_heads, head_dim),
+            qkv.new_empty(batch, num_kv_heads, head_dim))
 
 
 @torch.library.impl("kinetics::gated_act", "cuda")

@@ -14,6 +14,29 @@ from oracle import blocktopk_oracle as O
 
 HEAD_DIM = 128
 PAGE_SIZE = 16
+_head_dim = HEAD_DIM  # what make_problem() builds; see head_dim()
+
+
+class head_dim:
+    """``with head_dim(64): ...`` -- problems made inside have head rows of that many elements."""
+
+    def __init__(self, d: int):
+        assert d in (64, 128)
+        self.d = d
+
+    def __enter__(self):
+        global _head_dim
+        self.prev, _head_dim = _head_dim, self.d
+        return self.d
+
+    def __exit__(self, *exc):
+        global _head_dim
+        _head_dim = self.prev
+        return False
+
+
+def current_head_dim() -> int:
+    return _head_dim
 
 
 @dataclass
@@ -70,7 +93,7 @@ def make_problem(seed: int, lengths, num_kv_heads: int = 1, group: int = 4, topk
     rng = np.random.default_rng(seed)
     lengths = np.asarray(lengths, dtype=np.int64)
     B = len(lengths)
-    ps, D = page_size, HEAD_DIM
+    ps, D = page_size, _head_dim
     n_pages = (lengths + ps - 1) // ps
     total = int(n_pages.sum()) + extra_pages
     indptr = np.zeros(B + 1, dtype=np.int32)

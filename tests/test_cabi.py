@@ -51,7 +51,9 @@ def test_append_argument_errors(lib):
     assert append(lib, Hkv=0) == _lib.KIN_ERR_BAD_SHAPE
     assert append(lib, P=0) == _lib.KIN_ERR_BAD_SHAPE
     assert append(lib, kp=0) == _lib.KIN_ERR_BAD_SHAPE
-    assert append(lib, D=64) == _lib.KIN_ERR_UNSUPPORTED
+    assert append(lib, D=96) == _lib.KIN_ERR_UNSUPPORTED
+    assert b"64 and 128" in lib.kin_last_error()
+    assert append(lib, D=64, B=0) == _lib.KIN_OK              # the page path is built for head rows of 64 and 128
     assert append(lib, ps=24) == _lib.KIN_ERR_UNSUPPORTED
     assert append(lib, ps=128) == _lib.KIN_ERR_UNSUPPORTED
     assert append(lib, ps=32, B=0) == _lib.KIN_OK and append(lib, ps=64, B=0) == _lib.KIN_OK
@@ -158,9 +160,9 @@ def test_step_argument_errors(lib):
 
 def test_token_topk_argument_errors(lib):
     def tok(q=A, topk=8, sink=4, local=1, offset=0, sel=None, cnt=None, ws=A, wsb=1 << 20, B=2, Hq=4, Hkv=1, P=8, mp=4,
-            stride=0):
+            stride=0, D=128):
         return lib.kin_token_topk_decode(q, A, A, A, A, topk, sink, local, offset, sel, cnt, A, None, ws, wsb, B, Hq, Hkv,
-                                         128, 16, P, mp, stride, 0.0, None)
+                                         D, 16, P, mp, stride, 0.0, None)
 
     assert tok(q=None) == _lib.KIN_ERR_NULL_POINTER
     assert tok(topk=-1) == _lib.KIN_ERR_BAD_SHAPE
@@ -168,6 +170,8 @@ def test_token_topk_argument_errors(lib):
     assert tok(mp=0) == _lib.KIN_ERR_BAD_SHAPE
     assert tok(topk=5000) == _lib.KIN_ERR_UNSUPPORTED
     assert tok(local=2000) == _lib.KIN_ERR_UNSUPPORTED
+    assert tok(D=64) == _lib.KIN_ERR_UNSUPPORTED                      # the token-granular policies: head_dim 128 only
+    assert b"head_dim=64" in lib.kin_last_error()
     assert tok(sel=A, cnt=A, stride=12) == _lib.KIN_ERR_BAD_SHAPE      # 8 + 4 + 1 entries needed
     assert tok(sel=A, stride=13) == _lib.KIN_ERR_NULL_POINTER
     assert lib.kin_token_topk_workspace_bytes(2, 1, 4) == 256 + 2 * 4 * 16 * 4  # arrival counters + keys
@@ -215,7 +219,9 @@ def test_layer_row_kernel_argument_errors(lib):
     assert split(kw=None) == _lib.KIN_ERR_NULL_POINTER
     assert split(v=None) == _lib.KIN_ERR_NULL_POINTER
     assert split(Hq=0) == _lib.KIN_ERR_BAD_SHAPE
-    assert split(D=64) == _lib.KIN_ERR_UNSUPPORTED
+    assert split(D=96) == _lib.KIN_ERR_UNSUPPORTED
+    assert split(D=64, stride=384, B=0) == _lib.KIN_OK
+    assert split(D=64, stride=380) == _lib.KIN_ERR_BAD_SHAPE   # narrower than (Hq + 2*Hkv) * 64
     assert split(stride=760) == _lib.KIN_ERR_BAD_SHAPE     # narrower than (Hq + 2*Hkv) * 128
     assert split(q=A + 2) == _lib.KIN_ERR_MISALIGNED
     assert split(B=0) == _lib.KIN_OK

@@ -23,6 +23,24 @@ def bf(x):
     return x.to(_DT[0])
 
 
+class use_head_dim:
+    """``with use_head_dim(64): ...`` -- the helpers of this module build configurations and tensors
+    with head rows of that many elements (LiteSys reads head_dim from the model config,
+    LiteSys/litesys/attention/batch_cache.py:27)."""
+
+    def __init__(self, d):
+        self.d = d
+
+    def __enter__(self):
+        global D
+        self.prev, D = D, self.d
+
+    def __exit__(self, *exc):
+        global D
+        D = self.prev
+        return False
+
+
 def cfg_small():
     return SimpleNamespace(num_attention_heads=4, num_key_value_heads=2, head_dim=D, hidden_size=512, num_hidden_layers=2)
 
@@ -49,23 +67,43 @@ def test_rejects_what_it_does_not_implement():
         PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_block_topk=2)          # LiteSys: local required
     with pytest.raises(NotImplementedError):
         PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_block_topk=2, attn_local=4, attn_block_size=24)
+    # head rows of 64 elements: dense attention and the block policy, not the token-granular policies; other sizes: nothing
+    cfg64 = SimpleNamespace(num_attention_heads=4, num_key_value_heads=2, head_dim=64, hidden_size=256, num_hidden_layers=1)
+    PagedBatchKVManager(cfg64, 2, 64, DEV, torch.bfloat16, attn_block_topk=2, attn_local=4)
+    for token_policy in (dict(attn_topk=8, attn_local=4), dict(attn_local=4), dict(attn_block_topk=2, attn_local=4, attn_stride=8)):
+        with pytest.raises(NotImplementedError, match="head_dim 128"):
+            PagedBatchKVManager(cfg64, 2, 64, DEV, torch.bfloat16, **token_policy)
+    cfg96 = SimpleNamespace(num_attention_heads=4, num_key_value_heads=2, head_dim=96, hidden_size=384, num_hidden_layers=1)
+    with pytest.raises(NotImplementedError, match="head_dim 96"):
+        PagedBatchKVManager(cfg96, 2, 64, DEV, torch.bfloat16)
 
 
-@pytest.mark.parametrize("sparse,fused", [(dict(), None), (dict(attn_block_topk=3, attn_local=16), True),
-                                          (dict(attn_block_topk=3, attn_local=16), False),
-                                          (dict(attn_block_topk=2, attn_local=21), True),
-                                          (dict(attn_block_topk=2, attn_local=20, attn_block_size=32), True),
-                                          (dict(attn_block_topk=2, attn_local=33, attn_block_size=32), False),
-                                          (dict(attn_block_topk=1, attn_local=7, attn_block_size=64), True),
-                                          (dict(attn_local=24), False),
-                                          (dict(attn_topk=40, attn_local=10), None),
-                                          (dict(attn_block_topk=2, attn_local=9, attn_stride=8), None),
-                                          (dict(attn_block_topk=3, attn_local=5, attn_stride=4, attn_block_size=8), None)])
+_POLICIES = [(dict(), None), (dict(attn_block_topk=3, attn_local=16), True),
+             (dict(attn_block_topk=3, attn_local=16), False),
+             (dict(attn_block_topk=2, attn_local=21), True),
+             (dict(attn_block_topk=2, attn_local=20, attn_block_size=32), True),
+             (dict(attn_block_topk=2, attn_local=33, attn_block_size=32), False),
+             (dict(attn_block_topk=1, attn_local=7, attn_block_size=64), True),
+             (dict(attn_local=24), False),
+             (dict(attn_topk=40, attn_local=10), None),
+             (dict(attn_block_topk=2, attn_local=9, attn_stride=8), None),
+             (dict(attn_block_topk=3, attn_local=5, attn_stride=4, attn_block_size=8), None)]
+
+
+def _token_kernels(sparse):
+    return "attn_topk" in sparse or "attn_stride" in sparse or (bool(sparse) and "attn_block_topk" not in sparse)
+
+
+# head rows of 64 elements: dense attention and the block policy (the token-granular policies are built for 128 only)
+_CASES = [(s, f, 128) for s, f in _POLICIES] + [(s, f, 64) for s, f in _POLICIES if not _token_kernels(s)]
+
+
+@pytest.mark.parametrize("sparse,fused,head_dim", _CASES)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_prefill_then_decode_like_litesys(sparse, fused, dtype):
+def test_prefill_then_decode_like_litesys(sparse, fused, dtype, head_dim):
     _DT[0] = dtype
     try:
-        with O.element_format("f16" if dtype is torch.float16 else "bf16"):   # how the oracle reads the cache bits
+        with O.element_format("f16" if dtype is torch.float16 else "bf16"), use_head_dim(head_dim):   # how the oracle reads the cache bits
             _prefill_then_decode_like_litesys(sparse, fused)
     finally:
         _DT[0] = torch.bfloat16
@@ -464,8 +502,14 @@ def _fed_manager(max_batch, sparse, seed, prefill_lens):
     return m, hist
 
 
+@pytest.mark.parametrize("head_dim", [128, 64])
 @pytest.mark.parametrize("sparse", [dict(), dict(attn_block_topk=3, attn_local=16)])
-def test_manager_few_active_slots_in_any_order(sparse):
+def test_manager_few_active_slots_in_any_order(sparse, head_dim):
+    with use_head_dim(head_dim):
+        _manager_few_active_slots_in_any_order(sparse)
+
+
+def _manager_few_active_slots_in_any_order(sparse):
     """Five active slots of a 40-slot manager, in an order that is not the slots': q, k, v and the
     output follow the batch, the caches the slots.  The page table built by the first layer of a
     step is reused by the second (same batch_idx object) -- same bits as rebuilding it -- and the

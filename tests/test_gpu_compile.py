@@ -142,6 +142,7 @@ def test_functions_on_the_ops_compile_with_aot_eager(ops, path):
         return o + 0.0
 
     body = three if path == "three" else fused
+    torch._dynamo.reset()
     compiled = torch.compile(body, backend="aot_eager", fullgraph=True)
 
     def on_state(fn):
@@ -195,6 +196,7 @@ def test_decoder_layer_compiles(ops, backend, fused):
         import torch._inductor.config as inductor_config
 
         inductor_config.compile_threads = 1  # no pool of compile workers beside the GPU process
+    torch._dynamo.reset()  # many layers are compiled in one test process: each starts with an empty code cache
     ref_layer = make()
     eager = run(ref_layer, ref_layer.forward)
     layer = make()

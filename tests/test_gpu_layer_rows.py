@@ -53,7 +53,7 @@ def check_close(got_bits, want_bits, max_ulps=1):
     assert np.allclose(g, w, rtol=2e-2, atol=2e-2)
 
 
-@pytest.mark.parametrize("rows,hidden", [(1, 128), (37, 128), (16, 256), (6, 896), (33, 2048), (5, 1024), (9, 5120),
+@pytest.mark.parametrize("rows,hidden", [(1, 128), (37, 128), (1, 64), (777, 64), (16, 256), (6, 896), (33, 2048), (5, 1024), (9, 5120),
                                          (3, 8192), (1027, 4096), (4, 512)])
 @pytest.mark.parametrize("residual", [False, True])
 def test_rms_norm(ops, rows, hidden, residual):
@@ -117,14 +117,15 @@ def test_norm_ops_by_the_reference_names(ops):
         ops.rms_norm(ht[..., :1000].contiguous(), wt[:1000].contiguous(), 1e-6)
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("B,Hq,Hkv,pad", [(7, 4, 1, 0), (130, 8, 8, 0), (1, 5, 1, 0), (33, 8, 2, 64), (4096, 4, 1, 0)])
-def test_qkv_norm_split(ops, B, Hq, Hkv, pad):
+def test_qkv_norm_split(ops, B, Hq, Hkv, pad, D):
     rng = np.random.default_rng(B + Hq)
     width = (Hq + 2 * Hkv) * D
     buf = rand_bits(rng, (B, width + pad), 2.0)
     qw = O.f32_to_elem(1 + 0.3 * rng.standard_normal(D).astype(np.float32))
     kw = O.f32_to_elem(1 + 0.3 * rng.standard_normal(D).astype(np.float32))
-    wq, wk, wv = O.qkv_norm_split(buf[:, :width], qw, kw, 1e-6, Hq, Hkv)
+    wq, wk, wv = O.qkv_norm_split(buf[:, :width], qw, kw, 1e-6, Hq, Hkv, head_dim=D)
     bt = P.to_torch(buf, DEV)
     q, k, v = ops.qkv_norm_split(bt[:, :width], P.to_torch(qw, DEV), P.to_torch(kw, DEV), 1e-6, Hq, Hkv)
     torch.cuda.synchronize()

@@ -27,6 +27,15 @@ def ops():
     return _ops
 
 
+@pytest.fixture(params=[128, 64], ids=["D128", "D64"])
+def head_dim(request):
+    """Tests that take this fixture run twice: problems made inside have head rows of 128 and of 64
+    elements (the reference reads head_dim from the model config, benchmark/blocktopk_decoder.py:104;
+    LiteSys/litesys/attention/batch_cache.py:27)."""
+    with P.head_dim(request.param):
+        yield request.param
+
+
 class Gpu:
     """A Problem uploaded to the GPU."""
 
@@ -64,10 +73,11 @@ def workspace(ops, pb, max_pages, splits):
 
 
 @pytest.mark.parametrize("hkv,group", [(1, 4), (2, 2), (8, 2)])
-def test_append_bit_exact(ops, hkv, group):
+def test_append_bit_exact(ops, hkv, group, head_dim):
     lengths = [3 * PS + r + 1 for r in range(PS)] + [1, PS, 0, 5 * PS]
     pb = P.make_problem(200 + hkv, lengths, num_kv_heads=hkv, group=group)
     g = Gpu(pb)
+    assert g.kv.shape[-1] == head_dim and g.k.shape[-1] == head_dim and g.kbar.shape[-1] == head_dim
     check_table(ops, g)
     ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
     torch.cuda.synchronize()
@@ -82,7 +92,7 @@ def test_append_bit_exact(ops, hkv, group):
     assert np.array_equal(P.from_torch(g2.kv), want_kv)
 
 
-def test_build_kbar_bit_exact(ops):
+def test_build_kbar_bit_exact(ops, head_dim):
     lengths = [PS * 37, PS * 5 + 3, 1, 0, PS, PS * 64 + 16]
     pb = P.make_problem(210, lengths, num_kv_heads=2, group=2, build_kbar=False)
     g = Gpu(pb)
@@ -134,7 +144,7 @@ def check_selection(pb, sel, cnt, logical, scores, exact=False):
 
 
 @pytest.mark.parametrize("hkv,group,topk", [(1, 4, 8), (2, 2, 5), (8, 2, 16), (1, 8, 64), (1, 1, 3), (2, 16, 7), (1, 11, 20)])
-def test_score_topk_small(ops, hkv, group, topk):
+def test_score_topk_small(ops, hkv, group, topk, head_dim):
     lengths = [PS * 40 + 3, PS * 9, 1, 0, PS * 3 + 1, PS * 130 + 16, PS * topk + 1, PS * (topk + 1) + 1]
     pb = P.make_problem(300 + hkv + topk, lengths, num_kv_heads=hkv, group=group, topk=topk)
     g = Gpu(pb)
@@ -165,7 +175,7 @@ def test_score_topk_ties_take_lowest_index(ops):
     check_selection(pb2, sel, cnt, logical, scores, exact=True)
 
 
-def test_score_topk_many_candidates(ops):
+def test_score_topk_many_candidates(ops, head_dim):
     # 12000 candidate pages (192k tokens): dynamic LDS above the default allowance
     pb = P.make_problem(330, [PS * 12000 + 5, PS * 700 + 1, PS * 650 + 1], topk=700, kbar_slack=3)  # k > 512: bitonic path
     g = Gpu(pb)
@@ -183,7 +193,7 @@ def oracle_sparse(pb, kv=None):
 
 @pytest.mark.parametrize("hkv,group", [(1, 4), (1, 8), (8, 2), (2, 1), (1, 3), (2, 6), (1, 5), (2, 12), (1, 16), (4, 9)])
 @pytest.mark.parametrize("splits", [1, 3, 0])
-def test_sparse_decode_matches_oracle(ops, hkv, group, splits):
+def test_sparse_decode_matches_oracle(ops, hkv, group, splits, head_dim):
     lengths = [PS * 30 + r for r in (1, 2, 7, 15, 16)] + [1, 0, PS, PS * 3 + 4, PS * 100 + 9]
     pb = P.make_problem(400 + 10 * hkv + group, lengths, num_kv_heads=hkv, group=group, topk=12)
     sel, cnt, want, want_lse = oracle_sparse(pb)
@@ -202,7 +212,7 @@ def test_sparse_decode_matches_oracle(ops, hkv, group, splits):
 
 @pytest.mark.parametrize("hkv,group", [(1, 4), (8, 2), (1, 8), (2, 16), (1, 13)])
 @pytest.mark.parametrize("splits", [1, 4, 0])
-def test_dense_decode_matches_oracle(ops, hkv, group, splits):
+def test_dense_decode_matches_oracle(ops, hkv, group, splits, head_dim):
     lengths = [PS * 70 + 5, PS * 33, 1, 0, 17, PS * 257 + 16]
     pb = P.make_problem(500 + hkv + group, lengths, num_kv_heads=hkv, group=group, table="fragmented")
     want, want_lse = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len)
@@ -307,20 +317,20 @@ def check_step(ops, pb, splits=0):
     return same
 
 
-def test_decode_step_tiny_config(ops):
+def test_decode_step_tiny_config(ops, head_dim):
     """Batch 8, context 4096 (+1 appended), 1 KV head, 4 Q heads, budget 64 pages,
     random page table."""
     pb = P.make_problem(0, [4096 + 1] * 8, num_kv_heads=1, group=4, topk=64, table="random")
     assert check_step(ops, pb)
 
 
-def test_decode_step_qwen3_32b_share_small(ops):
+def test_decode_step_qwen3_32b_share_small(ops, head_dim):
     """8 Q heads per KV head, budget 256 pages, reference page layout p*B+b."""
     pb = P.make_problem(3, [8192 + 1] * 6, num_kv_heads=1, group=8, topk=256, table="strided")
     check_step(ops, pb)
 
 
-def test_decode_step_continuous_batching_mix(ops):
+def test_decode_step_continuous_batching_mix(ops, head_dim):
     """8 KV heads x 2, ragged lengths, per-KV-head selection, fragmented table,
     budget min(64, pages)."""
     rng = np.random.default_rng(4)
@@ -329,7 +339,7 @@ def test_decode_step_continuous_batching_mix(ops):
     check_step(ops, pb)
 
 
-def test_decode_step_fills_a_page(ops):
+def test_decode_step_fills_a_page(ops, head_dim):
     # the appended token completes a page: its mean key must appear, and the page
     # (being the last one) is attended but is not a candidate
     pb = P.make_problem(5, [PS * 21, PS * 2, PS], num_kv_heads=2, group=4, topk=4)
@@ -485,7 +495,7 @@ def test_selection_vs_the_references_bf16_scoring(ops, case):
 
 @pytest.mark.parametrize("page_size", [32, 64])
 @pytest.mark.parametrize("hkv,group", [(1, 4), (2, 8), (8, 2), (1, 3)])
-def test_pages_of_32_and_64_tokens(ops, page_size, hkv, group):
+def test_pages_of_32_and_64_tokens(ops, page_size, hkv, group, head_dim):
     """Every entry point of the page path on caches with 32- and 64-token pages
     (the reference's --page_size, benchmark/blocktopk.py:13): append and mean keys
     bit-exact, selection against the oracle, sparse / dense / fused attention within
@@ -555,7 +565,7 @@ def test_pages_of_32_and_64_tokens(ops, page_size, hkv, group):
     rng = np.random.default_rng(ps + hkv)
     new = np.array([min(int(L), int(rng.integers(0, 3 * ps))) for L in pb.lengths])
     append_indptr = np.concatenate([[0], np.cumsum(new)]).astype(np.int32)
-    k_new, v_new = P.randn_bf16(rng, (int(new.sum()), hkv, D)), P.randn_bf16(rng, (int(new.sum()), hkv, D))
+    k_new, v_new = P.randn_bf16(rng, (int(new.sum()), hkv, head_dim)), P.randn_bf16(rng, (int(new.sum()), hkv, head_dim))
     want_kv, want_kbar = pb.kv_cache.copy(), want.copy()
     O.append_paged_kv_ragged(k_new, v_new, append_indptr, want_kv, want_kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
     ops.append_paged_kv_ragged(P.to_torch(k_new, DEV), P.to_torch(v_new, DEV), P.int_tensor(append_indptr, DEV), g.kv, g.kbar,
@@ -574,7 +584,7 @@ def test_token_policies_reject_larger_pages(ops):
 
 @pytest.mark.parametrize("page_size", [16, 64])
 @pytest.mark.parametrize("hkv,group", [(1, 4), (2, 8), (8, 2)])
-def test_float16_caches(ops, hkv, group, page_size):
+def test_float16_caches(ops, hkv, group, page_size, head_dim):
     """The reference's --dtype float16 (benchmark/blocktopk.py:18): q, k, v, the
     cache, the mean keys and the output in IEEE half through the *_f16 entry
     points -- append and mean keys bit-exact, selection against the oracle, sparse
@@ -634,7 +644,7 @@ def test_float16_caches(ops, hkv, group, page_size):
         rng = np.random.default_rng(ps + hkv)
         new = np.array([min(int(L), int(rng.integers(0, 3 * ps))) for L in pb.lengths])
         append_indptr = np.concatenate([[0], np.cumsum(new)]).astype(np.int32)
-        k_new, v_new = P.randn_bf16(rng, (int(new.sum()), hkv, D)), P.randn_bf16(rng, (int(new.sum()), hkv, D))
+        k_new, v_new = P.randn_bf16(rng, (int(new.sum()), hkv, head_dim)), P.randn_bf16(rng, (int(new.sum()), hkv, head_dim))
         want_kv, want_kbar = pb.kv_cache.copy(), pb.kbar.copy()
         O.append_paged_kv_ragged(k_new, v_new, append_indptr, want_kv, want_kbar, pb.page_indices, pb.page_indptr, pb.last_page_len)
         ops.append_paged_kv_ragged(P.to_torch(k_new, DEV), P.to_torch(v_new, DEV), P.int_tensor(append_indptr, DEV), g.kv, g.kbar,
@@ -871,7 +881,7 @@ def test_full_size_continuous_batching_mix(ops):
     torch.cuda.empty_cache()
 
 
-def test_unused_cache_slots_may_hold_nan(ops):
+def test_unused_cache_slots_may_hold_nan(ops, head_dim):
     """Slots past a sequence's last token, padding slots in front of it and pages
     nobody owns are never initialised by a real cache: NaN and Inf bit patterns
     there must not reach the output (0 * NaN) on any path."""
@@ -915,7 +925,7 @@ def test_unused_cache_slots_may_hold_nan(ops):
 
 
 @pytest.mark.parametrize("hkv,group", [(1, 4), (2, 8), (8, 1)])
-def test_fused_step_split_scoring_for_few_long_sequences(ops, hkv, group):
+def test_fused_step_split_scoring_for_few_long_sequences(ops, hkv, group, head_dim):
     """Few lists with thousands of candidate pages: a team of workgroups per list shares
     the scoring (and the attention) and meets through the workspace; same cache bytes and
     page lists as without it, outputs equal to fp32 summation order and identical call
@@ -974,7 +984,7 @@ def test_fused_step_split_scoring_for_few_long_sequences(ops, hkv, group):
 
 
 @pytest.mark.parametrize("ps,fmt", [(16, "bf16"), (32, "bf16"), (64, "bf16"), (16, "f16")])
-def test_fused_step_split_attention_for_few_lists(ops, ps, fmt):
+def test_fused_step_split_attention_for_few_lists(ops, ps, fmt, head_dim):
     """Lists for at most half the CUs with long page lists: several workgroups per
     list, each scoring and selecting for itself and attending a share of the pages,
     the last to finish merging the partial results through the workspace.  Same
@@ -1094,7 +1104,7 @@ def test_seeded_sweep_of_split_scoring(ops):
 
 
 @pytest.mark.parametrize("hkv", [1, 2, 8])
-def test_ragged_append_bit_exact(ops, hkv):
+def test_ragged_append_bit_exact(ops, hkv, head_dim):
     """Multi-token appends of mixed lengths (none, one, page-crossing, page-filling,
     a long prefill) land bit for bit where the oracle puts them, and the mean keys
     of the completed pages are refreshed; also through the update_kv custom op."""
@@ -1104,7 +1114,7 @@ def test_ragged_append_bit_exact(ops, hkv):
     after = [a + n for a, n in zip(before, new)]
     pb = P.make_problem(600 + hkv, after, num_kv_heads=hkv, group=1, table="fragmented")
     nnz = sum(new)
-    k, v = P.randn_bf16(rng, (nnz, hkv, D)), P.randn_bf16(rng, (nnz, hkv, D))
+    k, v = P.randn_bf16(rng, (nnz, hkv, head_dim)), P.randn_bf16(rng, (nnz, hkv, head_dim))
     append_indptr = np.concatenate([[0], np.cumsum(new)]).astype(np.int32)
     for use_op in (False, True):
         g = Gpu(pb)
@@ -1582,7 +1592,7 @@ def test_custom_ops_trace_with_fullgraph(ops):
 
 
 @pytest.mark.parametrize("case", ["mixed", "hkv8", "g8", "fills", "ties", "long", "many", "many_g8", "mid"])
-def test_fused_step_equals_three_calls(ops, case):
+def test_fused_step_equals_three_calls(ops, case, head_dim):
     """kin_blocktopk_decode_step must give what append + score/select + attend
     give and match the oracle: cache bytes, mean keys and page lists bit for bit;
     the output bit for bit when the fused kernel runs 4 waves per list like the
@@ -1667,7 +1677,7 @@ def test_fused_step_full_size(ops):
 
 
 @pytest.mark.parametrize("fmt", ["bf16", "f16"])
-def test_slot_ids_put_the_mean_keys_with_the_cache_slot(ops, fmt):
+def test_slot_ids_put_the_mean_keys_with_the_cache_slot(ops, fmt, head_dim):
     """The reference's kernels index q, k, v and the output by position in the active
     batch and the cache by slot (LiteSys/litesys/attention/cache_utils.py:40-51,67-70).
     Here the page table is per active sequence already; slot_ids does the same for kbar:
@@ -1770,18 +1780,19 @@ def test_slot_ids_put_the_mean_keys_with_the_cache_slot(ops, fmt):
 # --------------------------------------------------------------------------- whole decoder layer
 
 
+@pytest.mark.parametrize("hd", [128, 64])
 @pytest.mark.parametrize("fmt", ["bf16", "f16"])
 @pytest.mark.parametrize("dense", [False, True])
-def test_decoder_layer_matches_fp32_reference(ops, dense, fmt):
+def test_decoder_layer_matches_fp32_reference(ops, dense, fmt, hd):
     """The drop-in layers: norms/GEMMs in PyTorch around the HIP attention.  The
     attention inside is checked against the oracle on the layer's own q, k, v;
     the rest against an fp32 restatement of the same layer.  In bfloat16 and in
     float16 (the reference moves the whole layer to --dtype, benchmark/blocktopk.py:18,37-40)."""
     with O.element_format(fmt):
-        _decoder_layer_case(ops, dense, torch.float16 if fmt == "f16" else torch.bfloat16)
+        _decoder_layer_case(ops, dense, torch.float16 if fmt == "f16" else torch.bfloat16, hd)
 
 
-def _decoder_layer_case(ops, dense, dt):
+def _decoder_layer_case(ops, dense, dt, D=D):
     from types import SimpleNamespace
 
     from kinetics_amd.decoder_layer import BlockTopkDecoderLayer, DenseDecoderLayer, init_weights, qwen3_config, rms_norm
@@ -1817,7 +1828,7 @@ def _decoder_layer_case(ops, dense, dt):
 
     x = rn(h32, W["input_layernorm_weight"]).to(dt).float()
     qkv = x @ W["wqkv.weight"].T + W["wqkv.bias"]
-    q32, k32, v32 = qkv.split((512, 128, 128), dim=-1)
+    q32, k32, v32 = qkv.split((4 * D, D, D), dim=-1)
     q32 = rn(q32.reshape(B, 4, D), W["qnorm_weight"])
     k32 = rn(k32.reshape(B, 1, D), W["knorm_weight"])
     assert torch.allclose(q.float().cpu(), q32, rtol=3e-2, atol=3e-2)
@@ -1834,7 +1845,7 @@ def _decoder_layer_case(ops, dense, dt):
         assert np.array_equal(layer.attn.topk_page_indices.cpu().numpy(), res["sel_pages"])
     assert np.array_equal(P.from_torch(st.kv_cache), kv_before)
     # the rest of the layer in fp32
-    o32 = torch.from_numpy(attn).float().to(dt).float().reshape(B, 1, 512)
+    o32 = torch.from_numpy(attn).float().to(dt).float().reshape(B, 1, 4 * D)
     h1 = h32 + o32 @ W["wo.weight"].T
     y = rn(h1, W["post_attention_layernorm_weight"])
     want = h1 + (torch.nn.functional.silu(y @ W["gate_proj.weight"].T) * (y @ W["up_proj.weight"].T)) @ W["down_proj.weight"].T
@@ -1843,6 +1854,7 @@ def _decoder_layer_case(ops, dense, dt):
     assert rms_norm(hidden, 1e-6, layer.input_layernorm_weight).dtype == dt
     # the whole forward traces without a graph break (the reference compiles it with fullgraph=True,
     # benchmark/blocktopk.py:41-43); backend "eager": no code generation, the same kernels run
+    torch._dynamo.reset()  # many layers are compiled in one test process: each starts with an empty code cache
     compiled = torch.compile(layer.forward, backend="eager", fullgraph=True)
     h_c = torch.randn(B, 1, 512, device=DEV).to(dt)
     want_c = layer(h_c.clone()).clone()
@@ -1864,7 +1876,7 @@ def _decoder_layer_case(ops, dense, dt):
 @pytest.mark.parametrize("sink,local,offset", [(1, 17, 0), (2, 33, 0), (0, 49, 0), (3, 1, 0), (1, 16, 12), (1, 5, 12),
                                                (2, 40, 7), (1, 1, 15)])
 @pytest.mark.parametrize("fused", [False, True])
-def test_sink_and_local_pages(ops, sink, local, offset, fused):
+def test_sink_and_local_pages(ops, sink, local, offset, fused, head_dim):
     """Pinned leading pages and trailing tokens (LiteSys' sink and local window),
     with and without padding slots at the start of the first page."""
     topk = 6
@@ -1942,7 +1954,7 @@ def test_topk_zero_is_sink_plus_local_window(ops):
 
 
 @pytest.mark.parametrize("page_size,fmt,trials", [(16, "bf16", 40), (32, "bf16", 15), (64, "bf16", 10), (16, "f16", 15), (64, "f16", 10)])
-def test_seeded_sweep_of_shapes(ops, page_size, fmt, trials):
+def test_seeded_sweep_of_shapes(ops, page_size, fmt, trials, head_dim):
     """Seeded random configurations -- head counts, group sizes 1..8, ragged
     lengths with empty and one-token sequences, budgets above and below the
     candidate count, pinned pages, table layouts, split counts, both step

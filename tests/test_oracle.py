@@ -266,8 +266,9 @@ def test_selection_matches_rule():
 def _depaged(pb, b, h):
     pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
     L = int(pb.lengths[b])
-    K = O.elem_to_f32(pb.kv_cache[pages, 0, :, h]).reshape(-1, D)[:L]
-    V = O.elem_to_f32(pb.kv_cache[pages, 1, :, h]).reshape(-1, D)[:L]
+    d = pb.kv_cache.shape[4]
+    K = O.elem_to_f32(pb.kv_cache[pages, 0, :, h]).reshape(-1, d)[:L]
+    V = O.elem_to_f32(pb.kv_cache[pages, 1, :, h]).reshape(-1, d)[:L]
     return K.astype(np.float64), V.astype(np.float64)
 
 
@@ -288,16 +289,19 @@ def test_float16_element_format_is_ieee_half():
     assert O._ELEMENT_FORMAT == "bf16"                            # the block restored the default
 
 
+@pytest.mark.parametrize("head_dim", [128, 64])
 @pytest.mark.parametrize("fmt", ["bf16", "f16"])
 @pytest.mark.parametrize("page_size", [16, 32, 64])
-def test_dense_attention_equals_torch_sdpa(page_size, fmt):
-    with O.element_format(fmt):
-        _dense_attention_equals_torch_sdpa(page_size)
+def test_dense_attention_equals_torch_sdpa(page_size, fmt, head_dim):
+    """Head rows of 64 elements too (LiteSys reads head_dim from the model config,
+    LiteSys/litesys/attention/batch_cache.py:27): the scale follows the row length."""
+    with O.element_format(fmt), P.head_dim(head_dim):
+        _dense_attention_equals_torch_sdpa(page_size, head_dim)
 
 
-def _dense_attention_equals_torch_sdpa(page_size):
+def _dense_attention_equals_torch_sdpa(page_size, D=D):
     pb = P.make_problem(41, [PS * 6 + 5, PS * 2, 9], num_kv_heads=2, group=4, page_size=page_size)
-    assert pb.kv_cache.shape[2] == page_size
+    assert pb.kv_cache.shape[2] == page_size and pb.kv_cache.shape[4] == D and pb.q.shape[2] == D
     out, lse = O.dense_paged_decode(pb.q, pb.kv_cache, pb.page_indices, pb.page_indptr, pb.last_page_len)
     qf = O.elem_to_f32(pb.q).astype(np.float64)
     for b in range(pb.B):
@@ -406,8 +410,14 @@ def test_decode_step_equals_masked_dense_formulation_float16():
         test_decode_step_equals_masked_dense_formulation(32)
 
 
+def test_decode_step_equals_masked_dense_formulation_head_dim_64():
+    with P.head_dim(64):
+        test_decode_step_equals_masked_dense_formulation(16, D=64)
+        test_decode_step_equals_masked_dense_formulation(64, D=64)
+
+
 @pytest.mark.parametrize("page_size", [16, 32, 64])
-def test_decode_step_equals_masked_dense_formulation(page_size):
+def test_decode_step_equals_masked_dense_formulation(page_size, D=D):
     """LiteSys expresses block sparsity as a -inf mask on full-context logits
     (sparsity_utils.py:39-45) followed by softmax and P.V; the gather form must
     give the same numbers, at every page size (the reference's --page_size,
