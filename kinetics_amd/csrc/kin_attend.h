@@ -35,7 +35,8 @@
 // 2 V rows -- the 16 lanes of a row group split into two halves of 8 chunks, the lower half taking tokens
 // 4*kg + 0..1 and the upper half 4*kg + 2..3 -- and the two halves' partial outputs are added at the end;
 // the wide form keeps 4 V rows per lane with both halves fetching the same chunks (its P V instruction
-// shares one probability between all 16 columns), so its columns 8..15 repeat columns 0..7.
+// shares one probability between all 16 columns) and lets the halves take the even and the odd elements
+// of a chunk (see page_pv_wide).
 #pragma once
 
 #include <cmath>
@@ -186,8 +187,24 @@ __device__ __forceinline__ void page_scores_wide(const uint4 (&ka)[KC], const ui
 // O += P V, wide form: A[i = head l%16][k = l/16] = p of token 4*kg + r, B[k = l/16][j = l%16] =
 // V[token 4*kg + r][8*(l%16) + u]; the instruction's K = 4 adds the four row groups, so lane
 // (kg, c16) accumulates O[head 4*kg + reg][d = 8*c16 + u] over all 16 tokens of the tile.
-template <bool F16 = false>
-__device__ __forceinline__ void page_pv_wide(const u32x4 (&vr)[4], const float (&pr)[4], floatx4 (&O)[8]) {
+//
+// With 64-element rows (HD = 64) a row has 8 chunks and the 16 columns carry two elements of a chunk instead:
+// lane (kg, c16) with c8 = c16 % 8 and hi = c16 / 8 supplies V[token 4*kg + r][8*c8 + 2*uu + hi] (both halves hold
+// chunk c8; `shift` = 16 * hi picks the element of dword uu), so a tile takes 16 instructions instead of 32 and the
+// lane accumulates O[uu][reg] = out[head 4*kg + reg][8*c8 + 2*uu + hi], uu = 0..3.
+template <bool F16 = false, int HD = kHeadDim>
+__device__ __forceinline__ void page_pv_wide(const u32x4 (&vr)[4], const float (&pr)[4], floatx4 (&O)[8], int shift) {
+  if constexpr (HD == 64) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const u32x4 vv = vr[r];
+      const float vf[4] = {elem_lo<F16>(vv.x >> shift), elem_lo<F16>(vv.y >> shift), elem_lo<F16>(vv.z >> shift),
+                           elem_lo<F16>(vv.w >> shift)};
+#pragma unroll
+      for (int uu = 0; uu < 4; ++uu) O[uu] = __builtin_amdgcn_mfma_f32_16x16x4f32(pr[r], vf[uu], O[uu], 0, 0, 0);
+    }
+    return;
+  }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const u32x4 vv = vr[r];
@@ -256,7 +273,7 @@ __device__ __forceinline__ void attend_finish(float m_run, float l_run, floatx4 
 
   if constexpr (NG == 4) {
     // Wide form: O is already summed over the row groups; the lanes of a head share m
-    // and hold partial sums l.  (HD = 64: lanes c16 >= 8 hold copies of lanes c16 - 8.)
+    // and hold partial sums l.
     float ll = l_run;
     ll += __shfl_xor(ll, 16);
     ll += __shfl_xor(ll, 32);
@@ -264,10 +281,16 @@ __device__ __forceinline__ void attend_finish(float m_run, float l_run, floatx4 
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int h = 4 * kg + i;
-      if (h < G && c16 < CPR) {
-        float* dst = ow + ((w * 16 + h) * HD + 8 * cc);
-        *reinterpret_cast<float4*>(dst) = make_float4(O[0][i], O[1][i], O[2][i], O[3][i]);
-        *reinterpret_cast<float4*>(dst + 4) = make_float4(O[4][i], O[5][i], O[6][i], O[7][i]);
+      if (h < G) {
+        if constexpr (HD == 64) {  // this lane's columns are 8*cc + 2*uu + (c16 >> 3), see page_pv_wide
+          float* dst = ow + ((w * 16 + h) * HD + 8 * cc + (c16 >> 3));
+#pragma unroll
+          for (int uu = 0; uu < 4; ++uu) dst[2 * uu] = O[uu][i];
+        } else {
+          float* dst = ow + ((w * 16 + h) * HD + 8 * cc);
+          *reinterpret_cast<float4*>(dst) = make_float4(O[0][i], O[1][i], O[2][i], O[3][i]);
+          *reinterpret_cast<float4*>(dst + 4) = make_float4(O[4][i], O[5][i], O[6][i], O[7][i]);
+        }
       }
     }
     if (l < 16) {
@@ -401,7 +424,7 @@ __device__ __forceinline__ void attend_list(const AttendArgs& a, IdAt id_at, uns
   };
   auto pv = [&](const u32x4 (&vr)[NV], const float (&pr)[4]) {
     if constexpr (NG == 4)
-      page_pv_wide<F16>(vr, pr, O);
+      page_pv_wide<F16, HD>(vr, pr, O, 16 * (c16 >> 3));
     else
       page_pv<F16, NV>(vr, pr, O, half);
   };

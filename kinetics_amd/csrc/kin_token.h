@@ -640,7 +640,7 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
   };
   auto pv = [&](const u32x4 (&vr)[4], const float (&pr)[4]) {
     if constexpr (NG == 4)
-      page_pv_wide<F16>(vr, pr, O);
+      page_pv_wide<F16>(vr, pr, O, 0);
     else
       page_pv<F16>(vr, pr, O, 0);
   };
