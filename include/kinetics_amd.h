@@ -392,6 +392,18 @@ size_t kin_step_workspace_bytes(int batch, int num_kv_heads, int kbar_pages);
  */
 #define KIN_STATIC_SCRATCH_BYTES (4u * 1024u * 1024u + 64u * 1024u)
 
+/*
+ * Patience of a team member (kin_blocktopk_decode_step, kin_token_topk_decode,
+ * kin_strided_topk_decode with few lists): the workgroups that share one list
+ * exchange their scores through the workspace, and a member polls at most `polls`
+ * times (about a third of a microsecond each; default 300) for the others before
+ * it scores the whole list for itself -- the same values, so results do not depend
+ * on it.  0: never wait (every member scores everything: what tests use to walk
+ * that path); negative: back to the default.  Process-wide, read at each launch.
+ * Returns the previous value.  No counterpart in the reference.
+ */
+int kin_set_team_spin_limit(int polls);
+
 size_t kin_static_scratch_bytes(void);
 
 int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_bf16_t* k, const kin_bf16_t* v,

@@ -62,6 +62,7 @@ SIGNATURES = {
     ),
     "kin_step_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "kin_static_scratch_bytes": (c_size_t, []),
+    "kin_set_team_spin_limit": (c_int, [c_int]),
     "kin_blocktopk_decode_step_static": (
         c_int,
         [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int64,

@@ -1,10 +1,15 @@
 // Status handling, shared argument checks and the page-table checker.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 
 #include "kin_common.h"
+#include "kin_step.h"
 
 namespace kin {
+
+static std::atomic<int> g_team_spin_limit{kTeamSpinLimit};
+int team_spin_limit() { return g_team_spin_limit.load(std::memory_order_relaxed); }
 
 static thread_local char g_last_error[512] = {0};
 
@@ -91,6 +96,10 @@ __global__ void check_page_table_kernel(const int32_t* __restrict__ page_indices
 extern "C" {
 
 int kin_version(void) { return 30100; }
+
+int kin_set_team_spin_limit(int polls) {
+  return kin::g_team_spin_limit.exchange(polls < 0 ? kin::kTeamSpinLimit : polls, std::memory_order_relaxed);
+}
 
 int kin_sel_list_capacity(int topk, int sink_pages, int local_tokens) {
   if (topk < 0 || sink_pages < 0 || local_tokens < 1) return 0;

@@ -48,6 +48,9 @@ struct StepParams {
 
 // Polls (about a third of a microsecond each) after which a team member stops waiting for the
 // others' keys and scores the whole list itself: some 100 us, several times what a slice takes.
+// The default of kin_set_team_spin_limit().
 constexpr int kTeamSpinLimit = 300;
+// The limit the next launches use (kin_api.hip).
+int team_spin_limit();
 
 }  // namespace kin

@@ -443,7 +443,7 @@ static int launch_step(const char* fn, bool f16, const uint16_t* q, const uint16
   p.team = plan.team;
   p.parts = plan.parts;
   p.head_blocks = plan.head_lists == items ? (int)xcd_grid_size(batch, num_kv_heads) : plan.head_lists;
-  p.spin_limit = kTeamSpinLimit;
+  p.spin_limit = team_spin_limit();
   p.ws_count = p.ws_count2 = nullptr;
   p.ws_keys = nullptr;
   p.ws_po = nullptr;

@@ -75,9 +75,8 @@ __device__ __forceinline__ void translate_slots(int32_t* list, int first, int co
 
 // LDS scratch of the two functions below.
 struct KeySelectShared {
-  uint32_t hist[256];
+  uint32_t hist[4][256];  // one histogram per radix digit (see radix_select_emit)
   uint32_t wave_gt[16], wave_eq[16];
-  uint32_t bin, remaining;
 };
 
 // Keys one trip to memory brings into registers: kSelLoads 16-byte loads per lane.
@@ -121,7 +120,7 @@ struct LdsKeys {  // 16-byte aligned LDS array of n (a multiple of 4) keys
 // "not a candidate"; at least k >= 1 keys are non-zero), then calls emit(pos, index)
 // for every key above it and for the lowest-indexed keys equal to it that complete
 // the k, pos = 0, 1, ... in ascending index order.
-// first_digit_counted: sh->hist already holds the histogram of the top byte of
+// first_digit_counted: sh->hist[0] already holds the histogram of the top byte of
 // the non-zero keys (counted while they were produced).  The writes of the keys
 // have completed (s_waitcnt + barrier, or the arrival counter of split scoring).
 // Up to NW * 4096 keys are loaded once and stay in registers through all passes;
@@ -130,51 +129,75 @@ template <int NW, typename Keys, typename Emit>
 __device__ __forceinline__ void radix_select_emit(const Keys& keys, int n_keys, uint32_t k,
                                                   bool first_digit_counted, KeySelectShared* sh, Emit emit) {
   constexpr int kChunk = NW * 256 * kSelLoads;
+  constexpr int NT = NW * 64;
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63;
   const bool single = n_keys <= kChunk;
   u32x4 kk[kSelLoads];
   if (single) load_key_chunk<NW>(keys, 0, kk);
+  KIN_STAMP(54);  // keys requested
+  // Loads of this wave that hold keys at all (the others read zeros past the end and are skipped:
+  // the passes below are bound by vector instructions, 64 keys per lane).
+  auto loads_with_keys = [&](int c0) -> int {
+    const int left = n_keys - (c0 + w * (256 * kSelLoads));
+    return left <= 0 ? 0 : (left >= 256 * kSelLoads ? kSelLoads : (left + 255) >> 8);
+  };
+  // The histograms of the digits still to be counted start at zero (one per digit: no wave
+  // clears what another still reads, so a digit costs one barrier).
+  for (int i = tid + (first_digit_counted ? 256 : 0); i < 4 * 256; i += NT) (&sh->hist[0][0])[i] = 0;
+  __syncthreads();
 
   uint32_t prefix = 0, mask = 0, remaining = k;
-  for (int shift = 24; shift >= 0; shift -= 8) {
-    if (shift != 24 || !first_digit_counted) {
-      if (tid < 256) sh->hist[tid] = 0;
-      __syncthreads();
+  bool whole_bin = false;  // every key that matches the digits fixed so far is wanted: no further digit needed
+  for (int pass = 0; pass < 4 && !whole_bin; ++pass) {
+    const int shift = 24 - 8 * pass;
+    if (pass != 0 || !first_digit_counted) {
+      uint32_t* hist = sh->hist[pass];
       for (int c0 = 0; c0 < n_keys; c0 += kChunk) {
         if (!single) load_key_chunk<NW>(keys, c0, kk);
+        const int nu = loads_with_keys(c0);
 #pragma unroll
         for (int u = 0; u < kSelLoads; ++u) {
-          const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
+          if (u < nu) {
+            const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
 #pragma unroll
-          for (int j = 0; j < 4; ++j)
-            if (k4[j] && (k4[j] & mask) == prefix) atomicAdd(&sh->hist[(k4[j] >> shift) & 255u], 1u);
+            for (int j = 0; j < 4; ++j)
+              if (k4[j] && (k4[j] & mask) == prefix) atomicAdd(&hist[(k4[j] >> shift) & 255u], 1u);
+          }
           __builtin_amdgcn_sched_barrier(0);  // keeps the lane masks of one load at a time in scalar registers
         }
       }
       __syncthreads();
     }
-    if (w == 0) radix_pick_bin(sh->hist, remaining, l, &sh->bin, &sh->remaining);
-    __syncthreads();
-    prefix |= sh->bin << shift;
+    uint32_t bin;
+    radix_pick_bin_uniform(sh->hist[pass], remaining, l, bin, remaining, whole_bin);  // every wave for itself: no hand-over
+    prefix |= bin << shift;
     mask |= 255u << shift;
-    remaining = sh->remaining;
+    KIN_STAMP(55 + pass);  // digit fixed
   }
-  const uint32_t thr = prefix;  // >= 1
+  uint32_t thr = prefix;  // the k-th largest key (>= 1) ...
+  if (whole_bin && mask != 0xffffffffu) {
+    // ... or, after an early exit, the largest value below every winner: all keys that start with
+    // `prefix` are taken, none is ranked among its equals.
+    thr = prefix ? prefix - 1u : 0u;
+    remaining = 0;
+  }
 
   // Ordered compaction, chunk by chunk: count per wave, prefix over the waves, emit.
-  const unsigned long long below = (1ull << l) - 1ull;
   uint32_t run_all = 0, eq_all = 0;  // winners / threshold-equal keys in the chunks before this one
   for (int c0 = 0; c0 < n_keys; c0 += kChunk) {
     if (!single) load_key_chunk<NW>(keys, c0, kk);
+    const int nu = loads_with_keys(c0);
     uint32_t gt = 0, eq = 0;
 #pragma unroll
     for (int u = 0; u < kSelLoads; ++u) {
-      const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
+      if (u < nu) {
+        const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        gt += (k4[j] > thr) ? 1u : 0u;
-        eq += (k4[j] == thr) ? 1u : 0u;
+        for (int j = 0; j < 4; ++j) {
+          gt += (k4[j] > thr) ? 1u : 0u;
+          eq += (k4[j] == thr) ? 1u : 0u;
+        }
       }
     }
 #pragma unroll
@@ -204,59 +227,48 @@ __device__ __forceinline__ void radix_select_emit(const Keys& keys, int n_keys, 
       eq_all = e_acc;
     }
     const int wave_base = c0 + w * (256 * kSelLoads) + 4 * l;
-    // The comparisons below repeat the counting pass's; an opaque copy of the threshold keeps
-    // the compiler from carrying 128 lane masks from there to here in scalar registers.
-    uint32_t thr_e = thr;
-    asm volatile("" : "+v"(thr_e));
+    const bool rank_equals = remaining > 0 && eq > 0;  // wave-uniform: some key of this wave's equals the threshold
 #pragma unroll
     for (int u = 0; u < kSelLoads; ++u) {
-      const int i0 = wave_base + u * 256;  // this lane's 4 consecutive indices
-      const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
-      // Keys equal to the threshold are rare: rank them (lane-major, then j) only when there are any.
-      bool is_eq[4];
-      uint32_t eq_mine = 0;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        is_eq[j] = k4[j] == thr_e;
-        eq_mine += is_eq[j] ? 1u : 0u;
-      }
-      uint32_t eq_before = eq_run;  // equal keys at lower indices
-      uint32_t eq_total = 0;
-      if (__ballot(eq_mine != 0) != 0ull) {
-#pragma unroll
+      if (u < nu) {  // wave-uniform: the loads behind hold no keys
+        const int i0 = wave_base + u * 256;  // this lane's 4 consecutive indices
+        const uint32_t k4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
+        // Lanes hold ascending indices, so positions come from prefix sums over the wave (DPP
+        // scans).  Keys equal to the threshold are rare: they are ranked only where there are any.
+        uint32_t eq_before = eq_run, eq_total = 0;
+        if (rank_equals) {
+          const uint32_t eq_mine = (k4[0] == thr ? 1u : 0u) + (k4[1] == thr ? 1u : 0u) + (k4[2] == thr ? 1u : 0u) +
+                                   (k4[3] == thr ? 1u : 0u);
+          const uint32_t incl = wave_inclusive_sum(eq_mine);
+          eq_before += incl - eq_mine;
+          eq_total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+        }
+        bool take[4];
+        uint32_t seen = 0, cnt = 0;
+  #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const unsigned long long be = __ballot(is_eq[j]);
-          eq_before += __popcll(be & below);
-          eq_total += __popcll(be);
+          const bool is_eq = k4[j] == thr;
+          take[j] = k4[j] > thr || (is_eq && eq_before + seen < remaining);
+          seen += is_eq ? 1u : 0u;
+          cnt += take[j] ? 1u : 0u;
         }
-      }
-      bool take[4];
-      uint32_t mine_eq_seen = 0;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        take[j] = k4[j] > thr_e || (is_eq[j] && eq_before + mine_eq_seen < remaining);
-        mine_eq_seen += is_eq[j] ? 1u : 0u;
-      }
-      uint32_t pos = run, total = 0;  // winners at lower indices (lower lanes hold lower indices)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const unsigned long long bt = __ballot(take[j]);
-        pos += __popcll(bt & below);
-        total += __popcll(bt);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        if (take[j]) {
-          emit((int)pos, i0 + j);
-          ++pos;
+        const uint32_t incl = wave_inclusive_sum(cnt);
+        uint32_t pos = run + incl - cnt;  // winners at lower indices
+  #pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (take[j]) {
+            emit((int)pos, i0 + j);
+            ++pos;
+          }
         }
+        run += (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+        eq_run += eq_total;
       }
-      run += total;
-      eq_run += eq_total;
-      __builtin_amdgcn_sched_barrier(0);  // one load's ballots at a time: they live in scalar registers
+      __builtin_amdgcn_sched_barrier(0);  // one load's scan at a time: interleaving them only costs registers
     }
     __syncthreads();  // wave_gt / wave_eq are rewritten by the next chunk
   }
+  KIN_STAMP(59);  // winners listed
 }
 
 // Streams the K plane of the pages pg0 <= p < pg1 (pg0 a multiple of 4) of the
@@ -400,7 +412,7 @@ __device__ __forceinline__ void token_score_keys(const TokenArgs& a, int pg0, in
 // Writes the token list (physical token ids) to a.list: sink tokens, the k
 // candidates with the largest keys in ascending position, local tokens; returns
 // its length.  When token_needs_scores(), a.keys is complete and, if
-// first_digit_counted, sh->hist holds the histogram of the keys' top byte.  Every
+// first_digit_counted, sh->hist[0] holds the histogram of the keys' top byte.  Every
 // thread of the workgroup calls this; it ends with a workgroup barrier.
 template <int NG, int NW, bool LDSK = false>
 __device__ __forceinline__ int token_select_list(const TokenArgs& a, KeySelectShared* sh, bool first_digit_counted) {
@@ -486,7 +498,7 @@ template <int NG, int NW, bool LDSK = false>
 __device__ __forceinline__ int strided_select_list(const TokenArgs& a, const StridedArgs& sa, KeySelectShared* sh) {
   constexpr int NT = NW * 64;
   __shared__ uint32_t wave_cnt[NW];
-  uint32_t* hist = sh->hist;
+  uint32_t* hist = sh->hist[0];
 
   const int tid = threadIdx.x;
   const int w = tid >> 6, l = tid & 63;
@@ -533,9 +545,20 @@ __device__ __forceinline__ int strided_select_list(const TokenArgs& a, const Str
         if (i < num_blocks) {
           const int off = (dyn_lo + i * sa.stride) * 4;
           float sum = 0.f;
-          for (int t = 0; t < sa.block; ++t)
-            sum += LDSK ? __uint_as_float(a.lds_keys[(off >> 2) + t])
-                        : __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(scores_rsrc, off + t * 4, 0, kDeviceScope));
+          if constexpr (LDSK) {
+            for (int t = 0; t < sa.block; ++t) sum += __uint_as_float(a.lds_keys[(off >> 2) + t]);
+          } else {
+            // 16 scores requested together (one memory round trip per 16 instead of one per score), added in token order
+            for (int t0 = 0; t0 < sa.block; t0 += 16) {
+              uint32_t x[16];
+#pragma unroll
+              for (int i = 0; i < 16; ++i)
+                x[i] = __builtin_amdgcn_raw_buffer_load_b32(scores_rsrc, off + (t0 + i) * 4, 0, kDeviceScope);
+#pragma unroll
+              for (int i = 0; i < 16; ++i)
+                if (t0 + i < sa.block) sum += __uint_as_float(x[i]);
+            }
+          }
           key = order_key(sum * inv);
           atomicAdd(&hist[key >> 24], 1u);
         }

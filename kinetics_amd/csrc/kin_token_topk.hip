@@ -2,9 +2,12 @@
 // KV head) every token of the context is scored, the sink tokens, the local
 // window and the top-k tokens in between are listed, and attended to
 // (token_score_keys() / token_select_list() / attend_tokens(), kin_token.h).
-// `chunks` workgroups share the scoring of one list, each a run of pages; the
-// last one to finish selects and attends.  Splitting keeps a few long lists from
-// leaving most of the GPU idle.
+// `chunks` workgroups share the scoring of one list, each a run of pages; the first
+// `parts` of them then select for themselves and attend a share of the token list,
+// and the last of those to finish merges the partial results (the team scheme of the
+// fused block top-k step).  Splitting keeps a few long lists from leaving most of
+// the GPU idle.
+#include "kin_step.h"
 #include "kin_token.h"
 
 namespace kin {
@@ -20,7 +23,13 @@ struct TokenTopkParams {
   uint16_t* out;
   float* lse;           // optional
   int chunks;           // workgroups per list
-  int32_t* count;       // workspace: [lists] arrival counters, zero at launch and left zero
+  int parts;            // of them, how many go on to select and attend a share of the list (1: the last arriver alone)
+  int spin_limit;       // polls a member waits for its team before it scores the whole list itself
+  int32_t* count;       // workspace: [lists] arrival counters of the scoring, zero at launch
+  int32_t* count2;      // workspace, parts > 1: [lists] arrival counters of the partial results, zero at launch
+  uint32_t* ws_hist;    // workspace, parts > 1: [lists, chunks, 256] first-digit histograms of the members' keys
+  uint32_t* ws_po;      // workspace, parts > 1: [lists, parts, G, 128] normalised partial outputs (fp32 bits)
+  uint32_t* ws_plse;    // workspace, parts > 1: [lists, parts, G] their base-2 log-sum-exps
   uint32_t* keys;       // workspace: [lists, max_pages_per_seq * 16] (token keys, or block keys)
   float* scores;        // workspace, strided blocks only: [lists, max_pages_per_seq * 16]
   int block, stride;    // strided blocks only
@@ -49,6 +58,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
   constexpr int NT = NW * 64;
 
   const int tid = threadIdx.x;
+  KIN_STAMP_RESET();
+  KIN_STAMP(0);
   const int list_id = blockIdx.x / p.chunks, chunk = blockIdx.x - list_id * p.chunks;
   int b, h;
   if (!xcd_list_of(list_id, p.batch, p.num_kv_heads, b, h)) return;
@@ -109,37 +120,103 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
     sa.winners = reinterpret_cast<int32_t*>(smem);
   }
   const bool scored = STRIDED ? strided_needs_scores(t, sa) : token_needs_scores(t);
-  if (!scored && chunk) return;  // nothing to share: chunk 0 does the list alone
-  const bool hist_on_the_fly = !STRIDED && p.chunks == 1;
+  const bool team = p.parts > 1;  // several members select and attend
+  if (!scored && chunk && !team) return;  // nothing to share: chunk 0 does the list alone
+  if (team && chunk >= p.parts && !scored) return;
+  bool first_digit_counted = !STRIDED && (p.chunks == 1 || team);
   if (scored) {
     const int per = ((n_pages + p.chunks - 1) / p.chunks + 3) & ~3;  // whole quads of pages
     const int pg0 = min(chunk * per, n_pages), pg1 = min(pg0 + per, n_pages);
-    if (hist_on_the_fly) {
-      if (tid < 256) sh.hist[tid] = 0;
+    if (first_digit_counted) {
+      if (tid < 256) sh.hist[0][tid] = 0;
       __syncthreads();
     }
     if (STRIDED) strided_score_tokens<NW, LDSK, F16>(t, sa, pg0, pg1);
-    else token_score_keys<NW, LDSK, F16>(t, pg0, pg1, hist_on_the_fly ? sh.hist : nullptr);
+    else token_score_keys<NW, LDSK, F16>(t, pg0, pg1, first_digit_counted ? sh.hist[0] : nullptr);
     // Every wave waits for its own stores to be acknowledged; after the barrier the
     // workgroup's scores are in memory.
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
+    KIN_STAMP(50);  // this workgroup's share of the tokens is scored
     if (p.chunks > 1) {
-      // The slices meet through memory without cache maintenance: scores and the
-      // arrival counter are written and read at device scope.  Whoever counts in
-      // last sees everybody's scores and carries on alone; the others are done.
-      if (tid == 0)
-        sh_last = (__hip_atomic_fetch_add(&p.count[item], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.chunks - 1)
-                      ? 1 : 0;
-      __syncthreads();
-      if (!sh_last) return;
-      if (tid == 0) __hip_atomic_store(&p.count[item], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+      // The slices meet through memory without cache maintenance: scores, histograms and the
+      // arrival counters are written and read at device scope.
+      uint32_t* my_hist = p.ws_hist + ((int64_t)item * p.chunks + chunk) * 256;
+      if (team && !STRIDED) {
+        if (tid < 256) __hip_atomic_store(my_hist + tid, sh.hist[0][tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+      }
+      if (!team) {
+        // Whoever counts in last sees everybody's scores and carries on alone; the others are done.
+        if (tid == 0)
+          sh_last = (__hip_atomic_fetch_add(&p.count[item], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.chunks - 1)
+                        ? 1 : 0;
+        __syncthreads();
+        if (!sh_last) return;
+      } else {
+        if (tid == 0) __hip_atomic_fetch_add(&p.count[item], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (chunk >= p.parts) return;  // a member that only scores is done
+        // The members that go on need everybody's scores.  The wait is bounded, and a member whose
+        // patience runs out scores the whole list for itself (the same values land in the same
+        // places): an optimisation, never a dependency between workgroups.
+        if (tid == 0) {
+          int seen = __hip_atomic_load(&p.count[item], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (int spins = 0; seen < p.chunks && spins < p.spin_limit; ++spins) {
+            __builtin_amdgcn_s_sleep(4);
+            seen = __hip_atomic_load(&p.count[item], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+          sh_last = seen >= p.chunks ? 1 : 0;
+        }
+        __syncthreads();
+        if (__builtin_amdgcn_readfirstlane(sh_last)) {
+          if (!STRIDED) {
+            // The list's first-digit histogram is the sum of the members': every thread takes one bin of
+            // every (NT / 256)-th member, 16 loads in flight at a time (reads past the last member return 0).
+            if (tid < 256) sh.hist[0][tid] = 0;
+            __syncthreads();
+            const __amdgpu_buffer_rsrc_t rh = make_rsrc(p.ws_hist + (int64_t)item * p.chunks * 256, p.chunks * 256 * 4);
+            constexpr int kStep = NT / 256;
+            const int bin = tid & 255;
+            uint32_t sum = 0;
+            for (int c0 = tid >> 8; c0 < p.chunks; c0 += 16 * kStep) {
+              uint32_t x[16];
+#pragma unroll
+              for (int i = 0; i < 16; ++i)
+                x[i] = __builtin_amdgcn_raw_buffer_load_b32(rh, ((c0 + i * kStep) * 256 + bin) * 4, 0, kDeviceScope);
+#pragma unroll
+              for (int i = 0; i < 16; ++i) sum += x[i];
+            }
+            if (sum) atomicAdd(&sh.hist[0][bin], sum);
+          }
+        } else {
+          if (!STRIDED) {
+            if (tid < 256) sh.hist[0][tid] = 0;
+            __syncthreads();
+            token_score_keys<NW, LDSK, F16>(t, 0, n_pages, sh.hist[0]);
+          } else {
+            strided_score_tokens<NW, LDSK, F16>(t, sa, 0, n_pages);
+          }
+          __builtin_amdgcn_s_waitcnt(0);
+        }
+        __syncthreads();
+      }
     }
   }
-  const int n = STRIDED ? strided_select_list<NG, NW, LDSK>(t, sa, &sh) : token_select_list<NG, NW, LDSK>(t, &sh, hist_on_the_fly);
-  if (sel_out)
+  if (team && chunk != 0) t.sel_tokens = nullptr;  // the token positions are reported once, by member 0
+  KIN_STAMP(51);  // every share is scored: the select starts
+  const int n = STRIDED ? strided_select_list<NG, NW, LDSK>(t, sa, &sh) : token_select_list<NG, NW, LDSK>(t, &sh, first_digit_counted);
+  KIN_STAMP(52);  // token list ready
+  if (sel_out && (!team || chunk == 0))
     for (int i = n + tid; i < p.sel_stride; i += NT) sel_out[i] = -1;
-  if (p.sel_count && tid == 0) p.sel_count[item] = n;
+  if (p.sel_count && tid == 0 && (!team || chunk == 0)) p.sel_count[item] = n;
+  // This member's share of the list: whole tiles of 16 entries.
+  int e0 = 0, e1 = n;
+  if (team) {
+    const int per = (((n + p.parts - 1) / p.parts) + kPageSize - 1) & ~(kPageSize - 1);
+    e0 = min(chunk * per, n);
+    e1 = min(e0 + per, n);
+  }
 
   AttendArgs a;
   a.q_bh = t.q_bh;
@@ -150,25 +227,60 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void token_topk_kernel(To
   a.num_pages = p.num_pages;
   a.G = G;
   a.scale_log2 = p.scale_log2;
-  a.n = n;
+  a.n = e1 - e0;
   a.p0 = 0;
-  a.p1 = n;
+  a.p1 = a.n;
   a.last_len = kPageSize;
   a.first_skip = 0;
   a.rotate = 0;
   a.page_size = kPageSize;
-  attend_tokens<NG, NW, F16>(a, list, smem, sm_m, sm_l, [&](int g, int d, float o, float lse2) {
-    p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(o);
-    if (p.lse && d == 0) p.lse[hq0 + g] = lse2 * kLn2;
+  attend_tokens<NG, NW, F16>(a, list + e0, smem, sm_m, sm_l, [&](int g, int d, float o, float lse2) {
+    if (team) {
+      // partial result, read by a workgroup that may sit on another XCD: device-scope stores
+      const int64_t row = ((int64_t)item * p.parts + chunk) * G + g;
+      __hip_atomic_store(p.ws_po + row * kHeadDim + d, __float_as_uint(o), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (d == 0) __hip_atomic_store(p.ws_plse + row, __float_as_uint(lse2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+      p.out[(hq0 + g) * kHeadDim + d] = (uint16_t)f32_to_elem<F16>(o);
+      if (p.lse && d == 0) p.lse[hq0 + g] = lse2 * kLn2;
+    }
   });
+  KIN_STAMP(53);  // listed tokens attended
+  if (!team) return;
+  // Every wave waits for its partial stores to be acknowledged, then the workgroup counts in;
+  // whoever counts in last sees all parts and merges them.
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (tid == 0)
+    sh_last = (__hip_atomic_fetch_add(&p.count2[item], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.parts - 1) ? 1 : 0;
+  __syncthreads();
+  if (!__builtin_amdgcn_readfirstlane(sh_last)) return;
+  merge_list_parts<NT, F16>(smem, p.ws_po, p.ws_plse, item, p.parts, G, p.out + hq0 * kHeadDim, p.lse ? p.lse + hq0 : nullptr);
+  KIN_STAMP(45);  // parts merged
 }
 
 }  // namespace kin
 
 namespace kin {
 
-// Bytes of the arrival counters in front of the score arrays.
-static size_t token_count_bytes(int64_t lists) { return ((size_t)lists * sizeof(int32_t) + 255) & ~(size_t)255; }
+// Bytes of the arrival counters (two per list) in front of the score arrays.
+static size_t token_count_bytes(int64_t lists) { return ((size_t)lists * 2 * sizeof(int32_t) + 255) & ~(size_t)255; }
+
+// Most members of a team that go on to select and attend: a share of at least 128 listed tokens each.
+constexpr int kMaxTokenParts = 16;
+static int token_team_parts(int chunks, int list_cap) {
+  int parts = list_cap / 128;
+  if (parts > chunks) parts = chunks;
+  if (parts > kMaxTokenParts) parts = kMaxTokenParts;
+  return parts < 2 ? 1 : parts;
+}
+// What teams need behind the score arrays: the members' first-digit histograms and the partial results
+// (sized for the largest group, so that the sizing entry points need not know the group).
+static size_t token_team_bytes(int64_t lists, int chunks) {
+  if (chunks <= 1) return 0;
+  const int parts = chunks < kMaxTokenParts ? chunks : kMaxTokenParts;
+  return (size_t)lists * chunks * 256 * sizeof(uint32_t) + (size_t)lists * parts * kMaxGroup * (kHeadDim + 1) * sizeof(float);
+}
 
 // Workgroups that share the scoring of one list (each at least 64 pages = 256 KiB
 // of keys; with 256 the 8 lists of a small batch occupied 64 CUs: 109 against 97 us
@@ -249,8 +361,14 @@ static int launch_token_policy(const char* fn, bool f16, const kin_bf16_t* q, co
   p.out = out;
   p.lse = lse;
   p.count = static_cast<int32_t*>(workspace);
+  p.count2 = p.count + items;
   p.keys = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + count_bytes);
   p.scores = strided ? reinterpret_cast<float*>(static_cast<char*>(workspace) + count_bytes + key_bytes) : nullptr;
+  p.parts = 1;
+  p.spin_limit = team_spin_limit();
+  p.ws_hist = nullptr;
+  p.ws_po = nullptr;
+  p.ws_plse = nullptr;
   p.block = block;
   p.stride = stride;
   p.list_cap = list_cap > 0 ? list_cap : 1;
@@ -287,6 +405,17 @@ static int launch_token_policy(const char* fn, bool f16, const kin_bf16_t* q, co
     nw = items > kNumCus && small <= 50 * 1024 ? 4 : 12;
   } else {
     p.chunks = token_score_chunks(items, max_pages_per_seq);
+    // Teams: the members that scored go on to select and attend a share of the list each, given
+    // the room for their histograms and partial results behind the score arrays.
+    const size_t team_bytes = token_team_bytes(items, p.chunks);
+    const int parts = token_team_parts(p.chunks, list_cap);
+    if (parts > 1 && workspace_bytes >= need + team_bytes) {
+      p.parts = parts;
+      char* w = static_cast<char*>(workspace) + need;
+      p.ws_hist = reinterpret_cast<uint32_t*>(w);
+      p.ws_po = p.ws_hist + (size_t)items * p.chunks * 256;
+      p.ws_plse = p.ws_po + (size_t)items * parts * p.group * kHeadDim;
+    }
     // Up to one list per CU: 12 waves once a sequence may have more keys than 8 waves hold in
     // registers through the select's passes (32 K; 8 lists of 32 K tokens: 97 -> 83 us), else 8.
     nw = items <= kNumCus && (int64_t)max_pages_per_seq * kPageSize > 8 * 4096 ? 12 : (items <= 2 * kNumCus ? 8 : 4);
@@ -322,7 +451,7 @@ static int launch_token_policy(const char* fn, bool f16, const kin_bf16_t* q, co
   hipStream_t hs = static_cast<hipStream_t>(stream);
   if (p.chunks > 1) {
     // a kernel, not a memset node: this launch sequence may be captured into a HIP graph
-    fill_zero_i32_kernel<<<(unsigned)((items + 255) / 256), 256, 0, hs>>>(p.count, (int)items);
+    fill_zero_i32_kernel<<<(unsigned)((2 * items + 255) / 256), 256, 0, hs>>>(p.count, (int)(2 * items));
     st = check_hip(hipGetLastError(), "fill_zero_i32_kernel launch");
     if (st) return st;
   }
@@ -332,18 +461,24 @@ static int launch_token_policy(const char* fn, bool f16, const kin_bf16_t* q, co
 
 }  // namespace kin
 
+#ifdef KIN_TUNE
+KIN_STAMP_ACCESSOR(kin_debug_stamps_token)
+#endif
+
 extern "C" {
 
 size_t kin_token_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq) {
   if (batch <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0) return 0;
   const int64_t lists = (int64_t)batch * num_kv_heads;
-  return kin::token_count_bytes(lists) + (size_t)lists * max_pages_per_seq * kin::kPageSize * sizeof(uint32_t);
+  return kin::token_count_bytes(lists) + (size_t)lists * max_pages_per_seq * kin::kPageSize * sizeof(uint32_t) +
+         kin::token_team_bytes(lists, kin::token_score_chunks(lists, max_pages_per_seq));
 }
 
 size_t kin_strided_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq) {
   if (batch <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0) return 0;
   const int64_t lists = (int64_t)batch * num_kv_heads;
-  return kin::token_count_bytes(lists) + 2 * (size_t)lists * max_pages_per_seq * kin::kPageSize * sizeof(uint32_t);
+  return kin::token_count_bytes(lists) + 2 * (size_t)lists * max_pages_per_seq * kin::kPageSize * sizeof(uint32_t) +
+         kin::token_team_bytes(lists, kin::token_score_chunks(lists, max_pages_per_seq));
 }
 
 int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const int32_t* page_indices,

@@ -46,6 +46,17 @@ PHASES = {
     31: "pages attended",
     44: "team: partial result stored, counted in",
     45: "team: parts merged, output written",
+    # the token-granular policies (kin_token_topk.hip)
+    50: "token policy: this workgroup's tokens scored",
+    51: "token policy: every share scored, select starts",
+    54: "token policy: keys requested",
+    55: "token policy: radix digit 0 fixed",
+    56: "token policy: radix digit 1 fixed",
+    57: "token policy: radix digit 2 fixed",
+    58: "token policy: radix digit 3 fixed",
+    59: "token policy: winners listed in position order",
+    52: "token policy: token list ready",
+    53: "token policy: listed tokens attended",
 }
 MAX_WGS, MAX_STAMPS = 1024, 64
 
@@ -62,6 +73,9 @@ def main() -> None:
     ap.add_argument("--workload", default="qwen3-8b-readme", choices=sorted(bench.WORKLOADS))
     ap.add_argument("--batch", type=int, default=None, help="override the workload's batch size")
     ap.add_argument("--topk", type=int, default=None, help="override the workload's page budget")
+    ap.add_argument("--policy", default="block", choices=["block", "token", "strided"],
+                    help="block: the fused block top-k step; token / strided: LiteSys' token-granular policies "
+                         "(token budget 16 x the page budget, 4 sink tokens, a local window of 16)")
     ap.add_argument("--warmup", type=int, default=10)
     args = ap.parse_args()
     if not PHASES_LIB_PATH.exists():
@@ -70,8 +84,9 @@ def main() -> None:
     for name, (restype, argtypes) in _lib.SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype, fn.argtypes = restype, argtypes
-    lib.kin_debug_stamps_step.restype = ctypes.c_int
-    lib.kin_debug_stamps_step.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    accessor = lib.kin_debug_stamps_step if args.policy == "block" else lib.kin_debug_stamps_token
+    accessor.restype = ctypes.c_int
+    accessor.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
     _lib._lib = lib  # this process only: the operators below call the diagnostic build
 
     B, ctx, Hkv, G, topk, _ = bench.WORKLOADS[args.workload]
@@ -81,17 +96,30 @@ def main() -> None:
     st = bench.build_state(torch, ops, B, ctx, Hkv, G, topk, dev, ragged=args.workload in bench.RAGGED)
     ws = torch.empty(max(16, ops.step_workspace_bytes(B, Hkv, st["kbar"].shape[2])), dtype=torch.uint8, device=dev)
 
+    max_pages = st["max_pages_used"]
+    if args.policy == "token":
+        ws = torch.empty(max(16, ops.token_topk_workspace_bytes(B, Hkv, max_pages)), dtype=torch.uint8, device=dev)
+    elif args.policy == "strided":
+        ws = torch.empty(max(16, ops.strided_topk_workspace_bytes(B, Hkv, max_pages)), dtype=torch.uint8, device=dev)
+
     def step():
-        ops.blocktopk_decode_step(st["q"], st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"], topk,
-                                  out=st["out"], workspace=ws)
+        if args.policy == "token":
+            ops.token_topk_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], 16 * topk, max_pages, sink_tokens=4,
+                                  local_tokens=16, out=st["out"], workspace=ws)
+        elif args.policy == "strided":
+            ops.strided_topk_decode(st["q"], st["kv"], st["indices"], st["indptr"], st["last"], topk, max_pages, block_size=16,
+                                    stride=8, sink_tokens=4, local_tokens=16, out=st["out"], workspace=ws)
+        else:
+            ops.blocktopk_decode_step(st["q"], st["k"], st["v"], st["kv"], st["kbar"], st["indices"], st["indptr"], st["last"], topk,
+                                      out=st["out"], workspace=ws)
 
     stamps = np.zeros(MAX_WGS * MAX_STAMPS * 2, dtype=np.int64)
     counts = np.zeros(MAX_WGS, dtype=np.int32)
 
     def read():
-        rc = lib.kin_debug_stamps_step(stamps.ctypes.data_as(ctypes.c_void_p), counts.ctypes.data_as(ctypes.c_void_p))
+        rc = accessor(stamps.ctypes.data_as(ctypes.c_void_p), counts.ctypes.data_as(ctypes.c_void_p))
         if rc != 0:
-            raise RuntimeError(f"kin_debug_stamps_step failed ({rc})")
+            raise RuntimeError(f"reading the stamps failed ({rc})")
 
     for _ in range(args.warmup):
         step()
@@ -107,7 +135,7 @@ def main() -> None:
     wgs = [w for w in range(MAX_WGS) if counts[w] > 0]
     t0 = min(int(table[w, 0, 1]) for w in wgs)
     lists = B * Hkv
-    print(f"== {args.workload}: batch {B}, {Hkv} KV x {G} Q heads, ctx {ctx}, {topk} pages per list: {lists} lists; "
+    print(f"== {args.workload}{'' if args.policy == 'block' else ' (' + args.policy + ' policy)'}: batch {B}, {Hkv} KV x {G} Q heads, ctx {ctx}, {topk} pages per list: {lists} lists; "
           f"{len(wgs)} workgroups stamped{' (the first 1024)' if len(wgs) == MAX_WGS else ''}; "
           f"{e0.elapsed_time(e1) * 1e3 / reps:.1f} us per launch by HIP events, {reps} launches back to back")
     print("   when the workgroups pass each boundary (us since the first workgroup started):")

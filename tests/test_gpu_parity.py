@@ -983,6 +983,56 @@ def test_fused_step_split_scoring_for_few_long_sequences(ops, hkv, group, head_d
     assert torch.equal(one.sel, a.sel)
 
 
+@pytest.mark.parametrize("policy", ["block", "token", "strided"])
+def test_team_members_that_do_not_wait_get_the_same_result(ops, policy):
+    """The workgroups that share a list wait for each other's scores only as an optimisation: with
+    no patience at all (kin_set_team_spin_limit(0)) a member that finds its team incomplete scores
+    the whole list for itself, and cache bytes, lists and outputs are those of the default."""
+    from kinetics_amd import _lib
+
+    lib = _lib.load()
+    if policy == "block":
+        pb = P.make_problem(7100, [PS * 2300 + 5, PS * 1100 + 16, PS * 600 + 1, 40], num_kv_heads=2, group=4, topk=200)
+    else:
+        pb = P.make_problem(7101, [PS * 2100 + 7, PS * 1030 + 16, PS * 300 + 1, 17], num_kv_heads=1, group=4)
+
+    def run():
+        g = Gpu(pb)
+        if policy == "block":
+            assert ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[2]) > 0        # a shape that forms teams
+            g.sel = torch.full((pb.B, pb.Hkv, pb.topk + 1), -7, dtype=torch.int32, device=DEV)
+            out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, pb.topk, sel_pages=g.sel,
+                                            sel_count=g.cnt)
+            lists = (g.sel.clone(), g.cnt.clone())
+        else:
+            ops.append_paged_kv(g.k, g.v, g.kv, None, g.indices, g.indptr, g.last)
+            cap = 700 + 4 + 16
+            sel = torch.full((pb.B, pb.Hkv, cap), -7, dtype=torch.int32, device=DEV)
+            cnt = torch.full((pb.B, pb.Hkv), -7, dtype=torch.int32, device=DEV)
+            if policy == "token":
+                out = ops.token_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, 700, pb.max_pages, sink_tokens=4, local_tokens=16,
+                                            sel_tokens=sel, sel_count=cnt)
+            else:
+                out = ops.strided_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, 43, pb.max_pages, block_size=16, stride=8,
+                                              sink_tokens=4, local_tokens=16, sel_tokens=sel, sel_count=cnt)
+            lists = (sel, cnt)
+        torch.cuda.synchronize()
+        return out.clone(), g.kv.clone(), g.kbar.clone(), lists
+
+    want = run()
+    prev = lib.kin_set_team_spin_limit(0)
+    try:
+        assert prev == 300
+        got = [run() for _ in range(3)]
+    finally:
+        assert lib.kin_set_team_spin_limit(-1) == 0
+    assert lib.kin_set_team_spin_limit(-1) == 300
+    for out, kv, kbar, lists in got:
+        assert torch.equal(kv, want[1]) and torch.equal(kbar, want[2])
+        assert torch.equal(lists[0], want[3][0]) and torch.equal(lists[1], want[3][1])
+        assert torch.equal(out.view(torch.int16), want[0].view(torch.int16))
+
+
 @pytest.mark.parametrize("ps,fmt", [(16, "bf16"), (32, "bf16"), (64, "bf16"), (16, "f16")])
 def test_fused_step_split_attention_for_few_lists(ops, ps, fmt, head_dim):
     """Lists for at most half the CUs with long page lists: several workgroups per
