@@ -439,12 +439,16 @@ int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_bf16_t* k, c
  * ascending order, local tokens -- padded with -1, and sel_count[b,h] = n
  * (-1 for a sequence with more than max_pages_per_seq pages, which is skipped:
  * out = 0).  workspace: kin_token_topk_workspace_bytes(...) bytes of scratch
- * (4 bytes per cache slot and KV head, plus an arrival counter per list; any
+ * (4 bytes per cache slot and KV head, plus two arrival counters per list and,
+ * for fewer than 128 lists, up to 2.4 MB of histograms and partial results; any
  * contents, 16-byte aligned; with 128 lists or more and max_pages_per_seq up
  * to ~2300 the per-token keys stay in on-chip memory and the scratch is not
  * touched, but its size is still checked).  Reads every key of the context
  * once: HBM traffic is about half of dense decode's.  When the lists are fewer than
- * the GPU's compute units, several workgroups share the scoring of a list;
+ * the GPU's compute units, a team of workgroups shares a list: every member scores a run of
+ * pages, the first members then select for themselves and attend a share of the
+ * token list each, the last one merges (a workspace without the room for that part
+ * gets the older scheme: the last workgroup to arrive selects and attends alone);
  * a small kernel that zeroes the counters is then launched first on the
  * same stream (no memset, so the call can be captured in a HIP graph).
  * Limits: topk_tokens <= 4096, sink_tokens <= 64, local_tokens <= 1024.
