@@ -39,8 +39,7 @@
  *                 (ref: benchmark/blocktopk_decoder.py:143,217-221).
  *
  * Supported shapes: head_dim 128 or 64 (the reference reads it from the model
- * config, benchmark/blocktopk_decoder.py:104; the token-granular policies
- * kin_token_topk_decode / kin_strided_topk_decode: 128 only); page_size 16, 32 or 64
+ * config, benchmark/blocktopk_decoder.py:104); page_size 16, 32 or 64
  * (the reference's --page_size, benchmark/blocktopk.py:13; the token-granular
  * policies: 16 only);
  * num_q_heads % num_kv_heads == 0 and group size num_q_heads/num_kv_heads <= 16.
@@ -84,8 +83,8 @@ enum kin_status {
  * winners in index order.  3.0.0: every entry point that touches kbar takes
  * slot_ids / num_slots in front of the stream (kbar laid out by cache slot).
  * 3.1.0: head_dim 64 in the page path (append, mean keys, selector, sparse and
- * dense decode, the fused step), in kin_qkv_norm_split and, for rows of 64
- * elements, in kin_rms_norm. */
+ * dense decode, the fused step, the token-granular policies), in
+ * kin_qkv_norm_split and, for rows of 64 elements, in kin_rms_norm. */
 int kin_version(void);
 
 /* Human-readable text of the last non-OK status on the calling thread

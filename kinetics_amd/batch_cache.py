@@ -118,9 +118,6 @@ class PagedBatchKVManager:
             self.token_local = int(kwargs["attn_local"])
         if self.head_dim not in ops.HEAD_DIMS:
             raise NotImplementedError(f"head_dim {self.head_dim}: the paged kernels are built for {ops.HEAD_DIMS}")
-        if self.head_dim != ops.HEAD_DIM and (self.token_topk is not None or self.strided is not None):
-            raise NotImplementedError(f"the token-granular policies (attn_topk, attn_stride, attn_local alone) are built for "
-                                      f"head_dim {ops.HEAD_DIM} only; the block policy and dense attention also take 64")
         self.layer_skip = list(kwargs.get("attn_layer_skip", [0]))
         self.sink_pages = 1 if self.sparse else 0
         self.local_tokens = int(kwargs["attn_local"]) if self.sparse else 1

@@ -21,7 +21,7 @@ OBJ_DIR = PKG_DIR / "build"
 # build for kinetics_amd/phase_timeline.py, never loaded by the operators.
 PHASES_LIB_PATH = PKG_DIR / "libkinetics_amd_phases.so"
 
-SOURCES = ["kin_api.hip", "kin_append.hip", "kin_score_topk.hip", "kin_decode.hip", "kin_step.hip", "kin_token_topk.hip",
+SOURCES = ["kin_api.hip", "kin_append.hip", "kin_score_topk.hip", "kin_decode.hip", "kin_step.hip", "kin_token_topk.hip", "kin_token_topk_small.hip",
            "kin_table.hip", "kin_layer.hip"]
 
 HIPCC_FLAGS = [

@@ -277,23 +277,26 @@ __device__ __forceinline__ void radix_select_emit(const Keys& keys, int n_keys, 
 // those pages (slots past the last token included).  emit must not branch around
 // vector memory operations (store through a descriptor, out of range when !valid).  16-byte loads straight to registers, 16 of them in flight per
 // lane; no LDS, no barrier.
-template <int NW, bool F16 = false, typename Emit>
+template <int NW, bool F16 = false, int HD = kHeadDim, typename Emit>
 __device__ __forceinline__ void stream_token_scores(const TokenArgs& a, int pg0, int pg1, Emit emit) {
+  constexpr int LPR = HD / 8;          // lanes that share a key row (16-byte chunks of it): 16 or 8
+  constexpr int RPI = 64 / LPR;        // key rows one load instruction of a wave covers: 4 or 8
+  constexpr int LPP = kPageSize / RPI; // loads per page (a K plane of 16 rows): 4 or 2
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int l = tid & 63, kg = l >> 4, c16 = l & 15;
+  const int l = tid & 63, rg = l / LPR, cc = l & (LPR - 1);
   const int G = a.G;
   const int32_t* table = a.table;
   // The mean over the group's heads of q_g . k_t is (mean_g q_g) . k_t: one dot
-  // product per token.  Lane owns columns d = 8*(lane%16) .. +7 of the mean query;
-  // 16 lanes share a key row, one load instruction of a wave covers 4 rows.
+  // product per token.  Lane owns columns d = 8*cc .. +7 of the mean query;
+  // LPR lanes share a key row, one load instruction of a wave covers RPI rows.
   float qm[8];
   {
 #pragma unroll
     for (int u = 0; u < 8; ++u) qm[u] = 0.f;
-    const uint16_t* qp = a.q_bh + 8 * c16;
+    const uint16_t* qp = a.q_bh + 8 * cc;
     for (int g = 0; g < G; ++g) {
-      const uint4 x = *reinterpret_cast<const uint4*>(qp + (int64_t)g * kHeadDim);
+      const uint4 x = *reinterpret_cast<const uint4*>(qp + (int64_t)g * HD);
       qm[0] += elem_lo<F16>(x.x); qm[1] += elem_hi<F16>(x.x);
       qm[2] += elem_lo<F16>(x.y); qm[3] += elem_hi<F16>(x.y);
       qm[4] += elem_lo<F16>(x.z); qm[5] += elem_hi<F16>(x.z);
@@ -303,19 +306,19 @@ __device__ __forceinline__ void stream_token_scores(const TokenArgs& a, int pg0,
 #pragma unroll
     for (int u = 0; u < 8; ++u) qm[u] *= inv;
   }
-  // A wave streams whole K planes (4 KiB contiguous, four 16-byte loads per lane:
-  // load i covers key rows 4*i .. 4*i+3), four consecutive pages at a time: the
+  // A wave streams whole K planes (16 rows, contiguous for one KV head; LPP 16-byte loads per lane:
+  // load i covers key rows RPI*i .. RPI*i + RPI-1), four consecutive pages at a time: the
   // quads pg0/4 + w, + NW, ... of the page range, the next quad in flight.  After
-  // a quad every lane holds one score -- lane (kg, c16) that of row 4*(c16%4) + kg
-  // of the quad's page c16/4 -- so one emit per quad covers 64 consecutive cache
+  // a quad every lane holds one score -- lane l that of the row l / LPR of the quad's load l % LPR
+  // (load j = LPP * page + i) -- so one emit per quad covers 64 consecutive cache
   // slots (256 B of keys: full lines, a quarter of the stores).
   constexpr int kPF = 4;
   const __attribute__((address_space(4))) int32_t* tab_c =
       reinterpret_cast<const __attribute__((address_space(4))) int32_t*>(reinterpret_cast<uintptr_t>(table));
-  const int voff = kg * a.row_bytes + c16 * 16;
-  const int row_step = 4 * a.row_bytes;
+  const int voff = rg * a.row_bytes + cc * 16;
+  const int row_step = RPI * a.row_bytes;
   const int k_span = kPageSize * a.row_bytes - (a.span < a.page_bytes ? a.page_bytes - a.span : 0);  // K plane only
-  auto load_page = [&](int p, u32x4 (&dst)[4]) {
+  auto load_page = [&](int p, u32x4 (&dst)[LPP]) {
     // Pages past the end (or with an id outside the cache) are read through an
     // empty descriptor: zeros, no memory traffic.
     const bool in = p < pg1;
@@ -323,9 +326,10 @@ __device__ __forceinline__ void stream_token_scores(const TokenArgs& a, int pg0,
     const bool ok = in && id >= 0 && (int64_t)id < a.num_pages;
     const __amdgpu_buffer_rsrc_t r = make_rsrc(a.kvb + (int64_t)(ok ? id : 0) * a.page_bytes, ok ? k_span : 0);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dst[i] = __builtin_amdgcn_raw_buffer_load_b128(r, voff + i * row_step, 0, kStreamLoad);
+    for (int i = 0; i < LPP; ++i) dst[i] = __builtin_amdgcn_raw_buffer_load_b128(r, voff + i * row_step, 0, kStreamLoad);
   };
-  const int my_page = c16 >> 2, my_row = 4 * (c16 & 3) + kg;
+  const int my_load = cc;                                   // the quad's load whose row this lane reports
+  const int my_page = my_load / LPP, my_row = RPI * (my_load % LPP) + rg;
   // The wave's quads are qi = w, w + NW, ... of the range's nq quads, visited from a
   // list-specific starting quad (a.rotate) and wrapping around: scores are stored by
   // position, so the order is free, and equal lists that run in step then read from
@@ -338,7 +342,7 @@ __device__ __forceinline__ void stream_token_scores(const TokenArgs& a, int pg0,
     const int qq = qi + rot;
     return pg0 + kPF * (qq >= nq ? qq - nq : qq);
   };
-  u32x4 x[kPF][4];
+  u32x4 x[kPF][LPP];
   {
     const int p0 = quad_page(w);
 #pragma unroll
@@ -354,22 +358,24 @@ __device__ __forceinline__ void stream_token_scores(const TokenArgs& a, int pg0,
     float mine = 0.f;
 #pragma unroll
     for (int u = 0; u < kPF; ++u) {
-      u32x4 kx[4];
+      u32x4 kx[LPP];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) kx[i] = x[u][i];
+      for (int i = 0; i < LPP; ++i) kx[i] = x[u][i];
       load_page(next + u, x[u]);
-      float acc[4];
+      float acc[LPP];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < LPP; ++i) {
         float s = 0.f;
         s = fmaf(qm[0], elem_lo<F16>(kx[i].x), s); s = fmaf(qm[1], elem_hi<F16>(kx[i].x), s);
         s = fmaf(qm[2], elem_lo<F16>(kx[i].y), s); s = fmaf(qm[3], elem_hi<F16>(kx[i].y), s);
         s = fmaf(qm[4], elem_lo<F16>(kx[i].z), s); s = fmaf(qm[5], elem_hi<F16>(kx[i].z), s);
         s = fmaf(qm[6], elem_lo<F16>(kx[i].w), s); s = fmaf(qm[7], elem_hi<F16>(kx[i].w), s);
-        acc[i] = row16_sum(s);
+        acc[i] = row_sum<LPR>(s);
       }
-      const int i_mine = c16 & 3;
-      const float pick = i_mine == 0 ? acc[0] : i_mine == 1 ? acc[1] : i_mine == 2 ? acc[2] : acc[3];
+      const int i_mine = my_load % LPP;
+      float pick = acc[0];
+#pragma unroll
+      for (int i = 1; i < LPP; ++i) pick = i_mine == i ? acc[i] : pick;
       if (my_page == u) mine = pick;
     }
     // Called by every lane, without a branch: conditionally executed memory operations in
@@ -393,13 +399,13 @@ __device__ __forceinline__ bool token_needs_scores(const TokenArgs& a) {
 // LDSK, into a.lds_keys; 0 marks "not a candidate", order_key is never 0 for a finite
 // score.  hist: 256 zeroed LDS counters that receive the histogram of the keys' top
 // byte, or null.  No barrier inside; the stores are complete after s_waitcnt(0).
-template <int NW, bool LDSK = false, bool F16 = false>
+template <int NW, bool LDSK = false, bool F16 = false, int HD = kHeadDim>
 __device__ __forceinline__ void token_score_keys(const TokenArgs& a, int pg0, int pg1, uint32_t* hist) {
   const int dyn_lo = a.pad + a.n_sink, dyn_hi = dyn_lo + a.n_dyn;  // cache slots of the candidates
   const __amdgpu_buffer_rsrc_t keys_rsrc = make_rsrc(a.keys, LDSK ? 0 : a.n_pages * kPageSize * 4);
   uint32_t* lds_keys = a.lds_keys;
   const int dump = a.n_pages * kPageSize;  // lanes without a row write here
-  stream_token_scores<NW, F16>(a, pg0, pg1, [&](int c, float score, bool valid) {
+  stream_token_scores<NW, F16, HD>(a, pg0, pg1, [&](int c, float score, bool valid) {
     const uint32_t key = (c >= dyn_lo && c < dyn_hi) ? order_key(score) : 0u;
     if constexpr (LDSK)
       lds_keys[valid ? c : dump] = key;
@@ -477,12 +483,12 @@ __device__ __forceinline__ bool strided_needs_scores(const TokenArgs& a, const S
 
 // fp32 scores of the tokens of the pages pg0 <= p < pg1 -> sa.scores (device-scope
 // stores) or, LDSK, -> a.lds_keys (as bit patterns).
-template <int NW, bool LDSK = false, bool F16 = false>
+template <int NW, bool LDSK = false, bool F16 = false, int HD = kHeadDim>
 __device__ __forceinline__ void strided_score_tokens(const TokenArgs& a, const StridedArgs& sa, int pg0, int pg1) {
   const __amdgpu_buffer_rsrc_t scores_rsrc = make_rsrc(sa.scores, LDSK ? 0 : a.n_pages * kPageSize * 4);
   uint32_t* lds_scores = a.lds_keys;
   const int dump = a.n_pages * kPageSize;
-  stream_token_scores<NW, F16>(a, pg0, pg1, [&](int c, float score, bool valid) {
+  stream_token_scores<NW, F16, HD>(a, pg0, pg1, [&](int c, float score, bool valid) {
     if constexpr (LDSK)
       lds_scores[valid ? c : dump] = __float_as_uint(score);
     else
@@ -620,52 +626,59 @@ __device__ __forceinline__ int strided_select_list(const TokenArgs& a, const Str
 // and online softmax as attend_list(); a "page" is any 16 consecutive list
 // entries, each K and V row fetched from its own address.
 // lds: attend_lds_bytes(NW); sm_m / sm_l: NW x (4*NG) floats each.
-template <int NG, int NW, bool F16 = false, typename Emit>
+template <int NG, int NW, bool F16 = false, int HD = kHeadDim, typename Emit>
 __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t* list, unsigned char* lds,
                                               float (*sm_m)[4 * NG], float (*sm_l)[4 * NG], Emit emit) {
+  constexpr int CPR = HD / 8;                   // 16-byte chunks of a head row
+  constexpr int KC = HD / 32;                   // matrix steps over the head dimension = LDS-direct loads per tile
+  constexpr int RPI = 64 / CPR;                 // K rows one LDS-direct load brings
+  constexpr int NV = attend_v_loads<NG, HD>();  // V rows per lane and tile
+  constexpr int kStage = kPageSize * HD * 2;    // bytes of one K stage
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int l = tid & 63, kg = l >> 4, c16 = l & 15, gq = l & 3;
+  const int l = tid & 63, kg = l >> 4, c16 = l & 15, gq = l & 3, cc = c16 & (CPR - 1);
+  const int half = NV == 2 ? (c16 >> 3) : 0;
+  const int vrow0 = 4 * kg + 2 * half;          // tile row of this lane's first V row
   const int G = a.G;
   const int n = a.n;
 
-  uint4 qB[4];
+  uint4 qB[KC];
   {
     const int g = min(NG == 4 ? c16 : gq, G - 1);
-    const uint16_t* qp = a.q_bh + (int64_t)g * kHeadDim + 8 * kg;
+    const uint16_t* qp = a.q_bh + (int64_t)g * HD + 8 * kg;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) qB[c] = *reinterpret_cast<const uint4*>(qp + 32 * c);
+    for (int c = 0; c < KC; ++c) qB[c] = *reinterpret_cast<const uint4*>(qp + 32 * c);
   }
 
   const int row_bytes = a.row_bytes;
   const int page_bytes = a.page_bytes;
   const char* kvb = a.kvb;
   const int64_t max_tok = a.num_pages * kPageSize;
-  unsigned char* kl = lds + w * (2 * 4096);
-  int kchunk[4], lds_r[4];
+  unsigned char* kl = lds + w * (kAttendStages * kStage);
+  int krow[KC], kchunk[KC], lds_r[KC];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    const int row = 4 * c + kg;                       // K row this lane helps to fetch with load c
-    kchunk[c] = ((c16 ^ row) & 15) * 16;              // the chunk that belongs at its LDS position
-    lds_r[c] = c16 * 256 + (((4 * c + kg) ^ c16) & 15) * 16;
+  for (int c = 0; c < KC; ++c) {
+    krow[c] = RPI * c + l / CPR;                                           // K row this lane helps to fetch with load c
+    kchunk[c] = ((cc ^ attend_swizzle<HD>(krow[c])) & (CPR - 1)) * 16;      // the chunk that belongs at its LDS position
+    lds_r[c] = c16 * (HD * 2) + (((4 * c + kg) ^ attend_swizzle<HD>(c16)) & (CPR - 1)) * 16;
   }
-  const int vchunk = kPageSize * row_bytes + c16 * 16;  // V plane of the page, this lane's columns
+  const int vchunk = kPageSize * row_bytes + cc * 16;  // V plane of the page, this lane's columns
 
   float m_run = kNegInf, l_run = 0.f;
   floatx4 O[8];
 #pragma unroll
   for (int u = 0; u < 8; ++u) O[u] = floatx4{0.f, 0.f, 0.f, 0.f};
-  auto scores = [&](const uint4 (&ka)[4], float (&pr)[4], int valid) {
+  auto scores = [&](const uint4 (&ka)[KC], float (&pr)[4], int valid) {
     if constexpr (NG == 4)
-      page_scores_wide<F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, 0, valid, kg);
+      page_scores_wide<F16, KC>(ka, qB, m_run, l_run, O, pr, a.scale_log2, 0, valid, kg);
     else
-      page_scores<F16>(ka, qB, m_run, l_run, O, pr, a.scale_log2, 0, valid, kg);
+      page_scores<F16, KC>(ka, qB, m_run, l_run, O, pr, a.scale_log2, 0, valid, kg);
   };
-  auto pv = [&](const u32x4 (&vr)[4], const float (&pr)[4]) {
+  auto pv = [&](const u32x4 (&vr)[NV], const float (&pr)[4]) {
     if constexpr (NG == 4)
-      page_pv_wide<F16>(vr, pr, O, 0);
+      page_pv_wide<F16, HD>(vr, pr, O, 16 * (c16 >> 3));
     else
-      page_pv<F16>(vr, pr, O, 0);
+      page_pv<F16, NV>(vr, pr, O, half);
   };
 
   // This wave takes the 16-entry groups w, w+NW, ...  Entries past the end (and
@@ -677,48 +690,48 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
     const int t = ok ? tok : 0;
     return kvb + (int64_t)(t >> 4) * page_bytes + (t & (kPageSize - 1)) * row_bytes;
   };
-  struct Ids { int k[4], v[4], valid; };
+  struct Ids { int k[KC], v[NV], valid; };
   auto fetch_ids = [&](int it) {
     Ids ids;
     const int base = (w + NW * it) * kPageSize;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int e = base + 4 * c + kg;
+    for (int c = 0; c < KC; ++c) {
+      const int e = base + krow[c];
       ids.k[c] = (e < n) ? list[e] : -1;
     }
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int e = base + 4 * kg + r;
+    for (int r = 0; r < NV; ++r) {
+      const int e = base + vrow0 + r;
       ids.v[r] = (e < n) ? list[e] : -1;
     }
     ids.valid = max(0, min(kPageSize, n - base));
     return ids;
   };
-  auto issue_v = [&](const Ids& ids, u32x4 (&vv)[4]) {
+  auto issue_v = [&](const Ids& ids, u32x4 (&vv)[NV]) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
+    for (int r = 0; r < NV; ++r)
       vv[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(row_ptr(ids.v[r]) + vchunk));
   };
   auto issue_k = [&](const Ids& ids, int stage) {
     __attribute__((address_space(3))) unsigned char* dst =
-        (__attribute__((address_space(3))) unsigned char*)(kl + stage * 4096);
+        (__attribute__((address_space(3))) unsigned char*)(kl + stage * kStage);
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
+    for (int c = 0; c < KC; ++c)
       __builtin_amdgcn_global_load_lds(
           reinterpret_cast<const __attribute__((address_space(1))) void*>(
               reinterpret_cast<uintptr_t>(row_ptr(ids.k[c]) + kchunk[c])),
           dst + c * 1024, 16, 0, kStreamLoad);
   };
-  auto read_k = [&](int stage, uint4 (&ka)[4]) {
+  auto read_k = [&](int stage, uint4 (&ka)[KC]) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) ka[c] = *reinterpret_cast<const uint4*>(kl + stage * 4096 + lds_r[c]);
+    for (int c = 0; c < KC; ++c) ka[c] = *reinterpret_cast<const uint4*>(kl + stage * kStage + lds_r[c]);
   };
 
-  // Same explicit wait as in attend_list(): when it executes, exactly the 4 V
+  // Same explicit wait as in attend_list(): when it executes, exactly the NV V
   // loads issued just before it may be outstanding.
   if (iters > 0) {
-    u32x4 vA[4], vB[4];
-    uint4 ka[4];
+    u32x4 vA[NV], vB[NV];
+    uint4 ka[KC];
     float pr[4];
     Ids idA = fetch_ids(0), idB;
     issue_k(idA, 0);
@@ -729,14 +742,14 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
         __builtin_amdgcn_sched_barrier(0);
         issue_v(idB, vB);
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(wait_vm_imm(4));
+        __builtin_amdgcn_s_waitcnt(wait_vm_imm(NV));
         __builtin_amdgcn_sched_barrier(0);
         read_k(0, ka);
         __builtin_amdgcn_sched_barrier(0);
         issue_k(idB, 1);
         __builtin_amdgcn_sched_barrier(0);
         scores(ka, pr, idA.valid);
-        if (idA.valid != kPageSize) clear_unused_v_rows<4>(vA, 0, idA.valid, 4 * kg);
+        if (idA.valid != kPageSize) clear_unused_v_rows<NV>(vA, 0, idA.valid, vrow0);
         pv(vA, pr);
       }
       {
@@ -744,19 +757,19 @@ __device__ __forceinline__ void attend_tokens(const AttendArgs& a, const int32_t
         __builtin_amdgcn_sched_barrier(0);
         issue_v(idA, vA);
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(wait_vm_imm(4));
+        __builtin_amdgcn_s_waitcnt(wait_vm_imm(NV));
         __builtin_amdgcn_sched_barrier(0);
         read_k(1, ka);
         __builtin_amdgcn_sched_barrier(0);
         issue_k(idA, 0);
         __builtin_amdgcn_sched_barrier(0);
         scores(ka, pr, idB.valid);
-        if (idB.valid != kPageSize) clear_unused_v_rows<4>(vB, 0, idB.valid, 4 * kg);
+        if (idB.valid != kPageSize) clear_unused_v_rows<NV>(vB, 0, idB.valid, vrow0);
         pv(vB, pr);
       }
     }
   }
-  attend_finish<NG, NW, kHeadDim>(m_run, l_run, O, G, lds, sm_m, sm_l, emit);
+  attend_finish<NG, NW, HD>(m_run, l_run, O, G, lds, sm_m, sm_l, emit);
 }
 
 }  // namespace kin

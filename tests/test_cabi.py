@@ -170,8 +170,9 @@ def test_token_topk_argument_errors(lib):
     assert tok(mp=0) == _lib.KIN_ERR_BAD_SHAPE
     assert tok(topk=5000) == _lib.KIN_ERR_UNSUPPORTED
     assert tok(local=2000) == _lib.KIN_ERR_UNSUPPORTED
-    assert tok(D=64) == _lib.KIN_ERR_UNSUPPORTED                      # the token-granular policies: head_dim 128 only
-    assert b"head_dim=64" in lib.kin_last_error()
+    assert tok(D=96) == _lib.KIN_ERR_UNSUPPORTED                      # head rows of 64 and 128 elements only
+    assert b"head_dim=96" in lib.kin_last_error()
+    assert tok(D=64, B=0) == _lib.KIN_OK
     assert tok(sel=A, cnt=A, stride=12) == _lib.KIN_ERR_BAD_SHAPE      # 8 + 4 + 1 entries needed
     assert tok(sel=A, stride=13) == _lib.KIN_ERR_NULL_POINTER
     assert lib.kin_token_topk_workspace_bytes(2, 1, 4) == 256 + 2 * 4 * 16 * 4  # arrival counters + keys

@@ -67,12 +67,11 @@ def test_rejects_what_it_does_not_implement():
         PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_block_topk=2)          # LiteSys: local required
     with pytest.raises(NotImplementedError):
         PagedBatchKVManager(cfg, 2, 64, DEV, torch.bfloat16, attn_block_topk=2, attn_local=4, attn_block_size=24)
-    # head rows of 64 elements: dense attention and the block policy, not the token-granular policies; other sizes: nothing
+    # head rows of 64 elements: every policy; other sizes: nothing
     cfg64 = SimpleNamespace(num_attention_heads=4, num_key_value_heads=2, head_dim=64, hidden_size=256, num_hidden_layers=1)
-    PagedBatchKVManager(cfg64, 2, 64, DEV, torch.bfloat16, attn_block_topk=2, attn_local=4)
-    for token_policy in (dict(attn_topk=8, attn_local=4), dict(attn_local=4), dict(attn_block_topk=2, attn_local=4, attn_stride=8)):
-        with pytest.raises(NotImplementedError, match="head_dim 128"):
-            PagedBatchKVManager(cfg64, 2, 64, DEV, torch.bfloat16, **token_policy)
+    for policy in (dict(attn_block_topk=2, attn_local=4), dict(attn_topk=8, attn_local=4), dict(attn_local=4),
+                   dict(attn_block_topk=2, attn_local=4, attn_stride=8)):
+        PagedBatchKVManager(cfg64, 2, 64, DEV, torch.bfloat16, **policy)
     cfg96 = SimpleNamespace(num_attention_heads=4, num_key_value_heads=2, head_dim=96, hidden_size=384, num_hidden_layers=1)
     with pytest.raises(NotImplementedError, match="head_dim 96"):
         PagedBatchKVManager(cfg96, 2, 64, DEV, torch.bfloat16)
@@ -90,12 +89,7 @@ _POLICIES = [(dict(), None), (dict(attn_block_topk=3, attn_local=16), True),
              (dict(attn_block_topk=3, attn_local=5, attn_stride=4, attn_block_size=8), None)]
 
 
-def _token_kernels(sparse):
-    return "attn_topk" in sparse or "attn_stride" in sparse or (bool(sparse) and "attn_block_topk" not in sparse)
-
-
-# head rows of 64 elements: dense attention and the block policy (the token-granular policies are built for 128 only)
-_CASES = [(s, f, 128) for s, f in _POLICIES] + [(s, f, 64) for s, f in _POLICIES if not _token_kernels(s)]
+_CASES = [(s, f, hd) for hd in (128, 64) for s, f in _POLICIES]
 
 
 @pytest.mark.parametrize("sparse,fused,head_dim", _CASES)

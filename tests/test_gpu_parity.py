@@ -984,7 +984,7 @@ def test_fused_step_split_scoring_for_few_long_sequences(ops, hkv, group, head_d
 
 
 @pytest.mark.parametrize("policy", ["block", "token", "strided"])
-def test_team_members_that_do_not_wait_get_the_same_result(ops, policy):
+def test_team_members_that_do_not_wait_get_the_same_result(ops, policy, head_dim):
     """The workgroups that share a list wait for each other's scores only as an optimisation: with
     no patience at all (kin_set_team_spin_limit(0)) a member that finds its team incomplete scores
     the whole list for itself, and cache bytes, lists and outputs are those of the default."""
@@ -1225,8 +1225,8 @@ def _check_token_topk(ops, pb, topk, sink, local, offset, what, max_pages=None):
         n_dyn = S - n_sink - n_local
         k_eff = min(topk, n_dyn)
         pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
-        K = O.elem_to_f32(kv[pages, 0]).reshape(-1, pb.Hkv, D)[offset : offset + S]
-        V = O.elem_to_f32(kv[pages, 1]).reshape(-1, pb.Hkv, D)[offset : offset + S]
+        K = O.elem_to_f32(kv[pages, 0]).reshape(-1, pb.Hkv, kv.shape[-1])[offset : offset + S]
+        V = O.elem_to_f32(kv[pages, 1]).reshape(-1, pb.Hkv, kv.shape[-1])[offset : offset + S]
         got_keep = np.zeros((pb.Hkv, S), dtype=bool)
         for h in range(pb.Hkv):
             n = cnt[b, h]
@@ -1251,7 +1251,7 @@ def _check_token_topk(ops, pb, topk, sink, local, offset, what, max_pages=None):
 
 @pytest.mark.parametrize("case", ["mixed", "hkv8", "g8", "g7", "many", "many_12_waves", "many_g16", "offset", "all",
                                   "window_only", "split", "split_many"])
-def test_token_topk_decode(ops, case):
+def test_token_topk_decode(ops, case, head_dim):
     """LiteSys' token-level top-k (sparsity_utils.py:6-21): sink tokens, the
     top-k tokens of the middle by group-mean logit, the local window."""
     if case == "mixed":
@@ -1336,8 +1336,8 @@ def _check_strided(ops, pb, topk, sink, local, block, stride, offset, what, need
             continue
         S = keeps[b].shape[1]
         pages = O.seq_pages(pb.page_indices, pb.page_indptr, b)
-        K = O.elem_to_f32(kv[pages, 0]).reshape(-1, pb.Hkv, D)[offset : offset + S]
-        V = O.elem_to_f32(kv[pages, 1]).reshape(-1, pb.Hkv, D)[offset : offset + S]
+        K = O.elem_to_f32(kv[pages, 0]).reshape(-1, pb.Hkv, kv.shape[-1])[offset : offset + S]
+        V = O.elem_to_f32(kv[pages, 1]).reshape(-1, pb.Hkv, kv.shape[-1])[offset : offset + S]
         got_keep = np.zeros((pb.Hkv, S), dtype=bool)
         for h in range(pb.Hkv):
             n = cnt[b, h]
@@ -1358,7 +1358,7 @@ def _check_strided(ops, pb, topk, sink, local, block, stride, offset, what, need
 
 
 @pytest.mark.parametrize("case", ["mixed", "hkv8_stride4", "g8", "g5", "many", "many_12_waves", "offset", "stride16", "split", "block8_stride3"])
-def test_strided_topk_decode(ops, case):
+def test_strided_topk_decode(ops, case, head_dim):
     """LiteSys' strided overlapping-block policy (sparsity_utils.py:49-105)."""
     block, stride, offset = 16, 8, 0
     if case == "mixed":
@@ -1400,7 +1400,7 @@ def test_strided_topk_decode(ops, case):
 
 
 @pytest.mark.parametrize("policy", ["token", "strided"])
-def test_token_policies_in_float16(ops, policy):
+def test_token_policies_in_float16(ops, policy, head_dim):
     """The kin_*_f16 twins of the token-granular policies: few long lists (shared
     scoring through HBM keys), and many lists (keys in LDS), against the oracle
     reading the same bits as float16."""
@@ -1420,7 +1420,7 @@ def test_token_policies_in_float16(ops, policy):
 
 
 @pytest.mark.parametrize("policy", ["token", "strided"])
-def test_token_policies_with_the_gpu_full_of_lists(ops, policy):
+def test_token_policies_with_the_gpu_full_of_lists(ops, policy, head_dim):
     """128 lists or more: one workgroup per list, and the per-token keys (scores,
     for the strided policy) stay in LDS when ``max_pages_per_seq`` lets them fit --
     one 12-wave workgroup per list up to 256 lists or for long sequences, 4-wave
@@ -1455,7 +1455,7 @@ def test_token_policies_with_the_gpu_full_of_lists(ops, policy):
 
 
 @pytest.mark.parametrize("lists", [1, 2])
-def test_token_topk_ties_pick_the_lowest_positions(ops, lists):
+def test_token_topk_ties_pick_the_lowest_positions(ops, lists, head_dim):
     """Equal scores are taken in ascending token position, also across the
     register-sized chunks the selecting workgroup walks the keys in (more than
     32768 keys at 8 waves) and across the workgroups that share the scoring."""
@@ -1465,14 +1465,14 @@ def test_token_topk_ties_pick_the_lowest_positions(ops, lists):
     ops.append_paged_kv(g.k, g.v, g.kv, None, g.indices, g.indptr, g.last)
     # list 0: every key identical -> every candidate ties; list 1 (if any): two score levels, the
     # higher one on every ninth token, fewer of them than the budget -> the rest by position
-    row = torch.randn(D, device=DEV).to(torch.bfloat16)
+    row = torch.randn(head_dim, device=DEV).to(torch.bfloat16)
     for b in range(lists):
         pages = g.indices[int(pb.page_indptr[b]): int(pb.page_indptr[b + 1])].long()
         g.kv[pages, 0] = row
         if b == 1:
-            K = g.kv[pages, 0].reshape(-1, D)        # [slots, D] copy
+            K = g.kv[pages, 0].reshape(-1, head_dim)  # [slots, D] copy
             K[::9] = row * 2
-            g.kv[pages, 0] = K.reshape(-1, PS, 1, D)
+            g.kv[pages, 0] = K.reshape(-1, PS, 1, head_dim)
     g.q[:] = row.float().sign().to(torch.bfloat16)   # q . row > 0: doubled rows score higher
     topk, sink, local = 4000, 4, 16
     sel = torch.full((lists, 1, topk + sink + local), -7, dtype=torch.int32, device=DEV)
@@ -1496,7 +1496,7 @@ def test_token_topk_ties_pick_the_lowest_positions(ops, lists):
         assert np.array_equal(mid, want), f"list {b}: first difference at {np.flatnonzero(mid != want)[:5]}"
 
 
-def test_seeded_sweep_of_token_policies(ops):
+def test_seeded_sweep_of_token_policies(ops, head_dim):
     """30 seeded random configurations of the two token-granular policies: head
     counts, groups 1..8, ragged lengths with empty and tiny sequences, budgets
     above and below the candidate count, sink / window / padding, block sizes and
