@@ -286,6 +286,7 @@ def cpu_model_name():
 
 LAST_LAUNCH_MS = []
 LAST_GRAPH_REPLAY_MS = None
+LAST_GRAPH_REPLAY_10_MS = None   # ten steps per graph
 
 
 @contextlib.contextmanager
@@ -306,11 +307,14 @@ def collector_paused():
 GRAPH_REPLAY_BELOW_MS = 0.1   # steps shorter than this are host-bound when launched eagerly
 
 
-def time_graph_replay(torch, step, steps, warmup):
-    """The step captured once as a HIP graph and replayed: what the GPU does when
+def time_graph_replay(torch, step, steps, warmup, per_graph=1):
+    """The step captured as a HIP graph and replayed: what the GPU does when
     the host is out of the way (the launch-overhead half of the reference's
-    torch.compile(mode="max-autotune"), benchmark/blocktopk.py:41-43).  All ``steps``
-    replays are queued back to back between two synchronisations; ms per step."""
+    torch.compile(mode="max-autotune"), benchmark/blocktopk.py:41-43).  The graph holds
+    ``per_graph`` consecutive steps (a served model replays one graph per forward pass,
+    a step per layer: each replay costs a few microseconds of its own, which one step per
+    graph pays in full); about ``steps`` steps in all are queued back to back between
+    two synchronisations; ms per step."""
     cur = torch.cuda.current_stream()
     side = torch.cuda.Stream()
     side.wait_stream(cur)
@@ -319,26 +323,29 @@ def time_graph_replay(torch, step, steps, warmup):
         step()
         side.synchronize()
         with torch.cuda.graph(graph, stream=side):
-            step()
+            for _ in range(per_graph):
+                step()
     cur.wait_stream(side)
     torch.cuda.synchronize()
+    replays = max(1, steps // per_graph)
     with collector_paused():
-        for _ in range(warmup):
+        for _ in range(max(1, warmup // per_graph)):
             graph.replay()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(steps):
+        for _ in range(replays):
             graph.replay()
         torch.cuda.synchronize()
-        dt = (time.perf_counter() - t0) / steps
+        dt = (time.perf_counter() - t0) / (replays * per_graph)
     del graph
     return dt * 1e3
 
 
 def time_step(torch, ops, st, B, Hkv, topk, steps, warmup, mode="auto"):
-    """W untimed and K timed decode steps on the state ``st``; HIP events on the
-    launch stream bracket every kernel.  Returns (ms_per_step, elapsed_s,
-    {kernel: mean ms}, fused?).  When the eager step is shorter than
+    """W untimed and K timed decode steps on the state ``st``, timed by the host clock between two
+    synchronisations and by HIP events on the launch stream: one pair around the timed region when
+    the step is one call (the fused step), a record between all launches when it is three.  Returns
+    (ms_per_step, elapsed_s, {kernel: mean ms}, fused?).  When the eager step is shorter than
     GRAPH_REPLAY_BELOW_MS, LAST_GRAPH_REPLAY_MS also holds the same step replayed
     as a HIP graph (None otherwise)."""
     device = st["q"].device
@@ -360,7 +367,16 @@ def time_step(torch, ops, st, B, Hkv, topk, steps, warmup, mode="auto"):
                                                                  out=st["out"], workspace=st["ws"])),
         ]
     K = steps
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(kernels) + 1)] for _ in range(K)]
+    # Events on the launch stream.  A step that is one kernel gets one pair around the K launches of the
+    # timed region: its average launch duration is their distance / K (the ~1 us between dependent
+    # launches included).  An event record is a packet of its own in the queue and holds the next kernel
+    # back by 2.5-5 us (qwen3-8b-readme: 38.6-40.6 us per step with no record between the launches, 41.2
+    # with one, 46.6 with two), so records between the launches would time themselves; the reference's
+    # loop has none either (benchmark/blocktopk.py:47-61).  A step of several kernels needs the records
+    # between them to tell the kernels apart, and pays for them.
+    per_launch = len(kernels) > 1
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(kernels) + 1)] for _ in range(K if per_launch else 0)]
+    region = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
     # the collection happens before the warm-up, so that nothing but a synchronise lies between the
     # warm-up and the timed steps (a GPU left idle for the tens of milliseconds of a collection runs
     # its next launches slower: 1.5 % on 20 timed steps)
@@ -370,22 +386,42 @@ def time_step(torch, ops, st, B, Hkv, topk, steps, warmup, mode="auto"):
                 fn()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for i in range(K):
-            ev[i][0].record()
-            for j, (_, fn) in enumerate(kernels):
+        region[0].record()
+        if per_launch:
+            for i in range(K):
+                ev[i][0].record()
+                for j, (_, fn) in enumerate(kernels):
+                    fn()
+                    ev[i][j + 1].record()
+        else:
+            fn = kernels[0][1]
+            for _ in range(K):
                 fn()
-                ev[i][j + 1].record()
+        region[1].record()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
-    kernel_ms = {name: statistics.fmean(e[j].elapsed_time(e[j + 1]) for e in ev) for j, (name, _) in enumerate(kernels)}
-    global LAST_LAUNCH_MS, LAST_GRAPH_REPLAY_MS
+        # after the timed region: a few launches bracketed one by one, for the spread between launches
+        P = K if per_launch else min(K, 20)
+        if not per_launch:
+            ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(P)]
+            for i in range(P):
+                ev[i][0].record()
+                fn()
+                ev[i][1].record()
+            torch.cuda.synchronize()
+    global LAST_LAUNCH_MS, LAST_GRAPH_REPLAY_MS, LAST_GRAPH_REPLAY_10_MS
     LAST_LAUNCH_MS = [round(sum(e[j].elapsed_time(e[j + 1]) for j in range(len(kernels))), 3) for e in ev]
-    LAST_GRAPH_REPLAY_MS = None
+    if per_launch:
+        kernel_ms = {name: statistics.fmean(e[j].elapsed_time(e[j + 1]) for e in ev) for j, (name, _) in enumerate(kernels)}
+    else:
+        kernel_ms = {kernels[0][0]: region[0].elapsed_time(region[1]) / K}
+    LAST_GRAPH_REPLAY_MS = LAST_GRAPH_REPLAY_10_MS = None
     if elapsed / K * 1e3 < GRAPH_REPLAY_BELOW_MS:
         def whole_step():
             for _, fn in kernels:
                 fn()
         LAST_GRAPH_REPLAY_MS = time_graph_replay(torch, whole_step, K, warmup)
+        LAST_GRAPH_REPLAY_10_MS = time_graph_replay(torch, whole_step, K, warmup, per_graph=10)
     return elapsed / K * 1e3, elapsed, kernel_ms, fused
 
 
@@ -471,6 +507,7 @@ def side_workload(torch, ops, name, steps, warmup, device, with_dense=True):
         # a step this short is host-bound when launched eagerly: the same launches replayed as one HIP graph
         out["graph_replay_ms_per_step"] = LAST_GRAPH_REPLAY_MS
         out["graph_replay_frac"] = ab["step"] / (LAST_GRAPH_REPLAY_MS * 1e-3) / 1e9 / HBM_PEAK_GBS
+        out["graph_of_10_steps_replay_ms_per_step"] = LAST_GRAPH_REPLAY_10_MS
     if fused:
         out["kernel_frac"] = ab["step"] / (kernel_ms["fused_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS
         tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
@@ -682,7 +719,7 @@ def main():
           f"KV {st['kv'].numel() * 2 / 1e9:.1f} GB resident at {hex(st['kv'].data_ptr())}, kbar at {hex(st['kbar'].data_ptr())}, "
           f"setup {time.perf_counter() - t_setup:.1f}s", file=sys.stderr, flush=True)
 
-    # -- the timed region: K steps; HIP events on the launch stream bracket each kernel
+    # -- the timed region: K steps between two synchronisations and two HIP events on the launch stream
     K = args.steps
     ms_step, elapsed, kernel_ms, fused = time_step(torch, ops, st, B, Hkv, topk, K, args.warmup, args.mode)
 
@@ -737,6 +774,7 @@ def main():
     if LAST_GRAPH_REPLAY_MS is not None:
         result["graph_replay_ms_per_step"] = LAST_GRAPH_REPLAY_MS
         result["graph_replay_frac"] = ab["step"] / (LAST_GRAPH_REPLAY_MS * 1e-3) / 1e9 / HBM_PEAK_GBS
+        result["graph_of_10_steps_replay_ms_per_step"] = LAST_GRAPH_REPLAY_10_MS
     if world:
         # the figure benchmark/blocktopk.py:82 prints divides the per-layer rate by world_size * num_hidden_layers;
         # it is built from the attention step alone here (the whole layer: --whole-layer)
