@@ -254,6 +254,8 @@ struct StepPlan {
 };
 
 constexpr int kMaxTeam = 64;
+// Most lists beyond one per CU that still get teams (see plan_step).
+constexpr int kMaxTailLists = 96;
 
 static size_t round256(size_t n) { return (n + 255) & ~(size_t)255; }
 
@@ -277,8 +279,14 @@ static size_t team_workspace_bytes(int64_t team_lists, int parts, int group, int
 // each.  Measured on MI355X (ctx 32 K, k = 128, G = 4, us per step; one workgroup per list |
 // teams | the earlier scheme, in which every part scored the whole list for itself): 8 lists
 // 38 | 30 | 35; 32 lists 45 | 35 | 45; 64 lists 48 | 42 | 50; 128 lists 54 | 56 | 56.
+// A batch of up to kMaxTailLists lists more than the GPU has CUs keeps one workgroup per list for the
+// first 256 and forms teams of 2-4 for the rest (first 256 lists alone | with tail teams, us per step:
+// ctx 32 K, k = 128, G = 4: 264 lists 95 | 81; 304 lists 101 | 93; 352 lists 108 | 104; 384 lists 109 |
+// 112 (not formed); G = 8, k = 256: 264 lists 171 | 137; 304 lists 175 | 149; 352 lists 180 | 165;
+// ctx 16 K, k = 64: 264 lists 55.9 | 50.0; 352 lists 61.4 | 59.9; 8 KV heads of G = 2, k = 64: 264
+// lists 71.5 | 60.6; 352 lists 78.3 | 75.4; the best team size falls from 4-8 at 8 extra lists to 2 at 96).
 // Tried and not kept, because one workgroup per list is faster there: teams of two or three for
-// 129 .. 400 lists (160 lists 53 | 73; 256 lists 74 | 92; 300 lists 102 | 109: the streaming
+// every list of 129 .. 400 (160 lists 53 | 73; 256 lists 74 | 92; 300 lists 102 | 109: the streaming
 // phases are bound by HBM either way, and the exchange, the second select and the merge add
 // 9 us to every list's critical path, a fill launch in front 4 more), and teams for the lists
 // of the second round of a batch a little larger than the GPU holds at once (1024 lists of
@@ -298,6 +306,16 @@ static StepPlan plan_step(int64_t items, int group, int kbar_pages, int64_t list
     if (team > kMaxTeam) team = kMaxTeam;
     parts = team < by_attend ? team : by_attend;
     head = 0;
+  } else if (items > kNumCus && items - kNumCus <= kMaxTailLists && (list_tiles >= 96 || kbar_pages >= 1024)) {
+    // A few lists more than CUs: one workgroup per list would leave a few CUs with two lists and
+    // the others waiting for them.  The lists beyond the first kNumCus get teams instead, small
+    // enough that every CU ends up with about the same bytes.
+    const int64_t tail = items - kNumCus;
+    team = tail <= 32 ? 4 : (tail <= 72 ? 3 : 2);
+    const int64_t useful = by_attend > by_score ? by_attend : by_score;
+    if (team > useful) team = useful;
+    parts = team < by_attend ? team : by_attend;
+    head = kNumCus;
   }
   if (parts < 1) parts = 1;
   if (team < 2) {

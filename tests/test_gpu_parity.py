@@ -983,7 +983,7 @@ def test_fused_step_split_scoring_for_few_long_sequences(ops, hkv, group, head_d
     assert torch.equal(one.sel, a.sel)
 
 
-@pytest.mark.parametrize("policy", ["block", "token", "strided"])
+@pytest.mark.parametrize("policy", ["block", "block_tail", "token", "strided"])
 def test_team_members_that_do_not_wait_get_the_same_result(ops, policy, head_dim):
     """The workgroups that share a list wait for each other's scores only as an optimisation: with
     no patience at all (kin_set_team_spin_limit(0)) a member that finds its team incomplete scores
@@ -993,12 +993,14 @@ def test_team_members_that_do_not_wait_get_the_same_result(ops, policy, head_dim
     lib = _lib.load()
     if policy == "block":
         pb = P.make_problem(7100, [PS * 2300 + 5, PS * 1100 + 16, PS * 600 + 1, 40], num_kv_heads=2, group=4, topk=200)
+    elif policy == "block_tail":  # 290 lists: the 34 beyond one per CU in teams of 3
+        pb = P.make_problem(7102, [PS * 120 + 5] * 144 + [40], num_kv_heads=2, group=4, topk=100)
     else:
         pb = P.make_problem(7101, [PS * 2100 + 7, PS * 1030 + 16, PS * 300 + 1, 17], num_kv_heads=1, group=4)
 
     def run():
         g = Gpu(pb)
-        if policy == "block":
+        if policy.startswith("block"):
             assert ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[2]) > 0        # a shape that forms teams
             g.sel = torch.full((pb.B, pb.Hkv, pb.topk + 1), -7, dtype=torch.int32, device=DEV)
             out = ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, pb.topk, sel_pages=g.sel,
@@ -1554,7 +1556,7 @@ def test_token_topk_rejects_short_workspace_and_long_sequences(ops):
 # --------------------------------------------------------------------------- graph capture / tracing
 
 
-@pytest.mark.parametrize("path", ["three", "three_split", "fused", "fused_split", "fused_parts", "token", "strided",
+@pytest.mark.parametrize("path", ["three", "three_split", "fused", "fused_split", "fused_parts", "fused_tail", "token", "strided",
                                   "token_split", "strided_split"])
 def test_step_replays_under_hip_graph(ops, path):
     """No allocation, no host sync, fixed buffers: every launch sequence can be
@@ -1564,6 +1566,8 @@ def test_step_replays_under_hip_graph(ops, path):
         pb = P.make_problem(801, [PS * 2300 + 3, PS * 2100 + 9], num_kv_heads=1, group=4, topk=32)
     elif path == "fused_parts":   # few lists with long page lists: fill kernel + several workgroups attend each list
         pb = P.make_problem(802, [PS * 400 + 3] * 5 + [PS * 90], num_kv_heads=2, group=4, topk=200)
+    elif path == "fused_tail":    # 280 lists: the 24 beyond one per CU in teams
+        pb = P.make_problem(803, [PS * 110 + 3] * 140, num_kv_heads=2, group=4, topk=100)
     else:
         pb = P.make_problem(800, [PS * 200 + 3] * 66, num_kv_heads=2, group=4, topk=32)
     g = Gpu(pb)
@@ -1572,14 +1576,14 @@ def test_step_replays_under_hip_graph(ops, path):
     step_ws = torch.empty(max(16, ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[2])), dtype=torch.uint8, device=DEV)
     tok_ws = torch.empty(max(16, ops.strided_topk_workspace_bytes(pb.B, pb.Hkv, pb.max_pages)), dtype=torch.uint8, device=DEV)
     tok_sel = torch.full((pb.B, pb.Hkv, 64 * 16 + 4 + 16), -1, dtype=torch.int32, device=DEV)
-    assert path.endswith(("_split", "_parts")) == (ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[2]) > 0)
+    assert path.endswith(("_split", "_parts", "_tail")) == (ops.step_workspace_bytes(pb.B, pb.Hkv, pb.kbar.shape[2]) > 0)
 
     def step():
         if path in ("three", "three_split"):
             ops.append_paged_kv(g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last)
             ops.block_score_topk(g.q, g.kbar, g.indices, g.indptr, g.last, pb.topk, g.sel, g.cnt, workspace=step_ws)
             ops.sparse_paged_decode(g.q, g.kv, g.sel, g.cnt, g.last, out=out, workspace=ws)
-        elif path in ("fused", "fused_split", "fused_parts"):
+        elif path in ("fused", "fused_split", "fused_parts", "fused_tail"):
             ops.blocktopk_decode_step(g.q, g.k, g.v, g.kv, g.kbar, g.indices, g.indptr, g.last, pb.topk, out=out,
                                       sel_pages=g.sel, sel_count=g.cnt, workspace=step_ws)
         else:
@@ -1641,7 +1645,8 @@ def test_custom_ops_trace_with_fullgraph(ops):
 # --------------------------------------------------------------------------- fused step
 
 
-@pytest.mark.parametrize("case", ["mixed", "hkv8", "g8", "fills", "ties", "long", "many", "many_g8", "mid"])
+@pytest.mark.parametrize("case", ["mixed", "hkv8", "g8", "fills", "ties", "long", "many", "many_g8", "mid", "tail_teams",
+                                  "tail_teams_g8"])
 def test_fused_step_equals_three_calls(ops, case, head_dim):
     """kin_blocktopk_decode_step must give what append + score/select + attend
     give and match the oracle: cache bytes, mean keys and page lists bit for bit;
@@ -1667,6 +1672,15 @@ def test_fused_step_equals_three_calls(ops, case, head_dim):
     elif case == "many_g8":    # > 256 lists with a group above 4: 4 waves per list
         rng = np.random.default_rng(907)
         pb = P.make_problem(907, [int(x) for x in rng.integers(1, PS * 30, size=300)], num_kv_heads=1, group=8, topk=6)
+    elif case == "tail_teams":  # a few lists more than CUs, page lists of 96 tiles or more: the lists beyond the first
+        # 256 are handled by teams of workgroups (here 44 of them, teams of 3; tiny and empty sequences among them)
+        rng = np.random.default_rng(909)
+        lengths = [int(x) for x in rng.integers(PS * 100, PS * 180, size=150)]
+        lengths[131], lengths[140], lengths[149] = 0, 5, PS * 3 + 1
+        pb = P.make_problem(909, lengths, num_kv_heads=2, group=4, topk=100)
+    elif case == "tail_teams_g8":  # the same with 8 heads per list and 14 lists in teams of 4
+        rng = np.random.default_rng(910)
+        pb = P.make_problem(910, [int(x) for x in rng.integers(PS * 110, PS * 150, size=270)], num_kv_heads=1, group=8, topk=110)
     else:                      # 257..512 lists: 4 waves per list, not every CU with three workgroups
         rng = np.random.default_rng(908)
         pb = P.make_problem(908, [int(x) for x in rng.integers(1, PS * 40, size=150)], num_kv_heads=2, group=3, topk=9)
@@ -1698,7 +1712,7 @@ def test_fused_step_equals_three_calls(ops, case, head_dim):
     if np.array_equal(sel, res["sel_pages"]):
         assert_out_close(out_b, res["out"], f"fused {case} vs oracle end to end")
     else:
-        assert case in ("long", "many", "many_g8", "mid")  # only near-ties may reorder; checked by selection_matches elsewhere
+        assert case in ("long", "many", "many_g8", "mid", "tail_teams", "tail_teams_g8")  # only near-ties may reorder; checked by selection_matches elsewhere
     # optional outputs may be omitted; no append when k, v are None
     c = Gpu(pb)
     ops.append_paged_kv(c.k, c.v, c.kv, c.kbar, c.indices, c.indptr, c.last)

@@ -78,6 +78,9 @@ def test_static_scratch_step_equals_workspace_step():
     _both_ways(ops, parts, sink=1, local=20, what="fourth call (split attention)", must_split=True)
     full = P.make_problem(9105, [PS * 1300 + 5] * 4, num_kv_heads=2, group=16, topk=1100)
     _both_ways(ops, full, sink=0, local=1, what="fifth call (split attention, 16 heads per list)", must_split=True)
+    # a few lists more than CUs: the 24 lists beyond the first 256 in teams
+    tail = P.make_problem(9107, [PS * 110 + 3] * 139 + [7], num_kv_heads=2, group=4, topk=100)
+    _both_ways(ops, tail, sink=0, local=1, what="call with 280 lists (teams for the last 24)", must_split=True)
     # and the first shape once more after them
     _both_ways(ops, big, sink=0, local=33, what="sixth call (first shape again)", must_split=True)
 
