@@ -321,10 +321,11 @@ int kin_dense_paged_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache,
  * shares a list: each scores a slice of the candidates, the keys meet in the
  * workspace, and the members each select for themselves (identical results),
  * attend a part of the listed pages and leave a partial result that the last to
- * finish merges.  A batch of up to 96 lists more than the GPU has compute units
- * (257 .. 352 lists) keeps one workgroup per list for the first 256 and forms
- * teams of 2 to 4 for the others, so that no compute unit is left with two
- * whole lists.  A member waits for its team's keys for a bounded time only
+ * finish merges.  A batch of up to 96 lists more than a multiple of the GPU's
+ * 256 compute units (257 .. 352 lists, 513 .. 608, ...) keeps one workgroup
+ * per list for that multiple and forms teams of 2 to 4 for the others, so that
+ * the launch does not end with a few compute units working on whole lists
+ * while the others wait.  A member waits for its team's keys for a bounded time only
  * and then scores the list alone, so the launch never depends on which
  * workgroups run at the same time.  Without sel_pages the winners are attended
  * in index order instead of score order (no sort).  slot_lens (optional, int32

@@ -51,6 +51,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
     h = list - b * p.num_kv_heads;
   } else if (p.head_lists == p.batch * p.num_kv_heads) {
     if (!xcd_list_of(blockIdx.x, p.batch, p.num_kv_heads, b, h)) return;
+  } else if (p.head_lists % (kNumXcds * p.num_kv_heads) == 0) {
+    // whole groups of 8 sequences in front of the teams: the same placement as without teams
+    xcd_list_of(blockIdx.x, p.head_lists / p.num_kv_heads, p.num_kv_heads, b, h);
   } else {
     b = blockIdx.x / p.num_kv_heads;
     h = blockIdx.x - b * p.num_kv_heads;
@@ -254,7 +257,7 @@ struct StepPlan {
 };
 
 constexpr int kMaxTeam = 64;
-// Most lists beyond one per CU that still get teams (see plan_step).
+// Most lists beyond a multiple of the CUs that still get teams (see plan_step).
 constexpr int kMaxTailLists = 96;
 
 static size_t round256(size_t n) { return (n + 255) & ~(size_t)255; }
@@ -279,12 +282,16 @@ static size_t team_workspace_bytes(int64_t team_lists, int parts, int group, int
 // each.  Measured on MI355X (ctx 32 K, k = 128, G = 4, us per step; one workgroup per list |
 // teams | the earlier scheme, in which every part scored the whole list for itself): 8 lists
 // 38 | 30 | 35; 32 lists 45 | 35 | 45; 64 lists 48 | 42 | 50; 128 lists 54 | 56 | 56.
-// A batch of up to kMaxTailLists lists more than the GPU has CUs keeps one workgroup per list for the
-// first 256 and forms teams of 2-4 for the rest (first 256 lists alone | with tail teams, us per step:
+// A batch of up to kMaxTailLists lists more than a multiple of the CUs keeps one workgroup per list for
+// that multiple and forms teams of 2-4 for the rest (one workgroup per list | with tail teams, us per step:
 // ctx 32 K, k = 128, G = 4: 264 lists 95 | 81; 304 lists 101 | 93; 352 lists 108 | 104; 384 lists 109 |
 // 112 (not formed); G = 8, k = 256: 264 lists 171 | 137; 304 lists 175 | 149; 352 lists 180 | 165;
 // ctx 16 K, k = 64: 264 lists 55.9 | 50.0; 352 lists 61.4 | 59.9; 8 KV heads of G = 2, k = 64: 264
-// lists 71.5 | 60.6; 352 lists 78.3 | 75.4; the best team size falls from 4-8 at 8 extra lists to 2 at 96).
+// lists 71.5 | 60.6; 352 lists 78.3 | 75.4; the best team size falls from 4-8 at 8 extra lists to 2 at 96;
+// ctx 32 K, k = 128, G = 4 again: 528 lists 154 | 141; 600: 166 | 164; 784: 228 | 210; 864: 241 | 237; 1040: 269 |
+// 259; 1552: 400 | 378; 2080: 521 | 499; 4128: 1078 | 1050; G = 8, k = 256: 528 lists 279 | 242; 816: 401 | 354;
+// 1040: 475 | 446; 1600: 703 | 664).  A batch that is a multiple of the CUs gains nothing from teams for its last
+// lists (4096 lists: 961 | 962-988; 1024 lists of 8 heads: 430 | 435-471).
 // Tried and not kept, because one workgroup per list is faster there: teams of two or three for
 // every list of 129 .. 400 (160 lists 53 | 73; 256 lists 74 | 92; 300 lists 102 | 109: the streaming
 // phases are bound by HBM either way, and the exchange, the second select and the merge add
@@ -306,16 +313,18 @@ static StepPlan plan_step(int64_t items, int group, int kbar_pages, int64_t list
     if (team > kMaxTeam) team = kMaxTeam;
     parts = team < by_attend ? team : by_attend;
     head = 0;
-  } else if (items > kNumCus && items - kNumCus <= kMaxTailLists && (list_tiles >= 96 || kbar_pages >= 1024)) {
-    // A few lists more than CUs: one workgroup per list would leave a few CUs with two lists and
-    // the others waiting for them.  The lists beyond the first kNumCus get teams instead, small
-    // enough that every CU ends up with about the same bytes.
-    const int64_t tail = items - kNumCus;
+  } else if (items > kNumCus && items % kNumCus != 0 && items % kNumCus <= kMaxTailLists &&
+             (list_tiles >= 96 || kbar_pages >= 1024)) {
+    // A few lists more than a multiple of the CUs: the GPU hands out workgroups in order, so the
+    // last few would run on a few CUs (beside another list each, or alone at the end) while the
+    // others wait for them.  Those lists get teams instead, small enough that every CU ends up
+    // with about the same bytes.
+    const int64_t tail = items % kNumCus;
     team = tail <= 32 ? 4 : (tail <= 72 ? 3 : 2);
     const int64_t useful = by_attend > by_score ? by_attend : by_score;
     if (team > useful) team = useful;
     parts = team < by_attend ? team : by_attend;
-    head = kNumCus;
+    head = items - tail;
   }
   if (parts < 1) parts = 1;
   if (team < 2) {
