@@ -454,6 +454,9 @@ int kin_blocktopk_decode_step_static(const kin_bf16_t* q, const kin_bf16_t* k, c
  * gets the older scheme: the last workgroup to arrive selects and attends alone);
  * a small kernel that zeroes the counters is then launched first on the
  * same stream (no memset, so the call can be captured in a HIP graph).
+ * A batch of up to 96 lists more than a multiple of the GPU's 256 compute units
+ * (when that multiple is whole sequences) is two launches, one after the other
+ * on the stream: the multiple, then the rest with the GPU to themselves.
  * Limits: topk_tokens <= 4096, sink_tokens <= 64, local_tokens <= 1024.
  */
 size_t kin_token_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq);

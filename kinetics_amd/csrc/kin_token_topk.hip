@@ -43,6 +43,32 @@ static int token_score_chunks(int64_t lists, int max_pages_per_seq) {
   return (int)(want < by_len ? want : by_len);
 }
 
+// Lists that a batch has beyond a multiple of the CUs, when they are few enough to be worth a launch of
+// their own (see launch_token_policy) and the multiple is whole sequences; else 0.
+constexpr int kMaxTokenTailLists = 96;
+static int64_t token_tail_lists(int64_t lists, int num_kv_heads) {
+  if (lists <= kNumCus || kNumCus % num_kv_heads != 0) return 0;
+  const int64_t tail = lists % kNumCus;
+  return tail <= kMaxTokenTailLists ? tail : 0;
+}
+// Workspace of one launch over `lists` lists: counters, keys (and scores: arrays = 2), what teams need.
+static size_t token_workspace_need(int64_t lists, int max_pages_per_seq, int arrays) {
+  return token_count_bytes(lists) + (size_t)arrays * lists * max_pages_per_seq * kPageSize * sizeof(uint32_t) +
+         token_team_bytes(lists, token_score_chunks(lists, max_pages_per_seq));
+}
+// The same for a call, which may be two launches that use the workspace one after the other.
+static size_t token_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq, int arrays) {
+  if (batch <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0) return 0;
+  const int64_t lists = (int64_t)batch * num_kv_heads;
+  size_t need = token_workspace_need(lists, max_pages_per_seq, arrays);
+  const int64_t tail = token_tail_lists(lists, num_kv_heads);
+  if (tail > 0) {
+    const size_t t = token_workspace_need(tail, max_pages_per_seq, arrays);
+    if (t > need) need = t;
+  }
+  return need;
+}
+
 // Shared by the two entry points.  topk counts tokens (block == 0) or blocks.
 static int launch_token_policy(const char* fn, bool f16, const kin_bf16_t* q, const kin_bf16_t* kv_cache,
                                const int32_t* page_indices, const int32_t* page_indptr, const int32_t* last_page_len,
@@ -50,7 +76,8 @@ static int launch_token_policy(const char* fn, bool f16, const kin_bf16_t* q, co
                                int first_page_offset, int32_t* sel_tokens, int32_t* sel_count, kin_bf16_t* out,
                                float* lse, void* workspace, size_t workspace_bytes, int batch, int num_q_heads,
                                int num_kv_heads, int head_dim, int page_size, int64_t num_pages,
-                               int max_pages_per_seq, int sel_stride, float sm_scale, kin_stream_t stream) {
+                               int max_pages_per_seq, int sel_stride, float sm_scale, kin_stream_t stream,
+                               bool may_split = true) {
   const bool strided = block > 0;
   if (!q || !kv_cache || !page_indices || !page_indptr || !last_page_len || !out)
     return fail(KIN_ERR_NULL_POINTER, "%s: null pointer argument", fn);
@@ -97,6 +124,30 @@ static int launch_token_policy(const char* fn, bool f16, const kin_bf16_t* q, co
     return fail(KIN_ERR_WORKSPACE, "%s: needs %zu workspace bytes, got %zu", fn, need,
                 workspace ? workspace_bytes : (size_t)0);
   if (!aligned16(workspace)) return fail(KIN_ERR_MISALIGNED, "%s: workspace must be 16-byte aligned", fn);
+
+  // A few lists more than a multiple of the CUs: the GPU hands out workgroups in order, so the last few
+  // lists would run on a few CUs after everybody else has finished (a 12-wave workgroup has a CU to
+  // itself: 300 lists are two rounds, the second of 44).  Two launches instead, one after the other on
+  // the stream: the whole rounds, then the rest with the GPU to themselves (shared scoring and teams,
+  // as for any small batch; the workspace is used by one launch at a time).  Measured, 2048 tokens of
+  // 32 K, one launch | two: 264 lists 545 | 423 us; 300: 575 | 497; 352: 616 | 590; 528: 942 | 835;
+  // 800: 1311 | 1223; 1056: 1670 | 1585.
+  if (may_split && token_tail_lists(items, num_kv_heads) > 0) {
+    const int b0 = (int)((items - token_tail_lists(items, num_kv_heads)) / num_kv_heads);
+    const int hq = num_q_heads, d = head_dim;
+    st = launch_token_policy(fn, f16, q, kv_cache, page_indices, page_indptr, last_page_len, topk, block, stride, sink_tokens,
+                             local_tokens, first_page_offset, sel_tokens, sel_count, out, lse, workspace, workspace_bytes, b0,
+                             num_q_heads, num_kv_heads, head_dim, page_size, num_pages, max_pages_per_seq, sel_stride, sm_scale,
+                             stream, false);
+    if (st) return st;
+    return launch_token_policy(fn, f16, q + (size_t)b0 * hq * d, kv_cache, page_indices, page_indptr + b0, last_page_len + b0, topk,
+                               block, stride, sink_tokens, local_tokens, first_page_offset,
+                               sel_tokens ? sel_tokens + (size_t)b0 * num_kv_heads * sel_stride : nullptr,
+                               sel_count ? sel_count + (size_t)b0 * num_kv_heads : nullptr, out + (size_t)b0 * hq * d,
+                               lse ? lse + (size_t)b0 * hq : nullptr, workspace, workspace_bytes, batch - b0, num_q_heads,
+                               num_kv_heads, head_dim, page_size, num_pages, max_pages_per_seq, sel_stride, sm_scale, stream,
+                               false);
+  }
 
   TokenTopkParams p;
   p.q = q;
@@ -213,17 +264,11 @@ KIN_STAMP_ACCESSOR(kin_debug_stamps_token)
 extern "C" {
 
 size_t kin_token_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq) {
-  if (batch <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0) return 0;
-  const int64_t lists = (int64_t)batch * num_kv_heads;
-  return kin::token_count_bytes(lists) + (size_t)lists * max_pages_per_seq * kin::kPageSize * sizeof(uint32_t) +
-         kin::token_team_bytes(lists, kin::token_score_chunks(lists, max_pages_per_seq));
+  return kin::token_workspace_bytes(batch, num_kv_heads, max_pages_per_seq, 1);
 }
 
 size_t kin_strided_topk_workspace_bytes(int batch, int num_kv_heads, int max_pages_per_seq) {
-  if (batch <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0) return 0;
-  const int64_t lists = (int64_t)batch * num_kv_heads;
-  return kin::token_count_bytes(lists) + 2 * (size_t)lists * max_pages_per_seq * kin::kPageSize * sizeof(uint32_t) +
-         kin::token_team_bytes(lists, kin::token_score_chunks(lists, max_pages_per_seq));
+  return kin::token_workspace_bytes(batch, num_kv_heads, max_pages_per_seq, 2);
 }
 
 int kin_token_topk_decode(const kin_bf16_t* q, const kin_bf16_t* kv_cache, const int32_t* page_indices,
