@@ -659,7 +659,7 @@ def main():
     ap.add_argument("--gen_len", type=int, default=32768)
     ap.add_argument("--batch_size", type=int, default=256)
     ap.add_argument("--topk_page", type=int, default=64)
-    ap.add_argument("--page_size", type=int, default=16, choices=[16, 32, 64],
+    ap.add_argument("--page_size", type=int, default=16, choices=[16, 32, 64, 128],
                     help="tokens per page of the cache (any workload; the reference's flag, benchmark/blocktopk.py:13)")
     ap.add_argument("--world_size", type=int, default=8)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float16"],

@@ -39,7 +39,7 @@
  *                 (ref: benchmark/blocktopk_decoder.py:143,217-221).
  *
  * Supported shapes: head_dim 128 or 64 (the reference reads it from the model
- * config, benchmark/blocktopk_decoder.py:104); page_size 16, 32 or 64
+ * config, benchmark/blocktopk_decoder.py:104); page_size 16, 32, 64 or 128
  * (the reference's --page_size, benchmark/blocktopk.py:13; the token-granular
  * policies: 16 only);
  * num_q_heads % num_kv_heads == 0 and group size num_q_heads/num_kv_heads <= 16.
@@ -557,7 +557,7 @@ int kin_build_slot_page_table(const int32_t* slot_ids, const int32_t* seq_lens, 
  * per-slot contiguous caches that also gives memory back: LiteSys sizes
  * [max_batch, H_kv, max_len, D] per layer up front and clear_cache zeroes a
  * slot (ref: LiteSys/litesys/attention/batch_cache.py:40-62,147-152); here the
- * slots draw pages (of 16, 32 or 64 tokens) from one pool of num_pool_pages pages through a
+ * slots draw pages (of 16, 32, 64 or 128 tokens) from one pool of num_pool_pages pages through a
  * free list that lives on the device, so the pool can be smaller than
  * max_slots * pages_per_slot and a finished request returns its pages.  No host
  * synchronisation anywhere; every call is a single small kernel.

@@ -103,8 +103,8 @@ class PagedBatchKVManager:
                         and 0 <= self.token_local <= 1024):
                     raise NotImplementedError("strided blocks: block size <= 64, budget <= 4096 tokens, attn_local <= 1024")
                 self.block_topk = None
-            elif kwargs.get("attn_block_size", PAGE) not in (16, 32, 64):
-                raise NotImplementedError("attn_block_size must be 16, 32 or 64 (a block is one page)")
+            elif kwargs.get("attn_block_size", PAGE) not in (16, 32, 64, 128):
+                raise NotImplementedError("attn_block_size must be 16, 32, 64 or 128 (a block is one page)")
         elif kwargs.get("attn_stride") is not None:
             raise NotImplementedError("attn_stride needs attn_block_topk")
         if kwargs.get("attn_local") is not None and self.block_topk is None and self.strided is None and self.token_topk is None:

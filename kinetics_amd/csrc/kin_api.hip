@@ -39,7 +39,7 @@ int check_common_dims(const char* fn, int batch, int num_q_heads, int num_kv_hea
     return fail(KIN_ERR_UNSUPPORTED, "%s: head_dim=%d unsupported (kernels are built for %s%d)", fn, head_dim,
                 small_head_dim_built ? "64 and " : "", kHeadDim);
   if (!supported_page_size(page_size))
-    return fail(KIN_ERR_UNSUPPORTED, "%s: page_size=%d unsupported (kernels are built for 16, 32 and 64)", fn, page_size);
+    return fail(KIN_ERR_UNSUPPORTED, "%s: page_size=%d unsupported (kernels are built for 16, 32, 64 and 128)", fn, page_size);
   if (num_q_heads / num_kv_heads > kMaxGroup)
     return fail(KIN_ERR_UNSUPPORTED, "%s: GQA group %d unsupported (max %d)", fn, num_q_heads / num_kv_heads,
                 kMaxGroup);

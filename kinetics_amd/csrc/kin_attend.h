@@ -222,7 +222,7 @@ struct AttendArgs {
   int row_bytes;         // bytes between token rows of a page (H_kv * HD * 2)
   int page_bytes;        // 2 * page_size * row_bytes
   int span;              // bytes addressable from kvb within one page
-  int page_size;         // tokens per page: 16, 32 or 64
+  int page_size;         // tokens per page: 16, 32, 64 or 128
   int64_t num_pages;
   int G;
   float scale_log2;      // sm_scale * log2(e)

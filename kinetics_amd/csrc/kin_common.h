@@ -11,7 +11,7 @@ namespace kin {
 constexpr int kHeadDim = 128;    // elements per head row (256 B in bf16): the default, and the largest, head dimension
 constexpr int kHeadDimSmall = 64;  // the second head dimension the page path is built for (128-byte rows)
 constexpr int kPageSize = 16;    // tokens of one attention tile (an MFMA tile is 16 keys); the smallest page
-constexpr int kMaxPageSize = 64; // pages hold 16, 32 or 64 tokens: 1, 2 or 4 tiles
+constexpr int kMaxPageSize = 128; // pages hold 16, 32, 64 or 128 tokens: 1, 2, 4 or 8 tiles
 constexpr int kRowBytes = kHeadDim * 2;
 constexpr int kMaxGroup = 16;    // largest supported num_q_heads / num_kv_heads
 constexpr int kMaxTopk = 2048;
@@ -31,10 +31,10 @@ constexpr int kMaxLocalTokens = (kMaxFixedPages - 1) * kPageSize + 1;
 // (for 16-token pages; larger pages need no more).
 __host__ __device__ inline int max_local_pages(int local_tokens) { return 1 + (local_tokens + kPageSize - 2) / kPageSize; }
 
-inline bool supported_page_size(int ps) { return ps == 16 || ps == 32 || ps == 64; }
+inline bool supported_page_size(int ps) { return ps == 16 || ps == 32 || ps == 64 || ps == 128; }
 inline bool supported_head_dim(int hd) { return hd == kHeadDim || hd == kHeadDimSmall; }
 // log2(page_size / 16): a page is 1 << page_tile_shift(ps) tiles of 16 tokens.
-__host__ __device__ inline int page_tile_shift(int ps) { return ps >= 64 ? 2 : (ps >= 32 ? 1 : 0); }
+__host__ __device__ inline int page_tile_shift(int ps) { return ps >= 128 ? 3 : (ps >= 64 ? 2 : (ps >= 32 ? 1 : 0)); }
 
 // Cache-policy bits for buffer loads of read-once data (K/V pages, mean keys):
 // the non-temporal hint keeps streams from displacing each other in L2/MALL and

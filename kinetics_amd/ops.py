@@ -256,7 +256,7 @@ def block_score_topk(q, kbar, page_indices, page_indptr, last_page_len, topk, se
     selected pages by descending score, local pages.  ``workspace`` (uint8,
     ``step_workspace_bytes``; optional) lets few, long sequences spread their
     scoring over the GPU.  ``page_size``: tokens per page of the cache the table
-    describes (16, 32 or 64)."""
+    describes (16, 32, 64 or 128)."""
     _require(q, "q", ELEM_DTYPES, 3)
     dev = q.device
     batch, num_q_heads, head_dim = q.shape

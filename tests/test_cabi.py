@@ -55,8 +55,8 @@ def test_append_argument_errors(lib):
     assert b"64 and 128" in lib.kin_last_error()
     assert append(lib, D=64, B=0) == _lib.KIN_OK              # the page path is built for head rows of 64 and 128
     assert append(lib, ps=24) == _lib.KIN_ERR_UNSUPPORTED
-    assert append(lib, ps=128) == _lib.KIN_ERR_UNSUPPORTED
-    assert append(lib, ps=32, B=0) == _lib.KIN_OK and append(lib, ps=64, B=0) == _lib.KIN_OK
+    assert append(lib, ps=256) == _lib.KIN_ERR_UNSUPPORTED
+    assert append(lib, ps=32, B=0) == _lib.KIN_OK and append(lib, ps=64, B=0) == _lib.KIN_OK and append(lib, ps=128, B=0) == _lib.KIN_OK
     assert append(lib, kv=A + 2) == _lib.KIN_ERR_MISALIGNED
     assert b"kv_cache" in lib.kin_last_error()
     assert append(lib, B=0) == _lib.KIN_OK  # nothing to do, nothing launched

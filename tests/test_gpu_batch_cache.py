@@ -83,6 +83,8 @@ _POLICIES = [(dict(), None), (dict(attn_block_topk=3, attn_local=16), True),
              (dict(attn_block_topk=2, attn_local=20, attn_block_size=32), True),
              (dict(attn_block_topk=2, attn_local=33, attn_block_size=32), False),
              (dict(attn_block_topk=1, attn_local=7, attn_block_size=64), True),
+             (dict(attn_block_topk=1, attn_local=40, attn_block_size=128), True),
+             (dict(attn_block_topk=2, attn_local=9, attn_block_size=128), False),
              (dict(attn_local=24), False),
              (dict(attn_topk=40, attn_local=10), None),
              (dict(attn_block_topk=2, attn_local=9, attn_stride=8), None),

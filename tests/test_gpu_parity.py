@@ -403,7 +403,7 @@ def test_properties_at_scale(ops):
 # --------------------------------------------------------------------------- layer objects + custom ops
 
 
-@pytest.mark.parametrize("PS", [16, 32, 64])
+@pytest.mark.parametrize("PS", [16, 32, 64, 128])
 @pytest.mark.parametrize("fused", [False, True])
 def test_layer_objects_follow_the_reference_call_order(ops, fused, PS):
     """The attention objects with the reference constructor's arguments, at each
@@ -493,7 +493,7 @@ def test_selection_vs_the_references_bf16_scoring(ops, case):
         assert diff[~same].max() <= 0.1
 
 
-@pytest.mark.parametrize("page_size", [32, 64])
+@pytest.mark.parametrize("page_size", [32, 64, 128])
 @pytest.mark.parametrize("hkv,group", [(1, 4), (2, 8), (8, 2), (1, 3)])
 def test_pages_of_32_and_64_tokens(ops, page_size, hkv, group, head_dim):
     """Every entry point of the page path on caches with 32- and 64-token pages
@@ -2026,7 +2026,7 @@ def test_topk_zero_is_sink_plus_local_window(ops):
 # --------------------------------------------------------------------------- seeded sweep over odd shapes
 
 
-@pytest.mark.parametrize("page_size,fmt,trials", [(16, "bf16", 40), (32, "bf16", 15), (64, "bf16", 10), (16, "f16", 15), (64, "f16", 10)])
+@pytest.mark.parametrize("page_size,fmt,trials", [(16, "bf16", 40), (32, "bf16", 15), (64, "bf16", 10), (128, "bf16", 10), (16, "f16", 15), (64, "f16", 10), (128, "f16", 6)])
 def test_seeded_sweep_of_shapes(ops, page_size, fmt, trials, head_dim):
     """Seeded random configurations -- head counts, group sizes 1..8, ragged
     lengths with empty and one-token sequences, budgets above and below the

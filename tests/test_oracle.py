@@ -291,7 +291,7 @@ def test_float16_element_format_is_ieee_half():
 
 @pytest.mark.parametrize("head_dim", [128, 64])
 @pytest.mark.parametrize("fmt", ["bf16", "f16"])
-@pytest.mark.parametrize("page_size", [16, 32, 64])
+@pytest.mark.parametrize("page_size", [16, 32, 64, 128])
 def test_dense_attention_equals_torch_sdpa(page_size, fmt, head_dim):
     """Head rows of 64 elements too (LiteSys reads head_dim from the model config,
     LiteSys/litesys/attention/batch_cache.py:27): the scale follows the row length."""
@@ -327,7 +327,7 @@ def test_repaging_leaves_dense_attention_unchanged():
     rows_v = [P.randn_bf16(rng, (L, Hkv, D)) for L in lengths]
     q = P.randn_bf16(rng, (len(lengths), Hkv * G, D))
     outs = []
-    for ps in (16, 32, 64):
+    for ps in (16, 32, 64, 128):
         n_pages = [(L + ps - 1) // ps for L in lengths]
         total = sum(n_pages) + 2
         perm = rng.permutation(total).astype(np.int32)
@@ -416,7 +416,7 @@ def test_decode_step_equals_masked_dense_formulation_head_dim_64():
         test_decode_step_equals_masked_dense_formulation(64, D=64)
 
 
-@pytest.mark.parametrize("page_size", [16, 32, 64])
+@pytest.mark.parametrize("page_size", [16, 32, 64, 128])
 def test_decode_step_equals_masked_dense_formulation(page_size, D=D):
     """LiteSys expresses block sparsity as a -inf mask on full-context logits
     (sparsity_utils.py:39-45) followed by softmax and P.V; the gather form must
@@ -536,7 +536,7 @@ def test_sink_and_local_pages_are_pinned_not_candidates():
     assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
 
 
-@pytest.mark.parametrize("page_size", [16, 32, 64])
+@pytest.mark.parametrize("page_size", [16, 32, 64, 128])
 def test_split_pages_against_token_level_definition(page_size):
     """Brute force: a page is a candidate iff it comes after the sink pages and
     ends at or before the first of the newest ``local_tokens`` tokens."""
@@ -584,7 +584,7 @@ def test_litesys_mask_hand_case():
     assert O.litesys_blockwise_topk_mask(np.arange(33.0), 33, 1, local).sum() == 4 + 16 + 13
 
 
-@pytest.mark.parametrize("page_size", [16, 32, 64])
+@pytest.mark.parametrize("page_size", [16, 32, 64, 128])
 def test_page_lists_with_offset_12_equal_litesys_mask_formulation(page_size):
     """The paged formulation (sink_pages=1, local_tokens=local, sequences stored
     page_size - 4 slots into their first page: 12 for LiteSys' default blocks of 16) and
