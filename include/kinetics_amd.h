@@ -83,8 +83,11 @@ enum kin_status {
  * winners in index order.  3.0.0: every entry point that touches kbar takes
  * slot_ids / num_slots in front of the stream (kbar laid out by cache slot).
  * 3.1.0: head_dim 64 in the page path (append, mean keys, selector, sparse and
- * dense decode, the fused step, the token-granular policies), in
- * kin_qkv_norm_split and, for rows of 64 elements, in kin_rms_norm. */
+ * dense decode, the fused step), in kin_qkv_norm_split and, for rows of 64
+ * elements, in kin_rms_norm.  3.2.0: head_dim 64 in the token-granular
+ * policies, pages of 128 tokens, teams (the fused step) or a launch of their
+ * own (the token-granular policies) for the lists that a batch has beyond a
+ * multiple of 256. */
 int kin_version(void);
 
 /* Human-readable text of the last non-OK status on the calling thread

@@ -95,7 +95,7 @@ __global__ void check_page_table_kernel(const int32_t* __restrict__ page_indices
 
 extern "C" {
 
-int kin_version(void) { return 30100; }
+int kin_version(void) { return 30200; }
 
 int kin_set_team_spin_limit(int polls) {
   return kin::g_team_spin_limit.exchange(polls < 0 ? kin::kTeamSpinLimit : polls, std::memory_order_relaxed);
