@@ -448,7 +448,8 @@ def time_token_policies(torch, ops, st, B, Hkv, G, topk, nt, traffic_of):
     device = st["q"].device
     ntok, sink, window = topk * PS, 4, 16
     res = {}
-    tok_bytes = sum(Hkv * (L * 256 + min(L, ntok + sink + window) * 512 + 512) + 2 * Hkv * G * 256 for L in st["lengths"])
+    row = 2 * D   # bytes of one head row
+    tok_bytes = sum(Hkv * (L * row + min(L, ntok + sink + window) * 2 * row + 2 * row) + 2 * Hkv * G * row for L in st["lengths"])
     ws_tok = torch.empty(max(16, ops.token_topk_workspace_bytes(B, Hkv, st["max_pages_used"])), dtype=torch.uint8, device=device)
     ws_str = torch.empty(max(16, ops.strided_topk_workspace_bytes(B, Hkv, st["max_pages_used"])), dtype=torch.uint8, device=device)
     calls = {
@@ -662,6 +663,9 @@ def main():
     ap.add_argument("--page_size", type=int, default=16, choices=[16, 32, 64, 128],
                     help="tokens per page of the cache (any workload; the reference's flag, benchmark/blocktopk.py:13)")
     ap.add_argument("--world_size", type=int, default=8)
+    ap.add_argument("--head_dim", type=int, default=128, choices=[128, 64],
+                    help="elements per head row (the reference reads it from the model config, "
+                         "benchmark/blocktopk_decoder.py:104; every BASELINE configuration has 128)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float16"],
                     help="element type of q, the cache, the mean keys and the output (the reference's flag, "
                          "benchmark/blocktopk.py:18)")
@@ -675,6 +679,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes) to scale profiler byte counters")
     args = ap.parse_args()
+    global D
+    D = args.head_dim
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the path is independent per (sequence, KV head) and is run on "
               "one GPU's share of the heads; --gpus above 1 is not supported.", file=sys.stderr)
