@@ -23,6 +23,11 @@
 
 namespace kin {
 
+// A list with fewer candidates and fewer tiles to attend than this is handled by one member of its team
+// alone (see the kernel): about 2.5 + 8 us of streaming for one workgroup, what a team's overhead costs.
+constexpr int kTeamMinCandidates = 256;
+constexpr int kTeamMinTiles = 24;
+
 // HD: elements of a head row, 128 or 64.
 template <int NG, int NW, bool F16, int HD = kHeadDim>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kernel(StepParams p) {
@@ -122,6 +127,18 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void blocktopk_step_kerne
   s.sorted = p.sel_pages != nullptr;
   int32_t* table_lds = reinterpret_cast<int32_t*>(smem + select_table_offset(p.kbar_pages, p.sort_cap));
   int n;
+  if (team > 1) {
+    // Teams are planned from the batch's capacity (kbar_pages, the page budget), not from the lengths,
+    // which only the GPU knows.  A list too short to be worth sharing -- the exchange, the second
+    // select and the merge cost about 10 us -- is member 0's alone: the others leave at once and
+    // nothing goes through the workspace.
+    const int tiles = (min(s.topk, s.n_cand) + s.n_sink + s.n_local) << page_tile_shift(p.page_size);
+    if (s.n_cand < kTeamMinCandidates && tiles < kTeamMinTiles) {
+      if (member != 0) return;
+      team = parts = 1;
+      append_token();
+    }
+  }
   if (team > 1) {
     // This member's slice of the candidates -> keys in HBM.
     const int titem = item - p.head_lists;
