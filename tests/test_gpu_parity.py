@@ -1540,6 +1540,28 @@ def test_seeded_sweep_of_token_policies(ops, head_dim):
             _check_token_topk(ops, pb, topk, sink, local, offset, what)
 
 
+@pytest.mark.parametrize("policy", ["token", "strided"])
+def test_token_policies_with_nothing_to_attend(ops, policy, head_dim):
+    """No budget, no sink tokens and no local window: nothing is listed, and like an empty page list
+    (kin_sparse_paged_decode) that gives out = 0 and lse = -inf, not the NaN of a softmax over nothing
+    (LiteSys cannot get there: its sink is always 4 tokens, sparsity_utils.py:6)."""
+    pb = P.make_problem(1330, [PS * 3 + 5, 40, PS * 120 + 1], num_kv_heads=2, group=4)   # (the strided policy lists a sequence shorter than a block whole)
+    g = Gpu(pb)
+    ops.append_paged_kv(g.k, g.v, g.kv, None, g.indices, g.indptr, g.last)
+    sel = torch.full((pb.B, pb.Hkv, 16), -7, dtype=torch.int32, device=DEV)
+    cnt = torch.full((pb.B, pb.Hkv), -7, dtype=torch.int32, device=DEV)
+    lse = torch.full((pb.B, pb.Hq), float("nan"), dtype=torch.float32, device=DEV)
+    if policy == "token":
+        out = ops.token_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, 0, pb.max_pages, sink_tokens=0, local_tokens=0, lse=lse,
+                                    sel_tokens=sel, sel_count=cnt)
+    else:
+        out = ops.strided_topk_decode(g.q, g.kv, g.indices, g.indptr, g.last, 0, pb.max_pages, block_size=16, stride=8, sink_tokens=0,
+                                      local_tokens=0, lse=lse, sel_tokens=sel, sel_count=cnt)
+    torch.cuda.synchronize()
+    assert (cnt == 0).all() and (sel == -1).all()
+    assert (out == 0).all() and torch.isneginf(lse).all()
+
+
 def test_token_topk_rejects_short_workspace_and_long_sequences(ops):
     pb = P.make_problem(1310, [PS * 6 + 2, PS * 2], num_kv_heads=1, group=4)
     g = Gpu(pb)
