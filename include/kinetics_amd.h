@@ -358,7 +358,8 @@ int kin_blocktopk_decode_step(const kin_bf16_t* q, const kin_bf16_t* k, const ki
 
 /*
  * Workspace kin_blocktopk_decode_step and kin_block_score_topk can use for the
- * given problem: 0 unless the lists are few.  Up to 128 lists (batch *
+ * given problem: 0 unless the lists are few, or up to 96 more than a multiple
+ * of 256 (then for those lists).  Up to 128 lists (batch *
  * num_kv_heads) the step may hand a list to a team of workgroups that meet
  * through this memory: two arrival counters per list, 4 bytes per candidate
  * page and list for the keys, and the partial results of the members that
