@@ -157,10 +157,14 @@ class PagedBatchKVManager:
                                dtype=torch.int32, device=dev)
         self._cnt = torch.zeros(B, Hkv, dtype=torch.int32, device=dev)
         # one workspace for every kernel and every number of active sequences
-        # (batches of a few lists more than a multiple of the GPU's 256 CUs form teams for those lists: the
-        # largest needs are at 32, 72 and 96 extra lists)
-        tails = {(m + t + Hkv - 1) // Hkv for m in range(256, B * Hkv + 1, 256) for t in (32, 72, 96)}
-        sizes = sorted({1 << i for i in range(B.bit_length())} | {B} | set(range(1, min(B, 128) + 1)) | {n for n in tails if n <= B})
+        # (the needs are not monotonic in the number of sequences: few lists are shared by teams of workgroups,
+        # lists just above a multiple of the GPU's 256 CUs are split or get teams; asking for every size costs
+        # tens of milliseconds, once)
+        if B <= 8192:
+            sizes = range(1, B + 1)
+        else:
+            tails = {(m + t) // Hkv + d for m in range(256, B * Hkv + 1, 256) for t in (32, 64, 72, 96) for d in (0, 1)}
+            sizes = sorted({1 << i for i in range(B.bit_length())} | {B} | set(range(1, 129)) | {n for n in tails if 1 <= n <= B})
         ws = 16
         for n in sizes:
             ws = max(ws, ops.decode_workspace_bytes(n, Hq, Hkv, P), ops.decode_workspace_bytes(n, Hq, Hkv, self._sel.shape[2]),

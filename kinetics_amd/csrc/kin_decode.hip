@@ -119,10 +119,10 @@ static int auto_splits(int batch, int num_kv_heads, int max_pages_per_list) {
   // Measured on dense decode (8 to 1024 lists of 65 to 2049 pages, 1 to 24 splits each):
   // up to 256 lists, a little under one workgroup per CU is best (more splits only add
   // partial results and merge work), never below 4 pages -- one per wave -- a split;
-  // between 256 and 768 lists only long lists gain from splitting (300 lists of 2049
+  // between 256 and 768 lists long lists gain from splitting (300 lists of 2049
   // pages: 0.94 ms whole, 0.77 ms in four to eight parts; 513 lists: 1.51 ms whole, 1.36
-  // in four -- whole lists cannot be balanced over the CUs), and from 768 lists on every
-  // CU holds its three workgroups anyway.
+  // in four -- whole lists cannot be balanced over the CUs), shorter ones only just above a
+  // multiple of the CUs (below), and from 768 lists on every CU holds its three workgroups anyway.
   const int64_t lists = (int64_t)batch * num_kv_heads;
   if (lists <= 0) return 1;
   int64_t want = 1;
@@ -130,6 +130,12 @@ static int auto_splits(int batch, int num_kv_heads, int max_pages_per_list) {
     want = (kNumCus - kNumCus / 8 + lists / 2) / lists;
   else if (lists < 3 * kNumCus && max_pages_per_list >= 1024)
     want = (8 * kNumCus + lists - 1) / lists;
+  else if (lists < 3 * kNumCus && lists % kNumCus != 0 && lists % kNumCus <= 96 && max_pages_per_list >= 32)
+    // A few lists more than a multiple of the CUs: whole lists would leave those few running on a few
+    // CUs beside or after the others.  In parts they spread (129-page lists: 264 lists 65 -> 55 us in
+    // four parts, 300: 67 -> 58, 352: 73 -> 66 in two, 528: 108 -> 100; 257-page lists of 8 heads:
+    // 264 lists 135 -> 108, 300: 138 -> 116, 528: 225 -> 201; 400 and 640 lists: whole lists win).
+    want = lists % kNumCus <= 64 ? 4 : 2;
   int64_t cap = max_pages_per_list / 4;
   if (want > cap) want = cap;
   if (want > 64) want = 64;

@@ -255,14 +255,19 @@ def test_auto_splits_policy(lib):
 
 
 def test_auto_splits_policy_follows_the_lists(lib):
-    """Few lists: about one workgroup per CU in total; just above 256 lists only
-    long lists are split; from 768 lists on none; never fewer than 4 pages a split."""
+    """Few lists: about one workgroup per CU in total; between 256 and 768 lists long lists are
+    split, shorter ones only just above a multiple of 256; from 768 lists on none; never fewer
+    than 4 pages a split."""
     assert lib.kin_decode_auto_splits(8, 1, 2049) == 28
     assert lib.kin_decode_auto_splits(64, 1, 2049) == 4
     assert lib.kin_decode_auto_splits(4, 8, 257) == 7
     assert lib.kin_decode_auto_splits(256, 1, 2049) == 1
     assert lib.kin_decode_auto_splits(300, 1, 2049) == 7
-    assert lib.kin_decode_auto_splits(300, 1, 513) == 1
+    assert lib.kin_decode_auto_splits(300, 1, 513) == 4        # 44 lists more than one per CU
+    assert lib.kin_decode_auto_splits(352, 1, 129) == 2 and lib.kin_decode_auto_splits(528, 1, 129) == 4
+    assert lib.kin_decode_auto_splits(400, 1, 513) == 1 and lib.kin_decode_auto_splits(512, 1, 513) == 1
+    assert lib.kin_decode_auto_splits(300, 1, 17) == 1         # too short to share
+    assert lib.kin_decode_auto_splits(800, 1, 129) == 1
     assert lib.kin_decode_auto_splits(768, 1, 2049) == 1
     assert lib.kin_decode_auto_splits(1, 1, 1 << 20) == 64
     assert lib.kin_decode_auto_splits(8, 1, 17) == 4
