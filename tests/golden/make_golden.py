@@ -33,12 +33,15 @@ CASES = {
     "sink_local": (1004, [PS * 9 + 5, PS * 3 + 1], 1, 4, 2, "random", False, 1, 17, 0),
     # LiteSys' geometry: 4 sink tokens in slots 12..15 of the first page, 20 local tokens
     "sink_local_offset12": (1005, [PS * 11 + 7, PS * 6, 14], 2, 2, 3, "random", False, 1, 20, 12),
+    # head rows of 64 elements (an eleventh entry: the head dimension; 128 when absent)
+    "head_dim_64": (1006, [PS * 7 + 9, PS * 2 + 16, 5], 2, 4, 3, "random", False, 1, 17, 0, 64),
 }
 
 
 def make(name):
-    seed, lengths, hkv, group, topk, table, equal, sink, local, offset = CASES[name]
-    pb = P.make_problem(seed, lengths, num_kv_heads=hkv, group=group, topk=topk, table=table, extra_pages=1, kbar_slack=1)
+    seed, lengths, hkv, group, topk, table, equal, sink, local, offset = CASES[name][:10]
+    with P.head_dim(CASES[name][10] if len(CASES[name]) > 10 else 128):
+        pb = P.make_problem(seed, lengths, num_kv_heads=hkv, group=group, topk=topk, table=table, extra_pages=1, kbar_slack=1)
     if equal:
         pb.kbar[:] = pb.kbar[0, 0, 0]
     inputs = dict(q=pb.q, k=pb.k, v=pb.v, kv_cache=pb.kv_cache.copy(), kbar=pb.kbar.copy(),
@@ -56,6 +59,6 @@ def make(name):
 
 
 if __name__ == "__main__":
-    for n in CASES:
+    for n in (sys.argv[1:] or CASES):   # all of them, or the ones named
         make(n)
         print("wrote", n, os.path.getsize(os.path.join(HERE, f"{n}.npz")), "bytes")
